@@ -1,0 +1,190 @@
+"""The reference's layer and decode drivers, chained from the oracle kernels
+(TEST INFRASTRUCTURE ONLY).
+
+  OracleModel.execute_with_paged_kv  inference/runtime/block.go:763-1081 (LLaMA arm:
+                                     RMSNorm, SwiGLU, serial residual, no bias)
+  OracleModel.decode_with_paged_kv   inference/runtime/decode.go:339-461
+  OracleModel.decode_batched         inference/runtime/decode.go:612-654 (sequential loop)
+  OracleModel.prefill_with_paged_kv  inference/runtime/decode.go:961-1096
+The KV pool holds real data here (numpy uint16 = f16 bits, or float32), addressed as
+inference/runtime/gpu_block_pool.go:15-19,107-108.
+"""
+import math
+from dataclasses import dataclass
+from typing import List
+
+import numpy as np
+
+from . import numerics as nx
+from .host_logic import GPUBlockPool
+
+
+@dataclass
+class ModelConfig:
+    num_layers: int
+    hidden: int
+    num_heads: int
+    num_kv_heads: int
+    head_dim: int
+    ffn: int
+    vocab: int
+    eps: float = 1e-5
+    rope_theta: float = 10000.0
+    block_size: int = 16  # inference/runtime/model.go:321
+
+
+@dataclass
+class QWeight:
+    fmt: int          # numerics.FMT_*
+    data: np.ndarray  # uint8 [N, row_bytes]
+    n: int
+    k: int
+
+
+@dataclass
+class LayerWeights:
+    attn_norm: np.ndarray
+    wq: QWeight
+    wk: QWeight
+    wv: QWeight
+    wo: QWeight
+    ffn_norm: np.ndarray
+    w1: QWeight
+    w3: QWeight
+    w2: QWeight
+
+
+def _mm(a, w: QWeight, m):
+    # block.go:506-552 matMulTransposed dispatch on the quant profile
+    return nx.matmul_quant(w.fmt, a, w.data, m, w.n, w.k)
+
+
+class OracleModel:
+    def __init__(self, cfg: ModelConfig, embedding_f32, layers: List[LayerWeights], final_norm,
+                 lm_head: QWeight, max_blocks, kv_fp16=True):
+        self.cfg = cfg
+        self.embedding = np.ascontiguousarray(embedding_f32, dtype=np.float32)
+        self.layers = layers
+        self.final_norm = final_norm
+        self.lm_head = lm_head
+        self.pool = GPUBlockPool(cfg.num_layers, cfg.num_kv_heads, cfg.head_dim, cfg.block_size,
+                                 max_blocks, use_fp16=kv_fp16)
+        elems = max_blocks * 2 * cfg.block_size * cfg.num_kv_heads * cfg.head_dim
+        dt = np.uint16 if kv_fp16 else np.float32
+        self.kv = [np.zeros(elems, dtype=dt) for _ in range(cfg.num_layers)]
+
+    # ---------------------------------------------------------------- one layer
+    def execute_with_paged_kv(self, x, seq_id, layer_idx, start_pos):
+        """x [seqLen, hidden] float32, updated copy returned. block.go:763-1081."""
+        c = self.cfg
+        lw = self.layers[layer_idx]
+        seq_len = x.shape[0]
+        norm = nx.rmsnorm(x, lw.attn_norm, seq_len, c.hidden, c.eps)           # :834-837
+        q = _mm(norm, lw.wq, seq_len)                                          # :841-854
+        k = _mm(norm, lw.wk, seq_len)
+        v = _mm(norm, lw.wv, seq_len)
+        q, k = nx.rope(q, k, c.head_dim, c.num_heads, c.num_kv_heads, seq_len, start_pos, 0,
+                       c.rope_theta, False)                                    # :858
+        scale = np.float32(1.0 / math.sqrt(float(c.head_dim)))                 # :862
+        slots = self.pool.store_kv_slots(layer_idx, seq_id, start_pos, seq_len)  # :868 / :878
+        bi = [s[0] for s in slots]
+        bo = [s[1] for s in slots]
+        nx.reshape_paged_kv(k, self.kv[layer_idx], bi, bo, c.num_kv_heads, c.head_dim, c.block_size, False)
+        nx.reshape_paged_kv(v, self.kv[layer_idx], bi, bo, c.num_kv_heads, c.head_dim, c.block_size, True)
+        if seq_len == 1:                                                       # :866-874
+            bt, nb, til = self.pool.attention_args(layer_idx, seq_id)
+            attn = nx.sdpa_paged_decode(q, self.kv[layer_idx], bt, nb, c.block_size, c.num_heads,
+                                        c.num_kv_heads, c.head_dim, scale, til).reshape(1, -1)
+        elif start_pos > 0:                                                    # :881-890
+            kv_lens = [start_pos + i + 1 for i in range(seq_len)]
+            bt = self.pool.seqs[seq_id].block_tables[layer_idx]
+            attn = nx.sdpa_paged_multiquery(q, self.kv[layer_idx], bt, kv_lens, c.block_size, c.num_heads,
+                                            c.num_kv_heads, c.head_dim, scale).reshape(seq_len, -1)
+        else:                                                                  # :893-895 dense causal on F32 K/V
+            attn = nx.sdpa_prefill(q, k, v, seq_len, c.num_heads, c.num_kv_heads, c.head_dim,
+                                   scale).reshape(seq_len, -1)
+        o = _mm(attn, lw.wo, seq_len)                                          # :981-983
+        x = nx.add(x, o)                                                       # :990
+        norm = nx.rmsnorm(x, lw.ffn_norm, seq_len, c.hidden, c.eps)            # :996-998
+        gate = _mm(norm, lw.w1, seq_len)                                       # :1043-1050
+        up = _mm(norm, lw.w3, seq_len)
+        act = nx.silu_mul(gate, up)                                            # :1056
+        down = _mm(act, lw.w2, seq_len)                                        # :1058-1061
+        return nx.add(x, down)                                                 # :1077
+
+    # ---------------------------------------------------------------- drivers
+    def _ensure_seq(self, seq_id):
+        if not self.pool.has_sequence(seq_id):                                 # decode.go:361-363
+            self.pool.create_sequence(seq_id)
+
+    def _head(self, state, rows):
+        c = self.cfg
+        state = nx.rmsnorm(state, self.final_norm, rows, c.hidden, c.eps)      # model.go:207-226
+        # model.go:352-422: quantized lm_head runs one M=1 call per row (same numbers)
+        return _mm(state, self.lm_head, rows)
+
+    def decode_with_paged_kv(self, token, seq_id, pos):
+        """decode.go:339-461 with one token -> logits [vocab]."""
+        c = self.cfg
+        self._ensure_seq(seq_id)
+        x = nx.embedding([token], self.embedding, c.vocab, c.hidden)           # decode.go:405-407
+        for i in range(c.num_layers):                                          # decode.go:432-437
+            x = self.execute_with_paged_kv(x, seq_id, i, pos)
+        return self._head(x, 1)[0]
+
+    def decode_batched(self, tokens, seq_ids, positions):
+        """decode.go:612-654: the batch is a loop over sequences -> logits [B, vocab]."""
+        assert len(tokens) == len(seq_ids) == len(positions)
+        return np.stack([self.decode_with_paged_kv(t, s, p) for t, s, p in zip(tokens, seq_ids, positions)])
+
+    def prefill_with_paged_kv(self, tokens, seq_id, start_pos):
+        """decode.go:961-1096 -> logits of the last token [vocab]."""
+        c = self.cfg
+        self._ensure_seq(seq_id)
+        n = len(tokens)
+        x = nx.embedding(tokens, self.embedding, c.vocab, c.hidden)
+        for i in range(c.num_layers):
+            x = self.execute_with_paged_kv(x, seq_id, i, start_pos)
+        last = x[n - 1:n]                                                      # decode.go:1057-1066
+        return self._head(last, 1)[0]
+
+    def verify_with_paged_kv(self, tokens, seq_id, start_pos):
+        """decode.go:1446-1569: logits for every position [n, vocab]."""
+        c = self.cfg
+        self._ensure_seq(seq_id)
+        n = len(tokens)
+        x = nx.embedding(tokens, self.embedding, c.vocab, c.hidden)
+        for i in range(c.num_layers):
+            x = self.execute_with_paged_kv(x, seq_id, i, start_pos)
+        return self._head(x, n)
+
+
+def random_model(cfg: ModelConfig, seed, fmt, head_fmt, emb_fmt=None, max_blocks=64, kv_fp16=True,
+                 fmt_overrides=None):
+    """Random-init model: N(0,0.02) weights quantized to `fmt`; norm weights = 1;
+    embedding table = dequantised `emb_fmt` matrix (loader rule,
+    inference/runtime/loader.go:79-200,275-288). fmt_overrides maps a weight name
+    (wq, wk, wv, wo, w1, w2, w3) to another format."""
+    from . import quantize as qz
+    rng = np.random.default_rng(seed)
+    fo = fmt_overrides or {}
+
+    def qw(name, n, k):
+        f = fo.get(name, fmt)
+        return QWeight(f, qz.random_quant(f, rng, n, k), n, k)
+
+    qd = cfg.num_heads * cfg.head_dim
+    kvd = cfg.num_kv_heads * cfg.head_dim
+    layers = []
+    for _ in range(cfg.num_layers):
+        layers.append(LayerWeights(
+            attn_norm=np.ones(cfg.hidden, dtype=np.float32),
+            wq=qw("wq", qd, cfg.hidden), wk=qw("wk", kvd, cfg.hidden), wv=qw("wv", kvd, cfg.hidden),
+            wo=qw("wo", cfg.hidden, qd),
+            ffn_norm=np.ones(cfg.hidden, dtype=np.float32),
+            w1=qw("w1", cfg.ffn, cfg.hidden), w3=qw("w3", cfg.ffn, cfg.hidden), w2=qw("w2", cfg.hidden, cfg.ffn)))
+    ef = emb_fmt if emb_fmt is not None else head_fmt
+    emb_q = qz.random_quant(ef, rng, cfg.vocab, cfg.hidden)
+    emb = nx.dequantize(ef, emb_q, cfg.vocab * cfg.hidden).reshape(cfg.vocab, cfg.hidden)
+    head = QWeight(head_fmt, qz.random_quant(head_fmt, rng, cfg.vocab, cfg.hidden), cfg.vocab, cfg.hidden)
+    return OracleModel(cfg, emb, layers, np.ones(cfg.hidden, dtype=np.float32), head, max_blocks, kv_fp16)
