@@ -1,0 +1,202 @@
+/*
+ * vexel_hip.h -- C ABI of libvexel_hip.so, an MI355X (gfx950) compute backend for
+ * vexel's batched-decode path.
+ *
+ * Every entry point replaces one method of the Go interfaces in
+ * inference/backend/backend.go of keithballinger/vexel (cited per function as
+ * backend.go:LINE). A cgo shim binds them 1:1. Conventions:
+ *   - every device pointer argument is a raw device address (the shim passes
+ *     DevicePtr.Addr()+DevicePtr.Offset(), tensor/device.go:38-51);
+ *   - functions return VX_OK (0) or an error code; vx_last_error() gives the text.
+ *     The Go methods return nothing: the shim panics on non-zero, as the Metal
+ *     backend panics on a missing pipeline (backend/metal/backend.go:775);
+ *   - all work is enqueued on the backend's single HIP stream (FIFO, like the one
+ *     Metal command queue); only vx_sync, vx_to_host and vx_argmax wait for it;
+ *   - the library is not re-entrant: one thread at a time per backend, which is how
+ *     the reference's scheduler goroutine uses it (scheduler/scheduler.go:126-165).
+ */
+#ifndef VEXEL_HIP_H
+#define VEXEL_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct vx_backend vx_backend;
+
+enum {
+    VX_OK = 0,
+    VX_ERR_INVALID = 1,     /* bad argument (shape, alignment, null pointer) */
+    VX_ERR_OOM = 2,         /* device allocation failed */
+    VX_ERR_HIP = 3,         /* a HIP runtime call failed */
+    VX_ERR_UNSUPPORTED = 4  /* format not implemented (Q5_K, Q5_0, BF16) */
+};
+
+/* Weight formats for the generic entry points (GGUF block layouts,
+ * inference/pkg/gguf/dequant.go). */
+enum { VX_Q4_0 = 1, VX_Q8_0 = 2, VX_Q4_K = 3, VX_Q6_K = 4 };
+
+/* ---- lifetime / errors ------------------------------------------------------ */
+/* metal.NewBackend (backend/metal/backend.go:238-409); Backend.Device (backend.go:311) */
+int vx_backend_create(int device_id, vx_backend **out);
+void vx_backend_destroy(vx_backend *be);
+int vx_backend_device(const vx_backend *be);
+const char *vx_last_error(void);
+
+/* ---- memory (backend.go:313-331, 8-10, 38-43) ------------------------------- */
+/* Backend.Alloc: buffer from the per-step pool, recycled by vx_reset_pool. NULL on failure. */
+void *vx_alloc(vx_backend *be, size_t bytes);
+/* AllocPermanent (runtime/gpu_block_pool.go:73-81, runtime/block.go:445-447): survives resets. */
+void *vx_alloc_permanent(vx_backend *be, size_t bytes);
+/* Backend.Free: releases a permanent buffer; a pool buffer is left to the next reset. */
+void vx_free(vx_backend *be, void *ptr);
+/* PoolResetter.ResetPool (backend.go:8-10): every vx_alloc buffer becomes reusable. */
+void vx_reset_pool(vx_backend *be);
+/* Backend.ToDevice / ToHost: the host buffer may be reused as soon as the call returns. */
+int vx_to_device(vx_backend *be, void *dst, const void *src_host, size_t bytes);
+int vx_to_host(vx_backend *be, void *dst_host, const void *src, size_t bytes);
+/* Backend.Sync */
+int vx_sync(vx_backend *be);
+/* BufferCopier.CopyBuffer / CopyBufferBatched (backend.go:38-43): device to device. */
+int vx_copy_buffer(vx_backend *be, const void *src, size_t src_off, void *dst, size_t dst_off, size_t bytes);
+/* Batcher (backend.go:25-34): one in-order stream needs no batching or barriers; kept
+ * so the shim can satisfy the interface. */
+int vx_begin_batch(vx_backend *be);
+int vx_end_batch(vx_backend *be);
+int vx_memory_barrier(vx_backend *be);
+
+/* ---- dense F32 kernels (backend.go:337-389) --------------------------------- */
+int vx_matmul(vx_backend *be, const float *a, const float *b, float *out, int m, int n, int k);             /* :338 */
+int vx_matmul_transposed(vx_backend *be, const float *a, const float *b, float *out, int m, int n, int k); /* :341 */
+int vx_rmsnorm(vx_backend *be, const float *x, const float *weight, float *out, int rows, int cols, float eps); /* :345 */
+/* :352. k may be NULL. rope_dim 0 = full head_dim. */
+int vx_rope(vx_backend *be, float *q, float *k, int head_dim, int num_heads, int num_kv_heads, int seq_len,
+            int start_pos, int rope_dim, float theta, int rope_neox);
+int vx_silu(vx_backend *be, const float *x, float *out, int n);                           /* :356 */
+int vx_silu_mul(vx_backend *be, const float *gate, const float *up, float *out, int n);   /* :360 */
+int vx_softmax(vx_backend *be, const float *x, float *out, int rows, int cols);           /* :364 */
+int vx_add(vx_backend *be, const float *a, const float *b, float *out, int n);            /* :367 */
+int vx_mul(vx_backend *be, const float *a, const float *b, float *out, int n);            /* :370 */
+/* :374. ids int32 on device; an id outside [0,vocab) leaves its output row untouched. */
+int vx_embedding(vx_backend *be, const int32_t *ids, int num_tokens, const float *table, float *out,
+                 int vocab_size, int dim);
+/* :382. K/V head-major [numKVHeads, kv_head_stride/headDim, headDim]. */
+int vx_sdpa(vx_backend *be, const float *q, const float *k, const float *v, float *out, int kv_len,
+            int num_q_heads, int num_kv_heads, int head_dim, float scale, int kv_head_stride);
+/* :389. Q/K/V/out token-major [seqLen, heads, headDim], causal. */
+int vx_sdpa_prefill(vx_backend *be, const float *q, const float *k, const float *v, float *out, int seq_len,
+                    int num_q_heads, int num_kv_heads, int head_dim, float scale);
+/* ArgmaxOps.Argmax (backend.go:199-203): first index of the strict maximum; waits for the stream. */
+int vx_argmax(vx_backend *be, const float *input, int n, int *out_index);
+
+/* ---- QuantizedMatMul (backend.go:47-81): C[M,N] = A[M,K] * B^T, B raw GGUF blocks --- */
+int vx_matmul_q4_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :50 */
+int vx_matmul_q4_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :55 */
+int vx_matmul_q6_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :60 */
+int vx_matmul_q8_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :75 */
+/* :65, :70, :80 -- not in any BASELINE config; return VX_ERR_UNSUPPORTED. */
+int vx_matmul_q5_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k);
+int vx_matmul_q5_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k);
+int vx_matmul_bf16(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k);
+
+/* ---- PagedKVOps (backend.go:415-466) ----------------------------------------- */
+/* Pool layout per physical block: K[blockSize,numKVHeads,headDim] then V[same]
+ * (runtime/gpu_block_pool.go:15-19). */
+int vx_reshape_paged_kv(vx_backend *be, const float *src, void *dst_base, const int32_t *page_table,
+                        const int32_t *block_offsets, int num_tokens, int num_kv_heads, int head_dim,
+                        int block_size, int is_value);                                             /* :424 */
+int vx_reshape_paged_kv_f16(vx_backend *be, const float *src, void *dst_base, const int32_t *page_table,
+                            const int32_t *block_offsets, int num_tokens, int num_kv_heads, int head_dim,
+                            int block_size, int is_value);                                         /* :457 */
+int vx_sdpa_paged_decode(vx_backend *be, const float *q, const void *kv_pool, const int32_t *block_table,
+                         float *out, int num_blocks, int block_size, int num_q_heads, int num_kv_heads,
+                         int head_dim, float scale, int tokens_in_last_block);                     /* :432 */
+int vx_sdpa_paged_decode_f16(vx_backend *be, const float *q, const void *kv_pool, const int32_t *block_table,
+                             float *out, int num_blocks, int block_size, int num_q_heads, int num_kv_heads,
+                             int head_dim, float scale, int tokens_in_last_block);                 /* :436 */
+/* :447. block_tables: host array of batch_size device pointers; seq_lens: host array.
+ * pool_is_f16 selects the pool element type (the Go method is called on an F32 pool). */
+int vx_sdpa_paged_decode_batched(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
+                                 const int32_t *const *block_tables, float *out, int batch_size, int max_blocks,
+                                 int block_size, int num_q_heads, int num_kv_heads, int head_dim, float scale,
+                                 const int32_t *seq_lens);
+/* :463. kv_lens: device int32[query_len]; query i attends to positions < kv_lens[i]. */
+int vx_sdpa_paged_decode_multiquery(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
+                                    const int32_t *block_table, float *out, const int32_t *kv_lens,
+                                    int num_blocks, int block_size, int num_q_heads, int num_kv_heads,
+                                    int head_dim, float scale, int query_len);
+
+/* ---- batched-decode entry points the reference lacks ------------------------- */
+/* (its batch is a host loop, runtime/decode.go:623-650; these run the whole batch in one
+ * launch and are defined per sequence by the sequential semantics above.) */
+
+/* gguf.Dequantize on the device (pkg/gguf/dequant.go:503-538), bit-exact; used for the
+ * loader rule that keeps token_embd in F32 (runtime/loader.go:275-288). n % block == 0. */
+int vx_dequantize(vx_backend *be, int fmt, const void *src, float *dst, int64_t n);
+
+/* Any of the four formats, with an optional fused residual: out = (residual ? residual : 0) + A*B^T.
+ * The add is the same single float32 add Backend.Add would do (runtime/block.go:990,1077). */
+int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, float *out, const float *residual,
+                    int m, int n, int k);
+
+/* RoPE with one position per row (row r rotated as Backend.RoPE with seqLen=1,
+ * startPos=positions[r]) fused with the paged scatter of K and V:
+ * slot_mapping[r] = physBlock*blockSize + offset (runtime/gpu_block_pool.go:250-252).
+ * q [rows,Hq,D] is rotated in place; k is rotated and stored; v is stored. */
+int vx_rope_store_paged(vx_backend *be, float *q, const float *k, const float *v, const int32_t *positions,
+                        const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int rows,
+                        int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta);
+
+/* Ragged batched paged attention with all metadata on the device: block_tables is a
+ * padded int32 [batch, max_blocks] matrix, kv_lens int32[batch]. One query per sequence.
+ * max_kv_len bounds the launch (>= every kv_lens[i]). */
+int vx_sdpa_paged_decode_ragged(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
+                                const int32_t *block_tables, const int32_t *kv_lens, float *out, int batch,
+                                int max_blocks, int block_size, int num_q_heads, int num_kv_heads, int head_dim,
+                                float scale, int max_kv_len);
+
+/* Tree verification (medusa/tree.go:186-202 mask rule): query i attends to every pool
+ * position < tree_base and to position tree_base+j iff tree_mask[i*query_len+j] != 0
+ * (uint8 on device). */
+int vx_sdpa_paged_tree(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
+                       const int32_t *block_table, float *out, const uint8_t *tree_mask, int tree_base,
+                       int block_size, int num_q_heads, int num_kv_heads, int head_dim, float scale,
+                       int query_len);
+
+/* Row-wise argmax on the device: out_idx[r] = ArgmaxOps.Argmax(logits + r*n, n). No wait. */
+int vx_argmax_rows(vx_backend *be, const float *logits, int rows, int n, int32_t *out_idx);
+
+/* Continuous-batching step metadata built on the device by prefix scans
+ * (host restatement: scheduler/scheduler.go:290-303 + runtime/gpu_block_pool.go:234-252,
+ * 359-363). Inputs (device int32): seq_slots[batch] = row of each sequence in the
+ * block-table matrix, positions[batch] = first new position, q_lens[batch] = new tokens
+ * (NULL = 1 each). free_list[free_cap] / free_count[1] are the pool's free stack; blocks
+ * are popped from the tail in batch order exactly as the per-sequence StoreKV calls would.
+ * Outputs (device int32): cu_seqlens[batch+1], token_pos[T], slot_mapping[T], kv_lens[batch],
+ * block tables updated in place, status[1] = 0 or 1 if the pool ran out of blocks.
+ * total_tokens = sum(q_lens) is given by the caller (T). */
+int vx_pack_batch(vx_backend *be, const int32_t *seq_slots, const int32_t *positions, const int32_t *q_lens,
+                  int batch, int total_tokens, int32_t *block_tables, int max_blocks, int32_t *num_blocks,
+                  int32_t *free_list, int32_t *free_count, int block_size, int32_t *cu_seqlens,
+                  int32_t *token_pos, int32_t *slot_mapping, int32_t *kv_lens, int32_t *status);
+
+/* Stream capture of a decode step into a hipGraph (replaces the Metal command-buffer
+ * batching of runtime/decode.go:426-431). Between begin and end every vx_* compute call
+ * is recorded instead of run; vx_graph_launch replays the recording. */
+typedef struct vx_graph vx_graph;
+int vx_graph_begin_capture(vx_backend *be);
+int vx_graph_end_capture(vx_backend *be, vx_graph **out);
+int vx_graph_launch(vx_backend *be, vx_graph *g);
+void vx_graph_destroy(vx_graph *g);
+
+/* Wall-clock helpers on the backend stream (HIP events), for benchmarks. */
+int vx_timer_start(vx_backend *be);
+int vx_timer_stop_ms(vx_backend *be, float *ms);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VEXEL_HIP_H */

@@ -1,0 +1,491 @@
+"""GPU parity: every C-ABI compute entry point against the CPU oracle on the same seeded
+inputs. Integer/byte results (dequantised weights, scatter layout, argmax, packing) are
+compared bit-exactly; floating point within the stated tolerances."""
+import math
+
+import numpy as np
+import pytest
+
+from oracle import numerics as nx
+from oracle import quantize as qz
+from oracle import host_logic as hl
+
+pytestmark = pytest.mark.gpu
+
+FMTS = [nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q4_K, nx.FMT_Q6_K]
+
+
+@pytest.fixture(scope="module")
+def be():
+    from vexel_amd.backend import HipBackend
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+def _close(got, want, rtol, atol, what=""):
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    lim = atol + rtol * np.abs(want.astype(np.float64))
+    assert np.all(err <= lim), "%s: max err %.3e (limit %.3e at worst element)" % (
+        what, err.max(), lim.reshape(-1)[err.argmax()])
+
+
+# ------------------------------------------------------------------ dequant: bit exact
+@pytest.mark.parametrize("fmt", FMTS)
+def test_dequantize_bit_exact(be, fmt):
+    rng = np.random.default_rng(100 + fmt)
+    n, k = 37, 1024
+    w = qz.random_quant(fmt, rng, n, k)
+    # adversarial header bits: random f16 scales including subnormals and negative values
+    raw = w.reshape(-1).copy()
+    want = nx.dequantize(fmt, raw, n * k)
+    dw = be.upload(raw)
+    dout = be.alloc(n * k * 4)
+    be.dequantize(fmt, dw, dout, n * k)
+    got = be.download(dout, (n * k,), np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    be.reset_pool()
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_dequantize_all_byte_patterns(be, fmt):
+    """Blocks filled with every byte value, finite random scales: covers every code."""
+    rng = np.random.default_rng(7)
+    bb, be_ = nx.BLOCK_BYTES[fmt], nx.BLOCK_ELEMS[fmt]
+    nblk = 512
+    raw = rng.integers(0, 256, size=(nblk, bb), dtype=np.uint8)
+    # keep f16 headers finite (exponent != 31) so NaN payload rules do not enter
+    def fix(col):
+        hi = raw[:, col + 1]
+        bad = (hi & 0x7C) == 0x7C
+        raw[bad, col + 1] = hi[bad] & 0xBF
+    if fmt in (nx.FMT_Q4_0, nx.FMT_Q8_0):
+        fix(0)
+    elif fmt == nx.FMT_Q4_K:
+        fix(0); fix(2)
+    else:
+        fix(208)
+    want = nx.dequantize(fmt, raw.reshape(-1), nblk * be_)
+    d = be.upload(raw)
+    o = be.alloc(nblk * be_ * 4)
+    be.dequantize(fmt, d, o, nblk * be_)
+    got = be.download(o, (nblk * be_,), np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    be.reset_pool()
+
+
+# ------------------------------------------------------------------ quantized matmul
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 32, 40])
+def test_matmul_quant_vs_oracle(be, fmt, m):
+    rng = np.random.default_rng(fmt * 100 + m)
+    n, k = 80, 1024
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    want = nx.matmul_quant(fmt, a, w, m, n, k)
+    da, dw = be.upload(a), be.upload(w)
+    dout = be.alloc(m * n * 4)
+    name = {nx.FMT_Q4_0: be.matmul_q4_0, nx.FMT_Q8_0: be.matmul_q8_0, nx.FMT_Q4_K: be.matmul_q4_k,
+            nx.FMT_Q6_K: be.matmul_q6_k}[fmt]
+    name(da, dw, dout, m, n, k)
+    got = be.download(dout, (m, n), np.float32)
+    # float32 summation-order level: far inside the 1e-2 abs / 1e-3 rel logits budget
+    scale = np.abs(want).max()
+    _close(got, want, 2e-5, 2e-6 * scale + 1e-7, "matmul fmt %d m %d" % (fmt, m))
+    be.reset_pool()
+
+
+@pytest.mark.parametrize("fmt", [nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q4_K])
+def test_matmul_rows_independent_of_batch(be, fmt):
+    """A row computed alone has the same bits as inside a batch (sequential-loop semantics of
+    the reference, backend/metal/backend.go:777-779)."""
+    rng = np.random.default_rng(9)
+    m, n, k = 32, 96, 2048
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    da, dw = be.upload(a), be.upload(w)
+    dout = be.alloc(m * n * 4)
+    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
+    full = be.download(dout, (m, n), np.float32)
+    for r in (0, 5, 31):
+        d1 = be.alloc(n * 4)
+        be.matmul_quant(fmt, da + r * k * 4, dw, d1, None, 1, n, k)
+        one = be.download(d1, (n,), np.float32)
+        assert np.array_equal(one.view(np.uint32), full[r].view(np.uint32))
+    be.reset_pool()
+
+
+def test_matmul_quant_residual_and_shapes(be):
+    rng = np.random.default_rng(11)
+    for (m, n, k) in [(2, 33, 512), (32, 4096, 4096), (5, 100, 11008)]:
+        w = qz.random_quant(nx.FMT_Q4_0, rng, n, k)
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        res = rng.standard_normal((m, n)).astype(np.float32)
+        want = nx.add(res, nx.matmul_q4_0(a, w, m, n, k))
+        da, dw, dr = be.upload(a), be.upload(w), be.upload(res)
+        be.matmul_quant(nx.FMT_Q4_0, da, dw, dr, dr, m, n, k)   # in place on the residual
+        got = be.download(dr, (m, n), np.float32)
+        _close(got, want, 2e-5, 1e-5, "residual %s" % ((m, n, k),))
+        be.reset_pool()
+
+
+def test_matmul_quant_unaligned_k_uses_fallback(be):
+    rng = np.random.default_rng(12)
+    m, n, k = 3, 20, 96   # K not a multiple of 256
+    w = qz.random_quant(nx.FMT_Q4_0, rng, n, k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    da, dw = be.upload(a), be.upload(w)
+    dout = be.alloc(m * n * 4)
+    be.matmul_q4_0(da, dw, dout, m, n, k)
+    _close(be.download(dout, (m, n), np.float32), nx.matmul_q4_0(a, w, m, n, k), 1e-5, 1e-6, "fallback")
+    be.reset_pool()
+
+
+def test_unsupported_formats_report(be):
+    from vexel_amd.backend import VexelError
+    for fn in (be.matmul_q5_k, be.matmul_q5_0, be.matmul_bf16):
+        with pytest.raises(VexelError) as e:
+            fn(0, 0, 0, 1, 32, 32)
+        assert e.value.code == 4
+
+
+def test_matmul_f32(be):
+    rng = np.random.default_rng(13)
+    m, n, k = 7, 45, 100
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal((n, k)).astype(np.float32)
+    da, db = be.upload(a), be.upload(b)
+    do = be.alloc(m * n * 4)
+    be.matmul_transposed(da, db, do, m, n, k)
+    _close(be.download(do, (m, n), np.float32), nx.matmul_t_f32(a, b, m, n, k), 1e-5, 1e-5, "matmul_t")
+    dbt = be.upload(np.ascontiguousarray(b.T))
+    be.matmul(da, dbt, do, m, n, k)
+    _close(be.download(do, (m, n), np.float32), nx.matmul_f32(a, b.T.copy(), m, n, k), 1e-5, 1e-5, "matmul")
+    be.reset_pool()
+
+
+# ------------------------------------------------------------------ elementwise
+def test_rmsnorm_rope_silu_add_softmax_embedding_argmax(be):
+    rng = np.random.default_rng(20)
+    rows, cols = 5, 2048
+    x = (rng.standard_normal((rows, cols)) * 2).astype(np.float32)
+    w = rng.standard_normal(cols).astype(np.float32)
+    dx, dw = be.upload(x), be.upload(w)
+    do = be.alloc(x.nbytes)
+    be.rmsnorm(dx, dw, do, rows, cols, 1e-5)
+    _close(be.download(do, x.shape, np.float32), nx.rmsnorm(x, w, rows, cols, 1e-5), 2e-6, 1e-7, "rmsnorm")
+
+    hq, hk, d, s = 8, 2, 64, 6
+    q = rng.standard_normal((s, hq, d)).astype(np.float32)
+    k = rng.standard_normal((s, hk, d)).astype(np.float32)
+    for neox, rd in ((False, 0), (True, 0), (False, 32)):
+        dq, dk = be.upload(q), be.upload(k)
+        be.rope(dq, dk, d, hq, hk, s, 1234, rd, 10000.0, neox)
+        wq, wk = nx.rope(q, k, d, hq, hk, s, 1234, rd, 10000.0, neox)
+        _close(be.download(dq, q.shape, np.float32), wq.reshape(q.shape), 0, 1e-6, "rope q")
+        _close(be.download(dk, k.shape, np.float32), wk.reshape(k.shape), 0, 1e-6, "rope k")
+    dq = be.upload(q)
+    be.rope(dq, 0, d, hq, 0, s, 0, 0, 500000.0, False)   # k = nil is allowed (cpu.go:269)
+    wq, _ = nx.rope(q, None, d, hq, 0, s, 0, 0, 500000.0, False)
+    _close(be.download(dq, q.shape, np.float32), wq.reshape(q.shape), 0, 1e-6, "rope q only")
+
+    n = 11008 * 3
+    g = (rng.standard_normal(n) * 3).astype(np.float32)
+    u = rng.standard_normal(n).astype(np.float32)
+    dg, du = be.upload(g), be.upload(u)
+    dn = be.alloc(n * 4)
+    be.silu_mul(dg, du, dn, n)
+    _close(be.download(dn, (n,), np.float32), nx.silu_mul(g, u), 1e-6, 1e-9, "silu_mul")
+    be.silu(dg, dn, n)
+    _close(be.download(dn, (n,), np.float32), nx.silu(g), 1e-6, 1e-9, "silu")
+    be.add(dg, du, dn, n)
+    assert np.array_equal(be.download(dn, (n,), np.float32), nx.add(g, u))
+    be.mul(dg, du, dn, n)
+    assert np.array_equal(be.download(dn, (n,), np.float32), nx.mul(g, u))
+
+    sm = (rng.standard_normal((4, 333)) * 5).astype(np.float32)
+    ds = be.upload(sm)
+    dso = be.alloc(sm.nbytes)
+    be.softmax(ds, dso, 4, 333)
+    _close(be.download(dso, sm.shape, np.float32), nx.softmax(sm, 4, 333), 2e-6, 1e-9, "softmax")
+
+    table = rng.standard_normal((50, 64)).astype(np.float32)
+    ids = np.array([3, 49, -1, 50, 0], dtype=np.int32)
+    dt, di = be.upload(table), be.upload(ids)
+    init = np.full((5, 64), 7.0, dtype=np.float32)
+    de = be.upload(init)
+    be.embedding(di, 5, dt, de, 50, 64)
+    assert np.array_equal(be.download(de, (5, 64), np.float32), nx.embedding(ids, table, 50, 64, out=init.copy()))
+
+    lg = rng.standard_normal((6, 32000)).astype(np.float32)
+    lg[1, 777] = lg[1, 20000] = 50.0          # tie -> lowest index
+    lg[2, :] = -np.inf                         # all -inf -> 0
+    lg[3, 5] = np.nan; lg[3, 9] = 60.0         # NaN never wins
+    lg[4, 31999] = 99.0
+    dl = be.upload(lg)
+    di = be.alloc(6 * 4)
+    be.argmax_rows(dl, 6, 32000, di)
+    got = be.download(di, (6,), np.int32)
+    assert list(got) == [nx.argmax(lg[r]) for r in range(6)]
+    assert be.argmax(dl + 4 * 32000 * 4, 32000) == 31999
+    be.reset_pool()
+
+
+# ------------------------------------------------------------------ attention
+def test_sdpa_and_prefill(be):
+    rng = np.random.default_rng(30)
+    for (hq, hk, d, L, stride) in [(1, 1, 4, 1, 1), (8, 2, 64, 300, 512), (4, 4, 128, 1500, 1500), (2, 1, 2, 3, 3)]:
+        q = rng.standard_normal((hq, d)).astype(np.float32)
+        k = rng.standard_normal((hk, stride, d)).astype(np.float32)
+        v = rng.standard_normal((hk, stride, d)).astype(np.float32)
+        sc = np.float32(1 / math.sqrt(d))
+        dq, dk, dv = be.upload(q), be.upload(k), be.upload(v)
+        do = be.alloc(q.nbytes)
+        be.sdpa(dq, dk, dv, do, L, hq, hk, d, sc, stride * d)
+        _close(be.download(do, q.shape, np.float32), nx.sdpa(q, k, v, L, hq, hk, d, sc, stride * d), 1e-5, 2e-6, "sdpa")
+        be.reset_pool()
+    s, hq, hk, d = 70, 4, 2, 64
+    q = rng.standard_normal((s, hq, d)).astype(np.float32)
+    k = rng.standard_normal((s, hk, d)).astype(np.float32)
+    v = rng.standard_normal((s, hk, d)).astype(np.float32)
+    sc = np.float32(1 / math.sqrt(d))
+    dq, dk, dv = be.upload(q), be.upload(k), be.upload(v)
+    do = be.alloc(q.nbytes)
+    be.sdpa_prefill(dq, dk, dv, do, s, hq, hk, d, sc)
+    _close(be.download(do, q.shape, np.float32), nx.sdpa_prefill(q, k, v, s, hq, hk, d, sc), 1e-5, 2e-6, "prefill")
+    be.reset_pool()
+
+
+def _make_pool(rng, f16, nblocks, bs, hk, d):
+    elems = nblocks * 2 * bs * hk * d
+    vals = rng.standard_normal(elems).astype(np.float32)
+    return nx.f32_to_f16_array(vals) if f16 else vals
+
+
+@pytest.mark.parametrize("f16", [False, True])
+def test_reshape_paged_kv_exact_layout(be, f16):
+    """inference/backend/metal/paged_test.go:10-128: exact equality of the scattered layout."""
+    rng = np.random.default_rng(31)
+    bs, hk, d, nblocks, t = 16, 4, 64, 12, 21
+    src = (rng.standard_normal((t, hk, d)) * 3).astype(np.float32)
+    bi = rng.integers(0, nblocks, t).astype(np.int32)
+    bo = rng.integers(0, bs, t).astype(np.int32)
+    # distinct (block, offset) pairs so the result does not depend on write order
+    pairs = set()
+    for i in range(t):
+        while (int(bi[i]), int(bo[i])) in pairs:
+            bo[i] = (bo[i] + 1) % bs
+            if bo[i] == 0:
+                bi[i] = (bi[i] + 1) % nblocks
+        pairs.add((int(bi[i]), int(bo[i])))
+    pool = _make_pool(rng, f16, nblocks, bs, hk, d)
+    want = pool.copy()
+    dpool, dsrc, dbi, dbo = be.upload(pool), be.upload(src), be.upload(bi), be.upload(bo)
+    fn = be.reshape_paged_kv_f16 if f16 else be.reshape_paged_kv
+    for isv in (False, True):
+        fn(dsrc, dpool, dbi, dbo, t, hk, d, bs, isv)
+        nx.reshape_paged_kv(src, want, bi, bo, hk, d, bs, isv)
+    got = be.download(dpool, pool.shape, pool.dtype)
+    assert np.array_equal(got, want)
+    be.reset_pool()
+
+
+@pytest.mark.parametrize("f16", [False, True])
+@pytest.mark.parametrize("shape", [(32, 4, 64), (32, 32, 128), (8, 8, 128), (4, 2, 32)])
+def test_paged_decode_single_batched_ragged(be, f16, shape):
+    hq, hk, d = shape
+    rng = np.random.default_rng(32 + hq + d)
+    bs, nblocks = 16, 200
+    pool = _make_pool(rng, f16, nblocks, bs, hk, d)
+    dpool = be.upload(pool)
+    sc = np.float32(1 / math.sqrt(d))
+    lens = [1, 15, 16, 17, 513, 700, 1024, 37]
+    perm = rng.permutation(nblocks)
+    tables, off = [], 0
+    for L in lens:
+        nb = (L + bs - 1) // bs
+        tables.append(perm[off:off + nb].astype(np.int32)); off += nb
+    B = len(lens)
+    q = rng.standard_normal((B, hq, d)).astype(np.float32)
+    dq = be.upload(q)
+    want = np.stack([nx.sdpa_paged_decode(q[i], pool, tables[i], len(tables[i]), bs, hq, hk, d, sc,
+                                          lens[i] - (len(tables[i]) - 1) * bs) for i in range(B)])
+    # single-sequence entry points
+    single = be.sdpa_paged_decode_f16 if f16 else be.sdpa_paged_decode
+    for i in (0, 3, 5):
+        dbt = be.upload(tables[i])
+        do = be.alloc(hq * d * 4)
+        single(dq + i * hq * d * 4, dpool, dbt, do, len(tables[i]), bs, hq, hk, d, sc,
+               lens[i] - (len(tables[i]) - 1) * bs)
+        _close(be.download(do, (hq, d), np.float32), want[i], 1e-5, 3e-6, "paged single %d" % i)
+    # Go-style batched (host arrays of device pointers)
+    ptrs = [be.upload(t) for t in tables]
+    mb = max(len(t) for t in tables)
+    do = be.alloc(q.nbytes)
+    be.sdpa_paged_decode_batched(dq, dpool, ptrs, do, B, mb, bs, hq, hk, d, sc, lens, pool_is_f16=f16)
+    _close(be.download(do, q.shape, np.float32), want, 1e-5, 3e-6, "paged batched")
+    # ragged (device matrix + device lengths)
+    mat = np.full((B, mb), -1, dtype=np.int32)
+    for i, t in enumerate(tables):
+        mat[i, :len(t)] = t
+    mat[mat < 0] = 0
+    dmat, dl = be.upload(mat), be.upload(np.array(lens, dtype=np.int32))
+    do2 = be.alloc(q.nbytes)
+    be.sdpa_paged_decode_ragged(dq, dpool, f16, dmat, dl, do2, B, mb, bs, hq, hk, d, sc, max(lens))
+    _close(be.download(do2, q.shape, np.float32), want, 1e-5, 3e-6, "paged ragged")
+    be.reset_pool()
+
+
+def test_paged_multiquery_and_tree(be):
+    rng = np.random.default_rng(34)
+    bs, hq, hk, d, nblocks = 16, 8, 2, 64, 40
+    for f16 in (False, True):
+        pool = _make_pool(rng, f16, nblocks, bs, hk, d)
+        dpool = be.upload(pool)
+        bt = rng.permutation(nblocks)[:20].astype(np.int32)
+        dbt = be.upload(bt)
+        sc = np.float32(1 / math.sqrt(d))
+        qn = 6
+        q = rng.standard_normal((qn, hq, d)).astype(np.float32)
+        dq = be.upload(q)
+        kvl = np.array([100 + i + 1 for i in range(qn)], dtype=np.int32)   # block.go:884-887
+        dk = be.upload(kvl)
+        do = be.alloc(q.nbytes)
+        be.sdpa_paged_decode_multiquery(dq, dpool, dbt, do, dk, len(bt), bs, hq, hk, d, sc, qn, pool_is_f16=f16)
+        want = nx.sdpa_paged_multiquery(q, pool, bt, kvl, bs, hq, hk, d, sc)
+        _close(be.download(do, q.shape, np.float32), want, 1e-5, 3e-6, "multiquery")
+        parent = [-1, -1, 0, 0, 1, 1]
+        mask = np.array(hl.build_tree_attention_mask(6, parent), dtype=np.uint8)
+        dm = be.upload(mask)
+        be.sdpa_paged_tree(dq, dpool, f16, dbt, do, dm, 200, bs, hq, hk, d, sc, qn)
+        want = nx.sdpa_paged_multiquery(q, pool, bt, None, bs, hq, hk, d, sc, tree_mask=mask, tree_base=200)
+        _close(be.download(do, q.shape, np.float32), want, 1e-5, 3e-6, "tree")
+        be.reset_pool()
+
+
+def test_rope_store_paged(be):
+    rng = np.random.default_rng(35)
+    rows, hq, hk, d, bs, nblocks = 9, 8, 2, 64, 16, 30
+    q = rng.standard_normal((rows, hq, d)).astype(np.float32)
+    k = rng.standard_normal((rows, hk, d)).astype(np.float32)
+    v = rng.standard_normal((rows, hk, d)).astype(np.float32)
+    pos = rng.integers(0, 4000, rows).astype(np.int32)
+    slots = rng.permutation(nblocks * bs)[:rows].astype(np.int32)
+    for f16 in (False, True):
+        pool = _make_pool(rng, f16, nblocks, bs, hk, d)
+        want_pool = pool.copy()
+        wq, wk = nx.rope_positions(q, k, d, hq, hk, pos, 0, 10000.0, False)
+        nx.reshape_paged_kv(wk, want_pool, slots // bs, slots % bs, hk, d, bs, False)
+        nx.reshape_paged_kv(v, want_pool, slots // bs, slots % bs, hk, d, bs, True)
+        dq, dk, dv = be.upload(q), be.upload(k), be.upload(v)
+        dpool, dp, ds = be.upload(pool), be.upload(pos), be.upload(slots)
+        be.rope_store_paged(dq, dk, dv, dp, ds, dpool, f16, rows, hq, hk, d, bs, 10000.0)
+        _close(be.download(dq, q.shape, np.float32), wq.reshape(q.shape), 0, 1e-6, "rope_store q")
+        got = be.download(dpool, pool.shape, pool.dtype)
+        if f16:
+            # K is rotated in float32 then rounded: allow the f16 neighbour where the f32 values differ in the last bit
+            diff = np.abs(nx.f16_to_f32_array(got) - nx.f16_to_f32_array(want_pool))
+            tol = np.abs(nx.f16_to_f32_array(want_pool)) * 2.0 ** -10 + 1e-7
+            assert np.all(diff <= tol)
+            assert np.mean(got != want_pool) < 1e-3
+        else:
+            _close(got, want_pool, 0, 1e-6, "rope_store pool")
+        be.reset_pool()
+
+
+# ------------------------------------------------------------------ packing: bit exact
+def test_pack_batch_bit_exact(be):
+    rng = np.random.default_rng(40)
+    bs, max_blocks, nslots, pool_blocks = 16, 20, 12, 150
+    for trial in range(6):
+        ref = hl.GPUBlockPool(1, 1, 8, bs, pool_blocks)
+        tables = np.zeros((nslots, max_blocks), dtype=np.int32)
+        nblk = np.zeros(nslots, dtype=np.int32)
+        ctx = rng.integers(0, 200, nslots)
+        for s in range(nslots):
+            ref.create_sequence(s)
+            if ctx[s] > 0:
+                ref.store_kv_slots(0, s, 0, int(ctx[s]))
+            bt = ref.seqs[s].block_tables[0]
+            tables[s, :len(bt)] = bt; nblk[s] = len(bt)
+        free = np.zeros(pool_blocks, dtype=np.int32)
+        fl = ref.free_lists[0]
+        free[:len(fl)] = fl
+        batch_slots = rng.permutation(nslots)[:rng.integers(1, nslots + 1)].astype(np.int32)
+        qlens = (rng.integers(1, 40, batch_slots.size) if trial % 2 else np.ones(batch_slots.size)).astype(np.int32)
+        pos = np.array([ctx[s] for s in batch_slots], dtype=np.int32)
+        T = int(qlens.sum())
+        want = hl.pack_batch(ref, 0, [int(s) for s in batch_slots], [int(p) for p in pos], [int(x) for x in qlens])
+        d = {k: be.upload(v) for k, v in dict(slots=batch_slots, pos=pos, ql=qlens, tables=tables, nblk=nblk,
+                                              free=free, fc=np.array([len(fl)], dtype=np.int32)).items()}
+        B = batch_slots.size
+        cu, tp, sm, kl, st = (be.alloc((B + 1) * 4), be.alloc(T * 4), be.alloc(T * 4), be.alloc(B * 4), be.alloc(4))
+        be.pack_batch(d["slots"], d["pos"], d["ql"] if trial % 2 else 0, B, T, d["tables"], max_blocks, d["nblk"],
+                      d["free"], d["fc"], bs, cu, tp, sm, kl, st)
+        assert be.download(st, (1,), np.int32)[0] == 0
+        assert list(be.download(cu, (B + 1,), np.int32)) == want["cu_seqlens"]
+        assert list(be.download(tp, (T,), np.int32)) == want["token_pos"]
+        assert list(be.download(sm, (T,), np.int32)) == want["slot_mapping"]
+        assert list(be.download(kl, (B,), np.int32)) == want["kv_lens"]
+        got_tables = be.download(d["tables"], tables.shape, np.int32)
+        got_nblk = be.download(d["nblk"], nblk.shape, np.int32)
+        for s in range(nslots):
+            bt = ref.seqs[s].block_tables[0]
+            assert got_nblk[s] == len(bt) and list(got_tables[s, :len(bt)]) == bt
+        assert be.download(d["fc"], (1,), np.int32)[0] == len(ref.free_lists[0])
+        be.reset_pool()
+    # exhaustion: status 1 and nothing changed
+    tables = np.zeros((1, 4), dtype=np.int32); nblk = np.zeros(1, dtype=np.int32)
+    free = np.arange(2, dtype=np.int32)
+    d_t, d_n, d_f, d_c = be.upload(tables), be.upload(nblk), be.upload(free), be.upload(np.array([2], dtype=np.int32))
+    d_s, d_p, d_q = be.upload(np.zeros(1, np.int32)), be.upload(np.zeros(1, np.int32)), be.upload(np.array([48], np.int32))
+    cu, tp, sm, kl, st = be.alloc(8), be.alloc(48 * 4), be.alloc(48 * 4), be.alloc(4), be.alloc(4)
+    be.pack_batch(d_s, d_p, d_q, 1, 48, d_t, 4, d_n, d_f, d_c, 16, cu, tp, sm, kl, st)
+    assert be.download(st, (1,), np.int32)[0] == 1
+    assert be.download(d_c, (1,), np.int32)[0] == 2 and be.download(d_n, (1,), np.int32)[0] == 0
+    be.reset_pool()
+
+
+def test_pool_alloc_reset_and_copy(be):
+    a = be.alloc(1000); b = be.alloc(1000)
+    assert a and b and a != b and a % 256 == 0
+    be.reset_pool()
+    assert be.alloc(1000) == a            # recycled after ResetPool
+    p = be.alloc_permanent(4096)
+    be.reset_pool()
+    x = np.arange(1024, dtype=np.float32)
+    be.to_device(p, x)
+    q = be.alloc_permanent(4096)
+    be.copy_buffer(p, 1024, q, 2048, 1024)
+    got = be.download(q + 2048, (256,), np.float32)
+    assert np.array_equal(got, x[256:512])
+    be.free(p); be.free(q)
+    be.begin_batch(); be.memory_barrier(); be.end_batch()
+
+
+def test_graph_capture_replays_match_eager(be):
+    rng = np.random.default_rng(50)
+    m, n, k = 4, 256, 1024
+    w = qz.random_quant(nx.FMT_Q4_0, rng, n, k)
+    dw = be.upload(w, permanent=True)
+    da = be.alloc_permanent(m * k * 4); do = be.alloc_permanent(m * n * 4); dn = be.alloc_permanent(m * n * 4)
+    nw = be.upload(np.ones(n, dtype=np.float32), permanent=True)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    be.to_device(da, a)
+    be.matmul_q4_0(da, dw, do, m, n, k)           # warm-up sizes the scratch
+    be.graph_begin_capture()
+    be.matmul_q4_0(da, dw, do, m, n, k)
+    be.rmsnorm(do, nw, dn, m, n, 1e-5)
+    g = be.graph_end_capture()
+    for it in range(4):
+        a = rng.standard_normal((m, k)).astype(np.float32)
+        be.to_device(da, a)
+        be.graph_launch(g)
+        got = be.download(dn, (m, n), np.float32)
+        be.matmul_q4_0(da, dw, do, m, n, k)
+        be.rmsnorm(do, nw, dn, m, n, 1e-5)
+        eager = be.download(dn, (m, n), np.float32)
+        assert np.array_equal(got, eager)
+    be.graph_destroy(g)
+    for p in (dw, da, do, dn, nw):
+        be.free(p)

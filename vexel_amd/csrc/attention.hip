@@ -1,0 +1,567 @@
+// Attention kernels.
+//
+//  * attn_generic_kernel: any head_dim <= 256, F32 or F16 K/V, three addressing modes
+//    (head-major contiguous, token-major causal prefill, paged through a block table),
+//    optional per-query kv length and optional tree mask. One workgroup per (query, head),
+//    online softmax over chunks of positions. Serves Backend.SDPA, SDPAPrefill and the
+//    single-sequence PagedKVOps methods.
+//  * paged_decode_f16_kernel + paged_merge_kernel: the batched-decode hot path. Ragged
+//    batch, F16 pool, one query per sequence, split over the KV length so a launch has
+//    thousands of workgroups whatever the mix of context lengths. HBM-bound: every K/V
+//    byte is read once with 16-byte loads, a token's head vector is one contiguous
+//    2*head_dim-byte run shared by head_dim/8 lanes.
+//
+// Arithmetic: float32 dot products and accumulation, softmax through exp2 of the
+// max-subtracted score; the CPU reference (backend/cpu/cpu.go:568-632) normalises the
+// weights before the V accumulation, here the accumulator is divided once at the end.
+#include <float.h>
+
+#include "common.h"
+
+using namespace vx;
+
+namespace {
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+enum { MODE_CONTIG = 0, MODE_PREFILL = 1, MODE_PAGED = 2 };
+
+struct AttnParams {
+    const float *q;
+    float *out;
+    const void *k;  // contiguous / prefill: K base; paged: pool base
+    const void *v;  // contiguous / prefill: V base; paged: unused
+    int mode;
+    int f16;
+    int num_q_heads, num_kv_heads, head_dim;
+    float scale;
+    // contiguous
+    int kv_head_stride;
+    int kv_len;  // fixed kv length (contiguous, single paged decode); ignored when kv_lens != nullptr
+    // paged
+    const int32_t *block_table;          // one table (single sequence / multiquery / tree)
+    const int32_t *const *bt_ptrs;       // per-query tables (batched), or nullptr
+    const int32_t *bt_matrix;            // padded [batch,max_blocks] matrix, or nullptr
+    int max_blocks;
+    int block_size;
+    const int32_t *kv_lens;              // per-query kv length (device), or nullptr
+    // tree mask
+    const uint8_t *tree_mask;
+    int tree_base;
+    int query_len;
+};
+
+__device__ __forceinline__ float ld_elem(const void *base, size_t idx, int f16) {
+    return f16 ? (float)((const _Float16 *)base)[idx] : ((const float *)base)[idx];
+}
+
+constexpr int GEN_THREADS = 256;
+constexpr int GEN_CHUNK = 1024;
+
+__global__ void __launch_bounds__(GEN_THREADS) attn_generic_kernel(AttnParams p) {
+    __shared__ float s_scores[GEN_CHUNK];
+    __shared__ float s_red[GEN_THREADS / 64];
+    __shared__ float s_acc[GEN_THREADS];
+    __shared__ float s_q[256];
+
+    const int h = blockIdx.x, qi = blockIdx.y, tid = threadIdx.x;
+    const int D = p.head_dim;
+    const int kvh = h / (p.num_q_heads / p.num_kv_heads);
+    const size_t qoff = ((size_t)qi * p.num_q_heads + h) * D;
+
+    int kv_len;
+    const int32_t *bt = nullptr;
+    if (p.mode == MODE_PREFILL) {
+        kv_len = qi + 1;
+    } else if (p.tree_mask) {
+        kv_len = p.tree_base + p.query_len;
+    } else {
+        kv_len = p.kv_lens ? p.kv_lens[qi] : p.kv_len;
+    }
+    if (p.mode == MODE_PAGED) {
+        if (p.bt_ptrs)
+            bt = p.bt_ptrs[qi];
+        else if (p.bt_matrix)
+            bt = p.bt_matrix + (size_t)qi * p.max_blocks;
+        else
+            bt = p.block_table;
+    }
+    for (int d = tid; d < D; d += GEN_THREADS) s_q[d] = p.q[qoff + d];
+    __syncthreads();
+
+    const size_t hs = (size_t)p.num_kv_heads * D;
+    const size_t part = (size_t)p.block_size * hs;
+    auto krow = [&](int pos) -> size_t {
+        if (p.mode == MODE_CONTIG) return (size_t)kvh * p.kv_head_stride + (size_t)pos * D;
+        if (p.mode == MODE_PREFILL) return ((size_t)pos * p.num_kv_heads + kvh) * D;
+        return (size_t)bt[pos / p.block_size] * 2 * part + (size_t)(pos % p.block_size) * hs + (size_t)kvh * D;
+    };
+    const void *vbase = (p.mode == MODE_PAGED) ? p.k : p.v;
+    const size_t vadd = (p.mode == MODE_PAGED) ? part : 0;
+
+    // accumulation layout: thread t owns dimension t % D for the position subset t / D
+    const int ng = (GEN_THREADS / D) > 0 ? (GEN_THREADS / D) : 1;
+    const int my_d = tid % D, my_g = tid / D;
+    const bool acc_active = my_g < ng && tid < ng * D;
+    float acc = 0.f, m_run = -INFINITY, l_run = 0.f;
+
+    for (int c0 = 0; c0 < kv_len; c0 += GEN_CHUNK) {
+        int cn = min(GEN_CHUNK, kv_len - c0);
+        float lmax = -INFINITY;
+        for (int i = tid; i < cn; i += GEN_THREADS) {
+            int pos = c0 + i;
+            float sc;
+            bool masked = p.tree_mask && pos >= p.tree_base &&
+                          !p.tree_mask[(size_t)qi * p.query_len + (pos - p.tree_base)];
+            if (masked) {
+                sc = -INFINITY;
+            } else {
+                size_t kb = krow(pos);
+                float dot = 0.f;
+                for (int d = 0; d < D; d++) dot = fmaf(s_q[d], ld_elem(p.k, kb + d, p.f16), dot);
+                sc = dot * p.scale;
+            }
+            s_scores[i] = sc;
+            lmax = fmaxf(lmax, sc);
+        }
+        // block max
+        for (int off = 32; off > 0; off >>= 1) lmax = fmaxf(lmax, __shfl_xor(lmax, off, 64));
+        __syncthreads();
+        if ((tid & 63) == 0) s_red[tid >> 6] = lmax;
+        __syncthreads();
+        float cmax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+        float m_new = fmaxf(m_run, cmax);
+        float alpha = (m_run == -INFINITY) ? 0.f : exp2f((m_run - m_new) * kLog2e);
+        float lsum = 0.f;
+        for (int i = tid; i < cn; i += GEN_THREADS) {
+            float sc = s_scores[i];
+            float e = (sc == -INFINITY) ? 0.f : exp2f((sc - m_new) * kLog2e);
+            s_scores[i] = e;
+            lsum += e;
+        }
+        for (int off = 32; off > 0; off >>= 1) lsum += __shfl_xor(lsum, off, 64);
+        __syncthreads();
+        if ((tid & 63) == 0) s_red[tid >> 6] = lsum;
+        __syncthreads();
+        float csum = s_red[0] + s_red[1] + s_red[2] + s_red[3];
+        l_run = l_run * alpha + csum;
+        m_run = m_new;
+        acc *= alpha;
+        if (acc_active) {
+            for (int i = my_g; i < cn; i += ng) {
+                float w = s_scores[i];
+                if (w != 0.f) acc = fmaf(w, ld_elem(vbase, krow(c0 + i) + vadd + my_d, p.f16), acc);
+            }
+        }
+        __syncthreads();
+    }
+    s_acc[tid] = acc_active ? acc : 0.f;
+    __syncthreads();
+    if (tid < D) {
+        float t = 0.f;
+        for (int g = 0; g < ng; g++) t += s_acc[g * D + tid];
+        p.out[qoff + tid] = (l_run > 0.f) ? t / l_run : 0.f;
+    }
+}
+
+// --------------------------------------------------------------------------------------------
+// Hot path: ragged batched decode over an F16 paged pool.
+//
+// grid = (num_kv_heads, splits, batch); block = 256 threads (4 waves).
+// A workgroup owns the tokens [split*TPW, min(kv_len,(split+1)*TPW)) of one (sequence, kv head)
+// and all G = Hq/Hkv query heads that share that kv head. A wave takes 16-token pool blocks
+// round-robin. Within a wave LPT = D/8 lanes hold one token's head vector (8 halves = 16 bytes
+// each), so one load instruction covers 64/LPT tokens.
+// Partials (m, l, acc[D]) per (sequence, q head, split) go to a scratch buffer; paged_merge_kernel
+// combines the splits.
+constexpr int TPW = 512;  // tokens per workgroup
+
+template <int D, int G>
+__global__ void __launch_bounds__(256) paged_decode_f16_kernel(
+    const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *const *__restrict__ bt_ptrs,
+    const int32_t *__restrict__ bt_matrix, int max_blocks, const int32_t *__restrict__ kv_lens,
+    float *__restrict__ partial, int num_q_heads, int num_kv_heads, int block_size, float scale, int max_splits) {
+    constexpr int LPT = D / 8;     // lanes per token
+    constexpr int TPI = 64 / LPT;  // tokens per load instruction
+    const int kvh = blockIdx.x, split = blockIdx.y, seq = blockIdx.z;
+    const int kv_len = kv_lens[seq];
+    const int t_begin = split * TPW;
+    if (t_begin >= kv_len) return;
+    const int t_end = min(kv_len, t_begin + TPW);
+    const int32_t *bt = bt_ptrs ? bt_ptrs[seq] : bt_matrix + (size_t)seq * max_blocks;
+
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tl = lane / LPT;  // token slot within a load
+    const int dl = lane % LPT;  // 8-element slice of the head vector
+    const size_t hs = (size_t)num_kv_heads * D;
+    const size_t part = (size_t)block_size * hs;
+
+    // query slices, pre-multiplied by scale*log2(e) so scores are in the exp2 domain
+    float qf[G][8];
+    const float qs = scale * kLog2e;
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        const float *qp = q + ((size_t)seq * num_q_heads + (size_t)kvh * G + g) * D + dl * 8;
+#pragma unroll
+        for (int e = 0; e < 8; e++) qf[g][e] = qp[e] * qs;
+    }
+    float acc[G][8], m_run[G], l_run[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+        m_run[g] = -INFINITY;
+        l_run[g] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[g][e] = 0.f;
+    }
+
+    // Token groups of U*TPI tokens, interleaved over the 4 waves. All 2*U loads of a group are
+    // issued before any arithmetic so each wave keeps 2*U KiB in flight.
+    constexpr int U = 4;
+    typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+    const int n_groups = (t_end - t_begin + U * TPI - 1) / (U * TPI);
+    for (int gi = wave; gi < n_groups; gi += 4) {
+        half8 kk[U], vv[U];
+        bool valid[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int tok = t_begin + (gi * U + u) * TPI + tl;
+            valid[u] = tok < t_end;
+            const int tk = valid[u] ? tok : t_end - 1;
+            const int blk = bt[tk / block_size];
+            const size_t base = (size_t)blk * 2 * part + (size_t)(tk % block_size) * hs + (size_t)kvh * D + dl * 8;
+            kk[u] = *(const half8 *)(pool + base);
+            vv[u] = *(const half8 *)(pool + base + part);
+        }
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+            float s[U];
+            float gm = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                float t = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; e++) t = fmaf(qf[g][e], (float)kk[u][e], t);
+#pragma unroll
+                for (int off = LPT / 2; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
+                s[u] = valid[u] ? t : -INFINITY;
+                gm = fmaxf(gm, s[u]);
+            }
+            // max over the token slots of the wave (every group has at least one valid token)
+#pragma unroll
+            for (int off = LPT; off < 64; off <<= 1) gm = fmaxf(gm, __shfl_xor(gm, off, 64));
+            const float m_new = fmaxf(m_run[g], gm);
+            const float alpha = exp2f(m_run[g] - m_new);  // m_new is finite; exp2(-inf) = 0 on the first group
+            m_run[g] = m_new;
+            float lsum = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[g][e] *= alpha;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float pw = exp2f(s[u] - m_new);  // 0 for invalid tokens
+                lsum += pw;
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[g][e] = fmaf(pw, (float)vv[u][e], acc[g][e]);
+            }
+            l_run[g] = l_run[g] * alpha + lsum;
+        }
+    }
+
+    // combine token slots inside the wave (m is already wave-uniform per g)
+#pragma unroll
+    for (int g = 0; g < G; g++) {
+#pragma unroll
+        for (int off = LPT; off < 64; off <<= 1) {
+            l_run[g] += __shfl_xor(l_run[g], off, 64);
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[g][e] += __shfl_xor(acc[g][e], off, 64);
+        }
+    }
+
+    // combine the 4 waves through LDS
+    __shared__ float s_m[4][G], s_l[4][G];
+    __shared__ float s_acc[4][G][D];
+    if (tl == 0) {
+#pragma unroll
+        for (int g = 0; g < G; g++) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) s_acc[wave][g][dl * 8 + e] = acc[g][e];
+            if (dl == 0) {
+                s_m[wave][g] = m_run[g];
+                s_l[wave][g] = l_run[g];
+            }
+        }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < G * D; idx += 256) {
+        const int g = idx / D, d = idx % D;
+        float M = fmaxf(fmaxf(s_m[0][g], s_m[1][g]), fmaxf(s_m[2][g], s_m[3][g]));
+        float L = 0.f, A = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float f = (s_m[w][g] == -INFINITY) ? 0.f : exp2f(s_m[w][g] - M);
+            L += s_l[w][g] * f;
+            A += s_acc[w][g][d] * f;
+        }
+        const int qh = kvh * G + g;
+        float *po = partial + (((size_t)seq * num_q_heads + qh) * max_splits + split) * (D + 2);
+        po[2 + d] = A;
+        if (d == 0) {
+            po[0] = M;
+            po[1] = L;
+        }
+    }
+}
+
+// grid = (num_q_heads, batch); block = D threads.
+template <int D>
+__global__ void __launch_bounds__(D) paged_merge_kernel(const float *__restrict__ partial,
+                                                        const int32_t *__restrict__ kv_lens, float *__restrict__ out,
+                                                        int num_q_heads, int max_splits) {
+    const int qh = blockIdx.x, seq = blockIdx.y, d = threadIdx.x;
+    const int kv_len = kv_lens[seq];
+    const int ns = (kv_len + TPW - 1) / TPW;
+    const float *pb = partial + ((size_t)seq * num_q_heads + qh) * max_splits * (D + 2);
+    float M = -INFINITY;
+    for (int s = 0; s < ns; s++) M = fmaxf(M, pb[(size_t)s * (D + 2)]);
+    float L = 0.f, A = 0.f;
+    for (int s = 0; s < ns; s++) {
+        const float *ps = pb + (size_t)s * (D + 2);
+        const float f = exp2f(ps[0] - M);
+        L += ps[1] * f;
+        A += ps[2 + d] * f;
+    }
+    out[((size_t)seq * num_q_heads + qh) * D + d] = (L > 0.f) ? A / L : 0.f;
+}
+
+template <int D, int G>
+int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *const *bt_ptrs,
+               const int32_t *bt_matrix, int max_blocks, const int32_t *kv_lens, float *out, int batch,
+               int num_q_heads, int num_kv_heads, int block_size, float scale, int max_kv_len) {
+    int max_splits = ceil_div(max_kv_len, TPW);
+    size_t need = (size_t)batch * num_q_heads * max_splits * (D + 2) * sizeof(float);
+    int rc = ensure_ws(be, &be->attn_ws, &be->attn_ws_bytes, need, "attention");
+    if (rc) return rc;
+    dim3 grid(num_kv_heads, max_splits, batch);
+    paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_ptrs, bt_matrix,
+                                                                max_blocks, kv_lens, (float *)be->attn_ws,
+                                                                num_q_heads, num_kv_heads, block_size, scale,
+                                                                max_splits);
+    VX_CHECK_LAUNCH();
+    paged_merge_kernel<D><<<dim3(num_q_heads, batch), D, 0, be->stream>>>((const float *)be->attn_ws, kv_lens, out,
+                                                                          num_q_heads, max_splits);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int run_generic(vx_backend *be, const AttnParams &p, int num_queries) {
+    VX_REQUIRE(p.head_dim > 0 && p.head_dim <= 256, "attention: head_dim %d not in 1..256", p.head_dim);
+    VX_REQUIRE(p.num_kv_heads > 0 && p.num_q_heads % p.num_kv_heads == 0,
+               "attention: %d query heads not a multiple of %d kv heads", p.num_q_heads, p.num_kv_heads);
+    if (num_queries == 0) return VX_OK;
+    attn_generic_kernel<<<dim3(p.num_q_heads, num_queries), GEN_THREADS, 0, be->stream>>>(p);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+// Ragged batched decode: hot kernel when the shape has an instantiation, generic otherwise.
+int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16, const int32_t *const *bt_ptrs,
+               const int32_t *bt_matrix, int max_blocks, const int32_t *kv_lens, float *out, int batch, int block_size,
+               int num_q_heads, int num_kv_heads, int head_dim, float scale, int max_kv_len) {
+    VX_REQUIRE(num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, "attention: bad head counts");
+    VX_REQUIRE(block_size > 0 && max_kv_len > 0, "attention: bad block size / kv length");
+    if (batch == 0) return VX_OK;
+    const int G = num_q_heads / num_kv_heads;
+    const bool aligned = ((uintptr_t)pool % 16) == 0;
+#define VX_HOT(DD, GG)                                                                                            \
+    if (pool_is_f16 && aligned && head_dim == DD && G == GG)                                                      \
+        return launch_hot<DD, GG>(be, q, pool, bt_ptrs, bt_matrix, max_blocks, kv_lens, out, batch, num_q_heads,   \
+                                  num_kv_heads, block_size, scale, max_kv_len);
+    VX_HOT(128, 1) VX_HOT(128, 2) VX_HOT(128, 4) VX_HOT(128, 8)
+    VX_HOT(64, 1) VX_HOT(64, 2) VX_HOT(64, 4) VX_HOT(64, 8)
+#undef VX_HOT
+    AttnParams p = {};
+    p.q = q;
+    p.out = out;
+    p.k = pool;
+    p.mode = MODE_PAGED;
+    p.f16 = pool_is_f16;
+    p.num_q_heads = num_q_heads;
+    p.num_kv_heads = num_kv_heads;
+    p.head_dim = head_dim;
+    p.scale = scale;
+    p.bt_ptrs = bt_ptrs;
+    p.bt_matrix = bt_matrix;
+    p.max_blocks = max_blocks;
+    p.block_size = block_size;
+    p.kv_lens = kv_lens;
+    return run_generic(be, p, batch);
+}
+
+}  // namespace
+
+extern "C" {
+
+int vx_sdpa(vx_backend *be, const float *q, const float *k, const float *v, float *out, int kv_len, int num_q_heads,
+            int num_kv_heads, int head_dim, float scale, int kv_head_stride) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && k && v && out && kv_len >= 1, "vx_sdpa: bad arguments");
+    AttnParams p = {};
+    p.q = q;
+    p.out = out;
+    p.k = k;
+    p.v = v;
+    p.mode = MODE_CONTIG;
+    p.num_q_heads = num_q_heads;
+    p.num_kv_heads = num_kv_heads;
+    p.head_dim = head_dim;
+    p.scale = scale;
+    p.kv_head_stride = kv_head_stride;
+    p.kv_len = kv_len;
+    return run_generic(be, p, 1);
+}
+
+int vx_sdpa_prefill(vx_backend *be, const float *q, const float *k, const float *v, float *out, int seq_len,
+                    int num_q_heads, int num_kv_heads, int head_dim, float scale) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && k && v && out && seq_len >= 0, "vx_sdpa_prefill: bad arguments");
+    AttnParams p = {};
+    p.q = q;
+    p.out = out;
+    p.k = k;
+    p.v = v;
+    p.mode = MODE_PREFILL;
+    p.num_q_heads = num_q_heads;
+    p.num_kv_heads = num_kv_heads;
+    p.head_dim = head_dim;
+    p.scale = scale;
+    return run_generic(be, p, seq_len);
+}
+
+static int paged_single(vx_backend *be, const float *q, const void *kv_pool, int f16, const int32_t *block_table,
+                        float *out, int num_blocks, int block_size, int num_q_heads, int num_kv_heads, int head_dim,
+                        float scale, int tokens_in_last_block) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && kv_pool && block_table && out, "vx_sdpa_paged_decode: null pointer");
+    VX_REQUIRE(num_blocks >= 1 && block_size >= 1 && tokens_in_last_block >= 1 && tokens_in_last_block <= block_size,
+               "vx_sdpa_paged_decode: bad block counts");
+    AttnParams p = {};
+    p.q = q;
+    p.out = out;
+    p.k = kv_pool;
+    p.mode = MODE_PAGED;
+    p.f16 = f16;
+    p.num_q_heads = num_q_heads;
+    p.num_kv_heads = num_kv_heads;
+    p.head_dim = head_dim;
+    p.scale = scale;
+    p.block_table = block_table;
+    p.block_size = block_size;
+    p.kv_len = (num_blocks - 1) * block_size + tokens_in_last_block;
+    return run_generic(be, p, 1);
+}
+
+int vx_sdpa_paged_decode(vx_backend *be, const float *q, const void *kv_pool, const int32_t *block_table, float *out,
+                         int num_blocks, int block_size, int num_q_heads, int num_kv_heads, int head_dim, float scale,
+                         int tokens_in_last_block) {
+    return paged_single(be, q, kv_pool, 0, block_table, out, num_blocks, block_size, num_q_heads, num_kv_heads,
+                        head_dim, scale, tokens_in_last_block);
+}
+
+int vx_sdpa_paged_decode_f16(vx_backend *be, const float *q, const void *kv_pool, const int32_t *block_table,
+                             float *out, int num_blocks, int block_size, int num_q_heads, int num_kv_heads,
+                             int head_dim, float scale, int tokens_in_last_block) {
+    return paged_single(be, q, kv_pool, 1, block_table, out, num_blocks, block_size, num_q_heads, num_kv_heads,
+                        head_dim, scale, tokens_in_last_block);
+}
+
+int vx_sdpa_paged_decode_batched(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
+                                 const int32_t *const *block_tables, float *out, int batch_size, int max_blocks,
+                                 int block_size, int num_q_heads, int num_kv_heads, int head_dim, float scale,
+                                 const int32_t *seq_lens) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && kv_pool && block_tables && out && seq_lens, "vx_sdpa_paged_decode_batched: null pointer");
+    VX_REQUIRE(!be->capturing, "vx_sdpa_paged_decode_batched takes host arrays and cannot be captured");
+    if (batch_size == 0) return VX_OK;
+    size_t pbytes = (size_t)batch_size * sizeof(void *), lbytes = (size_t)batch_size * sizeof(int32_t);
+    VX_REQUIRE(pbytes + lbytes <= be->misc_ws_bytes, "vx_sdpa_paged_decode_batched: batch too large");
+    int max_len = 0;
+    for (int i = 0; i < batch_size; i++) {
+        VX_REQUIRE(seq_lens[i] >= 1, "vx_sdpa_paged_decode_batched: sequence %d has length %d", i, seq_lens[i]);
+        max_len = seq_lens[i] > max_len ? seq_lens[i] : max_len;
+    }
+    char *dev = (char *)be->misc_ws;
+    VX_CHECK_HIP(hipMemcpyAsync(dev, block_tables, pbytes, hipMemcpyHostToDevice, be->stream));
+    VX_CHECK_HIP(hipMemcpyAsync(dev + pbytes, seq_lens, lbytes, hipMemcpyHostToDevice, be->stream));
+    VX_CHECK_HIP(hipStreamSynchronize(be->stream));  // host arrays belong to the caller after return
+    return run_ragged(be, q, kv_pool, pool_is_f16, (const int32_t *const *)dev, nullptr, max_blocks,
+                      (const int32_t *)(dev + pbytes), out, batch_size, block_size, num_q_heads, num_kv_heads,
+                      head_dim, scale, max_len);
+}
+
+int vx_sdpa_paged_decode_ragged(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
+                                const int32_t *block_tables, const int32_t *kv_lens, float *out, int batch,
+                                int max_blocks, int block_size, int num_q_heads, int num_kv_heads, int head_dim,
+                                float scale, int max_kv_len) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && kv_pool && block_tables && kv_lens && out, "vx_sdpa_paged_decode_ragged: null pointer");
+    VX_REQUIRE(max_kv_len <= max_blocks * block_size, "vx_sdpa_paged_decode_ragged: max_kv_len %d exceeds table capacity %d",
+               max_kv_len, max_blocks * block_size);
+    return run_ragged(be, q, kv_pool, pool_is_f16, nullptr, block_tables, max_blocks, kv_lens, out, batch, block_size,
+                      num_q_heads, num_kv_heads, head_dim, scale, max_kv_len);
+}
+
+int vx_sdpa_paged_decode_multiquery(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
+                                    const int32_t *block_table, float *out, const int32_t *kv_lens, int num_blocks,
+                                    int block_size, int num_q_heads, int num_kv_heads, int head_dim, float scale,
+                                    int query_len) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && kv_pool && block_table && out && kv_lens, "vx_sdpa_paged_decode_multiquery: null pointer");
+    VX_REQUIRE(num_blocks >= 1 && block_size >= 1 && query_len >= 0, "vx_sdpa_paged_decode_multiquery: bad counts");
+    AttnParams p = {};
+    p.q = q;
+    p.out = out;
+    p.k = kv_pool;
+    p.mode = MODE_PAGED;
+    p.f16 = pool_is_f16;
+    p.num_q_heads = num_q_heads;
+    p.num_kv_heads = num_kv_heads;
+    p.head_dim = head_dim;
+    p.scale = scale;
+    p.block_table = block_table;
+    p.block_size = block_size;
+    p.kv_lens = kv_lens;
+    return run_generic(be, p, query_len);
+}
+
+int vx_sdpa_paged_tree(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
+                       const int32_t *block_table, float *out, const uint8_t *tree_mask, int tree_base, int block_size,
+                       int num_q_heads, int num_kv_heads, int head_dim, float scale, int query_len) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && kv_pool && block_table && out && tree_mask, "vx_sdpa_paged_tree: null pointer");
+    VX_REQUIRE(tree_base >= 0 && block_size >= 1 && query_len >= 0, "vx_sdpa_paged_tree: bad counts");
+    AttnParams p = {};
+    p.q = q;
+    p.out = out;
+    p.k = kv_pool;
+    p.mode = MODE_PAGED;
+    p.f16 = pool_is_f16;
+    p.num_q_heads = num_q_heads;
+    p.num_kv_heads = num_kv_heads;
+    p.head_dim = head_dim;
+    p.scale = scale;
+    p.block_table = block_table;
+    p.block_size = block_size;
+    p.tree_mask = tree_mask;
+    p.tree_base = tree_base;
+    p.query_len = query_len;
+    return run_generic(be, p, query_len);
+}
+
+}  // extern "C"

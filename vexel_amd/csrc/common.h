@@ -1,0 +1,85 @@
+// Internal declarations shared by the HIP translation units of libvexel_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "vexel_hip.h"
+
+namespace vx {
+
+void set_error(const char *fmt, ...);
+
+#define VX_CHECK_HIP(expr)                                                                  \
+    do {                                                                                    \
+        hipError_t _e = (expr);                                                             \
+        if (_e != hipSuccess) {                                                             \
+            vx::set_error("%s failed: %s (%s:%d)", #expr, hipGetErrorString(_e), __FILE__, __LINE__); \
+            return VX_ERR_HIP;                                                              \
+        }                                                                                   \
+    } while (0)
+
+#define VX_REQUIRE(cond, ...)            \
+    do {                                 \
+        if (!(cond)) {                   \
+            vx::set_error(__VA_ARGS__);  \
+            return VX_ERR_INVALID;       \
+        }                                \
+    } while (0)
+
+// Checks the launch that was just issued (invalid configuration etc.).
+#define VX_CHECK_LAUNCH() VX_CHECK_HIP(hipGetLastError())
+
+struct PoolChunk {
+    char *base;
+    size_t size;
+    size_t used;
+};
+
+}  // namespace vx
+
+struct vx_backend {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    bool capturing = false;
+
+    // per-step pool (vx_alloc / vx_reset_pool)
+    std::vector<vx::PoolChunk> chunks;
+    size_t cur_chunk = 0;
+    // permanent allocations (vx_alloc_permanent / vx_free)
+    std::unordered_map<void *, size_t> permanent;
+
+    // library-owned scratch, grown on demand outside graph capture
+    void *gemm_ws = nullptr;     // split activations for the quantized GEMM
+    size_t gemm_ws_bytes = 0;
+    void *attn_ws = nullptr;     // split-KV partial results
+    size_t attn_ws_bytes = 0;
+    void *misc_ws = nullptr;     // small device staging (pointer tables, argmax result)
+    size_t misc_ws_bytes = 0;
+    void *host_stage = nullptr;  // pinned host staging
+    size_t host_stage_bytes = 0;
+
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+};
+
+struct vx_graph {
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+};
+
+namespace vx {
+
+// Makes be->device current on the calling thread (Go moves goroutines across OS threads).
+int enter(vx_backend *be);
+// Ensures a library scratch buffer holds at least `bytes`; fails during capture if it must grow.
+int ensure_ws(vx_backend *be, void **ptr, size_t *cap, size_t bytes, const char *what);
+
+static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
+static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace vx

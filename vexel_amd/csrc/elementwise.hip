@@ -1,0 +1,602 @@
+// Elementwise, normalisation, embedding, argmax, dequantisation and dense F32 matmul
+// kernels. Each entry point cites the Go method it replaces (include/vexel_hip.h).
+//
+// Arithmetic notes: where the reference CPU backend goes through float64 (sqrt, exp,
+// pow, cos, sin: backend/cpu/cpu.go:214,256-260,397,508) these kernels do the same in
+// double on the device, so the only differences from the CPU result are float32
+// summation order in reductions. Dequantisation is bit-exact: its products are written
+// with explicit round-to-nearest intrinsics so no multiply-add is fused.
+#include <float.h>
+
+#include "common.h"
+
+using namespace vx;
+
+namespace {
+
+constexpr int kThreads = 256;
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+
+// Block-wide sum for blockDim.x == kThreads; every thread gets the result.
+__device__ __forceinline__ float block_sum(float v, float *sm) {
+    v = wave_sum(v);
+    int w = threadIdx.x >> 6, l = threadIdx.x & 63;
+    __syncthreads();
+    if (l == 0) sm[w] = v;
+    __syncthreads();
+    float t = 0.f;
+    for (int i = 0; i < (int)(blockDim.x >> 6); i++) t += sm[i];
+    return t;
+}
+
+__device__ __forceinline__ float block_max(float v, float *sm) {
+    v = wave_max(v);
+    int w = threadIdx.x >> 6, l = threadIdx.x & 63;
+    __syncthreads();
+    if (l == 0) sm[w] = v;
+    __syncthreads();
+    float t = sm[0];
+    for (int i = 1; i < (int)(blockDim.x >> 6); i++) t = fmaxf(t, sm[i]);
+    return t;
+}
+
+// ---------------------------------------------------------------- RMSNorm (cpu.go:200-220)
+__global__ void __launch_bounds__(kThreads) rmsnorm_kernel(const float *x, const float *w, float *out, int cols,
+                                                           float eps) {
+    __shared__ float sm[kThreads / 64];
+    const float *xr = x + (size_t)blockIdx.x * cols;
+    float *orow = out + (size_t)blockIdx.x * cols;
+    float ss = 0.f;
+    for (int j = threadIdx.x; j < cols; j += kThreads) {
+        float v = xr[j];
+        ss += v * v;
+    }
+    ss = block_sum(ss, sm);
+    float mean = ss / (float)cols;
+    float rms = (float)sqrt((double)(mean + eps));
+    for (int j = threadIdx.x; j < cols; j += kThreads) orow[j] = (xr[j] / rms) * w[j];
+}
+
+// ---------------------------------------------------------------- RoPE (cpu.go:226-303)
+struct RopeCS {
+    float c, s;
+};
+
+__device__ __forceinline__ RopeCS rope_cs(int pos, int j, int eff_dim, float theta) {
+    double ex = (double)(2 * j) / (double)eff_dim;
+    float freq = (float)(1.0 / pow((double)theta, ex));
+    float angle = __fmul_rn((float)pos, freq);
+    RopeCS r;
+    r.c = (float)cos((double)angle);
+    r.s = (float)sin((double)angle);
+    return r;
+}
+
+__device__ __forceinline__ void rope_pair(float &a, float &b, RopeCS cs) {
+    float v1 = a, v2 = b;
+    a = __fsub_rn(__fmul_rn(v1, cs.c), __fmul_rn(v2, cs.s));
+    b = __fadd_rn(__fmul_rn(v1, cs.s), __fmul_rn(v2, cs.c));
+}
+
+// grid.x = seq row, threads over rotation pairs j.
+__global__ void rope_kernel(float *q, float *k, int head_dim, int num_heads, int num_kv_heads, int start_pos,
+                            int eff_dim, float theta, int neox, const int32_t *positions) {
+    int row = blockIdx.x;
+    int half = eff_dim / 2;
+    int pos = positions ? positions[row] : start_pos + row;
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+        RopeCS cs = rope_cs(pos, j, eff_dim, theta);
+        int i0 = neox ? j : 2 * j;
+        int i1 = neox ? j + half : 2 * j + 1;
+        float *qr = q + (size_t)row * num_heads * head_dim;
+        for (int h = 0; h < num_heads; h++) rope_pair(qr[h * head_dim + i0], qr[h * head_dim + i1], cs);
+        if (k) {
+            float *kr = k + (size_t)row * num_kv_heads * head_dim;
+            for (int h = 0; h < num_kv_heads; h++) rope_pair(kr[h * head_dim + i0], kr[h * head_dim + i1], cs);
+        }
+    }
+}
+
+// RoPE (interleaved pairs, full head_dim) + paged scatter of K and V.
+template <bool F16>
+__global__ void rope_store_paged_kernel(float *q, const float *k, const float *v, const int32_t *positions,
+                                        const int32_t *slot_mapping, void *pool, int num_q_heads, int num_kv_heads,
+                                        int head_dim, int block_size, float theta) {
+    int row = blockIdx.x;
+    int half = head_dim / 2;
+    int pos = positions[row];
+    int slot = slot_mapping[row];
+    int blk = slot / block_size, off = slot % block_size;
+    size_t hs = (size_t)num_kv_heads * head_dim;
+    size_t part = (size_t)block_size * hs;
+    size_t kbase = (size_t)blk * 2 * part + (size_t)off * hs;
+    size_t vbase = kbase + part;
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+        RopeCS cs = rope_cs(pos, j, head_dim, theta);
+        float *qr = q + (size_t)row * num_q_heads * head_dim;
+        for (int h = 0; h < num_q_heads; h++) rope_pair(qr[h * head_dim + 2 * j], qr[h * head_dim + 2 * j + 1], cs);
+        const float *kr = k + (size_t)row * hs;
+        const float *vr = v + (size_t)row * hs;
+        for (int h = 0; h < num_kv_heads; h++) {
+            float a = kr[h * head_dim + 2 * j], b = kr[h * head_dim + 2 * j + 1];
+            rope_pair(a, b, cs);
+            float va = vr[h * head_dim + 2 * j], vb = vr[h * head_dim + 2 * j + 1];
+            size_t o = (size_t)h * head_dim + 2 * j;
+            if (F16) {
+                _Float16 *p = (_Float16 *)pool;
+                p[kbase + o] = (_Float16)a;
+                p[kbase + o + 1] = (_Float16)b;
+                p[vbase + o] = (_Float16)va;
+                p[vbase + o + 1] = (_Float16)vb;
+            } else {
+                float *p = (float *)pool;
+                p[kbase + o] = a;
+                p[kbase + o + 1] = b;
+                p[vbase + o] = va;
+                p[vbase + o + 1] = vb;
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------- SiLU / SiLUMul / Add / Mul
+__device__ __forceinline__ float sigmoid_ref(float v) {  // cpu.go:384,397
+    return 1.0f / (1.0f + (float)exp((double)(-v)));
+}
+
+__global__ void silu_kernel(const float *x, float *out, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = __fmul_rn(x[i], sigmoid_ref(x[i]));
+}
+
+__global__ void silu_mul_kernel(const float *g, const float *u, float *out, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = __fmul_rn(__fmul_rn(g[i], sigmoid_ref(g[i])), u[i]);
+}
+
+__global__ void add_kernel(const float *a, const float *b, float *out, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = a[i] + b[i];
+}
+
+__global__ void mul_kernel(const float *a, const float *b, float *out, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = a[i] * b[i];
+}
+
+// ---------------------------------------------------------------- Softmax (cpu.go:490-518)
+__global__ void __launch_bounds__(kThreads) softmax_kernel(const float *x, float *out, int cols) {
+    __shared__ float sm[kThreads / 64];
+    const float *xr = x + (size_t)blockIdx.x * cols;
+    float *orow = out + (size_t)blockIdx.x * cols;
+    float mx = -INFINITY;
+    for (int j = threadIdx.x; j < cols; j += kThreads) mx = fmaxf(mx, xr[j]);
+    mx = block_max(mx, sm);
+    float s = 0.f;
+    for (int j = threadIdx.x; j < cols; j += kThreads) {
+        float e = (float)exp((double)(xr[j] - mx));
+        orow[j] = e;
+        s += e;
+    }
+    s = block_sum(s, sm);
+    float inv = 1.0f / s;
+    for (int j = threadIdx.x; j < cols; j += kThreads) orow[j] *= inv;
+}
+
+// ---------------------------------------------------------------- Embedding (cpu.go:543-555)
+__global__ void embedding_kernel(const int32_t *ids, const float *table, float *out, int vocab, int dim) {
+    int t = blockIdx.x;
+    int id = ids[t];
+    if (id < 0 || id >= vocab) return;  // row left untouched
+    const float *src = table + (size_t)id * dim;
+    float *dst = out + (size_t)t * dim;
+    for (int j = threadIdx.x; j < dim; j += blockDim.x) dst[j] = src[j];
+}
+
+// ---------------------------------------------------------------- Argmax (sampler.go:80-91)
+// One block per row. Strict '>' from -FLT_MAX; ties resolve to the lowest index; NaN never wins.
+__global__ void __launch_bounds__(1024) argmax_rows_kernel(const float *x, int n, int32_t *out) {
+    __shared__ float sv[16];
+    __shared__ int si[16];
+    const float *xr = x + (size_t)blockIdx.x * n;
+    float bv = -FLT_MAX;
+    int bi = 0;
+    for (int j = threadIdx.x; j < n; j += blockDim.x) {
+        float v = xr[j];
+        if (v > bv) {
+            bv = v;
+            bi = j;
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        float ov = __shfl_xor(bv, off, 64);
+        int oi = __shfl_xor(bi, off, 64);
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    int w = threadIdx.x >> 6, l = threadIdx.x & 63;
+    if (l == 0) {
+        sv[w] = bv;
+        si[w] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int i = 1; i < (int)(blockDim.x >> 6); i++)
+            if (sv[i] > bv || (sv[i] == bv && si[i] < bi)) {
+                bv = sv[i];
+                bi = si[i];
+            }
+        // an index found through a tie on -FLT_MAX is not a strict improvement: the reference returns 0
+        out[blockIdx.x] = (bv > -FLT_MAX) ? bi : 0;
+    }
+}
+
+// ---------------------------------------------------------------- Dequantise (dequant.go), bit-exact
+__device__ __forceinline__ float f16_bits_to_f32(uint16_t h) {
+    // IEEE half -> float is exact; matches dequant.go:231-261 for every non-NaN pattern.
+    _Float16 v;
+    __builtin_memcpy(&v, &h, 2);
+    return (float)v;
+}
+
+__device__ __forceinline__ uint16_t ld_u16(const uint8_t *p) { return (uint16_t)(p[0] | ((uint16_t)p[1] << 8)); }
+
+// one thread per block of 32 (Q4_0 / Q8_0)
+__global__ void dequant_q4_0_kernel(const uint8_t *src, float *dst, int64_t nblk) {
+    int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblk) return;
+    const uint8_t *p = src + b * 18;
+    float d = f16_bits_to_f32(ld_u16(p));
+    float *o = dst + b * 32;
+    for (int i = 0; i < 16; i++) {
+        uint8_t bv = p[2 + i];
+        o[i] = __fmul_rn(d, (float)((int)(bv & 0xF) - 8));
+        o[i + 16] = __fmul_rn(d, (float)((int)(bv >> 4) - 8));
+    }
+}
+
+__global__ void dequant_q8_0_kernel(const uint8_t *src, float *dst, int64_t nblk) {
+    int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblk) return;
+    const uint8_t *p = src + b * 34;
+    float d = f16_bits_to_f32(ld_u16(p));
+    float *o = dst + b * 32;
+    for (int i = 0; i < 32; i++) o[i] = __fmul_rn(d, (float)(int8_t)p[2 + i]);
+}
+
+__device__ __forceinline__ void scale_min_k4(int j, const uint8_t *q, uint8_t &sc, uint8_t &mn) {  // dequant.go:400-409
+    if (j < 4) {
+        sc = q[j] & 63;
+        mn = q[j + 4] & 63;
+    } else {
+        sc = (uint8_t)((q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4));
+        mn = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+// one 64-thread group per super-block of 256; thread t handles elements t, t+64, ...
+__global__ void dequant_q4_k_kernel(const uint8_t *src, float *dst, int64_t nblk) {
+    int64_t b = (int64_t)blockIdx.x * (blockDim.x / 64) + (threadIdx.x >> 6);
+    if (b >= nblk) return;
+    int t = threadIdx.x & 63;
+    const uint8_t *p = src + b * 144;
+    float d = f16_bits_to_f32(ld_u16(p)), dmin = f16_bits_to_f32(ld_u16(p + 2));
+    const uint8_t *scales = p + 4, *qs = p + 16;
+    float *o = dst + b * 256;
+    for (int e = t; e < 256; e += 64) {
+        int grp = e >> 6, l = e & 31, hi = (e >> 5) & 1;
+        uint8_t sc, mn;
+        scale_min_k4(grp * 2 + hi, scales, sc, mn);
+        float d1 = __fmul_rn(d, (float)sc), dm1 = __fmul_rn(dmin, (float)mn);
+        uint8_t bv = qs[grp * 32 + l];
+        int q = hi ? (bv >> 4) : (bv & 0xF);
+        o[e] = __fsub_rn(__fmul_rn(d1, (float)q), dm1);
+    }
+}
+
+__global__ void dequant_q6_k_kernel(const uint8_t *src, float *dst, int64_t nblk) {
+    int64_t b = (int64_t)blockIdx.x * (blockDim.x / 64) + (threadIdx.x >> 6);
+    if (b >= nblk) return;
+    int t = threadIdx.x & 63;
+    const uint8_t *p = src + b * 210;
+    const uint8_t *ql = p, *qh = p + 128, *sc = p + 192;
+    float d = f16_bits_to_f32(ld_u16(p + 208));
+    float *o = dst + b * 256;
+    int nn = t >> 5, l = t & 31, is = l >> 4;  // dequant.go:294-326
+    const uint8_t *qlp = ql + nn * 64, *qhp = qh + nn * 32;
+    const int8_t *scp = (const int8_t *)sc + nn * 8;
+    int q1 = (int)((qlp[l] & 0xF) | (((qhp[l] >> 0) & 3) << 4)) - 32;
+    int q2 = (int)((qlp[l + 32] & 0xF) | (((qhp[l] >> 2) & 3) << 4)) - 32;
+    int q3 = (int)((qlp[l] >> 4) | (((qhp[l] >> 4) & 3) << 4)) - 32;
+    int q4 = (int)((qlp[l + 32] >> 4) | (((qhp[l] >> 6) & 3) << 4)) - 32;
+    float *y = o + nn * 128;
+    y[l] = __fmul_rn(__fmul_rn(d, (float)scp[is + 0]), (float)q1);
+    y[l + 32] = __fmul_rn(__fmul_rn(d, (float)scp[is + 2]), (float)q2);
+    y[l + 64] = __fmul_rn(__fmul_rn(d, (float)scp[is + 4]), (float)q3);
+    y[l + 96] = __fmul_rn(__fmul_rn(d, (float)scp[is + 6]), (float)q4);
+}
+
+// ---------------------------------------------------------------- dense F32 matmul (cpu.go:106-197)
+// C[M,N] = A[M,K] * op(B); 32x32 output tile per block, k ascending inside each output.
+template <bool BT>
+__global__ void __launch_bounds__(256) matmul_f32_kernel(const float *a, const float *b, float *c, int m, int n,
+                                                         int k) {
+    __shared__ float as[32][33];
+    __shared__ float bs[32][33];
+    int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+    int row0 = blockIdx.y * 32, col0 = blockIdx.x * 32;
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int k0 = 0; k0 < k; k0 += 32) {
+        for (int r = ty; r < 32; r += 8) {
+            int gr = row0 + r, gk = k0 + tx;
+            as[r][tx] = (gr < m && gk < k) ? a[(size_t)gr * k + gk] : 0.f;
+            if (BT) {  // B is [N,K]
+                int gn = col0 + r;
+                bs[tx][r] = (gn < n && gk < k) ? b[(size_t)gn * k + gk] : 0.f;
+            } else {  // B is [K,N]
+                int gkk = k0 + r, gn = col0 + tx;
+                bs[r][tx] = (gkk < k && gn < n) ? b[(size_t)gkk * n + gn] : 0.f;
+            }
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int kk = 0; kk < 32; kk++) {
+            float bv = bs[kk][tx];
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[i] = fmaf(as[ty + 8 * i][kk], bv, acc[i]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        int gr = row0 + ty + 8 * i, gn = col0 + tx;
+        if (gr < m && gn < n) c[(size_t)gr * n + gn] = acc[i];
+    }
+}
+
+// ---------------------------------------------------------------- paged scatter (metal_bridge_darwin.m:8539-8642)
+template <bool F16>
+__global__ void reshape_paged_kv_kernel(const float *src, void *dst, const int32_t *blk_idx, const int32_t *blk_off,
+                                        int num_tokens, int num_kv_heads, int head_dim, int block_size, int is_value) {
+    size_t hs = (size_t)num_kv_heads * head_dim;
+    size_t total = (size_t)num_tokens * hs;
+    size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= total) return;
+    int t = (int)(gid / hs);
+    size_t r = gid % hs;
+    size_t part = (size_t)block_size * hs;
+    size_t di = (size_t)blk_idx[t] * 2 * part + (is_value ? part : 0) + (size_t)blk_off[t] * hs + r;
+    if (F16)
+        ((_Float16 *)dst)[di] = (_Float16)src[gid];  // round to nearest even, like Metal's (half)x
+    else
+        ((float *)dst)[di] = src[gid];
+}
+
+inline int grid1d(int64_t n, int threads) { return (int)((n + threads - 1) / threads); }
+
+}  // namespace
+
+extern "C" {
+
+int vx_rmsnorm(vx_backend *be, const float *x, const float *weight, float *out, int rows, int cols, float eps) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(x && weight && out && rows >= 0 && cols > 0, "vx_rmsnorm: bad arguments");
+    if (rows == 0) return VX_OK;
+    rmsnorm_kernel<<<rows, kThreads, 0, be->stream>>>(x, weight, out, cols, eps);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_rope(vx_backend *be, float *q, float *k, int head_dim, int num_heads, int num_kv_heads, int seq_len,
+            int start_pos, int rope_dim, float theta, int rope_neox) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && head_dim > 0 && num_heads > 0 && seq_len >= 0, "vx_rope: bad arguments");
+    int eff = rope_dim == 0 ? head_dim : rope_dim;
+    VX_REQUIRE(eff <= head_dim && eff % 2 == 0, "vx_rope: rope_dim %d invalid for head_dim %d", rope_dim, head_dim);
+    if (seq_len == 0) return VX_OK;
+    int threads = eff / 2 < 64 ? 64 : (eff / 2 > 256 ? 256 : eff / 2);
+    rope_kernel<<<seq_len, threads, 0, be->stream>>>(q, k, head_dim, num_heads, num_kv_heads, start_pos, eff, theta,
+                                                      rope_neox, nullptr);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_rope_store_paged(vx_backend *be, float *q, const float *k, const float *v, const int32_t *positions,
+                        const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int rows, int num_q_heads,
+                        int num_kv_heads, int head_dim, int block_size, float theta) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && k && v && positions && slot_mapping && kv_pool, "vx_rope_store_paged: null pointer");
+    VX_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && block_size > 0 && num_q_heads > 0 && num_kv_heads > 0,
+               "vx_rope_store_paged: bad shape");
+    if (rows == 0) return VX_OK;
+    int threads = head_dim / 2 < 64 ? 64 : head_dim / 2;
+    if (pool_is_f16)
+        rope_store_paged_kernel<true><<<rows, threads, 0, be->stream>>>(q, k, v, positions, slot_mapping, kv_pool,
+                                                                        num_q_heads, num_kv_heads, head_dim,
+                                                                        block_size, theta);
+    else
+        rope_store_paged_kernel<false><<<rows, threads, 0, be->stream>>>(q, k, v, positions, slot_mapping, kv_pool,
+                                                                         num_q_heads, num_kv_heads, head_dim,
+                                                                         block_size, theta);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+#define VX_EW(name, kernel, ...)                                                \
+    int rc = enter(be);                                                         \
+    if (rc) return rc;                                                          \
+    VX_REQUIRE(n >= 0, name ": negative n");                                    \
+    if (n == 0) return VX_OK;                                                   \
+    kernel<<<grid1d(n, kThreads), kThreads, 0, be->stream>>>(__VA_ARGS__, n);   \
+    VX_CHECK_LAUNCH();                                                          \
+    return VX_OK;
+
+int vx_silu(vx_backend *be, const float *x, float *out, int n) {
+    VX_REQUIRE(x && out, "vx_silu: null pointer");
+    VX_EW("vx_silu", silu_kernel, x, out)
+}
+
+int vx_silu_mul(vx_backend *be, const float *gate, const float *up, float *out, int n) {
+    VX_REQUIRE(gate && up && out, "vx_silu_mul: null pointer");
+    VX_EW("vx_silu_mul", silu_mul_kernel, gate, up, out)
+}
+
+int vx_add(vx_backend *be, const float *a, const float *b, float *out, int n) {
+    VX_REQUIRE(a && b && out, "vx_add: null pointer");
+    VX_EW("vx_add", add_kernel, a, b, out)
+}
+
+int vx_mul(vx_backend *be, const float *a, const float *b, float *out, int n) {
+    VX_REQUIRE(a && b && out, "vx_mul: null pointer");
+    VX_EW("vx_mul", mul_kernel, a, b, out)
+}
+
+int vx_softmax(vx_backend *be, const float *x, float *out, int rows, int cols) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(x && out && rows >= 0 && cols > 0, "vx_softmax: bad arguments");
+    if (rows == 0) return VX_OK;
+    softmax_kernel<<<rows, kThreads, 0, be->stream>>>(x, out, cols);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_embedding(vx_backend *be, const int32_t *ids, int num_tokens, const float *table, float *out, int vocab_size,
+                 int dim) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(ids && table && out && num_tokens >= 0 && dim > 0, "vx_embedding: bad arguments");
+    if (num_tokens == 0) return VX_OK;
+    embedding_kernel<<<num_tokens, kThreads, 0, be->stream>>>(ids, table, out, vocab_size, dim);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_argmax_rows(vx_backend *be, const float *logits, int rows, int n, int32_t *out_idx) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(logits && out_idx && rows >= 0 && n > 0, "vx_argmax_rows: bad arguments");
+    if (rows == 0) return VX_OK;
+    argmax_rows_kernel<<<rows, 1024, 0, be->stream>>>(logits, n, out_idx);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_argmax(vx_backend *be, const float *input, int n, int *out_index) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(input && out_index && n > 0, "vx_argmax: bad arguments");
+    VX_REQUIRE(!be->capturing, "vx_argmax during graph capture");
+    int32_t *dev = (int32_t *)be->misc_ws;
+    argmax_rows_kernel<<<1, 1024, 0, be->stream>>>(input, n, dev);
+    VX_CHECK_LAUNCH();
+    VX_CHECK_HIP(hipMemcpyAsync(be->host_stage, dev, 4, hipMemcpyDeviceToHost, be->stream));
+    VX_CHECK_HIP(hipStreamSynchronize(be->stream));
+    *out_index = *(int32_t *)be->host_stage;
+    return VX_OK;
+}
+
+int vx_dequantize(vx_backend *be, int fmt, const void *src, float *dst, int64_t n) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(src && dst && n >= 0, "vx_dequantize: bad arguments");
+    if (n == 0) return VX_OK;
+    const uint8_t *s = (const uint8_t *)src;
+    switch (fmt) {
+    case VX_Q4_0:
+        VX_REQUIRE(n % 32 == 0, "vx_dequantize: n must be a multiple of 32");
+        dequant_q4_0_kernel<<<grid1d(n / 32, kThreads), kThreads, 0, be->stream>>>(s, dst, n / 32);
+        break;
+    case VX_Q8_0:
+        VX_REQUIRE(n % 32 == 0, "vx_dequantize: n must be a multiple of 32");
+        dequant_q8_0_kernel<<<grid1d(n / 32, kThreads), kThreads, 0, be->stream>>>(s, dst, n / 32);
+        break;
+    case VX_Q4_K:
+        VX_REQUIRE(n % 256 == 0, "vx_dequantize: n must be a multiple of 256");
+        dequant_q4_k_kernel<<<grid1d(n / 256, 4), 256, 0, be->stream>>>(s, dst, n / 256);
+        break;
+    case VX_Q6_K:
+        VX_REQUIRE(n % 256 == 0, "vx_dequantize: n must be a multiple of 256");
+        dequant_q6_k_kernel<<<grid1d(n / 256, 4), 256, 0, be->stream>>>(s, dst, n / 256);
+        break;
+    default:
+        set_error("vx_dequantize: unknown format %d", fmt);
+        return VX_ERR_UNSUPPORTED;
+    }
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_matmul(vx_backend *be, const float *a, const float *b, float *out, int m, int n, int k) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(a && b && out && m >= 0 && n >= 0 && k >= 0, "vx_matmul: bad arguments");
+    if (m == 0 || n == 0) return VX_OK;
+    dim3 grid(ceil_div(n, 32), ceil_div(m, 32));
+    matmul_f32_kernel<false><<<grid, 256, 0, be->stream>>>(a, b, out, m, n, k);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_matmul_transposed(vx_backend *be, const float *a, const float *b, float *out, int m, int n, int k) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(a && b && out && m >= 0 && n >= 0 && k >= 0, "vx_matmul_transposed: bad arguments");
+    if (m == 0 || n == 0) return VX_OK;
+    dim3 grid(ceil_div(n, 32), ceil_div(m, 32));
+    matmul_f32_kernel<true><<<grid, 256, 0, be->stream>>>(a, b, out, m, n, k);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+static int reshape_paged(vx_backend *be, const float *src, void *dst_base, const int32_t *page_table,
+                         const int32_t *block_offsets, int num_tokens, int num_kv_heads, int head_dim,
+                         int block_size, int is_value, bool f16) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(src && dst_base && page_table && block_offsets, "vx_reshape_paged_kv: null pointer");
+    VX_REQUIRE(num_tokens >= 0 && num_kv_heads > 0 && head_dim > 0 && block_size > 0, "vx_reshape_paged_kv: bad shape");
+    if (num_tokens == 0) return VX_OK;
+    int64_t total = (int64_t)num_tokens * num_kv_heads * head_dim;
+    if (f16)
+        reshape_paged_kv_kernel<true><<<grid1d(total, kThreads), kThreads, 0, be->stream>>>(
+            src, dst_base, page_table, block_offsets, num_tokens, num_kv_heads, head_dim, block_size, is_value);
+    else
+        reshape_paged_kv_kernel<false><<<grid1d(total, kThreads), kThreads, 0, be->stream>>>(
+            src, dst_base, page_table, block_offsets, num_tokens, num_kv_heads, head_dim, block_size, is_value);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_reshape_paged_kv(vx_backend *be, const float *src, void *dst_base, const int32_t *page_table,
+                        const int32_t *block_offsets, int num_tokens, int num_kv_heads, int head_dim, int block_size,
+                        int is_value) {
+    return reshape_paged(be, src, dst_base, page_table, block_offsets, num_tokens, num_kv_heads, head_dim, block_size,
+                         is_value, false);
+}
+
+int vx_reshape_paged_kv_f16(vx_backend *be, const float *src, void *dst_base, const int32_t *page_table,
+                            const int32_t *block_offsets, int num_tokens, int num_kv_heads, int head_dim,
+                            int block_size, int is_value) {
+    return reshape_paged(be, src, dst_base, page_table, block_offsets, num_tokens, num_kv_heads, head_dim, block_size,
+                         is_value, true);
+}
+
+}  // extern "C"

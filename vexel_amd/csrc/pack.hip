@@ -1,0 +1,127 @@
+// Continuous-batching step metadata built on the device (vx_pack_batch).
+//
+// Host restatement of what this replaces: the per-sequence loop of
+// inference/runtime/decode.go:642-650 calling GPUBlockPool.StoreKV for every sequence
+// (inference/runtime/gpu_block_pool.go:234-252: ensure blocks up to (endPos-1)/blockSize by
+// popping the free list's tail, slot = (table[pos/bs], pos%bs)) and the length bookkeeping
+// of gpu_block_pool.go:318-320,354-363. Because the host loop visits sequences in batch
+// order and every layer's free list evolves identically, sequence i's new blocks are the
+// entries free[F-1-rank_i-j], rank_i = exclusive prefix sum of the blocks needed by the
+// sequences before it. Two prefix scans (blocks needed, new tokens) give every output.
+#include "common.h"
+
+using namespace vx;
+
+namespace {
+
+constexpr int PK_THREADS = 1024;
+
+// Exclusive scan over blockDim.x values held one per thread; returns the exclusive prefix and
+// writes the total to *total (same value in every thread).
+__device__ int block_exclusive_scan(int v, int *sm, int *total) {
+    const int tid = threadIdx.x;
+    sm[tid] = v;
+    __syncthreads();
+    for (int off = 1; off < PK_THREADS; off <<= 1) {
+        int t = (tid >= off) ? sm[tid - off] : 0;
+        __syncthreads();
+        sm[tid] += t;
+        __syncthreads();
+    }
+    int incl = sm[tid];
+    *total = sm[PK_THREADS - 1];
+    __syncthreads();
+    return incl - v;
+}
+
+__global__ void __launch_bounds__(PK_THREADS) pack_batch_kernel(
+    const int32_t *seq_slots, const int32_t *positions, const int32_t *q_lens, int batch, int total_tokens,
+    int32_t *block_tables, int max_blocks, int32_t *num_blocks, int32_t *free_list, int32_t *free_count,
+    int block_size, int32_t *cu_seqlens, int32_t *token_pos, int32_t *slot_mapping, int32_t *kv_lens,
+    int32_t *status) {
+    __shared__ int sm[PK_THREADS];
+    __shared__ int s_cu[PK_THREADS + 1];
+    const int tid = threadIdx.x;
+    const bool act = tid < batch;
+    int slot = 0, pos = 0, ql = 0, have = 0, need = 0;
+    if (act) {
+        slot = seq_slots[tid];
+        pos = positions[tid];
+        ql = q_lens ? q_lens[tid] : 1;
+        have = num_blocks[slot];
+        int end = pos + ql;
+        int want = end > 0 ? (end - 1) / block_size + 1 : 0;
+        need = want > have ? want - have : 0;
+    }
+    int total_need, total_q;
+    const int rank = block_exclusive_scan(need, sm, &total_need);
+    const int cu = block_exclusive_scan(ql, sm, &total_q);
+    const int F = *free_count;
+    bool fail = total_need > F || total_q != total_tokens;
+    if (act && have + need > max_blocks) fail = true;
+    // any thread's failure fails the step
+    sm[tid] = fail ? 1 : 0;
+    __syncthreads();
+    for (int off = PK_THREADS / 2; off > 0; off >>= 1) {
+        if (tid < off) sm[tid] |= sm[tid + off];
+        __syncthreads();
+    }
+    const bool any_fail = sm[0] != 0;
+    __syncthreads();
+    if (any_fail) {
+        if (tid == 0) *status = 1;
+        return;
+    }
+    if (act) {
+        for (int j = 0; j < need; j++)
+            block_tables[(size_t)slot * max_blocks + have + j] = free_list[F - 1 - (rank + j)];
+        num_blocks[slot] = have + need;
+        kv_lens[tid] = pos + ql;
+        s_cu[tid] = cu;
+        cu_seqlens[tid] = cu;
+    }
+    if (tid == 0) {
+        *free_count = F - total_need;
+        *status = 0;
+        s_cu[batch] = total_q;
+        cu_seqlens[batch] = total_q;
+    }
+    __syncthreads();
+    for (int t = tid; t < total_q; t += PK_THREADS) {
+        // binary search: largest i with s_cu[i] <= t
+        int lo = 0, hi = batch - 1;
+        while (lo < hi) {
+            int mid = (lo + hi + 1) >> 1;
+            if (s_cu[mid] <= t)
+                lo = mid;
+            else
+                hi = mid - 1;
+        }
+        const int p = positions[lo] + (t - s_cu[lo]);
+        token_pos[t] = p;
+        const int sl = seq_slots[lo];
+        slot_mapping[t] = block_tables[(size_t)sl * max_blocks + p / block_size] * block_size + p % block_size;
+    }
+}
+
+}  // namespace
+
+extern "C" int vx_pack_batch(vx_backend *be, const int32_t *seq_slots, const int32_t *positions,
+                             const int32_t *q_lens, int batch, int total_tokens, int32_t *block_tables,
+                             int max_blocks, int32_t *num_blocks, int32_t *free_list, int32_t *free_count,
+                             int block_size, int32_t *cu_seqlens, int32_t *token_pos, int32_t *slot_mapping,
+                             int32_t *kv_lens, int32_t *status) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(seq_slots && positions && block_tables && num_blocks && free_list && free_count && cu_seqlens &&
+                   token_pos && slot_mapping && kv_lens && status,
+               "vx_pack_batch: null pointer");
+    VX_REQUIRE(batch >= 1 && batch <= PK_THREADS, "vx_pack_batch: batch %d not in 1..%d", batch, PK_THREADS);
+    VX_REQUIRE(block_size >= 1 && max_blocks >= 1 && total_tokens >= 0, "vx_pack_batch: bad sizes");
+    pack_batch_kernel<<<1, PK_THREADS, 0, be->stream>>>(seq_slots, positions, q_lens, batch, total_tokens,
+                                                        block_tables, max_blocks, num_blocks, free_list, free_count,
+                                                        block_size, cu_seqlens, token_pos, slot_mapping, kv_lens,
+                                                        status);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
