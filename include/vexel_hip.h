@@ -151,12 +151,13 @@ int vx_rope_store_paged(vx_backend *be, float *q, const float *k, const float *v
                         int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta);
 
 /* Ragged batched paged attention with all metadata on the device: block_tables is a
- * padded int32 [batch, max_blocks] matrix, kv_lens int32[batch]. One query per sequence.
- * max_kv_len bounds the launch (>= every kv_lens[i]). */
+ * padded int32 [rows, max_blocks] matrix; sequence i uses row table_rows[i] (row i when
+ * table_rows is NULL); kv_lens int32[batch]. One query per sequence. max_kv_len bounds
+ * the launch (>= every kv_lens[i]). */
 int vx_sdpa_paged_decode_ragged(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
-                                const int32_t *block_tables, const int32_t *kv_lens, float *out, int batch,
-                                int max_blocks, int block_size, int num_q_heads, int num_kv_heads, int head_dim,
-                                float scale, int max_kv_len);
+                                const int32_t *block_tables, const int32_t *table_rows, const int32_t *kv_lens,
+                                float *out, int batch, int max_blocks, int block_size, int num_q_heads,
+                                int num_kv_heads, int head_dim, float scale, int max_kv_len);
 
 /* Tree verification (medusa/tree.go:186-202 mask rule): query i attends to every pool
  * position < tree_base and to position tree_base+j iff tree_mask[i*query_len+j] != 0
@@ -182,6 +183,12 @@ int vx_pack_batch(vx_backend *be, const int32_t *seq_slots, const int32_t *posit
                   int batch, int total_tokens, int32_t *block_tables, int max_blocks, int32_t *num_blocks,
                   int32_t *free_list, int32_t *free_count, int block_size, int32_t *cu_seqlens,
                   int32_t *token_pos, int32_t *slot_mapping, int32_t *kv_lens, int32_t *status);
+
+/* End of a device-driven decode step (host restatement: scheduler/scheduler.go:432-446 greedy arm +
+ * scheduler/sequence.go:136-141): out_log[step*batch + i] = next_tokens[i] where step = *step_counter,
+ * then tokens[i] = next_tokens[i], positions[i] += 1, *step_counter += 1. All device int32. */
+int vx_decode_advance(vx_backend *be, int32_t *tokens, int32_t *positions, const int32_t *next_tokens,
+                      int32_t *out_log, int32_t *step_counter, int batch);
 
 /* Stream capture of a decode step into a hipGraph (replaces the Metal command-buffer
  * batching of runtime/decode.go:426-431). Between begin and end every vx_* compute call

@@ -1,0 +1,91 @@
+/*
+ * vexel_host.h -- C API of libvexel_host.so: the host-side drivers of the batched-decode
+ * path (block pool bookkeeping, layer executor, decode / prefill drivers), written in C++
+ * above the C ABI of vexel_hip.h. In a Go build these are the Go packages themselves
+ * (inference/runtime); this library exists so the same logic can be built, tested and
+ * benchmarked where no Go toolchain is present. Each function names the Go method it mirrors.
+ */
+#ifndef VEXEL_HOST_H
+#define VEXEL_HOST_H
+
+#include <stdint.h>
+
+#include "vexel_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum { VH_OK = 0, VH_ERR = 1 };
+
+/* runtime.ModelConfig (inference/runtime/config.go) fields the path needs + pool sizing */
+typedef struct vh_config {
+    int num_layers, hidden, num_heads, num_kv_heads, head_dim, ffn, vocab;
+    float eps, rope_theta;
+    int block_size;          /* 16 in the reference (runtime/model.go:321) */
+    int pool_blocks;         /* physical blocks per layer (GPUBlockPool.maxBlocks) */
+    int max_seqs;            /* rows of the device block-table matrix */
+    int max_blocks_per_seq;  /* columns of the device block-table matrix */
+    int max_batch;           /* rows of the activation buffers */
+    int kv_fp16;             /* 1 = F16 pool (runtime/model.go:311), 0 = F32 */
+} vh_config;
+
+typedef struct vh_qweight {  /* tensor.Tensor with a QuantProfile: raw GGUF blocks on the device */
+    int fmt;                 /* VX_Q4_0 ... */
+    const void *data;
+    int n, k;
+} vh_qweight;
+
+typedef struct vh_layer_weights {  /* the BlockRuntime fields used by ExecuteWithPagedKV */
+    const float *attn_norm, *ffn_norm;
+    vh_qweight wq, wk, wv, wo, w1, w2, w3;
+} vh_layer_weights;
+
+typedef struct vh_model vh_model;
+
+const char *vh_last_error(void);
+
+/* NewModelRuntime + CreateGPUBlockPool (runtime/model.go:305-327): allocates the per-layer
+ * KV pool, the device mirror of the block tables and the activation buffers. */
+int vh_model_create(vx_backend *be, const vh_config *cfg, vh_model **out);
+void vh_model_destroy(vh_model *m);
+int vh_model_set_layer(vh_model *m, int layer, const vh_layer_weights *w);
+/* embedding: F32 [vocab,hidden] on the device (loader rule, runtime/loader.go:275-288) */
+int vh_model_set_head(vh_model *m, const float *embedding, const float *final_norm, const vh_qweight *lm_head);
+void *vh_kv_pool(vh_model *m, int layer);  /* device base of a layer's block pool */
+
+/* GPUBlockPool (runtime/gpu_block_pool.go) */
+int vh_pool_create_sequence(vh_model *m, int64_t seq_id);                       /* :126 */
+int vh_pool_delete_sequence(vh_model *m, int64_t seq_id);                       /* :138 */
+int vh_pool_truncate_sequence(vh_model *m, int64_t seq_id, int new_len);        /* :162 */
+int vh_pool_has_sequence(vh_model *m, int64_t seq_id);                          /* :193 */
+int vh_pool_share_blocks(vh_model *m, int64_t src, int64_t dst, int num_tokens);/* :572 */
+void vh_pool_block_stats(vh_model *m, int *total, int *free_blocks, int *shared);/* :610 (per layer x numLayers) */
+int vh_pool_seq_len(vh_model *m, int64_t seq_id);
+/* copies the sequence's block table (identical for every layer) into out; returns its length or -1 */
+int vh_pool_block_table(vh_model *m, int64_t seq_id, int32_t *out, int cap);
+/* installs a given block table / length for a sequence whose KV was written directly into the
+ * pool (synthetic pre-filled contexts of the benchmark configs); the blocks leave the free list */
+int vh_pool_adopt_blocks(vh_model *m, int64_t seq_id, const int32_t *blocks, int num_blocks, int seq_len);
+/* reads the device mirror back and compares it with the host state: 1 equal, 0 different, <0 error */
+int vh_pool_device_matches_host(vh_model *m);
+
+/* ModelRuntime.DecodeWithPagedKVBatched (runtime/decode.go:612-654): one token per sequence.
+ * logits_out: host [batch,vocab] or NULL; argmax_out: host [batch] or NULL. */
+int vh_decode_batched(vh_model *m, const int32_t *tokens, const int64_t *seq_ids, const int32_t *positions,
+                      int batch, float *logits_out, int32_t *argmax_out);
+/* ModelRuntime.PrefillWithPagedKV (runtime/decode.go:961-1096) when all_logits == 0: logits of the
+ * last token -> logits_out[vocab]. VerifySpeculativeWithPagedKV (decode.go:1446-1569) when
+ * all_logits != 0: logits of every position -> logits_out[n,vocab]. */
+int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int start_pos, int all_logits,
+               float *logits_out);
+/* Greedy decode of `steps` tokens for a fixed batch with the step captured in a hipGraph and all
+ * per-step metadata built on the device. out_tokens: host [steps,batch]. The host pool state is
+ * advanced by the same rule afterwards. use_graph = 0 runs the same device-driven step eagerly. */
+int vh_decode_graph(vh_model *m, const int32_t *first_tokens, const int64_t *seq_ids, const int32_t *positions,
+                    int batch, int steps, int use_graph, int32_t *out_tokens, float *ms_per_step);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

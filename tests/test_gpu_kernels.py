@@ -411,13 +411,14 @@ def test_pack_batch_bit_exact(be):
         free = np.zeros(pool_blocks, dtype=np.int32)
         fl = ref.free_lists[0]
         free[:len(fl)] = fl
+        free_count0 = len(fl)
         batch_slots = rng.permutation(nslots)[:rng.integers(1, nslots + 1)].astype(np.int32)
         qlens = (rng.integers(1, 40, batch_slots.size) if trial % 2 else np.ones(batch_slots.size)).astype(np.int32)
         pos = np.array([ctx[s] for s in batch_slots], dtype=np.int32)
         T = int(qlens.sum())
         want = hl.pack_batch(ref, 0, [int(s) for s in batch_slots], [int(p) for p in pos], [int(x) for x in qlens])
         d = {k: be.upload(v) for k, v in dict(slots=batch_slots, pos=pos, ql=qlens, tables=tables, nblk=nblk,
-                                              free=free, fc=np.array([len(fl)], dtype=np.int32)).items()}
+                                              free=free, fc=np.array([free_count0], dtype=np.int32)).items()}
         B = batch_slots.size
         cu, tp, sm, kl, st = (be.alloc((B + 1) * 4), be.alloc(T * 4), be.alloc(T * 4), be.alloc(B * 4), be.alloc(4))
         be.pack_batch(d["slots"], d["pos"], d["ql"] if trial % 2 else 0, B, T, d["tables"], max_blocks, d["nblk"],

@@ -1,0 +1,218 @@
+"""End-to-end parity of the decode drivers against the CPU oracle on identical seeded
+random-init weights and inputs (the BASELINE configs at sizes the oracle finishes in seconds:
+real head geometry and hidden sizes, fewer layers).
+
+Bars (BASELINE north star): logits within 1e-2 absolute / 1e-3 relative in float32; greedy
+tokens identical; block tables / slot state bit-exact."""
+import numpy as np
+import pytest
+
+from oracle import model as om
+from oracle import numerics as nx
+
+from helpers import gpu_model_from_oracle, install_context, assert_logits_close
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def be():
+    from vexel_amd.backend import HipBackend
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+def _greedy_margin(logits):
+    s = np.sort(logits)
+    return float(s[-1] - s[-2])
+
+
+def test_c1_prefill_then_greedy_decode(be):
+    """BASELINE config 1 shape (TinyLlama head geometry, Q4_0, Q8_0 embeddings and head), batch 1:
+    32-token prompt, greedy decode of 64 tokens. 2 layers so the CPU side stays in seconds."""
+    cfg = om.ModelConfig(num_layers=2, hidden=2048, num_heads=32, num_kv_heads=4, head_dim=64, ffn=5632,
+                         vocab=32000, eps=1e-5, rope_theta=10000.0)
+    omodel = om.random_model(cfg, 0, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=16)
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=16, max_batch=8)
+    rng = np.random.default_rng(0)
+    prompt = rng.integers(0, cfg.vocab, 32).tolist()
+    want = omodel.prefill_with_paged_kv(prompt, 1, 0)
+    got = mr.prefill_with_paged_kv(prompt, 1, 0)
+    worst = assert_logits_close(got, want, "prefill logits")
+    tok_o, tok_g = nx.argmax(want), int(np.argmax(got))
+    assert tok_o == tok_g
+    pos = len(prompt)
+    min_margin = 1e9
+    for step in range(64):
+        want = omodel.decode_with_paged_kv(tok_o, 1, pos)
+        got, am = mr.decode_with_paged_kv_batched([tok_g], [1], [pos])
+        worst = max(worst, assert_logits_close(got[0], want, "decode step %d" % step))
+        min_margin = min(min_margin, _greedy_margin(want))
+        tok_o = nx.argmax(want)
+        tok_g = int(am[0])
+        assert tok_o == tok_g, "greedy token differs at step %d (margin %.3e)" % (step, _greedy_margin(want))
+        pos += 1
+    assert mr.block_table(1) == omodel.pool.seqs[1].block_tables[0]
+    assert mr.seq_len(1) == omodel.pool.seqs[1].seq_len == 96
+    print("C1: worst logit error %.3e, smallest top-1 margin %.3e" % (worst, min_margin))
+    mr.close()
+
+
+def _ragged_setup(be, cfg, fmt, head_fmt, ctx_lens, seed, pool_blocks, fmt_overrides=None):
+    omodel = om.random_model(cfg, seed, fmt, head_fmt, max_blocks=pool_blocks, fmt_overrides=fmt_overrides)
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=pool_blocks, max_seqs=len(ctx_lens) + 2,
+                               max_blocks_per_seq=max(ctx_lens) // cfg.block_size + 8, max_batch=len(ctx_lens))
+    rng = np.random.default_rng(seed + 1)
+    perm = rng.permutation(pool_blocks)       # block tables are a seeded random permutation
+    off = 0
+    for i, L in enumerate(ctx_lens):
+        nb = (L + cfg.block_size - 1) // cfg.block_size
+        install_context(omodel, mr, be, 100 + i, perm[off:off + nb], L, rng)
+        off += nb
+    return omodel, mr, rng
+
+
+def test_c2_batched_decode_ragged_paged(be):
+    """BASELINE config 2 shape: 8 sequences, ragged contexts, KV pre-filled with N(0,1), permuted block
+    tables; batched decode steps against the oracle's sequential per-sequence loop."""
+    cfg = om.ModelConfig(num_layers=2, hidden=2048, num_heads=32, num_kv_heads=4, head_dim=64, ffn=5632,
+                         vocab=32000)
+    rng0 = np.random.default_rng(5)
+    ctx = [int(x) for x in rng0.integers(128, 700, 8)]
+    ctx[3] = 16 * 9            # exactly on a block boundary: the step must take a new block
+    omodel, mr, rng = _ragged_setup(be, cfg, nx.FMT_Q4_0, nx.FMT_Q8_0, ctx, 7, pool_blocks=400)
+    ids = [100 + i for i in range(8)]
+    toks = rng.integers(0, cfg.vocab, 8).tolist()
+    pos = list(ctx)
+    toks_g = list(toks)
+    for step in range(4):
+        want = omodel.decode_batched(toks, ids, pos)
+        got, am = mr.decode_with_paged_kv_batched(toks_g, ids, pos)
+        assert_logits_close(got, want, "C2 step %d" % step)
+        toks = [nx.argmax(want[i]) for i in range(8)]
+        toks_g = [int(a) for a in am]
+        assert toks == toks_g
+        pos = [p + 1 for p in pos]
+    for i, sid in enumerate(ids):
+        assert mr.block_table(sid) == omodel.pool.seqs[sid].block_tables[0]
+        assert mr.block_table(sid) == omodel.pool.seqs[sid].block_tables[cfg.num_layers - 1]
+    assert mr.block_stats()[1] == omodel.pool.block_stats()[1]
+    mr.close()
+
+
+def test_device_driven_graph_decode_matches_host_driven(be):
+    """The hipGraph-captured, device-packed greedy loop gives the same tokens as the host-driven
+    step and as the oracle, and leaves the device block tables equal to the host's."""
+    cfg = om.ModelConfig(num_layers=2, hidden=1024, num_heads=8, num_kv_heads=8, head_dim=128, ffn=2816,
+                         vocab=4096)
+    ctx = [30, 47, 16, 200, 333, 64]
+    steps = 20   # several sequences cross block boundaries
+    omodel, mr, rng = _ragged_setup(be, cfg, nx.FMT_Q4_0, nx.FMT_Q4_0, ctx, 11, pool_blocks=120)
+    ids = [100 + i for i in range(len(ctx))]
+    first = rng.integers(0, cfg.vocab, len(ctx)).tolist()
+    # oracle greedy loop
+    toks, pos, want_tokens = list(first), list(ctx), []
+    for s in range(steps):
+        lg = omodel.decode_batched(toks, ids, pos)
+        toks = [nx.argmax(lg[i]) for i in range(len(ctx))]
+        want_tokens.append(list(toks))
+        pos = [p + 1 for p in pos]
+    out, ms = mr.decode_graph(first, ids, ctx, steps, use_graph=True)
+    assert out.tolist() == want_tokens
+    assert mr.device_matches_host()
+    for sid in ids:
+        assert mr.block_table(sid) == omodel.pool.seqs[sid].block_tables[0]
+        assert mr.seq_len(sid) == omodel.pool.seqs[sid].seq_len
+    # continue on the device without re-uploading anything: replays of the cached graph
+    more, _ = mr.decode_graph(None, None, None, 5, use_graph=True, batch=len(ctx))
+    for s in range(5):
+        lg = omodel.decode_batched(toks, ids, pos)
+        toks = [nx.argmax(lg[i]) for i in range(len(ctx))]
+        assert more[s].tolist() == toks
+        pos = [p + 1 for p in pos]
+    assert mr.device_matches_host()
+    # eager device-driven steps (no graph) agree too
+    eager, _ = mr.decode_graph(None, None, None, 3, use_graph=False, batch=len(ctx))
+    for s in range(3):
+        lg = omodel.decode_batched(toks, ids, pos)
+        toks = [nx.argmax(lg[i]) for i in range(len(ctx))]
+        assert eager[s].tolist() == toks
+        pos = [p + 1 for p in pos]
+    mr.close()
+
+
+@pytest.mark.parametrize("name,fmt,head,over", [
+    ("q4_k_m mix", nx.FMT_Q4_K, nx.FMT_Q6_K, {"wv": nx.FMT_Q6_K, "w2": nx.FMT_Q6_K}),   # config 3
+    ("q8_0", nx.FMT_Q8_0, nx.FMT_Q8_0, None),                                            # config 4
+    ("q6_k", nx.FMT_Q6_K, nx.FMT_Q6_K, None),                                            # config 5
+])
+def test_other_formats_batched_decode(be, name, fmt, head, over):
+    """7B/8B head geometry (head_dim 128), one layer, 32 ragged sequences: the M=32 path."""
+    kvh = 8 if fmt == nx.FMT_Q8_0 else 32
+    cfg = om.ModelConfig(num_layers=1, hidden=4096, num_heads=32, num_kv_heads=kvh, head_dim=128, ffn=2048,
+                         vocab=2048, rope_theta=500000.0 if fmt == nx.FMT_Q8_0 else 10000.0)
+    rng0 = np.random.default_rng(21)
+    ctx = [int(x) for x in np.clip(np.exp(rng0.normal(np.log(200), 0.6, 32)), 64, 600)]
+    omodel, mr, rng = _ragged_setup(be, cfg, fmt, head, ctx, 23, pool_blocks=900, fmt_overrides=over)
+    ids = [100 + i for i in range(32)]
+    toks = rng.integers(0, cfg.vocab, 32).tolist()
+    want = omodel.decode_batched(toks, ids, ctx)
+    got, am = mr.decode_with_paged_kv_batched(toks, ids, ctx)
+    assert_logits_close(got, want, name)
+    assert [nx.argmax(want[i]) for i in range(32)] == [int(a) for a in am]
+    mr.close()
+
+
+def test_chunked_prefill_and_verify(be):
+    """Second chunk (startPos > 0) goes through multi-query paged attention over the f16 pool
+    (runtime/block.go:881-890); verify returns logits for every position."""
+    cfg = om.ModelConfig(num_layers=2, hidden=1024, num_heads=8, num_kv_heads=2, head_dim=128, ffn=2048,
+                         vocab=4096)
+    omodel = om.random_model(cfg, 31, nx.FMT_Q8_0, nx.FMT_Q8_0, max_blocks=32)
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=32, max_batch=4)
+    rng = np.random.default_rng(32)
+    toks = rng.integers(0, cfg.vocab, 70).tolist()
+    w1 = omodel.prefill_with_paged_kv(toks[:40], 5, 0)
+    g1 = mr.prefill_with_paged_kv(toks[:40], 5, 0)
+    assert_logits_close(g1, w1, "chunk 0")
+    w2 = omodel.prefill_with_paged_kv(toks[40:], 5, 40)
+    g2 = mr.prefill_with_paged_kv(toks[40:], 5, 40)
+    assert_logits_close(g2, w2, "chunk 1")
+    draft = rng.integers(0, cfg.vocab, 5).tolist()
+    wv = omodel.verify_with_paged_kv(draft, 5, 70)
+    gv = mr.prefill_with_paged_kv(draft, 5, 70, all_logits=True)
+    assert_logits_close(gv, wv, "verify")
+    # rollback after 2 accepted drafts (medusa_scheduler.go:852-861)
+    new_len = 70 + 1 + 2
+    omodel.pool.truncate_sequence(5, new_len)
+    mr.truncate_sequence(5, new_len)
+    assert mr.seq_len(5) == omodel.pool.seqs[5].seq_len == new_len
+    assert mr.block_table(5) == omodel.pool.seqs[5].block_tables[0]
+    assert mr.block_stats()[1] == omodel.pool.block_stats()[1]
+    mr.close()
+
+
+def test_pool_errors_and_lifecycle(be):
+    """Host-forced failure paths: pool exhaustion, unknown sequence, truncate no-ops."""
+    from vexel_amd.backend import VexelError
+    cfg = om.ModelConfig(num_layers=1, hidden=256, num_heads=2, num_kv_heads=2, head_dim=128, ffn=256, vocab=256)
+    omodel = om.random_model(cfg, 41, nx.FMT_Q4_0, nx.FMT_Q4_0, max_blocks=2)
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=2, max_seqs=4, max_blocks_per_seq=4, max_batch=4)
+    mr.prefill_with_paged_kv(list(range(32)), 1, 0)            # uses both blocks
+    with pytest.raises(VexelError) as e:
+        mr.decode_with_paged_kv_batched([1], [1], [32])       # needs a third block
+    assert "no free blocks" in str(e.value)
+    mr.truncate_sequence(999, 5)                               # unknown: no-op
+    mr.truncate_sequence(1, 100)                               # beyond length: no-op
+    assert mr.seq_len(1) == 32
+    mr.truncate_sequence(1, 16)
+    assert mr.block_stats() == (2, 1, 0)
+    mr.create_sequence(2)
+    mr.share_blocks(1, 2, 16)
+    assert mr.block_stats() == (2, 1, 1)
+    mr.delete_sequence(1)
+    assert mr.block_stats() == (2, 1, 0) and mr.has_sequence(2) and not mr.has_sequence(1)
+    with pytest.raises(VexelError):
+        mr.share_blocks(7, 2, 16)
+    mr.close()

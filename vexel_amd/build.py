@@ -8,6 +8,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libvexel_hip.so")
+HOST_LIB = os.path.join(HERE, "libvexel_host.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
 SOURCES = ["backend.hip", "elementwise.hip", "attention.hip", "qgemm.hip", "pack.hip"]
@@ -42,6 +43,17 @@ def build(verbose=True):
         raise RuntimeError("link failed:\n" + r.stderr)
     if verbose:
         print("built", LIB)
+    # host runtime: plain C++ above the C ABI (links the HIP library, finds it next to itself)
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I" + os.path.join(ROOT, "include"),
+           os.path.join(HERE, "host", "runtime.cpp"), "-o", HOST_LIB, "-L" + HERE, "-lvexel_hip",
+           "-Wl,-rpath,$ORIGIN", "-pthread"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("host runtime build failed:\n" + r.stderr)
+    if r.stderr.strip():
+        sys.stderr.write(r.stderr)
+    if verbose:
+        print("built", HOST_LIB)
     return LIB
 
 

@@ -41,7 +41,8 @@ struct AttnParams {
     // paged
     const int32_t *block_table;          // one table (single sequence / multiquery / tree)
     const int32_t *const *bt_ptrs;       // per-query tables (batched), or nullptr
-    const int32_t *bt_matrix;            // padded [batch,max_blocks] matrix, or nullptr
+    const int32_t *bt_matrix;            // padded [rows,max_blocks] matrix, or nullptr
+    const int32_t *bt_rows;              // row of each query in bt_matrix, or nullptr (row = query)
     int max_blocks;
     int block_size;
     const int32_t *kv_lens;              // per-query kv length (device), or nullptr
@@ -82,7 +83,7 @@ __global__ void __launch_bounds__(GEN_THREADS) attn_generic_kernel(AttnParams p)
         if (p.bt_ptrs)
             bt = p.bt_ptrs[qi];
         else if (p.bt_matrix)
-            bt = p.bt_matrix + (size_t)qi * p.max_blocks;
+            bt = p.bt_matrix + (size_t)(p.bt_rows ? p.bt_rows[qi] : qi) * p.max_blocks;
         else
             bt = p.block_table;
     }
@@ -179,7 +180,8 @@ constexpr int TPW = 512;  // tokens per workgroup
 template <int D, int G>
 __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *const *__restrict__ bt_ptrs,
-    const int32_t *__restrict__ bt_matrix, int max_blocks, const int32_t *__restrict__ kv_lens,
+    const int32_t *__restrict__ bt_matrix, const int32_t *__restrict__ bt_rows, int max_blocks,
+    const int32_t *__restrict__ kv_lens,
     float *__restrict__ partial, int num_q_heads, int num_kv_heads, int block_size, float scale, int max_splits) {
     constexpr int LPT = D / 8;     // lanes per token
     constexpr int TPI = 64 / LPT;  // tokens per load instruction
@@ -188,7 +190,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     const int t_begin = split * TPW;
     if (t_begin >= kv_len) return;
     const int t_end = min(kv_len, t_begin + TPW);
-    const int32_t *bt = bt_ptrs ? bt_ptrs[seq] : bt_matrix + (size_t)seq * max_blocks;
+    const int32_t *bt = bt_ptrs ? bt_ptrs[seq] : bt_matrix + (size_t)(bt_rows ? bt_rows[seq] : seq) * max_blocks;
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int tl = lane / LPT;  // token slot within a load
@@ -335,15 +337,15 @@ __global__ void __launch_bounds__(D) paged_merge_kernel(const float *__restrict_
 
 template <int D, int G>
 int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *const *bt_ptrs,
-               const int32_t *bt_matrix, int max_blocks, const int32_t *kv_lens, float *out, int batch,
-               int num_q_heads, int num_kv_heads, int block_size, float scale, int max_kv_len) {
+               const int32_t *bt_matrix, const int32_t *bt_rows, int max_blocks, const int32_t *kv_lens, float *out,
+               int batch, int num_q_heads, int num_kv_heads, int block_size, float scale, int max_kv_len) {
     int max_splits = ceil_div(max_kv_len, TPW);
     size_t need = (size_t)batch * num_q_heads * max_splits * (D + 2) * sizeof(float);
     int rc = ensure_ws(be, &be->attn_ws, &be->attn_ws_bytes, need, "attention");
     if (rc) return rc;
     dim3 grid(num_kv_heads, max_splits, batch);
     paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_ptrs, bt_matrix,
-                                                                max_blocks, kv_lens, (float *)be->attn_ws,
+                                                                bt_rows, max_blocks, kv_lens, (float *)be->attn_ws,
                                                                 num_q_heads, num_kv_heads, block_size, scale,
                                                                 max_splits);
     VX_CHECK_LAUNCH();
@@ -365,7 +367,8 @@ int run_generic(vx_backend *be, const AttnParams &p, int num_queries) {
 
 // Ragged batched decode: hot kernel when the shape has an instantiation, generic otherwise.
 int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16, const int32_t *const *bt_ptrs,
-               const int32_t *bt_matrix, int max_blocks, const int32_t *kv_lens, float *out, int batch, int block_size,
+               const int32_t *bt_matrix, const int32_t *bt_rows, int max_blocks, const int32_t *kv_lens, float *out,
+               int batch, int block_size,
                int num_q_heads, int num_kv_heads, int head_dim, float scale, int max_kv_len) {
     VX_REQUIRE(num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, "attention: bad head counts");
     VX_REQUIRE(block_size > 0 && max_kv_len > 0, "attention: bad block size / kv length");
@@ -374,7 +377,8 @@ int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16
     const bool aligned = ((uintptr_t)pool % 16) == 0;
 #define VX_HOT(DD, GG)                                                                                            \
     if (pool_is_f16 && aligned && head_dim == DD && G == GG)                                                      \
-        return launch_hot<DD, GG>(be, q, pool, bt_ptrs, bt_matrix, max_blocks, kv_lens, out, batch, num_q_heads,   \
+        return launch_hot<DD, GG>(be, q, pool, bt_ptrs, bt_matrix, bt_rows, max_blocks, kv_lens, out, batch,       \
+                                  num_q_heads,                                                                      \
                                   num_kv_heads, block_size, scale, max_kv_len);
     VX_HOT(128, 1) VX_HOT(128, 2) VX_HOT(128, 4) VX_HOT(128, 8)
     VX_HOT(64, 1) VX_HOT(64, 2) VX_HOT(64, 4) VX_HOT(64, 8)
@@ -391,6 +395,7 @@ int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16
     p.scale = scale;
     p.bt_ptrs = bt_ptrs;
     p.bt_matrix = bt_matrix;
+    p.bt_rows = bt_rows;
     p.max_blocks = max_blocks;
     p.block_size = block_size;
     p.kv_lens = kv_lens;
@@ -497,21 +502,22 @@ int vx_sdpa_paged_decode_batched(vx_backend *be, const float *q, const void *kv_
     VX_CHECK_HIP(hipMemcpyAsync(dev, block_tables, pbytes, hipMemcpyHostToDevice, be->stream));
     VX_CHECK_HIP(hipMemcpyAsync(dev + pbytes, seq_lens, lbytes, hipMemcpyHostToDevice, be->stream));
     VX_CHECK_HIP(hipStreamSynchronize(be->stream));  // host arrays belong to the caller after return
-    return run_ragged(be, q, kv_pool, pool_is_f16, (const int32_t *const *)dev, nullptr, max_blocks,
+    return run_ragged(be, q, kv_pool, pool_is_f16, (const int32_t *const *)dev, nullptr, nullptr, max_blocks,
                       (const int32_t *)(dev + pbytes), out, batch_size, block_size, num_q_heads, num_kv_heads,
                       head_dim, scale, max_len);
 }
 
 int vx_sdpa_paged_decode_ragged(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
-                                const int32_t *block_tables, const int32_t *kv_lens, float *out, int batch,
-                                int max_blocks, int block_size, int num_q_heads, int num_kv_heads, int head_dim,
-                                float scale, int max_kv_len) {
+                                const int32_t *block_tables, const int32_t *table_rows, const int32_t *kv_lens,
+                                float *out, int batch, int max_blocks, int block_size, int num_q_heads,
+                                int num_kv_heads, int head_dim, float scale, int max_kv_len) {
     int rc = enter(be);
     if (rc) return rc;
     VX_REQUIRE(q && kv_pool && block_tables && kv_lens && out, "vx_sdpa_paged_decode_ragged: null pointer");
     VX_REQUIRE(max_kv_len <= max_blocks * block_size, "vx_sdpa_paged_decode_ragged: max_kv_len %d exceeds table capacity %d",
                max_kv_len, max_blocks * block_size);
-    return run_ragged(be, q, kv_pool, pool_is_f16, nullptr, block_tables, max_blocks, kv_lens, out, batch, block_size,
+    return run_ragged(be, q, kv_pool, pool_is_f16, nullptr, block_tables, table_rows, max_blocks, kv_lens, out, batch,
+                      block_size,
                       num_q_heads, num_kv_heads, head_dim, scale, max_kv_len);
 }
 

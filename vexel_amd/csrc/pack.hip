@@ -125,3 +125,31 @@ extern "C" int vx_pack_batch(vx_backend *be, const int32_t *seq_slots, const int
     VX_CHECK_LAUNCH();
     return VX_OK;
 }
+
+namespace {
+__global__ void decode_advance_kernel(int32_t *tokens, int32_t *positions, const int32_t *next_tokens,
+                                      int32_t *out_log, int32_t *step_counter, int batch) {
+    const int i = threadIdx.x;
+    const int step = *step_counter;
+    __syncthreads();
+    if (i < batch) {
+        const int t = next_tokens[i];
+        out_log[(size_t)step * batch + i] = t;
+        tokens[i] = t;
+        positions[i] += 1;
+    }
+    if (i == 0) *step_counter = step + 1;
+}
+}  // namespace
+
+extern "C" int vx_decode_advance(vx_backend *be, int32_t *tokens, int32_t *positions, const int32_t *next_tokens,
+                                 int32_t *out_log, int32_t *step_counter, int batch) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(tokens && positions && next_tokens && out_log && step_counter, "vx_decode_advance: null pointer");
+    VX_REQUIRE(batch >= 1 && batch <= PK_THREADS, "vx_decode_advance: batch %d not in 1..%d", batch, PK_THREADS);
+    decode_advance_kernel<<<1, PK_THREADS, 0, be->stream>>>(tokens, positions, next_tokens, out_log, step_counter,
+                                                            batch);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}

@@ -1,0 +1,690 @@
+// Host runtime above the C ABI of include/vexel_hip.h: the part of vexel's Go runtime
+// that drives the batched-decode path, restated in C++ because no Go toolchain exists in
+// the build image. It calls the device only through the vx_* entry points, exactly as
+// the Go packages would through the cgo shim.
+//
+//   BlockPool      inference/runtime/gpu_block_pool.go (free list, ref counts, block tables,
+//                  truncate, share, stats). Every layer's bookkeeping is identical there, so
+//                  one table per sequence serves all layers here, with a device-resident
+//                  mirror (block-table matrix, free stack) that vx_pack_batch advances in
+//                  lock step with the host rule.
+//   execute_layer  inference/runtime/block.go:763-1081 (LLaMA arm) for a whole batch of
+//                  single-token sequences (block.go:1087-1119 loops over them instead).
+//   vh_decode_batched  inference/runtime/decode.go:612-654 (+339-461).
+//   vh_prefill     inference/runtime/decode.go:961-1096 / 1446-1569 for one sequence.
+//   vh_decode_graph  the decode step captured once in a hipGraph and replayed with all
+//                  per-step metadata built on the device; greedy sampling as
+//                  inference/pkg/sampler/sampler.go:80-91.
+#include <math.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <algorithm>
+#include <map>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "vexel_host.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return VH_ERR;
+}
+
+#define VXC(expr)                                                         \
+    do {                                                                  \
+        int _rc = (expr);                                                 \
+        if (_rc != VX_OK) return fail("%s: %s", #expr, vx_last_error());  \
+    } while (0)
+#define VHC(expr)                      \
+    do {                               \
+        if ((expr) != VH_OK) return VH_ERR; \
+    } while (0)
+
+struct SeqState {
+    std::vector<int32_t> table;  // logical block -> physical block (same for every layer)
+    int seq_len = 0;
+    int slot = -1;               // row in the device block-table matrix
+    bool dirty = true;           // device row differs from `table`
+};
+
+struct BlockPool {
+    int block_size = 16, max_blocks = 0;
+    std::vector<int32_t> free_list;               // gpu_block_pool.go:110-116
+    std::unordered_map<int32_t, int> ref_counts;  // gpu_block_pool.go:42-43
+    std::map<int64_t, SeqState> seqs;
+    std::mutex mu;                                // gpu_block_pool.go:46
+    std::vector<int> free_slots;
+    bool free_dirty = true;
+
+    int alloc_block(int32_t *out) {               // gpu_block_pool.go:200-209
+        if (free_list.empty()) return fail("no free blocks (max=%d)", max_blocks);
+        *out = free_list.back();
+        free_list.pop_back();
+        ref_counts[*out] = 1;
+        free_dirty = true;
+        return VH_OK;
+    }
+    void release_block(int32_t b) {               // gpu_block_pool.go:211-219
+        auto it = ref_counts.find(b);
+        int rc = it == ref_counts.end() ? 0 : it->second;
+        if (rc <= 1) {
+            if (it != ref_counts.end()) ref_counts.erase(it);
+            free_list.push_back(b);
+            free_dirty = true;
+        } else {
+            it->second = rc - 1;
+        }
+    }
+    int ensure_blocks(SeqState &s, int end_pos) {  // gpu_block_pool.go:234-245
+        if (end_pos <= 0) return VH_OK;
+        int last = (end_pos - 1) / block_size;
+        while ((int)s.table.size() <= last) {
+            int32_t b;
+            VHC(alloc_block(&b));
+            s.table.push_back(b);
+            s.dirty = true;
+        }
+        return VH_OK;
+    }
+};
+
+}  // namespace
+
+struct vh_model {
+    vx_backend *be = nullptr;
+    vh_config cfg{};
+    std::vector<vh_layer_weights> layers;
+    const float *embedding = nullptr;
+    const float *final_norm = nullptr;
+    vh_qweight lm_head{};
+    BlockPool pool;
+    std::vector<void *> kv;
+
+    int32_t *d_tables = nullptr, *d_num_blocks = nullptr, *d_free = nullptr, *d_free_count = nullptr;
+    int32_t *d_slots = nullptr, *d_positions = nullptr, *d_tokens = nullptr, *d_next = nullptr;
+    int32_t *d_cu = nullptr, *d_token_pos = nullptr, *d_slot_map = nullptr, *d_kv_lens = nullptr;
+    int32_t *d_status = nullptr, *d_step = nullptr, *d_log = nullptr;
+    int log_cap = 0;  // steps the log can hold
+
+    float *x = nullptr, *norm = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr;
+    float *gate = nullptr, *up = nullptr, *logits = nullptr;
+
+    vx_graph *graph = nullptr;
+    int graph_batch = 0;
+    std::vector<int64_t> dev_seq_ids;  // batch currently loaded in d_slots (device-driven mode)
+    std::vector<int32_t> dev_positions;
+};
+
+namespace {
+
+template <class T>
+int dev_alloc(vh_model *m, T **p, size_t count) {
+    *p = (T *)vx_alloc_permanent(m->be, (count ? count : 1) * sizeof(T));
+    if (!*p) return fail("vx_alloc_permanent(%zu): %s", count * sizeof(T), vx_last_error());
+    return VH_OK;
+}
+
+SeqState *find_seq(vh_model *m, int64_t id) {
+    auto it = m->pool.seqs.find(id);
+    return it == m->pool.seqs.end() ? nullptr : &it->second;
+}
+
+int create_seq_locked(vh_model *m, int64_t id) {  // gpu_block_pool.go:126-135 (replaces an existing entry)
+    BlockPool &p = m->pool;
+    auto it = p.seqs.find(id);
+    int slot;
+    if (it != p.seqs.end()) {
+        slot = it->second.slot;
+    } else {
+        if (p.free_slots.empty()) return fail("more than %d live sequences", m->cfg.max_seqs);
+        slot = p.free_slots.back();
+        p.free_slots.pop_back();
+    }
+    SeqState s;
+    s.slot = slot;
+    p.seqs[id] = s;
+    return VH_OK;
+}
+
+int sync_pool_to_device(vh_model *m) {
+    BlockPool &p = m->pool;
+    const int mb = m->cfg.max_blocks_per_seq;
+    for (auto &kv : p.seqs) {
+        SeqState &s = kv.second;
+        if (!s.dirty) continue;
+        if ((int)s.table.size() > mb)
+            return fail("sequence %lld needs %zu blocks, the table holds %d", (long long)kv.first, s.table.size(), mb);
+        if (!s.table.empty())
+            VXC(vx_to_device(m->be, m->d_tables + (size_t)s.slot * mb, s.table.data(), s.table.size() * 4));
+        int32_t nb = (int32_t)s.table.size();
+        VXC(vx_to_device(m->be, m->d_num_blocks + s.slot, &nb, 4));
+        s.dirty = false;
+    }
+    if (p.free_dirty) {
+        if (!p.free_list.empty()) VXC(vx_to_device(m->be, m->d_free, p.free_list.data(), p.free_list.size() * 4));
+        int32_t fc = (int32_t)p.free_list.size();
+        VXC(vx_to_device(m->be, m->d_free_count, &fc, 4));
+        p.free_dirty = false;
+    }
+    return VH_OK;
+}
+
+int matmul(vh_model *m, const float *a, const vh_qweight &w, float *out, const float *residual, int rows) {
+    if (!w.data) return fail("weight not set");
+    VXC(vx_matmul_quant(m->be, w.fmt, a, w.data, out, residual, rows, w.n, w.k));
+    return VH_OK;
+}
+
+// One layer for `rows` single-token sequences; positions, slots, tables and lengths are on the device.
+int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len) {
+    const vh_config &c = m->cfg;
+    const vh_layer_weights &w = m->layers[layer];
+    const float scale = (float)(1.0 / sqrt((double)c.head_dim));                          // block.go:862
+    VXC(vx_rmsnorm(m->be, m->x, w.attn_norm, m->norm, rows, c.hidden, c.eps));            // block.go:834-837
+    VHC(matmul(m, m->norm, w.wq, m->q, nullptr, rows));                                   // block.go:841-854
+    VHC(matmul(m, m->norm, w.wk, m->k, nullptr, rows));
+    VHC(matmul(m, m->norm, w.wv, m->v, nullptr, rows));
+    VXC(vx_rope_store_paged(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
+                            c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta));  // :858, :868
+    VXC(vx_sdpa_paged_decode_ragged(m->be, m->q, m->kv[layer], c.kv_fp16, m->d_tables, m->d_slots, m->d_kv_lens,
+                                    m->attn, rows, c.max_blocks_per_seq, c.block_size, c.num_heads, c.num_kv_heads,
+                                    c.head_dim, scale, max_kv_len));                       // block.go:872
+    VHC(matmul(m, m->attn, w.wo, m->x, m->x, rows));                                      // block.go:981-990
+    VXC(vx_rmsnorm(m->be, m->x, w.ffn_norm, m->norm, rows, c.hidden, c.eps));             // block.go:996-998
+    VHC(matmul(m, m->norm, w.w1, m->gate, nullptr, rows));                                // block.go:1043-1050
+    VHC(matmul(m, m->norm, w.w3, m->up, nullptr, rows));
+    VXC(vx_silu_mul(m->be, m->gate, m->up, m->gate, rows * c.ffn));                       // block.go:1056
+    VHC(matmul(m, m->gate, w.w2, m->x, m->x, rows));                                      // block.go:1058-1077
+    return VH_OK;
+}
+
+// embedding -> layers -> final norm -> lm_head -> argmax for a decode batch (decode.go:404-452)
+int forward_decode(vh_model *m, int rows, int max_kv_len) {
+    const vh_config &c = m->cfg;
+    VXC(vx_embedding(m->be, m->d_tokens, rows, m->embedding, m->x, c.vocab, c.hidden));
+    for (int l = 0; l < c.num_layers; l++) VHC(execute_layer_decode(m, l, rows, max_kv_len));
+    VXC(vx_rmsnorm(m->be, m->x, m->final_norm, m->norm, rows, c.hidden, c.eps));           // model.go:207-226
+    VHC(matmul(m, m->norm, m->lm_head, m->logits, nullptr, rows));                        // model.go:352-422
+    VXC(vx_argmax_rows(m->be, m->logits, rows, c.vocab, m->d_next));
+    return VH_OK;
+}
+
+int check_ready(vh_model *m) {
+    if (!m->embedding || !m->final_norm || !m->lm_head.data) return fail("model head / embedding not set");
+    for (auto &l : m->layers)
+        if (!l.attn_norm || !l.wq.data) return fail("a layer's weights are not set");
+    return VH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *vh_last_error(void) { return g_err; }
+
+int vh_model_create(vx_backend *be, const vh_config *cfg, vh_model **out) {
+    if (!be || !cfg || !out) return fail("null argument");
+    const vh_config &c = *cfg;
+    if (c.num_layers <= 0 || c.hidden <= 0 || c.num_heads <= 0 || c.num_kv_heads <= 0 || c.head_dim <= 0 ||
+        c.ffn <= 0 || c.vocab <= 0 || c.block_size <= 0 || c.pool_blocks <= 0 || c.max_seqs <= 0 ||
+        c.max_blocks_per_seq <= 0 || c.max_batch <= 0 || c.max_batch > 1024)
+        return fail("bad configuration");
+    if (c.num_heads % c.num_kv_heads) return fail("%d heads not a multiple of %d kv heads", c.num_heads, c.num_kv_heads);
+    vh_model *m = new vh_model();
+    m->be = be;
+    m->cfg = c;
+    m->layers.resize(c.num_layers);
+    m->pool.block_size = c.block_size;
+    m->pool.max_blocks = c.pool_blocks;
+    m->pool.free_list.resize(c.pool_blocks);
+    for (int i = 0; i < c.pool_blocks; i++) m->pool.free_list[i] = i;
+    for (int i = c.max_seqs - 1; i >= 0; i--) m->pool.free_slots.push_back(i);
+    const size_t kv_bytes = (size_t)c.pool_blocks * 2 * c.block_size * c.num_kv_heads * c.head_dim * (c.kv_fp16 ? 2 : 4);
+    m->kv.resize(c.num_layers, nullptr);
+    for (int l = 0; l < c.num_layers; l++) {
+        m->kv[l] = vx_alloc_permanent(be, kv_bytes);
+        if (!m->kv[l]) {
+            fail("KV pool layer %d (%zu bytes): %s", l, kv_bytes, vx_last_error());
+            vh_model_destroy(m);
+            return VH_ERR;
+        }
+    }
+    const size_t mb = c.max_batch;
+    int rc = VH_OK;
+    rc |= dev_alloc(m, &m->d_tables, (size_t)c.max_seqs * c.max_blocks_per_seq);
+    rc |= dev_alloc(m, &m->d_num_blocks, c.max_seqs);
+    rc |= dev_alloc(m, &m->d_free, c.pool_blocks);
+    rc |= dev_alloc(m, &m->d_free_count, 1);
+    rc |= dev_alloc(m, &m->d_slots, mb);
+    rc |= dev_alloc(m, &m->d_positions, mb);
+    rc |= dev_alloc(m, &m->d_tokens, mb);
+    rc |= dev_alloc(m, &m->d_next, mb);
+    rc |= dev_alloc(m, &m->d_cu, mb + 1);
+    rc |= dev_alloc(m, &m->d_token_pos, mb);
+    rc |= dev_alloc(m, &m->d_slot_map, mb);
+    rc |= dev_alloc(m, &m->d_kv_lens, mb);
+    rc |= dev_alloc(m, &m->d_status, 1);
+    rc |= dev_alloc(m, &m->d_step, 1);
+    rc |= dev_alloc(m, &m->x, mb * c.hidden);
+    rc |= dev_alloc(m, &m->norm, mb * c.hidden);
+    rc |= dev_alloc(m, &m->q, mb * c.num_heads * c.head_dim);
+    rc |= dev_alloc(m, &m->k, mb * c.num_kv_heads * c.head_dim);
+    rc |= dev_alloc(m, &m->v, mb * c.num_kv_heads * c.head_dim);
+    rc |= dev_alloc(m, &m->attn, mb * c.num_heads * c.head_dim);
+    rc |= dev_alloc(m, &m->gate, mb * c.ffn);
+    rc |= dev_alloc(m, &m->up, mb * c.ffn);
+    rc |= dev_alloc(m, &m->logits, mb * c.vocab);
+    if (rc) {
+        vh_model_destroy(m);
+        return VH_ERR;
+    }
+    std::vector<int32_t> zeros((size_t)c.max_seqs * c.max_blocks_per_seq, 0);
+    if (vx_to_device(be, m->d_tables, zeros.data(), zeros.size() * 4) ||
+        vx_to_device(be, m->d_num_blocks, zeros.data(), (size_t)c.max_seqs * 4)) {
+        fail("init: %s", vx_last_error());
+        vh_model_destroy(m);
+        return VH_ERR;
+    }
+    *out = m;
+    return VH_OK;
+}
+
+void vh_model_destroy(vh_model *m) {
+    if (!m) return;
+    if (m->graph) vx_graph_destroy(m->graph);
+    for (void *p : m->kv) vx_free(m->be, p);
+    void *bufs[] = {m->d_tables, m->d_num_blocks, m->d_free, m->d_free_count, m->d_slots, m->d_positions, m->d_tokens,
+                    m->d_next, m->d_cu, m->d_token_pos, m->d_slot_map, m->d_kv_lens, m->d_status, m->d_step, m->d_log,
+                    m->x, m->norm, m->q, m->k, m->v, m->attn, m->gate, m->up, m->logits};
+    for (void *p : bufs) vx_free(m->be, p);
+    delete m;
+}
+
+int vh_model_set_layer(vh_model *m, int layer, const vh_layer_weights *w) {
+    if (!m || !w || layer < 0 || layer >= m->cfg.num_layers) return fail("bad layer index");
+    const vh_config &c = m->cfg;
+    const int qd = c.num_heads * c.head_dim, kvd = c.num_kv_heads * c.head_dim;
+    if (w->wq.n != qd || w->wq.k != c.hidden || w->wk.n != kvd || w->wv.n != kvd || w->wo.n != c.hidden ||
+        w->wo.k != qd || w->w1.n != c.ffn || w->w3.n != c.ffn || w->w2.n != c.hidden || w->w2.k != c.ffn)
+        return fail("layer %d: weight shapes do not match the configuration", layer);
+    m->layers[layer] = *w;
+    return VH_OK;
+}
+
+int vh_model_set_head(vh_model *m, const float *embedding, const float *final_norm, const vh_qweight *lm_head) {
+    if (!m || !embedding || !final_norm || !lm_head) return fail("null argument");
+    if (lm_head->n != m->cfg.vocab || lm_head->k != m->cfg.hidden) return fail("lm_head shape mismatch");
+    m->embedding = embedding;
+    m->final_norm = final_norm;
+    m->lm_head = *lm_head;
+    return VH_OK;
+}
+
+void *vh_kv_pool(vh_model *m, int layer) {
+    return (m && layer >= 0 && layer < m->cfg.num_layers) ? m->kv[layer] : nullptr;
+}
+
+// ------------------------------------------------------------------ GPUBlockPool
+int vh_pool_create_sequence(vh_model *m, int64_t seq_id) {
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    return create_seq_locked(m, seq_id);
+}
+
+int vh_pool_delete_sequence(vh_model *m, int64_t seq_id) {  // gpu_block_pool.go:138-157
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    SeqState *s = find_seq(m, seq_id);
+    if (!s) return VH_OK;
+    for (int32_t b : s->table) m->pool.release_block(b);
+    m->pool.free_slots.push_back(s->slot);
+    m->pool.seqs.erase(seq_id);
+    return VH_OK;
+}
+
+int vh_pool_truncate_sequence(vh_model *m, int64_t seq_id, int new_len) {  // gpu_block_pool.go:162-190
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    SeqState *s = find_seq(m, seq_id);
+    if (!s || new_len >= s->seq_len) return VH_OK;
+    int keep = 0;
+    if (new_len > 0) keep = (new_len - 1) / m->pool.block_size + 1;
+    for (int i = keep; i < (int)s->table.size(); i++) m->pool.release_block(s->table[i]);
+    if (keep < (int)s->table.size()) {
+        s->table.resize(keep);
+        s->dirty = true;
+    }
+    s->seq_len = new_len;
+    return VH_OK;
+}
+
+int vh_pool_has_sequence(vh_model *m, int64_t seq_id) {
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    return find_seq(m, seq_id) ? 1 : 0;
+}
+
+int vh_pool_share_blocks(vh_model *m, int64_t src_id, int64_t dst_id, int num_tokens) {  // gpu_block_pool.go:572-607
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    SeqState *src = find_seq(m, src_id);
+    if (!src) return fail("source sequence %lld not found", (long long)src_id);
+    SeqState *dst = find_seq(m, dst_id);
+    if (!dst) return fail("destination sequence %lld not found", (long long)dst_id);
+    int nb = (num_tokens + m->pool.block_size - 1) / m->pool.block_size;
+    if (nb > (int)src->table.size())
+        return fail("source seq %lld has %zu blocks, need %d", (long long)src_id, src->table.size(), nb);
+    for (int i = 0; i < nb; i++) {
+        dst->table.push_back(src->table[i]);
+        m->pool.ref_counts[src->table[i]]++;
+    }
+    dst->dirty = true;
+    if (num_tokens > dst->seq_len) dst->seq_len = num_tokens;
+    return VH_OK;
+}
+
+void vh_pool_block_stats(vh_model *m, int *total, int *free_blocks, int *shared) {  // gpu_block_pool.go:610-624
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    int sh = 0;
+    for (auto &kv : m->pool.ref_counts)
+        if (kv.second > 1) sh++;
+    if (total) *total = m->pool.max_blocks * m->cfg.num_layers;
+    if (free_blocks) *free_blocks = (int)m->pool.free_list.size() * m->cfg.num_layers;
+    if (shared) *shared = sh * m->cfg.num_layers;
+}
+
+int vh_pool_seq_len(vh_model *m, int64_t seq_id) {
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    SeqState *s = find_seq(m, seq_id);
+    return s ? s->seq_len : -1;
+}
+
+int vh_pool_block_table(vh_model *m, int64_t seq_id, int32_t *out, int cap) {
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    SeqState *s = find_seq(m, seq_id);
+    if (!s) return -1;
+    int n = (int)s->table.size();
+    for (int i = 0; i < n && i < cap; i++) out[i] = s->table[i];
+    return n;
+}
+
+int vh_pool_adopt_blocks(vh_model *m, int64_t seq_id, const int32_t *blocks, int num_blocks, int seq_len) {
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    SeqState *s = find_seq(m, seq_id);
+    if (!s) return fail("sequence %lld not found", (long long)seq_id);
+    if (!s->table.empty()) return fail("sequence %lld already owns blocks", (long long)seq_id);
+    if (seq_len > num_blocks * m->pool.block_size || seq_len <= (num_blocks - 1) * m->pool.block_size)
+        return fail("%d tokens do not fill exactly %d blocks", seq_len, num_blocks);
+    BlockPool &p = m->pool;
+    for (int i = 0; i < num_blocks; i++) {
+        auto it = std::find(p.free_list.begin(), p.free_list.end(), blocks[i]);
+        if (it == p.free_list.end()) return fail("block %d is not free", blocks[i]);
+        p.free_list.erase(it);
+        p.ref_counts[blocks[i]] = 1;
+        s->table.push_back(blocks[i]);
+    }
+    p.free_dirty = true;
+    s->dirty = true;
+    s->seq_len = seq_len;
+    return VH_OK;
+}
+
+int vh_pool_device_matches_host(vh_model *m) {
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    const int mb = m->cfg.max_blocks_per_seq;
+    if (vx_sync(m->be)) return -1;
+    std::vector<int32_t> row(mb);
+    for (auto &kv : m->pool.seqs) {
+        SeqState &s = kv.second;
+        if (s.dirty) continue;  // not pushed yet: nothing to compare
+        int32_t nb = -1;
+        if (vx_to_host(m->be, &nb, m->d_num_blocks + s.slot, 4)) return -1;
+        if (nb != (int32_t)s.table.size()) return 0;
+        if (nb > 0 && vx_to_host(m->be, row.data(), m->d_tables + (size_t)s.slot * mb, (size_t)nb * 4)) return -1;
+        for (int i = 0; i < nb; i++)
+            if (row[i] != s.table[i]) return 0;
+    }
+    if (!m->pool.free_dirty) {
+        int32_t fc = -1;
+        if (vx_to_host(m->be, &fc, m->d_free_count, 4)) return -1;
+        if (fc != (int32_t)m->pool.free_list.size()) return 0;
+        std::vector<int32_t> fl(fc > 0 ? fc : 1);
+        if (fc > 0 && vx_to_host(m->be, fl.data(), m->d_free, (size_t)fc * 4)) return -1;
+        for (int i = 0; i < fc; i++)
+            if (fl[i] != m->pool.free_list[i]) return 0;
+    }
+    return 1;
+}
+
+// ------------------------------------------------------------------ decode (host-built metadata)
+int vh_decode_batched(vh_model *m, const int32_t *tokens, const int64_t *seq_ids, const int32_t *positions, int batch,
+                      float *logits_out, int32_t *argmax_out) {
+    if (!m || !tokens || !seq_ids || !positions) return fail("null argument");
+    if (batch == 0) return VH_OK;                                                    // decode.go:619-621
+    if (batch < 0 || batch > m->cfg.max_batch) return fail("batch %d exceeds max_batch %d", batch, m->cfg.max_batch);
+    VHC(check_ready(m));
+    const vh_config &c = m->cfg;
+    std::vector<int32_t> slots(batch), slot_map(batch), kv_lens(batch);
+    int max_kv = 1;
+    {
+        std::lock_guard<std::mutex> g(m->pool.mu);
+        for (int i = 0; i < batch; i++) {
+            if (tokens[i] < 0 || tokens[i] >= c.vocab) return fail("token %d out of range", tokens[i]);
+            if (!find_seq(m, seq_ids[i])) VHC(create_seq_locked(m, seq_ids[i]));       // decode.go:361-363
+            SeqState *s = find_seq(m, seq_ids[i]);
+            const int pos = positions[i];
+            VHC(m->pool.ensure_blocks(*s, pos + 1));                                  // gpu_block_pool.go:234-245
+            slot_map[i] = s->table[pos / c.block_size] * c.block_size + pos % c.block_size;  // :250-252
+            if (pos + 1 > s->seq_len) s->seq_len = pos + 1;                           // :318-320
+            kv_lens[i] = s->seq_len;                                                  // :354 (kvLen = seq.seqLen)
+            slots[i] = s->slot;
+            max_kv = std::max(max_kv, kv_lens[i]);
+        }
+        VHC(sync_pool_to_device(m));
+    }
+    vx_reset_pool(m->be);                                                            // decode.go:366-368
+    VXC(vx_to_device(m->be, m->d_tokens, tokens, (size_t)batch * 4));                 // decode.go:389-395
+    VXC(vx_to_device(m->be, m->d_token_pos, positions, (size_t)batch * 4));
+    VXC(vx_to_device(m->be, m->d_slots, slots.data(), (size_t)batch * 4));
+    VXC(vx_to_device(m->be, m->d_slot_map, slot_map.data(), (size_t)batch * 4));
+    VXC(vx_to_device(m->be, m->d_kv_lens, kv_lens.data(), (size_t)batch * 4));
+    VHC(forward_decode(m, batch, max_kv));
+    if (logits_out) VXC(vx_to_host(m->be, logits_out, m->logits, (size_t)batch * c.vocab * 4));
+    if (argmax_out) VXC(vx_to_host(m->be, argmax_out, m->d_next, (size_t)batch * 4));
+    VXC(vx_sync(m->be));                                                             // decode.go:651
+    return VH_OK;
+}
+
+// ------------------------------------------------------------------ prefill / verify of one sequence
+int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int start_pos, int all_logits,
+               float *logits_out) {
+    if (!m || !tokens || n <= 0 || start_pos < 0) return fail("bad arguments");
+    VHC(check_ready(m));
+    const vh_config &c = m->cfg;
+    std::vector<int32_t> page(n), offs(n), kvl(n), table;
+    int seq_len;
+    {
+        std::lock_guard<std::mutex> g(m->pool.mu);
+        if (!find_seq(m, seq_id)) VHC(create_seq_locked(m, seq_id));
+        SeqState *s = find_seq(m, seq_id);
+        VHC(m->pool.ensure_blocks(*s, start_pos + n));
+        for (int i = 0; i < n; i++) {
+            const int pos = start_pos + i;
+            page[i] = s->table[pos / c.block_size];
+            offs[i] = pos % c.block_size;
+            kvl[i] = start_pos + i + 1;                                               // block.go:884-887
+        }
+        if (start_pos + n > s->seq_len) s->seq_len = start_pos + n;
+        seq_len = s->seq_len;
+        table = s->table;
+        VHC(sync_pool_to_device(m));
+    }
+    vx_backend *be = m->be;
+    vx_reset_pool(be);
+    const size_t qd = (size_t)c.num_heads * c.head_dim, kvd = (size_t)c.num_kv_heads * c.head_dim;
+    auto fa = [&](size_t count) { return (float *)vx_alloc(be, count * 4); };
+    auto ia = [&](size_t count) { return (int32_t *)vx_alloc(be, count * 4); };
+    int32_t *d_tok = ia(n), *d_page = ia(n), *d_offs = ia(n), *d_kvl = ia(n), *d_bt = ia(table.size());
+    float *x = fa((size_t)n * c.hidden), *norm = fa((size_t)n * c.hidden), *q = fa(n * qd), *k = fa(n * kvd);
+    float *v = fa(n * kvd), *attn = fa(n * qd), *gate = fa((size_t)n * c.ffn), *up = fa((size_t)n * c.ffn);
+    const int out_rows = all_logits ? n : 1;
+    float *logits = fa((size_t)out_rows * c.vocab);
+    if (!d_tok || !d_page || !d_offs || !d_kvl || !d_bt || !x || !norm || !q || !k || !v || !attn || !gate || !up || !logits)
+        return fail("prefill buffers: %s", vx_last_error());
+    VXC(vx_to_device(be, d_tok, tokens, (size_t)n * 4));
+    VXC(vx_to_device(be, d_page, page.data(), (size_t)n * 4));
+    VXC(vx_to_device(be, d_offs, offs.data(), (size_t)n * 4));
+    VXC(vx_to_device(be, d_kvl, kvl.data(), (size_t)n * 4));
+    VXC(vx_to_device(be, d_bt, table.data(), table.size() * 4));
+    VXC(vx_embedding(be, d_tok, n, m->embedding, x, c.vocab, c.hidden));               // decode.go:1005-1010
+    const float scale = (float)(1.0 / sqrt((double)c.head_dim));
+    for (int l = 0; l < c.num_layers; l++) {
+        const vh_layer_weights &w = m->layers[l];
+        VXC(vx_rmsnorm(be, x, w.attn_norm, norm, n, c.hidden, c.eps));
+        VHC(matmul(m, norm, w.wq, q, nullptr, n));
+        VHC(matmul(m, norm, w.wk, k, nullptr, n));
+        VHC(matmul(m, norm, w.wv, v, nullptr, n));
+        VXC(vx_rope(be, q, k, c.head_dim, c.num_heads, c.num_kv_heads, n, start_pos, 0, c.rope_theta, 0));  // block.go:858
+        if (c.kv_fp16) {                                                               // gpu_block_pool.go:262-272
+            VXC(vx_reshape_paged_kv_f16(be, k, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 0));
+            VXC(vx_reshape_paged_kv_f16(be, v, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 1));
+        } else {
+            VXC(vx_reshape_paged_kv(be, k, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 0));
+            VXC(vx_reshape_paged_kv(be, v, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 1));
+        }
+        if (n == 1) {                                                                  // block.go:866-874
+            const int nb = (seq_len + c.block_size - 1) / c.block_size;
+            const int til = seq_len - (nb - 1) * c.block_size;                        // gpu_block_pool.go:359-363
+            if (c.kv_fp16)
+                VXC(vx_sdpa_paged_decode_f16(be, q, m->kv[l], d_bt, attn, nb, c.block_size, c.num_heads,
+                                             c.num_kv_heads, c.head_dim, scale, til));
+            else
+                VXC(vx_sdpa_paged_decode(be, q, m->kv[l], d_bt, attn, nb, c.block_size, c.num_heads, c.num_kv_heads,
+                                         c.head_dim, scale, til));
+        } else if (start_pos > 0) {                                                    // block.go:881-890
+            VXC(vx_sdpa_paged_decode_multiquery(be, q, m->kv[l], c.kv_fp16, d_bt, attn, d_kvl, (int)table.size(),
+                                                c.block_size, c.num_heads, c.num_kv_heads, c.head_dim, scale, n));
+        } else {                                                                       // block.go:893-895
+            VXC(vx_sdpa_prefill(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale));
+        }
+        VHC(matmul(m, attn, w.wo, x, x, n));
+        VXC(vx_rmsnorm(be, x, w.ffn_norm, norm, n, c.hidden, c.eps));
+        VHC(matmul(m, norm, w.w1, gate, nullptr, n));
+        VHC(matmul(m, norm, w.w3, up, nullptr, n));
+        VXC(vx_silu_mul(be, gate, up, gate, n * c.ffn));
+        VHC(matmul(m, gate, w.w2, x, x, n));
+    }
+    const float *last = all_logits ? x : x + (size_t)(n - 1) * c.hidden;                // decode.go:1057-1066
+    VXC(vx_rmsnorm(be, last, m->final_norm, norm, out_rows, c.hidden, c.eps));
+    VHC(matmul(m, norm, m->lm_head, logits, nullptr, out_rows));
+    if (logits_out) VXC(vx_to_host(be, logits_out, logits, (size_t)out_rows * c.vocab * 4));
+    VXC(vx_sync(be));
+    return VH_OK;
+}
+
+// ------------------------------------------------------------------ device-driven greedy decode
+static int device_step(vh_model *m, int batch) {
+    const vh_config &c = m->cfg;
+    VXC(vx_pack_batch(m->be, m->d_slots, m->d_positions, nullptr, batch, batch, m->d_tables, c.max_blocks_per_seq,
+                      m->d_num_blocks, m->d_free, m->d_free_count, c.block_size, m->d_cu, m->d_token_pos,
+                      m->d_slot_map, m->d_kv_lens, m->d_status));
+    VHC(forward_decode(m, batch, c.max_blocks_per_seq * c.block_size));
+    VXC(vx_decode_advance(m->be, m->d_tokens, m->d_positions, m->d_next, m->d_log, m->d_step, batch));
+    return VH_OK;
+}
+
+int vh_decode_graph(vh_model *m, const int32_t *first_tokens, const int64_t *seq_ids, const int32_t *positions,
+                    int batch, int steps, int use_graph, int32_t *out_tokens, float *ms_per_step) {
+    if (!m || batch <= 0 || steps <= 0) return fail("bad arguments");
+    if (batch > m->cfg.max_batch) return fail("batch %d exceeds max_batch %d", batch, m->cfg.max_batch);
+    VHC(check_ready(m));
+    const vh_config &c = m->cfg;
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    if (first_tokens) {
+        if (!seq_ids || !positions) return fail("seq_ids / positions missing");
+        std::vector<int32_t> slots(batch);
+        for (int i = 0; i < batch; i++) {
+            SeqState *s = find_seq(m, seq_ids[i]);
+            if (!s) return fail("sequence %lld not found", (long long)seq_ids[i]);
+            if (positions[i] != s->seq_len)
+                return fail("sequence %lld: position %d is not its length %d", (long long)seq_ids[i], positions[i], s->seq_len);
+            slots[i] = s->slot;
+        }
+        VHC(sync_pool_to_device(m));
+        VXC(vx_to_device(m->be, m->d_tokens, first_tokens, (size_t)batch * 4));
+        VXC(vx_to_device(m->be, m->d_positions, positions, (size_t)batch * 4));
+        VXC(vx_to_device(m->be, m->d_slots, slots.data(), (size_t)batch * 4));
+        m->dev_seq_ids.assign(seq_ids, seq_ids + batch);
+        m->dev_positions.assign(positions, positions + batch);
+    } else {
+        if ((int)m->dev_seq_ids.size() != batch) return fail("no batch of %d sequences is loaded on the device", batch);
+        VHC(sync_pool_to_device(m));  // lifecycle events since the last call (no-op when nothing changed)
+    }
+    if (m->log_cap < steps) {
+        if (m->d_log) vx_free(m->be, m->d_log);
+        m->d_log = nullptr;
+        VHC(dev_alloc(m, &m->d_log, (size_t)steps * c.max_batch));
+        m->log_cap = steps;
+        if (m->graph) {  // the graph holds the old log pointer
+            vx_graph_destroy(m->graph);
+            m->graph = nullptr;
+        }
+    }
+    int32_t zero = 0;
+    VXC(vx_to_device(m->be, m->d_step, &zero, 4));
+    vx_reset_pool(m->be);
+    int done = 0;
+    if (use_graph && (!m->graph || m->graph_batch != batch)) {
+        if (m->graph) vx_graph_destroy(m->graph);
+        m->graph = nullptr;
+        VHC(device_step(m, batch));  // eager: sizes the library scratch; it is step 0 of this call
+        done = 1;
+        VXC(vx_graph_begin_capture(m->be));
+        int rc = device_step(m, batch);
+        vx_graph *gr = nullptr;
+        int rc2 = vx_graph_end_capture(m->be, &gr);
+        if (rc != VH_OK) return VH_ERR;
+        if (rc2 != VX_OK) return fail("graph capture: %s", vx_last_error());
+        m->graph = gr;
+        m->graph_batch = batch;
+    }
+    VXC(vx_timer_start(m->be));
+    const int timed = steps - done;
+    for (int s = done; s < steps; s++) {
+        if (use_graph)
+            VXC(vx_graph_launch(m->be, m->graph));
+        else
+            VHC(device_step(m, batch));
+    }
+    float ms = 0.f;
+    VXC(vx_timer_stop_ms(m->be, &ms));
+    if (ms_per_step) *ms_per_step = timed > 0 ? ms / timed : 0.f;
+    int32_t status = 0;
+    VXC(vx_to_host(m->be, &status, m->d_status, 4));
+    if (status != 0) return fail("the block pool ran out of blocks during the device-driven steps");
+    std::vector<int32_t> log((size_t)steps * batch);
+    VXC(vx_to_host(m->be, log.data(), m->d_log, log.size() * 4));
+    if (out_tokens) memcpy(out_tokens, log.data(), log.size() * 4);
+    // advance the host pool by the same rule, in the same order (step-major, batch order)
+    for (int s = 0; s < steps; s++)
+        for (int i = 0; i < batch; i++) {
+            SeqState *st = find_seq(m, m->dev_seq_ids[i]);
+            const int pos = m->dev_positions[i] + s;
+            VHC(m->pool.ensure_blocks(*st, pos + 1));
+            if (pos + 1 > st->seq_len) st->seq_len = pos + 1;
+        }
+    for (int i = 0; i < batch; i++) {
+        m->dev_positions[i] += steps;
+        find_seq(m, m->dev_seq_ids[i])->dirty = false;  // the device made the same allocations itself
+    }
+    m->pool.free_dirty = false;
+    return VH_OK;
+}
+
+}  // extern "C"

@@ -58,10 +58,11 @@ SIGNATURES = {
     "vx_dequantize": (_i, [_vp, _i, _vp, _vp, _i64]),
     "vx_matmul_quant": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i]),
     "vx_rope_store_paged": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f]),
-    "vx_sdpa_paged_decode_ragged": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i]),
+    "vx_sdpa_paged_decode_ragged": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i]),
     "vx_sdpa_paged_tree": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),
     "vx_argmax_rows": (_i, [_vp, _vp, _i, _i, _vp]),
     "vx_pack_batch": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
+    "vx_decode_advance": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "vx_graph_begin_capture": (_i, [_vp]),
     "vx_graph_end_capture": (_i, [_vp, C.POINTER(_vp)]),
     "vx_graph_launch": (_i, [_vp, _vp]),

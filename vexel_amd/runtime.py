@@ -1,0 +1,209 @@
+"""ModelRuntime: Python handle on libvexel_host.so, the C++ restatement of the Go runtime
+pieces that drive the batched-decode path (inference/runtime: GPUBlockPool, BlockRuntime.
+ExecuteWithPagedKV, ModelRuntime.DecodeWithPagedKVBatched / PrefillWithPagedKV). Method
+names follow the Go methods in snake_case. Nothing is computed in Python."""
+import ctypes as C
+import os
+
+import numpy as np
+
+from . import lib as _l
+from .backend import HipBackend, VexelError
+
+HOST_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libvexel_host.so")
+
+
+class VhConfig(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("num_layers", "hidden", "num_heads", "num_kv_heads", "head_dim", "ffn",
+                                        "vocab")] + \
+               [("eps", C.c_float), ("rope_theta", C.c_float)] + \
+               [(n, C.c_int) for n in ("block_size", "pool_blocks", "max_seqs", "max_blocks_per_seq", "max_batch",
+                                        "kv_fp16")]
+
+
+class VhQWeight(C.Structure):
+    _fields_ = [("fmt", C.c_int), ("data", C.c_void_p), ("n", C.c_int), ("k", C.c_int)]
+
+
+class VhLayerWeights(C.Structure):
+    _fields_ = [("attn_norm", C.c_void_p), ("ffn_norm", C.c_void_p)] + \
+               [(n, VhQWeight) for n in ("wq", "wk", "wv", "wo", "w1", "w2", "w3")]
+
+
+_host = None
+
+
+def load_host():
+    global _host
+    if _host is None:
+        _l.load()
+        if not os.path.exists(HOST_LIB_PATH):
+            raise RuntimeError("%s is missing: build it with `python -m vexel_amd.build`" % HOST_LIB_PATH)
+        h = C.CDLL(HOST_LIB_PATH)
+        h.vh_last_error.restype = C.c_char_p
+        h.vh_kv_pool.restype = C.c_void_p
+        h.vh_kv_pool.argtypes = [C.c_void_p, C.c_int]
+        h.vh_model_create.argtypes = [C.c_void_p, C.POINTER(VhConfig), C.POINTER(C.c_void_p)]
+        h.vh_model_destroy.argtypes = [C.c_void_p]
+        h.vh_model_destroy.restype = None
+        h.vh_model_set_layer.argtypes = [C.c_void_p, C.c_int, C.POINTER(VhLayerWeights)]
+        h.vh_model_set_head.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(VhQWeight)]
+        for name in ("vh_pool_create_sequence", "vh_pool_delete_sequence", "vh_pool_has_sequence", "vh_pool_seq_len"):
+            getattr(h, name).argtypes = [C.c_void_p, C.c_int64]
+        h.vh_pool_truncate_sequence.argtypes = [C.c_void_p, C.c_int64, C.c_int]
+        h.vh_pool_share_blocks.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_int]
+        h.vh_pool_block_stats.argtypes = [C.c_void_p] + [C.POINTER(C.c_int)] * 3
+        h.vh_pool_block_stats.restype = None
+        h.vh_pool_block_table.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int]
+        h.vh_pool_adopt_blocks.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int]
+        h.vh_pool_device_matches_host.argtypes = [C.c_void_p]
+        h.vh_decode_batched.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
+        h.vh_prefill.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_int, C.c_void_p]
+        h.vh_decode_graph.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
+                                      C.c_void_p, C.POINTER(C.c_float)]
+        _host = h
+    return _host
+
+
+class ModelRuntime:
+    def __init__(self, be: HipBackend, num_layers, hidden, num_heads, num_kv_heads, head_dim, ffn, vocab,
+                 eps=1e-5, rope_theta=10000.0, block_size=16, pool_blocks=256, max_seqs=64,
+                 max_blocks_per_seq=None, max_batch=64, kv_fp16=True):
+        self._h = load_host()
+        self.be = be
+        if max_blocks_per_seq is None:
+            max_blocks_per_seq = pool_blocks
+        self.cfg = VhConfig(num_layers, hidden, num_heads, num_kv_heads, head_dim, ffn, vocab, eps, rope_theta,
+                            block_size, pool_blocks, max_seqs, max_blocks_per_seq, max_batch, int(bool(kv_fp16)))
+        m = C.c_void_p()
+        self._ck(self._h.vh_model_create(be._h, C.byref(self.cfg), C.byref(m)))
+        self._m = m
+        self._keep = []   # device buffers owned by this model
+
+    def _ck(self, rc):
+        if rc != 0:
+            raise VexelError(rc, self._h.vh_last_error().decode())
+
+    def close(self):
+        if self._m:
+            self._h.vh_model_destroy(self._m)
+            self._m = None
+            for p in self._keep:
+                self.be.free(p)
+            self._keep = []
+
+    # ---- weights
+    def _up(self, arr):
+        p = self.be.upload(np.ascontiguousarray(arr), permanent=True)
+        self._keep.append(p)
+        return p
+
+    def adopt_device_buffer(self, ptr):
+        """The model frees `ptr` (a vx_alloc_permanent buffer) when it is closed."""
+        self._keep.append(ptr)
+
+    @staticmethod
+    def qweight(fmt, dev_ptr, n, k):
+        return VhQWeight(fmt, dev_ptr, n, k)
+
+    def set_layer(self, layer, attn_norm, ffn_norm, weights):
+        """weights: dict name -> (fmt, numpy uint8 rows | device pointer, n, k) for wq wk wv wo w1 w2 w3."""
+        lw = VhLayerWeights()
+        lw.attn_norm = attn_norm if isinstance(attn_norm, int) else self._up(np.asarray(attn_norm, dtype=np.float32))
+        lw.ffn_norm = ffn_norm if isinstance(ffn_norm, int) else self._up(np.asarray(ffn_norm, dtype=np.float32))
+        for name in ("wq", "wk", "wv", "wo", "w1", "w2", "w3"):
+            fmt, data, n, k = weights[name]
+            ptr = data if isinstance(data, int) else self._up(data)
+            setattr(lw, name, VhQWeight(fmt, ptr, n, k))
+        self._ck(self._h.vh_model_set_layer(self._m, layer, C.byref(lw)))
+
+    def set_head(self, embedding_f32, final_norm, lm_head):
+        """embedding_f32: numpy [vocab,hidden] float32 or device pointer; lm_head: (fmt, data, n, k)."""
+        emb = embedding_f32 if isinstance(embedding_f32, int) else self._up(np.asarray(embedding_f32, dtype=np.float32))
+        fn = final_norm if isinstance(final_norm, int) else self._up(np.asarray(final_norm, dtype=np.float32))
+        fmt, data, n, k = lm_head
+        ptr = data if isinstance(data, int) else self._up(data)
+        qw = VhQWeight(fmt, ptr, n, k)
+        self._ck(self._h.vh_model_set_head(self._m, emb, fn, C.byref(qw)))
+
+    def kv_pool(self, layer):
+        return self._h.vh_kv_pool(self._m, layer)
+
+    # ---- GPUBlockPool
+    def create_sequence(self, seq_id):
+        self._ck(self._h.vh_pool_create_sequence(self._m, seq_id))
+
+    def delete_sequence(self, seq_id):
+        self._ck(self._h.vh_pool_delete_sequence(self._m, seq_id))
+
+    def truncate_sequence(self, seq_id, new_len):
+        self._ck(self._h.vh_pool_truncate_sequence(self._m, seq_id, new_len))
+
+    def has_sequence(self, seq_id):
+        return bool(self._h.vh_pool_has_sequence(self._m, seq_id))
+
+    def share_blocks(self, src, dst, num_tokens):
+        self._ck(self._h.vh_pool_share_blocks(self._m, src, dst, num_tokens))
+
+    def block_stats(self):
+        a, b, c = C.c_int(), C.c_int(), C.c_int()
+        self._h.vh_pool_block_stats(self._m, C.byref(a), C.byref(b), C.byref(c))
+        return a.value, b.value, c.value
+
+    def seq_len(self, seq_id):
+        return self._h.vh_pool_seq_len(self._m, seq_id)
+
+    def block_table(self, seq_id):
+        cap = self.cfg.max_blocks_per_seq + self.cfg.pool_blocks
+        buf = np.zeros(cap, dtype=np.int32)
+        n = self._h.vh_pool_block_table(self._m, seq_id, buf.ctypes.data, cap)
+        return None if n < 0 else [int(x) for x in buf[:n]]
+
+    def adopt_blocks(self, seq_id, blocks, seq_len):
+        b = np.ascontiguousarray(blocks, dtype=np.int32)
+        self._ck(self._h.vh_pool_adopt_blocks(self._m, seq_id, b.ctypes.data, b.size, seq_len))
+
+    def device_matches_host(self):
+        r = self._h.vh_pool_device_matches_host(self._m)
+        if r < 0:
+            raise VexelError(1, "device mirror read failed")
+        return bool(r)
+
+    # ---- drivers
+    def decode_with_paged_kv_batched(self, tokens, seq_ids, positions, want_logits=True):
+        """-> (logits [B,V] or None, argmax [B])"""
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        s = np.ascontiguousarray(seq_ids, dtype=np.int64)
+        p = np.ascontiguousarray(positions, dtype=np.int32)
+        b = t.size
+        logits = np.empty((b, self.cfg.vocab), dtype=np.float32) if want_logits else None
+        am = np.empty(b, dtype=np.int32)
+        self._ck(self._h.vh_decode_batched(self._m, t.ctypes.data, s.ctypes.data, p.ctypes.data, b,
+                                           logits.ctypes.data if want_logits else None, am.ctypes.data))
+        return logits, am
+
+    def prefill_with_paged_kv(self, tokens, seq_id, start_pos, all_logits=False):
+        t = np.ascontiguousarray(tokens, dtype=np.int32)
+        rows = t.size if all_logits else 1
+        logits = np.empty((rows, self.cfg.vocab), dtype=np.float32)
+        self._ck(self._h.vh_prefill(self._m, t.ctypes.data, t.size, seq_id, start_pos, int(all_logits),
+                                    logits.ctypes.data))
+        return logits if all_logits else logits[0]
+
+    def decode_graph(self, first_tokens, seq_ids, positions, steps, use_graph=True, batch=None):
+        """Greedy device-driven decode. first_tokens=None continues the batch loaded on the device.
+        -> (tokens [steps,B], ms_per_step of the timed steps)"""
+        if first_tokens is not None:
+            t = np.ascontiguousarray(first_tokens, dtype=np.int32)
+            s = np.ascontiguousarray(seq_ids, dtype=np.int64)
+            p = np.ascontiguousarray(positions, dtype=np.int32)
+            b = t.size
+            args = (t.ctypes.data, s.ctypes.data, p.ctypes.data)
+        else:
+            b = batch
+            args = (None, None, None)
+        out = np.empty((steps, b), dtype=np.int32)
+        ms = C.c_float()
+        self._ck(self._h.vh_decode_graph(self._m, *args, b, steps, int(bool(use_graph)), out.ctypes.data,
+                                         C.byref(ms)))
+        return out, ms.value
