@@ -1,0 +1,270 @@
+#!/usr/bin/env python3
+"""Benchmark of the batched-decode hot path on one MI355X.
+
+Workload (BASELINE.json north star): LLaMA-2-7B-shaped decoder (32 layers, hidden 4096, 32 MHA
+heads, head_dim 128, FFN 11008, vocab 32000), random-init N(0,0.02) weights quantized to Q4_0
+(token embedding and output head Q8_0, the rule of config 1), F16 paged KV (block 16) pre-filled
+with N(0,1), 32 ragged sequences with contexts lognormal(median 1024, sigma 0.6) clipped to
+[64, 4096] (seed 0), block tables a seeded permutation of the physical blocks. A step is one
+greedy decode step of all 32 sequences (pack -> 32 layers -> head -> argmax), replayed from a
+hipGraph with inputs resident in HBM.
+
+Prints ONE JSON line. torch is used only to make the synthetic weights / KV on the device.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+CFG = dict(num_layers=32, hidden=4096, num_heads=32, num_kv_heads=32, head_dim=128, ffn=11008, vocab=32000)
+BATCH = 32
+BLOCK = 16
+
+
+def ragged_contexts(seed=0, n=BATCH):
+    rng = np.random.default_rng(seed)
+    ctx = np.exp(rng.normal(math.log(1024.0), 0.6, n))
+    return [int(x) for x in np.clip(ctx, 64, 4096)]
+
+
+def q4_0_torch(torch, w):
+    n, k = w.shape
+    blk = w.view(n, k // 32, 32)
+    idx = blk.abs().argmax(dim=2, keepdim=True)
+    mx = blk.gather(2, idx)
+    d = mx / -8.0
+    inv = torch.where(d != 0, 1.0 / d, torch.zeros_like(d))
+    q = torch.clamp(torch.floor(blk * inv + 8.5), 0, 15).to(torch.uint8)
+    out = torch.empty((n, k // 32, 18), dtype=torch.uint8, device=w.device)
+    out[..., 0:2] = d.to(torch.float16).view(torch.uint8).view(n, k // 32, 2)
+    out[..., 2:] = q[..., :16] | (q[..., 16:] << 4)
+    return out.view(n, -1)
+
+
+def q8_0_torch(torch, w):
+    n, k = w.shape
+    blk = w.view(n, k // 32, 32)
+    d = blk.abs().amax(dim=2, keepdim=True) / 127.0
+    inv = torch.where(d != 0, 1.0 / d, torch.zeros_like(d))
+    q = torch.clamp(torch.round(blk * inv), -127, 127).to(torch.int8)
+    out = torch.empty((n, k // 32, 34), dtype=torch.uint8, device=w.device)
+    out[..., 0:2] = d.to(torch.float16).view(torch.uint8).view(n, k // 32, 2)
+    out[..., 2:] = q.view(torch.uint8)
+    return out.view(n, -1)
+
+
+def build_model(be, ctx, extra_tokens, layers):
+    """Synthetic 7B-shaped model + pre-filled contexts. Returns (ModelRuntime, seq_ids, keep)."""
+    import torch
+    from vexel_amd import lib
+    from vexel_amd.runtime import ModelRuntime
+    dev = torch.device("cuda:0")
+    c = dict(CFG)
+    c["num_layers"] = layers
+    need_blocks = sum((L + extra_tokens + BLOCK - 1) // BLOCK + 1 for L in ctx)
+    max_bps = (max(ctx) + extra_tokens + BLOCK - 1) // BLOCK + 1
+    mr = ModelRuntime(be, **c, pool_blocks=need_blocks, max_seqs=len(ctx), max_blocks_per_seq=max_bps,
+                      max_batch=len(ctx), kv_fp16=True)
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+
+    def to_ours(t):
+        torch.cuda.synchronize()
+        p = be.alloc_permanent(t.numel() * t.element_size())
+        mr.adopt_device_buffer(p)
+        be.copy_buffer(t.data_ptr(), 0, p, 0, t.numel() * t.element_size())
+        be.sync()
+        return p
+
+    def qw(n, k, fmt=lib.VX_Q4_0):
+        w = torch.randn((n, k), generator=g, device=dev, dtype=torch.float32) * 0.02
+        q = q4_0_torch(torch, w) if fmt == lib.VX_Q4_0 else q8_0_torch(torch, w)
+        return (fmt, to_ours(q), n, k)
+
+    h, qd, kvd, f, v = c["hidden"], c["num_heads"] * c["head_dim"], c["num_kv_heads"] * c["head_dim"], c["ffn"], c["vocab"]
+    ones = to_ours(torch.ones(h, device=dev, dtype=torch.float32))
+    for l in range(layers):
+        mr.set_layer(l, ones, ones, dict(wq=qw(qd, h), wk=qw(kvd, h), wv=qw(kvd, h), wo=qw(h, qd),
+                                         w1=qw(f, h), w3=qw(f, h), w2=qw(h, f)))
+    emb_q = qw(v, h, lib.VX_Q8_0)
+    emb = be.alloc_permanent(v * h * 4)
+    mr.adopt_device_buffer(emb)
+    be.dequantize(lib.VX_Q8_0, emb_q[1], emb, v * h)     # loader rule: token_embd kept in F32
+    mr.set_head(emb, ones, qw(v, h, lib.VX_Q8_0))
+    # KV: every physical block of every layer holds N(0,1) halves
+    per_block = 2 * BLOCK * kvd
+    for l in range(layers):
+        chunk = 256
+        for b0 in range(0, need_blocks, chunk):
+            nb = min(chunk, need_blocks - b0)
+            t = torch.randn(nb * per_block, generator=g, device=dev, dtype=torch.float32).to(torch.float16)
+            torch.cuda.synchronize()
+            be.copy_buffer(t.data_ptr(), 0, mr.kv_pool(l), b0 * per_block * 2, nb * per_block * 2)
+            be.sync()
+    rng = np.random.default_rng(0)
+    perm = rng.permutation(need_blocks)
+    ids, off = [], 0
+    for i, L in enumerate(ctx):
+        nb = (L + BLOCK - 1) // BLOCK
+        mr.create_sequence(i + 1)
+        mr.adopt_blocks(i + 1, perm[off:off + nb], L)
+        off += nb
+        ids.append(i + 1)
+    del t
+    torch.cuda.empty_cache()
+    return mr, ids
+
+
+def attention_bytes(ctx_lens, c):
+    """Algorithmic bytes of one ragged attention launch (one layer): K+V halves, block table, Q and out."""
+    kvd, qd = c["num_kv_heads"] * c["head_dim"], c["num_heads"] * c["head_dim"]
+    return sum(2 * L * kvd * 2 + ((L + BLOCK - 1) // BLOCK) * 4 + 2 * qd * 4 for L in ctx_lens)
+
+
+def time_attention_kernel(be, mr, ctx_now, c, layers, reps):
+    """Average duration of one ragged paged-attention launch (split-KV kernel + merge), HIP events on
+    the backend stream, cycling over the layers' pools so every launch streams from HBM."""
+    b = len(ctx_now)
+    qd = c["num_heads"] * c["head_dim"]
+    q = be.upload(np.random.default_rng(1).standard_normal((b, qd)).astype(np.float32), permanent=True)
+    out = be.alloc_permanent(b * qd * 4)
+    bts = np.zeros((b, mr.cfg.max_blocks_per_seq), dtype=np.int32)
+    for i in range(b):
+        t = mr.block_table(i + 1)
+        bts[i, :len(t)] = t
+    d_bt = be.upload(bts, permanent=True)
+    d_len = be.upload(np.array(ctx_now, dtype=np.int32), permanent=True)
+    scale = 1.0 / math.sqrt(c["head_dim"])
+    cap = mr.cfg.max_blocks_per_seq * BLOCK
+
+    def run(n):
+        for i in range(n):
+            be.sdpa_paged_decode_ragged(q, mr.kv_pool(i % layers), True, d_bt, d_len, out, b, mr.cfg.max_blocks_per_seq,
+                                        BLOCK, c["num_heads"], c["num_kv_heads"], c["head_dim"], scale, cap)
+    run(layers)
+    be.sync()
+    be.timer_start()
+    run(reps)
+    ms = be.timer_stop_ms()
+    for p in (q, out, d_bt, d_len):
+        be.free(p)
+    return ms / reps
+
+
+def cpu_baseline(be, mr, ctx, c, sample_layers=2, head_rows=2000):
+    """The reference CPU path (our C restatement, one core: the reference parallelises matmuls over M
+    only and decodes one sequence at a time, cpu.go:856-870, decode.go:642-650) timed on a bounded
+    sample: `sample_layers` layers + `head_rows` lm_head rows for one sequence, scaled to a full token."""
+    from oracle import numerics as nx
+    L = ctx[0]
+    hd, qd, kvd, f = c["hidden"], c["num_heads"] * c["head_dim"], c["num_kv_heads"] * c["head_dim"], c["ffn"]
+    rng = np.random.default_rng(2)
+    rb = lambda k: k // 32 * 18
+    w = {}
+    # weights of the sampled layers: random Q4_0 bytes of the real shapes (timing only)
+    for name, (n, k) in dict(wq=(qd, hd), wk=(kvd, hd), wv=(kvd, hd), wo=(hd, qd), w1=(f, hd), w3=(f, hd), w2=(hd, f)).items():
+        w[name] = (rng.integers(0, 256, size=(n, rb(k)), dtype=np.uint8), n, k)
+    head = rng.integers(0, 256, size=(head_rows, hd // 32 * 34), dtype=np.uint8)
+    per_block = 2 * BLOCK * kvd
+    nb = (L + BLOCK - 1) // BLOCK
+    pool = rng.integers(0, 0x3C00, size=nb * per_block, dtype=np.uint16)
+    bt = list(range(nb))
+    x = rng.standard_normal((1, hd)).astype(np.float32)
+    ones = np.ones(hd, dtype=np.float32)
+    scale = np.float32(1.0 / math.sqrt(c["head_dim"]))
+    t0 = time.perf_counter()
+    for _ in range(sample_layers):
+        nrm = nx.rmsnorm(x, ones, 1, hd, 1e-5)
+        q = nx.matmul_q4_0(nrm, w["wq"][0], 1, w["wq"][1], w["wq"][2])
+        k = nx.matmul_q4_0(nrm, w["wk"][0], 1, w["wk"][1], w["wk"][2])
+        v = nx.matmul_q4_0(nrm, w["wv"][0], 1, w["wv"][1], w["wv"][2])
+        q, k = nx.rope(q, k, c["head_dim"], c["num_heads"], c["num_kv_heads"], 1, L - 1, 0, 10000.0, False)
+        nx.reshape_paged_kv(k, pool, [bt[(L - 1) // BLOCK]], [(L - 1) % BLOCK], c["num_kv_heads"], c["head_dim"], BLOCK, False)
+        nx.reshape_paged_kv(v, pool, [bt[(L - 1) // BLOCK]], [(L - 1) % BLOCK], c["num_kv_heads"], c["head_dim"], BLOCK, True)
+        a = nx.sdpa_paged_decode(q, pool, bt, nb, BLOCK, c["num_heads"], c["num_kv_heads"], c["head_dim"], scale,
+                                 L - (nb - 1) * BLOCK).reshape(1, -1)
+        x = nx.add(x, nx.matmul_q4_0(a, w["wo"][0], 1, w["wo"][1], w["wo"][2]))
+        nrm = nx.rmsnorm(x, ones, 1, hd, 1e-5)
+        g = nx.matmul_q4_0(nrm, w["w1"][0], 1, w["w1"][1], w["w1"][2])
+        u = nx.matmul_q4_0(nrm, w["w3"][0], 1, w["w3"][1], w["w3"][2])
+        x = nx.add(x, nx.matmul_q4_0(nx.silu_mul(g, u), w["w2"][0], 1, w["w2"][1], w["w2"][2]))
+    t_layers = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    nx.matmul_quant(nx.FMT_Q8_0, nx.rmsnorm(x, ones, 1, hd, 1e-5), head, 1, head_rows, hd)
+    t_head = time.perf_counter() - t0
+    per_token = t_layers / sample_layers * c["num_layers"] + t_head / head_rows * c["vocab"]
+    return dict(value=1.0 / per_token, unit="tok/s", cores=1, kind="port",
+                sample="%d of %d layers + %d of %d lm_head rows for one sequence (ctx %d), extrapolated to a full "
+                       "token; host has %d cores, the reference path uses min(cores, M)=1"
+                       % (sample_layers, c["num_layers"], head_rows, c["vocab"], L, os.cpu_count()))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=32)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--layers", type=int, default=CFG["num_layers"], help="debug only: fewer layers is NOT the benchmark")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    from vexel_amd.backend import HipBackend
+    be = HipBackend(0)
+    ctx = ragged_contexts()
+    c = dict(CFG)
+    c["num_layers"] = args.layers
+    mr, ids = build_model(be, ctx, args.steps + args.warmup + 8, args.layers)
+    first = np.random.default_rng(3).integers(0, c["vocab"], BATCH).astype(np.int32)
+    use_graph = not args.no_graph
+    # warmup (untimed): first call runs one eager step, captures the graph, replays the rest
+    w = max(args.warmup, 2 if use_graph else 1)
+    mr.decode_graph(first, ids, ctx, w, use_graph=use_graph)
+    be.sync()
+    t0 = time.perf_counter()
+    toks, ms_events = mr.decode_graph(None, None, None, args.steps, use_graph=use_graph, batch=BATCH)
+    be.sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    ctx_now = [L + w + args.steps for L in ctx]
+    # dominant kernel: ragged paged attention (one launch per layer per step)
+    attn_ms = time_attention_kernel(be, mr, ctx_now, c, args.layers, reps=4 * args.layers)
+    attn_bytes = attention_bytes(ctx_now, c)
+    achieved = attn_bytes / (attn_ms * 1e-3) / 1e9
+    out = {
+        "metric": "decode tok/s, 7B Q4_0 x32 ragged seqs; % HBM peak in matvec + attn",
+        "value": BATCH * args.steps / wall,
+        "unit": "tok/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": w,
+        "ms_per_step": ms_per_step,
+        "ms_per_step_hip_events": ms_events,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "LLaMA-2-7B-shaped Q4_0 (Q8_0 embedding+head), %d layers, 32 ragged paged-KV seqs, "
+                               "ctx lognormal(median 1024, sigma 0.6) in [64,4096] seed 0, sum ctx %d, block 16, "
+                               "greedy decode, hipGraph=%s" % (args.layers, sum(ctx_now), use_graph),
+                   "global_batch": BATCH},
+        "roofline": {"bound": "hbm", "kernel": "paged_decode_f16_kernel<128,1> (+paged_merge_kernel)",
+                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": None, "bytes_per_launch": attn_bytes, "ms_per_launch": attn_ms},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(be, mr, ctx_now, c)
+    mr.close()
+    be.close()
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
