@@ -9,7 +9,8 @@ with N(0,1), 32 ragged sequences with contexts lognormal(median 1024, sigma 0.6)
 greedy decode step of all 32 sequences (pack -> 32 layers -> head -> argmax), replayed from a
 hipGraph with inputs resident in HBM.
 
-Prints ONE JSON line. torch is used only to make the synthetic weights / KV on the device.
+Prints ONE JSON line. The synthetic weights and KV contents are generated on the device by
+libvexel_synth.so (benchmark support built next to the backend); no torch in this process.
 """
 import argparse
 import json
@@ -36,62 +37,45 @@ def ragged_contexts(seed=0, n=BATCH):
     return [int(x) for x in np.clip(ctx, 64, 4096)]
 
 
-def q4_0_torch(torch, w):
-    n, k = w.shape
-    blk = w.view(n, k // 32, 32)
-    idx = blk.abs().argmax(dim=2, keepdim=True)
-    mx = blk.gather(2, idx)
-    d = mx / -8.0
-    inv = torch.where(d != 0, 1.0 / d, torch.zeros_like(d))
-    q = torch.clamp(torch.floor(blk * inv + 8.5), 0, 15).to(torch.uint8)
-    out = torch.empty((n, k // 32, 18), dtype=torch.uint8, device=w.device)
-    out[..., 0:2] = d.to(torch.float16).view(torch.uint8).view(n, k // 32, 2)
-    out[..., 2:] = q[..., :16] | (q[..., 16:] << 4)
-    return out.view(n, -1)
-
-
-def q8_0_torch(torch, w):
-    n, k = w.shape
-    blk = w.view(n, k // 32, 32)
-    d = blk.abs().amax(dim=2, keepdim=True) / 127.0
-    inv = torch.where(d != 0, 1.0 / d, torch.zeros_like(d))
-    q = torch.clamp(torch.round(blk * inv), -127, 127).to(torch.int8)
-    out = torch.empty((n, k // 32, 34), dtype=torch.uint8, device=w.device)
-    out[..., 0:2] = d.to(torch.float16).view(torch.uint8).view(n, k // 32, 2)
-    out[..., 2:] = q.view(torch.uint8)
-    return out.view(n, -1)
+def load_synth():
+    """libvexel_synth.so: device-side generators of the synthetic weights and KV (benchmark support)."""
+    import ctypes as C
+    path = os.path.join(ROOT, "vexel_amd", "libvexel_synth.so")
+    if not os.path.exists(path):
+        raise RuntimeError("%s is missing: run `python -m vexel_amd.build`" % path)
+    s = C.CDLL(path)
+    s.vxs_gaussian_quant.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_float, C.c_uint64]
+    s.vxs_gaussian_f16.argtypes = [C.c_void_p, C.c_int64, C.c_float, C.c_uint64]
+    return s
 
 
 def build_model(be, ctx, extra_tokens, layers):
-    """Synthetic 7B-shaped model + pre-filled contexts. Returns (ModelRuntime, seq_ids, keep)."""
-    import torch
+    """Synthetic 7B-shaped model + pre-filled contexts, generated on the device. -> (ModelRuntime, ids)"""
     from vexel_amd import lib
     from vexel_amd.runtime import ModelRuntime
-    dev = torch.device("cuda:0")
+    synth = load_synth()
     c = dict(CFG)
     c["num_layers"] = layers
     need_blocks = sum((L + extra_tokens + BLOCK - 1) // BLOCK + 1 for L in ctx)
     max_bps = (max(ctx) + extra_tokens + BLOCK - 1) // BLOCK + 1
     mr = ModelRuntime(be, **c, pool_blocks=need_blocks, max_seqs=len(ctx), max_blocks_per_seq=max_bps,
                       max_batch=len(ctx), kv_fp16=True)
-    g = torch.Generator(device=dev)
-    g.manual_seed(0)
-
-    def to_ours(t):
-        torch.cuda.synchronize()
-        p = be.alloc_permanent(t.numel() * t.element_size())
-        mr.adopt_device_buffer(p)
-        be.copy_buffer(t.data_ptr(), 0, p, 0, t.numel() * t.element_size())
-        be.sync()
-        return p
+    seed = [0]
 
     def qw(n, k, fmt=lib.VX_Q4_0):
-        w = torch.randn((n, k), generator=g, device=dev, dtype=torch.float32) * 0.02
-        q = q4_0_torch(torch, w) if fmt == lib.VX_Q4_0 else q8_0_torch(torch, w)
-        return (fmt, to_ours(q), n, k)
+        bb = 18 if fmt == lib.VX_Q4_0 else 34
+        nblk = n * (k // 32)
+        p = be.alloc_permanent(nblk * bb)
+        mr.adopt_device_buffer(p)
+        seed[0] += 1
+        rc = synth.vxs_gaussian_quant(fmt, p, nblk, 0.02, seed[0])
+        if rc != 0:
+            raise RuntimeError("vxs_gaussian_quant failed: %d" % rc)
+        return (fmt, p, n, k)
 
     h, qd, kvd, f, v = c["hidden"], c["num_heads"] * c["head_dim"], c["num_kv_heads"] * c["head_dim"], c["ffn"], c["vocab"]
-    ones = to_ours(torch.ones(h, device=dev, dtype=torch.float32))
+    ones = be.upload(np.ones(h, dtype=np.float32), permanent=True)
+    mr.adopt_device_buffer(ones)
     for l in range(layers):
         mr.set_layer(l, ones, ones, dict(wq=qw(qd, h), wk=qw(kvd, h), wv=qw(kvd, h), wo=qw(h, qd),
                                          w1=qw(f, h), w3=qw(f, h), w2=qw(h, f)))
@@ -99,17 +83,14 @@ def build_model(be, ctx, extra_tokens, layers):
     emb = be.alloc_permanent(v * h * 4)
     mr.adopt_device_buffer(emb)
     be.dequantize(lib.VX_Q8_0, emb_q[1], emb, v * h)     # loader rule: token_embd kept in F32
+    be.sync()
     mr.set_head(emb, ones, qw(v, h, lib.VX_Q8_0))
     # KV: every physical block of every layer holds N(0,1) halves
     per_block = 2 * BLOCK * kvd
     for l in range(layers):
-        chunk = 256
-        for b0 in range(0, need_blocks, chunk):
-            nb = min(chunk, need_blocks - b0)
-            t = torch.randn(nb * per_block, generator=g, device=dev, dtype=torch.float32).to(torch.float16)
-            torch.cuda.synchronize()
-            be.copy_buffer(t.data_ptr(), 0, mr.kv_pool(l), b0 * per_block * 2, nb * per_block * 2)
-            be.sync()
+        rc = synth.vxs_gaussian_f16(mr.kv_pool(l), need_blocks * per_block, 1.0, 1000 + l)
+        if rc != 0:
+            raise RuntimeError("vxs_gaussian_f16 failed: %d" % rc)
     rng = np.random.default_rng(0)
     perm = rng.permutation(need_blocks)
     ids, off = [], 0
@@ -119,8 +100,6 @@ def build_model(be, ctx, extra_tokens, layers):
         mr.adopt_blocks(i + 1, perm[off:off + nb], L)
         off += nb
         ids.append(i + 1)
-    del t
-    torch.cuda.empty_cache()
     return mr, ids
 
 

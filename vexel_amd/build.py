@@ -9,6 +9,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libvexel_hip.so")
 HOST_LIB = os.path.join(HERE, "libvexel_host.so")
+SYNTH_LIB = os.path.join(HERE, "libvexel_synth.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
 SOURCES = ["backend.hip", "elementwise.hip", "attention.hip", "qgemm.hip", "pack.hip"]
@@ -43,6 +44,13 @@ def build(verbose=True):
         raise RuntimeError("link failed:\n" + r.stderr)
     if verbose:
         print("built", LIB)
+    # benchmark support (synthetic weights / KV made on the device); not part of the C ABI
+    cmd = [HIPCC] + FLAGS + ["-shared", os.path.join(CSRC, "synth.hip"), "-o", SYNTH_LIB]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("synth build failed:\n" + r.stderr)
+    if verbose:
+        print("built", SYNTH_LIB)
     # host runtime: plain C++ above the C ABI (links the HIP library, finds it next to itself)
     cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I" + os.path.join(ROOT, "include"),
            os.path.join(HERE, "host", "runtime.cpp"), "-o", HOST_LIB, "-L" + HERE, "-lvexel_hip",
