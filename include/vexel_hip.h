@@ -142,6 +142,22 @@ int vx_dequantize(vx_backend *be, int fmt, const void *src, float *dst, int64_t 
 int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, float *out, const float *residual,
                     int m, int n, int k);
 
+/* "Prepare once, multiply many": the MFMA path consumes activations in a split, tiled f16 form
+ * kept in a backend-owned slot. A prepare call fills the slot from an [m,k] activation; every
+ * following vx_matmul_quant_prepared with the same (m,k) multiplies that activation by one more
+ * weight (Q/K/V share one, gate/up share one). k must be a multiple of 256 and pointers
+ * 16-byte aligned. Results equal vx_matmul_quant on the same values bit for bit.
+ *   vx_prepare_act       a itself
+ *   vx_rmsnorm_prepare   Backend.RMSNorm(x, weight) (backend.go:345); also stored to out when out != NULL
+ *   vx_silu_mul_prepare  Backend.SiLUMul(gate, up) (backend.go:360); also stored to out when out != NULL */
+int vx_prepare_act(vx_backend *be, const float *a, int m, int k);
+int vx_rmsnorm_prepare(vx_backend *be, const float *x, const float *weight, float *out, int rows, int cols, float eps);
+int vx_silu_mul_prepare(vx_backend *be, const float *gate, const float *up, float *out, int rows, int cols);
+int vx_matmul_quant_prepared(vx_backend *be, int fmt, const void *b, float *out, const float *residual, int m,
+                             int n, int k);
+/* 1 when (fmt, weight pointer alignment, k) can take the prepared MFMA path (Q4_0/Q8_0/Q4_K, k % 256 == 0). */
+int vx_matmul_quant_has_fast_path(int fmt, const void *b, int k);
+
 /* RoPE with one position per row (row r rotated as Backend.RoPE with seqLen=1,
  * startPos=positions[r]) fused with the paged scatter of K and V:
  * slot_mapping[r] = physBlock*blockSize + offset (runtime/gpu_block_pool.go:250-252).

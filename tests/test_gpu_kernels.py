@@ -115,6 +115,57 @@ def test_matmul_rows_independent_of_batch(be, fmt):
     be.reset_pool()
 
 
+def test_prepared_activation_paths(be):
+    """prepare-once / multiply-many equals the one-shot entry point bit for bit, and the fused
+    RMSNorm / SiLU*up prepares equal the separate ops."""
+    rng = np.random.default_rng(14)
+    m, n, k = 32, 160, 2048
+    a = (rng.standard_normal((m, k)) * 3).astype(np.float32)
+    wn = rng.standard_normal(k).astype(np.float32)
+    ws = {f: qz.random_quant(f, rng, n, k) for f in (nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q4_K)}
+    da, dwn = be.upload(a), be.upload(wn)
+    dws = {f: be.upload(w) for f, w in ws.items()}
+    d1, d2, dnorm = be.alloc(m * n * 4), be.alloc(m * n * 4), be.alloc(m * k * 4)
+    # plain prepare, three formats from one prepared activation
+    be.prepare_act(da, m, k)
+    for f in ws:
+        be.matmul_quant_prepared(f, dws[f], d1, None, m, n, k)
+        one = be.download(d1, (m, n), np.float32)
+        be.matmul_quant(f, da, dws[f], d2, None, m, n, k)
+        be.prepare_act(da, m, k)      # the one-shot call re-filled the slot; prepare again for the next format
+        assert np.array_equal(one.view(np.uint32), be.download(d2, (m, n), np.float32).view(np.uint32))
+    # fused rmsnorm + prepare
+    be.rmsnorm_prepare(da, dwn, dnorm, m, k, 1e-5)
+    want_norm = nx.rmsnorm(a, wn, m, k, 1e-5)
+    got_norm = be.download(dnorm, (m, k), np.float32)
+    _close(got_norm, want_norm, 2e-6, 1e-7, "rmsnorm_prepare f32 output")
+    be.matmul_quant_prepared(nx.FMT_Q4_0, dws[nx.FMT_Q4_0], d1, None, m, n, k)
+    got = be.download(d1, (m, n), np.float32)
+    want = nx.matmul_q4_0(want_norm, ws[nx.FMT_Q4_0], m, n, k)
+    _close(got, want, 3e-5, 3e-6 * np.abs(want).max(), "rmsnorm_prepare + matmul")
+    be.rmsnorm_prepare(da, dwn, None, m, k, 1e-5)     # no f32 copy: same prepared values
+    be.matmul_quant_prepared(nx.FMT_Q4_0, dws[nx.FMT_Q4_0], d2, None, m, n, k)
+    assert np.array_equal(got.view(np.uint32), be.download(d2, (m, n), np.float32).view(np.uint32))
+    # fused silu*up + prepare (staged and recomputing variants)
+    for kk in (2048, 14336):
+        g = (rng.standard_normal((3, kk)) * 2).astype(np.float32)
+        u = rng.standard_normal((3, kk)).astype(np.float32)
+        w2 = qz.random_quant(nx.FMT_Q4_0, rng, 48, kk)
+        dg, du, dw2 = be.upload(g), be.upload(u), be.upload(w2)
+        dact, do = be.alloc(3 * kk * 4), be.alloc(3 * 48 * 4)
+        be.silu_mul_prepare(dg, du, dact, 3, kk)
+        act = nx.silu_mul(g, u)
+        _close(be.download(dact, (3, kk), np.float32), act, 1e-6, 1e-9, "silu_mul_prepare f32 output")
+        be.matmul_quant_prepared(nx.FMT_Q4_0, dw2, do, None, 3, 48, kk)
+        want = nx.matmul_q4_0(act, w2, 3, 48, kk)
+        _close(be.download(do, (3, 48), np.float32), want, 3e-5, 3e-6 * np.abs(want).max(), "silu_mul_prepare + matmul")
+    # shape mismatch is an error, not a wrong answer
+    from vexel_amd.backend import VexelError
+    with pytest.raises(VexelError):
+        be.matmul_quant_prepared(nx.FMT_Q4_0, dws[nx.FMT_Q4_0], d1, None, m, n, 4096)
+    be.reset_pool()
+
+
 def test_matmul_quant_residual_and_shapes(be):
     rng = np.random.default_rng(11)
     for (m, n, k) in [(2, 33, 512), (32, 4096, 4096), (5, 100, 11008)]:

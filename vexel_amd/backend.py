@@ -209,6 +209,18 @@ class HipBackend:
     def matmul_quant(self, fmt, a, b, out, residual, m, n, k):
         self.call("vx_matmul_quant", fmt, a, b, out, residual, m, n, k)
 
+    def prepare_act(self, a, m, k):
+        self.call("vx_prepare_act", a, m, k)
+
+    def rmsnorm_prepare(self, x, weight, out, rows, cols, eps):
+        self.call("vx_rmsnorm_prepare", x, weight, out, rows, cols, eps)
+
+    def silu_mul_prepare(self, gate, up, out, rows, cols):
+        self.call("vx_silu_mul_prepare", gate, up, out, rows, cols)
+
+    def matmul_quant_prepared(self, fmt, b, out, residual, m, n, k):
+        self.call("vx_matmul_quant_prepared", fmt, b, out, residual, m, n, k)
+
     def rope_store_paged(self, q, k, v, positions, slot_mapping, kv_pool, pool_is_f16, rows, num_q_heads,
                          num_kv_heads, head_dim, block_size, theta):
         self.call("vx_rope_store_paged", q, k, v, positions, slot_mapping, kv_pool, int(bool(pool_is_f16)), rows,

@@ -88,6 +88,7 @@ void vx_backend_destroy(vx_backend *be) {
     for (auto &c : be->chunks) (void)hipFree(c.base);
     for (auto &kv : be->permanent) (void)hipFree(kv.first);
     if (be->gemm_ws) (void)hipFree(be->gemm_ws);
+    if (be->part_ws) (void)hipFree(be->part_ws);
     if (be->attn_ws) (void)hipFree(be->attn_ws);
     if (be->misc_ws) (void)hipFree(be->misc_ws);
     if (be->host_stage) (void)hipHostFree(be->host_stage);

@@ -55,8 +55,11 @@ struct vx_backend {
     std::unordered_map<void *, size_t> permanent;
 
     // library-owned scratch, grown on demand outside graph capture
-    void *gemm_ws = nullptr;     // split activations for the quantized GEMM
+    void *gemm_ws = nullptr;     // prepared (split, tiled) activations for the quantized GEMM
     size_t gemm_ws_bytes = 0;
+    int prep_m = 0, prep_k = 0;  // shape of the activation currently prepared in gemm_ws
+    void *part_ws = nullptr;     // split-K partial sums
+    size_t part_ws_bytes = 0;
     void *attn_ws = nullptr;     // split-KV partial results
     size_t attn_ws_bytes = 0;
     void *misc_ws = nullptr;     // small device staging (pointer tables, argmax result)

@@ -113,6 +113,8 @@ template <bool F16>
 __global__ void rope_store_paged_kernel(float *q, const float *k, const float *v, const int32_t *positions,
                                         const int32_t *slot_mapping, void *pool, int num_q_heads, int num_kv_heads,
                                         int head_dim, int block_size, float theta) {
+    // grid = (rows, head groups); thread = (rotation pair j, head lane); heads are strided over
+    // head lanes and head groups so the float64 cos/sin of a pair is computed once per thread.
     int row = blockIdx.x;
     int half = head_dim / 2;
     int pos = positions[row];
@@ -122,13 +124,17 @@ __global__ void rope_store_paged_kernel(float *q, const float *k, const float *v
     size_t part = (size_t)block_size * hs;
     size_t kbase = (size_t)blk * 2 * part + (size_t)off * hs;
     size_t vbase = kbase + part;
-    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+    const int lanes = blockDim.x / half;              // head lanes per block (>= 1)
+    const int hl = threadIdx.x / half;
+    const int hstride = lanes * gridDim.y;
+    const int h0 = blockIdx.y * lanes + hl;
+    for (int j = threadIdx.x % half; j < half && hl < lanes; j += half) {
         RopeCS cs = rope_cs(pos, j, head_dim, theta);
         float *qr = q + (size_t)row * num_q_heads * head_dim;
-        for (int h = 0; h < num_q_heads; h++) rope_pair(qr[h * head_dim + 2 * j], qr[h * head_dim + 2 * j + 1], cs);
+        for (int h = h0; h < num_q_heads; h += hstride) rope_pair(qr[h * head_dim + 2 * j], qr[h * head_dim + 2 * j + 1], cs);
         const float *kr = k + (size_t)row * hs;
         const float *vr = v + (size_t)row * hs;
-        for (int h = 0; h < num_kv_heads; h++) {
+        for (int h = h0; h < num_kv_heads; h += hstride) {
             float a = kr[h * head_dim + 2 * j], b = kr[h * head_dim + 2 * j + 1];
             rope_pair(a, b, cs);
             float va = vr[h * head_dim + 2 * j], vb = vr[h * head_dim + 2 * j + 1];
@@ -426,13 +432,20 @@ int vx_rope_store_paged(vx_backend *be, float *q, const float *k, const float *v
     VX_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && block_size > 0 && num_q_heads > 0 && num_kv_heads > 0,
                "vx_rope_store_paged: bad shape");
     if (rows == 0) return VX_OK;
-    int threads = head_dim / 2 < 64 ? 64 : head_dim / 2;
+    VX_REQUIRE(head_dim <= 512, "vx_rope_store_paged: head_dim %d too large", head_dim);
+    const int half = head_dim / 2;
+    const int lanes = 256 / half > 0 ? 256 / half : 1;
+    const int threads = lanes * half;
+    const int max_heads = num_q_heads > num_kv_heads ? num_q_heads : num_kv_heads;
+    int groups = ceil_div(max_heads, lanes * 2);  // about two heads per thread
+    if (groups < 1) groups = 1;
+    dim3 grid(rows, groups);
     if (pool_is_f16)
-        rope_store_paged_kernel<true><<<rows, threads, 0, be->stream>>>(q, k, v, positions, slot_mapping, kv_pool,
+        rope_store_paged_kernel<true><<<grid, threads, 0, be->stream>>>(q, k, v, positions, slot_mapping, kv_pool,
                                                                         num_q_heads, num_kv_heads, head_dim,
                                                                         block_size, theta);
     else
-        rope_store_paged_kernel<false><<<rows, threads, 0, be->stream>>>(q, k, v, positions, slot_mapping, kv_pool,
+        rope_store_paged_kernel<false><<<grid, threads, 0, be->stream>>>(q, k, v, positions, slot_mapping, kv_pool,
                                                                          num_q_heads, num_kv_heads, head_dim,
                                                                          block_size, theta);
     VX_CHECK_LAUNCH();

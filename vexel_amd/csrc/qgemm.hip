@@ -1,19 +1,29 @@
 // Quantized matmul C[M,N] = A[M,K] * B^T with B in raw GGUF blocks (Q4_0, Q8_0, Q4_K, Q6_K).
 // Replaces QuantizedMatMul.MatMulQ4_0/Q4_K/Q6_K/Q8_0 (inference/backend/backend.go:47-81).
 //
-// Fast path (Q4_0, Q8_0, Q4_K; K a multiple of 256, 16-byte aligned rows):
-//   1. split_act_kernel scales every activation row by a power of two, splits it into
-//      hi = f16(x) and lo = f16(x - hi) (together ~22 significant bits, the float32 level)
-//      and stores both in the k-order the weight unpacking produces.
-//   2. qgemm_kernel: a workgroup owns 16*R weight rows; its 4 waves split K. A wave stages
-//      its rows' raw blocks from HBM into LDS with coalesced 16-byte loads, unpacks the
-//      integer codes to exact f16 values in registers, and feeds v_mfma_f32_16x16x32_f16
-//      twice per 32-element block (hi, lo). The block scale d is applied to the float32
-//      MFMA result, never to the f16 operand, so the weight values entering the sum are
-//      exactly the integers of the format. The 4 partial sums are added in wave order.
-//   Each output element depends only on its own activation row and weight row, and the
-//   arithmetic does not depend on M, so a row gives the same bits alone or in a batch
-//   (the property the reference keeps by looping M=1 kernels, backend/metal/backend.go:777-779).
+// Fast path (Q4_0, Q8_0, Q4_K; K a multiple of 256, 16-byte aligned rows), two phases:
+//
+//  1. prepare: every activation row is scaled by a power of two and split into
+//     hi = f16(x), lo = f16(x - hi) (together ~22 significant bits, the float32 level). Both are
+//     written as ready-made MFMA operand tiles A[kstep][mtile][hi|lo][lane][8]: lane (g, r) of
+//     tile `mtile` holds row 16*mtile + r and the eight k-slots 8g..8g+7 of 32-element block
+//     `kstep`. Slot p of a block holds element PERM[p], the order in which every format's
+//     unpacking produces its eight values per lane, so one prepared activation serves any weight
+//     format. RMSNorm and SiLU*up have fused prepare variants; a prepared activation can be
+//     multiplied by several weights (Q/K/V, gate/up).
+//  2. qgemm_kernel: a workgroup owns 64*R weight rows (a wave 16*R of them) and one K slice.
+//     Per 256-element chunk the workgroup copies the activation tiles (contiguous, coalesced)
+//     into LDS once for its 4 waves, each wave stages its rows' raw blocks into LDS with 16-byte
+//     loads, unpacks the integer codes to exact f16 values in registers and issues
+//     v_mfma_f32_16x16x32_f16 twice per block (hi, lo). The block scale multiplies the float32
+//     MFMA result, never the f16 operand, so the weights entering the sum are exactly the
+//     format's integers. With KS > 1 slices the partial sums go to scratch and
+//     qgemm_reduce_kernel adds them in slice order (deterministic), applies the row scale and
+//     the optional residual.
+//  Each output element depends only on its own activation row and weight row and the launch
+//  shape depends on (N, K) only, so a row gives the same bits alone or inside a batch (the
+//  property the reference keeps by looping M=1 kernels, backend/metal/backend.go:777-779).
+//
 // Fallback (Q6_K, odd shapes): one wave per output column, float32 FMAs on the exact
 // dequantised values.
 #include "common.h"
@@ -32,105 +42,158 @@ __device__ __forceinline__ float h2f(uint16_t h) {
     return (float)v;
 }
 
-// ---------------------------------------------------------------- k-order of the MFMA operand
-// perm[p] = element index (within a 32-element block) that sits in operand position p, where
-// position p = 8*g + j is slot j of lane group g. inv is the inverse.
-struct Perm32 {
-    int8_t inv[32];
+// Slot j of lane group g (operand position p = 8g+j) holds block element
+//   {4g, 4g+2, 16+4g, 16+4g+2, 4g+1, 4g+3, 16+4g+1, 16+4g+3}[j]:
+// a lane needs elements 4g..4g+3 and 16+4g..16+4g+3, i.e. two aligned float4 of the source row.
+
+// ---------------------------------------------------------------- activation prepare
+// Workspace layout (be->gemm_ws): tiles [K/32][Mpad/16][2][64] half8, then inv_scale[Mpad],
+// then bsum[K/32][Mpad] (block sums of the scaled row, for Q4_K's min term).
+struct PrepView {
+    half8 *tiles;
+    float *inv_scale;
+    float *bsum;
 };
 
-constexpr Perm32 make_inv_q4_0() {
-    Perm32 r{};
-    for (int g = 0; g < 4; g++) {
-        const int e[8] = {4 * g, 4 * g + 2, 16 + 4 * g, 16 + 4 * g + 2, 4 * g + 1, 4 * g + 3, 16 + 4 * g + 1, 16 + 4 * g + 3};
-        for (int j = 0; j < 8; j++) r.inv[e[j]] = (int8_t)(8 * g + j);
-    }
-    return r;
-}
-constexpr Perm32 make_inv_ident() {
-    Perm32 r{};
-    for (int i = 0; i < 32; i++) r.inv[i] = (int8_t)i;
-    return r;
-}
-constexpr Perm32 make_inv_q4_k() {
-    Perm32 r{};
-    const int o[8] = {0, 2, 1, 3, 4, 6, 5, 7};
-    for (int g = 0; g < 4; g++)
-        for (int j = 0; j < 8; j++) r.inv[8 * g + o[j]] = (int8_t)(8 * g + j);
-    return r;
-}
+__host__ __device__ inline size_t prep_tiles_bytes(int mpad, int k) { return (size_t)(k / 32) * (mpad / 16) * 2 * 64 * 16; }
 
-__constant__ Perm32 c_inv_q4_0 = make_inv_q4_0();
-__constant__ Perm32 c_inv_q8_0 = make_inv_ident();
-__constant__ Perm32 c_inv_q4_k = make_inv_q4_k();
+enum { PREP_PLAIN = 0, PREP_RMSNORM = 1, PREP_SILU_MUL = 2 };
 
-// ---------------------------------------------------------------- activation split
-// grid = Mpad rows, block = 256. Outputs: hi/lo [Mpad,K] f16 (permuted inside each 32-block),
-// inv_scale[Mpad], bsum[K/32][Mpad] (block sums of the scaled row; used by Q4_K's min term).
-__global__ void __launch_bounds__(256) split_act_kernel(const float *__restrict__ a, int M, int K, int fmt,
-                                                        _Float16 *__restrict__ hi, _Float16 *__restrict__ lo,
-                                                        float *__restrict__ inv_scale, float *__restrict__ bsum,
-                                                        int Mpad) {
-    __shared__ float sm[4];
+__device__ __forceinline__ float sigmoid_ref(float v) { return 1.0f / (1.0f + (float)exp((double)(-v))); }
+
+// grid = Mpad rows, block = 256.
+//   PREP_PLAIN:    y = a
+//   PREP_RMSNORM:  y = (a / rms) * w            (backend/cpu/cpu.go:200-220), optional f32 copy to `fout`
+//   PREP_SILU_MUL: y = (a*sigmoid(a)) * b       (backend/cpu/cpu.go:390-400), optional f32 copy to `fout`
+// STAGE: keep the row's output values in LDS between the two passes (K*4 bytes of dynamic LDS);
+// otherwise pass 2 recomputes them.
+template <int MODE, bool STAGE>
+__global__ void __launch_bounds__(256) prepare_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                      float *__restrict__ fout, int M, int K, float eps,
+                                                      PrepView pv, int Mpad) {
+    extern __shared__ __attribute__((aligned(16))) float ybuf[];
+    __shared__ float sm[8];
     const int r = blockIdx.x, tid = threadIdx.x;
-    const Perm32 *pm = fmt == VX_Q4_0 ? &c_inv_q4_0 : (fmt == VX_Q4_K ? &c_inv_q4_k : &c_inv_q8_0);
+    const int mtiles = Mpad / 16, mt = r >> 4, ln = r & 15;
+    const int npairs = K / 8;  // (kstep, g) pairs: 8 output slots each
     if (r >= M) {
-        for (int k = tid; k < K; k += 256) {
-            hi[(size_t)r * K + k] = (_Float16)0.f;
-            lo[(size_t)r * K + k] = (_Float16)0.f;
+        const half8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int p = tid; p < npairs; p += 256) {
+            const int ks = p >> 2, g = p & 3;
+            half8 *t = pv.tiles + ((size_t)(ks * mtiles + mt) * 2) * 64 + g * 16 + ln;
+            t[0] = z;
+            t[64] = z;
+            if (g == 0) pv.bsum[(size_t)ks * Mpad + r] = 0.f;
         }
-        for (int b = tid; b < K / 32; b += 256) bsum[(size_t)b * Mpad + r] = 0.f;
-        if (tid == 0) inv_scale[r] = 0.f;
+        if (tid == 0) pv.inv_scale[r] = 0.f;
         return;
     }
     const float *ar = a + (size_t)r * K;
-    float amax = 0.f;
-    for (int k = tid; k < K; k += 256) amax = fmaxf(amax, fabsf(ar[k]));
-    for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-    if ((tid & 63) == 0) sm[tid >> 6] = amax;
+    const float *br = (MODE == PREP_RMSNORM) ? b : (b ? b + (size_t)r * K : nullptr);
+    // pass 1: row statistics (SiLU*up values are staged in LDS for pass 2 when STAGE)
+    float amax = 0.f, ss = 0.f;
+    for (int k = tid * 4; k < K; k += 1024) {
+        const float4 x = *(const float4 *)(ar + k);
+        float y[4] = {x.x, x.y, x.z, x.w};
+        if (MODE == PREP_RMSNORM) {
+            ss += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+        } else if (MODE == PREP_SILU_MUL) {
+            const float4 u = *(const float4 *)(br + k);
+            y[0] = __fmul_rn(__fmul_rn(x.x, sigmoid_ref(x.x)), u.x);
+            y[1] = __fmul_rn(__fmul_rn(x.y, sigmoid_ref(x.y)), u.y);
+            y[2] = __fmul_rn(__fmul_rn(x.z, sigmoid_ref(x.z)), u.z);
+            y[3] = __fmul_rn(__fmul_rn(x.w, sigmoid_ref(x.w)), u.w);
+        }
+        if (STAGE && MODE == PREP_SILU_MUL) *(float4 *)(ybuf + k) = make_float4(y[0], y[1], y[2], y[3]);
+        if (MODE == PREP_RMSNORM) {
+            const float4 w = *(const float4 *)(br + k);
+            y[0] *= w.x; y[1] *= w.y; y[2] *= w.z; y[3] *= w.w;
+        }
+        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(y[0]), fabsf(y[1])), fmaxf(fabsf(y[2]), fabsf(y[3]))));
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+        ss += __shfl_xor(ss, off, 64);
+    }
+    if ((tid & 63) == 0) {
+        sm[tid >> 6] = amax;
+        sm[4 + (tid >> 6)] = ss;
+    }
     __syncthreads();
     amax = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
+    float rms = 1.f;
+    if (MODE == PREP_RMSNORM) {
+        ss = sm[4] + sm[5] + sm[6] + sm[7];
+        rms = (float)sqrt((double)(ss / (float)K + eps));
+        amax = amax / rms * 1.0001f;  // bound of |(x/rms)*w| up to rounding
+    }
     float s = 1.f, inv = 1.f;
     if (amax > 0.f && amax < INFINITY) {
         int ex;
-        (void)frexpf(amax, &ex);      // amax = f * 2^ex, f in [0.5,1)
-        s = ldexpf(1.f, 14 - ex);     // amax*s in [2^13, 2^14)
-        inv = ldexpf(1.f, ex - 14);
+        (void)frexpf(amax, &ex);   // amax = f * 2^ex, f in [0.5,1)
+        s = ldexpf(1.f, 13 - ex);  // amax*s in [2^12, 2^13): far from the f16 limit 65504
+        inv = ldexpf(1.f, ex - 13);
     }
-    if (tid == 0) inv_scale[r] = inv;
-    for (int k = tid; k < K; k += 256) {
-        float x = ar[k] * s;
-        _Float16 h = (_Float16)x;
-        _Float16 l = (_Float16)(x - (float)h);
-        size_t o = (size_t)r * K + (k & ~31) + pm->inv[k & 31];
-        hi[o] = h;
-        lo[o] = l;
-        // 32 consecutive threads hold one block (256 % 32 == 0 and K % 32 == 0)
-        float t = x;
-        for (int off = 16; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
-        if ((tid & 31) == 0) bsum[(size_t)(k >> 5) * Mpad + r] = t;
+    if (tid == 0) pv.inv_scale[r] = inv;
+    // pass 2: one (kstep, g) pair per iteration = elements 4g..4g+3 and 16+4g..16+4g+3 of the block
+    for (int p = tid; p < npairs; p += 256) {
+        const int ks = p >> 2, g = p & 3;
+        const int k0 = ks * 32 + 4 * g;
+        const float *src = (STAGE && MODE == PREP_SILU_MUL) ? ybuf : ar;
+        float4 xa = *(const float4 *)(src + k0), xb = *(const float4 *)(src + k0 + 16);
+        float ya[4] = {xa.x, xa.y, xa.z, xa.w}, yb[4] = {xb.x, xb.y, xb.z, xb.w};
+        if (MODE == PREP_RMSNORM) {
+            const float4 wa = *(const float4 *)(br + k0), wb = *(const float4 *)(br + k0 + 16);
+            const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                ya[i] = __fmul_rn(ya[i] / rms, wv[i]);
+                yb[i] = __fmul_rn(yb[i] / rms, wv[4 + i]);
+            }
+        } else if (MODE == PREP_SILU_MUL && !STAGE) {
+            const float4 ua = *(const float4 *)(br + k0), ub = *(const float4 *)(br + k0 + 16);
+            const float uv[8] = {ua.x, ua.y, ua.z, ua.w, ub.x, ub.y, ub.z, ub.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                ya[i] = __fmul_rn(__fmul_rn(ya[i], sigmoid_ref(ya[i])), uv[i]);
+                yb[i] = __fmul_rn(__fmul_rn(yb[i], sigmoid_ref(yb[i])), uv[4 + i]);
+            }
+        }
+        if (MODE != PREP_PLAIN && fout) {
+            *(float4 *)(fout + (size_t)r * K + k0) = make_float4(ya[0], ya[1], ya[2], ya[3]);
+            *(float4 *)(fout + (size_t)r * K + k0 + 16) = make_float4(yb[0], yb[1], yb[2], yb[3]);
+        }
+        // slots: {4g, 4g+2, 16+4g, 16+4g+2, 4g+1, 4g+3, 16+4g+1, 16+4g+3}
+        const float v[8] = {ya[0] * s, ya[2] * s, yb[0] * s, yb[2] * s, ya[1] * s, ya[3] * s, yb[1] * s, yb[3] * s};
+        half8 h, l;
+        float bs = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            h[i] = (_Float16)v[i];
+            l[i] = (_Float16)(v[i] - (float)h[i]);
+            bs += v[i];
+        }
+        half8 *t = pv.tiles + ((size_t)(ks * mtiles + mt) * 2) * 64 + g * 16 + ln;
+        t[0] = h;
+        t[64] = l;
+        // the 4 lanes g = 0..3 of one kstep are adjacent threads (p = 4*ks + g)
+        bs += __shfl_xor(bs, 1, 64);
+        bs += __shfl_xor(bs, 2, 64);
+        if (g == 0) pv.bsum[(size_t)ks * Mpad + r] = bs;
     }
 }
 
-// ---------------------------------------------------------------- format policies (fast path)
-// CHUNK_STEPS 32-element MFMA steps per staged chunk, CHUNK_BYTES raw bytes per row per chunk.
+// ---------------------------------------------------------------- weight unpacking per format
 __device__ __forceinline__ uint32_t lds_u32_unaligned(const uint8_t *p) {
     uintptr_t a = (uintptr_t)p;
     const uint32_t *w = (const uint32_t *)(a & ~(uintptr_t)3);
     return __builtin_amdgcn_alignbyte(w[1], w[0], (uint32_t)(a & 3));
-}
-
-__device__ __forceinline__ uint32_t as_u32(half2v v) {
-    uint32_t u;
-    __builtin_memcpy(&u, &v, 4);
-    return u;
 }
 __device__ __forceinline__ half2v as_h2(uint32_t u) {
     half2v v;
     __builtin_memcpy(&v, &u, 4);
     return v;
 }
-
 __device__ __forceinline__ half8 pack8(half2v a, half2v b, half2v c, half2v d) {
     half8 r;
     r[0] = a[0]; r[1] = a[1]; r[2] = b[0]; r[3] = b[1];
@@ -138,27 +201,27 @@ __device__ __forceinline__ half8 pack8(half2v a, half2v b, half2v c, half2v d) {
     return r;
 }
 
-struct StepW {   // what one MFMA step needs from the weights
-    half8 b;     // exact integer codes as f16
-    float d;     // multiplies the MFMA result
-    float dm;    // multiplies the activation block sum and is subtracted (Q4_K), else 0
+struct StepW {  // what one MFMA step needs from the weights
+    half8 b;    // exact integer codes as f16, in slot order
+    float d;    // multiplies the MFMA result
+    float dm;   // multiplies the activation block sum and is subtracted (Q4_K), else 0
 };
 
+// CHUNK_BYTES = raw bytes per weight row for 8 steps (256 elements); all are multiples of 16.
 struct PQ4_0 {
-    static constexpr int CHUNK_STEPS = 16, CHUNK_BYTES = 288;  // sixteen 18-byte blocks
+    static constexpr int CHUNK_BYTES = 144;
     static constexpr bool HAS_MIN = false;
-    static __device__ __forceinline__ size_t row_bytes(int K) { return (size_t)K / 32 * 18; }
+    static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 32 * 18; }
     static __device__ __forceinline__ StepW load(const uint8_t *row, int step, int g) {
         const uint8_t *blk = row + step * 18;
-        uint32_t w = lds_u32_unaligned(blk + 2 + 4 * g);
+        const uint32_t w = lds_u32_unaligned(blk + 2 + 4 * g);  // bytes 4g..4g+3
         const half2v off = {(_Float16)1032.f, (_Float16)1032.f};
         const uint32_t m = 0x000F000Fu, mg = 0x64006400u;
-        half2v x0 = as_h2((w & m) | mg) - off;          // bytes 0,2 low nibbles
-        half2v x1 = as_h2(((w >> 4) & m) | mg) - off;   // bytes 0,2 high nibbles
-        half2v x2 = as_h2(((w >> 8) & m) | mg) - off;   // bytes 1,3 low nibbles
-        half2v x3 = as_h2(((w >> 12) & m) | mg) - off;  // bytes 1,3 high nibbles
         StepW r;
-        r.b = pack8(x0, x1, x2, x3);
+        r.b = pack8(as_h2((w & m) | mg) - off,          // low nibbles of bytes 0,2  -> 4g, 4g+2
+                    as_h2(((w >> 4) & m) | mg) - off,   // high nibbles of bytes 0,2 -> 16+4g, 16+4g+2
+                    as_h2(((w >> 8) & m) | mg) - off,   // low nibbles of bytes 1,3  -> 4g+1, 4g+3
+                    as_h2(((w >> 12) & m) | mg) - off); // high nibbles of bytes 1,3 -> 16+4g+1, 16+4g+3
         r.d = h2f(*(const uint16_t *)blk);
         r.dm = 0.f;
         return r;
@@ -166,25 +229,20 @@ struct PQ4_0 {
 };
 
 struct PQ8_0 {
-    static constexpr int CHUNK_STEPS = 8, CHUNK_BYTES = 272;
+    static constexpr int CHUNK_BYTES = 272;
     static constexpr bool HAS_MIN = false;
-    static __device__ __forceinline__ size_t row_bytes(int K) { return (size_t)K / 32 * 34; }
+    static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 32 * 34; }
     static __device__ __forceinline__ StepW load(const uint8_t *row, int step, int g) {
         const uint8_t *blk = row + step * 34;
-        const uint8_t *p = blk + 2 + 8 * g;
-        uintptr_t a = (uintptr_t)p;
-        const uint32_t *w = (const uint32_t *)(a & ~(uintptr_t)3);
-        uint32_t sh = (uint32_t)(a & 3);
-        uint32_t w0 = __builtin_amdgcn_alignbyte(w[1], w[0], sh) ^ 0x80808080u;
-        uint32_t w1 = __builtin_amdgcn_alignbyte(w[2], w[1], sh) ^ 0x80808080u;
+        const uint32_t w0 = lds_u32_unaligned(blk + 2 + 4 * g) ^ 0x80808080u;       // elements 4g..4g+3
+        const uint32_t w1 = lds_u32_unaligned(blk + 2 + 16 + 4 * g) ^ 0x80808080u;  // elements 16+4g..
         const half2v off = {(_Float16)1152.f, (_Float16)1152.f};  // 1024 + 128
         const uint32_t c64 = 0x64646464u;
-        half2v x0 = as_h2(__builtin_amdgcn_perm(w0, c64, 0x00050004u)) - off;
-        half2v x1 = as_h2(__builtin_amdgcn_perm(w0, c64, 0x00070006u)) - off;
-        half2v x2 = as_h2(__builtin_amdgcn_perm(w1, c64, 0x00050004u)) - off;
-        half2v x3 = as_h2(__builtin_amdgcn_perm(w1, c64, 0x00070006u)) - off;
         StepW r;
-        r.b = pack8(x0, x1, x2, x3);
+        r.b = pack8(as_h2(__builtin_amdgcn_perm(w0, c64, 0x00060004u)) - off,   // bytes 0,2 of w0
+                    as_h2(__builtin_amdgcn_perm(w1, c64, 0x00060004u)) - off,   // bytes 0,2 of w1
+                    as_h2(__builtin_amdgcn_perm(w0, c64, 0x00070005u)) - off,   // bytes 1,3 of w0
+                    as_h2(__builtin_amdgcn_perm(w1, c64, 0x00070005u)) - off);  // bytes 1,3 of w1
         r.d = h2f(*(const uint16_t *)blk);
         r.dm = 0.f;
         return r;
@@ -192,22 +250,17 @@ struct PQ8_0 {
 };
 
 struct PQ4_K {
-    static constexpr int CHUNK_STEPS = 16, CHUNK_BYTES = 288;  // two 144-byte super-blocks
+    static constexpr int CHUNK_BYTES = 144;  // one super-block = 8 sub-blocks of 32
     static constexpr bool HAS_MIN = true;
-    static __device__ __forceinline__ size_t row_bytes(int K) { return (size_t)K / 256 * 144; }
-    static __device__ __forceinline__ StepW load(const uint8_t *row, int step, int g) {
-        const uint8_t *sb = row + (step >> 3) * 144;
-        const int j = step & 7, gr = j >> 1, hi = j & 1;
-        const uint32_t *qp = (const uint32_t *)(sb + 16 + 32 * gr + 8 * g);
-        uint32_t w0 = qp[0] >> (4 * hi), w1 = qp[1] >> (4 * hi);
+    static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 256 * 144; }
+    static __device__ __forceinline__ StepW load(const uint8_t *sb, int j, int g) {
+        const int gr = j >> 1, hi = j & 1;
+        const uint32_t *qp = (const uint32_t *)(sb + 16 + 32 * gr);
+        const uint32_t w0 = qp[g] >> (4 * hi), w1 = qp[4 + g] >> (4 * hi);  // elements 4g.. and 16+4g..
         const half2v off = {(_Float16)1024.f, (_Float16)1024.f};
         const uint32_t m = 0x000F000Fu, mg = 0x64006400u;
-        half2v x0 = as_h2((w0 & m) | mg) - off;         // bytes 0,2
-        half2v x1 = as_h2(((w0 >> 8) & m) | mg) - off;  // bytes 1,3
-        half2v x2 = as_h2((w1 & m) | mg) - off;         // bytes 4,6
-        half2v x3 = as_h2(((w1 >> 8) & m) | mg) - off;  // bytes 5,7
         const uint8_t *q = sb + 4;
-        uint32_t sc, mn;  // dequant.go:400-409
+        uint32_t sc, mn;  // pkg/gguf/dequant.go:400-409
         if (j < 4) {
             sc = q[j] & 63;
             mn = q[j + 4] & 63;
@@ -215,137 +268,155 @@ struct PQ4_K {
             sc = (q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4);
             mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
         }
-        uint32_t hd = *(const uint32_t *)sb;
+        const uint32_t hd = *(const uint32_t *)sb;
         StepW r;
-        r.b = pack8(x0, x1, x2, x3);
+        r.b = pack8(as_h2((w0 & m) | mg) - off, as_h2((w1 & m) | mg) - off, as_h2(((w0 >> 8) & m) | mg) - off,
+                    as_h2(((w1 >> 8) & m) | mg) - off);
         r.d = h2f((uint16_t)(hd & 0xFFFF)) * (float)sc;
         r.dm = h2f((uint16_t)(hd >> 16)) * (float)mn;
         return r;
     }
 };
 
-constexpr int PITCH_PAD = 16;
+constexpr int CH = 8;  // MFMA steps (32 elements each) per chunk
 
-// grid.x = ceil(N / (16*R)); block = 256 (4 waves, K split by chunk index mod 4).
-// MT = number of 16-row activation tiles processed per pass over the weights.
+// grid = (row groups of 64*R rows, KS k-slices, groups of MT activation tiles); block = 256.
 template <class F, int R, int MT>
-__global__ void __launch_bounds__(256) qgemm_kernel(const uint8_t *__restrict__ W, const _Float16 *__restrict__ ahi,
-                                                    const _Float16 *__restrict__ alo,
-                                                    const float *__restrict__ inv_scale,
-                                                    const float *__restrict__ bsum, float *__restrict__ out,
-                                                    const float *__restrict__ residual, int M, int Mpad, int N, int K) {
-    constexpr int ROWS = 16 * R;
-    constexpr int PITCH = F::CHUNK_BYTES + PITCH_PAD;
-    constexpr int PIECES = ROWS * (F::CHUNK_BYTES / 16);
-    constexpr int NL = (PIECES + 63) / 64;
-    constexpr int WAVE_LDS = ROWS * PITCH;
-    constexpr int RED_FLOATS = 4 * R * MT * 4 * 64;
-    constexpr int LDS_BYTES = (4 * WAVE_LDS > RED_FLOATS * 4) ? 4 * WAVE_LDS : RED_FLOATS * 4;
-    __shared__ __attribute__((aligned(16))) uint8_t smem[LDS_BYTES];
+__global__ void __launch_bounds__(256) qgemm_kernel(const uint8_t *__restrict__ W, PrepView pv,
+                                                    float *__restrict__ out, const float *__restrict__ residual,
+                                                    float *__restrict__ partial, int M, int Mpad, int N, int K,
+                                                    int slice_chunks) {
+    constexpr int ROWS_W = 16 * R;
+    constexpr int PITCH = F::CHUNK_BYTES + 32;  // (PITCH/4) % 8 == 4: 16 rows x 4 lane groups spread over all banks
+    constexpr int WPIECES = ROWS_W * (F::CHUNK_BYTES / 16);
+    constexpr int WNL = (WPIECES + 63) / 64;
+    constexpr int APIECES = CH * MT * 2 * 64;  // 16-byte pieces of one activation chunk
+    constexpr int ANL = APIECES / 256;
+    __shared__ __attribute__((aligned(16))) half8 a_lds[APIECES];
+    __shared__ __attribute__((aligned(16))) uint8_t w_lds[4][ROWS_W * PITCH];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int ln = lane & 15, g = lane >> 4;
-    const int n0 = blockIdx.x * ROWS;
+    const int n0 = blockIdx.x * (64 * R) + wave * ROWS_W;
+    const int ks = blockIdx.y, mg = blockIdx.z;
+    const int m0 = mg * 16 * MT;
+    const int mtiles = Mpad / 16;
     const size_t row_bytes = F::row_bytes(K);
     const int steps_total = K / 32;
-    const int n_chunks = (steps_total + F::CHUNK_STEPS - 1) / F::CHUNK_STEPS;
-    uint8_t *wl = smem + wave * WAVE_LDS;
+    const int n_chunks = (steps_total + CH - 1) / CH;
+    const int c_begin = ks * slice_chunks;
+    const int c_end = min(c_begin + slice_chunks, n_chunks);
 
-    for (int m0 = 0; m0 < Mpad; m0 += 16 * MT) {
-        float4v run[R][MT];
+    float4v run[R][MT];
 #pragma unroll
-        for (int r = 0; r < R; r++)
+    for (int r = 0; r < R; r++)
 #pragma unroll
-            for (int t = 0; t < MT; t++) run[r][t] = (float4v){0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < MT; t++) run[r][t] = (float4v){0.f, 0.f, 0.f, 0.f};
 
-        uint4 stage[NL];
-        auto fetch = [&](int chunk) {
-            const size_t coff = (size_t)chunk * F::CHUNK_BYTES;
-            const int valid_bytes = (int)min((size_t)F::CHUNK_BYTES, row_bytes - coff);
+    half8 a_stage[ANL];
+    uint4 w_stage[WNL];
+    auto fetch = [&](int chunk) {
+        const int s0 = chunk * CH;
+        const int nsteps = min(CH, steps_total - s0);
 #pragma unroll
-            for (int i = 0; i < NL; i++) {
-                int pc = i * 64 + lane;
-                int row = pc / (F::CHUNK_BYTES / 16), col = pc % (F::CHUNK_BYTES / 16);
-                int n = min(n0 + row, N - 1);
-                bool ok = pc < PIECES && col * 16 < valid_bytes;
-                stage[i] = ok ? *(const uint4 *)(W + (size_t)n * row_bytes + coff + col * 16) : make_uint4(0, 0, 0, 0);
+        for (int i = 0; i < ANL; i++) {
+            const int p = i * 256 + tid;              // (s, t, hl, l)
+            const int l = p & 63, hl = (p >> 6) & 1, t = (p >> 7) % MT, s = p / (128 * MT);
+            const half8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+            a_stage[i] = (s < nsteps) ? pv.tiles[((size_t)((s0 + s) * mtiles + mg * MT + t) * 2 + hl) * 64 + l] : z;
+        }
+        const size_t coff = (size_t)chunk * F::CHUNK_BYTES;
+        const int valid = (int)min((size_t)F::CHUNK_BYTES, row_bytes - coff);
+#pragma unroll
+        for (int i = 0; i < WNL; i++) {
+            const int pc = i * 64 + lane;
+            const int row = pc / (F::CHUNK_BYTES / 16), col = pc % (F::CHUNK_BYTES / 16);
+            const int n = min(n0 + row, N - 1);
+            const bool ok = pc < WPIECES && col * 16 < valid;
+            w_stage[i] = ok ? *(const uint4 *)(W + (size_t)n * row_bytes + coff + col * 16) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto commit = [&]() {
+#pragma unroll
+        for (int i = 0; i < ANL; i++) a_lds[i * 256 + tid] = a_stage[i];
+#pragma unroll
+        for (int i = 0; i < WNL; i++) {
+            const int pc = i * 64 + lane;
+            const int row = pc / (F::CHUNK_BYTES / 16), col = pc % (F::CHUNK_BYTES / 16);
+            if (pc < WPIECES) *(uint4 *)(&w_lds[wave][row * PITCH + col * 16]) = w_stage[i];
+        }
+    };
+
+    if (c_begin < c_end) fetch(c_begin);
+    for (int chunk = c_begin; chunk < c_end; chunk++) {
+        __syncthreads();  // previous chunk's reads are done
+        commit();
+        __syncthreads();
+        if (chunk + 1 < c_end) fetch(chunk + 1);  // in flight while this chunk is computed
+        const int s0 = chunk * CH;
+        const int nsteps = min(CH, steps_total - s0);
+        for (int s = 0; s < nsteps; s++) {
+            half8 ah[MT], al[MT];
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                ah[t] = a_lds[((s * MT + t) * 2 + 0) * 64 + lane];
+                al[t] = a_lds[((s * MT + t) * 2 + 1) * 64 + lane];
             }
-        };
-        auto commit = [&]() {
 #pragma unroll
-            for (int i = 0; i < NL; i++) {
-                int pc = i * 64 + lane;
-                int row = pc / (F::CHUNK_BYTES / 16), col = pc % (F::CHUNK_BYTES / 16);
-                if (pc < PIECES) *(uint4 *)(wl + row * PITCH + col * 16) = stage[i];
-            }
-        };
-
-        int chunk = wave;
-        if (chunk < n_chunks) fetch(chunk);
-        for (; chunk < n_chunks; chunk += 4) {
-            __builtin_amdgcn_wave_barrier();
-            commit();
-            __builtin_amdgcn_wave_barrier();
-            if (chunk + 4 < n_chunks) fetch(chunk + 4);
-            const int s0 = chunk * F::CHUNK_STEPS;
-            const int nsteps = min(F::CHUNK_STEPS, steps_total - s0);
-            for (int s = 0; s < nsteps; s++) {
-                const size_t koff = (size_t)(s0 + s) * 32 + 8 * g;
-                half8 ah[MT], al[MT];
+            for (int r = 0; r < R; r++) {
+                const StepW sw = F::load(&w_lds[wave][(r * 16 + ln) * PITCH], s, g);
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
-                    const size_t ro = (size_t)(m0 + t * 16 + ln) * K + koff;
-                    ah[t] = *(const half8 *)(ahi + ro);
-                    al[t] = *(const half8 *)(alo + ro);
-                }
+                    float4v acc = {0.f, 0.f, 0.f, 0.f};
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah[t], sw.b, acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(al[t], sw.b, acc, 0, 0, 0);
+                    if (F::HAS_MIN) {
+                        const float4v bs = *(const float4v *)(pv.bsum + (size_t)(s0 + s) * Mpad + m0 + t * 16 + 4 * g);
 #pragma unroll
-                for (int r = 0; r < R; r++) {
-                    StepW sw = F::load(wl + (r * 16 + ln) * PITCH, s, g);
+                        for (int i = 0; i < 4; i++) run[r][t][i] += sw.d * acc[i] - sw.dm * bs[i];
+                    } else {
 #pragma unroll
-                    for (int t = 0; t < MT; t++) {
-                        float4v acc = {0.f, 0.f, 0.f, 0.f};
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah[t], sw.b, acc, 0, 0, 0);
-                        acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(al[t], sw.b, acc, 0, 0, 0);
-                        if (F::HAS_MIN) {
-                            const float4v bs = *(const float4v *)(bsum + (size_t)(s0 + s) * Mpad + m0 + t * 16 + 4 * g);
-#pragma unroll
-                            for (int i = 0; i < 4; i++) run[r][t][i] += sw.d * acc[i] - sw.dm * bs[i];
-                        } else {
-#pragma unroll
-                            for (int i = 0; i < 4; i++) run[r][t][i] += sw.d * acc[i];
-                        }
+                        for (int i = 0; i < 4; i++) run[r][t][i] += sw.d * acc[i];
                     }
                 }
             }
         }
-
-        // cross-wave reduction in wave order, then scale back, add the residual, store
-        __syncthreads();
-        float *red = (float *)smem;
-#pragma unroll
-        for (int r = 0; r < R; r++)
-#pragma unroll
-            for (int t = 0; t < MT; t++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) red[((wave * R + r) * MT + t) * 256 + i * 64 + lane] = run[r][t][i];
-        __syncthreads();
-        for (int idx = tid; idx < R * MT * 256; idx += 256) {
-            const int rt = idx / 256, e = idx % 256, i = e / 64, l2 = e % 64;
-            const int r = rt / MT, t = rt % MT;
-            float v = red[(0 * R * MT + rt) * 256 + e];
-            v += red[(1 * R * MT + rt) * 256 + e];
-            v += red[(2 * R * MT + rt) * 256 + e];
-            v += red[(3 * R * MT + rt) * 256 + e];
-            const int m = m0 + t * 16 + 4 * (l2 >> 4) + i;
-            const int n = n0 + r * 16 + (l2 & 15);
-            if (m < M && n < N) {
-                v *= inv_scale[m];
-                if (residual) v = residual[(size_t)m * N + n] + v;
-                out[(size_t)m * N + n] = v;
-            }
-        }
-        __syncthreads();
     }
+
+    // lane (g, ln) of tile (r, t) holds C[m = m0 + 16t + 4g + i][n = n0 + 16r + ln], i = 0..3
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int m = m0 + t * 16 + 4 * g + i;
+                const int n = n0 + r * 16 + ln;
+                if (m < M && n < N) {
+                    if (partial) {
+                        partial[((size_t)ks * M + m) * N + n] = run[r][t][i];
+                    } else {
+                        float v = run[r][t][i] * pv.inv_scale[m];
+                        if (residual) v = residual[(size_t)m * N + n] + v;
+                        out[(size_t)m * N + n] = v;
+                    }
+                }
+            }
+}
+
+// out[m][n] = residual + inv_scale[m] * (P[0] + P[1] + ... + P[KS-1]) in that order.
+__global__ void __launch_bounds__(256) qgemm_reduce_kernel(const float *__restrict__ partial,
+                                                           const float *__restrict__ inv_scale,
+                                                           float *__restrict__ out, const float *__restrict__ residual,
+                                                           int M, int N, int KS) {
+    const size_t total = (size_t)M * N;
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    float v = partial[i];
+    for (int s = 1; s < KS; s++) v += partial[(size_t)s * total + i];
+    v *= inv_scale[i / N];
+    if (residual) v = residual[i] + v;
+    out[i] = v;
 }
 
 // ---------------------------------------------------------------- fallback: exact dequantised values, float32 FMAs
@@ -379,7 +450,7 @@ __device__ __forceinline__ float deq_elem(int fmt, const uint8_t *row, int k) {
         int qq = hi ? (bv >> 4) : (bv & 0xF);
         return __fsub_rn(__fmul_rn(d1, (float)qq), dm1);
     }
-    // Q6_K, dequant.go:272-331
+    // Q6_K, pkg/gguf/dequant.go:272-331
     const uint8_t *b = row + (size_t)(k >> 8) * 210;
     int e = k & 255, nn = e >> 7, r = e & 127, quad = r >> 5, l = r & 31, is = l >> 4;
     const uint8_t *ql = b + nn * 64, *qh = b + 128 + nn * 32;
@@ -430,68 +501,176 @@ size_t fmt_row_bytes(int fmt, int k) {
     return 0;
 }
 
-template <class F, int R>
-int launch_fast_r(vx_backend *be, const uint8_t *W, const _Float16 *hi, const _Float16 *lo, const float *inv,
-                  const float *bsum, float *out, const float *residual, int M, int Mpad, int N, int K) {
-    int grid = ceil_div(N, 16 * R);
-    if (Mpad <= 16)
-        qgemm_kernel<F, R, 1><<<grid, 256, 0, be->stream>>>(W, hi, lo, inv, bsum, out, residual, M, Mpad, N, K);
-    else
-        qgemm_kernel<F, R, 2><<<grid, 256, 0, be->stream>>>(W, hi, lo, inv, bsum, out, residual, M, Mpad, N, K);
-    VX_CHECK_LAUNCH();
+int mpad_for(int m) { return m <= 16 ? 16 : ceil_div(m, 32) * 32; }
+
+PrepView prep_view(vx_backend *be, int mpad, int k) {
+    PrepView pv;
+    char *base = (char *)be->gemm_ws;
+    pv.tiles = (half8 *)base;
+    pv.inv_scale = (float *)(base + prep_tiles_bytes(mpad, k));
+    pv.bsum = pv.inv_scale + ceil_div(mpad, 64) * 64;
+    return pv;
+}
+
+// Makes the prepared-activation workspace hold an [m,k] activation; returns its view.
+int prep_begin(vx_backend *be, int m, int k, PrepView *pv) {
+    VX_REQUIRE(m >= 1 && k >= 256 && k % 256 == 0, "prepare: bad shape %dx%d (K must be a multiple of 256)", m, k);
+    const int mpad = mpad_for(m);
+    const size_t need = prep_tiles_bytes(mpad, k) + (size_t)ceil_div(mpad, 64) * 64 * 4 + (size_t)(k / 32) * mpad * 4;
+    int rc = ensure_ws(be, &be->gemm_ws, &be->gemm_ws_bytes, need, "prepared activations");
+    if (rc) return rc;
+    *pv = prep_view(be, mpad, k);
+    be->prep_m = m;
+    be->prep_k = k;
     return VX_OK;
 }
 
 template <class F>
-int launch_fast(vx_backend *be, const uint8_t *W, const _Float16 *hi, const _Float16 *lo, const float *inv,
-                const float *bsum, float *out, const float *residual, int M, int Mpad, int N, int K) {
-    // more rows per wave reuse each activation fetch, but the launch still has to fill 256 CUs
-    if (N >= 16 * 2 * 512) return launch_fast_r<F, 2>(be, W, hi, lo, inv, bsum, out, residual, M, Mpad, N, K);
-    return launch_fast_r<F, 1>(be, W, hi, lo, inv, bsum, out, residual, M, Mpad, N, K);
+int launch_fast(vx_backend *be, const uint8_t *W, float *out, const float *residual, int M, int N, int K) {
+    const int mpad = mpad_for(M);
+    const PrepView pv = prep_view(be, mpad, K);
+    constexpr int R = 2;
+    const int rg = ceil_div(N, 64 * R);
+    const int mgroups = mpad <= 16 ? 1 : mpad / 32;
+    const int n_chunks = ceil_div(K / 32, CH);
+    // enough workgroups to fill 256 CUs, at least 2 chunks per slice; depends on (N, K) only when M <= 32
+    int ks = 1;
+    if (mgroups == 1) {
+        ks = ceil_div(512, rg);
+        if (ks > n_chunks / 2) ks = n_chunks / 2;
+        if (ks < 1) ks = 1;
+    }
+    const int slice = ceil_div(n_chunks, ks);
+    ks = ceil_div(n_chunks, slice);
+    float *partial = nullptr;
+    if (ks > 1) {
+        const size_t need = (size_t)ks * M * N * sizeof(float);
+        int rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, need, "split-K partial sums");
+        if (rc) return rc;
+        partial = (float *)be->part_ws;
+    }
+    dim3 grid(rg, ks, mgroups);
+    if (mpad <= 16)
+        qgemm_kernel<F, R, 1><<<grid, 256, 0, be->stream>>>(W, pv, out, residual, partial, M, mpad, N, K, slice);
+    else
+        qgemm_kernel<F, R, 2><<<grid, 256, 0, be->stream>>>(W, pv, out, residual, partial, M, mpad, N, K, slice);
+    VX_CHECK_LAUNCH();
+    if (ks > 1) {
+        const size_t total = (size_t)M * N;
+        qgemm_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>(partial, pv.inv_scale, out,
+                                                                                      residual, M, N, ks);
+        VX_CHECK_LAUNCH();
+    }
+    return VX_OK;
+}
+
+bool fast_ok(int fmt, const void *b, int k) {
+    const size_t rb = fmt_row_bytes(fmt, k);
+    return fmt != VX_Q6_K && (k % 256 == 0) && (rb % 16 == 0) && ((uintptr_t)b % 16 == 0);
+}
+
+int check_fmt(int fmt, int k) {
+    if (fmt != VX_Q4_0 && fmt != VX_Q8_0 && fmt != VX_Q4_K && fmt != VX_Q6_K) {
+        set_error("quantized matmul: unknown format %d", fmt);
+        return VX_ERR_UNSUPPORTED;
+    }
+    const int blk = (fmt == VX_Q4_0 || fmt == VX_Q8_0) ? 32 : 256;
+    VX_REQUIRE(k > 0 && k % blk == 0, "quantized matmul: K=%d is not a multiple of the block size %d", k, blk);
+    return VX_OK;
+}
+
+int run_prepared(vx_backend *be, int fmt, const void *b, float *out, const float *residual, int m, int n, int k) {
+    const uint8_t *W = (const uint8_t *)b;
+    switch (fmt) {
+    case VX_Q4_0: return launch_fast<PQ4_0>(be, W, out, residual, m, n, k);
+    case VX_Q8_0: return launch_fast<PQ8_0>(be, W, out, residual, m, n, k);
+    default: return launch_fast<PQ4_K>(be, W, out, residual, m, n, k);
+    }
 }
 
 }  // namespace
 
 extern "C" {
 
+int vx_prepare_act(vx_backend *be, const float *a, int m, int k) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(a && ((uintptr_t)a % 16 == 0), "vx_prepare_act: null or unaligned activation");
+    PrepView pv;
+    rc = prep_begin(be, m, k, &pv);
+    if (rc) return rc;
+    const int mpad = mpad_for(m);
+    prepare_kernel<PREP_PLAIN, false><<<mpad, 256, 0, be->stream>>>(a, nullptr, nullptr, m, k, 0.f, pv, mpad);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_rmsnorm_prepare(vx_backend *be, const float *x, const float *weight, float *out, int rows, int cols, float eps) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(x && weight && ((uintptr_t)x % 16 == 0) && ((uintptr_t)weight % 16 == 0) && ((uintptr_t)out % 16 == 0),
+               "vx_rmsnorm_prepare: null or unaligned pointer");
+    PrepView pv;
+    rc = prep_begin(be, rows, cols, &pv);
+    if (rc) return rc;
+    const int mpad = mpad_for(rows);
+    prepare_kernel<PREP_RMSNORM, false><<<mpad, 256, 0, be->stream>>>(x, weight, out, rows, cols, eps, pv, mpad);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_silu_mul_prepare(vx_backend *be, const float *gate, const float *up, float *out, int rows, int cols) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(gate && up && ((uintptr_t)gate % 16 == 0) && ((uintptr_t)up % 16 == 0) && ((uintptr_t)out % 16 == 0),
+               "vx_silu_mul_prepare: null or unaligned pointer");
+    PrepView pv;
+    rc = prep_begin(be, rows, cols, &pv);
+    if (rc) return rc;
+    const int mpad = mpad_for(rows);
+    if ((size_t)cols * 4 <= 48 * 1024)
+        prepare_kernel<PREP_SILU_MUL, true><<<mpad, 256, (size_t)cols * 4, be->stream>>>(gate, up, out, rows, cols, 0.f,
+                                                                                          pv, mpad);
+    else
+        prepare_kernel<PREP_SILU_MUL, false><<<mpad, 256, 0, be->stream>>>(gate, up, out, rows, cols, 0.f, pv, mpad);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_matmul_quant_prepared(vx_backend *be, int fmt, const void *b, float *out, const float *residual, int m, int n,
+                             int k) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(b && out && n >= 1, "vx_matmul_quant_prepared: bad arguments");
+    rc = check_fmt(fmt, k);
+    if (rc) return rc;
+    VX_REQUIRE(be->prep_m == m && be->prep_k == k, "vx_matmul_quant_prepared: the prepared activation is %dx%d, not %dx%d",
+               be->prep_m, be->prep_k, m, k);
+    VX_REQUIRE(fast_ok(fmt, b, k), "vx_matmul_quant_prepared: format %d / K=%d / alignment has no MFMA path", fmt, k);
+    return run_prepared(be, fmt, b, out, residual, m, n, k);
+}
+
+int vx_matmul_quant_has_fast_path(int fmt, const void *b, int k) { return fast_ok(fmt, b, k) ? 1 : 0; }
+
 int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, float *out, const float *residual, int m,
                     int n, int k) {
     int rc = enter(be);
     if (rc) return rc;
     VX_REQUIRE(a && b && out, "vx_matmul_quant: null pointer");
-    VX_REQUIRE(m >= 0 && n >= 0 && k > 0, "vx_matmul_quant: bad shape %dx%dx%d", m, n, k);
-    int blk = (fmt == VX_Q4_0 || fmt == VX_Q8_0) ? 32 : 256;
-    if (fmt != VX_Q4_0 && fmt != VX_Q8_0 && fmt != VX_Q4_K && fmt != VX_Q6_K) {
-        set_error("vx_matmul_quant: unknown format %d", fmt);
-        return VX_ERR_UNSUPPORTED;
-    }
-    VX_REQUIRE(k % blk == 0, "vx_matmul_quant: K=%d is not a multiple of the block size %d", k, blk);
+    VX_REQUIRE(m >= 0 && n >= 0, "vx_matmul_quant: bad shape %dx%dx%d", m, n, k);
+    rc = check_fmt(fmt, k);
+    if (rc) return rc;
     if (m == 0 || n == 0) return VX_OK;
-    const size_t rb = fmt_row_bytes(fmt, k);
-    const bool fast = fmt != VX_Q6_K && (k % 256 == 0) && (rb % 16 == 0) && ((uintptr_t)b % 16 == 0);
-    if (!fast) {
+    if (!fast_ok(fmt, b, k) || ((uintptr_t)a % 16) != 0) {
+        const size_t rb = fmt_row_bytes(fmt, k);
         dim3 grid(n, ceil_div(m, FB_M));
         qgemm_fallback_kernel<<<grid, 64, 0, be->stream>>>(fmt, (const uint8_t *)b, a, out, residual, m, n, k, rb);
         VX_CHECK_LAUNCH();
         return VX_OK;
     }
-    const int mpad = ceil_div(m, 16) * 16 <= 16 ? 16 : ceil_div(m, 32) * 32;
-    const size_t hl = (size_t)mpad * k * sizeof(_Float16);
-    const size_t need = 2 * hl + (size_t)mpad * 4 + (size_t)(k / 32) * mpad * 4 + 256;
-    rc = ensure_ws(be, &be->gemm_ws, &be->gemm_ws_bytes, need, "quantized matmul");
+    rc = vx_prepare_act(be, a, m, k);
     if (rc) return rc;
-    _Float16 *hi = (_Float16 *)be->gemm_ws;
-    _Float16 *lo = (_Float16 *)((char *)be->gemm_ws + hl);
-    float *inv = (float *)((char *)be->gemm_ws + 2 * hl);
-    float *bsum = inv + mpad + (64 - mpad % 64) % 64;  // keep 16-byte alignment for float4 loads
-    split_act_kernel<<<mpad, 256, 0, be->stream>>>(a, m, k, fmt, hi, lo, inv, bsum, mpad);
-    VX_CHECK_LAUNCH();
-    const uint8_t *W = (const uint8_t *)b;
-    switch (fmt) {
-    case VX_Q4_0: return launch_fast<PQ4_0>(be, W, hi, lo, inv, bsum, out, residual, m, mpad, n, k);
-    case VX_Q8_0: return launch_fast<PQ8_0>(be, W, hi, lo, inv, bsum, out, residual, m, mpad, n, k);
-    default: return launch_fast<PQ4_K>(be, W, hi, lo, inv, bsum, out, residual, m, mpad, n, k);
-    }
+    return run_prepared(be, fmt, b, out, residual, m, n, k);
 }
 
 int vx_matmul_q4_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k) {

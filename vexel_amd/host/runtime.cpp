@@ -180,9 +180,51 @@ int sync_pool_to_device(vh_model *m) {
     return VH_OK;
 }
 
-int matmul(vh_model *m, const float *a, const vh_qweight &w, float *out, const float *residual, int rows) {
+bool fast(const vh_qweight &w) { return vx_matmul_quant_has_fast_path(w.fmt, w.data, w.k) != 0; }
+
+// out = act * w^T (+ residual) where `act` is both in the backend's prepared slot (when `prepared`) and,
+// unless every consumer takes the prepared path, in float32 at a_f32.
+int mm(vh_model *m, bool prepared, const float *a_f32, const vh_qweight &w, float *out, const float *residual, int rows) {
     if (!w.data) return fail("weight not set");
-    VXC(vx_matmul_quant(m->be, w.fmt, a, w.data, out, residual, rows, w.n, w.k));
+    if (prepared && fast(w)) {
+        VXC(vx_matmul_quant_prepared(m->be, w.fmt, w.data, out, residual, rows, w.n, w.k));
+        return VH_OK;
+    }
+    VXC(vx_matmul_quant(m->be, w.fmt, a_f32, w.data, out, residual, rows, w.n, w.k));
+    return VH_OK;
+}
+
+// RMSNorm feeding the given weights: fused norm + prepare when any of them has the MFMA path.
+int norm_for(vh_model *m, const float *x, const float *nw, float *norm, int rows, const vh_qweight *const *ws, int nws,
+             bool *prepared) {
+    const vh_config &c = m->cfg;
+    int nfast = 0;
+    for (int i = 0; i < nws; i++) nfast += fast(*ws[i]) ? 1 : 0;
+    *prepared = nfast > 0 && c.hidden % 256 == 0;
+    if (*prepared)
+        VXC(vx_rmsnorm_prepare(m->be, x, nw, nfast == nws ? nullptr : norm, rows, c.hidden, c.eps));
+    else
+        VXC(vx_rmsnorm(m->be, x, nw, norm, rows, c.hidden, c.eps));
+    return VH_OK;
+}
+
+// attention output -> Wo (+x), FFN norm, gate/up, SiLU*up, down (+x): block.go:981-1077, shared by decode and prefill
+int layer_tail(vh_model *m, const vh_layer_weights &w, float *x, float *norm, const float *attn, float *gate, float *up,
+               int rows) {
+    const vh_config &c = m->cfg;
+    VHC(mm(m, false, attn, w.wo, x, x, rows));                                            // block.go:981-990
+    bool prep;
+    const vh_qweight *w13[2] = {&w.w1, &w.w3};
+    VHC(norm_for(m, x, w.ffn_norm, norm, rows, w13, 2, &prep));                           // block.go:996-998
+    VHC(mm(m, prep, norm, w.w1, gate, nullptr, rows));                                    // block.go:1043-1050
+    VHC(mm(m, prep, norm, w.w3, up, nullptr, rows));
+    if (fast(w.w2) && c.ffn % 256 == 0) {                                                 // block.go:1056-1077
+        VXC(vx_silu_mul_prepare(m->be, gate, up, nullptr, rows, c.ffn));
+        VHC(mm(m, true, nullptr, w.w2, x, x, rows));
+    } else {
+        VXC(vx_silu_mul(m->be, gate, up, gate, rows * c.ffn));
+        VHC(mm(m, false, gate, w.w2, x, x, rows));
+    }
     return VH_OK;
 }
 
@@ -191,22 +233,18 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len) {
     const vh_config &c = m->cfg;
     const vh_layer_weights &w = m->layers[layer];
     const float scale = (float)(1.0 / sqrt((double)c.head_dim));                          // block.go:862
-    VXC(vx_rmsnorm(m->be, m->x, w.attn_norm, m->norm, rows, c.hidden, c.eps));            // block.go:834-837
-    VHC(matmul(m, m->norm, w.wq, m->q, nullptr, rows));                                   // block.go:841-854
-    VHC(matmul(m, m->norm, w.wk, m->k, nullptr, rows));
-    VHC(matmul(m, m->norm, w.wv, m->v, nullptr, rows));
+    bool prep;
+    const vh_qweight *qkv[3] = {&w.wq, &w.wk, &w.wv};
+    VHC(norm_for(m, m->x, w.attn_norm, m->norm, rows, qkv, 3, &prep));                    // block.go:834-837
+    VHC(mm(m, prep, m->norm, w.wq, m->q, nullptr, rows));                                 // block.go:841-854
+    VHC(mm(m, prep, m->norm, w.wk, m->k, nullptr, rows));
+    VHC(mm(m, prep, m->norm, w.wv, m->v, nullptr, rows));
     VXC(vx_rope_store_paged(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
                             c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta));  // :858, :868
     VXC(vx_sdpa_paged_decode_ragged(m->be, m->q, m->kv[layer], c.kv_fp16, m->d_tables, m->d_slots, m->d_kv_lens,
                                     m->attn, rows, c.max_blocks_per_seq, c.block_size, c.num_heads, c.num_kv_heads,
                                     c.head_dim, scale, max_kv_len));                       // block.go:872
-    VHC(matmul(m, m->attn, w.wo, m->x, m->x, rows));                                      // block.go:981-990
-    VXC(vx_rmsnorm(m->be, m->x, w.ffn_norm, m->norm, rows, c.hidden, c.eps));             // block.go:996-998
-    VHC(matmul(m, m->norm, w.w1, m->gate, nullptr, rows));                                // block.go:1043-1050
-    VHC(matmul(m, m->norm, w.w3, m->up, nullptr, rows));
-    VXC(vx_silu_mul(m->be, m->gate, m->up, m->gate, rows * c.ffn));                       // block.go:1056
-    VHC(matmul(m, m->gate, w.w2, m->x, m->x, rows));                                      // block.go:1058-1077
-    return VH_OK;
+    return layer_tail(m, w, m->x, m->norm, m->attn, m->gate, m->up, rows);
 }
 
 // embedding -> layers -> final norm -> lm_head -> argmax for a decode batch (decode.go:404-452)
@@ -214,8 +252,10 @@ int forward_decode(vh_model *m, int rows, int max_kv_len) {
     const vh_config &c = m->cfg;
     VXC(vx_embedding(m->be, m->d_tokens, rows, m->embedding, m->x, c.vocab, c.hidden));
     for (int l = 0; l < c.num_layers; l++) VHC(execute_layer_decode(m, l, rows, max_kv_len));
-    VXC(vx_rmsnorm(m->be, m->x, m->final_norm, m->norm, rows, c.hidden, c.eps));           // model.go:207-226
-    VHC(matmul(m, m->norm, m->lm_head, m->logits, nullptr, rows));                        // model.go:352-422
+    bool prep;
+    const vh_qweight *hw[1] = {&m->lm_head};
+    VHC(norm_for(m, m->x, m->final_norm, m->norm, rows, hw, 1, &prep));                    // model.go:207-226
+    VHC(mm(m, prep, m->norm, m->lm_head, m->logits, nullptr, rows));                      // model.go:352-422
     VXC(vx_argmax_rows(m->be, m->logits, rows, c.vocab, m->d_next));
     return VH_OK;
 }
@@ -546,10 +586,12 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
     const float scale = (float)(1.0 / sqrt((double)c.head_dim));
     for (int l = 0; l < c.num_layers; l++) {
         const vh_layer_weights &w = m->layers[l];
-        VXC(vx_rmsnorm(be, x, w.attn_norm, norm, n, c.hidden, c.eps));
-        VHC(matmul(m, norm, w.wq, q, nullptr, n));
-        VHC(matmul(m, norm, w.wk, k, nullptr, n));
-        VHC(matmul(m, norm, w.wv, v, nullptr, n));
+        bool prep;
+        const vh_qweight *qkv[3] = {&w.wq, &w.wk, &w.wv};
+        VHC(norm_for(m, x, w.attn_norm, norm, n, qkv, 3, &prep));
+        VHC(mm(m, prep, norm, w.wq, q, nullptr, n));
+        VHC(mm(m, prep, norm, w.wk, k, nullptr, n));
+        VHC(mm(m, prep, norm, w.wv, v, nullptr, n));
         VXC(vx_rope(be, q, k, c.head_dim, c.num_heads, c.num_kv_heads, n, start_pos, 0, c.rope_theta, 0));  // block.go:858
         if (c.kv_fp16) {                                                               // gpu_block_pool.go:262-272
             VXC(vx_reshape_paged_kv_f16(be, k, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 0));
@@ -573,16 +615,13 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
         } else {                                                                       // block.go:893-895
             VXC(vx_sdpa_prefill(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale));
         }
-        VHC(matmul(m, attn, w.wo, x, x, n));
-        VXC(vx_rmsnorm(be, x, w.ffn_norm, norm, n, c.hidden, c.eps));
-        VHC(matmul(m, norm, w.w1, gate, nullptr, n));
-        VHC(matmul(m, norm, w.w3, up, nullptr, n));
-        VXC(vx_silu_mul(be, gate, up, gate, n * c.ffn));
-        VHC(matmul(m, gate, w.w2, x, x, n));
+        VHC(layer_tail(m, w, x, norm, attn, gate, up, n));
     }
     const float *last = all_logits ? x : x + (size_t)(n - 1) * c.hidden;                // decode.go:1057-1066
-    VXC(vx_rmsnorm(be, last, m->final_norm, norm, out_rows, c.hidden, c.eps));
-    VHC(matmul(m, norm, m->lm_head, logits, nullptr, out_rows));
+    bool prep;
+    const vh_qweight *hw[1] = {&m->lm_head};
+    VHC(norm_for(m, last, m->final_norm, norm, out_rows, hw, 1, &prep));
+    VHC(mm(m, prep, norm, m->lm_head, logits, nullptr, out_rows));
     if (logits_out) VXC(vx_to_host(be, logits_out, logits, (size_t)out_rows * c.vocab * 4));
     VXC(vx_sync(be));
     return VH_OK;

@@ -57,6 +57,11 @@ SIGNATURES = {
     "vx_sdpa_paged_decode_multiquery": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),
     "vx_dequantize": (_i, [_vp, _i, _vp, _vp, _i64]),
     "vx_matmul_quant": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i]),
+    "vx_prepare_act": (_i, [_vp, _vp, _i, _i]),
+    "vx_rmsnorm_prepare": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f]),
+    "vx_silu_mul_prepare": (_i, [_vp, _vp, _vp, _vp, _i, _i]),
+    "vx_matmul_quant_prepared": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i]),
+    "vx_matmul_quant_has_fast_path": (_i, [_i, _vp, _i]),
     "vx_rope_store_paged": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f]),
     "vx_sdpa_paged_decode_ragged": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i]),
     "vx_sdpa_paged_tree": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),
