@@ -184,10 +184,12 @@ __global__ void __launch_bounds__(256) prepare_kernel(const float *__restrict__ 
 }
 
 // ---------------------------------------------------------------- weight unpacking per format
-__device__ __forceinline__ uint32_t lds_u32_unaligned(const uint8_t *p) {
-    uintptr_t a = (uintptr_t)p;
-    const uint32_t *w = (const uint32_t *)(a & ~(uintptr_t)3);
-    return __builtin_amdgcn_alignbyte(w[1], w[0], (uint32_t)(a & 3));
+// 4 bytes at byte offset `off` (any alignment) of an LDS array. Indexing the array keeps the access
+// in the LDS address space (ds_read2_b32); a pointer rebuilt from an integer would become a flat load.
+__device__ __forceinline__ uint32_t lds_u32_unaligned(const uint8_t *base, int off) {
+    const uint32_t *w = (const uint32_t *)base;
+    const int i = off >> 2;
+    return __builtin_amdgcn_alignbyte(w[i + 1], w[i], (uint32_t)(off & 3));
 }
 __device__ __forceinline__ half2v as_h2(uint32_t u) {
     half2v v;
@@ -212,9 +214,10 @@ struct PQ4_0 {
     static constexpr int CHUNK_BYTES = 144;
     static constexpr bool HAS_MIN = false;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 32 * 18; }
-    static __device__ __forceinline__ StepW load(const uint8_t *row, int step, int g) {
-        const uint8_t *blk = row + step * 18;
-        const uint32_t w = lds_u32_unaligned(blk + 2 + 4 * g);  // bytes 4g..4g+3
+    static __device__ __forceinline__ StepW load(const uint8_t *base, int row_off, int step, int g) {
+        const int bo = row_off + step * 18;
+        const uint8_t *blk = base + bo;
+        const uint32_t w = lds_u32_unaligned(base, bo + 2 + 4 * g);  // bytes 4g..4g+3
         const half2v off = {(_Float16)1032.f, (_Float16)1032.f};
         const uint32_t m = 0x000F000Fu, mg = 0x64006400u;
         StepW r;
@@ -232,10 +235,11 @@ struct PQ8_0 {
     static constexpr int CHUNK_BYTES = 272;
     static constexpr bool HAS_MIN = false;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 32 * 34; }
-    static __device__ __forceinline__ StepW load(const uint8_t *row, int step, int g) {
-        const uint8_t *blk = row + step * 34;
-        const uint32_t w0 = lds_u32_unaligned(blk + 2 + 4 * g) ^ 0x80808080u;       // elements 4g..4g+3
-        const uint32_t w1 = lds_u32_unaligned(blk + 2 + 16 + 4 * g) ^ 0x80808080u;  // elements 16+4g..
+    static __device__ __forceinline__ StepW load(const uint8_t *base, int row_off, int step, int g) {
+        const int bo = row_off + step * 34;
+        const uint8_t *blk = base + bo;
+        const uint32_t w0 = lds_u32_unaligned(base, bo + 2 + 4 * g) ^ 0x80808080u;       // elements 4g..4g+3
+        const uint32_t w1 = lds_u32_unaligned(base, bo + 2 + 16 + 4 * g) ^ 0x80808080u;  // elements 16+4g..
         const half2v off = {(_Float16)1152.f, (_Float16)1152.f};  // 1024 + 128
         const uint32_t c64 = 0x64646464u;
         StepW r;
@@ -253,7 +257,8 @@ struct PQ4_K {
     static constexpr int CHUNK_BYTES = 144;  // one super-block = 8 sub-blocks of 32
     static constexpr bool HAS_MIN = true;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 256 * 144; }
-    static __device__ __forceinline__ StepW load(const uint8_t *sb, int j, int g) {
+    static __device__ __forceinline__ StepW load(const uint8_t *base, int row_off, int j, int g) {
+        const uint8_t *sb = base + row_off;
         const int gr = j >> 1, hi = j & 1;
         const uint32_t *qp = (const uint32_t *)(sb + 16 + 32 * gr);
         const uint32_t w0 = qp[g] >> (4 * hi), w1 = qp[4 + g] >> (4 * hi);  // elements 4g.. and 16+4g..
@@ -364,7 +369,7 @@ __global__ void __launch_bounds__(256) qgemm_kernel(const uint8_t *__restrict__ 
             }
 #pragma unroll
             for (int r = 0; r < R; r++) {
-                const StepW sw = F::load(&w_lds[wave][(r * 16 + ln) * PITCH], s, g);
+                const StepW sw = F::load(&w_lds[wave][0], (r * 16 + ln) * PITCH, s, g);
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
                     float4v acc = {0.f, 0.f, 0.f, 0.f};
