@@ -158,6 +158,39 @@ int vx_matmul_quant_prepared(vx_backend *be, int fmt, const void *b, float *out,
 /* 1 when (fmt, weight pointer alignment, k) can take the prepared MFMA path (Q4_0/Q8_0/Q4_K, k % 256 == 0). */
 int vx_matmul_quant_has_fast_path(int fmt, const void *b, int k);
 
+/* Fused decode blocks (the reference's FusedOps idea, backend.go:128-158, re-cut for the batched
+ * paged path). They compute what the unfused call sequence computes, with each projection group
+ * (Q|K|V, gate|up) as one launch and the split-K partial sums consumed directly by the next stage
+ * instead of being reduced, stored and re-read. Results are deterministic and independent of the
+ * batch a row sits in; against the unfused sequence they differ only by the float32 summation order
+ * of the split-K slices (a group is sliced by its summed width). *_supported() is 1 when the weights allow it (same format within a group,
+ * MFMA path available, rows of 16, widths that are multiples of 256 and fit one workgroup's LDS);
+ * otherwise the entry points return VX_ERR_UNSUPPORTED before doing anything. */
+typedef struct vx_qweight {
+    int fmt;          /* VX_Q4_0 ... */
+    const void *data; /* raw GGUF blocks on the device, [n,k] */
+    int n, k;
+} vx_qweight;
+
+/* RMSNorm(x, norm_weight) -> Q|K|V projections (one launch) -> RoPE at positions[r] -> rotated Q to
+ * q_out [rows,Hq*D], rotated K and V scattered into the pool at slot_mapping[r]
+ * (runtime/block.go:834-868). With x_prepared != 0 the normalised activation left prepared by the
+ * previous vx_decode_ffn (next_norm_weight) is used and x / norm_weight are ignored. */
+int vx_decode_attn_qkv_supported(const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int head_dim);
+int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight, float eps, int x_prepared,
+                       const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int rows,
+                       const int32_t *positions, const int32_t *slot_mapping, void *kv_pool, int pool_is_f16,
+                       int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta, float *q_out);
+
+/* x += attn*Wo^T; h = RMSNorm(x, ffn_norm_weight); x += (SiLU(h*W1^T) * (h*W3^T)) * W2^T
+ * (runtime/block.go:981-1077), x [rows,hidden] updated in place. When next_norm_weight != NULL,
+ * RMSNorm(x, next_norm_weight) of the updated x is left prepared for the next vx_decode_attn_qkv
+ * (x_prepared = 1) or vx_matmul_quant_prepared (the output head). */
+int vx_decode_ffn_supported(const vx_qweight *wo, const vx_qweight *w1, const vx_qweight *w3, const vx_qweight *w2);
+int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight *wo, const float *ffn_norm_weight,
+                  float eps, const vx_qweight *w1, const vx_qweight *w3, const vx_qweight *w2, int rows,
+                  const float *next_norm_weight);
+
 /* RoPE with one position per row (row r rotated as Backend.RoPE with seqLen=1,
  * startPos=positions[r]) fused with the paged scatter of K and V:
  * slot_mapping[r] = physBlock*blockSize + offset (runtime/gpu_block_pool.go:250-252).

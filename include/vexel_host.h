@@ -30,11 +30,7 @@ typedef struct vh_config {
     int kv_fp16;             /* 1 = F16 pool (runtime/model.go:311), 0 = F32 */
 } vh_config;
 
-typedef struct vh_qweight {  /* tensor.Tensor with a QuantProfile: raw GGUF blocks on the device */
-    int fmt;                 /* VX_Q4_0 ... */
-    const void *data;
-    int n, k;
-} vh_qweight;
+typedef vx_qweight vh_qweight;  /* tensor.Tensor with a QuantProfile: raw GGUF blocks on the device */
 
 typedef struct vh_layer_weights {  /* the BlockRuntime fields used by ExecuteWithPagedKV */
     const float *attn_norm, *ffn_norm;
@@ -49,6 +45,10 @@ const char *vh_last_error(void);
  * KV pool, the device mirror of the block tables and the activation buffers. */
 int vh_model_create(vx_backend *be, const vh_config *cfg, vh_model **out);
 void vh_model_destroy(vh_model *m);
+/* Decode uses vx_decode_attn_qkv / vx_decode_ffn wherever they support the weights (default on).
+ * Off = the one-call-per-operation sequence of runtime/block.go; the two agree to float32
+ * summation order. */
+void vh_model_set_fused(vh_model *m, int on);
 int vh_model_set_layer(vh_model *m, int layer, const vh_layer_weights *w);
 /* embedding: F32 [vocab,hidden] on the device (loader rule, runtime/loader.go:275-288) */
 int vh_model_set_head(vh_model *m, const float *embedding, const float *final_norm, const vh_qweight *lm_head);

@@ -166,6 +166,100 @@ def test_prepared_activation_paths(be):
     be.reset_pool()
 
 
+@pytest.mark.parametrize("fmt,rows,hidden,ffn", [(nx.FMT_Q4_0, 1, 512, 1024), (nx.FMT_Q4_0, 32, 512, 14336),
+                                                 (nx.FMT_Q8_0, 5, 512, 1024), (nx.FMT_Q4_K, 40, 1024, 2048)])
+def test_fused_decode_blocks_equal_the_unfused_sequence(be, fmt, rows, hidden, ffn):
+    """vx_decode_attn_qkv / vx_decode_ffn give what the one-call-per-operation sequence of
+    runtime/block.go:834-1077 gives (float32 activations, F16 and F32 pools), including the chained
+    prepared activation for the next block. A fused projection group is one launch over the summed
+    width, so its split-K slices differ from the separate launches': values agree to float32 summation
+    order (1e-5 of the row magnitude), not bit for bit; a chained call equals a fresh one exactly."""
+    rng = np.random.default_rng(77 + rows)
+    hq, hk, d, bs, nblocks, eps, theta = hidden // 64, 2, 64, 16, 24, 1e-5, 10000.0
+    kvd = hk * d
+    W = {name: qz.random_quant(fmt, rng, n, k) for name, (n, k) in
+         dict(wq=(hidden, hidden), wk=(kvd, hidden), wv=(kvd, hidden), wo=(hidden, hidden), w1=(ffn, hidden),
+              w3=(ffn, hidden), w2=(hidden, ffn)).items()}
+    dims = dict(wq=(hidden, hidden), wk=(kvd, hidden), wv=(kvd, hidden), wo=(hidden, hidden), w1=(ffn, hidden),
+                w3=(ffn, hidden), w2=(hidden, ffn))
+    dW = {n: be.upload(w) for n, w in W.items()}
+    qw = {n: be.qweight(fmt, dW[n], *dims[n]) for n in W}
+    assert be.decode_attn_qkv_supported(qw["wq"], qw["wk"], qw["wv"], d)
+    assert be.decode_ffn_supported(qw["wo"], qw["w1"], qw["w3"], qw["w2"])
+    x = (rng.standard_normal((rows, hidden)) * 2).astype(np.float32)
+    n1, n2, n3 = (rng.standard_normal(hidden).astype(np.float32) for _ in range(3))
+    pos = rng.integers(0, 3000, rows).astype(np.int32)
+    slots = rng.permutation(nblocks * bs)[:rows].astype(np.int32)
+    dn1, dn2, dn3, dpos, dslots = (be.upload(a) for a in (n1, n2, n3, pos, slots))
+    f4 = lambda *shape: be.alloc(int(np.prod(shape)) * 4)
+    bits = lambda a: a.view(np.uint32) if a.dtype == np.float32 else a.view(np.uint16)
+
+    def near(got, want, what):
+        if got.dtype == np.uint16:   # F16 pool: the float32 values differ in the last bits, so allow the f16 neighbour
+            g, w = nx.f16_to_f32_array(got), nx.f16_to_f32_array(want)
+            assert np.all(np.abs(g - w) <= np.abs(w) * 2.0 ** -10 + 1e-4), what
+            assert np.mean(got != want) < 2e-2, what
+        else:
+            assert np.all(np.abs(got - want) <= 2e-5 * np.abs(want).max() + 1e-6), \
+                "%s: %g" % (what, np.abs(got - want).max())
+    for f16 in (True, False):
+        pool = _make_pool(rng, f16, nblocks, bs, hk, d)
+        # ---- unfused
+        dx, dpool = be.upload(x), be.upload(pool)
+        dq, dk, dv, dg, du = f4(rows, hidden), f4(rows, kvd), f4(rows, kvd), f4(rows, ffn), f4(rows, ffn)
+        be.rmsnorm_prepare(dx, dn1, None, rows, hidden, eps)
+        for name, out in (("wq", dq), ("wk", dk), ("wv", dv)):
+            be.matmul_quant_prepared(fmt, dW[name], out, None, rows, dims[name][0], hidden)
+        be.rope_store_paged(dq, dk, dv, dpos, dslots, dpool, f16, rows, hq, hk, d, bs, theta)
+        q_ref = be.download(dq, (rows, hidden), np.float32)
+        pool_ref = be.download(dpool, pool.shape, pool.dtype)
+        attn = (rng.standard_normal((rows, hidden))).astype(np.float32)   # stands in for the attention output
+        dattn = be.upload(attn)
+        be.matmul_quant(fmt, dattn, dW["wo"], dx, dx, rows, hidden, hidden)
+        be.rmsnorm_prepare(dx, dn2, None, rows, hidden, eps)
+        be.matmul_quant_prepared(fmt, dW["w1"], dg, None, rows, ffn, hidden)
+        be.matmul_quant_prepared(fmt, dW["w3"], du, None, rows, ffn, hidden)
+        be.silu_mul_prepare(dg, du, None, rows, ffn)
+        be.matmul_quant_prepared(fmt, dW["w2"], dx, dx, rows, hidden, ffn)
+        x_ref = be.download(dx, (rows, hidden), np.float32)
+        be.rmsnorm_prepare(dx, dn3, None, rows, hidden, eps)
+        be.matmul_quant_prepared(fmt, dW["wk"], dk, None, rows, kvd, hidden)
+        next_ref = be.download(dk, (rows, kvd), np.float32)
+        # ---- fused, without and with the chained prepare
+        for chain in (False, True):
+            dx2, dpool2, dq2 = be.upload(x), be.upload(pool), f4(rows, hidden)
+            be.decode_attn_qkv(dx2, dn1, eps, False, qw["wq"], qw["wk"], qw["wv"], rows, dpos, dslots, dpool2, f16,
+                               hq, hk, d, bs, theta, dq2)
+            near(be.download(dq2, (rows, hidden), np.float32), q_ref, "q")
+            near(be.download(dpool2, pool.shape, pool.dtype), pool_ref, "pool")
+            be.decode_ffn(dattn, dx2, qw["wo"], dn2, eps, qw["w1"], qw["w3"], qw["w2"], rows, dn3 if chain else None)
+            near(be.download(dx2, (rows, hidden), np.float32), x_ref, "x after the block")
+            if chain:
+                be.matmul_quant_prepared(fmt, dW["wk"], dk, None, rows, kvd, hidden)
+                near(be.download(dk, (rows, kvd), np.float32), next_ref, "projection of the chained activation")
+                # and the next block's attention half accepts the chained activation
+                be.decode_ffn(dattn, dx2, qw["wo"], dn2, eps, qw["w1"], qw["w3"], qw["w2"], rows, dn1)
+                dx3 = be.upload(be.download(dx2, (rows, hidden), np.float32))
+                dq3, dq4, dpool3, dpool4 = f4(rows, hidden), f4(rows, hidden), be.upload(pool), be.upload(pool)
+                be.decode_attn_qkv(0, 0, eps, True, qw["wq"], qw["wk"], qw["wv"], rows, dpos, dslots, dpool3, f16,
+                                   hq, hk, d, bs, theta, dq3)
+                be.decode_attn_qkv(dx3, dn1, eps, False, qw["wq"], qw["wk"], qw["wv"], rows, dpos, dslots, dpool4, f16,
+                                   hq, hk, d, bs, theta, dq4)
+                assert np.array_equal(bits(be.download(dq3, (rows, hidden), np.float32)),
+                                      bits(be.download(dq4, (rows, hidden), np.float32)))
+                assert np.array_equal(bits(be.download(dpool3, pool.shape, pool.dtype)),
+                                      bits(be.download(dpool4, pool.shape, pool.dtype)))
+            else:
+                from vexel_amd.backend import VexelError
+                with pytest.raises(VexelError):   # nothing was left prepared
+                    be.decode_attn_qkv(0, 0, eps, True, qw["wq"], qw["wk"], qw["wv"], rows, dpos, dslots, dpool2, f16,
+                                       hq, hk, d, bs, theta, dq2)
+    # mixed formats inside a group are refused, not mis-computed
+    other = be.qweight(nx.FMT_Q8_0 if fmt != nx.FMT_Q8_0 else nx.FMT_Q4_0, dW["wk"], kvd, hidden)
+    assert not be.decode_attn_qkv_supported(qw["wq"], other, qw["wv"], d)
+    be.reset_pool()
+
+
 def test_matmul_quant_residual_and_shapes(be):
     rng = np.random.default_rng(11)
     for (m, n, k) in [(2, 33, 512), (32, 4096, 4096), (5, 100, 11008)]:

@@ -101,6 +101,31 @@ def test_c2_batched_decode_ragged_paged(be):
     mr.close()
 
 
+def test_fused_and_unfused_runtime_give_identical_logits(be):
+    """The runtime's fused decode blocks and its one-call-per-operation sequence are the same function up
+    to the float32 summation order of the split-K slices: logits within 1e-3, same greedy tokens, over
+    several steps of a ragged batch (33 rows: more than one 16-row tile and a partial one)."""
+    cfg = om.ModelConfig(num_layers=3, hidden=1024, num_heads=16, num_kv_heads=4, head_dim=64, ffn=2816,
+                         vocab=4096)
+    rng0 = np.random.default_rng(21)
+    ctx = [int(x) for x in rng0.integers(5, 300, 33)]
+    runs = []
+    for fused in (True, False):
+        omodel, mr, rng = _ragged_setup(be, cfg, nx.FMT_Q4_0, nx.FMT_Q8_0, ctx, 23, pool_blocks=700)
+        mr.set_fused(fused)
+        ids = [100 + i for i in range(len(ctx))]
+        toks, pos, logs = rng.integers(0, cfg.vocab, len(ctx)).tolist(), list(ctx), []
+        for step in range(3):
+            got, am = mr.decode_with_paged_kv_batched(toks, ids, pos)
+            logs.append((got.copy(), [int(a) for a in am]))
+            toks, pos = [int(a) for a in am], [p + 1 for p in pos]
+        runs.append(logs)
+        mr.close()
+    for (a, ta), (b, tb) in zip(*runs):
+        assert np.abs(a - b).max() <= 1e-3 * max(1.0, np.abs(b).max())
+        assert ta == tb
+
+
 def test_device_driven_graph_decode_matches_host_driven(be):
     """The hipGraph-captured, device-packed greedy loop gives the same tokens as the host-driven
     step and as the oracle, and leaves the device block tables equal to the host's."""

@@ -13,6 +13,11 @@ import numpy as np
 from . import lib as _l
 
 
+class VxQWeight(C.Structure):
+    """vx_qweight of include/vexel_hip.h."""
+    _fields_ = [("fmt", C.c_int), ("data", C.c_void_p), ("n", C.c_int), ("k", C.c_int)]
+
+
 class VexelError(RuntimeError):
     def __init__(self, code, msg):
         super().__init__("vexel_hip error %d: %s" % (code, msg))
@@ -220,6 +225,27 @@ class HipBackend:
 
     def matmul_quant_prepared(self, fmt, b, out, residual, m, n, k):
         self.call("vx_matmul_quant_prepared", fmt, b, out, residual, m, n, k)
+
+    @staticmethod
+    def qweight(fmt, data, n, k):
+        """vx_qweight for the fused decode entry points (data: device pointer of the raw blocks)."""
+        return VxQWeight(fmt, data, n, k)
+
+    def decode_attn_qkv_supported(self, wq, wk, wv, head_dim):
+        return bool(self._lib.vx_decode_attn_qkv_supported(C.byref(wq), C.byref(wk), C.byref(wv), head_dim))
+
+    def decode_attn_qkv(self, x, norm_weight, eps, x_prepared, wq, wk, wv, rows, positions, slot_mapping, kv_pool,
+                        pool_is_f16, num_q_heads, num_kv_heads, head_dim, block_size, theta, q_out):
+        self.call("vx_decode_attn_qkv", x, norm_weight, eps, int(bool(x_prepared)), C.byref(wq), C.byref(wk),
+                  C.byref(wv), rows, positions, slot_mapping, kv_pool, int(bool(pool_is_f16)), num_q_heads,
+                  num_kv_heads, head_dim, block_size, theta, q_out)
+
+    def decode_ffn_supported(self, wo, w1, w3, w2):
+        return bool(self._lib.vx_decode_ffn_supported(C.byref(wo), C.byref(w1), C.byref(w3), C.byref(w2)))
+
+    def decode_ffn(self, attn, x, wo, ffn_norm_weight, eps, w1, w3, w2, rows, next_norm_weight=None):
+        self.call("vx_decode_ffn", attn, x, C.byref(wo), ffn_norm_weight, eps, C.byref(w1), C.byref(w3),
+                  C.byref(w2), rows, next_norm_weight)
 
     def rope_store_paged(self, q, k, v, positions, slot_mapping, kv_pool, pool_is_f16, rows, num_q_heads,
                          num_kv_heads, head_dim, block_size, theta):

@@ -166,37 +166,43 @@ __global__ void __launch_bounds__(GEN_THREADS) attn_generic_kernel(AttnParams p)
 }
 
 // --------------------------------------------------------------------------------------------
-// Hot path: ragged batched decode over an F16 paged pool.
+// Hot path: ragged batched decode over an F16 paged pool with 16-token blocks.
 //
 // grid = (num_kv_heads, splits, batch); block = 256 threads (4 waves).
 // A workgroup owns the tokens [split*TPW, min(kv_len,(split+1)*TPW)) of one (sequence, kv head)
 // and all G = Hq/Hkv query heads that share that kv head. A wave takes 16-token pool blocks
 // round-robin. Within a wave LPT = D/8 lanes hold one token's head vector (8 halves = 16 bytes
-// each), so one load instruction covers 64/LPT tokens.
+// each), so one load instruction covers TPI = 64/LPT tokens and a block needs NL = 16/TPI K loads
+// and as many V loads. The block id is wave-uniform (scalar load); all 2*NL loads of the next
+// block are in flight while the current block is reduced.
 // Partials (m, l, acc[D]) per (sequence, q head, split) go to a scratch buffer; paged_merge_kernel
 // combines the splits.
 constexpr int TPW = 512;  // tokens per workgroup
+constexpr int HOT_BS = 16;
 
 template <int D, int G>
 __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
-    const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *const *__restrict__ bt_ptrs,
-    const int32_t *__restrict__ bt_matrix, const int32_t *__restrict__ bt_rows, int max_blocks,
-    const int32_t *__restrict__ kv_lens,
-    float *__restrict__ partial, int num_q_heads, int num_kv_heads, int block_size, float scale, int max_splits) {
-    constexpr int LPT = D / 8;     // lanes per token
-    constexpr int TPI = 64 / LPT;  // tokens per load instruction
+    const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix,
+    const int32_t *__restrict__ bt_rows, int max_blocks, const int32_t *__restrict__ kv_lens,
+    float *__restrict__ partial, int num_q_heads, int num_kv_heads, float scale, int max_splits) {
+    constexpr int LPT = D / 8;       // lanes per token
+    constexpr int TPI = 64 / LPT;    // tokens per load instruction
+    constexpr int NL = HOT_BS / TPI; // load instructions per block and per K or V
+    typedef _Float16 half8 __attribute__((ext_vector_type(8)));
     const int kvh = blockIdx.x, split = blockIdx.y, seq = blockIdx.z;
     const int kv_len = kv_lens[seq];
     const int t_begin = split * TPW;
     if (t_begin >= kv_len) return;
     const int t_end = min(kv_len, t_begin + TPW);
-    const int32_t *bt = bt_ptrs ? bt_ptrs[seq] : bt_matrix + (size_t)(bt_rows ? bt_rows[seq] : seq) * max_blocks;
+    const int32_t *bt = bt_matrix + (size_t)(bt_rows ? bt_rows[seq] : seq) * max_blocks + t_begin / HOT_BS;
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int tl = lane / LPT;  // token slot within a load
     const int dl = lane % LPT;  // 8-element slice of the head vector
     const size_t hs = (size_t)num_kv_heads * D;
-    const size_t part = (size_t)block_size * hs;
+    const size_t part = (size_t)HOT_BS * hs;
+    const size_t lane_off = (size_t)tl * hs + (size_t)kvh * D + dl * 8;
 
     // query slices, pre-multiplied by scale*log2(e) so scores are in the exp2 domain
     float qf[G][8];
@@ -216,53 +222,60 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
         for (int e = 0; e < 8; e++) acc[g][e] = 0.f;
     }
 
-    // Token groups of U*TPI tokens, interleaved over the 4 waves. All 2*U loads of a group are
-    // issued before any arithmetic so each wave keeps 2*U KiB in flight.
-    constexpr int U = 4;
-    typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-    const int n_groups = (t_end - t_begin + U * TPI - 1) / (U * TPI);
-    for (int gi = wave; gi < n_groups; gi += 4) {
-        half8 kk[U], vv[U];
-        bool valid[U];
+    const int n_blocks = (t_end - t_begin + HOT_BS - 1) / HOT_BS;
+    half8 kk[NL], vv[NL], kn[NL], vn[NL];
+    auto issue = [&](int bi, half8 *kd, half8 *vd) {
+        const int blk = __builtin_amdgcn_readfirstlane(bt[bi]);
+        const _Float16 *base = pool + (size_t)blk * 2 * part + lane_off;
 #pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int tok = t_begin + (gi * U + u) * TPI + tl;
-            valid[u] = tok < t_end;
-            const int tk = valid[u] ? tok : t_end - 1;
-            const int blk = bt[tk / block_size];
-            const size_t base = (size_t)blk * 2 * part + (size_t)(tk % block_size) * hs + (size_t)kvh * D + dl * 8;
-            kk[u] = *(const half8 *)(pool + base);
-            vv[u] = *(const half8 *)(pool + base + part);
+        for (int u = 0; u < NL; u++) {
+            kd[u] = *(const half8 *)(base + (size_t)u * TPI * hs);
+            vd[u] = *(const half8 *)(base + part + (size_t)u * TPI * hs);
         }
+    };
+    if (wave < n_blocks) issue(wave, kn, vn);
+    for (int bi = wave; bi < n_blocks; bi += 4) {
+#pragma unroll
+        for (int u = 0; u < NL; u++) {
+            kk[u] = kn[u];
+            vv[u] = vn[u];
+        }
+        if (bi + 4 < n_blocks) issue(bi + 4, kn, vn);
+        __builtin_amdgcn_sched_barrier(0);
+        const int tok0 = t_begin + bi * HOT_BS + tl;
 #pragma unroll
         for (int g = 0; g < G; g++) {
-            float s[U];
+            float s[NL];
             float gm = -INFINITY;
 #pragma unroll
-            for (int u = 0; u < U; u++) {
+            for (int u = 0; u < NL; u++) {
                 float t = 0.f;
 #pragma unroll
                 for (int e = 0; e < 8; e++) t = fmaf(qf[g][e], (float)kk[u][e], t);
 #pragma unroll
                 for (int off = LPT / 2; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
-                s[u] = valid[u] ? t : -INFINITY;
+                s[u] = (tok0 + u * TPI < t_end) ? t : -INFINITY;
                 gm = fmaxf(gm, s[u]);
             }
-            // max over the token slots of the wave (every group has at least one valid token)
+            // max over the token slots of the wave (the block's first token is always valid)
 #pragma unroll
             for (int off = LPT; off < 64; off <<= 1) gm = fmaxf(gm, __shfl_xor(gm, off, 64));
             const float m_new = fmaxf(m_run[g], gm);
-            const float alpha = exp2f(m_run[g] - m_new);  // m_new is finite; exp2(-inf) = 0 on the first group
+            const float alpha = exp2f(m_run[g] - m_new);  // m_new is finite; exp2(-inf) = 0 on the first block
             m_run[g] = m_new;
             float lsum = 0.f;
 #pragma unroll
             for (int e = 0; e < 8; e++) acc[g][e] *= alpha;
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                const float pw = exp2f(s[u] - m_new);  // 0 for invalid tokens
+            for (int u = 0; u < NL; u++) {
+                const bool ok = tok0 + u * TPI < t_end;
+                const float pw = ok ? exp2f(s[u] - m_new) : 0.f;
                 lsum += pw;
 #pragma unroll
-                for (int e = 0; e < 8; e++) acc[g][e] = fmaf(pw, (float)vv[u][e], acc[g][e]);
+                for (int e = 0; e < 8; e++) {
+                    const float vf = ok ? (float)vv[u][e] : 0.f;  // slots past the end may hold anything
+                    acc[g][e] = fmaf(pw, vf, acc[g][e]);
+                }
             }
             l_run[g] = l_run[g] * alpha + lsum;
         }
@@ -314,6 +327,15 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     }
 }
 
+// Copies per-sequence block tables given as device pointers into a padded [batch, max_blocks] matrix.
+__global__ void gather_tables_kernel(const int32_t *const *bt_ptrs, const int32_t *seq_lens, int32_t *matrix,
+                                     int max_blocks, int block_size) {
+    const int seq = blockIdx.x;
+    const int nb = (seq_lens[seq] + block_size - 1) / block_size;
+    const int32_t *src = bt_ptrs[seq];
+    for (int i = threadIdx.x; i < max_blocks; i += blockDim.x) matrix[(size_t)seq * max_blocks + i] = i < nb ? src[i] : 0;
+}
+
 // grid = (num_q_heads, batch); block = D threads.
 template <int D>
 __global__ void __launch_bounds__(D) paged_merge_kernel(const float *__restrict__ partial,
@@ -336,18 +358,17 @@ __global__ void __launch_bounds__(D) paged_merge_kernel(const float *__restrict_
 }
 
 template <int D, int G>
-int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *const *bt_ptrs,
-               const int32_t *bt_matrix, const int32_t *bt_rows, int max_blocks, const int32_t *kv_lens, float *out,
-               int batch, int num_q_heads, int num_kv_heads, int block_size, float scale, int max_kv_len) {
+int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *bt_matrix, const int32_t *bt_rows,
+               int max_blocks, const int32_t *kv_lens, float *out, int batch, int num_q_heads, int num_kv_heads,
+               float scale, int max_kv_len) {
     int max_splits = ceil_div(max_kv_len, TPW);
     size_t need = (size_t)batch * num_q_heads * max_splits * (D + 2) * sizeof(float);
     int rc = ensure_ws(be, &be->attn_ws, &be->attn_ws_bytes, need, "attention");
     if (rc) return rc;
     dim3 grid(num_kv_heads, max_splits, batch);
-    paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_ptrs, bt_matrix,
-                                                                bt_rows, max_blocks, kv_lens, (float *)be->attn_ws,
-                                                                num_q_heads, num_kv_heads, block_size, scale,
-                                                                max_splits);
+    paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
+                                                                max_blocks, kv_lens, (float *)be->attn_ws, num_q_heads,
+                                                                num_kv_heads, scale, max_splits);
     VX_CHECK_LAUNCH();
     paged_merge_kernel<D><<<dim3(num_q_heads, batch), D, 0, be->stream>>>((const float *)be->attn_ws, kv_lens, out,
                                                                           num_q_heads, max_splits);
@@ -374,12 +395,11 @@ int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16
     VX_REQUIRE(block_size > 0 && max_kv_len > 0, "attention: bad block size / kv length");
     if (batch == 0) return VX_OK;
     const int G = num_q_heads / num_kv_heads;
-    const bool aligned = ((uintptr_t)pool % 16) == 0;
-#define VX_HOT(DD, GG)                                                                                            \
-    if (pool_is_f16 && aligned && head_dim == DD && G == GG)                                                      \
-        return launch_hot<DD, GG>(be, q, pool, bt_ptrs, bt_matrix, bt_rows, max_blocks, kv_lens, out, batch,       \
-                                  num_q_heads,                                                                      \
-                                  num_kv_heads, block_size, scale, max_kv_len);
+    const bool hot = pool_is_f16 && ((uintptr_t)pool % 16) == 0 && block_size == HOT_BS && bt_matrix && !bt_ptrs;
+#define VX_HOT(DD, GG)                                                                                         \
+    if (hot && head_dim == DD && G == GG)                                                                      \
+        return launch_hot<DD, GG>(be, q, pool, bt_matrix, bt_rows, max_blocks, kv_lens, out, batch, num_q_heads, \
+                                  num_kv_heads, scale, max_kv_len);
     VX_HOT(128, 1) VX_HOT(128, 2) VX_HOT(128, 4) VX_HOT(128, 8)
     VX_HOT(64, 1) VX_HOT(64, 2) VX_HOT(64, 4) VX_HOT(64, 8)
 #undef VX_HOT
@@ -502,9 +522,20 @@ int vx_sdpa_paged_decode_batched(vx_backend *be, const float *q, const void *kv_
     VX_CHECK_HIP(hipMemcpyAsync(dev, block_tables, pbytes, hipMemcpyHostToDevice, be->stream));
     VX_CHECK_HIP(hipMemcpyAsync(dev + pbytes, seq_lens, lbytes, hipMemcpyHostToDevice, be->stream));
     VX_CHECK_HIP(hipStreamSynchronize(be->stream));  // host arrays belong to the caller after return
-    return run_ragged(be, q, kv_pool, pool_is_f16, (const int32_t *const *)dev, nullptr, nullptr, max_blocks,
-                      (const int32_t *)(dev + pbytes), out, batch_size, block_size, num_q_heads, num_kv_heads,
-                      head_dim, scale, max_len);
+    const int32_t *d_lens = (const int32_t *)(dev + pbytes);
+    // gather the per-sequence tables into one padded matrix when it fits the staging buffer
+    const size_t moff = (pbytes + lbytes + 255) / 256 * 256;
+    const size_t mbytes = (size_t)batch_size * max_blocks * sizeof(int32_t);
+    if (max_blocks >= 1 && moff + mbytes <= be->misc_ws_bytes) {
+        int32_t *matrix = (int32_t *)(dev + moff);
+        gather_tables_kernel<<<batch_size, 256, 0, be->stream>>>((const int32_t *const *)dev, d_lens, matrix, max_blocks,
+                                                                block_size);
+        VX_CHECK_LAUNCH();
+        return run_ragged(be, q, kv_pool, pool_is_f16, nullptr, matrix, nullptr, max_blocks, d_lens, out, batch_size,
+                          block_size, num_q_heads, num_kv_heads, head_dim, scale, max_len);
+    }
+    return run_ragged(be, q, kv_pool, pool_is_f16, (const int32_t *const *)dev, nullptr, nullptr, max_blocks, d_lens,
+                      out, batch_size, block_size, num_q_heads, num_kv_heads, head_dim, scale, max_len);
 }
 
 int vx_sdpa_paged_decode_ragged(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,

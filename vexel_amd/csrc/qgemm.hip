@@ -26,6 +26,8 @@
 //
 // Fallback (Q6_K, odd shapes): one wave per output column, float32 FMAs on the exact
 // dequantised values.
+#include <stdlib.h>
+
 #include "common.h"
 
 using namespace vx;
@@ -47,7 +49,7 @@ __device__ __forceinline__ float h2f(uint16_t h) {
 // a lane needs elements 4g..4g+3 and 16+4g..16+4g+3, i.e. two aligned float4 of the source row.
 
 // ---------------------------------------------------------------- activation prepare
-// Workspace layout (be->gemm_ws): tiles [K/32][Mpad/16][2][64] half8, then inv_scale[Mpad],
+// Workspace layout (be->gemm_ws): inv_scale[Mpad], then tiles [K/32][Mpad/16][2][64] half8,
 // then bsum[K/32][Mpad] (block sums of the scaled row, for Q4_K's min term).
 struct PrepView {
     half8 *tiles;
@@ -67,18 +69,48 @@ __device__ __forceinline__ float sigmoid_ref(float v) { return 1.0f / (1.0f + (f
 //   PREP_SILU_MUL: y = (a*sigmoid(a)) * b       (backend/cpu/cpu.go:390-400), optional f32 copy to `fout`
 // STAGE: keep the row's output values in LDS between the two passes (K*4 bytes of dynamic LDS);
 // otherwise pass 2 recomputes them.
+constexpr int PREP_THREADS = 512;  // shared by every kernel that writes prepared tiles: the row statistics
+                                    // are summed in an order that depends on it, and fused and unfused
+                                    // producers must agree bit for bit
+
+// ss + a^2 + b^2 + c^2 + d^2 in one fixed order of fused multiply-adds
+__device__ __forceinline__ float sumsq4(float ss, float a, float b, float c, float d) {
+    return __fmaf_rn(d, d, __fmaf_rn(c, c, __fmaf_rn(b, b, __fmaf_rn(a, a, ss))));
+}
+
+// amax / sum of squares over the workgroup; every thread gets the totals
+__device__ __forceinline__ void row_stats(float &amax, float &ss, float *sm) {
+    constexpr int NW = PREP_THREADS / 64;
+    for (int off = 32; off > 0; off >>= 1) {
+        amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+        ss += __shfl_xor(ss, off, 64);
+    }
+    const int tid = threadIdx.x;
+    if ((tid & 63) == 0) {
+        sm[tid >> 6] = amax;
+        sm[NW + (tid >> 6)] = ss;
+    }
+    __syncthreads();
+    amax = sm[0];
+    ss = sm[NW];
+    for (int i = 1; i < NW; i++) {
+        amax = fmaxf(amax, sm[i]);
+        ss += sm[NW + i];
+    }
+}
+
 template <int MODE, bool STAGE>
-__global__ void __launch_bounds__(256) prepare_kernel(const float *__restrict__ a, const float *__restrict__ b,
+__global__ void __launch_bounds__(PREP_THREADS) prepare_kernel(const float *__restrict__ a, const float *__restrict__ b,
                                                       float *__restrict__ fout, int M, int K, float eps,
                                                       PrepView pv, int Mpad) {
     extern __shared__ __attribute__((aligned(16))) float ybuf[];
-    __shared__ float sm[8];
+    __shared__ float sm[2 * (PREP_THREADS / 64)];
     const int r = blockIdx.x, tid = threadIdx.x;
     const int mtiles = Mpad / 16, mt = r >> 4, ln = r & 15;
     const int npairs = K / 8;  // (kstep, g) pairs: 8 output slots each
     if (r >= M) {
         const half8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-        for (int p = tid; p < npairs; p += 256) {
+        for (int p = tid; p < npairs; p += PREP_THREADS) {
             const int ks = p >> 2, g = p & 3;
             half8 *t = pv.tiles + ((size_t)(ks * mtiles + mt) * 2) * 64 + g * 16 + ln;
             t[0] = z;
@@ -92,11 +124,11 @@ __global__ void __launch_bounds__(256) prepare_kernel(const float *__restrict__ 
     const float *br = (MODE == PREP_RMSNORM) ? b : (b ? b + (size_t)r * K : nullptr);
     // pass 1: row statistics (SiLU*up values are staged in LDS for pass 2 when STAGE)
     float amax = 0.f, ss = 0.f;
-    for (int k = tid * 4; k < K; k += 1024) {
+    for (int k = tid * 4; k < K; k += PREP_THREADS * 4) {
         const float4 x = *(const float4 *)(ar + k);
         float y[4] = {x.x, x.y, x.z, x.w};
         if (MODE == PREP_RMSNORM) {
-            ss += x.x * x.x + x.y * x.y + x.z * x.z + x.w * x.w;
+            ss = sumsq4(ss, x.x, x.y, x.z, x.w);
         } else if (MODE == PREP_SILU_MUL) {
             const float4 u = *(const float4 *)(br + k);
             y[0] = __fmul_rn(__fmul_rn(x.x, sigmoid_ref(x.x)), u.x);
@@ -111,19 +143,9 @@ __global__ void __launch_bounds__(256) prepare_kernel(const float *__restrict__ 
         }
         amax = fmaxf(amax, fmaxf(fmaxf(fabsf(y[0]), fabsf(y[1])), fmaxf(fabsf(y[2]), fabsf(y[3]))));
     }
-    for (int off = 32; off > 0; off >>= 1) {
-        amax = fmaxf(amax, __shfl_xor(amax, off, 64));
-        ss += __shfl_xor(ss, off, 64);
-    }
-    if ((tid & 63) == 0) {
-        sm[tid >> 6] = amax;
-        sm[4 + (tid >> 6)] = ss;
-    }
-    __syncthreads();
-    amax = fmaxf(fmaxf(sm[0], sm[1]), fmaxf(sm[2], sm[3]));
+    row_stats(amax, ss, sm);
     float rms = 1.f;
     if (MODE == PREP_RMSNORM) {
-        ss = sm[4] + sm[5] + sm[6] + sm[7];
         rms = (float)sqrt((double)(ss / (float)K + eps));
         amax = amax / rms * 1.0001f;  // bound of |(x/rms)*w| up to rounding
     }
@@ -136,7 +158,7 @@ __global__ void __launch_bounds__(256) prepare_kernel(const float *__restrict__ 
     }
     if (tid == 0) pv.inv_scale[r] = inv;
     // pass 2: one (kstep, g) pair per iteration = elements 4g..4g+3 and 16+4g..16+4g+3 of the block
-    for (int p = tid; p < npairs; p += 256) {
+    for (int p = tid; p < npairs; p += PREP_THREADS) {
         const int ks = p >> 2, g = p & 3;
         const int k0 = ks * 32 + 4 * g;
         const float *src = (STAGE && MODE == PREP_SILU_MUL) ? ybuf : ar;
@@ -285,12 +307,23 @@ struct PQ4_K {
 
 constexpr int CH = 8;  // MFMA steps (32 elements each) per chunk
 
+// Up to three weight matrices that share K and the activation (Q/K/V, gate/up) multiplied in one
+// launch: output column n belongs to segment sg = first with n < n_end[sg], local row n - n_end[sg-1].
+struct Segs {
+    const uint8_t *w[3];
+    int n_end[3];
+};
+__device__ __forceinline__ const uint8_t *seg_row(const Segs &sg, int n, size_t row_bytes) {
+    const int i = n < sg.n_end[0] ? 0 : (n < sg.n_end[1] ? 1 : 2);
+    const int local = n - (i == 0 ? 0 : sg.n_end[i - 1]);
+    return sg.w[i] + (size_t)local * row_bytes;
+}
+
 // grid = (row groups of 64*R rows, KS k-slices, groups of MT activation tiles); block = 256.
 template <class F, int R, int MT>
-__global__ void __launch_bounds__(256) qgemm_kernel(const uint8_t *__restrict__ W, PrepView pv,
-                                                    float *__restrict__ out, const float *__restrict__ residual,
-                                                    float *__restrict__ partial, int M, int Mpad, int N, int K,
-                                                    int slice_chunks) {
+__global__ void __launch_bounds__(256) qgemm_kernel(Segs segs, PrepView pv, float *__restrict__ out,
+                                                    const float *__restrict__ residual, float *__restrict__ partial,
+                                                    int M, int Mpad, int N, int K, int slice_chunks) {
     constexpr int ROWS_W = 16 * R;
     constexpr int PITCH = F::CHUNK_BYTES + 32;  // (PITCH/4) % 8 == 4: 16 rows x 4 lane groups spread over all banks
     constexpr int WPIECES = ROWS_W * (F::CHUNK_BYTES / 16);
@@ -338,7 +371,7 @@ __global__ void __launch_bounds__(256) qgemm_kernel(const uint8_t *__restrict__ 
             const int row = pc / (F::CHUNK_BYTES / 16), col = pc % (F::CHUNK_BYTES / 16);
             const int n = min(n0 + row, N - 1);
             const bool ok = pc < WPIECES && col * 16 < valid;
-            w_stage[i] = ok ? *(const uint4 *)(W + (size_t)n * row_bytes + coff + col * 16) : make_uint4(0, 0, 0, 0);
+            w_stage[i] = ok ? *(const uint4 *)(seg_row(segs, n, row_bytes) + coff + col * 16) : make_uint4(0, 0, 0, 0);
         }
     };
     auto commit = [&]() {
@@ -419,8 +452,8 @@ __global__ void __launch_bounds__(256) qgemm_reduce_kernel(const float *__restri
     if (i >= total) return;
     float v = partial[i];
     for (int s = 1; s < KS; s++) v += partial[(size_t)s * total + i];
-    v *= inv_scale[i / N];
-    if (residual) v = residual[i] + v;
+    v = __fmul_rn(v, inv_scale[i / N]);
+    if (residual) v = __fadd_rn(residual[i], v);
     out[i] = v;
 }
 
@@ -496,6 +529,198 @@ __global__ void __launch_bounds__(64) qgemm_fallback_kernel(int fmt, const uint8
     }
 }
 
+// ---------------------------------------------------------------- consumers of split-K partial sums
+// Sum of the KS slices of four consecutive columns, in slice order, times the activation row scale:
+// exactly what qgemm_reduce_kernel computes.
+__device__ __forceinline__ float4 psum4(const float *__restrict__ P, int KS, size_t slice_elems, size_t idx, float inv) {
+    float4 v = *(const float4 *)(P + idx);
+    for (int s = 1; s < KS; s++) {
+        const float4 t = *(const float4 *)(P + (size_t)s * slice_elems + idx);
+        v.x += t.x; v.y += t.y; v.z += t.z; v.w += t.w;
+    }
+    v.x = __fmul_rn(v.x, inv); v.y = __fmul_rn(v.y, inv); v.z = __fmul_rn(v.z, inv); v.w = __fmul_rn(v.w, inv);
+    return v;
+}
+
+enum { FUSE_ADD_RMSNORM = 0, FUSE_SILU_MUL = 1 };
+constexpr int FP_THREADS = PREP_THREADS;
+
+// grid = Mpad rows, block = FP_THREADS, dynamic LDS = K floats.
+//  FUSE_ADD_RMSNORM: v = x + inv_in * sum_ks P[ks][r][:K]  (the residual add of runtime/block.go:990,1077),
+//                    x <- v, prepared <- (v / rms) * w      (backend/cpu/cpu.go:200-220)
+//  FUSE_SILU_MUL:    g = inv_in * sum P[..][r][:K], u = inv_in * sum P[..][r][K:2K],
+//                    prepared <- (g*sigmoid(g)) * u          (backend/cpu/cpu.go:390-400)
+// inv_in is the row scale of the activation that produced P; it is read before this row's new
+// scale overwrites it. Values are bit-identical to reduce + RMSNorm/SiLUMul + prepare run separately.
+template <int MODE>
+__global__ void __launch_bounds__(FP_THREADS) fused_prepare_kernel(float *__restrict__ x, const float *__restrict__ P,
+                                                                   int KS, int M, int K, const float *__restrict__ w,
+                                                                   float eps, PrepView pv, int Mpad) {
+    extern __shared__ __attribute__((aligned(16))) float ybuf[];
+    __shared__ float sm[2 * (FP_THREADS / 64)];
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const int mtiles = Mpad / 16, mt = r >> 4, ln = r & 15;
+    const int npairs = K / 8;
+    if (r >= M) {
+        const half8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int p = tid; p < npairs; p += FP_THREADS) {
+            const int ks = p >> 2, g = p & 3;
+            half8 *t = pv.tiles + ((size_t)(ks * mtiles + mt) * 2) * 64 + g * 16 + ln;
+            t[0] = z;
+            t[64] = z;
+            if (g == 0) pv.bsum[(size_t)ks * Mpad + r] = 0.f;
+        }
+        if (tid == 0) pv.inv_scale[r] = 0.f;
+        return;
+    }
+    const float inv_in = pv.inv_scale[r];
+    const int ncols = (MODE == FUSE_SILU_MUL) ? 2 * K : K;
+    const size_t slice_elems = (size_t)M * ncols;
+    float amax = 0.f, ss = 0.f;
+    for (int k = tid * 4; k < K; k += FP_THREADS * 4) {
+        float y[4];
+        if (MODE == FUSE_ADD_RMSNORM) {
+            const float4 d = psum4(P, KS, slice_elems, (size_t)r * ncols + k, inv_in);
+            const float4 xo = *(const float4 *)(x + (size_t)r * K + k);
+            y[0] = __fadd_rn(xo.x, d.x); y[1] = __fadd_rn(xo.y, d.y); y[2] = __fadd_rn(xo.z, d.z); y[3] = __fadd_rn(xo.w, d.w);
+            *(float4 *)(x + (size_t)r * K + k) = make_float4(y[0], y[1], y[2], y[3]);
+            *(float4 *)(ybuf + k) = make_float4(y[0], y[1], y[2], y[3]);
+            ss = sumsq4(ss, y[0], y[1], y[2], y[3]);
+            const float4 wv = *(const float4 *)(w + k);
+            y[0] *= wv.x; y[1] *= wv.y; y[2] *= wv.z; y[3] *= wv.w;
+        } else {
+            const float4 gt = psum4(P, KS, slice_elems, (size_t)r * ncols + k, inv_in);
+            const float4 up = psum4(P, KS, slice_elems, (size_t)r * ncols + K + k, inv_in);
+            y[0] = __fmul_rn(__fmul_rn(gt.x, sigmoid_ref(gt.x)), up.x);
+            y[1] = __fmul_rn(__fmul_rn(gt.y, sigmoid_ref(gt.y)), up.y);
+            y[2] = __fmul_rn(__fmul_rn(gt.z, sigmoid_ref(gt.z)), up.z);
+            y[3] = __fmul_rn(__fmul_rn(gt.w, sigmoid_ref(gt.w)), up.w);
+            *(float4 *)(ybuf + k) = make_float4(y[0], y[1], y[2], y[3]);
+        }
+        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(y[0]), fabsf(y[1])), fmaxf(fabsf(y[2]), fabsf(y[3]))));
+    }
+    row_stats(amax, ss, sm);  // also orders the ybuf writes before pass 2
+    float rms = 1.f;
+    if (MODE == FUSE_ADD_RMSNORM) {
+        rms = (float)sqrt((double)(ss / (float)K + eps));
+        amax = amax / rms * 1.0001f;
+    }
+    float s = 1.f, inv = 1.f;
+    if (amax > 0.f && amax < INFINITY) {
+        int ex;
+        (void)frexpf(amax, &ex);
+        s = ldexpf(1.f, 13 - ex);
+        inv = ldexpf(1.f, ex - 13);
+    }
+    if (tid == 0) pv.inv_scale[r] = inv;
+    for (int p = tid; p < npairs; p += FP_THREADS) {
+        const int ks = p >> 2, g = p & 3;
+        const int k0 = ks * 32 + 4 * g;
+        const float4 xa = *(const float4 *)(ybuf + k0), xb = *(const float4 *)(ybuf + k0 + 16);
+        float ya[4] = {xa.x, xa.y, xa.z, xa.w}, yb[4] = {xb.x, xb.y, xb.z, xb.w};
+        if (MODE == FUSE_ADD_RMSNORM) {
+            const float4 wa = *(const float4 *)(w + k0), wb = *(const float4 *)(w + k0 + 16);
+            const float wv[8] = {wa.x, wa.y, wa.z, wa.w, wb.x, wb.y, wb.z, wb.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                ya[i] = __fmul_rn(ya[i] / rms, wv[i]);
+                yb[i] = __fmul_rn(yb[i] / rms, wv[4 + i]);
+            }
+        }
+        const float v[8] = {ya[0] * s, ya[2] * s, yb[0] * s, yb[2] * s, ya[1] * s, ya[3] * s, yb[1] * s, yb[3] * s};
+        half8 h, l;
+        float bs = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            h[i] = (_Float16)v[i];
+            l[i] = (_Float16)(v[i] - (float)h[i]);
+            bs += v[i];
+        }
+        half8 *t = pv.tiles + ((size_t)(ks * mtiles + mt) * 2) * 64 + g * 16 + ln;
+        t[0] = h;
+        t[64] = l;
+        bs += __shfl_xor(bs, 1, 64);
+        bs += __shfl_xor(bs, 2, 64);
+        if (g == 0) pv.bsum[(size_t)ks * Mpad + r] = bs;
+    }
+}
+
+// x <- x + inv_in * sum_ks P (residual add only; used after the last layer's down projection)
+__global__ void __launch_bounds__(256) add_partials_kernel(float *__restrict__ x, const float *__restrict__ P, int KS,
+                                                           int M, int K, const float *__restrict__ inv_scale) {
+    const size_t i4 = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i4 >= (size_t)M * K) return;
+    const float4 d = psum4(P, KS, (size_t)M * K, i4, inv_scale[i4 / K]);
+    float4 v = *(const float4 *)(x + i4);
+    v.x = __fadd_rn(v.x, d.x); v.y = __fadd_rn(v.y, d.y); v.z = __fadd_rn(v.z, d.z); v.w = __fadd_rn(v.w, d.w);
+    *(float4 *)(x + i4) = v;
+}
+
+// RoPE (backend/cpu/cpu.go:226-303, interleaved pairs, one position per row) + paged K/V scatter
+// (metal_bridge_darwin.m:8607-8642) reading the fused Q|K|V projection from its split-K partials.
+// grid = (rows, head groups); thread = (pair j, head lane).
+template <bool F16>
+__global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, int M, const float *__restrict__ inv_scale,
+                                           float *__restrict__ q_out, const int32_t *__restrict__ positions,
+                                           const int32_t *__restrict__ slot_mapping, void *__restrict__ pool,
+                                           int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta) {
+    const int row = blockIdx.x, half = head_dim / 2;
+    const int qd = num_q_heads * head_dim, kvd = num_kv_heads * head_dim, ncols = qd + 2 * kvd;
+    const size_t slice_elems = (size_t)M * ncols;
+    const float inv = inv_scale[row];
+    const int pos = positions[row], slot = slot_mapping[row];
+    const int blk = slot / block_size, off = slot % block_size;
+    const size_t part = (size_t)block_size * kvd;
+    const size_t kbase = (size_t)blk * 2 * part + (size_t)off * kvd, vbase = kbase + part;
+    const int lanes = blockDim.x / half, hl = threadIdx.x / half, j = threadIdx.x % half;
+    if (hl >= lanes) return;
+    const int hstride = lanes * gridDim.y, h0 = blockIdx.y * lanes + hl;
+    const double ex = (double)(2 * j) / (double)head_dim;
+    const float freq = (float)(1.0 / pow((double)theta, ex));
+    const float angle = __fmul_rn((float)pos, freq);
+    const float c = (float)cos((double)angle), sn = (float)sin((double)angle);
+    auto pair = [&](int col, float &a, float &b) {
+        const float *p0 = P + (size_t)row * ncols + col;
+        float2 v = *(const float2 *)p0;
+        for (int s = 1; s < KS; s++) {
+            const float2 t = *(const float2 *)(p0 + (size_t)s * slice_elems);
+            v.x += t.x;
+            v.y += t.y;
+        }
+        a = __fmul_rn(v.x, inv);
+        b = __fmul_rn(v.y, inv);
+    };
+    for (int h = h0; h < num_q_heads; h += hstride) {
+        float a, b;
+        pair(h * head_dim + 2 * j, a, b);
+        float2 o;
+        o.x = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, sn));
+        o.y = __fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, c));
+        *(float2 *)(q_out + (size_t)row * qd + h * head_dim + 2 * j) = o;
+    }
+    for (int h = h0; h < num_kv_heads; h += hstride) {
+        float a, b, va, vb;
+        pair(qd + h * head_dim + 2 * j, a, b);
+        pair(qd + kvd + h * head_dim + 2 * j, va, vb);
+        const float ka = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, sn));
+        const float kb = __fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, c));
+        const size_t o = (size_t)h * head_dim + 2 * j;
+        if (F16) {
+            _Float16 *pp = (_Float16 *)pool;
+            pp[kbase + o] = (_Float16)ka;
+            pp[kbase + o + 1] = (_Float16)kb;
+            pp[vbase + o] = (_Float16)va;
+            pp[vbase + o + 1] = (_Float16)vb;
+        } else {
+            float *pp = (float *)pool;
+            pp[kbase + o] = ka;
+            pp[kbase + o + 1] = kb;
+            pp[vbase + o] = va;
+            pp[vbase + o + 1] = vb;
+        }
+    }
+}
+
 size_t fmt_row_bytes(int fmt, int k) {
     switch (fmt) {
     case VX_Q4_0: return (size_t)k / 32 * 18;
@@ -510,10 +735,12 @@ int mpad_for(int m) { return m <= 16 ? 16 : ceil_div(m, 32) * 32; }
 
 PrepView prep_view(vx_backend *be, int mpad, int k) {
     PrepView pv;
+    // the row scales sit first, at an address that does not depend on K: a fused consumer reads the
+    // scales of the activation that produced its input while it prepares an activation of another width
     char *base = (char *)be->gemm_ws;
-    pv.tiles = (half8 *)base;
-    pv.inv_scale = (float *)(base + prep_tiles_bytes(mpad, k));
-    pv.bsum = pv.inv_scale + ceil_div(mpad, 64) * 64;
+    pv.inv_scale = (float *)base;
+    pv.tiles = (half8 *)(base + (size_t)ceil_div(mpad, 64) * 64 * 4);
+    pv.bsum = (float *)((char *)pv.tiles + prep_tiles_bytes(mpad, k));
     return pv;
 }
 
@@ -530,8 +757,30 @@ int prep_begin(vx_backend *be, int m, int k, PrepView *pv) {
     return VX_OK;
 }
 
+int gemm_target_wgs() {
+    static int v = 0;
+    if (v == 0) {
+        const char *e = getenv("VEXEL_HIP_GEMM_WGS");
+        v = e ? atoi(e) : 0;
+        if (v <= 0) v = 512;
+    }
+    return v;
+}
+
+// Launches the MFMA GEMM of the prepared activation against the segments. When `to_partials` (or when
+// more than one K slice is used) the raw sums go to be->part_ws as P[ks][M][N] and *ks_out slices must
+// be added by the consumer; otherwise out = residual + inv_scale * sums is written directly.
+// Grows the prepared-activation workspace for an [m, kmax] activation now, so that later prepares
+// of narrower activations inside one fused sequence cannot reallocate it (and lose the row scales).
+int prep_reserve(vx_backend *be, int m, int kmax) {
+    const int mpad = mpad_for(m);
+    const size_t need = prep_tiles_bytes(mpad, kmax) + (size_t)ceil_div(mpad, 64) * 64 * 4 + (size_t)(kmax / 32) * mpad * 4;
+    return ensure_ws(be, &be->gemm_ws, &be->gemm_ws_bytes, need, "prepared activations");
+}
+
 template <class F>
-int launch_fast(vx_backend *be, const uint8_t *W, float *out, const float *residual, int M, int N, int K) {
+int launch_gemm(vx_backend *be, const Segs &segs, int N, float *out, const float *residual, bool to_partials, int M,
+                int K, int *ks_out) {
     const int mpad = mpad_for(M);
     const PrepView pv = prep_view(be, mpad, K);
     constexpr int R = 2;
@@ -541,14 +790,14 @@ int launch_fast(vx_backend *be, const uint8_t *W, float *out, const float *resid
     // enough workgroups to fill 256 CUs, at least 2 chunks per slice; depends on (N, K) only when M <= 32
     int ks = 1;
     if (mgroups == 1) {
-        ks = ceil_div(512, rg);
+        ks = ceil_div(gemm_target_wgs(), rg);
         if (ks > n_chunks / 2) ks = n_chunks / 2;
         if (ks < 1) ks = 1;
     }
     const int slice = ceil_div(n_chunks, ks);
     ks = ceil_div(n_chunks, slice);
     float *partial = nullptr;
-    if (ks > 1) {
+    if (ks > 1 || to_partials) {
         const size_t need = (size_t)ks * M * N * sizeof(float);
         int rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, need, "split-K partial sums");
         if (rc) return rc;
@@ -556,17 +805,27 @@ int launch_fast(vx_backend *be, const uint8_t *W, float *out, const float *resid
     }
     dim3 grid(rg, ks, mgroups);
     if (mpad <= 16)
-        qgemm_kernel<F, R, 1><<<grid, 256, 0, be->stream>>>(W, pv, out, residual, partial, M, mpad, N, K, slice);
+        qgemm_kernel<F, R, 1><<<grid, 256, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slice);
     else
-        qgemm_kernel<F, R, 2><<<grid, 256, 0, be->stream>>>(W, pv, out, residual, partial, M, mpad, N, K, slice);
+        qgemm_kernel<F, R, 2><<<grid, 256, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slice);
     VX_CHECK_LAUNCH();
-    if (ks > 1) {
+    if (ks_out) *ks_out = ks;
+    if (partial && !to_partials) {
         const size_t total = (size_t)M * N;
         qgemm_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>(partial, pv.inv_scale, out,
                                                                                       residual, M, N, ks);
         VX_CHECK_LAUNCH();
     }
     return VX_OK;
+}
+
+int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out, const float *residual,
+                    bool to_partials, int M, int K, int *ks_out) {
+    switch (fmt) {
+    case VX_Q4_0: return launch_gemm<PQ4_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
+    case VX_Q8_0: return launch_gemm<PQ8_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
+    default: return launch_gemm<PQ4_K>(be, segs, N, out, residual, to_partials, M, K, ks_out);
+    }
 }
 
 bool fast_ok(int fmt, const void *b, int k) {
@@ -585,12 +844,10 @@ int check_fmt(int fmt, int k) {
 }
 
 int run_prepared(vx_backend *be, int fmt, const void *b, float *out, const float *residual, int m, int n, int k) {
-    const uint8_t *W = (const uint8_t *)b;
-    switch (fmt) {
-    case VX_Q4_0: return launch_fast<PQ4_0>(be, W, out, residual, m, n, k);
-    case VX_Q8_0: return launch_fast<PQ8_0>(be, W, out, residual, m, n, k);
-    default: return launch_fast<PQ4_K>(be, W, out, residual, m, n, k);
-    }
+    Segs segs;
+    segs.w[0] = segs.w[1] = segs.w[2] = (const uint8_t *)b;
+    segs.n_end[0] = segs.n_end[1] = segs.n_end[2] = n;
+    return launch_gemm_fmt(be, fmt, segs, n, out, residual, false, m, k, nullptr);
 }
 
 }  // namespace
@@ -605,7 +862,7 @@ int vx_prepare_act(vx_backend *be, const float *a, int m, int k) {
     rc = prep_begin(be, m, k, &pv);
     if (rc) return rc;
     const int mpad = mpad_for(m);
-    prepare_kernel<PREP_PLAIN, false><<<mpad, 256, 0, be->stream>>>(a, nullptr, nullptr, m, k, 0.f, pv, mpad);
+    prepare_kernel<PREP_PLAIN, false><<<mpad, PREP_THREADS, 0, be->stream>>>(a, nullptr, nullptr, m, k, 0.f, pv, mpad);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }
@@ -619,7 +876,7 @@ int vx_rmsnorm_prepare(vx_backend *be, const float *x, const float *weight, floa
     rc = prep_begin(be, rows, cols, &pv);
     if (rc) return rc;
     const int mpad = mpad_for(rows);
-    prepare_kernel<PREP_RMSNORM, false><<<mpad, 256, 0, be->stream>>>(x, weight, out, rows, cols, eps, pv, mpad);
+    prepare_kernel<PREP_RMSNORM, false><<<mpad, PREP_THREADS, 0, be->stream>>>(x, weight, out, rows, cols, eps, pv, mpad);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }
@@ -634,10 +891,10 @@ int vx_silu_mul_prepare(vx_backend *be, const float *gate, const float *up, floa
     if (rc) return rc;
     const int mpad = mpad_for(rows);
     if ((size_t)cols * 4 <= 48 * 1024)
-        prepare_kernel<PREP_SILU_MUL, true><<<mpad, 256, (size_t)cols * 4, be->stream>>>(gate, up, out, rows, cols, 0.f,
+        prepare_kernel<PREP_SILU_MUL, true><<<mpad, PREP_THREADS, (size_t)cols * 4, be->stream>>>(gate, up, out, rows, cols, 0.f,
                                                                                           pv, mpad);
     else
-        prepare_kernel<PREP_SILU_MUL, false><<<mpad, 256, 0, be->stream>>>(gate, up, out, rows, cols, 0.f, pv, mpad);
+        prepare_kernel<PREP_SILU_MUL, false><<<mpad, PREP_THREADS, 0, be->stream>>>(gate, up, out, rows, cols, 0.f, pv, mpad);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }
@@ -676,6 +933,146 @@ int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, floa
     rc = vx_prepare_act(be, a, m, k);
     if (rc) return rc;
     return run_prepared(be, fmt, b, out, residual, m, n, k);
+}
+
+static bool group_ok(const vx_qweight *const *ws, int nw) {
+    for (int i = 0; i < nw; i++) {
+        if (!ws[i] || !ws[i]->data) return false;
+        if (ws[i]->fmt != ws[0]->fmt || ws[i]->k != ws[0]->k) return false;
+        if (!fast_ok(ws[i]->fmt, ws[i]->data, ws[i]->k) || ws[i]->n % 16 != 0 || ws[i]->n <= 0) return false;
+    }
+    return true;
+}
+
+static Segs make_segs(const vx_qweight *const *ws, int nw, int *ntot) {
+    Segs sg;
+    int acc = 0;
+    for (int i = 0; i < 3; i++) {
+        const vx_qweight *w = ws[i < nw ? i : nw - 1];
+        if (i < nw) acc += w->n;
+        sg.w[i] = (const uint8_t *)w->data;
+        sg.n_end[i] = acc;
+    }
+    *ntot = acc;
+    return sg;
+}
+
+int vx_decode_attn_qkv_supported(const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int head_dim) {
+    const vx_qweight *ws[3] = {wq, wk, wv};
+    return group_ok(ws, 3) && head_dim % 2 == 0 && head_dim <= 512 && (size_t)wq->k * 4 <= 64 * 1024;
+}
+
+int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight, float eps, int x_prepared,
+                       const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int rows,
+                       const int32_t *positions, const int32_t *slot_mapping, void *kv_pool, int pool_is_f16,
+                       int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta, float *q_out) {
+    int rc = enter(be);
+    if (rc) return rc;
+    if (!vx_decode_attn_qkv_supported(wq, wk, wv, head_dim)) {
+        set_error("vx_decode_attn_qkv: weights have no fused MFMA path");
+        return VX_ERR_UNSUPPORTED;
+    }
+    VX_REQUIRE(positions && slot_mapping && kv_pool && q_out && rows >= 1, "vx_decode_attn_qkv: bad arguments");
+    VX_REQUIRE(wq->n == num_q_heads * head_dim && wk->n == num_kv_heads * head_dim && wv->n == wk->n && block_size >= 1,
+               "vx_decode_attn_qkv: weight shapes do not match the head geometry");
+    const int k = wq->k;
+    if (x_prepared) {
+        VX_REQUIRE(be->prep_m == rows && be->prep_k == k, "vx_decode_attn_qkv: no prepared %dx%d activation (have %dx%d)",
+                   rows, k, be->prep_m, be->prep_k);
+    } else {
+        rc = vx_rmsnorm_prepare(be, x, norm_weight, nullptr, rows, k, eps);
+        if (rc) return rc;
+    }
+    const vx_qweight *ws[3] = {wq, wk, wv};
+    int ntot, ks;
+    const Segs segs = make_segs(ws, 3, &ntot);
+    rc = launch_gemm_fmt(be, wq->fmt, segs, ntot, nullptr, nullptr, true, rows, k, &ks);
+    if (rc) return rc;
+    const PrepView pv = prep_view(be, mpad_for(rows), k);
+    const int half = head_dim / 2;
+    const int lanes = 256 / half > 0 ? 256 / half : 1;
+    const int max_heads = num_q_heads > num_kv_heads ? num_q_heads : num_kv_heads;
+    dim3 grid(rows, ceil_div(max_heads, lanes * 2));
+    if (pool_is_f16)
+        rope_store_partials_kernel<true><<<grid, lanes * half, 0, be->stream>>>(
+            (const float *)be->part_ws, ks, rows, pv.inv_scale, q_out, positions, slot_mapping, kv_pool, num_q_heads,
+            num_kv_heads, head_dim, block_size, theta);
+    else
+        rope_store_partials_kernel<false><<<grid, lanes * half, 0, be->stream>>>(
+            (const float *)be->part_ws, ks, rows, pv.inv_scale, q_out, positions, slot_mapping, kv_pool, num_q_heads,
+            num_kv_heads, head_dim, block_size, theta);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_decode_ffn_supported(const vx_qweight *wo, const vx_qweight *w1, const vx_qweight *w3, const vx_qweight *w2) {
+    const vx_qweight *a[1] = {wo}, *b[2] = {w1, w3}, *c[1] = {w2};
+    if (!group_ok(a, 1) || !group_ok(b, 2) || !group_ok(c, 1)) return 0;
+    if (w1->n != w3->n || w2->k != w1->n || w2->n != wo->n || w1->k != wo->n) return 0;
+    return (size_t)wo->n * 4 <= 64 * 1024 && (size_t)w1->n * 4 <= 64 * 1024 && wo->n % 256 == 0 && w1->n % 256 == 0;
+}
+
+int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight *wo, const float *ffn_norm_weight,
+                  float eps, const vx_qweight *w1, const vx_qweight *w3, const vx_qweight *w2, int rows,
+                  const float *next_norm_weight) {
+    int rc = enter(be);
+    if (rc) return rc;
+    if (!vx_decode_ffn_supported(wo, w1, w3, w2)) {
+        set_error("vx_decode_ffn: weights have no fused MFMA path");
+        return VX_ERR_UNSUPPORTED;
+    }
+    VX_REQUIRE(attn && x && ffn_norm_weight && rows >= 1, "vx_decode_ffn: bad arguments");
+    VX_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)ffn_norm_weight % 16 == 0) && ((uintptr_t)next_norm_weight % 16 == 0),
+               "vx_decode_ffn: unaligned pointer");
+    const int hidden = wo->n, ffn = w1->n, mpad = mpad_for(rows);
+    int ks, ntot;
+    rc = prep_reserve(be, rows, ffn > wo->k ? (ffn > hidden ? ffn : hidden) : (wo->k > hidden ? wo->k : hidden));
+    if (rc) return rc;
+    // attention output -> Wo -> partials
+    rc = vx_prepare_act(be, attn, rows, wo->k);
+    if (rc) return rc;
+    const vx_qweight *a[1] = {wo};
+    Segs segs = make_segs(a, 1, &ntot);
+    rc = launch_gemm_fmt(be, wo->fmt, segs, ntot, nullptr, nullptr, true, rows, wo->k, &ks);
+    if (rc) return rc;
+    // x += Wo(attn); prepared <- RMSNorm(x) * ffn_norm
+    PrepView pv;
+    rc = prep_begin(be, rows, hidden, &pv);
+    if (rc) return rc;
+    fused_prepare_kernel<FUSE_ADD_RMSNORM><<<mpad, FP_THREADS, (size_t)hidden * 4, be->stream>>>(
+        x, (const float *)be->part_ws, ks, rows, hidden, ffn_norm_weight, eps, pv, mpad);
+    VX_CHECK_LAUNCH();
+    // gate | up -> partials
+    const vx_qweight *b[2] = {w1, w3};
+    segs = make_segs(b, 2, &ntot);
+    rc = launch_gemm_fmt(be, w1->fmt, segs, ntot, nullptr, nullptr, true, rows, hidden, &ks);
+    if (rc) return rc;
+    // prepared <- SiLU(gate) * up
+    rc = prep_begin(be, rows, ffn, &pv);
+    if (rc) return rc;
+    fused_prepare_kernel<FUSE_SILU_MUL><<<mpad, FP_THREADS, (size_t)ffn * 4, be->stream>>>(
+        nullptr, (const float *)be->part_ws, ks, rows, ffn, nullptr, 0.f, pv, mpad);
+    VX_CHECK_LAUNCH();
+    // down -> partials
+    const vx_qweight *c[1] = {w2};
+    segs = make_segs(c, 1, &ntot);
+    rc = launch_gemm_fmt(be, w2->fmt, segs, ntot, nullptr, nullptr, true, rows, ffn, &ks);
+    if (rc) return rc;
+    if (next_norm_weight) {
+        rc = prep_begin(be, rows, hidden, &pv);
+        if (rc) return rc;
+        fused_prepare_kernel<FUSE_ADD_RMSNORM><<<mpad, FP_THREADS, (size_t)hidden * 4, be->stream>>>(
+            x, (const float *)be->part_ws, ks, rows, hidden, next_norm_weight, eps, pv, mpad);
+        VX_CHECK_LAUNCH();
+    } else {
+        const size_t total4 = (size_t)rows * hidden / 4;
+        add_partials_kernel<<<(unsigned)((total4 + 255) / 256), 256, 0, be->stream>>>(x, (const float *)be->part_ws, ks,
+                                                                                     rows, hidden, pv.inv_scale);
+        VX_CHECK_LAUNCH();
+        be->prep_m = 0;  // the slot no longer matches any activation the caller knows about
+        be->prep_k = 0;
+    }
+    return VX_OK;
 }
 
 int vx_matmul_q4_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k) {

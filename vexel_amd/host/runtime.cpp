@@ -120,6 +120,8 @@ struct vh_model {
     float *x = nullptr, *norm = nullptr, *q = nullptr, *k = nullptr, *v = nullptr, *attn = nullptr;
     float *gate = nullptr, *up = nullptr, *logits = nullptr;
 
+    bool fused = true;  // take the fused decode entry points where the weights allow it
+
     vx_graph *graph = nullptr;
     int graph_batch = 0;
     std::vector<int64_t> dev_seq_ids;  // batch currently loaded in d_slots (device-driven mode)
@@ -228,22 +230,44 @@ int layer_tail(vh_model *m, const vh_layer_weights &w, float *x, float *norm, co
     return VH_OK;
 }
 
+bool attn_fusable(const vh_model *m, int layer) {
+    if (!m->fused || layer >= m->cfg.num_layers) return false;
+    const vh_layer_weights &w = m->layers[layer];
+    return w.wq.data && w.wk.data && w.wv.data && vx_decode_attn_qkv_supported(&w.wq, &w.wk, &w.wv, m->cfg.head_dim) != 0;
+}
+
 // One layer for `rows` single-token sequences; positions, slots, tables and lengths are on the device.
-int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len) {
+// *chained says, on entry, that the backend's prepared slot already holds RMSNorm(x)*attn_norm of this
+// layer (left there by the previous layer's fused tail) and, on exit, the same for `next_norm`.
+int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const float *next_norm, bool *chained) {
     const vh_config &c = m->cfg;
     const vh_layer_weights &w = m->layers[layer];
     const float scale = (float)(1.0 / sqrt((double)c.head_dim));                          // block.go:862
-    bool prep;
-    const vh_qweight *qkv[3] = {&w.wq, &w.wk, &w.wv};
-    VHC(norm_for(m, m->x, w.attn_norm, m->norm, rows, qkv, 3, &prep));                    // block.go:834-837
-    VHC(mm(m, prep, m->norm, w.wq, m->q, nullptr, rows));                                 // block.go:841-854
-    VHC(mm(m, prep, m->norm, w.wk, m->k, nullptr, rows));
-    VHC(mm(m, prep, m->norm, w.wv, m->v, nullptr, rows));
-    VXC(vx_rope_store_paged(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
-                            c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta));  // :858, :868
+    if (attn_fusable(m, layer)) {                                                         // block.go:834-868
+        VXC(vx_decode_attn_qkv(m->be, m->x, w.attn_norm, c.eps, *chained ? 1 : 0, &w.wq, &w.wk, &w.wv, rows,
+                               m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, c.num_heads, c.num_kv_heads,
+                               c.head_dim, c.block_size, c.rope_theta, m->q));
+    } else {
+        if (*chained) return fail("internal: prepared activation handed to an unfused layer");
+        bool prep;
+        const vh_qweight *qkv[3] = {&w.wq, &w.wk, &w.wv};
+        VHC(norm_for(m, m->x, w.attn_norm, m->norm, rows, qkv, 3, &prep));                // block.go:834-837
+        VHC(mm(m, prep, m->norm, w.wq, m->q, nullptr, rows));                             // block.go:841-854
+        VHC(mm(m, prep, m->norm, w.wk, m->k, nullptr, rows));
+        VHC(mm(m, prep, m->norm, w.wv, m->v, nullptr, rows));
+        VXC(vx_rope_store_paged(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
+                                c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta));  // :858, :868
+    }
     VXC(vx_sdpa_paged_decode_ragged(m->be, m->q, m->kv[layer], c.kv_fp16, m->d_tables, m->d_slots, m->d_kv_lens,
                                     m->attn, rows, c.max_blocks_per_seq, c.block_size, c.num_heads, c.num_kv_heads,
                                     c.head_dim, scale, max_kv_len));                       // block.go:872
+    *chained = false;
+    if (m->fused && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
+        vx_decode_ffn_supported(&w.wo, &w.w1, &w.w3, &w.w2)) {                            // block.go:981-1077
+        VXC(vx_decode_ffn(m->be, m->attn, m->x, &w.wo, w.ffn_norm, c.eps, &w.w1, &w.w3, &w.w2, rows, next_norm));
+        *chained = next_norm != nullptr;
+        return VH_OK;
+    }
     return layer_tail(m, w, m->x, m->norm, m->attn, m->gate, m->up, rows);
 }
 
@@ -251,11 +275,21 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len) {
 int forward_decode(vh_model *m, int rows, int max_kv_len) {
     const vh_config &c = m->cfg;
     VXC(vx_embedding(m->be, m->d_tokens, rows, m->embedding, m->x, c.vocab, c.hidden));
-    for (int l = 0; l < c.num_layers; l++) VHC(execute_layer_decode(m, l, rows, max_kv_len));
-    bool prep;
-    const vh_qweight *hw[1] = {&m->lm_head};
-    VHC(norm_for(m, m->x, m->final_norm, m->norm, rows, hw, 1, &prep));                    // model.go:207-226
-    VHC(mm(m, prep, m->norm, m->lm_head, m->logits, nullptr, rows));                      // model.go:352-422
+    const bool head_prepared = m->fused && fast(m->lm_head) && c.hidden % 256 == 0;
+    bool chained = false;
+    for (int l = 0; l < c.num_layers; l++) {
+        const float *next_norm = l + 1 < c.num_layers ? (attn_fusable(m, l + 1) ? m->layers[l + 1].attn_norm : nullptr)
+                                                      : (head_prepared ? m->final_norm : nullptr);
+        VHC(execute_layer_decode(m, l, rows, max_kv_len, next_norm, &chained));
+    }
+    if (chained) {                                                                        // model.go:207-226, 352-422
+        VHC(mm(m, true, nullptr, m->lm_head, m->logits, nullptr, rows));
+    } else {
+        bool prep;
+        const vh_qweight *hw[1] = {&m->lm_head};
+        VHC(norm_for(m, m->x, m->final_norm, m->norm, rows, hw, 1, &prep));
+        VHC(mm(m, prep, m->norm, m->lm_head, m->logits, nullptr, rows));
+    }
     VXC(vx_argmax_rows(m->be, m->logits, rows, c.vocab, m->d_next));
     return VH_OK;
 }
@@ -369,6 +403,16 @@ int vh_model_set_head(vh_model *m, const float *embedding, const float *final_no
     m->final_norm = final_norm;
     m->lm_head = *lm_head;
     return VH_OK;
+}
+
+void vh_model_set_fused(vh_model *m, int on) {
+    if (!m) return;
+    m->fused = on != 0;
+    if (m->graph) {  // the captured step was recorded with the other kernel sequence
+        vx_graph_destroy(m->graph);
+        m->graph = nullptr;
+        m->graph_batch = 0;
+    }
 }
 
 void *vh_kv_pool(vh_model *m, int layer) {

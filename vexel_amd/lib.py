@@ -62,6 +62,10 @@ SIGNATURES = {
     "vx_silu_mul_prepare": (_i, [_vp, _vp, _vp, _vp, _i, _i]),
     "vx_matmul_quant_prepared": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i]),
     "vx_matmul_quant_has_fast_path": (_i, [_i, _vp, _i]),
+    "vx_decode_attn_qkv_supported": (_i, [_vp, _vp, _vp, _i]),
+    "vx_decode_attn_qkv": (_i, [_vp, _vp, _vp, _f, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
+    "vx_decode_ffn_supported": (_i, [_vp, _vp, _vp, _vp]),
+    "vx_decode_ffn": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _vp]),
     "vx_rope_store_paged": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f]),
     "vx_sdpa_paged_decode_ragged": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i]),
     "vx_sdpa_paged_tree": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),

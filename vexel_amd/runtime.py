@@ -8,7 +8,7 @@ import os
 import numpy as np
 
 from . import lib as _l
-from .backend import HipBackend, VexelError
+from .backend import HipBackend, VexelError, VxQWeight
 
 HOST_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libvexel_host.so")
 
@@ -21,8 +21,7 @@ class VhConfig(C.Structure):
                                         "kv_fp16")]
 
 
-class VhQWeight(C.Structure):
-    _fields_ = [("fmt", C.c_int), ("data", C.c_void_p), ("n", C.c_int), ("k", C.c_int)]
+VhQWeight = VxQWeight  # vh_qweight is a typedef of vx_qweight
 
 
 class VhLayerWeights(C.Structure):
@@ -46,6 +45,8 @@ def load_host():
         h.vh_model_create.argtypes = [C.c_void_p, C.POINTER(VhConfig), C.POINTER(C.c_void_p)]
         h.vh_model_destroy.argtypes = [C.c_void_p]
         h.vh_model_destroy.restype = None
+        h.vh_model_set_fused.argtypes = [C.c_void_p, C.c_int]
+        h.vh_model_set_fused.restype = None
         h.vh_model_set_layer.argtypes = [C.c_void_p, C.c_int, C.POINTER(VhLayerWeights)]
         h.vh_model_set_head.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(VhQWeight)]
         for name in ("vh_pool_create_sequence", "vh_pool_delete_sequence", "vh_pool_has_sequence", "vh_pool_seq_len"):
@@ -125,6 +126,12 @@ class ModelRuntime:
         ptr = data if isinstance(data, int) else self._up(data)
         qw = VhQWeight(fmt, ptr, n, k)
         self._ck(self._h.vh_model_set_head(self._m, emb, fn, C.byref(qw)))
+
+    def set_fused(self, on):
+        """Decode through the fused entry points where the weights allow it (default) or, when off,
+        through one backend call per operation as runtime/block.go does; the two agree to float32
+        summation order."""
+        self._h.vh_model_set_fused(self._m, int(bool(on)))
 
     def kv_pool(self, layer):
         return self._h.vh_kv_pool(self._m, layer)
