@@ -37,6 +37,7 @@ namespace {
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float h2f(uint16_t h) {
     _Float16 v;
@@ -313,10 +314,14 @@ struct Segs {
     const uint8_t *w[3];
     int n_end[3];
 };
+// Selects over values read once from the kernel arguments; indexing the arrays with a per-lane index
+// would turn every row lookup into dependent memory loads.
 __device__ __forceinline__ const uint8_t *seg_row(const Segs &sg, int n, size_t row_bytes) {
-    const int i = n < sg.n_end[0] ? 0 : (n < sg.n_end[1] ? 1 : 2);
-    const int local = n - (i == 0 ? 0 : sg.n_end[i - 1]);
-    return sg.w[i] + (size_t)local * row_bytes;
+    const uint8_t *w0 = sg.w[0], *w1 = sg.w[1], *w2 = sg.w[2];
+    const int e0 = sg.n_end[0], e1 = sg.n_end[1];
+    const uint8_t *base = n < e0 ? w0 : (n < e1 ? w1 : w2);
+    const int local = n < e0 ? n : (n < e1 ? n - e0 : n - e1);
+    return base + (size_t)local * row_bytes;
 }
 
 // grid = (row groups of 64*R rows, KS k-slices, groups of MT activation tiles); block = 256.
@@ -352,36 +357,35 @@ __global__ void __launch_bounds__(256) qgemm_kernel(Segs segs, PrepView pv, floa
         for (int t = 0; t < MT; t++) run[r][t] = (float4v){0.f, 0.f, 0.f, 0.f};
 
     half8 a_stage[ANL];
-    uint4 w_stage[WNL];
-    auto fetch = [&](int chunk) {
+    u32x4 w_stage[WNL];
+    // K is a multiple of 256, so every chunk has CH full steps and CHUNK_BYTES bytes per row. Every load is
+    // unconditional (addresses are clamped instead): a load under a branch makes the compiler wait for it
+    // inside the branch, which serialises the whole prefetch.
+    auto fetch = [&](int chunk) __attribute__((always_inline)) {
         const int s0 = chunk * CH;
-        const int nsteps = min(CH, steps_total - s0);
 #pragma unroll
         for (int i = 0; i < ANL; i++) {
             const int p = i * 256 + tid;              // (s, t, hl, l)
             const int l = p & 63, hl = (p >> 6) & 1, t = (p >> 7) % MT, s = p / (128 * MT);
-            const half8 z = {0, 0, 0, 0, 0, 0, 0, 0};
-            a_stage[i] = (s < nsteps) ? pv.tiles[((size_t)((s0 + s) * mtiles + mg * MT + t) * 2 + hl) * 64 + l] : z;
+            a_stage[i] = pv.tiles[((size_t)((s0 + s) * mtiles + mg * MT + t) * 2 + hl) * 64 + l];
         }
         const size_t coff = (size_t)chunk * F::CHUNK_BYTES;
-        const int valid = (int)min((size_t)F::CHUNK_BYTES, row_bytes - coff);
 #pragma unroll
         for (int i = 0; i < WNL; i++) {
-            const int pc = i * 64 + lane;
+            const int pc = min(i * 64 + lane, WPIECES - 1);
             const int row = pc / (F::CHUNK_BYTES / 16), col = pc % (F::CHUNK_BYTES / 16);
             const int n = min(n0 + row, N - 1);
-            const bool ok = pc < WPIECES && col * 16 < valid;
-            w_stage[i] = ok ? *(const uint4 *)(seg_row(segs, n, row_bytes) + coff + col * 16) : make_uint4(0, 0, 0, 0);
+            w_stage[i] = *(const u32x4 *)(seg_row(segs, n, row_bytes) + coff + col * 16);
         }
     };
-    auto commit = [&]() {
+    auto commit = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < ANL; i++) a_lds[i * 256 + tid] = a_stage[i];
 #pragma unroll
         for (int i = 0; i < WNL; i++) {
             const int pc = i * 64 + lane;
             const int row = pc / (F::CHUNK_BYTES / 16), col = pc % (F::CHUNK_BYTES / 16);
-            if (pc < WPIECES) *(uint4 *)(&w_lds[wave][row * PITCH + col * 16]) = w_stage[i];
+            if (pc < WPIECES) *(u32x4 *)(&w_lds[wave][row * PITCH + col * 16]) = w_stage[i];
         }
     };
 
@@ -392,8 +396,8 @@ __global__ void __launch_bounds__(256) qgemm_kernel(Segs segs, PrepView pv, floa
         __syncthreads();
         if (chunk + 1 < c_end) fetch(chunk + 1);  // in flight while this chunk is computed
         const int s0 = chunk * CH;
-        const int nsteps = min(CH, steps_total - s0);
-        for (int s = 0; s < nsteps; s++) {
+#pragma unroll 2
+        for (int s = 0; s < CH; s++) {
             half8 ah[MT], al[MT];
 #pragma unroll
             for (int t = 0; t < MT; t++) {
@@ -421,24 +425,46 @@ __global__ void __launch_bounds__(256) qgemm_kernel(Segs segs, PrepView pv, floa
         }
     }
 
-    // lane (g, ln) of tile (r, t) holds C[m = m0 + 16t + 4g + i][n = n0 + 16r + ln], i = 0..3
+    // lane (g, ln) of tile (r, t) holds C[m = m0 + 16t + 4g + i][n = n0 + 16r + ln], i = 0..3.
+    // Loads use clamped indices and come first, so they are all in flight together; only stores are predicated.
+    if (partial) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int m = m0 + t * 16 + 4 * g + i, n = n0 + r * 16 + ln;
+                    if (m < M && n < N) partial[((size_t)ks * M + m) * N + n] = run[r][t][i];
+                }
+        return;
+    }
+    float inv[MT][4], res[R][MT][4];
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) inv[t][i] = pv.inv_scale[m0 + t * 16 + 4 * g + i];  // < Mpad: always there
+    if (residual) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int m = min(m0 + t * 16 + 4 * g + i, M - 1), n = min(n0 + r * 16 + ln, N - 1);
+                    res[r][t][i] = residual[(size_t)m * N + n];
+                }
+    }
 #pragma unroll
     for (int r = 0; r < R; r++)
 #pragma unroll
         for (int t = 0; t < MT; t++)
 #pragma unroll
             for (int i = 0; i < 4; i++) {
-                const int m = m0 + t * 16 + 4 * g + i;
-                const int n = n0 + r * 16 + ln;
-                if (m < M && n < N) {
-                    if (partial) {
-                        partial[((size_t)ks * M + m) * N + n] = run[r][t][i];
-                    } else {
-                        float v = run[r][t][i] * pv.inv_scale[m];
-                        if (residual) v = residual[(size_t)m * N + n] + v;
-                        out[(size_t)m * N + n] = v;
-                    }
-                }
+                const int m = m0 + t * 16 + 4 * g + i, n = n0 + r * 16 + ln;
+                float v = __fmul_rn(run[r][t][i], inv[t][i]);
+                if (residual) v = __fadd_rn(res[r][t][i], v);
+                if (m < M && n < N) out[(size_t)m * N + n] = v;
             }
 }
 
