@@ -235,19 +235,23 @@ struct StepW {  // what one MFMA step needs from the weights
 // CHUNK_BYTES = raw bytes per weight row for 8 steps (256 elements); all are multiples of 16.
 struct PQ4_0 {
     static constexpr int CHUNK_BYTES = 144;
+    // 160-byte rows in LDS: 2-way bank conflicts on the 8-byte weight reads (a small part of the LDS
+    // traffic) in exchange for 52 KB per workgroup, so that three workgroups fit the CU's 160 KB
+    static constexpr int PITCH = 160;
+    static constexpr int MIN_WAVES = 3;
     static constexpr bool HAS_MIN = false;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 32 * 18; }
     static __device__ __forceinline__ StepW load(const uint8_t *base, int row_off, int step, int g) {
         const int bo = row_off + step * 18;
         const uint8_t *blk = base + bo;
         const uint32_t w = lds_u32_unaligned(base, bo + 2 + 4 * g);  // bytes 4g..4g+3
-        const half2v off = {(_Float16)1032.f, (_Float16)1032.f};
-        const uint32_t m = 0x000F000Fu, mg = 0x64006400u;
-        StepW r;
-        r.b = pack8(as_h2((w & m) | mg) - off,          // low nibbles of bytes 0,2  -> 4g, 4g+2
-                    as_h2(((w >> 4) & m) | mg) - off,   // high nibbles of bytes 0,2 -> 16+4g, 16+4g+2
-                    as_h2(((w >> 8) & m) | mg) - off,   // low nibbles of bytes 1,3  -> 4g+1, 4g+3
-                    as_h2(((w >> 12) & m) | mg) - off); // high nibbles of bytes 1,3 -> 16+4g+1, 16+4g+3
+        const half2v off = {(_Float16)1032.f, (_Float16)1032.f};  // 1024 + 8
+        const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu, c64 = 0x64646464u;
+        StepW r;  // byte b next to a 0x64 byte is the f16 1024 + b
+        r.b = pack8(as_h2(__builtin_amdgcn_perm(lo, c64, 0x00060004u)) - off,   // low nibbles of bytes 0,2  -> 4g, 4g+2
+                    as_h2(__builtin_amdgcn_perm(hi, c64, 0x00060004u)) - off,   // high nibbles of bytes 0,2 -> 16+4g, 16+4g+2
+                    as_h2(__builtin_amdgcn_perm(lo, c64, 0x00070005u)) - off,   // low nibbles of bytes 1,3  -> 4g+1, 4g+3
+                    as_h2(__builtin_amdgcn_perm(hi, c64, 0x00070005u)) - off);  // high nibbles of bytes 1,3 -> 16+4g+1, 16+4g+3
         r.d = h2f(*(const uint16_t *)blk);
         r.dm = 0.f;
         return r;
@@ -256,6 +260,8 @@ struct PQ4_0 {
 
 struct PQ8_0 {
     static constexpr int CHUNK_BYTES = 272;
+    static constexpr int PITCH = 304;  // (PITCH/4) % 8 == 4: 16 rows x 4 lane groups spread over all banks
+    static constexpr int MIN_WAVES = 2;
     static constexpr bool HAS_MIN = false;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 32 * 34; }
     static __device__ __forceinline__ StepW load(const uint8_t *base, int row_off, int step, int g) {
@@ -278,15 +284,17 @@ struct PQ8_0 {
 
 struct PQ4_K {
     static constexpr int CHUNK_BYTES = 144;  // one super-block = 8 sub-blocks of 32
+    static constexpr int PITCH = 160;
+    static constexpr int MIN_WAVES = 2;  // the min-term bookkeeping needs more registers than 3 waves leave
     static constexpr bool HAS_MIN = true;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 256 * 144; }
     static __device__ __forceinline__ StepW load(const uint8_t *base, int row_off, int j, int g) {
         const uint8_t *sb = base + row_off;
         const int gr = j >> 1, hi = j & 1;
         const uint32_t *qp = (const uint32_t *)(sb + 16 + 32 * gr);
-        const uint32_t w0 = qp[g] >> (4 * hi), w1 = qp[4 + g] >> (4 * hi);  // elements 4g.. and 16+4g..
+        const uint32_t w0 = (qp[g] >> (4 * hi)) & 0x0F0F0F0Fu, w1 = (qp[4 + g] >> (4 * hi)) & 0x0F0F0F0Fu;  // elements 4g.. and 16+4g..
         const half2v off = {(_Float16)1024.f, (_Float16)1024.f};
-        const uint32_t m = 0x000F000Fu, mg = 0x64006400u;
+        const uint32_t c64 = 0x64646464u;
         const uint8_t *q = sb + 4;
         uint32_t sc, mn;  // pkg/gguf/dequant.go:400-409
         if (j < 4) {
@@ -298,8 +306,8 @@ struct PQ4_K {
         }
         const uint32_t hd = *(const uint32_t *)sb;
         StepW r;
-        r.b = pack8(as_h2((w0 & m) | mg) - off, as_h2((w1 & m) | mg) - off, as_h2(((w0 >> 8) & m) | mg) - off,
-                    as_h2(((w1 >> 8) & m) | mg) - off);
+        r.b = pack8(as_h2(__builtin_amdgcn_perm(w0, c64, 0x00060004u)) - off, as_h2(__builtin_amdgcn_perm(w1, c64, 0x00060004u)) - off,
+                    as_h2(__builtin_amdgcn_perm(w0, c64, 0x00070005u)) - off, as_h2(__builtin_amdgcn_perm(w1, c64, 0x00070005u)) - off);
         r.d = h2f((uint16_t)(hd & 0xFFFF)) * (float)sc;
         r.dm = h2f((uint16_t)(hd >> 16)) * (float)mn;
         return r;
@@ -326,11 +334,11 @@ __device__ __forceinline__ const uint8_t *seg_row(const Segs &sg, int n, size_t 
 
 // grid = (row groups of 64*R rows, KS k-slices, groups of MT activation tiles); block = 256.
 template <class F, int R, int MT>
-__global__ void __launch_bounds__(256) qgemm_kernel(Segs segs, PrepView pv, float *__restrict__ out,
+__global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, PrepView pv, float *__restrict__ out,
                                                     const float *__restrict__ residual, float *__restrict__ partial,
-                                                    int M, int Mpad, int N, int K, int slice_chunks) {
+                                                    int M, int Mpad, int N, int K, int n_slices, int flags) {
     constexpr int ROWS_W = 16 * R;
-    constexpr int PITCH = F::CHUNK_BYTES + 32;  // (PITCH/4) % 8 == 4: 16 rows x 4 lane groups spread over all banks
+    constexpr int PITCH = F::PITCH;
     constexpr int WPIECES = ROWS_W * (F::CHUNK_BYTES / 16);
     constexpr int WNL = (WPIECES + 63) / 64;
     constexpr int APIECES = CH * MT * 2 * 64;  // 16-byte pieces of one activation chunk
@@ -347,8 +355,10 @@ __global__ void __launch_bounds__(256) qgemm_kernel(Segs segs, PrepView pv, floa
     const size_t row_bytes = F::row_bytes(K);
     const int steps_total = K / 32;
     const int n_chunks = (steps_total + CH - 1) / CH;
-    const int c_begin = ks * slice_chunks;
-    const int c_end = min(c_begin + slice_chunks, n_chunks);
+    // balanced slices: the first n_chunks % n_slices slices hold one chunk more
+    const int sl_base = n_chunks / n_slices, sl_rem = n_chunks % n_slices;
+    const int c_begin = ks * sl_base + min(ks, sl_rem);
+    const int c_end = c_begin + sl_base + (ks < sl_rem ? 1 : 0);
 
     float4v run[R][MT];
 #pragma unroll
@@ -388,15 +398,9 @@ __global__ void __launch_bounds__(256) qgemm_kernel(Segs segs, PrepView pv, floa
             if (pc < WPIECES) *(u32x4 *)(&w_lds[wave][row * PITCH + col * 16]) = w_stage[i];
         }
     };
-
-    if (c_begin < c_end) fetch(c_begin);
-    for (int chunk = c_begin; chunk < c_end; chunk++) {
-        __syncthreads();  // previous chunk's reads are done
-        commit();
-        __syncthreads();
-        if (chunk + 1 < c_end) fetch(chunk + 1);  // in flight while this chunk is computed
+    auto compute = [&](int chunk) __attribute__((always_inline)) {
         const int s0 = chunk * CH;
-#pragma unroll 2
+#pragma unroll
         for (int s = 0; s < CH; s++) {
             half8 ah[MT], al[MT];
 #pragma unroll
@@ -423,49 +427,71 @@ __global__ void __launch_bounds__(256) qgemm_kernel(Segs segs, PrepView pv, floa
                 }
             }
         }
+    };
+
+    if (c_begin < c_end) fetch(c_begin);
+    for (int chunk = c_begin; chunk < c_end; chunk++) {
+        __syncthreads();  // previous chunk's reads are done
+        commit();
+        __syncthreads();
+        if (chunk + 1 < c_end) fetch(chunk + 1);  // in flight while this chunk is computed
+        compute(chunk);
     }
 
-    // lane (g, ln) of tile (r, t) holds C[m = m0 + 16t + 4g + i][n = n0 + 16r + ln], i = 0..3.
-    // Loads use clamped indices and come first, so they are all in flight together; only stores are predicated.
-    if (partial) {
-#pragma unroll
-        for (int r = 0; r < R; r++)
-#pragma unroll
-            for (int t = 0; t < MT; t++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int m = m0 + t * 16 + 4 * g + i, n = n0 + r * 16 + ln;
-                    if (m < M && n < N) partial[((size_t)ks * M + m) * N + n] = run[r][t][i];
-                }
-        return;
-    }
-    float inv[MT][4], res[R][MT][4];
-#pragma unroll
-    for (int t = 0; t < MT; t++)
-#pragma unroll
-        for (int i = 0; i < 4; i++) inv[t][i] = pv.inv_scale[m0 + t * 16 + 4 * g + i];  // < Mpad: always there
-    if (residual) {
-#pragma unroll
-        for (int r = 0; r < R; r++)
-#pragma unroll
-            for (int t = 0; t < MT; t++)
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int m = min(m0 + t * 16 + 4 * g + i, M - 1), n = min(n0 + r * 16 + ln, N - 1);
-                    res[r][t][i] = residual[(size_t)m * N + n];
-                }
-    }
+    // lane (g, ln) of tile (r, t) holds C[m = m0 + 16t + 4g + i][n = n0 + 16r + ln], i = 0..3. Each wave
+    // transposes its [16*MT x ROWS_W] block through LDS (the activation buffer is free now) so that global
+    // memory sees 16-byte accesses covering whole 128-byte row segments.
+    constexpr int TP = ROWS_W + 4;  // floats per transposed row: rows 4 apart land 16 banks apart
+    static_assert(4 * 16 * MT * TP * 4 <= (int)sizeof(a_lds), "transpose area must fit the activation buffer");
+    __syncthreads();  // every wave is done reading a_lds
+    float *T = (float *)a_lds + wave * (16 * MT * TP);
 #pragma unroll
     for (int r = 0; r < R; r++)
 #pragma unroll
         for (int t = 0; t < MT; t++)
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int m = m0 + t * 16 + 4 * g + i, n = n0 + r * 16 + ln;
-                float v = __fmul_rn(run[r][t][i], inv[t][i]);
-                if (residual) v = __fadd_rn(res[r][t][i], v);
-                if (m < M && n < N) out[(size_t)m * N + n] = v;
+            for (int i = 0; i < 4; i++) T[(t * 16 + 4 * g + i) * TP + r * 16 + ln] = run[r][t][i];
+    __syncthreads();
+    constexpr int LPR = ROWS_W / 4;   // lanes per row of the block
+    constexpr int RPI = 64 / LPR;     // rows per access
+    const bool vec = (flags & 1) != 0;  // N % 4 == 0 and 16-byte aligned bases
+    const int nl = (lane % LPR) * 4, n = n0 + nl;
+#pragma unroll
+    for (int j = 0; j < 16 * MT / RPI; j++) {
+        const int ml = j * RPI + lane / LPR, m = m0 + ml;
+        const float4 c = *(const float4 *)(T + ml * TP + nl);
+        float v[4] = {c.x, c.y, c.z, c.w};
+        if (m >= M || n >= N) continue;
+        if (partial) {
+            float *dst = partial + ((size_t)ks * M + m) * N + n;
+            if (vec) {
+                *(float4 *)dst = c;
+            } else {
+                for (int e = 0; e < 4; e++)
+                    if (n + e < N) dst[e] = v[e];
             }
+            continue;
+        }
+        const float inv = pv.inv_scale[m];
+        float *dst = out + (size_t)m * N + n;
+        const float *rs = residual ? residual + (size_t)m * N + n : nullptr;
+        if (vec) {
+            float4 o;
+            o.x = __fmul_rn(v[0], inv); o.y = __fmul_rn(v[1], inv); o.z = __fmul_rn(v[2], inv); o.w = __fmul_rn(v[3], inv);
+            if (rs) {
+                const float4 q = *(const float4 *)rs;
+                o.x = __fadd_rn(q.x, o.x); o.y = __fadd_rn(q.y, o.y); o.z = __fadd_rn(q.z, o.z); o.w = __fadd_rn(q.w, o.w);
+            }
+            *(float4 *)dst = o;
+        } else {
+            for (int e = 0; e < 4; e++)
+                if (n + e < N) {
+                    float o = __fmul_rn(v[e], inv);
+                    if (rs) o = __fadd_rn(rs[e], o);
+                    dst[e] = o;
+                }
+        }
+    }
 }
 
 // out[m][n] = residual + inv_scale[m] * (P[0] + P[1] + ... + P[KS-1]) in that order.
@@ -783,19 +809,22 @@ int prep_begin(vx_backend *be, int m, int k, PrepView *pv) {
     return VX_OK;
 }
 
-int gemm_target_wgs() {
+// Workgroups the GEMM aims to keep resident: three per compute unit (VEXEL_HIP_GEMM_WGS overrides).
+int gemm_target_wgs(vx_backend *be) {
     static int v = 0;
     if (v == 0) {
         const char *e = getenv("VEXEL_HIP_GEMM_WGS");
         v = e ? atoi(e) : 0;
-        if (v <= 0) v = 512;
+        if (v <= 0) {
+            int cus = 0;
+            if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0)
+                cus = 256;
+            v = 3 * cus;
+        }
     }
     return v;
 }
 
-// Launches the MFMA GEMM of the prepared activation against the segments. When `to_partials` (or when
-// more than one K slice is used) the raw sums go to be->part_ws as P[ks][M][N] and *ks_out slices must
-// be added by the consumer; otherwise out = residual + inv_scale * sums is written directly.
 // Grows the prepared-activation workspace for an [m, kmax] activation now, so that later prepares
 // of narrower activations inside one fused sequence cannot reallocate it (and lose the row scales).
 int prep_reserve(vx_backend *be, int m, int kmax) {
@@ -813,15 +842,21 @@ int launch_gemm(vx_backend *be, const Segs &segs, int N, float *out, const float
     const int rg = ceil_div(N, 64 * R);
     const int mgroups = mpad <= 16 ? 1 : mpad / 32;
     const int n_chunks = ceil_div(K / 32, CH);
-    // enough workgroups to fill 256 CUs, at least 2 chunks per slice; depends on (N, K) only when M <= 32
+    // Split K only as far as it takes to put about three workgroups on every CU, and never below four
+    // chunks per slice: every extra slice costs a [M,N] float32 round trip through memory, which writes
+    // far slower than it reads. The count depends on (N, K) and the device only, never on M: a row has the
+    // same bits alone or in a batch.
     int ks = 1;
     if (mgroups == 1) {
-        ks = ceil_div(gemm_target_wgs(), rg);
-        if (ks > n_chunks / 2) ks = n_chunks / 2;
+        static int min_chunks = 0;
+        if (min_chunks == 0) {
+            const char *e = getenv("VEXEL_HIP_GEMM_MIN_CHUNKS");
+            min_chunks = e && atoi(e) > 0 ? atoi(e) : 4;
+        }
+        ks = gemm_target_wgs(be) / rg;
+        if (ks > n_chunks / min_chunks) ks = n_chunks / min_chunks;
         if (ks < 1) ks = 1;
     }
-    const int slice = ceil_div(n_chunks, ks);
-    ks = ceil_div(n_chunks, slice);
     float *partial = nullptr;
     if (ks > 1 || to_partials) {
         const size_t need = (size_t)ks * M * N * sizeof(float);
@@ -830,10 +865,12 @@ int launch_gemm(vx_backend *be, const Segs &segs, int N, float *out, const float
         partial = (float *)be->part_ws;
     }
     dim3 grid(rg, ks, mgroups);
+    const bool vec = N % 4 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)residual % 16) == 0;
+    const int flags = vec ? 1 : 0;
     if (mpad <= 16)
-        qgemm_kernel<F, R, 1><<<grid, 256, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slice);
+        qgemm_kernel<F, R, 1><<<grid, 256, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, ks, flags);
     else
-        qgemm_kernel<F, R, 2><<<grid, 256, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slice);
+        qgemm_kernel<F, R, 2><<<grid, 256, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, ks, flags);
     VX_CHECK_LAUNCH();
     if (ks_out) *ks_out = ks;
     if (partial && !to_partials) {
