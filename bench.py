@@ -13,6 +13,7 @@ Prints ONE JSON line. The synthetic weights and KV contents are generated on the
 libvexel_synth.so (benchmark support built next to the backend); no torch in this process.
 """
 import argparse
+import ctypes as C
 import json
 import math
 import os
@@ -31,6 +32,11 @@ BATCH = 32
 BLOCK = 16
 
 
+# HBM bytes per algorithmic byte of the attention launch, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs
+# scaled by a plain copy of known size (summary: profiles/paged_decode_attention_7b_x32_hbm_traffic.txt).
+ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.012
+
+
 def ragged_contexts(seed=0, n=BATCH):
     rng = np.random.default_rng(seed)
     ctx = np.exp(rng.normal(math.log(1024.0), 0.6, n))
@@ -39,13 +45,13 @@ def ragged_contexts(seed=0, n=BATCH):
 
 def load_synth():
     """libvexel_synth.so: device-side generators of the synthetic weights and KV (benchmark support)."""
-    import ctypes as C
     path = os.path.join(ROOT, "vexel_amd", "libvexel_synth.so")
     if not os.path.exists(path):
         raise RuntimeError("%s is missing: run `python -m vexel_amd.build`" % path)
     s = C.CDLL(path)
     s.vxs_gaussian_quant.argtypes = [C.c_int, C.c_void_p, C.c_int64, C.c_float, C.c_uint64]
     s.vxs_gaussian_f16.argtypes = [C.c_void_p, C.c_int64, C.c_float, C.c_uint64]
+    s.vxs_plain_copy.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
     return s
 
 
@@ -187,6 +193,20 @@ def cpu_baseline(be, mr, ctx, c, sample_layers=2, head_rows=2000):
                        % (sample_layers, c["num_layers"], head_rows, c["vocab"], L, os.cpu_count()))
 
 
+def counter_probe(be, mr, ctx, c, layers):
+    """Workload for hardware-counter runs: plain_copy_kernel moves 1 GiB (known traffic, the scale for
+    FETCH_SIZE / WRITE_SIZE), then the attention kernel runs 8 times on the benchmark contexts."""
+    synth = load_synth()
+    n = 1 << 30
+    src, dst = be.alloc_permanent(n), be.alloc_permanent(n)
+    rc = synth.vxs_plain_copy(C.c_void_p(dst), C.c_void_p(src), C.c_int64(n))
+    if rc:
+        raise RuntimeError("plain copy failed: %d" % rc)
+    ms = time_attention_kernel(be, mr, ctx, c, layers, reps=8)
+    print(json.dumps({"probe": "plain_copy_kernel 1 GiB + 8 attention launches", "attention_bytes": attention_bytes(ctx, c),
+                      "attention_ms": ms}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -195,6 +215,8 @@ def main():
     ap.add_argument("--layers", type=int, default=CFG["num_layers"], help="debug only: fewer layers is NOT the benchmark")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--counter-probe", action="store_true",
+                    help="for rocprofv3 --pmc runs: one 1 GiB plain copy and 8 attention launches, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -205,6 +227,9 @@ def main():
     c = dict(CFG)
     c["num_layers"] = args.layers
     mr, ids = build_model(be, ctx, args.steps + args.warmup + 8, args.layers)
+    if args.counter_probe:
+        counter_probe(be, mr, ctx, c, args.layers)
+        return
     first = np.random.default_rng(3).integers(0, c["vocab"], BATCH).astype(np.int32)
     use_graph = not args.no_graph
     # warmup (untimed): first call runs one eager step, captures the graph, replays the rest
@@ -236,7 +261,7 @@ def main():
                    "global_batch": BATCH},
         "roofline": {"bound": "hbm", "kernel": "paged_decode_f16_kernel<128,1> (+paged_merge_kernel)",
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": None, "bytes_per_launch": attn_bytes, "ms_per_launch": attn_ms},
+                     "traffic": ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE * attn_bytes, "bytes_per_launch": attn_bytes, "ms_per_launch": attn_ms},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(be, mr, ctx_now, c)

@@ -97,7 +97,24 @@ __global__ void gaussian_f16_kernel(_Float16 *dst, int64_t npairs, float stdv, u
 
 }  // namespace
 
+// Plain 16-byte-per-lane copy: a kernel of known traffic (bytes read = bytes written = n16*16) against
+// which hardware counters are calibrated.
+__global__ void plain_copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, int64_t n16) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n16) dst[i] = src[i];
+}
+
 extern "C" {
+
+// Copies `bytes` (a multiple of 16) with plain_copy_kernel. Returns 0 or a hipError_t value.
+int vxs_plain_copy(void *dst, const void *src, int64_t bytes) {
+    const int64_t n16 = bytes / 16;
+    if (n16 <= 0) return 0;
+    plain_copy_kernel<<<(unsigned)((n16 + 255) / 256), 256>>>((const uint4 *)src, (uint4 *)dst, n16);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    return (int)hipDeviceSynchronize();
+}
 
 // fmt: 1 = Q4_0, 2 = Q8_0. Returns 0 or a hipError_t value.
 int vxs_gaussian_quant(int fmt, void *dst, int64_t nblocks, float stdv, uint64_t seed) {
