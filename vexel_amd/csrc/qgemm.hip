@@ -235,9 +235,9 @@ struct StepW {  // what one MFMA step needs from the weights
 // CHUNK_BYTES = raw bytes per weight row for 8 steps (256 elements); all are multiples of 16.
 struct PQ4_0 {
     static constexpr int CHUNK_BYTES = 144;
-    // 160-byte rows in LDS: 2-way bank conflicts on the 8-byte weight reads (a small part of the LDS
-    // traffic) in exchange for 52 KB per workgroup, so that three workgroups fit the CU's 160 KB
-    static constexpr int PITCH = 160;
+    // Rows sit back to back in LDS: 144 bytes = 36 dwords, and 36*row mod 64 takes 16 distinct multiples of 4
+    // for the 16 rows of a tile, so the 4 lane groups of every row read 64 different banks.
+    static constexpr int PITCH = 144;
     static constexpr int MIN_WAVES = 3;
     static constexpr bool HAS_MIN = false;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 32 * 18; }
@@ -260,7 +260,7 @@ struct PQ4_0 {
 
 struct PQ8_0 {
     static constexpr int CHUNK_BYTES = 272;
-    static constexpr int PITCH = 304;  // (PITCH/4) % 8 == 4: 16 rows x 4 lane groups spread over all banks
+    static constexpr int PITCH = 272;  // 68 dwords: (PITCH/4) % 8 == 4, conflict free like Q4_0's 36
     static constexpr int MIN_WAVES = 2;
     static constexpr bool HAS_MIN = false;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 32 * 34; }
@@ -284,7 +284,7 @@ struct PQ8_0 {
 
 struct PQ4_K {
     static constexpr int CHUNK_BYTES = 144;  // one super-block = 8 sub-blocks of 32
-    static constexpr int PITCH = 160;
+    static constexpr int PITCH = 144;
     static constexpr int MIN_WAVES = 2;  // the min-term bookkeeping needs more registers than 3 waves leave
     static constexpr bool HAS_MIN = true;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 256 * 144; }
@@ -344,7 +344,7 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
     constexpr int APIECES = CH * MT * 2 * 64;  // 16-byte pieces of one activation chunk
     constexpr int ANL = APIECES / 256;
     __shared__ __attribute__((aligned(16))) half8 a_lds[APIECES];
-    __shared__ __attribute__((aligned(16))) uint8_t w_lds[4][ROWS_W * PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t w_lds[4][ROWS_W * PITCH + 16];  // +16: the unaligned dword read may touch 4 bytes past the last row
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int ln = lane & 15, g = lane >> 4;
