@@ -116,8 +116,9 @@ def attention_bytes(ctx_lens, c):
 
 
 def time_attention_kernel(be, mr, ctx_now, c, layers, reps):
-    """Average duration of one ragged paged-attention launch (split-KV kernel + merge), HIP events on
-    the backend stream, cycling over the layers' pools so every launch streams from HBM."""
+    """Average duration of one launch of the ragged paged-attention kernel, HIP events on the backend stream,
+    cycling over the layers' pools so every launch streams from HBM. The result is left in split form
+    (out = NULL), as in the decode step, where the next kernel merges the splits."""
     b = len(ctx_now)
     qd = c["num_heads"] * c["head_dim"]
     q = be.upload(np.random.default_rng(1).standard_normal((b, qd)).astype(np.float32), permanent=True)
@@ -133,7 +134,7 @@ def time_attention_kernel(be, mr, ctx_now, c, layers, reps):
 
     def run(n):
         for i in range(n):
-            be.sdpa_paged_decode_ragged(q, mr.kv_pool(i % layers), True, d_bt, d_len, out, b, mr.cfg.max_blocks_per_seq,
+            be.sdpa_paged_decode_ragged(q, mr.kv_pool(i % layers), True, d_bt, d_len, None, b, mr.cfg.max_blocks_per_seq,
                                         BLOCK, c["num_heads"], c["num_kv_heads"], c["head_dim"], scale, cap)
     run(layers)
     be.sync()
@@ -259,7 +260,7 @@ def main():
                                "ctx lognormal(median 1024, sigma 0.6) in [64,4096] seed 0, sum ctx %d, block 16, "
                                "greedy decode, hipGraph=%s" % (args.layers, sum(ctx_now), use_graph),
                    "global_batch": BATCH},
-        "roofline": {"bound": "hbm", "kernel": "paged_decode_f16_kernel<128,1> (+paged_merge_kernel)",
+        "roofline": {"bound": "hbm", "kernel": "paged_decode_f16_kernel<128,1>",
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE * attn_bytes, "bytes_per_launch": attn_bytes, "ms_per_launch": attn_ms},
     }

@@ -183,7 +183,8 @@ int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight,
                        int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta, float *q_out);
 
 /* x += attn*Wo^T; h = RMSNorm(x, ffn_norm_weight); x += (SiLU(h*W1^T) * (h*W3^T)) * W2^T
- * (runtime/block.go:981-1077), x [rows,hidden] updated in place. When next_norm_weight != NULL,
+ * (runtime/block.go:981-1077), x [rows,hidden] updated in place. attn may be NULL when the call follows a
+ * vx_sdpa_paged_decode_ragged with out = NULL for the same rows: the split-KV partials are merged here. When next_norm_weight != NULL,
  * RMSNorm(x, next_norm_weight) of the updated x is left prepared for the next vx_decode_attn_qkv
  * (x_prepared = 1) or vx_matmul_quant_prepared (the output head). */
 int vx_decode_ffn_supported(const vx_qweight *wo, const vx_qweight *w1, const vx_qweight *w3, const vx_qweight *w2);
@@ -202,7 +203,11 @@ int vx_rope_store_paged(vx_backend *be, float *q, const float *k, const float *v
 /* Ragged batched paged attention with all metadata on the device: block_tables is a
  * padded int32 [rows, max_blocks] matrix; sequence i uses row table_rows[i] (row i when
  * table_rows is NULL); kv_lens int32[batch]. One query per sequence. max_kv_len bounds
- * the launch (>= every kv_lens[i]). */
+ * the launch (>= every kv_lens[i]). With out = NULL the result stays in the backend as per-split partial
+ * sums for the next vx_decode_ffn(attn = NULL) to merge (one launch less); that form exists only where
+ * vx_sdpa_paged_decode_split_supported() is 1, otherwise the call returns VX_ERR_UNSUPPORTED. */
+int vx_sdpa_paged_decode_split_supported(int pool_is_f16, int block_size, int num_q_heads, int num_kv_heads,
+                                         int head_dim);
 int vx_sdpa_paged_decode_ragged(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
                                 const int32_t *block_tables, const int32_t *table_rows, const int32_t *kv_lens,
                                 float *out, int batch, int max_blocks, int block_size, int num_q_heads,

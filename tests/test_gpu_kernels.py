@@ -260,6 +260,50 @@ def test_fused_decode_blocks_equal_the_unfused_sequence(be, fmt, rows, hidden, f
     be.reset_pool()
 
 
+def test_decode_ffn_merges_split_attention(be):
+    """vx_sdpa_paged_decode_ragged(out = NULL) + vx_decode_ffn(attn = NULL) equals the merged attention output
+    fed to vx_decode_ffn (the split-KV partials are merged by the same formula inside the prepare kernel)."""
+    rng = np.random.default_rng(91)
+    fmt, rows, hidden, ffn = nx.FMT_Q4_0, 5, 512, 1024
+    hq, hk, d, bs, nblocks, eps = 8, 2, 64, 16, 160, 1e-5
+    dims = dict(wo=(hidden, hidden), w1=(ffn, hidden), w3=(ffn, hidden), w2=(hidden, ffn))
+    dW = {n: be.upload(qz.random_quant(fmt, rng, *dims[n])) for n in dims}
+    qw = {n: be.qweight(fmt, dW[n], *dims[n]) for n in dims}
+    assert be.lib_call("vx_sdpa_paged_decode_split_supported", 1, bs, hq, hk, d) == 1
+    lens = np.array([1, 16, 700, 513, 37], dtype=np.int32)          # several splits, block boundaries
+    max_blocks = 48
+    perm = rng.permutation(nblocks).astype(np.int32)
+    tables = np.zeros((rows, max_blocks), dtype=np.int32)
+    off = 0
+    for i, L in enumerate(lens):
+        nb = (L + bs - 1) // bs
+        tables[i, :nb] = perm[off:off + nb]
+        off += nb
+    pool = _make_pool(rng, True, nblocks, bs, hk, d)
+    q = rng.standard_normal((rows, hq * d)).astype(np.float32)
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    nw = rng.standard_normal(hidden).astype(np.float32)
+    dpool, dq, dt, dl, dnw = be.upload(pool), be.upload(q), be.upload(tables), be.upload(lens), be.upload(nw)
+    scale = 1.0 / math.sqrt(d)
+    dattn = be.alloc(rows * hidden * 4)
+    be.sdpa_paged_decode_ragged(dq, dpool, True, dt, dl, dattn, rows, max_blocks, bs, hq, hk, d, scale, max_blocks * bs)
+    dx1 = be.upload(x)
+    be.decode_ffn(dattn, dx1, qw["wo"], dnw, eps, qw["w1"], qw["w3"], qw["w2"], rows, None)
+    want = be.download(dx1, (rows, hidden), np.float32)
+    dx2 = be.upload(x)
+    be.sdpa_paged_decode_ragged(dq, dpool, True, dt, dl, None, rows, max_blocks, bs, hq, hk, d, scale, max_blocks * bs)
+    be.decode_ffn(None, dx2, qw["wo"], dnw, eps, qw["w1"], qw["w3"], qw["w2"], rows, None)
+    got = be.download(dx2, (rows, hidden), np.float32)
+    assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want).max())
+    from vexel_amd.backend import VexelError
+    with pytest.raises(VexelError):      # the pending split result was consumed
+        be.decode_ffn(None, dx2, qw["wo"], dnw, eps, qw["w1"], qw["w3"], qw["w2"], rows, None)
+    dpool32 = be.upload(_make_pool(rng, False, nblocks, bs, hk, d))
+    with pytest.raises(VexelError):      # no split form for an F32 pool
+        be.sdpa_paged_decode_ragged(dq, dpool32, False, dt, dl, None, rows, max_blocks, bs, hq, hk, d, scale, max_blocks * bs)
+    be.reset_pool()
+
+
 def test_matmul_quant_residual_and_shapes(be):
     rng = np.random.default_rng(11)
     for (m, n, k) in [(2, 33, 512), (32, 4096, 4096), (5, 100, 11008)]:

@@ -48,6 +48,10 @@ class HipBackend:
         if rc != 0:
             raise VexelError(rc, self._lib.vx_last_error().decode())
 
+    def lib_call(self, name, *args):
+        """Calls a C-ABI function that takes no backend handle and returns its int result."""
+        return getattr(self._lib, name)(*args)
+
     def call(self, name, *args):
         """Calls C-ABI function `name` with the backend handle prepended; raises on error."""
         self._ck(getattr(self._lib, name)(self._h, *args))

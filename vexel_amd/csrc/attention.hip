@@ -370,6 +370,16 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
                                                                 max_blocks, kv_lens, (float *)be->attn_ws, num_q_heads,
                                                                 num_kv_heads, scale, max_splits);
     VX_CHECK_LAUNCH();
+    be->split.batch = 0;
+    if (!out) {  // the caller merges: vx_decode_ffn(attn = NULL)
+        be->split.batch = batch;
+        be->split.num_q_heads = num_q_heads;
+        be->split.head_dim = D;
+        be->split.max_splits = max_splits;
+        be->split.tokens_per_split = TPW;
+        be->split.kv_lens = kv_lens;
+        return VX_OK;
+    }
     paged_merge_kernel<D><<<dim3(num_q_heads, batch), D, 0, be->stream>>>((const float *)be->attn_ws, kv_lens, out,
                                                                           num_q_heads, max_splits);
     VX_CHECK_LAUNCH();
@@ -403,6 +413,11 @@ int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16
     VX_HOT(128, 1) VX_HOT(128, 2) VX_HOT(128, 4) VX_HOT(128, 8)
     VX_HOT(64, 1) VX_HOT(64, 2) VX_HOT(64, 4) VX_HOT(64, 8)
 #undef VX_HOT
+    if (!out) {
+        set_error("vx_sdpa_paged_decode_ragged: out = NULL (split form) needs an F16 pool with 16-token blocks and a "
+                  "supported head geometry");
+        return VX_ERR_UNSUPPORTED;
+    }
     AttnParams p = {};
     p.q = q;
     p.out = out;
@@ -544,12 +559,19 @@ int vx_sdpa_paged_decode_ragged(vx_backend *be, const float *q, const void *kv_p
                                 int num_kv_heads, int head_dim, float scale, int max_kv_len) {
     int rc = enter(be);
     if (rc) return rc;
-    VX_REQUIRE(q && kv_pool && block_tables && kv_lens && out, "vx_sdpa_paged_decode_ragged: null pointer");
+    VX_REQUIRE(q && kv_pool && block_tables && kv_lens, "vx_sdpa_paged_decode_ragged: null pointer");
     VX_REQUIRE(max_kv_len <= max_blocks * block_size, "vx_sdpa_paged_decode_ragged: max_kv_len %d exceeds table capacity %d",
                max_kv_len, max_blocks * block_size);
     return run_ragged(be, q, kv_pool, pool_is_f16, nullptr, block_tables, table_rows, max_blocks, kv_lens, out, batch,
                       block_size,
                       num_q_heads, num_kv_heads, head_dim, scale, max_kv_len);
+}
+
+int vx_sdpa_paged_decode_split_supported(int pool_is_f16, int block_size, int num_q_heads, int num_kv_heads,
+                                         int head_dim) {
+    if (!pool_is_f16 || block_size != HOT_BS || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0) return 0;
+    const int G = num_q_heads / num_kv_heads;
+    return (head_dim == 128 || head_dim == 64) && (G == 1 || G == 2 || G == 4 || G == 8);
 }
 
 int vx_sdpa_paged_decode_multiquery(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,

@@ -61,6 +61,11 @@ struct vx_backend {
     void *part_ws = nullptr;     // split-K partial sums
     size_t part_ws_bytes = 0;
     void *attn_ws = nullptr;     // split-KV partial results
+    // attention left in split form by vx_sdpa_paged_decode_ragged(out = NULL), to be merged by vx_decode_ffn
+    struct {
+        int batch = 0, num_q_heads = 0, head_dim = 0, max_splits = 0, tokens_per_split = 0;
+        const int32_t *kv_lens = nullptr;
+    } split;
     size_t attn_ws_bytes = 0;
     void *misc_ws = nullptr;     // small device staging (pointer tables, argmax result)
     size_t misc_ws_bytes = 0;

@@ -70,7 +70,7 @@ __device__ __forceinline__ float sigmoid_ref(float v) { return 1.0f / (1.0f + (f
 //   PREP_SILU_MUL: y = (a*sigmoid(a)) * b       (backend/cpu/cpu.go:390-400), optional f32 copy to `fout`
 // STAGE: keep the row's output values in LDS between the two passes (K*4 bytes of dynamic LDS);
 // otherwise pass 2 recomputes them.
-constexpr int PREP_THREADS = 512;  // shared by every kernel that writes prepared tiles: the row statistics
+constexpr int PREP_THREADS = 1024;  // shared by every kernel that writes prepared tiles: the row statistics
                                     // are summed in an order that depends on it, and fused and unfused
                                     // producers must agree bit for bit
 
@@ -697,6 +697,83 @@ __global__ void __launch_bounds__(FP_THREADS) fused_prepare_kernel(float *__rest
     }
 }
 
+// Merges the split-KV attention partials (m, l, acc[D]) of row r (one sequence) exactly as the stand-alone merge
+// kernel does (out = sum_s acc_s*2^(m_s-M) / sum_s l_s*2^(m_s-M)) and prepares the [Hq*D] result as the Wo
+// projection's activation. grid = Mpad rows, block = PREP_THREADS, dynamic LDS = K floats.
+__global__ void __launch_bounds__(PREP_THREADS) merge_prepare_kernel(const float *__restrict__ part,
+                                                                     const int32_t *__restrict__ kv_lens, int M, int K,
+                                                                     int D, int max_splits, int tokens_per_split,
+                                                                     PrepView pv, int Mpad) {
+    extern __shared__ __attribute__((aligned(16))) float ybuf[];
+    __shared__ float sm[2 * (PREP_THREADS / 64)];
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const int mtiles = Mpad / 16, mt = r >> 4, ln = r & 15;
+    const int npairs = K / 8;
+    if (r >= M) {
+        const half8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+        for (int p = tid; p < npairs; p += PREP_THREADS) {
+            const int ks = p >> 2, g = p & 3;
+            half8 *t = pv.tiles + ((size_t)(ks * mtiles + mt) * 2) * 64 + g * 16 + ln;
+            t[0] = z;
+            t[64] = z;
+            if (g == 0) pv.bsum[(size_t)ks * Mpad + r] = 0.f;
+        }
+        if (tid == 0) pv.inv_scale[r] = 0.f;
+        return;
+    }
+    const int ns = (kv_lens[r] + tokens_per_split - 1) / tokens_per_split;
+    const int P = D + 2;
+    float amax = 0.f, ss = 0.f;
+    for (int k = tid * 4; k < K; k += PREP_THREADS * 4) {
+        const int h = k / D, d = k % D;
+        const float *pb = part + ((size_t)r * (K / D) + h) * max_splits * P;
+        float Mx = -INFINITY;
+        for (int s = 0; s < ns; s++) Mx = fmaxf(Mx, pb[(size_t)s * P]);
+        float L = 0.f, A[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < ns; s++) {
+            const float *ps = pb + (size_t)s * P;
+            const float f = exp2f(ps[0] - Mx);
+            L += ps[1] * f;
+            const float2 a = *(const float2 *)(ps + 2 + d), b = *(const float2 *)(ps + 4 + d);
+            A[0] += a.x * f; A[1] += a.y * f; A[2] += b.x * f; A[3] += b.y * f;
+        }
+        float y[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) y[e] = (L > 0.f) ? A[e] / L : 0.f;
+        *(float4 *)(ybuf + k) = make_float4(y[0], y[1], y[2], y[3]);
+        amax = fmaxf(amax, fmaxf(fmaxf(fabsf(y[0]), fabsf(y[1])), fmaxf(fabsf(y[2]), fabsf(y[3]))));
+    }
+    row_stats(amax, ss, sm);  // also orders the ybuf writes before pass 2
+    float s = 1.f, inv = 1.f;
+    if (amax > 0.f && amax < INFINITY) {
+        int ex;
+        (void)frexpf(amax, &ex);
+        s = ldexpf(1.f, 13 - ex);
+        inv = ldexpf(1.f, ex - 13);
+    }
+    if (tid == 0) pv.inv_scale[r] = inv;
+    for (int p = tid; p < npairs; p += PREP_THREADS) {
+        const int ks = p >> 2, g = p & 3;
+        const int k0 = ks * 32 + 4 * g;
+        const float4 xa = *(const float4 *)(ybuf + k0), xb = *(const float4 *)(ybuf + k0 + 16);
+        const float v[8] = {xa.x * s, xa.z * s, xb.x * s, xb.z * s, xa.y * s, xa.w * s, xb.y * s, xb.w * s};
+        half8 h, l;
+        float bs = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            h[i] = (_Float16)v[i];
+            l[i] = (_Float16)(v[i] - (float)h[i]);
+            bs += v[i];
+        }
+        half8 *t = pv.tiles + ((size_t)(ks * mtiles + mt) * 2) * 64 + g * 16 + ln;
+        t[0] = h;
+        t[64] = l;
+        bs += __shfl_xor(bs, 1, 64);
+        bs += __shfl_xor(bs, 2, 64);
+        if (g == 0) pv.bsum[(size_t)ks * Mpad + r] = bs;
+    }
+}
+
 // x <- x + inv_in * sum_ks P (residual add only; used after the last layer's down projection)
 __global__ void __launch_bounds__(256) add_partials_kernel(float *__restrict__ x, const float *__restrict__ P, int KS,
                                                            int M, int K, const float *__restrict__ inv_scale) {
@@ -1084,7 +1161,13 @@ int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight 
         set_error("vx_decode_ffn: weights have no fused MFMA path");
         return VX_ERR_UNSUPPORTED;
     }
-    VX_REQUIRE(attn && x && ffn_norm_weight && rows >= 1, "vx_decode_ffn: bad arguments");
+    VX_REQUIRE(x && ffn_norm_weight && rows >= 1, "vx_decode_ffn: bad arguments");
+    if (!attn) {
+        VX_REQUIRE(be->split.batch == rows && be->split.num_q_heads * be->split.head_dim == wo->k,
+                   "vx_decode_ffn: attn = NULL but no matching split-form attention result is pending "
+                   "(call vx_sdpa_paged_decode_ragged with out = NULL right before)");
+        VX_REQUIRE(be->split.head_dim % 4 == 0 && (size_t)wo->k * 4 <= 64 * 1024, "vx_decode_ffn: head geometry");
+    }
     VX_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)ffn_norm_weight % 16 == 0) && ((uintptr_t)next_norm_weight % 16 == 0),
                "vx_decode_ffn: unaligned pointer");
     const int hidden = wo->n, ffn = w1->n, mpad = mpad_for(rows);
@@ -1092,8 +1175,19 @@ int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight 
     rc = prep_reserve(be, rows, ffn > wo->k ? (ffn > hidden ? ffn : hidden) : (wo->k > hidden ? wo->k : hidden));
     if (rc) return rc;
     // attention output -> Wo -> partials
-    rc = vx_prepare_act(be, attn, rows, wo->k);
-    if (rc) return rc;
+    if (attn) {
+        rc = vx_prepare_act(be, attn, rows, wo->k);
+        if (rc) return rc;
+    } else {
+        PrepView pa;
+        rc = prep_begin(be, rows, wo->k, &pa);
+        if (rc) return rc;
+        merge_prepare_kernel<<<mpad, PREP_THREADS, (size_t)wo->k * 4, be->stream>>>(
+            (const float *)be->attn_ws, be->split.kv_lens, rows, wo->k, be->split.head_dim, be->split.max_splits,
+            be->split.tokens_per_split, pa, mpad);
+        VX_CHECK_LAUNCH();
+        be->split.batch = 0;
+    }
     const vx_qweight *a[1] = {wo};
     Segs segs = make_segs(a, 1, &ntot);
     rc = launch_gemm_fmt(be, wo->fmt, segs, ntot, nullptr, nullptr, true, rows, wo->k, &ks);

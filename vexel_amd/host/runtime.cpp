@@ -258,13 +258,18 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
         VXC(vx_rope_store_paged(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
                                 c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta));  // :858, :868
     }
+    const bool ffn_fused = m->fused && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
+                           vx_decode_ffn_supported(&w.wo, &w.w1, &w.w3, &w.w2);
+    // the fused tail can merge the attention's split-KV partials itself
+    const bool split = ffn_fused && (size_t)w.wo.k * 4 <= 64 * 1024 && c.head_dim % 4 == 0 &&
+                       vx_sdpa_paged_decode_split_supported(c.kv_fp16, c.block_size, c.num_heads, c.num_kv_heads, c.head_dim);
     VXC(vx_sdpa_paged_decode_ragged(m->be, m->q, m->kv[layer], c.kv_fp16, m->d_tables, m->d_slots, m->d_kv_lens,
-                                    m->attn, rows, c.max_blocks_per_seq, c.block_size, c.num_heads, c.num_kv_heads,
-                                    c.head_dim, scale, max_kv_len));                       // block.go:872
+                                    split ? nullptr : m->attn, rows, c.max_blocks_per_seq, c.block_size, c.num_heads,
+                                    c.num_kv_heads, c.head_dim, scale, max_kv_len));       // block.go:872
     *chained = false;
-    if (m->fused && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
-        vx_decode_ffn_supported(&w.wo, &w.w1, &w.w3, &w.w2)) {                            // block.go:981-1077
-        VXC(vx_decode_ffn(m->be, m->attn, m->x, &w.wo, w.ffn_norm, c.eps, &w.w1, &w.w3, &w.w2, rows, next_norm));
+    if (ffn_fused) {                                                                      // block.go:981-1077
+        VXC(vx_decode_ffn(m->be, split ? nullptr : m->attn, m->x, &w.wo, w.ffn_norm, c.eps, &w.w1, &w.w3, &w.w2, rows,
+                          next_norm));
         *chained = next_norm != nullptr;
         return VH_OK;
     }
