@@ -238,13 +238,23 @@ struct PQ4_0 {
     // Rows sit back to back in LDS: 144 bytes = 36 dwords, and 36*row mod 64 takes 16 distinct multiples of 4
     // for the 16 rows of a tile, so the 4 lane groups of every row read 64 different banks.
     static constexpr int PITCH = 144;
-    static constexpr int MIN_WAVES = 3;
+    static constexpr int MIN_WAVES = 2;
     static constexpr bool HAS_MIN = false;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 32 * 18; }
-    static __device__ __forceinline__ StepW load(const uint8_t *base, int row_off, int step, int g) {
-        const int bo = row_off + step * 18;
-        const uint8_t *blk = base + bo;
-        const uint32_t w = lds_u32_unaligned(base, bo + 2 + 4 * g);  // bytes 4g..4g+3
+    struct Raw { uint32_t lo, hi, sh; uint16_t d; };
+    // LDS reads of one step (no arithmetic on the loaded values): two dwords around the 4 nibble bytes, the scale
+    static __device__ __forceinline__ Raw read(const uint8_t *base, int row_off, int step, int g) {
+        const int bo = row_off + step * 18, off = bo + 2 + 4 * g;  // bytes 4g..4g+3 of the block
+        const uint32_t *w = (const uint32_t *)base;
+        Raw r;
+        r.lo = w[off >> 2];
+        r.hi = w[(off >> 2) + 1];
+        r.sh = (uint32_t)(off & 3);
+        r.d = *(const uint16_t *)(base + bo);
+        return r;
+    }
+    static __device__ __forceinline__ StepW unpack(const Raw &x, int) {
+        const uint32_t w = __builtin_amdgcn_alignbyte(x.hi, x.lo, x.sh);
         const half2v off = {(_Float16)1032.f, (_Float16)1032.f};  // 1024 + 8
         const uint32_t lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu, c64 = 0x64646464u;
         StepW r;  // byte b next to a 0x64 byte is the f16 1024 + b
@@ -252,7 +262,7 @@ struct PQ4_0 {
                     as_h2(__builtin_amdgcn_perm(hi, c64, 0x00060004u)) - off,   // high nibbles of bytes 0,2 -> 16+4g, 16+4g+2
                     as_h2(__builtin_amdgcn_perm(lo, c64, 0x00070005u)) - off,   // low nibbles of bytes 1,3  -> 4g+1, 4g+3
                     as_h2(__builtin_amdgcn_perm(hi, c64, 0x00070005u)) - off);  // high nibbles of bytes 1,3 -> 16+4g+1, 16+4g+3
-        r.d = h2f(*(const uint16_t *)blk);
+        r.d = h2f(x.d);
         r.dm = 0.f;
         return r;
     }
@@ -264,11 +274,22 @@ struct PQ8_0 {
     static constexpr int MIN_WAVES = 2;
     static constexpr bool HAS_MIN = false;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 32 * 34; }
-    static __device__ __forceinline__ StepW load(const uint8_t *base, int row_off, int step, int g) {
-        const int bo = row_off + step * 34;
-        const uint8_t *blk = base + bo;
-        const uint32_t w0 = lds_u32_unaligned(base, bo + 2 + 4 * g) ^ 0x80808080u;       // elements 4g..4g+3
-        const uint32_t w1 = lds_u32_unaligned(base, bo + 2 + 16 + 4 * g) ^ 0x80808080u;  // elements 16+4g..
+    struct Raw { uint32_t a0, a1, b0, b1, sh; uint16_t d; };
+    static __device__ __forceinline__ Raw read(const uint8_t *base, int row_off, int step, int g) {
+        const int bo = row_off + step * 34, off = bo + 2 + 4 * g;  // elements 4g..4g+3; 16+4g.. are 16 bytes on
+        const uint32_t *w = (const uint32_t *)base;
+        Raw r;
+        r.a0 = w[off >> 2];
+        r.a1 = w[(off >> 2) + 1];
+        r.b0 = w[(off >> 2) + 4];
+        r.b1 = w[(off >> 2) + 5];
+        r.sh = (uint32_t)(off & 3);
+        r.d = *(const uint16_t *)(base + bo);
+        return r;
+    }
+    static __device__ __forceinline__ StepW unpack(const Raw &x, int) {
+        const uint32_t w0 = __builtin_amdgcn_alignbyte(x.a1, x.a0, x.sh) ^ 0x80808080u;
+        const uint32_t w1 = __builtin_amdgcn_alignbyte(x.b1, x.b0, x.sh) ^ 0x80808080u;
         const half2v off = {(_Float16)1152.f, (_Float16)1152.f};  // 1024 + 128
         const uint32_t c64 = 0x64646464u;
         StepW r;
@@ -276,7 +297,7 @@ struct PQ8_0 {
                     as_h2(__builtin_amdgcn_perm(w1, c64, 0x00060004u)) - off,   // bytes 0,2 of w1
                     as_h2(__builtin_amdgcn_perm(w0, c64, 0x00070005u)) - off,   // bytes 1,3 of w0
                     as_h2(__builtin_amdgcn_perm(w1, c64, 0x00070005u)) - off);  // bytes 1,3 of w1
-        r.d = h2f(*(const uint16_t *)blk);
+        r.d = h2f(x.d);
         r.dm = 0.f;
         return r;
     }
@@ -288,28 +309,40 @@ struct PQ4_K {
     static constexpr int MIN_WAVES = 2;  // the min-term bookkeeping needs more registers than 3 waves leave
     static constexpr bool HAS_MIN = true;
     static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 256 * 144; }
-    static __device__ __forceinline__ StepW load(const uint8_t *base, int row_off, int j, int g) {
-        const uint8_t *sb = base + row_off;
-        const int gr = j >> 1, hi = j & 1;
-        const uint32_t *qp = (const uint32_t *)(sb + 16 + 32 * gr);
-        const uint32_t w0 = (qp[g] >> (4 * hi)) & 0x0F0F0F0Fu, w1 = (qp[4 + g] >> (4 * hi)) & 0x0F0F0F0Fu;  // elements 4g.. and 16+4g..
+    struct Raw { uint32_t w0, w1, hd, s0, s1, s2; };
+    static __device__ __forceinline__ Raw read(const uint8_t *base, int row_off, int j, int g) {
+        const uint32_t *sb = (const uint32_t *)(base + row_off);
+        const uint32_t *qp = sb + 4 + 8 * (j >> 1);
+        Raw r;
+        r.w0 = qp[g];      // elements 4g..4g+3 of both sub-blocks of the pair (low / high nibbles)
+        r.w1 = qp[4 + g];  // elements 16+4g..
+        r.hd = sb[0];      // d, dmin
+        r.s0 = sb[1];      // the 12 bytes of 6-bit scales and mins
+        r.s1 = sb[2];
+        r.s2 = sb[3];
+        return r;
+    }
+    static __device__ __forceinline__ StepW unpack(const Raw &x, int j) {
+        const uint32_t w0 = (x.w0 >> (4 * (j & 1))) & 0x0F0F0F0Fu, w1 = (x.w1 >> (4 * (j & 1))) & 0x0F0F0F0Fu;
         const half2v off = {(_Float16)1024.f, (_Float16)1024.f};
         const uint32_t c64 = 0x64646464u;
-        const uint8_t *q = sb + 4;
+        auto q = [&](int i) -> uint32_t {  // byte i of the scales field
+            const uint32_t wd = i < 4 ? x.s0 : (i < 8 ? x.s1 : x.s2);
+            return (wd >> (8 * (i & 3))) & 0xFFu;
+        };
         uint32_t sc, mn;  // pkg/gguf/dequant.go:400-409
         if (j < 4) {
-            sc = q[j] & 63;
-            mn = q[j + 4] & 63;
+            sc = q(j) & 63;
+            mn = q(j + 4) & 63;
         } else {
-            sc = (q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4);
-            mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+            sc = (q(j + 4) & 0x0F) | ((q(j - 4) >> 6) << 4);
+            mn = (q(j + 4) >> 4) | ((q(j) >> 6) << 4);
         }
-        const uint32_t hd = *(const uint32_t *)sb;
         StepW r;
         r.b = pack8(as_h2(__builtin_amdgcn_perm(w0, c64, 0x00060004u)) - off, as_h2(__builtin_amdgcn_perm(w1, c64, 0x00060004u)) - off,
                     as_h2(__builtin_amdgcn_perm(w0, c64, 0x00070005u)) - off, as_h2(__builtin_amdgcn_perm(w1, c64, 0x00070005u)) - off);
-        r.d = h2f((uint16_t)(hd & 0xFFFF)) * (float)sc;
-        r.dm = h2f((uint16_t)(hd >> 16)) * (float)mn;
+        r.d = h2f((uint16_t)(x.hd & 0xFFFF)) * (float)sc;
+        r.dm = h2f((uint16_t)(x.hd >> 16)) * (float)mn;
         return r;
     }
 };
@@ -398,35 +431,101 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
             if (pc < WPIECES) *(u32x4 *)(&w_lds[wave][row * PITCH + col * 16]) = w_stage[i];
         }
     };
-    auto compute = [&](int chunk) __attribute__((always_inline)) {
-        const int s0 = chunk * CH;
+    // One chunk = CH steps, software-pipelined by hand. A SIMD issues a wave's instructions in order and a
+    // 16x16x32 MFMA keeps the matrix pipe busy for 16 cycles, so eight MFMAs back to back stall the wave for
+    // most of a step while its ~60 vector instructions (nibble unpacking, block-scale FMAs) wait their turn.
+    // Each step therefore issues its MFMAs interleaved with vector work that does not depend on them: the
+    // scale FMAs of the previous step and the unpacking of the next step's weights, whose LDS reads were
+    // issued a step earlier. sched_group_barrier pins that interleaving.
+    struct StepA { half8 h[MT], l[MT]; };
+    auto lds_a = [&](int s) __attribute__((always_inline)) {
+        StepA a;
 #pragma unroll
-        for (int s = 0; s < CH; s++) {
-            half8 ah[MT], al[MT];
+        for (int t = 0; t < MT; t++) {
+            a.h[t] = a_lds[((s * MT + t) * 2 + 0) * 64 + lane];
+            a.l[t] = a_lds[((s * MT + t) * 2 + 1) * 64 + lane];
+        }
+        return a;
+    };
+    auto scale_add = [&](const float4v (&acc)[R][MT], const StepW (&w)[R], const float4v (&bs)[MT]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
 #pragma unroll
             for (int t = 0; t < MT; t++) {
-                ah[t] = a_lds[((s * MT + t) * 2 + 0) * 64 + lane];
-                al[t] = a_lds[((s * MT + t) * 2 + 1) * 64 + lane];
-            }
+                if (F::HAS_MIN) {
 #pragma unroll
-            for (int r = 0; r < R; r++) {
-                const StepW sw = F::load(&w_lds[wave][0], (r * 16 + ln) * PITCH, s, g);
+                    for (int i = 0; i < 4; i++) run[r][t][i] += w[r].d * acc[r][t][i] - w[r].dm * bs[t][i];
+                } else {
 #pragma unroll
-                for (int t = 0; t < MT; t++) {
-                    float4v acc = {0.f, 0.f, 0.f, 0.f};
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah[t], sw.b, acc, 0, 0, 0);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(al[t], sw.b, acc, 0, 0, 0);
-                    if (F::HAS_MIN) {
-                        const float4v bs = *(const float4v *)(pv.bsum + (size_t)(s0 + s) * Mpad + m0 + t * 16 + 4 * g);
-#pragma unroll
-                        for (int i = 0; i < 4; i++) run[r][t][i] += sw.d * acc[i] - sw.dm * bs[i];
-                    } else {
-#pragma unroll
-                        for (int i = 0; i < 4; i++) run[r][t][i] += sw.d * acc[i];
-                    }
+                    for (int i = 0; i < 4; i++) run[r][t][i] += w[r].d * acc[r][t][i];
                 }
             }
+    };
+    auto compute = [&](int chunk) __attribute__((always_inline)) {
+        const int s0 = chunk * CH;
+        const uint8_t *wl = &w_lds[wave][0];
+        StepA a_cur = lds_a(0), a_nxt = a_cur;
+        typename F::Raw raw_n[R], raw_nn[R];
+        StepW w_cur[R], w_nxt[R], w_old[R];
+        float4v acc_old[R][MT], bs_old[MT] = {}, bs_cur[MT] = {};
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            raw_n[r] = F::read(wl, (r * 16 + ln) * PITCH, 0, g);
+            w_old[r] = w_nxt[r] = w_cur[r] = F::unpack(raw_n[r], 0);
+            raw_nn[r] = raw_n[r] = F::read(wl, (r * 16 + ln) * PITCH, 1, g);
+#pragma unroll
+            for (int t = 0; t < MT; t++) acc_old[r][t] = (float4v){0.f, 0.f, 0.f, 0.f};
         }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < CH; s++) {
+            // LDS reads for later steps go out first
+            if (s + 1 < CH) a_nxt = lds_a(s + 1);
+            if (s + 2 < CH) {
+#pragma unroll
+                for (int r = 0; r < R; r++) raw_nn[r] = F::read(wl, (r * 16 + ln) * PITCH, s + 2, g);
+            }
+            if (F::HAS_MIN) {
+#pragma unroll
+                for (int t = 0; t < MT; t++) bs_cur[t] = *(const float4v *)(pv.bsum + (size_t)(s0 + s) * Mpad + m0 + t * 16 + 4 * g);
+            }
+            float4v acc[R][MT];
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int t = 0; t < MT; t++)
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur.h[t], w_cur[r].b, (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int t = 0; t < MT; t++)
+                    acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_cur.l[t], w_cur[r].b, acc[r][t], 0, 0, 0);
+            // vector work independent of this step's MFMAs
+            if (s > 0) scale_add(acc_old, w_old, bs_old);
+            if (s + 1 < CH) {
+#pragma unroll
+                for (int r = 0; r < R; r++) w_nxt[r] = F::unpack(raw_n[r], s + 1);
+            }
+            // one MFMA, then a share of the vector instructions
+#pragma unroll
+            for (int i = 0; i < 2 * R * MT; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                w_old[r] = w_cur[r];
+                w_cur[r] = w_nxt[r];
+                raw_n[r] = raw_nn[r];
+#pragma unroll
+                for (int t = 0; t < MT; t++) acc_old[r][t] = acc[r][t];
+            }
+#pragma unroll
+            for (int t = 0; t < MT; t++) bs_old[t] = bs_cur[t];
+            a_cur = a_nxt;
+        }
+        scale_add(acc_old, w_old, bs_old);
     };
 
     if (c_begin < c_end) fetch(c_begin);
