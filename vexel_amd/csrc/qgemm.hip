@@ -740,13 +740,30 @@ __global__ void __launch_bounds__(FP_THREADS) fused_prepare_kernel(float *__rest
             const float4 wv = *(const float4 *)(w + k);
             y[0] *= wv.x; y[1] *= wv.y; y[2] *= wv.z; y[3] *= wv.w;
         } else {
+            // two column groups per trip, their loads issued together: the trip count is what this
+            // latency-bound loop pays for (the second group is clamped and dropped past the row's end)
+            const int k2 = k + FP_THREADS * 4;
+            const bool has2 = k2 < K;
+            const int kb = has2 ? k2 : k;
             const float4 gt = psum4(P, KS, slice_elems, (size_t)r * ncols + k, inv_in);
             const float4 up = psum4(P, KS, slice_elems, (size_t)r * ncols + K + k, inv_in);
+            const float4 gt2 = psum4(P, KS, slice_elems, (size_t)r * ncols + kb, inv_in);
+            const float4 up2 = psum4(P, KS, slice_elems, (size_t)r * ncols + K + kb, inv_in);
             y[0] = __fmul_rn(__fmul_rn(gt.x, sigmoid_ref(gt.x)), up.x);
             y[1] = __fmul_rn(__fmul_rn(gt.y, sigmoid_ref(gt.y)), up.y);
             y[2] = __fmul_rn(__fmul_rn(gt.z, sigmoid_ref(gt.z)), up.z);
             y[3] = __fmul_rn(__fmul_rn(gt.w, sigmoid_ref(gt.w)), up.w);
             *(float4 *)(ybuf + k) = make_float4(y[0], y[1], y[2], y[3]);
+            if (has2) {
+                float z[4];
+                z[0] = __fmul_rn(__fmul_rn(gt2.x, sigmoid_ref(gt2.x)), up2.x);
+                z[1] = __fmul_rn(__fmul_rn(gt2.y, sigmoid_ref(gt2.y)), up2.y);
+                z[2] = __fmul_rn(__fmul_rn(gt2.z, sigmoid_ref(gt2.z)), up2.z);
+                z[3] = __fmul_rn(__fmul_rn(gt2.w, sigmoid_ref(gt2.w)), up2.w);
+                *(float4 *)(ybuf + k2) = make_float4(z[0], z[1], z[2], z[3]);
+                amax = fmaxf(amax, fmaxf(fmaxf(fabsf(z[0]), fabsf(z[1])), fmaxf(fabsf(z[2]), fabsf(z[3]))));
+            }
+            k += FP_THREADS * 4;  // the second group is done
         }
         amax = fmaxf(amax, fmaxf(fmaxf(fabsf(y[0]), fabsf(y[1])), fmaxf(fabsf(y[2]), fabsf(y[3]))));
     }
