@@ -194,6 +194,59 @@ def cpu_baseline(be, mr, ctx, c, sample_layers=2, head_rows=2000):
                        % (sample_layers, c["num_layers"], head_rows, c["vocab"], L, os.cpu_count()))
 
 
+def kernel_report(be):
+    """Per-kernel timings through the C ABI, inputs resident in HBM, HIP events on the backend stream. Every
+    weight shape cycles over enough distinct copies (> 400 MB) that nothing is served from the 256 MB
+    memory-side cache. Algorithmic bytes of a quantized matmul: N*K*bytes_per_element + M*K*4 + M*N*4."""
+    synth = load_synth()
+    bpe = {1: 18 / 32, 2: 34 / 32}
+    names = {1: "Q4_0", 2: "Q8_0"}
+    shapes = [("Q|K|V", 12288, 4096), ("Wo", 4096, 4096), ("gate|up", 22016, 4096), ("down", 4096, 11008),
+              ("lm_head", 32000, 4096)]
+    a = np.random.default_rng(0).standard_normal((32, 11008)).astype(np.float32)
+    da = be.upload(a, permanent=True)
+    print("%-8s %-5s %3s %6s %6s %9s %9s %7s" % ("matmul", "fmt", "M", "N", "K", "us/call", "GB/s", "of 8TB"))
+    for fmt in (1, 2):
+        for name, n, k in shapes:
+            rb = int(k * bpe[fmt])
+            copies = max(2, int(400e6 // (n * rb)) + 1)
+            ws = []
+            for i in range(copies):
+                p = be.alloc_permanent(n * rb)
+                rc = synth.vxs_gaussian_quant(fmt, p, n * (k // 32), 0.02, 77 + i)
+                if rc:
+                    raise RuntimeError("synthetic weight generation failed: %d" % rc)
+                ws.append(p)
+            for m in (1, 32):
+                out = be.alloc_permanent(m * n * 4)
+                be.prepare_act(da, m, k)
+                for w in ws[:2]:
+                    be.matmul_quant_prepared(fmt, w, out, None, m, n, k)
+                be.sync()
+                reps = 3
+                be.timer_start()
+                for _ in range(reps):
+                    for w in ws:
+                        be.matmul_quant_prepared(fmt, w, out, None, m, n, k)
+                us = be.timer_stop_ms() * 1e3 / (reps * copies)
+                nbytes = n * rb + m * k * 4 + m * n * 4
+                gbs = nbytes / us / 1e3
+                print("%-8s %-5s %3d %6d %6d %9.1f %9.0f %7.3f" % (name, names[fmt], m, n, k, us, gbs, gbs / HBM_PEAK_GBS))
+                be.free(out)
+            for w in ws:
+                be.free(w)
+    be.free(da)
+    # attention at the north-star contexts
+    ctx = ragged_contexts()
+    c = dict(CFG)
+    mr, ids = build_model(be, ctx, 8, 4)
+    ms = time_attention_kernel(be, mr, ctx, c, 4, reps=40)
+    nb = attention_bytes(ctx, c)
+    print("paged decode attention, 32 ragged sequences (sum ctx %d), one layer: %.1f us, %.0f GB/s, %.3f of 8 TB/s"
+          % (sum(ctx), ms * 1e3, nb / ms / 1e6, nb / ms / 1e6 / HBM_PEAK_GBS))
+    mr.close()
+
+
 def counter_probe(be, mr, ctx, c, layers):
     """Workload for hardware-counter runs: plain_copy_kernel moves 1 GiB (known traffic, the scale for
     FETCH_SIZE / WRITE_SIZE), then the attention kernel runs 8 times on the benchmark contexts."""
@@ -216,6 +269,9 @@ def main():
     ap.add_argument("--layers", type=int, default=CFG["num_layers"], help="debug only: fewer layers is NOT the benchmark")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--kernel-report", action="store_true",
+                    help="time the path's kernels one by one (quantized GEMM shapes per format, attention) and print a "
+                         "table of achieved GB/s against the 8 TB/s HBM peak, then exit")
     ap.add_argument("--counter-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: one 1 GiB plain copy and 8 attention launches, then exit")
     args = ap.parse_args()
@@ -224,6 +280,9 @@ def main():
         sys.exit(2)
     from vexel_amd.backend import HipBackend
     be = HipBackend(0)
+    if args.kernel_report:
+        kernel_report(be)
+        return
     ctx = ragged_contexts()
     c = dict(CFG)
     c["num_layers"] = args.layers

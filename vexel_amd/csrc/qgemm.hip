@@ -51,10 +51,11 @@ __device__ __forceinline__ float h2f(uint16_t h) {
 
 // ---------------------------------------------------------------- activation prepare
 // Workspace layout (be->gemm_ws): inv_scale[Mpad], then tiles [K/32][Mpad/16][2][64] half8,
-// then bsum[K/32][Mpad] (block sums of the scaled row, for Q4_K's min term).
+// then bsum[K/32][Mpad] (block sums of the scaled row, for Q4_K's min term), then cscale[K/256][Mpad].
 struct PrepView {
     half8 *tiles;
-    float *inv_scale;
+    float *inv_scale;  // [Mpad] row factor: multiplies the finished dot products of the row
+    float *cscale;     // [K/256][Mpad] factor of each 256-column chunk's partial dot product
     float *bsum;
 };
 
@@ -119,6 +120,7 @@ __global__ void __launch_bounds__(PREP_THREADS) prepare_kernel(const float *__re
             if (g == 0) pv.bsum[(size_t)ks * Mpad + r] = 0.f;
         }
         if (tid == 0) pv.inv_scale[r] = 0.f;
+        for (int c = tid; c < K / 256; c += blockDim.x) pv.cscale[(size_t)c * Mpad + r] = 0.f;
         return;
     }
     const float *ar = a + (size_t)r * K;
@@ -158,6 +160,7 @@ __global__ void __launch_bounds__(PREP_THREADS) prepare_kernel(const float *__re
         inv = ldexpf(1.f, ex - 13);
     }
     if (tid == 0) pv.inv_scale[r] = inv;
+    for (int c = tid; c < K / 256; c += blockDim.x) pv.cscale[(size_t)c * Mpad + r] = 1.f;
     // pass 2: one (kstep, g) pair per iteration = elements 4g..4g+3 and 16+4g..16+4g+3 of the block
     for (int p = tid; p < npairs; p += PREP_THREADS) {
         const int ks = p >> 2, g = p & 3;
@@ -401,6 +404,7 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
 
     half8 a_stage[ANL];
     u32x4 w_stage[WNL];
+    float4v cs_stage[MT], cs_cur[MT];  // the chunk's factors for this lane's rows m0 + 16t + 4g + (0..3)
     // K is a multiple of 256, so every chunk has CH full steps and CHUNK_BYTES bytes per row. Every load is
     // unconditional (addresses are clamped instead): a load under a branch makes the compiler wait for it
     // inside the branch, which serialises the whole prefetch.
@@ -412,6 +416,8 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
             const int l = p & 63, hl = (p >> 6) & 1, t = (p >> 7) % MT, s = p / (128 * MT);
             a_stage[i] = pv.tiles[((size_t)((s0 + s) * mtiles + mg * MT + t) * 2 + hl) * 64 + l];
         }
+#pragma unroll
+        for (int t = 0; t < MT; t++) cs_stage[t] = *(const float4v *)(pv.cscale + (size_t)chunk * Mpad + m0 + t * 16 + 4 * g);
         const size_t coff = (size_t)chunk * F::CHUNK_BYTES;
 #pragma unroll
         for (int i = 0; i < WNL; i++) {
@@ -422,6 +428,8 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
         }
     };
     auto commit = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < MT; t++) cs_cur[t] = cs_stage[t];
 #pragma unroll
         for (int i = 0; i < ANL; i++) a_lds[i * 256 + tid] = a_stage[i];
 #pragma unroll
@@ -447,6 +455,7 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
         }
         return a;
     };
+    float4v crun[R][MT];  // the chunk's own sum, folded into run with the chunk's factors at its end
     auto scale_add = [&](const float4v (&acc)[R][MT], const StepW (&w)[R], const float4v (&bs)[MT]) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < R; r++)
@@ -454,16 +463,20 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
             for (int t = 0; t < MT; t++) {
                 if (F::HAS_MIN) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) run[r][t][i] += w[r].d * acc[r][t][i] - w[r].dm * bs[t][i];
+                    for (int i = 0; i < 4; i++) crun[r][t][i] += w[r].d * acc[r][t][i] - w[r].dm * bs[t][i];
                 } else {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) run[r][t][i] += w[r].d * acc[r][t][i];
+                    for (int i = 0; i < 4; i++) crun[r][t][i] += w[r].d * acc[r][t][i];
                 }
             }
     };
     auto compute = [&](int chunk) __attribute__((always_inline)) {
         const int s0 = chunk * CH;
         const uint8_t *wl = &w_lds[wave][0];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++) crun[r][t] = (float4v){0.f, 0.f, 0.f, 0.f};
         StepA a_cur = lds_a(0), a_nxt = a_cur;
         typename F::Raw raw_n[R], raw_nn[R];
         StepW w_cur[R], w_nxt[R], w_old[R];
@@ -526,6 +539,12 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
             a_cur = a_nxt;
         }
         scale_add(acc_old, w_old, bs_old);
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) run[r][t][i] += cs_cur[t][i] * crun[r][t][i];
     };
 
     if (c_begin < c_end) fetch(c_begin);
@@ -722,6 +741,7 @@ __global__ void __launch_bounds__(FP_THREADS) fused_prepare_kernel(float *__rest
             if (g == 0) pv.bsum[(size_t)ks * Mpad + r] = 0.f;
         }
         if (tid == 0) pv.inv_scale[r] = 0.f;
+        for (int c = tid; c < K / 256; c += blockDim.x) pv.cscale[(size_t)c * Mpad + r] = 0.f;
         return;
     }
     const float inv_in = pv.inv_scale[r];
@@ -781,6 +801,7 @@ __global__ void __launch_bounds__(FP_THREADS) fused_prepare_kernel(float *__rest
         inv = ldexpf(1.f, ex - 13);
     }
     if (tid == 0) pv.inv_scale[r] = inv;
+    for (int c = tid; c < K / 256; c += blockDim.x) pv.cscale[(size_t)c * Mpad + r] = 1.f;
     for (int p = tid; p < npairs; p += FP_THREADS) {
         const int ks = p >> 2, g = p & 3;
         const int k0 = ks * 32 + 4 * g;
@@ -835,6 +856,7 @@ __global__ void __launch_bounds__(PREP_THREADS) merge_prepare_kernel(const float
             if (g == 0) pv.bsum[(size_t)ks * Mpad + r] = 0.f;
         }
         if (tid == 0) pv.inv_scale[r] = 0.f;
+        for (int c = tid; c < K / 256; c += blockDim.x) pv.cscale[(size_t)c * Mpad + r] = 0.f;
         return;
     }
     const int ns = (kv_lens[r] + tokens_per_split - 1) / tokens_per_split;
@@ -868,6 +890,7 @@ __global__ void __launch_bounds__(PREP_THREADS) merge_prepare_kernel(const float
         inv = ldexpf(1.f, ex - 13);
     }
     if (tid == 0) pv.inv_scale[r] = inv;
+    for (int c = tid; c < K / 256; c += blockDim.x) pv.cscale[(size_t)c * Mpad + r] = 1.f;
     for (int p = tid; p < npairs; p += PREP_THREADS) {
         const int ks = p >> 2, g = p & 3;
         const int k0 = ks * 32 + 4 * g;
@@ -986,6 +1009,7 @@ PrepView prep_view(vx_backend *be, int mpad, int k) {
     pv.inv_scale = (float *)base;
     pv.tiles = (half8 *)(base + (size_t)ceil_div(mpad, 64) * 64 * 4);
     pv.bsum = (float *)((char *)pv.tiles + prep_tiles_bytes(mpad, k));
+    pv.cscale = pv.bsum + (size_t)(k / 32) * mpad;
     return pv;
 }
 
@@ -993,7 +1017,8 @@ PrepView prep_view(vx_backend *be, int mpad, int k) {
 int prep_begin(vx_backend *be, int m, int k, PrepView *pv) {
     VX_REQUIRE(m >= 1 && k >= 256 && k % 256 == 0, "prepare: bad shape %dx%d (K must be a multiple of 256)", m, k);
     const int mpad = mpad_for(m);
-    const size_t need = prep_tiles_bytes(mpad, k) + (size_t)ceil_div(mpad, 64) * 64 * 4 + (size_t)(k / 32) * mpad * 4;
+    const size_t need = prep_tiles_bytes(mpad, k) + (size_t)ceil_div(mpad, 64) * 64 * 4 + (size_t)(k / 32) * mpad * 4 +
+                        (size_t)(k / 256) * mpad * 4;
     int rc = ensure_ws(be, &be->gemm_ws, &be->gemm_ws_bytes, need, "prepared activations");
     if (rc) return rc;
     *pv = prep_view(be, mpad, k);
@@ -1022,7 +1047,8 @@ int gemm_target_wgs(vx_backend *be) {
 // of narrower activations inside one fused sequence cannot reallocate it (and lose the row scales).
 int prep_reserve(vx_backend *be, int m, int kmax) {
     const int mpad = mpad_for(m);
-    const size_t need = prep_tiles_bytes(mpad, kmax) + (size_t)ceil_div(mpad, 64) * 64 * 4 + (size_t)(kmax / 32) * mpad * 4;
+    const size_t need = prep_tiles_bytes(mpad, kmax) + (size_t)ceil_div(mpad, 64) * 64 * 4 + (size_t)(kmax / 32) * mpad * 4 +
+                        (size_t)(kmax / 256) * mpad * 4;
     return ensure_ws(be, &be->gemm_ws, &be->gemm_ws_bytes, need, "prepared activations");
 }
 
