@@ -245,10 +245,12 @@ def test_fused_decode_blocks_equal_the_unfused_sequence(be, fmt, rows, hidden, f
                                    hq, hk, d, bs, theta, dq3)
                 be.decode_attn_qkv(dx3, dn1, eps, False, qw["wq"], qw["wk"], qw["wv"], rows, dpos, dslots, dpool4, f16,
                                    hq, hk, d, bs, theta, dq4)
-                assert np.array_equal(bits(be.download(dq3, (rows, hidden), np.float32)),
-                                      bits(be.download(dq4, (rows, hidden), np.float32)))
-                assert np.array_equal(bits(be.download(dpool3, pool.shape, pool.dtype)),
-                                      bits(be.download(dpool4, pool.shape, pool.dtype)))
+                # (the chained activation is prepared per 256-column chunk with 1/rms applied to the products,
+                # the fresh one per row with x/rms prepared: same values up to float32 rounding)
+                near(be.download(dq3, (rows, hidden), np.float32), be.download(dq4, (rows, hidden), np.float32),
+                     "q from the chained activation")
+                near(be.download(dpool3, pool.shape, pool.dtype), be.download(dpool4, pool.shape, pool.dtype),
+                     "pool from the chained activation")
             else:
                 from vexel_amd.backend import VexelError
                 with pytest.raises(VexelError):   # nothing was left prepared

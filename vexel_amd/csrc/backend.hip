@@ -77,6 +77,8 @@ int vx_backend_create(int device_id, vx_backend **out) {
     VX_CHECK_HIP(hipHostMalloc(&be->host_stage, be->host_stage_bytes, hipHostMallocDefault));
     be->misc_ws_bytes = 1 << 20;
     VX_CHECK_HIP(hipMalloc(&be->misc_ws, be->misc_ws_bytes));
+    VX_CHECK_HIP(hipMalloc(&be->prep_sync, VX_PREP_SYNC_BYTES));
+    VX_CHECK_HIP(hipMemset(be->prep_sync, 0, VX_PREP_SYNC_BYTES));  // arrival counters start at zero and reset themselves
     *out = be;
     return VX_OK;
 }
@@ -91,6 +93,7 @@ void vx_backend_destroy(vx_backend *be) {
     if (be->part_ws) (void)hipFree(be->part_ws);
     if (be->attn_ws) (void)hipFree(be->attn_ws);
     if (be->misc_ws) (void)hipFree(be->misc_ws);
+    if (be->prep_sync) (void)hipFree(be->prep_sync);
     if (be->host_stage) (void)hipHostFree(be->host_stage);
     if (be->ev0) (void)hipEventDestroy(be->ev0);
     if (be->ev1) (void)hipEventDestroy(be->ev1);

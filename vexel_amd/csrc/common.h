@@ -43,6 +43,11 @@ struct PoolChunk {
 
 }  // namespace vx
 
+// chunk-parallel prepares: up to 64 rows x 64 chunks of 256 columns; two [64][64] float arrays of per-chunk sums of squares
+#define VX_PREP_SYNC_ROWS 64
+#define VX_PREP_SYNC_CHUNKS 64
+#define VX_PREP_SYNC_BYTES (2 * VX_PREP_SYNC_CHUNKS * VX_PREP_SYNC_ROWS * 4)
+
 struct vx_backend {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -58,6 +63,10 @@ struct vx_backend {
     void *gemm_ws = nullptr;     // prepared (split, tiled) activations for the quantized GEMM
     size_t gemm_ws_bytes = 0;
     int prep_m = 0, prep_k = 0;  // shape of the activation currently prepared in gemm_ws
+    int rowfac_slot = 0;         // which of the two row-factor arrays at the head of gemm_ws is current
+    void *prep_sync = nullptr;   // per-chunk sums of squares of the chunk-parallel RMSNorm prepares (two slots)
+    int prep_norm_k = 0;         // > 0: the prepared activation is x*w of an RMSNorm over that many columns whose
+    float prep_norm_eps = 0.f;   //      1/rms is still to be taken from the current slot of prep_sync
     void *part_ws = nullptr;     // split-K partial sums
     size_t part_ws_bytes = 0;
     void *attn_ws = nullptr;     // split-KV partial results

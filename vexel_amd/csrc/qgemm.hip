@@ -725,7 +725,8 @@ constexpr int FP_THREADS = PREP_THREADS;
 template <int MODE>
 __global__ void __launch_bounds__(FP_THREADS) fused_prepare_kernel(float *__restrict__ x, const float *__restrict__ P,
                                                                    int KS, int M, int K, const float *__restrict__ w,
-                                                                   float eps, PrepView pv, int Mpad) {
+                                                                   float eps, PrepView pv, int Mpad,
+                                                                   const float *__restrict__ inv_in_rows) {
     extern __shared__ __attribute__((aligned(16))) float ybuf[];
     __shared__ float sm[2 * (FP_THREADS / 64)];
     const int r = blockIdx.x, tid = threadIdx.x;
@@ -744,7 +745,7 @@ __global__ void __launch_bounds__(FP_THREADS) fused_prepare_kernel(float *__rest
         for (int c = tid; c < K / 256; c += blockDim.x) pv.cscale[(size_t)c * Mpad + r] = 0.f;
         return;
     }
-    const float inv_in = pv.inv_scale[r];
+    const float inv_in = inv_in_rows[r];
     const int ncols = (MODE == FUSE_SILU_MUL) ? 2 * K : K;
     const size_t slice_elems = (size_t)M * ncols;
     float amax = 0.f, ss = 0.f;
@@ -913,6 +914,165 @@ __global__ void __launch_bounds__(PREP_THREADS) merge_prepare_kernel(const float
     }
 }
 
+// ---------------------------------------------------------------- chunk-parallel prepares (decode batches)
+// One wave per (256-column chunk, row): lane l owns columns 4l..4l+3 of the chunk. Nothing spans the row except
+// RMSNorm's sum of squares, which goes through per-chunk partial sums and an arrival counter: the last wave of
+// a row to arrive adds the partials in chunk order (so the result does not depend on who arrives last) and
+// writes the row factor 1/rms; nobody waits for anybody. The prepared values are x*w (not yet divided by rms)
+// scaled per chunk; the GEMM multiplies each chunk's dot product by cscale and the row's result by inv_scale.
+// The sums of squares of a row's chunks, from which whoever consumes the activation's products takes 1/rms.
+struct RowNorm {
+    const float *sspart;  // [VX_PREP_SYNC_CHUNKS][VX_PREP_SYNC_ROWS], NULL when the rows carry no pending RMSNorm
+    int n_chunks;
+    float inv_k, eps;
+};
+
+__device__ __forceinline__ float wave_max(float v) {
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+// Scales the wave's 256 values by a power of two chosen from their maximum, splits them hi + lo and writes the
+// MFMA-ready tiles, the block sums and the chunk factor of (row r, chunk c).
+__device__ __forceinline__ void write_chunk(const PrepView &pv, int r, int c, const float (&y)[4], int Mpad) {
+    const int lane = threadIdx.x & 63;
+    const float amax = wave_max(fmaxf(fmaxf(fabsf(y[0]), fabsf(y[1])), fmaxf(fabsf(y[2]), fabsf(y[3]))));
+    float s = 1.f, inv = 1.f;
+    if (amax > 0.f && amax < INFINITY) {
+        int ex;
+        (void)frexpf(amax, &ex);
+        s = ldexpf(1.f, 13 - ex);
+        inv = ldexpf(1.f, ex - 13);
+    }
+    if (lane == 0) pv.cscale[(size_t)c * Mpad + r] = inv;
+    // lane l = 8*step + 4*half + g holds block elements 16*half + 4g .. +3; slot order of lane group g is
+    // {4g, 4g+2, 16+4g, 16+4g+2, 4g+1, 4g+3, 16+4g+1, 16+4g+3}: the low-half lane fetches the high half's values
+    const float a[4] = {y[0] * s, y[1] * s, y[2] * s, y[3] * s};
+    float b[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) b[i] = __shfl_down(a[i], 4, 64);
+    float bs = a[0] + a[1] + a[2] + a[3];
+    bs += __shfl_xor(bs, 1, 64);
+    bs += __shfl_xor(bs, 2, 64);
+    bs += __shfl_xor(bs, 4, 64);
+    const int step = c * 8 + (lane >> 3), half = (lane >> 2) & 1, g = lane & 3;
+    if (half == 0) {
+        const float v[8] = {a[0], a[2], b[0], b[2], a[1], a[3], b[1], b[3]};
+        half8 h, l;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            h[i] = (_Float16)v[i];
+            l[i] = (_Float16)(v[i] - (float)h[i]);
+        }
+        const int mtiles = Mpad / 16, mt = r >> 4, ln = r & 15;
+        half8 *t = pv.tiles + ((size_t)(step * mtiles + mt) * 2) * 64 + g * 16 + ln;
+        t[0] = h;
+        t[64] = l;
+        if (g == 0) pv.bsum[(size_t)step * Mpad + r] = bs;
+    }
+}
+
+// Factor of row r's finished dot products: the stored row factor times, for a pending RMSNorm, 1/rms from the
+// chunks' sums of squares (added by a fixed butterfly over the wave, so every caller gets the same bits).
+// Must be called by all 64 lanes of a wave.
+__device__ __forceinline__ float row_factor(const float *__restrict__ inv_rows, const RowNorm &rn, int r) {
+    float f = inv_rows[r];
+    if (rn.sspart) {
+        const int lane = threadIdx.x & 63;
+        const float ss = wave_sum(lane < rn.n_chunks ? rn.sspart[lane * VX_PREP_SYNC_ROWS + r] : 0.f);
+        const float rms = (float)sqrt((double)(ss * rn.inv_k + rn.eps));  // backend/cpu/cpu.go:214
+        f = f / rms;
+    }
+    return f;
+}
+
+// Writes inv_scale[r] *= 1/rms for every row, for consumers that read plain row factors. grid = rows, block = 64.
+__global__ void __launch_bounds__(64) finalize_row_norm_kernel(float *__restrict__ inv_rows, RowNorm rn) {
+    const float f = row_factor(inv_rows, rn, blockIdx.x);
+    if (threadIdx.x == 0) inv_rows[blockIdx.x] = f;
+}
+
+// grid = (K/256, Mpad), block = 64.
+//   x_new = x + inv_in[r] * sum_s P[s][r][:]   (P may be NULL: x_new = x), x <- x_new when P is given,
+//   prepared <- x_new * w, its chunks' sums of squares to ss_out for the pending 1/rms (backend/cpu/cpu.go:200-220)
+__global__ void __launch_bounds__(64) chunk_add_norm_kernel(float *__restrict__ x, const float *__restrict__ P, int KS, int M,
+                                                            int K, const float *__restrict__ w, float eps, PrepView pv,
+                                                            int Mpad, const float *__restrict__ inv_in_rows, RowNorm rn_in,
+                                                            float *__restrict__ ss_out) {
+    const int c = blockIdx.x, r = blockIdx.y, lane = threadIdx.x;
+    const int k = c * 256 + lane * 4;
+    float y[4] = {0.f, 0.f, 0.f, 0.f};
+    float ss = 0.f;
+    if (r < M) {
+        float4 v = *(const float4 *)(x + (size_t)r * K + k);
+        if (P) {
+            const float4 d = psum4(P, KS, (size_t)M * K, (size_t)r * K + k, row_factor(inv_in_rows, rn_in, r));
+            v.x = __fadd_rn(v.x, d.x); v.y = __fadd_rn(v.y, d.y); v.z = __fadd_rn(v.z, d.z); v.w = __fadd_rn(v.w, d.w);
+            *(float4 *)(x + (size_t)r * K + k) = v;
+        }
+        ss = wave_sum(sumsq4(0.f, v.x, v.y, v.z, v.w));
+        const float4 wv = *(const float4 *)(w + k);
+        y[0] = v.x * wv.x; y[1] = v.y * wv.y; y[2] = v.z * wv.z; y[3] = v.w * wv.w;
+    }
+    write_chunk(pv, r, c, y, Mpad);
+    if (lane == 0) {
+        ss_out[c * VX_PREP_SYNC_ROWS + r] = ss;
+        if (c == 0) pv.inv_scale[r] = r < M ? 1.f : 0.f;
+    }
+}
+
+//   g = inv_in[r] * sum_s P[s][r][:K], u = inv_in[r] * sum_s P[s][r][K:2K], prepared <- (g*sigmoid(g)) * u, row factor 1
+__global__ void __launch_bounds__(64) chunk_silu_kernel(const float *__restrict__ P, int KS, int M, int K, PrepView pv, int Mpad,
+                                                        const float *__restrict__ inv_in_rows, RowNorm rn_in) {
+    const int c = blockIdx.x, r = blockIdx.y, lane = threadIdx.x;
+    const int k = c * 256 + lane * 4;
+    float y[4] = {0.f, 0.f, 0.f, 0.f};
+    if (r < M) {
+        const float inv_in = row_factor(inv_in_rows, rn_in, r);
+        const size_t slice = (size_t)M * 2 * K;
+        const float4 gt = psum4(P, KS, slice, (size_t)r * 2 * K + k, inv_in);
+        const float4 up = psum4(P, KS, slice, (size_t)r * 2 * K + K + k, inv_in);
+        y[0] = __fmul_rn(__fmul_rn(gt.x, sigmoid_ref(gt.x)), up.x);
+        y[1] = __fmul_rn(__fmul_rn(gt.y, sigmoid_ref(gt.y)), up.y);
+        y[2] = __fmul_rn(__fmul_rn(gt.z, sigmoid_ref(gt.z)), up.z);
+        y[3] = __fmul_rn(__fmul_rn(gt.w, sigmoid_ref(gt.w)), up.w);
+    }
+    write_chunk(pv, r, c, y, Mpad);
+    if (c == 0 && lane == 0) pv.inv_scale[r] = r < M ? 1.f : 0.f;
+}
+
+//   merged split-KV attention output of row r (as paged_merge_kernel computes it), row factor 1
+__global__ void __launch_bounds__(64) chunk_merge_kernel(const float *__restrict__ part, const int32_t *__restrict__ kv_lens,
+                                                         int M, int K, int D, int max_splits, int tokens_per_split,
+                                                         PrepView pv, int Mpad) {
+    const int c = blockIdx.x, r = blockIdx.y, lane = threadIdx.x;
+    const int k = c * 256 + lane * 4;
+    float y[4] = {0.f, 0.f, 0.f, 0.f};
+    if (r < M) {
+        const int ns = (kv_lens[r] + tokens_per_split - 1) / tokens_per_split;
+        const int P = D + 2, h = k / D, d = k % D;
+        const float *pb = part + ((size_t)r * (K / D) + h) * max_splits * P;
+        float Mx = -INFINITY;
+        for (int s = 0; s < ns; s++) Mx = fmaxf(Mx, pb[(size_t)s * P]);
+        float L = 0.f, A[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < ns; s++) {
+            const float *ps = pb + (size_t)s * P;
+            const float f = exp2f(ps[0] - Mx);
+            L += ps[1] * f;
+            const float2 a = *(const float2 *)(ps + 2 + d), b = *(const float2 *)(ps + 4 + d);
+            A[0] += a.x * f; A[1] += a.y * f; A[2] += b.x * f; A[3] += b.y * f;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; e++) y[e] = (L > 0.f) ? A[e] / L : 0.f;
+    }
+    write_chunk(pv, r, c, y, Mpad);
+    if (c == 0 && lane == 0) pv.inv_scale[r] = r < M ? 1.f : 0.f;
+}
+
 // x <- x + inv_in * sum_ks P (residual add only; used after the last layer's down projection)
 __global__ void __launch_bounds__(256) add_partials_kernel(float *__restrict__ x, const float *__restrict__ P, int KS,
                                                            int M, int K, const float *__restrict__ inv_scale) {
@@ -928,14 +1088,14 @@ __global__ void __launch_bounds__(256) add_partials_kernel(float *__restrict__ x
 // (metal_bridge_darwin.m:8607-8642) reading the fused Q|K|V projection from its split-K partials.
 // grid = (rows, head groups); thread = (pair j, head lane).
 template <bool F16>
-__global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, int M, const float *__restrict__ inv_scale,
+__global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, int M, const float *__restrict__ inv_scale, RowNorm rn,
                                            float *__restrict__ q_out, const int32_t *__restrict__ positions,
                                            const int32_t *__restrict__ slot_mapping, void *__restrict__ pool,
                                            int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta) {
     const int row = blockIdx.x, half = head_dim / 2;
     const int qd = num_q_heads * head_dim, kvd = num_kv_heads * head_dim, ncols = qd + 2 * kvd;
     const size_t slice_elems = (size_t)M * ncols;
-    const float inv = inv_scale[row];
+    const float inv = row_factor(inv_scale, rn, row);  // every wave of the block, before any lane leaves
     const int pos = positions[row], slot = slot_mapping[row];
     const int blk = slot / block_size, off = slot % block_size;
     const size_t part = (size_t)block_size * kvd;
@@ -1005,9 +1165,12 @@ PrepView prep_view(vx_backend *be, int mpad, int k) {
     PrepView pv;
     // the row scales sit first, at an address that does not depend on K: a fused consumer reads the
     // scales of the activation that produced its input while it prepares an activation of another width
+    // two arrays, used alternately (prep_begin switches): the kernel that prepares the next activation writes
+    // the new factors while it still reads the previous ones
     char *base = (char *)be->gemm_ws;
-    pv.inv_scale = (float *)base;
-    pv.tiles = (half8 *)(base + (size_t)ceil_div(mpad, 64) * 64 * 4);
+    const size_t rf = (size_t)ceil_div(mpad, 64) * 64 * 4;
+    pv.inv_scale = (float *)(base + be->rowfac_slot * rf);
+    pv.tiles = (half8 *)(base + 2 * rf);
     pv.bsum = (float *)((char *)pv.tiles + prep_tiles_bytes(mpad, k));
     pv.cscale = pv.bsum + (size_t)(k / 32) * mpad;
     return pv;
@@ -1017,10 +1180,12 @@ PrepView prep_view(vx_backend *be, int mpad, int k) {
 int prep_begin(vx_backend *be, int m, int k, PrepView *pv) {
     VX_REQUIRE(m >= 1 && k >= 256 && k % 256 == 0, "prepare: bad shape %dx%d (K must be a multiple of 256)", m, k);
     const int mpad = mpad_for(m);
-    const size_t need = prep_tiles_bytes(mpad, k) + (size_t)ceil_div(mpad, 64) * 64 * 4 + (size_t)(k / 32) * mpad * 4 +
+    const size_t need = prep_tiles_bytes(mpad, k) + 2 * (size_t)ceil_div(mpad, 64) * 64 * 4 + (size_t)(k / 32) * mpad * 4 +
                         (size_t)(k / 256) * mpad * 4;
     int rc = ensure_ws(be, &be->gemm_ws, &be->gemm_ws_bytes, need, "prepared activations");
     if (rc) return rc;
+    be->rowfac_slot ^= 1;
+    be->prep_norm_k = 0;
     *pv = prep_view(be, mpad, k);
     be->prep_m = m;
     be->prep_k = k;
@@ -1047,7 +1212,7 @@ int gemm_target_wgs(vx_backend *be) {
 // of narrower activations inside one fused sequence cannot reallocate it (and lose the row scales).
 int prep_reserve(vx_backend *be, int m, int kmax) {
     const int mpad = mpad_for(m);
-    const size_t need = prep_tiles_bytes(mpad, kmax) + (size_t)ceil_div(mpad, 64) * 64 * 4 + (size_t)(kmax / 32) * mpad * 4 +
+    const size_t need = prep_tiles_bytes(mpad, kmax) + 2 * (size_t)ceil_div(mpad, 64) * 64 * 4 + (size_t)(kmax / 32) * mpad * 4 +
                         (size_t)(kmax / 256) * mpad * 4;
     return ensure_ws(be, &be->gemm_ws, &be->gemm_ws_bytes, need, "prepared activations");
 }
@@ -1125,10 +1290,36 @@ int check_fmt(int fmt, int k) {
     return VX_OK;
 }
 
+// Pending RMSNorm of the currently prepared activation (none: sspart = NULL).
+RowNorm cur_row_norm(const vx_backend *be) {
+    RowNorm rn = {nullptr, 0, 0.f, 0.f};
+    if (be->prep_norm_k > 0) {
+        rn.sspart = (const float *)be->prep_sync + (size_t)be->rowfac_slot * VX_PREP_SYNC_CHUNKS * VX_PREP_SYNC_ROWS;
+        rn.n_chunks = be->prep_norm_k / 256;
+        rn.inv_k = 1.0f / (float)be->prep_norm_k;
+        rn.eps = be->prep_norm_eps;
+    }
+    return rn;
+}
+float *cur_ss_out(vx_backend *be) {
+    return (float *)be->prep_sync + (size_t)be->rowfac_slot * VX_PREP_SYNC_CHUNKS * VX_PREP_SYNC_ROWS;
+}
+// Folds a pending 1/rms into the plain row factors, for consumers that read only those.
+int finalize_row_norm(vx_backend *be) {
+    if (be->prep_norm_k <= 0) return VX_OK;
+    const PrepView pv = prep_view(be, mpad_for(be->prep_m), be->prep_k);
+    finalize_row_norm_kernel<<<be->prep_m, 64, 0, be->stream>>>(pv.inv_scale, cur_row_norm(be));
+    VX_CHECK_LAUNCH();
+    be->prep_norm_k = 0;
+    return VX_OK;
+}
+
 int run_prepared(vx_backend *be, int fmt, const void *b, float *out, const float *residual, int m, int n, int k) {
     Segs segs;
     segs.w[0] = segs.w[1] = segs.w[2] = (const uint8_t *)b;
     segs.n_end[0] = segs.n_end[1] = segs.n_end[2] = n;
+    int rc = finalize_row_norm(be);  // the GEMM epilogue and the reduce kernel read plain row factors
+    if (rc) return rc;
     return launch_gemm_fmt(be, fmt, segs, n, out, residual, false, m, k, nullptr);
 }
 
@@ -1239,6 +1430,8 @@ static Segs make_segs(const vx_qweight *const *ws, int nw, int *ntot) {
     return sg;
 }
 
+// The chunk-parallel prepares cover decode-sized batches; larger ones keep the one-workgroup-per-row kernels.
+bool chunk_prepare_ok(int rows, int k) { return mpad_for(rows) <= VX_PREP_SYNC_ROWS && k / 256 <= VX_PREP_SYNC_CHUNKS; }
 int vx_decode_attn_qkv_supported(const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int head_dim) {
     const vx_qweight *ws[3] = {wq, wk, wv};
     return group_ok(ws, 3) && head_dim % 2 == 0 && head_dim <= 512 && (size_t)wq->k * 4 <= 64 * 1024;
@@ -1273,15 +1466,20 @@ int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight,
     const PrepView pv = prep_view(be, mpad_for(rows), k);
     const int half = head_dim / 2;
     const int lanes = 256 / half > 0 ? 256 / half : 1;
+    if ((lanes * half) % 64 != 0) {  // the row factor is a whole-wave computation
+        rc = finalize_row_norm(be);
+        if (rc) return rc;
+    }
+    const RowNorm rn = cur_row_norm(be);
     const int max_heads = num_q_heads > num_kv_heads ? num_q_heads : num_kv_heads;
     dim3 grid(rows, ceil_div(max_heads, lanes * 2));
     if (pool_is_f16)
         rope_store_partials_kernel<true><<<grid, lanes * half, 0, be->stream>>>(
-            (const float *)be->part_ws, ks, rows, pv.inv_scale, q_out, positions, slot_mapping, kv_pool, num_q_heads,
+            (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
             num_kv_heads, head_dim, block_size, theta);
     else
         rope_store_partials_kernel<false><<<grid, lanes * half, 0, be->stream>>>(
-            (const float *)be->part_ws, ks, rows, pv.inv_scale, q_out, positions, slot_mapping, kv_pool, num_q_heads,
+            (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
             num_kv_heads, head_dim, block_size, theta);
     VX_CHECK_LAUNCH();
     return VX_OK;
@@ -1324,9 +1522,14 @@ int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight 
         PrepView pa;
         rc = prep_begin(be, rows, wo->k, &pa);
         if (rc) return rc;
-        merge_prepare_kernel<<<mpad, PREP_THREADS, (size_t)wo->k * 4, be->stream>>>(
-            (const float *)be->attn_ws, be->split.kv_lens, rows, wo->k, be->split.head_dim, be->split.max_splits,
-            be->split.tokens_per_split, pa, mpad);
+        if (chunk_prepare_ok(rows, wo->k))
+            chunk_merge_kernel<<<dim3(wo->k / 256, mpad), 64, 0, be->stream>>>(
+                (const float *)be->attn_ws, be->split.kv_lens, rows, wo->k, be->split.head_dim, be->split.max_splits,
+                be->split.tokens_per_split, pa, mpad);
+        else
+            merge_prepare_kernel<<<mpad, PREP_THREADS, (size_t)wo->k * 4, be->stream>>>(
+                (const float *)be->attn_ws, be->split.kv_lens, rows, wo->k, be->split.head_dim, be->split.max_splits,
+                be->split.tokens_per_split, pa, mpad);
         VX_CHECK_LAUNCH();
         be->split.batch = 0;
     }
@@ -1336,10 +1539,19 @@ int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight 
     if (rc) return rc;
     // x += Wo(attn); prepared <- RMSNorm(x) * ffn_norm
     PrepView pv;
+    const float *inv_in = prep_view(be, mpad, wo->k).inv_scale;  // row factors of the activation that produced the partials
+    RowNorm rn_in = cur_row_norm(be);                            // (none pending here: the attention output)
     rc = prep_begin(be, rows, hidden, &pv);
     if (rc) return rc;
-    fused_prepare_kernel<FUSE_ADD_RMSNORM><<<mpad, FP_THREADS, (size_t)hidden * 4, be->stream>>>(
-        x, (const float *)be->part_ws, ks, rows, hidden, ffn_norm_weight, eps, pv, mpad);
+    const bool chunked = chunk_prepare_ok(rows, hidden) && chunk_prepare_ok(rows, ffn);
+    if (chunked) {
+        chunk_add_norm_kernel<<<dim3(hidden / 256, mpad), 64, 0, be->stream>>>(
+            x, (const float *)be->part_ws, ks, rows, hidden, ffn_norm_weight, eps, pv, mpad, inv_in, rn_in, cur_ss_out(be));
+        be->prep_norm_k = hidden;
+        be->prep_norm_eps = eps;
+    } else
+        fused_prepare_kernel<FUSE_ADD_RMSNORM><<<mpad, FP_THREADS, (size_t)hidden * 4, be->stream>>>(
+            x, (const float *)be->part_ws, ks, rows, hidden, ffn_norm_weight, eps, pv, mpad, inv_in);
     VX_CHECK_LAUNCH();
     // gate | up -> partials
     const vx_qweight *b[2] = {w1, w3};
@@ -1347,10 +1559,16 @@ int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight 
     rc = launch_gemm_fmt(be, w1->fmt, segs, ntot, nullptr, nullptr, true, rows, hidden, &ks);
     if (rc) return rc;
     // prepared <- SiLU(gate) * up
+    inv_in = pv.inv_scale;
+    rn_in = cur_row_norm(be);
     rc = prep_begin(be, rows, ffn, &pv);
     if (rc) return rc;
-    fused_prepare_kernel<FUSE_SILU_MUL><<<mpad, FP_THREADS, (size_t)ffn * 4, be->stream>>>(
-        nullptr, (const float *)be->part_ws, ks, rows, ffn, nullptr, 0.f, pv, mpad);
+    if (chunked)
+        chunk_silu_kernel<<<dim3(ffn / 256, mpad), 64, 0, be->stream>>>((const float *)be->part_ws, ks, rows, ffn, pv, mpad,
+                                                                        inv_in, rn_in);
+    else
+        fused_prepare_kernel<FUSE_SILU_MUL><<<mpad, FP_THREADS, (size_t)ffn * 4, be->stream>>>(
+            nullptr, (const float *)be->part_ws, ks, rows, ffn, nullptr, 0.f, pv, mpad, inv_in);
     VX_CHECK_LAUNCH();
     // down -> partials
     const vx_qweight *c[1] = {w2};
@@ -1358,10 +1576,19 @@ int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight 
     rc = launch_gemm_fmt(be, w2->fmt, segs, ntot, nullptr, nullptr, true, rows, ffn, &ks);
     if (rc) return rc;
     if (next_norm_weight) {
+        inv_in = pv.inv_scale;
+        rn_in = cur_row_norm(be);
         rc = prep_begin(be, rows, hidden, &pv);
         if (rc) return rc;
-        fused_prepare_kernel<FUSE_ADD_RMSNORM><<<mpad, FP_THREADS, (size_t)hidden * 4, be->stream>>>(
-            x, (const float *)be->part_ws, ks, rows, hidden, next_norm_weight, eps, pv, mpad);
+        if (chunked) {
+            chunk_add_norm_kernel<<<dim3(hidden / 256, mpad), 64, 0, be->stream>>>(
+                x, (const float *)be->part_ws, ks, rows, hidden, next_norm_weight, eps, pv, mpad, inv_in, rn_in,
+                cur_ss_out(be));
+            be->prep_norm_k = hidden;
+            be->prep_norm_eps = eps;
+        } else
+            fused_prepare_kernel<FUSE_ADD_RMSNORM><<<mpad, FP_THREADS, (size_t)hidden * 4, be->stream>>>(
+                x, (const float *)be->part_ws, ks, rows, hidden, next_norm_weight, eps, pv, mpad, inv_in);
         VX_CHECK_LAUNCH();
     } else {
         const size_t total4 = (size_t)rows * hidden / 4;
