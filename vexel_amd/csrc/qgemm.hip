@@ -1472,7 +1472,7 @@ int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight,
     }
     const RowNorm rn = cur_row_norm(be);
     const int max_heads = num_q_heads > num_kv_heads ? num_q_heads : num_kv_heads;
-    dim3 grid(rows, ceil_div(max_heads, lanes * 2));
+    dim3 grid(rows, ceil_div(max_heads, lanes));
     if (pool_is_f16)
         rope_store_partials_kernel<true><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
