@@ -180,6 +180,18 @@ __global__ void __launch_bounds__(GEN_THREADS) attn_generic_kernel(AttnParams p)
 constexpr int TPW = 512;  // tokens per workgroup
 constexpr int HOT_BS = 16;
 
+// Sum over the N adjacent lanes (N = 8 or 16, aligned) that hold one token's head vector, by DPP inside a
+// 16-lane row (no LDS traffic): quads, then the mirrored quad of the half, then the mirrored half.
+template <int N>
+__device__ __forceinline__ float token_sum(float t) {
+    static_assert(N == 8 || N == 16, "a head vector spans 8 or 16 lanes");
+    t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0xb1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+    t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x4e, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+    t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x141, 0xf, 0xf, false));  // row_half_mirror
+    if (N == 16) t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x140, 0xf, 0xf, false));  // row_mirror
+    return t;
+}
+
 template <int D, int G>
 __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix,
@@ -252,8 +264,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
                 float t = 0.f;
 #pragma unroll
                 for (int e = 0; e < 8; e++) t = fmaf(qf[g][e], (float)kk[u][e], t);
-#pragma unroll
-                for (int off = LPT / 2; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
+                t = token_sum<LPT>(t);
                 s[u] = (tok0 + u * TPI < t_end) ? t : -INFINITY;
                 gm = fmaxf(gm, s[u]);
             }
