@@ -221,13 +221,19 @@ def kernel_report(be):
                 out = be.alloc_permanent(m * n * 4)
                 be.prepare_act(da, m, k)
                 for w in ws[:2]:
-                    be.matmul_quant_prepared(fmt, w, out, None, m, n, k)
+                    if m == 1:
+                        be.matmul_quant(fmt, da, w, out, None, m, n, k)
+                    else:
+                        be.matmul_quant_prepared(fmt, w, out, None, m, n, k)
                 be.sync()
                 reps = 3
                 be.timer_start()
                 for _ in range(reps):
                     for w in ws:
-                        be.matmul_quant_prepared(fmt, w, out, None, m, n, k)
+                        if m == 1:   # the matrix-vector kernel reads the float32 activation itself
+                            be.matmul_quant(fmt, da, w, out, None, m, n, k)
+                        else:
+                            be.matmul_quant_prepared(fmt, w, out, None, m, n, k)
                 us = be.timer_stop_ms() * 1e3 / (reps * copies)
                 nbytes = n * rb + m * k * 4 + m * n * 4
                 gbs = nbytes / us / 1e3

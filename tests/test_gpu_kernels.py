@@ -97,8 +97,10 @@ def test_matmul_quant_vs_oracle(be, fmt, m):
 
 @pytest.mark.parametrize("fmt", [nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q4_K])
 def test_matmul_rows_independent_of_batch(be, fmt):
-    """A row computed alone has the same bits as inside a batch (sequential-loop semantics of
-    the reference, backend/metal/backend.go:777-779)."""
+    """A row has the same bits in a batch of 2 as in a batch of 32 (the batched kernel's launch shape and
+    summation order do not depend on M; cf. the reference's loop of M=1 kernels, backend/metal/backend.go:777-779).
+    A single row (M = 1) goes through the matrix-vector kernel, whose float32 summation order differs: it agrees
+    to rounding, not bit for bit."""
     rng = np.random.default_rng(9)
     m, n, k = 32, 96, 2048
     w = qz.random_quant(fmt, rng, n, k)
@@ -107,11 +109,37 @@ def test_matmul_rows_independent_of_batch(be, fmt):
     dout = be.alloc(m * n * 4)
     be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
     full = be.download(dout, (m, n), np.float32)
-    for r in (0, 5, 31):
+    for r in (0, 5, 30):
+        d2 = be.alloc(2 * n * 4)
+        be.matmul_quant(fmt, da + r * k * 4, dw, d2, None, 2, n, k)
+        two = be.download(d2, (2, n), np.float32)
+        assert np.array_equal(two.view(np.uint32), full[r:r + 2].view(np.uint32))
         d1 = be.alloc(n * 4)
         be.matmul_quant(fmt, da + r * k * 4, dw, d1, None, 1, n, k)
         one = be.download(d1, (n,), np.float32)
-        assert np.array_equal(one.view(np.uint32), full[r].view(np.uint32))
+        assert np.all(np.abs(one - full[r]) <= 2e-6 * np.abs(full[r]).max() + 1e-7)
+    be.reset_pool()
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("n,k", [(80, 1024), (33, 256), (7, 4096), (96, 11008), (40, 14336)])
+def test_matvec_single_row(be, fmt, n, k):
+    """M = 1 (the reference's decode call): segments that start at odd 16-byte phases, rows that are not a
+    multiple of 16 bytes (Q6_K at K = 11008), row groups running past N, with and without the residual. Shapes
+    the matrix-vector kernel declines (a matrix that is not a multiple of 16 bytes long) fall to the other paths
+    and must give the same answer."""
+    rng = np.random.default_rng(fmt * 1000 + n + k)
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((1, k)).astype(np.float32)
+    res = rng.standard_normal((1, n)).astype(np.float32)
+    want = nx.matmul_quant(fmt, a, w, 1, n, k)
+    da, dw, dres = be.upload(a), be.upload(w), be.upload(res)
+    dout = be.alloc(n * 4)
+    scale = np.abs(want).max()
+    be.matmul_quant(fmt, da, dw, dout, None, 1, n, k)
+    _close(be.download(dout, (1, n), np.float32), want, 2e-5, 3e-6 * scale + 1e-7, "matvec fmt %d %dx%d" % (fmt, n, k))
+    be.matmul_quant(fmt, da, dw, dout, dres, 1, n, k)
+    _close(be.download(dout, (1, n), np.float32), want + res, 2e-5, 3e-6 * scale + 1e-6, "matvec + residual")
     be.reset_pool()
 
 

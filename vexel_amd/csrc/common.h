@@ -96,6 +96,10 @@ int enter(vx_backend *be);
 // Ensures a library scratch buffer holds at least `bytes`; fails during capture if it must grow.
 int ensure_ws(vx_backend *be, void **ptr, size_t *cap, size_t bytes, const char *what);
 
+// qmatvec.hip: out[n] = a . W[n] (+ residual[n]) for one activation row; VX_ERR_UNSUPPORTED (nothing launched, no
+// error text) when the shape is outside the kernel's range.
+int run_matvec(vx_backend *be, int fmt, const float *a, const void *b, float *out, const float *residual, int n, int k);
+
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }
 

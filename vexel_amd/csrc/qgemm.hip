@@ -1396,6 +1396,11 @@ int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, floa
     rc = check_fmt(fmt, k);
     if (rc) return rc;
     if (m == 0 || n == 0) return VX_OK;
+    static const bool no_matvec = getenv("VEXEL_HIP_NO_MATVEC") != nullptr;  // keeps M = 1 on the batched kernel
+    if (m == 1 && !no_matvec) {  // a single row: the streaming matrix-vector kernel
+        rc = run_matvec(be, fmt, a, b, out, residual, n, k);
+        if (rc != VX_ERR_UNSUPPORTED) return rc;
+    }
     if (!fast_ok(fmt, b, k) || ((uintptr_t)a % 16) != 0) {
         const size_t rb = fmt_row_bytes(fmt, k);
         dim3 grid(n, ceil_div(m, FB_M));

@@ -202,7 +202,8 @@ int norm_for(vh_model *m, const float *x, const float *nw, float *norm, int rows
     const vh_config &c = m->cfg;
     int nfast = 0;
     for (int i = 0; i < nws; i++) nfast += fast(*ws[i]) ? 1 : 0;
-    *prepared = nfast > 0 && c.hidden % 256 == 0;
+    // a single row goes through the matrix-vector kernel, which reads the float32 activation
+    *prepared = rows > 1 && nfast > 0 && c.hidden % 256 == 0;
     if (*prepared)
         VXC(vx_rmsnorm_prepare(m->be, x, nw, nfast == nws ? nullptr : norm, rows, c.hidden, c.eps));
     else
@@ -220,7 +221,7 @@ int layer_tail(vh_model *m, const vh_layer_weights &w, float *x, float *norm, co
     VHC(norm_for(m, x, w.ffn_norm, norm, rows, w13, 2, &prep));                           // block.go:996-998
     VHC(mm(m, prep, norm, w.w1, gate, nullptr, rows));                                    // block.go:1043-1050
     VHC(mm(m, prep, norm, w.w3, up, nullptr, rows));
-    if (fast(w.w2) && c.ffn % 256 == 0) {                                                 // block.go:1056-1077
+    if (rows > 1 && fast(w.w2) && c.ffn % 256 == 0) {                                     // block.go:1056-1077
         VXC(vx_silu_mul_prepare(m->be, gate, up, nullptr, rows, c.ffn));
         VHC(mm(m, true, nullptr, w.w2, x, x, rows));
     } else {
@@ -243,7 +244,7 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
     const vh_config &c = m->cfg;
     const vh_layer_weights &w = m->layers[layer];
     const float scale = (float)(1.0 / sqrt((double)c.head_dim));                          // block.go:862
-    if (attn_fusable(m, layer)) {                                                         // block.go:834-868
+    if (rows > 1 && attn_fusable(m, layer)) {                                             // block.go:834-868
         VXC(vx_decode_attn_qkv(m->be, m->x, w.attn_norm, c.eps, *chained ? 1 : 0, &w.wq, &w.wk, &w.wv, rows,
                                m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, c.num_heads, c.num_kv_heads,
                                c.head_dim, c.block_size, c.rope_theta, m->q));
@@ -258,7 +259,7 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
         VXC(vx_rope_store_paged(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
                                 c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta));  // :858, :868
     }
-    const bool ffn_fused = m->fused && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
+    const bool ffn_fused = rows > 1 && m->fused && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
                            vx_decode_ffn_supported(&w.wo, &w.w1, &w.w3, &w.w2);
     // the fused tail can merge the attention's split-KV partials itself
     const bool split = ffn_fused && (size_t)w.wo.k * 4 <= 64 * 1024 && c.head_dim % 4 == 0 &&
@@ -280,10 +281,10 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
 int forward_decode(vh_model *m, int rows, int max_kv_len) {
     const vh_config &c = m->cfg;
     VXC(vx_embedding(m->be, m->d_tokens, rows, m->embedding, m->x, c.vocab, c.hidden));
-    const bool head_prepared = m->fused && fast(m->lm_head) && c.hidden % 256 == 0;
+    const bool head_prepared = rows > 1 && m->fused && fast(m->lm_head) && c.hidden % 256 == 0;
     bool chained = false;
     for (int l = 0; l < c.num_layers; l++) {
-        const float *next_norm = l + 1 < c.num_layers ? (attn_fusable(m, l + 1) ? m->layers[l + 1].attn_norm : nullptr)
+        const float *next_norm = l + 1 < c.num_layers ? (rows > 1 && attn_fusable(m, l + 1) ? m->layers[l + 1].attn_norm : nullptr)
                                                       : (head_prepared ? m->final_norm : nullptr);
         VHC(execute_layer_decode(m, l, rows, max_kv_len, next_norm, &chained));
     }
