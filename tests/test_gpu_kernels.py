@@ -463,16 +463,20 @@ def test_sdpa_and_prefill(be):
         be.sdpa(dq, dk, dv, do, L, hq, hk, d, sc, stride * d)
         _close(be.download(do, q.shape, np.float32), nx.sdpa(q, k, v, L, hq, hk, d, sc, stride * d), 1e-5, 2e-6, "sdpa")
         be.reset_pool()
-    s, hq, hk, d = 70, 4, 2, 64
-    q = rng.standard_normal((s, hq, d)).astype(np.float32)
-    k = rng.standard_normal((s, hk, d)).astype(np.float32)
-    v = rng.standard_normal((s, hk, d)).astype(np.float32)
-    sc = np.float32(1 / math.sqrt(d))
-    dq, dk, dv = be.upload(q), be.upload(k), be.upload(v)
-    do = be.alloc(q.nbytes)
-    be.sdpa_prefill(dq, dk, dv, do, s, hq, hk, d, sc)
-    _close(be.download(do, q.shape, np.float32), nx.sdpa_prefill(q, k, v, s, hq, hk, d, sc), 1e-5, 2e-6, "prefill")
-    be.reset_pool()
+    # causal prefill: the tiled matrix-core kernel (head_dim 64 / 128; one query, ragged tile ends, exact tile
+    # multiples, GQA) and the generic kernel (other head sizes)
+    for (s, hq, hk, d) in [(70, 4, 2, 64), (1, 2, 2, 128), (33, 4, 1, 128), (64, 2, 2, 64), (129, 8, 2, 128),
+                           (200, 2, 1, 64), (40, 2, 2, 32)]:
+        q = rng.standard_normal((s, hq, d)).astype(np.float32)
+        k = rng.standard_normal((s, hk, d)).astype(np.float32)
+        v = rng.standard_normal((s, hk, d)).astype(np.float32)
+        sc = np.float32(1 / math.sqrt(d))
+        dq, dk, dv = be.upload(q), be.upload(k), be.upload(v)
+        do = be.alloc(q.nbytes)
+        be.sdpa_prefill(dq, dk, dv, do, s, hq, hk, d, sc)
+        _close(be.download(do, q.shape, np.float32), nx.sdpa_prefill(q, k, v, s, hq, hk, d, sc), 1e-5, 3e-6,
+               "prefill s=%d hq=%d hk=%d d=%d" % (s, hq, hk, d))
+        be.reset_pool()
 
 
 def _make_pool(rng, f16, nblocks, bs, hk, d):

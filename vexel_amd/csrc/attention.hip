@@ -368,6 +368,150 @@ __global__ void __launch_bounds__(D) paged_merge_kernel(const float *__restrict_
     out[((size_t)seq * num_q_heads + qh) * D + d] = (L > 0.f) ? A / L : 0.f;
 }
 
+// --------------------------------------------------------------------------------------------
+// Dense causal prefill (Backend.SDPAPrefill, backend.go:389; math of backend/cpu/cpu.go:568-632 per query):
+// FlashAttention-2 style. grid = (query tiles of 64, Hq); block = 256 = 4 waves of 16 queries.
+// Per 32-key tile: K and V go to LDS as float32 (all four waves share them), S = Q K^T and O += P V run on the
+// float32 matrix cores (v_mfma_f32_16x16x4_f32: exact float32 products, float32 accumulation, so the numerics stay
+// at the reference's float32 level), the softmax is online in the exp2 domain, P crosses from the MFMA output
+// layout to the operand layout through a wave-private LDS tile. LDS row pitches are chosen so that each
+// operand read hits 64 different banks: K rows 132 floats (16 keys x 4 d), V rows 144 (4 keys x 16 d),
+// P rows 36.
+constexpr int FA_BQ = 64, FA_BK = 32;
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+template <int N>
+__device__ __forceinline__ float row16_max(float t) {  // max over the 16 lanes of a row; every lane gets it
+    t = fmaxf(t, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0xb1, 0xf, 0xf, false)));
+    t = fmaxf(t, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x4e, 0xf, 0xf, false)));
+    t = fmaxf(t, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x141, 0xf, 0xf, false)));
+    t = fmaxf(t, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x140, 0xf, 0xf, false)));
+    return t;
+}
+
+template <int D>
+__global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restrict__ q, const float *__restrict__ k,
+                                                          const float *__restrict__ v, float *__restrict__ out, int S,
+                                                          int num_q_heads, int num_kv_heads, float scale) {
+    constexpr int KP = D + 4, VP = D + 16, PP = FA_BK + 4;
+    __shared__ __attribute__((aligned(16))) float Ks[FA_BK * KP];
+    __shared__ __attribute__((aligned(16))) float Vs[FA_BK * VP];
+    __shared__ __attribute__((aligned(16))) float Ps[4][16 * PP];
+    const int qt = blockIdx.x, h = blockIdx.y, kvh = h / (num_q_heads / num_kv_heads);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int c16 = lane & 15, g = lane >> 4;
+    const int q0 = qt * FA_BQ + wave * 16;  // the wave's first query
+    const size_t qs = (size_t)num_q_heads * D, ks = (size_t)num_kv_heads * D;
+
+    // Q as the A operand: lane (row c16, k = 4s + g), pre-multiplied by scale*log2(e)
+    float qa[D / 4];
+    {
+        const int qi = min(q0 + c16, S - 1);
+        const float *qp = q + (size_t)qi * qs + (size_t)h * D + g;
+        const float f = scale * kLog2e;
+#pragma unroll
+        for (int s = 0; s < D / 4; s++) qa[s] = qp[4 * s] * f;
+    }
+    float4v o[D / 16];
+#pragma unroll
+    for (int db = 0; db < D / 16; db++) o[db] = (float4v){0.f, 0.f, 0.f, 0.f};
+    float m_run[4], l_run[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        m_run[i] = -INFINITY;
+        l_run[i] = 0.f;
+    }
+    const int last_q = min(qt * FA_BQ + FA_BQ - 1, S - 1);
+    const int n_tiles = last_q / FA_BK + 1;  // keys 0 .. last_q
+    for (int kt = 0; kt < n_tiles; kt++) {
+        __syncthreads();  // the previous tile's reads are done
+        for (int idx = tid; idx < FA_BK * (D / 4); idx += 256) {
+            const int key = idx / (D / 4), d4 = (idx % (D / 4)) * 4;
+            const int ki = kt * FA_BK + key;
+            float4 kv4 = make_float4(0.f, 0.f, 0.f, 0.f), vv4 = kv4;
+            if (ki < S) {
+                kv4 = *(const float4 *)(k + (size_t)ki * ks + (size_t)kvh * D + d4);
+                vv4 = *(const float4 *)(v + (size_t)ki * ks + (size_t)kvh * D + d4);
+            }
+            *(float4 *)(Ks + key * KP + d4) = kv4;
+            *(float4 *)(Vs + key * VP + d4) = vv4;
+        }
+        __syncthreads();
+        if (kt * FA_BK > min(q0 + 15, S - 1)) continue;  // every key of the tile is after the wave's queries
+        // S = Q K^T for the wave's 16 queries x 32 keys: lane holds S[row 4g+i][key cb*16 + c16]
+        float4v sc[FA_BK / 16];
+#pragma unroll
+        for (int cb = 0; cb < FA_BK / 16; cb++) {
+            float4v acc = {0.f, 0.f, 0.f, 0.f};
+            const float *kb = Ks + (cb * 16 + c16) * KP + g;
+#pragma unroll
+            for (int s = 0; s < D / 4; s++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[s], kb[4 * s], acc, 0, 0, 0);
+            sc[cb] = acc;
+        }
+        // causal mask, online softmax per row
+        float alpha[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int qi = q0 + 4 * g + i;
+            float mx = -INFINITY;
+#pragma unroll
+            for (int cb = 0; cb < FA_BK / 16; cb++) {
+                const int ki = kt * FA_BK + cb * 16 + c16;
+                if (ki > qi || ki >= S) sc[cb][i] = -INFINITY;
+                mx = fmaxf(mx, sc[cb][i]);
+            }
+            mx = row16_max<16>(mx);
+            const float m_new = fmaxf(m_run[i], mx);
+            // a row whose keys are all masked so far keeps m = -inf: exp2(-inf - -inf) must not be evaluated
+            alpha[i] = (m_new == -INFINITY) ? 1.f : exp2f(m_run[i] - m_new);
+            float rs = 0.f;
+#pragma unroll
+            for (int cb = 0; cb < FA_BK / 16; cb++) {
+                const float pw = (sc[cb][i] == -INFINITY) ? 0.f : exp2f(sc[cb][i] - m_new);
+                sc[cb][i] = pw;
+                rs += pw;
+            }
+            // sum over the 16 key lanes
+            rs += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, rs), 0xb1, 0xf, 0xf, false));
+            rs += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, rs), 0x4e, 0xf, 0xf, false));
+            rs += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, rs), 0x141, 0xf, 0xf, false));
+            rs += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, rs), 0x140, 0xf, 0xf, false));
+            l_run[i] = l_run[i] * alpha[i] + rs;
+            m_run[i] = m_new;
+        }
+#pragma unroll
+        for (int db = 0; db < D / 16; db++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) o[db][i] *= alpha[i];
+        // P: MFMA output layout -> operand layout through the wave's LDS tile
+        float *pt = &Ps[wave][0];
+#pragma unroll
+        for (int cb = 0; cb < FA_BK / 16; cb++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) pt[(4 * g + i) * PP + cb * 16 + c16] = sc[cb][i];
+        // (wave-private tile: the wave's own LDS accesses are ordered)
+        float pa[FA_BK / 4];
+#pragma unroll
+        for (int s = 0; s < FA_BK / 4; s++) pa[s] = pt[c16 * PP + 4 * s + g];
+        // O += P V: lane holds O[row 4g+i][d = db*16 + c16]
+#pragma unroll
+        for (int db = 0; db < D / 16; db++) {
+            const float *vb = Vs + g * VP + db * 16 + c16;
+#pragma unroll
+            for (int s = 0; s < FA_BK / 4; s++) o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[s], vb[4 * s * VP], o[db], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int qi = q0 + 4 * g + i;
+        if (qi >= S) continue;
+        const float inv = l_run[i] > 0.f ? 1.f / l_run[i] : 0.f;
+        float *op = out + (size_t)qi * qs + (size_t)h * D + c16;
+#pragma unroll
+        for (int db = 0; db < D / 16; db++) op[db * 16] = o[db][i] * inv;
+    }
+}
+
 template <int D, int G>
 int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *bt_matrix, const int32_t *bt_rows,
                int max_blocks, const int32_t *kv_lens, float *out, int batch, int num_q_heads, int num_kv_heads,
@@ -477,6 +621,17 @@ int vx_sdpa_prefill(vx_backend *be, const float *q, const float *k, const float 
     int rc = enter(be);
     if (rc) return rc;
     VX_REQUIRE(q && k && v && out && seq_len >= 0, "vx_sdpa_prefill: bad arguments");
+    VX_REQUIRE(num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, "vx_sdpa_prefill: bad head counts");
+    if (seq_len == 0) return VX_OK;
+    if ((head_dim == 64 || head_dim == 128) && ((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0) {
+        const dim3 grid(ceil_div(seq_len, FA_BQ), num_q_heads);
+        if (head_dim == 128)
+            prefill_fa2_kernel<128><<<grid, 256, 0, be->stream>>>(q, k, v, out, seq_len, num_q_heads, num_kv_heads, scale);
+        else
+            prefill_fa2_kernel<64><<<grid, 256, 0, be->stream>>>(q, k, v, out, seq_len, num_q_heads, num_kv_heads, scale);
+        VX_CHECK_LAUNCH();
+        return VX_OK;
+    }
     AttnParams p = {};
     p.q = q;
     p.out = out;
