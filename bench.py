@@ -34,7 +34,7 @@ BLOCK = 16
 
 # HBM bytes per algorithmic byte of the attention launch, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs
 # scaled by a plain copy of known size (summary: profiles/paged_decode_attention_7b_x32_hbm_traffic.txt).
-ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.012
+ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.008
 
 
 def ragged_contexts(seed=0, n=BATCH):
@@ -251,6 +251,26 @@ def kernel_report(be):
     print("paged decode attention, 32 ragged sequences (sum ctx %d), one layer: %.1f us, %.0f GB/s, %.3f of 8 TB/s"
           % (sum(ctx), ms * 1e3, nb / ms / 1e6, nb / ms / 1e6 / HBM_PEAK_GBS))
     mr.close()
+    # dense causal prefill attention of one 512-token chunk, 7B head geometry (float32 matrix cores)
+    S, hq, d = 512, c["num_heads"], c["head_dim"]
+    rng = np.random.default_rng(5)
+    dq = be.upload(rng.standard_normal((S, hq * d)).astype(np.float32), permanent=True)
+    dk = be.upload(rng.standard_normal((S, hq * d)).astype(np.float32), permanent=True)
+    dv = be.upload(rng.standard_normal((S, hq * d)).astype(np.float32), permanent=True)
+    do = be.alloc_permanent(S * hq * d * 4)
+    scale = 1.0 / math.sqrt(d)
+    for _ in range(3):
+        be.sdpa_prefill(dq, dk, dv, do, S, hq, hq, d, scale)
+    be.sync()
+    be.timer_start()
+    for _ in range(20):
+        be.sdpa_prefill(dq, dk, dv, do, S, hq, hq, d, scale)
+    ms = be.timer_stop_ms() / 20
+    flops = 4.0 * hq * d * S * (S + 1) / 2
+    print("causal prefill attention, S=512, %d heads x %d: %.1f us, %.1f TFLOP/s, %.3f of the 157.3 TFLOP/s float32 MFMA peak"
+          % (hq, d, ms * 1e3, flops / ms / 1e9, flops / ms / 1e9 / 157.3))
+    for p_ in (dq, dk, dv, do):
+        be.free(p_)
 
 
 def counter_probe(be, mr, ctx, c, layers):
@@ -275,6 +295,8 @@ def main():
     ap.add_argument("--layers", type=int, default=CFG["num_layers"], help="debug only: fewer layers is NOT the benchmark")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--seqs", type=int, default=BATCH, help="debug only: another batch size is NOT the benchmark "
+                                                             "(1 = single-stream decode through the matrix-vector kernel)")
     ap.add_argument("--kernel-report", action="store_true",
                     help="time the path's kernels one by one (quantized GEMM shapes per format, attention) and print a "
                          "table of achieved GB/s against the 8 TB/s HBM peak, then exit")
@@ -289,21 +311,22 @@ def main():
     if args.kernel_report:
         kernel_report(be)
         return
-    ctx = ragged_contexts()
+    ctx = ragged_contexts(n=args.seqs) if args.seqs != BATCH else ragged_contexts()
+    nseq = len(ctx)
     c = dict(CFG)
     c["num_layers"] = args.layers
     mr, ids = build_model(be, ctx, args.steps + args.warmup + 8, args.layers)
     if args.counter_probe:
         counter_probe(be, mr, ctx, c, args.layers)
         return
-    first = np.random.default_rng(3).integers(0, c["vocab"], BATCH).astype(np.int32)
+    first = np.random.default_rng(3).integers(0, c["vocab"], nseq).astype(np.int32)
     use_graph = not args.no_graph
     # warmup (untimed): first call runs one eager step, captures the graph, replays the rest
     w = max(args.warmup, 2 if use_graph else 1)
     mr.decode_graph(first, ids, ctx, w, use_graph=use_graph)
     be.sync()
     t0 = time.perf_counter()
-    toks, ms_events = mr.decode_graph(None, None, None, args.steps, use_graph=use_graph, batch=BATCH)
+    toks, ms_events = mr.decode_graph(None, None, None, args.steps, use_graph=use_graph, batch=nseq)
     be.sync()
     wall = time.perf_counter() - t0
     ms_per_step = wall * 1e3 / args.steps
@@ -314,17 +337,17 @@ def main():
     achieved = attn_bytes / (attn_ms * 1e-3) / 1e9
     out = {
         "metric": "decode tok/s, 7B Q4_0 x32 ragged seqs; % HBM peak in matvec + attn",
-        "value": BATCH * args.steps / wall,
+        "value": nseq * args.steps / wall,
         "unit": "tok/s",
         "n_gpus": 1, "steps": args.steps, "warmup": w,
         "ms_per_step": ms_per_step,
         "ms_per_step_hip_events": ms_events,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "LLaMA-2-7B-shaped Q4_0 (Q8_0 embedding+head), %d layers, 32 ragged paged-KV seqs, "
+        "config": {"workload": "LLaMA-2-7B-shaped Q4_0 (Q8_0 embedding+head), %d layers, %d ragged paged-KV seqs, "
                                "ctx lognormal(median 1024, sigma 0.6) in [64,4096] seed 0, sum ctx %d, block 16, "
-                               "greedy decode, hipGraph=%s" % (args.layers, sum(ctx_now), use_graph),
-                   "global_batch": BATCH},
+                               "greedy decode, hipGraph=%s" % (args.layers, nseq, sum(ctx_now), use_graph),
+                   "global_batch": nseq},
         "roofline": {"bound": "hbm", "kernel": "paged_decode_f16_kernel<128,1>",
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE * attn_bytes, "bytes_per_launch": attn_bytes, "ms_per_launch": attn_ms},
