@@ -155,8 +155,9 @@ int vx_rmsnorm_prepare(vx_backend *be, const float *x, const float *weight, floa
 int vx_silu_mul_prepare(vx_backend *be, const float *gate, const float *up, float *out, int rows, int cols);
 int vx_matmul_quant_prepared(vx_backend *be, int fmt, const void *b, float *out, const float *residual, int m,
                              int n, int k);
-/* 1 when (fmt, weight pointer alignment, k) can take the prepared MFMA path (Q4_0/Q8_0/Q4_K, k % 256 == 0). */
-int vx_matmul_quant_has_fast_path(int fmt, const void *b, int k);
+/* 1 when the [n,k] matrix can take the prepared MFMA path: k % 256 == 0, a 16-byte aligned pointer, and rows
+ * that are a multiple of 16 bytes (Q6_K: the whole matrix is, e.g. n % 8 == 0). */
+int vx_matmul_quant_has_fast_path(int fmt, const void *b, int n, int k);
 
 /* Fused decode blocks (the reference's FusedOps idea, backend.go:128-158, re-cut for the batched
  * paged path). They compute what the unfused call sequence computes, with each projection group

@@ -95,7 +95,7 @@ def test_matmul_quant_vs_oracle(be, fmt, m):
     be.reset_pool()
 
 
-@pytest.mark.parametrize("fmt", [nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q4_K])
+@pytest.mark.parametrize("fmt", FMTS)
 def test_matmul_rows_independent_of_batch(be, fmt):
     """A row has the same bits in a batch of 2 as in a batch of 32 (the batched kernel's launch shape and
     summation order do not depend on M; cf. the reference's loop of M=1 kernels, backend/metal/backend.go:777-779).
@@ -195,7 +195,8 @@ def test_prepared_activation_paths(be):
 
 
 @pytest.mark.parametrize("fmt,rows,hidden,ffn", [(nx.FMT_Q4_0, 1, 512, 1024), (nx.FMT_Q4_0, 32, 512, 14336),
-                                                 (nx.FMT_Q8_0, 5, 512, 1024), (nx.FMT_Q4_K, 40, 1024, 2048)])
+                                                 (nx.FMT_Q8_0, 5, 512, 1024), (nx.FMT_Q4_K, 40, 1024, 2048),
+                                                 (nx.FMT_Q6_K, 32, 512, 2816), (nx.FMT_Q6_K, 3, 1024, 1024)])
 def test_fused_decode_blocks_equal_the_unfused_sequence(be, fmt, rows, hidden, ffn):
     """vx_decode_attn_qkv / vx_decode_ffn give what the one-call-per-operation sequence of
     runtime/block.go:834-1077 gives (float32 activations, F16 and F32 pools), including the chained

@@ -229,15 +229,25 @@ __device__ __forceinline__ half8 pack8(half2v a, half2v b, half2v c, half2v d) {
     return r;
 }
 
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ half4v first16(half8 v) { return __builtin_shufflevector(v, v, 0, 1, 4, 5); }
+__device__ __forceinline__ half4v second16(half8 v) { return __builtin_shufflevector(v, v, 2, 3, 6, 7); }
+
 struct StepW {  // what one MFMA step needs from the weights
     half8 b;    // exact integer codes as f16, in slot order
     float d;    // multiplies the MFMA result
-    float dm;   // multiplies the activation block sum and is subtracted (Q4_K), else 0
+    float dm;   // multiplies the activation block sum and is subtracted (Q4_K); Q6_K: the scale of the
+                // step's second 16 elements (d is that of the first 16); else 0
 };
 
-// CHUNK_BYTES = raw bytes per weight row for 8 steps (256 elements); all are multiples of 16.
+// CHUNK_BYTES = raw bytes per weight row for 8 steps (256 elements). ROW_PIECES = 16-byte pieces staged per
+// row and chunk: CHUNK_BYTES / 16 where rows start on 16-byte boundaries (ALIGNED), else enough to cover the
+// chunk from the aligned address below its first byte. TWO_SCALES: a step's two halves of 16 elements carry
+// different scales, so a step is two 16x16x16 MFMAs per activation half instead of one 16x16x32.
 struct PQ4_0 {
     static constexpr int CHUNK_BYTES = 144;
+    static constexpr int ROW_PIECES = CHUNK_BYTES / 16;
+    static constexpr bool ALIGNED = true, TWO_SCALES = false;
     // Rows sit back to back in LDS: 144 bytes = 36 dwords, and 36*row mod 64 takes 16 distinct multiples of 4
     // for the 16 rows of a tile, so the 4 lane groups of every row read 64 different banks.
     static constexpr int PITCH = 144;
@@ -273,6 +283,8 @@ struct PQ4_0 {
 
 struct PQ8_0 {
     static constexpr int CHUNK_BYTES = 272;
+    static constexpr int ROW_PIECES = CHUNK_BYTES / 16;
+    static constexpr bool ALIGNED = true, TWO_SCALES = false;
     static constexpr int PITCH = 272;  // 68 dwords: (PITCH/4) % 8 == 4, conflict free like Q4_0's 36
     static constexpr int MIN_WAVES = 2;
     static constexpr bool HAS_MIN = false;
@@ -308,6 +320,8 @@ struct PQ8_0 {
 
 struct PQ4_K {
     static constexpr int CHUNK_BYTES = 144;  // one super-block = 8 sub-blocks of 32
+    static constexpr int ROW_PIECES = CHUNK_BYTES / 16;
+    static constexpr bool ALIGNED = true, TWO_SCALES = false;
     static constexpr int PITCH = 144;
     static constexpr int MIN_WAVES = 2;  // the min-term bookkeeping needs more registers than 3 waves leave
     static constexpr bool HAS_MIN = true;
@@ -354,6 +368,55 @@ constexpr int CH = 8;  // MFMA steps (32 elements each) per chunk
 
 // Up to three weight matrices that share K and the activation (Q/K/V, gate/up) multiplied in one
 // launch: output column n belongs to segment sg = first with n < n_end[sg], local row n - n_end[sg-1].
+// Q6_K: 210-byte super-blocks (ql[128] | qh[64] | int8 scales[16] | f16 d), so rows start on 2-byte
+// boundaries only. Element e = 128n + 32qt + p of a super-block: low nibble source ql[64n + 32(qt&1) + p]
+// >> 4(qt>>1), high two bits qh[32n + p] >> 2qt, scale[8n + 2qt + p/16] (inference/pkg/gguf/dequant.go:272-331).
+struct PQ6_K {
+    static constexpr int CHUNK_BYTES = 210;
+    static constexpr int ROW_PIECES = 14;  // shift <= 14 bytes, 14 + 210 = 224
+    static constexpr bool ALIGNED = false, TWO_SCALES = true;
+    static constexpr int PITCH = 240;  // 60 dwords: (PITCH/4) % 8 == 4
+    static constexpr int MIN_WAVES = 2;
+    static constexpr bool HAS_MIN = false;
+    static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 256 * 210; }
+    struct Raw { uint32_t l0, l1, l2, l3, h0, h1, h2, h3, sh; uint16_t sc, d; };
+    static __device__ __forceinline__ Raw read(const uint8_t *base, int row_off, int j, int g) {
+        const int n = j >> 2, qt = j & 3;
+        const int lo = row_off + 64 * n + 32 * (qt & 1) + 4 * g;  // positions 4g..4g+3; 16+4g.. are 16 bytes on
+        const int ho = row_off + 128 + 32 * n + 4 * g;
+        const uint32_t *w = (const uint32_t *)base;
+        Raw r;
+        r.l0 = w[lo >> 2];
+        r.l1 = w[(lo >> 2) + 1];
+        r.l2 = w[(lo >> 2) + 4];
+        r.l3 = w[(lo >> 2) + 5];
+        r.h0 = w[ho >> 2];
+        r.h1 = w[(ho >> 2) + 1];
+        r.h2 = w[(ho >> 2) + 4];
+        r.h3 = w[(ho >> 2) + 5];
+        r.sh = (uint32_t)(row_off & 3);  // every offset above differs from row_off by a multiple of 4
+        r.sc = *(const uint16_t *)(base + row_off + 192 + 8 * n + 2 * qt);
+        r.d = *(const uint16_t *)(base + row_off + 208);
+        return r;
+    }
+    static __device__ __forceinline__ StepW unpack(const Raw &x, int j) {
+        const int qt = j & 3;
+        const uint32_t ql0 = __builtin_amdgcn_alignbyte(x.l1, x.l0, x.sh), ql1 = __builtin_amdgcn_alignbyte(x.l3, x.l2, x.sh);
+        const uint32_t qh0 = __builtin_amdgcn_alignbyte(x.h1, x.h0, x.sh), qh1 = __builtin_amdgcn_alignbyte(x.h3, x.h2, x.sh);
+        const uint32_t w0 = ((ql0 >> (4 * (qt >> 1))) & 0x0F0F0F0Fu) | (((qh0 >> (2 * qt)) & 0x03030303u) << 4);
+        const uint32_t w1 = ((ql1 >> (4 * (qt >> 1))) & 0x0F0F0F0Fu) | (((qh1 >> (2 * qt)) & 0x03030303u) << 4);
+        const half2v off = {(_Float16)1056.f, (_Float16)1056.f};  // 1024 + 32
+        const uint32_t c64 = 0x64646464u;
+        StepW r;
+        r.b = pack8(as_h2(__builtin_amdgcn_perm(w0, c64, 0x00060004u)) - off, as_h2(__builtin_amdgcn_perm(w1, c64, 0x00060004u)) - off,
+                    as_h2(__builtin_amdgcn_perm(w0, c64, 0x00070005u)) - off, as_h2(__builtin_amdgcn_perm(w1, c64, 0x00070005u)) - off);
+        const float d = h2f(x.d);
+        r.d = d * (float)(int8_t)(x.sc & 0xFF);
+        r.dm = d * (float)(int8_t)(x.sc >> 8);
+        return r;
+    }
+};
+
 struct Segs {
     const uint8_t *w[3];
     int n_end[3];
@@ -375,7 +438,7 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
                                                     int M, int Mpad, int N, int K, int n_slices, int flags) {
     constexpr int ROWS_W = 16 * R;
     constexpr int PITCH = F::PITCH;
-    constexpr int WPIECES = ROWS_W * (F::CHUNK_BYTES / 16);
+    constexpr int WPIECES = ROWS_W * F::ROW_PIECES;
     constexpr int WNL = (WPIECES + 63) / 64;
     constexpr int APIECES = CH * MT * 2 * 64;  // 16-byte pieces of one activation chunk
     constexpr int ANL = APIECES / 256;
@@ -422,9 +485,14 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
 #pragma unroll
         for (int i = 0; i < WNL; i++) {
             const int pc = min(i * 64 + lane, WPIECES - 1);
-            const int row = pc / (F::CHUNK_BYTES / 16), col = pc % (F::CHUNK_BYTES / 16);
+            const int row = pc / F::ROW_PIECES, col = pc % F::ROW_PIECES;
             const int n = min(n0 + row, N - 1);
-            w_stage[i] = *(const u32x4 *)(seg_row(segs, n, row_bytes) + coff + col * 16);
+            const uint8_t *src = seg_row(segs, n, row_bytes) + coff;
+            // Unaligned rows are staged from the 16-byte boundary below their first byte; the pieces then end
+            // at the boundary at or above the chunk's last byte, which is inside the matrix because its size
+            // is a multiple of 16 (checked on the host).
+            if (!F::ALIGNED) src = (const uint8_t *)((uintptr_t)src & ~(uintptr_t)15);
+            w_stage[i] = *(const u32x4 *)(src + col * 16);
         }
     };
     auto commit = [&]() __attribute__((always_inline)) {
@@ -435,7 +503,7 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
 #pragma unroll
         for (int i = 0; i < WNL; i++) {
             const int pc = i * 64 + lane;
-            const int row = pc / (F::CHUNK_BYTES / 16), col = pc % (F::CHUNK_BYTES / 16);
+            const int row = pc / F::ROW_PIECES, col = pc % F::ROW_PIECES;
             if (pc < WPIECES) *(u32x4 *)(&w_lds[wave][row * PITCH + col * 16]) = w_stage[i];
         }
     };
@@ -481,11 +549,17 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
         typename F::Raw raw_n[R], raw_nn[R];
         StepW w_cur[R], w_nxt[R], w_old[R];
         float4v acc_old[R][MT], bs_old[MT] = {}, bs_cur[MT] = {};
+        int roff[R];  // where this lane's row of tile r starts in the wave's staging area
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            raw_n[r] = F::read(wl, (r * 16 + ln) * PITCH, 0, g);
+            roff[r] = (r * 16 + ln) * PITCH;
+            if (!F::ALIGNED) {
+                const int n = min(n0 + r * 16 + ln, N - 1);
+                roff[r] += (int)((uintptr_t)(seg_row(segs, n, row_bytes) + (size_t)chunk * F::CHUNK_BYTES) & 15);
+            }
+            raw_n[r] = F::read(wl, roff[r], 0, g);
             w_old[r] = w_nxt[r] = w_cur[r] = F::unpack(raw_n[r], 0);
-            raw_nn[r] = raw_n[r] = F::read(wl, (r * 16 + ln) * PITCH, 1, g);
+            raw_nn[r] = raw_n[r] = F::read(wl, roff[r], 1, g);
 #pragma unroll
             for (int t = 0; t < MT; t++) acc_old[r][t] = (float4v){0.f, 0.f, 0.f, 0.f};
         }
@@ -496,7 +570,7 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
             if (s + 1 < CH) a_nxt = lds_a(s + 1);
             if (s + 2 < CH) {
 #pragma unroll
-                for (int r = 0; r < R; r++) raw_nn[r] = F::read(wl, (r * 16 + ln) * PITCH, s + 2, g);
+                for (int r = 0; r < R; r++) raw_nn[r] = F::read(wl, roff[r], s + 2, g);
             }
             if (F::HAS_MIN) {
 #pragma unroll
@@ -547,13 +621,81 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
                 for (int i = 0; i < 4; i++) run[r][t][i] += cs_cur[t][i] * crun[r][t][i];
     };
 
+    // The same for formats whose step has two scales: four 16x16x16 MFMAs per tile and step, scaled as
+    // soon as the next tile's MFMAs have been issued, so that only two tiles' results are live at a time
+    // (the staging of unaligned rows and the wider raw reads leave fewer registers for pipelining).
+    auto compute_two_scales = [&](int chunk) __attribute__((always_inline)) {
+        const uint8_t *wl = &w_lds[wave][0];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++) crun[r][t] = (float4v){0.f, 0.f, 0.f, 0.f};
+        int roff[R];
+        typename F::Raw raw_n[R];
+        StepW w_cur[R], w_nxt[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const int n = min(n0 + r * 16 + ln, N - 1);
+            roff[r] = (r * 16 + ln) * PITCH +
+                      (int)((uintptr_t)(seg_row(segs, n, row_bytes) + (size_t)chunk * F::CHUNK_BYTES) & 15);
+            raw_n[r] = F::read(wl, roff[r], 0, g);
+            w_nxt[r] = w_cur[r] = F::unpack(raw_n[r], 0);
+            raw_n[r] = F::read(wl, roff[r], 1, g);
+        }
+        StepA a_cur = lds_a(0), a_nxt = a_cur;
+        const float4v z = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < CH; s++) {
+            if (s + 1 < CH) {
+                a_nxt = lds_a(s + 1);
+#pragma unroll
+                for (int r = 0; r < R; r++) w_nxt[r] = F::unpack(raw_n[r], s + 1);
+            }
+            if (s + 2 < CH) {
+#pragma unroll
+                for (int r = 0; r < R; r++) raw_n[r] = F::read(wl, roff[r], s + 2, g);
+            }
+            float4v p1 = z, p2 = z;  // the previous tile's two sums
+            int pr = 0, pt = 0;
+#pragma unroll
+            for (int i = 0; i <= R * MT; i++) {
+                float4v c1 = z, c2 = z;
+                const int r = i / MT, t = i % MT;
+                if (i < R * MT) {
+                    // slots 0,1,4,5 of an operand are the step's first 16 elements, slots 2,3,6,7 its second 16
+                    c1 = __builtin_amdgcn_mfma_f32_16x16x16f16(first16(a_cur.h[t]), first16(w_cur[r].b), z, 0, 0, 0);
+                    c2 = __builtin_amdgcn_mfma_f32_16x16x16f16(second16(a_cur.h[t]), second16(w_cur[r].b), z, 0, 0, 0);
+                    c1 = __builtin_amdgcn_mfma_f32_16x16x16f16(first16(a_cur.l[t]), first16(w_cur[r].b), c1, 0, 0, 0);
+                    c2 = __builtin_amdgcn_mfma_f32_16x16x16f16(second16(a_cur.l[t]), second16(w_cur[r].b), c2, 0, 0, 0);
+                }
+                if (i > 0) {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) crun[pr][pt][e] += w_cur[pr].d * p1[e] + w_cur[pr].dm * p2[e];
+                }
+                p1 = c1, p2 = c2, pr = r, pt = t;
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) w_cur[r] = w_nxt[r];
+            a_cur = a_nxt;
+        }
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) run[r][t][i] += cs_cur[t][i] * crun[r][t][i];
+    };
+
     if (c_begin < c_end) fetch(c_begin);
     for (int chunk = c_begin; chunk < c_end; chunk++) {
         __syncthreads();  // previous chunk's reads are done
         commit();
         __syncthreads();
         if (chunk + 1 < c_end) fetch(chunk + 1);  // in flight while this chunk is computed
-        compute(chunk);
+        if constexpr (F::TWO_SCALES)
+            compute_two_scales(chunk);
+        else
+            compute(chunk);
     }
 
     // lane (g, ln) of tile (r, t) holds C[m = m0 + 16t + 4g + i][n = n0 + 16r + ln], i = 0..3. Each wave
@@ -1271,13 +1413,17 @@ int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out
     switch (fmt) {
     case VX_Q4_0: return launch_gemm<PQ4_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
     case VX_Q8_0: return launch_gemm<PQ8_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
+    case VX_Q6_K: return launch_gemm<PQ6_K>(be, segs, N, out, residual, to_partials, M, K, ks_out);
     default: return launch_gemm<PQ4_K>(be, segs, N, out, residual, to_partials, M, K, ks_out);
     }
 }
 
-bool fast_ok(int fmt, const void *b, int k) {
+// Q6_K rows are 210 bytes per 256 elements and need not start on 16-byte boundaries; its kernel stages
+// them from the boundary below, which needs the whole matrix to be a multiple of 16 bytes.
+bool fast_ok(int fmt, const void *b, int n, int k) {
     const size_t rb = fmt_row_bytes(fmt, k);
-    return fmt != VX_Q6_K && (k % 256 == 0) && (rb % 16 == 0) && ((uintptr_t)b % 16 == 0);
+    if (k % 256 != 0 || ((uintptr_t)b % 16) != 0 || n < 1) return false;
+    return fmt == VX_Q6_K ? ((size_t)n * rb) % 16 == 0 : rb % 16 == 0;
 }
 
 int check_fmt(int fmt, int k) {
@@ -1381,11 +1527,11 @@ int vx_matmul_quant_prepared(vx_backend *be, int fmt, const void *b, float *out,
     if (rc) return rc;
     VX_REQUIRE(be->prep_m == m && be->prep_k == k, "vx_matmul_quant_prepared: the prepared activation is %dx%d, not %dx%d",
                be->prep_m, be->prep_k, m, k);
-    VX_REQUIRE(fast_ok(fmt, b, k), "vx_matmul_quant_prepared: format %d / K=%d / alignment has no MFMA path", fmt, k);
+    VX_REQUIRE(fast_ok(fmt, b, n, k), "vx_matmul_quant_prepared: format %d / N=%d / K=%d / alignment has no MFMA path", fmt, n, k);
     return run_prepared(be, fmt, b, out, residual, m, n, k);
 }
 
-int vx_matmul_quant_has_fast_path(int fmt, const void *b, int k) { return fast_ok(fmt, b, k) ? 1 : 0; }
+int vx_matmul_quant_has_fast_path(int fmt, const void *b, int n, int k) { return fast_ok(fmt, b, n, k) ? 1 : 0; }
 
 int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, float *out, const float *residual, int m,
                     int n, int k) {
@@ -1401,7 +1547,7 @@ int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, floa
         rc = run_matvec(be, fmt, a, b, out, residual, n, k);
         if (rc != VX_ERR_UNSUPPORTED) return rc;
     }
-    if (!fast_ok(fmt, b, k) || ((uintptr_t)a % 16) != 0) {
+    if (!fast_ok(fmt, b, n, k) || ((uintptr_t)a % 16) != 0) {
         const size_t rb = fmt_row_bytes(fmt, k);
         dim3 grid(n, ceil_div(m, FB_M));
         qgemm_fallback_kernel<<<grid, 64, 0, be->stream>>>(fmt, (const uint8_t *)b, a, out, residual, m, n, k, rb);
@@ -1417,7 +1563,7 @@ static bool group_ok(const vx_qweight *const *ws, int nw) {
     for (int i = 0; i < nw; i++) {
         if (!ws[i] || !ws[i]->data) return false;
         if (ws[i]->fmt != ws[0]->fmt || ws[i]->k != ws[0]->k) return false;
-        if (!fast_ok(ws[i]->fmt, ws[i]->data, ws[i]->k) || ws[i]->n % 16 != 0 || ws[i]->n <= 0) return false;
+        if (!fast_ok(ws[i]->fmt, ws[i]->data, ws[i]->n, ws[i]->k) || ws[i]->n % 16 != 0 || ws[i]->n <= 0) return false;
     }
     return true;
 }

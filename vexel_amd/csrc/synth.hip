@@ -29,6 +29,25 @@ __device__ __forceinline__ float2 normal_pair(uint64_t seed, uint64_t i) {
     return make_float2(rad * c, rad * s);
 }
 
+// one thread per super-block: random bytes, then f16 headers of about 2^-10 at byte offsets h0 / h1 (h1 < 0: none)
+__global__ void random_kquant_kernel(uint8_t *dst, int64_t nblocks, int block_bytes, int h0, int h1, uint64_t seed) {
+    int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblocks) return;
+    uint8_t *o = dst + b * block_bytes;
+    for (int i = 0; i < block_bytes; i += 2) {  // block sizes are even
+        const uint64_t r = splitmix64(seed ^ splitmix64((uint64_t)b * 128 + i / 2));
+        o[i] = (uint8_t)r;
+        o[i + 1] = (uint8_t)(r >> 8);
+    }
+    const uint64_t r = splitmix64(seed + 0x5bd1e995ull * (uint64_t)b);
+    o[h0] = (uint8_t)r;
+    o[h0 + 1] = 0x14;  // 2^-10 * (1 + mantissa)
+    if (h1 >= 0) {
+        o[h1] = (uint8_t)(r >> 8);
+        o[h1 + 1] = 0x10;
+    }
+}
+
 __global__ void gaussian_q4_0_kernel(uint8_t *dst, int64_t nblocks, float stdv, uint64_t seed) {
     int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (b >= nblocks) return;
@@ -111,6 +130,19 @@ int vxs_plain_copy(void *dst, const void *src, int64_t bytes) {
     const int64_t n16 = bytes / 16;
     if (n16 <= 0) return 0;
     plain_copy_kernel<<<(unsigned)((n16 + 255) / 256), 256>>>((const uint4 *)src, (uint4 *)dst, n16);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
+    return (int)hipDeviceSynchronize();
+}
+
+// fmt: 3 = Q4_K (144-byte super-blocks), 4 = Q6_K (210-byte): uniformly random codes and sub-block scales
+// under small finite f16 super-block scales. Timing input only: the values follow no distribution a
+// quantizer would produce.
+int vxs_random_kquant(int fmt, void *dst, int64_t nblocks, uint64_t seed) {
+    if (nblocks <= 0) return 0;
+    if (fmt != 3 && fmt != 4) return -1;
+    random_kquant_kernel<<<(unsigned)((nblocks + 255) / 256), 256>>>((uint8_t *)dst, nblocks, fmt == 3 ? 144 : 210,
+                                                                      fmt == 3 ? 0 : 208, fmt == 3 ? 2 : -1, seed);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     return (int)hipDeviceSynchronize();

@@ -182,7 +182,7 @@ int sync_pool_to_device(vh_model *m) {
     return VH_OK;
 }
 
-bool fast(const vh_qweight &w) { return vx_matmul_quant_has_fast_path(w.fmt, w.data, w.k) != 0; }
+bool fast(const vh_qweight &w) { return vx_matmul_quant_has_fast_path(w.fmt, w.data, w.n, w.k) != 0; }
 
 // out = act * w^T (+ residual) where `act` is both in the backend's prepared slot (when `prepared`) and,
 // unless every consumer takes the prepared path, in float32 at a_f32.

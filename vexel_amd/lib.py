@@ -61,7 +61,7 @@ SIGNATURES = {
     "vx_rmsnorm_prepare": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f]),
     "vx_silu_mul_prepare": (_i, [_vp, _vp, _vp, _vp, _i, _i]),
     "vx_matmul_quant_prepared": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i]),
-    "vx_matmul_quant_has_fast_path": (_i, [_i, _vp, _i]),
+    "vx_matmul_quant_has_fast_path": (_i, [_i, _vp, _i, _i]),
     "vx_decode_attn_qkv_supported": (_i, [_vp, _vp, _vp, _i]),
     "vx_decode_attn_qkv": (_i, [_vp, _vp, _vp, _f, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
     "vx_decode_ffn_supported": (_i, [_vp, _vp, _vp, _vp]),
