@@ -3,7 +3,8 @@
 // W holds raw GGUF blocks (inference/pkg/gguf/dequant.go). HBM bound: every weight byte is read once with 16-byte
 // loads, the arithmetic is plain float32 on the vector ALU (no matrix cores at M = 1).
 //
-// Shape of the work. grid = ceil(N / RG) workgroups of 256 threads; a workgroup owns RG consecutive weight rows.
+// Shape of the work. Workgroups of 256 threads; a workgroup takes groups of RG consecutive weight rows, one group
+// per trip of its loop, and loads the next group's weights while it computes the current one.
 //   * K is cut in four segments of whole "units" (a 32-element block for Q4_0 / Q8_0, a 256-element super-block for
 //     Q4_K / Q6_K); wave w takes segment w of every row of the group.
 //   * A wave's 64 lanes are 2 row lanes x 32 block lanes: lane l works on 32-element blocks (l % 32) + 32 t,
@@ -19,6 +20,7 @@
 //     d * (sum a*q - off * sum a). The 32 block lanes are added by DPP inside 16-lane rows plus one cross-row
 //     exchange, the four waves through LDS, in a fixed order.
 #include "common.h"
+#include <algorithm>
 
 using namespace vx;
 
@@ -63,44 +65,145 @@ __device__ __forceinline__ float half_wave_sum(float t) {
     return t;
 }
 
-// ---- per-format decoders: contribution of 32-element block `jl` of the staged segment `seg` (LDS byte offset of the
-// segment's first byte inside `base`), given the block's activations x[32] and their sums over elements 0-15 / 16-31.
+// ---- per-format decoders. X holds what a lane keeps of one 32-element block of the activation row (set once by
+// prep from the block's 32 floats); block() is the contribution of block `jl` of the staged segment `seg` (LDS
+// byte offset of the segment's first byte inside `base`).
+//
+// The arithmetic is integer: 4-byte dot products (v_dot4) of the weight codes, which ARE bytes or nibbles, with
+// the activations as fixed-point integers. A block's activations are scaled by the power of two that puts the
+// largest magnitude in [2^(BITS-2), 2^(BITS-1)) and rounded to integers xi (an error of at most 2^-(BITS-1) of
+// the block's largest activation per element). Plane p holds byte p of the two's-complement xi of the 32
+// elements, four to a dword in element order: xi = b0 + 256 b1 + 65536 b2 with b0, b1 unsigned and b2 signed,
+// so sum(code * xi) = S0 + 256 S1 + 65536 S2 with Sp = sum(code * bp), exact in int32 for the BITS each format
+// picks. The block's scale and the inverse power of two are applied to the float of that integer.
+template <int BITS>
+struct XInt {
+    uint32_t p[3][8];  // plane, dword j = elements 4j .. 4j+3
+    int s0, s1;        // sum of xi over elements 0-15 / 16-31
+    float inv;         // activation = xi * inv
+    __device__ __forceinline__ void prep(const float *v) {
+        float m = 0.f;
+#pragma unroll
+        for (int i = 0; i < 32; i++) m = fmaxf(m, fabsf(v[i]));
+        // scale = 2^(BITS - 2 - exponent(m)); zero, denormal-range and non-finite maxima take 1 (such rows give
+        // zeros or garbage either way: the float path would too)
+        const int ex = (int)((__float_as_uint(m) >> 23) & 0xFF);
+        const bool usable = ex > BITS && ex < 255;
+        const float scale = usable ? __uint_as_float((uint32_t)(127 + BITS - 2 + 127 - ex) << 23) : 1.f;
+        inv = usable ? __uint_as_float((uint32_t)(ex - (BITS - 2)) << 23) : 1.f;
+        s0 = s1 = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            uint32_t xi[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) {
+                // adding 1.5 * 2^23 rounds v * scale (|.| < 2^22) to an integer, to nearest even, in the low
+                // mantissa bits: the float's bits are 0x4B400000 + xi
+                const uint32_t bits = __float_as_uint(fmaf(v[4 * j + k], scale, 12582912.f));
+                xi[k] = bits - 0x4B400000u;
+                if (j < 4) s0 += (int)xi[k];
+                else s1 += (int)xi[k];
+            }
+            // v_perm_b32(hi, lo, sel): selector bytes 0-3 pick from lo, 4-7 from hi
+            const uint32_t a01 = __builtin_amdgcn_perm(xi[1], xi[0], 0x05010400u);  // x0.b0 x1.b0 x0.b1 x1.b1
+            const uint32_t a23 = __builtin_amdgcn_perm(xi[3], xi[2], 0x05010400u);
+            const uint32_t c01 = __builtin_amdgcn_perm(xi[1], xi[0], 0x0c0c0602u);  // x0.b2 x1.b2 0 0
+            const uint32_t c23 = __builtin_amdgcn_perm(xi[3], xi[2], 0x0c0c0602u);
+            p[0][j] = __builtin_amdgcn_perm(a23, a01, 0x05040100u);
+            p[1][j] = __builtin_amdgcn_perm(a23, a01, 0x07060302u);
+            p[2][j] = __builtin_amdgcn_perm(c23, c01, 0x05040100u);
+        }
+    }
+    // acc[p] += sum over the 4 unsigned code bytes of c times byte p of elements 4j .. 4j+3 (codes below 128)
+    __device__ __forceinline__ void dot(int (&acc)[3], uint32_t c, int j) const {
+        acc[0] = (int)__builtin_amdgcn_udot4(c, p[0][j], (uint32_t)acc[0], false);
+        acc[1] = (int)__builtin_amdgcn_udot4(c, p[1][j], (uint32_t)acc[1], false);
+        acc[2] = __builtin_amdgcn_sdot4((int)c, (int)p[2][j], acc[2], false);
+    }
+    // sum of the bytes of plane pl over all 32 elements
+    __device__ __forceinline__ int plane_sum(int pl) const {
+        uint32_t t = 0;
+#pragma unroll
+        for (int j = 0; j < 8; j++) t = __builtin_amdgcn_udot4(0x01010101u, p[pl][j], t, false);
+        return (int)t;
+    }
+};
+
+// N consecutive dwords starting at byte offset `off` (any alignment) of a 4-byte aligned LDS array: N + 1
+// aligned reads at constant offsets from one address, then one byte alignment each.
+template <int N>
+__device__ __forceinline__ void lds_dwords(const uint8_t *base, int off, uint32_t (&w)[N]) {
+    const uint32_t *p = (const uint32_t *)base + (off >> 2);
+    const uint32_t sh = (uint32_t)(off & 3);
+    uint32_t raw[N + 1];
+#pragma unroll
+    for (int i = 0; i <= N; i++) raw[i] = p[i];
+#pragma unroll
+    for (int i = 0; i < N; i++) w[i] = __builtin_amdgcn_alignbyte(raw[i + 1], raw[i], sh);
+}
+
 struct VQ4_0 {  // dequant.go:16-56: [f16 d][16 bytes], element i = low nibble of byte i, i+16 = high nibble, (q-8)*d
     static constexpr int UNIT_BLOCKS = 1, UNIT_BYTES = 18;
-    static __device__ __forceinline__ float block(const uint8_t *base, int seg, int jl, const float *x, float s0, float s1) {
+    typedef XInt<23> X;  // |xi| < 2^22: |sum q xi| <= 15 * 2^22 * 32 < 2^31
+    static __device__ __forceinline__ float block(const uint8_t *base, int seg, int jl, const X &x) {
         const int o = seg + jl * 18;
-        float acc = 0.f;
+        uint32_t w[4];
+        lds_dwords<4>(base, o + 2, w);
+        int acc[3] = {0, 0, 0};
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const uint32_t w = lds_u32(base, o + 2 + 4 * i);
-            acc = dot4(acc, w & 0x0F0F0F0Fu, x + 4 * i);
-            acc = dot4(acc, (w >> 4) & 0x0F0F0F0Fu, x + 16 + 4 * i);
+            x.dot(acc, w[i] & 0x0F0F0F0Fu, i);
+            x.dot(acc, (w[i] >> 4) & 0x0F0F0F0Fu, 4 + i);
         }
-        return h2f((uint16_t)lds_u16(base, o)) * (acc - 8.f * (s0 + s1));
+        const int t = acc[0] + (acc[1] << 8) + (acc[2] << 16) - 8 * (x.s0 + x.s1);  // sum (q - 8) xi, exact
+        return h2f((uint16_t)lds_u16(base, o)) * ((float)t * x.inv);
     }
 };
 
 struct VQ8_0 {  // dequant.go:62-90: [f16 d][32 x int8], d*q
     static constexpr int UNIT_BLOCKS = 1, UNIT_BYTES = 34;
-    static __device__ __forceinline__ float block(const uint8_t *base, int seg, int jl, const float *x, float s0, float s1) {
+    struct X : XInt<23> {
+        int b0, b1;  // byte sums of planes 0 and 1
+        __device__ __forceinline__ void prep(const float *v) {
+            XInt<23>::prep(v);
+            b0 = plane_sum(0);
+            b1 = plane_sum(1);
+        }
+    };
+    static __device__ __forceinline__ float block(const uint8_t *base, int seg, int jl, const X &x) {
         const int o = seg + jl * 34;
-        float acc = 0.f;
+        uint32_t w[8];
+        lds_dwords<8>(base, o + 2, w);
+        // the unsigned planes take the codes as q + 128 (unsigned), corrected by 128 * the plane's byte sum;
+        // the signed top plane takes them as they are
+        uint32_t u0 = 0, u1 = 0;
+        int s2 = 0;
 #pragma unroll
-        for (int i = 0; i < 8; i++) acc = dot4(acc, lds_u32(base, o + 2 + 4 * i) ^ 0x80808080u, x + 4 * i);  // q + 128
-        return h2f((uint16_t)lds_u16(base, o)) * (acc - 128.f * (s0 + s1));
+        for (int i = 0; i < 8; i++) {
+            const uint32_t c = w[i] ^ 0x80808080u;
+            u0 = __builtin_amdgcn_udot4(c, x.p[0][i], u0, false);
+            u1 = __builtin_amdgcn_udot4(c, x.p[1][i], u1, false);
+            s2 = __builtin_amdgcn_sdot4((int)w[i], (int)x.p[2][i], s2, false);
+        }
+        // |S2| can reach 2^18, so the top plane joins in float32 (|S0 + 256 S1| < 2^31 stays exact)
+        const int low = ((int)u0 - 128 * x.b0) + (((int)u1 - 128 * x.b1) << 8);
+        const float t = (float)s2 * 65536.f + (float)low;
+        return h2f((uint16_t)lds_u16(base, o)) * (t * x.inv);
     }
 };
 
 struct VQ4_K {  // dequant.go:342-409: 144-byte super-block, 8 sub-blocks of 32: d*sc*q - dmin*m
     static constexpr int UNIT_BLOCKS = 8, UNIT_BYTES = 144;
-    static __device__ __forceinline__ float block(const uint8_t *base, int seg, int jl, const float *x, float s0, float s1) {
+    typedef XInt<23> X;
+    static __device__ __forceinline__ float block(const uint8_t *base, int seg, int jl, const X &x) {
         const int j = jl & 7;
         const int sb = seg + (jl >> 3) * 144;  // 16-byte aligned: rows and segments are whole super-blocks
         const uint32_t *S = (const uint32_t *)(base + sb);
         const uint32_t *qp = S + 4 + 8 * (j >> 1);
-        float acc = 0.f;
+        int acc[3] = {0, 0, 0};
 #pragma unroll
-        for (int i = 0; i < 8; i++) acc = dot4(acc, (qp[i] >> (4 * (j & 1))) & 0x0F0F0F0Fu, x + 4 * i);
+        for (int i = 0; i < 8; i++) x.dot(acc, (qp[i] >> (4 * (j & 1))) & 0x0F0F0F0Fu, i);
+        const int t = acc[0] + (acc[1] << 8) + (acc[2] << 16);
         const uint8_t *q = base + sb + 4;
         uint32_t sc, mn;  // getScaleMinK4, dequant.go:400-409
         if (j < 4) {
@@ -111,115 +214,162 @@ struct VQ4_K {  // dequant.go:342-409: 144-byte super-block, 8 sub-blocks of 32:
             mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
         }
         const uint32_t hd = S[0];
-        return h2f((uint16_t)(hd & 0xFFFF)) * (float)sc * acc - h2f((uint16_t)(hd >> 16)) * (float)mn * (s0 + s1);
+        return (h2f((uint16_t)(hd & 0xFFFF)) * (float)sc * (float)t - h2f((uint16_t)(hd >> 16)) * (float)mn * (float)(x.s0 + x.s1)) * x.inv;
     }
 };
 
 struct VQ6_K {  // dequant.go:272-331: 210-byte super-block [ql 128][qh 64][int8 sc 16][f16 d]
     static constexpr int UNIT_BLOCKS = 8, UNIT_BYTES = 210;
-    static __device__ __forceinline__ float block(const uint8_t *base, int seg, int jl, const float *x, float s0, float s1) {
+    typedef XInt<22> X;  // |xi| < 2^21; per 16 elements: |sum q6 xi| <= 63 * 2^21 * 16 < 2^31
+    static __device__ __forceinline__ float block(const uint8_t *base, int seg, int jl, const X &x) {
         const int j = jl & 7, n = j >> 2, qt = j & 3;  // half n, quarter qt: elements 128n + 32qt + (0..31)
         const int S = seg + (jl >> 3) * 210;
         const int ql = S + 64 * n + 32 * (qt & 1), qh = S + 128 + 32 * n;
-        float a0 = 0.f, a1 = 0.f;
+        uint32_t wl[8], wh[8];
+        lds_dwords<8>(base, ql, wl);
+        lds_dwords<8>(base, qh, wh);
+        int a[3] = {0, 0, 0}, b[3] = {0, 0, 0};
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const uint32_t lo = (lds_u32(base, ql + 4 * i) >> (4 * (qt >> 1))) & 0x0F0F0F0Fu;
-            const uint32_t hi = (lds_u32(base, qh + 4 * i) >> (2 * qt)) & 0x03030303u;
-            const uint32_t q = lo | (hi << 4);  // 6-bit code, value q - 32
-            if (i < 4) a0 = dot4(a0, q, x + 4 * i);
-            else a1 = dot4(a1, q, x + 4 * i);
+            const uint32_t lo = (wl[i] >> (4 * (qt >> 1))) & 0x0F0F0F0Fu;
+            const uint32_t hi = (wh[i] >> (2 * qt)) & 0x03030303u;
+            const uint32_t q = lo | (hi << 4);  // 6-bit codes, value q - 32
+            if (i < 4) x.dot(a, q, i);
+            else x.dot(b, q, i);
         }
+        const int ta = a[0] + (a[1] << 8) + (a[2] << 16) - 32 * x.s0;  // elements 0-15
+        const int tb = b[0] + (b[1] << 8) + (b[2] << 16) - 32 * x.s1;
         const uint32_t sc = lds_u16(base, S + 192 + 8 * n + 2 * qt);  // scales of elements 0-15 and 16-31
         const float sa = (float)(int8_t)(sc & 0xFF), sb = (float)(int8_t)(sc >> 8);
         const float d = h2f((uint16_t)lds_u16(base, S + 208));
-        return d * (sa * (a0 - 32.f * s0) + sb * (a1 - 32.f * s1));
+        return d * ((sa * (float)ta + sb * (float)tb) * x.inv);
     }
 };
 
-template <class F, int T>
+template <class F, int T, int LP>
 __global__ void __launch_bounds__(MV_THREADS) qmatvec_kernel(const uint8_t *__restrict__ W, const float *__restrict__ a,
                                                              float *__restrict__ out, const float *__restrict__ residual,
-                                                             int N, int K, size_t row_bytes, int lp, int units_per_wave) {
+                                                             int N, int K, size_t row_bytes, int units_per_wave,
+                                                             int n_groups) {
+    constexpr int PASSES = 1 << LP, RG = MV_MAX_RG >> LP;  // 64-piece passes per staged row; rows per group
     __shared__ __attribute__((aligned(16))) uint8_t stage[MV_WAVES][MV_WAVE_LDS];
-    __shared__ float part[MV_WAVES][MV_MAX_RG];
+    __shared__ float part[2][MV_WAVES][MV_MAX_RG];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bl = lane & 31, rp = lane >> 5;
     const int n_units = K / (32 * F::UNIT_BLOCKS);
     const int u0 = min(wave * units_per_wave, n_units), u1 = min(u0 + units_per_wave, n_units);
     const int seg_blocks = (u1 - u0) * F::UNIT_BLOCKS;
-    const int passes = 1 << lp, rg = MV_MAX_RG >> lp;  // 64-piece passes per staged row; rows per group
-    const int row0 = blockIdx.x * rg;
+
+    // Staging geometry of the wave's segment: 16-byte pieces from the aligned address at or below the segment.
+    // Row r of a group: pieces from (row start + seg_off) & ~15; its first segment byte lands at byte sh_r of its
+    // LDS row. Rows have different sh_r when row_bytes is not a multiple of 16.
+    // A wave whose segment is empty (fewer units than waves) stages the row's last unit instead and adds
+    // nothing (seg_blocks = 0): its loads stay inside the matrix without a special case.
+    const size_t seg_off = (size_t)min(u0, n_units - 1) * F::UNIT_BYTES;
+    const int seg_bytes = max(u1 - u0, 1) * F::UNIT_BYTES;
+    uint8_t *my = &stage[wave][0];
+    const int rstride = (seg_bytes + 15 + 16 + 15) & ~15;  // room for the leading offset and the trailing over-read
+    const int ppr = rstride / 16;                            // pieces per row (<= 64 * PASSES)
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    constexpr int NP = MV_MAX_RG;  // load slots per lane: slot i = (row i >> LP, pass i & (PASSES - 1))
+    u32x4 pc[NP];
+    // Every load is unconditional: loads under a branch would be waited for one by one. A row's address math is
+    // scalar (one row per slot); a lane only clamps its piece index to the row's last piece, so that no load
+    // leaves the matrix. A group past the end loads the last row eight times (cache hits, results unused).
+    auto issue = [&](int grp) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NP; i++) {
+            const int r = i >> LP;
+            const int row = min(grp * RG + r, N - 1);
+            const size_t start = row_bytes * (size_t)row + seg_off;
+            const uint8_t *first = W + (start & ~(size_t)15);
+            const uint32_t last_piece = (uint32_t)(((start & 15) + (size_t)seg_bytes - 1) >> 4);
+            const uint32_t c = min((uint32_t)(((i & (PASSES - 1)) << 6) + lane), last_piece);
+            pc[i] = *(const u32x4 *)(first + c * 16u);
+        }
+    };
+    int grp = blockIdx.x;
+    issue(grp);  // the first group's weights are on their way while the activations are read
+    __builtin_amdgcn_sched_barrier(0);  // keeps the activation loads behind the weight loads
 
     // the lane's activations (one global read each for the whole kernel)
-    float x[T][32], s0[T], s1[T];
+    typename F::X x[T];
 #pragma unroll
     for (int t = 0; t < T; t++) {
         const int jl = bl + 32 * t;
-        // every load is unconditional (a lane without a block re-reads the vector's start): loads under a branch
-        // would be waited for one by one
+        // a lane without a block re-reads the vector's start
         const float *ap = a + (jl < seg_blocks ? (size_t)(u0 * F::UNIT_BLOCKS + jl) * 32 : 0);
-        s0[t] = s1[t] = 0.f;
+        float v[32];
 #pragma unroll
         for (int i = 0; i < 8; i++) {
-            const float4 v = *(const float4 *)(ap + 4 * i);
-            x[t][4 * i] = v.x; x[t][4 * i + 1] = v.y; x[t][4 * i + 2] = v.z; x[t][4 * i + 3] = v.w;
+            const float4 q = *(const float4 *)(ap + 4 * i);
+            v[4 * i] = q.x; v[4 * i + 1] = q.y; v[4 * i + 2] = q.z; v[4 * i + 3] = q.w;
         }
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            s0[t] += x[t][i];
-            s1[t] += x[t][16 + i];
-        }
+        x[t].prep(v);
     }
 
-    // stage the wave's segment of the group's rows: 16-byte pieces from the aligned address at or below the segment
-    const size_t seg_off = (size_t)u0 * F::UNIT_BYTES;
-    const int seg_bytes = (u1 - u0) * F::UNIT_BYTES;
-    uint8_t *my = &stage[wave][0];
-    // Row r of the group: pieces from (row start + seg_off) & ~15; its first segment byte lands at byte sh_r of its
-    // LDS row. Rows have different sh_r when row_bytes is not a multiple of 16.
-    const int rstride = (seg_bytes + 15 + 16 + 15) & ~15;  // room for the leading offset and the trailing over-read
-    const int ppr = rstride / 16;                            // pieces per row (<= 64 * passes)
-    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-    constexpr int NP = MV_MAX_RG;  // load slots per lane: slot i = (row i >> lp, pass i & (passes - 1))
-    u32x4 pc[NP];
+    // A workgroup walks over row groups grp, grp + gridDim.x, ...: while it works on one group out of LDS, the
+    // next group's weights are in flight into registers. All its threads make the same number of trips.
+    for (int it = 0; grp < n_groups; grp += gridDim.x, it++) {
+        const int row0 = grp * RG;
 #pragma unroll
-    for (int i = 0; i < NP; i++) {
-        const int r = i >> lp, c = min(((i & (passes - 1)) << 6) + lane, ppr - 1);
-        const int row = min(row0 + r, N - 1);
-        const size_t start = row_bytes * (size_t)row + seg_off;
-        const size_t first = start & ~(size_t)15;
-        // pieces past the segment's end (the slack of rstride) are clamped to its last piece: never outside the matrix
-        const size_t last = (start + (size_t)max(seg_bytes, 1) - 1) & ~(size_t)15;
-        const size_t addr = seg_bytes > 0 ? min(first + (size_t)c * 16, last) : 0;  // an empty segment reads the matrix start
-        pc[i] = *(const u32x4 *)(W + addr);
-    }
-#pragma unroll
-    for (int i = 0; i < NP; i++) {
-        const int r = i >> lp, c = ((i & (passes - 1)) << 6) + lane;
-        if (c < ppr) *(u32x4 *)(my + (size_t)r * rstride + (size_t)c * 16) = pc[i];
-    }
-    // the wave reads only what it wrote: its own LDS operations are ordered, no barrier needed here
-
-    for (int r = rp; r < rg; r += 2) {
-        const int row = min(row0 + r, N - 1);
-        const int sh = (int)((row_bytes * (size_t)row + seg_off) & 15);
-        float acc = 0.f;
-#pragma unroll
-        for (int t = 0; t < T; t++) {
-            const int jl = bl + 32 * t;
-            if (jl < seg_blocks) acc += F::block(my, r * rstride + sh, jl, x[t], s0[t], s1[t]);
+        for (int i = 0; i < NP; i++) {
+            const int r = i >> LP, c = ((i & (PASSES - 1)) << 6) + lane;
+            if (c < ppr) *(u32x4 *)(my + r * rstride + c * 16) = pc[i];
         }
-        acc = half_wave_sum(acc);
-        if (bl == 0) part[wave][r] = acc;
+        // the wave reads only what it wrote: its own LDS operations are ordered, no barrier needed here
+        issue(grp + (int)gridDim.x);
+
+        float acc[RG / 2];
+#pragma unroll
+        for (int rr = 0; rr < RG / 2; rr++) {  // the lane's rows rp, rp + 2, ...: independent, so their LDS reads overlap
+            const int r = rp + 2 * rr;
+            const int row = min(row0 + r, N - 1);
+            const int sh = (int)((row_bytes * (size_t)row + seg_off) & 15);
+            acc[rr] = 0.f;
+#pragma unroll
+            for (int t = 0; t < T; t++) {
+                const int jl = bl + 32 * t;
+                if (jl < seg_blocks) acc[rr] += F::block(my, r * rstride + sh, jl, x[t]);
+            }
+        }
+#pragma unroll
+        for (int rr = 0; rr < RG / 2; rr++) {
+            const float v = half_wave_sum(acc[rr]);
+            if (bl == 0) part[it & 1][wave][rp + 2 * rr] = v;
+        }
+        __syncthreads();  // the other parity of part[] is written next trip, after its readers passed this barrier
+        if (tid < RG && row0 + tid < N) {
+            const float(*pp)[MV_MAX_RG] = part[it & 1];
+            float v = (pp[0][tid] + pp[1][tid]) + (pp[2][tid] + pp[3][tid]);
+            if (residual) v = __fadd_rn(residual[row0 + tid], v);
+            out[row0 + tid] = v;
+        }
     }
-    __syncthreads();
-    if (tid < rg && row0 + tid < N) {
-        float v = (part[0][tid] + part[1][tid]) + (part[2][tid] + part[3][tid]);
-        if (residual) v = __fadd_rn(residual[row0 + tid], v);
-        out[row0 + tid] = v;
+}
+
+int device_cus(vx_backend *be) {
+    static int cus = 0;
+    if (cus == 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0) cus = 256;
     }
+    return cus;
+}
+
+// Launches qmatvec_kernel<F, T, LP> on as many workgroups as are resident at once (registers and LDS, asked once
+// per instantiation), each walking over several row groups.
+template <class F, int T, int LP>
+void launch_tl(vx_backend *be, const uint8_t *W, const float *a, float *out, const float *residual, int n, int k,
+               size_t rb, int upw) {
+    static int per_cu = 0;
+    if (per_cu == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, qmatvec_kernel<F, T, LP>, MV_THREADS, 0) != hipSuccess || per_cu < 1)
+            per_cu = 1;
+    }
+    const int n_groups = ceil_div(n, MV_MAX_RG >> LP);
+    const dim3 grid(std::min(n_groups, per_cu * device_cus(be)));
+    qmatvec_kernel<F, T, LP><<<grid, MV_THREADS, 0, be->stream>>>(W, a, out, residual, n, k, rb, upw, n_groups);
 }
 
 template <class F>
@@ -234,15 +384,14 @@ int launch(vx_backend *be, const uint8_t *W, const float *a, float *out, const f
     int lp = 0;
     while ((64 << lp) < rstride / 16) lp++;
     if (lp > 2 || (MV_MAX_RG >> lp) * rstride > MV_WAVE_LDS) return VX_ERR_UNSUPPORTED;
-    const int rg = MV_MAX_RG >> lp;
     const size_t rb = (size_t)n_units * F::UNIT_BYTES;
-    const dim3 grid(ceil_div(n, rg));
-#define VX_MV(TT)                                                                                                    \
-    case TT:                                                                                                         \
-        qmatvec_kernel<F, TT><<<grid, MV_THREADS, 0, be->stream>>>(W, a, out, residual, n, k, rb, lp, upw);             \
+#define VX_MV(TT, LL)                                                          \
+    case TT * 4 + LL:                                                          \
+        launch_tl<F, TT, LL>(be, W, a, out, residual, n, k, rb, upw);          \
         break;
-    switch (T) {
-        VX_MV(1) VX_MV(2) VX_MV(3) VX_MV(4)
+    switch (T * 4 + lp) {
+        VX_MV(1, 0) VX_MV(1, 1) VX_MV(2, 0) VX_MV(2, 1) VX_MV(2, 2) VX_MV(3, 1) VX_MV(3, 2) VX_MV(4, 1) VX_MV(4, 2)
+    default: return VX_ERR_UNSUPPORTED;
     }
 #undef VX_MV
     VX_CHECK_LAUNCH();
