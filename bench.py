@@ -116,7 +116,7 @@ def attention_bytes(ctx_lens, c):
     return sum(2 * L * kvd * 2 + ((L + BLOCK - 1) // BLOCK) * 4 + 2 * qd * 4 for L in ctx_lens)
 
 
-def time_attention_kernel(be, mr, ctx_now, c, layers, reps):
+def time_attention_kernel(be, mr, ctx_now, c, layers, reps, from_step=False):
     """Average duration of one launch of the ragged paged-attention kernel, HIP events on the backend stream,
     cycling over the layers' pools so every launch streams from HBM. The result is left in split form
     (out = NULL), as in the decode step, where the next kernel merges the splits."""
@@ -124,25 +124,37 @@ def time_attention_kernel(be, mr, ctx_now, c, layers, reps):
     qd = c["num_heads"] * c["head_dim"]
     q = be.upload(np.random.default_rng(1).standard_normal((b, qd)).astype(np.float32), permanent=True)
     out = be.alloc_permanent(b * qd * 4)
-    bts = np.zeros((b, mr.cfg.max_blocks_per_seq), dtype=np.int32)
-    for i in range(b):
-        t = mr.block_table(i + 1)
-        bts[i, :len(t)] = t
-    d_bt = be.upload(bts, permanent=True)
-    d_len = be.upload(np.array(ctx_now, dtype=np.int32), permanent=True)
+    own = []
+    if from_step:
+        # exactly the decode step's call: its block-table matrix, row indices and kv lengths (ctx_now), for
+        # which the step's packing kernel has left the attention work list in the backend
+        d_bt, d_rows, d_len = mr.step_buffers()
+        got = be.download(d_len, (b,), np.int32)
+        if list(got) != list(ctx_now):
+            raise RuntimeError("the step's kv lengths are not the expected contexts")
+    else:
+        bts = np.zeros((b, mr.cfg.max_blocks_per_seq), dtype=np.int32)
+        for i in range(b):
+            t = mr.block_table(i + 1)
+            bts[i, :len(t)] = t
+        d_bt = be.upload(bts, permanent=True)
+        d_len = be.upload(np.array(ctx_now, dtype=np.int32), permanent=True)
+        d_rows = None
+        own = [d_bt, d_len]
     scale = 1.0 / math.sqrt(c["head_dim"])
     cap = mr.cfg.max_blocks_per_seq * BLOCK
 
     def run(n):
         for i in range(n):
             be.sdpa_paged_decode_ragged(q, mr.kv_pool(i % layers), True, d_bt, d_len, None, b, mr.cfg.max_blocks_per_seq,
-                                        BLOCK, c["num_heads"], c["num_kv_heads"], c["head_dim"], scale, cap)
+                                        BLOCK, c["num_heads"], c["num_kv_heads"], c["head_dim"], scale, cap,
+                                        table_rows=d_rows)
     run(layers)
     be.sync()
     be.timer_start()
     run(reps)
     ms = be.timer_stop_ms()
-    for p in (q, out, d_bt, d_len):
+    for p in [q, out] + own:
         be.free(p)
     return ms / reps
 
@@ -336,7 +348,7 @@ def main():
     ms_per_step = wall * 1e3 / args.steps
     ctx_now = [L + w + args.steps for L in ctx]
     # dominant kernel: ragged paged attention (one launch per layer per step)
-    attn_ms = time_attention_kernel(be, mr, ctx_now, c, args.layers, reps=4 * args.layers)
+    attn_ms = time_attention_kernel(be, mr, ctx_now, c, args.layers, reps=4 * args.layers, from_step=True)
     attn_bytes = attention_bytes(ctx_now, c)
     achieved = attn_bytes / (attn_ms * 1e-3) / 1e9
     out = {

@@ -53,6 +53,10 @@ int vh_model_set_layer(vh_model *m, int layer, const vh_layer_weights *w);
 /* embedding: F32 [vocab,hidden] on the device (loader rule, runtime/loader.go:275-288) */
 int vh_model_set_head(vh_model *m, const float *embedding, const float *final_norm, const vh_qweight *lm_head);
 void *vh_kv_pool(vh_model *m, int layer);  /* device base of a layer's block pool */
+/* Device arrays the last decode step ran on: the block-table matrix [slots, max_blocks_per_seq], the matrix
+ * row of every batch entry and the kv lengths (int32 each). For measuring or re-running the step's attention
+ * call in isolation; contents change with every step. */
+void vh_step_buffers(vh_model *m, const int32_t **block_tables, const int32_t **table_rows, const int32_t **kv_lens);
 
 /* GPUBlockPool (runtime/gpu_block_pool.go) */
 int vh_pool_create_sequence(vh_model *m, int64_t seq_id);                       /* :126 */

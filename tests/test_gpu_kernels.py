@@ -560,6 +560,55 @@ def test_paged_decode_single_batched_ragged(be, f16, shape):
     be.reset_pool()
 
 
+def test_attention_work_list_from_pack_batch(be):
+    """vx_pack_batch leaves a work list for the ragged decode attention (full 512-token items first, partial last
+    items from the longest down). The attention call that passes the packed kv_lens array takes the list; a call
+    with a copy of the same lengths in another array walks the (split, sequence) grid. Both give the same bits,
+    and match the oracle; writing the lengths through the library drops the list."""
+    rng = np.random.default_rng(36)
+    bs, hq, hk, d, nblocks = 16, 8, 2, 128, 400
+    pool = _make_pool(rng, True, nblocks, bs, hk, d)
+    dpool = be.upload(pool)
+    sc = np.float32(1 / math.sqrt(d))
+    pos = np.array([0, 511, 512, 700, 1023, 1536, 40, 1100, 255], dtype=np.int32)   # kv_len = pos + 1
+    B, mb = pos.size, 100
+    perm = rng.permutation(nblocks)
+    tables = np.zeros((B, mb), dtype=np.int32)
+    nblk = np.zeros(B, dtype=np.int32)
+    off = 0
+    for i, p_ in enumerate(pos):
+        nb = (int(p_) + 1 + bs - 1) // bs          # blocks already there, the new token's included
+        tables[i, :nb] = perm[off:off + nb]; nblk[i] = nb; off += nb
+    free = perm[off:].astype(np.int32)
+    d_t, d_n, d_f, d_c = be.upload(tables), be.upload(nblk), be.upload(free), be.upload(np.array([free.size], np.int32))
+    d_s, d_p = be.upload(np.arange(B, dtype=np.int32)), be.upload(pos)
+    cu, tp, sm, kl, st = be.alloc((B + 1) * 4), be.alloc(B * 4), be.alloc(B * 4), be.alloc(B * 4), be.alloc(4)
+    be.pack_batch(d_s, d_p, 0, B, B, d_t, mb, d_n, d_f, d_c, bs, cu, tp, sm, kl, st)
+    assert be.download(st, (1,), np.int32)[0] == 0
+    lens = be.download(kl, (B,), np.int32)
+    assert list(lens) == [int(p_) + 1 for p_ in pos]
+    q = rng.standard_normal((B, hq, d)).astype(np.float32)
+    dq = be.upload(q)
+    want = np.stack([nx.sdpa_paged_decode(q[i], pool, tables[i, :nblk[i]], int(nblk[i]), bs, hq, hk, d, sc,
+                                          int(lens[i]) - (int(nblk[i]) - 1) * bs) for i in range(B)])
+    o_list, o_grid, o_after = be.alloc(q.nbytes), be.alloc(q.nbytes), be.alloc(q.nbytes)
+    be.sdpa_paged_decode_ragged(dq, dpool, True, d_t, kl, o_list, B, mb, bs, hq, hk, d, sc, mb * bs)
+    kl2 = be.alloc(B * 4)
+    be.copy_buffer(kl, 0, kl2, 0, B * 4)
+    be.sdpa_paged_decode_ragged(dq, dpool, True, d_t, kl2, o_grid, B, mb, bs, hq, hk, d, sc, mb * bs)
+    got = be.download(o_list, q.shape, np.float32)
+    assert np.array_equal(got.view(np.uint32), be.download(o_grid, q.shape, np.float32).view(np.uint32))
+    _close(got, want, 1e-5, 3e-6, "attention over the packed work list")
+    # shorter lengths written into the packed array: the stale list must not be used
+    short = np.maximum(lens // 2, 1).astype(np.int32)
+    be.to_device(kl, short)
+    be.sdpa_paged_decode_ragged(dq, dpool, True, d_t, kl, o_after, B, mb, bs, hq, hk, d, sc, mb * bs)
+    want2 = np.stack([nx.sdpa_paged_decode(q[i], pool, tables[i, :nblk[i]], (int(short[i]) + bs - 1) // bs, bs, hq, hk, d, sc,
+                                           int(short[i]) - ((int(short[i]) + bs - 1) // bs - 1) * bs) for i in range(B)])
+    _close(be.download(o_after, q.shape, np.float32), want2, 1e-5, 3e-6, "attention after the lengths were rewritten")
+    be.reset_pool()
+
+
 def test_paged_multiquery_and_tree(be):
     rng = np.random.default_rng(34)
     bs, hq, hk, d, nblocks = 16, 8, 2, 64, 40

@@ -177,7 +177,7 @@ __global__ void __launch_bounds__(GEN_THREADS) attn_generic_kernel(AttnParams p)
 // block are in flight while the current block is reduced.
 // Partials (m, l, acc[D]) per (sequence, q head, split) go to a scratch buffer; paged_merge_kernel
 // combines the splits.
-constexpr int TPW = 512;  // tokens per workgroup
+constexpr int TPW = ATTN_TPW;  // tokens per workgroup
 constexpr int HOT_BS = 16;
 
 // Sum over the N adjacent lanes (N = 8 or 16, aligned) that hold one token's head vector, by DPP inside a
@@ -196,12 +196,20 @@ template <int D, int G>
 __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix,
     const int32_t *__restrict__ bt_rows, int max_blocks, const int32_t *__restrict__ kv_lens,
-    float *__restrict__ partial, int num_q_heads, int num_kv_heads, float scale, int max_splits) {
+    float *__restrict__ partial, int num_q_heads, int num_kv_heads, float scale, int max_splits,
+    const int32_t *__restrict__ items) {
     constexpr int LPT = D / 8;       // lanes per token
     constexpr int TPI = 64 / LPT;    // tokens per load instruction
     constexpr int NL = HOT_BS / TPI; // load instructions per block and per K or V
     typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-    const int kvh = blockIdx.x, split = blockIdx.y, seq = blockIdx.z;
+    const int kvh = blockIdx.x;
+    int split = blockIdx.y, seq = blockIdx.z;
+    if (items) {  // work list: grid.y runs over the items, the workgroups past the list's end are the grid's last
+        if ((int)blockIdx.y >= items[0]) return;
+        const int code = items[1 + blockIdx.y];
+        seq = code >> 16;
+        split = code & 0xFFFF;
+    }
     const int kv_len = kv_lens[seq];
     const int t_begin = split * TPW;
     if (t_begin >= kv_len) return;
@@ -520,10 +528,16 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
     size_t need = (size_t)batch * num_q_heads * max_splits * (D + 2) * sizeof(float);
     int rc = ensure_ws(be, &be->attn_ws, &be->attn_ws_bytes, need, "attention");
     if (rc) return rc;
-    dim3 grid(num_kv_heads, max_splits, batch);
+    // With a work list from vx_pack_batch for these lengths the grid's second dimension runs over its items
+    // (at most max_splits per sequence, as max_kv_len bounds every length); otherwise over (split, sequence).
+    const bool listed = be->items.valid && be->items.kv_lens == kv_lens && be->items.batch == batch &&
+                        (size_t)batch * max_splits + 1 <= be->items.bytes / sizeof(int32_t) &&
+                        (size_t)batch * max_splits <= 65535;
+    dim3 grid(num_kv_heads, listed ? batch * max_splits : max_splits, listed ? 1 : batch);
     paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
                                                                 max_blocks, kv_lens, (float *)be->attn_ws, num_q_heads,
-                                                                num_kv_heads, scale, max_splits);
+                                                                num_kv_heads, scale, max_splits,
+                                                                listed ? be->items.buf : nullptr);
     VX_CHECK_LAUNCH();
     be->split.batch = 0;
     if (!out) {  // the caller merges: vx_decode_ffn(attn = NULL)

@@ -92,6 +92,7 @@ void vx_backend_destroy(vx_backend *be) {
     if (be->gemm_ws) (void)hipFree(be->gemm_ws);
     if (be->part_ws) (void)hipFree(be->part_ws);
     if (be->attn_ws) (void)hipFree(be->attn_ws);
+    if (be->items.buf) (void)hipFree(be->items.buf);
     if (be->misc_ws) (void)hipFree(be->misc_ws);
     if (be->prep_sync) (void)hipFree(be->prep_sync);
     if (be->host_stage) (void)hipHostFree(be->host_stage);
@@ -152,6 +153,7 @@ void vx_free(vx_backend *be, void *ptr) {
     if (!ptr || enter(be) != VX_OK) return;
     auto it = be->permanent.find(ptr);
     if (it == be->permanent.end()) return;  // pool buffer: recycled by vx_reset_pool
+    items_written(be, ptr, it->second);
     (void)hipStreamSynchronize(be->stream);
     (void)hipFree(ptr);
     be->permanent.erase(it);
@@ -161,6 +163,7 @@ void vx_reset_pool(vx_backend *be) {
     if (!be) return;
     for (auto &c : be->chunks) c.used = 0;
     be->cur_chunk = 0;
+    be->items.valid = false;  // a kv_lens array taken from the pool is about to be reused
 }
 
 int vx_to_device(vx_backend *be, void *dst, const void *src_host, size_t bytes) {
@@ -169,6 +172,7 @@ int vx_to_device(vx_backend *be, void *dst, const void *src_host, size_t bytes) 
     if (!dst || bytes == 0) return VX_OK;  // CPUBackend.ToDevice ignores nil / empty (cpu.go:57-63)
     VX_REQUIRE(src_host != nullptr, "vx_to_device: null source");
     VX_REQUIRE(!be->capturing, "vx_to_device during graph capture");
+    items_written(be, dst, bytes);
     VX_CHECK_HIP(hipMemcpyAsync(dst, src_host, bytes, hipMemcpyHostToDevice, be->stream));
     VX_CHECK_HIP(hipStreamSynchronize(be->stream));
     return VX_OK;
@@ -198,6 +202,7 @@ int vx_copy_buffer(vx_backend *be, const void *src, size_t src_off, void *dst, s
     if (rc) return rc;
     if (bytes == 0) return VX_OK;
     VX_REQUIRE(src && dst, "vx_copy_buffer: null pointer");
+    items_written(be, (char *)dst + dst_off, bytes);
     VX_CHECK_HIP(hipMemcpyAsync((char *)dst + dst_off, (const char *)src + src_off, bytes,
                                 hipMemcpyDeviceToDevice, be->stream));
     return VX_OK;

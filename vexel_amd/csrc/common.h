@@ -76,6 +76,17 @@ struct vx_backend {
         const int32_t *kv_lens = nullptr;
     } split;
     size_t attn_ws_bytes = 0;
+    // Work list of the ragged decode attention, written on the device by vx_pack_batch next to kv_lens:
+    // buf[0] = number of items, buf[1 + i] = (batch index << 16) | split, full splits first, then the
+    // sequences' partial last splits from the longest down. Valid for attention calls that pass the same
+    // kv_lens pointer and batch, until the library is asked to write into that array by other means.
+    struct {
+        int32_t *buf = nullptr;
+        size_t bytes = 0;
+        const int32_t *kv_lens = nullptr;
+        int batch = 0;
+        bool valid = false;
+    } items;
     void *misc_ws = nullptr;     // small device staging (pointer tables, argmax result)
     size_t misc_ws_bytes = 0;
     void *host_stage = nullptr;  // pinned host staging
@@ -90,6 +101,15 @@ struct vx_graph {
 };
 
 namespace vx {
+
+constexpr int ATTN_TPW = 512;  // tokens of one (sequence, kv head) that one attention workgroup takes
+
+// Drops the attention work list when [dst, dst + bytes) overlaps the kv_lens array it was built from.
+inline void items_written(vx_backend *be, const void *dst, size_t bytes) {
+    if (!be->items.valid) return;
+    const char *a = (const char *)dst, *k = (const char *)be->items.kv_lens;
+    if (a < k + (size_t)be->items.batch * 4 && k < a + bytes) be->items.valid = false;
+}
 
 // Makes be->device current on the calling thread (Go moves goroutines across OS threads).
 int enter(vx_backend *be);

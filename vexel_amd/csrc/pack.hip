@@ -38,7 +38,7 @@ __global__ void __launch_bounds__(PK_THREADS) pack_batch_kernel(
     const int32_t *seq_slots, const int32_t *positions, const int32_t *q_lens, int batch, int total_tokens,
     int32_t *block_tables, int max_blocks, int32_t *num_blocks, int32_t *free_list, int32_t *free_count,
     int block_size, int32_t *cu_seqlens, int32_t *token_pos, int32_t *slot_mapping, int32_t *kv_lens,
-    int32_t *status) {
+    int32_t *status, int32_t *items, int items_cap) {
     __shared__ int sm[PK_THREADS];
     __shared__ int s_cu[PK_THREADS + 1];
     const int tid = threadIdx.x;
@@ -69,8 +69,35 @@ __global__ void __launch_bounds__(PK_THREADS) pack_batch_kernel(
     const bool any_fail = sm[0] != 0;
     __syncthreads();
     if (any_fail) {
-        if (tid == 0) *status = 1;
+        if (tid == 0) {
+            *status = 1;
+            if (items) items[0] = 0;
+        }
         return;
+    }
+    if (items) {
+        // The attention work list: one item per ATTN_TPW tokens of a sequence. Equal (full) items first, in
+        // batch order; then the partial last items from the longest down, so that the kernel's last
+        // workgroups are its smallest.
+        const int len = act ? pos + ql : 0;
+        const int full = len / ATTN_TPW, rest = len % ATTN_TPW;
+        int total_full;
+        const int off = block_exclusive_scan(full, sm, &total_full);
+        sm[tid] = rest;
+        __syncthreads();
+        int before = 0, partials = 0;  // partial items ahead of this one; partial items in all
+        for (int j = 0; j < batch; j++) {
+            const int rj = sm[j];
+            partials += rj > 0;
+            before += (rj > rest) || (rj == rest && rj > 0 && j < tid);
+        }
+        __syncthreads();
+        const int n_items = total_full + partials;
+        if (n_items <= items_cap) {
+            for (int s2 = 0; s2 < full; s2++) items[1 + off + s2] = (tid << 16) | s2;
+            if (rest > 0) items[1 + total_full + before] = (tid << 16) | full;
+        }
+        if (tid == 0) items[0] = n_items <= items_cap ? n_items : -1;  // -1: the list did not fit, not to be used
     }
     if (act) {
         for (int j = 0; j < need; j++)
@@ -118,11 +145,24 @@ extern "C" int vx_pack_batch(vx_backend *be, const int32_t *seq_slots, const int
                "vx_pack_batch: null pointer");
     VX_REQUIRE(batch >= 1 && batch <= PK_THREADS, "vx_pack_batch: batch %d not in 1..%d", batch, PK_THREADS);
     VX_REQUIRE(block_size >= 1 && max_blocks >= 1 && total_tokens >= 0, "vx_pack_batch: bad sizes");
+    // room for the attention work list: every sequence at the longest context its block table allows
+    const size_t per_seq = ((size_t)max_blocks * block_size + ATTN_TPW - 1) / ATTN_TPW;
+    const size_t cap = (size_t)batch * per_seq;
+    int32_t *items = nullptr;
+    be->items.valid = false;
+    if (batch <= 32767 && per_seq <= 65535 &&
+        ensure_ws(be, (void **)&be->items.buf, &be->items.bytes, (cap + 1) * sizeof(int32_t), "attention work list") == VX_OK)
+        items = be->items.buf;
     pack_batch_kernel<<<1, PK_THREADS, 0, be->stream>>>(seq_slots, positions, q_lens, batch, total_tokens,
                                                         block_tables, max_blocks, num_blocks, free_list, free_count,
                                                         block_size, cu_seqlens, token_pos, slot_mapping, kv_lens,
-                                                        status);
+                                                        status, items, (int)cap);
     VX_CHECK_LAUNCH();
+    if (items) {
+        be->items.kv_lens = kv_lens;
+        be->items.batch = batch;
+        be->items.valid = true;
+    }
     return VX_OK;
 }
 

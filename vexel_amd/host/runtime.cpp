@@ -425,6 +425,12 @@ void *vh_kv_pool(vh_model *m, int layer) {
     return (m && layer >= 0 && layer < m->cfg.num_layers) ? m->kv[layer] : nullptr;
 }
 
+void vh_step_buffers(vh_model *m, const int32_t **block_tables, const int32_t **table_rows, const int32_t **kv_lens) {
+    if (block_tables) *block_tables = m ? m->d_tables : nullptr;
+    if (table_rows) *table_rows = m ? m->d_slots : nullptr;
+    if (kv_lens) *kv_lens = m ? m->d_kv_lens : nullptr;
+}
+
 // ------------------------------------------------------------------ GPUBlockPool
 int vh_pool_create_sequence(vh_model *m, int64_t seq_id) {
     std::lock_guard<std::mutex> g(m->pool.mu);

@@ -42,6 +42,8 @@ def load_host():
         h.vh_last_error.restype = C.c_char_p
         h.vh_kv_pool.restype = C.c_void_p
         h.vh_kv_pool.argtypes = [C.c_void_p, C.c_int]
+        h.vh_step_buffers.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
+        h.vh_step_buffers.restype = None
         h.vh_model_create.argtypes = [C.c_void_p, C.POINTER(VhConfig), C.POINTER(C.c_void_p)]
         h.vh_model_destroy.argtypes = [C.c_void_p]
         h.vh_model_destroy.restype = None
@@ -135,6 +137,12 @@ class ModelRuntime:
 
     def kv_pool(self, layer):
         return self._h.vh_kv_pool(self._m, layer)
+
+    def step_buffers(self):
+        """(block-table matrix, table rows, kv lengths): device addresses of the last decode step's metadata."""
+        p = [C.c_void_p(), C.c_void_p(), C.c_void_p()]
+        self._h.vh_step_buffers(self._m, C.byref(p[0]), C.byref(p[1]), C.byref(p[2]))
+        return tuple(x.value for x in p)
 
     # ---- GPUBlockPool
     def create_sequence(self, seq_id):
