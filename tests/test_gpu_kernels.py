@@ -143,6 +143,26 @@ def test_matvec_single_row(be, fmt, n, k):
     be.reset_pool()
 
 
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("m,n,k", [(5, 96, 11008), (32, 40, 14336), (16, 7, 4096), (33, 200, 256)])
+def test_matmul_batched_shapes(be, fmt, m, n, k):
+    """M >= 2 at the 7B / 8B reduction lengths: Q6_K rows of 9030 bytes (every even 16-byte phase), row groups
+    running past N, one-chunk reductions, M just past a tile boundary; with and without the residual."""
+    rng = np.random.default_rng(fmt * 77 + m + n)
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    want = nx.matmul_quant(fmt, a, w, m, n, k)
+    da, dw, dres = be.upload(a), be.upload(w), be.upload(res)
+    dout = be.alloc(m * n * 4)
+    scale = np.abs(want).max()
+    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
+    _close(be.download(dout, (m, n), np.float32), want, 2e-5, 3e-6 * scale + 1e-7, "matmul fmt %d %dx%dx%d" % (fmt, m, n, k))
+    be.matmul_quant(fmt, da, dw, dout, dres, m, n, k)
+    _close(be.download(dout, (m, n), np.float32), want + res, 2e-5, 3e-6 * scale + 1e-6, "matmul + residual")
+    be.reset_pool()
+
+
 def test_prepared_activation_paths(be):
     """prepare-once / multiply-many equals the one-shot entry point bit for bit, and the fused
     RMSNorm / SiLU*up prepares equal the separate ops."""

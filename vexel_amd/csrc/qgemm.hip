@@ -1359,11 +1359,12 @@ int prep_reserve(vx_backend *be, int m, int kmax) {
     return ensure_ws(be, &be->gemm_ws, &be->gemm_ws_bytes, need, "prepared activations");
 }
 
-template <class F, int R>
-int launch_gemm_r(vx_backend *be, const Segs &segs, int N, float *out, const float *residual, bool to_partials, int M,
-                  int K, int *ks_out) {
+template <class F>
+int launch_gemm(vx_backend *be, const Segs &segs, int N, float *out, const float *residual, bool to_partials, int M,
+                int K, int *ks_out) {
     const int mpad = mpad_for(M);
     const PrepView pv = prep_view(be, mpad, K);
+    constexpr int R = 2;
     const int rg = ceil_div(N, 64 * R);
     const int mgroups = mpad <= 16 ? 1 : mpad / 32;
     const int n_chunks = ceil_div(K / 32, CH);
@@ -1405,15 +1406,6 @@ int launch_gemm_r(vx_backend *be, const Segs &segs, int N, float *out, const flo
         VX_CHECK_LAUNCH();
     }
     return VX_OK;
-}
-
-template <class F>
-int launch_gemm(vx_backend *be, const Segs &segs, int N, float *out, const float *residual, bool to_partials, int M,
-                int K, int *ks_out) {
-    static const int r_env = getenv("VEXEL_HIP_GEMM_R") ? atoi(getenv("VEXEL_HIP_GEMM_R")) : 0;
-    static const int r1_max_n = getenv("VEXEL_HIP_GEMM_R1_MAX_N") ? atoi(getenv("VEXEL_HIP_GEMM_R1_MAX_N")) : 0;
-    if (r_env == 1 || N <= r1_max_n) return launch_gemm_r<F, 1>(be, segs, N, out, residual, to_partials, M, K, ks_out);
-    return launch_gemm_r<F, 2>(be, segs, N, out, residual, to_partials, M, K, ks_out);
 }
 
 int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out, const float *residual,
