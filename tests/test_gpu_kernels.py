@@ -97,18 +97,26 @@ def test_matmul_quant_vs_oracle(be, fmt, m):
 
 @pytest.mark.parametrize("fmt", FMTS)
 def test_matmul_rows_independent_of_batch(be, fmt):
-    """A row has the same bits in a batch of 2 as in a batch of 32 (the batched kernel's launch shape and
-    summation order do not depend on M; cf. the reference's loop of M=1 kernels, backend/metal/backend.go:777-779).
-    A single row (M = 1) goes through the matrix-vector kernel, whose float32 summation order differs: it agrees
-    to rounding, not bit for bit."""
+    """A row has the same bits in a batch of 2, of 32 and of 72 (the k-slices and the order their sums are added in
+    depend on the matrix and the device only; up to 32 rows the slices are separate workgroups, beyond that one
+    workgroup walks them in the same order; cf. the reference's loop of M=1 kernels,
+    backend/metal/backend.go:777-779). A single row (M = 1) goes through the matrix-vector kernel, whose
+    arithmetic differs: it agrees to rounding, not bit for bit."""
     rng = np.random.default_rng(9)
     m, n, k = 32, 96, 2048
     w = qz.random_quant(fmt, rng, n, k)
-    a = rng.standard_normal((m, k)).astype(np.float32)
-    da, dw = be.upload(a), be.upload(w)
+    big = rng.standard_normal((72, k)).astype(np.float32)
+    a = big[:m]
+    da, dw = be.upload(big), be.upload(w)
     dout = be.alloc(m * n * 4)
     be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
     full = be.download(dout, (m, n), np.float32)
+    dbig = be.alloc(72 * n * 4)
+    be.matmul_quant(fmt, da, dw, dbig, None, 72, n, k)
+    many = be.download(dbig, (72, n), np.float32)
+    assert np.array_equal(many[:m].view(np.uint32), full.view(np.uint32))
+    want = nx.matmul_quant(fmt, big, w, 72, n, k)
+    _close(many, want, 2e-5, 3e-6 * np.abs(want).max() + 1e-7, "72-row batch")
     for r in (0, 5, 30):
         d2 = be.alloc(2 * n * 4)
         be.matmul_quant(fmt, da + r * k * 4, dw, d2, None, 2, n, k)

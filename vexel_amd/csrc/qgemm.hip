@@ -29,6 +29,8 @@
 #include <stdlib.h>
 
 #include "common.h"
+#include <cstring>
+#include <algorithm>
 
 using namespace vx;
 
@@ -432,7 +434,7 @@ __device__ __forceinline__ const uint8_t *seg_row(const Segs &sg, int n, size_t 
 }
 
 // grid = (row groups of 64*R rows, KS k-slices, groups of MT activation tiles); block = 256.
-template <class F, int R, int MT>
+template <class F, int R, int MT, bool SERIAL>
 __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, PrepView pv, float *__restrict__ out,
                                                     const float *__restrict__ residual, float *__restrict__ partial,
                                                     int M, int Mpad, int N, int K, int n_slices, int flags) {
@@ -456,8 +458,11 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
     const int n_chunks = (steps_total + CH - 1) / CH;
     // balanced slices: the first n_chunks % n_slices slices hold one chunk more
     const int sl_base = n_chunks / n_slices, sl_rem = n_chunks % n_slices;
-    const int c_begin = ks * sl_base + min(ks, sl_rem);
-    const int c_end = c_begin + sl_base + (ks < sl_rem ? 1 : 0);
+    // SERIAL: this workgroup walks all slices itself, one after the other, and adds their sums in slice order:
+    // the same bits as one workgroup per slice plus the reduction, without the partial sums' round trip
+    constexpr bool serial = SERIAL;
+    const int c_begin = serial ? 0 : ks * sl_base + min(ks, sl_rem);
+    const int c_end = serial ? n_chunks : c_begin + sl_base + (ks < sl_rem ? 1 : 0);
 
     float4v run[R][MT];
 #pragma unroll
@@ -686,8 +691,22 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
                 for (int i = 0; i < 4; i++) run[r][t][i] += cs_cur[t][i] * crun[r][t][i];
     };
 
+    float4v total[SERIAL ? R : 1][SERIAL ? MT : 1];  // serial mode: the finished slices' sum (touched at slice ends only)
+    int slice = 0, slice_end = sl_base + (0 < sl_rem ? 1 : 0);
     if (c_begin < c_end) fetch(c_begin);
     for (int chunk = c_begin; chunk < c_end; chunk++) {
+        if constexpr (SERIAL) if (chunk == slice_end) {  // a slice is complete: fold it in, start the next from zero
+#pragma unroll
+            for (int r = 0; r < R; r++)
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++) total[r][t][i] = slice == 0 ? run[r][t][i] : total[r][t][i] + run[r][t][i];
+                    run[r][t] = (float4v){0.f, 0.f, 0.f, 0.f};
+                }
+            slice++;
+            slice_end += sl_base + (slice < sl_rem ? 1 : 0);
+        }
         __syncthreads();  // previous chunk's reads are done
         commit();
         __syncthreads();
@@ -696,6 +715,14 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
             compute_two_scales(chunk);
         else
             compute(chunk);
+    }
+    if constexpr (SERIAL) if (slice > 0) {
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) run[r][t][i] = total[r][t][i] + run[r][t][i];
     }
 
     // lane (g, ln) of tile (r, t) holds C[m = m0 + 16t + 4g + i][n = n0 + 16r + ln], i = 0..3. Each wave
@@ -1334,20 +1361,37 @@ int prep_begin(vx_backend *be, int m, int k, PrepView *pv) {
     return VX_OK;
 }
 
-// Workgroups the GEMM aims to keep resident: three per compute unit (VEXEL_HIP_GEMM_WGS overrides).
-int gemm_target_wgs(vx_backend *be) {
-    static int v = 0;
-    if (v == 0) {
-        const char *e = getenv("VEXEL_HIP_GEMM_WGS");
-        v = e ? atoi(e) : 0;
-        if (v <= 0) {
-            int cus = 0;
-            if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0)
-                cus = 256;
-            v = 3 * cus;
+// Number of k-slices for a GEMM of rg row groups (128 weight rows each) and n_chunks 256-column chunks: the count
+// that minimises a small model of the kernel's critical path, fitted to measurements of the 7B shapes at 32
+// rows. A compute unit holds two workgroups at a time; two together take about 1.4 times as long as one alone,
+// a third waits. Each slice costs a fixed 0.2 chunk times (the consumer's pass over it) plus its [M,N] float32
+// partial sums' trip through memory, which grows with the matrix' height.
+// VEXEL_HIP_KS="NxK:slices,..." (row groups x chunks, e.g. "96x16:4") overrides the choice for tuning.
+int gemm_slices(vx_backend *be, int rg, int n_chunks) {
+    static int cus = 0;
+    if (cus == 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0) cus = 256;
+    }
+    static const char *env = getenv("VEXEL_HIP_KS");
+    if (env) {
+        char key[64];
+        snprintf(key, sizeof key, "%dx%d:", rg, n_chunks);
+        const char *p = strstr(env, key);
+        if (p) return std::max(1, std::min(n_chunks, atoi(p + strlen(key))));
+    }
+    int best = 1;
+    float best_cost = 0.f;
+    for (int ks = 1; ks <= std::min(n_chunks, 32); ks++) {
+        const int per_cu = ceil_div(rg * ks, cus);  // workgroups on the busiest compute unit
+        const float rounds = (float)(per_cu / 2) * 1.4f + (float)(per_cu % 2);
+        const float per_slice = 0.2f + 0.8f * (float)rg / (float)cus;
+        const float cost = (float)ceil_div(n_chunks, ks) * rounds + per_slice * (float)ks;
+        if (ks == 1 || cost < best_cost) {
+            best = ks;
+            best_cost = cost;
         }
     }
-    return v;
+    return best;
 }
 
 // Grows the prepared-activation workspace for an [m, kmax] activation now, so that later prepares
@@ -1368,21 +1412,12 @@ int launch_gemm(vx_backend *be, const Segs &segs, int N, float *out, const float
     const int rg = ceil_div(N, 64 * R);
     const int mgroups = mpad <= 16 ? 1 : mpad / 32;
     const int n_chunks = ceil_div(K / 32, CH);
-    // Split K only as far as it takes to put about three workgroups on every CU, and never below four
-    // chunks per slice: every extra slice costs a [M,N] float32 round trip through memory, which writes
-    // far slower than it reads. The count depends on (N, K) and the device only, never on M: a row has the
-    // same bits alone or in a batch.
-    int ks = 1;
-    if (mgroups == 1) {
-        static int min_chunks = 0;
-        if (min_chunks == 0) {
-            const char *e = getenv("VEXEL_HIP_GEMM_MIN_CHUNKS");
-            min_chunks = e && atoi(e) > 0 ? atoi(e) : 4;
-        }
-        ks = gemm_target_wgs(be) / rg;
-        if (ks > n_chunks / min_chunks) ks = n_chunks / min_chunks;
-        if (ks < 1) ks = 1;
-    }
+    // How many slices to cut K into depends on (N, K) and the device only, never on M: a row has the same bits
+    // alone or in a batch. Up to 32 rows every slice is a workgroup of its own (grid.y) and the slices' sums go
+    // through memory; beyond that one workgroup per row group walks the slices in order (no partial sums).
+    const int n_slices = gemm_slices(be, rg, n_chunks);
+    const bool serial = mgroups > 1 && n_slices > 1;
+    const int ks = serial ? 1 : n_slices;
     float *partial = nullptr;
     if (ks > 1 || to_partials) {
         const size_t need = (size_t)ks * M * N * sizeof(float);
@@ -1394,9 +1429,11 @@ int launch_gemm(vx_backend *be, const Segs &segs, int N, float *out, const float
     const bool vec = N % 4 == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)residual % 16) == 0;
     const int flags = vec ? 1 : 0;
     if (mpad <= 16)
-        qgemm_kernel<F, R, 1><<<grid, 256, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, ks, flags);
+        qgemm_kernel<F, R, 1, false><<<grid, 256, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, n_slices, flags);
+    else if (!serial)
+        qgemm_kernel<F, R, 2, false><<<grid, 256, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, n_slices, flags);
     else
-        qgemm_kernel<F, R, 2><<<grid, 256, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, ks, flags);
+        qgemm_kernel<F, R, 2, true><<<grid, 256, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, n_slices, flags);
     VX_CHECK_LAUNCH();
     if (ks_out) *ks_out = ks;
     if (partial && !to_partials) {
