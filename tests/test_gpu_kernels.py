@@ -151,6 +151,27 @@ def test_matvec_single_row(be, fmt, n, k):
     be.reset_pool()
 
 
+@pytest.mark.parametrize("fmt", [nx.FMT_Q4_0, nx.FMT_Q6_K])
+def test_matmul_rows_independent_at_prefill_size(be, fmt):
+    """1024 rows against a 2048-row matrix: enough (row group, activation group) pairs that one workgroup walks
+    the k-slices in order instead of one workgroup per slice. Rows keep the bits they have in a batch of 2."""
+    rng = np.random.default_rng(19)
+    m, n, k = 1024, 2048, 512
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    da, dw = be.upload(a), be.upload(w)
+    dout = be.alloc(m * n * 4)
+    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
+    full = be.download(dout, (m, n), np.float32)
+    for r in (0, 517, 1022):
+        d2 = be.alloc(2 * n * 4)
+        be.matmul_quant(fmt, da + r * k * 4, dw, d2, None, 2, n, k)
+        assert np.array_equal(be.download(d2, (2, n), np.float32).view(np.uint32), full[r:r + 2].view(np.uint32))
+    want = nx.matmul_quant(fmt, a[:64], w, 64, n, k)
+    _close(full[:64], want, 2e-5, 3e-6 * np.abs(want).max() + 1e-7, "1024-row batch")
+    be.reset_pool()
+
+
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("m,n,k", [(5, 96, 11008), (32, 40, 14336), (16, 7, 4096), (33, 200, 256)])
 def test_matmul_batched_shapes(be, fmt, m, n, k):

@@ -1367,11 +1367,16 @@ int prep_begin(vx_backend *be, int m, int k, PrepView *pv) {
 // a third waits. Each slice costs a fixed 0.2 chunk times (the consumer's pass over it) plus its [M,N] float32
 // partial sums' trip through memory, which grows with the matrix' height.
 // VEXEL_HIP_KS="NxK:slices,..." (row groups x chunks, e.g. "96x16:4") overrides the choice for tuning.
-int gemm_slices(vx_backend *be, int rg, int n_chunks) {
+int gemm_cus(vx_backend *be) {
     static int cus = 0;
     if (cus == 0) {
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0) cus = 256;
     }
+    return cus;
+}
+
+int gemm_slices(vx_backend *be, int rg, int n_chunks) {
+    const int cus = gemm_cus(be);
     static const char *env = getenv("VEXEL_HIP_KS");
     if (env) {
         char key[64];
@@ -1413,10 +1418,12 @@ int launch_gemm(vx_backend *be, const Segs &segs, int N, float *out, const float
     const int mgroups = mpad <= 16 ? 1 : mpad / 32;
     const int n_chunks = ceil_div(K / 32, CH);
     // How many slices to cut K into depends on (N, K) and the device only, never on M: a row has the same bits
-    // alone or in a batch. Up to 32 rows every slice is a workgroup of its own (grid.y) and the slices' sums go
-    // through memory; beyond that one workgroup per row group walks the slices in order (no partial sums).
+    // alone or in a batch. With few rows every slice is a workgroup of its own (grid.y) and the slices' sums go
+    // through memory; once the row groups and 32-row activation groups alone fill the device twice over, one
+    // workgroup per (row group, activation group) walks the slices in order instead (no partial sums). Both
+    // forms add the same numbers in the same order.
     const int n_slices = gemm_slices(be, rg, n_chunks);
-    const bool serial = mgroups > 1 && n_slices > 1;
+    const bool serial = mgroups > 1 && n_slices > 1 && rg * mgroups >= 2 * gemm_cus(be);
     const int ks = serial ? 1 : n_slices;
     float *partial = nullptr;
     if (ks > 1 || to_partials) {
