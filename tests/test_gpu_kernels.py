@@ -245,10 +245,13 @@ def test_prepared_activation_paths(be):
 
 @pytest.mark.parametrize("fmt,rows,hidden,ffn", [(nx.FMT_Q4_0, 1, 512, 1024), (nx.FMT_Q4_0, 32, 512, 14336),
                                                  (nx.FMT_Q8_0, 5, 512, 1024), (nx.FMT_Q4_K, 40, 1024, 2048),
-                                                 (nx.FMT_Q6_K, 32, 512, 2816), (nx.FMT_Q6_K, 3, 1024, 1024)])
+                                                 (nx.FMT_Q6_K, 32, 512, 2816), (nx.FMT_Q6_K, 3, 1024, 1024),
+                                                 (nx.FMT_Q8_0, 1, 512, 1024), (nx.FMT_Q4_K, 1, 1024, 2048),
+                                                 (nx.FMT_Q6_K, 1, 1024, 2816), (nx.FMT_Q4_0, 1, 4096, 11008)])
 def test_fused_decode_blocks_equal_the_unfused_sequence(be, fmt, rows, hidden, ffn):
     """vx_decode_attn_qkv / vx_decode_ffn give what the one-call-per-operation sequence of
-    runtime/block.go:834-1077 gives (float32 activations, F16 and F32 pools), including the chained
+    runtime/block.go:834-1077 gives (float32 activations, F16 and F32 pools; one row goes through the
+    matrix-vector kernel with RMSNorm, SiLU*up and the residual adds folded in), including the chained
     prepared activation for the next block. A fused projection group is one launch over the summed
     width, so its split-K slices differ from the separate launches': values agree to float32 summation
     order (1e-5 of the row magnitude), not bit for bit; a chained call equals a fresh one exactly."""
@@ -375,6 +378,14 @@ def test_decode_ffn_merges_split_attention(be):
     be.decode_ffn(None, dx2, qw["wo"], dnw, eps, qw["w1"], qw["w3"], qw["w2"], rows, None)
     got = be.download(dx2, (rows, hidden), np.float32)
     assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want).max())
+    # one row (the matrix-vector path merges the partials while it reads its activation): sequence 2, 700 tokens
+    one = slice(2, 3)
+    dq1, dt1, dl1 = be.upload(q[one]), be.upload(tables[one]), be.upload(lens[one])
+    dx3 = be.upload(x[one])
+    be.sdpa_paged_decode_ragged(dq1, dpool, True, dt1, dl1, None, 1, max_blocks, bs, hq, hk, d, scale, max_blocks * bs)
+    be.decode_ffn(None, dx3, qw["wo"], dnw, eps, qw["w1"], qw["w3"], qw["w2"], 1, None)
+    got1 = be.download(dx3, (1, hidden), np.float32)
+    assert np.all(np.abs(got1 - want[one]) <= 2e-5 * np.abs(want).max())
     from vexel_amd.backend import VexelError
     with pytest.raises(VexelError):      # the pending split result was consumed
         be.decode_ffn(None, dx2, qw["wo"], dnw, eps, qw["w1"], qw["w3"], qw["w2"], rows, None)

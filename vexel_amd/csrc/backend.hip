@@ -79,6 +79,12 @@ int vx_backend_create(int device_id, vx_backend **out) {
     VX_CHECK_HIP(hipMalloc(&be->misc_ws, be->misc_ws_bytes));
     VX_CHECK_HIP(hipMalloc(&be->prep_sync, VX_PREP_SYNC_BYTES));
     VX_CHECK_HIP(hipMemset(be->prep_sync, 0, VX_PREP_SYNC_BYTES));  // arrival counters start at zero and reset themselves
+    {
+        float ones[64];
+        for (float &o : ones) o = 1.0f;
+        VX_CHECK_HIP(hipMalloc((void **)&be->ones, sizeof ones));
+        VX_CHECK_HIP(hipMemcpy(be->ones, ones, sizeof ones, hipMemcpyHostToDevice));
+    }
     *out = be;
     return VX_OK;
 }
@@ -95,6 +101,7 @@ void vx_backend_destroy(vx_backend *be) {
     if (be->items.buf) (void)hipFree(be->items.buf);
     if (be->misc_ws) (void)hipFree(be->misc_ws);
     if (be->prep_sync) (void)hipFree(be->prep_sync);
+    if (be->ones) (void)hipFree(be->ones);
     if (be->host_stage) (void)hipHostFree(be->host_stage);
     if (be->ev0) (void)hipEventDestroy(be->ev0);
     if (be->ev1) (void)hipEventDestroy(be->ev1);

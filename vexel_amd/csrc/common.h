@@ -87,6 +87,7 @@ struct vx_backend {
         int batch = 0;
         bool valid = false;
     } items;
+    float *ones = nullptr;       // 64 floats of 1.0 on the device (row factors of an unscaled activation)
     void *misc_ws = nullptr;     // small device staging (pointer tables, argmax result)
     size_t misc_ws_bytes = 0;
     void *host_stage = nullptr;  // pinned host staging
@@ -119,6 +120,22 @@ int ensure_ws(vx_backend *be, void **ptr, size_t *cap, size_t bytes, const char 
 // qmatvec.hip: out[n] = a . W[n] (+ residual[n]) for one activation row; VX_ERR_UNSUPPORTED (nothing launched, no
 // error text) when the shape is outside the kernel's range.
 int run_matvec(vx_backend *be, int fmt, const float *a, const void *b, float *out, const float *residual, int n, int k);
+// Where the matrix-vector kernel takes its activation row from: x itself; x * norm_w with the results divided
+// by rms(x) (RMSNorm folded in); or the attention output of one query merged from its split-KV partials.
+struct MatvecSource {
+    const float *x = nullptr;
+    const float *norm_w = nullptr;
+    float eps = 0.f;
+    const float *attn_partial = nullptr;
+    const int32_t *kv_len = nullptr;
+    int head_dim = 0, max_splits = 0, tokens_per_split = 0;
+};
+// Whether run_matvec_fused would take these matrices (format, K, alignment).
+bool matvec_ok(int fmt, const void *const *ws, const int *ns, int nw, int k);
+// Up to three matrices of one format and K with their rows concatenated (out has the summed height); pair != 0:
+// two matrices of equal height n, out[i] = silu(W0[i] . a) * (W1[i] . a), i < n.
+int run_matvec_fused(vx_backend *be, int fmt, const void *const *ws, const int *ns, int nw, int k, const MatvecSource &src,
+                     float *out, const float *residual, int pair);
 
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 static inline int64_t ceil_div64(int64_t a, int64_t b) { return (a + b - 1) / b; }

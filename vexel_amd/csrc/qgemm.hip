@@ -1646,6 +1646,33 @@ int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight,
     VX_REQUIRE(wq->n == num_q_heads * head_dim && wk->n == num_kv_heads * head_dim && wv->n == wk->n && block_size >= 1,
                "vx_decode_attn_qkv: weight shapes do not match the head geometry");
     const int k = wq->k;
+    static const bool no_matvec = getenv("VEXEL_HIP_NO_MATVEC") != nullptr;
+    if (rows == 1 && !x_prepared && !no_matvec && pool_is_f16 && head_dim % 2 == 0) {
+        // A single row: Q|K|V by one matrix-vector launch with the RMSNorm folded in (the row enters as x * w,
+        // the dot products are divided by rms(x)), then RoPE and the KV store from that launch's output.
+        const void *mw[3] = {wq->data, wk->data, wv->data};
+        const int mn[3] = {wq->n, wk->n, wv->n};
+        const int ntot1 = wq->n + wk->n + wv->n;
+        if (x && norm_weight && matvec_ok(wq->fmt, mw, mn, 3, k)) {
+            rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, (size_t)ntot1 * sizeof(float), "split-K partial sums");
+            if (rc) return rc;
+            MatvecSource src;
+            src.x = x;
+            src.norm_w = norm_weight;
+            src.eps = eps;
+            rc = run_matvec_fused(be, wq->fmt, mw, mn, 3, k, src, (float *)be->part_ws, nullptr, 0);
+            if (rc) return rc;
+            const int half1 = head_dim / 2;
+            const int lanes1 = 256 / half1 > 0 ? 256 / half1 : 1;
+            const int max_heads1 = num_q_heads > num_kv_heads ? num_q_heads : num_kv_heads;
+            const RowNorm none = {nullptr, 0, 0.f, 0.f};
+            rope_store_partials_kernel<true><<<dim3(1, ceil_div(max_heads1, lanes1)), lanes1 * half1, 0, be->stream>>>(
+                (const float *)be->part_ws, 1, 1, be->ones, none, q_out, positions, slot_mapping, kv_pool, num_q_heads,
+                num_kv_heads, head_dim, block_size, theta);
+            VX_CHECK_LAUNCH();
+            return VX_OK;
+        }
+    }
     if (x_prepared) {
         VX_REQUIRE(be->prep_m == rows && be->prep_k == k, "vx_decode_attn_qkv: no prepared %dx%d activation (have %dx%d)",
                    rows, k, be->prep_m, be->prep_k);
@@ -1706,6 +1733,47 @@ int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight 
     VX_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)ffn_norm_weight % 16 == 0) && ((uintptr_t)next_norm_weight % 16 == 0),
                "vx_decode_ffn: unaligned pointer");
     const int hidden = wo->n, ffn = w1->n, mpad = mpad_for(rows);
+    static const bool no_matvec = getenv("VEXEL_HIP_NO_MATVEC") != nullptr;
+    if (rows == 1 && !no_matvec) {
+        // A single row: three matrix-vector launches. Wo takes the attention output (merged from the split
+        // partials on the fly when attn is NULL) and adds the residual; gate|up take x * ffn_norm / rms(x) and
+        // leave SiLU(gate) * up; down adds the residual.
+        const void *m1[1] = {wo->data}, *m2[2] = {w1->data, w3->data}, *m3[1] = {w2->data};
+        const int n1[1] = {wo->n}, n2[2] = {w1->n, w3->n}, n3[1] = {w2->n};
+        const bool merge_ok = attn || (be->split.head_dim % 32 == 0 && be->split.head_dim >= 32);
+        if (merge_ok && matvec_ok(wo->fmt, m1, n1, 1, wo->k) && matvec_ok(w1->fmt, m2, n2, 2, hidden) &&
+            matvec_ok(w2->fmt, m3, n3, 1, ffn)) {
+            rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, (size_t)ffn * sizeof(float), "split-K partial sums");
+            if (rc) return rc;
+            float *h = (float *)be->part_ws;
+            MatvecSource s1, s2, s3;
+            if (attn) {
+                VX_REQUIRE((uintptr_t)attn % 16 == 0, "vx_decode_ffn: unaligned pointer");
+                s1.x = attn;
+            } else {
+                s1.attn_partial = (const float *)be->attn_ws;
+                s1.kv_len = be->split.kv_lens;
+                s1.head_dim = be->split.head_dim;
+                s1.max_splits = be->split.max_splits;
+                s1.tokens_per_split = be->split.tokens_per_split;
+                be->split.batch = 0;
+            }
+            rc = run_matvec_fused(be, wo->fmt, m1, n1, 1, wo->k, s1, x, x, 0);
+            if (rc) return rc;
+            s2.x = x;
+            s2.norm_w = ffn_norm_weight;
+            s2.eps = eps;
+            rc = run_matvec_fused(be, w1->fmt, m2, n2, 2, hidden, s2, h, nullptr, 1);
+            if (rc) return rc;
+            s3.x = h;
+            rc = run_matvec_fused(be, w2->fmt, m3, n3, 1, ffn, s3, x, x, 0);
+            if (rc) return rc;
+            be->prep_m = 0;
+            be->prep_k = 0;
+            if (next_norm_weight) return vx_rmsnorm_prepare(be, x, next_norm_weight, nullptr, 1, hidden, eps);
+            return VX_OK;
+        }
+    }
     int ks, ntot;
     rc = prep_reserve(be, rows, ffn > wo->k ? (ffn > hidden ? ffn : hidden) : (wo->k > hidden ? wo->k : hidden));
     if (rc) return rc;

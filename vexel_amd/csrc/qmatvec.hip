@@ -246,20 +246,44 @@ struct VQ6_K {  // dequant.go:272-331: 210-byte super-block [ql 128][qh 64][int8
     }
 };
 
+// What one launch works on. Up to three weight matrices of one format and K, their rows concatenated (Q|K|V,
+// gate|up); where the activation row comes from; what happens to the dot products.
+struct MvArgs {
+    const uint8_t *w0, *w1, *w2;  // matrix i holds the concatenated rows [end_{i-1}, end_i)
+    int end0, end1;
+    int N, K;                     // concatenated rows; columns
+    size_t row_bytes;
+    int units_per_wave, n_groups;
+    int mode;                     // MV_PLAIN, MV_RMSNORM, MV_MERGED_ATTENTION
+    const float *x;               // the activation row (MV_PLAIN, MV_RMSNORM)
+    const float *norm_w;          // MV_RMSNORM: the row is x * norm_w and the dot products are divided by rms(x)
+    float eps;
+    const float *attn_partial;    // MV_MERGED_ATTENTION: split-KV partials (m, l, acc[D]) of one query,
+    const int32_t *kv_len;        //   [head][split][D + 2], merged on the fly (the row is the attention output)
+    int head_dim, max_splits, tokens_per_split;
+    int pair;                     // > 0: rows i and pair + i belong together, out[i] = silu(dot_i) * dot_{pair+i}
+    float *out;
+    const float *residual;        // added to the result (not with pair)
+};
+enum { MV_PLAIN = 0, MV_RMSNORM = 1, MV_MERGED_ATTENTION = 2 };
+
+__device__ __forceinline__ float mv_sigmoid(float v) { return 1.0f / (1.0f + (float)exp((double)(-v))); }  // cpu.go:384,397
+
 template <class F, int T, int LP>
-__global__ void __launch_bounds__(MV_THREADS) qmatvec_kernel(const uint8_t *__restrict__ W, const float *__restrict__ a,
-                                                             float *__restrict__ out, const float *__restrict__ residual,
-                                                             int N, int K, size_t row_bytes, int units_per_wave,
-                                                             int n_groups) {
+__global__ void __launch_bounds__(MV_THREADS) qmatvec_kernel(const MvArgs p) {
     constexpr int PASSES = 1 << LP, RG = MV_MAX_RG >> LP;  // 64-piece passes per staged row; rows per group
     __shared__ __attribute__((aligned(16))) uint8_t stage[MV_WAVES][MV_WAVE_LDS];
     __shared__ float part[2][MV_WAVES][MV_MAX_RG];
+    __shared__ float s_ss[MV_WAVES];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int bl = lane & 31, rp = lane >> 5;
+    const int N = p.N, K = p.K;
+    const size_t row_bytes = p.row_bytes;
     const int n_units = K / (32 * F::UNIT_BLOCKS);
-    const int u0 = min(wave * units_per_wave, n_units), u1 = min(u0 + units_per_wave, n_units);
+    const int u0 = min(wave * p.units_per_wave, n_units), u1 = min(u0 + p.units_per_wave, n_units);
     const int seg_blocks = (u1 - u0) * F::UNIT_BLOCKS;
+    const int pair = p.pair;
 
     // Staging geometry of the wave's segment: 16-byte pieces from the aligned address at or below the segment.
     // Row r of a group: pieces from (row start + seg_off) & ~15; its first segment byte lands at byte sh_r of its
@@ -274,16 +298,28 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec_kernel(const uint8_t *__re
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     constexpr int NP = MV_MAX_RG;  // load slots per lane: slot i = (row i >> LP, pass i & (PASSES - 1))
     u32x4 pc[NP];
+    // Row r of group grp in the concatenated row space. With pair the group's first half are rows of the first
+    // matrix and the second half the same rows of the second. Rows past the end repeat the last row.
+    auto crow = [&](int grp, int r) __attribute__((always_inline)) {
+        if (pair > 0) return (r / (RG / 2)) * pair + min(grp * (RG / 2) + r % (RG / 2), pair - 1);
+        return min(grp * RG + r, N - 1);
+    };
+    // Byte offset of a concatenated row inside its matrix, and the matrix (selects over values read once from
+    // the kernel arguments: indexing an argument array by row would turn into dependent loads).
+    auto row_off = [&](int row) __attribute__((always_inline)) {
+        const int local = row < p.end0 ? row : (row < p.end1 ? row - p.end0 : row - p.end1);
+        return row_bytes * (size_t)local + seg_off;
+    };
+    auto row_base = [&](int row) __attribute__((always_inline)) { return row < p.end0 ? p.w0 : (row < p.end1 ? p.w1 : p.w2); };
     // Every load is unconditional: loads under a branch would be waited for one by one. A row's address math is
     // scalar (one row per slot); a lane only clamps its piece index to the row's last piece, so that no load
     // leaves the matrix. A group past the end loads the last row eight times (cache hits, results unused).
     auto issue = [&](int grp) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < NP; i++) {
-            const int r = i >> LP;
-            const int row = min(grp * RG + r, N - 1);
-            const size_t start = row_bytes * (size_t)row + seg_off;
-            const uint8_t *first = W + (start & ~(size_t)15);
+            const int row = crow(grp, i >> LP);
+            const size_t start = row_off(row);
+            const uint8_t *first = row_base(row) + (start & ~(size_t)15);
             const uint32_t last_piece = (uint32_t)(((start & 15) + (size_t)seg_bytes - 1) >> 4);
             const uint32_t c = min((uint32_t)(((i & (PASSES - 1)) << 6) + lane), last_piece);
             pc[i] = *(const u32x4 *)(first + c * 16u);
@@ -293,26 +329,71 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec_kernel(const uint8_t *__re
     issue(grp);  // the first group's weights are on their way while the activations are read
     __builtin_amdgcn_sched_barrier(0);  // keeps the activation loads behind the weight loads
 
-    // the lane's activations (one global read each for the whole kernel)
+    // the lane's activations (read once for the whole kernel)
     typename F::X x[T];
+    float ss = 0.f;  // MV_RMSNORM: sum of squares of the lane's elements
 #pragma unroll
     for (int t = 0; t < T; t++) {
         const int jl = bl + 32 * t;
-        // a lane without a block re-reads the vector's start
-        const float *ap = a + (jl < seg_blocks ? (size_t)(u0 * F::UNIT_BLOCKS + jl) * 32 : 0);
+        const bool have = jl < seg_blocks;
+        const size_t e0 = have ? (size_t)(u0 * F::UNIT_BLOCKS + jl) * 32 : 0;  // a lane without a block re-reads the row's start
         float v[32];
+        if (p.mode == MV_MERGED_ATTENTION) {
+            // paged_merge_kernel's arithmetic for the 32 elements of this block (one head)
+            const int D = p.head_dim, qh = (int)(e0 / D), d0 = (int)(e0 % D);
+            const int ns = (p.kv_len[0] + p.tokens_per_split - 1) / p.tokens_per_split;
+            const float *pb = p.attn_partial + (size_t)qh * p.max_splits * (D + 2);
+            float M = -INFINITY, L = 0.f;
+            for (int sp = 0; sp < ns; sp++) M = fmaxf(M, pb[(size_t)sp * (D + 2)]);
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const float4 q = *(const float4 *)(ap + 4 * i);
-            v[4 * i] = q.x; v[4 * i + 1] = q.y; v[4 * i + 2] = q.z; v[4 * i + 3] = q.w;
+            for (int i = 0; i < 32; i++) v[i] = 0.f;
+            for (int sp = 0; sp < ns; sp++) {
+                const float *ps = pb + (size_t)sp * (D + 2);
+                const float f = exp2f(ps[0] - M);
+                L += ps[1] * f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float4 q = *(const float4 *)(ps + 2 + d0 + 4 * i);  // 8-byte aligned only: D + 2 floats per split
+                    v[4 * i] += q.x * f; v[4 * i + 1] += q.y * f; v[4 * i + 2] += q.z * f; v[4 * i + 3] += q.w * f;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < 32; i++) v[i] = L > 0.f ? v[i] / L : 0.f;
+        } else {
+            const float *ap = p.x + e0;
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float4 q = *(const float4 *)(ap + 4 * i);
+                v[4 * i] = q.x; v[4 * i + 1] = q.y; v[4 * i + 2] = q.z; v[4 * i + 3] = q.w;
+            }
+            if (p.mode == MV_RMSNORM) {
+                const float *wp = p.norm_w + e0;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    const float4 q = *(const float4 *)(wp + 4 * i);
+                    const float wv[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        if (have && rp == 0) ss = fmaf(v[4 * i + e], v[4 * i + e], ss);  // every element counted once
+                        v[4 * i + e] *= wv[e];
+                    }
+                }
+            }
         }
         x[t].prep(v);
+    }
+    float row_fac = 1.f;
+    if (p.mode == MV_RMSNORM) {  // 1/rms of the whole row: lanes, then waves, in a fixed order (cpu.go:200-220)
+        ss = half_wave_sum(ss);   // the second half-wave holds zeros
+        if (lane == 0) s_ss[wave] = ss;
+        __syncthreads();
+        const float tot = (s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3]);
+        row_fac = 1.0f / (float)sqrt((double)(tot / (float)K + p.eps));
     }
 
     // A workgroup walks over row groups grp, grp + gridDim.x, ...: while it works on one group out of LDS, the
     // next group's weights are in flight into registers. All its threads make the same number of trips.
-    for (int it = 0; grp < n_groups; grp += gridDim.x, it++) {
-        const int row0 = grp * RG;
+    for (int it = 0; grp < p.n_groups; grp += gridDim.x, it++) {
 #pragma unroll
         for (int i = 0; i < NP; i++) {
             const int r = i >> LP, c = ((i & (PASSES - 1)) << 6) + lane;
@@ -325,8 +406,7 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec_kernel(const uint8_t *__re
 #pragma unroll
         for (int rr = 0; rr < RG / 2; rr++) {  // the lane's rows rp, rp + 2, ...: independent, so their LDS reads overlap
             const int r = rp + 2 * rr;
-            const int row = min(row0 + r, N - 1);
-            const int sh = (int)((row_bytes * (size_t)row + seg_off) & 15);
+            const int sh = (int)(row_off(crow(grp, r)) & 15);
             acc[rr] = 0.f;
 #pragma unroll
             for (int t = 0; t < T; t++) {
@@ -340,11 +420,19 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec_kernel(const uint8_t *__re
             if (bl == 0) part[it & 1][wave][rp + 2 * rr] = v;
         }
         __syncthreads();  // the other parity of part[] is written next trip, after its readers passed this barrier
-        if (tid < RG && row0 + tid < N) {
-            const float(*pp)[MV_MAX_RG] = part[it & 1];
-            float v = (pp[0][tid] + pp[1][tid]) + (pp[2][tid] + pp[3][tid]);
-            if (residual) v = __fadd_rn(residual[row0 + tid], v);
-            out[row0 + tid] = v;
+        const float(*pp)[MV_MAX_RG] = part[it & 1];
+        if (pair > 0) {
+            const int i = grp * (RG / 2) + tid;
+            if (tid < RG / 2 && i < pair) {
+                const int j = tid + RG / 2;
+                const float g = ((pp[0][tid] + pp[1][tid]) + (pp[2][tid] + pp[3][tid])) * row_fac;
+                const float u = ((pp[0][j] + pp[1][j]) + (pp[2][j] + pp[3][j])) * row_fac;
+                p.out[i] = __fmul_rn(__fmul_rn(g, mv_sigmoid(g)), u);  // cpu.go:390-400
+            }
+        } else if (tid < RG && grp * RG + tid < N) {
+            float v = ((pp[0][tid] + pp[1][tid]) + (pp[2][tid] + pp[3][tid])) * row_fac;
+            if (p.residual) v = __fadd_rn(p.residual[grp * RG + tid], v);
+            p.out[grp * RG + tid] = v;
         }
     }
 }
@@ -360,21 +448,21 @@ int device_cus(vx_backend *be) {
 // Launches qmatvec_kernel<F, T, LP> on as many workgroups as are resident at once (registers and LDS, asked once
 // per instantiation), each walking over several row groups.
 template <class F, int T, int LP>
-void launch_tl(vx_backend *be, const uint8_t *W, const float *a, float *out, const float *residual, int n, int k,
-               size_t rb, int upw) {
+void launch_tl(vx_backend *be, MvArgs &a) {
     static int per_cu = 0;
     if (per_cu == 0) {
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, qmatvec_kernel<F, T, LP>, MV_THREADS, 0) != hipSuccess || per_cu < 1)
             per_cu = 1;
     }
-    const int n_groups = ceil_div(n, MV_MAX_RG >> LP);
-    const dim3 grid(std::min(n_groups, per_cu * device_cus(be)));
-    qmatvec_kernel<F, T, LP><<<grid, MV_THREADS, 0, be->stream>>>(W, a, out, residual, n, k, rb, upw, n_groups);
+    constexpr int RG = MV_MAX_RG >> LP;
+    a.n_groups = a.pair > 0 ? ceil_div(a.pair, RG / 2) : ceil_div(a.N, RG);
+    const dim3 grid(std::min(a.n_groups, per_cu * device_cus(be)));
+    qmatvec_kernel<F, T, LP><<<grid, MV_THREADS, 0, be->stream>>>(a);
 }
 
 template <class F>
-int launch(vx_backend *be, const uint8_t *W, const float *a, float *out, const float *residual, int n, int k) {
-    const int n_units = k / (32 * F::UNIT_BLOCKS);
+int launch(vx_backend *be, MvArgs &a) {
+    const int n_units = a.K / (32 * F::UNIT_BLOCKS);
     const int upw = ceil_div(n_units, MV_WAVES);
     const int seg_blocks = upw * F::UNIT_BLOCKS;
     const int T = ceil_div(seg_blocks, 32);
@@ -384,10 +472,11 @@ int launch(vx_backend *be, const uint8_t *W, const float *a, float *out, const f
     int lp = 0;
     while ((64 << lp) < rstride / 16) lp++;
     if (lp > 2 || (MV_MAX_RG >> lp) * rstride > MV_WAVE_LDS) return VX_ERR_UNSUPPORTED;
-    const size_t rb = (size_t)n_units * F::UNIT_BYTES;
-#define VX_MV(TT, LL)                                                          \
-    case TT * 4 + LL:                                                          \
-        launch_tl<F, TT, LL>(be, W, a, out, residual, n, k, rb, upw);          \
+    a.row_bytes = (size_t)n_units * F::UNIT_BYTES;
+    a.units_per_wave = upw;
+#define VX_MV(TT, LL)                   \
+    case TT * 4 + LL:                   \
+        launch_tl<F, TT, LL>(be, a);    \
         break;
     switch (T * 4 + lp) {
         VX_MV(1, 0) VX_MV(1, 1) VX_MV(2, 0) VX_MV(2, 1) VX_MV(2, 2) VX_MV(3, 1) VX_MV(3, 2) VX_MV(4, 1) VX_MV(4, 2)
@@ -398,30 +487,108 @@ int launch(vx_backend *be, const uint8_t *W, const float *a, float *out, const f
     return VX_OK;
 }
 
+// Bytes of one weight row, 0 when the format or K has no matrix-vector kernel.
+size_t mv_row_bytes(int fmt, int k) {
+    switch (fmt) {
+    case VX_Q4_0: return k % 32 == 0 ? (size_t)(k / 32) * 18 : 0;
+    case VX_Q8_0: return k % 32 == 0 ? (size_t)(k / 32) * 34 : 0;
+    case VX_Q4_K: return k % 256 == 0 ? (size_t)(k / 256) * 144 : 0;
+    case VX_Q6_K: return k % 256 == 0 ? (size_t)(k / 256) * 210 : 0;
+    }
+    return 0;
+}
+
+// Whether qmatvec_kernel has an instantiation for rows of this format and length.
+template <class F>
+bool shape_ok(int k) {
+    const int n_units = k / (32 * F::UNIT_BLOCKS);
+    const int upw = ceil_div(n_units, MV_WAVES);
+    const int T = ceil_div(upw * F::UNIT_BLOCKS, 32);
+    if (n_units < 1 || T > MV_MAX_T) return false;
+    const int rstride = (upw * F::UNIT_BYTES + 15 + 16 + 15) & ~15;
+    int lp = 0;
+    while ((64 << lp) < rstride / 16) lp++;
+    if (lp > 2 || (MV_MAX_RG >> lp) * rstride > MV_WAVE_LDS) return false;
+    switch (T * 4 + lp) {
+    case 4: case 5: case 8: case 9: case 10: case 13: case 14: case 17: case 18: return true;
+    }
+    return false;
+}
+
+int launch_fmt(vx_backend *be, int fmt, MvArgs &a) {
+    switch (fmt) {
+    case VX_Q4_0: return launch<VQ4_0>(be, a);
+    case VX_Q8_0: return launch<VQ8_0>(be, a);
+    case VX_Q4_K: return launch<VQ4_K>(be, a);
+    case VX_Q6_K: return launch<VQ6_K>(be, a);
+    }
+    return VX_ERR_UNSUPPORTED;
+}
+
 }  // namespace
 
 namespace vx {
 
+bool matvec_ok(int fmt, const void *const *ws, const int *ns, int nw, int k) {
+    const size_t rb = mv_row_bytes(fmt, k);
+    if (rb == 0 || nw < 1 || nw > 3) return false;
+    for (int i = 0; i < nw; i++)
+        if (ns[i] < 1 || ((uintptr_t)ws[i] % 16) != 0 || ((size_t)ns[i] * rb) % 16 != 0) return false;
+    switch (fmt) {
+    case VX_Q4_0: return shape_ok<VQ4_0>(k);
+    case VX_Q8_0: return shape_ok<VQ8_0>(k);
+    case VX_Q4_K: return shape_ok<VQ4_K>(k);
+    case VX_Q6_K: return shape_ok<VQ6_K>(k);
+    }
+    return false;
+}
+
 // out[n] = a . W[n] (+ residual[n]) for one activation row. VX_ERR_UNSUPPORTED (nothing launched) when the shape is
 // outside the kernel's range: the caller then takes another path.
 int run_matvec(vx_backend *be, int fmt, const float *a, const void *b, float *out, const float *residual, int n, int k) {
-    if (((uintptr_t)b % 16) != 0 || ((uintptr_t)a % 16) != 0 || n < 1) return VX_ERR_UNSUPPORTED;
-    const uint8_t *W = (const uint8_t *)b;
-    switch (fmt) {
-    case VX_Q4_0:
-        if (k % 32 != 0 || ((size_t)n * (k / 32) * 18) % 16 != 0) return VX_ERR_UNSUPPORTED;
-        return launch<VQ4_0>(be, W, a, out, residual, n, k);
-    case VX_Q8_0:
-        if (k % 32 != 0 || ((size_t)n * (k / 32) * 34) % 16 != 0) return VX_ERR_UNSUPPORTED;
-        return launch<VQ8_0>(be, W, a, out, residual, n, k);
-    case VX_Q4_K:
-        if (k % 256 != 0) return VX_ERR_UNSUPPORTED;
-        return launch<VQ4_K>(be, W, a, out, residual, n, k);
-    case VX_Q6_K:
-        if (k % 256 != 0 || ((size_t)n * (k / 256) * 210) % 16 != 0) return VX_ERR_UNSUPPORTED;
-        return launch<VQ6_K>(be, W, a, out, residual, n, k);
+    MatvecSource src;
+    src.x = a;
+    const void *ws[1] = {b};
+    const int ns[1] = {n};
+    return run_matvec_fused(be, fmt, ws, ns, 1, k, src, out, residual, 0);
+}
+
+// The general form: nw <= 3 matrices of one format and K, rows concatenated; the activation row from `src`;
+// pair != 0: two matrices of equal height, out[i] = silu(row i of the first) * (row i of the second).
+int run_matvec_fused(vx_backend *be, int fmt, const void *const *ws, const int *ns, int nw, int k, const MatvecSource &src,
+                     float *out, const float *residual, int pair) {
+    const size_t rb = mv_row_bytes(fmt, k);
+    if (rb == 0 || nw < 1 || nw > 3) return VX_ERR_UNSUPPORTED;
+    MvArgs a = {};
+    const uint8_t *w[3] = {nullptr, nullptr, nullptr};
+    int end[3] = {0, 0, 0}, tot = 0;
+    for (int i = 0; i < 3; i++) {
+        const int j = i < nw ? i : nw - 1;
+        if (i < nw) {
+            // aligned 16-byte pieces must stay inside each matrix: aligned base, a whole number of pieces
+            if (ns[i] < 1 || ((uintptr_t)ws[i] % 16) != 0 || ((size_t)ns[i] * rb) % 16 != 0) return VX_ERR_UNSUPPORTED;
+            tot += ns[i];
+        }
+        w[i] = (const uint8_t *)ws[j];
+        end[i] = tot;
     }
-    return VX_ERR_UNSUPPORTED;
+    if (pair && (nw != 2 || ns[0] != ns[1] || residual)) return VX_ERR_UNSUPPORTED;
+    a.w0 = w[0]; a.w1 = w[1]; a.w2 = w[2];
+    a.end0 = end[0]; a.end1 = end[1];
+    a.N = tot; a.K = k;
+    a.pair = pair ? ns[0] : 0;
+    a.out = out; a.residual = residual;
+    if (src.attn_partial) {
+        if (!src.kv_len || src.head_dim < 32 || src.head_dim % 32 != 0 || k % src.head_dim != 0) return VX_ERR_UNSUPPORTED;
+        a.mode = MV_MERGED_ATTENTION;
+        a.attn_partial = src.attn_partial; a.kv_len = src.kv_len;
+        a.head_dim = src.head_dim; a.max_splits = src.max_splits; a.tokens_per_split = src.tokens_per_split;
+    } else {
+        if (!src.x || ((uintptr_t)src.x % 16) != 0 || ((uintptr_t)src.norm_w % 16) != 0) return VX_ERR_UNSUPPORTED;
+        a.mode = src.norm_w ? MV_RMSNORM : MV_PLAIN;
+        a.x = src.x; a.norm_w = src.norm_w; a.eps = src.eps;
+    }
+    return launch_fmt(be, fmt, a);
 }
 
 }  // namespace vx

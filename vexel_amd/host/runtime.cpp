@@ -244,7 +244,7 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
     const vh_config &c = m->cfg;
     const vh_layer_weights &w = m->layers[layer];
     const float scale = (float)(1.0 / sqrt((double)c.head_dim));                          // block.go:862
-    if (rows > 1 && attn_fusable(m, layer)) {                                             // block.go:834-868
+    if (attn_fusable(m, layer)) {   // block.go:834-868; one row: matrix-vector launches inside the same entry points
         VXC(vx_decode_attn_qkv(m->be, m->x, w.attn_norm, c.eps, *chained ? 1 : 0, &w.wq, &w.wk, &w.wv, rows,
                                m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, c.num_heads, c.num_kv_heads,
                                c.head_dim, c.block_size, c.rope_theta, m->q));
@@ -259,7 +259,7 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
         VXC(vx_rope_store_paged(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
                                 c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta));  // :858, :868
     }
-    const bool ffn_fused = rows > 1 && m->fused && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
+    const bool ffn_fused = m->fused && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
                            vx_decode_ffn_supported(&w.wo, &w.w1, &w.w3, &w.w2);
     // the fused tail can merge the attention's split-KV partials itself
     const bool split = ffn_fused && (size_t)w.wo.k * 4 <= 64 * 1024 && c.head_dim % 4 == 0 &&
