@@ -31,6 +31,9 @@ typedef struct vh_config {
 } vh_config;
 
 typedef vx_qweight vh_qweight;  /* tensor.Tensor with a QuantProfile: raw GGUF blocks on the device */
+/* vh_qweight.fmt for a plain float32 [n,k] matrix (a dequantized or tied output head, runtime/loader.go:187-203,
+ * 596-600); accepted for the output head only. */
+enum { VH_F32 = 0 };
 
 typedef struct vh_layer_weights {  /* the BlockRuntime fields used by ExecuteWithPagedKV */
     const float *attn_norm, *ffn_norm;
@@ -45,6 +48,7 @@ const char *vh_last_error(void);
  * KV pool, the device mirror of the block tables and the activation buffers. */
 int vh_model_create(vx_backend *be, const vh_config *cfg, vh_model **out);
 void vh_model_destroy(vh_model *m);
+void vh_model_get_config(const vh_model *m, vh_config *out);  /* the configuration the model was created with */
 /* Decode uses vx_decode_attn_qkv / vx_decode_ffn wherever they support the weights (default on).
  * Off = the one-call-per-operation sequence of runtime/block.go; the two agree to float32
  * summation order. */
@@ -88,6 +92,59 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
  * advanced by the same rule afterwards. use_graph = 0 runs the same device-driven step eagerly. */
 int vh_decode_graph(vh_model *m, const int32_t *first_tokens, const int64_t *seq_ids, const int32_t *positions,
                     int batch, int steps, int use_graph, int32_t *out_tokens, float *ms_per_step);
+
+/* ---- GGUF checkpoints (inference/pkg/gguf/gguf.go; loader rule of inference/runtime/loader.go) ---------- */
+#define VH_GGUF_MAX_DIMS 4
+typedef struct vh_gguf vh_gguf;
+typedef struct vh_gguf_tensor {  /* gguf.TensorInfo (gguf.go:200-207) plus where its bytes are */
+    const char *name;            /* owned by the reader */
+    int n_dims;
+    uint64_t dims[VH_GGUF_MAX_DIMS]; /* file order: dims[0] is the innermost dimension (K of an [N,K] matrix) */
+    uint32_t type;               /* gguf.TensorType (gguf.go:38-60) */
+    uint64_t offset;             /* from the start of the data section */
+    uint64_t n_bytes;            /* ceil(elements / block) * bytes per block (gguf.go:594-604) */
+    const void *data;            /* host address inside the file mapping; NULL when the file ends before it */
+} vh_gguf_tensor;
+typedef struct vh_gguf_config {  /* File.extractModelConfig (gguf.go:504-582); 0 = key absent */
+    char architecture[64];
+    int num_layers, hidden, num_heads, num_kv_heads, ffn, context_length, vocab, rope_dim_count, head_dim;
+    float rope_theta;            /* 10000 when absent */
+    float rms_eps;
+} vh_gguf_config;
+/* gguf.Open (gguf.go:249-335): magic, version 2..3, metadata, tensor table, aligned data offset. The file is
+ * mapped read-only; nothing is copied until a tensor is used. */
+int vh_gguf_open(const char *path, vh_gguf **out);
+void vh_gguf_close(vh_gguf *g);
+uint32_t vh_gguf_version(const vh_gguf *g);
+int64_t vh_gguf_data_offset(const vh_gguf *g);
+int vh_gguf_num_tensors(const vh_gguf *g);
+int vh_gguf_tensor_at(const vh_gguf *g, int i, vh_gguf_tensor *out);
+int vh_gguf_find_tensor(const vh_gguf *g, const char *name, vh_gguf_tensor *out);  /* File.GetTensor (gguf.go:584-591) */
+int vh_gguf_num_metadata(const vh_gguf *g);
+const char *vh_gguf_metadata_key(const vh_gguf *g, int i);                         /* file order */
+int vh_gguf_meta_type(const vh_gguf *g, const char *key);                          /* gguf.MetadataType, -1 if absent */
+uint32_t vh_gguf_meta_u32(const vh_gguf *g, const char *key);                      /* MetadataValue.AsUint32 (gguf.go:158-169) */
+uint64_t vh_gguf_meta_u64(const vh_gguf *g, const char *key);                      /* AsUint64 (:172-181) */
+float vh_gguf_meta_f32(const vh_gguf *g, const char *key);                         /* AsFloat32 (:189-198) */
+const char *vh_gguf_meta_str(const vh_gguf *g, const char *key);                   /* NULL unless a string */
+int64_t vh_gguf_meta_array_len(const vh_gguf *g, const char *key);                 /* -1 unless an array */
+int vh_gguf_get_config(const vh_gguf *g, vh_gguf_config *out);
+/* gguf.GetLayerTensorName (pkg/gguf/loader.go:121-228), LLaMA-family names; others pass through. */
+int vh_gguf_tensor_name(const char *hf_name, char *out, size_t cap);
+
+typedef struct vh_load_options {  /* what the checkpoint does not say: the KV pool and batch geometry */
+    int block_size;               /* 0 = 16 */
+    int pool_blocks, max_seqs, max_blocks_per_seq, max_batch, kv_fp16;
+} vh_load_options;
+/* ModelRuntime.LoadWeightsGGUF + CopyWeightsToDevice (runtime/loader.go:28-212, 560-700) for LLaMA-family
+ * checkpoints: Q4_0 / Q8_0 / Q4_K / Q6_K projection matrices and output head go to the device as raw blocks,
+ * token_embd and the norm vectors as float32 (F32, F16 or one of those four types in the file), a missing
+ * output.weight is the embedding. One difference: a Q4_0 output head stays Q4_0 here, where the reference
+ * dequantizes it to float32 at load (same values, float32 summation order aside). The model owns the device
+ * copies; vh_model_destroy frees them. */
+int vh_model_load_gguf(vx_backend *be, const char *path, const vh_load_options *opt, vh_model **out);
+/* Hands a vx_alloc_permanent buffer to the model, which frees it in vh_model_destroy. */
+void vh_model_adopt_buffer(vh_model *m, void *device_ptr);
 
 #ifdef __cplusplus
 }

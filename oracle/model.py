@@ -55,7 +55,10 @@ class LayerWeights:
 
 
 def _mm(a, w: QWeight, m):
-    # block.go:506-552 matMulTransposed dispatch on the quant profile
+    # block.go:506-552 matMulTransposed dispatch on the quant profile; fmt 0 = a float32 [n,k] matrix
+    # (a dequantized or tied output head, model.go:394-404 -> Backend.MatMulTransposed)
+    if w.fmt == 0:
+        return nx.matmul_t_f32(a, w.data, m, w.n, w.k)
     return nx.matmul_quant(w.fmt, a, w.data, m, w.n, w.k)
 
 

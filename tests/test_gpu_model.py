@@ -218,6 +218,98 @@ def test_chunked_prefill_and_verify(be):
     mr.close()
 
 
+GGUF_TYPE = {nx.FMT_Q4_0: 2, nx.FMT_Q8_0: 8, nx.FMT_Q4_K: 12, nx.FMT_Q6_K: 14}
+
+
+@pytest.mark.parametrize("case", ["q4_k_m mix with output", "tied q8_0 embedding", "tied f16 embedding, q4_0"])
+def test_load_gguf_checkpoint(be, tmp_path, case):
+    """A checkpoint written as a GGUF file (oracle/gguf.py writer: llama.* metadata, llama.cpp tensor names) and read
+    back by the C++ loader gives the logits and greedy tokens of the oracle model built from the same tensors:
+    raw quantized projection matrices and head, token_embd and norms converted to float32 (from a quantized type,
+    F16 and F32), a missing output.weight tied to the embedding (runtime/loader.go:28-212, 596-600)."""
+    import os
+    from oracle import gguf as og
+    from oracle import quantize as qz
+    from vexel_amd.runtime import ModelRuntime
+    rng = np.random.default_rng(55)
+    cfg = om.ModelConfig(num_layers=2, hidden=512, num_heads=8, num_kv_heads=2, head_dim=64, ffn=1024, vocab=768,
+                         eps=1e-6, rope_theta=500000.0)
+    fmt = nx.FMT_Q4_0 if "q4_0" in case else nx.FMT_Q4_K
+    over = {"wv": nx.FMT_Q6_K, "w2": nx.FMT_Q6_K} if "mix" in case else {}
+    qd, kvd = cfg.num_heads * cfg.head_dim, cfg.num_kv_heads * cfg.head_dim
+    tensors, layers = [], []
+    f16 = lambda a: nx.f16_to_f32_array(nx.f32_to_f16_array(a.astype(np.float32)))
+    for l in range(cfg.num_layers):
+        ws = {}
+        for name, gname, n, k in (("wq", "attn_q", qd, cfg.hidden), ("wk", "attn_k", kvd, cfg.hidden),
+                                  ("wv", "attn_v", kvd, cfg.hidden), ("wo", "attn_output", cfg.hidden, qd),
+                                  ("w1", "ffn_gate", cfg.ffn, cfg.hidden), ("w3", "ffn_up", cfg.ffn, cfg.hidden),
+                                  ("w2", "ffn_down", cfg.hidden, cfg.ffn)):
+            f = over.get(name, fmt)
+            data = qz.random_quant(f, rng, n, k)
+            ws[name] = om.QWeight(f, data, n, k)
+            tensors.append(("blk.%d.%s.weight" % (l, gname), [k, n], GGUF_TYPE[f], data.tobytes()))
+        an = (1 + 0.1 * rng.standard_normal(cfg.hidden)).astype(np.float32)
+        fn = f16(1 + 0.1 * rng.standard_normal(cfg.hidden))          # stored as F16 in the file
+        tensors.append(("blk.%d.attn_norm.weight" % l, [cfg.hidden], og.T_F32, an.tobytes()))
+        tensors.append(("blk.%d.ffn_norm.weight" % l, [cfg.hidden], og.T_F16, nx.f32_to_f16_array(fn).tobytes()))
+        layers.append(om.LayerWeights(attn_norm=an, ffn_norm=fn, **ws))
+    final_norm = (1 + 0.1 * rng.standard_normal(cfg.hidden)).astype(np.float32)
+    tensors.append(("output_norm.weight", [cfg.hidden], og.T_F32, final_norm.tobytes()))
+    if "f16 embedding" in case:
+        emb = f16(0.05 * rng.standard_normal((cfg.vocab, cfg.hidden)))
+        tensors.append(("token_embd.weight", [cfg.hidden, cfg.vocab], og.T_F16, nx.f32_to_f16_array(emb.reshape(-1)).tobytes()))
+        head = om.QWeight(0, emb, cfg.vocab, cfg.hidden)               # tied, float32
+    else:
+        ef = nx.FMT_Q8_0 if "q8_0" in case else nx.FMT_Q4_0
+        eq = qz.random_quant(ef, rng, cfg.vocab, cfg.hidden)
+        emb = nx.dequantize(ef, eq, cfg.vocab * cfg.hidden).reshape(cfg.vocab, cfg.hidden)
+        tensors.append(("token_embd.weight", [cfg.hidden, cfg.vocab], GGUF_TYPE[ef], eq.tobytes()))
+        if "tied" in case:
+            head = om.QWeight(ef, eq, cfg.vocab, cfg.hidden)           # tied, raw blocks
+        else:
+            hq = qz.random_quant(nx.FMT_Q6_K, rng, cfg.vocab, cfg.hidden)
+            tensors.append(("output.weight", [cfg.hidden, cfg.vocab], GGUF_TYPE[nx.FMT_Q6_K], hq.tobytes()))
+            head = om.QWeight(nx.FMT_Q6_K, hq, cfg.vocab, cfg.hidden)
+    md = [("general.architecture", og.MT_STRING, "llama"), ("llama.block_count", og.MT_U32, cfg.num_layers),
+          ("llama.embedding_length", og.MT_U32, cfg.hidden), ("llama.attention.head_count", og.MT_U32, cfg.num_heads),
+          ("llama.attention.head_count_kv", og.MT_U32, cfg.num_kv_heads), ("llama.feed_forward_length", og.MT_U32, cfg.ffn),
+          ("llama.context_length", og.MT_U32, 2048), ("llama.rope.freq_base", og.MT_F32, cfg.rope_theta),
+          ("llama.attention.layer_norm_rms_epsilon", og.MT_F32, cfg.eps),
+          ("tokenizer.ggml.tokens", og.MT_ARRAY, (og.MT_STRING, ["t%d" % i for i in range(cfg.vocab)]))]
+    rng.shuffle(tensors)                                               # file order is not the loader's order
+    path = os.path.join(tmp_path, "model.gguf")
+    with open(path, "wb") as fh:
+        fh.write(og.build(md, [tuple(t) for t in tensors]))
+    omodel = om.OracleModel(cfg, emb, layers, final_norm, head, max_blocks=16)
+    mr = ModelRuntime.from_gguf(be, path, pool_blocks=16, max_seqs=4, max_batch=48)
+    c = mr.cfg
+    assert (c.num_layers, c.hidden, c.num_heads, c.num_kv_heads, c.head_dim, c.ffn, c.vocab) == \
+           (cfg.num_layers, cfg.hidden, cfg.num_heads, cfg.num_kv_heads, cfg.head_dim, cfg.ffn, cfg.vocab)
+    assert np.float32(c.eps) == np.float32(cfg.eps) and np.float32(c.rope_theta) == np.float32(cfg.rope_theta)
+    prompt = rng.integers(0, cfg.vocab, 40).tolist()
+    want = omodel.prefill_with_paged_kv(prompt, 1, 0)
+    got = mr.prefill_with_paged_kv(prompt, 1, 0)
+    assert_logits_close(got, want, "prefill logits from the loaded checkpoint")
+    tok, pos = nx.argmax(want), len(prompt)
+    assert tok == int(np.argmax(got))
+    for step in range(8):
+        want = omodel.decode_with_paged_kv(tok, 1, pos)
+        got, am = mr.decode_with_paged_kv_batched([tok], [1], [pos])
+        assert_logits_close(got[0], want, "decode step %d" % step)
+        tok = nx.argmax(want)
+        assert tok == int(am[0])
+        pos += 1
+    mr.close()
+    # a checkpoint the loader cannot take says why
+    from vexel_amd.backend import VexelError
+    bad = [t for t in tensors if t[0] != "blk.1.ffn_up.weight"]
+    with open(path, "wb") as fh:
+        fh.write(og.build(md, [tuple(t) for t in bad]))
+    with pytest.raises(VexelError, match="ffn_up"):
+        ModelRuntime.from_gguf(be, path, pool_blocks=16, max_seqs=4, max_batch=48)
+
+
 def test_pool_errors_and_lifecycle(be):
     """Host-forced failure paths: pool exhaustion, unknown sequence, truncate no-ops."""
     from vexel_amd.backend import VexelError

@@ -456,7 +456,10 @@ void launch_tl(vx_backend *be, MvArgs &a) {
     }
     constexpr int RG = MV_MAX_RG >> LP;
     a.n_groups = a.pair > 0 ? ceil_div(a.pair, RG / 2) : ceil_div(a.N, RG);
-    const dim3 grid(std::min(a.n_groups, per_cu * device_cus(be)));
+    // as many workgroups as fit at once, or fewer when that makes every workgroup's number of trips equal
+    const int resident = per_cu * device_cus(be);
+    const int trips = ceil_div(a.n_groups, resident);
+    const dim3 grid(ceil_div(a.n_groups, trips));
     qmatvec_kernel<F, T, LP><<<grid, MV_THREADS, 0, be->stream>>>(a);
 }
 

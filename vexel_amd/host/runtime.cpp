@@ -108,6 +108,7 @@ struct vh_model {
     const float *embedding = nullptr;
     const float *final_norm = nullptr;
     vh_qweight lm_head{};
+    std::vector<void *> adopted;  // device buffers a loader handed over (vh_model_adopt_buffer)
     BlockPool pool;
     std::vector<void *> kv;
 
@@ -188,6 +189,12 @@ bool fast(const vh_qweight &w) { return vx_matmul_quant_has_fast_path(w.fmt, w.d
 // unless every consumer takes the prepared path, in float32 at a_f32.
 int mm(vh_model *m, bool prepared, const float *a_f32, const vh_qweight &w, float *out, const float *residual, int rows) {
     if (!w.data) return fail("weight not set");
+    if (w.fmt == VH_F32) {  // a float32 output head: Backend.MatMulTransposed (model.go:394-404)
+        if (!a_f32) return fail("internal: a float32 matrix needs the float32 activation");
+        VXC(vx_matmul_transposed(m->be, a_f32, (const float *)w.data, out, rows, w.n, w.k));
+        if (residual) VXC(vx_add(m->be, out, residual, out, rows * w.n));
+        return VH_OK;
+    }
     if (prepared && fast(w)) {
         VXC(vx_matmul_quant_prepared(m->be, w.fmt, w.data, out, residual, rows, w.n, w.k));
         return VH_OK;
@@ -312,6 +319,15 @@ int check_ready(vh_model *m) {
 extern "C" {
 
 const char *vh_last_error(void) { return g_err; }
+void vh_set_error(const char *text) { snprintf(g_err, sizeof(g_err), "%s", text ? text : ""); }  // for gguf.cpp
+
+void vh_model_get_config(const vh_model *m, vh_config *out) {
+    if (m && out) *out = m->cfg;
+}
+
+void vh_model_adopt_buffer(vh_model *m, void *device_ptr) {
+    if (m && device_ptr) m->adopted.push_back(device_ptr);
+}
 
 int vh_model_create(vx_backend *be, const vh_config *cfg, vh_model **out) {
     if (!be || !cfg || !out) return fail("null argument");
@@ -388,6 +404,7 @@ void vh_model_destroy(vh_model *m) {
                     m->d_next, m->d_cu, m->d_token_pos, m->d_slot_map, m->d_kv_lens, m->d_status, m->d_step, m->d_log,
                     m->x, m->norm, m->q, m->k, m->v, m->attn, m->gate, m->up, m->logits};
     for (void *p : bufs) vx_free(m->be, p);
+    for (void *p : m->adopted) vx_free(m->be, p);
     delete m;
 }
 

@@ -22,6 +22,12 @@ class VhConfig(C.Structure):
 
 
 VhQWeight = VxQWeight  # vh_qweight is a typedef of vx_qweight
+VH_F32 = 0             # vh_qweight.fmt of a float32 output head
+
+
+class VhLoadOptions(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("block_size", "pool_blocks", "max_seqs", "max_blocks_per_seq", "max_batch",
+                                        "kv_fp16")]
 
 
 class VhLayerWeights(C.Structure):
@@ -47,6 +53,9 @@ def load_host():
         h.vh_model_create.argtypes = [C.c_void_p, C.POINTER(VhConfig), C.POINTER(C.c_void_p)]
         h.vh_model_destroy.argtypes = [C.c_void_p]
         h.vh_model_destroy.restype = None
+        h.vh_model_get_config.argtypes = [C.c_void_p, C.POINTER(VhConfig)]
+        h.vh_model_get_config.restype = None
+        h.vh_model_load_gguf.argtypes = [C.c_void_p, C.c_char_p, C.POINTER(VhLoadOptions), C.POINTER(C.c_void_p)]
         h.vh_model_set_fused.argtypes = [C.c_void_p, C.c_int]
         h.vh_model_set_fused.restype = None
         h.vh_model_set_layer.argtypes = [C.c_void_p, C.c_int, C.POINTER(VhLayerWeights)]
@@ -82,6 +91,25 @@ class ModelRuntime:
         self._ck(self._h.vh_model_create(be._h, C.byref(self.cfg), C.byref(m)))
         self._m = m
         self._keep = []   # device buffers owned by this model
+
+    @classmethod
+    def from_gguf(cls, be: HipBackend, path, block_size=16, pool_blocks=256, max_seqs=64, max_blocks_per_seq=None,
+                  max_batch=64, kv_fp16=True):
+        """ModelRuntime.LoadWeightsGGUF + CopyWeightsToDevice (runtime/loader.go): a LLaMA-family checkpoint read
+        by the C++ loader; the model owns the device copies of the weights."""
+        self = cls.__new__(cls)
+        self._h = load_host()
+        self.be = be
+        opt = VhLoadOptions(block_size, pool_blocks, max_seqs, max_blocks_per_seq or pool_blocks, max_batch,
+                            int(bool(kv_fp16)))
+        m = C.c_void_p()
+        self._m = None
+        self._keep = []
+        self._ck(self._h.vh_model_load_gguf(be._h, os.fsencode(path), C.byref(opt), C.byref(m)))
+        self._m = m
+        self.cfg = VhConfig()
+        self._h.vh_model_get_config(m, C.byref(self.cfg))
+        return self
 
     def _ck(self, rc):
         if rc != 0:
