@@ -146,6 +146,35 @@ int vh_model_load_gguf(vx_backend *be, const char *path, const vh_load_options *
 /* Hands a vx_alloc_permanent buffer to the model, which frees it in vh_model_destroy. */
 void vh_model_adopt_buffer(vh_model *m, void *device_ptr);
 
+/* ---- continuous-batching scheduler (inference/scheduler/scheduler.go, sequence.go; pkg/sampler/sampler.go) ---- */
+enum { VH_SEQ_PENDING = 0, VH_SEQ_PREFILL = 1, VH_SEQ_DECODING = 2, VH_SEQ_FINISHED = 3 };  /* sequence.go:15-20 */
+typedef struct vh_scheduler vh_scheduler;
+typedef struct vh_sched_config {  /* scheduler.Config (scheduler.go:24-36) */
+    int max_batch_size;           /* ready sequences per step */
+    int max_tokens;               /* generation limit per sequence, 0 = none */
+    int eos_token;                /* the stop token (scheduler.go:110-116) */
+    int prefill_chunk;            /* 0 = a prompt is prefilled in one call (scheduler.go:483-500); > 0 = in pieces of
+                                     this many tokens, one piece per step */
+} vh_sched_config;
+int vh_sched_create(vh_model *m, const vh_sched_config *cfg, vh_scheduler **out);
+void vh_sched_destroy(vh_scheduler *s);
+/* Scheduler.AddSequence (scheduler.go:645-677) with the prompt already tokenized; max_tokens 0 = the scheduler's. */
+int vh_sched_add_sequence(vh_scheduler *s, int64_t seq_id, const int32_t *prompt, int n, int max_tokens);
+/* Sequence.SetSamplingParams (sequence.go:150-160); temperature 0 = greedy. The uniform draws come from a
+ * SplitMix64 stream started at seed. */
+int vh_sched_set_sampling(vh_scheduler *s, int64_t seq_id, float temperature, int top_k, float top_p, uint64_t seed);
+int vh_sched_remove_sequence(vh_scheduler *s, int64_t seq_id);             /* scheduler.go:679-699 */
+int vh_sched_sequence_count(const vh_scheduler *s);                        /* scheduler.go:702-706 */
+int vh_sched_state(const vh_scheduler *s, int64_t seq_id);                 /* VH_SEQ_*, -1 if unknown */
+int vh_sched_position(const vh_scheduler *s, int64_t seq_id);
+int vh_sched_generated(const vh_scheduler *s, int64_t seq_id, int32_t *out, int cap);
+/* One Scheduler.step (scheduler.go:166-201): ready sequences in ascending id (the reference's map order is
+ * unspecified), prompts fed first, then one batched decode; *tokens_out = tokens generated. */
+int vh_sched_step(vh_scheduler *s, int *tokens_out);
+/* sampler.Argmax (sampler.go:80-91) and Sampler.Sample (sampler.go:48-77) on host logits, the uniform draw r given. */
+int vh_argmax(const float *logits, int n);
+int vh_sample(const float *logits, int n, float temperature, int top_k, float top_p, float r);
+
 #ifdef __cplusplus
 }
 #endif

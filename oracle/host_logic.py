@@ -6,8 +6,11 @@ candidate trees follow inference/medusa/tree.go; greedy verification and rollbac
 follow inference/scheduler/medusa_scheduler.go:852,934-977. All results are integers
 and are compared bit-exactly.
 """
+import math
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Tuple
+
+import numpy as np
 
 
 # --------------------------------------------------------------------------- block pool
@@ -460,3 +463,168 @@ def greedy_tree_accept(tokens, parent_idx, root_argmax, node_argmax):
             return accepted, want
         accepted.append(nxt)
         cur, want = nxt, node_argmax[nxt]
+
+
+# --------------------------------------------------------------------------- sampler and scheduler step
+def sampler_argmax(logits):
+    """sampler.go:80-91: first index of the strict maximum, starting from -MaxFloat32."""
+    best, idx = -np.finfo(np.float32).max, 0
+    for i, v in enumerate(np.asarray(logits, dtype=np.float32)):
+        if v > best:
+            best, idx = v, i
+    return idx
+
+
+def sampler_sample(logits, temperature, top_k, top_p, r):
+    """Sampler.Sample (sampler.go:48-77, 94-203) in float32, the uniform draw r given. Ties at the nucleus cutoff keep
+    the lower index (the reference's sort.Slice is unstable: its order among equal probabilities is unspecified)."""
+    f32 = np.float32
+    logits = np.asarray(logits, dtype=f32)
+    if temperature == 0:
+        return sampler_argmax(logits)
+    scaled = logits / f32(temperature)
+    mx = -np.finfo(f32).max
+    for v in scaled:
+        if v > mx:
+            mx = v
+    probs = np.empty_like(scaled)
+    s = f32(0)
+    for i, v in enumerate(scaled):
+        probs[i] = f32(math.exp(float(f32(v - mx))))
+        s = f32(s + probs[i])
+    probs = probs / s
+    n = len(probs)
+    if 0 < top_k < n:
+        threshold = np.sort(probs)[::-1][top_k - 1]
+        s = f32(0)
+        for i in range(n):
+            if probs[i] < threshold:
+                probs[i] = 0
+            else:
+                s = f32(s + probs[i])
+        if s > 0:
+            probs = probs / s
+    if 0 < top_p < 1.0:
+        order = sorted(range(n), key=lambda i: (-float(probs[i]), i))
+        cum, cutoff = f32(0), n
+        for j, i in enumerate(order):
+            cum = f32(cum + probs[i])
+            if cum > f32(top_p):
+                cutoff = j + 1
+                break
+        keep = set(order[:cutoff])
+        s = f32(0)
+        for i in range(n):
+            if i not in keep:
+                probs[i] = 0
+            else:
+                s = f32(s + probs[i])
+        if s > 0:
+            probs = probs / s
+    cum = f32(0)
+    for i in range(n):
+        cum = f32(cum + probs[i])
+        if f32(r) < cum:
+            return i
+    return n - 1
+
+
+def splitmix_uniform(state):
+    """The uniform stream of sampled requests: SplitMix64, top 24 bits. Returns (r, new state)."""
+    mask = (1 << 64) - 1
+    state = (state + 0x9E3779B97F4A7C15) & mask
+    z = state
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & mask
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & mask
+    z ^= z >> 31
+    return float(np.float32(z >> 40) * np.float32(1.0 / 16777216.0)), state
+
+
+PENDING, PREFILL, DECODING, FINISHED = range(4)  # sequence.go:15-20
+
+
+class SchedSeq:
+    def __init__(self, prompt, max_tokens=0):
+        self.prompt, self.generated = list(prompt), []
+        self.prompt_pos = self.position = 0
+        self.state, self.max_tokens = PENDING, max_tokens
+        self.sampling = None   # (temperature, top_k, top_p, rng state)
+
+    def prefill_complete(self):  # sequence.go:205-207
+        return self.prompt_pos >= len(self.prompt)
+
+    def reached_max(self, global_max):  # sequence.go:196-202
+        limit = self.max_tokens if self.max_tokens > 0 else global_max
+        return limit > 0 and len(self.generated) >= limit
+
+
+class Scheduler:
+    """Scheduler.step (scheduler.go:166-483) over any model with prefill_with_paged_kv / decode_batched, sequences
+    taken in ascending id; prefill_chunk > 0 feeds prompts in pieces, one per step."""
+
+    def __init__(self, model, max_batch_size, max_tokens, eos_token, prefill_chunk=0):
+        self.model, self.max_batch_size, self.max_tokens = model, max_batch_size, max_tokens
+        self.eos, self.chunk = eos_token, prefill_chunk
+        self.seqs: Dict[int, SchedSeq] = {}
+
+    def add_sequence(self, seq_id, prompt, max_tokens=0):
+        self.model.pool.create_sequence(seq_id)
+        self.seqs[seq_id] = SchedSeq(prompt, max_tokens)
+
+    def remove_sequence(self, seq_id):
+        if seq_id in self.seqs:
+            del self.seqs[seq_id]
+            if self.model.pool.has_sequence(seq_id):
+                self.model.pool.delete_sequence(seq_id)
+
+    def _pick(self, q, logits):
+        if q.sampling is None or q.sampling[0] == 0:
+            return sampler_argmax(logits)
+        t, k, p, st = q.sampling
+        r, st = splitmix_uniform(st)
+        q.sampling = (t, k, p, st)
+        return sampler_sample(logits, t, k, p, r)
+
+    def step(self):
+        batch = [i for i in sorted(self.seqs) if self.seqs[i].state in (PENDING, PREFILL, DECODING)][:self.max_batch_size]
+        if not batch:
+            for i in [i for i, q in self.seqs.items() if q.state == FINISHED]:
+                self.remove_sequence(i)   # the reference only forgets it here; its KV blocks would leak
+            return 0
+        produced = 0
+        for i in batch:
+            q = self.seqs[i]
+            if q.state not in (PENDING, PREFILL) or not q.prompt or q.prefill_complete():
+                continue
+            left = len(q.prompt) - q.prompt_pos
+            n = min(left, self.chunk) if self.chunk > 0 else left
+            logits = self.model.prefill_with_paged_kv(q.prompt[q.prompt_pos:q.prompt_pos + n], i, q.prompt_pos)
+            q.prompt_pos += n
+            q.position = q.prompt_pos
+            if not q.prefill_complete():
+                q.state = PREFILL
+                continue
+            tok = self._pick(q, logits)
+            q.generated.append(tok)
+            produced += 1
+            q.state = FINISHED if tok == self.eos else DECODING
+        dec = [i for i in batch if self.seqs[i].state == DECODING or
+               (self.seqs[i].state == PENDING and self.seqs[i].prefill_complete())]
+        if dec:
+            toks, pos = [], []
+            for i in dec:
+                q = self.seqs[i]
+                toks.append(q.generated[-1] if q.generated else 1)
+                pos.append(q.position if q.generated else 0)
+            logits = self.model.decode_batched(toks, dec, pos)
+            for row, i in enumerate(dec):
+                q = self.seqs[i]
+                q.position += 1
+                if q.state == PENDING:
+                    q.state = DECODING
+                tok = self._pick(q, logits[row])
+                q.generated.append(tok)
+                produced += 1
+                if tok == self.eos or q.reached_max(self.max_tokens):
+                    q.state = FINISHED
+        return produced

@@ -310,6 +310,69 @@ def test_load_gguf_checkpoint(be, tmp_path, case):
         ModelRuntime.from_gguf(be, path, pool_blocks=16, max_seqs=4, max_batch=48)
 
 
+@pytest.mark.parametrize("chunk", [0, 16])
+def test_scheduler_loop_matches_oracle(be, chunk):
+    """Continuous batching (scheduler/scheduler.go:166-483, sequence.go): six requests with prompts of 0 to 45 tokens
+    join at different steps; at most four run per step; one stops on the EOS token, the others on their own or
+    the scheduler's length limit; finished sequences are removed and their blocks return to the pool. After every
+    step the C++ scheduler and its oracle restatement over the CPU model agree on every sequence's state, position
+    and generated tokens; at the end on block tables and pool statistics. chunk = 16 feeds prompts in pieces."""
+    from oracle import host_logic as hl
+    from vexel_amd.runtime import Scheduler
+    cfg = om.ModelConfig(num_layers=2, hidden=512, num_heads=8, num_kv_heads=2, head_dim=64, ffn=1024, vocab=1024)
+    omodel = om.random_model(cfg, 71, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=48)
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=48, max_seqs=8, max_blocks_per_seq=8, max_batch=48)
+    rng = np.random.default_rng(72)
+    prompts = {11: 45, 12: 0, 13: 7, 14: 33, 15: 16, 16: 1}
+    prompts = {i: rng.integers(0, cfg.vocab, n).tolist() for i, n in prompts.items()}
+    limits = {11: 9, 12: 0, 13: 5, 14: 0, 15: 12, 16: 3}
+    arrivals = {0: [11, 12, 13], 2: [14, 15], 5: [16]}
+    # the EOS token: what sequence 14 generates third in a dry run of the oracle (so that one request stops on it)
+    dry_model = om.random_model(cfg, 71, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=48)
+    dry = hl.Scheduler(dry_model, 4, 14, -1, chunk)
+    dry.add_sequence(14, prompts[14])
+    for _ in range(6):
+        dry.step()
+    eos = dry.seqs[14].generated[2]
+    want = hl.Scheduler(omodel, 4, 14, eos, chunk)
+    got = Scheduler(mr, 4, max_tokens=14, eos_token=eos, prefill_chunk=chunk)
+    finished_at = {}
+    for step in range(40):
+        for i in arrivals.get(step, []):
+            want.add_sequence(i, prompts[i], limits[i])
+            got.add_sequence(i, prompts[i], limits[i])
+        nw, ng = want.step(), got.step()
+        assert nw == ng, "tokens produced in step %d" % step
+        for i, q in want.seqs.items():
+            assert got.state(i) == q.state and got.position(i) == q.position, (step, i)
+            assert got.generated(i) == q.generated, (step, i)
+            if q.state == hl.FINISHED and i not in finished_at:
+                finished_at[i] = step
+        assert got.sequence_count() == len(want.seqs)
+        for i in [i for i, q in want.seqs.items() if q.state == hl.FINISHED and finished_at[i] < step]:
+            assert mr.block_table(i) == omodel.pool.seqs[i].block_tables[0]
+            want.remove_sequence(i)
+            got.remove_sequence(i)
+        assert mr.block_stats()[1] == omodel.pool.block_stats()[1]
+        if step > 6 and not want.seqs:
+            break
+    assert not want.seqs and got.sequence_count() == 0 and len(finished_at) == 6
+    assert mr.block_stats()[1] == omodel.pool.block_stats()[1] == 48 * cfg.num_layers
+    # a sampled request runs to its limit inside the vocabulary (its draws follow the library's own stream)
+    got.add_sequence(30, prompts[13], 6)
+    got.set_sampling(30, 0.8, 20, 0.95, 1234)
+    for _ in range(8):
+        got.step()
+        if got.state(30) == hl.FINISHED:
+            break
+    toks = got.generated(30)
+    assert got.state(30) == hl.FINISHED and 1 <= len(toks) <= 6 and all(0 <= t < cfg.vocab for t in toks)
+    got.step()                                   # nothing left to run: the finished request is dropped, its blocks freed
+    assert got.sequence_count() == 0 and mr.block_stats()[1] == 48 * cfg.num_layers
+    got.close()
+    mr.close()
+
+
 def test_pool_errors_and_lifecycle(be):
     """Host-forced failure paths: pool exhaustion, unknown sequence, truncate no-ops."""
     from vexel_amd.backend import VexelError

@@ -53,7 +53,8 @@ def build(verbose=True):
         print("built", SYNTH_LIB)
     # host runtime: plain C++ above the C ABI (links the HIP library, finds it next to itself)
     cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-I" + os.path.join(ROOT, "include"),
-           os.path.join(HERE, "host", "runtime.cpp"), os.path.join(HERE, "host", "gguf.cpp"), "-o", HOST_LIB, "-L" + HERE, "-lvexel_hip",
+           os.path.join(HERE, "host", "runtime.cpp"), os.path.join(HERE, "host", "gguf.cpp"),
+           os.path.join(HERE, "host", "scheduler.cpp"), "-o", HOST_LIB, "-L" + HERE, "-lvexel_hip",
            "-Wl,-rpath,$ORIGIN", "-pthread"]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:

@@ -77,6 +77,84 @@ def load_host():
     return _host
 
 
+class VhSchedConfig(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("max_batch_size", "max_tokens", "eos_token", "prefill_chunk")]
+
+
+class Scheduler:
+    """scheduler.Scheduler over a ModelRuntime: add_sequence / step / remove_sequence; the loop is the caller's."""
+
+    def __init__(self, mr, max_batch_size, max_tokens=0, eos_token=2, prefill_chunk=0):
+        self._h = load_host()
+        h = self._h
+        if not getattr(h, "_sched_bound", False):
+            h.vh_sched_create.argtypes = [C.c_void_p, C.POINTER(VhSchedConfig), C.POINTER(C.c_void_p)]
+            h.vh_sched_destroy.argtypes = [C.c_void_p]
+            h.vh_sched_destroy.restype = None
+            h.vh_sched_add_sequence.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int, C.c_int]
+            h.vh_sched_set_sampling.argtypes = [C.c_void_p, C.c_int64, C.c_float, C.c_int, C.c_float, C.c_uint64]
+            h.vh_sched_remove_sequence.argtypes = [C.c_void_p, C.c_int64]
+            h.vh_sched_sequence_count.argtypes = [C.c_void_p]
+            h.vh_sched_state.argtypes = [C.c_void_p, C.c_int64]
+            h.vh_sched_position.argtypes = [C.c_void_p, C.c_int64]
+            h.vh_sched_generated.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int]
+            h.vh_sched_step.argtypes = [C.c_void_p, C.POINTER(C.c_int)]
+            h.vh_argmax.argtypes = [C.c_void_p, C.c_int]
+            h.vh_sample.argtypes = [C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_float]
+            h._sched_bound = True
+        self.mr = mr
+        cfg = VhSchedConfig(max_batch_size, max_tokens, eos_token, prefill_chunk)
+        s = C.c_void_p()
+        self._s = None
+        self._ck(h.vh_sched_create(mr._m, C.byref(cfg), C.byref(s)))
+        self._s = s
+
+    def _ck(self, rc):
+        if rc != 0:
+            raise VexelError(rc, self._h.vh_last_error().decode())
+
+    def close(self):
+        if self._s:
+            self._h.vh_sched_destroy(self._s)
+            self._s = None
+
+    def add_sequence(self, seq_id, prompt, max_tokens=0):
+        p = np.ascontiguousarray(prompt, dtype=np.int32)
+        self._ck(self._h.vh_sched_add_sequence(self._s, seq_id, p.ctypes.data, p.size, max_tokens))
+
+    def set_sampling(self, seq_id, temperature, top_k, top_p, seed):
+        self._ck(self._h.vh_sched_set_sampling(self._s, seq_id, temperature, top_k, top_p, seed))
+
+    def remove_sequence(self, seq_id):
+        self._ck(self._h.vh_sched_remove_sequence(self._s, seq_id))
+
+    def sequence_count(self):
+        return self._h.vh_sched_sequence_count(self._s)
+
+    def state(self, seq_id):
+        return self._h.vh_sched_state(self._s, seq_id)
+
+    def position(self, seq_id):
+        return self._h.vh_sched_position(self._s, seq_id)
+
+    def generated(self, seq_id):
+        n = self._h.vh_sched_generated(self._s, seq_id, None, 0)
+        if n < 0:
+            return None
+        out = np.zeros(max(n, 1), dtype=np.int32)
+        self._h.vh_sched_generated(self._s, seq_id, out.ctypes.data, n)
+        return [int(x) for x in out[:n]]
+
+    def step(self):
+        n = C.c_int()
+        self._ck(self._h.vh_sched_step(self._s, C.byref(n)))
+        return n.value
+
+    def sample(self, logits, temperature, top_k, top_p, r):
+        a = np.ascontiguousarray(logits, dtype=np.float32)
+        return self._h.vh_sample(a.ctypes.data, a.size, temperature, top_k, top_p, r)
+
+
 class ModelRuntime:
     def __init__(self, be: HipBackend, num_layers, hidden, num_heads, num_kv_heads, head_dim, ffn, vocab,
                  eps=1e-5, rope_theta=10000.0, block_size=16, pool_blocks=256, max_seqs=64,
