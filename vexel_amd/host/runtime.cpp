@@ -115,6 +115,7 @@ struct vh_model {
     int32_t *d_tables = nullptr, *d_num_blocks = nullptr, *d_free = nullptr, *d_free_count = nullptr;
     int32_t *d_slots = nullptr, *d_positions = nullptr, *d_tokens = nullptr, *d_next = nullptr;
     int32_t *d_cu = nullptr, *d_token_pos = nullptr, *d_slot_map = nullptr, *d_kv_lens = nullptr;
+    int32_t *d_pos_in = nullptr;  // positions of a host-driven step, input of the packing kernel
     int32_t *d_status = nullptr, *d_step = nullptr, *d_log = nullptr;
     int log_cap = 0;  // steps the log can hold
 
@@ -370,6 +371,7 @@ int vh_model_create(vx_backend *be, const vh_config *cfg, vh_model **out) {
     rc |= dev_alloc(m, &m->d_token_pos, mb);
     rc |= dev_alloc(m, &m->d_slot_map, mb);
     rc |= dev_alloc(m, &m->d_kv_lens, mb);
+    rc |= dev_alloc(m, &m->d_pos_in, mb);
     rc |= dev_alloc(m, &m->d_status, 1);
     rc |= dev_alloc(m, &m->d_step, 1);
     rc |= dev_alloc(m, &m->x, mb * c.hidden);
@@ -401,7 +403,7 @@ void vh_model_destroy(vh_model *m) {
     if (m->graph) vx_graph_destroy(m->graph);
     for (void *p : m->kv) vx_free(m->be, p);
     void *bufs[] = {m->d_tables, m->d_num_blocks, m->d_free, m->d_free_count, m->d_slots, m->d_positions, m->d_tokens,
-                    m->d_next, m->d_cu, m->d_token_pos, m->d_slot_map, m->d_kv_lens, m->d_status, m->d_step, m->d_log,
+                    m->d_next, m->d_cu, m->d_token_pos, m->d_slot_map, m->d_kv_lens, m->d_pos_in, m->d_status, m->d_step, m->d_log,
                     m->x, m->norm, m->q, m->k, m->v, m->attn, m->gate, m->up, m->logits};
     for (void *p : bufs) vx_free(m->be, p);
     for (void *p : m->adopted) vx_free(m->be, p);
@@ -603,10 +605,21 @@ int vh_decode_batched(vh_model *m, const int32_t *tokens, const int64_t *seq_ids
     }
     vx_reset_pool(m->be);                                                            // decode.go:366-368
     VXC(vx_to_device(m->be, m->d_tokens, tokens, (size_t)batch * 4));                 // decode.go:389-395
-    VXC(vx_to_device(m->be, m->d_token_pos, positions, (size_t)batch * 4));
     VXC(vx_to_device(m->be, m->d_slots, slots.data(), (size_t)batch * 4));
-    VXC(vx_to_device(m->be, m->d_slot_map, slot_map.data(), (size_t)batch * 4));
-    VXC(vx_to_device(m->be, m->d_kv_lens, kv_lens.data(), (size_t)batch * 4));
+    bool at_end = true;  // every sequence decodes at its end: kv length = position + 1
+    for (int i = 0; i < batch; i++) at_end = at_end && kv_lens[i] == positions[i] + 1;
+    if (at_end) {
+        // The blocks are there already (host pool, mirrored above), so the packing kernel allocates nothing and
+        // only derives slots and lengths on the device, and leaves the attention's work list with them.
+        VXC(vx_to_device(m->be, m->d_pos_in, positions, (size_t)batch * 4));
+        VXC(vx_pack_batch(m->be, m->d_slots, m->d_pos_in, nullptr, batch, batch, m->d_tables, c.max_blocks_per_seq,
+                          m->d_num_blocks, m->d_free, m->d_free_count, c.block_size, m->d_cu, m->d_token_pos,
+                          m->d_slot_map, m->d_kv_lens, m->d_status));
+    } else {
+        VXC(vx_to_device(m->be, m->d_token_pos, positions, (size_t)batch * 4));
+        VXC(vx_to_device(m->be, m->d_slot_map, slot_map.data(), (size_t)batch * 4));
+        VXC(vx_to_device(m->be, m->d_kv_lens, kv_lens.data(), (size_t)batch * 4));
+    }
     VHC(forward_decode(m, batch, max_kv));
     if (logits_out) VXC(vx_to_host(m->be, logits_out, m->logits, (size_t)batch * c.vocab * 4));
     if (argmax_out) VXC(vx_to_host(m->be, argmax_out, m->d_next, (size_t)batch * 4));
