@@ -307,6 +307,49 @@ def counter_probe(be, mr, ctx, c, layers):
                       "attention_ms": ms}))
 
 
+def prefill_probe(be, rows=512, reps=10):
+    """Workload for MFMA counters (rocprofv3 --pmc SQ_INSTS_VALU_MFMA_MOPS_F16 ...): the four 7B-shaped Q4_0
+    projections with `rows` activation rows through the batched MFMA kernel, and one causal prefill attention of
+    `rows` tokens (32 heads x 128), `reps` launches each; prints flops and event-timed durations."""
+    synth = load_synth()
+    shapes = [("Q|K|V", 12288, 4096), ("Wo", 4096, 4096), ("gate|up", 22016, 4096), ("down", 4096, 11008)]
+    a = np.random.default_rng(0).standard_normal((rows, 11008)).astype(np.float32)
+    da = be.upload(a, permanent=True)
+    out = {"rows": rows, "gemm": [], "note": "the GEMM's MFMA work is twice 2*M*N*K: activations enter as hi + lo f16"}
+    for name, n, k in shapes:
+        rb = k // 32 * 18
+        w = be.alloc_permanent(n * rb)
+        if synth.vxs_gaussian_quant(1, w, n * (k // 32), 0.02, 91):
+            raise RuntimeError("synthetic weight generation failed")
+        o = be.alloc_permanent(rows * n * 4)
+        be.prepare_act(da, rows, k)
+        be.matmul_quant_prepared(1, w, o, None, rows, n, k)
+        be.sync()
+        be.timer_start()
+        for _ in range(reps):
+            be.matmul_quant_prepared(1, w, o, None, rows, n, k)
+        ms = be.timer_stop_ms() / reps
+        flops = 2.0 * rows * n * k
+        out["gemm"].append({"name": name, "n": n, "k": k, "ms": ms, "algorithmic_tflops": flops / ms / 1e9,
+                            "mfma_tflops": 2 * flops / ms / 1e9})
+        be.free(w)
+        be.free(o)
+    hq, d = CFG["num_heads"], CFG["head_dim"]
+    rng = np.random.default_rng(5)
+    bufs = [be.upload(rng.standard_normal((rows, hq * d)).astype(np.float32), permanent=True) for _ in range(3)]
+    do = be.alloc_permanent(rows * hq * d * 4)
+    scale = 1.0 / math.sqrt(d)
+    be.sdpa_prefill(bufs[0], bufs[1], bufs[2], do, rows, hq, hq, d, scale)
+    be.sync()
+    be.timer_start()
+    for _ in range(reps):
+        be.sdpa_prefill(bufs[0], bufs[1], bufs[2], do, rows, hq, hq, d, scale)
+    ms = be.timer_stop_ms() / reps
+    flops = 4.0 * hq * d * rows * (rows + 1) / 2
+    out["prefill_attention"] = {"tokens": rows, "ms": ms, "tflops": flops / ms / 1e9}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -322,6 +365,9 @@ def main():
                          "table of achieved GB/s against the 8 TB/s HBM peak, then exit")
     ap.add_argument("--counter-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: one 1 GiB plain copy and 8 attention launches, then exit")
+    ap.add_argument("--prefill-probe", action="store_true",
+                    help="for rocprofv3 --pmc runs of the MFMA kernels: 512-row GEMMs of the 7B shapes and one "
+                         "512-token prefill attention, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -330,6 +376,9 @@ def main():
     be = HipBackend(0)
     if args.kernel_report:
         kernel_report(be)
+        return
+    if args.prefill_probe:
+        prefill_probe(be)
         return
     ctx = ragged_contexts(n=args.seqs) if args.seqs != BATCH else ragged_contexts()
     nseq = len(ctx)
