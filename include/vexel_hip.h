@@ -236,7 +236,7 @@ int vx_argmax_rows(vx_backend *be, const float *logits, int rows, int n, int32_t
  * total_tokens = sum(q_lens) is given by the caller (T).
  * The call also leaves, inside the backend, a work list for vx_sdpa_paged_decode_ragged: one item per 512 tokens
  * of every sequence, equal items first, the partial last items from the longest down. An attention call that
- * passes this kv_lens array and batch walks the list (no empty workgroups inside its grid, the smallest last);
+ * passes this kv_lens array, seq_slots as its table_rows and the same batch walks the list (no empty workgroups inside its grid, the smallest last);
  * the list is dropped when the array is written through vx_to_device / vx_copy_buffer, freed, or the pool is
  * reset. A caller that rewrites kv_lens with kernels of its own must do so in another array. */
 int vx_pack_batch(vx_backend *be, const int32_t *seq_slots, const int32_t *positions, const int32_t *q_lens,

@@ -622,7 +622,7 @@ def test_paged_decode_single_batched_ragged(be, f16, shape):
 
 def test_attention_work_list_from_pack_batch(be):
     """vx_pack_batch leaves a work list for the ragged decode attention (full 512-token items first, partial last
-    items from the longest down). The attention call that passes the packed kv_lens array takes the list; a call
+    items from the longest down). The attention call that passes the packed kv_lens array and row indices takes the list; a call
     with a copy of the same lengths in another array walks the (split, sequence) grid. Both give the same bits,
     and match the oracle; writing the lengths through the library drops the list."""
     rng = np.random.default_rng(36)
@@ -652,7 +652,7 @@ def test_attention_work_list_from_pack_batch(be):
     want = np.stack([nx.sdpa_paged_decode(q[i], pool, tables[i, :nblk[i]], int(nblk[i]), bs, hq, hk, d, sc,
                                           int(lens[i]) - (int(nblk[i]) - 1) * bs) for i in range(B)])
     o_list, o_grid, o_after = be.alloc(q.nbytes), be.alloc(q.nbytes), be.alloc(q.nbytes)
-    be.sdpa_paged_decode_ragged(dq, dpool, True, d_t, kl, o_list, B, mb, bs, hq, hk, d, sc, mb * bs)
+    be.sdpa_paged_decode_ragged(dq, dpool, True, d_t, kl, o_list, B, mb, bs, hq, hk, d, sc, mb * bs, table_rows=d_s)
     kl2 = be.alloc(B * 4)
     be.copy_buffer(kl, 0, kl2, 0, B * 4)
     be.sdpa_paged_decode_ragged(dq, dpool, True, d_t, kl2, o_grid, B, mb, bs, hq, hk, d, sc, mb * bs)
@@ -662,7 +662,7 @@ def test_attention_work_list_from_pack_batch(be):
     # shorter lengths written into the packed array: the stale list must not be used
     short = np.maximum(lens // 2, 1).astype(np.int32)
     be.to_device(kl, short)
-    be.sdpa_paged_decode_ragged(dq, dpool, True, d_t, kl, o_after, B, mb, bs, hq, hk, d, sc, mb * bs)
+    be.sdpa_paged_decode_ragged(dq, dpool, True, d_t, kl, o_after, B, mb, bs, hq, hk, d, sc, mb * bs, table_rows=d_s)
     want2 = np.stack([nx.sdpa_paged_decode(q[i], pool, tables[i, :nblk[i]], (int(short[i]) + bs - 1) // bs, bs, hq, hk, d, sc,
                                            int(short[i]) - ((int(short[i]) + bs - 1) // bs - 1) * bs) for i in range(B)])
     _close(be.download(o_after, q.shape, np.float32), want2, 1e-5, 3e-6, "attention after the lengths were rewritten")

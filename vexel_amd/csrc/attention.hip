@@ -203,18 +203,22 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     constexpr int NL = HOT_BS / TPI; // load instructions per block and per K or V
     typedef _Float16 half8 __attribute__((ext_vector_type(8)));
     const int kvh = blockIdx.x;
-    int split = blockIdx.y, seq = blockIdx.z;
+    int split = blockIdx.y, seq = blockIdx.z, kv_len, row;
     if (items) {  // work list: grid.y runs over the items, the workgroups past the list's end are the grid's last
         if ((int)blockIdx.y >= items[0]) return;
-        const int code = items[1 + blockIdx.y];
-        seq = code >> 16;
-        split = code & 0xFFFF;
+        const int4 rec = ((const int4 *)(items + 4))[blockIdx.y];  // (sequence, split, kv length, table row)
+        seq = rec.x;
+        split = rec.y;
+        kv_len = rec.z;
+        row = rec.w;
+    } else {
+        kv_len = kv_lens[seq];
+        row = bt_rows ? bt_rows[seq] : seq;
     }
-    const int kv_len = kv_lens[seq];
     const int t_begin = split * TPW;
     if (t_begin >= kv_len) return;
     const int t_end = min(kv_len, t_begin + TPW);
-    const int32_t *bt = bt_matrix + (size_t)(bt_rows ? bt_rows[seq] : seq) * max_blocks + t_begin / HOT_BS;
+    const int32_t *bt = bt_matrix + (size_t)row * max_blocks + t_begin / HOT_BS;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -530,8 +534,9 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
     if (rc) return rc;
     // With a work list from vx_pack_batch for these lengths the grid's second dimension runs over its items
     // (at most max_splits per sequence, as max_kv_len bounds every length); otherwise over (split, sequence).
-    const bool listed = be->items.valid && be->items.kv_lens == kv_lens && be->items.batch == batch &&
-                        (size_t)batch * max_splits + 1 <= be->items.bytes / sizeof(int32_t) &&
+    const bool listed = be->items.valid && be->items.kv_lens == kv_lens && be->items.table_rows == bt_rows &&
+                        be->items.batch == batch &&
+                        ((size_t)batch * max_splits + 1) * 4 <= be->items.bytes / sizeof(int32_t) &&
                         (size_t)batch * max_splits <= 65535;
     dim3 grid(num_kv_heads, listed ? batch * max_splits : max_splits, listed ? 1 : batch);
     paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,

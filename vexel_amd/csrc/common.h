@@ -77,13 +77,15 @@ struct vx_backend {
     } split;
     size_t attn_ws_bytes = 0;
     // Work list of the ragged decode attention, written on the device by vx_pack_batch next to kv_lens:
-    // buf[0] = number of items, buf[1 + i] = (batch index << 16) | split, full splits first, then the
-    // sequences' partial last splits from the longest down. Valid for attention calls that pass the same
-    // kv_lens pointer and batch, until the library is asked to write into that array by other means.
+    // buf[0] = number of items, then from buf[4] one record of four ints per item (batch index, split, kv
+    // length, block-table row), full splits first, then the sequences' partial last splits from the longest
+    // down. Valid for attention calls that pass the same kv_lens and table-row pointers and batch, until the
+    // library is asked to write into the kv_lens array by other means.
     struct {
         int32_t *buf = nullptr;
         size_t bytes = 0;
         const int32_t *kv_lens = nullptr;
+        const int32_t *table_rows = nullptr;
         int batch = 0;
         bool valid = false;
     } items;

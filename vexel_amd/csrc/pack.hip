@@ -94,8 +94,9 @@ __global__ void __launch_bounds__(PK_THREADS) pack_batch_kernel(
         __syncthreads();
         const int n_items = total_full + partials;
         if (n_items <= items_cap) {
-            for (int s2 = 0; s2 < full; s2++) items[1 + off + s2] = (tid << 16) | s2;
-            if (rest > 0) items[1 + total_full + before] = (tid << 16) | full;
+            int4 *rec = (int4 *)(items + 4);  // one 16-byte record per item: everything a workgroup needs to start
+            for (int s2 = 0; s2 < full; s2++) rec[off + s2] = make_int4(tid, s2, len, slot);
+            if (rest > 0) rec[total_full + before] = make_int4(tid, full, len, slot);
         }
         if (tid == 0) items[0] = n_items <= items_cap ? n_items : -1;  // -1: the list did not fit, not to be used
     }
@@ -151,7 +152,7 @@ extern "C" int vx_pack_batch(vx_backend *be, const int32_t *seq_slots, const int
     int32_t *items = nullptr;
     be->items.valid = false;
     if (batch <= 32767 && per_seq <= 65535 &&
-        ensure_ws(be, (void **)&be->items.buf, &be->items.bytes, (cap + 1) * sizeof(int32_t), "attention work list") == VX_OK)
+        ensure_ws(be, (void **)&be->items.buf, &be->items.bytes, (cap + 1) * 4 * sizeof(int32_t), "attention work list") == VX_OK)
         items = be->items.buf;
     pack_batch_kernel<<<1, PK_THREADS, 0, be->stream>>>(seq_slots, positions, q_lens, batch, total_tokens,
                                                         block_tables, max_blocks, num_blocks, free_list, free_count,
@@ -160,6 +161,7 @@ extern "C" int vx_pack_batch(vx_backend *be, const int32_t *seq_slots, const int
     VX_CHECK_LAUNCH();
     if (items) {
         be->items.kv_lens = kv_lens;
+        be->items.table_rows = seq_slots;
         be->items.batch = batch;
         be->items.valid = true;
     }
