@@ -222,6 +222,16 @@ int vx_sdpa_paged_tree(vx_backend *be, const float *q, const void *kv_pool, int 
                        int block_size, int num_q_heads, int num_kv_heads, int head_dim, float scale,
                        int query_len);
 
+/* Moves token rows (K and V of every KV head) inside one layer's paged pool: slot = physical block *
+ * block_size + offset in the block. Chain c is the moves chain_offsets[c] .. chain_offsets[c+1]-1 (device
+ * int32 arrays), applied in order, so a later move of a chain may read what an earlier one wrote; different
+ * chains must not touch the same slots. No counterpart in the reference, whose verification keeps one path
+ * that is contiguous already (scheduler/medusa_scheduler.go:852-861 only truncates); after a whole tree has
+ * been verified the accepted path's rows have to move up before the truncation. */
+int vx_paged_kv_move(vx_backend *be, void *kv_pool, int pool_is_f16, const int32_t *chain_offsets,
+                     const int32_t *src_slots, const int32_t *dst_slots, int num_chains, int num_kv_heads,
+                     int head_dim, int block_size);
+
 /* Row-wise argmax on the device: out_idx[r] = ArgmaxOps.Argmax(logits + r*n, n). No wait. */
 int vx_argmax_rows(vx_backend *be, const float *logits, int rows, int n, int32_t *out_idx);
 

@@ -82,6 +82,25 @@ int vh_pool_device_matches_host(vh_model *m);
  * logits_out: host [batch,vocab] or NULL; argmax_out: host [batch] or NULL. */
 int vh_decode_batched(vh_model *m, const int32_t *tokens, const int64_t *seq_ids, const int32_t *positions,
                       int batch, float *logits_out, int32_t *argmax_out);
+/* Speculative verification of a whole candidate tree for each of n_seqs sequences in one forward pass, greedy
+ * acceptance and rollback. The reference's runTreeMedusaDecodeStep (scheduler/medusa_scheduler.go:733-861)
+ * handles one sequence and verifies only the most confident path with VerifySpeculativeWithPagedKV
+ * (runtime/decode.go:1446-1569); here every path is verified at once under the ancestor mask of
+ * medusa/tree.go:186-202, and each root-to-node path sees exactly what that linear verification shows it.
+ *   Sequence i: input_tokens[i] goes to position start_pos[i], which must be the sequence's KV length; its
+ *   n_nodes[i] candidates follow in CandidateTree.Linearize order (tree.go:144-178), tokens and parent indices
+ *   (-1 = child of the input token) concatenated over the sequences in node_tokens / parent_idx.
+ *   Acceptance: from the argmax of the input token's logits, descend into the child whose token equals the
+ *   current argmax (first such child), continue with that node's argmax; the argmax nobody matches is the
+ *   final token. accepted_nodes receives the accepted node indices (within the sequence's tree, path order)
+ *   at the sequence's offset in the concatenated node arrays; num_accepted[i] and final_tokens[i] per sequence.
+ *   Rollback (medusa_scheduler.go:852-861): the accepted nodes' K/V rows move to the positions after the input
+ *   token and the sequence is truncated to start_pos + 1 + accepted (gpu_block_pool.go:162-190).
+ * logits_out: host [n_seqs + sum n_nodes, vocab] (per sequence: input token row, then node rows) or NULL. */
+int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_t *input_tokens,
+                   const int32_t *start_pos, const int32_t *n_nodes, const int32_t *node_tokens,
+                   const int32_t *parent_idx, int32_t *num_accepted, int32_t *accepted_nodes, int32_t *final_tokens,
+                   float *logits_out);
 /* ModelRuntime.PrefillWithPagedKV (runtime/decode.go:961-1096) when all_logits == 0: logits of the
  * last token -> logits_out[vocab]. VerifySpeculativeWithPagedKV (decode.go:1446-1569) when
  * all_logits != 0: logits of every position -> logits_out[n,vocab]. */

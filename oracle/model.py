@@ -6,6 +6,9 @@
   OracleModel.decode_with_paged_kv   inference/runtime/decode.go:339-461
   OracleModel.decode_batched         inference/runtime/decode.go:612-654 (sequential loop)
   OracleModel.prefill_with_paged_kv  inference/runtime/decode.go:961-1096
+  OracleModel.verify_tree/tree_step  whole-tree form of scheduler/medusa_scheduler.go:733-861 (the reference
+                                     verifies one path; pinned by equality with verify_with_paged_kv on every
+                                     root-to-node path)
 The KV pool holds real data here (numpy uint16 = f16 bits, or float32), addressed as
 inference/runtime/gpu_block_pool.go:15-19,107-108.
 """
@@ -160,6 +163,93 @@ class OracleModel:
         for i in range(c.num_layers):
             x = self.execute_with_paged_kv(x, seq_id, i, start_pos)
         return self._head(x, n)
+
+
+    # ---------------------------------------------------------------- tree verification
+    def _execute_tree_layer(self, x, seq_id, layer_idx, start_pos, positions, mask):
+        """block.go:763-1081 for the rows [input token, candidate nodes]: row r is stored at pool position
+        start_pos + r, rotated at positions[r] (start_pos + its depth in the tree) and attends to every earlier
+        pool position and to the rows the mask names (tree.go:186-202)."""
+        c = self.cfg
+        lw = self.layers[layer_idx]
+        rows = x.shape[0]
+        norm = nx.rmsnorm(x, lw.attn_norm, rows, c.hidden, c.eps)
+        q = _mm(norm, lw.wq, rows)
+        k = _mm(norm, lw.wk, rows)
+        v = _mm(norm, lw.wv, rows)
+        q, k = nx.rope_positions(q, k, c.head_dim, c.num_heads, c.num_kv_heads, positions, 0, c.rope_theta, False)
+        scale = np.float32(1.0 / math.sqrt(float(c.head_dim)))
+        slots = self.pool.store_kv_slots(layer_idx, seq_id, start_pos, rows)
+        bi = [s[0] for s in slots]
+        bo = [s[1] for s in slots]
+        nx.reshape_paged_kv(k, self.kv[layer_idx], bi, bo, c.num_kv_heads, c.head_dim, c.block_size, False)
+        nx.reshape_paged_kv(v, self.kv[layer_idx], bi, bo, c.num_kv_heads, c.head_dim, c.block_size, True)
+        bt = self.pool.seqs[seq_id].block_tables[layer_idx]
+        attn = nx.sdpa_paged_multiquery(q, self.kv[layer_idx], bt, None, c.block_size, c.num_heads, c.num_kv_heads,
+                                        c.head_dim, scale, tree_mask=mask, tree_base=start_pos).reshape(rows, -1)
+        o = _mm(attn, lw.wo, rows)
+        x = nx.add(x, o)
+        norm = nx.rmsnorm(x, lw.ffn_norm, rows, c.hidden, c.eps)
+        act = nx.silu_mul(_mm(norm, lw.w1, rows), _mm(norm, lw.w3, rows))
+        return nx.add(x, _mm(act, lw.w2, rows))
+
+    def verify_tree(self, input_token, node_tokens, parent_idx, seq_id, start_pos):
+        """Logits [1 + nodes, vocab] of one pass over the input token and a candidate tree given as
+        CandidateTree.Linearize returns it (tree.go:144-178: parent_idx -1 = child of the input token). Every
+        root-to-node path sees what VerifySpeculativeWithPagedKV (decode.go:1446-1569) would show it on
+        [input token, path tokens]: same positions, same visible keys. The rows' K/V stay in the pool at
+        start_pos .. start_pos + nodes."""
+        from .host_logic import build_tree_attention_mask, tree_depths
+        c = self.cfg
+        self._ensure_seq(seq_id)
+        n = len(node_tokens)
+        rows = n + 1
+        # row 0 is the input token: every node descends from it
+        parents = [-1] + [p + 1 for p in parent_idx]
+        mask = np.array(build_tree_attention_mask(rows, parents), dtype=np.uint8).reshape(rows, rows)
+        positions = [start_pos + d for d in tree_depths(parents)]
+        x = nx.embedding([input_token] + list(node_tokens), self.embedding, c.vocab, c.hidden)
+        for i in range(c.num_layers):
+            x = self._execute_tree_layer(x, seq_id, i, start_pos, positions, mask)
+        return self._head(x, rows)
+
+    def _move_kv_row(self, layer, seq_id, src_pos, dst_pos):
+        c = self.cfg
+        bt = self.pool.seqs[seq_id].block_tables[layer]
+        row = c.num_kv_heads * c.head_dim
+        blk = 2 * c.block_size * row                                       # gpu_block_pool.go:107-108
+        for half in (0, 1):                                                # K rows, then V rows of the block
+            s = bt[src_pos // c.block_size] * blk + half * c.block_size * row + (src_pos % c.block_size) * row
+            d = bt[dst_pos // c.block_size] * blk + half * c.block_size * row + (dst_pos % c.block_size) * row
+            self.kv[layer][d:d + row] = self.kv[layer][s:s + row].copy()
+
+    def tree_step(self, input_token, node_tokens, parent_idx, seq_id, start_pos):
+        """verify_tree, greedy acceptance over the whole tree, then the rollback of
+        medusa_scheduler.go:852-861: the accepted nodes' K/V move up to the positions right after the input
+        token (a path is not contiguous in the pool) and the sequence is truncated to
+        start_pos + 1 + accepted. -> (accepted node indices, final token, logits)."""
+        logits = self.verify_tree(input_token, node_tokens, parent_idx, seq_id, start_pos)
+        return self._accept_and_roll_back(logits, node_tokens, parent_idx, seq_id, start_pos)
+
+    def tree_step_batched(self, input_tokens, trees, seq_ids, start_positions):
+        """tree_step for several sequences whose trees are verified in the same pass: every sequence's rows
+        take their blocks first (in the order given), then every sequence is rolled back (same order).
+        -> [(accepted node indices, final token, logits)] per sequence."""
+        logits = [self.verify_tree(t, tr[0], tr[1], sid, sp)
+                  for t, tr, sid, sp in zip(input_tokens, trees, seq_ids, start_positions)]
+        return [self._accept_and_roll_back(lg, tr[0], tr[1], sid, sp)
+                for lg, tr, sid, sp in zip(logits, trees, seq_ids, start_positions)]
+
+    def _accept_and_roll_back(self, logits, node_tokens, parent_idx, seq_id, start_pos):
+        from .host_logic import greedy_tree_accept, argmax_list, cache_len_after_verify
+        am = [argmax_list(row) for row in logits]
+        accepted, final = greedy_tree_accept(list(node_tokens), list(parent_idx), am[0], am[1:])
+        for layer in range(self.cfg.num_layers):
+            for k, node in enumerate(accepted):                            # ascending: a source is never overwritten
+                if node != k:
+                    self._move_kv_row(layer, seq_id, start_pos + 1 + node, start_pos + 1 + k)
+        self.pool.truncate_sequence(seq_id, cache_len_after_verify(start_pos, len(accepted)))
+        return accepted, final, logits
 
 
 def random_model(cfg: ModelConfig, seed, fmt, head_fmt, emb_fmt=None, max_blocks=64, kv_fp16=True,

@@ -696,6 +696,36 @@ def test_paged_multiquery_and_tree(be):
         be.reset_pool()
 
 
+def test_paged_kv_move_chains(be):
+    """Rows move inside the pool in chain order: a later move of a chain reads what an earlier one wrote."""
+    rng = np.random.default_rng(36)
+    bs, hk, d, nblocks = 16, 2, 64, 12
+    for f16 in (False, True):
+        pool = _make_pool(rng, f16, nblocks, bs, hk, d)
+        dpool = be.upload(pool)
+        # chain 0: the accepted path of a tree (rows 3, 8, 9 move up to 1, 2, 3: row 3 is read, then overwritten);
+        # chain 1: a move across blocks; chain 2: a swap-like pair that depends on the order
+        base0, base1 = 5 * bs + 2, 7 * bs + 14
+        chains = [[(base0 + 3, base0 + 1), (base0 + 8, base0 + 2), (base0 + 9, base0 + 3)],
+                  [(base1 + 5, base1 + 1)],
+                  [(20, 21), (21, 22)]]
+        off = np.cumsum([0] + [len(c) for c in chains]).astype(np.int32)
+        src = np.array([m[0] for c in chains for m in c], dtype=np.int32)
+        dst = np.array([m[1] for c in chains for m in c], dtype=np.int32)
+        be.paged_kv_move(dpool, f16, be.upload(off), be.upload(src), be.upload(dst), len(chains), hk, d, bs)
+        want = pool.copy()
+        row = hk * d
+        for c in chains:
+            for sl, dl in c:
+                for half in (0, 1):
+                    so = (sl // bs) * 2 * bs * row + half * bs * row + (sl % bs) * row
+                    do = (dl // bs) * 2 * bs * row + half * bs * row + (dl % bs) * row
+                    want[do:do + row] = want[so:so + row].copy()
+        got = be.download(dpool, pool.shape, pool.dtype)
+        assert np.array_equal(got.view(np.uint16 if f16 else np.uint32), want.view(np.uint16 if f16 else np.uint32))
+        be.reset_pool()
+
+
 def test_rope_store_paged(be):
     rng = np.random.default_rng(35)
     rows, hq, hk, d, bs, nblocks = 9, 8, 2, 64, 16, 30

@@ -218,6 +218,59 @@ def test_chunked_prefill_and_verify(be):
     mr.close()
 
 
+def test_c5_tree_verification_batched(be):
+    """BASELINE config 5 at oracle size: Q6_K weights, several sequences at ragged contexts, a 15-node candidate
+    tree (4 heads x top-2) per sequence verified in one pass under tree masks over the paged f16 pool, greedy
+    acceptance, rollback in the block tables; two rounds, the second on top of the first one's rollback."""
+    import copy
+    from oracle import host_logic as hl
+    cfg = om.ModelConfig(num_layers=2, hidden=1024, num_heads=8, num_kv_heads=8, head_dim=128, ffn=2816, vocab=4096)
+    ctx = [291, 256, 517, 333]     # 256: the input token opens a new block
+    omodel, mr, rng = _ragged_setup(be, cfg, nx.FMT_Q6_K, nx.FMT_Q6_K, ctx, 41, pool_blocks=160)
+    ids = [100 + i for i in range(4)]
+    inputs = rng.integers(0, cfg.vocab, 4).tolist()
+    start = list(ctx)
+    moved = 0
+    for rnd in range(2):
+        trees = []
+        for i, sid in enumerate(ids):
+            # sequences 0 and 2 get their own greedy continuation planted down one branch (3 and 1 levels deep)
+            plant = []
+            if i in (0, 2):
+                probe = copy.deepcopy(omodel)
+                tok = inputs[i]
+                for d in range(3 if i == 0 else 1):
+                    tok = nx.argmax(probe.decode_with_paged_kv(tok, sid, start[i] + d))
+                    plant.append(tok)
+            toks = [rng.choice(cfg.vocab, 2, replace=False).tolist() for _ in range(4)]
+            for h, t in enumerate(plant):
+                toks[h][(h + 1) % 2] = t
+                if toks[h][0] == toks[h][1]:
+                    toks[h][h % 2] = (t + 1) % cfg.vocab
+            tree = hl.build_candidate_tree_from_topk(toks, [[2.0, 1.0]] * 4, 15)
+            trees.append(tree.linearize())
+        want = omodel.tree_step_batched(inputs, trees, ids, start)
+        acc, fin, logits = mr.verify_tree(ids, inputs, start, trees)
+        for i, sid in enumerate(ids):
+            assert_logits_close(logits[i], want[i][2], "C5 round %d seq %d" % (rnd, i))
+            assert acc[i] == want[i][0] and fin[i] == want[i][1]
+            assert mr.seq_len(sid) == omodel.pool.seqs[sid].seq_len == start[i] + 1 + len(acc[i])
+            assert mr.block_table(sid) == omodel.pool.seqs[sid].block_tables[0]
+            moved += sum(1 for k, node in enumerate(acc[i]) if node != k)
+        assert len(acc[0]) >= 3 and len(acc[2]) >= 1
+        assert mr.block_stats()[1] == omodel.pool.block_stats()[1]
+        inputs = list(fin)
+        start = [start[i] + 1 + len(acc[i]) for i in range(4)]
+    assert moved > 0   # the rollback had rows to move
+    # the compacted K/V rows serve an ordinary decode step
+    wl = omodel.decode_batched(inputs, ids, start)
+    gl, am = mr.decode_with_paged_kv_batched(inputs, ids, start)
+    assert_logits_close(gl, wl, "C5 decode after rollback")
+    assert [nx.argmax(wl[i]) for i in range(4)] == [int(a) for a in am]
+    assert mr.device_matches_host()
+    mr.close()
+
+
 GGUF_TYPE = {nx.FMT_Q4_0: 2, nx.FMT_Q8_0: 8, nx.FMT_Q4_K: 12, nx.FMT_Q6_K: 14}
 
 

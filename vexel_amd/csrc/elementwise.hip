@@ -392,6 +392,21 @@ __global__ void reshape_paged_kv_kernel(const float *src, void *dst, const int32
         ((float *)dst)[di] = src[gid];
 }
 
+// Moves token rows inside a paged pool. Chain c holds the moves chain_offsets[c] .. chain_offsets[c+1]-1, applied
+// in that order; a thread owns the same words of every row, so a move may read a row an earlier move of its
+// chain wrote. grid = (chains, 2: K rows, V rows).
+__global__ void move_paged_kv_kernel(uint32_t *pool, const int32_t *chain_offsets, const int32_t *src_slots,
+                                     const int32_t *dst_slots, int row_words, int block_size) {
+    const int c = blockIdx.x, half = blockIdx.y;
+    const size_t part = (size_t)block_size * row_words;
+    for (int i = chain_offsets[c]; i < chain_offsets[c + 1]; i++) {
+        const int s = src_slots[i], d = dst_slots[i];
+        const uint32_t *src = pool + (size_t)(s / block_size) * 2 * part + half * part + (size_t)(s % block_size) * row_words;
+        uint32_t *dst = pool + (size_t)(d / block_size) * 2 * part + half * part + (size_t)(d % block_size) * row_words;
+        for (int w = threadIdx.x; w < row_words; w += blockDim.x) dst[w] = src[w];
+    }
+}
+
 inline int grid1d(int64_t n, int threads) { return (int)((n + threads - 1) / threads); }
 
 }  // namespace
@@ -610,6 +625,22 @@ int vx_reshape_paged_kv_f16(vx_backend *be, const float *src, void *dst_base, co
                             int block_size, int is_value) {
     return reshape_paged(be, src, dst_base, page_table, block_offsets, num_tokens, num_kv_heads, head_dim, block_size,
                          is_value, true);
+}
+
+int vx_paged_kv_move(vx_backend *be, void *kv_pool, int pool_is_f16, const int32_t *chain_offsets,
+                     const int32_t *src_slots, const int32_t *dst_slots, int num_chains, int num_kv_heads, int head_dim,
+                     int block_size) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(kv_pool && chain_offsets && src_slots && dst_slots, "vx_paged_kv_move: null pointer");
+    VX_REQUIRE(num_chains >= 0 && num_kv_heads > 0 && head_dim > 0 && block_size > 0, "vx_paged_kv_move: bad shape");
+    const int64_t row_bytes = (int64_t)num_kv_heads * head_dim * (pool_is_f16 ? 2 : 4);
+    VX_REQUIRE(row_bytes % 4 == 0, "vx_paged_kv_move: a token row must be a whole number of 32-bit words");
+    if (num_chains == 0) return VX_OK;
+    move_paged_kv_kernel<<<dim3(num_chains, 2), kThreads, 0, be->stream>>>((uint32_t *)kv_pool, chain_offsets, src_slots,
+                                                                        dst_slots, (int)(row_bytes / 4), block_size);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
 }
 
 }  // extern "C"

@@ -713,6 +713,164 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
     return VH_OK;
 }
 
+// ------------------------------------------------------------------ tree verification of a batch of sequences
+int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_t *input_tokens, const int32_t *start_pos,
+                   const int32_t *n_nodes, const int32_t *node_tokens, const int32_t *parent_idx, int32_t *num_accepted,
+                   int32_t *accepted_nodes, int32_t *final_tokens, float *logits_out) {
+    if (!m || n_seqs < 0 || !seq_ids || !input_tokens || !start_pos || !n_nodes || !num_accepted || !final_tokens)
+        return fail("bad arguments");
+    if (n_seqs == 0) return VH_OK;
+    VHC(check_ready(m));
+    const vh_config &c = m->cfg;
+    struct SeqRows { int row0, rows, node0, start, slot; };
+    std::vector<SeqRows> sr(n_seqs);
+    int total = 0, nodes_total = 0;
+    for (int i = 0; i < n_seqs; i++) {
+        if (n_nodes[i] < 0 || start_pos[i] < 0) return fail("sequence %d: bad counts", i);
+        sr[i] = {total, 1 + n_nodes[i], nodes_total, start_pos[i], -1};
+        total += 1 + n_nodes[i];
+        nodes_total += n_nodes[i];
+    }
+    if (nodes_total > 0 && (!node_tokens || !parent_idx || !accepted_nodes)) return fail("null node arrays");
+    for (int i = 0; i < n_seqs; i++)
+        for (int j = i + 1; j < n_seqs; j++)
+            if (seq_ids[i] == seq_ids[j]) return fail("sequence %lld appears twice", (long long)seq_ids[i]);
+    // rows: [input token, nodes] per sequence; row r of a sequence lives at pool position start + r and is rotated
+    // at start + its depth; it sees the rows of its ancestors (tree.go:186-202) and everything before start
+    std::vector<int32_t> tok(total), pos(total), slot_map(total);
+    std::vector<uint8_t> mask;
+    std::vector<size_t> mask_off(n_seqs);
+    {
+        std::lock_guard<std::mutex> g(m->pool.mu);
+        for (int i = 0; i < n_seqs; i++) {
+            const SeqRows &q = sr[i];
+            if (input_tokens[i] < 0 || input_tokens[i] >= c.vocab) return fail("token %d out of range", input_tokens[i]);
+            if (!find_seq(m, seq_ids[i])) VHC(create_seq_locked(m, seq_ids[i]));
+            SeqState *s = find_seq(m, seq_ids[i]);
+            if (s->seq_len != q.start)
+                return fail("sequence %lld holds %d tokens, verification starts at %d", (long long)seq_ids[i], s->seq_len, q.start);
+            VHC(m->pool.ensure_blocks(*s, q.start + q.rows));                               // gpu_block_pool.go:234-245
+            if ((int)s->table.size() > c.max_blocks_per_seq)
+                return fail("sequence %lld needs %zu blocks, the table holds %d", (long long)seq_ids[i], s->table.size(),
+                            c.max_blocks_per_seq);
+            mask_off[i] = mask.size();
+            mask.resize(mask.size() + (size_t)q.rows * q.rows, 0);
+            uint8_t *mk = mask.data() + mask_off[i];
+            std::vector<int> depth(q.rows, 0);
+            for (int r = 0; r < q.rows; r++) {
+                int parent = -1;  // row index of the parent; the input token has none
+                if (r > 0) {
+                    const int node = r - 1, p = parent_idx[q.node0 + node];
+                    if (p < -1 || p >= node) return fail("sequence %d: parent of node %d is %d", i, node, p);
+                    const int t = node_tokens[q.node0 + node];
+                    if (t < 0 || t >= c.vocab) return fail("token %d out of range", t);
+                    tok[q.row0 + r] = t;
+                    parent = p + 1;
+                    depth[r] = depth[parent] + 1;
+                    memcpy(mk + (size_t)r * q.rows, mk + (size_t)parent * q.rows, q.rows);  // the parent's ancestors
+                } else {
+                    tok[q.row0] = input_tokens[i];
+                }
+                mk[(size_t)r * q.rows + r] = 1;
+                const int p = q.start + r;
+                pos[q.row0 + r] = q.start + depth[r];
+                slot_map[q.row0 + r] = s->table[p / c.block_size] * c.block_size + p % c.block_size;  // :250-252
+            }
+            s->seq_len = q.start + q.rows;
+            sr[i].slot = s->slot;
+        }
+        VHC(sync_pool_to_device(m));
+    }
+    vx_backend *be = m->be;
+    vx_reset_pool(be);
+    const int n = total;
+    const size_t qd = (size_t)c.num_heads * c.head_dim, kvd = (size_t)c.num_kv_heads * c.head_dim;
+    auto fa = [&](size_t count) { return (float *)vx_alloc(be, count * 4); };
+    auto ia = [&](size_t count) { return (int32_t *)vx_alloc(be, count * 4); };
+    int32_t *d_tok = ia(n), *d_pos = ia(n), *d_slot = ia(n), *d_am = ia(n);
+    uint8_t *d_mask = (uint8_t *)vx_alloc(be, mask.size());
+    float *x = fa((size_t)n * c.hidden), *norm = fa((size_t)n * c.hidden), *q = fa(n * qd), *k = fa(n * kvd);
+    float *v = fa(n * kvd), *attn = fa(n * qd), *gate = fa((size_t)n * c.ffn), *up = fa((size_t)n * c.ffn);
+    float *logits = fa((size_t)n * c.vocab);
+    if (!d_tok || !d_pos || !d_slot || !d_am || !d_mask || !x || !norm || !q || !k || !v || !attn || !gate || !up || !logits)
+        return fail("verification buffers: %s", vx_last_error());
+    VXC(vx_to_device(be, d_tok, tok.data(), (size_t)n * 4));
+    VXC(vx_to_device(be, d_pos, pos.data(), (size_t)n * 4));
+    VXC(vx_to_device(be, d_slot, slot_map.data(), (size_t)n * 4));
+    VXC(vx_to_device(be, d_mask, mask.data(), mask.size()));
+    VXC(vx_embedding(be, d_tok, n, m->embedding, x, c.vocab, c.hidden));
+    const float scale = (float)(1.0 / sqrt((double)c.head_dim));
+    for (int l = 0; l < c.num_layers; l++) {
+        const vh_layer_weights &w = m->layers[l];
+        bool prep;
+        const vh_qweight *qkv[3] = {&w.wq, &w.wk, &w.wv};
+        VHC(norm_for(m, x, w.attn_norm, norm, n, qkv, 3, &prep));
+        VHC(mm(m, prep, norm, w.wq, q, nullptr, n));
+        VHC(mm(m, prep, norm, w.wk, k, nullptr, n));
+        VHC(mm(m, prep, norm, w.wv, v, nullptr, n));
+        VXC(vx_rope_store_paged(be, q, k, v, d_pos, d_slot, m->kv[l], c.kv_fp16, n, c.num_heads, c.num_kv_heads,
+                                c.head_dim, c.block_size, c.rope_theta));
+        for (int i = 0; i < n_seqs; i++) {
+            const SeqRows &s = sr[i];
+            VXC(vx_sdpa_paged_tree(be, q + s.row0 * qd, m->kv[l], c.kv_fp16, m->d_tables + (size_t)s.slot * c.max_blocks_per_seq,
+                                   attn + s.row0 * qd, d_mask + mask_off[i], s.start, c.block_size, c.num_heads,
+                                   c.num_kv_heads, c.head_dim, scale, s.rows));
+        }
+        VHC(layer_tail(m, w, x, norm, attn, gate, up, n));
+    }
+    bool prep;
+    const vh_qweight *hw[1] = {&m->lm_head};
+    VHC(norm_for(m, x, m->final_norm, norm, n, hw, 1, &prep));
+    VHC(mm(m, prep, norm, m->lm_head, logits, nullptr, n));
+    VXC(vx_argmax_rows(be, logits, n, c.vocab, d_am));
+    std::vector<int32_t> am(n);
+    VXC(vx_to_host(be, am.data(), d_am, (size_t)n * 4));
+    if (logits_out) VXC(vx_to_host(be, logits_out, logits, (size_t)n * c.vocab * 4));
+    VXC(vx_sync(be));
+
+    // greedy acceptance per sequence, then the moves that make each accepted path contiguous
+    std::vector<int32_t> chain_off(1, 0), src, dst;
+    for (int i = 0; i < n_seqs; i++) {
+        const SeqRows &s = sr[i];
+        int cur = -1, want = am[s.row0], acc = 0;
+        for (;;) {
+            int next = -1;
+            for (int node = cur + 1; node < s.rows - 1; node++)
+                if (parent_idx[s.node0 + node] == cur && node_tokens[s.node0 + node] == want) {
+                    next = node;
+                    break;
+                }
+            if (next < 0) break;
+            accepted_nodes[s.node0 + acc] = next;
+            if (next != acc) {  // pool position start+1+next -> start+1+acc
+                src.push_back(slot_map[s.row0 + 1 + next]);
+                dst.push_back(slot_map[s.row0 + 1 + acc]);
+            }
+            acc++;
+            cur = next;
+            want = am[s.row0 + 1 + next];
+        }
+        num_accepted[i] = acc;
+        final_tokens[i] = want;
+        if ((int)src.size() > chain_off.back()) chain_off.push_back((int32_t)src.size());
+    }
+    if (!src.empty()) {
+        const int chains = (int)chain_off.size() - 1;
+        int32_t *d_co = ia(chain_off.size()), *d_src = ia(src.size()), *d_dst = ia(dst.size());
+        if (!d_co || !d_src || !d_dst) return fail("verification buffers: %s", vx_last_error());
+        VXC(vx_to_device(be, d_co, chain_off.data(), chain_off.size() * 4));
+        VXC(vx_to_device(be, d_src, src.data(), src.size() * 4));
+        VXC(vx_to_device(be, d_dst, dst.data(), dst.size() * 4));
+        for (int l = 0; l < c.num_layers; l++)
+            VXC(vx_paged_kv_move(be, m->kv[l], c.kv_fp16, d_co, d_src, d_dst, chains, c.num_kv_heads, c.head_dim,
+                                 c.block_size));
+        VXC(vx_sync(be));
+    }
+    for (int i = 0; i < n_seqs; i++)                                                       // medusa_scheduler.go:852-861
+        VHC(vh_pool_truncate_sequence(m, seq_ids[i], sr[i].start + 1 + num_accepted[i]));
+    return VH_OK;
+}
+
 // ------------------------------------------------------------------ device-driven greedy decode
 static int device_step(vh_model *m, int batch) {
     const vh_config &c = m->cfg;

@@ -71,6 +71,7 @@ SIGNATURES = {
     "vx_sdpa_paged_decode_ragged": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i]),
     "vx_sdpa_paged_tree": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),
     "vx_argmax_rows": (_i, [_vp, _vp, _i, _i, _vp]),
+    "vx_paged_kv_move": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i]),
     "vx_pack_batch": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "vx_decode_advance": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i]),
     "vx_graph_begin_capture": (_i, [_vp]),

@@ -71,6 +71,7 @@ def load_host():
         h.vh_pool_device_matches_host.argtypes = [C.c_void_p]
         h.vh_decode_batched.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]
         h.vh_prefill.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int64, C.c_int, C.c_int, C.c_void_p]
+        h.vh_verify_tree.argtypes = [C.c_void_p, C.c_int] + [C.c_void_p] * 10
         h.vh_decode_graph.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int,
                                       C.c_void_p, C.POINTER(C.c_float)]
         _host = h
@@ -310,6 +311,35 @@ class ModelRuntime:
         self._ck(self._h.vh_prefill(self._m, t.ctypes.data, t.size, seq_id, start_pos, int(all_logits),
                                     logits.ctypes.data))
         return logits if all_logits else logits[0]
+
+    def verify_tree(self, seq_ids, input_tokens, start_pos, trees, want_logits=True):
+        """One verification pass over a candidate tree per sequence (vh_verify_tree). trees: one
+        (node tokens, parent indices) pair per sequence, in CandidateTree.Linearize order.
+        -> ([accepted node indices per sequence], [final token per sequence], [logits (1 + nodes, vocab) per
+        sequence] or None)"""
+        n = len(seq_ids)
+        s = np.ascontiguousarray(seq_ids, dtype=np.int64)
+        t = np.ascontiguousarray(input_tokens, dtype=np.int32)
+        sp = np.ascontiguousarray(start_pos, dtype=np.int32)
+        nn = np.array([len(tr[0]) for tr in trees], dtype=np.int32)
+        toks = np.ascontiguousarray([x for tr in trees for x in tr[0]] or [0], dtype=np.int32)
+        par = np.ascontiguousarray([x for tr in trees for x in tr[1]] or [0], dtype=np.int32)
+        nacc = np.zeros(n, dtype=np.int32)
+        acc = np.zeros(max(1, int(nn.sum())), dtype=np.int32)
+        fin = np.zeros(n, dtype=np.int32)
+        rows = n + int(nn.sum())
+        logits = np.empty((rows, self.cfg.vocab), dtype=np.float32) if want_logits else None
+        self._ck(self._h.vh_verify_tree(self._m, n, s.ctypes.data, t.ctypes.data, sp.ctypes.data, nn.ctypes.data,
+                                        toks.ctypes.data, par.ctypes.data, nacc.ctypes.data, acc.ctypes.data,
+                                        fin.ctypes.data, logits.ctypes.data if want_logits else None))
+        accepted, per_seq, node0, row0 = [], [], 0, 0
+        for i in range(n):
+            accepted.append([int(x) for x in acc[node0:node0 + nacc[i]]])
+            if want_logits:
+                per_seq.append(logits[row0:row0 + 1 + nn[i]])
+            node0 += int(nn[i])
+            row0 += 1 + int(nn[i])
+        return accepted, [int(x) for x in fin], (per_seq if want_logits else None)
 
     def decode_graph(self, first_tokens, seq_ids, positions, steps, use_graph=True, batch=None):
         """Greedy device-driven decode. first_tokens=None continues the batch loaded on the device.
