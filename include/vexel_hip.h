@@ -32,12 +32,12 @@ enum {
     VX_ERR_INVALID = 1,     /* bad argument (shape, alignment, null pointer) */
     VX_ERR_OOM = 2,         /* device allocation failed */
     VX_ERR_HIP = 3,         /* a HIP runtime call failed */
-    VX_ERR_UNSUPPORTED = 4  /* format not implemented (Q5_K, Q5_0, BF16) */
+    VX_ERR_UNSUPPORTED = 4  /* unknown weight format, or a fused form the given shapes do not have */
 };
 
 /* Weight formats for the generic entry points (GGUF block layouts,
  * inference/pkg/gguf/dequant.go). */
-enum { VX_Q4_0 = 1, VX_Q8_0 = 2, VX_Q4_K = 3, VX_Q6_K = 4 };
+enum { VX_Q4_0 = 1, VX_Q8_0 = 2, VX_Q4_K = 3, VX_Q6_K = 4, VX_Q5_0 = 5, VX_Q5_K = 6, VX_BF16 = 7 };
 
 /* ---- lifetime / errors ------------------------------------------------------ */
 /* metal.NewBackend (backend/metal/backend.go:238-409); Backend.Device (backend.go:311) */
@@ -97,10 +97,11 @@ int vx_matmul_q4_0(vx_backend *be, const float *a, const void *b, float *out, in
 int vx_matmul_q4_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :55 */
 int vx_matmul_q6_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :60 */
 int vx_matmul_q8_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :75 */
-/* :65, :70, :80 -- not in any BASELINE config; return VX_ERR_UNSUPPORTED. */
-int vx_matmul_q5_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k);
-int vx_matmul_q5_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k);
-int vx_matmul_bf16(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k);
+/* Not in any BASELINE config: one wave per weight row on the exact dequantised values (pkg/gguf/dequant.go:
+ * 423-500, 100-145, 215-228), no tiled or matrix-vector fast path. */
+int vx_matmul_q5_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :65 */
+int vx_matmul_q5_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :70 */
+int vx_matmul_bf16(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :80 */
 
 /* ---- PagedKVOps (backend.go:415-466) ----------------------------------------- */
 /* Pool layout per physical block: K[blockSize,numKVHeads,headDim] then V[same]

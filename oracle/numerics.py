@@ -12,9 +12,9 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB_PATH = os.path.join(_HERE, "libvexel_oracle.so")
 
-FMT_Q4_0, FMT_Q8_0, FMT_Q4_K, FMT_Q6_K = 1, 2, 3, 4
-BLOCK_ELEMS = {FMT_Q4_0: 32, FMT_Q8_0: 32, FMT_Q4_K: 256, FMT_Q6_K: 256}
-BLOCK_BYTES = {FMT_Q4_0: 18, FMT_Q8_0: 34, FMT_Q4_K: 144, FMT_Q6_K: 210}
+FMT_Q4_0, FMT_Q8_0, FMT_Q4_K, FMT_Q6_K, FMT_Q5_0, FMT_Q5_K, FMT_BF16 = 1, 2, 3, 4, 5, 6, 7
+BLOCK_ELEMS = {FMT_Q4_0: 32, FMT_Q8_0: 32, FMT_Q4_K: 256, FMT_Q6_K: 256, FMT_Q5_0: 32, FMT_Q5_K: 256, FMT_BF16: 1}
+BLOCK_BYTES = {FMT_Q4_0: 18, FMT_Q8_0: 34, FMT_Q4_K: 144, FMT_Q6_K: 210, FMT_Q5_0: 22, FMT_Q5_K: 176, FMT_BF16: 2}
 
 
 def build(force=False):
@@ -89,11 +89,12 @@ def f16_to_f32_array(h):
 
 # ---------------------------------------------------------------- dequant
 _DEQ = {FMT_Q4_0: "vxo_dequant_q4_0", FMT_Q8_0: "vxo_dequant_q8_0",
-        FMT_Q4_K: "vxo_dequant_q4_k", FMT_Q6_K: "vxo_dequant_q6_k"}
+        FMT_Q4_K: "vxo_dequant_q4_k", FMT_Q6_K: "vxo_dequant_q6_k", FMT_Q5_0: "vxo_dequant_q5_0",
+        FMT_Q5_K: "vxo_dequant_q5_k", FMT_BF16: "vxo_dequant_bf16"}
 
 
 def dequantize(fmt, data, n):
-    """gguf.Dequantize, dequant.go:503-538 (Q4_0/Q8_0/Q4_K/Q6_K arms)."""
+    """gguf.Dequantize, dequant.go:503-538 (Q4_0/Q8_0/Q4_K/Q6_K/Q5_0/Q5_K/BF16 arms)."""
     data = _u8(data).reshape(-1)
     out = np.empty(n, dtype=np.float32)
     getattr(_lib, _DEQ[fmt])(_p(data), C.c_int64(data.size), C.c_int64(n), _p(out))

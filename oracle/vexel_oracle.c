@@ -275,6 +275,84 @@ VXO_API void vxo_dequant_q6_k(const uint8_t *data, int64_t nbytes, int64_t n, fl
     }
 }
 
+/* inference/pkg/gguf/dequant.go:100-145: q = low nibble | bit j (or j+16) of qh << 4; element (q - 16) * d */
+VXO_API void vxo_dequant_q5_0(const uint8_t *data, int64_t nbytes, int64_t n, float *out) {
+    const int64_t bs = 32, bb = 22;
+    int64_t nblk = (n + bs - 1) / bs;
+    memset(out, 0, (size_t)n * sizeof(float));
+    for (int64_t b = 0; b < nblk; b++) {
+        int64_t off = b * bb;
+        if (off + bb > nbytes) break;
+        float d = vxo_f16_to_f32(rd_u16(data + off));
+        uint32_t qh = (uint32_t)data[off + 2] | ((uint32_t)data[off + 3] << 8) | ((uint32_t)data[off + 4] << 16) |
+                      ((uint32_t)data[off + 5] << 24);
+        for (int j = 0; j < 16; j++) {
+            uint8_t bv = data[off + 6 + j];
+            int64_t idx = b * bs + j;
+            if (idx < n) {
+                uint8_t xh0 = (uint8_t)(((qh >> j) << 4) & 0x10);
+                int q = (int)(bv & 0x0F) | (int)xh0;
+                out[idx] = (float)(q - 16) * d;
+            }
+            idx = b * bs + j + 16;
+            if (idx < n) {
+                uint8_t xh1 = (uint8_t)(((qh >> (j + 16)) << 4) & 0x10);
+                int q = (int)(bv >> 4) | (int)xh1;
+                out[idx] = (float)(q - 16) * d;
+            }
+        }
+    }
+}
+
+/* inference/pkg/gguf/dequant.go:423-500: Q4_K's header and 6-bit scales, then qh[32] (bit 2*group + half of
+ * qh[l] is the fifth bit of element 64*group + 32*half + l) and the nibbles. d1 = d*float32(sc) and
+ * dm1 = dmin*float32(m) are rounded first; the element is d1*q - dm1. */
+VXO_API void vxo_dequant_q5_k(const uint8_t *data, int64_t nbytes, int64_t n, float *out) {
+    const int64_t bs = 256, bb = 176;
+    int64_t nblk = (n + bs - 1) / bs;
+    memset(out, 0, (size_t)n * sizeof(float));
+    for (int64_t b = 0; b < nblk; b++) {
+        int64_t off = b * bb;
+        if (off + bb > nbytes) break;
+        float d = vxo_f16_to_f32(rd_u16(data + off));
+        float dmin = vxo_f16_to_f32(rd_u16(data + off + 2));
+        const uint8_t *scales = data + off + 4;
+        const uint8_t *qh = data + off + 16;
+        const uint8_t *qs = data + off + 48;
+        int qoff = 0, is = 0;
+        uint8_t u1 = 1, u2 = 2;
+        for (int j = 0; j < 256; j += 64) {
+            uint8_t sc1, m1, sc2, m2;
+            vxo_get_scale_min_k4(is + 0, scales, &sc1, &m1);
+            float d1 = d * (float)sc1;
+            float dm1 = dmin * (float)m1;
+            vxo_get_scale_min_k4(is + 1, scales, &sc2, &m2);
+            float d2 = d * (float)sc2;
+            float dm2 = dmin * (float)m2;
+            for (int l = 0; l < 32; l++) {
+                int64_t i1 = b * bs + j + l, i2 = b * bs + j + l + 32;
+                uint8_t hb1 = (qh[l] & u1) ? 16 : 0, hb2 = (qh[l] & u2) ? 16 : 0;
+                if (i1 < n) out[i1] = d1 * (float)(uint8_t)((qs[qoff + l] & 0x0F) + hb1) - dm1;
+                if (i2 < n) out[i2] = d2 * (float)(uint8_t)((qs[qoff + l] >> 4) + hb2) - dm2;
+            }
+            qoff += 32;
+            is += 2;
+            u1 = (uint8_t)(u1 << 2);
+            u2 = (uint8_t)(u2 << 2);
+        }
+    }
+}
+
+/* inference/pkg/gguf/dequant.go:215-228: the 16 bits are the upper half of the float32 */
+VXO_API void vxo_dequant_bf16(const uint8_t *data, int64_t nbytes, int64_t n, float *out) {
+    memset(out, 0, (size_t)n * sizeof(float));
+    for (int64_t i = 0; i < n; i++) {
+        if (i * 2 + 2 > nbytes) break;
+        uint32_t u = (uint32_t)rd_u16(data + i * 2) << 16;
+        memcpy(out + i, &u, 4);
+    }
+}
+
 /* inference/pkg/gguf/dequant.go:200-211 */
 VXO_API void vxo_dequant_f16(const uint8_t *data, int64_t nbytes, int64_t n, float *out) {
     memset(out, 0, (size_t)n * sizeof(float));
@@ -353,6 +431,9 @@ VXO_API int vxo_matmul_quant_via_dequant(int fmt, const float *a, const uint8_t 
     case 2: row_bytes = (int64_t)k / 32 * 34; break;
     case 3: row_bytes = (int64_t)k / 256 * 144; break;
     case 4: row_bytes = (int64_t)k / 256 * 210; break;
+    case 5: row_bytes = (int64_t)k / 32 * 22; break;
+    case 6: row_bytes = (int64_t)k / 256 * 176; break;
+    case 7: row_bytes = (int64_t)k * 2; break;
     default: return -1;
     }
     float *w = (float *)malloc((size_t)k * sizeof(float));
@@ -364,6 +445,9 @@ VXO_API int vxo_matmul_quant_via_dequant(int fmt, const float *a, const uint8_t 
         case 2: vxo_dequant_q8_0(row, row_bytes, k, w); break;
         case 3: vxo_dequant_q4_k(row, row_bytes, k, w); break;
         case 4: vxo_dequant_q6_k(row, row_bytes, k, w); break;
+        case 5: vxo_dequant_q5_0(row, row_bytes, k, w); break;
+        case 6: vxo_dequant_q5_k(row, row_bytes, k, w); break;
+        case 7: vxo_dequant_bf16(row, row_bytes, k, w); break;
         }
         for (int i = 0; i < m; i++) {
             const float *arow = a + (int64_t)i * k;

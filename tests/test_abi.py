@@ -31,9 +31,9 @@ def test_library_exports_every_declared_symbol():
 def test_error_text_is_available_without_a_gpu():
     l = lib.load()
     assert isinstance(l.vx_last_error(), bytes)
-    # the reference's unimplemented formats answer without touching the device
-    assert l.vx_matmul_q5_k(None, None, None, None, 1, 32, 32) == lib.VX_ERR_UNSUPPORTED
-    assert b"not implemented" in l.vx_last_error()
+    # a call without a backend is refused before anything touches the device
+    assert l.vx_matmul_q5_k(None, None, None, None, 1, 32, 32) == lib.VX_ERR_INVALID
+    assert b"null backend" in l.vx_last_error()
 
 
 def test_every_entry_point_cites_the_reference():

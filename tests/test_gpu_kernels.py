@@ -74,6 +74,56 @@ def test_dequantize_all_byte_patterns(be, fmt):
     be.reset_pool()
 
 
+@pytest.mark.parametrize("fmt", [nx.FMT_Q5_0, nx.FMT_Q5_K, nx.FMT_BF16])
+def test_dequantize_other_formats_bit_exact(be, fmt):
+    """Q5_0, Q5_K, BF16 (pkg/gguf/dequant.go:100-145, 423-500, 215-228): random weights, then blocks of random
+    bytes with finite f16 headers (every code, every fifth-bit position)."""
+    rng = np.random.default_rng(300 + fmt)
+    n, k = 11, 1024
+    raw = qz.random_quant(fmt, rng, n, k).reshape(-1).copy()
+    bb, be_ = nx.BLOCK_BYTES[fmt], nx.BLOCK_ELEMS[fmt]
+    rnd = rng.integers(0, 256, size=(2048 // be_ * 8, bb), dtype=np.uint8)
+    if fmt == nx.FMT_BF16:
+        rnd[(rnd[:, 1] & 0x7F) == 0x7F, 1] &= 0xBF          # no NaN / Inf patterns
+    else:
+        for col in ((0,) if fmt == nx.FMT_Q5_0 else (0, 2)):
+            hi = rnd[:, col + 1]
+            bad = (hi & 0x7C) == 0x7C
+            rnd[bad, col + 1] = hi[bad] & 0xBF
+    for data in (raw, rnd.reshape(-1)):
+        cnt = data.size // bb * be_
+        want = nx.dequantize(fmt, data, cnt)
+        d = be.upload(data)
+        o = be.alloc(cnt * 4)
+        be.dequantize(fmt, d, o, cnt)
+        got = be.download(o, (cnt,), np.float32)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    be.reset_pool()
+
+
+@pytest.mark.parametrize("fmt", [nx.FMT_Q5_0, nx.FMT_Q5_K, nx.FMT_BF16])
+@pytest.mark.parametrize("m", [1, 3, 8, 9, 32])
+def test_matmul_other_formats_vs_oracle(be, fmt, m):
+    """MatMulQ5_0 / MatMulQ5_K / MatMulBF16 (backend.go:65-80) against Dequantize + the naive product."""
+    rng = np.random.default_rng(fmt * 100 + m)
+    n, k = 70, 1536
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    want = nx.matmul_quant(fmt, a, w, m, n, k)
+    da, dw = be.upload(a), be.upload(w)
+    dout = be.alloc(m * n * 4)
+    {nx.FMT_Q5_0: be.matmul_q5_0, nx.FMT_Q5_K: be.matmul_q5_k, nx.FMT_BF16: be.matmul_bf16}[fmt](da, dw, dout, m, n, k)
+    got = be.download(dout, (m, n), np.float32)
+    _close(got, want, 2e-5, 2e-6 * np.abs(want).max() + 1e-7, "matmul fmt %d m %d" % (fmt, m))
+    # an activation that is not 16-byte aligned takes the element-wise path: same values to rounding
+    if m == 3:
+        big = be.alloc((m * k + 1) * 4)
+        be.copy_buffer(da, 0, big, 4, m * k * 4)
+        be.matmul_quant(fmt, big + 4, dw, dout, None, m, n, k)
+        _close(be.download(dout, (m, n), np.float32), want, 2e-5, 2e-6 * np.abs(want).max() + 1e-7, "unaligned")
+    be.reset_pool()
+
+
 # ------------------------------------------------------------------ quantized matmul
 @pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 32, 40])
@@ -421,12 +471,19 @@ def test_matmul_quant_unaligned_k_uses_fallback(be):
     be.reset_pool()
 
 
-def test_unsupported_formats_report(be):
+def test_unknown_format_and_bad_shape_report(be):
     from vexel_amd.backend import VexelError
-    for fn in (be.matmul_q5_k, be.matmul_q5_0, be.matmul_bf16):
-        with pytest.raises(VexelError) as e:
-            fn(0, 0, 0, 1, 32, 32)
-        assert e.value.code == 4
+    d = be.alloc(4096)
+    with pytest.raises(VexelError) as e:
+        be.matmul_quant(9, d, d, d, None, 1, 4, 32)          # no such format
+    assert e.value.code == 4
+    with pytest.raises(VexelError) as e:
+        be.matmul_q5_k(d, d, d, 1, 4, 128)                   # K is not a whole number of 256-element blocks
+    assert e.value.code == 1
+    with pytest.raises(VexelError) as e:
+        be.matmul_q5_0(0, 0, 0, 1, 32, 32)
+    assert e.value.code == 1
+    be.reset_pool()
 
 
 def test_matmul_f32(be):

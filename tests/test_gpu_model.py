@@ -271,10 +271,12 @@ def test_c5_tree_verification_batched(be):
     mr.close()
 
 
-GGUF_TYPE = {nx.FMT_Q4_0: 2, nx.FMT_Q8_0: 8, nx.FMT_Q4_K: 12, nx.FMT_Q6_K: 14}
+GGUF_TYPE = {nx.FMT_Q4_0: 2, nx.FMT_Q8_0: 8, nx.FMT_Q4_K: 12, nx.FMT_Q6_K: 14, nx.FMT_Q5_0: 6, nx.FMT_Q5_K: 13,
+             nx.FMT_BF16: 30}
 
 
-@pytest.mark.parametrize("case", ["q4_k_m mix with output", "tied q8_0 embedding", "tied f16 embedding, q4_0"])
+@pytest.mark.parametrize("case", ["q4_k_m mix with output", "tied q8_0 embedding", "tied f16 embedding, q4_0",
+                                  "q5_k mix with q5_0 and bf16, tied q5_0 embedding"])
 def test_load_gguf_checkpoint(be, tmp_path, case):
     """A checkpoint written as a GGUF file (oracle/gguf.py writer: llama.* metadata, llama.cpp tensor names) and read
     back by the C++ loader gives the logits and greedy tokens of the oracle model built from the same tensors:
@@ -287,8 +289,10 @@ def test_load_gguf_checkpoint(be, tmp_path, case):
     rng = np.random.default_rng(55)
     cfg = om.ModelConfig(num_layers=2, hidden=512, num_heads=8, num_kv_heads=2, head_dim=64, ffn=1024, vocab=768,
                          eps=1e-6, rope_theta=500000.0)
-    fmt = nx.FMT_Q4_0 if "q4_0" in case else nx.FMT_Q4_K
+    fmt = nx.FMT_Q4_0 if "q4_0" in case else nx.FMT_Q5_K if "q5_k" in case else nx.FMT_Q4_K
     over = {"wv": nx.FMT_Q6_K, "w2": nx.FMT_Q6_K} if "mix" in case else {}
+    if "q5_k" in case:
+        over = {"wv": nx.FMT_Q5_0, "wo": nx.FMT_BF16, "w2": nx.FMT_Q5_0}
     qd, kvd = cfg.num_heads * cfg.head_dim, cfg.num_kv_heads * cfg.head_dim
     tensors, layers = [], []
     f16 = lambda a: nx.f16_to_f32_array(nx.f32_to_f16_array(a.astype(np.float32)))
@@ -314,7 +318,7 @@ def test_load_gguf_checkpoint(be, tmp_path, case):
         tensors.append(("token_embd.weight", [cfg.hidden, cfg.vocab], og.T_F16, nx.f32_to_f16_array(emb.reshape(-1)).tobytes()))
         head = om.QWeight(0, emb, cfg.vocab, cfg.hidden)               # tied, float32
     else:
-        ef = nx.FMT_Q8_0 if "q8_0" in case else nx.FMT_Q4_0
+        ef = nx.FMT_Q8_0 if "q8_0" in case else nx.FMT_Q5_0 if "q5_0 embedding" in case else nx.FMT_Q4_0
         eq = qz.random_quant(ef, rng, cfg.vocab, cfg.hidden)
         emb = nx.dequantize(ef, eq, cfg.vocab * cfg.hidden).reshape(cfg.vocab, cfg.hidden)
         tensors.append(("token_embd.weight", [cfg.hidden, cfg.vocab], GGUF_TYPE[ef], eq.tobytes()))

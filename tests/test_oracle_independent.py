@@ -128,6 +128,63 @@ def test_q6_k_closed_form():
         assert np.array_equal(nx.dequantize(nx.FMT_Q6_K, blk, 256), vals.astype(np.float32))
 
 
+def test_q5_0_closed_form_every_code_in_every_position():
+    """element = float32(q - 16) * d; the encoder states the layout on its own (bit i of qh = fifth bit of
+    element i), so a swapped half or a wrong bit index fails."""
+    rng = np.random.default_rng(7)
+    for shift in range(32):
+        vals = np.array([(i * 7 + shift) % 32 for i in range(32)])
+        blk = qz.encode_q5_0_block(1.0, vals)
+        assert np.array_equal(nx.dequantize(nx.FMT_Q5_0, blk, 32), (vals - 16).astype(np.float32))
+    for _ in range(20):
+        d = float(rng.uniform(1e-4, 0.1)) * (1 if rng.random() < 0.5 else -1)
+        vals = rng.integers(0, 32, 32)
+        r = nx.dequantize(nx.FMT_Q5_0, qz.encode_q5_0_block(d, vals), 32)
+        want = np.array([np.float32(np.float32(v - 16) * _f16(d)) for v in vals], dtype=np.float32)
+        assert np.array_equal(r, want)
+
+
+def test_q5_k_closed_form():
+    """element = (d*sc)*q - (dmin*m) with q in [0,31]: Q4_K's arithmetic with a fifth bit from qh."""
+    rng = np.random.default_rng(8)
+    # a single high bit set: exactly one element differs from the four-bit block
+    for e in (0, 31, 32, 100, 223, 255):
+        vals = np.zeros(256, dtype=int)
+        vals[e] = 16
+        blk = qz.encode_q5_k_block(1.0, 0.0, np.ones(8, dtype=int), np.zeros(8, dtype=int), vals)
+        assert np.array_equal(nx.dequantize(nx.FMT_Q5_K, blk, 256), vals.astype(np.float32))
+    for _ in range(20):
+        d, dmin = float(rng.uniform(1e-4, 0.1)), float(rng.uniform(1e-4, 0.1))
+        sc = rng.integers(0, 64, 8); mn = rng.integers(0, 64, 8)
+        vals = rng.integers(0, 32, 256)
+        r = nx.dequantize(nx.FMT_Q5_K, qz.encode_q5_k_block(d, dmin, sc, mn, vals), 256)
+        df, dmf = _f16(d), _f16(dmin)
+        want = np.empty(256, dtype=np.float32)
+        for i in range(256):
+            sb = i // 32
+            d1 = np.float32(df * np.float32(sc[sb]))
+            dm1 = np.float32(dmf * np.float32(mn[sb]))
+            want[i] = np.float32(np.float32(d1 * np.float32(vals[i])) - dm1)
+        assert np.array_equal(r, want)
+    # with the fifth bits clear a Q5_K block decodes as the Q4_K block with the same header and nibbles
+    vals = rng.integers(0, 16, 256)
+    sc = rng.integers(0, 64, 8); mn = rng.integers(0, 64, 8)
+    assert np.array_equal(nx.dequantize(nx.FMT_Q5_K, qz.encode_q5_k_block(0.01, 0.02, sc, mn, vals), 256),
+                          nx.dequantize(nx.FMT_Q4_K, qz.encode_q4_k_block(0.01, 0.02, sc, mn, vals), 256))
+
+
+def test_bf16_all_patterns_against_numpy():
+    h = np.arange(65536, dtype=np.uint16)
+    got = nx.dequantize(nx.FMT_BF16, h.view(np.uint8), 65536)
+    want = (h.astype(np.uint32) << 16).view(np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # the synthetic-weight maker rounds to nearest even
+    w = np.array([[1.0, 1.00390625, 1.005859375, -3.0e-5]], dtype=np.float32)
+    back = nx.dequantize(nx.FMT_BF16, qz.quantize_bf16(w), 4)
+    assert back[0] == 1.0 and back[1] == 1.0 and back[2] == np.float32(1.0078125)
+    assert abs(back[3] + 3.0e-5) < 3.0e-5 * 2 ** -8
+
+
 def test_multi_block_and_partial_count():
     rng = np.random.default_rng(6)
     w = rng.standard_normal((3, 128)).astype(np.float32)
@@ -139,7 +196,8 @@ def test_multi_block_and_partial_count():
 
 
 # ----------------------------------------------------------------- matmul
-@pytest.mark.parametrize("fmt", [nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q4_K, nx.FMT_Q6_K])
+@pytest.mark.parametrize("fmt", [nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q4_K, nx.FMT_Q6_K, nx.FMT_Q5_0, nx.FMT_Q5_K,
+                                 nx.FMT_BF16])
 def test_quant_matmul_vs_float64_of_exact_dequant(fmt):
     rng = np.random.default_rng(10 + fmt)
     m, n, k = 3, 5, 512

@@ -41,9 +41,32 @@ def test_q4_0_kat():
     assert r[2] == -8.0 and r[18] == -8.0
 
 
+# ---- dequant_test.go:142-161
+def test_bf16_kat():
+    data = np.array([0x80, 0x3F, 0x00, 0x40], dtype=np.uint8)
+    assert np.array_equal(nx.dequantize(nx.FMT_BF16, data, 2), np.array([1.0, 2.0], dtype=np.float32))
+
+
+# ---- dequant_test.go:184-250 (all_zero, split_halves, with_scale)
+def test_q5_0_kats():
+    data = np.zeros(22, dtype=np.uint8)
+    data[0:2] = [0x00, 0x3C]
+    data[2:6] = 0xFF
+    assert np.array_equal(nx.dequantize(nx.FMT_Q5_0, data, 32), np.zeros(32, dtype=np.float32))
+    data[2:6] = [0x00, 0x00, 0xFF, 0xFF]
+    data[6:22] = 0x88
+    r = nx.dequantize(nx.FMT_Q5_0, data, 32)
+    assert np.all(r[:16] == -8.0) and np.all(r[16:] == 8.0)
+    data = np.zeros(22, dtype=np.uint8)
+    data[0:2] = [0x00, 0x38]
+    data[6] = 0x0F
+    r = nx.dequantize(nx.FMT_Q5_0, data, 32)
+    assert r[0] == -0.5 and r[16] == -8.0
+
+
 # ---- dequant_test.go:307-320: a buffer too short for one block dequantises to zeros
 def test_short_buffer_zeros():
-    for fmt in (nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q4_K, nx.FMT_Q6_K):
+    for fmt in (nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q4_K, nx.FMT_Q6_K, nx.FMT_Q5_0, nx.FMT_Q5_K):
         data = np.full(nx.BLOCK_BYTES[fmt] - 1, 0xFF, dtype=np.uint8)
         assert np.all(nx.dequantize(fmt, data, 32) == 0)
     data = np.full(100, 0x55, dtype=np.uint8)  # 100 bytes < 144

@@ -314,6 +314,49 @@ __global__ void dequant_q4_k_kernel(const uint8_t *src, float *dst, int64_t nblk
     }
 }
 
+// pkg/gguf/dequant.go:423-500: Q4_K's arithmetic with a fifth bit from qh
+__global__ void dequant_q5_k_kernel(const uint8_t *src, float *dst, int64_t nblk) {
+    int64_t b = (int64_t)blockIdx.x * (blockDim.x / 64) + (threadIdx.x >> 6);
+    if (b >= nblk) return;
+    int t = threadIdx.x & 63;
+    const uint8_t *p = src + b * 176;
+    float d = f16_bits_to_f32(ld_u16(p)), dmin = f16_bits_to_f32(ld_u16(p + 2));
+    const uint8_t *scales = p + 4, *qh = p + 16, *qs = p + 48;
+    float *o = dst + b * 256;
+    for (int e = t; e < 256; e += 64) {
+        int grp = e >> 6, l = e & 31, hi = (e >> 5) & 1;
+        uint8_t sc, mn;
+        scale_min_k4(grp * 2 + hi, scales, sc, mn);
+        float d1 = __fmul_rn(d, (float)sc), dm1 = __fmul_rn(dmin, (float)mn);
+        uint8_t bv = qs[grp * 32 + l];
+        int q = (hi ? (bv >> 4) : (bv & 0xF)) + (((qh[l] >> (grp * 2 + hi)) & 1) << 4);
+        o[e] = __fsub_rn(__fmul_rn(d1, (float)q), dm1);
+    }
+}
+
+// pkg/gguf/dequant.go:100-145; thread = one block of 32
+__global__ void dequant_q5_0_kernel(const uint8_t *src, float *dst, int64_t nblk) {
+    int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (b >= nblk) return;
+    const uint8_t *p = src + b * 22;
+    float d = f16_bits_to_f32(ld_u16(p));
+    uint32_t qh = (uint32_t)ld_u16(p + 2) | ((uint32_t)ld_u16(p + 4) << 16);
+    float *o = dst + b * 32;
+    for (int j = 0; j < 16; j++) {
+        uint8_t bv = p[6 + j];
+        int q0 = (int)(bv & 0xF) | (int)(((qh >> j) & 1) << 4);
+        int q1 = (int)(bv >> 4) | (int)(((qh >> (j + 16)) & 1) << 4);
+        o[j] = __fmul_rn((float)(q0 - 16), d);
+        o[j + 16] = __fmul_rn((float)(q1 - 16), d);
+    }
+}
+
+// pkg/gguf/dequant.go:215-228
+__global__ void dequant_bf16_kernel(const uint8_t *src, float *dst, int64_t n) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = __uint_as_float((uint32_t)ld_u16(src + 2 * i) << 16);
+}
+
 __global__ void dequant_q6_k_kernel(const uint8_t *src, float *dst, int64_t nblk) {
     int64_t b = (int64_t)blockIdx.x * (blockDim.x / 64) + (threadIdx.x >> 6);
     if (b >= nblk) return;
@@ -563,6 +606,17 @@ int vx_dequantize(vx_backend *be, int fmt, const void *src, float *dst, int64_t 
     case VX_Q6_K:
         VX_REQUIRE(n % 256 == 0, "vx_dequantize: n must be a multiple of 256");
         dequant_q6_k_kernel<<<grid1d(n / 256, 4), 256, 0, be->stream>>>(s, dst, n / 256);
+        break;
+    case VX_Q5_0:
+        VX_REQUIRE(n % 32 == 0, "vx_dequantize: n must be a multiple of 32");
+        dequant_q5_0_kernel<<<grid1d(n / 32, kThreads), kThreads, 0, be->stream>>>(s, dst, n / 32);
+        break;
+    case VX_Q5_K:
+        VX_REQUIRE(n % 256 == 0, "vx_dequantize: n must be a multiple of 256");
+        dequant_q5_k_kernel<<<grid1d(n / 256, 4), 256, 0, be->stream>>>(s, dst, n / 256);
+        break;
+    case VX_BF16:
+        dequant_bf16_kernel<<<grid1d(n, kThreads), kThreads, 0, be->stream>>>(s, dst, n);
         break;
     default:
         set_error("vx_dequantize: unknown format %d", fmt);

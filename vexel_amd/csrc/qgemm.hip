@@ -827,6 +827,36 @@ __device__ __forceinline__ float deq_elem(int fmt, const uint8_t *row, int k) {
         int qq = hi ? (bv >> 4) : (bv & 0xF);
         return __fsub_rn(__fmul_rn(d1, (float)qq), dm1);
     }
+    if (fmt == VX_Q5_0) {  // pkg/gguf/dequant.go:100-145
+        const uint8_t *b = row + (size_t)(k >> 5) * 22;
+        const int i = k & 31;
+        const uint32_t qh = (uint32_t)b[2] | ((uint32_t)b[3] << 8) | ((uint32_t)b[4] << 16) | ((uint32_t)b[5] << 24);
+        const uint8_t bv = b[6 + (i & 15)];
+        const int q = (int)((i < 16) ? (bv & 0xF) : (bv >> 4)) | (int)(((qh >> i) & 1) << 4);
+        return __fmul_rn((float)(q - 16), h2f((uint16_t)(b[0] | (b[1] << 8))));
+    }
+    if (fmt == VX_Q5_K) {  // pkg/gguf/dequant.go:423-500
+        const uint8_t *b = row + (size_t)(k >> 8) * 176;
+        const int e = k & 255, grp = e >> 6, l = e & 31, hi = (e >> 5) & 1, j = grp * 2 + hi;
+        const uint8_t *q = b + 4;
+        uint32_t sc, mn;
+        if (j < 4) {
+            sc = q[j] & 63;
+            mn = q[j + 4] & 63;
+        } else {
+            sc = (q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4);
+            mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+        }
+        const float d1 = __fmul_rn(h2f((uint16_t)(b[0] | (b[1] << 8))), (float)sc);
+        const float dm1 = __fmul_rn(h2f((uint16_t)(b[2] | (b[3] << 8))), (float)mn);
+        const uint8_t bv = b[48 + grp * 32 + l];
+        const int qq = (int)(hi ? (bv >> 4) : (bv & 0xF)) + (int)(((b[16 + l] >> j) & 1) << 4);
+        return __fsub_rn(__fmul_rn(d1, (float)qq), dm1);
+    }
+    if (fmt == VX_BF16) {  // pkg/gguf/dequant.go:215-228
+        const uint32_t u = ((uint32_t)row[2 * (size_t)k] | ((uint32_t)row[2 * (size_t)k + 1] << 8)) << 16;
+        return __uint_as_float(u);
+    }
     // Q6_K, pkg/gguf/dequant.go:272-331
     const uint8_t *b = row + (size_t)(k >> 8) * 210;
     int e = k & 255, nn = e >> 7, r = e & 127, quad = r >> 5, l = r & 31, is = l >> 4;
@@ -856,6 +886,82 @@ __global__ void __launch_bounds__(64) qgemm_fallback_kernel(int fmt, const uint8
 #pragma unroll
         for (int i = 0; i < FB_M; i++)
             if (m0 + i < M) acc[i] = fmaf(a[(size_t)(m0 + i) * K + k], w, acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < FB_M; i++) {
+        float v = acc[i];
+        for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+        if (lane == 0 && m0 + i < M) {
+            if (residual) v = residual[(size_t)(m0 + i) * N + n] + v;
+            out[(size_t)(m0 + i) * N + n] = v;
+        }
+    }
+}
+
+// Formats without a tiled path (Q5_0, Q5_K, BF16): one wave per weight row, lane l takes elements 4l..4l+3 of every
+// 256-element stretch (coalesced float4 activation loads, the row's bytes shared through the cache), exact
+// dequantised values, float32 FMAs, a butterfly sum. grid = (N, ceil(M/FB_M)); block = 64.
+template <int FMT>
+__device__ __forceinline__ void deq4(const uint8_t *row, int k0, float (&w)[4]) {
+    if (FMT == VX_BF16) {
+        const uint16_t *p = (const uint16_t *)(row + 2 * (size_t)k0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = __uint_as_float((uint32_t)p[i] << 16);
+    } else if (FMT == VX_Q5_0) {
+        const uint8_t *b = row + (size_t)(k0 >> 5) * 22;
+        const uint16_t *h = (const uint16_t *)b;  // blocks start on even addresses
+        const int i0 = k0 & 31, j0 = i0 & 15;
+        const float d = h2f(h[0]);
+        const uint32_t qh = ((uint32_t)h[1] | ((uint32_t)h[2] << 16)) >> i0;
+        const uint32_t qs = ((uint32_t)h[3 + (j0 >> 1)] | ((uint32_t)h[4 + (j0 >> 1)] << 16)) >> (i0 & 16 ? 4 : 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int q = (int)((qs >> (8 * i)) & 0xF) | (int)(((qh >> i) & 1) << 4);
+            w[i] = __fmul_rn((float)(q - 16), d);
+        }
+    } else {  // Q5_K
+        const uint8_t *b = row + (size_t)(k0 >> 8) * 176;
+        const int e = k0 & 255, grp = e >> 6, l = e & 31, hi = (e >> 5) & 1, j = grp * 2 + hi;
+        const uint8_t *q = b + 4;
+        uint32_t sc, mn;
+        if (j < 4) {
+            sc = q[j] & 63;
+            mn = q[j + 4] & 63;
+        } else {
+            sc = (q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4);
+            mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+        }
+        const uint16_t *h = (const uint16_t *)b;
+        const float d1 = __fmul_rn(h2f(h[0]), (float)sc), dm1 = __fmul_rn(h2f(h[1]), (float)mn);
+        const uint16_t *qs16 = (const uint16_t *)(b + 48 + grp * 32 + l), *qh16 = (const uint16_t *)(b + 16 + l);
+        const uint32_t qs = ((uint32_t)qs16[0] | ((uint32_t)qs16[1] << 16)) >> (hi ? 4 : 0);
+        const uint32_t qh = ((uint32_t)qh16[0] | ((uint32_t)qh16[1] << 16)) >> j;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int qq = (int)((qs >> (8 * i)) & 0xF) + (int)(((qh >> (8 * i)) & 1) << 4);
+            w[i] = __fsub_rn(__fmul_rn(d1, (float)qq), dm1);
+        }
+    }
+}
+
+template <int FMT>
+__global__ void __launch_bounds__(64) qrow4_kernel(const uint8_t *__restrict__ W, const float *__restrict__ a,
+                                                   float *__restrict__ out, const float *__restrict__ residual, int M, int N,
+                                                   int K, size_t row_bytes) {
+    const int n = blockIdx.x, m0 = blockIdx.y * FB_M, lane = threadIdx.x;
+    const uint8_t *row = W + (size_t)n * row_bytes;
+    float acc[FB_M];
+#pragma unroll
+    for (int i = 0; i < FB_M; i++) acc[i] = 0.f;
+    for (int k0 = lane * 4; k0 < K; k0 += 256) {
+        float w[4];
+        deq4<FMT>(row, k0, w);
+#pragma unroll
+        for (int i = 0; i < FB_M; i++) {
+            const int m = min(m0 + i, M - 1);  // rows past M repeat the last one; their sums are dropped
+            const float4 x = *(const float4 *)(a + (size_t)m * K + k0);
+            acc[i] = fmaf(x.w, w[3], fmaf(x.z, w[2], fmaf(x.y, w[1], fmaf(x.x, w[0], acc[i]))));
+        }
     }
 #pragma unroll
     for (int i = 0; i < FB_M; i++) {
@@ -1324,6 +1430,9 @@ size_t fmt_row_bytes(int fmt, int k) {
     case VX_Q8_0: return (size_t)k / 32 * 34;
     case VX_Q4_K: return (size_t)k / 256 * 144;
     case VX_Q6_K: return (size_t)k / 256 * 210;
+    case VX_Q5_0: return (size_t)k / 32 * 22;
+    case VX_Q5_K: return (size_t)k / 256 * 176;
+    case VX_BF16: return (size_t)k * 2;
     }
     return 0;
 }
@@ -1466,16 +1575,17 @@ int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out
 // them from the boundary below, which needs the whole matrix to be a multiple of 16 bytes.
 bool fast_ok(int fmt, const void *b, int n, int k) {
     const size_t rb = fmt_row_bytes(fmt, k);
+    if (fmt < VX_Q4_0 || fmt > VX_Q6_K) return false;  // Q5_0, Q5_K, BF16: the row kernel
     if (k % 256 != 0 || ((uintptr_t)b % 16) != 0 || n < 1) return false;
     return fmt == VX_Q6_K ? ((size_t)n * rb) % 16 == 0 : rb % 16 == 0;
 }
 
 int check_fmt(int fmt, int k) {
-    if (fmt != VX_Q4_0 && fmt != VX_Q8_0 && fmt != VX_Q4_K && fmt != VX_Q6_K) {
+    if (fmt < VX_Q4_0 || fmt > VX_BF16) {
         set_error("quantized matmul: unknown format %d", fmt);
         return VX_ERR_UNSUPPORTED;
     }
-    const int blk = (fmt == VX_Q4_0 || fmt == VX_Q8_0) ? 32 : 256;
+    const int blk = fmt == VX_BF16 ? 1 : (fmt == VX_Q4_0 || fmt == VX_Q8_0 || fmt == VX_Q5_0) ? 32 : 256;
     VX_REQUIRE(k > 0 && k % blk == 0, "quantized matmul: K=%d is not a multiple of the block size %d", k, blk);
     return VX_OK;
 }
@@ -1594,6 +1704,14 @@ int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, floa
     if (!fast_ok(fmt, b, n, k) || ((uintptr_t)a % 16) != 0) {
         const size_t rb = fmt_row_bytes(fmt, k);
         dim3 grid(n, ceil_div(m, FB_M));
+        if (fmt > VX_Q6_K && k % 4 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 2) == 0) {
+            const uint8_t *w = (const uint8_t *)b;
+            if (fmt == VX_Q5_0) qrow4_kernel<VX_Q5_0><<<grid, 64, 0, be->stream>>>(w, a, out, residual, m, n, k, rb);
+            else if (fmt == VX_Q5_K) qrow4_kernel<VX_Q5_K><<<grid, 64, 0, be->stream>>>(w, a, out, residual, m, n, k, rb);
+            else qrow4_kernel<VX_BF16><<<grid, 64, 0, be->stream>>>(w, a, out, residual, m, n, k, rb);
+            VX_CHECK_LAUNCH();
+            return VX_OK;
+        }
         qgemm_fallback_kernel<<<grid, 64, 0, be->stream>>>(fmt, (const uint8_t *)b, a, out, residual, m, n, k, rb);
         VX_CHECK_LAUNCH();
         return VX_OK;
@@ -1877,12 +1995,14 @@ int vx_matmul_q8_0(vx_backend *be, const float *a, const void *b, float *out, in
     return vx_matmul_quant(be, VX_Q8_0, a, b, out, nullptr, m, n, k);
 }
 
-static int unsupported(const char *name) {
-    set_error("%s: format not implemented by this backend", name);
-    return VX_ERR_UNSUPPORTED;
+int vx_matmul_q5_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k) {
+    return vx_matmul_quant(be, VX_Q5_K, a, b, out, nullptr, m, n, k);
 }
-int vx_matmul_q5_k(vx_backend *, const float *, const void *, float *, int, int, int) { return unsupported("vx_matmul_q5_k"); }
-int vx_matmul_q5_0(vx_backend *, const float *, const void *, float *, int, int, int) { return unsupported("vx_matmul_q5_0"); }
-int vx_matmul_bf16(vx_backend *, const float *, const void *, float *, int, int, int) { return unsupported("vx_matmul_bf16"); }
+int vx_matmul_q5_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k) {
+    return vx_matmul_quant(be, VX_Q5_0, a, b, out, nullptr, m, n, k);
+}
+int vx_matmul_bf16(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k) {
+    return vx_matmul_quant(be, VX_BF16, a, b, out, nullptr, m, n, k);
+}
 
 }  // extern "C"

@@ -384,7 +384,7 @@ int vh_gguf_tensor_name(const char *hf_name, char *out, size_t cap) {
 // ------------------------------------------------------------------ the loader rule
 namespace {
 
-enum { T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q8_0 = 8, T_Q4_K = 12, T_Q6_K = 14 };
+enum { T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q5_0 = 6, T_Q8_0 = 8, T_Q4_K = 12, T_Q5_K = 13, T_Q6_K = 14, T_BF16 = 30 };
 
 int quant_fmt(uint32_t type) {  // GGUF tensor type -> VX_* format of the quantized matmuls, 0 if it has none
     switch (type) {
@@ -392,9 +392,14 @@ int quant_fmt(uint32_t type) {  // GGUF tensor type -> VX_* format of the quanti
     case T_Q8_0: return VX_Q8_0;
     case T_Q4_K: return VX_Q4_K;
     case T_Q6_K: return VX_Q6_K;
+    case T_Q5_0: return VX_Q5_0;
+    case T_Q5_K: return VX_Q5_K;
+    case T_BF16: return VX_BF16;
     }
     return 0;
 }
+
+int fmt_block(int fmt) { return fmt == VX_BF16 ? 1 : (fmt == VX_Q4_0 || fmt == VX_Q8_0 || fmt == VX_Q5_0) ? 32 : 256; }
 
 float f16_to_f32(uint16_t h) {  // dequant.go:231-261
     const uint32_t sign = (uint32_t)(h >> 15) << 31;
@@ -450,7 +455,7 @@ struct Loader {
             return gfail("%s: shape [%llu, %llu] does not match the configuration's [%d, %d]", name.c_str(),
                          (unsigned long long)t.dims[1], (unsigned long long)t.dims[0], n, k);
         const int fmt = quant_fmt(t.type);
-        if (!fmt) return gfail("%s: tensor type %u has no quantized matmul here (Q4_0, Q8_0, Q4_K, Q6_K do)", name.c_str(), t.type);
+        if (!fmt) return gfail("%s: tensor type %u has no quantized matmul here (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K, BF16 do)", name.c_str(), t.type);
         void *p = dev_copy(t.data, (size_t)t.n_bytes);
         if (!p) return gfail("%s: device copy failed: %s", name.c_str(), vx_last_error());
         w->fmt = fmt;
@@ -475,7 +480,7 @@ struct Loader {
             for (int64_t i = 0; i < n; i++) tmp[(size_t)i] = f16_to_f32(h[i]);
             dst = dev_copy(tmp.data(), (size_t)n * 4);
         } else if (const int fmt = quant_fmt(t.type)) {
-            if (n % (fmt == VX_Q4_0 || fmt == VX_Q8_0 ? 32 : 256) != 0) return gfail("%s: not a whole number of blocks", name.c_str());
+            if (n % fmt_block(fmt) != 0) return gfail("%s: not a whole number of blocks", name.c_str());
             void *raw = vx_alloc_permanent(be, (size_t)t.n_bytes);
             dst = vx_alloc_permanent(be, (size_t)n * 4);
             bool ok = raw && dst && vx_to_device(be, raw, t.data, (size_t)t.n_bytes) == VX_OK &&
