@@ -156,8 +156,8 @@ typedef struct vh_load_options {  /* what the checkpoint does not say: the KV po
     int pool_blocks, max_seqs, max_blocks_per_seq, max_batch, kv_fp16;
 } vh_load_options;
 /* ModelRuntime.LoadWeightsGGUF + CopyWeightsToDevice (runtime/loader.go:28-212, 560-700) for LLaMA-family
- * checkpoints: Q4_0 / Q8_0 / Q4_K / Q6_K projection matrices and output head go to the device as raw blocks,
- * token_embd and the norm vectors as float32 (F32, F16 or one of those four types in the file), a missing
+ * checkpoints: Q4_0 / Q8_0 / Q4_K / Q6_K / Q5_0 / Q5_K / BF16 projection matrices and output head go to the
+ * device as raw blocks, token_embd and the norm vectors as float32 (F32, F16 or one of those types in the file), a missing
  * output.weight is the embedding. One difference: a Q4_0 output head stays Q4_0 here, where the reference
  * dequantizes it to float32 at load (same values, float32 summation order aside). The model owns the device
  * copies; vh_model_destroy frees them. */
