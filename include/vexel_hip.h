@@ -223,6 +223,21 @@ int vx_sdpa_paged_tree(vx_backend *be, const float *q, const void *kv_pool, int 
                        int block_size, int num_q_heads, int num_kv_heads, int head_dim, float scale,
                        int query_len);
 
+/* Tree verification for many sequences in two launches. The query rows come in entries of
+ * vx_sdpa_paged_tree_rows_per_entry() consecutive rows (0: this geometry has no batched form); the rows of an
+ * entry belong to one tree, whose sequence is block-table row entry_table_rows[e] with entry_kv_lens[e] tokens
+ * before the tree. A tree's own keys sit at pool positions kv_len .. kv_len + n - 1 of its sequence (stored
+ * before the call). row_info: int32[rows][4] = (block-table row, kv_len, row index inside its tree, rows n of the
+ * tree); row i of a tree sees key j where tree_masks[mask_offsets[row] + i*n + j] != 0 (medusa/tree.go:186-202).
+ * Rows that only pad an entry repeat a real row. F16 pool with 16-token blocks; all arrays on the device. The
+ * context is read once per entry (not once per row); no counterpart in the reference, which verifies one path. */
+int vx_sdpa_paged_tree_rows_per_entry(int pool_is_f16, int block_size, int num_q_heads, int num_kv_heads, int head_dim);
+int vx_sdpa_paged_tree_batched(vx_backend *be, const float *q, const void *kv_pool, const int32_t *block_tables,
+                               int max_blocks, const int32_t *entry_table_rows, const int32_t *entry_kv_lens,
+                               int entries, const int32_t *row_info, const uint8_t *tree_masks,
+                               const int32_t *mask_offsets, float *out, int rows, int max_tree_rows,
+                               int num_q_heads, int num_kv_heads, int head_dim, float scale, int max_kv_len);
+
 /* Moves token rows (K and V of every KV head) inside one layer's paged pool: slot = physical block *
  * block_size + offset in the block. Chain c is the moves chain_offsets[c] .. chain_offsets[c+1]-1 (device
  * int32 arrays), applied in order, so a later move of a chain may read what an earlier one wrote; different

@@ -297,7 +297,8 @@ def test_prepared_activation_paths(be):
                                                  (nx.FMT_Q8_0, 5, 512, 1024), (nx.FMT_Q4_K, 40, 1024, 2048),
                                                  (nx.FMT_Q6_K, 32, 512, 2816), (nx.FMT_Q6_K, 3, 1024, 1024),
                                                  (nx.FMT_Q8_0, 1, 512, 1024), (nx.FMT_Q4_K, 1, 1024, 2048),
-                                                 (nx.FMT_Q6_K, 1, 1024, 2816), (nx.FMT_Q4_0, 1, 4096, 11008)])
+                                                 (nx.FMT_Q6_K, 1, 1024, 2816), (nx.FMT_Q4_0, 1, 4096, 11008),
+                                                 (nx.FMT_Q4_0, 100, 512, 1024), (nx.FMT_Q6_K, 256, 512, 1024)])
 def test_fused_decode_blocks_equal_the_unfused_sequence(be, fmt, rows, hidden, ffn):
     """vx_decode_attn_qkv / vx_decode_ffn give what the one-call-per-operation sequence of
     runtime/block.go:834-1077 gives (float32 activations, F16 and F32 pools; one row goes through the
@@ -751,6 +752,65 @@ def test_paged_multiquery_and_tree(be):
         want = nx.sdpa_paged_multiquery(q, pool, bt, None, bs, hq, hk, d, sc, tree_mask=mask, tree_base=200)
         _close(be.download(do, q.shape, np.float32), want, 1e-5, 3e-6, "tree")
         be.reset_pool()
+
+
+@pytest.mark.parametrize("hq,hk,d", [(8, 8, 128), (8, 2, 64), (16, 2, 128)])
+def test_paged_tree_batched(be, hq, hk, d):
+    """Every tree of a batch in two launches: against the oracle's masked multi-query attention per sequence and,
+    to rounding, the per-sequence entry point. Ragged contexts (one empty, one a multiple of the 512-token split),
+    trees of different sizes, entries padded with repeated rows."""
+    rng = np.random.default_rng(37)
+    bs, nblocks = 16, 160
+    rg = be._lib.vx_sdpa_paged_tree_rows_per_entry(1, bs, hq, hk, d)
+    assert rg == 8 // (hq // hk)
+    pool = _make_pool(rng, True, nblocks, bs, hk, d)
+    dpool = be.upload(pool)
+    starts = [0, 37, 512, 700]
+    parents = [[-1, -1, 0, 0, 1, 1, 2, 2, 3, 3, 4, 4, 5, 5, 6], [-1, 0, 1], [-1, -1, -1, 0, 1, 2, 3, 3, 3, 8], [-1]]
+    mb = (max(starts) + 16 + bs - 1) // bs + 1
+    perm = rng.permutation(nblocks)
+    tables = np.zeros((len(starts), mb), dtype=np.int32)
+    off = 0
+    for i, st in enumerate(starts):
+        nb = (st + len(parents[i]) + bs - 1) // bs
+        tables[i, :nb] = perm[off:off + nb]
+        off += nb
+    sc = np.float32(1 / math.sqrt(d))
+    qs, masks, info, moff, ent_rows, ent_lens, row0 = [], [], [], [], [], [], []
+    mask_bytes = 0
+    for i, par in enumerate(parents):
+        n = len(par)
+        pad = (n + rg - 1) // rg * rg
+        q = rng.standard_normal((n, hq, d)).astype(np.float32)
+        mask = np.array(hl.build_tree_attention_mask(n, par), dtype=np.uint8)
+        row0.append(sum(x.shape[0] for x in qs))
+        qs.append(np.concatenate([q, np.repeat(q[-1:], pad - n, axis=0)]))
+        for r in range(pad):
+            info.append([i, starts[i], min(r, n - 1), n])
+            moff.append(mask_bytes)
+        masks.append(mask)
+        mask_bytes += mask.size
+        ent_rows += [i] * (pad // rg)
+        ent_lens += [starts[i]] * (pad // rg)
+    qall = np.concatenate(qs)
+    rows = qall.shape[0]
+    dq, dt = be.upload(qall), be.upload(tables)
+    dm = be.upload(np.concatenate(masks))
+    do = be.alloc(qall.nbytes)
+    be.call("vx_sdpa_paged_tree_batched", dq, dpool, dt, mb, be.upload(np.array(ent_rows, dtype=np.int32)),
+            be.upload(np.array(ent_lens, dtype=np.int32)), len(ent_rows), be.upload(np.array(info, dtype=np.int32)), dm,
+            be.upload(np.array(moff, dtype=np.int32)), do, rows, max(len(p) for p in parents), hq, hk, d, sc, max(starts))
+    got = be.download(do, qall.shape, np.float32)
+    for i, par in enumerate(parents):
+        n = len(par)
+        want = nx.sdpa_paged_multiquery(qs[i][:n], pool, tables[i], None, bs, hq, hk, d, sc, tree_mask=masks[i],
+                                        tree_base=starts[i])
+        _close(got[row0[i]:row0[i] + n], want, 1e-5, 3e-6, "batched tree, sequence %d" % i)
+        one = be.alloc(n * hq * d * 4)
+        be.sdpa_paged_tree(dq + row0[i] * hq * d * 4, dpool, True, dt + i * mb * 4, one, be.upload(masks[i]), starts[i], bs,
+                           hq, hk, d, sc, n)
+        _close(got[row0[i]:row0[i] + n], be.download(one, (n, hq, d), np.float32), 1e-5, 3e-6, "against the per-sequence call")
+    be.reset_pool()
 
 
 def test_paged_kv_move_chains(be):

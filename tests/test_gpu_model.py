@@ -218,13 +218,16 @@ def test_chunked_prefill_and_verify(be):
     mr.close()
 
 
-def test_c5_tree_verification_batched(be):
+@pytest.mark.parametrize("kv_heads,max_nodes", [(8, 15), (2, 10)])
+def test_c5_tree_verification_batched(be, kv_heads, max_nodes):
     """BASELINE config 5 at oracle size: Q6_K weights, several sequences at ragged contexts, a 15-node candidate
     tree (4 heads x top-2) per sequence verified in one pass under tree masks over the paged f16 pool, greedy
-    acceptance, rollback in the block tables; two rounds, the second on top of the first one's rollback."""
+    acceptance, rollback in the block tables; two rounds, the second on top of the first one's rollback.
+    Second case: grouped-query heads and 11-row trees, which do not fill the attention's entries of query rows."""
     import copy
     from oracle import host_logic as hl
-    cfg = om.ModelConfig(num_layers=2, hidden=1024, num_heads=8, num_kv_heads=8, head_dim=128, ffn=2816, vocab=4096)
+    cfg = om.ModelConfig(num_layers=2, hidden=1024, num_heads=8, num_kv_heads=kv_heads, head_dim=128, ffn=2816,
+                         vocab=4096)
     ctx = [291, 256, 517, 333]     # 256: the input token opens a new block
     omodel, mr, rng = _ragged_setup(be, cfg, nx.FMT_Q6_K, nx.FMT_Q6_K, ctx, 41, pool_blocks=160)
     ids = [100 + i for i in range(4)]
@@ -247,7 +250,7 @@ def test_c5_tree_verification_batched(be):
                 toks[h][(h + 1) % 2] = t
                 if toks[h][0] == toks[h][1]:
                     toks[h][h % 2] = (t + 1) % cfg.vocab
-            tree = hl.build_candidate_tree_from_topk(toks, [[2.0, 1.0]] * 4, 15)
+            tree = hl.build_candidate_tree_from_topk(toks, [[2.0, 1.0]] * 4, max_nodes)
             trees.append(tree.linearize())
         want = omodel.tree_step_batched(inputs, trees, ids, start)
         acc, fin, logits = mr.verify_tree(ids, inputs, start, trees)
@@ -257,7 +260,8 @@ def test_c5_tree_verification_batched(be):
             assert mr.seq_len(sid) == omodel.pool.seqs[sid].seq_len == start[i] + 1 + len(acc[i])
             assert mr.block_table(sid) == omodel.pool.seqs[sid].block_tables[0]
             moved += sum(1 for k, node in enumerate(acc[i]) if node != k)
-        assert len(acc[0]) >= 3 and len(acc[2]) >= 1
+        # (a 10-node tree stops inside its third level: the planted branch may end after two)
+        assert len(acc[0]) >= (3 if max_nodes == 15 else 2) and len(acc[2]) >= 1
         assert mr.block_stats()[1] == omodel.pool.block_stats()[1]
         inputs = list(fin)
         start = [start[i] + 1 + len(acc[i]) for i in range(4)]

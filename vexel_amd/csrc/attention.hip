@@ -192,12 +192,15 @@ __device__ __forceinline__ float token_sum(float t) {
     return t;
 }
 
-template <int D, int G>
+// RG > 1: an entry of the batch is RG consecutive query rows that share one sequence's context (the rows of a
+// candidate tree): the workgroup serves the G*RG queries (row, head) of its kv head from one pass over the K/V.
+template <int D, int G, int RG = 1>
 __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix,
     const int32_t *__restrict__ bt_rows, int max_blocks, const int32_t *__restrict__ kv_lens,
     float *__restrict__ partial, int num_q_heads, int num_kv_heads, float scale, int max_splits,
     const int32_t *__restrict__ items) {
+    constexpr int GG = G * RG;       // queries per K/V row
     constexpr int LPT = D / 8;       // lanes per token
     constexpr int TPI = 64 / LPT;    // tokens per load instruction
     constexpr int NL = HOT_BS / TPI; // load instructions per block and per K or V
@@ -229,17 +232,17 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     const size_t lane_off = (size_t)tl * hs + (size_t)kvh * D + dl * 8;
 
     // query slices, pre-multiplied by scale*log2(e) so scores are in the exp2 domain
-    float qf[G][8];
+    float qf[GG][8];
     const float qs = scale * kLog2e;
 #pragma unroll
-    for (int g = 0; g < G; g++) {
-        const float *qp = q + ((size_t)seq * num_q_heads + (size_t)kvh * G + g) * D + dl * 8;
+    for (int g = 0; g < GG; g++) {
+        const float *qp = q + (((size_t)seq * RG + g / G) * num_q_heads + (size_t)kvh * G + g % G) * D + dl * 8;
 #pragma unroll
         for (int e = 0; e < 8; e++) qf[g][e] = qp[e] * qs;
     }
-    float acc[G][8], m_run[G], l_run[G];
+    float acc[GG][8], m_run[GG], l_run[GG];
 #pragma unroll
-    for (int g = 0; g < G; g++) {
+    for (int g = 0; g < GG; g++) {
         m_run[g] = -INFINITY;
         l_run[g] = 0.f;
 #pragma unroll
@@ -268,7 +271,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
         __builtin_amdgcn_sched_barrier(0);
         const int tok0 = t_begin + bi * HOT_BS + tl;
 #pragma unroll
-        for (int g = 0; g < G; g++) {
+        for (int g = 0; g < GG; g++) {
             float s[NL];
             float gm = -INFINITY;
 #pragma unroll
@@ -306,7 +309,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
 
     // combine token slots inside the wave (m is already wave-uniform per g)
 #pragma unroll
-    for (int g = 0; g < G; g++) {
+    for (int g = 0; g < GG; g++) {
 #pragma unroll
         for (int off = LPT; off < 64; off <<= 1) {
             l_run[g] += __shfl_xor(l_run[g], off, 64);
@@ -316,11 +319,11 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     }
 
     // combine the 4 waves through LDS
-    __shared__ float s_m[4][G], s_l[4][G];
-    __shared__ float s_acc[4][G][D];
+    __shared__ float s_m[4][GG], s_l[4][GG];
+    __shared__ float s_acc[4][GG][D];
     if (tl == 0) {
 #pragma unroll
-        for (int g = 0; g < G; g++) {
+        for (int g = 0; g < GG; g++) {
 #pragma unroll
             for (int e = 0; e < 8; e++) s_acc[wave][g][dl * 8 + e] = acc[g][e];
             if (dl == 0) {
@@ -330,7 +333,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
         }
     }
     __syncthreads();
-    for (int idx = tid; idx < G * D; idx += 256) {
+    for (int idx = tid; idx < GG * D; idx += 256) {
         const int g = idx / D, d = idx % D;
         float M = fmaxf(fmaxf(s_m[0][g], s_m[1][g]), fmaxf(s_m[2][g], s_m[3][g]));
         float L = 0.f, A = 0.f;
@@ -340,8 +343,8 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
             L += s_l[w][g] * f;
             A += s_acc[w][g][d] * f;
         }
-        const int qh = kvh * G + g;
-        float *po = partial + (((size_t)seq * num_q_heads + qh) * max_splits + split) * (D + 2);
+        const int qh = kvh * G + g % G;
+        float *po = partial + ((((size_t)seq * RG + g / G) * num_q_heads + qh) * max_splits + split) * (D + 2);
         po[2 + d] = A;
         if (d == 0) {
             po[0] = M;
@@ -378,6 +381,64 @@ __global__ void __launch_bounds__(D) paged_merge_kernel(const float *__restrict_
         A += ps[2 + d] * f;
     }
     out[((size_t)seq * num_q_heads + qh) * D + d] = (L > 0.f) ? A / L : 0.f;
+}
+
+// The rows of candidate trees: query row `row` of head qh has its context (pool positions < start, read by
+// paged_decode_f16_kernel<D, G, RG>) as split partials; this adds the tree's own keys, which sit at pool positions
+// start .. start + n - 1 of the same sequence and are visible where the row's mask says so (medusa/tree.go:186-202),
+// and normalises. info[row] = (block-table row, start, row index inside its tree, rows of the tree);
+// grid = (num_q_heads, rows); block = D threads.
+template <int D>
+__global__ void __launch_bounds__(D) tree_merge_kernel(const float *__restrict__ partial, const float *__restrict__ q,
+                                                       const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix,
+                                                       int max_blocks, const int4 *__restrict__ info,
+                                                       const uint8_t *__restrict__ masks, const int32_t *__restrict__ mask_off,
+                                                       float *__restrict__ out, int num_q_heads, int num_kv_heads, float scale,
+                                                       int max_splits) {
+    constexpr int MAXN = 64;  // rows of one tree (checked on the host)
+    const int qh = blockIdx.x, row = blockIdx.y, d = threadIdx.x;
+    const int4 inf = info[row];
+    const int start = inf.y, r = inf.z, n = inf.w;
+    const int kvh = qh / (num_q_heads / num_kv_heads);
+    const int32_t *bt = bt_matrix + (size_t)inf.x * max_blocks;
+    const uint8_t *mk = masks + mask_off[row] + (size_t)r * n;
+    const size_t hs = (size_t)num_kv_heads * D, part = (size_t)HOT_BS * hs;
+    __shared__ float s_q[D];
+    __shared__ float s_s[MAXN];
+    s_q[d] = q[((size_t)row * num_q_heads + qh) * D + d] * (scale * kLog2e);
+    __syncthreads();
+    if (d < n) {  // one key per thread: its score in the exp2 domain, -inf where the mask hides it
+        float t = -INFINITY;
+        if (mk[d]) {
+            const int pos = start + d;
+            const _Float16 *kp = pool + (size_t)bt[pos / HOT_BS] * 2 * part + (size_t)(pos % HOT_BS) * hs + (size_t)kvh * D;
+            t = 0.f;
+            for (int e = 0; e < D; e++) t = fmaf(s_q[e], (float)kp[e], t);
+        }
+        s_s[d] = t;
+    }
+    __syncthreads();
+    const int ns = (start + TPW - 1) / TPW;
+    const float *pb = partial + ((size_t)row * num_q_heads + qh) * max_splits * (D + 2);
+    float M = -INFINITY;
+    for (int s = 0; s < ns; s++) M = fmaxf(M, pb[(size_t)s * (D + 2)]);
+    for (int j = 0; j < n; j++) M = fmaxf(M, s_s[j]);
+    float L = 0.f, A = 0.f;
+    for (int s = 0; s < ns; s++) {
+        const float *ps = pb + (size_t)s * (D + 2);
+        const float f = exp2f(ps[0] - M);
+        L += ps[1] * f;
+        A += ps[2 + d] * f;
+    }
+    for (int j = 0; j < n; j++) {
+        if (s_s[j] == -INFINITY) continue;
+        const int pos = start + j;
+        const _Float16 *vp = pool + (size_t)bt[pos / HOT_BS] * 2 * part + part + (size_t)(pos % HOT_BS) * hs + (size_t)kvh * D;
+        const float f = exp2f(s_s[j] - M);
+        L += f;
+        A = fmaf(f, (float)vp[d], A);
+    }
+    out[((size_t)row * num_q_heads + qh) * D + d] = (L > 0.f) ? A / L : 0.f;
 }
 
 // --------------------------------------------------------------------------------------------
@@ -806,6 +867,66 @@ int vx_sdpa_paged_tree(vx_backend *be, const float *q, const void *kv_pool, int 
     p.tree_base = tree_base;
     p.query_len = query_len;
     return run_generic(be, p, query_len);
+}
+
+int vx_sdpa_paged_tree_rows_per_entry(int pool_is_f16, int block_size, int num_q_heads, int num_kv_heads, int head_dim) {
+    if (!pool_is_f16 || block_size != HOT_BS || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0) return 0;
+    if (head_dim != 128 && head_dim != 64) return 0;
+    const int G = num_q_heads / num_kv_heads;
+    return (G == 1 || G == 2 || G == 4 || G == 8) ? 8 / G : 0;
+}
+
+int vx_sdpa_paged_tree_batched(vx_backend *be, const float *q, const void *kv_pool, const int32_t *block_tables,
+                               int max_blocks, const int32_t *entry_table_rows, const int32_t *entry_kv_lens, int entries,
+                               const int32_t *row_info, const uint8_t *tree_masks, const int32_t *mask_offsets, float *out,
+                               int rows, int max_tree_rows, int num_q_heads, int num_kv_heads, int head_dim, float scale,
+                               int max_kv_len) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && kv_pool && block_tables && entry_table_rows && entry_kv_lens && row_info && tree_masks && mask_offsets && out,
+               "vx_sdpa_paged_tree_batched: null pointer");
+    const int rg = vx_sdpa_paged_tree_rows_per_entry(1, HOT_BS, num_q_heads, num_kv_heads, head_dim);
+    if (rg == 0) {
+        set_error("vx_sdpa_paged_tree_batched: head geometry %d/%d x %d has no batched form", num_q_heads, num_kv_heads, head_dim);
+        return VX_ERR_UNSUPPORTED;
+    }
+    VX_REQUIRE(entries >= 0 && rows == entries * rg, "vx_sdpa_paged_tree_batched: %d rows are not %d entries of %d rows", rows,
+               entries, rg);
+    VX_REQUIRE(max_tree_rows >= 1 && max_tree_rows <= 64 && max_tree_rows <= head_dim,
+               "vx_sdpa_paged_tree_batched: a tree of %d rows (at most 64)", max_tree_rows);
+    VX_REQUIRE(((uintptr_t)kv_pool % 16) == 0 && max_kv_len >= 0, "vx_sdpa_paged_tree_batched: bad pool alignment / length");
+    if (rows == 0) return VX_OK;
+    const int max_splits = max_kv_len > 0 ? ceil_div(max_kv_len, TPW) : 1;
+    const size_t need = (size_t)rows * num_q_heads * max_splits * (head_dim + 2) * sizeof(float);
+    rc = ensure_ws(be, &be->attn_ws, &be->attn_ws_bytes, need, "attention");
+    if (rc) return rc;
+    be->split.batch = 0;
+    const _Float16 *pool = (const _Float16 *)kv_pool;
+    float *ws = (float *)be->attn_ws;
+    const int G = num_q_heads / num_kv_heads;
+    const dim3 grid(num_kv_heads, max_splits, entries);
+    if (max_kv_len > 0) {
+#define VX_TREE(DD, GG, RR)                                                                                              \
+    if (head_dim == DD && G == GG)                                                                                        \
+        paged_decode_f16_kernel<DD, GG, RR><<<grid, 256, 0, be->stream>>>(q, pool, block_tables, entry_table_rows, max_blocks, \
+                                                                        entry_kv_lens, ws, num_q_heads, num_kv_heads, scale, \
+                                                                        max_splits, nullptr);
+        VX_TREE(128, 1, 8) VX_TREE(128, 2, 4) VX_TREE(128, 4, 2) VX_TREE(128, 8, 1)
+        VX_TREE(64, 1, 8) VX_TREE(64, 2, 4) VX_TREE(64, 4, 2) VX_TREE(64, 8, 1)
+#undef VX_TREE
+        VX_CHECK_LAUNCH();
+    }
+    const dim3 mgrid(num_q_heads, rows);
+    if (head_dim == 128)
+        tree_merge_kernel<128><<<mgrid, 128, 0, be->stream>>>(ws, q, pool, block_tables, max_blocks, (const int4 *)row_info,
+                                                             tree_masks, mask_offsets, out, num_q_heads, num_kv_heads, scale,
+                                                             max_splits);
+    else
+        tree_merge_kernel<64><<<mgrid, 64, 0, be->stream>>>(ws, q, pool, block_tables, max_blocks, (const int4 *)row_info,
+                                                           tree_masks, mask_offsets, out, num_q_heads, num_kv_heads, scale,
+                                                           max_splits);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
 }
 
 }  // extern "C"

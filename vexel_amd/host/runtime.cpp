@@ -722,13 +722,22 @@ int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_
     if (n_seqs == 0) return VH_OK;
     VHC(check_ready(m));
     const vh_config &c = m->cfg;
-    struct SeqRows { int row0, rows, node0, start, slot; };
+    struct SeqRows { int row0, rows, node0, start, slot, pad; };
     std::vector<SeqRows> sr(n_seqs);
-    int total = 0, nodes_total = 0;
+    int total = 0, nodes_total = 0, max_rows = 1;
     for (int i = 0; i < n_seqs; i++) {
         if (n_nodes[i] < 0 || start_pos[i] < 0) return fail("sequence %d: bad counts", i);
-        sr[i] = {total, 1 + n_nodes[i], nodes_total, start_pos[i], -1};
-        total += 1 + n_nodes[i];
+        max_rows = std::max(max_rows, 1 + n_nodes[i]);
+    }
+    // With the batched tree attention a sequence's rows fill whole entries of `rg` rows: the rows that pad the
+    // last entry repeat the sequence's last row (same token, position and pool slot), their results are dropped.
+    static const bool per_sequence = getenv("VEXEL_HIP_TREE_PER_SEQUENCE") != nullptr;
+    const int rg0 = vx_sdpa_paged_tree_rows_per_entry(c.kv_fp16, c.block_size, c.num_heads, c.num_kv_heads, c.head_dim);
+    const int rg = (rg0 > 0 && max_rows <= 64 && max_rows <= c.head_dim && !per_sequence) ? rg0 : 0;
+    for (int i = 0; i < n_seqs; i++) {
+        const int rows = 1 + n_nodes[i], pad = rg ? (rows + rg - 1) / rg * rg : rows;
+        sr[i] = {total, rows, nodes_total, start_pos[i], -1, pad};
+        total += pad;
         nodes_total += n_nodes[i];
     }
     if (nodes_total > 0 && (!node_tokens || !parent_idx || !accepted_nodes)) return fail("null node arrays");
@@ -776,6 +785,11 @@ int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_
                 pos[q.row0 + r] = q.start + depth[r];
                 slot_map[q.row0 + r] = s->table[p / c.block_size] * c.block_size + p % c.block_size;  // :250-252
             }
+            for (int r = q.rows; r < q.pad; r++) {
+                tok[q.row0 + r] = tok[q.row0 + q.rows - 1];
+                pos[q.row0 + r] = pos[q.row0 + q.rows - 1];
+                slot_map[q.row0 + r] = slot_map[q.row0 + q.rows - 1];
+            }
             s->seq_len = q.start + q.rows;
             sr[i].slot = s->slot;
         }
@@ -798,34 +812,97 @@ int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_
     VXC(vx_to_device(be, d_pos, pos.data(), (size_t)n * 4));
     VXC(vx_to_device(be, d_slot, slot_map.data(), (size_t)n * 4));
     VXC(vx_to_device(be, d_mask, mask.data(), mask.size()));
-    VXC(vx_embedding(be, d_tok, n, m->embedding, x, c.vocab, c.hidden));
-    const float scale = (float)(1.0 / sqrt((double)c.head_dim));
-    for (int l = 0; l < c.num_layers; l++) {
-        const vh_layer_weights &w = m->layers[l];
-        bool prep;
-        const vh_qweight *qkv[3] = {&w.wq, &w.wk, &w.wv};
-        VHC(norm_for(m, x, w.attn_norm, norm, n, qkv, 3, &prep));
-        VHC(mm(m, prep, norm, w.wq, q, nullptr, n));
-        VHC(mm(m, prep, norm, w.wk, k, nullptr, n));
-        VHC(mm(m, prep, norm, w.wv, v, nullptr, n));
-        VXC(vx_rope_store_paged(be, q, k, v, d_pos, d_slot, m->kv[l], c.kv_fp16, n, c.num_heads, c.num_kv_heads,
-                                c.head_dim, c.block_size, c.rope_theta));
+    int32_t *d_ent_rows = nullptr, *d_ent_lens = nullptr, *d_info = nullptr, *d_moff = nullptr;
+    int entries = 0, max_start = 0;
+    if (rg) {
+        std::vector<int32_t> ent_rows, ent_lens, info((size_t)n * 4), moff(n);
         for (int i = 0; i < n_seqs; i++) {
             const SeqRows &s = sr[i];
-            VXC(vx_sdpa_paged_tree(be, q + s.row0 * qd, m->kv[l], c.kv_fp16, m->d_tables + (size_t)s.slot * c.max_blocks_per_seq,
-                                   attn + s.row0 * qd, d_mask + mask_off[i], s.start, c.block_size, c.num_heads,
-                                   c.num_kv_heads, c.head_dim, scale, s.rows));
+            max_start = std::max(max_start, s.start);
+            for (int e = 0; e < s.pad / rg; e++) {
+                ent_rows.push_back(s.slot);
+                ent_lens.push_back(s.start);
+            }
+            for (int r = 0; r < s.pad; r++) {
+                int32_t *f = &info[(size_t)(s.row0 + r) * 4];
+                f[0] = s.slot, f[1] = s.start, f[2] = std::min(r, s.rows - 1), f[3] = s.rows;
+                moff[s.row0 + r] = (int32_t)mask_off[i];
+            }
         }
-        VHC(layer_tail(m, w, x, norm, attn, gate, up, n));
+        entries = (int)ent_rows.size();
+        d_ent_rows = ia(entries), d_ent_lens = ia(entries), d_info = ia((size_t)n * 4), d_moff = ia(n);
+        if (!d_ent_rows || !d_ent_lens || !d_info || !d_moff) return fail("verification buffers: %s", vx_last_error());
+        VXC(vx_to_device(be, d_ent_rows, ent_rows.data(), (size_t)entries * 4));
+        VXC(vx_to_device(be, d_ent_lens, ent_lens.data(), (size_t)entries * 4));
+        VXC(vx_to_device(be, d_info, info.data(), (size_t)n * 16));
+        VXC(vx_to_device(be, d_moff, moff.data(), (size_t)n * 4));
     }
-    bool prep;
-    const vh_qweight *hw[1] = {&m->lm_head};
-    VHC(norm_for(m, x, m->final_norm, norm, n, hw, 1, &prep));
-    VHC(mm(m, prep, norm, m->lm_head, logits, nullptr, n));
+    VXC(vx_embedding(be, d_tok, n, m->embedding, x, c.vocab, c.hidden));
+    const float scale = (float)(1.0 / sqrt((double)c.head_dim));
+    // the layers as in forward_decode: fused projection groups where the weights allow them, each fused tail
+    // leaving the next norm's activation prepared
+    const bool head_prepared = n > 1 && m->fused && fast(m->lm_head) && c.hidden % 256 == 0;
+    bool chained = false;
+    for (int l = 0; l < c.num_layers; l++) {
+        const vh_layer_weights &w = m->layers[l];
+        if (attn_fusable(m, l)) {
+            VXC(vx_decode_attn_qkv(be, x, w.attn_norm, c.eps, chained ? 1 : 0, &w.wq, &w.wk, &w.wv, n, d_pos, d_slot, m->kv[l],
+                                   c.kv_fp16, c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta, q));
+        } else {
+            if (chained) return fail("internal: prepared activation handed to an unfused layer");
+            bool prep;
+            const vh_qweight *qkv[3] = {&w.wq, &w.wk, &w.wv};
+            VHC(norm_for(m, x, w.attn_norm, norm, n, qkv, 3, &prep));
+            VHC(mm(m, prep, norm, w.wq, q, nullptr, n));
+            VHC(mm(m, prep, norm, w.wk, k, nullptr, n));
+            VHC(mm(m, prep, norm, w.wv, v, nullptr, n));
+            VXC(vx_rope_store_paged(be, q, k, v, d_pos, d_slot, m->kv[l], c.kv_fp16, n, c.num_heads, c.num_kv_heads,
+                                    c.head_dim, c.block_size, c.rope_theta));
+        }
+        if (rg) {  // every tree in two launches, each sequence's context read once per entry of rg rows
+            VXC(vx_sdpa_paged_tree_batched(be, q, m->kv[l], m->d_tables, c.max_blocks_per_seq, d_ent_rows, d_ent_lens, entries,
+                                           d_info, d_mask, d_moff, attn, n, max_rows, c.num_heads, c.num_kv_heads, c.head_dim,
+                                           scale, max_start));
+        } else {
+            for (int i = 0; i < n_seqs; i++) {
+                const SeqRows &s = sr[i];
+                VXC(vx_sdpa_paged_tree(be, q + s.row0 * qd, m->kv[l], c.kv_fp16,
+                                       m->d_tables + (size_t)s.slot * c.max_blocks_per_seq, attn + s.row0 * qd,
+                                       d_mask + mask_off[i], s.start, c.block_size, c.num_heads, c.num_kv_heads, c.head_dim,
+                                       scale, s.rows));
+            }
+        }
+        chained = false;
+        const bool ffn_fused = m->fused && n > 1 && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
+                               vx_decode_ffn_supported(&w.wo, &w.w1, &w.w3, &w.w2);
+        if (ffn_fused) {
+            const float *next_norm = l + 1 < c.num_layers ? (attn_fusable(m, l + 1) ? m->layers[l + 1].attn_norm : nullptr)
+                                                          : (head_prepared ? m->final_norm : nullptr);
+            VXC(vx_decode_ffn(be, attn, x, &w.wo, w.ffn_norm, c.eps, &w.w1, &w.w3, &w.w2, n, next_norm));
+            chained = next_norm != nullptr;
+        } else {
+            VHC(layer_tail(m, w, x, norm, attn, gate, up, n));
+        }
+    }
+    if (chained) {
+        VHC(mm(m, true, nullptr, m->lm_head, logits, nullptr, n));
+    } else {
+        bool prep;
+        const vh_qweight *hw[1] = {&m->lm_head};
+        VHC(norm_for(m, x, m->final_norm, norm, n, hw, 1, &prep));
+        VHC(mm(m, prep, norm, m->lm_head, logits, nullptr, n));
+    }
     VXC(vx_argmax_rows(be, logits, n, c.vocab, d_am));
     std::vector<int32_t> am(n);
     VXC(vx_to_host(be, am.data(), d_am, (size_t)n * 4));
-    if (logits_out) VXC(vx_to_host(be, logits_out, logits, (size_t)n * c.vocab * 4));
+    if (logits_out) {
+        size_t out_row = 0;
+        for (int i = 0; i < n_seqs; i++) {  // the real rows of each sequence
+            VXC(vx_to_host(be, logits_out + out_row * c.vocab, logits + (size_t)sr[i].row0 * c.vocab,
+                           (size_t)sr[i].rows * c.vocab * 4));
+            out_row += sr[i].rows;
+        }
+    }
     VXC(vx_sync(be));
 
     // greedy acceptance per sequence, then the moves that make each accepted path contiguous
