@@ -251,6 +251,15 @@ int vx_paged_kv_move(vx_backend *be, void *kv_pool, int pool_is_f16, const int32
 /* Row-wise argmax on the device: out_idx[r] = ArgmaxOps.Argmax(logits + r*n, n). No wait. */
 int vx_argmax_rows(vx_backend *be, const float *logits, int rows, int n, int32_t *out_idx);
 
+/* Sampler.Sample (pkg/sampler/sampler.go:48-204) for every row of logits[rows, n] on the device: temperature
+ * scaling, softmax, top-k (0 or >= n: off), top-p (<= 0 or >= 1: off) and the draw, with the row's uniform number
+ * in [0, 1) given by the caller in place of the reference's rand.Float32(). temperature 0 is Argmax. All sums are
+ * float32 in the reference's order, so the token is the reference's for the same draw; among equal probabilities
+ * at the nucleus boundary the lower index stays (the reference's sort leaves that open). All arrays on the device;
+ * out_idx int32[rows]. No wait. */
+int vx_sample_rows(vx_backend *be, const float *logits, int rows, int n, const float *temperature,
+                   const int32_t *top_k, const float *top_p, const float *uniform, int32_t *out_idx);
+
 /* Continuous-batching step metadata built on the device by prefix scans
  * (host restatement: scheduler/scheduler.go:290-303 + runtime/gpu_block_pool.go:234-252,
  * 359-363). Inputs (device int32): seq_slots[batch] = row of each sequence in the

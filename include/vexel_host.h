@@ -82,6 +82,11 @@ int vh_pool_device_matches_host(vh_model *m);
  * logits_out: host [batch,vocab] or NULL; argmax_out: host [batch] or NULL. */
 int vh_decode_batched(vh_model *m, const int32_t *tokens, const int64_t *seq_ids, const int32_t *positions,
                       int batch, float *logits_out, int32_t *argmax_out);
+/* Sampler.Sample (pkg/sampler/sampler.go:48-77) on the device for the `rows` rows of logits the last
+ * vh_decode_batched left there, one (temperature, top_k, top_p, uniform draw in [0, 1)) per row from host arrays;
+ * temperature 0 is the greedy choice. tokens_out: host int32[rows]. */
+int vh_sample_last_logits(vh_model *m, int rows, const float *temperature, const int32_t *top_k, const float *top_p,
+                          const float *uniform, int32_t *tokens_out);
 /* Speculative verification of a whole candidate tree for each of n_seqs sequences in one forward pass, greedy
  * acceptance and rollback. The reference's runTreeMedusaDecodeStep (scheduler/medusa_scheduler.go:733-861)
  * handles one sequence and verifies only the most confident path with VerifySpeculativeWithPagedKV

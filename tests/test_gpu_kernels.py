@@ -813,6 +813,36 @@ def test_paged_tree_batched(be, hq, hk, d):
     be.reset_pool()
 
 
+def test_sample_rows_matches_the_reference_sampler(be):
+    """Sampler.Sample (pkg/sampler/sampler.go:48-204) on the device against its restatement with the same uniform
+    draws: greedy rows, plain temperature sampling, top-k, top-p and both, flat and peaked distributions, draws at
+    both ends of [0, 1), equal probabilities at the cut-offs, a vocabulary that is not a power of two."""
+    rng = np.random.default_rng(38)
+    n = 3001
+    cases = []
+    for temp, k, p in [(0.0, 0, 0.0), (1.0, 0, 0.0), (0.7, 40, 0.0), (0.7, 0, 0.9), (1.3, 50, 0.95), (0.5, 1, 0.0),
+                       (1.0, n, 1.0), (1.0, 5, 0.5), (2.0, 0, 0.999), (0.1, 0, 0.3), (1.0, 300, 0.2)]:
+        for r in (float(rng.random()), 0.0, 0.99999994):
+            cases.append((temp, k, p, r))
+    rows = len(cases)
+    logits = (rng.standard_normal((rows, n)) * rng.choice([0.2, 1.0, 4.0], size=(rows, 1))).astype(np.float32)
+    logits[3, 100:140] = logits[3, 100]                     # runs of equal logits: ties at the top-k / top-p cuts
+    logits[9, :] = 0.25
+    logits[12, 7] = logits[12, 2000] = logits[12].max() + 1
+    logits[20, 500:2500] = logits[20, 499]
+    temp = np.array([c[0] for c in cases], dtype=np.float32)
+    topk = np.array([c[1] for c in cases], dtype=np.int32)
+    topp = np.array([c[2] for c in cases], dtype=np.float32)
+    uni = np.array([c[3] for c in cases], dtype=np.float32)
+    out = be.alloc(rows * 4)
+    be.sample_rows(be.upload(logits), rows, n, be.upload(temp), be.upload(topk), be.upload(topp), be.upload(uni), out)
+    got = be.download(out, (rows,), np.int32)
+    want = [hl.sampler_sample(logits[i], float(temp[i]), int(topk[i]), float(topp[i]), float(uni[i])) for i in range(rows)]
+    assert got.tolist() == want
+    assert len(set(want)) > rows // 3                        # the cases do pick different tokens
+    be.reset_pool()
+
+
 def test_paged_kv_move_chains(be):
     """Rows move inside the pool in chain order: a later move of a chain reads what an earlier one wrote."""
     rng = np.random.default_rng(36)

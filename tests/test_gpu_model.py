@@ -377,7 +377,8 @@ def test_scheduler_loop_matches_oracle(be, chunk):
     join at different steps; at most four run per step; one stops on the EOS token, the others on their own or
     the scheduler's length limit; finished sequences are removed and their blocks return to the pool. After every
     step the C++ scheduler and its oracle restatement over the CPU model agree on every sequence's state, position
-    and generated tokens; at the end on block tables and pool statistics. chunk = 16 feeds prompts in pieces."""
+    and generated tokens; at the end on block tables and pool statistics. chunk = 16 feeds prompts in pieces.
+    Two of the requests sample (temperature, top-k, top-p) from the same uniform stream on both sides."""
     from oracle import host_logic as hl
     from vexel_amd.runtime import Scheduler
     cfg = om.ModelConfig(num_layers=2, hidden=512, num_heads=8, num_kv_heads=2, head_dim=64, ffn=1024, vocab=1024)
@@ -398,10 +399,15 @@ def test_scheduler_loop_matches_oracle(be, chunk):
     want = hl.Scheduler(omodel, 4, 14, eos, chunk)
     got = Scheduler(mr, 4, max_tokens=14, eos_token=eos, prefill_chunk=chunk)
     finished_at = {}
+    # two requests are sampled (in decode steps on the device, after their prompt on the host), the others greedy
+    sampled = {13: (0.8, 20, 0.95, 1234), 15: (1.1, 0, 0.9, 99)}
     for step in range(40):
         for i in arrivals.get(step, []):
             want.add_sequence(i, prompts[i], limits[i])
             got.add_sequence(i, prompts[i], limits[i])
+            if i in sampled:          # same parameters and the same uniform stream on both sides
+                want.seqs[i].sampling = sampled[i]
+                got.set_sampling(i, *sampled[i])
         nw, ng = want.step(), got.step()
         assert nw == ng, "tokens produced in step %d" % step
         for i, q in want.seqs.items():

@@ -266,6 +266,9 @@ class HipBackend:
         self.call("vx_sdpa_paged_tree", q, kv_pool, int(bool(pool_is_f16)), block_table, out, tree_mask,
                   tree_base, block_size, num_q_heads, num_kv_heads, head_dim, scale, query_len)
 
+    def sample_rows(self, logits, rows, n, temperature, top_k, top_p, uniform, out_idx):
+        self.call("vx_sample_rows", logits, rows, n, temperature, top_k, top_p, uniform, out_idx)
+
     def paged_kv_move(self, kv_pool, pool_is_f16, chain_offsets, src_slots, dst_slots, num_chains, num_kv_heads,
                       head_dim, block_size):
         self.call("vx_paged_kv_move", kv_pool, int(bool(pool_is_f16)), chain_offsets, src_slots, dst_slots,

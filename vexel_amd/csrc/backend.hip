@@ -98,6 +98,7 @@ void vx_backend_destroy(vx_backend *be) {
     if (be->gemm_ws) (void)hipFree(be->gemm_ws);
     if (be->part_ws) (void)hipFree(be->part_ws);
     if (be->attn_ws) (void)hipFree(be->attn_ws);
+    if (be->sample_ws) (void)hipFree(be->sample_ws);
     if (be->items.buf) (void)hipFree(be->items.buf);
     if (be->misc_ws) (void)hipFree(be->misc_ws);
     if (be->prep_sync) (void)hipFree(be->prep_sync);

@@ -90,6 +90,8 @@ struct vx_backend {
         bool valid = false;
     } items;
     float *ones = nullptr;       // 64 floats of 1.0 on the device (row factors of an unscaled activation)
+    void *sample_ws = nullptr;   // probabilities and sort keys of vx_sample_rows
+    size_t sample_ws_bytes = 0;
     void *misc_ws = nullptr;     // small device staging (pointer tables, argmax result)
     size_t misc_ws_bytes = 0;
     void *host_stage = nullptr;  // pinned host staging

@@ -627,6 +627,27 @@ int vh_decode_batched(vh_model *m, const int32_t *tokens, const int64_t *seq_ids
     return VH_OK;
 }
 
+// Sampler.Sample (pkg/sampler/sampler.go:48-77) for the rows of the last decode step, on the device.
+int vh_sample_last_logits(vh_model *m, int rows, const float *temperature, const int32_t *top_k, const float *top_p,
+                          const float *uniform, int32_t *tokens_out) {
+    if (!m || rows < 0 || !temperature || !top_k || !top_p || !uniform || !tokens_out) return fail("bad arguments");
+    if (rows == 0) return VH_OK;
+    if (rows > m->cfg.max_batch) return fail("%d rows exceed max_batch %d", rows, m->cfg.max_batch);
+    vx_backend *be = m->be;
+    float *d_t = (float *)vx_alloc(be, (size_t)rows * 4), *d_p = (float *)vx_alloc(be, (size_t)rows * 4);
+    float *d_u = (float *)vx_alloc(be, (size_t)rows * 4);
+    int32_t *d_k = (int32_t *)vx_alloc(be, (size_t)rows * 4), *d_out = (int32_t *)vx_alloc(be, (size_t)rows * 4);
+    if (!d_t || !d_p || !d_u || !d_k || !d_out) return fail("sampling buffers: %s", vx_last_error());
+    VXC(vx_to_device(be, d_t, temperature, (size_t)rows * 4));
+    VXC(vx_to_device(be, d_k, top_k, (size_t)rows * 4));
+    VXC(vx_to_device(be, d_p, top_p, (size_t)rows * 4));
+    VXC(vx_to_device(be, d_u, uniform, (size_t)rows * 4));
+    VXC(vx_sample_rows(be, m->logits, rows, m->cfg.vocab, d_t, d_k, d_p, d_u, d_out));
+    VXC(vx_to_host(be, tokens_out, d_out, (size_t)rows * 4));
+    VXC(vx_sync(be));
+    return VH_OK;
+}
+
 // ------------------------------------------------------------------ prefill / verify of one sequence
 int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int start_pos, int all_logits,
                float *logits_out) {

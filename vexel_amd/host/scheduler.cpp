@@ -13,7 +13,8 @@
 //    the reference only forgets it (scheduler.go:182-187), after which RemoveSequence cannot find it any more.
 //  * Sampled requests draw their uniform numbers from a SplitMix64 stream seeded per sequence, not from Go's
 //    math/rand (whose generator table is no part of the reference's tree). Greedy requests (temperature 0) use the
-//    device argmax and never move logits to the host.
+//    device argmax; in decode steps sampled requests are sampled on the device too (vh_sample_last_logits, the
+//    same sums in the same order), so logits move to the host only for the token that follows a prompt.
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
@@ -300,15 +301,22 @@ int vh_sched_step(vh_scheduler *s, int *tokens_out) {
     if (!ids.empty()) {
         const int b = (int)ids.size();
         std::vector<int32_t> am((size_t)b);
-        if (need_logits) s->logits.resize((size_t)b * V);
-        if (vh_decode_batched(s->m, tokens.data(), ids.data(), positions.data(), b, need_logits ? s->logits.data() : nullptr,
-                              am.data()) != VH_OK)
-            return VH_ERR;
+        if (vh_decode_batched(s->m, tokens.data(), ids.data(), positions.data(), b, nullptr, am.data()) != VH_OK) return VH_ERR;
+        if (need_logits) {  // sampled requests: the sampler runs on the device, on the logits the step left there
+            std::vector<float> temp((size_t)b, 0.f), tp((size_t)b, 0.f), uni((size_t)b, 0.f);
+            std::vector<int32_t> tk((size_t)b, 0);
+            for (int i = 0; i < b; i++) {
+                Seq &q = s->seqs[ids[i]];
+                if (!q.sampled) continue;  // temperature 0: the greedy choice
+                temp[i] = q.temperature, tk[i] = q.top_k, tp[i] = q.top_p, uni[i] = next_uniform(&q.rng);
+            }
+            if (vh_sample_last_logits(s->m, b, temp.data(), tk.data(), tp.data(), uni.data(), am.data()) != VH_OK) return VH_ERR;
+        }
         for (int i = 0; i < b; i++) {  // scheduler.go:404-456
             Seq &q = s->seqs[ids[i]];
             q.position++;  // AdvancePosition (the prompt is complete here)
             if (q.state == VH_SEQ_PENDING) q.state = VH_SEQ_DECODING;
-            const int tok = pick(q, need_logits ? s->logits.data() + (size_t)i * V : nullptr, am[i]);
+            const int tok = am[i];
             q.generated.push_back(tok);
             produced++;
             if (is_stop(tok) || q.reached_max(s->cfg.max_tokens)) q.state = VH_SEQ_FINISHED;
