@@ -75,6 +75,10 @@ int vx_rmsnorm(vx_backend *be, const float *x, const float *weight, float *out, 
 /* :352. k may be NULL. rope_dim 0 = full head_dim. */
 int vx_rope(vx_backend *be, float *q, float *k, int head_dim, int num_heads, int num_kv_heads, int seq_len,
             int start_pos, int rope_dim, float theta, int rope_neox);
+/* RoPEShift of the CPU backend (backend/cpu/backend.go:244-276, interface.go:37-44): every K vector of
+ * k[num_tokens, num_kv_heads, head_dim] is rotated by the angle of position `shift` (interleaved pairs), which
+ * turns RoPE(p) into RoPE(p + shift); shift 0 changes nothing. */
+int vx_rope_shift(vx_backend *be, float *k, int head_dim, int num_kv_heads, int num_tokens, int shift, float theta);
 int vx_silu(vx_backend *be, const float *x, float *out, int n);                           /* :356 */
 int vx_silu_mul(vx_backend *be, const float *gate, const float *up, float *out, int n);   /* :360 */
 int vx_softmax(vx_backend *be, const float *x, float *out, int rows, int cols);           /* :364 */

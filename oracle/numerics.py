@@ -191,6 +191,13 @@ def rope_positions(q, k, head_dim, num_heads, num_kv_heads, positions, rope_dim,
     return q, k2
 
 
+def rope_shift(k, head_dim, num_kv_heads, num_tokens, shift, theta):
+    """backend/cpu/backend.go:244-276; returns the rotated copy."""
+    k2 = _f32(k).copy()
+    _lib.vxo_rope_shift(_p(k2), head_dim, num_kv_heads, num_tokens, shift, C.c_float(theta))
+    return k2
+
+
 def silu(x):
     x = _f32(x)
     out = np.empty_like(x)

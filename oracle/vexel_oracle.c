@@ -525,6 +525,26 @@ VXO_API void vxo_rope_positions(float *q, float *k, int head_dim, int num_heads,
     if (k) rope_one(k, (int64_t)rows * num_kv_heads, num_kv_heads, head_dim, 0, eff, theta, neox, positions);
 }
 
+/* inference/backend/cpu/backend.go:244-276 (RoPEShift): every K vector rotated by the angle of position `shift`,
+ * interleaved pairs over the whole head; shift 0 returns at once. */
+VXO_API void vxo_rope_shift(float *k, int head_dim, int num_kv_heads, int num_tokens, int shift, float theta) {
+    if (shift == 0) return;
+    for (int t = 0; t < num_tokens; t++)
+        for (int h = 0; h < num_kv_heads; h++) {
+            int64_t offset = (int64_t)t * num_kv_heads * head_dim + (int64_t)h * head_dim;
+            for (int j = 0; j < head_dim / 2; j++) {
+                int idx = j * 2;
+                double ex = (double)(2 * j) / (double)head_dim;
+                float freq = (float)(1.0 / pow((double)theta, ex));
+                float angle = (float)shift * freq;
+                float c = (float)cos((double)angle), sn = (float)sin((double)angle);
+                float v1 = k[offset + idx], v2 = k[offset + idx + 1];
+                k[offset + idx] = v1 * c - v2 * sn;
+                k[offset + idx + 1] = v1 * sn + v2 * c;
+            }
+        }
+}
+
 /* inference/backend/cpu/cpu.go:378-387 */
 VXO_API void vxo_silu(const float *x, float *out, int64_t n) {
     for (int64_t i = 0; i < n; i++) {

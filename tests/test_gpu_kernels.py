@@ -873,6 +873,23 @@ def test_paged_kv_move_chains(be):
         be.reset_pool()
 
 
+def test_rope_shift(be):
+    """RoPEShift (backend/cpu/backend.go:244-276) against the oracle (to the last bits of the float64 cos / sin, as
+    for RoPE itself); shift 0 leaves the buffer alone."""
+    rng = np.random.default_rng(39)
+    hd, hk, toks = 128, 4, 37
+    k = rng.standard_normal(toks * hk * hd).astype(np.float32)
+    dk = be.upload(k)
+    be.rope_shift(dk, hd, hk, toks, 0, 10000.0)
+    assert np.array_equal(be.download(dk, k.shape, np.float32), k)
+    for shift, theta in ((3, 10000.0), (4095, 500000.0)):
+        dk = be.upload(k)
+        be.rope_shift(dk, hd, hk, toks, shift, theta)
+        want = nx.rope_shift(k, hd, hk, toks, shift, theta)
+        _close(be.download(dk, k.shape, np.float32), want, 0, 1e-6, "rope shift %d" % shift)
+    be.reset_pool()
+
+
 def test_rope_store_paged(be):
     rng = np.random.default_rng(35)
     rows, hq, hk, d, bs, nblocks = 9, 8, 2, 64, 16, 30

@@ -179,6 +179,24 @@ def test_rope_kats():
     assert not (q[0] == 1.0 and q[1] == 0.0)
 
 
+# ---- inference/backend/cpu/rope_shift_test.go:9-90: RoPE(2) then shift 3 is RoPE(5); shift 0 is the identity;
+# a shift changes several tokens at once
+def test_rope_shift_kats():
+    theta, hd, hk = 10000.0, 4, 2
+    base = np.array([1, 2, 3, 4, 5, 6, 7, 8], dtype=np.float32)
+    _, k5 = nx.rope(np.zeros(8, dtype=np.float32), base, hd, hk, hk, 1, 5, 0, theta, False)
+    _, k2 = nx.rope(np.zeros(8, dtype=np.float32), base, hd, hk, hk, 1, 2, 0, theta, False)
+    k23 = nx.rope_shift(k2, hd, hk, 1, 3, theta)
+    assert np.max(np.abs(k5 - k23)) <= 1e-5
+    assert np.array_equal(nx.rope_shift(base, hd, hk, 1, 0, theta), base)
+    many = np.arange(1, 3 * hk * hd + 1, dtype=np.float32)
+    moved = nx.rope_shift(many, hd, hk, 3, 10, theta)
+    assert np.count_nonzero(moved != many) > 0
+    # a shift is the rotation RoPE gives a one-token call at that position, for every token alike
+    _, want = nx.rope_positions(np.zeros(3 * hk * hd, dtype=np.float32), many, hd, hk, hk, [10, 10, 10], 0, theta, False)
+    assert np.array_equal(moved.view(np.uint32), want.reshape(-1).view(np.uint32))
+
+
 # ---- test/golden/golden_test.go:267-319: position 0 is the identity
 def test_rope_pos0_identity():
     rng = np.random.default_rng(1)

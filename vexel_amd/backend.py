@@ -266,6 +266,9 @@ class HipBackend:
         self.call("vx_sdpa_paged_tree", q, kv_pool, int(bool(pool_is_f16)), block_table, out, tree_mask,
                   tree_base, block_size, num_q_heads, num_kv_heads, head_dim, scale, query_len)
 
+    def rope_shift(self, k, head_dim, num_kv_heads, num_tokens, shift, theta):
+        self.call("vx_rope_shift", k, head_dim, num_kv_heads, num_tokens, shift, theta)
+
     def sample_rows(self, logits, rows, n, temperature, top_k, top_p, uniform, out_idx):
         self.call("vx_sample_rows", logits, rows, n, temperature, top_k, top_p, uniform, out_idx)
 

@@ -91,10 +91,10 @@ __device__ __forceinline__ void rope_pair(float &a, float &b, RopeCS cs) {
 
 // grid.x = seq row, threads over rotation pairs j.
 __global__ void rope_kernel(float *q, float *k, int head_dim, int num_heads, int num_kv_heads, int start_pos,
-                            int eff_dim, float theta, int neox, const int32_t *positions) {
+                            int eff_dim, float theta, int neox, const int32_t *positions, int row_step) {
     int row = blockIdx.x;
     int half = eff_dim / 2;
-    int pos = positions ? positions[row] : start_pos + row;
+    int pos = positions ? positions[row] : start_pos + row * row_step;  // row_step 0: one position for every row
     for (int j = threadIdx.x; j < half; j += blockDim.x) {
         RopeCS cs = rope_cs(pos, j, eff_dim, theta);
         int i0 = neox ? j : 2 * j;
@@ -476,7 +476,19 @@ int vx_rope(vx_backend *be, float *q, float *k, int head_dim, int num_heads, int
     if (seq_len == 0) return VX_OK;
     int threads = eff / 2 < 64 ? 64 : (eff / 2 > 256 ? 256 : eff / 2);
     rope_kernel<<<seq_len, threads, 0, be->stream>>>(q, k, head_dim, num_heads, num_kv_heads, start_pos, eff, theta,
-                                                      rope_neox, nullptr);
+                                                      rope_neox, nullptr, 1);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_rope_shift(vx_backend *be, float *k, int head_dim, int num_kv_heads, int num_tokens, int shift, float theta) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(k && head_dim > 0 && head_dim % 2 == 0 && num_kv_heads > 0 && num_tokens >= 0, "vx_rope_shift: bad arguments");
+    if (shift == 0 || num_tokens == 0) return VX_OK;  // backend/cpu/backend.go:248-250
+    int threads = head_dim / 2 < 64 ? 64 : (head_dim / 2 > 256 ? 256 : head_dim / 2);
+    rope_kernel<<<num_tokens, threads, 0, be->stream>>>(nullptr, k, head_dim, 0, num_kv_heads, shift, head_dim, theta, 0,
+                                                         nullptr, 0);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }

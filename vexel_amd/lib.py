@@ -73,6 +73,7 @@ SIGNATURES = {
     "vx_argmax_rows": (_i, [_vp, _vp, _i, _i, _vp]),
     "vx_sdpa_paged_tree_rows_per_entry": (_i, [_i, _i, _i, _i, _i]),
     "vx_sdpa_paged_tree_batched": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),
+    "vx_rope_shift": (_i, [_vp, _vp, _i, _i, _i, _i, _f]),
     "vx_sample_rows": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "vx_paged_kv_move": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i]),
     "vx_pack_batch": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
