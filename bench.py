@@ -417,7 +417,7 @@ def main():
                                "ctx lognormal(median 1024, sigma 0.6) in [64,4096] seed 0, sum ctx %d, block 16, "
                                "greedy decode, hipGraph=%s" % (args.layers, nseq, sum(ctx_now), use_graph),
                    "global_batch": nseq},
-        "roofline": {"bound": "hbm", "kernel": "paged_decode_f16_kernel<128,1>",
+        "roofline": {"bound": "hbm", "kernel": "paged_decode_f16_kernel<128,1,1>",
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE * attn_bytes, "bytes_per_launch": attn_bytes, "ms_per_launch": attn_ms},
     }
