@@ -28,6 +28,19 @@ def test_library_exports_every_declared_symbol():
     lib.load()
 
 
+def test_host_library_exports_every_declared_symbol():
+    """include/vexel_host.h against libvexel_host.so (the host runtime above the C ABI)."""
+    text = open(os.path.join(ROOT, "include", "vexel_host.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    names = set(re.findall(r"\b(vh_[a-z0-9_]+)\s*\(", text))
+    assert len(names) > 40
+    path = os.path.join(ROOT, "vexel_amd", "libvexel_host.so")
+    assert os.path.exists(path), "build the library first: python -m vexel_amd.build"
+    dll = ctypes.CDLL(path)
+    for name in sorted(names):
+        assert hasattr(dll, name), "missing export " + name
+
+
 def test_error_text_is_available_without_a_gpu():
     l = lib.load()
     assert isinstance(l.vx_last_error(), bytes)
