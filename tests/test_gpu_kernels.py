@@ -840,6 +840,17 @@ def test_sample_rows_matches_the_reference_sampler(be):
     want = [hl.sampler_sample(logits[i], float(temp[i]), int(topk[i]), float(topp[i]), float(uni[i])) for i in range(rows)]
     assert got.tolist() == want
     assert len(set(want)) > rows // 3                        # the cases do pick different tokens
+    # tiny and odd vocabularies, one row and many
+    for n2, rows2 in ((1, 1), (5, 3), (257, 40), (4096, 2)):
+        lg = rng.standard_normal((rows2, n2)).astype(np.float32)
+        t2 = rng.choice([0.0, 0.6, 1.0], rows2).astype(np.float32)
+        k2 = rng.integers(0, n2 + 2, rows2).astype(np.int32)
+        p2 = rng.choice([0.0, 0.5, 0.9, 1.0], rows2).astype(np.float32)
+        u2 = rng.random(rows2).astype(np.float32)
+        o2 = be.alloc(rows2 * 4)
+        be.sample_rows(be.upload(lg), rows2, n2, be.upload(t2), be.upload(k2), be.upload(p2), be.upload(u2), o2)
+        w2 = [hl.sampler_sample(lg[i], float(t2[i]), int(k2[i]), float(p2[i]), float(u2[i])) for i in range(rows2)]
+        assert be.download(o2, (rows2,), np.int32).tolist() == w2, (n2, rows2)
     be.reset_pool()
 
 
