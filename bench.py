@@ -56,42 +56,53 @@ def load_synth():
     return s
 
 
-def build_model(be, ctx, extra_tokens, layers):
-    """Synthetic 7B-shaped model + pre-filled contexts, generated on the device. -> (ModelRuntime, ids)"""
+def build_model(be, ctx, extra_tokens, layers, cfg=None, fmts=None, max_batch=None):
+    """Synthetic model (7B-shaped Q4_0 unless cfg / fmts say otherwise) + pre-filled contexts, generated on the
+    device. fmts: weight name (wq, wk, wv, wo, w1, w3, w2, head) -> VX_* format, "*" the default.
+    -> (ModelRuntime, ids)"""
     from vexel_amd import lib
     from vexel_amd.runtime import ModelRuntime
     synth = load_synth()
-    c = dict(CFG)
+    c = dict(cfg or CFG)
     c["num_layers"] = layers
+    fmts = fmts or {"*": lib.VX_Q4_0, "head": lib.VX_Q8_0}
+    fm = lambda name: fmts.get(name, fmts["*"])
     need_blocks = sum((L + extra_tokens + BLOCK - 1) // BLOCK + 1 for L in ctx)
     max_bps = (max(ctx) + extra_tokens + BLOCK - 1) // BLOCK + 1
     mr = ModelRuntime(be, **c, pool_blocks=need_blocks, max_seqs=len(ctx), max_blocks_per_seq=max_bps,
-                      max_batch=len(ctx), kv_fp16=True)
+                      max_batch=max_batch or len(ctx), kv_fp16=True)
     seed = [0]
 
     def qw(n, k, fmt=lib.VX_Q4_0):
-        bb = 18 if fmt == lib.VX_Q4_0 else 34
-        nblk = n * (k // 32)
-        p = be.alloc_permanent(nblk * bb)
-        mr.adopt_device_buffer(p)
         seed[0] += 1
-        rc = synth.vxs_gaussian_quant(fmt, p, nblk, 0.02, seed[0])
+        if fmt in (lib.VX_Q4_0, lib.VX_Q8_0):
+            bb = 18 if fmt == lib.VX_Q4_0 else 34
+            nblk = n * (k // 32)
+            p = be.alloc_permanent(nblk * bb)
+            rc = synth.vxs_gaussian_quant(fmt, p, nblk, 0.02, seed[0])
+        else:                                    # Q4_K / Q6_K: random valid super-blocks
+            bb = 144 if fmt == lib.VX_Q4_K else 210
+            nblk = n * (k // 256)
+            p = be.alloc_permanent(nblk * bb + 16)
+            rc = synth.vxs_random_kquant(fmt, p, nblk, seed[0])
+        mr.adopt_device_buffer(p)
         if rc != 0:
-            raise RuntimeError("vxs_gaussian_quant failed: %d" % rc)
+            raise RuntimeError("synthetic weights failed: %d" % rc)
         return (fmt, p, n, k)
 
     h, qd, kvd, f, v = c["hidden"], c["num_heads"] * c["head_dim"], c["num_kv_heads"] * c["head_dim"], c["ffn"], c["vocab"]
     ones = be.upload(np.ones(h, dtype=np.float32), permanent=True)
     mr.adopt_device_buffer(ones)
     for l in range(layers):
-        mr.set_layer(l, ones, ones, dict(wq=qw(qd, h), wk=qw(kvd, h), wv=qw(kvd, h), wo=qw(h, qd),
-                                         w1=qw(f, h), w3=qw(f, h), w2=qw(h, f)))
+        mr.set_layer(l, ones, ones, dict(wq=qw(qd, h, fm("wq")), wk=qw(kvd, h, fm("wk")), wv=qw(kvd, h, fm("wv")),
+                                         wo=qw(h, qd, fm("wo")), w1=qw(f, h, fm("w1")), w3=qw(f, h, fm("w3")),
+                                         w2=qw(h, f, fm("w2"))))
     emb_q = qw(v, h, lib.VX_Q8_0)
     emb = be.alloc_permanent(v * h * 4)
     mr.adopt_device_buffer(emb)
     be.dequantize(lib.VX_Q8_0, emb_q[1], emb, v * h)     # loader rule: token_embd kept in F32
     be.sync()
-    mr.set_head(emb, ones, qw(v, h, lib.VX_Q8_0))
+    mr.set_head(emb, ones, qw(v, h, fm("head")))
     # KV: every physical block of every layer holds N(0,1) halves
     per_block = 2 * BLOCK * kvd
     for l in range(layers):
@@ -350,6 +361,71 @@ def prefill_probe(be, rows=512, reps=10):
     print(json.dumps(out))
 
 
+def configs_report(be):
+    """Throughput of the BASELINE configs other than the north star, each at its real shape (synthetic weights and
+    contexts, greedy decode replayed from a hipGraph; config 4 as its two ingredients; config 5 as one verification
+    step). Informational: the benchmark line is the north-star workload."""
+    from vexel_amd import lib
+    from oracle import host_logic as hl
+    tiny = dict(num_layers=22, hidden=2048, num_heads=32, num_kv_heads=4, head_dim=64, ffn=5632, vocab=32000)
+    l8b = dict(num_layers=32, hidden=4096, num_heads=32, num_kv_heads=8, head_dim=128, ffn=14336, vocab=128256,
+               rope_theta=500000.0)
+    q4km = {"*": lib.VX_Q4_K, "wv": lib.VX_Q6_K, "w2": lib.VX_Q6_K, "head": lib.VX_Q6_K}
+
+    def decode_rate(name, cfg, fmts, ctx, steps):
+        mr, ids = build_model(be, ctx, steps + 16, cfg["num_layers"], cfg, fmts)
+        first = np.random.default_rng(3).integers(0, cfg["vocab"], len(ctx)).astype(np.int32)
+        mr.decode_graph(first, ids, ctx, 4, use_graph=True)
+        be.sync()
+        t0 = time.perf_counter()
+        mr.decode_graph(None, None, None, steps, use_graph=True, batch=len(ctx))
+        be.sync()
+        dt = time.perf_counter() - t0
+        print("%-64s %8.1f tok/s  %7.3f ms/step" % (name, len(ctx) * steps / dt, dt * 1e3 / steps), flush=True)
+        return mr, ids
+
+    rng = np.random.default_rng(0)
+    mr, _ = decode_rate("config 1: TinyLlama-shaped Q4_0, 1 sequence, ctx 32 + 64 steps", tiny, None, [32], 64)
+    mr.close()
+    ctx2 = [int(x) for x in rng.integers(128, 2049, 8)]
+    mr, _ = decode_rate("config 2: TinyLlama-shaped Q4_0, 8 ragged sequences (sum ctx %d)" % sum(ctx2), tiny, None, ctx2, 128)
+    mr.close()
+    ctx3 = ragged_contexts()
+    mr, _ = decode_rate("config 3: 7B-shaped Q4_K_M mix, 32 ragged sequences (sum ctx %d)" % sum(ctx3), CFG, q4km, ctx3, 64)
+    mr.close()
+    ctx4 = [int(x) for x in np.clip(np.exp(rng.normal(math.log(512.0), 0.6, 64)), 16, 4096)]
+    mr, ids = decode_rate("config 4 (decode part): 8B-shaped Q8_0, 64 sequences (sum ctx %d)" % sum(ctx4), l8b,
+                          {"*": lib.VX_Q8_0}, ctx4 + [640], 32)   # the 65th sequence only reserves blocks for the chunk
+    chunk = rng.integers(0, l8b["vocab"], 512).tolist()
+    mr.delete_sequence(ids[-1])
+    mr.prefill_with_paged_kv(chunk[:64], 1000, 0)           # sizes the workspaces
+    mr.delete_sequence(1000)
+    be.sync()
+    t0 = time.perf_counter()
+    mr.prefill_with_paged_kv(chunk, 1001, 0)
+    be.sync()
+    dt = time.perf_counter() - t0
+    print("%-64s %8.1f tok/s  %7.3f ms/chunk" % ("config 4 (prefill part): one 512-token chunk", 512 / dt, dt * 1e3), flush=True)
+    mr.close()
+    ctx5 = [int(x) for x in rng.integers(256, 2049, 16)]
+    mr, ids = build_model(be, ctx5, 64, 32, CFG, {"*": lib.VX_Q6_K}, max_batch=16)
+    start, inputs = list(ctx5), rng.integers(0, 32000, 16).tolist()
+    for it in range(4):
+        trees = []
+        for _ in range(16):
+            toks = [rng.choice(32000, 2, replace=False).tolist() for _ in range(4)]
+            trees.append(hl.build_candidate_tree_from_topk(toks, [[2.0, 1.0]] * 4, 15).linearize())
+        be.sync()
+        t0 = time.perf_counter()
+        acc, fin, _ = mr.verify_tree(ids, inputs, start, trees, want_logits=False)
+        dt = time.perf_counter() - t0
+        start = [start[i] + 1 + len(acc[i]) for i in range(16)]
+        inputs = fin
+    print("%-64s %8.1f rows/s %7.3f ms/step" % ("config 5: 7B-shaped Q6_K, 16 sequences (sum ctx %d), 15-node trees" % sum(ctx5),
+                                                  256 / dt, dt * 1e3), flush=True)
+    mr.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -365,6 +441,8 @@ def main():
                          "table of achieved GB/s against the 8 TB/s HBM peak, then exit")
     ap.add_argument("--counter-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: one 1 GiB plain copy and 8 attention launches, then exit")
+    ap.add_argument("--configs-report", action="store_true",
+                    help="decode / prefill / verification rates of BASELINE configs 1-5 at their real shapes, then exit")
     ap.add_argument("--prefill-probe", action="store_true",
                     help="for rocprofv3 --pmc runs of the MFMA kernels: 512-row GEMMs of the 7B shapes and one "
                          "512-token prefill attention, then exit")
@@ -379,6 +457,9 @@ def main():
         return
     if args.prefill_probe:
         prefill_probe(be)
+        return
+    if args.configs_report:
+        configs_report(be)
         return
     ctx = ragged_contexts(n=args.seqs) if args.seqs != BATCH else ragged_contexts()
     nseq = len(ctx)
