@@ -446,6 +446,10 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
     constexpr int ANL = APIECES / 256;
     __shared__ __attribute__((aligned(16))) half8 a_lds[APIECES];
     __shared__ __attribute__((aligned(16))) uint8_t w_lds[4][ROWS_W * PITCH + 16];  // +16: the unaligned dword read may touch 4 bytes past the last row
+    // formats with a min term: the chunk's activation block sums, [step][tile][row], staged with the tiles
+    constexpr int NBS = CH * MT * 16;
+    static_assert(NBS <= 256, "one block sum per thread");
+    __shared__ __attribute__((aligned(16))) float bs_lds[F::HAS_MIN ? NBS : 4];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int ln = lane & 15, g = lane >> 4;
@@ -473,6 +477,7 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
     half8 a_stage[ANL];
     u32x4 w_stage[WNL];
     float4v cs_stage[MT], cs_cur[MT];  // the chunk's factors for this lane's rows m0 + 16t + 4g + (0..3)
+    float bs_stage = 0.f;
     // K is a multiple of 256, so every chunk has CH full steps and CHUNK_BYTES bytes per row. Every load is
     // unconditional (addresses are clamped instead): a load under a branch makes the compiler wait for it
     // inside the branch, which serialises the whole prefetch.
@@ -486,6 +491,10 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
         }
 #pragma unroll
         for (int t = 0; t < MT; t++) cs_stage[t] = *(const float4v *)(pv.cscale + (size_t)chunk * Mpad + m0 + t * 16 + 4 * g);
+        if (F::HAS_MIN) {
+            const int i = tid % NBS;  // (step, tile, row); threads past NBS repeat a load and store nothing
+            bs_stage = pv.bsum[(size_t)(s0 + i / (MT * 16)) * Mpad + m0 + i % (MT * 16)];
+        }
         const size_t coff = (size_t)chunk * F::CHUNK_BYTES;
 #pragma unroll
         for (int i = 0; i < WNL; i++) {
@@ -503,6 +512,7 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
     auto commit = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int t = 0; t < MT; t++) cs_cur[t] = cs_stage[t];
+        if (F::HAS_MIN && tid < NBS) bs_lds[tid] = bs_stage;
 #pragma unroll
         for (int i = 0; i < ANL; i++) a_lds[i * 256 + tid] = a_stage[i];
 #pragma unroll
@@ -536,7 +546,8 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
             for (int t = 0; t < MT; t++) {
                 if (F::HAS_MIN) {
 #pragma unroll
-                    for (int i = 0; i < 4; i++) crun[r][t][i] += w[r].d * acc[r][t][i] - w[r].dm * bs[t][i];
+                    for (int i = 0; i < 4; i++)  // two fused multiply-adds per output (one expression would cost three operations)
+                        crun[r][t][i] = __builtin_fmaf(-w[r].dm, bs[t][i], __builtin_fmaf(w[r].d, acc[r][t][i], crun[r][t][i]));
                 } else {
 #pragma unroll
                     for (int i = 0; i < 4; i++) crun[r][t][i] += w[r].d * acc[r][t][i];
@@ -544,7 +555,6 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
             }
     };
     auto compute = [&](int chunk) __attribute__((always_inline)) {
-        const int s0 = chunk * CH;
         const uint8_t *wl = &w_lds[wave][0];
 #pragma unroll
         for (int r = 0; r < R; r++)
@@ -579,7 +589,7 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
             }
             if (F::HAS_MIN) {
 #pragma unroll
-                for (int t = 0; t < MT; t++) bs_cur[t] = *(const float4v *)(pv.bsum + (size_t)(s0 + s) * Mpad + m0 + t * 16 + 4 * g);
+                for (int t = 0; t < MT; t++) bs_cur[t] = *(const float4v *)&bs_lds[(s * MT + t) * 16 + 4 * g];
             }
             float4v acc[R][MT];
 #pragma unroll
@@ -675,7 +685,8 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
                 }
                 if (i > 0) {
 #pragma unroll
-                    for (int e = 0; e < 4; e++) crun[pr][pt][e] += w_cur[pr].d * p1[e] + w_cur[pr].dm * p2[e];
+                    for (int e = 0; e < 4; e++)
+                        crun[pr][pt][e] = __builtin_fmaf(w_cur[pr].dm, p2[e], __builtin_fmaf(w_cur[pr].d, p1[e], crun[pr][pt][e]));
                 }
                 p1 = c1, p2 = c2, pr = r, pt = t;
             }
