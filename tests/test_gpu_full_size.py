@@ -150,3 +150,32 @@ def test_pack_batch_at_maximum_batch_and_context(be):
     assert int(be.download(d_fc, (1,), np.int32)[0]) == len(pool.free_lists[0])
     assert be.download(d_free, (len(pool.free_lists[0]),), np.int32).tolist() == pool.free_lists[0]
     be.reset_pool()
+
+
+def test_north_star_shape_batched_equals_sequence_by_sequence(be):
+    """The whole north-star model (7B shape, 32 layers, Q4_0, 32 ragged sequences up to 4096 tokens) is beyond the
+    oracle's reach, but the reference's batched decode is by definition its single-sequence decode in a loop
+    (runtime/decode.go:612-654): the batched step (MFMA GEMMs, work-list attention, fused blocks) must give each
+    sequence the logits the one-sequence path (matrix-vector kernels, one-row attention) gives it alone, within the
+    logits budget, and the same greedy token; checked for a sample of the sequences over two steps."""
+    import os, sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+    ctx = bench.ragged_contexts()
+    mr, ids = bench.build_model(be, ctx, 8, 32)
+    mr2, ids2 = bench.build_model(be, ctx, 8, 32)           # same seeds: the same weights and contexts
+    rng = np.random.default_rng(405)
+    toks = rng.integers(0, 32000, len(ids)).tolist()
+    pos = list(ctx)
+    sample = [0, int(np.argmax(ctx)), int(np.argmin(ctx)), 17]
+    for step in range(2):
+        got, am = mr.decode_with_paged_kv_batched(toks, ids, pos)
+        for i in sample:
+            one, am1 = mr2.decode_with_paged_kv_batched([toks[i]], [ids2[i]], [pos[i]])
+            err = np.abs(got[i].astype(np.float64) - one[0].astype(np.float64))
+            assert np.all(err <= 1e-2 + 1e-3 * np.abs(one[0])), "sequence %d step %d: max err %.3e" % (i, step, err.max())
+            assert int(am[i]) == int(am1[0])
+        toks = [int(a) for a in am]
+        pos = [p + 1 for p in pos]
+    mr.close()
+    mr2.close()
