@@ -362,7 +362,7 @@ def prefill_probe(be, rows=512, reps=10):
 
 
 def configs_report(be):
-    """Throughput of the BASELINE configs other than the north star, each at its real shape (synthetic weights and
+    """Throughput of the benchmark configs other than the north star, each at its real shape (synthetic weights and
     contexts, greedy decode replayed from a hipGraph; config 4 as its two ingredients; config 5 as one verification
     step). Informational: the benchmark line is the north-star workload."""
     from vexel_amd import lib
@@ -442,7 +442,7 @@ def main():
     ap.add_argument("--counter-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: one 1 GiB plain copy and 8 attention launches, then exit")
     ap.add_argument("--configs-report", action="store_true",
-                    help="decode / prefill / verification rates of BASELINE configs 1-5 at their real shapes, then exit")
+                    help="decode / prefill / verification rates of benchmark configs 1-5 at their real shapes, then exit")
     ap.add_argument("--prefill-probe", action="store_true",
                     help="for rocprofv3 --pmc runs of the MFMA kernels: 512-row GEMMs of the 7B shapes and one "
                          "512-token prefill attention, then exit")

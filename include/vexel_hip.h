@@ -101,7 +101,7 @@ int vx_matmul_q4_0(vx_backend *be, const float *a, const void *b, float *out, in
 int vx_matmul_q4_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :55 */
 int vx_matmul_q6_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :60 */
 int vx_matmul_q8_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :75 */
-/* Not in any BASELINE config: one wave per weight row on the exact dequantised values (pkg/gguf/dequant.go:
+/* Not in any benchmark config: one wave per weight row on the exact dequantised values (pkg/gguf/dequant.go:
  * 423-500, 100-145, 215-228), no tiled or matrix-vector fast path. */
 int vx_matmul_q5_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :65 */
 int vx_matmul_q5_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :70 */

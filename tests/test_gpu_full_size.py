@@ -1,4 +1,4 @@
-"""The hot kernels at the BASELINE configs' full shapes. The oracle cannot run whole matrices of this size in
+"""The hot kernels at the benchmark configs' full shapes. The oracle cannot run whole matrices of this size in
 seconds, so every check takes the full-size GPU result and compares a sample of it (rows of the weight matrix,
 whole attention heads) with the oracle computed on exactly those rows, plus properties that hold at any size."""
 import math

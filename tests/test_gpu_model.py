@@ -1,8 +1,8 @@
 """End-to-end parity of the decode drivers against the CPU oracle on identical seeded
-random-init weights and inputs (the BASELINE configs at sizes the oracle finishes in seconds:
+random-init weights and inputs (the benchmark configs at sizes the oracle finishes in seconds:
 real head geometry and hidden sizes, fewer layers).
 
-Bars (BASELINE north star): logits within 1e-2 absolute / 1e-3 relative in float32; greedy
+Bars (the benchmark's north star): logits within 1e-2 absolute / 1e-3 relative in float32; greedy
 tokens identical; block tables / slot state bit-exact."""
 import numpy as np
 import pytest
@@ -29,7 +29,7 @@ def _greedy_margin(logits):
 
 
 def test_c1_prefill_then_greedy_decode(be):
-    """BASELINE config 1 shape (TinyLlama head geometry, Q4_0, Q8_0 embeddings and head), batch 1:
+    """benchmark config 1 shape (TinyLlama head geometry, Q4_0, Q8_0 embeddings and head), batch 1:
     32-token prompt, greedy decode of 64 tokens. 2 layers so the CPU side stays in seconds."""
     cfg = om.ModelConfig(num_layers=2, hidden=2048, num_heads=32, num_kv_heads=4, head_dim=64, ffn=5632,
                          vocab=32000, eps=1e-5, rope_theta=10000.0)
@@ -74,7 +74,7 @@ def _ragged_setup(be, cfg, fmt, head_fmt, ctx_lens, seed, pool_blocks, fmt_overr
 
 
 def test_c2_batched_decode_ragged_paged(be):
-    """BASELINE config 2 shape: 8 sequences, ragged contexts, KV pre-filled with N(0,1), permuted block
+    """benchmark config 2 shape: 8 sequences, ragged contexts, KV pre-filled with N(0,1), permuted block
     tables; batched decode steps against the oracle's sequential per-sequence loop."""
     cfg = om.ModelConfig(num_layers=2, hidden=2048, num_heads=32, num_kv_heads=4, head_dim=64, ffn=5632,
                          vocab=32000)
@@ -220,7 +220,7 @@ def test_chunked_prefill_and_verify(be):
 
 @pytest.mark.parametrize("kv_heads,max_nodes", [(8, 15), (2, 10)])
 def test_c5_tree_verification_batched(be, kv_heads, max_nodes):
-    """BASELINE config 5 at oracle size: Q6_K weights, several sequences at ragged contexts, a 15-node candidate
+    """benchmark config 5 at oracle size: Q6_K weights, several sequences at ragged contexts, a 15-node candidate
     tree (4 heads x top-2) per sequence verified in one pass under tree masks over the paged f16 pool, greedy
     acceptance, rollback in the block tables; two rounds, the second on top of the first one's rollback.
     Second case: grouped-query heads and 11-row trees, which do not fill the attention's entries of query rows."""

@@ -280,7 +280,7 @@ def test_tree_paths_linearize_mask():
 
 
 def test_tree_15_nodes_4x2():
-    """BASELINE config 5: 4 heads x top-2 capped at 15 nodes = 2+4+8+1."""
+    """benchmark config 5: 4 heads x top-2 capped at 15 nodes = 2+4+8+1."""
     toks = [[10, 11], [20, 21], [30, 31], [40, 41]]
     vals = [[2.0, 1.0]] * 4
     t = hl.build_candidate_tree_from_topk(toks, vals, 15)

@@ -1,5 +1,5 @@
 // Benchmark support, not part of the backend's C ABI: fills device buffers with synthetic
-// data of the shapes the BASELINE configs name, without any host round trip:
+// data of the shapes the benchmark configs name, without any host round trip:
 //   vxs_gaussian_quant  N(0,std) values quantized to Q4_0 / Q8_0 blocks (llama.cpp convention:
 //                       Q4_0 d = signed absmax / -8, q = min(15, floor(x/d + 8.5));
 //                       Q8_0 d = absmax / 127, q = round(x/d))
