@@ -179,7 +179,7 @@ def test_matmul_rows_independent_of_batch(be, fmt):
     be.reset_pool()
 
 
-@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("fmt", FMTS + [nx.FMT_Q5_0, nx.FMT_Q5_K])
 @pytest.mark.parametrize("n,k", [(80, 1024), (33, 256), (7, 4096), (96, 11008), (40, 14336)])
 def test_matvec_single_row(be, fmt, n, k):
     """M = 1 (the reference's decode call): segments that start at odd 16-byte phases, rows that are not a

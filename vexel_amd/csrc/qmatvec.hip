@@ -246,6 +246,55 @@ struct VQ6_K {  // dequant.go:272-331: 210-byte super-block [ql 128][qh 64][int8
     }
 };
 
+// the 4 low bits of b, one each into bit 4 of the 4 bytes of a dword (bit i -> byte i)
+__device__ __forceinline__ uint32_t fifth_bits(uint32_t b) { return ((b * 0x00204081u) & 0x01010101u) << 4; }
+
+struct VQ5_0 {  // dequant.go:100-145: [f16 d][u32 qh][16 bytes], element i = nibble as Q4_0 | bit i of qh << 4, (q-16)*d
+    static constexpr int UNIT_BLOCKS = 1, UNIT_BYTES = 22;
+    typedef XInt<22> X;  // |xi| < 2^21: |sum q xi| <= 31 * 2^21 * 32 < 2^31
+    static __device__ __forceinline__ float block(const uint8_t *base, int seg, int jl, const X &x) {
+        const int o = seg + jl * 22;
+        uint32_t w[5];
+        lds_dwords<5>(base, o + 2, w);
+        const uint32_t qh = w[0];
+        int acc[3] = {0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            x.dot(acc, (w[1 + i] & 0x0F0F0F0Fu) | fifth_bits((qh >> (4 * i)) & 15u), i);
+            x.dot(acc, ((w[1 + i] >> 4) & 0x0F0F0F0Fu) | fifth_bits((qh >> (16 + 4 * i)) & 15u), 4 + i);
+        }
+        const int t = acc[0] + (acc[1] << 8) + (acc[2] << 16) - 16 * (x.s0 + x.s1);  // sum (q - 16) xi, exact
+        return h2f((uint16_t)lds_u16(base, o)) * ((float)t * x.inv);
+    }
+};
+
+struct VQ5_K {  // dequant.go:423-500: 176-byte super-block [d][dmin][12 scale bytes][qh 32][qs 128]: d*sc*q - dmin*m
+    static constexpr int UNIT_BLOCKS = 8, UNIT_BYTES = 176;
+    typedef XInt<22> X;
+    static __device__ __forceinline__ float block(const uint8_t *base, int seg, int jl, const X &x) {
+        const int j = jl & 7;
+        const int sb = seg + (jl >> 3) * 176;  // 16-byte aligned: rows and segments are whole super-blocks
+        const uint32_t *S = (const uint32_t *)(base + sb);
+        const uint32_t *qp = S + 12 + 8 * (j >> 1);
+        int acc[3] = {0, 0, 0};
+#pragma unroll
+        for (int i = 0; i < 8; i++)  // bit j of qh byte l is the fifth bit of element l of sub-block j
+            x.dot(acc, ((qp[i] >> (4 * (j & 1))) & 0x0F0F0F0Fu) | (((S[4 + i] >> j) & 0x01010101u) << 4), i);
+        const int t = acc[0] + (acc[1] << 8) + (acc[2] << 16);
+        const uint8_t *q = base + sb + 4;
+        uint32_t sc, mn;  // getScaleMinK4, dequant.go:400-409
+        if (j < 4) {
+            sc = q[j] & 63;
+            mn = q[j + 4] & 63;
+        } else {
+            sc = (q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4);
+            mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+        }
+        const uint32_t hd = S[0];
+        return (h2f((uint16_t)(hd & 0xFFFF)) * (float)sc * (float)t - h2f((uint16_t)(hd >> 16)) * (float)mn * (float)(x.s0 + x.s1)) * x.inv;
+    }
+};
+
 // What one launch works on. Up to three weight matrices of one format and K, their rows concatenated (Q|K|V,
 // gate|up); where the activation row comes from; what happens to the dot products.
 struct MvArgs {
@@ -497,6 +546,8 @@ size_t mv_row_bytes(int fmt, int k) {
     case VX_Q8_0: return k % 32 == 0 ? (size_t)(k / 32) * 34 : 0;
     case VX_Q4_K: return k % 256 == 0 ? (size_t)(k / 256) * 144 : 0;
     case VX_Q6_K: return k % 256 == 0 ? (size_t)(k / 256) * 210 : 0;
+    case VX_Q5_0: return k % 32 == 0 ? (size_t)(k / 32) * 22 : 0;
+    case VX_Q5_K: return k % 256 == 0 ? (size_t)(k / 256) * 176 : 0;
     }
     return 0;
 }
@@ -524,6 +575,8 @@ int launch_fmt(vx_backend *be, int fmt, MvArgs &a) {
     case VX_Q8_0: return launch<VQ8_0>(be, a);
     case VX_Q4_K: return launch<VQ4_K>(be, a);
     case VX_Q6_K: return launch<VQ6_K>(be, a);
+    case VX_Q5_0: return launch<VQ5_0>(be, a);
+    case VX_Q5_K: return launch<VQ5_K>(be, a);
     }
     return VX_ERR_UNSUPPORTED;
 }
@@ -542,6 +595,8 @@ bool matvec_ok(int fmt, const void *const *ws, const int *ns, int nw, int k) {
     case VX_Q8_0: return shape_ok<VQ8_0>(k);
     case VX_Q4_K: return shape_ok<VQ4_K>(k);
     case VX_Q6_K: return shape_ok<VQ6_K>(k);
+    case VX_Q5_0: return shape_ok<VQ5_0>(k);
+    case VX_Q5_K: return shape_ok<VQ5_K>(k);
     }
     return false;
 }
