@@ -93,6 +93,30 @@ int vx_sdpa(vx_backend *be, const float *q, const float *k, const float *v, floa
 /* :389. Q/K/V/out token-major [seqLen, heads, headDim], causal. */
 int vx_sdpa_prefill(vx_backend *be, const float *q, const float *k, const float *v, float *out, int seq_len,
                     int num_q_heads, int num_kv_heads, int head_dim, float scale);
+
+/* ---- optional interfaces of other architectures (backend.go:205-263; CPU bodies in backend/cpu/cpu.go) ---- */
+/* LayerNormOps.LayerNorm (backend.go:207-212, cpu.go:404-436): (x - mean) / sqrt(var + eps) * weight + bias per
+ * row, var = the mean squared deviation (divisor cols). */
+int vx_layernorm(vx_backend *be, const float *x, const float *weight, const float *bias, float *out, int rows,
+                 int cols, float eps);
+/* GELUOps (backend.go:216-226, cpu.go:440-473): 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))); gelu(gate) * up. */
+int vx_gelu(vx_backend *be, const float *x, float *out, int n);
+int vx_gelu_mul(vx_backend *be, const float *gate, const float *up, float *out, int n);
+/* BiasOps.AddBias (backend.go:249-253, cpu.go:476-487): out[r][c] = x[r][c] + bias[c]; out may be x. */
+int vx_add_bias(vx_backend *be, const float *x, const float *bias, float *out, int rows, int cols);
+/* ScaleOps.ScaleBuffer (backend.go:257-261, cpu.go:558-563): buf[i] *= scale in place. */
+int vx_scale_buffer(vx_backend *be, float *buf, float scale, int n);
+/* SoftCapAttentionOps (backend.go:231-241, cpu.go:705-841): vx_sdpa / vx_sdpa_prefill whose scaled scores pass
+ * through softcap * tanh(score / softcap) before the softmax; softcap 0 is the plain kernel. */
+int vx_sdpa_softcap(vx_backend *be, const float *q, const float *k, const float *v, float *out, int kv_len,
+                    int num_q_heads, int num_kv_heads, int head_dim, float scale, float softcap, int kv_head_stride);
+int vx_sdpa_prefill_softcap(vx_backend *be, const float *q, const float *k, const float *v, float *out, int seq_len,
+                            int num_q_heads, int num_kv_heads, int head_dim, float scale, float softcap);
+/* ScaledRoPEOps.RoPEWithFreqs (backend.go:247-249, cpu.go:308-375): RoPE over the whole head with pair j turning
+ * by position * freqs[j] (head_dim / 2 floats on the device). k may be NULL. */
+int vx_rope_with_freqs(vx_backend *be, float *q, float *k, const float *freqs, int head_dim, int num_heads,
+                       int num_kv_heads, int seq_len, int start_pos, int rope_neox);
+
 /* ArgmaxOps.Argmax (backend.go:199-203): first index of the strict maximum; waits for the stream. */
 int vx_argmax(vx_backend *be, const float *input, int n, int *out_index);
 

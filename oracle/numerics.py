@@ -191,6 +191,17 @@ def rope_positions(q, k, head_dim, num_heads, num_kv_heads, positions, rope_dim,
     return q, k2
 
 
+def rope_with_freqs(q, k, freqs, head_dim, num_heads, num_kv_heads, seq_len, start_pos, neox):
+    """cpu.go:308-375; returns rotated copies (q, k)."""
+    q = _f32(q).copy()
+    k2 = None if k is None else _f32(k).copy()
+    f = _f32(freqs)
+    assert f.size >= head_dim // 2
+    _lib.vxo_rope_with_freqs(_p(q), None if k2 is None else _p(k2), _p(f), head_dim, num_heads, num_kv_heads, seq_len,
+                             start_pos, int(bool(neox)))
+    return q, k2
+
+
 def rope_shift(k, head_dim, num_kv_heads, num_tokens, shift, theta):
     """backend/cpu/backend.go:244-276; returns the rotated copy."""
     k2 = _f32(k).copy()
@@ -211,6 +222,45 @@ def silu_mul(gate, up):
     out = np.empty_like(gate)
     _lib.vxo_silu_mul(_p(gate), _p(up), _p(out), C.c_int64(gate.size))
     return out
+
+
+def layernorm(x, weight, bias, rows, cols, eps):
+    """cpu.go:404-436"""
+    x, weight, bias = _f32(x), _f32(weight), _f32(bias)
+    out = np.empty((rows, cols), dtype=np.float32)
+    _lib.vxo_layernorm(_p(x), _p(weight), _p(bias), _p(out), rows, cols, C.c_float(eps))
+    return out
+
+
+def gelu(x):
+    """cpu.go:440-454"""
+    x = _f32(x)
+    out = np.empty_like(x)
+    _lib.vxo_gelu(_p(x), _p(out), C.c_int64(x.size))
+    return out
+
+
+def gelu_mul(gate, up):
+    """cpu.go:457-473"""
+    gate, up = _f32(gate), _f32(up)
+    out = np.empty_like(gate)
+    _lib.vxo_gelu_mul(_p(gate), _p(up), _p(out), C.c_int64(gate.size))
+    return out
+
+
+def add_bias(x, bias, rows, cols):
+    """cpu.go:476-487"""
+    x, bias = _f32(x), _f32(bias)
+    out = np.empty((rows, cols), dtype=np.float32)
+    _lib.vxo_add_bias(_p(x), _p(bias), _p(out), rows, cols)
+    return out
+
+
+def scale_buffer(buf, scale):
+    """cpu.go:558-563; returns the scaled copy."""
+    b = _f32(buf).copy()
+    _lib.vxo_scale_buffer(_p(b), C.c_float(scale), C.c_int64(b.size))
+    return b
 
 
 def softmax(x, rows, cols):
@@ -266,6 +316,24 @@ def sdpa_prefill(q, k, v, seq_len, num_q_heads, num_kv_heads, head_dim, scale):
     out = np.empty((seq_len, num_q_heads, head_dim), dtype=np.float32)
     _lib.vxo_sdpa_prefill(_p(q), _p(k), _p(v), _p(out), seq_len, num_q_heads, num_kv_heads, head_dim,
                           C.c_float(scale))
+    return out
+
+
+def sdpa_softcap(q, k, v, kv_len, num_q_heads, num_kv_heads, head_dim, scale, softcap, kv_head_stride):
+    """cpu.go:705-765"""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    out = np.empty((num_q_heads, head_dim), dtype=np.float32)
+    _lib.vxo_sdpa_softcap(_p(q), _p(k), _p(v), _p(out), kv_len, num_q_heads, num_kv_heads, head_dim,
+                          C.c_float(scale), C.c_float(softcap), kv_head_stride)
+    return out
+
+
+def sdpa_prefill_softcap(q, k, v, seq_len, num_q_heads, num_kv_heads, head_dim, scale, softcap):
+    """cpu.go:770-841"""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    out = np.empty((seq_len, num_q_heads, head_dim), dtype=np.float32)
+    _lib.vxo_sdpa_prefill_softcap(_p(q), _p(k), _p(v), _p(out), seq_len, num_q_heads, num_kv_heads, head_dim,
+                                  C.c_float(scale), C.c_float(softcap))
     return out
 
 

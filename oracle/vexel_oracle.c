@@ -545,6 +545,31 @@ VXO_API void vxo_rope_shift(float *k, int head_dim, int num_kv_heads, int num_to
         }
 }
 
+static void rope_freqs_one(float *data, int64_t total_vectors, int heads, int head_dim, int start_pos,
+                           const float *freqs, int neox) {
+    int half = head_dim / 2;
+    for (int64_t i = 0; i < total_vectors; i++) {
+        int pos = start_pos + (int)(i / heads);
+        int64_t off = i * head_dim;
+        for (int j = 0; j < half; j++) {
+            int i0 = neox ? j : 2 * j, i1 = neox ? j + half : 2 * j + 1;
+            float angle = (float)pos * freqs[j];
+            float c = (float)cos((double)angle), sn = (float)sin((double)angle);
+            float v1 = data[off + i0], v2 = data[off + i1];
+            data[off + i0] = v1 * c - v2 * sn;
+            data[off + i1] = v1 * sn + v2 * c;
+        }
+    }
+}
+
+/* inference/backend/cpu/cpu.go:308-375 (RoPEWithFreqs): RoPE over the whole head with the inverse frequency of
+ * pair j read from freqs[j] (head_dim / 2 values) instead of computed from theta. k may be NULL. */
+VXO_API void vxo_rope_with_freqs(float *q, float *k, const float *freqs, int head_dim, int num_heads, int num_kv_heads,
+                                 int seq_len, int start_pos, int neox) {
+    rope_freqs_one(q, (int64_t)seq_len * num_heads, num_heads, head_dim, start_pos, freqs, neox);
+    if (k) rope_freqs_one(k, (int64_t)seq_len * num_kv_heads, num_kv_heads, head_dim, start_pos, freqs, neox);
+}
+
 /* inference/backend/cpu/cpu.go:378-387 */
 VXO_API void vxo_silu(const float *x, float *out, int64_t n) {
     for (int64_t i = 0; i < n; i++) {
@@ -561,6 +586,60 @@ VXO_API void vxo_silu_mul(const float *gate, const float *up, float *out, int64_
         float sg = 1.0f / (1.0f + (float)exp((double)(-g)));
         out[i] = (g * sg) * up[i];
     }
+}
+
+/* inference/backend/cpu/cpu.go:404-436 (LayerNorm): mean and variance by sequential float32 sums over the row,
+ * 1/sqrt in float64 rounded to float32, then ((x - mean) * invStd) * w + b. */
+VXO_API void vxo_layernorm(const float *x, const float *w, const float *b, float *out, int rows, int cols, float eps) {
+    for (int i = 0; i < rows; i++) {
+        int64_t off = (int64_t)i * cols;
+        float sum = 0;
+        for (int j = 0; j < cols; j++) sum += x[off + j];
+        float mean = sum / (float)cols;
+        float vs = 0;
+        for (int j = 0; j < cols; j++) {
+            float diff = x[off + j] - mean;
+            vs += diff * diff;
+        }
+        float variance = vs / (float)cols;
+        float inv_std = 1.0f / (float)sqrt((double)(variance + eps));
+        for (int j = 0; j < cols; j++) {
+            float normalized = (x[off + j] - mean) * inv_std;
+            out[off + j] = normalized * w[j] + b[j];
+        }
+    }
+}
+
+/* The tanh form of GELU as cpu.go:440-454 evaluates it: the untyped constants take float32 beside a float32
+ * operand, every product is float32, tanh is taken in float64 of the float32 argument. */
+static float gelu_one(float val) {
+    const float sqrt_two_pi = 0.7978845608f, coeff = 0.044715f;
+    float x3 = val * val * val;
+    float inner = coeff * x3;
+    float arg = sqrt_two_pi * (val + inner);
+    float th = (float)tanh((double)arg);
+    return 0.5f * val * (1.0f + th);
+}
+
+/* inference/backend/cpu/cpu.go:440-454 */
+VXO_API void vxo_gelu(const float *x, float *out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = gelu_one(x[i]);
+}
+
+/* inference/backend/cpu/cpu.go:457-473 (GELUMul): gelu(gate) * up */
+VXO_API void vxo_gelu_mul(const float *gate, const float *up, float *out, int64_t n) {
+    for (int64_t i = 0; i < n; i++) out[i] = gelu_one(gate[i]) * up[i];
+}
+
+/* inference/backend/cpu/cpu.go:476-487 (AddBias): out[r][c] = x[r][c] + bias[c] */
+VXO_API void vxo_add_bias(const float *x, const float *bias, float *out, int rows, int cols) {
+    for (int i = 0; i < rows; i++)
+        for (int j = 0; j < cols; j++) out[(int64_t)i * cols + j] = x[(int64_t)i * cols + j] + bias[j];
+}
+
+/* inference/backend/cpu/cpu.go:558-563 (ScaleBuffer), in place */
+VXO_API void vxo_scale_buffer(float *buf, float scale, int64_t n) {
+    for (int64_t i = 0; i < n; i++) buf[i] *= scale;
 }
 
 /* inference/backend/cpu/cpu.go:490-518 */
@@ -621,13 +700,16 @@ VXO_API int vxo_argmax(const float *x, int n) {
 
 /* One query head against kv_len (k,v) rows fetched through callbacks-free strided
  * access: k_at(p) = kbase + p*kstride. Body of inference/backend/cpu/cpu.go:589-630. */
-static void sdpa_head(const float *qh, float *oh, int kv_len, int head_dim, float scale,
-                      const float *const *krows, const float *const *vrows, float *scores) {
+static void sdpa_head_capped(const float *qh, float *oh, int kv_len, int head_dim, float scale, float softcap,
+                             const float *const *krows, const float *const *vrows, float *scores) {
     for (int p = 0; p < kv_len; p++) {
         const float *kv = krows[p];
         float dot = 0;
         for (int d = 0; d < head_dim; d++) dot += qh[d] * kv[d];
-        scores[p] = dot * scale;
+        float score = dot * scale;
+        /* cpu.go:735-737, 802-804: the only difference of the soft-capped forms */
+        if (softcap > 0) score = softcap * (float)tanh((double)(score / softcap));
+        scores[p] = score;
     }
     float mx = scores[0];
     for (int p = 0; p < kv_len; p++)
@@ -645,6 +727,11 @@ static void sdpa_head(const float *qh, float *oh, int kv_len, int head_dim, floa
         float w = scores[p];
         for (int d = 0; d < head_dim; d++) oh[d] += w * vv[d];
     }
+}
+
+static void sdpa_head(const float *qh, float *oh, int kv_len, int head_dim, float scale,
+                      const float *const *krows, const float *const *vrows, float *scores) {
+    sdpa_head_capped(qh, oh, kv_len, head_dim, scale, 0.0f, krows, vrows, scores);
 }
 
 /* inference/backend/cpu/cpu.go:568-632. K/V head-major [numKVHeads, stride/headDim, headDim]. */
@@ -685,6 +772,53 @@ VXO_API void vxo_sdpa_prefill(const float *q, const float *k, const float *v, fl
                 vr[p] = v + ((int64_t)p * num_kv_heads + kvh) * head_dim;
             }
             sdpa_head(q + qo, out + qo, mk, head_dim, scale, kr, vr, scores);
+        }
+    free(scores);
+    free(kr);
+    free(vr);
+}
+
+/* inference/backend/cpu/cpu.go:705-765 (SDPASoftCap): SDPA whose scaled scores pass through
+ * softcap * tanh(score / softcap) when softcap > 0. */
+VXO_API void vxo_sdpa_softcap(const float *q, const float *k, const float *v, float *out, int kv_len,
+                              int num_q_heads, int num_kv_heads, int head_dim, float scale, float softcap,
+                              int kv_head_stride) {
+    int hpk = num_q_heads / num_kv_heads;
+    size_t cap = (size_t)(kv_len > 0 ? kv_len : 1);
+    float *scores = (float *)malloc(cap * sizeof(float));
+    const float **kr = (const float **)malloc(cap * sizeof(float *));
+    const float **vr = (const float **)malloc(cap * sizeof(float *));
+    for (int h = 0; h < num_q_heads; h++) {
+        int64_t base = (int64_t)(h / hpk) * kv_head_stride;
+        for (int p = 0; p < kv_len; p++) {
+            kr[p] = k + base + (int64_t)p * head_dim;
+            vr[p] = v + base + (int64_t)p * head_dim;
+        }
+        sdpa_head_capped(q + (int64_t)h * head_dim, out + (int64_t)h * head_dim, kv_len, head_dim, scale, softcap, kr,
+                         vr, scores);
+    }
+    free(scores);
+    free(kr);
+    free(vr);
+}
+
+/* inference/backend/cpu/cpu.go:770-841 (SDPAPrefillSoftCap): causal, token-major. */
+VXO_API void vxo_sdpa_prefill_softcap(const float *q, const float *k, const float *v, float *out, int seq_len,
+                                      int num_q_heads, int num_kv_heads, int head_dim, float scale, float softcap) {
+    int hpk = num_q_heads / num_kv_heads;
+    size_t cap = (size_t)(seq_len > 0 ? seq_len : 1);
+    float *scores = (float *)malloc(cap * sizeof(float));
+    const float **kr = (const float **)malloc(cap * sizeof(float *));
+    const float **vr = (const float **)malloc(cap * sizeof(float *));
+    for (int qp = 0; qp < seq_len; qp++)
+        for (int h = 0; h < num_q_heads; h++) {
+            int kvh = h / hpk;
+            int64_t qo = ((int64_t)qp * num_q_heads + h) * head_dim;
+            for (int p = 0; p <= qp; p++) {
+                kr[p] = k + ((int64_t)p * num_kv_heads + kvh) * head_dim;
+                vr[p] = v + ((int64_t)p * num_kv_heads + kvh) * head_dim;
+            }
+            sdpa_head_capped(q + qo, out + qo, qp + 1, head_dim, scale, softcap, kr, vr, scores);
         }
     free(scores);
     free(kr);

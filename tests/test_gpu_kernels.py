@@ -1028,3 +1028,98 @@ def test_graph_capture_replays_match_eager(be):
     be.graph_destroy(g)
     for p in (dw, da, do, dn, nw):
         be.free(p)
+
+
+# ------------------------------------------------------------------ optional interfaces of other architectures
+def test_layernorm_gelu_bias_scale(be):
+    """LayerNormOps, GELUOps, BiasOps, ScaleOps (backend.go:205-263) against the oracle's restatement of the CPU
+    backend. The element-wise ones follow the reference's float32 operation order and are compared bit for bit."""
+    rng = np.random.default_rng(61)
+    for rows, cols in ((5, 2560), (3, 80), (1, 1)):
+        x = (rng.standard_normal((rows, cols)) * 2 + 0.5).astype(np.float32)
+        w = rng.standard_normal(cols).astype(np.float32)
+        b = rng.standard_normal(cols).astype(np.float32)
+        dx, dw, db = be.upload(x), be.upload(w), be.upload(b)
+        do = be.alloc(x.nbytes)
+        be.layernorm(dx, dw, db, do, rows, cols, 1e-5)
+        _close(be.download(do, x.shape, np.float32), nx.layernorm(x, w, b, rows, cols, 1e-5), 1e-5, 2e-6, "layernorm")
+        be.add_bias(dx, db, do, rows, cols)
+        assert np.array_equal(be.download(do, x.shape, np.float32), nx.add_bias(x, b, rows, cols))
+        be.add_bias(dx, db, dx, rows, cols)                          # in place
+        assert np.array_equal(be.download(dx, x.shape, np.float32), nx.add_bias(x, b, rows, cols))
+    n = 100003
+    g = np.concatenate([(rng.standard_normal(n - 6) * 3), [0.0, -0.0, 40.0, -40.0, 1e-20, 9.5]]).astype(np.float32)
+    u = rng.standard_normal(n).astype(np.float32)
+    dg, du = be.upload(g), be.upload(u)
+    do = be.alloc(n * 4)
+    be.gelu(dg, do, n)
+    got, want = be.download(do, (n,), np.float32), nx.gelu(g)
+    _close(got, want, 2e-7, 1e-9, "gelu")
+    assert np.mean(got.view(np.uint32) == want.view(np.uint32)) > 0.999
+    be.gelu_mul(dg, du, do, n)
+    _close(be.download(do, (n,), np.float32), nx.gelu_mul(g, u), 2e-7, 1e-9, "gelu_mul")
+    be.scale_buffer(du, float(np.float32(math.sqrt(2304.0))), n)
+    assert np.array_equal(be.download(du, (n,), np.float32), nx.scale_buffer(u, np.float32(math.sqrt(2304.0))))
+    be.gelu(dg, do, 0)                                              # nothing to do
+    be.reset_pool()
+
+
+@pytest.mark.parametrize("hq,hk,d,n,cap", [(8, 4, 256, 300, 30.0), (1, 1, 4, 4, 5.0), (32, 8, 128, 1500, 50.0),
+                                            (4, 4, 80, 33, 0.0)])
+def test_sdpa_softcap(be, hq, hk, d, n, cap):
+    """SDPASoftCap (backend.go:235, cpu.go:705-765): Gemma 2's geometry (heads of 256, cap 30), the reference
+    test's 4-key case, a context longer than one chunk of the kernel, and cap 0 = plain SDPA."""
+    rng = np.random.default_rng(62 + n)
+    q = (rng.standard_normal((hq, d)) * 3).astype(np.float32)
+    k = (rng.standard_normal((hk, n, d)) * 3).astype(np.float32)
+    v = rng.standard_normal((hk, n, d)).astype(np.float32)
+    sc = float(np.float32(1 / math.sqrt(d)))
+    dq, dk, dv = be.upload(q), be.upload(k), be.upload(v)
+    do = be.alloc(q.nbytes)
+    be.sdpa_softcap(dq, dk, dv, do, n, hq, hk, d, sc, cap, n * d)
+    want = nx.sdpa_softcap(q, k, v, n, hq, hk, d, sc, cap, n * d)
+    _close(be.download(do, q.shape, np.float32), want, 1e-5, 3e-6, "sdpa_softcap")
+    if cap > 0:
+        assert np.abs(want - nx.sdpa(q, k, v, n, hq, hk, d, sc, n * d)).max() > 1e-3   # the cap mattered
+    be.reset_pool()
+
+
+@pytest.mark.parametrize("hq,hk,d,s,cap", [(4, 2, 128, 70, 50.0), (8, 4, 64, 33, 30.0), (8, 4, 256, 40, 50.0),
+                                            (4, 2, 128, 70, 0.0)])
+def test_sdpa_prefill_softcap(be, hq, hk, d, s, cap):
+    """SDPAPrefillSoftCap (backend.go:239, cpu.go:770-841) on the MFMA kernel (heads of 64 / 128) and the generic
+    one (256), with scores well into the curved part of the cap."""
+    rng = np.random.default_rng(63 + s + d)
+    q = (rng.standard_normal((s, hq, d)) * 3).astype(np.float32)
+    k = (rng.standard_normal((s, hk, d)) * 3).astype(np.float32)
+    v = rng.standard_normal((s, hk, d)).astype(np.float32)
+    sc = float(np.float32(1 / math.sqrt(d)))
+    dq, dk, dv = be.upload(q), be.upload(k), be.upload(v)
+    do = be.alloc(q.nbytes)
+    be.sdpa_prefill_softcap(dq, dk, dv, do, s, hq, hk, d, sc, cap)
+    want = nx.sdpa_prefill_softcap(q, k, v, s, hq, hk, d, sc, cap)
+    # scores reach tens here (inputs scaled by 3): a float32 rounding of a score of 30 moves its weight by 2e-6
+    _close(be.download(do, q.shape, np.float32), want, 5e-5, 2e-5, "sdpa_prefill_softcap")
+    if cap > 0:
+        assert np.abs(want - nx.sdpa_prefill(q, k, v, s, hq, hk, d, sc)).max() > 1e-3
+    be.reset_pool()
+
+
+@pytest.mark.parametrize("neox", [False, True])
+def test_rope_with_freqs(be, neox):
+    """ScaledRoPEOps.RoPEWithFreqs (backend.go:247-249, cpu.go:308-375) with frequencies that no theta gives
+    (scaled_rope_test.go:134-138), with and without K."""
+    rng = np.random.default_rng(64)
+    d, hq, hk, s, start = 64, 8, 4, 5, 1000
+    freqs = (0.01 * np.arange(1, d // 2 + 1)).astype(np.float32)
+    q = rng.standard_normal((s, hq, d)).astype(np.float32)
+    k = rng.standard_normal((s, hk, d)).astype(np.float32)
+    wq, wk = nx.rope_with_freqs(q, k, freqs, d, hq, hk, s, start, neox)
+    dq, dk, df = be.upload(q), be.upload(k), be.upload(freqs)
+    be.rope_with_freqs(dq, dk, df, d, hq, hk, s, start, neox)
+    _close(be.download(dq, q.shape, np.float32), wq, 0, 1e-6, "rope_with_freqs q")
+    _close(be.download(dk, k.shape, np.float32), wk, 0, 1e-6, "rope_with_freqs k")
+    dq = be.upload(q)
+    be.rope_with_freqs(dq, None, df, d, hq, hk, s, start, neox)
+    _close(be.download(dq, q.shape, np.float32), wq, 0, 1e-6, "rope_with_freqs, no k")
+    be.reset_pool()

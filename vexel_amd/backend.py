@@ -150,6 +150,33 @@ class HipBackend:
     def sdpa_prefill(self, q, k, v, out, seq_len, num_q_heads, num_kv_heads, head_dim, scale):
         self.call("vx_sdpa_prefill", q, k, v, out, seq_len, num_q_heads, num_kv_heads, head_dim, scale)
 
+    # ---- optional interfaces (backend.go:205-263)
+    def layernorm(self, x, weight, bias, out, rows, cols, eps):
+        self.call("vx_layernorm", x, weight, bias, out, rows, cols, eps)
+
+    def gelu(self, x, out, n):
+        self.call("vx_gelu", x, out, n)
+
+    def gelu_mul(self, gate, up, out, n):
+        self.call("vx_gelu_mul", gate, up, out, n)
+
+    def add_bias(self, x, bias, out, rows, cols):
+        self.call("vx_add_bias", x, bias, out, rows, cols)
+
+    def scale_buffer(self, buf, scale, n):
+        self.call("vx_scale_buffer", buf, scale, n)
+
+    def sdpa_softcap(self, q, k, v, out, kv_len, num_q_heads, num_kv_heads, head_dim, scale, softcap, kv_head_stride):
+        self.call("vx_sdpa_softcap", q, k, v, out, kv_len, num_q_heads, num_kv_heads, head_dim, scale, softcap,
+                  kv_head_stride)
+
+    def sdpa_prefill_softcap(self, q, k, v, out, seq_len, num_q_heads, num_kv_heads, head_dim, scale, softcap):
+        self.call("vx_sdpa_prefill_softcap", q, k, v, out, seq_len, num_q_heads, num_kv_heads, head_dim, scale, softcap)
+
+    def rope_with_freqs(self, q, k, freqs, head_dim, num_heads, num_kv_heads, seq_len, start_pos, neox):
+        self.call("vx_rope_with_freqs", q, k, freqs, head_dim, num_heads, num_kv_heads, seq_len, start_pos,
+                  int(bool(neox)))
+
     def argmax(self, inp, n):
         r = C.c_int()
         self.call("vx_argmax", inp, n, C.byref(r))

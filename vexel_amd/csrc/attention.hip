@@ -35,6 +35,7 @@ struct AttnParams {
     int f16;
     int num_q_heads, num_kv_heads, head_dim;
     float scale;
+    float softcap;  // > 0: scaled scores pass through softcap * tanh(score / softcap) (cpu.go:735-737)
     // contiguous
     int kv_head_stride;
     int kv_len;  // fixed kv length (contiguous, single paged decode); ignored when kv_lens != nullptr
@@ -121,6 +122,7 @@ __global__ void __launch_bounds__(GEN_THREADS) attn_generic_kernel(AttnParams p)
                 float dot = 0.f;
                 for (int d = 0; d < D; d++) dot = fmaf(s_q[d], ld_elem(p.k, kb + d, p.f16), dot);
                 sc = dot * p.scale;
+                if (p.softcap > 0.f) sc = p.softcap * (float)tanh((double)(sc / p.softcap));
             }
             s_scores[i] = sc;
             lmax = fmaxf(lmax, sc);
@@ -462,10 +464,13 @@ __device__ __forceinline__ float row16_max(float t) {  // max over the 16 lanes 
     return t;
 }
 
-template <int D>
+// CAP: the scores (held in log2 units, score * log2 e) pass through cap2 * tanh(. / cap2) with
+// cap2 = softcap * log2 e, which is softcap * tanh(score / softcap) in those units.
+template <int D, bool CAP = false>
 __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restrict__ q, const float *__restrict__ k,
                                                           const float *__restrict__ v, float *__restrict__ out, int S,
-                                                          int num_q_heads, int num_kv_heads, float scale) {
+                                                          int num_q_heads, int num_kv_heads, float scale,
+                                                          float softcap = 0.f) {
     constexpr int KP = D + 4, VP = D + 16, PP = FA_BK + 4;
     __shared__ __attribute__((aligned(16))) float Ks[FA_BK * KP];
     __shared__ __attribute__((aligned(16))) float Vs[FA_BK * VP];
@@ -520,6 +525,13 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
 #pragma unroll
             for (int s = 0; s < D / 4; s++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[s], kb[4 * s], acc, 0, 0, 0);
             sc[cb] = acc;
+        }
+        if (CAP) {
+            const float cap2 = softcap * kLog2e, inv_cap2 = 1.f / cap2;
+#pragma unroll
+            for (int cb = 0; cb < FA_BK / 16; cb++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) sc[cb][i] = cap2 * tanhf(sc[cb][i] * inv_cap2);
         }
         // causal mask, online softmax per row
         float alpha[4];
@@ -676,12 +688,14 @@ int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16
 
 extern "C" {
 
-int vx_sdpa(vx_backend *be, const float *q, const float *k, const float *v, float *out, int kv_len, int num_q_heads,
-            int num_kv_heads, int head_dim, float scale, int kv_head_stride) {
+static int sdpa_dense(vx_backend *be, const float *q, const float *k, const float *v, float *out, int kv_len,
+                      int num_q_heads, int num_kv_heads, int head_dim, float scale, float softcap, int kv_head_stride) {
     int rc = enter(be);
     if (rc) return rc;
     VX_REQUIRE(q && k && v && out && kv_len >= 1, "vx_sdpa: bad arguments");
+    VX_REQUIRE(softcap >= 0.f, "vx_sdpa_softcap: negative softcap");
     AttnParams p = {};
+    p.softcap = softcap;
     p.q = q;
     p.out = out;
     p.k = k;
@@ -696,16 +710,32 @@ int vx_sdpa(vx_backend *be, const float *q, const float *k, const float *v, floa
     return run_generic(be, p, 1);
 }
 
-int vx_sdpa_prefill(vx_backend *be, const float *q, const float *k, const float *v, float *out, int seq_len,
-                    int num_q_heads, int num_kv_heads, int head_dim, float scale) {
+int vx_sdpa(vx_backend *be, const float *q, const float *k, const float *v, float *out, int kv_len, int num_q_heads,
+            int num_kv_heads, int head_dim, float scale, int kv_head_stride) {
+    return sdpa_dense(be, q, k, v, out, kv_len, num_q_heads, num_kv_heads, head_dim, scale, 0.f, kv_head_stride);
+}
+
+int vx_sdpa_softcap(vx_backend *be, const float *q, const float *k, const float *v, float *out, int kv_len,
+                    int num_q_heads, int num_kv_heads, int head_dim, float scale, float softcap, int kv_head_stride) {
+    return sdpa_dense(be, q, k, v, out, kv_len, num_q_heads, num_kv_heads, head_dim, scale, softcap, kv_head_stride);
+}
+
+static int sdpa_prefill_dense(vx_backend *be, const float *q, const float *k, const float *v, float *out, int seq_len,
+                              int num_q_heads, int num_kv_heads, int head_dim, float scale, float softcap) {
     int rc = enter(be);
     if (rc) return rc;
     VX_REQUIRE(q && k && v && out && seq_len >= 0, "vx_sdpa_prefill: bad arguments");
     VX_REQUIRE(num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, "vx_sdpa_prefill: bad head counts");
+    VX_REQUIRE(softcap >= 0.f, "vx_sdpa_prefill_softcap: negative softcap");
     if (seq_len == 0) return VX_OK;
     if ((head_dim == 64 || head_dim == 128) && ((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0) {
         const dim3 grid(ceil_div(seq_len, FA_BQ), num_q_heads);
-        if (head_dim == 128)
+        if (softcap > 0.f) {
+            if (head_dim == 128)
+                prefill_fa2_kernel<128, true><<<grid, 256, 0, be->stream>>>(q, k, v, out, seq_len, num_q_heads, num_kv_heads, scale, softcap);
+            else
+                prefill_fa2_kernel<64, true><<<grid, 256, 0, be->stream>>>(q, k, v, out, seq_len, num_q_heads, num_kv_heads, scale, softcap);
+        } else if (head_dim == 128)
             prefill_fa2_kernel<128><<<grid, 256, 0, be->stream>>>(q, k, v, out, seq_len, num_q_heads, num_kv_heads, scale);
         else
             prefill_fa2_kernel<64><<<grid, 256, 0, be->stream>>>(q, k, v, out, seq_len, num_q_heads, num_kv_heads, scale);
@@ -713,6 +743,7 @@ int vx_sdpa_prefill(vx_backend *be, const float *q, const float *k, const float 
         return VX_OK;
     }
     AttnParams p = {};
+    p.softcap = softcap;
     p.q = q;
     p.out = out;
     p.k = k;
@@ -723,6 +754,16 @@ int vx_sdpa_prefill(vx_backend *be, const float *q, const float *k, const float 
     p.head_dim = head_dim;
     p.scale = scale;
     return run_generic(be, p, seq_len);
+}
+
+int vx_sdpa_prefill(vx_backend *be, const float *q, const float *k, const float *v, float *out, int seq_len,
+                    int num_q_heads, int num_kv_heads, int head_dim, float scale) {
+    return sdpa_prefill_dense(be, q, k, v, out, seq_len, num_q_heads, num_kv_heads, head_dim, scale, 0.f);
+}
+
+int vx_sdpa_prefill_softcap(vx_backend *be, const float *q, const float *k, const float *v, float *out, int seq_len,
+                            int num_q_heads, int num_kv_heads, int head_dim, float scale, float softcap) {
+    return sdpa_prefill_dense(be, q, k, v, out, seq_len, num_q_heads, num_kv_heads, head_dim, scale, softcap);
 }
 
 static int paged_single(vx_backend *be, const float *q, const void *kv_pool, int f16, const int32_t *block_table,

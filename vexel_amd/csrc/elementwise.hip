@@ -181,6 +181,78 @@ __global__ void mul_kernel(const float *a, const float *b, float *out, int n) {
     if (i < n) out[i] = a[i] * b[i];
 }
 
+// ---------------------------------------------------------------- LayerNorm (cpu.go:404-436)
+__global__ void __launch_bounds__(kThreads) layernorm_kernel(const float *x, const float *w, const float *b, float *out,
+                                                             int cols, float eps) {
+    __shared__ float sm[kThreads / 64];
+    const float *xr = x + (size_t)blockIdx.x * cols;
+    float *orow = out + (size_t)blockIdx.x * cols;
+    float s = 0.f;
+    for (int j = threadIdx.x; j < cols; j += kThreads) s += xr[j];
+    const float mean = block_sum(s, sm) / (float)cols;
+    float vs = 0.f;
+    for (int j = threadIdx.x; j < cols; j += kThreads) {
+        const float d = xr[j] - mean;
+        vs = fmaf(d, d, vs);
+    }
+    const float variance = block_sum(vs, sm) / (float)cols;
+    const float inv_std = 1.0f / (float)sqrt((double)(variance + eps));
+    for (int j = threadIdx.x; j < cols; j += kThreads) orow[j] = (xr[j] - mean) * inv_std * w[j] + b[j];
+}
+
+// ---------------------------------------------------------------- GELU, tanh form (cpu.go:440-473)
+__device__ __forceinline__ float gelu_ref(float v) {
+    // plain operators under contract(off): v + 0.044715 x^3 stays a product and a sum as in the reference (the
+    // __f*_rn helpers are ordinary inline functions whose operations the compiler still fuses)
+#pragma clang fp contract(off)
+    const float x3 = v * v * v;
+    const float arg = 0.7978845608f * (v + 0.044715f * x3);
+    const float th = (float)tanh((double)arg);
+    return 0.5f * v * (1.0f + th);
+}
+
+__global__ void gelu_kernel(const float *x, float *out, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = gelu_ref(x[i]);
+}
+
+__global__ void gelu_mul_kernel(const float *g, const float *u, float *out, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = __fmul_rn(gelu_ref(g[i]), u[i]);
+}
+
+// cpu.go:476-487: out[r][c] = x[r][c] + bias[c]; n = rows * cols
+__global__ void add_bias_kernel(const float *x, const float *bias, float *out, int cols, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = x[i] + bias[i % cols];
+}
+
+// cpu.go:558-563
+__global__ void scale_kernel(float *buf, float scale, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) buf[i] = __fmul_rn(buf[i], scale);
+}
+
+// cpu.go:308-375: RoPE over the whole head, pair j turning by position * freqs[j]. grid.x = row.
+__global__ void rope_freqs_kernel(float *q, float *k, const float *freqs, int head_dim, int num_heads, int num_kv_heads,
+                                  int start_pos, int neox) {
+    const int row = blockIdx.x, half = head_dim / 2;
+    const int pos = start_pos + row;
+    for (int j = threadIdx.x; j < half; j += blockDim.x) {
+        const float angle = __fmul_rn((float)pos, freqs[j]);
+        RopeCS cs;
+        cs.c = (float)cos((double)angle);
+        cs.s = (float)sin((double)angle);
+        const int i0 = neox ? j : 2 * j, i1 = neox ? j + half : 2 * j + 1;
+        float *qr = q + (size_t)row * num_heads * head_dim;
+        for (int h = 0; h < num_heads; h++) rope_pair(qr[h * head_dim + i0], qr[h * head_dim + i1], cs);
+        if (k) {
+            float *kr = k + (size_t)row * num_kv_heads * head_dim;
+            for (int h = 0; h < num_kv_heads; h++) rope_pair(kr[h * head_dim + i0], kr[h * head_dim + i1], cs);
+        }
+    }
+}
+
 // ---------------------------------------------------------------- Softmax (cpu.go:490-518)
 __global__ void __launch_bounds__(kThreads) softmax_kernel(const float *x, float *out, int cols) {
     __shared__ float sm[kThreads / 64];
@@ -539,6 +611,58 @@ int vx_silu(vx_backend *be, const float *x, float *out, int n) {
 int vx_silu_mul(vx_backend *be, const float *gate, const float *up, float *out, int n) {
     VX_REQUIRE(gate && up && out, "vx_silu_mul: null pointer");
     VX_EW("vx_silu_mul", silu_mul_kernel, gate, up, out)
+}
+
+int vx_gelu(vx_backend *be, const float *x, float *out, int n) {
+    VX_REQUIRE(x && out, "vx_gelu: null pointer");
+    VX_EW("vx_gelu", gelu_kernel, x, out)
+}
+
+int vx_gelu_mul(vx_backend *be, const float *gate, const float *up, float *out, int n) {
+    VX_REQUIRE(gate && up && out, "vx_gelu_mul: null pointer");
+    VX_EW("vx_gelu_mul", gelu_mul_kernel, gate, up, out)
+}
+
+int vx_scale_buffer(vx_backend *be, float *buf, float scale, int n) {
+    VX_REQUIRE(buf, "vx_scale_buffer: null pointer");
+    VX_EW("vx_scale_buffer", scale_kernel, buf, scale)
+}
+
+int vx_add_bias(vx_backend *be, const float *x, const float *bias, float *out, int rows, int cols) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(x && bias && out && rows >= 0 && cols > 0, "vx_add_bias: bad arguments");
+    VX_REQUIRE((int64_t)rows * cols <= INT32_MAX, "vx_add_bias: %d x %d elements exceed 2^31", rows, cols);
+    const int n = rows * cols;
+    if (n == 0) return VX_OK;
+    add_bias_kernel<<<grid1d(n, kThreads), kThreads, 0, be->stream>>>(x, bias, out, cols, n);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_layernorm(vx_backend *be, const float *x, const float *weight, const float *bias, float *out, int rows, int cols,
+                 float eps) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(x && weight && bias && out && rows >= 0 && cols > 0, "vx_layernorm: bad arguments");
+    if (rows == 0) return VX_OK;
+    layernorm_kernel<<<rows, kThreads, 0, be->stream>>>(x, weight, bias, out, cols, eps);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_rope_with_freqs(vx_backend *be, float *q, float *k, const float *freqs, int head_dim, int num_heads,
+                       int num_kv_heads, int seq_len, int start_pos, int rope_neox) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && freqs && head_dim > 0 && head_dim % 2 == 0 && num_heads > 0 && seq_len >= 0 && (!k || num_kv_heads > 0),
+               "vx_rope_with_freqs: bad arguments");
+    if (seq_len == 0) return VX_OK;
+    int threads = head_dim / 2 < 64 ? 64 : (head_dim / 2 > 256 ? 256 : head_dim / 2);
+    rope_freqs_kernel<<<seq_len, threads, 0, be->stream>>>(q, k, freqs, head_dim, num_heads, num_kv_heads, start_pos,
+                                                           rope_neox);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
 }
 
 int vx_add(vx_backend *be, const float *a, const float *b, float *out, int n) {

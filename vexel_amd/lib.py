@@ -42,6 +42,14 @@ SIGNATURES = {
     "vx_sdpa": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i]),
     "vx_sdpa_prefill": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f]),
     "vx_argmax": (_i, [_vp, _vp, _i, C.POINTER(_i)]),
+    "vx_layernorm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f]),
+    "vx_gelu": (_i, [_vp, _vp, _vp, _i]),
+    "vx_gelu_mul": (_i, [_vp, _vp, _vp, _vp, _i]),
+    "vx_add_bias": (_i, [_vp, _vp, _vp, _vp, _i, _i]),
+    "vx_scale_buffer": (_i, [_vp, _vp, _f, _i]),
+    "vx_sdpa_softcap": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _f, _i]),
+    "vx_sdpa_prefill_softcap": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _f]),
+    "vx_rope_with_freqs": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i]),
     "vx_matmul_q4_0": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "vx_matmul_q4_k": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "vx_matmul_q6_k": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
