@@ -1,8 +1,9 @@
 """The reference's layer and decode drivers, chained from the oracle kernels
 (TEST INFRASTRUCTURE ONLY).
 
-  OracleModel.execute_with_paged_kv  inference/runtime/block.go:763-1081 (LLaMA arm:
-                                     RMSNorm, SwiGLU, serial residual, no bias)
+  OracleModel.execute_with_paged_kv  inference/runtime/block.go:763-1081 (every arm: RMSNorm / LayerNorm, SwiGLU /
+                                     GELU / GeGLU, serial / parallel residual, biases, partial and NeoX RoPE,
+                                     post-norms, the soft-capped first prefill chunk)
   OracleModel.decode_with_paged_kv   inference/runtime/decode.go:339-461
   OracleModel.decode_batched         inference/runtime/decode.go:612-654 (sequential loop)
   OracleModel.prefill_with_paged_kv  inference/runtime/decode.go:961-1096
@@ -14,7 +15,7 @@ inference/runtime/gpu_block_pool.go:15-19,107-108.
 """
 import math
 from dataclasses import dataclass
-from typing import List
+from typing import List, Optional
 
 import numpy as np
 
@@ -34,6 +35,15 @@ class ModelConfig:
     eps: float = 1e-5
     rope_theta: float = 10000.0
     block_size: int = 16  # inference/runtime/model.go:321
+    # the architecture switches of runtime/config.go:14-62,120-131 and block.go:245-254,339-340; the defaults are LLaMA
+    norm_type: str = "rms"            # "rms" | "layer" (NormType)
+    mlp_type: str = "swiglu"          # "swiglu" | "gelu" | "geglu" (MLPType)
+    parallel_residual: bool = False   # x + attn(norm(x)) + mlp(norm(x))
+    rope_dim: int = 0                 # rotated dimensions, 0 = the whole head
+    rope_neox: bool = False           # pairs (j, j + half) instead of (2j, 2j+1)
+    attn_softcap: float = 0.0         # AttentionLogitSoftCap
+    post_norms: bool = False          # HasPostNorms
+    embedding_scale: float = 0.0      # EmbeddingScale, <= 0 = none (decode.go:197-205)
 
 
 @dataclass
@@ -53,8 +63,19 @@ class LayerWeights:
     wo: QWeight
     ffn_norm: np.ndarray
     w1: QWeight
-    w3: QWeight
+    w3: Optional[QWeight]                     # unused by the GELU MLP (block.go:265)
     w2: QWeight
+    # block.go:266-283: LayerNorm biases, projection biases, Gemma 2's post-norms; None = the tensor is absent
+    attn_norm_bias: Optional[np.ndarray] = None
+    ffn_norm_bias: Optional[np.ndarray] = None
+    wq_bias: Optional[np.ndarray] = None
+    wk_bias: Optional[np.ndarray] = None
+    wv_bias: Optional[np.ndarray] = None
+    wo_bias: Optional[np.ndarray] = None
+    w1_bias: Optional[np.ndarray] = None
+    w2_bias: Optional[np.ndarray] = None
+    post_attn_norm: Optional[np.ndarray] = None
+    post_ffn_norm: Optional[np.ndarray] = None
 
 
 def _mm(a, w: QWeight, m):
@@ -65,10 +86,20 @@ def _mm(a, w: QWeight, m):
     return nx.matmul_quant(w.fmt, a, w.data, m, w.n, w.k)
 
 
+def _mm_bias(a, w: QWeight, bias, m):
+    """block.go:555-560 (matMulTransposedWithBias): the product, then AddBias when the bias tensor exists."""
+    out = _mm(a, w, m)
+    return out if bias is None else nx.add_bias(out, bias, m, w.n)
+
+
 class OracleModel:
     def __init__(self, cfg: ModelConfig, embedding_f32, layers: List[LayerWeights], final_norm,
-                 lm_head: QWeight, max_blocks, kv_fp16=True):
+                 lm_head: QWeight, max_blocks, kv_fp16=True, final_norm_bias=None):
         self.cfg = cfg
+        # block.go:972-976 keeps the attention output in the buffer the gated MLPs write W3's product to: the
+        # parallel residual exists for the GELU MLP only
+        assert not cfg.parallel_residual or cfg.mlp_type == "gelu"
+        self.final_norm_bias = final_norm_bias
         self.embedding = np.ascontiguousarray(embedding_f32, dtype=np.float32)
         self.layers = layers
         self.final_norm = final_norm
@@ -80,43 +111,77 @@ class OracleModel:
         self.kv = [np.zeros(elems, dtype=dt) for _ in range(cfg.num_layers)]
 
     # ---------------------------------------------------------------- one layer
+    def _norm(self, x, weight, bias, rows):
+        """block.go:562-576 (applyNorm): LayerNorm with its bias, or RMSNorm, which ignores the bias."""
+        c = self.cfg
+        if c.norm_type == "layer":
+            b = bias if bias is not None else np.zeros(c.hidden, dtype=np.float32)
+            return nx.layernorm(x, weight, b, rows, c.hidden, c.eps)
+        return nx.rmsnorm(x, weight, rows, c.hidden, c.eps)
+
+    def _mlp(self, norm, lw, seq_len):
+        """block.go:1001-1063: the GELU MLP with biases, or the gated one (SiLU or GELU gate) without."""
+        c = self.cfg
+        if c.mlp_type == "gelu":
+            gate = nx.gelu(_mm_bias(norm, lw.w1, lw.w1_bias, seq_len))         # :1010-1021
+            return _mm_bias(gate, lw.w2, lw.w2_bias, seq_len)                  # :1036
+        gate = _mm(norm, lw.w1, seq_len)                                       # :1043-1050
+        up = _mm(norm, lw.w3, seq_len)
+        act = nx.gelu_mul(gate, up) if c.mlp_type == "geglu" else nx.silu_mul(gate, up)  # :1051-1056
+        return _mm(act, lw.w2, seq_len)                                        # :1058-1061
+
     def execute_with_paged_kv(self, x, seq_id, layer_idx, start_pos):
         """x [seqLen, hidden] float32, updated copy returned. block.go:763-1081."""
         c = self.cfg
         lw = self.layers[layer_idx]
         seq_len = x.shape[0]
-        norm = nx.rmsnorm(x, lw.attn_norm, seq_len, c.hidden, c.eps)           # :834-837
-        q = _mm(norm, lw.wq, seq_len)                                          # :841-854
-        k = _mm(norm, lw.wk, seq_len)
-        v = _mm(norm, lw.wv, seq_len)
-        q, k = nx.rope(q, k, c.head_dim, c.num_heads, c.num_kv_heads, seq_len, start_pos, 0,
-                       c.rope_theta, False)                                    # :858
+        norm = self._norm(x, lw.attn_norm, lw.attn_norm_bias, seq_len)         # :834-837
+        q = _mm_bias(norm, lw.wq, lw.wq_bias, seq_len)                         # :841-854
+        k = _mm_bias(norm, lw.wk, lw.wk_bias, seq_len)
+        v = _mm_bias(norm, lw.wv, lw.wv_bias, seq_len)
+        q, k = nx.rope(q, k, c.head_dim, c.num_heads, c.num_kv_heads, seq_len, start_pos, c.rope_dim,
+                       c.rope_theta, c.rope_neox)                              # :858 (applyRoPE, :497-503)
         scale = np.float32(1.0 / math.sqrt(float(c.head_dim)))                 # :862
         slots = self.pool.store_kv_slots(layer_idx, seq_id, start_pos, seq_len)  # :868 / :878
         bi = [s[0] for s in slots]
         bo = [s[1] for s in slots]
         nx.reshape_paged_kv(k, self.kv[layer_idx], bi, bo, c.num_kv_heads, c.head_dim, c.block_size, False)
         nx.reshape_paged_kv(v, self.kv[layer_idx], bi, bo, c.num_kv_heads, c.head_dim, c.block_size, True)
-        if seq_len == 1:                                                       # :866-874
+        if seq_len == 1:                                                       # :866-874 (no soft cap on this arm)
             bt, nb, til = self.pool.attention_args(layer_idx, seq_id)
             attn = nx.sdpa_paged_decode(q, self.kv[layer_idx], bt, nb, c.block_size, c.num_heads,
                                         c.num_kv_heads, c.head_dim, scale, til).reshape(1, -1)
-        elif start_pos > 0:                                                    # :881-890
+        elif start_pos > 0:                                                    # :881-890 (nor on this one)
             kv_lens = [start_pos + i + 1 for i in range(seq_len)]
             bt = self.pool.seqs[seq_id].block_tables[layer_idx]
             attn = nx.sdpa_paged_multiquery(q, self.kv[layer_idx], bt, kv_lens, c.block_size, c.num_heads,
                                             c.num_kv_heads, c.head_dim, scale).reshape(seq_len, -1)
+        elif c.attn_softcap > 0:                                               # :891-892
+            attn = nx.sdpa_prefill_softcap(q, k, v, seq_len, c.num_heads, c.num_kv_heads, c.head_dim, scale,
+                                           c.attn_softcap).reshape(seq_len, -1)
         else:                                                                  # :893-895 dense causal on F32 K/V
             attn = nx.sdpa_prefill(q, k, v, seq_len, c.num_heads, c.num_kv_heads, c.head_dim,
                                    scale).reshape(seq_len, -1)
-        o = _mm(attn, lw.wo, seq_len)                                          # :981-983
-        x = nx.add(x, o)                                                       # :990
-        norm = nx.rmsnorm(x, lw.ffn_norm, seq_len, c.hidden, c.eps)            # :996-998
-        gate = _mm(norm, lw.w1, seq_len)                                       # :1043-1050
-        up = _mm(norm, lw.w3, seq_len)
-        act = nx.silu_mul(gate, up)                                            # :1056
-        down = _mm(act, lw.w2, seq_len)                                        # :1058-1061
-        return nx.add(x, down)                                                 # :1077
+        o = _mm_bias(attn, lw.wo, lw.wo_bias, seq_len)                         # :981-983
+        if c.post_norms and lw.post_attn_norm is not None:                     # :985-987
+            o = nx.rmsnorm(o, lw.post_attn_norm, seq_len, c.hidden, c.eps)
+        if not c.parallel_residual:
+            x = nx.add(x, o)                                                   # :989-991
+            if lw.ffn_norm is not None:                                        # :996-998
+                norm = self._norm(x, lw.ffn_norm, lw.ffn_norm_bias, seq_len)
+        down = self._mlp(norm, lw, seq_len)                                    # :1001-1063
+        if c.post_norms and lw.post_ffn_norm is not None:                      # :1066-1069
+            down = nx.rmsnorm(down, lw.post_ffn_norm, seq_len, c.hidden, c.eps)
+        if c.parallel_residual:                                                # :1072-1075
+            x = nx.add(x, o)
+        return nx.add(x, down)                                                 # :1075-1077
+
+    def _embed(self, tokens):
+        c = self.cfg
+        x = nx.embedding(tokens, self.embedding, c.vocab, c.hidden)           # decode.go:405-407
+        if c.embedding_scale > 0:                                              # decode.go:197-205, 408
+            x = nx.scale_buffer(x, c.embedding_scale)
+        return x
 
     # ---------------------------------------------------------------- drivers
     def _ensure_seq(self, seq_id):
@@ -125,7 +190,7 @@ class OracleModel:
 
     def _head(self, state, rows):
         c = self.cfg
-        state = nx.rmsnorm(state, self.final_norm, rows, c.hidden, c.eps)      # model.go:207-226
+        state = self._norm(state, self.final_norm, self.final_norm_bias, rows)  # model.go:207-226
         # model.go:352-422: quantized lm_head runs one M=1 call per row (same numbers)
         return _mm(state, self.lm_head, rows)
 
@@ -133,7 +198,7 @@ class OracleModel:
         """decode.go:339-461 with one token -> logits [vocab]."""
         c = self.cfg
         self._ensure_seq(seq_id)
-        x = nx.embedding([token], self.embedding, c.vocab, c.hidden)           # decode.go:405-407
+        x = self._embed([token])
         for i in range(c.num_layers):                                          # decode.go:432-437
             x = self.execute_with_paged_kv(x, seq_id, i, pos)
         return self._head(x, 1)[0]
@@ -148,7 +213,7 @@ class OracleModel:
         c = self.cfg
         self._ensure_seq(seq_id)
         n = len(tokens)
-        x = nx.embedding(tokens, self.embedding, c.vocab, c.hidden)
+        x = self._embed(tokens)
         for i in range(c.num_layers):
             x = self.execute_with_paged_kv(x, seq_id, i, start_pos)
         last = x[n - 1:n]                                                      # decode.go:1057-1066
@@ -159,7 +224,7 @@ class OracleModel:
         c = self.cfg
         self._ensure_seq(seq_id)
         n = len(tokens)
-        x = nx.embedding(tokens, self.embedding, c.vocab, c.hidden)
+        x = self._embed(tokens)
         for i in range(c.num_layers):
             x = self.execute_with_paged_kv(x, seq_id, i, start_pos)
         return self._head(x, n)
@@ -201,6 +266,7 @@ class OracleModel:
         start_pos .. start_pos + nodes."""
         from .host_logic import build_tree_attention_mask, tree_depths
         c = self.cfg
+        assert is_llama(c), "tree verification is restated for the LLaMA arm only"
         self._ensure_seq(seq_id)
         n = len(node_tokens)
         rows = n + 1
@@ -280,4 +346,31 @@ def random_model(cfg: ModelConfig, seed, fmt, head_fmt, emb_fmt=None, max_blocks
     emb_q = qz.random_quant(ef, rng, cfg.vocab, cfg.hidden)
     emb = nx.dequantize(ef, emb_q, cfg.vocab * cfg.hidden).reshape(cfg.vocab, cfg.hidden)
     head = QWeight(head_fmt, qz.random_quant(head_fmt, rng, cfg.vocab, cfg.hidden), cfg.vocab, cfg.hidden)
-    return OracleModel(cfg, emb, layers, np.ones(cfg.hidden, dtype=np.float32), head, max_blocks, kv_fp16)
+    final_norm, final_bias = np.ones(cfg.hidden, dtype=np.float32), None
+    if not is_llama(cfg):
+        # the tensors the other architectures add, from a stream of their own (the LLaMA draws above are unchanged):
+        # norm weights around 1, small biases, so that a dropped or misplaced one moves the logits visibly
+        r2 = np.random.default_rng(seed + 7919)
+        vec = lambda n, mean, sd: (mean + sd * r2.standard_normal(n)).astype(np.float32)
+        bias = cfg.norm_type == "layer" or cfg.mlp_type == "gelu"           # HasBias models (Phi)
+        for lw in layers:
+            lw.attn_norm, lw.ffn_norm = vec(cfg.hidden, 1.0, 0.1), vec(cfg.hidden, 1.0, 0.1)
+            if cfg.norm_type == "layer":
+                lw.attn_norm_bias, lw.ffn_norm_bias = vec(cfg.hidden, 0.0, 0.05), vec(cfg.hidden, 0.0, 0.05)
+            if bias:
+                lw.wq_bias, lw.wk_bias, lw.wv_bias = vec(qd, 0.0, 0.05), vec(kvd, 0.0, 0.05), vec(kvd, 0.0, 0.05)
+                lw.wo_bias = vec(cfg.hidden, 0.0, 0.05)
+            if cfg.mlp_type == "gelu":
+                lw.w1_bias, lw.w2_bias, lw.w3 = vec(cfg.ffn, 0.0, 0.05), vec(cfg.hidden, 0.0, 0.05), None
+            if cfg.post_norms:
+                lw.post_attn_norm, lw.post_ffn_norm = vec(cfg.hidden, 1.0, 0.1), vec(cfg.hidden, 1.0, 0.1)
+        final_norm = vec(cfg.hidden, 1.0, 0.1)
+        if cfg.norm_type == "layer":
+            final_bias = vec(cfg.hidden, 0.0, 0.05)
+    return OracleModel(cfg, emb, layers, final_norm, head, max_blocks, kv_fp16, final_norm_bias=final_bias)
+
+
+def is_llama(cfg: ModelConfig):
+    """Every architecture switch at its default."""
+    return (cfg.norm_type == "rms" and cfg.mlp_type == "swiglu" and not cfg.parallel_residual and cfg.rope_dim == 0
+            and not cfg.rope_neox and cfg.attn_softcap == 0 and not cfg.post_norms and cfg.embedding_scale <= 0)
