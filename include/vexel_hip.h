@@ -229,6 +229,11 @@ int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight 
 int vx_rope_store_paged(vx_backend *be, float *q, const float *k, const float *v, const int32_t *positions,
                         const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int rows,
                         int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta);
+/* The same with Backend.RoPE's ropeDim / ropeNeox (backend.go:352): the first rope_dim dimensions of a head turn
+ * (0 = all), in pairs (j, j + rope_dim/2) when rope_neox; the others are stored as they are. */
+int vx_rope_store_paged_ex(vx_backend *be, float *q, const float *k, const float *v, const int32_t *positions,
+                           const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int rows, int num_q_heads,
+                           int num_kv_heads, int head_dim, int block_size, float theta, int rope_dim, int rope_neox);
 
 /* Ragged batched paged attention with all metadata on the device: block_tables is a
  * padded int32 [rows, max_blocks] matrix; sequence i uses row table_rows[i] (row i when

@@ -40,6 +40,25 @@ typedef struct vh_layer_weights {  /* the BlockRuntime fields used by ExecuteWit
     vh_qweight wq, wk, wv, wo, w1, w2, w3;
 } vh_layer_weights;
 
+/* The architecture switches of runtime/config.go:14-62,120-131 and block.go:245-254,339-340. All zero = LLaMA. */
+enum { VH_NORM_RMS = 0, VH_NORM_LAYER = 1 };                  /* NormType */
+enum { VH_MLP_SWIGLU = 0, VH_MLP_GELU = 1, VH_MLP_GEGLU = 2 }; /* MLPType */
+typedef struct vh_arch {
+    int norm_type, mlp_type;
+    int parallel_residual;   /* x + attn(norm(x)) + mlp(norm(x)); with the GELU MLP only (block.go:972-976) */
+    int rope_dim;            /* rotated dimensions of a head, 0 = all (RoPEDim) */
+    int rope_neox;           /* pairs (j, j + rope_dim/2) instead of (2j, 2j+1) */
+    int post_norms;          /* HasPostNorms: RMSNorm of the attention and MLP outputs before the residual */
+    float attn_softcap;      /* AttentionLogitSoftCap: applied where block.go applies it on the paged path, the
+                                first prefill chunk (block.go:891-892) */
+    float embedding_scale;   /* EmbeddingScale, <= 0 = none (decode.go:197-205) */
+} vh_arch;
+typedef struct vh_layer_extras {  /* the BlockRuntime tensors beside vh_layer_weights (block.go:266-283); NULL = absent */
+    const float *attn_norm_bias, *ffn_norm_bias;
+    const float *wq_bias, *wk_bias, *wv_bias, *wo_bias, *w1_bias, *w2_bias;
+    const float *post_attn_norm, *post_ffn_norm;
+} vh_layer_extras;
+
 typedef struct vh_model vh_model;
 
 const char *vh_last_error(void);
@@ -54,6 +73,13 @@ void vh_model_get_config(const vh_model *m, vh_config *out);  /* the configurati
  * summation order. */
 void vh_model_set_fused(vh_model *m, int on);
 int vh_model_set_layer(vh_model *m, int layer, const vh_layer_weights *w);
+/* A model with any switch or extra tensor set runs ExecuteWithPagedKV's general sequence, one backend call per
+ * operation (block.go:834-1077), in vh_prefill, vh_decode_batched, vh_decode_graph and the scheduler; the fused
+ * decode entry points and vh_verify_tree are for the LLaMA arm. With the GELU MLP a layer's w3 may be empty.
+ * All pointers are float32 device vectors that outlive the model's use of them. */
+int vh_model_set_architecture(vh_model *m, const vh_arch *arch);
+int vh_model_set_layer_extras(vh_model *m, int layer, const vh_layer_extras *extras);
+int vh_model_set_final_norm_bias(vh_model *m, const float *bias);  /* Model.FinalNormBias (model.go:36, 207-219) */
 /* embedding: F32 [vocab,hidden] on the device (loader rule, runtime/loader.go:275-288) */
 int vh_model_set_head(vh_model *m, const float *embedding, const float *final_norm, const vh_qweight *lm_head);
 void *vh_kv_pool(vh_model *m, int layer);  /* device base of a layer's block pool */

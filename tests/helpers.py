@@ -13,12 +13,22 @@ def gpu_model_from_oracle(be, omodel, pool_blocks, max_seqs=64, max_blocks_per_s
                       eps=c.eps, rope_theta=c.rope_theta, block_size=c.block_size, pool_blocks=pool_blocks,
                       max_seqs=max_seqs, max_blocks_per_seq=max_blocks_per_seq, max_batch=max_batch,
                       kv_fp16=omodel.pool.use_fp16)
+    from oracle.model import is_llama
+    from vexel_amd.runtime import EXTRA_NAMES
+    if not is_llama(c):
+        mr.set_architecture(c.norm_type, c.mlp_type, c.parallel_residual, c.rope_dim, c.rope_neox, c.post_norms,
+                            c.attn_softcap, c.embedding_scale)
     for i, lw in enumerate(omodel.layers):
         ws = {n: (getattr(lw, n).fmt, getattr(lw, n).data, getattr(lw, n).n, getattr(lw, n).k)
-              for n in ("wq", "wk", "wv", "wo", "w1", "w2", "w3")}
+              for n in ("wq", "wk", "wv", "wo", "w1", "w2", "w3") if getattr(lw, n) is not None}
         mr.set_layer(i, lw.attn_norm, lw.ffn_norm, ws)
+        extras = {n: getattr(lw, n) for n in EXTRA_NAMES if getattr(lw, n) is not None}
+        if extras:
+            mr.set_layer_extras(i, **extras)
     h = omodel.lm_head
     mr.set_head(omodel.embedding, omodel.final_norm, (h.fmt, h.data, h.n, h.k))
+    if omodel.final_norm_bias is not None:
+        mr.set_final_norm_bias(omodel.final_norm_bias)
     return mr
 
 

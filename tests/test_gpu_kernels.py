@@ -901,9 +901,12 @@ def test_rope_shift(be):
     be.reset_pool()
 
 
-def test_rope_store_paged(be):
+@pytest.mark.parametrize("rope_dim,neox,d", [(0, False, 64), (0, True, 64), (32, True, 80), (32, False, 64), (128, True, 128)])
+def test_rope_store_paged(be, rope_dim, neox, d):
+    """Interleaved whole-head RoPE (LLaMA) and the ropeDim / ropeNeox forms of Backend.RoPE (Phi-2: 32 of 80
+    dimensions, split pairs; Qwen / Gemma: the whole head, split pairs), fused with the paged store."""
     rng = np.random.default_rng(35)
-    rows, hq, hk, d, bs, nblocks = 9, 8, 2, 64, 16, 30
+    rows, hq, hk, bs, nblocks = 9, 8, 2, 16, 30
     q = rng.standard_normal((rows, hq, d)).astype(np.float32)
     k = rng.standard_normal((rows, hk, d)).astype(np.float32)
     v = rng.standard_normal((rows, hk, d)).astype(np.float32)
@@ -912,12 +915,12 @@ def test_rope_store_paged(be):
     for f16 in (False, True):
         pool = _make_pool(rng, f16, nblocks, bs, hk, d)
         want_pool = pool.copy()
-        wq, wk = nx.rope_positions(q, k, d, hq, hk, pos, 0, 10000.0, False)
+        wq, wk = nx.rope_positions(q, k, d, hq, hk, pos, rope_dim, 10000.0, neox)
         nx.reshape_paged_kv(wk, want_pool, slots // bs, slots % bs, hk, d, bs, False)
         nx.reshape_paged_kv(v, want_pool, slots // bs, slots % bs, hk, d, bs, True)
         dq, dk, dv = be.upload(q), be.upload(k), be.upload(v)
         dpool, dp, ds = be.upload(pool), be.upload(pos), be.upload(slots)
-        be.rope_store_paged(dq, dk, dv, dp, ds, dpool, f16, rows, hq, hk, d, bs, 10000.0)
+        be.rope_store_paged(dq, dk, dv, dp, ds, dpool, f16, rows, hq, hk, d, bs, 10000.0, rope_dim, neox)
         _close(be.download(dq, q.shape, np.float32), wq.reshape(q.shape), 0, 1e-6, "rope_store q")
         got = be.download(dpool, pool.shape, pool.dtype)
         if f16:

@@ -465,3 +465,91 @@ def test_pool_errors_and_lifecycle(be):
     with pytest.raises(VexelError):
         mr.share_blocks(7, 2, 16)
     mr.close()
+
+
+# ------------------------------------------------------------------ the architectures beside LLaMA
+def _arch_config(name):
+    """Small models with the layer shapes of Phi-2 (LayerNorm, biases, 32 of 80 head dimensions rotated in split
+    pairs, GELU MLP, parallel residual), Gemma 2 (scaled embeddings, GeGLU, post-norms, soft-capped attention, heads
+    of 256) and Qwen 2 (Q/K/V biases, split-pair RoPE, theta 1e6)."""
+    import math
+    if name == "phi":
+        return om.ModelConfig(num_layers=2, hidden=640, num_heads=8, num_kv_heads=8, head_dim=80, ffn=2560, vocab=1000,
+                              norm_type="layer", mlp_type="gelu", parallel_residual=True, rope_dim=32, rope_neox=True)
+    if name == "gemma":
+        return om.ModelConfig(num_layers=2, hidden=512, num_heads=4, num_kv_heads=2, head_dim=256, ffn=1024, vocab=1000,
+                              eps=1e-6, mlp_type="geglu", post_norms=True, attn_softcap=50.0, rope_neox=True,
+                              embedding_scale=float(np.float32(math.sqrt(512.0))))
+    return om.ModelConfig(num_layers=2, hidden=512, num_heads=8, num_kv_heads=2, head_dim=64, ffn=1536, vocab=1000,
+                          eps=1e-6, rope_neox=True, rope_theta=1000000.0)
+
+
+@pytest.mark.parametrize("name", ["phi", "gemma", "qwen"])
+def test_other_architectures_prefill_decode_graph(be, name):
+    """ExecuteWithPagedKV's general sequence (block.go:834-1077) through vh_prefill (first chunk and a later one),
+    vh_decode_batched and the device-driven vh_decode_graph, against the oracle's layer for the same switches."""
+    cfg = _arch_config(name)
+    omodel = om.random_model(cfg, 21, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=24)
+    if name == "qwen":
+        rng = np.random.default_rng(22)
+        for lw in omodel.layers:
+            lw.wq_bias = (0.05 * rng.standard_normal(512)).astype(np.float32)
+            lw.wk_bias = (0.05 * rng.standard_normal(128)).astype(np.float32)
+            lw.wv_bias = (0.05 * rng.standard_normal(128)).astype(np.float32)
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=24, max_seqs=4, max_batch=8)
+    rng = np.random.default_rng(23)
+    prompts = {1: rng.integers(0, cfg.vocab, 21).tolist(), 2: rng.integers(0, cfg.vocab, 35).tolist()}
+    toks, worst = {}, 0.0
+    for sid, p in prompts.items():
+        want = omodel.prefill_with_paged_kv(p[:17], sid, 0)
+        got = mr.prefill_with_paged_kv(p[:17], sid, 0)
+        worst = max(worst, assert_logits_close(got, want, "%s first chunk" % name))
+        want = omodel.prefill_with_paged_kv(p[17:], sid, 17)
+        got = mr.prefill_with_paged_kv(p[17:], sid, 17)
+        worst = max(worst, assert_logits_close(got, want, "%s second chunk" % name))
+        toks[sid] = nx.argmax(want)
+        assert toks[sid] == int(np.argmax(got))
+    ids = [1, 2]
+    pos = [len(prompts[1]), len(prompts[2])]
+    cur = [toks[1], toks[2]]
+    for step in range(12):
+        want = omodel.decode_batched(cur, ids, pos)
+        got, am = mr.decode_with_paged_kv_batched(cur, ids, pos)
+        worst = max(worst, assert_logits_close(got, want, "%s decode step %d" % (name, step)))
+        nxt = [nx.argmax(w) for w in want]
+        assert nxt == [int(a) for a in am]
+        cur, pos = nxt, [p + 1 for p in pos]
+    # the device-driven loop continues from here; the oracle follows step by step
+    out, _ = mr.decode_graph(cur, ids, pos, 6)
+    for step in range(6):
+        want = omodel.decode_batched(cur, ids, pos)
+        cur, pos = [nx.argmax(w) for w in want], [p + 1 for p in pos]
+        assert out[step].tolist() == cur, "graph step %d" % step
+    assert mr.block_table(1) == omodel.pool.seqs[1].block_tables[0]
+    assert mr.device_matches_host()
+    with pytest.raises(RuntimeError, match="LLaMA arm only"):
+        mr.verify_tree([1], [cur[0]], [pos[0]], [([5, 6], [-1, 0])])
+    print("%s: worst logit error %.3e" % (name, worst))
+    mr.close()
+
+
+def test_architecture_switches_are_validated(be):
+    cfg = om.ModelConfig(num_layers=1, hidden=256, num_heads=4, num_kv_heads=2, head_dim=64, ffn=512, vocab=300)
+    omodel = om.random_model(cfg, 3, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=8)
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=8, max_seqs=2, max_batch=2)
+    with pytest.raises(RuntimeError, match="parallel residual"):
+        mr.set_architecture(parallel_residual=True)                 # gated MLP
+    with pytest.raises(RuntimeError, match="rope_dim"):
+        mr.set_architecture(rope_dim=66)
+    with pytest.raises(RuntimeError, match="rope_dim"):
+        mr.set_architecture(rope_dim=31)
+    with pytest.raises(RuntimeError, match="soft cap"):
+        mr.set_architecture(attn_softcap=-1.0)
+    # rope_dim = head_dim is the default sequence's arithmetic: same logits, bit for bit, as the unfused LLaMA arm
+    mr.set_fused(False)
+    prompt = list(range(30, 49))
+    a = mr.prefill_with_paged_kv(prompt, 1, 0)
+    mr.set_architecture(rope_dim=64)
+    b = mr.prefill_with_paged_kv(prompt, 2, 0)
+    assert_logits_close(b, a, "rope_dim = head_dim")
+    mr.close()

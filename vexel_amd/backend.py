@@ -279,9 +279,9 @@ class HipBackend:
                   C.byref(w2), rows, next_norm_weight)
 
     def rope_store_paged(self, q, k, v, positions, slot_mapping, kv_pool, pool_is_f16, rows, num_q_heads,
-                         num_kv_heads, head_dim, block_size, theta):
-        self.call("vx_rope_store_paged", q, k, v, positions, slot_mapping, kv_pool, int(bool(pool_is_f16)), rows,
-                  num_q_heads, num_kv_heads, head_dim, block_size, theta)
+                         num_kv_heads, head_dim, block_size, theta, rope_dim=0, rope_neox=False):
+        self.call("vx_rope_store_paged_ex", q, k, v, positions, slot_mapping, kv_pool, int(bool(pool_is_f16)), rows,
+                  num_q_heads, num_kv_heads, head_dim, block_size, theta, rope_dim, int(bool(rope_neox)))
 
     def sdpa_paged_decode_ragged(self, q, kv_pool, pool_is_f16, block_tables, kv_lens, out, batch, max_blocks,
                                  block_size, num_q_heads, num_kv_heads, head_dim, scale, max_kv_len, table_rows=None):

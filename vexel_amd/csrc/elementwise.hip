@@ -108,15 +108,17 @@ __global__ void rope_kernel(float *q, float *k, int head_dim, int num_heads, int
     }
 }
 
-// RoPE (interleaved pairs, full head_dim) + paged scatter of K and V.
+// RoPE + paged scatter of K and V. The first eff_dim dimensions of a head turn, in pairs (2j, 2j+1) or, neox,
+// (j, j + eff_dim/2); the rest is copied. Thread j of a head handles rotation pair j, or past the rotated part the
+// two elements eff_dim + 2(j - eff_dim/2) and the one after: head_dim/2 threads cover the head either way.
 template <bool F16>
 __global__ void rope_store_paged_kernel(float *q, const float *k, const float *v, const int32_t *positions,
                                         const int32_t *slot_mapping, void *pool, int num_q_heads, int num_kv_heads,
-                                        int head_dim, int block_size, float theta) {
-    // grid = (rows, head groups); thread = (rotation pair j, head lane); heads are strided over
+                                        int head_dim, int block_size, float theta, int eff_dim, int neox) {
+    // grid = (rows, head groups); thread = (pair j, head lane); heads are strided over
     // head lanes and head groups so the float64 cos/sin of a pair is computed once per thread.
     int row = blockIdx.x;
-    int half = head_dim / 2;
+    int half = head_dim / 2, he = eff_dim / 2;
     int pos = positions[row];
     int slot = slot_mapping[row];
     int blk = slot / block_size, off = slot % block_size;
@@ -129,28 +131,33 @@ __global__ void rope_store_paged_kernel(float *q, const float *k, const float *v
     const int hstride = lanes * gridDim.y;
     const int h0 = blockIdx.y * lanes + hl;
     for (int j = threadIdx.x % half; j < half && hl < lanes; j += half) {
-        RopeCS cs = rope_cs(pos, j, head_dim, theta);
+        const bool turn = j < he;
+        const int i0 = turn ? (neox ? j : 2 * j) : eff_dim + 2 * (j - he);
+        const int i1 = turn ? (neox ? j + he : 2 * j + 1) : i0 + 1;
+        RopeCS cs = {1.f, 0.f};
+        if (turn) cs = rope_cs(pos, j, eff_dim, theta);
         float *qr = q + (size_t)row * num_q_heads * head_dim;
-        for (int h = h0; h < num_q_heads; h += hstride) rope_pair(qr[h * head_dim + 2 * j], qr[h * head_dim + 2 * j + 1], cs);
+        if (turn)
+            for (int h = h0; h < num_q_heads; h += hstride) rope_pair(qr[h * head_dim + i0], qr[h * head_dim + i1], cs);
         const float *kr = k + (size_t)row * hs;
         const float *vr = v + (size_t)row * hs;
         for (int h = h0; h < num_kv_heads; h += hstride) {
-            float a = kr[h * head_dim + 2 * j], b = kr[h * head_dim + 2 * j + 1];
-            rope_pair(a, b, cs);
-            float va = vr[h * head_dim + 2 * j], vb = vr[h * head_dim + 2 * j + 1];
-            size_t o = (size_t)h * head_dim + 2 * j;
+            float a = kr[h * head_dim + i0], b = kr[h * head_dim + i1];
+            if (turn) rope_pair(a, b, cs);
+            float va = vr[h * head_dim + i0], vb = vr[h * head_dim + i1];
+            size_t o0 = (size_t)h * head_dim + i0, o1 = (size_t)h * head_dim + i1;
             if (F16) {
                 _Float16 *p = (_Float16 *)pool;
-                p[kbase + o] = (_Float16)a;
-                p[kbase + o + 1] = (_Float16)b;
-                p[vbase + o] = (_Float16)va;
-                p[vbase + o + 1] = (_Float16)vb;
+                p[kbase + o0] = (_Float16)a;
+                p[kbase + o1] = (_Float16)b;
+                p[vbase + o0] = (_Float16)va;
+                p[vbase + o1] = (_Float16)vb;
             } else {
                 float *p = (float *)pool;
-                p[kbase + o] = a;
-                p[kbase + o + 1] = b;
-                p[vbase + o] = va;
-                p[vbase + o + 1] = vb;
+                p[kbase + o0] = a;
+                p[kbase + o1] = b;
+                p[vbase + o0] = va;
+                p[vbase + o1] = vb;
             }
         }
     }
@@ -565,14 +572,17 @@ int vx_rope_shift(vx_backend *be, float *k, int head_dim, int num_kv_heads, int 
     return VX_OK;
 }
 
-int vx_rope_store_paged(vx_backend *be, float *q, const float *k, const float *v, const int32_t *positions,
-                        const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int rows, int num_q_heads,
-                        int num_kv_heads, int head_dim, int block_size, float theta) {
+int vx_rope_store_paged_ex(vx_backend *be, float *q, const float *k, const float *v, const int32_t *positions,
+                           const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int rows, int num_q_heads,
+                           int num_kv_heads, int head_dim, int block_size, float theta, int rope_dim, int rope_neox) {
     int rc = enter(be);
     if (rc) return rc;
     VX_REQUIRE(q && k && v && positions && slot_mapping && kv_pool, "vx_rope_store_paged: null pointer");
     VX_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && block_size > 0 && num_q_heads > 0 && num_kv_heads > 0,
                "vx_rope_store_paged: bad shape");
+    const int eff = rope_dim == 0 ? head_dim : rope_dim;
+    VX_REQUIRE(eff > 0 && eff <= head_dim && eff % 2 == 0, "vx_rope_store_paged: rope_dim %d invalid for head_dim %d", rope_dim,
+               head_dim);
     if (rows == 0) return VX_OK;
     VX_REQUIRE(head_dim <= 512, "vx_rope_store_paged: head_dim %d too large", head_dim);
     const int half = head_dim / 2;
@@ -585,13 +595,20 @@ int vx_rope_store_paged(vx_backend *be, float *q, const float *k, const float *v
     if (pool_is_f16)
         rope_store_paged_kernel<true><<<grid, threads, 0, be->stream>>>(q, k, v, positions, slot_mapping, kv_pool,
                                                                         num_q_heads, num_kv_heads, head_dim,
-                                                                        block_size, theta);
+                                                                        block_size, theta, eff, rope_neox);
     else
         rope_store_paged_kernel<false><<<grid, threads, 0, be->stream>>>(q, k, v, positions, slot_mapping, kv_pool,
                                                                          num_q_heads, num_kv_heads, head_dim,
-                                                                         block_size, theta);
+                                                                         block_size, theta, eff, rope_neox);
     VX_CHECK_LAUNCH();
     return VX_OK;
+}
+
+int vx_rope_store_paged(vx_backend *be, float *q, const float *k, const float *v, const int32_t *positions,
+                        const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int rows, int num_q_heads,
+                        int num_kv_heads, int head_dim, int block_size, float theta) {
+    return vx_rope_store_paged_ex(be, q, k, v, positions, slot_mapping, kv_pool, pool_is_f16, rows, num_q_heads,
+                                  num_kv_heads, head_dim, block_size, theta, 0, 0);
 }
 
 #define VX_EW(name, kernel, ...)                                                \

@@ -124,6 +124,12 @@ struct vh_model {
 
     bool fused = true;  // take the fused decode entry points where the weights allow it
 
+    vh_arch arch{};                       // all zero: the LLaMA arm
+    std::vector<vh_layer_extras> extras;  // per layer, all NULL by default
+    const float *final_norm_bias = nullptr;
+    float *zeros = nullptr;               // [hidden] zeros: the bias of a LayerNorm whose bias tensor is absent
+    bool general = false;                 // some switch or extra tensor is set: the one-call-per-operation sequence
+
     vx_graph *graph = nullptr;
     int graph_batch = 0;
     std::vector<int64_t> dev_seq_ids;  // batch currently loaded in d_slots (device-driven mode)
@@ -239,8 +245,77 @@ int layer_tail(vh_model *m, const vh_layer_weights &w, float *x, float *norm, co
     return VH_OK;
 }
 
+// ---- the general sequence of block.go:834-1077 for the architectures beside LLaMA ----
+
+// applyNorm (block.go:562-576): LayerNorm with its bias, or RMSNorm, which ignores the bias
+int g_norm(vh_model *m, const float *x, const float *w, const float *b, float *out, int rows) {
+    const vh_config &c = m->cfg;
+    if (m->arch.norm_type == VH_NORM_LAYER)
+        VXC(vx_layernorm(m->be, x, w, b ? b : m->zeros, out, rows, c.hidden, c.eps));
+    else
+        VXC(vx_rmsnorm(m->be, x, w, out, rows, c.hidden, c.eps));
+    return VH_OK;
+}
+
+// matMulTransposedWithBias (block.go:555-560)
+int g_mm(vh_model *m, const float *a, const vh_qweight &w, const float *bias, float *out, int rows) {
+    VHC(mm(m, false, a, w, out, nullptr, rows));
+    if (bias) VXC(vx_add_bias(m->be, out, bias, out, rows, w.n));
+    return VH_OK;
+}
+
+// block.go:834-854: the attention norm and the three projections
+int g_qkv(vh_model *m, int layer, const float *x, float *norm, float *q, float *k, float *v, int rows) {
+    const vh_layer_weights &w = m->layers[layer];
+    const vh_layer_extras &e = m->extras[layer];
+    VHC(g_norm(m, x, w.attn_norm, e.attn_norm_bias, norm, rows));
+    VHC(g_mm(m, norm, w.wq, e.wq_bias, q, rows));
+    VHC(g_mm(m, norm, w.wk, e.wk_bias, k, rows));
+    VHC(g_mm(m, norm, w.wv, e.wv_bias, v, rows));
+    return VH_OK;
+}
+
+// block.go:972-1077: Wo, post-norm, residual(s), FFN norm, MLP. `norm` holds the attention norm's output on entry.
+int g_tail(vh_model *m, int layer, float *x, float *norm, const float *attn, float *gate, float *up, int rows) {
+    const vh_config &c = m->cfg;
+    const vh_arch &a = m->arch;
+    const vh_layer_weights &w = m->layers[layer];
+    const vh_layer_extras &e = m->extras[layer];
+    vx_backend *be = m->be;
+    float *o = a.parallel_residual ? up : norm;                                        // :972-978
+    VHC(g_mm(m, attn, w.wo, e.wo_bias, o, rows));                                      // :981-983
+    if (a.post_norms && e.post_attn_norm) VXC(vx_rmsnorm(be, o, e.post_attn_norm, o, rows, c.hidden, c.eps));  // :985-987
+    if (!a.parallel_residual) {
+        VXC(vx_add(be, x, o, x, rows * c.hidden));                                     // :989-991
+        if (w.ffn_norm) VHC(g_norm(m, x, w.ffn_norm, e.ffn_norm_bias, norm, rows));    // :996-998
+    }
+    if (a.mlp_type == VH_MLP_GELU) {                                                   // :1004-1037
+        VHC(g_mm(m, norm, w.w1, e.w1_bias, gate, rows));
+        VXC(vx_gelu(be, gate, gate, rows * c.ffn));
+        VHC(g_mm(m, gate, w.w2, e.w2_bias, norm, rows));
+    } else {                                                                           // :1040-1062
+        VHC(mm(m, false, norm, w.w1, gate, nullptr, rows));
+        VHC(mm(m, false, norm, w.w3, up, nullptr, rows));
+        if (a.mlp_type == VH_MLP_GEGLU)
+            VXC(vx_gelu_mul(be, gate, up, gate, rows * c.ffn));
+        else
+            VXC(vx_silu_mul(be, gate, up, gate, rows * c.ffn));
+        VHC(mm(m, false, gate, w.w2, norm, nullptr, rows));
+    }
+    if (a.post_norms && e.post_ffn_norm) VXC(vx_rmsnorm(be, norm, e.post_ffn_norm, norm, rows, c.hidden, c.eps));  // :1066-1069
+    if (a.parallel_residual) VXC(vx_add(be, x, o, x, rows * c.hidden));                // :1072-1075
+    VXC(vx_add(be, x, norm, x, rows * c.hidden));
+    return VH_OK;
+}
+
+// embedding scale (decode.go:197-205) and the final norm (model.go:207-226) of the general sequence
+int g_scale_embedding(vh_model *m, float *x, int rows) {
+    if (m->arch.embedding_scale > 0.f) VXC(vx_scale_buffer(m->be, x, m->arch.embedding_scale, rows * m->cfg.hidden));
+    return VH_OK;
+}
+
 bool attn_fusable(const vh_model *m, int layer) {
-    if (!m->fused || layer >= m->cfg.num_layers) return false;
+    if (!m->fused || m->general || layer >= m->cfg.num_layers) return false;
     const vh_layer_weights &w = m->layers[layer];
     return w.wq.data && w.wk.data && w.wv.data && vx_decode_attn_qkv_supported(&w.wq, &w.wk, &w.wv, m->cfg.head_dim) != 0;
 }
@@ -252,6 +327,17 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
     const vh_config &c = m->cfg;
     const vh_layer_weights &w = m->layers[layer];
     const float scale = (float)(1.0 / sqrt((double)c.head_dim));                          // block.go:862
+    if (m->general) {
+        if (*chained) return fail("internal: prepared activation handed to a general layer");
+        VHC(g_qkv(m, layer, m->x, m->norm, m->q, m->k, m->v, rows));
+        VXC(vx_rope_store_paged_ex(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
+                                   c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta, m->arch.rope_dim,
+                                   m->arch.rope_neox));                               // :858, :868
+        VXC(vx_sdpa_paged_decode_ragged(m->be, m->q, m->kv[layer], c.kv_fp16, m->d_tables, m->d_slots, m->d_kv_lens,
+                                        m->attn, rows, c.max_blocks_per_seq, c.block_size, c.num_heads, c.num_kv_heads,
+                                        c.head_dim, scale, max_kv_len));               // :872 (no soft cap on this arm)
+        return g_tail(m, layer, m->x, m->norm, m->attn, m->gate, m->up, rows);
+    }
     if (attn_fusable(m, layer)) {   // block.go:834-868; one row: matrix-vector launches inside the same entry points
         VXC(vx_decode_attn_qkv(m->be, m->x, w.attn_norm, c.eps, *chained ? 1 : 0, &w.wq, &w.wk, &w.wv, rows,
                                m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, c.num_heads, c.num_kv_heads,
@@ -289,7 +375,8 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
 int forward_decode(vh_model *m, int rows, int max_kv_len) {
     const vh_config &c = m->cfg;
     VXC(vx_embedding(m->be, m->d_tokens, rows, m->embedding, m->x, c.vocab, c.hidden));
-    const bool head_prepared = rows > 1 && m->fused && fast(m->lm_head) && c.hidden % 256 == 0;
+    VHC(g_scale_embedding(m, m->x, rows));
+    const bool head_prepared = rows > 1 && m->fused && !m->general && fast(m->lm_head) && c.hidden % 256 == 0;
     bool chained = false;
     for (int l = 0; l < c.num_layers; l++) {
         const float *next_norm = l + 1 < c.num_layers ? (rows > 1 && attn_fusable(m, l + 1) ? m->layers[l + 1].attn_norm : nullptr)
@@ -298,6 +385,9 @@ int forward_decode(vh_model *m, int rows, int max_kv_len) {
     }
     if (chained) {                                                                        // model.go:207-226, 352-422
         VHC(mm(m, true, nullptr, m->lm_head, m->logits, nullptr, rows));
+    } else if (m->general) {
+        VHC(g_norm(m, m->x, m->final_norm, m->final_norm_bias, m->norm, rows));
+        VHC(mm(m, false, m->norm, m->lm_head, m->logits, nullptr, rows));
     } else {
         bool prep;
         const vh_qweight *hw[1] = {&m->lm_head};
@@ -312,6 +402,9 @@ int check_ready(vh_model *m) {
     if (!m->embedding || !m->final_norm || !m->lm_head.data) return fail("model head / embedding not set");
     for (auto &l : m->layers)
         if (!l.attn_norm || !l.wq.data) return fail("a layer's weights are not set");
+    if (m->arch.mlp_type != VH_MLP_GELU)
+        for (auto &l : m->layers)
+            if (!l.w3.data) return fail("a layer has no w3 and the MLP is gated");
     return VH_OK;
 }
 
@@ -342,6 +435,7 @@ int vh_model_create(vx_backend *be, const vh_config *cfg, vh_model **out) {
     m->be = be;
     m->cfg = c;
     m->layers.resize(c.num_layers);
+    m->extras.resize(c.num_layers);
     m->pool.block_size = c.block_size;
     m->pool.max_blocks = c.pool_blocks;
     m->pool.free_list.resize(c.pool_blocks);
@@ -404,7 +498,7 @@ void vh_model_destroy(vh_model *m) {
     for (void *p : m->kv) vx_free(m->be, p);
     void *bufs[] = {m->d_tables, m->d_num_blocks, m->d_free, m->d_free_count, m->d_slots, m->d_positions, m->d_tokens,
                     m->d_next, m->d_cu, m->d_token_pos, m->d_slot_map, m->d_kv_lens, m->d_pos_in, m->d_status, m->d_step, m->d_log,
-                    m->x, m->norm, m->q, m->k, m->v, m->attn, m->gate, m->up, m->logits};
+                    m->x, m->norm, m->q, m->k, m->v, m->attn, m->gate, m->up, m->logits, m->zeros};
     for (void *p : bufs) vx_free(m->be, p);
     for (void *p : m->adopted) vx_free(m->be, p);
     delete m;
@@ -415,7 +509,7 @@ int vh_model_set_layer(vh_model *m, int layer, const vh_layer_weights *w) {
     const vh_config &c = m->cfg;
     const int qd = c.num_heads * c.head_dim, kvd = c.num_kv_heads * c.head_dim;
     if (w->wq.n != qd || w->wq.k != c.hidden || w->wk.n != kvd || w->wv.n != kvd || w->wo.n != c.hidden ||
-        w->wo.k != qd || w->w1.n != c.ffn || w->w3.n != c.ffn || w->w2.n != c.hidden || w->w2.k != c.ffn)
+        w->wo.k != qd || w->w1.n != c.ffn || (w->w3.data && w->w3.n != c.ffn) || w->w2.n != c.hidden || w->w2.k != c.ffn)
         return fail("layer %d: weight shapes do not match the configuration", layer);
     m->layers[layer] = *w;
     return VH_OK;
@@ -427,6 +521,65 @@ int vh_model_set_head(vh_model *m, const float *embedding, const float *final_no
     m->embedding = embedding;
     m->final_norm = final_norm;
     m->lm_head = *lm_head;
+    return VH_OK;
+}
+
+static void drop_graph(vh_model *m) {  // a captured step was recorded with another kernel sequence
+    if (m->graph) {
+        vx_graph_destroy(m->graph);
+        m->graph = nullptr;
+        m->graph_batch = 0;
+    }
+}
+
+static void refresh_general(vh_model *m) {
+    const vh_arch &a = m->arch;
+    bool g = a.norm_type || a.mlp_type || a.parallel_residual || a.rope_dim || a.rope_neox || a.post_norms ||
+             a.attn_softcap > 0.f || a.embedding_scale > 0.f || m->final_norm_bias;
+    for (const vh_layer_extras &e : m->extras)
+        g = g || e.attn_norm_bias || e.ffn_norm_bias || e.wq_bias || e.wk_bias || e.wv_bias || e.wo_bias || e.w1_bias ||
+            e.w2_bias || e.post_attn_norm || e.post_ffn_norm;
+    if (g != m->general) drop_graph(m);
+    m->general = g;
+}
+
+int vh_model_set_architecture(vh_model *m, const vh_arch *arch) {
+    if (!m || !arch) return fail("null argument");
+    const vh_arch &a = *arch;
+    if (a.norm_type < 0 || a.norm_type > VH_NORM_LAYER || a.mlp_type < 0 || a.mlp_type > VH_MLP_GEGLU)
+        return fail("unknown norm type %d / MLP type %d", a.norm_type, a.mlp_type);
+    if (a.parallel_residual && a.mlp_type != VH_MLP_GELU)
+        return fail("the parallel residual goes with the GELU MLP only");  // block.go:972-976 shares a buffer with W3's product
+    if (a.rope_dim < 0 || a.rope_dim > m->cfg.head_dim || a.rope_dim % 2 != 0)
+        return fail("rope_dim %d invalid for head_dim %d", a.rope_dim, m->cfg.head_dim);
+    if (a.attn_softcap < 0.f) return fail("negative attention soft cap");
+    if (a.mlp_type == VH_MLP_GELU && m->cfg.ffn < m->cfg.hidden && a.parallel_residual)
+        return fail("the parallel residual keeps the attention output in an [rows, ffn] buffer: ffn %d < hidden %d", m->cfg.ffn,
+                    m->cfg.hidden);
+    if (a.norm_type == VH_NORM_LAYER && !m->zeros) {
+        std::vector<float> z((size_t)m->cfg.hidden, 0.f);
+        m->zeros = (float *)vx_alloc_permanent(m->be, z.size() * 4);
+        if (!m->zeros) return fail("zero bias: %s", vx_last_error());
+        VXC(vx_to_device(m->be, m->zeros, z.data(), z.size() * 4));
+    }
+    m->arch = a;
+    drop_graph(m);
+    refresh_general(m);
+    return VH_OK;
+}
+
+int vh_model_set_layer_extras(vh_model *m, int layer, const vh_layer_extras *extras) {
+    if (!m || !extras || layer < 0 || layer >= m->cfg.num_layers) return fail("bad layer index");
+    m->extras[layer] = *extras;
+    drop_graph(m);
+    refresh_general(m);
+    return VH_OK;
+}
+
+int vh_model_set_final_norm_bias(vh_model *m, const float *bias) {
+    if (!m) return fail("null argument");
+    m->final_norm_bias = bias;
+    refresh_general(m);
     return VH_OK;
 }
 
@@ -690,16 +843,22 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
     VXC(vx_to_device(be, d_kvl, kvl.data(), (size_t)n * 4));
     VXC(vx_to_device(be, d_bt, table.data(), table.size() * 4));
     VXC(vx_embedding(be, d_tok, n, m->embedding, x, c.vocab, c.hidden));               // decode.go:1005-1010
+    VHC(g_scale_embedding(m, x, n));                                                   // decode.go:1030
     const float scale = (float)(1.0 / sqrt((double)c.head_dim));
     for (int l = 0; l < c.num_layers; l++) {
         const vh_layer_weights &w = m->layers[l];
-        bool prep;
-        const vh_qweight *qkv[3] = {&w.wq, &w.wk, &w.wv};
-        VHC(norm_for(m, x, w.attn_norm, norm, n, qkv, 3, &prep));
-        VHC(mm(m, prep, norm, w.wq, q, nullptr, n));
-        VHC(mm(m, prep, norm, w.wk, k, nullptr, n));
-        VHC(mm(m, prep, norm, w.wv, v, nullptr, n));
-        VXC(vx_rope(be, q, k, c.head_dim, c.num_heads, c.num_kv_heads, n, start_pos, 0, c.rope_theta, 0));  // block.go:858
+        if (m->general) {
+            VHC(g_qkv(m, l, x, norm, q, k, v, n));
+        } else {
+            bool prep;
+            const vh_qweight *qkv[3] = {&w.wq, &w.wk, &w.wv};
+            VHC(norm_for(m, x, w.attn_norm, norm, n, qkv, 3, &prep));
+            VHC(mm(m, prep, norm, w.wq, q, nullptr, n));
+            VHC(mm(m, prep, norm, w.wk, k, nullptr, n));
+            VHC(mm(m, prep, norm, w.wv, v, nullptr, n));
+        }
+        VXC(vx_rope(be, q, k, c.head_dim, c.num_heads, c.num_kv_heads, n, start_pos, m->arch.rope_dim, c.rope_theta,
+                    m->arch.rope_neox));                                               // block.go:858 (applyRoPE, :497-503)
         if (c.kv_fp16) {                                                               // gpu_block_pool.go:262-272
             VXC(vx_reshape_paged_kv_f16(be, k, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 0));
             VXC(vx_reshape_paged_kv_f16(be, v, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 1));
@@ -719,16 +878,27 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
         } else if (start_pos > 0) {                                                    // block.go:881-890
             VXC(vx_sdpa_paged_decode_multiquery(be, q, m->kv[l], c.kv_fp16, d_bt, attn, d_kvl, (int)table.size(),
                                                 c.block_size, c.num_heads, c.num_kv_heads, c.head_dim, scale, n));
+        } else if (m->arch.attn_softcap > 0.f) {                                       // block.go:891-892
+            VXC(vx_sdpa_prefill_softcap(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale,
+                                        m->arch.attn_softcap));
         } else {                                                                       // block.go:893-895
             VXC(vx_sdpa_prefill(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale));
         }
-        VHC(layer_tail(m, w, x, norm, attn, gate, up, n));
+        if (m->general)
+            VHC(g_tail(m, l, x, norm, attn, gate, up, n));
+        else
+            VHC(layer_tail(m, w, x, norm, attn, gate, up, n));
     }
     const float *last = all_logits ? x : x + (size_t)(n - 1) * c.hidden;                // decode.go:1057-1066
-    bool prep;
-    const vh_qweight *hw[1] = {&m->lm_head};
-    VHC(norm_for(m, last, m->final_norm, norm, out_rows, hw, 1, &prep));
-    VHC(mm(m, prep, norm, m->lm_head, logits, nullptr, out_rows));
+    if (m->general) {
+        VHC(g_norm(m, last, m->final_norm, m->final_norm_bias, norm, out_rows));
+        VHC(mm(m, false, norm, m->lm_head, logits, nullptr, out_rows));
+    } else {
+        bool prep;
+        const vh_qweight *hw[1] = {&m->lm_head};
+        VHC(norm_for(m, last, m->final_norm, norm, out_rows, hw, 1, &prep));
+        VHC(mm(m, prep, norm, m->lm_head, logits, nullptr, out_rows));
+    }
     if (logits_out) VXC(vx_to_host(be, logits_out, logits, (size_t)out_rows * c.vocab * 4));
     VXC(vx_sync(be));
     return VH_OK;
@@ -738,6 +908,7 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
 int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_t *input_tokens, const int32_t *start_pos,
                    const int32_t *n_nodes, const int32_t *node_tokens, const int32_t *parent_idx, int32_t *num_accepted,
                    int32_t *accepted_nodes, int32_t *final_tokens, float *logits_out) {
+    if (m && m->general) return fail("vh_verify_tree: the LLaMA arm only");
     if (!m || n_seqs < 0 || !seq_ids || !input_tokens || !start_pos || !n_nodes || !num_accepted || !final_tokens)
         return fail("bad arguments");
     if (n_seqs == 0) return VH_OK;

@@ -75,6 +75,7 @@ SIGNATURES = {
     "vx_decode_ffn_supported": (_i, [_vp, _vp, _vp, _vp]),
     "vx_decode_ffn": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _vp]),
     "vx_rope_store_paged": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f]),
+    "vx_rope_store_paged_ex": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i]),
     "vx_sdpa_paged_decode_split_supported": (_i, [_i, _i, _i, _i, _i]),
     "vx_sdpa_paged_decode_ragged": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i]),
     "vx_sdpa_paged_tree": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),

@@ -35,6 +35,22 @@ class VhLayerWeights(C.Structure):
                [(n, VhQWeight) for n in ("wq", "wk", "wv", "wo", "w1", "w2", "w3")]
 
 
+class VhArch(C.Structure):
+    _fields_ = [(n, C.c_int) for n in ("norm_type", "mlp_type", "parallel_residual", "rope_dim", "rope_neox",
+                                        "post_norms")] + [("attn_softcap", C.c_float), ("embedding_scale", C.c_float)]
+
+
+EXTRA_NAMES = ("attn_norm_bias", "ffn_norm_bias", "wq_bias", "wk_bias", "wv_bias", "wo_bias", "w1_bias", "w2_bias",
+               "post_attn_norm", "post_ffn_norm")
+
+
+class VhLayerExtras(C.Structure):
+    _fields_ = [(n, C.c_void_p) for n in EXTRA_NAMES]
+
+
+NORM_TYPES = {"rms": 0, "layer": 1}
+MLP_TYPES = {"swiglu": 0, "gelu": 1, "geglu": 2}
+
 _host = None
 
 
@@ -60,6 +76,9 @@ def load_host():
         h.vh_model_set_fused.restype = None
         h.vh_model_set_layer.argtypes = [C.c_void_p, C.c_int, C.POINTER(VhLayerWeights)]
         h.vh_model_set_head.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.POINTER(VhQWeight)]
+        h.vh_model_set_architecture.argtypes = [C.c_void_p, C.POINTER(VhArch)]
+        h.vh_model_set_layer_extras.argtypes = [C.c_void_p, C.c_int, C.POINTER(VhLayerExtras)]
+        h.vh_model_set_final_norm_bias.argtypes = [C.c_void_p, C.c_void_p]
         for name in ("vh_pool_create_sequence", "vh_pool_delete_sequence", "vh_pool_has_sequence", "vh_pool_seq_len"):
             getattr(h, name).argtypes = [C.c_void_p, C.c_int64]
         h.vh_pool_truncate_sequence.argtypes = [C.c_void_p, C.c_int64, C.c_int]
@@ -222,10 +241,33 @@ class ModelRuntime:
         lw.attn_norm = attn_norm if isinstance(attn_norm, int) else self._up(np.asarray(attn_norm, dtype=np.float32))
         lw.ffn_norm = ffn_norm if isinstance(ffn_norm, int) else self._up(np.asarray(ffn_norm, dtype=np.float32))
         for name in ("wq", "wk", "wv", "wo", "w1", "w2", "w3"):
+            if weights.get(name) is None:          # w3 of a GELU MLP
+                continue
             fmt, data, n, k = weights[name]
             ptr = data if isinstance(data, int) else self._up(data)
             setattr(lw, name, VhQWeight(fmt, ptr, n, k))
         self._ck(self._h.vh_model_set_layer(self._m, layer, C.byref(lw)))
+
+    def set_architecture(self, norm_type="rms", mlp_type="swiglu", parallel_residual=False, rope_dim=0, rope_neox=False,
+                         post_norms=False, attn_softcap=0.0, embedding_scale=0.0):
+        """The switches of runtime/config.go:14-62,120-131; any non-default one selects block.go's general sequence."""
+        a = VhArch(NORM_TYPES[norm_type], MLP_TYPES[mlp_type], int(bool(parallel_residual)), rope_dim,
+                   int(bool(rope_neox)), int(bool(post_norms)), attn_softcap, embedding_scale)
+        self._ck(self._h.vh_model_set_architecture(self._m, C.byref(a)))
+
+    def set_layer_extras(self, layer, **tensors):
+        """Biases and post-norm weights of a layer (block.go:266-283): float32 vectors by name, absent = None."""
+        e = VhLayerExtras()
+        for name, arr in tensors.items():
+            if name not in EXTRA_NAMES:
+                raise KeyError(name)
+            if arr is not None:
+                setattr(e, name, arr if isinstance(arr, int) else self._up(np.asarray(arr, dtype=np.float32)))
+        self._ck(self._h.vh_model_set_layer_extras(self._m, layer, C.byref(e)))
+
+    def set_final_norm_bias(self, bias):
+        self._ck(self._h.vh_model_set_final_norm_bias(
+            self._m, bias if isinstance(bias, int) else self._up(np.asarray(bias, dtype=np.float32))))
 
     def set_head(self, embedding_f32, final_norm, lm_head):
         """embedding_f32: numpy [vocab,hidden] float32 or device pointer; lm_head: (fmt, data, n, k)."""
