@@ -117,6 +117,19 @@ int vx_sdpa_prefill_softcap(vx_backend *be, const float *q, const float *k, cons
 int vx_rope_with_freqs(vx_backend *be, float *q, float *k, const float *freqs, int head_dim, int num_heads,
                        int num_kv_heads, int seq_len, int start_pos, int rope_neox);
 
+/* ---- Medusa prediction heads (inference/medusa/heads.go) ---- */
+/* Heads.ForwardAll (heads.go:83-128) for `rows` (<= 8) hidden states at once: for every head h,
+ * intermediate[h][r] = SiLU(hidden[r] . FC1[h]) and logits[h][r] = intermediate[h][r] . FC2[h], with SiLU(x) =
+ * x / (1 + exp(-x)). fc1 [heads][hidden][hidden] and fc2 [heads][hidden][vocab] are float32 with the input index
+ * first, as Head.FC1 / FC2 hold them; hidden [rows][hidden]; intermediate [heads][rows][hidden] (caller's scratch);
+ * logits [heads][rows][vocab]. hidden and vocab must be multiples of 4. */
+int vx_medusa_forward(vx_backend *be, const float *hidden, const float *fc1, const float *fc2, float *intermediate,
+                      float *logits, int rows, int num_heads, int hidden_size, int vocab_size);
+/* topK (heads.go:146-171) per row of x [rows][n]: the indices of the k largest values, largest first, a tie to the
+ * lower index; out_idx [rows][k] int32, out_val [rows][k] (may be NULL) on the device. Values not above -MaxFloat32
+ * and NaN are never taken: the index is then -1. */
+int vx_topk_rows(vx_backend *be, const float *x, int rows, int n, int k, int32_t *out_idx, float *out_val);
+
 /* ArgmaxOps.Argmax (backend.go:199-203): first index of the strict maximum; waits for the stream. */
 int vx_argmax(vx_backend *be, const float *input, int n, int *out_index);
 

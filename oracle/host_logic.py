@@ -340,6 +340,22 @@ def build_candidate_tree_from_topk(head_topk_tokens, head_topk_vals, max_nodes):
     return tree
 
 
+def medusa_top_k(values, k):
+    """heads.go:146-171 (topK): k rounds, each taking the first strictly largest value not yet used, starting from
+    -MaxFloat32; a round that finds nothing yields -1."""
+    k = min(k, len(values))
+    used, out = [False] * len(values), []
+    for _ in range(k):
+        best_idx, best_val = -1, -3.4028234663852886e38
+        for j, v in enumerate(values):
+            if not used[j] and v > best_val:
+                best_val, best_idx = v, j
+        out.append(best_idx)
+        if best_idx >= 0:
+            used[best_idx] = True
+    return out
+
+
 def top_k_with_values(values, k):
     """tree.go:242-271 for inputs without ties among the top k."""
     k = min(k, len(values))

@@ -263,6 +263,16 @@ def scale_buffer(buf, scale):
     return b
 
 
+def medusa_forward(hidden, fc1, fc2):
+    """heads.go:83-117 for one head: hidden [H], fc1 [H,H], fc2 [H,V] (input index first) -> (intermediate, logits)."""
+    hidden, fc1, fc2 = _f32(hidden), _f32(fc1), _f32(fc2)
+    h, v = fc1.shape[0], fc2.shape[1]
+    assert fc1.shape == (h, h) and fc2.shape == (h, v) and hidden.shape == (h,)
+    inter, logits = np.empty(h, dtype=np.float32), np.empty(v, dtype=np.float32)
+    _lib.vxo_medusa_forward(_p(hidden), _p(fc1), _p(fc2), _p(inter), _p(logits), h, v)
+    return inter, logits
+
+
 def softmax(x, rows, cols):
     """cpu.go:490-518"""
     x = _f32(x)

@@ -694,6 +694,23 @@ VXO_API int vxo_argmax(const float *x, int n) {
     return mi;
 }
 
+/* inference/medusa/heads.go:83-117 (Heads.Forward) for one head: intermediate = silu(hidden . FC1) with
+ * silu(x) = x / (1 + exp(-x)) (heads.go:20-22), logits = intermediate . FC2; FC1 is [hidden, hidden] and FC2
+ * [hidden, vocab], both indexed [in * out_size + out]; every sum runs over the input index in order. */
+VXO_API void vxo_medusa_forward(const float *hidden, const float *fc1, const float *fc2, float *intermediate,
+                                float *logits, int hidden_size, int vocab_size) {
+    for (int i = 0; i < hidden_size; i++) {
+        float sum = 0;
+        for (int j = 0; j < hidden_size; j++) sum += hidden[j] * fc1[(int64_t)j * hidden_size + i];
+        intermediate[i] = sum / (1.0f + (float)exp((double)(-sum)));
+    }
+    for (int i = 0; i < vocab_size; i++) {
+        float sum = 0;
+        for (int j = 0; j < hidden_size; j++) sum += intermediate[j] * fc2[(int64_t)j * vocab_size + i];
+        logits[i] = sum;
+    }
+}
+
 /* ------------------------------------------------------------------------- */
 /* attention                                                                 */
 /* ------------------------------------------------------------------------- */

@@ -1126,3 +1126,59 @@ def test_rope_with_freqs(be, neox):
     be.rope_with_freqs(dq, None, df, d, hq, hk, s, start, neox)
     _close(be.download(dq, q.shape, np.float32), wq, 0, 1e-6, "rope_with_freqs, no k")
     be.reset_pool()
+
+
+# ------------------------------------------------------------------ Medusa heads
+@pytest.mark.parametrize("rows,heads,h,v", [(1, 4, 64, 100), (1, 4, 512, 4000), (3, 2, 256, 1000), (8, 1, 128, 260),
+                                             (5, 3, 100, 36)])
+def test_medusa_forward(be, rows, heads, h, v):
+    """Heads.ForwardAll (medusa/heads.go:83-128) for a few hidden states at once against the oracle's Forward per
+    head and row; then the heads' top-k (heads.go:146-171) against the oracle's selection."""
+    rng = np.random.default_rng(70 + rows + h)
+    hidden = (rng.random((rows, h)) * 2 - 1).astype(np.float32)
+    fc1 = ((rng.random((heads, h, h)) * 2 - 1) * math.sqrt(2.0 / h)).astype(np.float32)
+    fc2 = ((rng.random((heads, h, v)) * 2 - 1) * math.sqrt(2.0 / h)).astype(np.float32)
+    dh, d1, d2 = be.upload(hidden), be.upload(fc1), be.upload(fc2)
+    di, dl = be.alloc(heads * rows * h * 4), be.alloc(heads * rows * v * 4)
+    be.medusa_forward(dh, d1, d2, di, dl, rows, heads, h, v)
+    got_i = be.download(di, (heads, rows, h), np.float32)
+    got_l = be.download(dl, (heads, rows, v), np.float32)
+    for hd in range(heads):
+        for r in range(rows):
+            wi, wl = nx.medusa_forward(hidden[r], fc1[hd], fc2[hd])
+            _close(got_i[hd, r], wi, 1e-5, 2e-6, "medusa intermediate")
+            _close(got_l[hd, r], wl, 1e-5, 5e-6, "medusa logits")
+    k = 5
+    dk, dv = be.alloc(heads * rows * k * 4), be.alloc(heads * rows * k * 4)
+    be.topk_rows(dl, heads * rows, v, k, dk, dv)
+    idx = be.download(dk, (heads * rows, k), np.int32)
+    val = be.download(dv, (heads * rows, k), np.float32)
+    flat = got_l.reshape(heads * rows, v)
+    for r in range(heads * rows):
+        assert idx[r].tolist() == hl.medusa_top_k(flat[r].tolist(), k)
+        assert np.array_equal(val[r], flat[r][idx[r]])
+    be.reset_pool()
+
+
+def test_topk_rows_ties_and_unusable_values(be):
+    x = np.array([[0.5, 2.0, 2.0, -1.0, 3.0, 2.0],
+                  [-np.inf, 1.0, np.nan, -np.inf, -np.inf, np.nan],
+                  [7.0, 7.0, 7.0, 7.0, 7.0, 7.0]], dtype=np.float32)
+    dx = be.upload(x)
+    dk, dv = be.alloc(3 * 6 * 4), be.alloc(3 * 6 * 4)
+    be.topk_rows(dx, 3, 6, 6, dk, dv)
+    idx = be.download(dk, (3, 6), np.int32)
+    for r in range(3):
+        assert idx[r].tolist() == hl.medusa_top_k(x[r].tolist(), 6)
+    assert idx[0].tolist() == [4, 1, 2, 5, 0, 3] and idx[1].tolist() == [1, -1, -1, -1, -1, -1]
+    big = np.random.default_rng(71).standard_normal((2, 128256)).astype(np.float32)
+    big[1, 77] = big[1, 100000] = big[1].max() + 1                  # a tie at the top: the lower index first
+    db = be.upload(big)
+    dk = be.alloc(2 * 10 * 4)
+    be.topk_rows(db, 2, 128256, 10, dk)
+    idx = be.download(dk, (2, 10), np.int32)
+    for r in range(2):
+        assert idx[r].tolist() == np.argsort(-big[r].astype(np.float64), kind="stable")[:10].tolist()
+    with pytest.raises(RuntimeError, match="exceeds the row length"):
+        be.topk_rows(dx, 3, 6, 7, dk)
+    be.reset_pool()

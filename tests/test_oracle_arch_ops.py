@@ -197,3 +197,31 @@ def test_rope_with_custom_freqs_closed_form(neox):
     # position 0: no rotation
     same, _ = nx.rope_with_freqs(q[:1], None, freqs, d, heads, heads, 1, 0, neox)
     assert np.array_equal(same, q[:1])
+
+
+# ---- inference/medusa/medusa_test.go:250-318 (SiLU values, the forward pass spelled out) and heads.go:146-171
+def test_medusa_forward_and_topk():
+    from oracle import host_logic as hl
+    rng = np.random.default_rng(39)
+    h, v = 64, 100                                                  # medusa_test.go:12-14
+    hidden = (rng.random(h) * 2 - 1).astype(np.float32)
+    fc1 = ((rng.random((h, h)) * 2 - 1) * math.sqrt(2.0 / h)).astype(np.float32)   # heads.go:60-75
+    fc2 = ((rng.random((h, v)) * 2 - 1) * math.sqrt(2.0 / h)).astype(np.float32)
+    inter, logits = nx.medusa_forward(hidden, fc1, fc2)
+    pre = hidden.astype(np.float64) @ fc1.astype(np.float64)
+    want_inter = pre / (1.0 + np.exp(-pre))
+    assert np.max(np.abs(inter - want_inter)) <= 2e-6
+    assert np.max(np.abs(logits - want_inter @ fc2.astype(np.float64))) <= 5e-6
+    # medusa_test.go:297-317: silu(-1) ≈ -0.2689, silu(0) = 0, silu(1) ≈ 0.7311, through a one-column identity FC1
+    eye = np.eye(4, dtype=np.float32)
+    got, _ = nx.medusa_forward([-1.0, 0.0, 1.0, -2.0], eye, eye)
+    assert abs(got[0] + 0.2689) < 1e-4 and got[1] == 0.0 and abs(got[2] - 0.7311) < 1e-4 and abs(got[3] + 0.2384) < 1e-4
+    # a transposed FC1 would be a different product
+    t_inter, _ = nx.medusa_forward(hidden, fc1.T.copy(), fc2)
+    assert np.max(np.abs(t_inter - inter)) > 1e-2
+    # top-k: largest first, the first of equal values, -1 when nothing is above -MaxFloat32
+    assert hl.medusa_top_k([0.5, 2.0, 2.0, -1.0, 3.0], 4) == [4, 1, 2, 0]
+    assert hl.medusa_top_k([float("-inf"), 1.0], 2) == [1, -1]
+    assert hl.medusa_top_k([1.0, float("nan"), 2.0], 3) == [2, 0, -1]
+    top = hl.medusa_top_k(logits.tolist(), 5)
+    assert top == np.argsort(-logits.astype(np.float64), kind="stable")[:5].tolist()

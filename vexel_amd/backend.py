@@ -150,6 +150,13 @@ class HipBackend:
     def sdpa_prefill(self, q, k, v, out, seq_len, num_q_heads, num_kv_heads, head_dim, scale):
         self.call("vx_sdpa_prefill", q, k, v, out, seq_len, num_q_heads, num_kv_heads, head_dim, scale)
 
+    # ---- Medusa heads (medusa/heads.go)
+    def medusa_forward(self, hidden, fc1, fc2, intermediate, logits, rows, num_heads, hidden_size, vocab_size):
+        self.call("vx_medusa_forward", hidden, fc1, fc2, intermediate, logits, rows, num_heads, hidden_size, vocab_size)
+
+    def topk_rows(self, x, rows, n, k, out_idx, out_val=None):
+        self.call("vx_topk_rows", x, rows, n, k, out_idx, out_val)
+
     # ---- optional interfaces (backend.go:205-263)
     def layernorm(self, x, weight, bias, out, rows, cols, eps):
         self.call("vx_layernorm", x, weight, bias, out, rows, cols, eps)

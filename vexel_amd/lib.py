@@ -42,6 +42,8 @@ SIGNATURES = {
     "vx_sdpa": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f, _i]),
     "vx_sdpa_prefill": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _f]),
     "vx_argmax": (_i, [_vp, _vp, _i, C.POINTER(_i)]),
+    "vx_medusa_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
+    "vx_topk_rows": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
     "vx_layernorm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f]),
     "vx_gelu": (_i, [_vp, _vp, _vp, _i]),
     "vx_gelu_mul": (_i, [_vp, _vp, _vp, _vp, _i]),
