@@ -112,6 +112,9 @@ int vx_sdpa_softcap(vx_backend *be, const float *q, const float *k, const float 
                     int num_q_heads, int num_kv_heads, int head_dim, float scale, float softcap, int kv_head_stride);
 int vx_sdpa_prefill_softcap(vx_backend *be, const float *q, const float *k, const float *v, float *out, int seq_len,
                             int num_q_heads, int num_kv_heads, int head_dim, float scale, float softcap);
+/* ModelRuntime.ApplyFinalLogitSoftCap (runtime/model.go:336-350; the reference runs it on the host copy of the logits
+ * a request is sampled from): logits[i] = cap * tanh(logits[i] / cap) in float64, in place; cap <= 0 = off. */
+int vx_logit_softcap(vx_backend *be, float *logits, int n, float cap);
 /* ScaledRoPEOps.RoPEWithFreqs (backend.go:247-249, cpu.go:308-375): RoPE over the whole head with pair j turning
  * by position * freqs[j] (head_dim / 2 floats on the device). k may be NULL. */
 int vx_rope_with_freqs(vx_backend *be, float *q, float *k, const float *freqs, int head_dim, int num_heads,

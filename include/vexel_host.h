@@ -52,6 +52,9 @@ typedef struct vh_arch {
     float attn_softcap;      /* AttentionLogitSoftCap: applied where block.go applies it on the paged path, the
                                 first prefill chunk (block.go:891-892) */
     float embedding_scale;   /* EmbeddingScale, <= 0 = none (decode.go:197-205) */
+    float final_softcap;     /* FinalLogitSoftCap (model.go:336-350): applied, as in the reference, to the logits a
+                                request is sampled from (scheduler.go:772-773), not to what vh_prefill and
+                                vh_decode_batched return, and not before a greedy arg-max */
 } vh_arch;
 typedef struct vh_layer_extras {  /* the BlockRuntime tensors beside vh_layer_weights (block.go:266-283); NULL = absent */
     const float *attn_norm_bias, *ffn_norm_bias;
@@ -78,6 +81,7 @@ int vh_model_set_layer(vh_model *m, int layer, const vh_layer_weights *w);
  * decode entry points and vh_verify_tree are for the LLaMA arm. With the GELU MLP a layer's w3 may be empty.
  * All pointers are float32 device vectors that outlive the model's use of them. */
 int vh_model_set_architecture(vh_model *m, const vh_arch *arch);
+void vh_model_get_architecture(const vh_model *m, vh_arch *out);
 int vh_model_set_layer_extras(vh_model *m, int layer, const vh_layer_extras *extras);
 int vh_model_set_final_norm_bias(vh_model *m, const float *bias);  /* Model.FinalNormBias (model.go:36, 207-219) */
 /* embedding: F32 [vocab,hidden] on the device (loader rule, runtime/loader.go:275-288) */

@@ -599,6 +599,10 @@ class Scheduler:
         t, k, p, st = q.sampling
         r, st = splitmix_uniform(st)
         q.sampling = (t, k, p, st)
+        cap = getattr(getattr(self.model, "cfg", None), "final_softcap", 0.0)
+        if cap > 0:                      # scheduler.go:772-773 -> model.go:336-350, sampled requests only
+            from . import numerics as nx
+            logits = nx.logit_softcap(logits, cap)
         return sampler_sample(logits, t, k, p, r)
 
     def step(self):

@@ -44,6 +44,7 @@ class ModelConfig:
     attn_softcap: float = 0.0         # AttentionLogitSoftCap
     post_norms: bool = False          # HasPostNorms
     embedding_scale: float = 0.0      # EmbeddingScale, <= 0 = none (decode.go:197-205)
+    final_softcap: float = 0.0        # FinalLogitSoftCap: on the logits a request is sampled from (scheduler.go:772-773)
 
 
 @dataclass
@@ -373,4 +374,5 @@ def random_model(cfg: ModelConfig, seed, fmt, head_fmt, emb_fmt=None, max_blocks
 def is_llama(cfg: ModelConfig):
     """Every architecture switch at its default."""
     return (cfg.norm_type == "rms" and cfg.mlp_type == "swiglu" and not cfg.parallel_residual and cfg.rope_dim == 0
-            and not cfg.rope_neox and cfg.attn_softcap == 0 and not cfg.post_norms and cfg.embedding_scale <= 0)
+            and not cfg.rope_neox and cfg.attn_softcap == 0 and not cfg.post_norms and cfg.embedding_scale <= 0
+            and cfg.final_softcap <= 0)

@@ -263,6 +263,13 @@ def scale_buffer(buf, scale):
     return b
 
 
+def logit_softcap(logits, cap):
+    """model.go:336-350; returns the capped copy."""
+    out = _f32(logits).copy()
+    _lib.vxo_logit_softcap(_p(out), C.c_int64(out.size), C.c_float(cap))
+    return out
+
+
 def medusa_forward(hidden, fc1, fc2):
     """heads.go:83-117 for one head: hidden [H], fc1 [H,H], fc2 [H,V] (input index first) -> (intermediate, logits)."""
     hidden, fc1, fc2 = _f32(hidden), _f32(fc1), _f32(fc2)

@@ -694,6 +694,14 @@ VXO_API int vxo_argmax(const float *x, int n) {
     return mi;
 }
 
+/* inference/runtime/model.go:336-350 (ApplyFinalLogitSoftCap): float32(float64(cap) * tanh(float64(x) * invCap))
+ * with invCap = 1.0 / float64(cap), in place; cap <= 0 changes nothing. */
+VXO_API void vxo_logit_softcap(float *logits, int64_t n, float cap) {
+    if (cap <= 0) return;
+    double inv_cap = 1.0 / (double)cap;
+    for (int64_t i = 0; i < n; i++) logits[i] = (float)((double)cap * tanh((double)logits[i] * inv_cap));
+}
+
 /* inference/medusa/heads.go:83-117 (Heads.Forward) for one head: intermediate = silu(hidden . FC1) with
  * silu(x) = x / (1 + exp(-x)) (heads.go:20-22), logits = intermediate . FC2; FC1 is [hidden, hidden] and FC2
  * [hidden, vocab], both indexed [in * out_size + out]; every sum runs over the input index in order. */

@@ -17,7 +17,7 @@ def gpu_model_from_oracle(be, omodel, pool_blocks, max_seqs=64, max_blocks_per_s
     from vexel_amd.runtime import EXTRA_NAMES
     if not is_llama(c):
         mr.set_architecture(c.norm_type, c.mlp_type, c.parallel_residual, c.rope_dim, c.rope_neox, c.post_norms,
-                            c.attn_softcap, c.embedding_scale)
+                            c.attn_softcap, c.embedding_scale, c.final_softcap)
     for i, lw in enumerate(omodel.layers):
         ws = {n: (getattr(lw, n).fmt, getattr(lw, n).data, getattr(lw, n).n, getattr(lw, n).k)
               for n in ("wq", "wk", "wv", "wo", "w1", "w2", "w3") if getattr(lw, n) is not None}

@@ -1064,6 +1064,15 @@ def test_layernorm_gelu_bias_scale(be):
     be.scale_buffer(du, float(np.float32(math.sqrt(2304.0))), n)
     assert np.array_equal(be.download(du, (n,), np.float32), nx.scale_buffer(u, np.float32(math.sqrt(2304.0))))
     be.gelu(dg, do, 0)                                              # nothing to do
+    # ApplyFinalLogitSoftCap (model.go:336-350): float64 tanh, bit for bit but for the device's tanh
+    lg = np.concatenate([rng.standard_normal(n - 4) * 40, [0.0, 1e30, -1e30, 1e-8]]).astype(np.float32)
+    dl = be.upload(lg)
+    be.logit_softcap(dl, n, 30.0)
+    got, want = be.download(dl, (n,), np.float32), nx.logit_softcap(lg, 30.0)
+    _close(got, want, 2e-7, 1e-9, "logit_softcap")
+    assert np.mean(got.view(np.uint32) == want.view(np.uint32)) > 0.999
+    be.logit_softcap(dl, n, 0.0)                                    # disabled: unchanged
+    assert np.array_equal(be.download(dl, (n,), np.float32), got)
     be.reset_pool()
 
 

@@ -553,3 +553,48 @@ def test_architecture_switches_are_validated(be):
     b = mr.prefill_with_paged_kv(prompt, 2, 0)
     assert_logits_close(b, a, "rope_dim = head_dim")
     mr.close()
+
+
+def test_scheduler_caps_the_logits_of_sampled_requests(be):
+    """FinalLogitSoftCap (model.go:336-350) reaches only the logits a request is sampled from (scheduler.go:772-773):
+    a Gemma-2-like model with a small cap, two sampled requests and a greedy one, C++ scheduler against its oracle
+    restatement token by token; without the cap the sampled requests would have drawn other tokens."""
+    import copy
+    from oracle import host_logic as hl
+    from vexel_amd.runtime import Scheduler
+    cfg = _arch_config("gemma")
+    cfg.final_softcap = 0.5
+    omodel = om.random_model(cfg, 81, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=24)
+    plain = copy.deepcopy(omodel)
+    plain.cfg = copy.copy(cfg)
+    plain.cfg.final_softcap = 0.0
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=24, max_seqs=4, max_batch=8)
+    rng = np.random.default_rng(82)
+    prompts = {1: rng.integers(0, cfg.vocab, 9).tolist(), 2: rng.integers(0, cfg.vocab, 20).tolist(),
+               3: rng.integers(0, cfg.vocab, 5).tolist()}
+    sampled = {1: (1.5, 0, 1.0, 7), 3: (0.9, 50, 0.95, 8)}
+    want, other = hl.Scheduler(omodel, 4, 10, -1), hl.Scheduler(plain, 4, 10, -1)
+    got = Scheduler(mr, 4, max_tokens=10, eos_token=-1)
+    for i, p in prompts.items():
+        for sch in (want, other):
+            sch.add_sequence(i, p, 10)
+            if i in sampled:
+                sch.seqs[i].sampling = sampled[i]
+        got.add_sequence(i, p, 10)
+        if i in sampled:
+            got.set_sampling(i, *sampled[i])
+    capped, uncapped = {}, {}
+    for step in range(12):
+        nw, ng = want.step(), got.step()
+        other.step()
+        assert nw == ng
+        for i, q in want.seqs.items():
+            assert got.generated(i) == q.generated, (step, i)
+            capped[i] = list(q.generated)
+        for i, q in other.seqs.items():
+            uncapped[i] = list(q.generated)
+    assert all(len(capped[i]) == 10 for i in prompts)
+    assert capped[1] != uncapped[1] and capped[3] != uncapped[3]
+    assert capped[2] == uncapped[2]                                 # the greedy request never sees the cap
+    got.close()
+    mr.close()

@@ -225,3 +225,15 @@ def test_medusa_forward_and_topk():
     assert hl.medusa_top_k([1.0, float("nan"), 2.0], 3) == [2, 0, -1]
     top = hl.medusa_top_k(logits.tolist(), 5)
     assert top == np.argsort(-logits.astype(np.float64), kind="stable")[:5].tolist()
+
+
+# ---- runtime/model.go:336-350 (ApplyFinalLogitSoftCap)
+def test_logit_softcap_closed_form():
+    x = np.concatenate([np.linspace(-200, 200, 4001), [0.0, 1e-8, 1e30, -1e30]]).astype(np.float32)
+    got = nx.logit_softcap(x, 30.0)
+    want = 30.0 * np.tanh(x.astype(np.float64) / 30.0)
+    assert np.max(np.abs(got - want)) <= 2e-6
+    assert np.all(np.abs(got) <= 30.0) and got[-2] == 30.0 and got[-1] == -30.0
+    assert np.all(np.diff(got[:4001]) >= 0)                        # monotone: the greedy choice is unchanged
+    assert np.max(np.abs(got[1900:2101] - x[1900:2101])) < 0.4     # near 0 it is almost the identity
+    assert np.array_equal(nx.logit_softcap(x, 0.0), x)             # disabled

@@ -170,6 +170,9 @@ class HipBackend:
     def add_bias(self, x, bias, out, rows, cols):
         self.call("vx_add_bias", x, bias, out, rows, cols)
 
+    def logit_softcap(self, logits, n, cap):
+        self.call("vx_logit_softcap", logits, n, cap)
+
     def scale_buffer(self, buf, scale, n):
         self.call("vx_scale_buffer", buf, scale, n)
 

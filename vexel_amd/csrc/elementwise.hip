@@ -240,6 +240,12 @@ __global__ void scale_kernel(float *buf, float scale, int n) {
     if (i < n) buf[i] = __fmul_rn(buf[i], scale);
 }
 
+// model.go:336-350: float32(float64(cap) * tanh(float64(x) / cap)) with the quotient as a product by 1 / float64(cap)
+__global__ void logit_softcap_kernel(float *x, double cap, double inv_cap, int n) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = (float)(cap * tanh((double)x[i] * inv_cap));
+}
+
 // cpu.go:308-375: RoPE over the whole head, pair j turning by position * freqs[j]. grid.x = row.
 __global__ void rope_freqs_kernel(float *q, float *k, const float *freqs, int head_dim, int num_heads, int num_kv_heads,
                                   int start_pos, int neox) {
@@ -643,6 +649,12 @@ int vx_gelu_mul(vx_backend *be, const float *gate, const float *up, float *out, 
 int vx_scale_buffer(vx_backend *be, float *buf, float scale, int n) {
     VX_REQUIRE(buf, "vx_scale_buffer: null pointer");
     VX_EW("vx_scale_buffer", scale_kernel, buf, scale)
+}
+
+int vx_logit_softcap(vx_backend *be, float *logits, int n, float cap) {
+    VX_REQUIRE(logits, "vx_logit_softcap: null pointer");
+    if (cap <= 0.f) return enter(be);  // disabled (model.go:342-344)
+    VX_EW("vx_logit_softcap", logit_softcap_kernel, logits, (double)cap, 1.0 / (double)cap)
 }
 
 int vx_add_bias(vx_backend *be, const float *x, const float *bias, float *out, int rows, int cols) {

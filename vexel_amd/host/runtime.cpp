@@ -552,7 +552,7 @@ int vh_model_set_architecture(vh_model *m, const vh_arch *arch) {
         return fail("the parallel residual goes with the GELU MLP only");  // block.go:972-976 shares a buffer with W3's product
     if (a.rope_dim < 0 || a.rope_dim > m->cfg.head_dim || a.rope_dim % 2 != 0)
         return fail("rope_dim %d invalid for head_dim %d", a.rope_dim, m->cfg.head_dim);
-    if (a.attn_softcap < 0.f) return fail("negative attention soft cap");
+    if (a.attn_softcap < 0.f || a.final_softcap < 0.f) return fail("negative soft cap");
     if (a.mlp_type == VH_MLP_GELU && m->cfg.ffn < m->cfg.hidden && a.parallel_residual)
         return fail("the parallel residual keeps the attention output in an [rows, ffn] buffer: ffn %d < hidden %d", m->cfg.ffn,
                     m->cfg.hidden);
@@ -566,6 +566,10 @@ int vh_model_set_architecture(vh_model *m, const vh_arch *arch) {
     drop_graph(m);
     refresh_general(m);
     return VH_OK;
+}
+
+void vh_model_get_architecture(const vh_model *m, vh_arch *out) {
+    if (m && out) *out = m->arch;
 }
 
 int vh_model_set_layer_extras(vh_model *m, int layer, const vh_layer_extras *extras) {
@@ -795,6 +799,10 @@ int vh_sample_last_logits(vh_model *m, int rows, const float *temperature, const
     VXC(vx_to_device(be, d_k, top_k, (size_t)rows * 4));
     VXC(vx_to_device(be, d_p, top_p, (size_t)rows * 4));
     VXC(vx_to_device(be, d_u, uniform, (size_t)rows * 4));
+    if (m->arch.final_softcap > 0.f)  // scheduler.go:772-773: the logits a request is sampled from are capped first
+        for (int r = 0; r < rows; r++)
+            if (temperature[r] > 0.f)
+                VXC(vx_logit_softcap(be, m->logits + (size_t)r * m->cfg.vocab, m->cfg.vocab, m->arch.final_softcap));
     VXC(vx_sample_rows(be, m->logits, rows, m->cfg.vocab, d_t, d_k, d_p, d_u, d_out));
     VXC(vx_to_host(be, tokens_out, d_out, (size_t)rows * 4));
     VXC(vx_sync(be));

@@ -257,8 +257,14 @@ int vh_sched_step(vh_scheduler *s, int *tokens_out) {
         return VH_OK;
     }
     auto is_stop = [&](int tok) { return tok == s->cfg.eos_token; };  // scheduler.go:110-116 (primary EOS)
-    auto pick = [&](Seq &q, const float *row, int device_argmax) {
+    vh_arch arch;
+    vh_model_get_architecture(s->m, &arch);
+    auto pick = [&](Seq &q, float *row, int device_argmax) {
         if (!q.sampled) return device_argmax >= 0 ? device_argmax : vh_argmax(row, V);
+        if (arch.final_softcap > 0.f) {  // model.go:336-350 on the host copy (scheduler.go:772-773)
+            const double cap = (double)arch.final_softcap, inv_cap = 1.0 / cap;
+            for (int i = 0; i < V; i++) row[i] = (float)(cap * tanh((double)row[i] * inv_cap));
+        }
         return vh_sample(row, V, q.temperature, q.top_k, q.top_p, next_uniform(&q.rng));
     };
     int produced = 0;

@@ -44,6 +44,7 @@ SIGNATURES = {
     "vx_argmax": (_i, [_vp, _vp, _i, C.POINTER(_i)]),
     "vx_medusa_forward": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i]),
     "vx_topk_rows": (_i, [_vp, _vp, _i, _i, _i, _vp, _vp]),
+    "vx_logit_softcap": (_i, [_vp, _vp, _i, _f]),
     "vx_layernorm": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _f]),
     "vx_gelu": (_i, [_vp, _vp, _vp, _i]),
     "vx_gelu_mul": (_i, [_vp, _vp, _vp, _vp, _i]),

@@ -37,7 +37,8 @@ class VhLayerWeights(C.Structure):
 
 class VhArch(C.Structure):
     _fields_ = [(n, C.c_int) for n in ("norm_type", "mlp_type", "parallel_residual", "rope_dim", "rope_neox",
-                                        "post_norms")] + [("attn_softcap", C.c_float), ("embedding_scale", C.c_float)]
+                                        "post_norms")] + [("attn_softcap", C.c_float), ("embedding_scale", C.c_float),
+                                                         ("final_softcap", C.c_float)]
 
 
 EXTRA_NAMES = ("attn_norm_bias", "ffn_norm_bias", "wq_bias", "wk_bias", "wv_bias", "wo_bias", "w1_bias", "w2_bias",
@@ -249,10 +250,10 @@ class ModelRuntime:
         self._ck(self._h.vh_model_set_layer(self._m, layer, C.byref(lw)))
 
     def set_architecture(self, norm_type="rms", mlp_type="swiglu", parallel_residual=False, rope_dim=0, rope_neox=False,
-                         post_norms=False, attn_softcap=0.0, embedding_scale=0.0):
+                         post_norms=False, attn_softcap=0.0, embedding_scale=0.0, final_softcap=0.0):
         """The switches of runtime/config.go:14-62,120-131; any non-default one selects block.go's general sequence."""
         a = VhArch(NORM_TYPES[norm_type], MLP_TYPES[mlp_type], int(bool(parallel_residual)), rope_dim,
-                   int(bool(rope_neox)), int(bool(post_norms)), attn_softcap, embedding_scale)
+                   int(bool(rope_neox)), int(bool(post_norms)), attn_softcap, embedding_scale, final_softcap)
         self._ck(self._h.vh_model_set_architecture(self._m, C.byref(a)))
 
     def set_layer_extras(self, layer, **tensors):
