@@ -426,6 +426,41 @@ def configs_report(be):
     mr.close()
 
 
+def medusa_report(be):
+    """Medusa head inference (medusa/heads.go:83-171) at the 7B shape: all heads' FC1 / FC2 in one pass, then the
+    per-head top-k. Weights are float32; GB/s counts the weight bytes against the 8 TB/s HBM peak."""
+    rng = np.random.default_rng(0)
+    print("heads hidden  vocab rows  forward ms  GB/s  of 8TB  top-10 ms")
+    for heads, h, v, rows in ((4, 4096, 32000, 1), (4, 4096, 32000, 8), (4, 2048, 32000, 1), (4, 4096, 128256, 1)):
+        d1 = be.alloc_permanent(heads * h * h * 4)
+        d2 = be.alloc_permanent(heads * h * v * 4)
+        piece = (rng.standard_normal(h * 1000) * 0.02).astype(np.float32)
+        for base, total in ((d1, heads * h * h), (d2, heads * h * v)):
+            off = 0
+            while off < total:
+                n = min(piece.size, total - off)
+                be.to_device(base + off * 4, piece[:n])
+                off += n
+        dh = be.upload(rng.standard_normal((rows, h)).astype(np.float32), permanent=True)
+        di, dl = be.alloc_permanent(heads * rows * h * 4), be.alloc_permanent(heads * rows * v * 4)
+        dk, dv = be.alloc_permanent(heads * rows * 10 * 4), be.alloc_permanent(heads * rows * 10 * 4)
+        for _ in range(3):
+            be.medusa_forward(dh, d1, d2, di, dl, rows, heads, h, v)
+        be.sync()
+        be.timer_start()
+        for _ in range(20):
+            be.medusa_forward(dh, d1, d2, di, dl, rows, heads, h, v)
+        ms = be.timer_stop_ms() / 20
+        be.timer_start()
+        for _ in range(20):
+            be.topk_rows(dl, heads * rows, v, 10, dk, dv)
+        ms_k = be.timer_stop_ms() / 20
+        gbs = heads * (h * h + h * v) * 4 / ms / 1e6
+        print("%5d %6d %6d %4d  %10.3f %5.0f  %6.3f  %9.3f" % (heads, h, v, rows, ms, gbs, gbs / 8000, ms_k), flush=True)
+        for ptr in (d1, d2, dh, di, dl, dk, dv):
+            be.free(ptr)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -446,6 +481,8 @@ def main():
     ap.add_argument("--prefill-probe", action="store_true",
                     help="for rocprofv3 --pmc runs of the MFMA kernels: 512-row GEMMs of the 7B shapes and one "
                          "512-token prefill attention, then exit")
+    ap.add_argument("--medusa-report", action="store_true",
+                    help="time the Medusa heads' forward pass and top-k at the 7B shape, then exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -460,6 +497,9 @@ def main():
         return
     if args.configs_report:
         configs_report(be)
+        return
+    if args.medusa_report:
+        medusa_report(be)
         return
     ctx = ragged_contexts(n=args.seqs) if args.seqs != BATCH else ragged_contexts()
     nseq = len(ctx)

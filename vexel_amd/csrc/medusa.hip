@@ -75,7 +75,16 @@ __global__ void kn_reduce_kernel(const float *__restrict__ P, float *__restrict_
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
     float t = 0.f;
-    for (int s = 0; s < splits; s++) t += P[(size_t)s * total + i];
+    int s = 0;
+    for (; s + 4 <= splits; s += 4) {  // four loads in flight, added in split order
+        const float p0 = P[(size_t)s * total + i], p1 = P[(size_t)(s + 1) * total + i];
+        const float p2 = P[(size_t)(s + 2) * total + i], p3 = P[(size_t)(s + 3) * total + i];
+        t += p0;
+        t += p1;
+        t += p2;
+        t += p3;
+    }
+    for (; s < splits; s++) t += P[(size_t)s * total + i];
     if (SILU) t = t / (1.0f + (float)exp((double)(-t)));  // heads.go:20-22
     out[i] = t;
 }
