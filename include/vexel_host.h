@@ -164,6 +164,7 @@ typedef struct vh_gguf_config {  /* File.extractModelConfig (gguf.go:504-582); 0
     int num_layers, hidden, num_heads, num_kv_heads, ffn, context_length, vocab, rope_dim_count, head_dim;
     float rope_theta;            /* 10000 when absent */
     float rms_eps;
+    float attn_softcap, final_softcap; /* <arch>.attn_logit_softcapping / final_logit_softcapping (gguf.go:560-566) */
 } vh_gguf_config;
 /* gguf.Open (gguf.go:249-335): magic, version 2..3, metadata, tensor table, aligned data offset. The file is
  * mapped read-only; nothing is copied until a tensor is used. */
@@ -190,8 +191,12 @@ typedef struct vh_load_options {  /* what the checkpoint does not say: the KV po
     int block_size;               /* 0 = 16 */
     int pool_blocks, max_seqs, max_blocks_per_seq, max_batch, kv_fp16;
 } vh_load_options;
-/* ModelRuntime.LoadWeightsGGUF + CopyWeightsToDevice (runtime/loader.go:28-212, 560-700) for LLaMA-family
- * checkpoints: Q4_0 / Q8_0 / Q4_K / Q6_K / Q5_0 / Q5_K / BF16 projection matrices and output head go to the
+/* ModelRuntime.LoadWeightsGGUF + CopyWeightsToDevice (runtime/loader.go:28-212, 560-700). general.architecture
+ * selects the switches as ModelConfigFromGGUF does (runtime/config.go:388-470): llama / mistral; qwen2 (Q/K/V biases,
+ * split-pair RoPE); gemma and gemma2 (GeGLU, embeddings times sqrt(hidden); gemma2 also post-norms and the soft
+ * caps); phi / phi2 (LayerNorm and biases, GELU MLP, parallel residual, partial split-pair RoPE, the fused
+ * attn_qkv matrix used in place as three row ranges, loader.go:610-640). Any other architecture is refused. For
+ * all of them: Q4_0 / Q8_0 / Q4_K / Q6_K / Q5_0 / Q5_K / BF16 projection matrices and output head go to the
  * device as raw blocks, token_embd and the norm vectors as float32 (F32, F16 or one of those types in the file), a missing
  * output.weight is the embedding. One difference: a Q4_0 output head stays Q4_0 here, where the reference
  * dequantizes it to float32 at load (same values, float32 summation order aside). The model owns the device

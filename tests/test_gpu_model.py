@@ -598,3 +598,97 @@ def test_scheduler_caps_the_logits_of_sampled_requests(be):
     assert capped[2] == uncapped[2]                                 # the greedy request never sees the cap
     got.close()
     mr.close()
+
+
+def _gguf_from_oracle(omodel, arch, extra_md=()):
+    """The oracle model as the tensors and metadata a GGUF file of that architecture holds (pkg/gguf/loader.go:121-228
+    names): Phi with its fused attn_qkv matrix and bias, fc1 / fc2 as ffn_up / ffn_down, no ffn_norm."""
+    from oracle import gguf as og
+    cfg = omodel.cfg
+    f32 = lambda name, a: (name, [int(a.size)], og.T_F32, np.ascontiguousarray(a, dtype=np.float32).tobytes())
+    mat = lambda name, q: (name, [q.k, q.n], GGUF_TYPE[q.fmt], q.data.tobytes())
+    tensors = []
+    for l, lw in enumerate(omodel.layers):
+        b = "blk.%d." % l
+        tensors.append(f32(b + "attn_norm.weight", lw.attn_norm))
+        if arch == "phi2":
+            fused = np.concatenate([lw.wq.data, lw.wk.data, lw.wv.data], axis=0)
+            tensors.append((b + "attn_qkv.weight", [lw.wq.k, lw.wq.n + 2 * lw.wk.n], GGUF_TYPE[lw.wq.fmt], fused.tobytes()))
+            tensors.append(f32(b + "attn_qkv.bias", np.concatenate([lw.wq_bias, lw.wk_bias, lw.wv_bias])))
+            tensors += [f32(b + "attn_norm.bias", lw.attn_norm_bias), f32(b + "attn_output.bias", lw.wo_bias),
+                        f32(b + "ffn_up.bias", lw.w1_bias), f32(b + "ffn_down.bias", lw.w2_bias)]
+            tensors.append(mat(b + "ffn_up.weight", lw.w1))
+        else:
+            tensors += [mat(b + "attn_q.weight", lw.wq), mat(b + "attn_k.weight", lw.wk), mat(b + "attn_v.weight", lw.wv),
+                        mat(b + "ffn_gate.weight", lw.w1), mat(b + "ffn_up.weight", lw.w3),
+                        f32(b + "ffn_norm.weight", lw.ffn_norm)]
+            if lw.wq_bias is not None:
+                tensors += [f32(b + "attn_q.bias", lw.wq_bias), f32(b + "attn_k.bias", lw.wk_bias),
+                            f32(b + "attn_v.bias", lw.wv_bias)]
+            if lw.post_attn_norm is not None:
+                tensors += [f32(b + "post_attention_norm.weight", lw.post_attn_norm),
+                            f32(b + "post_ffw_norm.weight", lw.post_ffn_norm)]
+        tensors += [mat(b + "attn_output.weight", lw.wo), mat(b + "ffn_down.weight", lw.w2)]
+    tensors.append(f32("output_norm.weight", omodel.final_norm))
+    if omodel.final_norm_bias is not None:
+        tensors.append(f32("output_norm.bias", omodel.final_norm_bias))
+    tensors.append(("token_embd.weight", [cfg.hidden, cfg.vocab], og.T_F32, omodel.embedding.tobytes()))
+    tensors.append(mat("output.weight", omodel.lm_head))
+    p = arch + "."
+    md = [("general.architecture", og.MT_STRING, arch), (p + "block_count", og.MT_U32, cfg.num_layers),
+          (p + "embedding_length", og.MT_U32, cfg.hidden), (p + "attention.head_count", og.MT_U32, cfg.num_heads),
+          (p + "attention.head_count_kv", og.MT_U32, cfg.num_kv_heads), (p + "feed_forward_length", og.MT_U32, cfg.ffn),
+          (p + "context_length", og.MT_U32, 2048), (p + "rope.freq_base", og.MT_F32, cfg.rope_theta),
+          (p + "attention.layer_norm_rms_epsilon", og.MT_F32, cfg.eps)] + list(extra_md)
+    return og.build(md, tensors)
+
+
+@pytest.mark.parametrize("arch", ["phi2", "gemma2", "qwen2"])
+def test_load_gguf_other_architectures(be, tmp_path, arch):
+    """general.architecture selects the switches as ModelConfigFromGGUF does (runtime/config.go:388-470) and the
+    loader finds each architecture's tensors (runtime/loader.go:290-385): the loaded model gives the oracle's logits
+    and greedy tokens. Gemma 2 takes interleaved RoPE pairs here, as the reference's table has it."""
+    import copy, os
+    from oracle import gguf as og
+    from vexel_amd.backend import VexelError
+    from vexel_amd.runtime import ModelRuntime
+    cfg = _arch_config({"phi2": "phi", "gemma2": "gemma", "qwen2": "qwen"}[arch])
+    extra = []
+    if arch == "gemma2":
+        cfg.rope_neox, cfg.final_softcap = False, 30.0
+        extra = [("gemma2.attention.key_length", og.MT_U32, cfg.head_dim), ("gemma2.attn_logit_softcapping", og.MT_F32, 50.0),
+                 ("gemma2.final_logit_softcapping", og.MT_F32, 30.0)]
+    if arch == "phi2":
+        cfg.eps = 1e-5
+        extra = [("phi2.rope.dimension_count", og.MT_U32, cfg.rope_dim)]
+    omodel = om.random_model(cfg, 91, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=16)
+    if arch == "qwen2":
+        rng = np.random.default_rng(92)
+        for lw in omodel.layers:
+            lw.wq_bias = (0.05 * rng.standard_normal(512)).astype(np.float32)
+            lw.wk_bias = (0.05 * rng.standard_normal(128)).astype(np.float32)
+            lw.wv_bias = (0.05 * rng.standard_normal(128)).astype(np.float32)
+    path = os.path.join(tmp_path, arch + ".gguf")
+    with open(path, "wb") as fh:
+        fh.write(_gguf_from_oracle(omodel, arch, extra))
+    mr = ModelRuntime.from_gguf(be, path, pool_blocks=16, max_seqs=4, max_batch=8)
+    assert mr.cfg.head_dim == cfg.head_dim
+    prompt = np.random.default_rng(93).integers(0, cfg.vocab, 23).tolist()
+    want = omodel.prefill_with_paged_kv(prompt, 1, 0)
+    got = mr.prefill_with_paged_kv(prompt, 1, 0)
+    assert_logits_close(got, want, arch + " prefill from the loaded checkpoint")
+    tok, pos = nx.argmax(want), len(prompt)
+    assert tok == int(np.argmax(got))
+    for step in range(6):
+        want = omodel.decode_with_paged_kv(tok, 1, pos)
+        got, am = mr.decode_with_paged_kv_batched([tok], [1], [pos])
+        assert_logits_close(got[0], want, "%s decode step %d" % (arch, step))
+        tok, pos = nx.argmax(want), pos + 1
+        assert tok == int(am[0])
+    mr.close()
+    # an architecture without a loader is refused by name
+    blob = _gguf_from_oracle(omodel, arch, extra).replace(arch.encode(), b"x" * len(arch))
+    with open(path, "wb") as fh:
+        fh.write(blob)
+    with pytest.raises(VexelError, match="no loader here"):
+        ModelRuntime.from_gguf(be, path, pool_blocks=16, max_seqs=4, max_batch=8)

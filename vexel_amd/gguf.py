@@ -16,7 +16,8 @@ class VhGGUFConfig(C.Structure):
     _fields_ = [("architecture", C.c_char * 64)] + \
                [(n, C.c_int) for n in ("num_layers", "hidden", "num_heads", "num_kv_heads", "ffn", "context_length",
                                         "vocab", "rope_dim_count", "head_dim")] + \
-               [("rope_theta", C.c_float), ("rms_eps", C.c_float)]
+               [("rope_theta", C.c_float), ("rms_eps", C.c_float), ("attn_softcap", C.c_float),
+                ("final_softcap", C.c_float)]
 
 
 def _bind(h):

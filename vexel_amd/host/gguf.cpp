@@ -6,6 +6,7 @@
 // blocks on the device, token_embd and the norm vectors become float32, a missing output.weight falls back to
 // the embedding. Nothing here touches the GPU except vh_model_load_gguf.
 #include <fcntl.h>
+#include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
 #include <string.h>
@@ -332,6 +333,8 @@ int vh_gguf_get_config(const vh_gguf *g, vh_gguf_config *c) {
     u32("rope.dimension_count", &c->rope_dim_count);
     if (const Meta *m = find_meta(g, prefix + "attention.layer_norm_rms_epsilon")) c->rms_eps = as_f32(*m);
     u32("attention.key_length", &c->head_dim);
+    if (const Meta *m = find_meta(g, prefix + "attn_logit_softcapping")) c->attn_softcap = as_f32(*m);
+    if (const Meta *m = find_meta(g, prefix + "final_logit_softcapping")) c->final_softcap = as_f32(*m);
     if (const Meta *m = find_meta(g, "tokenizer.ggml.tokens"))
         if (m->type == MT_ARRAY) c->vocab = (int)m->arr_len;
     return VH_OK;
@@ -464,6 +467,15 @@ struct Loader {
         w->k = k;
         return VH_OK;
     }
+    bool has(const std::string &name) {
+        vh_gguf_tensor t;
+        return vh_gguf_find_tensor(g, name.c_str(), &t) == VH_OK;
+    }
+    // as_f32 for a tensor that may be absent (*out stays NULL then)
+    int opt_f32(const std::string &name, int64_t elems, const float **out) {
+        *out = nullptr;
+        return has(name) ? as_f32(name, elems, out) : (int)VH_OK;
+    }
     // Any supported type as float32 on the device (loader.go:187-203: gguf.Dequantize at load).
     int as_f32(const std::string &name, int64_t elems, const float **out) {
         vh_gguf_tensor t;
@@ -545,9 +557,38 @@ extern "C" int vh_model_load_gguf(vx_backend *be, const char *path, const vh_loa
     c.max_blocks_per_seq = opt->max_blocks_per_seq;
     c.max_batch = opt->max_batch;
     c.kv_fp16 = opt->kv_fp16;
-    if (gc.rope_dim_count != 0 && gc.rope_dim_count != c.head_dim)
-        return done(gfail("partial rotary embedding (%d of %d dimensions) is not supported", gc.rope_dim_count, c.head_dim));
+    // ModelConfigFromGGUF (runtime/config.go:388-470): the architecture's switches
+    const std::string archname = gc.architecture;
+    vh_arch a;
+    memset(&a, 0, sizeof a);
+    bool qkv_bias = false, all_bias = false, fused_qkv = false;
+    if (archname.empty() || archname == "llama" || archname == "mistral") {
+    } else if (archname == "qwen2") {
+        qkv_bias = true;
+        a.rope_neox = 1;
+    } else if (archname == "gemma" || archname == "gemma2") {
+        a.mlp_type = VH_MLP_GEGLU;
+        a.embedding_scale = (float)sqrt((double)c.hidden);
+        if (archname == "gemma2") {
+            a.post_norms = 1;
+            a.attn_softcap = gc.attn_softcap != 0.f ? gc.attn_softcap : 50.0f;  // config.go:443-446
+            a.final_softcap = gc.final_softcap;
+        }
+    } else if (archname == "phi" || archname == "phi2") {
+        a.norm_type = VH_NORM_LAYER;
+        a.mlp_type = VH_MLP_GELU;
+        a.parallel_residual = 1;
+        a.rope_neox = 1;
+        all_bias = fused_qkv = true;
+    } else {
+        return done(gfail("%s: architecture '%s' has no loader here (llama, mistral, qwen2, gemma, gemma2, phi, phi2 do)", path,
+                          archname.c_str()));
+    }
+    if (gc.rope_dim_count < 0 || gc.rope_dim_count > c.head_dim || gc.rope_dim_count % 2 != 0)
+        return done(gfail("rope.dimension_count %d invalid for heads of %d", gc.rope_dim_count, c.head_dim));
+    a.rope_dim = gc.rope_dim_count == c.head_dim ? 0 : gc.rope_dim_count;  // config.go:487 (0 = the whole head)
     if (vh_model_create(be, &c, &L.m) != VH_OK) return done(VH_ERR);
+    if (vh_model_set_architecture(L.m, &a) != VH_OK) return done(VH_ERR);
     auto adopt_all = [&]() {
         for (void *p : L.owned) vh_model_adopt_buffer(L.m, p);
         L.owned.clear();
@@ -556,15 +597,58 @@ extern "C" int vh_model_load_gguf(vx_backend *be, const char *path, const vh_loa
     for (int l = 0; l < c.num_layers; l++) {
         const std::string b = "blk." + std::to_string(l) + ".";
         vh_layer_weights w;
+        vh_layer_extras e;
         memset(&w, 0, sizeof w);
-        int rc = L.as_f32(b + "attn_norm.weight", c.hidden, &w.attn_norm) || L.as_f32(b + "ffn_norm.weight", c.hidden, &w.ffn_norm) ||
-                 L.matrix(b + "attn_q.weight", qd, c.hidden, &w.wq) || L.matrix(b + "attn_k.weight", kvd, c.hidden, &w.wk) ||
-                 L.matrix(b + "attn_v.weight", kvd, c.hidden, &w.wv) || L.matrix(b + "attn_output.weight", c.hidden, qd, &w.wo) ||
-                 L.matrix(b + "ffn_gate.weight", c.ffn, c.hidden, &w.w1) || L.matrix(b + "ffn_up.weight", c.ffn, c.hidden, &w.w3) ||
+        memset(&e, 0, sizeof e);
+        int rc = L.as_f32(b + "attn_norm.weight", c.hidden, &w.attn_norm) || L.matrix(b + "attn_output.weight", c.hidden, qd, &w.wo) ||
                  L.matrix(b + "ffn_down.weight", c.hidden, c.ffn, &w.w2);
+        if (!rc && fused_qkv) {
+            // Phi's attn_qkv [q + 2 kv rows, hidden]: Wq, Wk, Wv are its row ranges, in place (loader.go:610-640, 1018-1060)
+            vh_qweight all;
+            memset(&all, 0, sizeof all);
+            rc = L.matrix(b + "attn_qkv.weight", qd + 2 * kvd, c.hidden, &all);
+            if (!rc) {
+                vh_gguf_tensor t;
+                L.find(b + "attn_qkv.weight", &t);
+                const size_t row_bytes = (size_t)t.n_bytes / (size_t)(qd + 2 * kvd);
+                const uint8_t *base = (const uint8_t *)all.data;
+                w.wq = vh_qweight{all.fmt, base, qd, c.hidden};
+                w.wk = vh_qweight{all.fmt, base + (size_t)qd * row_bytes, kvd, c.hidden};
+                w.wv = vh_qweight{all.fmt, base + (size_t)(qd + kvd) * row_bytes, kvd, c.hidden};
+                const float *bias = nullptr;
+                rc = L.opt_f32(b + "attn_qkv.bias", qd + 2 * kvd, &bias);
+                if (!rc && bias) e.wq_bias = bias, e.wk_bias = bias + qd, e.wv_bias = bias + qd + kvd;
+            }
+        } else if (!rc) {
+            rc = L.matrix(b + "attn_q.weight", qd, c.hidden, &w.wq) || L.matrix(b + "attn_k.weight", kvd, c.hidden, &w.wk) ||
+                 L.matrix(b + "attn_v.weight", kvd, c.hidden, &w.wv);
+            if (!rc && (qkv_bias || all_bias))
+                rc = L.opt_f32(b + "attn_q.bias", qd, &e.wq_bias) || L.opt_f32(b + "attn_k.bias", kvd, &e.wk_bias) ||
+                     L.opt_f32(b + "attn_v.bias", kvd, &e.wv_bias);
+        }
+        if (!rc && a.mlp_type == VH_MLP_GELU) {  // fc1 = ffn_up, fc2 = ffn_down (pkg/gguf/loader.go:190-198)
+            rc = L.matrix(b + "ffn_up.weight", c.ffn, c.hidden, &w.w1);
+        } else if (!rc) {
+            rc = L.matrix(b + "ffn_gate.weight", c.ffn, c.hidden, &w.w1) || L.matrix(b + "ffn_up.weight", c.ffn, c.hidden, &w.w3);
+        }
+        if (!rc && !a.parallel_residual) rc = L.as_f32(b + "ffn_norm.weight", c.hidden, &w.ffn_norm);
+        if (!rc && all_bias)
+            rc = L.opt_f32(b + "attn_norm.bias", c.hidden, &e.attn_norm_bias) || L.opt_f32(b + "attn_output.bias", c.hidden, &e.wo_bias) ||
+                 L.opt_f32(b + "ffn_up.bias", c.ffn, &e.w1_bias) || L.opt_f32(b + "ffn_down.bias", c.hidden, &e.w2_bias) ||
+                 (a.parallel_residual ? (int)VH_OK : L.opt_f32(b + "ffn_norm.bias", c.hidden, &e.ffn_norm_bias));
+        if (!rc && a.post_norms)  // loader.go:366-371
+            rc = L.as_f32(b + "post_attention_norm.weight", c.hidden, &e.post_attn_norm) ||
+                 L.as_f32(b + "post_ffw_norm.weight", c.hidden, &e.post_ffn_norm);
         adopt_all();
         if (rc) return done(VH_ERR);
-        if (vh_model_set_layer(L.m, l, &w) != VH_OK) return done(VH_ERR);
+        if (vh_model_set_layer(L.m, l, &w) != VH_OK || vh_model_set_layer_extras(L.m, l, &e) != VH_OK) return done(VH_ERR);
+    }
+    if (a.norm_type == VH_NORM_LAYER) {  // model.norm.bias (pkg/gguf/loader.go:126)
+        const float *fb = nullptr;
+        const int rc = L.opt_f32("output_norm.bias", c.hidden, &fb);
+        adopt_all();
+        if (rc) return done(VH_ERR);
+        if (fb && vh_model_set_final_norm_bias(L.m, fb) != VH_OK) return done(VH_ERR);
     }
     const float *embedding = nullptr, *final_norm = nullptr;
     if (L.as_f32("token_embd.weight", (int64_t)c.vocab * c.hidden, &embedding) || L.as_f32("output_norm.weight", c.hidden, &final_norm)) {
