@@ -223,21 +223,29 @@ def kernel_report(be):
     weight shape cycles over enough distinct copies (> 400 MB) that nothing is served from the 256 MB
     memory-side cache. Algorithmic bytes of a quantized matmul: N*K*bytes_per_element + M*K*4 + M*N*4."""
     synth = load_synth()
-    bpe = {1: 18 / 32, 2: 34 / 32, 3: 144 / 256, 4: 210 / 256}
-    names = {1: "Q4_0", 2: "Q8_0", 3: "Q4_K", 4: "Q6_K"}
+    bpe = {1: 18 / 32, 2: 34 / 32, 3: 144 / 256, 4: 210 / 256, 5: 22 / 32, 6: 176 / 256}
+    names = {1: "Q4_0", 2: "Q8_0", 3: "Q4_K", 4: "Q6_K", 5: "Q5_0", 6: "Q5_K"}
     shapes = [("Q|K|V", 12288, 4096), ("Wo", 4096, 4096), ("gate|up", 22016, 4096), ("down", 4096, 11008),
               ("lm_head", 32000, 4096)]
     a = np.random.default_rng(0).standard_normal((32, 11008)).astype(np.float32)
     da = be.upload(a, permanent=True)
     print("%-8s %-5s %3s %6s %6s %9s %9s %7s" % ("matmul", "fmt", "M", "N", "K", "us/call", "GB/s", "of 8TB"))
-    for fmt in (1, 2, 3, 4):
+    for fmt in (1, 2, 3, 4, 5, 6):
         for name, n, k in shapes:
             rb = int(k * bpe[fmt])
             copies = max(2, int(400e6 // (n * rb)) + 1)
             ws = []
             for i in range(copies):
                 p = be.alloc_permanent(n * rb)
-                if fmt <= 2:
+                if fmt >= 5:   # random codes from the host; the f16 scale fields set to small finite values
+                    blk = 22 if fmt == 5 else 176
+                    raw = np.random.default_rng(77 + i).integers(0, 256, (n * rb // blk, blk), dtype=np.uint8)
+                    raw[:, 0:2] = np.frombuffer(np.float16(0.01).tobytes(), dtype=np.uint8)
+                    if fmt == 6:
+                        raw[:, 2:4] = np.frombuffer(np.float16(0.005).tobytes(), dtype=np.uint8)
+                    be.to_device(p, raw)
+                    rc = 0
+                elif fmt <= 2:
                     rc = synth.vxs_gaussian_quant(fmt, p, n * (k // 32), 0.02, 77 + i)
                 else:   # timing does not depend on the codes
                     rc = synth.vxs_random_kquant(fmt, p, n * (k // 256), 77 + i)

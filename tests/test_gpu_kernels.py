@@ -13,6 +13,7 @@ from oracle import host_logic as hl
 pytestmark = pytest.mark.gpu
 
 FMTS = [nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q4_K, nx.FMT_Q6_K]
+FMTS_MFMA = FMTS + [nx.FMT_Q5_0, nx.FMT_Q5_K]      # the formats with matrix-vector and MFMA kernels
 
 
 @pytest.fixture(scope="module")
@@ -125,7 +126,7 @@ def test_matmul_other_formats_vs_oracle(be, fmt, m):
 
 
 # ------------------------------------------------------------------ quantized matmul
-@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("fmt", FMTS_MFMA)
 @pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 32, 40])
 def test_matmul_quant_vs_oracle(be, fmt, m):
     rng = np.random.default_rng(fmt * 100 + m)
@@ -136,7 +137,7 @@ def test_matmul_quant_vs_oracle(be, fmt, m):
     da, dw = be.upload(a), be.upload(w)
     dout = be.alloc(m * n * 4)
     name = {nx.FMT_Q4_0: be.matmul_q4_0, nx.FMT_Q8_0: be.matmul_q8_0, nx.FMT_Q4_K: be.matmul_q4_k,
-            nx.FMT_Q6_K: be.matmul_q6_k}[fmt]
+            nx.FMT_Q6_K: be.matmul_q6_k, nx.FMT_Q5_0: be.matmul_q5_0, nx.FMT_Q5_K: be.matmul_q5_k}[fmt]
     name(da, dw, dout, m, n, k)
     got = be.download(dout, (m, n), np.float32)
     # float32 summation-order level: far inside the 1e-2 abs / 1e-3 rel logits budget
@@ -145,7 +146,7 @@ def test_matmul_quant_vs_oracle(be, fmt, m):
     be.reset_pool()
 
 
-@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("fmt", FMTS_MFMA)
 def test_matmul_rows_independent_of_batch(be, fmt):
     """A row has the same bits in a batch of 2, of 32 and of 72 (the k-slices and the order their sums are added in
     depend on the matrix and the device only; up to 32 rows the slices are separate workgroups, beyond that one
@@ -179,7 +180,7 @@ def test_matmul_rows_independent_of_batch(be, fmt):
     be.reset_pool()
 
 
-@pytest.mark.parametrize("fmt", FMTS + [nx.FMT_Q5_0, nx.FMT_Q5_K])
+@pytest.mark.parametrize("fmt", FMTS_MFMA)
 @pytest.mark.parametrize("n,k", [(80, 1024), (33, 256), (7, 4096), (96, 11008), (40, 14336)])
 def test_matvec_single_row(be, fmt, n, k):
     """M = 1 (the reference's decode call): segments that start at odd 16-byte phases, rows that are not a
@@ -222,7 +223,7 @@ def test_matmul_rows_independent_at_prefill_size(be, fmt):
     be.reset_pool()
 
 
-@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("fmt", FMTS_MFMA)
 @pytest.mark.parametrize("m,n,k", [(5, 96, 11008), (32, 40, 14336), (16, 7, 4096), (33, 200, 256)])
 def test_matmul_batched_shapes(be, fmt, m, n, k):
     """M >= 2 at the 7B / 8B reduction lengths: Q6_K rows of 9030 bytes (every even 16-byte phase), row groups

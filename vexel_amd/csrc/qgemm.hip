@@ -366,6 +366,97 @@ struct PQ4_K {
     }
 };
 
+// bit i of the 4 low bits of b into bit 4 of byte i
+__device__ __forceinline__ uint32_t fifth_bits4(uint32_t b) { return ((b * 0x00204081u) & 0x01010101u) << 4; }
+
+// Q5_0 (dequant.go:100-145): 22-byte blocks [f16 d][u32 qh][16 nibble bytes]; element i = nibble | bit i of qh << 4,
+// value (q - 16) d. Eight blocks are 176 bytes, so rows and chunks start on 16-byte boundaries.
+struct PQ5_0 {
+    static constexpr int CHUNK_BYTES = 176;
+    static constexpr int ROW_PIECES = CHUNK_BYTES / 16;
+    static constexpr bool ALIGNED = true, TWO_SCALES = false;
+    static constexpr int PITCH = 176;  // 44 dwords: (PITCH/4) % 8 == 4
+    static constexpr int MIN_WAVES = 2;
+    static constexpr bool HAS_MIN = false;
+    static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 32 * 22; }
+    struct Raw { uint32_t lo, hi, sh, q0, q1, qsh, g; uint16_t d; };
+    static __device__ __forceinline__ Raw read(const uint8_t *base, int row_off, int step, int g) {
+        const int bo = row_off + step * 22, off = bo + 6 + 4 * g;  // nibble bytes 4g..4g+3; qh sits at bo + 2
+        const uint32_t *w = (const uint32_t *)base;
+        Raw r;
+        r.lo = w[off >> 2];
+        r.hi = w[(off >> 2) + 1];
+        r.sh = (uint32_t)(off & 3);
+        r.q0 = w[(bo + 2) >> 2];
+        r.q1 = w[((bo + 2) >> 2) + 1];
+        r.qsh = (uint32_t)((bo + 2) & 3);
+        r.g = (uint32_t)g;
+        r.d = *(const uint16_t *)(base + bo);
+        return r;
+    }
+    static __device__ __forceinline__ StepW unpack(const Raw &x, int) {
+        const uint32_t w = __builtin_amdgcn_alignbyte(x.hi, x.lo, x.sh);
+        const uint32_t qh = __builtin_amdgcn_alignbyte(x.q1, x.q0, x.qsh);
+        const half2v off = {(_Float16)1040.f, (_Float16)1040.f};  // 1024 + 16
+        const uint32_t lo = (w & 0x0F0F0F0Fu) | fifth_bits4((qh >> (4 * x.g)) & 15u);
+        const uint32_t hi = ((w >> 4) & 0x0F0F0F0Fu) | fifth_bits4((qh >> (16 + 4 * x.g)) & 15u);
+        const uint32_t c64 = 0x64646464u;
+        StepW r;
+        r.b = pack8(as_h2(__builtin_amdgcn_perm(lo, c64, 0x00060004u)) - off, as_h2(__builtin_amdgcn_perm(hi, c64, 0x00060004u)) - off,
+                    as_h2(__builtin_amdgcn_perm(lo, c64, 0x00070005u)) - off, as_h2(__builtin_amdgcn_perm(hi, c64, 0x00070005u)) - off);
+        r.d = h2f(x.d);
+        r.dm = 0.f;
+        return r;
+    }
+};
+
+// Q5_K (dequant.go:423-500): Q4_K's header and 6-bit scales, then qh[32] and qs[128]; bit j of qh byte l is the
+// fifth bit of element l of sub-block j.
+struct PQ5_K {
+    static constexpr int CHUNK_BYTES = 176;
+    static constexpr int ROW_PIECES = CHUNK_BYTES / 16;
+    static constexpr bool ALIGNED = true, TWO_SCALES = false;
+    static constexpr int PITCH = 176;
+    static constexpr int MIN_WAVES = 2;
+    static constexpr bool HAS_MIN = true;
+    static __host__ __device__ size_t row_bytes(int K) { return (size_t)K / 256 * 176; }
+    // what a step keeps between its LDS reads and its MFMA: the sub-block's fifth bits (bit 0 of each byte: elements
+    // 4g.., bit 1: 16+4g..) and its 6-bit scale and min are picked out at once, so that fewer registers stay live
+    struct Raw { uint32_t w0, w1, h, hd, scmn; };
+    static __device__ __forceinline__ Raw read(const uint8_t *base, int row_off, int j, int g) {
+        const uint32_t *sb = (const uint32_t *)(base + row_off);
+        const uint32_t *qp = sb + 12 + 8 * (j >> 1);
+        Raw r;
+        r.w0 = qp[g];      // elements 4g..4g+3 of both sub-blocks of the pair (low / high nibbles)
+        r.w1 = qp[4 + g];  // elements 16+4g..
+        r.h = ((sb[4 + g] >> j) & 0x01010101u) | (((sb[8 + g] >> j) & 0x01010101u) << 1);
+        r.hd = sb[0];
+        const uint8_t *q = base + row_off + 4;  // pkg/gguf/dequant.go:400-409
+        uint32_t sc, mn;
+        if (j < 4) {
+            sc = q[j] & 63;
+            mn = q[j + 4] & 63;
+        } else {
+            sc = (q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4);
+            mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+        }
+        r.scmn = sc | (mn << 8);
+        return r;
+    }
+    static __device__ __forceinline__ StepW unpack(const Raw &x, int j) {
+        const uint32_t w0 = ((x.w0 >> (4 * (j & 1))) & 0x0F0F0F0Fu) | ((x.h & 0x01010101u) << 4);
+        const uint32_t w1 = ((x.w1 >> (4 * (j & 1))) & 0x0F0F0F0Fu) | ((x.h & 0x02020202u) << 3);
+        const half2v off = {(_Float16)1024.f, (_Float16)1024.f};
+        const uint32_t c64 = 0x64646464u;
+        StepW r;
+        r.b = pack8(as_h2(__builtin_amdgcn_perm(w0, c64, 0x00060004u)) - off, as_h2(__builtin_amdgcn_perm(w1, c64, 0x00060004u)) - off,
+                    as_h2(__builtin_amdgcn_perm(w0, c64, 0x00070005u)) - off, as_h2(__builtin_amdgcn_perm(w1, c64, 0x00070005u)) - off);
+        r.d = h2f((uint16_t)(x.hd & 0xFFFF)) * (float)(x.scmn & 0xFFu);
+        r.dm = h2f((uint16_t)(x.hd >> 16)) * (float)(x.scmn >> 8);
+        return r;
+    }
+};
+
 constexpr int CH = 8;  // MFMA steps (32 elements each) per chunk
 
 // Up to three weight matrices that share K and the activation (Q/K/V, gate/up) multiplied in one
@@ -1578,6 +1669,8 @@ int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out
     case VX_Q4_0: return launch_gemm<PQ4_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
     case VX_Q8_0: return launch_gemm<PQ8_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
     case VX_Q6_K: return launch_gemm<PQ6_K>(be, segs, N, out, residual, to_partials, M, K, ks_out);
+    case VX_Q5_0: return launch_gemm<PQ5_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
+    case VX_Q5_K: return launch_gemm<PQ5_K>(be, segs, N, out, residual, to_partials, M, K, ks_out);
     default: return launch_gemm<PQ4_K>(be, segs, N, out, residual, to_partials, M, K, ks_out);
     }
 }
@@ -1586,7 +1679,7 @@ int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out
 // them from the boundary below, which needs the whole matrix to be a multiple of 16 bytes.
 bool fast_ok(int fmt, const void *b, int n, int k) {
     const size_t rb = fmt_row_bytes(fmt, k);
-    if (fmt < VX_Q4_0 || fmt > VX_Q6_K) return false;  // Q5_0, Q5_K, BF16: the row kernel
+    if (fmt < VX_Q4_0 || fmt > VX_Q5_K) return false;  // BF16: the row kernel
     if (k % 256 != 0 || ((uintptr_t)b % 16) != 0 || n < 1) return false;
     return fmt == VX_Q6_K ? ((size_t)n * rb) % 16 == 0 : rb % 16 == 0;
 }
