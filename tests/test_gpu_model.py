@@ -171,6 +171,8 @@ def test_device_driven_graph_decode_matches_host_driven(be):
     ("q4_k_m mix", nx.FMT_Q4_K, nx.FMT_Q6_K, {"wv": nx.FMT_Q6_K, "w2": nx.FMT_Q6_K}),   # config 3
     ("q8_0", nx.FMT_Q8_0, nx.FMT_Q8_0, None),                                            # config 4
     ("q6_k", nx.FMT_Q6_K, nx.FMT_Q6_K, None),                                            # config 5
+    ("q5_k_m mix", nx.FMT_Q5_K, nx.FMT_Q6_K, {"wv": nx.FMT_Q6_K, "w2": nx.FMT_Q6_K}),   # llama.cpp's Q5_K_M recipe
+    ("q5_0", nx.FMT_Q5_0, nx.FMT_Q8_0, None),
 ])
 def test_other_formats_batched_decode(be, name, fmt, head, over):
     """7B/8B head geometry (head_dim 128), one layer, 32 ragged sequences: the M=32 path."""
