@@ -17,6 +17,10 @@
  *   - none of the arithmetic kernels below is unpinned; see the test files.
  *   - vxo_matmul_q4_0 / vxo_sdpa last-ulp summation order: pinned only by
  *     restating the loop order (no reference vector fixes the last ulp).
+ *   - the operators of the other architectures (vxo_layernorm, vxo_gelu[_mul], vxo_add_bias,
+ *     vxo_scale_buffer, vxo_sdpa[_prefill]_softcap, vxo_rope_with_freqs, vxo_logit_softcap) and
+ *     vxo_medusa_forward: pinned in tests/test_oracle_arch_ops.py by the reference's own test
+ *     values and float64 closed forms; their last-ulp operation order likewise by restatement only.
  */
 #include <math.h>
 #include <stdint.h>
