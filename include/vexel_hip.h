@@ -227,6 +227,14 @@ int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight,
                        const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int rows,
                        const int32_t *positions, const int32_t *slot_mapping, void *kv_pool, int pool_is_f16,
                        int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta, float *q_out);
+/* The same for projections with biases (added before the rotation, as block.go:555-560 then :497-503 do) and with
+ * Backend.RoPE's ropeDim / ropeNeox: Qwen 2's layer (Q/K/V biases, split pairs) on the fused path. NULL biases,
+ * rope_dim 0 and rope_neox 0 are vx_decode_attn_qkv. */
+int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weight, float eps, int x_prepared,
+                          const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, const float *q_bias,
+                          const float *k_bias, const float *v_bias, int rows, const int32_t *positions,
+                          const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int num_q_heads, int num_kv_heads,
+                          int head_dim, int block_size, float theta, int rope_dim, int rope_neox, float *q_out);
 
 /* x += attn*Wo^T; h = RMSNorm(x, ffn_norm_weight); x += (SiLU(h*W1^T) * (h*W3^T)) * W2^T
  * (runtime/block.go:981-1077), x [rows,hidden] updated in place. attn may be NULL when the call follows a

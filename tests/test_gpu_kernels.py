@@ -1192,3 +1192,51 @@ def test_topk_rows_ties_and_unusable_values(be):
     with pytest.raises(RuntimeError, match="exceeds the row length"):
         be.topk_rows(dx, 3, 6, 7, dk)
     be.reset_pool()
+
+
+@pytest.mark.parametrize("rows", [1, 5, 32])
+@pytest.mark.parametrize("rope_dim,neox,bias,d", [(0, True, True, 64), (32, True, True, 128), (0, False, True, 64),
+                                                  (64, False, False, 128)])
+def test_decode_attn_qkv_with_bias_and_rope_forms(be, rows, rope_dim, neox, bias, d):
+    """vx_decode_attn_qkv_ex: RMSNorm -> Q|K|V (+ biases) -> RoPE in the ropeDim / ropeNeox forms -> paged store, in
+    its one-row (matrix-vector) and batched (MFMA) forms, against the oracle's operation sequence
+    (block.go:834-868 with matMulTransposedWithBias and applyRoPE)."""
+    rng = np.random.default_rng(80 + rows + d)
+    hq, hk, hidden, bs, nblocks = 8, 2, 1024, 16, 40
+    qd, kvd = hq * d, hk * d
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    ws = [qz.random_quant(nx.FMT_Q4_0, rng, n, hidden) for n in (qd, kvd, kvd)]
+    bs_ = [(0.1 * rng.standard_normal(n)).astype(np.float32) if bias else None for n in (qd, kvd, kvd)]
+    pos = rng.integers(0, 3000, rows).astype(np.int32)
+    slots = rng.permutation(nblocks * bs)[:rows].astype(np.int32)
+    pool = _make_pool(rng, True, nblocks, bs, hk, d)
+    norm = nx.rmsnorm(x, nw, rows, hidden, 1e-5)
+    proj = [nx.matmul_quant(nx.FMT_Q4_0, norm, w, rows, n, hidden) for w, n in zip(ws, (qd, kvd, kvd))]
+    if bias:
+        proj = [nx.add_bias(p, b, rows, n) for p, b, n in zip(proj, bs_, (qd, kvd, kvd))]
+    wq, wk = nx.rope_positions(proj[0], proj[1], d, hq, hk, pos, rope_dim, 10000.0, neox)
+    want_pool = pool.copy()
+    nx.reshape_paged_kv(wk, want_pool, slots // bs, slots % bs, hk, d, bs, False)
+    nx.reshape_paged_kv(proj[2], want_pool, slots // bs, slots % bs, hk, d, bs, True)
+    dx, dn = be.upload(x), be.upload(nw)
+    dws = [be.qweight(nx.FMT_Q4_0, be.upload(w), n, hidden) for w, n in zip(ws, (qd, kvd, kvd))]
+    dbs = [be.upload(b) if b is not None else None for b in bs_]
+    dpool, dp, ds = be.upload(pool), be.upload(pos), be.upload(slots)
+    dq = be.alloc(rows * qd * 4)
+    be.decode_attn_qkv_ex(dx, dn, 1e-5, False, dws[0], dws[1], dws[2], dbs[0], dbs[1], dbs[2], rows, dp, ds, dpool, True,
+                          hq, hk, d, bs, 10000.0, rope_dim, neox, dq)
+    got_q = be.download(dq, (rows, qd), np.float32)
+    scale = np.abs(wq).max()
+    _close(got_q, wq.reshape(rows, qd), 2e-5, 3e-6 * scale + 1e-7, "fused q")
+    got = nx.f16_to_f32_array(be.download(dpool, pool.shape, pool.dtype))
+    ref = nx.f16_to_f32_array(want_pool)
+    assert np.all(np.abs(got - ref) <= np.abs(ref) * 2.0 ** -9 + 1e-5)        # f16 neighbours where f32 differs in its last bits
+    untouched = np.ones(pool.shape, dtype=bool)
+    per_blk = 2 * bs * hk * d
+    for sl in slots:
+        b, o = sl // bs, sl % bs
+        untouched[b * per_blk + o * hk * d: b * per_blk + (o + 1) * hk * d] = False
+        untouched[b * per_blk + bs * hk * d + o * hk * d: b * per_blk + bs * hk * d + (o + 1) * hk * d] = False
+    assert np.array_equal(be.download(dpool, pool.shape, pool.dtype)[untouched], pool[untouched])
+    be.reset_pool()

@@ -1464,6 +1464,78 @@ __global__ void __launch_bounds__(256) add_partials_kernel(float *__restrict__ x
 // RoPE (backend/cpu/cpu.go:226-303, interleaved pairs, one position per row) + paged K/V scatter
 // (metal_bridge_darwin.m:8607-8642) reading the fused Q|K|V projection from its split-K partials.
 // grid = (rows, head groups); thread = (pair j, head lane).
+// GEN: the general form (biases added to the projections before the rotation as matMulTransposedWithBias +
+// applyRoPE do, block.go:497-503,555-560; rope_dim of the head's dimensions rotated, in split pairs when neox).
+struct QkvExtra {
+    const float *q_bias, *k_bias, *v_bias;  // [qd], [kvd], [kvd] or nullptr
+    int eff_dim, neox;
+};
+
+template <bool F16, bool GEN>
+__global__ void rope_store_general_kernel(const float *__restrict__ P, int KS, int M, const float *__restrict__ inv_scale, RowNorm rn,
+                                          float *__restrict__ q_out, const int32_t *__restrict__ positions,
+                                          const int32_t *__restrict__ slot_mapping, void *__restrict__ pool,
+                                          int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta,
+                                          QkvExtra ex) {
+    static_assert(GEN, "the interleaved whole-head form is rope_store_partials_kernel");
+    const int row = blockIdx.x, half = head_dim / 2, he = ex.eff_dim / 2;
+    const int qd = num_q_heads * head_dim, kvd = num_kv_heads * head_dim, ncols = qd + 2 * kvd;
+    const size_t slice_elems = (size_t)M * ncols;
+    const float inv = row_factor(inv_scale, rn, row);  // every wave of the block, before any lane leaves
+    const int pos = positions[row], slot = slot_mapping[row];
+    const int blk = slot / block_size, off = slot % block_size;
+    const size_t part = (size_t)block_size * kvd;
+    const size_t kbase = (size_t)blk * 2 * part + (size_t)off * kvd, vbase = kbase + part;
+    const int lanes = blockDim.x / half, hl = threadIdx.x / half, j = threadIdx.x % half;
+    if (hl >= lanes) return;
+    const int hstride = lanes * gridDim.y, h0 = blockIdx.y * lanes + hl;
+    // thread j: rotation pair j, or past the rotated part two neighbouring dimensions that are only carried over
+    const bool turn = j < he;
+    const int i0 = turn ? (ex.neox ? j : 2 * j) : ex.eff_dim + 2 * (j - he);
+    const int i1 = turn ? (ex.neox ? j + he : 2 * j + 1) : i0 + 1;
+    float c = 1.f, sn = 0.f;
+    if (turn) {
+        const double e = (double)(2 * j) / (double)ex.eff_dim;
+        const float freq = (float)(1.0 / pow((double)theta, e));
+        const float angle = __fmul_rn((float)pos, freq);
+        c = (float)cos((double)angle);
+        sn = (float)sin((double)angle);
+    }
+    auto elem = [&](int col, const float *bias, int bcol) {
+        const float *p0 = P + (size_t)row * ncols + col;
+        float v = *p0;
+        for (int s = 1; s < KS; s++) v += p0[(size_t)s * slice_elems];
+        v = __fmul_rn(v, inv);
+        return bias ? __fadd_rn(v, bias[bcol]) : v;
+    };
+    for (int h = h0; h < num_q_heads; h += hstride) {
+        const int b0 = h * head_dim + i0, b1 = h * head_dim + i1;
+        const float a = elem(b0, ex.q_bias, b0), b = elem(b1, ex.q_bias, b1);
+        q_out[(size_t)row * qd + b0] = turn ? __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, sn)) : a;
+        q_out[(size_t)row * qd + b1] = turn ? __fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, c)) : b;
+    }
+    for (int h = h0; h < num_kv_heads; h += hstride) {
+        const int b0 = h * head_dim + i0, b1 = h * head_dim + i1;
+        const float a = elem(qd + b0, ex.k_bias, b0), b = elem(qd + b1, ex.k_bias, b1);
+        const float va = elem(qd + kvd + b0, ex.v_bias, b0), vb = elem(qd + kvd + b1, ex.v_bias, b1);
+        const float ka = turn ? __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, sn)) : a;
+        const float kb = turn ? __fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, c)) : b;
+        if (F16) {
+            _Float16 *pp = (_Float16 *)pool;
+            pp[kbase + b0] = (_Float16)ka;
+            pp[kbase + b1] = (_Float16)kb;
+            pp[vbase + b0] = (_Float16)va;
+            pp[vbase + b1] = (_Float16)vb;
+        } else {
+            float *pp = (float *)pool;
+            pp[kbase + b0] = ka;
+            pp[kbase + b1] = kb;
+            pp[vbase + b0] = va;
+            pp[vbase + b1] = vb;
+        }
+    }
+}
+
 template <bool F16>
 __global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, int M, const float *__restrict__ inv_scale, RowNorm rn,
                                            float *__restrict__ q_out, const int32_t *__restrict__ positions,
@@ -1858,8 +1930,24 @@ int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight,
                        const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int rows,
                        const int32_t *positions, const int32_t *slot_mapping, void *kv_pool, int pool_is_f16,
                        int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta, float *q_out) {
+    return vx_decode_attn_qkv_ex(be, x, norm_weight, eps, x_prepared, wq, wk, wv, nullptr, nullptr, nullptr, rows, positions,
+                                 slot_mapping, kv_pool, pool_is_f16, num_q_heads, num_kv_heads, head_dim, block_size, theta, 0, 0,
+                                 q_out);
+}
+
+int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weight, float eps, int x_prepared,
+                          const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, const float *q_bias,
+                          const float *k_bias, const float *v_bias, int rows, const int32_t *positions,
+                          const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int num_q_heads, int num_kv_heads,
+                          int head_dim, int block_size, float theta, int rope_dim, int rope_neox, float *q_out) {
     int rc = enter(be);
     if (rc) return rc;
+    const int eff_dim = rope_dim == 0 ? head_dim : rope_dim;
+    VX_REQUIRE(eff_dim > 0 && eff_dim <= head_dim && eff_dim % 2 == 0, "vx_decode_attn_qkv: rope_dim %d invalid for head_dim %d",
+               rope_dim, head_dim);
+    // the interleaved whole-head form without biases keeps its own kernel
+    const bool gen = q_bias || k_bias || v_bias || rope_neox || eff_dim != head_dim;
+    const QkvExtra ex = {q_bias, k_bias, v_bias, eff_dim, rope_neox};
     if (!vx_decode_attn_qkv_supported(wq, wk, wv, head_dim)) {
         set_error("vx_decode_attn_qkv: weights have no fused MFMA path");
         return VX_ERR_UNSUPPORTED;
@@ -1888,9 +1976,14 @@ int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight,
             const int lanes1 = 256 / half1 > 0 ? 256 / half1 : 1;
             const int max_heads1 = num_q_heads > num_kv_heads ? num_q_heads : num_kv_heads;
             const RowNorm none = {nullptr, 0, 0.f, 0.f};
-            rope_store_partials_kernel<true><<<dim3(1, ceil_div(max_heads1, lanes1)), lanes1 * half1, 0, be->stream>>>(
-                (const float *)be->part_ws, 1, 1, be->ones, none, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-                num_kv_heads, head_dim, block_size, theta);
+            if (gen)
+                rope_store_general_kernel<true, true><<<dim3(1, ceil_div(max_heads1, lanes1)), lanes1 * half1, 0, be->stream>>>(
+                    (const float *)be->part_ws, 1, 1, be->ones, none, q_out, positions, slot_mapping, kv_pool, num_q_heads,
+                    num_kv_heads, head_dim, block_size, theta, ex);
+            else
+                rope_store_partials_kernel<true><<<dim3(1, ceil_div(max_heads1, lanes1)), lanes1 * half1, 0, be->stream>>>(
+                    (const float *)be->part_ws, 1, 1, be->ones, none, q_out, positions, slot_mapping, kv_pool, num_q_heads,
+                    num_kv_heads, head_dim, block_size, theta);
             VX_CHECK_LAUNCH();
             return VX_OK;
         }
@@ -1917,7 +2010,15 @@ int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight,
     const RowNorm rn = cur_row_norm(be);
     const int max_heads = num_q_heads > num_kv_heads ? num_q_heads : num_kv_heads;
     dim3 grid(rows, ceil_div(max_heads, lanes));
-    if (pool_is_f16)
+    if (gen && pool_is_f16)
+        rope_store_general_kernel<true, true><<<grid, lanes * half, 0, be->stream>>>(
+            (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
+            num_kv_heads, head_dim, block_size, theta, ex);
+    else if (gen)
+        rope_store_general_kernel<false, true><<<grid, lanes * half, 0, be->stream>>>(
+            (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
+            num_kv_heads, head_dim, block_size, theta, ex);
+    else if (pool_is_f16)
         rope_store_partials_kernel<true><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
             num_kv_heads, head_dim, block_size, theta);

@@ -129,6 +129,8 @@ struct vh_model {
     const float *final_norm_bias = nullptr;
     float *zeros = nullptr;               // [hidden] zeros: the bias of a LayerNorm whose bias tensor is absent
     bool general = false;                 // some switch or extra tensor is set: the one-call-per-operation sequence
+    bool fused_ok = true;                 // the layer differs from LLaMA's at most by Q/K/V biases and the RoPE form
+                                          // (Qwen 2): decode may still take the fused entry points
 
     vx_graph *graph = nullptr;
     int graph_batch = 0;
@@ -315,7 +317,7 @@ int g_scale_embedding(vh_model *m, float *x, int rows) {
 }
 
 bool attn_fusable(const vh_model *m, int layer) {
-    if (!m->fused || m->general || layer >= m->cfg.num_layers) return false;
+    if (!m->fused || (m->general && !m->fused_ok) || layer >= m->cfg.num_layers) return false;
     const vh_layer_weights &w = m->layers[layer];
     return w.wq.data && w.wk.data && w.wv.data && vx_decode_attn_qkv_supported(&w.wq, &w.wk, &w.wv, m->cfg.head_dim) != 0;
 }
@@ -327,7 +329,7 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
     const vh_config &c = m->cfg;
     const vh_layer_weights &w = m->layers[layer];
     const float scale = (float)(1.0 / sqrt((double)c.head_dim));                          // block.go:862
-    if (m->general) {
+    if (m->general && !attn_fusable(m, layer)) {
         if (*chained) return fail("internal: prepared activation handed to a general layer");
         VHC(g_qkv(m, layer, m->x, m->norm, m->q, m->k, m->v, rows));
         VXC(vx_rope_store_paged_ex(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
@@ -339,9 +341,11 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
         return g_tail(m, layer, m->x, m->norm, m->attn, m->gate, m->up, rows);
     }
     if (attn_fusable(m, layer)) {   // block.go:834-868; one row: matrix-vector launches inside the same entry points
-        VXC(vx_decode_attn_qkv(m->be, m->x, w.attn_norm, c.eps, *chained ? 1 : 0, &w.wq, &w.wk, &w.wv, rows,
-                               m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, c.num_heads, c.num_kv_heads,
-                               c.head_dim, c.block_size, c.rope_theta, m->q));
+        const vh_layer_extras &e = m->extras[layer];
+        VXC(vx_decode_attn_qkv_ex(m->be, m->x, w.attn_norm, c.eps, *chained ? 1 : 0, &w.wq, &w.wk, &w.wv, e.wq_bias, e.wk_bias,
+                                  e.wv_bias, rows, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, c.num_heads,
+                                  c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta, m->arch.rope_dim, m->arch.rope_neox,
+                                  m->q));
     } else {
         if (*chained) return fail("internal: prepared activation handed to an unfused layer");
         bool prep;
@@ -376,7 +380,7 @@ int forward_decode(vh_model *m, int rows, int max_kv_len) {
     const vh_config &c = m->cfg;
     VXC(vx_embedding(m->be, m->d_tokens, rows, m->embedding, m->x, c.vocab, c.hidden));
     VHC(g_scale_embedding(m, m->x, rows));
-    const bool head_prepared = rows > 1 && m->fused && !m->general && fast(m->lm_head) && c.hidden % 256 == 0;
+    const bool head_prepared = rows > 1 && m->fused && (!m->general || m->fused_ok) && fast(m->lm_head) && c.hidden % 256 == 0;
     bool chained = false;
     for (int l = 0; l < c.num_layers; l++) {
         const float *next_norm = l + 1 < c.num_layers ? (rows > 1 && attn_fusable(m, l + 1) ? m->layers[l + 1].attn_norm : nullptr)
@@ -385,7 +389,7 @@ int forward_decode(vh_model *m, int rows, int max_kv_len) {
     }
     if (chained) {                                                                        // model.go:207-226, 352-422
         VHC(mm(m, true, nullptr, m->lm_head, m->logits, nullptr, rows));
-    } else if (m->general) {
+    } else if (m->general && !m->fused_ok) {
         VHC(g_norm(m, m->x, m->final_norm, m->final_norm_bias, m->norm, rows));
         VHC(mm(m, false, m->norm, m->lm_head, m->logits, nullptr, rows));
     } else {
@@ -539,8 +543,13 @@ static void refresh_general(vh_model *m) {
     for (const vh_layer_extras &e : m->extras)
         g = g || e.attn_norm_bias || e.ffn_norm_bias || e.wq_bias || e.wk_bias || e.wv_bias || e.wo_bias || e.w1_bias ||
             e.w2_bias || e.post_attn_norm || e.post_ffn_norm;
-    if (g != m->general) drop_graph(m);
+    bool f = !a.norm_type && !a.mlp_type && !a.parallel_residual && !a.post_norms && !m->final_norm_bias;
+    for (const vh_layer_extras &e : m->extras)
+        f = f && !e.attn_norm_bias && !e.ffn_norm_bias && !e.wo_bias && !e.w1_bias && !e.w2_bias && !e.post_attn_norm &&
+            !e.post_ffn_norm;
+    if (g != m->general || f != m->fused_ok) drop_graph(m);
     m->general = g;
+    m->fused_ok = f;
 }
 
 int vh_model_set_architecture(vh_model *m, const vh_arch *arch) {

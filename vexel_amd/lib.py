@@ -74,6 +74,8 @@ SIGNATURES = {
     "vx_matmul_quant_prepared": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i]),
     "vx_matmul_quant_has_fast_path": (_i, [_i, _vp, _i, _i]),
     "vx_decode_attn_qkv_supported": (_i, [_vp, _vp, _vp, _i]),
+    "vx_decode_attn_qkv_ex": (_i, [_vp, _vp, _vp, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i,
+                                   _f, _i, _i, _vp]),
     "vx_decode_attn_qkv": (_i, [_vp, _vp, _vp, _f, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
     "vx_decode_ffn_supported": (_i, [_vp, _vp, _vp, _vp]),
     "vx_decode_ffn": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _vp]),
