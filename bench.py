@@ -56,9 +56,10 @@ def load_synth():
     return s
 
 
-def build_model(be, ctx, extra_tokens, layers, cfg=None, fmts=None, max_batch=None):
+def build_model(be, ctx, extra_tokens, layers, cfg=None, fmts=None, max_batch=None, arch=None):
     """Synthetic model (7B-shaped Q4_0 unless cfg / fmts say otherwise) + pre-filled contexts, generated on the
     device. fmts: weight name (wq, wk, wv, wo, w1, w3, w2, head) -> VX_* format, "*" the default.
+    arch: the switches of ModelRuntime.set_architecture plus "bias": "qkv" | "all" (small random bias vectors).
     -> (ModelRuntime, ids)"""
     from vexel_amd import lib
     from vexel_amd.runtime import ModelRuntime
@@ -72,6 +73,15 @@ def build_model(be, ctx, extra_tokens, layers, cfg=None, fmts=None, max_batch=No
     mr = ModelRuntime(be, **c, pool_blocks=need_blocks, max_seqs=len(ctx), max_blocks_per_seq=max_bps,
                       max_batch=max_batch or len(ctx), kv_fp16=True)
     seed = [0]
+    arch = dict(arch or {})
+    bias_kind = arch.pop("bias", None)
+    if arch:
+        mr.set_architecture(**arch)
+    gelu_mlp = arch.get("mlp_type") == "gelu"
+
+    def vec(n, mean):
+        seed[0] += 1
+        return (mean + 0.02 * np.random.default_rng(seed[0]).standard_normal(n)).astype(np.float32)
 
     def qw(n, k, fmt=lib.VX_Q4_0):
         seed[0] += 1
@@ -95,8 +105,17 @@ def build_model(be, ctx, extra_tokens, layers, cfg=None, fmts=None, max_batch=No
     mr.adopt_device_buffer(ones)
     for l in range(layers):
         mr.set_layer(l, ones, ones, dict(wq=qw(qd, h, fm("wq")), wk=qw(kvd, h, fm("wk")), wv=qw(kvd, h, fm("wv")),
-                                         wo=qw(h, qd, fm("wo")), w1=qw(f, h, fm("w1")), w3=qw(f, h, fm("w3")),
-                                         w2=qw(h, f, fm("w2"))))
+                                         wo=qw(h, qd, fm("wo")), w1=qw(f, h, fm("w1")),
+                                         w3=None if gelu_mlp else qw(f, h, fm("w3")), w2=qw(h, f, fm("w2"))))
+        extras = {}
+        if bias_kind in ("qkv", "all"):
+            extras.update(wq_bias=vec(qd, 0.0), wk_bias=vec(kvd, 0.0), wv_bias=vec(kvd, 0.0))
+        if bias_kind == "all":
+            extras.update(wo_bias=vec(h, 0.0), w1_bias=vec(f, 0.0), w2_bias=vec(h, 0.0), attn_norm_bias=vec(h, 0.0))
+        if arch.get("post_norms"):
+            extras.update(post_attn_norm=vec(h, 1.0), post_ffn_norm=vec(h, 1.0))
+        if extras:
+            mr.set_layer_extras(l, **extras)
     emb_q = qw(v, h, lib.VX_Q8_0)
     emb = be.alloc_permanent(v * h * 4)
     mr.adopt_device_buffer(emb)
@@ -469,6 +488,36 @@ def medusa_report(be):
             be.free(ptr)
 
 
+def arch_report(be):
+    """Batched greedy decode (32 ragged sequences, device-driven hipGraph loop) for the layer graphs beside LLaMA at
+    the shapes of published models, Q4_0 weights: Qwen 2 7B (fused decode blocks with the bias / split-pair epilogue),
+    Phi-2 and Gemma 2 2B (one call per operation)."""
+    from vexel_amd import lib
+    models = [
+        ("LLaMA-2 7B", dict(hidden=4096, num_heads=32, num_kv_heads=32, head_dim=128, ffn=11008, vocab=32000, eps=1e-5,
+                            rope_theta=10000.0), 32, None),
+        ("Qwen 2 7B", dict(hidden=3584, num_heads=28, num_kv_heads=4, head_dim=128, ffn=18944, vocab=152064, eps=1e-6,
+                           rope_theta=1000000.0), 28, dict(rope_neox=True, bias="qkv")),
+        ("Phi-2 2.7B", dict(hidden=2560, num_heads=32, num_kv_heads=32, head_dim=80, ffn=10240, vocab=51200, eps=1e-5,
+                            rope_theta=10000.0), 32,
+         dict(norm_type="layer", mlp_type="gelu", parallel_residual=True, rope_dim=32, rope_neox=True, bias="all")),
+        ("Gemma 2 2B", dict(hidden=2304, num_heads=8, num_kv_heads=4, head_dim=256, ffn=9216, vocab=256000, eps=1e-6,
+                            rope_theta=10000.0), 26,
+         dict(mlp_type="geglu", post_norms=True, attn_softcap=50.0, final_softcap=30.0, embedding_scale=48.0)),
+    ]
+    ctx = ragged_contexts()
+    print("%-12s %6s %7s %10s %9s" % ("model", "layers", "batch", "ms/step", "tok/s"))
+    for name, cfg, layers, arch in models:
+        c = dict(CFG)
+        c.update(cfg)
+        mr, ids = build_model(be, ctx, 48, layers, cfg=c, arch=arch)
+        first = np.random.default_rng(3).integers(0, c["vocab"], len(ctx)).astype(np.int32)
+        mr.decode_graph(first, ids, list(ctx), 4)
+        _, ms = mr.decode_graph(None, None, None, 24, batch=len(ctx))
+        print("%-12s %6d %7d %10.3f %9.0f" % (name, layers, len(ctx), ms, len(ctx) / ms * 1e3), flush=True)
+        mr.close()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -489,6 +538,8 @@ def main():
     ap.add_argument("--prefill-probe", action="store_true",
                     help="for rocprofv3 --pmc runs of the MFMA kernels: 512-row GEMMs of the 7B shapes and one "
                          "512-token prefill attention, then exit")
+    ap.add_argument("--arch-report", action="store_true",
+                    help="batched decode rates of the Qwen 2 / Phi-2 / Gemma 2 layer graphs at published shapes, then exit")
     ap.add_argument("--medusa-report", action="store_true",
                     help="time the Medusa heads' forward pass and top-k at the 7B shape, then exit")
     args = ap.parse_args()
@@ -508,6 +559,9 @@ def main():
         return
     if args.medusa_report:
         medusa_report(be)
+        return
+    if args.arch_report:
+        arch_report(be)
         return
     ctx = ragged_contexts(n=args.seqs) if args.seqs != BATCH else ragged_contexts()
     nseq = len(ctx)

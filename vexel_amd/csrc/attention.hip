@@ -182,15 +182,17 @@ __global__ void __launch_bounds__(GEN_THREADS) attn_generic_kernel(AttnParams p)
 constexpr int TPW = ATTN_TPW;  // tokens per workgroup
 constexpr int HOT_BS = 16;
 
-// Sum over the N adjacent lanes (N = 8 or 16, aligned) that hold one token's head vector, by DPP inside a
-// 16-lane row (no LDS traffic): quads, then the mirrored quad of the half, then the mirrored half.
+// Sum over the N adjacent lanes (N = 8, 16 or 32, aligned) that hold one token's head vector, by DPP inside a
+// 16-lane row (no LDS traffic): quads, then the mirrored quad of the half, then the mirrored half; heads of 256
+// span two rows, joined by one cross-row exchange.
 template <int N>
 __device__ __forceinline__ float token_sum(float t) {
-    static_assert(N == 8 || N == 16, "a head vector spans 8 or 16 lanes");
+    static_assert(N == 8 || N == 16 || N == 32, "a head vector spans 8, 16 or 32 lanes");
     t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0xb1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
     t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x4e, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
     t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x141, 0xf, 0xf, false));  // row_half_mirror
-    if (N == 16) t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x140, 0xf, 0xf, false));  // row_mirror
+    if (N >= 16) t += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, t), 0x140, 0xf, 0xf, false));  // row_mirror
+    if (N == 32) t += __shfl_xor(t, 16, 64);
     return t;
 }
 
@@ -203,7 +205,11 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     float *__restrict__ partial, int num_q_heads, int num_kv_heads, float scale, int max_splits,
     const int32_t *__restrict__ items) {
     constexpr int GG = G * RG;       // queries per K/V row
-    constexpr int LPT = D / 8;       // lanes per token
+    constexpr int DL = D / 8;        // 8-element slices of a head vector
+    // lanes per token: the next power of two; the lanes past DL (heads of 80 or 96) repeat the last slice's loads
+    // with a zero query, so they add nothing and write nothing
+    constexpr int LPT = DL <= 8 ? 8 : (DL <= 16 ? 16 : 32);
+    static_assert(D % 8 == 0 && DL <= 32, "head vectors are whole 16-byte slices on at most 32 lanes");
     constexpr int TPI = 64 / LPT;    // tokens per load instruction
     constexpr int NL = HOT_BS / TPI; // load instructions per block and per K or V
     typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -228,7 +234,8 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int tl = lane / LPT;  // token slot within a load
-    const int dl = lane % LPT;  // 8-element slice of the head vector
+    const int dl = DL == LPT ? lane % LPT : min(lane % LPT, DL - 1);  // 8-element slice of the head vector
+    const bool live = DL == LPT ? true : lane % LPT < DL;
     const size_t hs = (size_t)num_kv_heads * D;
     const size_t part = (size_t)HOT_BS * hs;
     const size_t lane_off = (size_t)tl * hs + (size_t)kvh * D + dl * 8;
@@ -240,7 +247,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     for (int g = 0; g < GG; g++) {
         const float *qp = q + (((size_t)seq * RG + g / G) * num_q_heads + (size_t)kvh * G + g % G) * D + dl * 8;
 #pragma unroll
-        for (int e = 0; e < 8; e++) qf[g][e] = qp[e] * qs;
+        for (int e = 0; e < 8; e++) qf[g][e] = live ? qp[e] * qs : 0.f;
     }
     float acc[GG][8], m_run[GG], l_run[GG];
 #pragma unroll
@@ -323,7 +330,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     // combine the 4 waves through LDS
     __shared__ float s_m[4][GG], s_l[4][GG];
     __shared__ float s_acc[4][GG][D];
-    if (tl == 0) {
+    if (tl == 0 && live) {
 #pragma unroll
         for (int g = 0; g < GG; g++) {
 #pragma unroll
@@ -659,6 +666,13 @@ int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16
                                   num_kv_heads, scale, max_kv_len);
     VX_HOT(128, 1) VX_HOT(128, 2) VX_HOT(128, 4) VX_HOT(128, 8)
     VX_HOT(64, 1) VX_HOT(64, 2) VX_HOT(64, 4) VX_HOT(64, 8)
+    // group sizes that are no power of two (Qwen 2 7B: 28 / 4 heads, LLaMA 3.2 3B: 24 / 8, Qwen 2 1.5B: 12 / 2)
+    VX_HOT(128, 3) VX_HOT(128, 5) VX_HOT(128, 6) VX_HOT(128, 7)
+    VX_HOT(64, 3) VX_HOT(64, 5) VX_HOT(64, 6) VX_HOT(64, 7)
+    // heads of 256 (Gemma): 32 lanes per token; the K/V registers of a 16-token block leave room for 1 or 2 query heads
+    VX_HOT(256, 1) VX_HOT(256, 2)
+    // heads of 80 (Phi-2) and 96 (Phi-3 mini) on 16 lanes per token, 10 or 12 of them live
+    VX_HOT(80, 1) VX_HOT(96, 1)
 #undef VX_HOT
     if (!out) {
         set_error("vx_sdpa_paged_decode_ragged: out = NULL (split form) needs an F16 pool with 16-token blocks and a "
@@ -858,7 +872,8 @@ int vx_sdpa_paged_decode_split_supported(int pool_is_f16, int block_size, int nu
                                          int head_dim) {
     if (!pool_is_f16 || block_size != HOT_BS || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0) return 0;
     const int G = num_q_heads / num_kv_heads;
-    return (head_dim == 128 || head_dim == 64) && (G == 1 || G == 2 || G == 4 || G == 8);
+    return ((head_dim == 128 || head_dim == 64) && G >= 1 && G <= 8) || (head_dim == 256 && G <= 2) ||
+           ((head_dim == 80 || head_dim == 96) && G == 1);
 }
 
 int vx_sdpa_paged_decode_multiquery(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
