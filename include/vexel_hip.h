@@ -264,7 +264,10 @@ int vx_rope_store_paged_ex(vx_backend *be, float *q, const float *k, const float
  * table_rows is NULL); kv_lens int32[batch]. One query per sequence. max_kv_len bounds
  * the launch (>= every kv_lens[i]). With out = NULL the result stays in the backend as per-split partial
  * sums for the next vx_decode_ffn(attn = NULL) to merge (one launch less); that form exists only where
- * vx_sdpa_paged_decode_split_supported() is 1, otherwise the call returns VX_ERR_UNSUPPORTED. */
+ * vx_sdpa_paged_decode_split_supported() is 1, otherwise the call returns VX_ERR_UNSUPPORTED.
+ * That is also where the streaming split-KV kernel runs (F16 pool, 16-token blocks): heads of 64 or 128 with 1 to 8
+ * query heads per KV head, heads of 256 with 1 or 2, heads of 80 or 96 with 1; other geometries take the generic
+ * kernel (any head_dim <= 256), same results, far slower. */
 int vx_sdpa_paged_decode_split_supported(int pool_is_f16, int block_size, int num_q_heads, int num_kv_heads,
                                          int head_dim);
 int vx_sdpa_paged_decode_ragged(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
