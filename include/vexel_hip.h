@@ -129,7 +129,7 @@ int vx_rope_with_freqs(vx_backend *be, float *q, float *k, const float *freqs, i
 int vx_medusa_forward(vx_backend *be, const float *hidden, const float *fc1, const float *fc2, float *intermediate,
                       float *logits, int rows, int num_heads, int hidden_size, int vocab_size);
 /* topK (heads.go:146-171) per row of x [rows][n]: the indices of the k largest values, largest first, a tie to the
- * lower index; out_idx [rows][k] int32, out_val [rows][k] (may be NULL) on the device. Values not above -MaxFloat32
+ * lower index; out_idx [rows][k] int32, out_val [rows][k] (may be NULL) on the device; k <= min(n, 256). Values not above -MaxFloat32
  * and NaN are never taken: the index is then -1. */
 int vx_topk_rows(vx_backend *be, const float *x, int rows, int n, int k, int32_t *out_idx, float *out_val);
 

@@ -1192,6 +1192,8 @@ def test_topk_rows_ties_and_unusable_values(be):
         assert idx[r].tolist() == np.argsort(-big[r].astype(np.float64), kind="stable")[:10].tolist()
     with pytest.raises(RuntimeError, match="exceeds the row length"):
         be.topk_rows(dx, 3, 6, 7, dk)
+    with pytest.raises(RuntimeError, match="above 256"):
+        be.topk_rows(db, 2, 128256, 257, dk)
     be.reset_pool()
 
 

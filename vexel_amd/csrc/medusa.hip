@@ -209,6 +209,7 @@ int vx_topk_rows(vx_backend *be, const float *x, int rows, int n, int k, int32_t
     if (rc) return rc;
     VX_REQUIRE(x && out_idx && rows >= 0 && n >= 1 && k >= 0, "vx_topk_rows: bad arguments");
     VX_REQUIRE(k <= n, "vx_topk_rows: k %d exceeds the row length %d", k, n);
+    VX_REQUIRE(k <= 256, "vx_topk_rows: k %d above 256 (the selection makes one pass over the row per pick)", k);
     if (rows == 0 || k == 0) return VX_OK;
     topk_rows_kernel<<<rows, 1024, 0, be->stream>>>(x, n, k, out_idx, out_val);
     VX_CHECK_LAUNCH();
