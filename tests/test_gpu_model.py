@@ -482,22 +482,26 @@ def _arch_config(name):
         return om.ModelConfig(num_layers=2, hidden=512, num_heads=4, num_kv_heads=2, head_dim=256, ffn=1024, vocab=1000,
                               eps=1e-6, mlp_type="geglu", post_norms=True, attn_softcap=50.0, rope_neox=True,
                               embedding_scale=float(np.float32(math.sqrt(512.0))))
+    if name == "qwen_g7":   # 7 query heads per KV head (Qwen 2 7B's 28 / 4) at heads of 128: the fused blocks and the
+        return om.ModelConfig(num_layers=2, hidden=1024, num_heads=14, num_kv_heads=2, head_dim=128, ffn=1536,  # split merge
+                              vocab=1000, eps=1e-6, rope_neox=True, rope_theta=1000000.0)
     return om.ModelConfig(num_layers=2, hidden=512, num_heads=8, num_kv_heads=2, head_dim=64, ffn=1536, vocab=1000,
                           eps=1e-6, rope_neox=True, rope_theta=1000000.0)
 
 
-@pytest.mark.parametrize("name", ["phi", "gemma", "qwen"])
+@pytest.mark.parametrize("name", ["phi", "gemma", "qwen", "qwen_g7"])
 def test_other_architectures_prefill_decode_graph(be, name):
     """ExecuteWithPagedKV's general sequence (block.go:834-1077) through vh_prefill (first chunk and a later one),
     vh_decode_batched and the device-driven vh_decode_graph, against the oracle's layer for the same switches."""
     cfg = _arch_config(name)
     omodel = om.random_model(cfg, 21, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=24)
-    if name == "qwen":
+    if name.startswith("qwen"):
         rng = np.random.default_rng(22)
+        qd, kvd = cfg.num_heads * cfg.head_dim, cfg.num_kv_heads * cfg.head_dim
         for lw in omodel.layers:
-            lw.wq_bias = (0.05 * rng.standard_normal(512)).astype(np.float32)
-            lw.wk_bias = (0.05 * rng.standard_normal(128)).astype(np.float32)
-            lw.wv_bias = (0.05 * rng.standard_normal(128)).astype(np.float32)
+            lw.wq_bias = (0.05 * rng.standard_normal(qd)).astype(np.float32)
+            lw.wk_bias = (0.05 * rng.standard_normal(kvd)).astype(np.float32)
+            lw.wv_bias = (0.05 * rng.standard_normal(kvd)).astype(np.float32)
     mr = gpu_model_from_oracle(be, omodel, pool_blocks=24, max_seqs=4, max_batch=8)
     rng = np.random.default_rng(23)
     prompts = {1: rng.integers(0, cfg.vocab, 21).tolist(), 2: rng.integers(0, cfg.vocab, 35).tolist()}
