@@ -20,6 +20,9 @@
 //     format's integers. With KS > 1 slices the partial sums go to scratch and
 //     qgemm_reduce_kernel adds them in slice order (deterministic), applies the row scale and
 //     the optional residual.
+//     Decode batches (at most two activation tiles per workgroup) whose weight rows fit one round of
+//     workgroups take qgemm_wave_kernel (qgemm_wave.h) instead: one workgroup per compute unit, its
+//     waves split K, activation tiles go from L2 straight to registers.
 //  Each output element depends only on its own activation row and weight row and the launch
 //  shape depends on (N, K) only, so a row gives the same bits alone or inside a batch (the
 //  property the reference keeps by looping M=1 kernels, backend/metal/backend.go:777-779).
@@ -883,6 +886,8 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
     }
 }
 
+#include "qgemm_wave.h"
+
 // out[m][n] = residual + inv_scale[m] * (P[0] + P[1] + ... + P[KS-1]) in that order.
 __global__ void __launch_bounds__(256) qgemm_reduce_kernel(const float *__restrict__ partial,
                                                            const float *__restrict__ inv_scale,
@@ -1735,8 +1740,118 @@ int launch_gemm(vx_backend *be, const Segs &segs, int N, float *out, const float
     return VX_OK;
 }
 
+// ---- the wave-private kernel (qgemm_wave.h): which shapes take it, and how the matrix is cut
+struct WavePlan {
+    int r;   // weight tiles (16 rows) per workgroup; 0: the shape stays on qgemm_kernel
+    int ks;  // K slices
+};
+
+// Depends on the format and the matrix only, never on M, so that a row's bits do not depend on the batch it sits
+// in. One workgroup per compute unit: the plan with the shortest modelled time among those whose workgroups all
+// run at once. VEXEL_HIP_WPLAN="NxK:R,KS;..." overrides (tuning).
+WavePlan wave_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K) {
+    WavePlan none = {0, 1};
+    static const char *off = getenv("VEXEL_HIP_WAVE_OFF");
+    if (off && atoi(off)) return none;
+    if (fmt != VX_Q4_0 && fmt != VX_Q8_0 && fmt != VX_Q4_K) return none;
+    if (K % 256 != 0 || N % 16 != 0 || N < 64) return none;
+    const int cus = gemm_cus(be), tiles = N / 16, n_chunks = K / 256;
+    auto fits = [&](int r) {
+        if (N < 16 * r) return false;
+        for (int i = 0; i < 2; i++)
+            if (segs.n_end[i] < N && segs.n_end[i] % (16 * r) != 0) return false;
+        return true;
+    };
+    static const char *env = getenv("VEXEL_HIP_WPLAN");
+    if (env) {
+        char key[64];
+        snprintf(key, sizeof key, "%dx%d:", N, K);
+        const char *p = strstr(env, key);
+        if (p) {
+            int r = 0, ks = 1;
+            if (sscanf(p + strlen(key), "%d,%d", &r, &ks) == 2 && fits(r)) return WavePlan{r, std::max(1, std::min(ks, n_chunks))};
+        }
+    }
+    // more than 6 tiles a workgroup would spill registers: taller matrices (output heads) stay on qgemm_kernel
+    if (tiles > (fmt == VX_Q8_0 ? 4 : 6) * cus) return none;
+    static const int rs[] = {1, 2, 3, 4, 6};
+    WavePlan best = none;
+    float best_cost = 0.f;
+    for (int r : rs) {
+        if (!fits(r) || (fmt == VX_Q8_0 && r > 4)) continue;  // Q8_0's wider staging leaves room for 4 tiles
+        const int rg = ceil_div(tiles, r);
+        for (int ks = 1; ks <= std::min(n_chunks, 8); ks++) {
+            if (rg * ks > cus) continue;
+            const int wg_chunks = ceil_div(n_chunks, ks), wave_chunks = ceil_div(wg_chunks, 8);
+            // In cycles, fitted to the 7B shapes at 32 rows: a wave's tile steps share a SIMD with one other
+            // wave's (about 220 cycles a tile step for the pair); a compute unit pulls the 32 KB of activation
+            // tiles of a chunk at about 32 bytes a cycle; each extra slice costs its partial sums' trip through
+            // memory and the consumer's pass over them.
+            const float compute = (float)wave_chunks * 8.f * (float)r * 220.f;
+            const float operand = (float)wg_chunks * 1024.f;
+            const float part = ks > 1 ? (float)ks * (float)N * 0.06f + 1500.f : 0.f;
+            const float cost = std::max(compute, operand) + part;
+            if (best.r == 0 || cost < best_cost) {
+                best = WavePlan{r, ks};
+                best_cost = cost;
+            }
+        }
+    }
+    return best;
+}
+
+template <class W, int R>
+int launch_gemm_wave(vx_backend *be, const Segs &segs, int N, float *out, const float *residual, bool to_partials, int M,
+                     int K, int ks, int *ks_out) {
+    constexpr int NW = 8;
+    const int mpad = mpad_for(M);
+    const PrepView pv = prep_view(be, mpad, K);
+    const int rg = ceil_div(N, 16 * R), mgroups = mpad <= 16 ? 1 : mpad / 32;
+    float *partial = nullptr;
+    if (ks > 1 || to_partials) {
+        int rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, (size_t)ks * M * N * sizeof(float), "split-K partial sums");
+        if (rc) return rc;
+        partial = (float *)be->part_ws;
+    }
+    dim3 grid(rg, ks, mgroups);
+    const bool vec = ((uintptr_t)out % 16) == 0 && ((uintptr_t)residual % 16) == 0;
+    const int n_chunks = K / 256, slices = ((n_chunks / ks) << 16) | (n_chunks % ks);  // the kernel takes the division done
+    if (mpad <= 16)
+        qgemm_wave_kernel<W, R, 1, NW><<<grid, 64 * NW, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slices, vec ? 1 : 0);
+    else
+        qgemm_wave_kernel<W, R, 2, NW><<<grid, 64 * NW, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slices, vec ? 1 : 0);
+    VX_CHECK_LAUNCH();
+    if (ks_out) *ks_out = ks;
+    if (partial && !to_partials) {
+        const size_t total = (size_t)M * N;
+        qgemm_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>(partial, pv.inv_scale, out, residual, M, N, ks);
+        VX_CHECK_LAUNCH();
+    }
+    return VX_OK;
+}
+
+template <class W>
+int launch_gemm_wave_r(vx_backend *be, const WavePlan &pl, const Segs &segs, int N, float *out, const float *residual,
+                       bool to_partials, int M, int K, int *ks_out) {
+    switch (pl.r) {
+    case 1: return launch_gemm_wave<W, 1>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
+    case 2: return launch_gemm_wave<W, 2>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
+    case 3: return launch_gemm_wave<W, 3>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
+    case 4: return launch_gemm_wave<W, 4>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
+    case 6: return launch_gemm_wave<W, 6>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
+    }
+    set_error("wave GEMM: no kernel for %d tiles per workgroup", pl.r);
+    return VX_ERR_INVALID;
+}
+
 int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out, const float *residual,
                     bool to_partials, int M, int K, int *ks_out) {
+    const WavePlan pl = wave_plan(be, fmt, segs, N, K);
+    if (pl.r > 0) {
+        if (fmt == VX_Q4_0) return launch_gemm_wave_r<WQ4_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out);
+        if (fmt == VX_Q8_0) return launch_gemm_wave_r<WQ8_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out);
+        return launch_gemm_wave_r<WQ4_K>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out);
+    }
     switch (fmt) {
     case VX_Q4_0: return launch_gemm<PQ4_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
     case VX_Q8_0: return launch_gemm<PQ8_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
