@@ -352,6 +352,12 @@ typedef struct vx_graph vx_graph;
 int vx_graph_begin_capture(vx_backend *be);
 int vx_graph_end_capture(vx_backend *be, vx_graph **out);
 int vx_graph_launch(vx_backend *be, vx_graph *g);
+/* A recording holds the addresses of the library's own scratch buffers (prepared activations, split-K and
+ * split-KV partial sums, the attention work list). They move when a later eager call needs more room than any
+ * call before it; the counter returned here goes up by one each time that happens. A caller that keeps a graph
+ * records the counter after vx_graph_end_capture and captures again, instead of launching, once it has changed.
+ * No counterpart in the reference (its command buffers are rebuilt every step). */
+uint64_t vx_scratch_generation(const vx_backend *be);
 void vx_graph_destroy(vx_graph *g);
 
 /* Wall-clock helpers on the backend stream (HIP events), for benchmarks. */

@@ -59,10 +59,11 @@ def test_c1_prefill_then_greedy_decode(be):
     mr.close()
 
 
-def _ragged_setup(be, cfg, fmt, head_fmt, ctx_lens, seed, pool_blocks, fmt_overrides=None):
+def _ragged_setup(be, cfg, fmt, head_fmt, ctx_lens, seed, pool_blocks, fmt_overrides=None, max_blocks_per_seq=None):
     omodel = om.random_model(cfg, seed, fmt, head_fmt, max_blocks=pool_blocks, fmt_overrides=fmt_overrides)
     mr = gpu_model_from_oracle(be, omodel, pool_blocks=pool_blocks, max_seqs=len(ctx_lens) + 2,
-                               max_blocks_per_seq=max(ctx_lens) // cfg.block_size + 8, max_batch=len(ctx_lens))
+                               max_blocks_per_seq=max_blocks_per_seq or max(ctx_lens) // cfg.block_size + 8,
+                               max_batch=len(ctx_lens))
     rng = np.random.default_rng(seed + 1)
     perm = rng.permutation(pool_blocks)       # block tables are a seeded random permutation
     off = 0
@@ -164,6 +165,74 @@ def test_device_driven_graph_decode_matches_host_driven(be):
         toks = [nx.argmax(lg[i]) for i in range(len(ctx))]
         assert eager[s].tolist() == toks
         pos = [p + 1 for p in pos]
+    mr.close()
+
+
+def _greedy_oracle(omodel, toks, ids, pos, steps):
+    toks, pos, out = list(toks), list(pos), []
+    for _ in range(steps):
+        lg = omodel.decode_batched(toks, ids, pos)
+        toks = [nx.argmax(lg[i]) for i in range(len(ids))]
+        out.append(list(toks))
+        pos = [p + 1 for p in pos]
+    return out, toks, pos
+
+
+def test_graph_decode_after_the_scratch_buffers_moved():
+    """A kept graph holds the library's scratch addresses. A prefill of more rows than the decode batch makes
+    those buffers grow (and move); the next device-driven call must notice and record the step again instead of
+    replaying the old graph over freed memory."""
+    from vexel_amd.backend import HipBackend
+    own = HipBackend(0)   # a backend of its own: its scratch is as small as this test's first calls leave it
+    cfg = om.ModelConfig(num_layers=2, hidden=512, num_heads=8, num_kv_heads=2, head_dim=64, ffn=1024, vocab=1024)
+    ctx = [20, 33, 50]
+    omodel, mr, rng = _ragged_setup(own, cfg, nx.FMT_Q4_0, nx.FMT_Q8_0, ctx, 41, pool_blocks=96, max_blocks_per_seq=24)
+    ids = [100 + i for i in range(3)]
+    first = rng.integers(0, cfg.vocab, 3).tolist()
+    want, toks, pos = _greedy_oracle(omodel, first, ids, ctx, 4)
+    out, _ = mr.decode_graph(first, ids, ctx, 4, use_graph=True)
+    assert out.tolist() == want
+    gen = own.scratch_generation()
+    # another request arrives: a 300-token prompt goes through the same library scratch
+    prompt = rng.integers(0, cfg.vocab, 300).tolist()
+    omodel.pool.create_sequence(7)
+    mr.create_sequence(7)
+    assert_logits_close(mr.prefill_with_paged_kv(prompt, 7, 0), omodel.prefill_with_paged_kv(prompt, 7, 0), "prefill between graphs")
+    assert own.scratch_generation() > gen, "the prefill was meant to outgrow the decode batch's scratch"
+    want2, toks, pos = _greedy_oracle(omodel, toks, ids, pos, 6)
+    more, _ = mr.decode_graph(None, None, None, 6, use_graph=True, batch=3)
+    assert more.tolist() == want2
+    assert mr.device_matches_host()
+    mr.close()
+    own.close()
+
+
+def test_device_driven_decode_refuses_steps_the_pool_cannot_hold(be):
+    """More steps than the free blocks allow are refused before anything runs on the device: tables, free list and
+    the K/V rows stay as they were, and a shorter run afterwards matches the oracle."""
+    from vexel_amd.backend import VexelError
+    cfg = om.ModelConfig(num_layers=2, hidden=512, num_heads=8, num_kv_heads=2, head_dim=64, ffn=1024, vocab=1024)
+    ctx = [30, 47, 16]    # 2 + 3 + 1 blocks of the pool's 9: three are free
+    omodel, mr, rng = _ragged_setup(be, cfg, nx.FMT_Q4_0, nx.FMT_Q8_0, ctx, 43, pool_blocks=9)
+    ids = [100 + i for i in range(3)]
+    first = rng.integers(0, cfg.vocab, 3).tolist()
+    # 40 steps: sequence 0 would need 5 blocks (+3), sequence 1 six (+3), sequence 2 four (+3)
+    with pytest.raises(VexelError, match="free blocks"):
+        mr.decode_graph(first, ids, ctx, 40, use_graph=True)
+    assert mr.device_matches_host()
+    for sid, c in zip(ids, ctx):
+        assert mr.seq_len(sid) == c
+    # one sequence over its own limit
+    with pytest.raises(VexelError, match="max_blocks_per_seq"):
+        mr.decode_graph(first, ids, ctx, 16 * 20, use_graph=True)
+    want, toks, pos = _greedy_oracle(omodel, first, ids, ctx, 6)   # within the three free blocks
+    out, _ = mr.decode_graph(first, ids, ctx, 6, use_graph=True)
+    assert out.tolist() == want
+    assert mr.device_matches_host()
+    # the batch on the device loses a sequence: continuing is refused, not a null dereference
+    mr.delete_sequence(ids[1])
+    with pytest.raises(VexelError, match="deleted"):
+        mr.decode_graph(None, None, None, 1, use_graph=True, batch=3)
     mr.close()
 
 

@@ -42,6 +42,7 @@ int ensure_ws(vx_backend *be, void **ptr, size_t *cap, size_t bytes, const char 
         return VX_ERR_OOM;
     }
     *cap = want;
+    be->scratch_gen++;
     return VX_OK;
 }
 
@@ -52,6 +53,8 @@ using namespace vx;
 extern "C" {
 
 const char *vx_last_error(void) { return g_err; }
+
+uint64_t vx_scratch_generation(const vx_backend *be) { return be ? be->scratch_gen : 0; }
 
 int vx_backend_create(int device_id, vx_backend **out) {
     if (!out) {

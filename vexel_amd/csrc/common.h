@@ -59,7 +59,9 @@ struct vx_backend {
     // permanent allocations (vx_alloc_permanent / vx_free)
     std::unordered_map<void *, size_t> permanent;
 
-    // library-owned scratch, grown on demand outside graph capture
+    // library-owned scratch, grown on demand outside graph capture; scratch_gen counts the reallocations
+    // (a captured graph holds the old addresses)
+    uint64_t scratch_gen = 0;
     void *gemm_ws = nullptr;     // prepared (split, tiled) activations for the quantized GEMM
     size_t gemm_ws_bytes = 0;
     int prep_m = 0, prep_k = 0;  // shape of the activation currently prepared in gemm_ws

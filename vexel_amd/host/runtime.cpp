@@ -134,6 +134,7 @@ struct vh_model {
 
     vx_graph *graph = nullptr;
     int graph_batch = 0;
+    uint64_t graph_scratch_gen = 0;  // vx_scratch_generation() when the graph was captured
     std::vector<int64_t> dev_seq_ids;  // batch currently loaded in d_slots (device-driven mode)
     std::vector<int32_t> dev_positions;
 };
@@ -1158,6 +1159,26 @@ int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_
 }
 
 // ------------------------------------------------------------------ device-driven greedy decode
+// The device-driven steps allocate blocks on the device and cannot stop half way: the host, which knows every
+// table and the free count, checks before the first launch that `steps` more tokens per sequence fit
+// (gpu_block_pool.go:234-245 applied steps times), and fails without touching the device when they do not.
+static int check_room(vh_model *m, const int64_t *seq_ids, const int32_t *positions, int batch, int steps) {
+    const int bs = m->pool.block_size;
+    long long need = 0;
+    for (int i = 0; i < batch; i++) {
+        const SeqState *s = find_seq(m, seq_ids[i]);
+        const int blocks = (positions[i] + steps - 1) / bs + 1;  // blocks holding positions 0 .. positions[i] + steps - 1
+        if (blocks > m->cfg.max_blocks_per_seq)
+            return fail("sequence %lld: %d more tokens need %d blocks, max_blocks_per_seq is %d", (long long)seq_ids[i], steps,
+                        blocks, m->cfg.max_blocks_per_seq);
+        need += std::max(0, blocks - (int)s->table.size());
+    }
+    if (need > (long long)m->pool.free_list.size())
+        return fail("%d more tokens for %d sequences need %lld free blocks, the pool has %zu", steps, batch, need,
+                    m->pool.free_list.size());
+    return VH_OK;
+}
+
 static int device_step(vh_model *m, int batch) {
     const vh_config &c = m->cfg;
     VXC(vx_pack_batch(m->be, m->d_slots, m->d_positions, nullptr, batch, batch, m->d_tables, c.max_blocks_per_seq,
@@ -1185,6 +1206,7 @@ int vh_decode_graph(vh_model *m, const int32_t *first_tokens, const int64_t *seq
                 return fail("sequence %lld: position %d is not its length %d", (long long)seq_ids[i], positions[i], s->seq_len);
             slots[i] = s->slot;
         }
+        VHC(check_room(m, seq_ids, positions, batch, steps));
         VHC(sync_pool_to_device(m));
         VXC(vx_to_device(m->be, m->d_tokens, first_tokens, (size_t)batch * 4));
         VXC(vx_to_device(m->be, m->d_positions, positions, (size_t)batch * 4));
@@ -1193,6 +1215,10 @@ int vh_decode_graph(vh_model *m, const int32_t *first_tokens, const int64_t *seq
         m->dev_positions.assign(positions, positions + batch);
     } else {
         if ((int)m->dev_seq_ids.size() != batch) return fail("no batch of %d sequences is loaded on the device", batch);
+        for (int i = 0; i < batch; i++)
+            if (!find_seq(m, m->dev_seq_ids[i]))
+                return fail("sequence %lld of the batch on the device was deleted; pass the batch again", (long long)m->dev_seq_ids[i]);
+        VHC(check_room(m, m->dev_seq_ids.data(), m->dev_positions.data(), batch, steps));
         VHC(sync_pool_to_device(m));  // lifecycle events since the last call (no-op when nothing changed)
     }
     if (m->log_cap < steps) {
@@ -1209,7 +1235,9 @@ int vh_decode_graph(vh_model *m, const int32_t *first_tokens, const int64_t *seq
     VXC(vx_to_device(m->be, m->d_step, &zero, 4));
     vx_reset_pool(m->be);
     int done = 0;
-    if (use_graph && (!m->graph || m->graph_batch != batch)) {
+    // a recording holds the library's scratch addresses: once an eager call in between (a longer prefill, a tree
+    // verification, a larger batch) has made one of them grow, it is stale
+    if (use_graph && (!m->graph || m->graph_batch != batch || m->graph_scratch_gen != vx_scratch_generation(m->be))) {
         if (m->graph) vx_graph_destroy(m->graph);
         m->graph = nullptr;
         VHC(device_step(m, batch));  // eager: sizes the library scratch; it is step 0 of this call
@@ -1222,6 +1250,7 @@ int vh_decode_graph(vh_model *m, const int32_t *first_tokens, const int64_t *seq
         if (rc2 != VX_OK) return fail("graph capture: %s", vx_last_error());
         m->graph = gr;
         m->graph_batch = batch;
+        m->graph_scratch_gen = vx_scratch_generation(m->be);
     }
     VXC(vx_timer_start(m->be));
     const int timed = steps - done;
@@ -1236,7 +1265,14 @@ int vh_decode_graph(vh_model *m, const int32_t *first_tokens, const int64_t *seq
     if (ms_per_step) *ms_per_step = timed > 0 ? ms / timed : 0.f;
     int32_t status = 0;
     VXC(vx_to_host(m->be, &status, m->d_status, 4));
-    if (status != 0) return fail("the block pool ran out of blocks during the device-driven steps");
+    if (status != 0) {
+        // check_room() rules this out; should it happen all the same, the device tables are no longer the host's:
+        // have the next call rebuild them
+        for (auto &kv : m->pool.seqs) kv.second.dirty = true;
+        m->pool.free_dirty = true;
+        m->dev_seq_ids.clear();
+        return fail("the block pool ran out of blocks during the device-driven steps");
+    }
     std::vector<int32_t> log((size_t)steps * batch);
     VXC(vx_to_host(m->be, log.data(), m->d_log, log.size() * 4));
     if (out_tokens) memcpy(out_tokens, log.data(), log.size() * 4);

@@ -18,6 +18,7 @@ SIGNATURES = {
     "vx_backend_destroy": (None, [_vp]),
     "vx_backend_device": (_i, [_vp]),
     "vx_last_error": (C.c_char_p, []),
+    "vx_scratch_generation": (C.c_uint64, [_vp]),
     "vx_alloc": (_vp, [_vp, _sz]),
     "vx_alloc_permanent": (_vp, [_vp, _sz]),
     "vx_free": (None, [_vp, _vp]),
