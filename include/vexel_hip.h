@@ -141,8 +141,9 @@ int vx_matmul_q4_0(vx_backend *be, const float *a, const void *b, float *out, in
 int vx_matmul_q4_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :55 */
 int vx_matmul_q6_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :60 */
 int vx_matmul_q8_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :75 */
-/* Not in any benchmark config: one wave per weight row on the exact dequantised values (pkg/gguf/dequant.go:
- * 423-500, 100-145, 215-228), no tiled or matrix-vector fast path. */
+/* Not in any benchmark config. Q5_K and Q5_0 (pkg/gguf/dequant.go:423-500, 100-145) run on the same two kernels
+ * as the formats above (the streaming matrix-vector kernel for one row, the MFMA kernel for more); BF16
+ * (dequant.go:215-228) has one wave per weight row on the exact values only. */
 int vx_matmul_q5_k(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :65 */
 int vx_matmul_q5_0(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :70 */
 int vx_matmul_bf16(vx_backend *be, const float *a, const void *b, float *out, int m, int n, int k); /* :80 */
@@ -262,7 +263,9 @@ int vx_rope_store_paged_ex(vx_backend *be, float *q, const float *k, const float
 /* Ragged batched paged attention with all metadata on the device: block_tables is a
  * padded int32 [rows, max_blocks] matrix; sequence i uses row table_rows[i] (row i when
  * table_rows is NULL); kv_lens int32[batch]. One query per sequence. max_kv_len bounds
- * the launch (>= every kv_lens[i]). With out = NULL the result stays in the backend as per-split partial
+ * the launch (>= every kv_lens[i]; the lengths live on the device, so the host cannot check the promise: the
+ * streaming kernels attend a longer sequence over its first max_kv_len tokens, rounded up to whole splits, and stay
+ * inside their buffers; max_blocks * block_size is always a safe value). With out = NULL the result stays in the backend as per-split partial
  * sums for the next vx_decode_ffn(attn = NULL) to merge (one launch less); that form exists only where
  * vx_sdpa_paged_decode_split_supported() is 1, otherwise the call returns VX_ERR_UNSUPPORTED.
  * That is also where the streaming split-KV kernel runs (F16 pool, 16-token blocks): heads of 64 or 128 with 1 to 8

@@ -226,8 +226,12 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
         kv_len = kv_lens[seq];
         row = bt_rows ? bt_rows[seq] : seq;
     }
+    // The caller's max_kv_len sized the partial sums (max_splits per sequence and head). A length above it is
+    // attended over its first max_splits * TPW tokens by every kernel of the path alike: defined, and inside the
+    // buffers.
+    kv_len = min(kv_len, max_splits * TPW);
     const int t_begin = split * TPW;
-    if (t_begin >= kv_len) return;
+    if (split >= max_splits || t_begin >= kv_len) return;
     const int t_end = min(kv_len, t_begin + TPW);
     const int32_t *bt = bt_matrix + (size_t)row * max_blocks + t_begin / HOT_BS;
 
@@ -378,7 +382,7 @@ __global__ void __launch_bounds__(D) paged_merge_kernel(const float *__restrict_
                                                         int num_q_heads, int max_splits) {
     const int qh = blockIdx.x, seq = blockIdx.y, d = threadIdx.x;
     const int kv_len = kv_lens[seq];
-    const int ns = (kv_len + TPW - 1) / TPW;
+    const int ns = min((kv_len + TPW - 1) / TPW, max_splits);  // a length over the caller's bound: its first max_splits splits
     const float *pb = partial + ((size_t)seq * num_q_heads + qh) * max_splits * (D + 2);
     float M = -INFINITY;
     for (int s = 0; s < ns; s++) M = fmaxf(M, pb[(size_t)s * (D + 2)]);

@@ -81,7 +81,7 @@ int vx_backend_create(int device_id, vx_backend **out) {
     be->misc_ws_bytes = 1 << 20;
     VX_CHECK_HIP(hipMalloc(&be->misc_ws, be->misc_ws_bytes));
     VX_CHECK_HIP(hipMalloc(&be->prep_sync, VX_PREP_SYNC_BYTES));
-    VX_CHECK_HIP(hipMemset(be->prep_sync, 0, VX_PREP_SYNC_BYTES));  // arrival counters start at zero and reset themselves
+    VX_CHECK_HIP(hipMemset(be->prep_sync, 0, VX_PREP_SYNC_BYTES));  // per-chunk sums of squares: every slot a prepare reads was written by the kernel before it
     {
         float ones[64];
         for (float &o : ones) o = 1.0f;

@@ -1242,7 +1242,7 @@ __global__ void __launch_bounds__(PREP_THREADS) merge_prepare_kernel(const float
         for (int c = tid; c < K / 256; c += blockDim.x) pv.cscale[(size_t)c * Mpad + r] = 0.f;
         return;
     }
-    const int ns = (kv_lens[r] + tokens_per_split - 1) / tokens_per_split;
+    const int ns = min((kv_lens[r] + tokens_per_split - 1) / tokens_per_split, max_splits);
     const int P = D + 2;
     float amax = 0.f, ss = 0.f;
     for (int k = tid * 4; k < K; k += PREP_THREADS * 4) {
@@ -1435,7 +1435,7 @@ __global__ void __launch_bounds__(64) chunk_merge_kernel(const float *__restrict
     const int k = c * 256 + lane * 4;
     float y[4] = {0.f, 0.f, 0.f, 0.f};
     if (r < M) {
-        const int ns = (kv_lens[r] + tokens_per_split - 1) / tokens_per_split;
+        const int ns = min((kv_lens[r] + tokens_per_split - 1) / tokens_per_split, max_splits);
         const int P = D + 2, h = k / D, d = k % D;
         const float *pb = part + ((size_t)r * (K / D) + h) * max_splits * P;
         float Mx = -INFINITY;
