@@ -277,6 +277,19 @@ int vx_sdpa_paged_decode_ragged(vx_backend *be, const float *q, const void *kv_p
                                 const int32_t *block_tables, const int32_t *table_rows, const int32_t *kv_lens,
                                 float *out, int batch, int max_blocks, int block_size, int num_q_heads,
                                 int num_kv_heads, int head_dim, float scale, int max_kv_len);
+/* vx_sdpa_paged_decode_ragged for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc): the same kernels, same arguments and bit-identical results, with
+ * the per-split partial sums in a fixed 8 MiB area that every device holds from the moment the library is loaded
+ * until the process ends, instead of the backend's growable scratch. It has no counterpart in the reference. The
+ * call allocates and frees nothing. It needs out != NULL and a geometry of the streaming kernel
+ * (vx_sdpa_paged_decode_split_supported() == 1), else VX_ERR_UNSUPPORTED; batch * num_q_heads *
+ * ceil(max_kv_len / 512) * (head_dim + 2) * 4 bytes must fit the area (32 sequences x 32 heads of 128 up to 4096
+ * tokens take 4.3 MB), else VX_ERR_INVALID with the sizes in vx_last_error(). All calls on one device, from any
+ * backend, share the area: two of them in flight at once race. */
+int vx_sdpa_paged_decode_ragged_noalloc(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
+                                        const int32_t *block_tables, const int32_t *table_rows, const int32_t *kv_lens,
+                                        float *out, int batch, int max_blocks, int block_size, int num_q_heads,
+                                        int num_kv_heads, int head_dim, float scale, int max_kv_len);
 
 /* Tree verification (medusa/tree.go:186-202 mask rule): query i attends to every pool
  * position < tree_base and to position tree_base+j iff tree_mask[i*query_len+j] != 0

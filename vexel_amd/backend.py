@@ -309,6 +309,12 @@ class HipBackend:
         self.call("vx_sdpa_paged_decode_ragged", q, kv_pool, int(bool(pool_is_f16)), block_tables, table_rows,
                   kv_lens, out, batch, max_blocks, block_size, num_q_heads, num_kv_heads, head_dim, scale, max_kv_len)
 
+    def sdpa_paged_decode_ragged_noalloc(self, q, kv_pool, pool_is_f16, block_tables, kv_lens, out, batch, max_blocks,
+                                         block_size, num_q_heads, num_kv_heads, head_dim, scale, max_kv_len,
+                                         table_rows=None):
+        self.call("vx_sdpa_paged_decode_ragged_noalloc", q, kv_pool, int(bool(pool_is_f16)), block_tables, table_rows,
+                  kv_lens, out, batch, max_blocks, block_size, num_q_heads, num_kv_heads, head_dim, scale, max_kv_len)
+
     def sdpa_paged_tree(self, q, kv_pool, pool_is_f16, block_table, out, tree_mask, tree_base, block_size,
                         num_q_heads, num_kv_heads, head_dim, scale, query_len):
         self.call("vx_sdpa_paged_tree", q, kv_pool, int(bool(pool_is_f16)), block_table, out, tree_mask,

@@ -608,14 +608,32 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
     }
 }
 
+// The partial sums of a call that must not allocate: one fixed area per device, shared by every such call on that
+// device (calls that overlap there race). Host code never uses the array's name as an address: attn_noalloc_init
+// asks the runtime where the current device keeps its copy, and that pointer is what the kernels get.
+constexpr size_t FIXED_WS_BYTES = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[FIXED_WS_BYTES];
+
+// fixed: the call takes the fixed area (and fails when it is too small) instead of the growable one
 template <int D, int G>
 int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *bt_matrix, const int32_t *bt_rows,
                int max_blocks, const int32_t *kv_lens, float *out, int batch, int num_q_heads, int num_kv_heads,
-               float scale, int max_kv_len) {
+               float scale, int max_kv_len, bool fixed) {
     int max_splits = ceil_div(max_kv_len, TPW);
     size_t need = (size_t)batch * num_q_heads * max_splits * (D + 2) * sizeof(float);
-    int rc = ensure_ws(be, &be->attn_ws, &be->attn_ws_bytes, need, "attention");
-    if (rc) return rc;
+    float *ws;
+    if (fixed) {
+        if (need > FIXED_WS_BYTES || !be->attn_fixed_ws) {
+            set_error("vx_sdpa_paged_decode_ragged_noalloc: %d sequences x %d heads x %d splits of %d tokens need %zu bytes of "
+                      "partial sums, the fixed area holds %zu", batch, num_q_heads, max_splits, TPW, need, FIXED_WS_BYTES);
+            return VX_ERR_INVALID;
+        }
+        ws = (float *)be->attn_fixed_ws;
+    } else {
+        int rc = ensure_ws(be, &be->attn_ws, &be->attn_ws_bytes, need, "attention");
+        if (rc) return rc;
+        ws = (float *)be->attn_ws;
+    }
     // With a work list from vx_pack_batch for these lengths the grid's second dimension runs over its items
     // (at most max_splits per sequence, as max_kv_len bounds every length); otherwise over (split, sequence).
     const bool listed = be->items.valid && be->items.kv_lens == kv_lens && be->items.table_rows == bt_rows &&
@@ -624,11 +642,11 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
                         (size_t)batch * max_splits <= 65535;
     dim3 grid(num_kv_heads, listed ? batch * max_splits : max_splits, listed ? 1 : batch);
     paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
-                                                                max_blocks, kv_lens, (float *)be->attn_ws, num_q_heads,
+                                                                max_blocks, kv_lens, ws, num_q_heads,
                                                                 num_kv_heads, scale, max_splits,
                                                                 listed ? be->items.buf : nullptr);
     VX_CHECK_LAUNCH();
-    be->split.batch = 0;
+    if (!fixed) be->split.batch = 0;  // (the fixed area is not where vx_decode_ffn looks for a split result)
     if (!out) {  // the caller merges: vx_decode_ffn(attn = NULL)
         be->split.batch = batch;
         be->split.num_q_heads = num_q_heads;
@@ -638,8 +656,7 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
         be->split.kv_lens = kv_lens;
         return VX_OK;
     }
-    paged_merge_kernel<D><<<dim3(num_q_heads, batch), D, 0, be->stream>>>((const float *)be->attn_ws, kv_lens, out,
-                                                                          num_q_heads, max_splits);
+    paged_merge_kernel<D><<<dim3(num_q_heads, batch), D, 0, be->stream>>>(ws, kv_lens, out, num_q_heads, max_splits);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }
@@ -658,7 +675,7 @@ int run_generic(vx_backend *be, const AttnParams &p, int num_queries) {
 int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16, const int32_t *const *bt_ptrs,
                const int32_t *bt_matrix, const int32_t *bt_rows, int max_blocks, const int32_t *kv_lens, float *out,
                int batch, int block_size,
-               int num_q_heads, int num_kv_heads, int head_dim, float scale, int max_kv_len) {
+               int num_q_heads, int num_kv_heads, int head_dim, float scale, int max_kv_len, bool fixed = false) {
     VX_REQUIRE(num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, "attention: bad head counts");
     VX_REQUIRE(block_size > 0 && max_kv_len > 0, "attention: bad block size / kv length");
     if (batch == 0) return VX_OK;
@@ -667,7 +684,7 @@ int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16
 #define VX_HOT(DD, GG)                                                                                         \
     if (hot && head_dim == DD && G == GG)                                                                      \
         return launch_hot<DD, GG>(be, q, pool, bt_matrix, bt_rows, max_blocks, kv_lens, out, batch, num_q_heads, \
-                                  num_kv_heads, scale, max_kv_len);
+                                  num_kv_heads, scale, max_kv_len, fixed);
     VX_HOT(128, 1) VX_HOT(128, 2) VX_HOT(128, 4) VX_HOT(128, 8)
     VX_HOT(64, 1) VX_HOT(64, 2) VX_HOT(64, 4) VX_HOT(64, 8)
     // group sizes that are no power of two (Qwen 2 7B: 28 / 4 heads, LLaMA 3.2 3B: 24 / 8, Qwen 2 1.5B: 12 / 2)
@@ -678,6 +695,11 @@ int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16
     // heads of 80 (Phi-2) and 96 (Phi-3 mini) on 16 lanes per token, 10 or 12 of them live
     VX_HOT(80, 1) VX_HOT(96, 1)
 #undef VX_HOT
+    if (fixed) {
+        set_error("vx_sdpa_paged_decode_ragged_noalloc: only the geometries of the streaming kernel (see "
+                  "vx_sdpa_paged_decode_split_supported) run without scratch allocation");
+        return VX_ERR_UNSUPPORTED;
+    }
     if (!out) {
         set_error("vx_sdpa_paged_decode_ragged: out = NULL (split form) needs an F16 pool with 16-token blocks and a "
                   "supported head geometry");
@@ -703,6 +725,15 @@ int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16
 }
 
 }  // namespace
+
+namespace vx {
+int attn_noalloc_init(vx_backend *be) {
+    void *p = nullptr;
+    VX_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));  // the current device's copy of the array
+    be->attn_fixed_ws = p;
+    return VX_OK;
+}
+}  // namespace vx
 
 extern "C" {
 
@@ -870,6 +901,19 @@ int vx_sdpa_paged_decode_ragged(vx_backend *be, const float *q, const void *kv_p
     return run_ragged(be, q, kv_pool, pool_is_f16, nullptr, block_tables, table_rows, max_blocks, kv_lens, out, batch,
                       block_size,
                       num_q_heads, num_kv_heads, head_dim, scale, max_kv_len);
+}
+
+int vx_sdpa_paged_decode_ragged_noalloc(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
+                                        const int32_t *block_tables, const int32_t *table_rows, const int32_t *kv_lens,
+                                        float *out, int batch, int max_blocks, int block_size, int num_q_heads,
+                                        int num_kv_heads, int head_dim, float scale, int max_kv_len) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(q && kv_pool && block_tables && kv_lens && out, "vx_sdpa_paged_decode_ragged_noalloc: null pointer");
+    VX_REQUIRE(batch >= 0 && max_kv_len > 0 && max_kv_len <= max_blocks * block_size,
+               "vx_sdpa_paged_decode_ragged_noalloc: max_kv_len %d not in 1..table capacity %d", max_kv_len, max_blocks * block_size);
+    return run_ragged(be, q, kv_pool, pool_is_f16, nullptr, block_tables, table_rows, max_blocks, kv_lens, out, batch,
+                      block_size, num_q_heads, num_kv_heads, head_dim, scale, max_kv_len, true);
 }
 
 int vx_sdpa_paged_decode_split_supported(int pool_is_f16, int block_size, int num_q_heads, int num_kv_heads,

@@ -73,6 +73,13 @@ int vx_backend_create(int device_id, vx_backend **out) {
     }
     vx_backend *be = new vx_backend();
     be->device = device_id;
+    {
+        int rc = attn_noalloc_init(be);
+        if (rc) {
+            delete be;
+            return rc;
+        }
+    }
     VX_CHECK_HIP(hipStreamCreateWithFlags(&be->stream, hipStreamNonBlocking));
     VX_CHECK_HIP(hipEventCreate(&be->ev0));
     VX_CHECK_HIP(hipEventCreate(&be->ev1));

@@ -72,6 +72,7 @@ struct vx_backend {
     void *part_ws = nullptr;     // split-K partial sums
     size_t part_ws_bytes = 0;
     void *attn_ws = nullptr;     // split-KV partial results
+    void *attn_fixed_ws = nullptr;  // this device's copy of the fixed-size partial-sum area (never allocated or freed)
     // attention left in split form by vx_sdpa_paged_decode_ragged(out = NULL), to be merged by vx_decode_ffn
     struct {
         int batch = 0, num_q_heads = 0, head_dim = 0, max_splits = 0, tokens_per_split = 0;
@@ -122,6 +123,9 @@ inline void items_written(vx_backend *be, const void *dst, size_t bytes) {
 int enter(vx_backend *be);
 // Ensures a library scratch buffer holds at least `bytes`; fails during capture if it must grow.
 int ensure_ws(vx_backend *be, void **ptr, size_t *cap, size_t bytes, const char *what);
+// Looks up, once per backend and with its device current, where that device keeps the fixed partial-sum area of
+// vx_sdpa_paged_decode_ragged_noalloc (attention.hip); called by vx_backend_create.
+int attn_noalloc_init(vx_backend *be);
 
 // qmatvec.hip: out[n] = a . W[n] (+ residual[n]) for one activation row; VX_ERR_UNSUPPORTED (nothing launched, no
 // error text) when the shape is outside the kernel's range.

@@ -84,6 +84,7 @@ SIGNATURES = {
     "vx_rope_store_paged_ex": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i]),
     "vx_sdpa_paged_decode_split_supported": (_i, [_i, _i, _i, _i, _i]),
     "vx_sdpa_paged_decode_ragged": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i]),
+    "vx_sdpa_paged_decode_ragged_noalloc": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i]),
     "vx_sdpa_paged_tree": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),
     "vx_argmax_rows": (_i, [_vp, _vp, _i, _i, _vp]),
     "vx_sdpa_paged_tree_rows_per_entry": (_i, [_i, _i, _i, _i, _i]),
