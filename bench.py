@@ -83,30 +83,51 @@ def build_model(be, ctx, extra_tokens, layers, cfg=None, fmts=None, max_batch=No
         seed[0] += 1
         return (mean + 0.02 * np.random.default_rng(seed[0]).standard_normal(n)).astype(np.float32)
 
-    def qw(n, k, fmt=lib.VX_Q4_0):
+    def qbytes(n, k, fmt):
+        return n * (k // 32) * (18 if fmt == lib.VX_Q4_0 else 34) if fmt in (lib.VX_Q4_0, lib.VX_Q8_0) else \
+            n * (k // 256) * (144 if fmt == lib.VX_Q4_K else 210)
+
+    def qfill(p, n, k, fmt):
         seed[0] += 1
         if fmt in (lib.VX_Q4_0, lib.VX_Q8_0):
-            bb = 18 if fmt == lib.VX_Q4_0 else 34
-            nblk = n * (k // 32)
-            p = be.alloc_permanent(nblk * bb)
-            rc = synth.vxs_gaussian_quant(fmt, p, nblk, 0.02, seed[0])
+            rc = synth.vxs_gaussian_quant(fmt, p, n * (k // 32), 0.02, seed[0])
         else:                                    # Q4_K / Q6_K: random valid super-blocks
-            bb = 144 if fmt == lib.VX_Q4_K else 210
-            nblk = n * (k // 256)
-            p = be.alloc_permanent(nblk * bb + 16)
-            rc = synth.vxs_random_kquant(fmt, p, nblk, seed[0])
-        mr.adopt_device_buffer(p)
+            rc = synth.vxs_random_kquant(fmt, p, n * (k // 256), seed[0])
         if rc != 0:
             raise RuntimeError("synthetic weights failed: %d" % rc)
         return (fmt, p, n, k)
 
+    def qw(n, k, fmt=lib.VX_Q4_0):
+        p = be.alloc_permanent(qbytes(n, k, fmt) + 16)
+        mr.adopt_device_buffer(p)
+        return qfill(p, n, k, fmt)
+
+    def qgroup(shapes):
+        """The matrices one launch multiplies together (Q|K|V, gate|up), back to back in one buffer when they
+        share format and width and every part starts on a 16-byte boundary; else one buffer each."""
+        sizes = [qbytes(n, k, fmt) for n, k, fmt in shapes]
+        if len({(k, fmt) for _, k, fmt in shapes}) != 1 or any(sz % 16 for sz in sizes):
+            return [qw(n, k, fmt) for n, k, fmt in shapes]
+        p = be.alloc_permanent(sum(sizes) + 16)
+        mr.adopt_device_buffer(p)
+        out, off = [], 0
+        for (n, k, fmt), sz in zip(shapes, sizes):
+            out.append(qfill(p + off, n, k, fmt))
+            off += sz
+        return out
+
     h, qd, kvd, f, v = c["hidden"], c["num_heads"] * c["head_dim"], c["num_kv_heads"] * c["head_dim"], c["ffn"], c["vocab"]
+    layer_weights = []   # per layer: name -> (fmt, device pointer, n, k); kept on the runtime object for the GEMM timing
+    mr.layer_weights = layer_weights
     ones = be.upload(np.ones(h, dtype=np.float32), permanent=True)
     mr.adopt_device_buffer(ones)
     for l in range(layers):
-        mr.set_layer(l, ones, ones, dict(wq=qw(qd, h, fm("wq")), wk=qw(kvd, h, fm("wk")), wv=qw(kvd, h, fm("wv")),
-                                         wo=qw(h, qd, fm("wo")), w1=qw(f, h, fm("w1")),
-                                         w3=None if gelu_mlp else qw(f, h, fm("w3")), w2=qw(h, f, fm("w2"))))
+        wq, wk, wv = qgroup([(qd, h, fm("wq")), (kvd, h, fm("wk")), (kvd, h, fm("wv"))])
+        wo = qw(h, qd, fm("wo"))
+        w1, w3 = (qw(f, h, fm("w1")), None) if gelu_mlp else qgroup([(f, h, fm("w1")), (f, h, fm("w3"))])
+        w2 = qw(h, f, fm("w2"))
+        mr.set_layer(l, ones, ones, dict(wq=wq, wk=wk, wv=wv, wo=wo, w1=w1, w3=w3, w2=w2))
+        layer_weights.append(dict(wq=wq, wk=wk, wv=wv, wo=wo, w1=w1, w3=w3, w2=w2))
         extras = {}
         if bias_kind in ("qkv", "all"):
             extras.update(wq_bias=vec(qd, 0.0), wk_bias=vec(kvd, 0.0), wv_bias=vec(kvd, 0.0))
@@ -189,10 +210,14 @@ def time_attention_kernel(be, mr, ctx_now, c, layers, reps, from_step=False):
     return ms / reps
 
 
-def cpu_baseline(be, mr, ctx, c, sample_layers=2, head_rows=2000):
+def cpu_baseline(be, mr, ctx, c, sample_layers=2, head_rows=2000, threads=1):
     """The reference CPU path (our C restatement, one core: the reference parallelises matmuls over M
     only and decodes one sequence at a time, cpu.go:856-870, decode.go:642-650) timed on a bounded
-    sample: `sample_layers` layers + `head_rows` lm_head rows for one sequence, scaled to a full token."""
+    sample: `sample_layers` layers + `head_rows` lm_head rows for one sequence, scaled to a full token.
+    The random bytes that stand for the weights are not the GPU run's weights: values differ, timing does not
+    depend on them. threads > 1: every matmul's weight rows are cut into that many slices computed side by side
+    (NOT what the reference does; shown beside the one-core figure for scale)."""
+    from concurrent.futures import ThreadPoolExecutor
     from oracle import numerics as nx
     L = ctx[0]
     hd, qd, kvd, f = c["hidden"], c["num_heads"] * c["head_dim"], c["num_kv_heads"] * c["head_dim"], c["ffn"]
@@ -210,31 +235,107 @@ def cpu_baseline(be, mr, ctx, c, sample_layers=2, head_rows=2000):
     x = rng.standard_normal((1, hd)).astype(np.float32)
     ones = np.ones(hd, dtype=np.float32)
     scale = np.float32(1.0 / math.sqrt(c["head_dim"]))
+    ex = ThreadPoolExecutor(max_workers=threads) if threads > 1 else None
+
+    def rows_parallel(fn, a, wbytes, n, k):
+        """fn(a, weight rows, 1, rows, k) on `threads` slices of the rows (the C code runs without the GIL)"""
+        if ex is None:
+            return fn(a, wbytes, 1, n, k)
+        cuts = [n * i // threads for i in range(threads + 1)]
+        parts = list(ex.map(lambda i: fn(a, wbytes[cuts[i]:cuts[i + 1]], 1, cuts[i + 1] - cuts[i], k), range(threads)))
+        return np.concatenate(parts, axis=1)
+
+    mm = lambda a, name: rows_parallel(nx.matmul_q4_0, a, w[name][0], w[name][1], w[name][2])
     t0 = time.perf_counter()
     for _ in range(sample_layers):
         nrm = nx.rmsnorm(x, ones, 1, hd, 1e-5)
-        q = nx.matmul_q4_0(nrm, w["wq"][0], 1, w["wq"][1], w["wq"][2])
-        k = nx.matmul_q4_0(nrm, w["wk"][0], 1, w["wk"][1], w["wk"][2])
-        v = nx.matmul_q4_0(nrm, w["wv"][0], 1, w["wv"][1], w["wv"][2])
+        q, k, v = mm(nrm, "wq"), mm(nrm, "wk"), mm(nrm, "wv")
         q, k = nx.rope(q, k, c["head_dim"], c["num_heads"], c["num_kv_heads"], 1, L - 1, 0, 10000.0, False)
         nx.reshape_paged_kv(k, pool, [bt[(L - 1) // BLOCK]], [(L - 1) % BLOCK], c["num_kv_heads"], c["head_dim"], BLOCK, False)
         nx.reshape_paged_kv(v, pool, [bt[(L - 1) // BLOCK]], [(L - 1) % BLOCK], c["num_kv_heads"], c["head_dim"], BLOCK, True)
         a = nx.sdpa_paged_decode(q, pool, bt, nb, BLOCK, c["num_heads"], c["num_kv_heads"], c["head_dim"], scale,
                                  L - (nb - 1) * BLOCK).reshape(1, -1)
-        x = nx.add(x, nx.matmul_q4_0(a, w["wo"][0], 1, w["wo"][1], w["wo"][2]))
+        x = nx.add(x, mm(a, "wo"))
         nrm = nx.rmsnorm(x, ones, 1, hd, 1e-5)
-        g = nx.matmul_q4_0(nrm, w["w1"][0], 1, w["w1"][1], w["w1"][2])
-        u = nx.matmul_q4_0(nrm, w["w3"][0], 1, w["w3"][1], w["w3"][2])
-        x = nx.add(x, nx.matmul_q4_0(nx.silu_mul(g, u), w["w2"][0], 1, w["w2"][1], w["w2"][2]))
+        g, u = mm(nrm, "w1"), mm(nrm, "w3")
+        x = nx.add(x, mm(nx.silu_mul(g, u), "w2"))
     t_layers = time.perf_counter() - t0
     t0 = time.perf_counter()
-    nx.matmul_quant(nx.FMT_Q8_0, nx.rmsnorm(x, ones, 1, hd, 1e-5), head, 1, head_rows, hd)
+    rows_parallel(lambda a_, w_, m_, n_, k_: nx.matmul_quant(nx.FMT_Q8_0, a_, w_, m_, n_, k_),
+                  nx.rmsnorm(x, ones, 1, hd, 1e-5), head, head_rows, hd)
     t_head = time.perf_counter() - t0
+    if ex is not None:
+        ex.shutdown()
     per_token = t_layers / sample_layers * c["num_layers"] + t_head / head_rows * c["vocab"]
-    return dict(value=1.0 / per_token, unit="tok/s", cores=1, kind="port",
-                sample="%d of %d layers + %d of %d lm_head rows for one sequence (ctx %d), extrapolated to a full "
-                       "token; host has %d cores, the reference path uses min(cores, M)=1"
-                       % (sample_layers, c["num_layers"], head_rows, c["vocab"], L, os.cpu_count()))
+    what = "%d of %d layers + %d of %d lm_head rows for one sequence (ctx %d), extrapolated to a full token; random " \
+           "bytes stand for the weights (values differ from the GPU run's, the time does not depend on them); " \
+           % (sample_layers, c["num_layers"], head_rows, c["vocab"], L)
+    if threads == 1:
+        what += "host has %d cores, the reference path uses min(cores, M)=1" % os.cpu_count()
+    else:
+        what += "NOT reference behaviour: each matmul's weight rows cut into %d slices run side by side " \
+                "(attention and the element-wise steps on one core)" % threads
+    return dict(value=1.0 / per_token, unit="tok/s", cores=threads, kind="port", sample=what)
+
+
+def time_step_gemms(be, mr, c, rows):
+    """The decode step's four projection launches per layer (Q|K|V, Wo, gate|up, down) at `rows` activation rows,
+    timed with HIP events on the backend's stream over the model's own weights: every layer's matrices once per
+    pass, so each launch streams its weights from HBM as in the step. Algorithmic bytes per launch:
+    N*K*bytes_per_element + rows*K*4 + rows*N*4. -> dict for the bench line."""
+    bpe = {1: 18 / 32, 2: 34 / 32, 3: 144 / 256, 4: 210 / 256}
+    lw = mr.layer_weights
+    h, f = c["hidden"], c["ffn"]
+    rng = np.random.default_rng(9)
+    acts = {k: be.upload(rng.standard_normal((rows, k)).astype(np.float32), permanent=True) for k in {h, f, lw[0]["wo"][3]}}
+
+    def group(names):
+        """(fmt, pointer, total rows, k) of matrices laid out back to back, else None"""
+        ws = [lw[0][n] for n in names]
+        fmt, k = ws[0][0], ws[0][3]
+        per_layer = []
+        for l in lw:
+            p, n = l[names[0]][1], 0
+            for nm in names:
+                if l[nm][1] != p + int(n * k * bpe[fmt]) or l[nm][0] != fmt or l[nm][3] != k:
+                    return None
+                n += l[nm][2]
+            per_layer.append(p)
+        return fmt, per_layer, n, k
+
+    shapes = [("Q|K|V", group(["wq", "wk", "wv"])), ("Wo", group(["wo"])), ("gate|up", group(["w1", "w3"])),
+              ("down", group(["w2"]))]
+    if any(g is None for _, g in shapes):
+        for p in acts.values():
+            be.free(p)
+        return None
+    nmax = max(g[2] for _, g in shapes)
+    out = be.alloc_permanent(rows * nmax * 4)
+    res, total_us, total_bytes = {}, 0.0, 0
+    for name, (fmt, ptrs, n, k) in shapes:
+        be.prepare_act(acts[k], rows, k)
+        for p in ptrs[:2]:
+            be.matmul_quant_prepared(fmt, p, out, None, rows, n, k)
+        be.sync()
+        reps = 3
+        be.timer_start()
+        for _ in range(reps):
+            for p in ptrs:
+                be.matmul_quant_prepared(fmt, p, out, None, rows, n, k)
+        us = be.timer_stop_ms() * 1e3 / (reps * len(ptrs))
+        nbytes = int(n * k * bpe[fmt]) + rows * k * 4 + rows * n * 4
+        res[name] = {"n": n, "k": k, "us": round(us, 2), "bytes": nbytes, "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        total_us += us
+        total_bytes += nbytes
+    be.free(out)
+    for p in acts.values():
+        be.free(p)
+    return {"bound": "hbm", "kernel": "qgemm_wave_kernel (the step's four projection launches per layer, M=%d)" % rows,
+            "achieved": total_bytes / total_us / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": total_bytes / total_us / 1e3 / HBM_PEAK_GBS, "bytes_per_layer": total_bytes,
+            "us_per_layer": total_us, "launches": res,
+            "note": "HIP events around back-to-back launches over all layers' weights; a launch with split K "
+                    "includes its reduction kernel"}
 
 
 def kernel_report(be):
@@ -598,14 +699,21 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "LLaMA-2-7B-shaped Q4_0 (Q8_0 embedding+head), %d layers, %d ragged paged-KV seqs, "
                                "ctx lognormal(median 1024, sigma 0.6) in [64,4096] seed 0, sum ctx %d, block 16, "
-                               "greedy decode, hipGraph=%s" % (args.layers, nseq, sum(ctx_now), use_graph),
+                               "greedy decode, hipGraph=%s; float32 activations enter the batched matmuls as two f16 halves "
+                               "(hi + lo, about 22 significant bits) with float32 accumulation, a single row's "
+                               "matrix-vector products as 22-bit fixed point" % (args.layers, nseq, sum(ctx_now), use_graph),
                    "global_batch": nseq},
         "roofline": {"bound": "hbm", "kernel": "paged_decode_f16_kernel<128,1,1>",
                      "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
                      "traffic": ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE * attn_bytes, "bytes_per_launch": attn_bytes, "ms_per_launch": attn_ms},
     }
+    gm = time_step_gemms(be, mr, c, nseq) if nseq >= 2 else None
+    if gm:
+        out["roofline_matmul"] = gm
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(be, mr, ctx_now, c)
+        out["cpu_baseline_all_cores"] = cpu_baseline(be, mr, ctx_now, c, sample_layers=4, head_rows=8000,
+                                                     threads=min(16, os.cpu_count() or 1))
     mr.close()
     be.close()
     print(json.dumps(out))

@@ -132,13 +132,46 @@ def matmul_t_f32(a, b, m, n, k):
     return out
 
 
+_ROW_THREADS = 1
+_ROW_POOL = None
+
+
+def set_row_threads(n):
+    """Long test runs only: the quantized matmuls cut their weight rows into n slices computed side by side. Every
+    output element is still the same loop over the same numbers in the same order, so the bits do not change;
+    only the wall time does. (The reference itself runs these loops on one core at M = 1.)"""
+    global _ROW_THREADS, _ROW_POOL
+    from concurrent.futures import ThreadPoolExecutor
+    if _ROW_POOL is not None:
+        _ROW_POOL.shutdown()
+        _ROW_POOL = None
+    _ROW_THREADS = max(1, int(n))
+    if _ROW_THREADS > 1:
+        _ROW_POOL = ThreadPoolExecutor(max_workers=_ROW_THREADS)
+
+
+def _rows_parallel(fn, bq, m, n, k, row_bytes):
+    """fn(weight bytes of rows [r0, r1), r1 - r0) -> [m, r1 - r0] on slices of the weight rows"""
+    t = _ROW_THREADS
+    if t <= 1 or n < 4 * t or m * n * k < (1 << 22):
+        return fn(bq, n)
+    rows = _u8(bq).reshape(n, row_bytes)
+    cuts = [n * i // t for i in range(t + 1)]
+    parts = list(_ROW_POOL.map(lambda i: fn(rows[cuts[i]:cuts[i + 1]], cuts[i + 1] - cuts[i]), range(t)))
+    return np.concatenate(parts, axis=1)
+
+
 def matmul_q4_0(a, bq, m, n, k):
     """cpu.go:842-911"""
     a, bq = _f32(a), _u8(bq)
     assert bq.size == n * (k // 32) * 18
-    out = np.empty((m, n), dtype=np.float32)
-    _lib.vxo_matmul_q4_0(_p(a), _p(bq), _p(out), m, n, k)
-    return out
+
+    def run(rows, nr):
+        rows = _u8(rows)
+        out = np.empty((m, nr), dtype=np.float32)
+        _lib.vxo_matmul_q4_0(_p(a), _p(rows), _p(out), m, nr, k)
+        return out
+    return _rows_parallel(run, bq, m, n, k, k // 32 * 18)
 
 
 def matmul_quant(fmt, a, bq, m, n, k):
@@ -149,10 +182,14 @@ def matmul_quant(fmt, a, bq, m, n, k):
         return matmul_q4_0(a, bq, m, n, k)
     a, bq = _f32(a), _u8(bq)
     assert bq.size == n * (k // BLOCK_ELEMS[fmt]) * BLOCK_BYTES[fmt]
-    out = np.empty((m, n), dtype=np.float32)
-    rc = _lib.vxo_matmul_quant_via_dequant(fmt, _p(a), _p(bq), _p(out), m, n, k)
-    assert rc == 0
-    return out
+
+    def run(rows, nr):
+        rows = _u8(rows)
+        out = np.empty((m, nr), dtype=np.float32)
+        rc = _lib.vxo_matmul_quant_via_dequant(fmt, _p(a), _p(rows), _p(out), m, nr, k)
+        assert rc == 0
+        return out
+    return _rows_parallel(run, bq, m, n, k, k // BLOCK_ELEMS[fmt] * BLOCK_BYTES[fmt])
 
 
 def matmul_quant_via_dequant(fmt, a, bq, m, n, k):

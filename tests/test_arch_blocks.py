@@ -17,7 +17,8 @@ PHI = om.ModelConfig(**BASE, norm_type="layer", mlp_type="gelu", parallel_residu
 GEMMA = om.ModelConfig(**BASE, mlp_type="geglu", post_norms=True, attn_softcap=5.0, rope_neox=True,
                        embedding_scale=float(np.float32(math.sqrt(256.0))), eps=1e-6)
 QWEN = om.ModelConfig(**BASE, rope_neox=True, rope_theta=1000000.0)
-ARCHS = {"phi": PHI, "gemma": GEMMA, "qwen": QWEN}
+LLAMA = om.ModelConfig(**BASE)          # the plain layer: RMSNorm, SwiGLU, no biases, interleaved RoPE pairs (2j, 2j+1)
+ARCHS = {"phi": PHI, "gemma": GEMMA, "qwen": QWEN, "llama": LLAMA}
 
 
 def make(name, seed=11):
@@ -126,7 +127,7 @@ class Float64Model:
 
 
 # ---------------------------------------------------------------- checks
-@pytest.mark.parametrize("name", ["phi", "gemma", "qwen"])
+@pytest.mark.parametrize("name", ["phi", "gemma", "qwen", "llama"])
 def test_oracle_block_matches_float64_model(name):
     m = make(name)
     ref = Float64Model(m)
@@ -155,6 +156,23 @@ def test_the_comparison_sees_a_dropped_bias(name, drop):
     prompt = np.random.default_rng(12).integers(0, 300, 19).tolist()
     got = m.prefill_with_paged_kv(prompt, 3, 0)
     want = Float64Model(m, drop=drop).forward(prompt, 0)
+    assert np.abs(got - want).max() > 5e-3 * float(np.abs(want).max())
+
+
+def test_the_comparison_sees_the_rope_pairing_of_the_llama_layer():
+    """The float64 model with split pairs (j, j + D/2) in place of LLaMA's interleaved (2j, 2j+1) is a different
+    function: the llama case above would not pass with the wrong pairing on either side."""
+    import dataclasses
+    m = make("llama")
+    prompt = np.random.default_rng(12).integers(0, 300, 19).tolist()
+    got = m.prefill_with_paged_kv(prompt, 3, 0)
+    wrong = Float64Model(m)
+    wrong.c = dataclasses.replace(m.cfg, rope_neox=True) if dataclasses.is_dataclass(m.cfg) else m.cfg
+    if not dataclasses.is_dataclass(m.cfg):
+        import copy
+        wrong.c = copy.copy(m.cfg)
+        wrong.c.rope_neox = True
+    want = wrong.forward(prompt, 0)
     assert np.abs(got - want).max() > 5e-3 * float(np.abs(want).max())
 
 

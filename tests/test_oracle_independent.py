@@ -538,3 +538,20 @@ def test_greedy_tree_accept_equals_best_linear_path():
     assert hl.verify_tree_path([11, 20], [11, 20, 99]) == (2, 99)
     acc, final = hl.greedy_tree_accept(tokens, parent, 55, [0] * 6)
     assert acc == [] and final == 55
+
+
+@pytest.mark.parametrize("fmt", [nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q6_K])
+def test_row_sliced_matmul_has_the_same_bits(fmt):
+    """set_row_threads() cuts the weight rows into slices computed side by side (long GPU parity runs use it to
+    shorten the oracle's share): every output element is the same loop, so the result is bit-identical."""
+    rng = np.random.default_rng(300 + fmt)
+    m, n, k = 3, 1536, 1024
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    one = nx.matmul_quant(fmt, a, w, m, n, k)
+    nx.set_row_threads(5)
+    try:
+        cut = nx.matmul_quant(fmt, a, w, m, n, k)
+    finally:
+        nx.set_row_threads(1)
+    assert np.array_equal(one.view(np.uint32), cut.view(np.uint32))

@@ -2021,13 +2021,27 @@ static bool group_ok(const vx_qweight *const *ws, int nw) {
     return true;
 }
 
+// Matrices that follow one another in memory (a loader that lays Q|K|V or gate|up out back to back) become one
+// segment: the kernels then cut the rows where they like instead of at the matrices' boundaries.
 static Segs make_segs(const vx_qweight *const *ws, int nw, int *ntot) {
     Segs sg;
-    int acc = 0;
-    for (int i = 0; i < 3; i++) {
-        const vx_qweight *w = ws[i < nw ? i : nw - 1];
-        if (i < nw) acc += w->n;
-        sg.w[i] = (const uint8_t *)w->data;
+    int acc = 0, ns = 0;
+    const uint8_t *next = nullptr;  // where a matrix would have to start to continue the current segment
+    for (int i = 0; i < nw; i++) {
+        const vx_qweight *w = ws[i];
+        const uint8_t *p = (const uint8_t *)w->data;
+        acc += w->n;
+        if (ns > 0 && p == next) {
+            sg.n_end[ns - 1] = acc;
+        } else {
+            sg.w[ns] = p;
+            sg.n_end[ns] = acc;
+            ns++;
+        }
+        next = p + (size_t)w->n * fmt_row_bytes(w->fmt, w->k);
+    }
+    for (int i = ns; i < 3; i++) {  // unused slots repeat the last segment
+        sg.w[i] = sg.w[ns - 1];
         sg.n_end[i] = acc;
     }
     *ntot = acc;

@@ -241,11 +241,24 @@ class ModelRuntime:
         lw = VhLayerWeights()
         lw.attn_norm = attn_norm if isinstance(attn_norm, int) else self._up(np.asarray(attn_norm, dtype=np.float32))
         lw.ffn_norm = ffn_norm if isinstance(ffn_norm, int) else self._up(np.asarray(ffn_norm, dtype=np.float32))
+        ptrs = {}
+        # matrices that one launch multiplies together go into one device buffer, back to back, when they come
+        # from the host in one format and width: the kernels then see a single row range
+        for group in (("wq", "wk", "wv"), ("w1", "w3")):
+            ws = [weights.get(n_) for n_ in group]
+            if all(w is not None and not isinstance(w[1], int) for w in ws) and len({(w[0], w[3]) for w in ws}) == 1:
+                rows = [np.ascontiguousarray(w[1]).reshape(w[2], -1) for w in ws]
+                if len({r.shape[1] for r in rows}) == 1 and rows[0].shape[1] % 16 == 0:
+                    base = self._up(np.concatenate(rows, axis=0))
+                    off = 0
+                    for n_, r in zip(group, rows):
+                        ptrs[n_] = base + off
+                        off += r.nbytes
         for name in ("wq", "wk", "wv", "wo", "w1", "w2", "w3"):
             if weights.get(name) is None:          # w3 of a GELU MLP
                 continue
             fmt, data, n, k = weights[name]
-            ptr = data if isinstance(data, int) else self._up(data)
+            ptr = ptrs.get(name) or (data if isinstance(data, int) else self._up(data))
             setattr(lw, name, VhQWeight(fmt, ptr, n, k))
         self._ck(self._h.vh_model_set_layer(self._m, layer, C.byref(lw)))
 
