@@ -314,6 +314,15 @@ int vx_sdpa_paged_tree_batched(vx_backend *be, const float *q, const void *kv_po
                                const int32_t *mask_offsets, float *out, int rows, int max_tree_rows,
                                int num_q_heads, int num_kv_heads, int head_dim, float scale, int max_kv_len);
 
+/* Copies num_tokens token rows (K and V of every KV head) from src_slots[i] to dst_slots[i] of one layer's paged
+ * pool (device int32 arrays, slot = physical block * block_size + offset; the two sets must not overlap) and
+ * rotates the K rows by the angle of position `shift` on the way: RoPEShift (backend/cpu/backend.go:244-276,
+ * interleaved pairs) applied where the reference applies it to a gathered copy when it reads a cached fragment
+ * (kv/paged_cache.go:225-283). An F16 pool keeps the rotated K rounded to half precision. shift 0 is a plain copy. */
+int vx_paged_kv_copy_shifted(vx_backend *be, void *kv_pool, int pool_is_f16, const int32_t *src_slots,
+                             const int32_t *dst_slots, int num_tokens, int num_kv_heads, int head_dim, int block_size,
+                             int shift, float theta);
+
 /* Moves token rows (K and V of every KV head) inside one layer's paged pool: slot = physical block *
  * block_size + offset in the block. Chain c is the moves chain_offsets[c] .. chain_offsets[c+1]-1 (device
  * int32 arrays), applied in order, so a later move of a chain may read what an earlier one wrote; different

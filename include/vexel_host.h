@@ -99,6 +99,23 @@ int vh_pool_truncate_sequence(vh_model *m, int64_t seq_id, int new_len);        
 int vh_pool_has_sequence(vh_model *m, int64_t seq_id);                          /* :193 */
 int vh_pool_share_blocks(vh_model *m, int64_t src, int64_t dst, int num_tokens);/* :572 */
 void vh_pool_block_stats(vh_model *m, int *total, int *free_blocks, int *shared);/* :610 (per layer x numLayers) */
+/* Named fragments (kv/fragment.go:18-101, kv/paged_cache.go:285-343): the K/V of a finished sequence kept under a
+ * name and put at the end of other sequences without running the model over those tokens again.
+ *   vh_fragment_cache   PagedKVCache.CacheContent: the sequence's blocks get one more reference each and stay alive
+ *                       after the sequence is deleted; a fragment of the same name is released first; an unknown
+ *                       sequence caches nothing.
+ *   vh_fragment_insert  PagedKVCache.InsertFragment: *num_tokens = tokens added (0 and VH_OK for an unknown name;
+ *                       an unknown sequence is created). insert_pos must be the sequence's length. The reference
+ *                       shares the blocks and rotates K by insert_pos at every read; here the rows are copied once
+ *                       into the sequence's own blocks with K rotated (vx_paged_kv_copy_shifted), so attention reads
+ *                       the pool as it is.
+ *   vh_fragment_delete  FragmentCache.Delete; vh_fragment_tokens: CachedFragment.NumTokens or -1;
+ *   vh_fragment_count   len(FragmentCache.List()). */
+int vh_fragment_cache(vh_model *m, const char *name, int64_t seq_id);
+int vh_fragment_insert(vh_model *m, int64_t seq_id, const char *name, int insert_pos, int *num_tokens);
+int vh_fragment_delete(vh_model *m, const char *name);
+int vh_fragment_tokens(vh_model *m, const char *name);
+int vh_fragment_count(vh_model *m);
 int vh_pool_seq_len(vh_model *m, int64_t seq_id);
 /* copies the sequence's block table (identical for every layer) into out; returns its length or -1 */
 int vh_pool_block_table(vh_model *m, int64_t seq_id, int32_t *out, int cap);

@@ -163,6 +163,35 @@ class GPUBlockPool:
         if num_tokens > dst.seq_len:
             dst.seq_len = num_tokens
 
+    # ---- named fragments: kv/fragment.go:18-101 and kv/paged_cache.go:285-343 over this pool's counters
+    def cache_content(self, name, seq_id):
+        """PagedKVCache.CacheContent: the sequence's blocks, one more reference each; replaces a fragment of that name."""
+        seq = self.seqs.get(seq_id)
+        if seq is None:
+            return None                                       # paged_cache.go:331-333
+        frags = self.__dict__.setdefault("fragments", {})
+        if name in frags:                                     # fragment.go:41-43
+            self._release_fragment(frags.pop(name))
+        blocks = [list(bt) for bt in seq.block_tables]
+        for layer in range(self.num_layers):
+            for b in blocks[layer]:                           # fragment.go:46-50
+                self.ref_counts[layer][b] = self.ref_counts[layer].get(b, 0) + 1
+        frags[name] = (seq.seq_len, blocks)
+        return frags[name]
+
+    def _release_fragment(self, frag):                        # fragment.go:83-89
+        for layer, blocks in enumerate(frag[1]):
+            for b in blocks:
+                self._release(layer, b)
+
+    def delete_fragment(self, name):                          # fragment.go:71-79
+        frags = self.__dict__.setdefault("fragments", {})
+        if name in frags:
+            self._release_fragment(frags.pop(name))
+
+    def fragment(self, name):                                 # fragment.go:63-68
+        return self.__dict__.setdefault("fragments", {}).get(name)
+
     # gpu_block_pool.go:610-624
     def block_stats(self):
         total = self.max_blocks * self.num_layers

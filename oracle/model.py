@@ -280,6 +280,36 @@ class OracleModel:
             x = self._execute_tree_layer(x, seq_id, i, start_pos, positions, mask)
         return self._head(x, rows)
 
+    def insert_fragment(self, seq_id, name, insert_pos):
+        """PagedKVCache.InsertFragment (kv/paged_cache.go:285-322) with the read-time RoPE shift of
+        GetKVSliceForAttention (:225-283) done once, at insertion: the fragment's token rows go to positions
+        insert_pos.. of the sequence, K rotated by RoPEShift(insert_pos) (backend/cpu/backend.go:244-276) and, in
+        an F16 pool, rounded to half precision again; V as it is. -> tokens inserted (0 for an unknown name)."""
+        c, pool = self.cfg, self.pool
+        frag = pool.fragment(name)
+        if frag is None:
+            return 0
+        if not pool.has_sequence(seq_id):
+            pool.create_sequence(seq_id)
+        st = pool.seqs[seq_id]
+        assert insert_pos == st.seq_len, "a fragment goes to the end of the sequence"
+        n, blocks = frag
+        row = c.num_kv_heads * c.head_dim
+        blk = 2 * c.block_size * row                                       # gpu_block_pool.go:107-108
+        for layer in range(c.num_layers if n > 0 else 0):
+            slots = pool.store_kv_slots(layer, seq_id, insert_pos, n)      # the blocks StoreKV would take, :234-252
+            for t in range(n):
+                src = blocks[layer][t // c.block_size] * blk + (t % c.block_size) * row
+                dst = slots[t][0] * blk + slots[t][1] * row
+                k = self.kv[layer][src:src + row]
+                kf = nx.f16_to_f32_array(k) if pool.use_fp16 else k.astype(np.float32)
+                kf = nx.rope_shift(kf, c.head_dim, c.num_kv_heads, 1, insert_pos, c.rope_theta).reshape(-1)
+                self.kv[layer][dst:dst + row] = nx.f32_to_f16_array(kf) if pool.use_fp16 else kf
+                v0, v1 = src + c.block_size * row, dst + c.block_size * row
+                self.kv[layer][v1:v1 + row] = self.kv[layer][v0:v0 + row].copy()
+        st.seq_len = insert_pos + n
+        return n
+
     def _move_kv_row(self, layer, seq_id, src_pos, dst_pos):
         c = self.cfg
         bt = self.pool.seqs[seq_id].block_tables[layer]

@@ -619,6 +619,116 @@ def test_batched_greedy_64_steps_7b_geometry_32_sequences(be):
     mr.close()
 
 
+def test_prefix_sharing_decodes_over_shared_blocks(be):
+    """gpu_block_pool.go:568-607 end to end: sequence B takes the first two blocks of A's prompt by reference,
+    prefills only the rest, and both decode. B's logits are those of a sequence that prefilled the whole prompt in
+    the same two pieces (the second piece reads the f16 pool either way, runtime/block.go:875-895); the shared
+    blocks survive A's deletion and B keeps decoding over them; oracle and device agree on tables and counts."""
+    cfg = om.ModelConfig(num_layers=2, hidden=512, num_heads=8, num_kv_heads=2, head_dim=64, ffn=1024, vocab=1024)
+    omodel = om.random_model(cfg, 91, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=40)
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=40, max_seqs=8, max_blocks_per_seq=8, max_batch=64)
+    rng = np.random.default_rng(92)
+    prompt = rng.integers(0, cfg.vocab, 45).tolist()
+    A, B, Cq = 1, 2, 3
+    for sid in (A, B, Cq):
+        omodel.pool.create_sequence(sid)
+        mr.create_sequence(sid)
+    assert_logits_close(mr.prefill_with_paged_kv(prompt, A, 0), omodel.prefill_with_paged_kv(prompt, A, 0), "A")
+    omodel.pool.share_blocks(A, B, 32)
+    mr.share_blocks(A, B, 32)
+    assert mr.block_stats() == omodel.pool.block_stats() and mr.block_stats()[2] == 2 * cfg.num_layers
+    wb = omodel.prefill_with_paged_kv(prompt[32:], B, 32)
+    gb = mr.prefill_with_paged_kv(prompt[32:], B, 32)
+    assert_logits_close(gb, wb, "B after the shared prefix")
+    assert mr.block_table(B)[:2] == mr.block_table(A)[:2] == omodel.pool.seqs[A].block_tables[0][:2]
+    # a sequence that computes the same prompt itself, in the same two pieces
+    mr.prefill_with_paged_kv(prompt[:32], Cq, 0)
+    gc = mr.prefill_with_paged_kv(prompt[32:], Cq, 32)
+    assert np.abs(gb - gc).max() <= 1e-5 * np.abs(gc).max()
+    mr.delete_sequence(Cq)
+    omodel.pool.delete_sequence(Cq)
+    # both decode, then A goes away and B goes on over the blocks it shares no longer with anyone
+    toks, pos = [7, nx.argmax(wb)], [45, 45]
+    for step in range(3):
+        want = omodel.decode_batched(toks, [A, B], pos)
+        got, am = mr.decode_with_paged_kv_batched(toks, [A, B], pos)
+        assert_logits_close(got, want, "shared decode %d" % step)
+        toks = [nx.argmax(want[i]) for i in range(2)]
+        assert toks == [int(a) for a in am]
+        pos = [p + 1 for p in pos]
+    omodel.pool.delete_sequence(A)
+    mr.delete_sequence(A)
+    assert mr.block_stats() == omodel.pool.block_stats() and mr.block_stats()[2] == 0
+    for step in range(3):
+        want = omodel.decode_batched(toks[1:], [B], pos[1:])
+        got, am = mr.decode_with_paged_kv_batched(toks[1:], [B], pos[1:])
+        assert_logits_close(got, want, "B alone %d" % step)
+        toks = [toks[0], nx.argmax(want[0])]
+        assert toks[1] == int(am[0])
+        pos = [p + 1 for p in pos]
+    assert mr.block_table(B) == omodel.pool.seqs[B].block_tables[0]
+    mr.close()
+
+
+@pytest.mark.parametrize("kv_f16", [True, False])
+def test_fragment_cache_insert_with_rope_shift(be, kv_f16):
+    """kv/fragment.go + kv/paged_cache.go:285-343: a prefilled document is cached under a name, its sequence
+    deleted; two other sequences put it behind prompts of different lengths (K rotated by 13 and by 32 positions on
+    insertion, V copied) and decode. Pool contents are compared bit for bit with the oracle's (same float32
+    operations, same rounding to the pool's type), logits within the usual tolerance, tables and counts exactly."""
+    cfg = om.ModelConfig(num_layers=2, hidden=512, num_heads=8, num_kv_heads=2, head_dim=64, ffn=1024, vocab=1024)
+    omodel = om.random_model(cfg, 93, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=48, kv_fp16=kv_f16)
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=48, max_seqs=8, max_blocks_per_seq=8, max_batch=64)
+    rng = np.random.default_rng(94)
+    # the document's K/V: the same values on both sides (a prefill would leave last-bit differences between the two
+    # implementations in the source rows, and the comparison below is exact)
+    install_context(omodel, mr, be, 1, [5, 9, 2], 37, rng)
+    omodel.pool.cache_content("doc", 1)
+    mr.cache_fragment("doc", 1)
+    omodel.pool.delete_sequence(1)
+    mr.delete_sequence(1)
+    assert mr.fragment_tokens("doc") == 37 and mr.fragment_count() == 1 and mr.fragment_tokens("other") == -1
+    assert mr.block_stats() == omodel.pool.block_stats()
+    per_block = 2 * cfg.block_size * cfg.num_kv_heads * cfg.head_dim
+    esz, dt = (2, np.uint16) if kv_f16 else (4, np.float32)
+    for sid, plen in ((2, 13), (3, 32)):
+        head = rng.integers(0, cfg.vocab, plen).tolist()
+        omodel.pool.create_sequence(sid)
+        mr.create_sequence(sid)
+        assert_logits_close(mr.prefill_with_paged_kv(head, sid, 0), omodel.prefill_with_paged_kv(head, sid, 0), "head")
+        assert omodel.insert_fragment(sid, "doc", plen) == 37
+        assert mr.insert_fragment(sid, "doc", plen) == 37
+        assert mr.seq_len(sid) == plen + 37 == omodel.pool.seqs[sid].seq_len
+        assert mr.block_table(sid) == omodel.pool.seqs[sid].block_tables[0]
+        row = cfg.num_kv_heads * cfg.head_dim
+        for layer in range(cfg.num_layers):        # the inserted rows, K and V, bit for bit
+            for b in set(mr.block_table(sid)[plen // 16:]):
+                got = be.download(mr.kv_pool(layer) + b * per_block * esz, (per_block,), dt)
+                want = np.ascontiguousarray(omodel.kv[layer][b * per_block:(b + 1) * per_block])
+                lb = mr.block_table(sid).index(b)
+                for off in range(16):
+                    if plen <= lb * 16 + off < plen + 37:
+                        for base in (off * row, 16 * row + off * row):
+                            assert np.array_equal(got[base:base + row].view(np.uint8), want[base:base + row].view(np.uint8)), \
+                                (sid, layer, b, off)
+        tok, pos = 5, plen + 37
+        for step in range(3):
+            want = omodel.decode_with_paged_kv(tok, sid, pos)
+            got, am = mr.decode_with_paged_kv_batched([tok], [sid], [pos])
+            assert_logits_close(got[0], want, "decode after the fragment %d" % step)
+            tok = nx.argmax(want)
+            assert tok == int(am[0])
+            pos += 1
+    assert mr.insert_fragment(2, "no such fragment", mr.seq_len(2)) == 0
+    from vexel_amd.backend import VexelError
+    with pytest.raises(VexelError, match="end of sequence"):
+        mr.insert_fragment(2, "doc", 3)
+    omodel.pool.delete_fragment("doc")
+    mr.delete_fragment("doc")
+    assert mr.fragment_count() == 0 and mr.block_stats() == omodel.pool.block_stats()
+    mr.close()
+
+
 def test_pool_errors_and_lifecycle(be):
     """Host-forced failure paths: pool exhaustion, unknown sequence, truncate no-ops."""
     from vexel_amd.backend import VexelError

@@ -555,3 +555,65 @@ def test_row_sliced_matmul_has_the_same_bits(fmt):
     finally:
         nx.set_row_threads(1)
     assert np.array_equal(one.view(np.uint32), cut.view(np.uint32))
+
+
+# ----------------------------------------------------------------- named fragments
+def test_fragment_cache_reference_counts_by_hand():
+    """kv/fragment.go:36-89 and kv/paged_cache.go:285-343 on the pool's counters, worked by hand for a 4-block
+    pool of block size 4: caching adds one reference per block and keeps the blocks alive after the sequence is
+    gone; a second fragment of the same name releases the first; deleting the last holder frees the blocks."""
+    p = hl.GPUBlockPool(num_layers=2, num_kv_heads=1, head_dim=2, block_size=4, max_blocks=4)
+    p.create_sequence(1)
+    p.store_kv_slots(0, 1, 0, 6), p.store_kv_slots(1, 1, 0, 6)       # two blocks per layer: 3 and 2 (tail first)
+    assert p.seqs[1].block_tables == [[3, 2], [3, 2]]
+    assert p.cache_content("sys", 1) == (6, [[3, 2], [3, 2]])
+    assert p.ref_counts[0] == {3: 2, 2: 2} and p.block_stats() == (8, 4, 4)
+    p.delete_sequence(1)                                             # the fragment still holds them
+    assert p.ref_counts[0] == {3: 1, 2: 1} and p.block_stats() == (8, 4, 0)
+    assert p.cache_content("nobody", 99) is None                     # an unknown sequence caches nothing
+    p.create_sequence(2)
+    p.store_kv_slots(0, 2, 0, 3), p.store_kv_slots(1, 2, 0, 3)       # block 1
+    p.cache_content("sys", 2)                                        # same name: blocks 3 and 2 go back to the pool
+    assert p.fragment("sys") == (3, [[1], [1]])
+    assert p.free_lists[0] == [0, 3, 2] and p.ref_counts[0] == {1: 2}
+    p.delete_fragment("sys")
+    p.delete_sequence(2)
+    assert p.free_lists[0] == [0, 3, 2, 1] and p.ref_counts == [{}, {}] and p.fragment("sys") is None
+
+
+def test_fragment_inserted_at_p_holds_the_keys_of_positions_p_onward():
+    """What the shift has to achieve, checked without the shift code: in layer 0 a token's K before RoPE depends on
+    the token alone, so a fragment of tokens F cached from positions 0..n-1 and inserted at position p must leave,
+    in layer 0, the K rows that a prefill of the same tokens at positions p..p+n-1 computes (to the half-precision
+    rounding of rotating an already rounded row), and V rows that are bit-identical."""
+    from oracle import model as om
+    cfg = om.ModelConfig(num_layers=2, hidden=128, num_heads=4, num_kv_heads=2, head_dim=32, ffn=256, vocab=200)
+    m = om.random_model(cfg, 17, nx.FMT_Q8_0, nx.FMT_Q8_0, max_blocks=24)
+    rng = np.random.default_rng(18)
+    frag, head = rng.integers(0, 200, 21).tolist(), rng.integers(0, 200, 11).tolist()
+    m.pool.create_sequence(1)
+    m.prefill_with_paged_kv(frag, 1, 0)
+    m.pool.cache_content("doc", 1)
+    m.pool.delete_sequence(1)
+    m.pool.create_sequence(2)
+    m.prefill_with_paged_kv(head, 2, 0)
+    assert m.insert_fragment(2, "doc", 11) == 21 and m.pool.seqs[2].seq_len == 32
+    assert m.insert_fragment(2, "no such name", 32) == 0
+    m.pool.create_sequence(3)                                        # the same 32 tokens computed in place
+    m.prefill_with_paged_kv(head + frag, 3, 0)
+    row, bs = cfg.num_kv_heads * cfg.head_dim, cfg.block_size
+    blk = 2 * bs * row
+
+    def rows(seq, pos, v):
+        bt = m.pool.seqs[seq].block_tables[0]
+        o = bt[pos // bs] * blk + (bs * row if v else 0) + (pos % bs) * row
+        return nx.f16_to_f32_array(m.kv[0][o:o + row])
+    for pos in range(11, 32):
+        assert np.array_equal(rows(2, pos, True), rows(3, pos, True))                 # V: position-free in layer 0
+        k_ins, k_ref = rows(2, pos, False), rows(3, pos, False)
+        assert np.abs(k_ins - k_ref).max() <= 2.5e-3 * np.abs(k_ref).max() + 1e-4    # two half-precision roundings
+    # the rotation really happened: the unshifted rows are far from the reference
+    m.pool.create_sequence(4)
+    m.prefill_with_paged_kv(frag, 4, 0)
+    far = max(np.abs(rows(4, t, False) - rows(3, 11 + t, False)).max() for t in range(21))
+    assert far > 0.1 * max(np.abs(rows(3, 11 + t, False)).max() for t in range(21))

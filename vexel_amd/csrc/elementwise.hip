@@ -535,6 +535,45 @@ __global__ void move_paged_kv_kernel(uint32_t *pool, const int32_t *chain_offset
     }
 }
 
+
+// Copies token rows between slots of one layer's paged pool (K and V of every KV head); the K rows are rotated by
+// the angle of position `shift` on the way (interleaved pairs), which turns RoPE(p) into RoPE(p + shift):
+// backend/cpu/backend.go:244-276 applied to pool rows. cs: [head_dim/2] (cos, sin) pairs of the shift, worked out
+// on the host in the reference's precision chain. The products are rounded before they are added, as the
+// reference's separate float32 operations are. grid = tokens, block = 256.
+template <typename T>
+__global__ void __launch_bounds__(256) copy_shift_paged_kv_kernel(T *pool, const int32_t *__restrict__ src_slots,
+                                                                  const int32_t *__restrict__ dst_slots,
+                                                                  const float2 *__restrict__ cs, int num_kv_heads,
+                                                                  int head_dim, int block_size, int rotate) {
+    const int i = blockIdx.x;
+    const int s = src_slots[i], d = dst_slots[i];
+    const int row = num_kv_heads * head_dim, half = head_dim / 2;
+    const size_t part = (size_t)block_size * row;
+    const T *ks = pool + (size_t)(s / block_size) * 2 * part + (size_t)(s % block_size) * row;
+    T *kd = pool + (size_t)(d / block_size) * 2 * part + (size_t)(d % block_size) * row;
+    for (int p = threadIdx.x; p < num_kv_heads * half; p += blockDim.x) {
+        const int h = p / half, j = p % half;
+        const float v1 = (float)ks[h * head_dim + 2 * j], v2 = (float)ks[h * head_dim + 2 * j + 1];
+        float o1 = v1, o2 = v2;
+        if (rotate) {
+            const float2 c = cs[j];
+            // Every product and every sum has to exist as a rounded float32 of its own, as in the reference's
+            // separate operations: left alone, the compiler fuses a product into the sum, and the sum into the
+            // conversion to half precision (one mixed-precision instruction that rounds once, from the unrounded
+            // sum, and lands on the other side of a tie now and then).
+            float p1 = v1 * c.x, p2 = v2 * c.y, p3 = v1 * c.y, p4 = v2 * c.x;
+            asm volatile("" : "+v"(p1), "+v"(p2), "+v"(p3), "+v"(p4));
+            o1 = p1 - p2;
+            o2 = p3 + p4;
+            asm volatile("" : "+v"(o1), "+v"(o2));
+        }
+        kd[h * head_dim + 2 * j] = (T)o1;
+        kd[h * head_dim + 2 * j + 1] = (T)o2;
+    }
+    for (int e = threadIdx.x; e < row; e += blockDim.x) kd[part + e] = ks[part + e];  // the V row, as it is
+}
+
 inline int grid1d(int64_t n, int threads) { return (int)((n + threads - 1) / threads); }
 
 }  // namespace
@@ -574,6 +613,45 @@ int vx_rope_shift(vx_backend *be, float *k, int head_dim, int num_kv_heads, int 
     int threads = head_dim / 2 < 64 ? 64 : (head_dim / 2 > 256 ? 256 : head_dim / 2);
     rope_kernel<<<num_tokens, threads, 0, be->stream>>>(nullptr, k, head_dim, 0, num_kv_heads, shift, head_dim, theta, 0,
                                                          nullptr, 0);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_paged_kv_copy_shifted(vx_backend *be, void *kv_pool, int pool_is_f16, const int32_t *src_slots,
+                             const int32_t *dst_slots, int num_tokens, int num_kv_heads, int head_dim, int block_size,
+                             int shift, float theta) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(kv_pool && src_slots && dst_slots && num_tokens >= 0, "vx_paged_kv_copy_shifted: bad arguments");
+    VX_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && num_kv_heads > 0 && block_size > 0, "vx_paged_kv_copy_shifted: bad shape");
+    if (num_tokens == 0) return VX_OK;
+    const int half = head_dim / 2;
+    VX_REQUIRE((size_t)half * sizeof(float2) <= be->host_stage_bytes && (size_t)half * sizeof(float2) <= be->misc_ws_bytes,
+               "vx_paged_kv_copy_shifted: head_dim %d too large", head_dim);
+    if (shift != 0) {
+        // the table must not change under a copy still in flight from the call before
+        VX_CHECK_HIP(hipStreamSynchronize(be->stream));
+        float2 *t = (float2 *)be->host_stage;
+        for (int j = 0; j < half; j++) {                       // backend/cpu/backend.go:262-266
+            const double ex = (double)(2 * j) / (double)head_dim;
+            const float freq = (float)(1.0 / pow((double)theta, ex));
+            const float angle = (float)shift * freq;
+            // through volatile doubles: the compiler may otherwise shrink (float)cos((double)x) to cosf(x), whose
+            // last bit is not the correctly rounded double result's
+            volatile double cd = cos((double)angle), sd = sin((double)angle);
+            t[j] = make_float2((float)cd, (float)sd);
+        }
+        VX_CHECK_HIP(hipMemcpyAsync(be->misc_ws, t, (size_t)half * sizeof(float2), hipMemcpyHostToDevice, be->stream));
+        VX_CHECK_HIP(hipStreamSynchronize(be->stream));        // the staging buffer is free again for the next caller
+    }
+    if (pool_is_f16)
+        copy_shift_paged_kv_kernel<_Float16><<<num_tokens, 256, 0, be->stream>>>((_Float16 *)kv_pool, src_slots, dst_slots,
+                                                                                 (const float2 *)be->misc_ws, num_kv_heads,
+                                                                                 head_dim, block_size, shift != 0);
+    else
+        copy_shift_paged_kv_kernel<float><<<num_tokens, 256, 0, be->stream>>>((float *)kv_pool, src_slots, dst_slots,
+                                                                              (const float2 *)be->misc_ws, num_kv_heads,
+                                                                              head_dim, block_size, shift != 0);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }

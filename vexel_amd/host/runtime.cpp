@@ -24,6 +24,7 @@
 #include <algorithm>
 #include <map>
 #include <mutex>
+#include <string>
 #include <unordered_map>
 #include <vector>
 
@@ -58,8 +59,14 @@ struct SeqState {
     bool dirty = true;           // device row differs from `table`
 };
 
+struct Fragment {                 // kv/fragment.go:9-16
+    int num_tokens = 0;
+    std::vector<int32_t> blocks;  // the cached sequence's table (the same for every layer), one reference each
+};
+
 struct BlockPool {
     int block_size = 16, max_blocks = 0;
+    std::map<std::string, Fragment> fragments;    // kv/fragment.go:19-23
     std::vector<int32_t> free_list;               // gpu_block_pool.go:110-116
     std::unordered_map<int32_t, int> ref_counts;  // gpu_block_pool.go:42-43
     std::map<int64_t, SeqState> seqs;
@@ -668,6 +675,100 @@ int vh_pool_share_blocks(vh_model *m, int64_t src_id, int64_t dst_id, int num_to
     }
     dst->dirty = true;
     if (num_tokens > dst->seq_len) dst->seq_len = num_tokens;
+    return VH_OK;
+}
+
+// ------------------------------------------------------------------ named fragments (kv/fragment.go, kv/paged_cache.go:285-343)
+static void release_fragment(vh_model *m, const Fragment &f) {  // fragment.go:83-89
+    for (int32_t b : f.blocks) m->pool.release_block(b);
+}
+
+int vh_fragment_cache(vh_model *m, const char *name, int64_t seq_id) {  // paged_cache.go:324-343, fragment.go:36-60
+    if (!m || !name) return fail("bad arguments");
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    SeqState *s = find_seq(m, seq_id);
+    if (!s) return VH_OK;  // paged_cache.go:331-333: an unknown sequence caches nothing
+    auto old = m->pool.fragments.find(name);
+    if (old != m->pool.fragments.end()) {  // fragment.go:41-43: a fragment of that name gives its blocks back first
+        release_fragment(m, old->second);
+        m->pool.fragments.erase(old);
+    }
+    Fragment f;
+    f.num_tokens = s->seq_len;
+    f.blocks = s->table;
+    for (int32_t b : f.blocks) m->pool.ref_counts[b]++;  // fragment.go:46-50 (AddRef)
+    m->pool.fragments[name] = f;
+    return VH_OK;
+}
+
+int vh_fragment_tokens(vh_model *m, const char *name) {  // fragment.go:63-68; -1: no such fragment
+    if (!m || !name) return -1;
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    auto it = m->pool.fragments.find(name);
+    return it == m->pool.fragments.end() ? -1 : it->second.num_tokens;
+}
+
+int vh_fragment_count(vh_model *m) {  // fragment.go:92-101
+    if (!m) return 0;
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    return (int)m->pool.fragments.size();
+}
+
+int vh_fragment_delete(vh_model *m, const char *name) {  // fragment.go:71-79
+    if (!m || !name) return fail("bad arguments");
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    auto it = m->pool.fragments.find(name);
+    if (it == m->pool.fragments.end()) return VH_OK;
+    release_fragment(m, it->second);
+    m->pool.fragments.erase(it);
+    return VH_OK;
+}
+
+// The reference shares the fragment's blocks with the sequence and rotates K by insert_pos every time it reads
+// them (paged_cache.go:225-283). Here the rotation happens once, at insertion: the fragment's rows are copied
+// into the sequence's own blocks with K turned by insert_pos, so the attention kernels read the pool as it is and
+// the fragment's blocks stay untouched for the next insertion at another position.
+int vh_fragment_insert(vh_model *m, int64_t seq_id, const char *name, int insert_pos, int *num_tokens) {
+    if (num_tokens) *num_tokens = 0;
+    if (!m || !name || insert_pos < 0) return fail("bad arguments");
+    const vh_config &c = m->cfg;
+    if (m->arch.rope_neox || (m->arch.rope_dim != 0 && m->arch.rope_dim != c.head_dim))
+        return fail("fragments are rotated as RoPEShift rotates (whole head, pairs 2j and 2j+1): not this model's RoPE");
+    std::lock_guard<std::mutex> g(m->pool.mu);
+    auto it = m->pool.fragments.find(name);
+    if (it == m->pool.fragments.end()) return VH_OK;  // paged_cache.go:290-293: nothing to insert
+    SeqState *s = find_seq(m, seq_id);
+    if (!s) {  // paged_cache.go:296-300: the sequence comes into being
+        VHC(create_seq_locked(m, seq_id));
+        s = find_seq(m, seq_id);
+    }
+    if (insert_pos != s->seq_len)
+        return fail("fragment \"%s\" can only go to the end of sequence %lld (length %d), not to position %d", name,
+                    (long long)seq_id, s->seq_len, insert_pos);
+    const Fragment &f = it->second;
+    const int n = f.num_tokens, bs = m->pool.block_size;
+    if ((insert_pos + n - 1) / bs + 1 > c.max_blocks_per_seq && n > 0)
+        return fail("sequence %lld: %d tokens at position %d exceed max_blocks_per_seq %d", (long long)seq_id, n, insert_pos,
+                    c.max_blocks_per_seq);
+    VHC(m->pool.ensure_blocks(*s, insert_pos + n));
+    if (n > 0) {
+        std::vector<int32_t> slots(2 * (size_t)n);
+        for (int t = 0; t < n; t++) {
+            slots[t] = f.blocks[t / bs] * bs + t % bs;
+            const int p = insert_pos + t;
+            slots[n + t] = s->table[p / bs] * bs + p % bs;
+        }
+        int32_t *d_slots = (int32_t *)vx_alloc(m->be, slots.size() * 4);
+        if (!d_slots) return fail("vx_alloc: %s", vx_last_error());
+        VXC(vx_to_device(m->be, d_slots, slots.data(), slots.size() * 4));
+        for (int l = 0; l < c.num_layers; l++)
+            VXC(vx_paged_kv_copy_shifted(m->be, m->kv[l], c.kv_fp16, d_slots, d_slots + n, n, c.num_kv_heads, c.head_dim, bs,
+                                         insert_pos, c.rope_theta));
+        VXC(vx_sync(m->be));
+    }
+    s->seq_len = insert_pos + n;  // paged_cache.go:316-319
+    s->dirty = true;
+    if (num_tokens) *num_tokens = n;
     return VH_OK;
 }
 

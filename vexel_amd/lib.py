@@ -91,6 +91,7 @@ SIGNATURES = {
     "vx_sdpa_paged_tree_batched": (_i, [_vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),
     "vx_rope_shift": (_i, [_vp, _vp, _i, _i, _i, _i, _f]),
     "vx_sample_rows": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+    "vx_paged_kv_copy_shifted": (_i, [_vp, _vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _f]),
     "vx_paged_kv_move": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i]),
     "vx_pack_batch": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "vx_decode_advance": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _i]),

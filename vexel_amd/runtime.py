@@ -84,6 +84,11 @@ def load_host():
             getattr(h, name).argtypes = [C.c_void_p, C.c_int64]
         h.vh_pool_truncate_sequence.argtypes = [C.c_void_p, C.c_int64, C.c_int]
         h.vh_pool_share_blocks.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_int]
+        h.vh_fragment_cache.argtypes = [C.c_void_p, C.c_char_p, C.c_int64]
+        h.vh_fragment_insert.argtypes = [C.c_void_p, C.c_int64, C.c_char_p, C.c_int, C.POINTER(C.c_int)]
+        h.vh_fragment_delete.argtypes = [C.c_void_p, C.c_char_p]
+        h.vh_fragment_tokens.argtypes = [C.c_void_p, C.c_char_p]
+        h.vh_fragment_count.argtypes = [C.c_void_p]
         h.vh_pool_block_stats.argtypes = [C.c_void_p] + [C.POINTER(C.c_int)] * 3
         h.vh_pool_block_stats.restype = None
         h.vh_pool_block_table.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int]
@@ -322,6 +327,25 @@ class ModelRuntime:
 
     def share_blocks(self, src, dst, num_tokens):
         self._ck(self._h.vh_pool_share_blocks(self._m, src, dst, num_tokens))
+
+    # ---- named fragments (kv/fragment.go, kv/paged_cache.go:285-343)
+    def cache_fragment(self, name, seq_id):
+        self._ck(self._h.vh_fragment_cache(self._m, name.encode(), seq_id))
+
+    def insert_fragment(self, seq_id, name, insert_pos):
+        """-> tokens inserted (0 when no fragment has that name)"""
+        n = C.c_int(0)
+        self._ck(self._h.vh_fragment_insert(self._m, seq_id, name.encode(), insert_pos, C.byref(n)))
+        return n.value
+
+    def delete_fragment(self, name):
+        self._ck(self._h.vh_fragment_delete(self._m, name.encode()))
+
+    def fragment_tokens(self, name):
+        return self._h.vh_fragment_tokens(self._m, name.encode())
+
+    def fragment_count(self):
+        return self._h.vh_fragment_count(self._m)
 
     def block_stats(self):
         a, b, c = C.c_int(), C.c_int(), C.c_int()
