@@ -523,7 +523,7 @@ def configs_report(be):
     mr.close()
     ctx4 = [int(x) for x in np.clip(np.exp(rng.normal(math.log(512.0), 0.6, 64)), 16, 4096)]
     mr, ids = decode_rate("config 4 (decode part): 8B-shaped Q8_0, 64 sequences (sum ctx %d)" % sum(ctx4), l8b,
-                          {"*": lib.VX_Q8_0}, ctx4 + [640], 32)   # the 65th sequence only reserves blocks for the chunk
+                          {"*": lib.VX_Q8_0}, ctx4 + [4200], 32)   # the 65th sequence only reserves blocks for the chunks
     chunk = rng.integers(0, l8b["vocab"], 512).tolist()
     mr.delete_sequence(ids[-1])
     mr.prefill_with_paged_kv(chunk[:64], 1000, 0)           # sizes the workspaces
@@ -534,6 +534,27 @@ def configs_report(be):
     be.sync()
     dt = time.perf_counter() - t0
     print("%-64s %8.1f tok/s  %7.3f ms/chunk" % ("config 4 (prefill part): one 512-token chunk", 512 / dt, dt * 1e3), flush=True)
+    # later chunks of a long prompt: 512 tokens at start positions 512 and 3584 (paged multi-query attention over the
+    # f16 pool, runtime/block.go:881-890); the contexts before them are adopted blocks of the synthetic pool
+    mr.delete_sequence(1001)
+    for start in (512, 3584):
+        sid = 2000 + start
+        free_now = mr.block_stats()[1] // l8b["num_layers"]
+        need = (start + 512 + BLOCK - 1) // BLOCK
+        if free_now < need + 2:
+            print("config 4 later chunk at %d: skipped, %d free blocks" % (start, free_now), flush=True)
+            continue
+        mr.create_sequence(sid)
+        for p0 in range(0, start, 512):          # the earlier chunks, untimed
+            mr.prefill_with_paged_kv(chunk, sid, p0)
+        be.sync()
+        t0 = time.perf_counter()
+        mr.prefill_with_paged_kv(chunk, sid, start)
+        be.sync()
+        dt = time.perf_counter() - t0
+        print("%-64s %8.1f tok/s  %7.3f ms/chunk" % ("config 4 (prefill part): 512-token chunk at position %d" % start,
+                                                      512 / dt, dt * 1e3), flush=True)
+        mr.delete_sequence(sid)
     mr.close()
     ctx5 = [int(x) for x in rng.integers(256, 2049, 16)]
     mr, ids = build_model(be, ctx5, 64, 32, CFG, {"*": lib.VX_Q6_K}, max_batch=16)

@@ -109,6 +109,39 @@ def test_paged_attention_at_full_context_and_head_geometry(be):
         be.reset_pool()
 
 
+def test_prompt_chunk_of_512_at_position_3584_8b_geometry(be):
+    """Benchmark config 4's largest later chunk: 512 query rows at start position 3584 (the last chunk of a
+    4096-token prompt), 32 / 8 heads of 128, F16 pool, on the tiled multi-query kernel. Sampled rows (tile edges, the
+    first and the last) against the oracle's per-row attention; every row against the single-query split-KV decode
+    kernel of the same library, which was checked against the oracle at these lengths above."""
+    rng = np.random.default_rng(405)
+    bs, hq, hk, d, start, qn = 16, 32, 8, 128, 3584, 512
+    nb = (start + qn) // bs
+    nblocks = nb + 5
+    pool = nx.f32_to_f16_array(rng.standard_normal(nblocks * 2 * bs * hk * d).astype(np.float32))
+    bt = rng.permutation(nblocks)[:nb].astype(np.int32)
+    q = rng.standard_normal((qn, hq, d)).astype(np.float32)
+    kvl = np.arange(start + 1, start + qn + 1, dtype=np.int32)
+    sc = np.float32(1 / math.sqrt(d))
+    dq, dpool, dbt, dk = be.upload(q), be.upload(pool, permanent=True), be.upload(bt), be.upload(kvl)
+    do = be.alloc(q.nbytes)
+    be.sdpa_paged_decode_multiquery(dq, dpool, dbt, do, dk, nb, bs, hq, hk, d, sc, qn, pool_is_f16=True)
+    got = be.download(do, q.shape, np.float32)
+    for i in (0, 1, 63, 64, 255, 256, 510, 511):
+        L = int(kvl[i])
+        n_i = (L + bs - 1) // bs
+        want = nx.sdpa_paged_decode(q[i], pool, bt[:n_i], n_i, bs, hq, hk, d, sc, L - (n_i - 1) * bs)
+        _close(got[i], want.reshape(hq, d), 1e-5, 3e-6, "chunk row %d" % i)
+    # all 512 rows as 512 one-query sequences that share the table
+    tables = np.tile(bt, (qn, 1))
+    dt, do2 = be.upload(tables), be.alloc(q.nbytes)
+    be.sdpa_paged_decode_ragged(dq, dpool, True, dt, dk, do2, qn, nb, bs, hq, hk, d, sc, start + qn)
+    ref = be.download(do2, q.shape, np.float32)
+    _close(got, ref, 2e-5, 6e-6, "tiled chunk against the split-KV decode kernel")
+    be.free(dpool)
+    be.reset_pool()
+
+
 def test_pack_batch_at_maximum_batch_and_context(be):
     """The packing kernel at 64 sequences whose positions sit on every kind of boundary up to 4096 tokens:
     bit-exact against the host pool's own bookkeeping."""

@@ -756,6 +756,41 @@ def test_paged_multiquery_and_tree(be):
         be.reset_pool()
 
 
+@pytest.mark.parametrize("hq,hk,d,qn,start", [(8, 2, 128, 200, 137), (8, 8, 64, 70, 0), (4, 1, 128, 16, 500),
+                                              (32, 8, 128, 65, 40)])
+def test_paged_multiquery_tiled(be, hq, hk, d, qn, start):
+    """SDPAPagedDecodeMultiquery on the tiled kernel (F16 pool, 16 or more query rows): the later chunk of a prompt
+    (row i sees start + i + 1 keys, runtime/block.go:884-887), with the chunk's rows crossing 64-row tile and 32-key
+    tile boundaries, against the oracle's per-row attention."""
+    rng = np.random.default_rng(340 + qn)
+    bs, nblocks = 16, 60
+    pool = _make_pool(rng, True, nblocks, bs, hk, d)
+    dpool = be.upload(pool)
+    bt = rng.permutation(nblocks)[:(start + qn + bs - 1) // bs + 1].astype(np.int32)
+    sc = np.float32(1 / math.sqrt(d))
+    q = rng.standard_normal((qn, hq, d)).astype(np.float32)
+    kvl = np.array([start + i + 1 for i in range(qn)], dtype=np.int32)
+    dq, dbt, dk, do = be.upload(q), be.upload(bt), be.upload(kvl), be.alloc(q.nbytes)
+    be.sdpa_paged_decode_multiquery(dq, dpool, dbt, do, dk, len(bt), bs, hq, hk, d, sc, qn, pool_is_f16=True)
+    want = nx.sdpa_paged_multiquery(q, pool, bt, kvl, bs, hq, hk, d, sc)
+    _close(be.download(do, q.shape, np.float32), want, 1e-5, 3e-6, "tiled multiquery, causal chunk")
+    # lengths in no order, some rows seeing a single key, one row none at all (its output is zero)
+    kvl2 = rng.integers(1, start + qn + 1, qn).astype(np.int32)
+    kvl2[3], kvl2[qn - 1] = 1, start + qn
+    be.to_device(dk, kvl2)
+    be.sdpa_paged_decode_multiquery(dq, dpool, dbt, do, dk, len(bt), bs, hq, hk, d, sc, qn, pool_is_f16=True)
+    want = nx.sdpa_paged_multiquery(q, pool, bt, kvl2, bs, hq, hk, d, sc)
+    _close(be.download(do, q.shape, np.float32), want, 1e-5, 3e-6, "tiled multiquery, ragged lengths")
+    kvl2[5] = 0
+    be.to_device(dk, kvl2)
+    be.sdpa_paged_decode_multiquery(dq, dpool, dbt, do, dk, len(bt), bs, hq, hk, d, sc, qn, pool_is_f16=True)
+    got = be.download(do, q.shape, np.float32)
+    assert not got[5].any()
+    keep = [i for i in range(qn) if i != 5]
+    _close(got[keep], want[keep], 1e-5, 3e-6, "tiled multiquery, one empty row")
+    be.reset_pool()
+
+
 @pytest.mark.parametrize("hq,hk,d", [(8, 8, 128), (8, 2, 64), (16, 2, 128)])
 def test_paged_tree_batched(be, hq, hk, d):
     """Every tree of a batch in two launches: against the oracle's masked multi-query attention per sequence and,

@@ -477,20 +477,47 @@ __device__ __forceinline__ float row16_max(float t) {  // max over the 16 lanes 
 
 // CAP: the scores (held in log2 units, score * log2 e) pass through cap2 * tanh(. / cap2) with
 // cap2 = softcap * log2 e, which is softcap * tanh(score / softcap) in those units.
-template <int D, bool CAP = false>
+// PAGED: the keys and values are the rows of one sequence in an F16 paged pool (block table `paged.table`), and query
+// row i attends to the first paged.kv_lens[i] of them (Backend.SDPAPagedDecodeMultiquery, backend.go:456-466: the
+// later chunks of a prompt, kv_lens[i] = startPos + i + 1, and linear verification, runtime/block.go:881-890)
+// instead of to rows 0..i of dense float32 K and V.
+struct PagedSrc {
+    const _Float16 *pool;
+    const int32_t *table;
+    const int32_t *kv_lens;
+    int block_size;
+};
+
+template <int D, bool CAP = false, bool PAGED = false>
 __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restrict__ q, const float *__restrict__ k,
                                                           const float *__restrict__ v, float *__restrict__ out, int S,
                                                           int num_q_heads, int num_kv_heads, float scale,
-                                                          float softcap = 0.f) {
+                                                          float softcap = 0.f, PagedSrc paged = PagedSrc()) {
     constexpr int KP = D + 4, VP = D + 16, PP = FA_BK + 4;
     __shared__ __attribute__((aligned(16))) float Ks[FA_BK * KP];
     __shared__ __attribute__((aligned(16))) float Vs[FA_BK * VP];
     __shared__ __attribute__((aligned(16))) float Ps[4][16 * PP];
+    __shared__ int len_max[5];  // PAGED: the longest key range among each wave's 16 queries, [4]: among all 64
     const int qt = blockIdx.x, h = blockIdx.y, kvh = h / (num_q_heads / num_kv_heads);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c16 = lane & 15, g = lane >> 4;
     const int q0 = qt * FA_BQ + wave * 16;  // the wave's first query
     const size_t qs = (size_t)num_q_heads * D, ks = (size_t)num_kv_heads * D;
+    int lim[4];  // keys 0 .. lim[i]-1 are visible to the lane's query row 4g + i
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int qi = q0 + 4 * g + i;
+        lim[i] = PAGED ? (qi < S ? max(paged.kv_lens[qi], 0) : 0) : min(qi + 1, S);
+    }
+    if (PAGED) {
+        if (tid < 5) len_max[tid] = 0;
+        __syncthreads();
+        const int m4 = max(max(lim[0], lim[1]), max(lim[2], lim[3]));
+        atomicMax(&len_max[wave], m4);
+        atomicMax(&len_max[4], m4);
+        __syncthreads();
+    }
+    const int wave_keys = PAGED ? len_max[wave] : min(q0 + 15, S - 1) + 1;  // keys any of the wave's queries sees
 
     // Q as the A operand: lane (row c16, k = 4s + g), pre-multiplied by scale*log2(e)
     float qa[D / 4];
@@ -511,14 +538,25 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
         l_run[i] = 0.f;
     }
     const int last_q = min(qt * FA_BQ + FA_BQ - 1, S - 1);
-    const int n_tiles = last_q / FA_BK + 1;  // keys 0 .. last_q
+    const int n_keys = PAGED ? len_max[4] : last_q + 1;  // keys 0 .. n_keys-1 are visible to some query of the tile
+    const int n_tiles = (n_keys + FA_BK - 1) / FA_BK;
     for (int kt = 0; kt < n_tiles; kt++) {
         __syncthreads();  // the previous tile's reads are done
         for (int idx = tid; idx < FA_BK * (D / 4); idx += 256) {
             const int key = idx / (D / 4), d4 = (idx % (D / 4)) * 4;
             const int ki = kt * FA_BK + key;
             float4 kv4 = make_float4(0.f, 0.f, 0.f, 0.f), vv4 = kv4;
-            if (ki < S) {
+            if (PAGED) {
+                if (ki < n_keys) {
+                    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+                    const size_t part = (size_t)paged.block_size * ks;  // a block's K rows, then its V rows
+                    const _Float16 *kp = paged.pool + (size_t)paged.table[ki / paged.block_size] * 2 * part +
+                                         (size_t)(ki % paged.block_size) * ks + (size_t)kvh * D + d4;
+                    const half4 kh = *(const half4 *)kp, vh = *(const half4 *)(kp + part);
+                    kv4 = make_float4((float)kh[0], (float)kh[1], (float)kh[2], (float)kh[3]);
+                    vv4 = make_float4((float)vh[0], (float)vh[1], (float)vh[2], (float)vh[3]);
+                }
+            } else if (ki < S) {
                 kv4 = *(const float4 *)(k + (size_t)ki * ks + (size_t)kvh * D + d4);
                 vv4 = *(const float4 *)(v + (size_t)ki * ks + (size_t)kvh * D + d4);
             }
@@ -526,7 +564,7 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
             *(float4 *)(Vs + key * VP + d4) = vv4;
         }
         __syncthreads();
-        if (kt * FA_BK > min(q0 + 15, S - 1)) continue;  // every key of the tile is after the wave's queries
+        if (kt * FA_BK >= wave_keys) continue;  // every key of the tile is beyond what the wave's queries see
         // S = Q K^T for the wave's 16 queries x 32 keys: lane holds S[row 4g+i][key cb*16 + c16]
         float4v sc[FA_BK / 16];
 #pragma unroll
@@ -548,12 +586,11 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
         float alpha[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const int qi = q0 + 4 * g + i;
             float mx = -INFINITY;
 #pragma unroll
             for (int cb = 0; cb < FA_BK / 16; cb++) {
                 const int ki = kt * FA_BK + cb * 16 + c16;
-                if (ki > qi || ki >= S) sc[cb][i] = -INFINITY;
+                if (ki >= lim[i]) sc[cb][i] = -INFINITY;
                 mx = fmaxf(mx, sc[cb][i]);
             }
             mx = row16_max<16>(mx);
@@ -932,6 +969,22 @@ int vx_sdpa_paged_decode_multiquery(vx_backend *be, const float *q, const void *
     if (rc) return rc;
     VX_REQUIRE(q && kv_pool && block_table && out && kv_lens, "vx_sdpa_paged_decode_multiquery: null pointer");
     VX_REQUIRE(num_blocks >= 1 && block_size >= 1 && query_len >= 0, "vx_sdpa_paged_decode_multiquery: bad counts");
+    VX_REQUIRE(head_dim > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, "vx_sdpa_paged_decode_multiquery: bad head counts");
+    // Chunks of a prompt and verification rows over an F16 pool: the tiled kernel (K/V tiles of 32 keys staged in
+    // LDS for 64 queries, float32 matrix cores). A handful of rows, other head sizes and float32 pools keep the
+    // one-workgroup-per-query kernel.
+    if (pool_is_f16 && query_len >= 16 && (head_dim == 64 || head_dim == 128) && ((uintptr_t)kv_pool % 8) == 0) {
+        PagedSrc src = {(const _Float16 *)kv_pool, block_table, kv_lens, block_size};
+        dim3 grid(ceil_div(query_len, FA_BQ), num_q_heads);
+        if (head_dim == 128)
+            prefill_fa2_kernel<128, false, true><<<grid, 256, 0, be->stream>>>(q, nullptr, nullptr, out, query_len, num_q_heads,
+                                                                               num_kv_heads, scale, 0.f, src);
+        else
+            prefill_fa2_kernel<64, false, true><<<grid, 256, 0, be->stream>>>(q, nullptr, nullptr, out, query_len, num_q_heads,
+                                                                              num_kv_heads, scale, 0.f, src);
+        VX_CHECK_LAUNCH();
+        return VX_OK;
+    }
     AttnParams p = {};
     p.q = q;
     p.out = out;
