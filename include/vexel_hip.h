@@ -224,6 +224,15 @@ typedef struct vx_qweight {
  * (runtime/block.go:834-868). With x_prepared != 0 the normalised activation left prepared by the
  * previous vx_decode_ffn (next_norm_weight) is used and x / norm_weight are ignored. */
 int vx_decode_attn_qkv_supported(const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int head_dim);
+/* Optional, once per decode step before the layers' vx_decode_attn_qkv calls: works out cos / sin of every (row,
+ * dimension pair) for positions[0 .. rows-1] (up to 64 rows, heads up to 256) and keeps them in the backend. While the
+ * table stands, a vx_decode_attn_qkv call with the same positions pointer, at most 32 rows, an unbiased interleaved
+ * whole-head RoPE and weights laid out for a single K slice rotates and stores its rows inside the projection launch
+ * (one launch per layer less), with the same arithmetic. The table falls when the library writes to a caller's
+ * buffer (vx_pack_batch, vx_decode_advance, vx_to_device, vx_copy_buffer); a caller that changes the positions by
+ * other means must call this again (or not at all: without a table nothing changes). No counterpart in the reference,
+ * which recomputes the angles in every layer (backend/cpu/cpu.go:226-303). */
+int vx_rope_table_prepare(vx_backend *be, const int32_t *positions, int rows, int head_dim, float theta);
 int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight, float eps, int x_prepared,
                        const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int rows,
                        const int32_t *positions, const int32_t *slot_mapping, void *kv_pool, int pool_is_f16,

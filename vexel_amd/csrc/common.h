@@ -44,6 +44,8 @@ struct PoolChunk {
 }  // namespace vx
 
 // chunk-parallel prepares: up to 64 rows x 64 chunks of 256 columns; two [64][64] float arrays of per-chunk sums of squares
+#define VX_ROPE_TAB_ROWS 64
+#define VX_ROPE_TAB_PAIRS 128
 #define VX_PREP_SYNC_ROWS 64
 #define VX_PREP_SYNC_CHUNKS 64
 #define VX_PREP_SYNC_BYTES (2 * VX_PREP_SYNC_CHUNKS * VX_PREP_SYNC_ROWS * 4)
@@ -71,6 +73,13 @@ struct vx_backend {
     float prep_norm_eps = 0.f;   //      1/rms is still to be taken from the current slot of prep_sync
     void *part_ws = nullptr;     // split-K partial sums
     size_t part_ws_bytes = 0;
+    // cos / sin of every (row, pair) of the step's positions (vx_rope_table_prepare): [VX_ROPE_TAB_ROWS][head_dim/2]
+    // float2, valid while the key below matches and the library has written nothing since (write_epoch)
+    void *rope_tab = nullptr;
+    const int32_t *rope_tab_pos = nullptr;
+    int rope_tab_rows = 0, rope_tab_dim = 0;
+    float rope_tab_theta = 0.f;
+    uint64_t rope_tab_epoch = 0, write_epoch = 1;
     void *attn_ws = nullptr;     // split-KV partial results
     void *attn_fixed_ws = nullptr;  // this device's copy of the fixed-size partial-sum area (never allocated or freed)
     // attention left in split form by vx_sdpa_paged_decode_ragged(out = NULL), to be merged by vx_decode_ffn
@@ -114,6 +123,7 @@ constexpr int ATTN_TPW = 512;  // tokens of one (sequence, kv head) that one att
 
 // Drops the attention work list when [dst, dst + bytes) overlaps the kv_lens array it was built from.
 inline void items_written(vx_backend *be, const void *dst, size_t bytes) {
+    be->write_epoch++;  // the library wrote into a caller's buffer: a kept RoPE table may describe other positions now
     if (!be->items.valid) return;
     const char *a = (const char *)dst, *k = (const char *)be->items.kv_lens;
     if (a < k + (size_t)be->items.batch * 4 && k < a + bytes) be->items.valid = false;

@@ -141,6 +141,7 @@ extern "C" int vx_pack_batch(vx_backend *be, const int32_t *seq_slots, const int
                              int32_t *kv_lens, int32_t *status) {
     int rc = enter(be);
     if (rc) return rc;
+    be->write_epoch++;  // positions and slots change
     VX_REQUIRE(seq_slots && positions && block_tables && num_blocks && free_list && free_count && cu_seqlens &&
                    token_pos && slot_mapping && kv_lens && status,
                "vx_pack_batch: null pointer");
@@ -188,6 +189,7 @@ extern "C" int vx_decode_advance(vx_backend *be, int32_t *tokens, int32_t *posit
                                  int32_t *out_log, int32_t *step_counter, int batch) {
     int rc = enter(be);
     if (rc) return rc;
+    be->write_epoch++;  // positions move on
     VX_REQUIRE(tokens && positions && next_tokens && out_log && step_counter, "vx_decode_advance: null pointer");
     VX_REQUIRE(batch >= 1 && batch <= PK_THREADS, "vx_decode_advance: batch %d not in 1..%d", batch, PK_THREADS);
     decode_advance_kernel<<<1, PK_THREADS, 0, be->stream>>>(tokens, positions, next_tokens, out_log, step_counter,

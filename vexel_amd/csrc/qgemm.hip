@@ -886,8 +886,6 @@ __global__ void __launch_bounds__(256, F::MIN_WAVES) qgemm_kernel(Segs segs, Pre
     }
 }
 
-#include "qgemm_wave.h"
-
 // out[m][n] = residual + inv_scale[m] * (P[0] + P[1] + ... + P[KS-1]) in that order.
 __global__ void __launch_bounds__(256) qgemm_reduce_kernel(const float *__restrict__ partial,
                                                            const float *__restrict__ inv_scale,
@@ -1378,6 +1376,19 @@ __global__ void __launch_bounds__(64) finalize_row_norm_kernel(float *__restrict
     if (threadIdx.x == 0) inv_rows[blockIdx.x] = f;
 }
 
+// What the Q|K|V launch needs to finish its rows itself (RoPE, the rotated Q to q_out, K and V into the paged
+// pool: rope_store_partials_kernel's work) when one K slice holds the whole sum. q_out == NULL: not in use.
+struct QkvEpi {
+    float *q_out;
+    void *pool;
+    const int32_t *slots;
+    const float2 *cs_tab;  // [row][head_dim / 2] (cos, sin) of the row's position
+    RowNorm rn;
+    int qd, kvd, head_dim, block_size, pool_f16;
+};
+
+#include "qgemm_wave.h"
+
 // grid = (K/256, Mpad), block = 64.
 //   x_new = x + inv_in[r] * sum_s P[s][r][:]   (P may be NULL: x_new = x), x <- x_new when P is given,
 //   prepared <- x_new * w, its chunks' sums of squares to ss_out for the pending 1/rms (backend/cpu/cpu.go:200-220)
@@ -1603,6 +1614,16 @@ __global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, 
     }
 }
 
+// (cos, sin) of every (row, pair): rope_store_partials_kernel's angle arithmetic (backend/cpu/cpu.go:226-303 for one
+// position per row), once per step instead of once per layer. grid = rows, block = head_dim / 2.
+__global__ void rope_table_kernel(const int32_t *__restrict__ positions, float2 *__restrict__ tab, int head_dim, float theta) {
+    const int row = blockIdx.x, j = threadIdx.x, half = head_dim / 2;
+    const double ex = (double)(2 * j) / (double)head_dim;
+    const float freq = (float)(1.0 / pow((double)theta, ex));
+    const float angle = __fmul_rn((float)positions[row], freq);
+    tab[(size_t)row * half + j] = make_float2((float)cos((double)angle), (float)sin((double)angle));
+}
+
 size_t fmt_row_bytes(int fmt, int k) {
     switch (fmt) {
     case VX_Q4_0: return (size_t)k / 32 * 18;
@@ -1785,11 +1806,11 @@ WavePlan wave_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K) {
             const int wg_chunks = ceil_div(n_chunks, ks), wave_chunks = ceil_div(wg_chunks, 8);
             // In cycles, fitted to the 7B shapes at 32 rows: a wave's tile steps share a SIMD with one other
             // wave's (about 220 cycles a tile step for the pair); a compute unit pulls the 32 KB of activation
-            // tiles of a chunk at about 32 bytes a cycle; each extra slice costs its partial sums' trip through
-            // memory and the consumer's pass over them.
+            // tiles of a chunk at about 32 bytes a cycle; slicing K costs the partial sums' trip through memory, the
+            // consumer's pass over every slice, and the epilogues that only a whole sum can run.
             const float compute = (float)wave_chunks * 8.f * (float)r * 220.f;
             const float operand = (float)wg_chunks * 1024.f;
-            const float part = ks > 1 ? (float)ks * (float)N * 0.06f + 1500.f : 0.f;
+            const float part = ks > 1 ? (float)ks * (float)N * 0.06f + 5000.f : 0.f;
             const float cost = std::max(compute, operand) + part;
             if (best.r == 0 || cost < best_cost) {
                 best = WavePlan{r, ks};
@@ -1802,7 +1823,7 @@ WavePlan wave_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K) {
 
 template <class W, int R>
 int launch_gemm_wave(vx_backend *be, const Segs &segs, int N, float *out, const float *residual, bool to_partials, int M,
-                     int K, int ks, int *ks_out) {
+                     int K, int ks, int *ks_out, const QkvEpi &epi) {
     constexpr int NW = 8;
     const int mpad = mpad_for(M);
     const PrepView pv = prep_view(be, mpad, K);
@@ -1817,9 +1838,9 @@ int launch_gemm_wave(vx_backend *be, const Segs &segs, int N, float *out, const 
     const bool vec = ((uintptr_t)out % 16) == 0 && ((uintptr_t)residual % 16) == 0;
     const int n_chunks = K / 256, slices = ((n_chunks / ks) << 16) | (n_chunks % ks);  // the kernel takes the division done
     if (mpad <= 16)
-        qgemm_wave_kernel<W, R, 1, NW><<<grid, 64 * NW, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slices, vec ? 1 : 0);
+        qgemm_wave_kernel<W, R, 1, NW><<<grid, 64 * NW, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slices, vec ? 1 : 0, epi);
     else
-        qgemm_wave_kernel<W, R, 2, NW><<<grid, 64 * NW, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slices, vec ? 1 : 0);
+        qgemm_wave_kernel<W, R, 2, NW><<<grid, 64 * NW, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slices, vec ? 1 : 0, epi);
     VX_CHECK_LAUNCH();
     if (ks_out) *ks_out = ks;
     if (partial && !to_partials) {
@@ -1832,25 +1853,26 @@ int launch_gemm_wave(vx_backend *be, const Segs &segs, int N, float *out, const 
 
 template <class W>
 int launch_gemm_wave_r(vx_backend *be, const WavePlan &pl, const Segs &segs, int N, float *out, const float *residual,
-                       bool to_partials, int M, int K, int *ks_out) {
+                       bool to_partials, int M, int K, int *ks_out, const QkvEpi &epi) {
     switch (pl.r) {
-    case 1: return launch_gemm_wave<W, 1>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
-    case 2: return launch_gemm_wave<W, 2>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
-    case 3: return launch_gemm_wave<W, 3>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
-    case 4: return launch_gemm_wave<W, 4>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
-    case 6: return launch_gemm_wave<W, 6>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
+    case 1: return launch_gemm_wave<W, 1>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
+    case 2: return launch_gemm_wave<W, 2>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
+    case 3: return launch_gemm_wave<W, 3>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
+    case 4: return launch_gemm_wave<W, 4>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
+    case 6: return launch_gemm_wave<W, 6>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
     }
     set_error("wave GEMM: no kernel for %d tiles per workgroup", pl.r);
     return VX_ERR_INVALID;
 }
 
 int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out, const float *residual,
-                    bool to_partials, int M, int K, int *ks_out) {
+                    bool to_partials, int M, int K, int *ks_out, const QkvEpi *epi_in = nullptr) {
+    const QkvEpi epi = epi_in ? *epi_in : QkvEpi{};  // (with an epilogue the caller has checked that the wave plan applies)
     const WavePlan pl = wave_plan(be, fmt, segs, N, K);
     if (pl.r > 0) {
-        if (fmt == VX_Q4_0) return launch_gemm_wave_r<WQ4_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out);
-        if (fmt == VX_Q8_0) return launch_gemm_wave_r<WQ8_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out);
-        return launch_gemm_wave_r<WQ4_K>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out);
+        if (fmt == VX_Q4_0) return launch_gemm_wave_r<WQ4_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
+        if (fmt == VX_Q8_0) return launch_gemm_wave_r<WQ8_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
+        return launch_gemm_wave_r<WQ4_K>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
     }
     switch (fmt) {
     case VX_Q4_0: return launch_gemm<PQ4_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
@@ -2050,6 +2072,22 @@ static Segs make_segs(const vx_qweight *const *ws, int nw, int *ntot) {
 
 // The chunk-parallel prepares cover decode-sized batches; larger ones keep the one-workgroup-per-row kernels.
 bool chunk_prepare_ok(int rows, int k) { return mpad_for(rows) <= VX_PREP_SYNC_ROWS && k / 256 <= VX_PREP_SYNC_CHUNKS; }
+int vx_rope_table_prepare(vx_backend *be, const int32_t *positions, int rows, int head_dim, float theta) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(positions && rows >= 1 && head_dim >= 2 && head_dim % 2 == 0, "vx_rope_table_prepare: bad arguments");
+    be->rope_tab_pos = nullptr;
+    if (rows > VX_ROPE_TAB_ROWS || head_dim / 2 > VX_ROPE_TAB_PAIRS) return VX_OK;  // no table: the calls keep their own arithmetic
+    rope_table_kernel<<<rows, head_dim / 2, 0, be->stream>>>(positions, (float2 *)be->rope_tab, head_dim, theta);
+    VX_CHECK_LAUNCH();
+    be->rope_tab_pos = positions;
+    be->rope_tab_rows = rows;
+    be->rope_tab_dim = head_dim;
+    be->rope_tab_theta = theta;
+    be->rope_tab_epoch = be->write_epoch;
+    return VX_OK;
+}
+
 int vx_decode_attn_qkv_supported(const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int head_dim) {
     const vx_qweight *ws[3] = {wq, wk, wv};
     return group_ok(ws, 3) && head_dim % 2 == 0 && head_dim <= 512 && (size_t)wq->k * 4 <= 64 * 1024;
@@ -2127,6 +2165,29 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
     const vx_qweight *ws[3] = {wq, wk, wv};
     int ntot, ks;
     const Segs segs = make_segs(ws, 3, &ntot);
+    // One K slice, one activation group, the plain RoPE form and a table of this step's angles: the GEMM's workgroups
+    // finish their own rows (no partial sums, no second launch).
+    {
+        const WavePlan pl = wave_plan(be, wq->fmt, segs, ntot, k);
+        const bool table = be->rope_tab_pos == positions && be->rope_tab_rows >= rows && be->rope_tab_dim == head_dim &&
+                           be->rope_tab_theta == theta && be->rope_tab_epoch == be->write_epoch;
+        static const bool no_epi = getenv("VEXEL_HIP_NO_QKV_EPILOGUE") != nullptr;
+        if (!no_epi && !gen && table && pl.r > 0 && pl.ks == 1 && mpad_for(rows) <= 32 && (head_dim & (head_dim - 1)) == 0 &&
+            head_dim >= 4 && ((uintptr_t)kv_pool % 16) == 0 && ((uintptr_t)q_out % 16) == 0) {
+            QkvEpi epi;
+            epi.q_out = q_out;
+            epi.pool = kv_pool;
+            epi.slots = slot_mapping;
+            epi.cs_tab = (const float2 *)be->rope_tab;
+            epi.rn = cur_row_norm(be);
+            epi.qd = wq->n;
+            epi.kvd = wk->n;
+            epi.head_dim = head_dim;
+            epi.block_size = block_size;
+            epi.pool_f16 = pool_is_f16;
+            return launch_gemm_fmt(be, wq->fmt, segs, ntot, nullptr, nullptr, false, rows, k, nullptr, &epi);
+        }
+    }
     rc = launch_gemm_fmt(be, wq->fmt, segs, ntot, nullptr, nullptr, true, rows, k, &ks);
     if (rc) return rc;
     const PrepView pv = prep_view(be, mpad_for(rows), k);

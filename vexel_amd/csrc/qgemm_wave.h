@@ -141,7 +141,8 @@ template <class W, int R, int MT> struct WaveGeom {
 template <class W, int R, int MT, int NW>
 __global__ void __launch_bounds__(64 * NW, 1) qgemm_wave_kernel(Segs segs, PrepView pv, float *__restrict__ out,
                                                                const float *__restrict__ residual, float *__restrict__ partial,
-                                                               int M, int Mpad, int N, int K, int n_slices, int flags) {
+                                                               int M, int Mpad, int N, int K, int n_slices, int flags,
+                                                               QkvEpi epi) {
     typedef WaveGeom<W, R, MT> G;
     constexpr int ROWS = G::ROWS;
     // steps an activation load runs ahead of its use: a step of few tiles is short, so its operand must be
@@ -345,6 +346,15 @@ __global__ void __launch_bounds__(64 * NW, 1) qgemm_wave_kernel(Segs segs, PrepV
 #pragma unroll
                 for (int e = 0; e < 4; e++) T[(t * 16 + 4 * g + e) * TP + r * 16 + ln] = run[r][t][e];
     }
+    // Q|K|V rows finished here: the row factors (with the pending 1/rms of the RMSNorm that fed the activation) are
+    // whole-wave computations, one row at a time
+    __shared__ float s_fac[16 * MT];
+    if (epi.q_out) {
+        for (int r = wave; r < 16 * MT; r += NW) {
+            const float f = row_factor(pv.inv_scale, epi.rn, m0 + r);
+            if (lane == 0) s_fac[r] = f;
+        }
+    }
     __syncthreads();
     constexpr int F4 = 16 * MT * ROWS / 4;  // float4 groups of the block
     constexpr int NT = 64 * NW;
@@ -361,6 +371,38 @@ __global__ void __launch_bounds__(64 * NW, 1) qgemm_wave_kernel(Segs segs, PrepV
         }
         const int m = m0 + ml, n = n0 + nl;
         if (m >= M || n < n_own) continue;
+        if (epi.q_out) {
+            // columns n .. n+3 of row m: two RoPE pairs of a Q or K head, or four V values (the arithmetic of
+            // rope_store_partials_kernel, which does this for launches that leave partial sums)
+            const float inv = s_fac[ml];
+            const float a0 = __fmul_rn(c.x, inv), b0 = __fmul_rn(c.y, inv), a1 = __fmul_rn(c.z, inv), b1 = __fmul_rn(c.w, inv);
+            const bool is_q = n < epi.qd, is_v = n >= epi.qd + epi.kvd;
+            const int o = is_q ? n : (is_v ? n - epi.qd - epi.kvd : n - epi.qd);
+            float4 r4 = make_float4(a0, b0, a1, b1);
+            if (!is_v) {
+                const float2 *cs = epi.cs_tab + (size_t)m * (epi.head_dim >> 1) + ((o & (epi.head_dim - 1)) >> 1);
+                const float2 c0 = cs[0], c1 = cs[1];
+                r4.x = __fsub_rn(__fmul_rn(a0, c0.x), __fmul_rn(b0, c0.y));
+                r4.y = __fadd_rn(__fmul_rn(a0, c0.y), __fmul_rn(b0, c0.x));
+                r4.z = __fsub_rn(__fmul_rn(a1, c1.x), __fmul_rn(b1, c1.y));
+                r4.w = __fadd_rn(__fmul_rn(a1, c1.y), __fmul_rn(b1, c1.x));
+            }
+            if (is_q) {
+                *(float4 *)(epi.q_out + (size_t)m * epi.qd + o) = r4;
+                continue;
+            }
+            const int slot = epi.slots[m], blk = slot / epi.block_size, off = slot - blk * epi.block_size;
+            const size_t part = (size_t)epi.block_size * epi.kvd;
+            const size_t at = (size_t)blk * 2 * part + (size_t)off * epi.kvd + (is_v ? part : 0) + o;
+            if (epi.pool_f16) {
+                typedef _Float16 half4w __attribute__((ext_vector_type(4)));
+                const half4w h4 = {(_Float16)r4.x, (_Float16)r4.y, (_Float16)r4.z, (_Float16)r4.w};
+                *(half4w *)((_Float16 *)epi.pool + at) = h4;
+            } else {
+                *(float4 *)((float *)epi.pool + at) = r4;
+            }
+            continue;
+        }
         if (partial) {
             *(float4 *)(partial + ((size_t)ks * M + m) * N + n) = c;
             continue;
