@@ -276,7 +276,11 @@ int vx_rope_store_paged_ex(vx_backend *be, float *q, const float *k, const float
  * streaming kernels attend a longer sequence over its first max_kv_len tokens, rounded up to whole splits, and stay
  * inside their buffers; max_blocks * block_size is always a safe value). With out = NULL the result stays in the backend as per-split partial
  * sums for the next vx_decode_ffn(attn = NULL) to merge (one launch less); that form exists only where
- * vx_sdpa_paged_decode_split_supported() is 1, otherwise the call returns VX_ERR_UNSUPPORTED.
+ * vx_sdpa_paged_decode_split_supported() is 1, otherwise the call returns VX_ERR_UNSUPPORTED. Where a workgroup's
+ * columns (query heads per KV head x head_dim) divide 256 or are a multiple of it, 2 to 64 rows, the workgroup that
+ * finishes a sequence's 256 columns last also merges them, splits in index order, and writes them as the output
+ * projection's prepared operand (no merge launch at all); any call between the two that prepares another
+ * activation makes vx_decode_ffn merge from the partial sums as before.
  * That is also where the streaming split-KV kernel runs (F16 pool, 16-token blocks): heads of 64 or 128 with 1 to 8
  * query heads per KV head, heads of 256 with 1 or 2, heads of 80 or 96 with 1; other geometries take the generic
  * kernel (any head_dim <= 256), same results, far slower. */

@@ -395,13 +395,17 @@ def test_fused_decode_blocks_equal_the_unfused_sequence(be, fmt, rows, hidden, f
     be.reset_pool()
 
 
-def test_decode_ffn_merges_split_attention(be):
+# (query heads, kv heads, head size): a workgroup's columns are one 256-column chunk, a quarter or half of one,
+# four of them, and (3 query heads of 128 per kv head) no whole number either way
+@pytest.mark.parametrize("hq,hk,d", [(8, 2, 64), (8, 8, 64), (4, 4, 128), (8, 1, 128), (6, 2, 128)])
+def test_decode_ffn_merges_split_attention(be, hq, hk, d):
     """vx_sdpa_paged_decode_ragged(out = NULL) + vx_decode_ffn(attn = NULL) equals the merged attention output
-    fed to vx_decode_ffn (the split-KV partials are merged by the same formula inside the prepare kernel)."""
+    fed to vx_decode_ffn (the split-KV partials are merged by the same formula, by the attention kernel's last
+    workgroup of each chunk or by the prepare kernel)."""
     rng = np.random.default_rng(91)
     fmt, rows, hidden, ffn = nx.FMT_Q4_0, 5, 512, 1024
-    hq, hk, d, bs, nblocks, eps = 8, 2, 64, 16, 160, 1e-5
-    dims = dict(wo=(hidden, hidden), w1=(ffn, hidden), w3=(ffn, hidden), w2=(hidden, ffn))
+    bs, nblocks, eps = 16, 160, 1e-5
+    dims = dict(wo=(hidden, hq * d), w1=(ffn, hidden), w3=(ffn, hidden), w2=(hidden, ffn))
     dW = {n: be.upload(qz.random_quant(fmt, rng, *dims[n])) for n in dims}
     qw = {n: be.qweight(fmt, dW[n], *dims[n]) for n in dims}
     assert be.lib_call("vx_sdpa_paged_decode_split_supported", 1, bs, hq, hk, d) == 1
@@ -420,16 +424,22 @@ def test_decode_ffn_merges_split_attention(be):
     nw = rng.standard_normal(hidden).astype(np.float32)
     dpool, dq, dt, dl, dnw = be.upload(pool), be.upload(q), be.upload(tables), be.upload(lens), be.upload(nw)
     scale = 1.0 / math.sqrt(d)
-    dattn = be.alloc(rows * hidden * 4)
-    be.sdpa_paged_decode_ragged(dq, dpool, True, dt, dl, dattn, rows, max_blocks, bs, hq, hk, d, scale, max_blocks * bs)
-    dx1 = be.upload(x)
-    be.decode_ffn(dattn, dx1, qw["wo"], dnw, eps, qw["w1"], qw["w3"], qw["w2"], rows, None)
-    want = be.download(dx1, (rows, hidden), np.float32)
-    dx2 = be.upload(x)
-    be.sdpa_paged_decode_ragged(dq, dpool, True, dt, dl, None, rows, max_blocks, bs, hq, hk, d, scale, max_blocks * bs)
-    be.decode_ffn(None, dx2, qw["wo"], dnw, eps, qw["w1"], qw["w3"], qw["w2"], rows, None)
-    got = be.download(dx2, (rows, hidden), np.float32)
-    assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want).max())
+    dattn = be.alloc(rows * hq * d * 4)
+    # twice, the second time with other lengths (fewer splits, one sequence without tokens: zeros): whatever the
+    # first call counted is gone
+    for lens_i in (lens, np.array([300, 0, 512, 40, 31], dtype=np.int32)):
+        dl = be.upload(lens_i)
+        be.sdpa_paged_decode_ragged(dq, dpool, True, dt, dl, dattn, rows, max_blocks, bs, hq, hk, d, scale, max_blocks * bs)
+        dx1 = be.upload(x)
+        be.decode_ffn(dattn, dx1, qw["wo"], dnw, eps, qw["w1"], qw["w3"], qw["w2"], rows, None)
+        want_i = be.download(dx1, (rows, hidden), np.float32)
+        dx2 = be.upload(x)
+        be.sdpa_paged_decode_ragged(dq, dpool, True, dt, dl, None, rows, max_blocks, bs, hq, hk, d, scale, max_blocks * bs)
+        be.decode_ffn(None, dx2, qw["wo"], dnw, eps, qw["w1"], qw["w3"], qw["w2"], rows, None)
+        got = be.download(dx2, (rows, hidden), np.float32)
+        assert np.all(np.abs(got - want_i) <= 1e-5 * np.abs(want_i).max())
+        if lens_i is lens:
+            want = want_i
     # one row (the matrix-vector path merges the partials while it reads its activation): sequence 2, 700 tokens
     one = slice(2, 3)
     dq1, dt1, dl1 = be.upload(q[one]), be.upload(tables[one]), be.upload(lens[one])

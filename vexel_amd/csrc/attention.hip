@@ -17,6 +17,7 @@
 #include <float.h>
 
 #include "common.h"
+#include "prep_tiles.h"
 
 using namespace vx;
 
@@ -196,6 +197,15 @@ __device__ __forceinline__ float token_sum(float t) {
     return t;
 }
 
+// Where the workgroup that finishes a sequence's 256-column chunk last leaves the chunk merged over its splits,
+// as the prepared activation of the output projection (cnt == nullptr: nobody merges, the partial sums are the
+// result). cnt[sequence * units + unit] counts the arrivals and is zero again when the launch ends.
+struct MergeOut {
+    PrepView pv;
+    int32_t *cnt = nullptr;
+    int mpad = 0;
+};
+
 // RG > 1: an entry of the batch is RG consecutive query rows that share one sequence's context (the rows of a
 // candidate tree): the workgroup serves the G*RG queries (row, head) of its kv head from one pass over the K/V.
 template <int D, int G, int RG = 1>
@@ -203,7 +213,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix,
     const int32_t *__restrict__ bt_rows, int max_blocks, const int32_t *__restrict__ kv_lens,
     float *__restrict__ partial, int num_q_heads, int num_kv_heads, float scale, int max_splits,
-    const int32_t *__restrict__ items) {
+    const int32_t *__restrict__ items, MergeOut mg) {
     constexpr int GG = G * RG;       // queries per K/V row
     constexpr int DL = D / 8;        // 8-element slices of a head vector
     // lanes per token: the next power of two; the lanes past DL (heads of 80 or 96) repeat the last slice's loads
@@ -231,12 +241,29 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     // buffers.
     kv_len = min(kv_len, max_splits * TPW);
     const int t_begin = split * TPW;
-    if (split >= max_splits || t_begin >= kv_len) return;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int GD = G * D;                          // this workgroup's columns of the output
+    constexpr bool MERGES = RG == 1 && (GD % 256 == 0 || 256 % GD == 0);
+    constexpr int CH = GD >= 256 ? GD / 256 : 1;       // 256-column chunks inside them
+    constexpr int HPC = GD >= 256 ? 1 : 256 / GD;      // kv heads that share a chunk
+    if (split >= max_splits || t_begin >= kv_len) {
+        // a sequence without tokens has nobody to merge for it: zeros, as the merge of no splits gives
+        if constexpr (MERGES) {
+            if (mg.cnt && kv_len == 0 && split == 0 && kvh % HPC == 0) {
+                const float zero[4] = {0.f, 0.f, 0.f, 0.f};
+                for (int ch = wave; ch < CH; ch += 4) {
+                    const int c = kvh / HPC * CH + ch;
+                    write_chunk(mg.pv, seq, c, zero, mg.mpad);
+                    if (c == 0 && lane == 0) mg.pv.inv_scale[seq] = 1.f;
+                }
+            }
+        }
+        return;
+    }
     const int t_end = min(kv_len, t_begin + TPW);
     const int32_t *bt = bt_matrix + (size_t)row * max_blocks + t_begin / HOT_BS;
 
-    const int tid = threadIdx.x, lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int tl = lane / LPT;  // token slot within a load
     const int dl = DL == LPT ? lane % LPT : min(lane % LPT, DL - 1);  // 8-element slice of the head vector
     const bool live = DL == LPT ? true : lane % LPT < DL;
@@ -358,10 +385,42 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
         }
         const int qh = kvh * G + g % G;
         float *po = partial + ((((size_t)seq * RG + g / G) * num_q_heads + qh) * max_splits + split) * (D + 2);
-        po[2 + d] = A;
+        // (device-scope stores: written through to where a workgroup on another die reads them, see below)
+        __hip_atomic_store(po + 2 + d, A, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (d == 0) {
-            po[0] = M;
-            po[1] = L;
+            __hip_atomic_store(po, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(po + 1, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    // The last workgroup to arrive at a (sequence, chunk of 256 output columns) merges the chunk's splits in
+    // index order - the sums do not depend on who that is - and writes it as the next GEMM's operand.
+    if constexpr (MERGES) {
+        if (!mg.cnt) return;
+        // Ordering without device-wide cache write-backs and invalidations (a release / acquire fence pair at
+        // device scope costs this kernel several times its run time: every workgroup would flush and drop its
+        // die's L2): the partial sums above are device-scope stores and are read back by device-scope loads, which
+        // the dies' caches do not hold back or serve stale; each wave waits until its stores are acknowledged
+        // before the workgroup's barrier, thread 0 counts the arrival after the barrier, and whoever counts the
+        // last one reads only after that atomic has returned.
+        __shared__ int s_last;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const int ns = (kv_len + TPW - 1) / TPW;  // workgroups of one kv head that arrive for this sequence
+        const int unit = kvh / HPC;
+        if (tid == 0) {
+            int32_t *cnt = mg.cnt + (size_t)seq * (num_kv_heads / HPC) + unit;
+            const int last = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ns * HPC - 1;
+            if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // (nobody else comes before the next launch)
+            s_last = last;
+        }
+        __syncthreads();
+        if (!s_last) return;
+        for (int ch = wave; ch < CH; ch += 4) {
+            const int c = unit * CH + ch;
+            float y[4];
+            split_merge4<true>(partial, ns, num_q_heads, D, max_splits, seq, c * 256 + lane * 4, y);
+            write_chunk(mg.pv, seq, c, y, mg.mpad);
+            if (c == 0 && lane == 0) mg.pv.inv_scale[seq] = 1.f;
         }
     }
 }
@@ -678,13 +737,31 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
                         ((size_t)batch * max_splits + 1) * 4 <= be->items.bytes / sizeof(int32_t) &&
                         (size_t)batch * max_splits <= 65535;
     dim3 grid(num_kv_heads, listed ? batch * max_splits : max_splits, listed ? 1 : batch);
+    // out == NULL leaves the result to vx_decode_ffn(attn = NULL): as split partial sums, and - where the shape
+    // allows - already merged and prepared as that call's first operand by the workgroups that finish last.
+    MergeOut mg;
+    static const bool no_merge = getenv("VEXEL_HIP_NO_ATTN_MERGE") != nullptr;
+    constexpr int GD = G * D;
+    constexpr int HPC = (GD < 256 && 256 % GD == 0) ? 256 / GD : 0;  // kv heads that share a chunk
+    const bool mergeable = GD % 256 == 0 || (HPC > 0 && num_kv_heads % HPC == 0);
+    if (!out && !fixed && !no_merge && batch >= 2 && mergeable && be->attn_cnt &&
+        (size_t)batch * num_kv_heads <= VX_ATTN_CNT) {
+        int mpad = 0;
+        const int rc = prep_begin_chunked(be, batch, num_q_heads * D, &mg.pv, &mpad);
+        if (rc == VX_OK) {
+            mg.cnt = be->attn_cnt;
+            mg.mpad = mpad;
+        } else if (rc != VX_ERR_UNSUPPORTED)
+            return rc;
+    }
     paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
                                                                 max_blocks, kv_lens, ws, num_q_heads,
                                                                 num_kv_heads, scale, max_splits,
-                                                                listed ? be->items.buf : nullptr);
+                                                                listed ? be->items.buf : nullptr, mg);
     VX_CHECK_LAUNCH();
     if (!fixed) be->split.batch = 0;  // (the fixed area is not where vx_decode_ffn looks for a split result)
     if (!out) {  // the caller merges: vx_decode_ffn(attn = NULL)
+        be->split.merged = mg.cnt != nullptr;
         be->split.batch = batch;
         be->split.num_q_heads = num_q_heads;
         be->split.head_dim = D;
@@ -1067,7 +1144,7 @@ int vx_sdpa_paged_tree_batched(vx_backend *be, const float *q, const void *kv_po
     if (head_dim == DD && G == GG)                                                                                        \
         paged_decode_f16_kernel<DD, GG, RR><<<grid, 256, 0, be->stream>>>(q, pool, block_tables, entry_table_rows, max_blocks, \
                                                                         entry_kv_lens, ws, num_q_heads, num_kv_heads, scale, \
-                                                                        max_splits, nullptr);
+                                                                        max_splits, nullptr, MergeOut{});
         VX_TREE(128, 1, 8) VX_TREE(128, 2, 4) VX_TREE(128, 4, 2) VX_TREE(128, 8, 1)
         VX_TREE(64, 1, 8) VX_TREE(64, 2, 4) VX_TREE(64, 4, 2) VX_TREE(64, 8, 1)
 #undef VX_TREE

@@ -88,6 +88,8 @@ int vx_backend_create(int device_id, vx_backend **out) {
     be->misc_ws_bytes = 1 << 20;
     VX_CHECK_HIP(hipMalloc(&be->misc_ws, be->misc_ws_bytes));
     VX_CHECK_HIP(hipMalloc(&be->rope_tab, (size_t)VX_ROPE_TAB_ROWS * VX_ROPE_TAB_PAIRS * 2 * sizeof(float)));
+    VX_CHECK_HIP(hipMalloc((void **)&be->attn_cnt, VX_ATTN_CNT * sizeof(int32_t)));
+    VX_CHECK_HIP(hipMemset(be->attn_cnt, 0, VX_ATTN_CNT * sizeof(int32_t)));  // (whoever arrives last at a counter puts it back to zero)
     VX_CHECK_HIP(hipMalloc(&be->prep_sync, VX_PREP_SYNC_BYTES));
     VX_CHECK_HIP(hipMemset(be->prep_sync, 0, VX_PREP_SYNC_BYTES));  // per-chunk sums of squares: every slot a prepare reads was written by the kernel before it
     {
@@ -114,6 +116,7 @@ void vx_backend_destroy(vx_backend *be) {
     if (be->misc_ws) (void)hipFree(be->misc_ws);
     if (be->prep_sync) (void)hipFree(be->prep_sync);
     if (be->rope_tab) (void)hipFree(be->rope_tab);
+    if (be->attn_cnt) (void)hipFree(be->attn_cnt);
     if (be->ones) (void)hipFree(be->ones);
     if (be->host_stage) (void)hipHostFree(be->host_stage);
     if (be->ev0) (void)hipEventDestroy(be->ev0);

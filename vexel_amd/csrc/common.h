@@ -45,6 +45,7 @@ struct PoolChunk {
 
 // chunk-parallel prepares: up to 64 rows x 64 chunks of 256 columns; two [64][64] float arrays of per-chunk sums of squares
 #define VX_ROPE_TAB_ROWS 64
+#define VX_ATTN_CNT 16384
 #define VX_ROPE_TAB_PAIRS 128
 #define VX_PREP_SYNC_ROWS 64
 #define VX_PREP_SYNC_CHUNKS 64
@@ -86,7 +87,9 @@ struct vx_backend {
     struct {
         int batch = 0, num_q_heads = 0, head_dim = 0, max_splits = 0, tokens_per_split = 0;
         const int32_t *kv_lens = nullptr;
+        int merged = 0;  // the attention kernel also left the merged rows as the prepared activation (gemm_ws)
     } split;
+    int32_t *attn_cnt = nullptr;  // arrival counters of the merging attention kernel, VX_ATTN_CNT of them, zero between launches
     size_t attn_ws_bytes = 0;
     // Work list of the ragged decode attention, written on the device by vx_pack_batch next to kv_lens:
     // buf[0] = number of items, then from buf[4] one record of four ints per item (batch index, split, kv

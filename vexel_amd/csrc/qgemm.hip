@@ -35,11 +35,12 @@
 #include <cstring>
 #include <algorithm>
 
+#include "prep_tiles.h"
+
 using namespace vx;
 
 namespace {
 
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
@@ -55,16 +56,7 @@ __device__ __forceinline__ float h2f(uint16_t h) {
 // a lane needs elements 4g..4g+3 and 16+4g..16+4g+3, i.e. two aligned float4 of the source row.
 
 // ---------------------------------------------------------------- activation prepare
-// Workspace layout (be->gemm_ws): inv_scale[Mpad], then tiles [K/32][Mpad/16][2][64] half8,
-// then bsum[K/32][Mpad] (block sums of the scaled row, for Q4_K's min term), then cscale[K/256][Mpad].
-struct PrepView {
-    half8 *tiles;
-    float *inv_scale;  // [Mpad] row factor: multiplies the finished dot products of the row
-    float *cscale;     // [K/256][Mpad] factor of each 256-column chunk's partial dot product
-    float *bsum;
-};
-
-__host__ __device__ inline size_t prep_tiles_bytes(int mpad, int k) { return (size_t)(k / 32) * (mpad / 16) * 2 * 64 * 16; }
+// (PrepView, the workspace layout and write_chunk: prep_tiles.h)
 
 enum { PREP_PLAIN = 0, PREP_RMSNORM = 1, PREP_SILU_MUL = 2 };
 
@@ -1307,53 +1299,9 @@ struct RowNorm {
     float inv_k, eps;
 };
 
-__device__ __forceinline__ float wave_max(float v) {
-    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-    return v;
-}
 __device__ __forceinline__ float wave_sum(float v) {
     for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     return v;
-}
-
-// Scales the wave's 256 values by a power of two chosen from their maximum, splits them hi + lo and writes the
-// MFMA-ready tiles, the block sums and the chunk factor of (row r, chunk c).
-__device__ __forceinline__ void write_chunk(const PrepView &pv, int r, int c, const float (&y)[4], int Mpad) {
-    const int lane = threadIdx.x & 63;
-    const float amax = wave_max(fmaxf(fmaxf(fabsf(y[0]), fabsf(y[1])), fmaxf(fabsf(y[2]), fabsf(y[3]))));
-    float s = 1.f, inv = 1.f;
-    if (amax > 0.f && amax < INFINITY) {
-        int ex;
-        (void)frexpf(amax, &ex);
-        s = ldexpf(1.f, 13 - ex);
-        inv = ldexpf(1.f, ex - 13);
-    }
-    if (lane == 0) pv.cscale[(size_t)c * Mpad + r] = inv;
-    // lane l = 8*step + 4*half + g holds block elements 16*half + 4g .. +3; slot order of lane group g is
-    // {4g, 4g+2, 16+4g, 16+4g+2, 4g+1, 4g+3, 16+4g+1, 16+4g+3}: the low-half lane fetches the high half's values
-    const float a[4] = {y[0] * s, y[1] * s, y[2] * s, y[3] * s};
-    float b[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++) b[i] = __shfl_down(a[i], 4, 64);
-    float bs = a[0] + a[1] + a[2] + a[3];
-    bs += __shfl_xor(bs, 1, 64);
-    bs += __shfl_xor(bs, 2, 64);
-    bs += __shfl_xor(bs, 4, 64);
-    const int step = c * 8 + (lane >> 3), half = (lane >> 2) & 1, g = lane & 3;
-    if (half == 0) {
-        const float v[8] = {a[0], a[2], b[0], b[2], a[1], a[3], b[1], b[3]};
-        half8 h, l;
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            h[i] = (_Float16)v[i];
-            l[i] = (_Float16)(v[i] - (float)h[i]);
-        }
-        const int mtiles = Mpad / 16, mt = r >> 4, ln = r & 15;
-        half8 *t = pv.tiles + ((size_t)(step * mtiles + mt) * 2) * 64 + g * 16 + ln;
-        t[0] = h;
-        t[64] = l;
-        if (g == 0) pv.bsum[(size_t)step * Mpad + r] = bs;
-    }
 }
 
 // Factor of row r's finished dot products: the stored row factor times, for a pending RMSNorm, 1/rms from the
@@ -1447,20 +1395,7 @@ __global__ void __launch_bounds__(64) chunk_merge_kernel(const float *__restrict
     float y[4] = {0.f, 0.f, 0.f, 0.f};
     if (r < M) {
         const int ns = min((kv_lens[r] + tokens_per_split - 1) / tokens_per_split, max_splits);
-        const int P = D + 2, h = k / D, d = k % D;
-        const float *pb = part + ((size_t)r * (K / D) + h) * max_splits * P;
-        float Mx = -INFINITY;
-        for (int s = 0; s < ns; s++) Mx = fmaxf(Mx, pb[(size_t)s * P]);
-        float L = 0.f, A[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int s = 0; s < ns; s++) {
-            const float *ps = pb + (size_t)s * P;
-            const float f = exp2f(ps[0] - Mx);
-            L += ps[1] * f;
-            const float2 a = *(const float2 *)(ps + 2 + d), b = *(const float2 *)(ps + 4 + d);
-            A[0] += a.x * f; A[1] += a.y * f; A[2] += b.x * f; A[3] += b.y * f;
-        }
-#pragma unroll
-        for (int e = 0; e < 4; e++) y[e] = (L > 0.f) ? A[e] / L : 0.f;
+        split_merge4(part, ns, K / D, D, max_splits, r, k, y);
     }
     write_chunk(pv, r, c, y, Mpad);
     if (c == 0 && lane == 0) pv.inv_scale[r] = r < M ? 1.f : 0.f;
@@ -1664,6 +1599,7 @@ int prep_begin(vx_backend *be, int m, int k, PrepView *pv) {
     if (rc) return rc;
     be->rowfac_slot ^= 1;
     be->prep_norm_k = 0;
+    be->split.merged = 0;  // whatever the attention kernel prepared is overwritten
     *pv = prep_view(be, mpad, k);
     be->prep_m = m;
     be->prep_k = k;
@@ -2072,6 +2008,16 @@ static Segs make_segs(const vx_qweight *const *ws, int nw, int *ntot) {
 
 // The chunk-parallel prepares cover decode-sized batches; larger ones keep the one-workgroup-per-row kernels.
 bool chunk_prepare_ok(int rows, int k) { return mpad_for(rows) <= VX_PREP_SYNC_ROWS && k / 256 <= VX_PREP_SYNC_CHUNKS; }
+
+extern "C++" {
+namespace vx {
+int prep_begin_chunked(vx_backend *be, int m, int k, PrepView *pv, int *mpad) {
+    if (k < 256 || k % 256 != 0 || !chunk_prepare_ok(m, k)) return VX_ERR_UNSUPPORTED;
+    *mpad = mpad_for(m);
+    return prep_begin(be, m, k, pv);
+}
+}  // namespace vx
+}
 int vx_rope_table_prepare(vx_backend *be, const int32_t *positions, int rows, int head_dim, float theta) {
     int rc = enter(be);
     if (rc) return rc;
@@ -2288,12 +2234,21 @@ int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight 
         }
     }
     int ks, ntot;
+    // (the attention kernel may already have left the merged result in the prepared form: only where the workspace
+    // still is where that kernel wrote it)
+    const void *ws_before = be->gemm_ws;
+    const size_t ws_bytes_before = be->gemm_ws_bytes;
     rc = prep_reserve(be, rows, ffn > wo->k ? (ffn > hidden ? ffn : hidden) : (wo->k > hidden ? wo->k : hidden));
     if (rc) return rc;
+    const bool merged = !attn && be->split.merged && be->gemm_ws == ws_before && be->gemm_ws_bytes == ws_bytes_before &&
+                        be->prep_m == rows && be->prep_k == wo->k;
+    be->split.merged = 0;
     // attention output -> Wo -> partials
     if (attn) {
         rc = vx_prepare_act(be, attn, rows, wo->k);
         if (rc) return rc;
+    } else if (merged) {
+        be->split.batch = 0;
     } else {
         PrepView pa;
         rc = prep_begin(be, rows, wo->k, &pa);
