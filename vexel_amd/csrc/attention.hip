@@ -204,7 +204,19 @@ struct MergeOut {
     PrepView pv;
     int32_t *cnt = nullptr;
     int mpad = 0;
+    float *plain = nullptr;  // != nullptr: the merged rows as plain float32 [row][heads * D] instead (a single row's matrix-vector product reads that)
 };
+
+// The wave's 256 merged columns (chunk c of row `row`, four per lane): as a chunk of the prepared operand or as floats.
+__device__ __forceinline__ void put_merged(const MergeOut &mg, int row, int c, const float (&y)[4], int K) {
+    const int lane = threadIdx.x & 63;
+    if (mg.plain) {
+        *(float4 *)(mg.plain + (size_t)row * K + c * 256 + lane * 4) = make_float4(y[0], y[1], y[2], y[3]);
+        return;
+    }
+    write_chunk(mg.pv, row, c, y, mg.mpad);
+    if (c == 0 && lane == 0) mg.pv.inv_scale[row] = 1.f;
+}
 
 // RG > 1: an entry of the batch is RG consecutive query rows that share one sequence's context (the rows of a
 // candidate tree): the workgroup serves the G*RG queries (row, head) of its kv head from one pass over the K/V.
@@ -213,7 +225,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix,
     const int32_t *__restrict__ bt_rows, int max_blocks, const int32_t *__restrict__ kv_lens,
     float *__restrict__ partial, int num_q_heads, int num_kv_heads, float scale, int max_splits,
-    const int32_t *__restrict__ items, MergeOut mg) {
+    const int32_t *__restrict__ items, MergeOut mg, int tps) {
     constexpr int GG = G * RG;       // queries per K/V row
     constexpr int DL = D / 8;        // 8-element slices of a head vector
     // lanes per token: the next power of two; the lanes past DL (heads of 80 or 96) repeat the last slice's loads
@@ -239,8 +251,8 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     // The caller's max_kv_len sized the partial sums (max_splits per sequence and head). A length above it is
     // attended over its first max_splits * TPW tokens by every kernel of the path alike: defined, and inside the
     // buffers.
-    kv_len = min(kv_len, max_splits * TPW);
-    const int t_begin = split * TPW;
+    kv_len = min(kv_len, max_splits * tps);  // (tps: tokens per split, a multiple of the block size; ATTN_TPW with a work list)
+    const int t_begin = split * tps;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     constexpr int GD = G * D;                          // this workgroup's columns of the output
@@ -252,16 +264,12 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
         if constexpr (MERGES) {
             if (mg.cnt && kv_len == 0 && split == 0 && kvh % HPC == 0) {
                 const float zero[4] = {0.f, 0.f, 0.f, 0.f};
-                for (int ch = wave; ch < CH; ch += 4) {
-                    const int c = kvh / HPC * CH + ch;
-                    write_chunk(mg.pv, seq, c, zero, mg.mpad);
-                    if (c == 0 && lane == 0) mg.pv.inv_scale[seq] = 1.f;
-                }
+                for (int ch = wave; ch < CH; ch += 4) put_merged(mg, seq, kvh / HPC * CH + ch, zero, num_q_heads * D);
             }
         }
         return;
     }
-    const int t_end = min(kv_len, t_begin + TPW);
+    const int t_end = min(kv_len, t_begin + tps);
     const int32_t *bt = bt_matrix + (size_t)row * max_blocks + t_begin / HOT_BS;
 
     const int tl = lane / LPT;  // token slot within a load
@@ -405,7 +413,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
         __shared__ int s_last;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        const int ns = (kv_len + TPW - 1) / TPW;  // workgroups of one kv head that arrive for this sequence
+        const int ns = (kv_len + tps - 1) / tps;  // workgroups of one kv head that arrive for this sequence
         const int unit = kvh / HPC;
         if (tid == 0) {
             int32_t *cnt = mg.cnt + (size_t)seq * (num_kv_heads / HPC) + unit;
@@ -419,8 +427,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
             const int c = unit * CH + ch;
             float y[4];
             split_merge4<true>(partial, ns, num_q_heads, D, max_splits, seq, c * 256 + lane * 4, y);
-            write_chunk(mg.pv, seq, c, y, mg.mpad);
-            if (c == 0 && lane == 0) mg.pv.inv_scale[seq] = 1.f;
+            put_merged(mg, seq, c, y, num_q_heads * D);
         }
     }
 }
@@ -438,10 +445,10 @@ __global__ void gather_tables_kernel(const int32_t *const *bt_ptrs, const int32_
 template <int D>
 __global__ void __launch_bounds__(D) paged_merge_kernel(const float *__restrict__ partial,
                                                         const int32_t *__restrict__ kv_lens, float *__restrict__ out,
-                                                        int num_q_heads, int max_splits) {
+                                                        int num_q_heads, int max_splits, int tps) {
     const int qh = blockIdx.x, seq = blockIdx.y, d = threadIdx.x;
     const int kv_len = kv_lens[seq];
-    const int ns = min((kv_len + TPW - 1) / TPW, max_splits);  // a length over the caller's bound: its first max_splits splits
+    const int ns = min((kv_len + tps - 1) / tps, max_splits);  // a length over the caller's bound: its first max_splits splits
     const float *pb = partial + ((size_t)seq * num_q_heads + qh) * max_splits * (D + 2);
     float M = -INFINITY;
     for (int s = 0; s < ns; s++) M = fmaxf(M, pb[(size_t)s * (D + 2)]);
@@ -715,13 +722,22 @@ template <int D, int G>
 int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *bt_matrix, const int32_t *bt_rows,
                int max_blocks, const int32_t *kv_lens, float *out, int batch, int num_q_heads, int num_kv_heads,
                float scale, int max_kv_len, bool fixed) {
-    int max_splits = ceil_div(max_kv_len, TPW);
-    size_t need = (size_t)batch * num_q_heads * max_splits * (D + 2) * sizeof(float);
+    // Tokens per split: ATTN_TPW; a quarter of it at least when that many splits would leave most of the chip
+    // idle (a single sequence). The work list from vx_pack_batch is cut in ATTN_TPW tokens, so it serves the first only.
+    int tps = TPW;
+    static const int cus = [&] {
+        int n = 0;
+        return (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, be->device) == hipSuccess && n > 0) ? n : 256;
+    }();
+    while (tps > TPW / 4 && (size_t)batch * num_kv_heads * ceil_div(max_kv_len, tps) < (size_t)2 * cus) tps /= 2;
+    int max_splits = ceil_div(max_kv_len, tps);
+    const size_t partial_floats = ((size_t)batch * num_q_heads * max_splits * (D + 2) + 3) & ~(size_t)3;
+    const size_t need = (partial_floats + (batch == 1 ? (size_t)num_q_heads * D : 0)) * sizeof(float);
     float *ws;
     if (fixed) {
         if (need > FIXED_WS_BYTES || !be->attn_fixed_ws) {
             set_error("vx_sdpa_paged_decode_ragged_noalloc: %d sequences x %d heads x %d splits of %d tokens need %zu bytes of "
-                      "partial sums, the fixed area holds %zu", batch, num_q_heads, max_splits, TPW, need, FIXED_WS_BYTES);
+                      "partial sums, the fixed area holds %zu", batch, num_q_heads, max_splits, tps, need, FIXED_WS_BYTES);
             return VX_ERR_INVALID;
         }
         ws = (float *)be->attn_fixed_ws;
@@ -732,45 +748,52 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
     }
     // With a work list from vx_pack_batch for these lengths the grid's second dimension runs over its items
     // (at most max_splits per sequence, as max_kv_len bounds every length); otherwise over (split, sequence).
-    const bool listed = be->items.valid && be->items.kv_lens == kv_lens && be->items.table_rows == bt_rows &&
+    const bool listed = tps == TPW && be->items.valid && be->items.kv_lens == kv_lens && be->items.table_rows == bt_rows &&
                         be->items.batch == batch &&
                         ((size_t)batch * max_splits + 1) * 4 <= be->items.bytes / sizeof(int32_t) &&
                         (size_t)batch * max_splits <= 65535;
     dim3 grid(num_kv_heads, listed ? batch * max_splits : max_splits, listed ? 1 : batch);
     // out == NULL leaves the result to vx_decode_ffn(attn = NULL): as split partial sums, and - where the shape
-    // allows - already merged and prepared as that call's first operand by the workgroups that finish last.
+    // allows - already merged by the workgroups that finish last: prepared as that call's first operand, or, for
+    // a single row, as plain floats behind the partial sums (what the matrix-vector product reads).
     MergeOut mg;
+    float *plain = nullptr;
     static const bool no_merge = getenv("VEXEL_HIP_NO_ATTN_MERGE") != nullptr;
     constexpr int GD = G * D;
     constexpr int HPC = (GD < 256 && 256 % GD == 0) ? 256 / GD : 0;  // kv heads that share a chunk
     const bool mergeable = GD % 256 == 0 || (HPC > 0 && num_kv_heads % HPC == 0);
-    if (!out && !fixed && !no_merge && batch >= 2 && mergeable && be->attn_cnt &&
-        (size_t)batch * num_kv_heads <= VX_ATTN_CNT) {
-        int mpad = 0;
-        const int rc = prep_begin_chunked(be, batch, num_q_heads * D, &mg.pv, &mpad);
-        if (rc == VX_OK) {
+    if (!out && !fixed && !no_merge && mergeable && be->attn_cnt && (size_t)batch * num_kv_heads <= VX_ATTN_CNT) {
+        if (batch == 1) {
             mg.cnt = be->attn_cnt;
-            mg.mpad = mpad;
-        } else if (rc != VX_ERR_UNSUPPORTED)
-            return rc;
+            mg.plain = plain = ws + partial_floats;
+        } else {
+            int mpad = 0;
+            const int rc = prep_begin_chunked(be, batch, num_q_heads * D, &mg.pv, &mpad);
+            if (rc == VX_OK) {
+                mg.cnt = be->attn_cnt;
+                mg.mpad = mpad;
+            } else if (rc != VX_ERR_UNSUPPORTED)
+                return rc;
+        }
     }
     paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
                                                                 max_blocks, kv_lens, ws, num_q_heads,
                                                                 num_kv_heads, scale, max_splits,
-                                                                listed ? be->items.buf : nullptr, mg);
+                                                                listed ? be->items.buf : nullptr, mg, tps);
     VX_CHECK_LAUNCH();
     if (!fixed) be->split.batch = 0;  // (the fixed area is not where vx_decode_ffn looks for a split result)
     if (!out) {  // the caller merges: vx_decode_ffn(attn = NULL)
-        be->split.merged = mg.cnt != nullptr;
+        be->split.merged = mg.cnt != nullptr && !plain;
+        be->split.plain = plain;
         be->split.batch = batch;
         be->split.num_q_heads = num_q_heads;
         be->split.head_dim = D;
         be->split.max_splits = max_splits;
-        be->split.tokens_per_split = TPW;
+        be->split.tokens_per_split = tps;
         be->split.kv_lens = kv_lens;
         return VX_OK;
     }
-    paged_merge_kernel<D><<<dim3(num_q_heads, batch), D, 0, be->stream>>>(ws, kv_lens, out, num_q_heads, max_splits);
+    paged_merge_kernel<D><<<dim3(num_q_heads, batch), D, 0, be->stream>>>(ws, kv_lens, out, num_q_heads, max_splits, tps);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }
@@ -1144,7 +1167,7 @@ int vx_sdpa_paged_tree_batched(vx_backend *be, const float *q, const void *kv_po
     if (head_dim == DD && G == GG)                                                                                        \
         paged_decode_f16_kernel<DD, GG, RR><<<grid, 256, 0, be->stream>>>(q, pool, block_tables, entry_table_rows, max_blocks, \
                                                                         entry_kv_lens, ws, num_q_heads, num_kv_heads, scale, \
-                                                                        max_splits, nullptr, MergeOut{});
+                                                                        max_splits, nullptr, MergeOut{}, TPW);
         VX_TREE(128, 1, 8) VX_TREE(128, 2, 4) VX_TREE(128, 4, 2) VX_TREE(128, 8, 1)
         VX_TREE(64, 1, 8) VX_TREE(64, 2, 4) VX_TREE(64, 4, 2) VX_TREE(64, 8, 1)
 #undef VX_TREE

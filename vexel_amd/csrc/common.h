@@ -88,6 +88,7 @@ struct vx_backend {
         int batch = 0, num_q_heads = 0, head_dim = 0, max_splits = 0, tokens_per_split = 0;
         const int32_t *kv_lens = nullptr;
         int merged = 0;  // the attention kernel also left the merged rows as the prepared activation (gemm_ws)
+        const float *plain = nullptr;  // a single row: the attention kernel also left the merged row here, as floats
     } split;
     int32_t *attn_cnt = nullptr;  // arrival counters of the merging attention kernel, VX_ATTN_CNT of them, zero between launches
     size_t attn_ws_bytes = 0;

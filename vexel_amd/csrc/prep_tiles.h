@@ -66,7 +66,8 @@ __device__ __forceinline__ void write_chunk(const PrepView &pv, int r, int c, co
 
 // Columns k .. k+3 of row r's attention output from its split partial sums (per row and head: max_splits records
 // of [running maximum, sum of weights, D weighted value sums], the first ns of them written), as
-// paged_merge_kernel computes it: splits added in index order.
+// paged_merge_kernel computes it for up to eight splits (splits added in index order; beyond eight, in groups of eight
+// under a running maximum).
 // DEVICE_SCOPE: the records were written by other workgroups of the running launch with device-scope stores; every
 // value is read by a device-scope load, which is served from where those stores went and not from this compute
 // unit's or this die's cache.
@@ -78,28 +79,29 @@ __device__ __forceinline__ void split_merge4(const float *__restrict__ part, int
     };
     const int P = D + 2, h = k / D, d = k % D;
     const float *pb = part + ((size_t)r * num_heads + h) * max_splits * P;
-    // (four splits' loads in flight at a time: the device-scope ones each cost a trip to memory)
-    float Mx = -INFINITY;
-    for (int s0 = 0; s0 < ns; s0 += 4) {
-        float m[4];
+    // Eight splits at a time, all their loads in flight together (a device-scope load is a trip to memory): the
+    // running maximum moves up between the groups and what was added so far is rescaled, the first group from zero.
+    float Mx = -INFINITY, L = 0.f, A[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < ns; s0 += 8) {
+        float v[8][6];
 #pragma unroll
-        for (int j = 0; j < 4; j++) m[j] = s0 + j < ns ? ld(pb + (size_t)(s0 + j) * P) : -INFINITY;
-#pragma unroll
-        for (int j = 0; j < 4; j++) Mx = fmaxf(Mx, m[j]);
-    }
-    float L = 0.f, A[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < ns; s0 += 4) {
-        float v[4][6];
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < 8; j++) {
             const float *ps = pb + (size_t)min(s0 + j, ns - 1) * P;
             v[j][0] = ld(ps);
             v[j][1] = ld(ps + 1);
 #pragma unroll
             for (int e = 0; e < 4; e++) v[j][2 + e] = ld(ps + 2 + d + e);
         }
+        float Mn = Mx;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
+        for (int j = 0; j < 8; j++) Mn = fmaxf(Mn, s0 + j < ns ? v[j][0] : -INFINITY);
+        const float keep = (Mx == -INFINITY) ? 0.f : exp2f(Mx - Mn);
+        Mx = Mn;
+        L *= keep;
+#pragma unroll
+        for (int e = 0; e < 4; e++) A[e] *= keep;
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
             if (s0 + j >= ns) break;
             const float f = exp2f(v[j][0] - Mx);
             L += v[j][1] * f;

@@ -2209,6 +2209,9 @@ int vx_decode_ffn(vx_backend *be, const float *attn, float *x, const vx_qweight 
             if (attn) {
                 VX_REQUIRE((uintptr_t)attn % 16 == 0, "vx_decode_ffn: unaligned pointer");
                 s1.x = attn;
+            } else if (be->split.plain) {
+                s1.x = be->split.plain;
+                be->split.batch = 0;
             } else {
                 s1.attn_partial = (const float *)be->attn_ws;
                 s1.kv_len = be->split.kv_lens;

@@ -486,6 +486,241 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec_kernel(const MvArgs p) {
     }
 }
 
+int device_cus(vx_backend *be);
+
+// ---- Q4_0, second form: whole rows per wave, the activation's integer planes in LDS.
+// The kernel above spends most of its instructions around its loads (per-trip address arithmetic, a workgroup
+// barrier per 8 rows, every workgroup preparing its lanes' activations again per K segment). Here a workgroup
+// prepares the row's planes once, into LDS; after that its waves do not meet again. A wave takes passes of NR
+// consecutive rows (with `pair`: NR/2 rows of each matrix): their bytes are one contiguous run, read as aligned
+// 16-byte pieces, lane l piece l + 64 i - the pattern memory serves fastest - into registers, the next pass in
+// flight while the current one is worked on; the pieces go to the wave's own LDS rows, from where lane l takes
+// block t*64 + l of every row of the pass (18-byte stride, any alignment) against the planes of that block, read
+// once per step for all NR rows. One butterfly over the wave per row at the end of the pass. The arithmetic of a
+// block is VQ4_0::block's.
+constexpr int MV2_XSTRIDE = 28;  // dwords per block in LDS: planes [3][8], sum of xi, inv; padded to whole 16-byte pieces
+
+// x: the block's 28 dwords; w: its 16 code bytes; d: its scale
+__device__ __forceinline__ float mv2_q4_0_dot(const uint32_t (&w)[4], uint32_t d, const uint32_t (&x)[MV2_XSTRIDE]) {
+    int a0 = 0, a1 = 0, a2 = 0;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const uint32_t lo = w[i] & 0x0F0F0F0Fu, hi = (w[i] >> 4) & 0x0F0F0F0Fu;
+        a0 = (int)__builtin_amdgcn_udot4(lo, x[i], (uint32_t)a0, false);
+        a1 = (int)__builtin_amdgcn_udot4(lo, x[8 + i], (uint32_t)a1, false);
+        a2 = __builtin_amdgcn_sdot4((int)lo, (int)x[16 + i], a2, false);
+        a0 = (int)__builtin_amdgcn_udot4(hi, x[4 + i], (uint32_t)a0, false);
+        a1 = (int)__builtin_amdgcn_udot4(hi, x[12 + i], (uint32_t)a1, false);
+        a2 = __builtin_amdgcn_sdot4((int)hi, (int)x[20 + i], a2, false);
+    }
+    const int t = a0 + (a1 << 8) + (a2 << 16) - 8 * (int)x[24];  // sum (q - 8) xi, exact
+    return h2f((uint16_t)d) * ((float)t * __uint_as_float(x[25]));
+}
+
+__device__ __forceinline__ float wave_sum64(float t) {
+    t = half_wave_sum(t);
+    return t + __shfl_xor(t, 32, 64);
+}
+
+// NR rows per pass, NPL 16-byte pieces per lane and pass (64 * NPL >= NR * row_bytes / 16). Every matrix (with
+// `pair`: each of the two) holds a multiple of NR (NR/2) rows and whole 16-byte rows: the host checks.
+template <int NR, int NPL>
+__global__ void __launch_bounds__(MV_THREADS) qmatvec2_kernel(const MvArgs p, int n_passes) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) uint32_t smem[];  // planes [nblocks + 1][MV2_XSTRIDE] (the last block zeros), then the waves' rows
+    __shared__ float s_ss[MV_WAVES];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int K = p.K, nblocks = K / 32, pair = p.pair;
+    const int T = (nblocks + 63) / 64;
+    const int rb = (int)p.row_bytes;
+    const int total = NR * (rb / 16);         // pieces of a pass
+    const int half_pieces = total / 2;        // pair: pieces of each matrix' share
+    uint8_t *my = (uint8_t *)(smem + (size_t)(nblocks + 1) * MV2_XSTRIDE) + (size_t)wave * (NR * rb + 16);
+
+    // Pass q: rows [q * NR, q * NR + NR) of the concatenated rows; with pair, rows [q * NR/2, ...) of both matrices.
+    auto issue = [&](int q, u32x4 (&pc)[NPL]) __attribute__((always_inline)) {
+        const uint8_t *b0, *b1;
+        if (pair > 0) {
+            b0 = p.w0 + (size_t)q * (NR / 2) * rb;
+            b1 = p.w1 + (size_t)q * (NR / 2) * rb - (size_t)half_pieces * 16;
+        } else {
+            const int row = q * NR;
+            const uint8_t *base = row < p.end0 ? p.w0 : (row < p.end1 ? p.w1 : p.w2);
+            const int local = row < p.end0 ? row : (row < p.end1 ? row - p.end0 : row - p.end1);
+            b0 = b1 = base + (size_t)local * rb;
+        }
+#pragma unroll
+        for (int i = 0; i < NPL; i++) {
+            const int c = min(lane + 64 * i, total - 1);
+            const uint8_t *b = (pair > 0 && c >= half_pieces) ? b1 : b0;
+            pc[i] = *(const u32x4 *)(b + (size_t)c * 16);
+        }
+    };
+    const int n_waves = gridDim.x * MV_WAVES;
+    int q = blockIdx.x * MV_WAVES + wave;
+
+    // The activation's first loads go ahead of the weights': behind them they would wait for all of those.
+    float4 xv[8], nv[8];
+    if (tid < nblocks) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) xv[i] = *(const float4 *)(p.x + (size_t)tid * 32 + 4 * i);
+        if (p.mode == MV_RMSNORM) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) nv[i] = *(const float4 *)(p.norm_w + (size_t)tid * 32 + 4 * i);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    u32x4 pc[NPL];
+    if (q < n_passes) issue(q, pc);
+    __builtin_amdgcn_sched_barrier(0);
+
+    // activation -> integer planes in LDS (XInt<23>), one block per thread and trip
+    float ss = 0.f;
+    for (int j = tid; j < nblocks; j += MV_THREADS) {
+        if (j != tid) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) xv[i] = *(const float4 *)(p.x + (size_t)j * 32 + 4 * i);
+            if (p.mode == MV_RMSNORM) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) nv[i] = *(const float4 *)(p.norm_w + (size_t)j * 32 + 4 * i);
+            }
+        }
+        float v[32];
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            v[4 * i] = xv[i].x; v[4 * i + 1] = xv[i].y; v[4 * i + 2] = xv[i].z; v[4 * i + 3] = xv[i].w;
+        }
+        if (p.mode == MV_RMSNORM) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                const float wv[4] = {nv[i].x, nv[i].y, nv[i].z, nv[i].w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    ss = fmaf(v[4 * i + e], v[4 * i + e], ss);
+                    v[4 * i + e] *= wv[e];
+                }
+            }
+        }
+        XInt<23> x;
+        x.prep(v);
+        uint32_t *dst = smem + (size_t)j * MV2_XSTRIDE;
+#pragma unroll
+        for (int pl = 0; pl < 3; pl++) {
+            *(u32x4 *)(dst + pl * 8) = u32x4{x.p[pl][0], x.p[pl][1], x.p[pl][2], x.p[pl][3]};
+            *(u32x4 *)(dst + pl * 8 + 4) = u32x4{x.p[pl][4], x.p[pl][5], x.p[pl][6], x.p[pl][7]};
+        }
+        *(u32x4 *)(dst + 24) = u32x4{(uint32_t)(x.s0 + x.s1), __float_as_uint(x.inv), 0u, 0u};
+    }
+    if (tid < MV2_XSTRIDE) smem[(size_t)nblocks * MV2_XSTRIDE + tid] = 0u;
+    float row_fac = 1.f;
+    if (p.mode == MV_RMSNORM) {  // 1/rms of the row: lanes by a fixed butterfly, then the waves in order (cpu.go:200-220)
+        for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+        if (lane == 0) s_ss[wave] = ss;
+    }
+    __syncthreads();
+    if (p.mode == MV_RMSNORM) {
+        const float tot = (s_ss[0] + s_ss[1]) + (s_ss[2] + s_ss[3]);
+        row_fac = 1.0f / (float)sqrt((double)(tot / (float)K + p.eps));
+    }
+
+    // one pass: its pieces to the wave's LDS rows, the next pass on its way into the same registers, then the rows'
+    // dot products
+    auto pass = [&](int q, u32x4 (&pc)[NPL]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NPL; i++) {
+            const int c = lane + 64 * i;
+            if (c < total) *(u32x4 *)(my + (size_t)c * 16) = pc[i];
+        }
+        // (the wave reads only what it wrote itself: its LDS operations are ordered, no barrier)
+        if (q + n_waves < n_passes) issue(q + n_waves, pc);
+        float acc[NR];
+#pragma unroll
+        for (int r = 0; r < NR; r++) acc[r] = 0.f;
+        for (int t = 0; t < T; t++) {
+            const int j = t * 64 + lane;
+            const int jx = j < nblocks ? j : nblocks;   // past the row's end: the zero planes
+            const int jw = min(j, nblocks - 1);
+            uint32_t x[MV2_XSTRIDE];
+#pragma unroll
+            for (int i = 0; i < MV2_XSTRIDE / 4; i++) {
+                const u32x4 f = *(const u32x4 *)(smem + (size_t)jx * MV2_XSTRIDE + 4 * i);
+                x[4 * i] = f[0]; x[4 * i + 1] = f[1]; x[4 * i + 2] = f[2]; x[4 * i + 3] = f[3];
+            }
+#pragma unroll
+            for (int r = 0; r < NR; r++) {
+                const int o = r * rb + jw * 18;
+                uint32_t w[4];
+                lds_dwords<4>(my, o + 2, w);
+                acc[r] += mv2_q4_0_dot(w, lds_u16(my, o), x);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < NR; r++) acc[r] = wave_sum64(acc[r]) * row_fac;
+        if (pair > 0) {
+            float g = acc[0], u = acc[NR / 2];
+#pragma unroll
+            for (int r = 1; r < NR / 2; r++) {
+                g = lane == r ? acc[r] : g;
+                u = lane == r ? acc[NR / 2 + r] : u;
+            }
+            if (lane < NR / 2) p.out[q * (NR / 2) + lane] = __fmul_rn(__fmul_rn(g, mv_sigmoid(g)), u);  // cpu.go:390-400
+        } else {
+            float v = acc[0];
+#pragma unroll
+            for (int r = 1; r < NR; r++) v = lane == r ? acc[r] : v;
+            if (lane < NR) {
+                const int row = q * NR + lane;
+                if (p.residual) v = __fadd_rn(p.residual[row], v);
+                p.out[row] = v;
+            }
+        }
+    };
+    for (; q < n_passes; q += n_waves) pass(q, pc);
+}
+
+template <int NR, int NPL>
+void launch_second(vx_backend *be, MvArgs &a, size_t lds) {
+    static int per_cu = 0;
+    if (per_cu == 0) {
+        (void)hipFuncSetAttribute((const void *)qmatvec2_kernel<NR, NPL>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, qmatvec2_kernel<NR, NPL>, MV_THREADS, lds) != hipSuccess || per_cu < 1)
+            per_cu = 1;
+    }
+    const int n_passes = a.pair > 0 ? a.pair / (NR / 2) : a.N / NR;
+    // as many workgroups as fit at once, or fewer when that makes every wave's number of passes equal
+    const int wgs = ceil_div(n_passes, MV_WAVES);
+    const int trips = ceil_div(wgs, per_cu * device_cus(be));
+    qmatvec2_kernel<NR, NPL><<<ceil_div(wgs, trips), MV_THREADS, lds, be->stream>>>(a, n_passes);
+}
+
+// Launches the second form when it serves the call: Q4_0, an activation row from memory, rows of whole 16-byte
+// pieces, every matrix a whole number of passes.
+bool launch_second_form(vx_backend *be, int fmt, MvArgs &a) {
+    static const bool off = getenv("VEXEL_HIP_MATVEC_FIRST_FORM") != nullptr;
+    if (off || fmt != VX_Q4_0 || a.mode == MV_MERGED_ATTENTION) return false;
+    const int nblocks = a.K / 32;
+    const size_t rb = (size_t)nblocks * 18;
+    if (rb % 16 != 0) return false;
+    int nr, npl;
+    if (4 * rb / 16 <= 64 * 9) nr = 4, npl = 9;         // K <= 4096
+    else if (2 * rb / 16 <= 64 * 9) nr = 2, npl = 9;    // K <= 8192
+    else if (2 * rb / 16 <= 64 * 13) nr = 2, npl = 13;  // K <= 11776
+    else return false;
+    const int unit = a.pair > 0 ? nr / 2 : nr;
+    if (a.pair > 0) {
+        if (a.pair % unit != 0) return false;
+    } else if (a.end0 % unit != 0 || a.end1 % unit != 0 || a.N % unit != 0)
+        return false;
+    const size_t lds = (size_t)(nblocks + 1) * MV2_XSTRIDE * 4 + MV_WAVES * (nr * rb + 16);
+    if (lds > 120 * 1024) return false;
+    a.row_bytes = rb;
+    if (nr == 4) launch_second<4, 9>(be, a, lds);
+    else if (npl == 9) launch_second<2, 9>(be, a, lds);
+    else launch_second<2, 13>(be, a, lds);
+    return true;
+}
+
 int device_cus(vx_backend *be) {
     static int cus = 0;
     if (cus == 0) {
@@ -570,6 +805,10 @@ bool shape_ok(int k) {
 }
 
 int launch_fmt(vx_backend *be, int fmt, MvArgs &a) {
+    if (launch_second_form(be, fmt, a)) {
+        VX_CHECK_LAUNCH();
+        return VX_OK;
+    }
     switch (fmt) {
     case VX_Q4_0: return launch<VQ4_0>(be, a);
     case VX_Q8_0: return launch<VQ8_0>(be, a);
