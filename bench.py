@@ -34,7 +34,9 @@ BLOCK = 16
 
 # HBM bytes per algorithmic byte of the attention launch, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs
 # scaled by a plain copy of known size (summary: profiles/paged_decode_attention_7b_x32_hbm_traffic.txt).
-ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.008
+ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.013
+# the same for the step's four projection launches per layer at 32 rows (reductions of the k-slices included)
+GEMM_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.27
 
 
 def ragged_contexts(seed=0, n=BATCH):
@@ -332,7 +334,9 @@ def time_step_gemms(be, mr, c, rows):
         be.free(p)
     return {"bound": "hbm", "kernel": "qgemm_wave_kernel (the step's four projection launches per layer, M=%d)" % rows,
             "achieved": total_bytes / total_us / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": total_bytes / total_us / 1e3 / HBM_PEAK_GBS, "bytes_per_layer": total_bytes,
+            "frac": total_bytes / total_us / 1e3 / HBM_PEAK_GBS,
+            "traffic": GEMM_TRAFFIC_PER_ALGORITHMIC_BYTE * total_bytes if rows == BATCH else None,
+            "bytes_per_layer": total_bytes,
             "us_per_layer": total_us, "launches": res,
             "note": "HIP events around back-to-back launches over all layers' weights; a launch with split K "
                     "includes its reduction kernel"}
@@ -434,7 +438,8 @@ def kernel_report(be):
 
 def counter_probe(be, mr, ctx, c, layers):
     """Workload for hardware-counter runs: plain_copy_kernel moves 1 GiB (known traffic, the scale for
-    FETCH_SIZE / WRITE_SIZE), then the attention kernel runs 8 times on the benchmark contexts."""
+    FETCH_SIZE / WRITE_SIZE), then the attention kernel runs 8 times on the benchmark contexts, then the step's
+    four quantized projection launches per layer run over every layer's weights."""
     synth = load_synth()
     n = 1 << 30
     src, dst = be.alloc_permanent(n), be.alloc_permanent(n)
@@ -442,8 +447,10 @@ def counter_probe(be, mr, ctx, c, layers):
     if rc:
         raise RuntimeError("plain copy failed: %d" % rc)
     ms = time_attention_kernel(be, mr, ctx, c, layers, reps=8)
-    print(json.dumps({"probe": "plain_copy_kernel 1 GiB + 8 attention launches", "attention_bytes": attention_bytes(ctx, c),
-                      "attention_ms": ms}))
+    gm = time_step_gemms(be, mr, c, len(ctx))   # every layer's four projection launches, weights streamed from HBM
+    print(json.dumps({"probe": "plain_copy_kernel 1 GiB + 8 attention launches + the step's projection launches",
+                      "attention_bytes": attention_bytes(ctx, c), "attention_ms": ms,
+                      "projection_launches": gm["launches"] if gm else None}))
 
 
 def prefill_probe(be, rows=512, reps=10):
