@@ -148,11 +148,10 @@ def test_matmul_quant_vs_oracle(be, fmt, m):
 
 @pytest.mark.parametrize("fmt", FMTS_MFMA)
 def test_matmul_rows_independent_of_batch(be, fmt):
-    """A row has the same bits in a batch of 2, of 32 and of 72 (the k-slices and the order their sums are added in
-    depend on the matrix and the device only; up to 32 rows the slices are separate workgroups, beyond that one
-    workgroup walks them in the same order; cf. the reference's loop of M=1 kernels,
-    backend/metal/backend.go:777-779). A single row (M = 1) goes through the matrix-vector kernel, whose
-    arithmetic differs: it agrees to rounding, not bit for bit."""
+    """A row has the same bits in a batch of 2 and of 32, and the same bits in a batch of 40 and of 72: the k-slices
+    and the order their sums are added in depend on the matrix, the device and the kernel only, and the kernel
+    changes at 32 rows (cf. the reference's loop of M=1 kernels, backend/metal/backend.go:777-779). Across that
+    boundary, and for a single row (M = 1, the matrix-vector kernel), rows agree to rounding, not bit for bit."""
     rng = np.random.default_rng(9)
     m, n, k = 32, 96, 2048
     w = qz.random_quant(fmt, rng, n, k)
@@ -165,9 +164,12 @@ def test_matmul_rows_independent_of_batch(be, fmt):
     dbig = be.alloc(72 * n * 4)
     be.matmul_quant(fmt, da, dw, dbig, None, 72, n, k)
     many = be.download(dbig, (72, n), np.float32)
-    assert np.array_equal(many[:m].view(np.uint32), full.view(np.uint32))
+    d40 = be.alloc(40 * n * 4)
+    be.matmul_quant(fmt, da, dw, d40, None, 40, n, k)
+    assert np.array_equal(many[:40].view(np.uint32), be.download(d40, (40, n), np.float32).view(np.uint32))
     want = nx.matmul_quant(fmt, big, w, 72, n, k)
     _close(many, want, 2e-5, 3e-6 * np.abs(want).max() + 1e-7, "72-row batch")
+    assert np.all(np.abs(many[:m] - full) <= 2e-6 * np.abs(full).max() + 1e-7)
     for r in (0, 5, 30):
         d2 = be.alloc(2 * n * 4)
         be.matmul_quant(fmt, da + r * k * 4, dw, d2, None, 2, n, k)
@@ -205,7 +207,7 @@ def test_matvec_single_row(be, fmt, n, k):
 @pytest.mark.parametrize("fmt", [nx.FMT_Q4_0, nx.FMT_Q6_K])
 def test_matmul_rows_independent_at_prefill_size(be, fmt):
     """1024 rows against a 2048-row matrix: enough (row group, activation group) pairs that one workgroup walks
-    the k-slices in order instead of one workgroup per slice. Rows keep the bits they have in a batch of 2."""
+    the k-slices in order instead of one workgroup per slice. Rows keep the bits they have in a batch of 34."""
     rng = np.random.default_rng(19)
     m, n, k = 1024, 2048, 512
     w = qz.random_quant(fmt, rng, n, k)
@@ -214,10 +216,10 @@ def test_matmul_rows_independent_at_prefill_size(be, fmt):
     dout = be.alloc(m * n * 4)
     be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
     full = be.download(dout, (m, n), np.float32)
-    for r in (0, 517, 1022):
-        d2 = be.alloc(2 * n * 4)
-        be.matmul_quant(fmt, da + r * k * 4, dw, d2, None, 2, n, k)
-        assert np.array_equal(be.download(d2, (2, n), np.float32).view(np.uint32), full[r:r + 2].view(np.uint32))
+    for r in (0, 517, 990):
+        d2 = be.alloc(34 * n * 4)
+        be.matmul_quant(fmt, da + r * k * 4, dw, d2, None, 34, n, k)
+        assert np.array_equal(be.download(d2, (34, n), np.float32).view(np.uint32), full[r:r + 34].view(np.uint32))
     want = nx.matmul_quant(fmt, a[:64], w, 64, n, k)
     _close(full[:64], want, 2e-5, 3e-6 * np.abs(want).max() + 1e-7, "1024-row batch")
     be.reset_pool()

@@ -1706,8 +1706,11 @@ struct WavePlan {
 // Depends on the format and the matrix only, never on M, so that a row's bits do not depend on the batch it sits
 // in. One workgroup per compute unit: the plan with the shortest modelled time among those whose workgroups all
 // run at once. VEXEL_HIP_WPLAN="NxK:R,KS;..." overrides (tuning).
-WavePlan wave_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K) {
+// (up to 32 activation rows: with more, every further 32 rows would stage and unpack the weights again from
+// eight waves' separate slices, and qgemm_kernel's shared staging is quicker)
+WavePlan wave_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K, int M) {
     WavePlan none = {0, 1};
+    if (M > 32) return none;
     static const char *off = getenv("VEXEL_HIP_WAVE_OFF");
     if (off && atoi(off)) return none;
     if (fmt != VX_Q4_0 && fmt != VX_Q8_0 && fmt != VX_Q4_K) return none;
@@ -1804,7 +1807,7 @@ int launch_gemm_wave_r(vx_backend *be, const WavePlan &pl, const Segs &segs, int
 int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out, const float *residual,
                     bool to_partials, int M, int K, int *ks_out, const QkvEpi *epi_in = nullptr) {
     const QkvEpi epi = epi_in ? *epi_in : QkvEpi{};  // (with an epilogue the caller has checked that the wave plan applies)
-    const WavePlan pl = wave_plan(be, fmt, segs, N, K);
+    const WavePlan pl = wave_plan(be, fmt, segs, N, K, M);
     if (pl.r > 0) {
         if (fmt == VX_Q4_0) return launch_gemm_wave_r<WQ4_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
         if (fmt == VX_Q8_0) return launch_gemm_wave_r<WQ8_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
@@ -2114,7 +2117,7 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
     // One K slice, one activation group, the plain RoPE form and a table of this step's angles: the GEMM's workgroups
     // finish their own rows (no partial sums, no second launch).
     {
-        const WavePlan pl = wave_plan(be, wq->fmt, segs, ntot, k);
+        const WavePlan pl = wave_plan(be, wq->fmt, segs, ntot, k, rows);
         const bool table = be->rope_tab_pos == positions && be->rope_tab_rows >= rows && be->rope_tab_dim == head_dim &&
                            be->rope_tab_theta == theta && be->rope_tab_epoch == be->write_epoch;
         static const bool no_epi = getenv("VEXEL_HIP_NO_QKV_EPILOGUE") != nullptr;
