@@ -225,6 +225,36 @@ def test_matmul_rows_independent_at_prefill_size(be, fmt):
     be.reset_pool()
 
 
+@pytest.mark.parametrize("m,n,k", [(100, 208, 512), (256, 1024, 2048), (130, 4096, 256), (97, 48, 1024)])
+def test_matmul_many_rows_q8_0(be, m, n, k):
+    """Q8_0 with more than 96 rows (prompt chunks): the kernel whose waves split the weight rows. Heights that
+    leave waves and whole workgroups past the matrix' end, one and several K slices, a last group of activation
+    rows that is partly padding; with and without the residual."""
+    rng = np.random.default_rng(m + n + k)
+    fmt = nx.FMT_Q8_0
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    want = nx.matmul_quant(fmt, a, w, m, n, k)
+    da, dw, dres = be.upload(a), be.upload(w), be.upload(res)
+    dout = be.alloc(m * n * 4)
+    scale = np.abs(want).max()
+    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
+    got = be.download(dout, (m, n), np.float32)
+    _close(got, want, 2e-5, 3e-6 * scale + 1e-7, "many rows %dx%dx%d" % (m, n, k))
+    be.matmul_quant(fmt, da, dw, dout, dres, m, n, k)
+    _close(be.download(dout, (m, n), np.float32), want + res, 2e-5, 3e-6 * scale + 1e-6, "many rows + residual")
+    # (this kernel's K slices depend on how many groups of 64 rows the batch has: a row keeps its bits between
+    # batches of the same number of groups, and agrees to rounding otherwise)
+    m2 = min(m + 20, (m + 63) // 64 * 64)
+    if m2 > m:
+        a2 = np.concatenate([a, rng.standard_normal((m2 - m, k)).astype(np.float32)])
+        d2 = be.alloc(m2 * n * 4)
+        be.matmul_quant(fmt, be.upload(a2), dw, d2, None, m2, n, k)
+        assert np.array_equal(be.download(d2, (m2, n), np.float32)[:m].view(np.uint32), got.view(np.uint32))
+    be.reset_pool()
+
+
 @pytest.mark.parametrize("fmt", FMTS_MFMA)
 @pytest.mark.parametrize("m,n,k", [(5, 96, 11008), (32, 40, 14336), (16, 7, 4096), (33, 200, 256)])
 def test_matmul_batched_shapes(be, fmt, m, n, k):

@@ -1804,8 +1804,79 @@ int launch_gemm_wave_r(vx_backend *be, const WavePlan &pl, const Segs &segs, int
     return VX_ERR_INVALID;
 }
 
+// The many-rows kernel's cut for (N, K) at M rows: R tiles per wave (128 R weight rows per workgroup) and K slices;
+// r = 0: not served. Wide cuts first; slices only when even 128-row workgroups leave compute units idle.
+// VEXEL_HIP_RPLAN="NxK:R,KS;..." overrides, VEXEL_HIP_ROWS_MIN=<rows> moves the smallest batch it takes.
+WavePlan rows_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K, int M) {
+    WavePlan none = {0, 1};
+    static const int min_rows = getenv("VEXEL_HIP_ROWS_MIN") ? atoi(getenv("VEXEL_HIP_ROWS_MIN")) : 97;
+    // Q8_0 only: measured against qgemm_kernel at 128 / 256 / 512 rows it takes 0.86 / 0.83 / 0.75 of the time there,
+    // while Q4_0 comes out even (its unpack is cheaper to repeat) and Q4_K's decoder does not fit the registers
+    if (M < min_rows || fmt != VX_Q8_0) return none;
+    if (K % 256 != 0 || N % 16 != 0 || N < 16) return none;
+    const int cus = gemm_cus(be), n_chunks = K / 256, mgroups = ceil_div(mpad_for(M), 64);
+    auto fits = [&](int r) {
+        if (N % (16 * r) != 0) return false;
+        for (int i = 0; i < 2; i++)
+            if (segs.n_end[i] < N && segs.n_end[i] % (16 * r) != 0) return false;
+        return true;
+    };
+    static const char *env = getenv("VEXEL_HIP_RPLAN");
+    if (env) {
+        char key[64];
+        snprintf(key, sizeof key, "%dx%d:", N, K);
+        const char *p = strstr(env, key);
+        if (p) {
+            int r = 0, ks = 1;
+            if (sscanf(p + strlen(key), "%d,%d", &r, &ks) == 2 && (r == 1 || r == 2) && fits(r))
+                return WavePlan{r, std::max(1, std::min(ks, n_chunks))};
+        }
+    }
+    for (int r : {2, 1}) {  // (four tiles a wave need more registers than there are)
+        if (!fits(r)) continue;
+        const int wgs = ceil_div(N, 128 * r) * mgroups;
+        if (wgs * 2 >= cus || r == 1) return WavePlan{r, std::max(1, std::min(std::min(n_chunks, 8), cus / std::max(wgs, 1)))};
+    }
+    return none;
+}
+
+template <class W, int R>
+int launch_gemm_rows(vx_backend *be, const Segs &segs, int N, float *out, const float *residual, bool to_partials, int M,
+                     int K, int ks, int *ks_out) {
+    const int mpad = mpad_for(M);
+    const PrepView pv = prep_view(be, mpad, K);
+    float *partial = nullptr;
+    if (ks > 1 || to_partials) {
+        int rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, (size_t)ks * M * N * sizeof(float), "split-K partial sums");
+        if (rc) return rc;
+        partial = (float *)be->part_ws;
+    }
+    const int n_chunks = K / 256, slices = ((n_chunks / ks) << 16) | (n_chunks % ks);
+    dim3 grid(ceil_div(N, 128 * R), ks, ceil_div(mpad, 64));
+    qgemm_rows_kernel<W, R, 4><<<grid, 512, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slices);
+    VX_CHECK_LAUNCH();
+    if (ks_out) *ks_out = ks;
+    if (partial && !to_partials) {
+        const size_t total = (size_t)M * N;
+        qgemm_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>(partial, pv.inv_scale, out, residual, M, N, ks);
+        VX_CHECK_LAUNCH();
+    }
+    return VX_OK;
+}
+
+template <class W>
+int launch_gemm_rows_r(vx_backend *be, const WavePlan &pl, const Segs &segs, int N, float *out, const float *residual,
+                       bool to_partials, int M, int K, int *ks_out) {
+    if (pl.r == 1) return launch_gemm_rows<W, 1>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
+    return launch_gemm_rows<W, 2>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
+}
+
 int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out, const float *residual,
                     bool to_partials, int M, int K, int *ks_out, const QkvEpi *epi_in = nullptr) {
+    const WavePlan rp = rows_plan(be, fmt, segs, N, K, M);
+    if (rp.r > 0) {
+        return launch_gemm_rows_r<WQ8_0>(be, rp, segs, N, out, residual, to_partials, M, K, ks_out);
+    }
     const QkvEpi epi = epi_in ? *epi_in : QkvEpi{};  // (with an epilogue the caller has checked that the wave plan applies)
     const WavePlan pl = wave_plan(be, fmt, segs, N, K, M);
     if (pl.r > 0) {

@@ -422,3 +422,210 @@ __global__ void __launch_bounds__(64 * NW, 1) qgemm_wave_kernel(Segs segs, PrepV
         }
     }
 }
+
+// ---------------------------------------------------------------------------------------------------------------
+// The same arithmetic for many activation rows (prompt chunks, candidate trees), cut the other way: the eight
+// waves of a workgroup take 16*R weight rows EACH (128*R rows per workgroup) and walk the K slice together, against
+// 16*MT activation rows whose tiles the workgroup brings into LDS once per half chunk for all eight. Per step a
+// wave unpacks its R weight tiles once and feeds R*MT MFMA pairs from them, so the unpack and the weight staging
+// are spread over MT*16 rows instead of 32, and an activation tile is fetched from L2 once per 128*R weight rows.
+// Weight staging (global -> registers -> the wave's own LDS rows) is the wave-private kernel's; the activation
+// tiles are double-buffered in LDS with one workgroup barrier per half chunk.
+// grid = (ceil(N / (128 R)), K slices, ceil(Mpad / (16 MT))); block = 512.
+template <class W, int R, int MT>
+__global__ void __launch_bounds__(512, 1) qgemm_rows_kernel(Segs segs, PrepView pv, float *__restrict__ out,
+                                                           const float *__restrict__ residual, float *__restrict__ partial,
+                                                           int M, int Mpad, int N, int K, int n_slices) {
+    constexpr int NW = 8, ROWS = 16 * R;
+    constexpr int NG = (ROWS + W::GROWS - 1) / W::GROWS;
+    constexpr int LAST_ROWS = ROWS - (NG - 1) * W::GROWS;
+    constexpr int W_BYTES = (ROWS * W::PITCH + 16 + 15) / 16 * 16;
+    constexpr int A_HALF = WSS * MT * 2 * 64;  // half8 pieces of a half chunk's activation tiles
+    static_assert(MT * 2 * 64 == 512, "one piece per thread and step");
+    typedef typename PieceOf<W::PIECE>::type piece_t;
+    __shared__ __attribute__((aligned(16))) uint8_t w_lds[NW][W_BYTES];
+    __shared__ half8 a_lds[2][A_HALF];
+
+    const int tid = threadIdx.x, lane = tid & 63, ln = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n_own = (blockIdx.x * NW + wave) * ROWS;  // first row this wave writes
+    const int n0 = max(min(n_own, N - ROWS), 0);         // (a wave past the matrix' end works on its last rows and writes nothing)
+    const int ks = blockIdx.y, mg = blockIdx.z, m0 = mg * 16 * MT, mtiles = Mpad / 16;
+    const size_t row_bytes = W::row_bytes(K);
+    const int sl_base = n_slices >> 16, sl_rem = n_slices & 0xFFFF;
+    const int c_begin = ks * sl_base + min(ks, sl_rem);
+    const int c_end = c_begin + sl_base + (ks < sl_rem ? 1 : 0);
+    const int n_half = 2 * (c_end - c_begin);
+
+    const uint8_t *wg_rows;
+    {
+        const int e0 = segs.n_end[0], e1 = segs.n_end[1];
+        const uint8_t *base = n0 < e0 ? segs.w[0] : (n0 < e1 ? segs.w[1] : segs.w[2]);
+        const int local = n0 < e0 ? n0 : (n0 < e1 ? n0 - e0 : n0 - e1);
+        wg_rows = base + (size_t)local * row_bytes;
+    }
+    uint8_t *const region = &w_lds[wave][0];
+    uint32_t voff[W::GI], voff_last[W::GI], hinc[W::GI], hinc_last[W::GI];
+    int loff[W::GI], loff_last[W::GI];
+#pragma unroll
+    for (int j = 0; j < W::GI; j++) {
+        const int pc = j * 64 + lane;
+        const int lrow = pc / W::NP, lcol = pc % W::NP;
+        const bool ok = lrow < W::GROWS, ok_l = lrow < LAST_ROWS;
+        const int row = ok ? lrow : 0, col = ok ? lcol : 0, row_l = ok_l ? lrow : 0, col_l = ok_l ? lcol : 0;
+        voff[j] = (uint32_t)(row * row_bytes) + W::src_off(0, col);
+        voff_last[j] = (uint32_t)(row_l * row_bytes) + W::src_off(0, col_l);
+        hinc[j] = (uint32_t)(W::src_off(1, col) - W::src_off(0, col));
+        hinc_last[j] = (uint32_t)(W::src_off(1, col_l) - W::src_off(0, col_l));
+        loff[j] = row * W::PITCH + col * W::PIECE;
+        loff_last[j] = row_l * W::PITCH + col_l * W::PIECE;
+    }
+    // this thread's piece of a step's activation tiles: tile tid / 128 of the group (hi and lo halves, 64 lanes each);
+    // a tile past the padded rows repeats the last one (its products are not stored)
+    const int a_tile = min(mg * MT + tid / 128, mtiles - 1);
+    const half8 *a_src = pv.tiles + ((size_t)a_tile * 2) * 64 + (tid & 127);
+
+    float4v run[R][MT];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int t = 0; t < MT; t++) run[r][t] = (float4v){0.f, 0.f, 0.f, 0.f};
+
+    piece_t st[NG * W::GI];
+    half8 areg[WSS];
+    // half chunk q of the slice: chunk c_begin + q / 2, half q % 2 (past the end: the last again)
+    auto fetch = [&](int q) __attribute__((always_inline)) {
+        const int qq = min(q, n_half - 1);
+        const int chunk = c_begin + (qq >> 1), h = qq & 1;
+        const uint8_t *src = wg_rows + (size_t)chunk * W::CHUNK_BYTES;
+#pragma unroll
+        for (int i = 0; i < NG; i++)
+#pragma unroll
+            for (int j = 0; j < W::GI; j++) {
+                const uint32_t vo = i == NG - 1 ? voff_last[j] + (h ? hinc_last[j] : 0u) : voff[j] + (h ? hinc[j] : 0u);
+                st[i * W::GI + j] = *(const piece_t *)(src + (size_t)i * W::GROWS * row_bytes + vo);
+            }
+        const int s0 = chunk * 8 + h * WSS;
+#pragma unroll
+        for (int sp = 0; sp < WSS; sp++) areg[sp] = a_src[(size_t)(s0 + sp) * mtiles * 128];
+    };
+    auto commit = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < NG; i++)
+#pragma unroll
+            for (int j = 0; j < W::GI; j++)
+                *(piece_t *)(region + i * W::GROWS * W::PITCH + (i == NG - 1 ? loff_last[j] : loff[j])) = st[i * W::GI + j];
+#pragma unroll
+        for (int sp = 0; sp < WSS; sp++) a_lds[buf][sp * 512 + tid] = areg[sp];
+    };
+    auto load_cs = [&](int chunk, float4v (&cs)[MT]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            const int mt = min(mg * MT + t, mtiles - 1);
+            cs[t] = *(const float4v *)(pv.cscale + (size_t)chunk * Mpad + mt * 16 + 4 * g);
+        }
+    };
+    const uint8_t *const lane_row = region + ln * W::PITCH;
+
+    if (n_half > 0) {
+        float4v cs[MT], cs_prev[MT];
+        fetch(0);
+        load_cs(c_begin, cs);
+        commit(0);
+        __syncthreads();
+        for (int q = 0; q < n_half; q++) {
+            const int chunk = c_begin + (q >> 1), h = q & 1;
+            fetch(q + 1);
+            if (h == 0 && q > 0) {
+                // a new chunk: the sums move to its activation scale
+                float4v cn[MT];
+                load_cs(chunk, cn);
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    float4v f;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) f[e] = pow2_ratio(cs[t][e], cn[t][e]);
+#pragma unroll
+                    for (int r = 0; r < R; r++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) run[r][t][e] *= f[e];
+                    cs[t] = cn[t];
+                }
+            }
+            const half8 *ab = &a_lds[q & 1][0];
+#pragma unroll
+            for (int sp = 0; sp < WSS; sp++) {
+                const int j = h * WSS + sp, s = chunk * 8 + j;
+                half8 ah[MT], al[MT];
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    ah[t] = ab[sp * 512 + (t * 2 + 0) * 64 + lane];
+                    al[t] = ab[sp * 512 + (t * 2 + 1) * 64 + lane];
+                }
+                float4v bs[MT];
+                if (W::HAS_MIN) {
+#pragma unroll
+                    for (int t = 0; t < MT; t++) {
+                        const int mt = min(mg * MT + t, mtiles - 1);
+                        bs[t] = *(const float4v *)(pv.bsum + (size_t)s * Mpad + mt * 16 + 4 * g);
+                    }
+                }
+                typename W::Raw raw = W::read(lane_row, sp, g);
+#pragma unroll
+                for (int r = 0; r < R; r++) {
+                    const StepW w = W::unpack(raw, sp, j);
+                    if (r + 1 < R) raw = W::read(lane_row + (r + 1) * 16 * W::PITCH, sp, g);
+                    float4v acc[MT];
+#pragma unroll
+                    for (int t = 0; t < MT; t++)
+                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah[t], w.b, (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                    for (int t = 0; t < MT; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al[t], w.b, acc[t], 0, 0, 0);
+#pragma unroll
+                    for (int t = 0; t < MT; t++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            if (W::HAS_MIN)
+                                run[r][t][e] = __builtin_fmaf(-w.dm, bs[t][e], __builtin_fmaf(w.d, acc[t][e], run[r][t][e]));
+                            else
+                                run[r][t][e] = __builtin_fmaf(w.d, acc[t][e], run[r][t][e]);
+                        }
+                }
+            }
+            // the next half chunk: this wave's weights into its own rows (it is done reading them), the activation
+            // tiles into the buffer that every wave finished with before the previous barrier
+            commit((q + 1) & 1);
+            __syncthreads();
+        }
+#pragma unroll
+        for (int t = 0; t < MT; t++) cs_prev[t] = cs[t];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) run[r][t][e] *= cs_prev[t][e];
+    }
+
+    // lane (g, ln) of tile (r, t) holds C[m0 + 16t + 4g + e][n0 + 16r + ln]
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int m = m0 + 16 * t + 4 * g + e;
+            if (m >= M) continue;
+            const float inv = partial ? 1.f : pv.inv_scale[m];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                const int n = n0 + 16 * r + ln;
+                if (n < n_own) continue;
+                if (partial) {
+                    partial[((size_t)ks * M + m) * N + n] = run[r][t][e];
+                } else {
+                    float v = __fmul_rn(run[r][t][e], inv);
+                    if (residual) v = __fadd_rn(residual[(size_t)m * N + n], v);
+                    out[(size_t)m * N + n] = v;
+                }
+            }
+        }
+}
