@@ -523,13 +523,31 @@ __global__ void __launch_bounds__(D) tree_merge_kernel(const float *__restrict__
 // --------------------------------------------------------------------------------------------
 // Dense causal prefill (Backend.SDPAPrefill, backend.go:389; math of backend/cpu/cpu.go:568-632 per query):
 // FlashAttention-2 style. grid = (query tiles of 64, Hq); block = 256 = 4 waves of 16 queries.
-// Per 32-key tile: K and V go to LDS as float32 (all four waves share them), S = Q K^T and O += P V run on the
-// float32 matrix cores (v_mfma_f32_16x16x4_f32: exact float32 products, float32 accumulation, so the numerics stay
-// at the reference's float32 level), the softmax is online in the exp2 domain, P crosses from the MFMA output
-// layout to the operand layout through a wave-private LDS tile. LDS row pitches are chosen so that each
-// operand read hits 64 different banks: K rows 132 floats (16 keys x 4 d), V rows 144 (4 keys x 16 d),
-// P rows 36.
+// Per 32-key tile: K goes to LDS as f16 rows, V transposed ([d][key], so that a lane's eight keys of one column are
+// 16 contiguous bytes); S = Q K^T and O += P V run on v_mfma_f32_16x16x32_f16 with every float32 operand split in
+// two f16 halves (x = hi + lo, about 22 significant bits, float32 accumulation): Q and P always, K and V when they
+// come as float32 (dense prefill; the products hi*hi + hi*lo + lo*hi, the lo*lo term is below float32's last bit),
+// not when they are the f16 rows of the paged pool, which are exact. The softmax is online in the exp2 domain; P
+// crosses from the MFMA output layout to the operand layout through a wave-private LDS tile. LDS row pitches are
+// an odd number of 16-byte slots, so the 16 lanes of an operand read land in 16 different slots.
 constexpr int FA_BQ = 64, FA_BK = 32;
+
+// x = h + l in two f16 halves. The float32 value, its rounded half and their difference each pass through a register
+// of their own: left to itself the compiler folds the operations that produced x into mixed-precision
+// multiply-adds that round once from the unrounded product, and the halves then add up to less than x's 24 bits
+// (measured: attention outputs off by 3e-5 instead of 1e-6).
+struct HalfPair { _Float16 h, l; };
+__device__ __forceinline__ HalfPair split_hl(float x) {
+    asm volatile("" : "+v"(x));
+    HalfPair r;
+    r.h = (_Float16)x;
+    float hf = (float)r.h;
+    asm volatile("" : "+v"(hf));
+    float d = x - hf;
+    asm volatile("" : "+v"(d));
+    r.l = (_Float16)d;
+    return r;
+}
 typedef float float4v __attribute__((ext_vector_type(4)));
 
 template <int N>
@@ -559,9 +577,10 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
                                                           const float *__restrict__ v, float *__restrict__ out, int S,
                                                           int num_q_heads, int num_kv_heads, float scale,
                                                           float softcap = 0.f, PagedSrc paged = PagedSrc()) {
-    constexpr int KP = D + 4, VP = D + 16, PP = FA_BK + 4;
-    __shared__ __attribute__((aligned(16))) float Ks[FA_BK * KP];
-    __shared__ __attribute__((aligned(16))) float Vs[FA_BK * VP];
+    constexpr int KP = D + 8, VP = FA_BK + 8, PP = FA_BK + 4;  // halves per K row, halves per V^T row, floats per P row
+    constexpr int NLO = PAGED ? 1 : 2;                           // [0]: hi halves, [1]: lo halves (float32 sources only)
+    __shared__ __attribute__((aligned(16))) _Float16 Ks[NLO][FA_BK * KP];
+    __shared__ __attribute__((aligned(16))) _Float16 Vt[NLO][D * VP];
     __shared__ __attribute__((aligned(16))) float Ps[4][16 * PP];
     __shared__ int len_max[5];  // PAGED: the longest key range among each wave's 16 queries, [4]: among all 64
     const int qt = blockIdx.x, h = blockIdx.y, kvh = h / (num_q_heads / num_kv_heads);
@@ -585,14 +604,23 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
     }
     const int wave_keys = PAGED ? len_max[wave] : min(q0 + 15, S - 1) + 1;  // keys any of the wave's queries sees
 
-    // Q as the A operand: lane (row c16, k = 4s + g), pre-multiplied by scale*log2(e)
-    float qa[D / 4];
+    // Q as the A operand: lane (row c16, columns 32s + 8g .. + 7), pre-multiplied by scale*log2(e), hi + lo
+    half8 qh[D / 32], ql[D / 32];
     {
         const int qi = min(q0 + c16, S - 1);
-        const float *qp = q + (size_t)qi * qs + (size_t)h * D + g;
+        const float *qp = q + (size_t)qi * qs + (size_t)h * D + 8 * g;
         const float f = scale * kLog2e;
 #pragma unroll
-        for (int s = 0; s < D / 4; s++) qa[s] = qp[4 * s] * f;
+        for (int s = 0; s < D / 32; s++) {
+            const float4 a = *(const float4 *)(qp + 32 * s), b = *(const float4 *)(qp + 32 * s + 4);
+            const float x[8] = {a.x * f, a.y * f, a.z * f, a.w * f, b.x * f, b.y * f, b.z * f, b.w * f};
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const HalfPair t = split_hl(x[e]);
+                qh[s][e] = t.h;
+                ql[s][e] = t.l;
+            }
+        }
     }
     float4v o[D / 16];
 #pragma unroll
@@ -608,26 +636,39 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
     const int n_tiles = (n_keys + FA_BK - 1) / FA_BK;
     for (int kt = 0; kt < n_tiles; kt++) {
         __syncthreads();  // the previous tile's reads are done
-        for (int idx = tid; idx < FA_BK * (D / 4); idx += 256) {
-            const int key = idx / (D / 4), d4 = (idx % (D / 4)) * 4;
+        for (int idx = tid; idx < FA_BK * (D / 8); idx += 256) {
+            const int key = idx % FA_BK, d8 = (idx / FA_BK) * 8;  // (lanes run over keys: V^T's 2-byte stores fill whole rows)
             const int ki = kt * FA_BK + key;
-            float4 kv4 = make_float4(0.f, 0.f, 0.f, 0.f), vv4 = kv4;
+            half8 kh = {0, 0, 0, 0, 0, 0, 0, 0}, vh = kh, kl = kh, vl = kh;
             if (PAGED) {
                 if (ki < n_keys) {
-                    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
                     const size_t part = (size_t)paged.block_size * ks;  // a block's K rows, then its V rows
                     const _Float16 *kp = paged.pool + (size_t)paged.table[ki / paged.block_size] * 2 * part +
-                                         (size_t)(ki % paged.block_size) * ks + (size_t)kvh * D + d4;
-                    const half4 kh = *(const half4 *)kp, vh = *(const half4 *)(kp + part);
-                    kv4 = make_float4((float)kh[0], (float)kh[1], (float)kh[2], (float)kh[3]);
-                    vv4 = make_float4((float)vh[0], (float)vh[1], (float)vh[2], (float)vh[3]);
+                                         (size_t)(ki % paged.block_size) * ks + (size_t)kvh * D + d8;
+                    kh = *(const half8 *)kp;
+                    vh = *(const half8 *)(kp + part);
                 }
             } else if (ki < S) {
-                kv4 = *(const float4 *)(k + (size_t)ki * ks + (size_t)kvh * D + d4);
-                vv4 = *(const float4 *)(v + (size_t)ki * ks + (size_t)kvh * D + d4);
+                const float *kp = k + (size_t)ki * ks + (size_t)kvh * D + d8, *vp = v + (size_t)ki * ks + (size_t)kvh * D + d8;
+                const float4 k0 = *(const float4 *)kp, k1 = *(const float4 *)(kp + 4);
+                const float4 v0 = *(const float4 *)vp, v1 = *(const float4 *)(vp + 4);
+                const float kx[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
+                const float vx[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const HalfPair tk = split_hl(kx[e]), tv = split_hl(vx[e]);
+                    kh[e] = tk.h; kl[e] = tk.l;
+                    vh[e] = tv.h; vl[e] = tv.l;
+                }
             }
-            *(float4 *)(Ks + key * KP + d4) = kv4;
-            *(float4 *)(Vs + key * VP + d4) = vv4;
+            *(half8 *)(&Ks[0][key * KP + d8]) = kh;
+#pragma unroll
+            for (int e = 0; e < 8; e++) Vt[0][(d8 + e) * VP + key] = vh[e];
+            if (!PAGED) {
+                *(half8 *)(&Ks[NLO - 1][key * KP + d8]) = kl;
+#pragma unroll
+                for (int e = 0; e < 8; e++) Vt[NLO - 1][(d8 + e) * VP + key] = vl[e];
+            }
         }
         __syncthreads();
         if (kt * FA_BK >= wave_keys) continue;  // every key of the tile is beyond what the wave's queries see
@@ -636,9 +677,17 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
 #pragma unroll
         for (int cb = 0; cb < FA_BK / 16; cb++) {
             float4v acc = {0.f, 0.f, 0.f, 0.f};
-            const float *kb = Ks + (cb * 16 + c16) * KP + g;
+            const int ko = (cb * 16 + c16) * KP + 8 * g;  // key cb*16 + c16, columns 32s + 8g .. + 7
 #pragma unroll
-            for (int s = 0; s < D / 4; s++) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[s], kb[4 * s], acc, 0, 0, 0);
+            for (int s = 0; s < D / 32; s++) {
+                const half8 b = *(const half8 *)(&Ks[0][ko + 32 * s]);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh[s], b, acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(ql[s], b, acc, 0, 0, 0);
+                if (!PAGED) {
+                    const half8 bl = *(const half8 *)(&Ks[NLO - 1][ko + 32 * s]);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(qh[s], bl, acc, 0, 0, 0);
+                }
+            }
             sc[cb] = acc;
         }
         if (CAP) {
@@ -689,15 +738,29 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
 #pragma unroll
             for (int i = 0; i < 4; i++) pt[(4 * g + i) * PP + cb * 16 + c16] = sc[cb][i];
         // (wave-private tile: the wave's own LDS accesses are ordered)
-        float pa[FA_BK / 4];
+        // P as the A operand: lane (row c16, keys 8g .. 8g + 7), hi + lo
+        half8 ph, pl;
+        {
+            const float4 a = *(const float4 *)(pt + c16 * PP + 8 * g), b = *(const float4 *)(pt + c16 * PP + 8 * g + 4);
+            const float x[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
-        for (int s = 0; s < FA_BK / 4; s++) pa[s] = pt[c16 * PP + 4 * s + g];
-        // O += P V: lane holds O[row 4g+i][d = db*16 + c16]
+            for (int e = 0; e < 8; e++) {
+                const HalfPair t = split_hl(x[e]);
+                ph[e] = t.h;
+                pl[e] = t.l;
+            }
+        }
+        // O += P V: lane holds O[row 4g+i][d = db*16 + c16]; B operand: column d, keys 8g .. 8g + 7 of V^T
 #pragma unroll
         for (int db = 0; db < D / 16; db++) {
-            const float *vb = Vs + g * VP + db * 16 + c16;
-#pragma unroll
-            for (int s = 0; s < FA_BK / 4; s++) o[db] = __builtin_amdgcn_mfma_f32_16x16x4f32(pa[s], vb[4 * s * VP], o[db], 0, 0, 0);
+            const int vo = (db * 16 + c16) * VP + 8 * g;
+            const half8 vb = *(const half8 *)(&Vt[0][vo]);
+            o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ph, vb, o[db], 0, 0, 0);
+            o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pl, vb, o[db], 0, 0, 0);
+            if (!PAGED) {
+                const half8 vl = *(const half8 *)(&Vt[NLO - 1][vo]);
+                o[db] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ph, vl, o[db], 0, 0, 0);
+            }
         }
     }
 #pragma unroll
@@ -761,7 +824,8 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
     static const bool no_merge = getenv("VEXEL_HIP_NO_ATTN_MERGE") != nullptr;
     constexpr int GD = G * D;
     constexpr int HPC = (GD < 256 && 256 % GD == 0) ? 256 / GD : 0;  // kv heads that share a chunk
-    const bool mergeable = GD % 256 == 0 || (HPC > 0 && num_kv_heads % HPC == 0);
+    bool mergeable = GD % 256 == 0;
+    if constexpr (HPC > 0) mergeable = num_kv_heads % HPC == 0;
     if (!out && !fixed && !no_merge && mergeable && be->attn_cnt && (size_t)batch * num_kv_heads <= VX_ATTN_CNT) {
         if (batch == 1) {
             mg.cnt = be->attn_cnt;
