@@ -146,7 +146,17 @@ int attn_noalloc_init(vx_backend *be);
 int run_matvec(vx_backend *be, int fmt, const float *a, const void *b, float *out, const float *residual, int n, int k);
 // Where the matrix-vector kernel takes its activation row from: x itself; x * norm_w with the results divided
 // by rms(x) (RMSNorm folded in); or the attention output of one query merged from its split-KV partials.
+// RoPE (interleaved pairs over the whole head) and the paged K/V store as the epilogue of a single row's fused
+// Q|K|V matrix-vector product: rows [0, qd) are Q, [qd, qd + kvd) K, then V. q_out == nullptr: none.
+struct MatvecRope {
+    float *q_out = nullptr;
+    void *pool = nullptr;          // F16 paged pool of the layer
+    const int32_t *slot = nullptr; // the row's slot in the pool (device)
+    const float2 *cs_tab = nullptr; // (cos, sin) of the row's position per pair (vx_rope_table_prepare)
+    int qd = 0, kvd = 0, head_dim = 0, block_size = 0;
+};
 struct MatvecSource {
+    MatvecRope rope;
     const float *x = nullptr;
     const float *norm_w = nullptr;
     float eps = 0.f;

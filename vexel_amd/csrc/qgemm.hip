@@ -2157,6 +2157,24 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
             src.x = x;
             src.norm_w = norm_weight;
             src.eps = eps;
+            // With this step's table of angles the launch finishes the row itself: RoPE, Q out, K and V into the pool.
+            static const bool no_epi = getenv("VEXEL_HIP_NO_QKV_EPILOGUE") != nullptr;
+            const bool table1 = be->rope_tab_pos == positions && be->rope_tab_rows >= 1 && be->rope_tab_dim == head_dim &&
+                                be->rope_tab_theta == theta && be->rope_tab_epoch == be->write_epoch;
+            if (!gen && !no_epi && table1) {
+                src.rope.q_out = q_out;
+                src.rope.pool = kv_pool;
+                src.rope.slot = slot_mapping;
+                src.rope.cs_tab = (const float2 *)be->rope_tab;
+                src.rope.qd = wq->n;
+                src.rope.kvd = wk->n;
+                src.rope.head_dim = head_dim;
+                src.rope.block_size = block_size;
+                rc = run_matvec_fused(be, wq->fmt, mw, mn, 3, k, src, (float *)be->part_ws, nullptr, 0);
+                if (rc == VX_OK) return VX_OK;
+                if (rc != VX_ERR_UNSUPPORTED) return rc;
+                src.rope = MatvecRope();
+            }
             rc = run_matvec_fused(be, wq->fmt, mw, mn, 3, k, src, (float *)be->part_ws, nullptr, 0);
             if (rc) return rc;
             const int half1 = head_dim / 2;

@@ -313,6 +313,7 @@ struct MvArgs {
     int pair;                     // > 0: rows i and pair + i belong together, out[i] = silu(dot_i) * dot_{pair+i}
     float *out;
     const float *residual;        // added to the result (not with pair)
+    MatvecRope rope;              // qmatvec2_kernel only: the rows are Q|K|V of one token, finished in the epilogue
 };
 enum { MV_PLAIN = 0, MV_RMSNORM = 1, MV_MERGED_ATTENTION = 2 };
 
@@ -669,7 +670,29 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec2_kernel(const MvArgs p, in
             float v = acc[0];
 #pragma unroll
             for (int r = 1; r < NR; r++) v = lane == r ? acc[r] : v;
-            if (lane < NR) {
+            if (p.rope.q_out) {
+                // rows 2j and 2j + 1 of a head are a RoPE pair (backend/cpu/cpu.go:226-303) and sit in lanes 2i, 2i + 1
+                const float other = __shfl_xor(v, 1, 64);
+                if (lane < NR) {
+                    const int row = q * NR + lane, qd = p.rope.qd, kvd = p.rope.kvd;
+                    const bool is_q = row < qd, is_v = row >= qd + kvd;
+                    const int o = is_q ? row : (is_v ? row - qd - kvd : row - qd);
+                    float res = v;
+                    if (!is_v) {
+                        const float2 cs = p.rope.cs_tab[(o & (p.rope.head_dim - 1)) >> 1];
+                        const float a = (lane & 1) ? other : v, b = (lane & 1) ? v : other;
+                        res = (lane & 1) ? __fadd_rn(__fmul_rn(a, cs.y), __fmul_rn(b, cs.x))
+                                         : __fsub_rn(__fmul_rn(a, cs.x), __fmul_rn(b, cs.y));
+                    }
+                    if (is_q) {
+                        p.rope.q_out[o] = res;
+                    } else {
+                        const int slot = p.rope.slot[0], blk = slot / p.rope.block_size, off = slot - blk * p.rope.block_size;
+                        const size_t part = (size_t)p.rope.block_size * kvd;
+                        ((_Float16 *)p.rope.pool)[(size_t)blk * 2 * part + (size_t)off * kvd + (is_v ? part : 0) + o] = (_Float16)res;
+                    }
+                }
+            } else if (lane < NR) {
                 const int row = q * NR + lane;
                 if (p.residual) v = __fadd_rn(p.residual[row], v);
                 p.out[row] = v;
@@ -707,6 +730,9 @@ bool launch_second_form(vx_backend *be, int fmt, MvArgs &a) {
     else if (2 * rb / 16 <= 64 * 9) nr = 2, npl = 9;    // K <= 8192
     else if (2 * rb / 16 <= 64 * 13) nr = 2, npl = 13;  // K <= 11776
     else return false;
+    if (a.rope.q_out && (a.pair > 0 || a.residual || nr % 2 != 0 || a.rope.qd % nr != 0 || a.rope.kvd % nr != 0 ||
+                         (a.rope.head_dim & (a.rope.head_dim - 1)) != 0 || a.N != a.rope.qd + 2 * a.rope.kvd))
+        return false;
     const int unit = a.pair > 0 ? nr / 2 : nr;
     if (a.pair > 0) {
         if (a.pair % unit != 0) return false;
@@ -809,6 +835,7 @@ int launch_fmt(vx_backend *be, int fmt, MvArgs &a) {
         VX_CHECK_LAUNCH();
         return VX_OK;
     }
+    if (a.rope.q_out) return VX_ERR_UNSUPPORTED;  // only that kernel finishes Q|K|V rows itself
     switch (fmt) {
     case VX_Q4_0: return launch<VQ4_0>(be, a);
     case VX_Q8_0: return launch<VQ8_0>(be, a);
@@ -875,6 +902,8 @@ int run_matvec_fused(vx_backend *be, int fmt, const void *const *ws, const int *
     a.N = tot; a.K = k;
     a.pair = pair ? ns[0] : 0;
     a.out = out; a.residual = residual;
+    a.rope = src.rope;
+    if (a.rope.q_out && src.attn_partial) return VX_ERR_UNSUPPORTED;
     if (src.attn_partial) {
         if (!src.kv_len || src.head_dim < 32 || src.head_dim % 32 != 0 || k % src.head_dim != 0) return VX_ERR_UNSUPPORTED;
         a.mode = MV_MERGED_ATTENTION;

@@ -391,7 +391,7 @@ int forward_decode(vh_model *m, int rows, int max_kv_len) {
     const bool head_prepared = rows > 1 && m->fused && (!m->general || m->fused_ok) && fast(m->lm_head) && c.hidden % 256 == 0;
     bool chained = false;
     // the step's RoPE angles once for all layers: the fused Q|K|V launches then rotate and store their own rows
-    if (rows > 1 && m->fused && !m->general) VXC(vx_rope_table_prepare(m->be, m->d_token_pos, rows, c.head_dim, c.rope_theta));
+    if (m->fused && !m->general) VXC(vx_rope_table_prepare(m->be, m->d_token_pos, rows, c.head_dim, c.rope_theta));
     for (int l = 0; l < c.num_layers; l++) {
         const float *next_norm = l + 1 < c.num_layers ? (rows > 1 && attn_fusable(m, l + 1) ? m->layers[l + 1].attn_norm : nullptr)
                                                       : (head_prepared ? m->final_norm : nullptr);
