@@ -125,6 +125,35 @@ def test_matmul_other_formats_vs_oracle(be, fmt, m):
     be.reset_pool()
 
 
+@pytest.mark.parametrize("m,n,k", [(2, 64, 256), (32, 256, 2048), (40, 512, 1024), (7, 1040, 512), (100, 96, 768),
+                                   (1, 71, 4096), (1, 256, 11008), (1, 3, 8)])
+def test_matmul_bf16_fast_paths(be, m, n, k):
+    """MatMulBF16 (backend.go:80) where the matrix-core kernel (two rows and more, K a multiple of 256, N of 16:
+    the bf16 weights become f16 exactly) and the streaming matrix-vector kernel (one row) take it; with and without
+    the residual; weights down to f16's smallest normal magnitudes."""
+    rng = np.random.default_rng(m * 7 + n + k)
+    fmt = nx.FMT_BF16
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    want = nx.matmul_quant(fmt, a, w, m, n, k)
+    da, dw, dres = be.upload(a), be.upload(w), be.upload(res)
+    dout = be.alloc(m * n * 4)
+    scale = np.abs(want).max()
+    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
+    _close(be.download(dout, (m, n), np.float32), want, 2e-5, 3e-6 * scale + 1e-7, "bf16 %dx%dx%d" % (m, n, k))
+    be.matmul_quant(fmt, da, dw, dout, dres, m, n, k)
+    _close(be.download(dout, (m, n), np.float32), want + res, 2e-5, 3e-6 * scale + 1e-6, "bf16 + residual")
+    # small weights: 2^-14 .. 2^-10 (f16 keeps all eight bits of a bf16 there)
+    wf = (rng.standard_normal(n * k) * 2.0 ** -12).astype(np.float32)
+    ws = (wf.view(np.uint32) >> 16).astype(np.uint16)
+    want2 = a.astype(np.float64) @ (ws.astype(np.uint32) << 16).view(np.float32).reshape(n, k).astype(np.float64).T
+    be.matmul_quant(fmt, da, be.upload(ws), dout, None, m, n, k)
+    got2 = be.download(dout, (m, n), np.float32)
+    assert np.all(np.abs(got2 - want2) <= 2e-5 * np.abs(want2) + 3e-6 * np.abs(want2).max())
+    be.reset_pool()
+
+
 # ------------------------------------------------------------------ quantized matmul
 @pytest.mark.parametrize("fmt", FMTS_MFMA)
 @pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 32, 40])

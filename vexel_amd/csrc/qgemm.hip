@@ -1710,10 +1710,10 @@ struct WavePlan {
 // eight waves' separate slices, and qgemm_kernel's shared staging is quicker)
 WavePlan wave_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K, int M) {
     WavePlan none = {0, 1};
-    if (M > 32) return none;
+    if (M > 32 && fmt != VX_BF16) return none;  // (BF16 has no other matrix-core kernel: it takes the groups of 32 rows)
     static const char *off = getenv("VEXEL_HIP_WAVE_OFF");
     if (off && atoi(off)) return none;
-    if (fmt != VX_Q4_0 && fmt != VX_Q8_0 && fmt != VX_Q4_K) return none;
+    if (fmt != VX_Q4_0 && fmt != VX_Q8_0 && fmt != VX_Q4_K && fmt != VX_BF16) return none;
     if (K % 256 != 0 || N % 16 != 0 || N < 64) return none;
     const int cus = gemm_cus(be), tiles = N / 16, n_chunks = K / 256;
     auto fits = [&](int r) {
@@ -1733,15 +1733,16 @@ WavePlan wave_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K, int 
         }
     }
     // more than 6 tiles a workgroup would spill registers: taller matrices (output heads) stay on qgemm_kernel
-    if (tiles > (fmt == VX_Q8_0 ? 4 : 6) * cus) return none;
+    const int max_r = fmt == VX_Q8_0 ? 4 : (fmt == VX_BF16 ? 2 : 6);  // (wider staging leaves room for fewer tiles)
+    if (tiles > max_r * cus && fmt != VX_BF16) return none;
     static const int rs[] = {1, 2, 3, 4, 6};
     WavePlan best = none;
     float best_cost = 0.f;
     for (int r : rs) {
-        if (!fits(r) || (fmt == VX_Q8_0 && r > 4)) continue;  // Q8_0's wider staging leaves room for 4 tiles
+        if (!fits(r) || r > max_r) continue;
         const int rg = ceil_div(tiles, r);
         for (int ks = 1; ks <= std::min(n_chunks, 8); ks++) {
-            if (rg * ks > cus) continue;
+            if (rg * ks > cus && !(fmt == VX_BF16 && ks == 1 && r == max_r)) continue;  // (a tall BF16 matrix: several rounds of workgroups)
             const int wg_chunks = ceil_div(n_chunks, ks), wave_chunks = ceil_div(wg_chunks, 8);
             // In cycles, fitted to the 7B shapes at 32 rows: a wave's tile steps share a SIMD with one other
             // wave's (about 220 cycles a tile step for the pair); a compute unit pulls the 32 KB of activation
@@ -1793,12 +1794,14 @@ int launch_gemm_wave(vx_backend *be, const Segs &segs, int N, float *out, const 
 template <class W>
 int launch_gemm_wave_r(vx_backend *be, const WavePlan &pl, const Segs &segs, int N, float *out, const float *residual,
                        bool to_partials, int M, int K, int *ks_out, const QkvEpi &epi) {
-    switch (pl.r) {
-    case 1: return launch_gemm_wave<W, 1>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
-    case 2: return launch_gemm_wave<W, 2>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
-    case 3: return launch_gemm_wave<W, 3>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
-    case 4: return launch_gemm_wave<W, 4>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
-    case 6: return launch_gemm_wave<W, 6>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
+    if (pl.r == 1) return launch_gemm_wave<W, 1>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
+    if (pl.r == 2) return launch_gemm_wave<W, 2>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
+    if constexpr (W::PITCH < 256) {  // (the narrow formats: more tiles fit the registers and the LDS)
+        switch (pl.r) {
+        case 3: return launch_gemm_wave<W, 3>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
+        case 4: return launch_gemm_wave<W, 4>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
+        case 6: return launch_gemm_wave<W, 6>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out, epi);
+        }
     }
     set_error("wave GEMM: no kernel for %d tiles per workgroup", pl.r);
     return VX_ERR_INVALID;
@@ -1882,6 +1885,7 @@ int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out
     if (pl.r > 0) {
         if (fmt == VX_Q4_0) return launch_gemm_wave_r<WQ4_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
         if (fmt == VX_Q8_0) return launch_gemm_wave_r<WQ8_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
+        if (fmt == VX_BF16) return launch_gemm_wave_r<WBF16>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
         return launch_gemm_wave_r<WQ4_K>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
     }
     switch (fmt) {
@@ -2023,6 +2027,19 @@ int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, floa
     if (m == 1 && !no_matvec) {  // a single row: the streaming matrix-vector kernel
         rc = run_matvec(be, fmt, a, b, out, residual, n, k);
         if (rc != VX_ERR_UNSUPPORTED) return rc;
+    }
+    if (fmt == VX_BF16 && m >= 2 && k % 256 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0) {
+        // the matrix cores: bf16 -> f16 is exact for weights, the activations enter as hi + lo as everywhere
+        Segs segs;
+        segs.w[0] = segs.w[1] = segs.w[2] = (const uint8_t *)b;
+        segs.n_end[0] = segs.n_end[1] = segs.n_end[2] = n;
+        if (wave_plan(be, fmt, segs, n, k, m).r > 0) {
+            rc = vx_prepare_act(be, a, m, k);
+            if (rc) return rc;
+            rc = finalize_row_norm(be);
+            if (rc) return rc;
+            return launch_gemm_fmt(be, fmt, segs, n, out, residual, false, m, k, nullptr);
+        }
     }
     if (!fast_ok(fmt, b, n, k) || ((uintptr_t)a % 16) != 0) {
         const size_t rb = fmt_row_bytes(fmt, k);

@@ -124,6 +124,41 @@ struct WQ4_K {
     }
 };
 
+// BF16 (pkg/gguf/dequant.go:215-228): no blocks and no scales. A bf16 value's eight significant bits fit f16's eleven,
+// so its conversion to f16 is exact wherever the value lies inside f16's range. The weights are converted times 64
+// (added to the exponent field; 1/64 is the step's scale): exact for magnitudes from 2^-23 to 1023, an absolute error
+// below 2^-31 under that, and a wrong (saturated) value from 1024 up, which weight matrices do not hold.
+// A stage is the row's 128 elements, 256 bytes.
+struct WBF16 {
+    static constexpr int CHUNK_BYTES = 512, PIECE = 16, NP = 16, PITCH = 272, GI = 1, GROWS = 4;
+    static constexpr bool HAS_MIN = false;
+    static __host__ __device__ size_t row_bytes(int K) { return (size_t)K * 2; }
+    static __device__ __forceinline__ int src_off(int h, int col) { return 256 * h + 16 * col; }
+    struct Raw { uint32_t a0, a1, b0, b1; };  // elements 4g..4g+3 and 16+4g..16+4g+3 of the step
+    static __device__ __forceinline__ Raw read(const uint8_t *row, int sp, int g) {
+        const uint32_t *p = (const uint32_t *)(row + 64 * sp) + 2 * g;
+        Raw x;
+        x.a0 = p[0];
+        x.a1 = p[1];
+        x.b0 = p[8];
+        x.b1 = p[9];
+        return x;
+    }
+    static __device__ __forceinline__ half2v cvt2(uint32_t lo_bits, uint32_t hi_bits) {  // two bf16 patterns in the high halves
+        return __builtin_bit_cast(half2v, __builtin_amdgcn_cvt_pkrtz(__uint_as_float(lo_bits), __uint_as_float(hi_bits)));
+    }
+    static __device__ __forceinline__ StepW unpack(const Raw &x, int, int) {
+        constexpr uint32_t E = 6u << 23;  // times 64 (a zero becomes 2^-121 and converts to zero)
+        auto lo = [](uint32_t w) { return (w << 16) + E; };
+        auto hi = [](uint32_t w) { return (w & 0xFFFF0000u) + E; };
+        StepW r;  // slot order {4g, 4g+2, 16+4g, 16+4g+2, 4g+1, 4g+3, 16+4g+1, 16+4g+3}
+        r.b = pack8(cvt2(lo(x.a0), lo(x.a1)), cvt2(lo(x.b0), lo(x.b1)), cvt2(hi(x.a0), hi(x.a1)), cvt2(hi(x.b0), hi(x.b1)));
+        r.d = 1.f / 64.f;
+        r.dm = 0.f;
+        return r;
+    }
+};
+
 // ratio of two chunk factors (positive powers of two): the difference of their exponent fields
 __device__ __forceinline__ float pow2_ratio(float num, float den) {
     return __uint_as_float(__float_as_uint(num) - __float_as_uint(den) + 0x3F800000u);

@@ -747,6 +747,58 @@ bool launch_second_form(vx_backend *be, int fmt, MvArgs &a) {
     return true;
 }
 
+// ---- BF16, one activation row: out[n] = sum_k a[k] * W[n][k] in float32 (the bf16 pattern is the high half of the
+// float32 it stands for, pkg/gguf/dequant.go:215-228). The activation row sits in LDS as floats; a wave takes two rows
+// at a time, every lane 16 bytes (eight weights) of each per trip, up to eight trips' loads in flight, and adds its
+// lanes by one butterfly per row. HBM bound: 2 bytes per weight.
+__global__ void __launch_bounds__(MV_THREADS) bf16_matvec_kernel(const uint8_t *__restrict__ W, const float *__restrict__ a,
+                                                                float *__restrict__ out, const float *__restrict__ residual,
+                                                                int N, int K) {
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __attribute__((aligned(16))) float xs[];  // [K]
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    for (int i = tid * 4; i < K; i += MV_THREADS * 4) *(float4 *)(xs + i) = *(const float4 *)(a + i);
+    __syncthreads();
+    const int n_waves = gridDim.x * MV_WAVES, pieces = K / 8;  // 16-byte pieces of a row
+    constexpr int U = 8;
+    for (int pr = blockIdx.x * MV_WAVES + wave; 2 * pr < N; pr += n_waves) {
+        const int r0 = 2 * pr, r1 = min(r0 + 1, N - 1);
+        const uint8_t *w0 = W + (size_t)r0 * K * 2, *w1 = W + (size_t)r1 * K * 2;
+        float acc0 = 0.f, acc1 = 0.f;
+        for (int p0 = 0; p0 < pieces; p0 += 64 * U) {
+            u32x4 q0[U], q1[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int pc = min(p0 + 64 * u + lane, pieces - 1);  // (past the row's end: the last piece again, not added)
+                q0[u] = *(const u32x4 *)(w0 + (size_t)pc * 16);
+                q1[u] = *(const u32x4 *)(w1 + (size_t)pc * 16);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int pc = p0 + 64 * u + lane;
+                if (pc < pieces) {
+                    const float4 xa = *(const float4 *)(xs + pc * 8), xb = *(const float4 *)(xs + pc * 8 + 4);
+                    const float x[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        acc0 = fmaf(x[2 * e], __uint_as_float(q0[u][e] << 16), acc0);
+                        acc0 = fmaf(x[2 * e + 1], __uint_as_float(q0[u][e] & 0xFFFF0000u), acc0);
+                        acc1 = fmaf(x[2 * e], __uint_as_float(q1[u][e] << 16), acc1);
+                        acc1 = fmaf(x[2 * e + 1], __uint_as_float(q1[u][e] & 0xFFFF0000u), acc1);
+                    }
+                }
+            }
+        }
+        acc0 = wave_sum64(acc0);
+        acc1 = wave_sum64(acc1);
+        if (lane == 0) {
+            out[r0] = residual ? __fadd_rn(residual[r0], acc0) : acc0;
+            if (r0 + 1 < N) out[r0 + 1] = residual ? __fadd_rn(residual[r0 + 1], acc1) : acc1;
+        }
+    }
+}
+
 int device_cus(vx_backend *be) {
     static int cus = 0;
     if (cus == 0) {
@@ -870,6 +922,18 @@ bool matvec_ok(int fmt, const void *const *ws, const int *ns, int nw, int k) {
 // out[n] = a . W[n] (+ residual[n]) for one activation row. VX_ERR_UNSUPPORTED (nothing launched) when the shape is
 // outside the kernel's range: the caller then takes another path.
 int run_matvec(vx_backend *be, int fmt, const float *a, const void *b, float *out, const float *residual, int n, int k) {
+    if (fmt == VX_BF16) {
+        if (k % 8 != 0 || (size_t)k * 4 > 96 * 1024 || ((uintptr_t)b % 16) != 0 || ((uintptr_t)a % 16) != 0) return VX_ERR_UNSUPPORTED;
+        static int per_cu = 0;
+        if (per_cu == 0) {
+            (void)hipFuncSetAttribute((const void *)bf16_matvec_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+            per_cu = 1;
+        }
+        const int wgs = std::min(ceil_div(ceil_div(n, 2), MV_WAVES), 4 * device_cus(be));
+        bf16_matvec_kernel<<<wgs, MV_THREADS, (size_t)k * 4, be->stream>>>((const uint8_t *)b, a, out, residual, n, k);
+        VX_CHECK_LAUNCH();
+        return VX_OK;
+    }
     MatvecSource src;
     src.x = a;
     const void *ws[1] = {b};
