@@ -280,7 +280,9 @@ int vx_rope_store_paged_ex(vx_backend *be, float *q, const float *k, const float
  * columns (query heads per KV head x head_dim) divide 256 or are a multiple of it, 2 to 64 rows, the workgroup that
  * finishes a sequence's 256 columns last also merges them, splits in index order, and writes them as the output
  * projection's prepared operand (no merge launch at all); any call between the two that prepares another
- * activation makes vx_decode_ffn merge from the partial sums as before.
+ * activation makes vx_decode_ffn merge from the partial sums as before. A call with out = NULL therefore replaces
+ * whatever activation the backend held prepared (vx_prepare_act, vx_rmsnorm_prepare, ...): prepare again before a
+ * vx_matmul_quant_prepared that is not the vx_decode_ffn this call is for.
  * That is also where the streaming split-KV kernel runs (F16 pool, 16-token blocks): heads of 64 or 128 with 1 to 8
  * query heads per KV head, heads of 256 with 1 or 2, heads of 80 or 96 with 1; other geometries take the generic
  * kernel (any head_dim <= 256), same results, far slower. */
