@@ -525,7 +525,8 @@ __device__ __forceinline__ float wave_sum64(float t) {
 
 // NR rows per pass, NPL 16-byte pieces per lane and pass (64 * NPL >= NR * row_bytes / 16). Every matrix (with
 // `pair`: each of the two) holds a multiple of NR (NR/2) rows and whole 16-byte rows: the host checks.
-template <int NR, int NPL>
+// TT: steps of 64 blocks per row when known at compile time (the loop is then unrolled and its LDS reads overlap), 0: any.
+template <int NR, int NPL, int TT = 0>
 __global__ void __launch_bounds__(MV_THREADS) qmatvec2_kernel(const MvArgs p, int n_passes) {
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
     extern __shared__ __attribute__((aligned(16))) uint32_t smem[];  // planes [nblocks + 1][MV2_XSTRIDE] (the last block zeros), then the waves' rows
@@ -533,7 +534,7 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec2_kernel(const MvArgs p, in
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int K = p.K, nblocks = K / 32, pair = p.pair;
-    const int T = (nblocks + 63) / 64;
+    const int T = TT > 0 ? TT : (nblocks + 63) / 64;
     const int rb = (int)p.row_bytes;
     const int total = NR * (rb / 16);         // pieces of a pass
     const int half_pieces = total / 2;        // pair: pieces of each matrix' share
@@ -638,7 +639,8 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec2_kernel(const MvArgs p, in
         float acc[NR];
 #pragma unroll
         for (int r = 0; r < NR; r++) acc[r] = 0.f;
-        for (int t = 0; t < T; t++) {
+#pragma unroll
+        for (int t = 0; t < (TT > 0 ? TT : T); t++) {
             const int j = t * 64 + lane;
             const int jx = j < nblocks ? j : nblocks;   // past the row's end: the zero planes
             const int jw = min(j, nblocks - 1);
@@ -702,19 +704,19 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec2_kernel(const MvArgs p, in
     for (; q < n_passes; q += n_waves) pass(q, pc);
 }
 
-template <int NR, int NPL>
+template <int NR, int NPL, int TT = 0>
 void launch_second(vx_backend *be, MvArgs &a, size_t lds) {
     static int per_cu = 0;
     if (per_cu == 0) {
-        (void)hipFuncSetAttribute((const void *)qmatvec2_kernel<NR, NPL>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, qmatvec2_kernel<NR, NPL>, MV_THREADS, lds) != hipSuccess || per_cu < 1)
+        (void)hipFuncSetAttribute((const void *)qmatvec2_kernel<NR, NPL, TT>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, qmatvec2_kernel<NR, NPL, TT>, MV_THREADS, lds) != hipSuccess || per_cu < 1)
             per_cu = 1;
     }
     const int n_passes = a.pair > 0 ? a.pair / (NR / 2) : a.N / NR;
     // as many workgroups as fit at once, or fewer when that makes every wave's number of passes equal
     const int wgs = ceil_div(n_passes, MV_WAVES);
     const int trips = ceil_div(wgs, per_cu * device_cus(be));
-    qmatvec2_kernel<NR, NPL><<<ceil_div(wgs, trips), MV_THREADS, lds, be->stream>>>(a, n_passes);
+    qmatvec2_kernel<NR, NPL, TT><<<ceil_div(wgs, trips), MV_THREADS, lds, be->stream>>>(a, n_passes);
 }
 
 // Launches the second form when it serves the call: Q4_0, an activation row from memory, rows of whole 16-byte
@@ -741,8 +743,11 @@ bool launch_second_form(vx_backend *be, int fmt, MvArgs &a) {
     const size_t lds = (size_t)(nblocks + 1) * MV2_XSTRIDE * 4 + MV_WAVES * (nr * rb + 16);
     if (lds > 120 * 1024) return false;
     a.row_bytes = rb;
-    if (nr == 4) launch_second<4, 9>(be, a, lds);
+    const int steps = (nblocks + 63) / 64;
+    if (nr == 4 && steps == 2) launch_second<4, 9, 2>(be, a, lds);       // K = 4096
+    else if (nr == 4) launch_second<4, 9>(be, a, lds);
     else if (npl == 9) launch_second<2, 9>(be, a, lds);
+    else if (steps == 6) launch_second<2, 13, 6>(be, a, lds);           // K = 11008
     else launch_second<2, 13>(be, a, lds);
     return true;
 }
