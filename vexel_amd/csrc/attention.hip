@@ -5,14 +5,17 @@
 //    optional per-query kv length and optional tree mask. One workgroup per (query, head),
 //    online softmax over chunks of positions. Serves Backend.SDPA, SDPAPrefill and the
 //    single-sequence PagedKVOps methods.
-//  * paged_decode_f16_kernel + paged_merge_kernel: the batched-decode hot path. Ragged
-//    batch, F16 pool, one query per sequence, split over the KV length so a launch has
-//    thousands of workgroups whatever the mix of context lengths. HBM-bound: every K/V
-//    byte is read once with 16-byte loads, a token's head vector is one contiguous
-//    2*head_dim-byte run shared by head_dim/8 lanes.
+//  * paged_decode_f16_kernel (+ paged_merge_kernel where the caller wants plain rows): the
+//    batched-decode hot path. Ragged batch, F16 pool, one query per sequence, split over the KV
+//    length so a launch has thousands of workgroups whatever the mix of context lengths.
+//    HBM-bound: every K/V byte is read once with 16-byte loads, a token's head vector is one
+//    contiguous 2*head_dim-byte run shared by head_dim/8 lanes. When the result goes on to the
+//    output projection the kernel merges its own splits (the last workgroup of a chunk does it).
+//  * prefill_fa2_kernel: tiled causal prefill and paged multi-query attention on the f16
+//    matrix cores (operands as two f16 halves).
 //
-// Arithmetic: float32 dot products and accumulation, softmax through exp2 of the
-// max-subtracted score; the CPU reference (backend/cpu/cpu.go:568-632) normalises the
+// Arithmetic: float32 dot products and accumulation (the tiled kernel: f16 products of
+// two-halves operands, float32 accumulation), softmax through exp2 of the max-subtracted score; the CPU reference (backend/cpu/cpu.go:568-632) normalises the
 // weights before the V accumulation, here the accumulator is divided once at the end.
 #include <float.h>
 
@@ -179,8 +182,8 @@ __global__ void __launch_bounds__(GEN_THREADS) attn_generic_kernel(AttnParams p)
 // and as many V loads. The block id is wave-uniform (scalar load); all 2*NL loads of the next
 // block are in flight while the current block is reduced.
 // Partials (m, l, acc[D]) per (sequence, q head, split) go to a scratch buffer; paged_merge_kernel
-// combines the splits.
-constexpr int TPW = ATTN_TPW;  // tokens per workgroup
+// combines the splits, or the kernel itself does (MergeOut).
+constexpr int TPW = ATTN_TPW;  // tokens per workgroup (smaller, a kernel argument, for batches that would not fill the chip)
 constexpr int HOT_BS = 16;
 
 // Sum over the N adjacent lanes (N = 8, 16 or 32, aligned) that hold one token's head vector, by DPP inside a

@@ -20,12 +20,15 @@
 //     format's integers. With KS > 1 slices the partial sums go to scratch and
 //     qgemm_reduce_kernel adds them in slice order (deterministic), applies the row scale and
 //     the optional residual.
-//     Decode batches (at most two activation tiles per workgroup) whose weight rows fit one round of
-//     workgroups take qgemm_wave_kernel (qgemm_wave.h) instead: one workgroup per compute unit, its
-//     waves split K, activation tiles go from L2 straight to registers.
+//     Decode batches (2 to 32 rows) whose weight rows fit one round of workgroups take
+//     qgemm_wave_kernel (qgemm_wave.h) instead: one workgroup per compute unit, its waves split K,
+//     activation tiles go from L2 straight to registers; BF16 matrices take it at any batch size.
+//     Q8_0 batches of more than 96 rows take qgemm_rows_kernel (same header): the waves split the
+//     weight rows and share 64 activation rows' tiles through LDS.
 //  Each output element depends only on its own activation row and weight row and the launch
-//  shape depends on (N, K) only, so a row gives the same bits alone or inside a batch (the
-//  property the reference keeps by looping M=1 kernels, backend/metal/backend.go:777-779).
+//  shape depends on (N, K) and on which of these kernels the batch size selects, so a row gives
+//  the same bits in any two batches of one range (the property the reference keeps by looping
+//  M=1 kernels, backend/metal/backend.go:777-779).
 //
 // Fallback (Q6_K, odd shapes): one wave per output column, float32 FMAs on the exact
 // dequantised values.
