@@ -450,6 +450,15 @@ def test_fused_decode_blocks_equal_the_unfused_sequence(be, fmt, rows, hidden, f
                 with pytest.raises(VexelError):   # nothing was left prepared
                     be.decode_attn_qkv(0, 0, eps, True, qw["wq"], qw["wk"], qw["wv"], rows, dpos, dslots, dpool2, f16,
                                        hq, hk, d, bs, theta, dq2)
+        # ---- with the step's table of RoPE angles the projection launch finishes its own rows where it can (one
+        # K slice, up to 32 rows; a single row: the matrix-vector kernel's epilogue): same Q and pool
+        if rows <= 64:
+            dx5, dpool5, dq5 = be.upload(x), be.upload(pool), f4(rows, hidden)
+            be.rope_table_prepare(dpos, rows, d, theta)   # (after the uploads: writes to device memory drop the table)
+            be.decode_attn_qkv(dx5, dn1, eps, False, qw["wq"], qw["wk"], qw["wv"], rows, dpos, dslots, dpool5, f16,
+                               hq, hk, d, bs, theta, dq5)
+            near(be.download(dq5, (rows, hidden), np.float32), q_ref, "q with the angle table")
+            near(be.download(dpool5, pool.shape, pool.dtype), pool_ref, "pool with the angle table")
     # mixed formats inside a group are refused, not mis-computed
     other = be.qweight(nx.FMT_Q8_0 if fmt != nx.FMT_Q8_0 else nx.FMT_Q4_0, dW["wk"], kvd, hidden)
     assert not be.decode_attn_qkv_supported(qw["wq"], other, qw["wv"], d)

@@ -285,6 +285,9 @@ class HipBackend:
                   C.byref(wv), rows, positions, slot_mapping, kv_pool, int(bool(pool_is_f16)), num_q_heads,
                   num_kv_heads, head_dim, block_size, theta, q_out)
 
+    def rope_table_prepare(self, positions, rows, head_dim, theta):
+        self.call("vx_rope_table_prepare", positions, rows, head_dim, theta)
+
     def decode_attn_qkv_ex(self, x, norm_weight, eps, x_prepared, wq, wk, wv, q_bias, k_bias, v_bias, rows, positions,
                            slot_mapping, kv_pool, pool_is_f16, num_q_heads, num_kv_heads, head_dim, block_size, theta,
                            rope_dim, rope_neox, q_out):
