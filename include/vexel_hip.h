@@ -222,7 +222,9 @@ typedef struct vx_qweight {
 /* RMSNorm(x, norm_weight) -> Q|K|V projections (one launch) -> RoPE at positions[r] -> rotated Q to
  * q_out [rows,Hq*D], rotated K and V scattered into the pool at slot_mapping[r]
  * (runtime/block.go:834-868). With x_prepared != 0 the normalised activation left prepared by the
- * previous vx_decode_ffn (next_norm_weight) is used and x / norm_weight are ignored. */
+ * previous vx_decode_ffn (next_norm_weight) is used and x / norm_weight are ignored. wq and wk share a format;
+ * wv may have another one (the Q4_K_M mixes keep attn_v in Q6_K): it then is a launch of its own between the shared
+ * prepare and the shared RoPE + store. */
 int vx_decode_attn_qkv_supported(const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int head_dim);
 /* Optional, once per decode step before the layers' vx_decode_attn_qkv calls: works out cos / sin of every (row,
  * dimension pair) for positions[0 .. rows-1] (up to 64 rows, heads up to 256) and keeps them in the backend. While the

@@ -465,6 +465,45 @@ def test_fused_decode_blocks_equal_the_unfused_sequence(be, fmt, rows, hidden, f
     be.reset_pool()
 
 
+@pytest.mark.parametrize("rows", [1, 5, 32, 40])
+@pytest.mark.parametrize("fqk,fv", [(nx.FMT_Q4_K, nx.FMT_Q6_K), (nx.FMT_Q4_0, nx.FMT_Q8_0)])
+def test_decode_attn_qkv_with_v_in_another_format(be, rows, fqk, fv):
+    """The Q4_K_M mixes keep attn_v in Q6_K beside Q4_K attn_q / attn_k: the fused attention half takes V as a launch
+    of its own between the shared prepare and the shared RoPE + store, and gives what the one-call-per-operation
+    sequence gives (runtime/block.go:834-905)."""
+    rng = np.random.default_rng(300 + rows)
+    hidden, hq, hk, d, bs, nblocks, eps, theta = 1024, 16, 4, 64, 16, 24, 1e-5, 10000.0
+    kvd = hk * d
+    dims = dict(wq=(hidden, hidden), wk=(kvd, hidden), wv=(kvd, hidden))
+    fm = dict(wq=fqk, wk=fqk, wv=fv)
+    dW = {n: be.upload(qz.random_quant(fm[n], rng, *dims[n])) for n in dims}
+    qw = {n: be.qweight(fm[n], dW[n], *dims[n]) for n in dims}
+    assert be.decode_attn_qkv_supported(qw["wq"], qw["wk"], qw["wv"], d)
+    x = (rng.standard_normal((rows, hidden)) * 2).astype(np.float32)
+    n1 = rng.standard_normal(hidden).astype(np.float32)
+    pos = rng.integers(0, 3000, rows).astype(np.int32)
+    slots = rng.permutation(nblocks * bs)[:rows].astype(np.int32)
+    pool = _make_pool(rng, True, nblocks, bs, hk, d)
+    dn1, dpos, dslots = be.upload(n1), be.upload(pos), be.upload(slots)
+    f4 = lambda *shape: be.alloc(int(np.prod(shape)) * 4)
+    dx, dpool = be.upload(x), be.upload(pool)
+    dq, dk, dv = f4(rows, hidden), f4(rows, kvd), f4(rows, kvd)
+    be.rmsnorm_prepare(dx, dn1, None, rows, hidden, eps)
+    for name, out in (("wq", dq), ("wk", dk), ("wv", dv)):
+        be.matmul_quant_prepared(fm[name], dW[name], out, None, rows, dims[name][0], hidden)
+    be.rope_store_paged(dq, dk, dv, dpos, dslots, dpool, True, rows, hq, hk, d, bs, theta)
+    q_ref = be.download(dq, (rows, hidden), np.float32)
+    pool_ref = nx.f16_to_f32_array(be.download(dpool, pool.shape, pool.dtype))
+    dx2, dpool2, dq2 = be.upload(x), be.upload(pool), f4(rows, hidden)
+    be.decode_attn_qkv(dx2, dn1, eps, False, qw["wq"], qw["wk"], qw["wv"], rows, dpos, dslots, dpool2, True,
+                       hq, hk, d, bs, theta, dq2)
+    q = be.download(dq2, (rows, hidden), np.float32)
+    assert np.all(np.abs(q - q_ref) <= 2e-5 * np.abs(q_ref).max() + 1e-6)
+    got = nx.f16_to_f32_array(be.download(dpool2, pool.shape, pool.dtype))
+    assert np.all(np.abs(got - pool_ref) <= np.abs(pool_ref) * 2.0 ** -10 + 1e-4)
+    be.reset_pool()
+
+
 # (query heads, kv heads, head size): a workgroup's columns are one 256-column chunk, a quarter or half of one,
 # four of them, and (3 query heads of 128 per kv head) no whole number either way
 @pytest.mark.parametrize("hq,hk,d", [(8, 2, 64), (8, 8, 64), (4, 4, 128), (8, 1, 128), (6, 2, 128)])

@@ -110,6 +110,7 @@ void vx_backend_destroy(vx_backend *be) {
     for (auto &kv : be->permanent) (void)hipFree(kv.first);
     if (be->gemm_ws) (void)hipFree(be->gemm_ws);
     if (be->part_ws) (void)hipFree(be->part_ws);
+    if (be->part_ws2) (void)hipFree(be->part_ws2);
     if (be->attn_ws) (void)hipFree(be->attn_ws);
     if (be->sample_ws) (void)hipFree(be->sample_ws);
     if (be->items.buf) (void)hipFree(be->items.buf);

@@ -74,6 +74,8 @@ struct vx_backend {
     float prep_norm_eps = 0.f;   //      1/rms is still to be taken from the current slot of prep_sync
     void *part_ws = nullptr;     // split-K partial sums
     size_t part_ws_bytes = 0;
+    void *part_ws2 = nullptr;    // a second one: the V projection's, where V is a launch of its own beside Q|K
+    size_t part_ws2_bytes = 0;
     // cos / sin of every (row, pair) of the step's positions (vx_rope_table_prepare): [VX_ROPE_TAB_ROWS][head_dim/2]
     // float2, valid while the key below matches and the library has written nothing since (write_epoch)
     void *rope_tab = nullptr;

@@ -1420,6 +1420,12 @@ __global__ void __launch_bounds__(256) add_partials_kernel(float *__restrict__ x
 // grid = (rows, head groups); thread = (pair j, head lane).
 // GEN: the general form (biases added to the projections before the rotation as matMulTransposedWithBias +
 // applyRoPE do, block.go:497-503,555-560; rope_dim of the head's dimensions rotated, in split pairs when neox).
+// Where the V projection's partial sums are when V was a launch of its own (a weight format other than Q's and K's):
+// [KS][M][ncols], the head vectors from column 0. P == NULL: behind Q and K in the common buffer.
+struct VSrc {
+    const float *P;
+    int KS, ncols;
+};
 struct QkvExtra {
     const float *q_bias, *k_bias, *v_bias;  // [qd], [kvd], [kvd] or nullptr
     int eff_dim, neox;
@@ -1430,10 +1436,10 @@ __global__ void rope_store_general_kernel(const float *__restrict__ P, int KS, i
                                           float *__restrict__ q_out, const int32_t *__restrict__ positions,
                                           const int32_t *__restrict__ slot_mapping, void *__restrict__ pool,
                                           int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta,
-                                          QkvExtra ex) {
+                                          QkvExtra ex, VSrc vs) {
     static_assert(GEN, "the interleaved whole-head form is rope_store_partials_kernel");
     const int row = blockIdx.x, half = head_dim / 2, he = ex.eff_dim / 2;
-    const int qd = num_q_heads * head_dim, kvd = num_kv_heads * head_dim, ncols = qd + 2 * kvd;
+    const int qd = num_q_heads * head_dim, kvd = num_kv_heads * head_dim, ncols = vs.P ? qd + kvd : qd + 2 * kvd;
     const size_t slice_elems = (size_t)M * ncols;
     const float inv = row_factor(inv_scale, rn, row);  // every wave of the block, before any lane leaves
     const int pos = positions[row], slot = slot_mapping[row];
@@ -1462,6 +1468,14 @@ __global__ void rope_store_general_kernel(const float *__restrict__ P, int KS, i
         v = __fmul_rn(v, inv);
         return bias ? __fadd_rn(v, bias[bcol]) : v;
     };
+    auto velem = [&](int bcol) {
+        if (!vs.P) return elem(qd + kvd + bcol, ex.v_bias, bcol);
+        const float *p0 = vs.P + (size_t)row * vs.ncols + bcol;
+        float v = *p0;
+        for (int s = 1; s < vs.KS; s++) v += p0[(size_t)s * M * vs.ncols];
+        v = __fmul_rn(v, inv);
+        return ex.v_bias ? __fadd_rn(v, ex.v_bias[bcol]) : v;
+    };
     for (int h = h0; h < num_q_heads; h += hstride) {
         const int b0 = h * head_dim + i0, b1 = h * head_dim + i1;
         const float a = elem(b0, ex.q_bias, b0), b = elem(b1, ex.q_bias, b1);
@@ -1471,7 +1485,7 @@ __global__ void rope_store_general_kernel(const float *__restrict__ P, int KS, i
     for (int h = h0; h < num_kv_heads; h += hstride) {
         const int b0 = h * head_dim + i0, b1 = h * head_dim + i1;
         const float a = elem(qd + b0, ex.k_bias, b0), b = elem(qd + b1, ex.k_bias, b1);
-        const float va = elem(qd + kvd + b0, ex.v_bias, b0), vb = elem(qd + kvd + b1, ex.v_bias, b1);
+        const float va = velem(b0), vb = velem(b1);
         const float ka = turn ? __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, sn)) : a;
         const float kb = turn ? __fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, c)) : b;
         if (F16) {
@@ -1494,9 +1508,10 @@ template <bool F16>
 __global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, int M, const float *__restrict__ inv_scale, RowNorm rn,
                                            float *__restrict__ q_out, const int32_t *__restrict__ positions,
                                            const int32_t *__restrict__ slot_mapping, void *__restrict__ pool,
-                                           int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta) {
+                                           int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta,
+                                           VSrc vs) {
     const int row = blockIdx.x, half = head_dim / 2;
-    const int qd = num_q_heads * head_dim, kvd = num_kv_heads * head_dim, ncols = qd + 2 * kvd;
+    const int qd = num_q_heads * head_dim, kvd = num_kv_heads * head_dim, ncols = vs.P ? qd + kvd : qd + 2 * kvd;
     const size_t slice_elems = (size_t)M * ncols;
     const float inv = row_factor(inv_scale, rn, row);  // every wave of the block, before any lane leaves
     const int pos = positions[row], slot = slot_mapping[row];
@@ -1521,6 +1536,21 @@ __global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, 
         a = __fmul_rn(v.x, inv);
         b = __fmul_rn(v.y, inv);
     };
+    auto vpair = [&](int col, float &a, float &b) {
+        if (!vs.P) {
+            pair(qd + kvd + col, a, b);
+            return;
+        }
+        const float *p0 = vs.P + (size_t)row * vs.ncols + col;
+        float2 v = *(const float2 *)p0;
+        for (int s = 1; s < vs.KS; s++) {
+            const float2 t = *(const float2 *)(p0 + (size_t)s * M * vs.ncols);
+            v.x += t.x;
+            v.y += t.y;
+        }
+        a = __fmul_rn(v.x, inv);
+        b = __fmul_rn(v.y, inv);
+    };
     for (int h = h0; h < num_q_heads; h += hstride) {
         float a, b;
         pair(h * head_dim + 2 * j, a, b);
@@ -1532,7 +1562,7 @@ __global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, 
     for (int h = h0; h < num_kv_heads; h += hstride) {
         float a, b, va, vb;
         pair(qd + h * head_dim + 2 * j, a, b);
-        pair(qd + kvd + h * head_dim + 2 * j, va, vb);
+        vpair(h * head_dim + 2 * j, va, vb);
         const float ka = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, sn));
         const float kb = __fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, c));
         const size_t o = (size_t)h * head_dim + 2 * j;
@@ -2128,9 +2158,12 @@ int vx_rope_table_prepare(vx_backend *be, const int32_t *positions, int rows, in
     return VX_OK;
 }
 
+// Q and K of one format; V of the same, or of another with a matrix-core path (the Q4_K_M mixes keep attn_v in Q6_K):
+// it then is a launch of its own between the shared prepare and the shared RoPE + store.
 int vx_decode_attn_qkv_supported(const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int head_dim) {
-    const vx_qweight *ws[3] = {wq, wk, wv};
-    return group_ok(ws, 3) && head_dim % 2 == 0 && head_dim <= 512 && (size_t)wq->k * 4 <= 64 * 1024;
+    const vx_qweight *ws[3] = {wq, wk, wv}, *wvs[1] = {wv};
+    const bool ok = group_ok(ws, 3) || (group_ok(ws, 2) && group_ok(wvs, 1) && wv->k == wq->k);
+    return ok && head_dim % 2 == 0 && head_dim <= 512 && (size_t)wq->k * 4 <= 64 * 1024;
 }
 
 int vx_decode_attn_qkv(vx_backend *be, const float *x, const float *norm_weight, float eps, int x_prepared,
@@ -2170,7 +2203,36 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
         const void *mw[3] = {wq->data, wk->data, wv->data};
         const int mn[3] = {wq->n, wk->n, wv->n};
         const int ntot1 = wq->n + wk->n + wv->n;
-        if (x && norm_weight && matvec_ok(wq->fmt, mw, mn, 3, k)) {
+        const bool mixed1 = wv->fmt != wq->fmt;
+        if (x && norm_weight && mixed1 && matvec_ok(wq->fmt, mw, mn, 2, k) && matvec_ok(wv->fmt, mw + 2, mn + 2, 1, k)) {
+            // V in another format: its own launch, the outputs side by side
+            rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, (size_t)ntot1 * sizeof(float), "split-K partial sums");
+            if (rc) return rc;
+            MatvecSource src;
+            src.x = x;
+            src.norm_w = norm_weight;
+            src.eps = eps;
+            rc = run_matvec_fused(be, wq->fmt, mw, mn, 2, k, src, (float *)be->part_ws, nullptr, 0);
+            if (rc) return rc;
+            rc = run_matvec_fused(be, wv->fmt, mw + 2, mn + 2, 1, k, src, (float *)be->part_ws + wq->n + wk->n, nullptr, 0);
+            if (rc) return rc;
+            const int half1 = head_dim / 2;
+            const int lanes1 = 256 / half1 > 0 ? 256 / half1 : 1;
+            const int max_heads1 = num_q_heads > num_kv_heads ? num_q_heads : num_kv_heads;
+            const RowNorm none = {nullptr, 0, 0.f, 0.f};
+            const VSrc same = {nullptr, 0, 0};
+            if (gen)
+                rope_store_general_kernel<true, true><<<dim3(1, ceil_div(max_heads1, lanes1)), lanes1 * half1, 0, be->stream>>>(
+                    (const float *)be->part_ws, 1, 1, be->ones, none, q_out, positions, slot_mapping, kv_pool, num_q_heads,
+                    num_kv_heads, head_dim, block_size, theta, ex, same);
+            else
+                rope_store_partials_kernel<true><<<dim3(1, ceil_div(max_heads1, lanes1)), lanes1 * half1, 0, be->stream>>>(
+                    (const float *)be->part_ws, 1, 1, be->ones, none, q_out, positions, slot_mapping, kv_pool, num_q_heads,
+                    num_kv_heads, head_dim, block_size, theta, same);
+            VX_CHECK_LAUNCH();
+            return VX_OK;
+        }
+        if (x && norm_weight && !mixed1 && matvec_ok(wq->fmt, mw, mn, 3, k)) {
             rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, (size_t)ntot1 * sizeof(float), "split-K partial sums");
             if (rc) return rc;
             MatvecSource src;
@@ -2204,11 +2266,11 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
             if (gen)
                 rope_store_general_kernel<true, true><<<dim3(1, ceil_div(max_heads1, lanes1)), lanes1 * half1, 0, be->stream>>>(
                     (const float *)be->part_ws, 1, 1, be->ones, none, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-                    num_kv_heads, head_dim, block_size, theta, ex);
+                    num_kv_heads, head_dim, block_size, theta, ex, VSrc{nullptr, 0, 0});
             else
                 rope_store_partials_kernel<true><<<dim3(1, ceil_div(max_heads1, lanes1)), lanes1 * half1, 0, be->stream>>>(
                     (const float *)be->part_ws, 1, 1, be->ones, none, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-                    num_kv_heads, head_dim, block_size, theta);
+                    num_kv_heads, head_dim, block_size, theta, VSrc{nullptr, 0, 0});
             VX_CHECK_LAUNCH();
             return VX_OK;
         }
@@ -2221,11 +2283,26 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
         if (rc) return rc;
     }
     const vx_qweight *ws[3] = {wq, wk, wv};
+    const bool mixed = wv->fmt != wq->fmt;
     int ntot, ks;
-    const Segs segs = make_segs(ws, 3, &ntot);
+    const Segs segs = make_segs(ws, mixed ? 2 : 3, &ntot);
+    VSrc vs = {nullptr, 0, 0};
+    if (mixed) {
+        // V first, into the second partial-sum area (the two change places around its launch), then Q|K as usual
+        const vx_qweight *wvs[1] = {wv};
+        int nv, ksv;
+        const Segs sv = make_segs(wvs, 1, &nv);
+        std::swap(be->part_ws, be->part_ws2);
+        std::swap(be->part_ws_bytes, be->part_ws2_bytes);
+        rc = launch_gemm_fmt(be, wv->fmt, sv, nv, nullptr, nullptr, true, rows, k, &ksv);
+        std::swap(be->part_ws, be->part_ws2);
+        std::swap(be->part_ws_bytes, be->part_ws2_bytes);
+        if (rc) return rc;
+        vs = VSrc{(const float *)be->part_ws2, ksv, nv};
+    }
     // One K slice, one activation group, the plain RoPE form and a table of this step's angles: the GEMM's workgroups
     // finish their own rows (no partial sums, no second launch).
-    {
+    if (!mixed) {
         const WavePlan pl = wave_plan(be, wq->fmt, segs, ntot, k, rows);
         const bool table = be->rope_tab_pos == positions && be->rope_tab_rows >= rows && be->rope_tab_dim == head_dim &&
                            be->rope_tab_theta == theta && be->rope_tab_epoch == be->write_epoch;
@@ -2261,19 +2338,19 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
     if (gen && pool_is_f16)
         rope_store_general_kernel<true, true><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-            num_kv_heads, head_dim, block_size, theta, ex);
+            num_kv_heads, head_dim, block_size, theta, ex, vs);
     else if (gen)
         rope_store_general_kernel<false, true><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-            num_kv_heads, head_dim, block_size, theta, ex);
+            num_kv_heads, head_dim, block_size, theta, ex, vs);
     else if (pool_is_f16)
         rope_store_partials_kernel<true><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-            num_kv_heads, head_dim, block_size, theta);
+            num_kv_heads, head_dim, block_size, theta, vs);
     else
         rope_store_partials_kernel<false><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-            num_kv_heads, head_dim, block_size, theta);
+            num_kv_heads, head_dim, block_size, theta, vs);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }
