@@ -177,28 +177,32 @@ def test_matmul_quant_vs_oracle(be, fmt, m):
 
 @pytest.mark.parametrize("fmt", FMTS_MFMA)
 def test_matmul_rows_independent_of_batch(be, fmt):
-    """A row has the same bits in a batch of 2 and of 32, and the same bits in a batch of 40 and of 72: the k-slices
-    and the order their sums are added in depend on the matrix, the device and the kernel only, and the kernel
-    changes at 32 rows (cf. the reference's loop of M=1 kernels, backend/metal/backend.go:777-779). Across that
-    boundary, and for a single row (M = 1, the matrix-vector kernel), rows agree to rounding, not bit for bit."""
+    """A row has the same bits in a batch of 2 and of 32, in a batch of 40 and of 64, and in a batch of 72 and of
+    90: the k-slices and the order their sums are added in depend on the matrix, the device and the kernel only, and
+    the kernel (or its cut of the matrix) changes at 32 and at 64 rows (cf. the reference's loop of M=1 kernels,
+    backend/metal/backend.go:777-779). Across those boundaries, and for a single row (M = 1, the matrix-vector
+    kernel), rows agree to rounding, not bit for bit."""
     rng = np.random.default_rng(9)
     m, n, k = 32, 96, 2048
     w = qz.random_quant(fmt, rng, n, k)
-    big = rng.standard_normal((72, k)).astype(np.float32)
+    big = rng.standard_normal((90, k)).astype(np.float32)
     a = big[:m]
     da, dw = be.upload(big), be.upload(w)
-    dout = be.alloc(m * n * 4)
-    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
-    full = be.download(dout, (m, n), np.float32)
-    dbig = be.alloc(72 * n * 4)
-    be.matmul_quant(fmt, da, dw, dbig, None, 72, n, k)
-    many = be.download(dbig, (72, n), np.float32)
-    d40 = be.alloc(40 * n * 4)
-    be.matmul_quant(fmt, da, dw, d40, None, 40, n, k)
-    assert np.array_equal(many[:40].view(np.uint32), be.download(d40, (40, n), np.float32).view(np.uint32))
-    want = nx.matmul_quant(fmt, big, w, 72, n, k)
-    _close(many, want, 2e-5, 3e-6 * np.abs(want).max() + 1e-7, "72-row batch")
+
+    def batch(rows):
+        d = be.alloc(rows * n * 4)
+        be.matmul_quant(fmt, da, dw, d, None, rows, n, k)
+        return be.download(d, (rows, n), np.float32)
+
+    full, many = batch(m), batch(90)
+    assert np.array_equal(many[:72].view(np.uint32), batch(72).view(np.uint32))
+    mid = batch(64)
+    assert np.array_equal(mid[:40].view(np.uint32), batch(40).view(np.uint32))
+    want = nx.matmul_quant(fmt, big, w, 90, n, k)
+    _close(many, want, 2e-5, 3e-6 * np.abs(want).max() + 1e-7, "90-row batch")
+    _close(mid, want[:64], 2e-5, 3e-6 * np.abs(want).max() + 1e-7, "64-row batch")
     assert np.all(np.abs(many[:m] - full) <= 2e-6 * np.abs(full).max() + 1e-7)
+    assert np.all(np.abs(mid[:m] - full) <= 2e-6 * np.abs(full).max() + 1e-7)
     for r in (0, 5, 30):
         d2 = be.alloc(2 * n * 4)
         be.matmul_quant(fmt, da + r * k * 4, dw, d2, None, 2, n, k)
@@ -233,10 +237,31 @@ def test_matvec_single_row(be, fmt, n, k):
     be.reset_pool()
 
 
+@pytest.mark.parametrize("fmt", [nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q4_K])
+@pytest.mark.parametrize("m,n,k", [(33, 4112, 512), (48, 12304, 256), (64, 96, 4096), (50, 1040, 2048)])
+def test_matmul_33_to_64_rows(be, fmt, m, n, k):
+    """Batches of 33 to 64 rows (four activation tiles a step in the kernel whose waves split K): a matrix tall
+    enough for several rounds of workgroups, heights that leave the last workgroup overlapping its neighbour, several
+    K slices, rows of padding in the last tile; with and without the residual."""
+    rng = np.random.default_rng(m + n + k + fmt)
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    want = nx.matmul_quant(fmt, a, w, m, n, k)
+    da, dw, dres = be.upload(a), be.upload(w), be.upload(res)
+    dout = be.alloc(m * n * 4)
+    scale = np.abs(want).max()
+    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
+    _close(be.download(dout, (m, n), np.float32), want, 2e-5, 3e-6 * scale + 1e-7, "%dx%dx%d" % (m, n, k))
+    be.matmul_quant(fmt, da, dw, dout, dres, m, n, k)
+    _close(be.download(dout, (m, n), np.float32), want + res, 2e-5, 3e-6 * scale + 1e-6, "with the residual")
+    be.reset_pool()
+
+
 @pytest.mark.parametrize("fmt", [nx.FMT_Q4_0, nx.FMT_Q6_K])
 def test_matmul_rows_independent_at_prefill_size(be, fmt):
     """1024 rows against a 2048-row matrix: enough (row group, activation group) pairs that one workgroup walks
-    the k-slices in order instead of one workgroup per slice. Rows keep the bits they have in a batch of 34."""
+    the k-slices in order instead of one workgroup per slice. Rows keep the bits they have in a batch of 70."""
     rng = np.random.default_rng(19)
     m, n, k = 1024, 2048, 512
     w = qz.random_quant(fmt, rng, n, k)
@@ -245,10 +270,10 @@ def test_matmul_rows_independent_at_prefill_size(be, fmt):
     dout = be.alloc(m * n * 4)
     be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
     full = be.download(dout, (m, n), np.float32)
-    for r in (0, 517, 990):
-        d2 = be.alloc(34 * n * 4)
-        be.matmul_quant(fmt, da + r * k * 4, dw, d2, None, 34, n, k)
-        assert np.array_equal(be.download(d2, (34, n), np.float32).view(np.uint32), full[r:r + 34].view(np.uint32))
+    for r in (0, 517, 954):
+        d2 = be.alloc(70 * n * 4)
+        be.matmul_quant(fmt, da + r * k * 4, dw, d2, None, 70, n, k)
+        assert np.array_equal(be.download(d2, (70, n), np.float32).view(np.uint32), full[r:r + 70].view(np.uint32))
     want = nx.matmul_quant(fmt, a[:64], w, 64, n, k)
     _close(full[:64], want, 2e-5, 3e-6 * np.abs(want).max() + 1e-7, "1024-row batch")
     be.reset_pool()
@@ -796,6 +821,54 @@ def test_paged_decode_single_batched_ragged(be, f16, shape):
     do2 = be.alloc(q.nbytes)
     be.sdpa_paged_decode_ragged(dq, dpool, f16, dmat, dl, do2, B, mb, bs, hq, hk, d, sc, max(lens))
     _close(be.download(do2, q.shape, np.float32), want, 1e-5, 3e-6, "paged ragged")
+    be.reset_pool()
+
+
+@pytest.mark.parametrize("hq,hk,d", [(8, 2, 128), (16, 2, 64), (6, 2, 128)])
+def test_paged_decode_grouped_queries_value_ranges(be, hq, hk, d):
+    """The grouped-query kernel scales every query row by a power of two before it splits it into two f16 halves and
+    carries the softmax weights times 2^10: rows of very large and very small magnitude, a zero row, a row with one
+    dominant element, scores peaked on one token with a long tail of small weights, contexts that end inside a
+    block and on a split boundary."""
+    rng = np.random.default_rng(77 + hq + d)
+    bs, nblocks = 16, 200
+    pool = _make_pool(rng, True, nblocks, bs, hk, d)
+    dpool = be.upload(pool)
+    sc = np.float32(1 / math.sqrt(d))
+    lens = [700, 37, 513, 16, 1024, 256, 300]
+    B, mb = len(lens), 64
+    perm = rng.permutation(nblocks)
+    mat = np.zeros((B, mb), dtype=np.int32)
+    tables, off = [], 0
+    for i, L in enumerate(lens):
+        nb = (L + bs - 1) // bs
+        mat[i, :nb] = perm[off:off + nb]
+        tables.append(mat[i, :nb].copy()); off += nb
+    q = rng.standard_normal((B, hq, d)).astype(np.float32)
+    q[0] *= 1e3
+    q[1] *= 1e-6
+    q[2, 1] = 0.0
+    q[3, :, 5] = 4000.0
+    q[4] *= 30.0                       # peaked: one token takes nearly all the weight, a thousand share the rest
+    q[5, 0] *= 1e-20
+    q[6, ::2] *= 200.0
+    want = np.stack([nx.sdpa_paged_decode(q[i], pool, tables[i], len(tables[i]), bs, hq, hk, d, sc,
+                                          lens[i] - (len(tables[i]) - 1) * bs) for i in range(B)])
+    dq, dmat, dl = be.upload(q), be.upload(mat), be.upload(np.array(lens, dtype=np.int32))
+    do = be.alloc(q.nbytes)
+    be.sdpa_paged_decode_ragged(dq, dpool, True, dmat, dl, do, B, mb, bs, hq, hk, d, sc, mb * bs)
+    got = be.download(do, q.shape, np.float32)
+    assert np.isfinite(got).all()
+    # A query row enters with 22 significant bits relative to its largest element, so a score s carries an error of
+    # about 2^-22 |s| (float32 dot products: 2^-24 |s| and their own rounding); where the scores reach into the
+    # hundreds that shows in the weights, and the bar widens with the largest score of the sequence.
+    errs = []
+    for i in range(B):
+        smax = float(np.abs(q[i]).max() * 6.0 * math.sqrt(d) * sc * math.sqrt(2.0)) if lens[i] > 16 else 0.0
+        tol = 3e-6 + 2.0 ** -21 * min(smax, 64.0)
+        e = np.abs(got[i].astype(np.float64) - want[i]) - 1e-5 * np.abs(want[i])
+        errs.append((i, float(e.max()), tol))
+    assert all(e <= t for _, e, t in errs), errs
     be.reset_pool()
 
 

@@ -11,10 +11,12 @@
 //    HBM-bound: every K/V byte is read once with 16-byte loads, a token's head vector is one
 //    contiguous 2*head_dim-byte run shared by head_dim/8 lanes. When the result goes on to the
 //    output projection the kernel merges its own splits (the last workgroup of a chunk does it).
+//  * paged_decode_gqa_kernel: the same for grouped queries (2 to 16 queries per K/V row, heads of 64 or
+//    128) and for the batched tree attention's entries, on the f16 matrix cores; same splits, same merge.
 //  * prefill_fa2_kernel: tiled causal prefill and paged multi-query attention on the f16
 //    matrix cores (operands as two f16 halves).
 //
-// Arithmetic: float32 dot products and accumulation (the tiled kernel: f16 products of
+// Arithmetic: float32 dot products and accumulation (the matrix-core kernels: f16 products of
 // two-halves operands, float32 accumulation), softmax through exp2 of the max-subtracted score; the CPU reference (backend/cpu/cpu.go:568-632) normalises the
 // weights before the V accumulation, here the accumulator is divided once at the end.
 #include <float.h>
@@ -186,6 +188,24 @@ __global__ void __launch_bounds__(GEN_THREADS) attn_generic_kernel(AttnParams p)
 constexpr int TPW = ATTN_TPW;  // tokens per workgroup (smaller, a kernel argument, for batches that would not fill the chip)
 constexpr int HOT_BS = 16;
 
+// x = h + l in two f16 halves. The float32 value, its rounded half and their difference each pass through a register
+// of their own: left to itself the compiler folds the operations that produced x into mixed-precision
+// multiply-adds that round once from the unrounded product, and the halves then add up to less than x's 24 bits
+// (measured: attention outputs off by 3e-5 instead of 1e-6).
+struct HalfPair { _Float16 h, l; };
+__device__ __forceinline__ HalfPair split_hl(float x) {
+    asm volatile("" : "+v"(x));
+    HalfPair r;
+    r.h = (_Float16)x;
+    float hf = (float)r.h;
+    asm volatile("" : "+v"(hf));
+    float d = x - hf;
+    asm volatile("" : "+v"(d));
+    r.l = (_Float16)d;
+    return r;
+}
+typedef float float4v __attribute__((ext_vector_type(4)));
+
 // Sum over the N adjacent lanes (N = 8, 16 or 32, aligned) that hold one token's head vector, by DPP inside a
 // 16-lane row (no LDS traffic): quads, then the mirrored quad of the half, then the mirrored half; heads of 256
 // span two rows, joined by one cross-row exchange.
@@ -219,6 +239,73 @@ __device__ __forceinline__ void put_merged(const MergeOut &mg, int row, int c, c
     }
     write_chunk(mg.pv, row, c, y, mg.mpad);
     if (c == 0 && lane == 0) mg.pv.inv_scale[row] = 1.f;
+}
+
+// What follows once each of the workgroup's 4 waves has left its (m, l, acc) of the G*RG queries in LDS: the waves'
+// sums are combined, written as the split's partial sums and, with mg.cnt, merged over the splits by the workgroup
+// that arrives last at its chunk of 256 output columns.
+template <int D, int G, int RG>
+__device__ __forceinline__ void finish_split(const float (&s_m)[4][G * RG], const float (&s_l)[4][G * RG],
+                                             const float (&s_acc)[4][G * RG][D], float *__restrict__ partial, int seq,
+                                             int kvh, int split, int kv_len, int num_q_heads, int num_kv_heads,
+                                             int max_splits, const MergeOut &mg, int tps) {
+    constexpr int GG = G * RG;
+    constexpr int GD = G * D;                          // this workgroup's columns of the output
+    constexpr bool MERGES = RG == 1 && (GD % 256 == 0 || 256 % GD == 0);
+    constexpr int CH = GD >= 256 ? GD / 256 : 1;       // 256-column chunks inside them
+    constexpr int HPC = GD >= 256 ? 1 : 256 / GD;      // kv heads that share a chunk
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    __syncthreads();
+    for (int idx = tid; idx < GG * D; idx += 256) {
+        const int g = idx / D, d = idx % D;
+        float M = fmaxf(fmaxf(s_m[0][g], s_m[1][g]), fmaxf(s_m[2][g], s_m[3][g]));
+        float L = 0.f, A = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float f = (s_m[w][g] == -INFINITY) ? 0.f : exp2f(s_m[w][g] - M);
+            L += s_l[w][g] * f;
+            A += s_acc[w][g][d] * f;
+        }
+        const int qh = kvh * G + g % G;
+        float *po = partial + ((((size_t)seq * RG + g / G) * num_q_heads + qh) * max_splits + split) * (D + 2);
+        // (device-scope stores: written through to where a workgroup on another die reads them, see below)
+        __hip_atomic_store(po + 2 + d, A, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (d == 0) {
+            __hip_atomic_store(po, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(po + 1, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    // The last workgroup to arrive at a (sequence, chunk of 256 output columns) merges the chunk's splits in
+    // index order - the sums do not depend on who that is - and writes it as the next GEMM's operand.
+    if constexpr (MERGES) {
+        if (!mg.cnt) return;
+        // Ordering without device-wide cache write-backs and invalidations (a release / acquire fence pair at
+        // device scope costs this kernel several times its run time: every workgroup would flush and drop its
+        // die's L2): the partial sums above are device-scope stores and are read back by device-scope loads, which
+        // the dies' caches do not hold back or serve stale; each wave waits until its stores are acknowledged
+        // before the workgroup's barrier, thread 0 counts the arrival after the barrier, and whoever counts the
+        // last one reads only after that atomic has returned.
+        __shared__ int s_last;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        const int ns = (kv_len + tps - 1) / tps;  // workgroups of one kv head that arrive for this sequence
+        const int unit = kvh / HPC;
+        if (tid == 0) {
+            int32_t *cnt = mg.cnt + (size_t)seq * (num_kv_heads / HPC) + unit;
+            const int last = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ns * HPC - 1;
+            if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // (nobody else comes before the next launch)
+            s_last = last;
+        }
+        __syncthreads();
+        if (!s_last) return;
+        for (int ch = wave; ch < CH; ch += 4) {
+            const int c = unit * CH + ch;
+            float y[4];
+            split_merge4<true>(partial, ns, num_q_heads, D, max_splits, seq, c * 256 + lane * 4, y);
+            put_merged(mg, seq, c, y, num_q_heads * D);
+        }
+    }
 }
 
 // RG > 1: an entry of the batch is RG consecutive query rows that share one sequence's context (the rows of a
@@ -383,56 +470,207 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
             }
         }
     }
-    __syncthreads();
-    for (int idx = tid; idx < GG * D; idx += 256) {
-        const int g = idx / D, d = idx % D;
-        float M = fmaxf(fmaxf(s_m[0][g], s_m[1][g]), fmaxf(s_m[2][g], s_m[3][g]));
-        float L = 0.f, A = 0.f;
+    finish_split<D, G, RG>(s_m, s_l, s_acc, partial, seq, kvh, split, kv_len, num_q_heads, num_kv_heads, max_splits, mg, tps);
+}
+
+// The same split of the work for grouped queries (G*RG = 2 .. 16 queries per K/V row) on the matrix cores: the vector
+// form above repeats its multiply-adds, reductions and exponentials per query and is bound by them from G = 2 on.
+// Per 16-token block a wave forms
+//   S^T[token][query] = K Q^T   with v_mfma_f32_16x16x32_f16: A = K (exact f16), B = Q^T as hi + lo f16 halves of
+//                               the row scaled by a power of two (so that the halves carry 22 bits of every element
+//                               relative to the row's largest), D/32 steps x 2 halves;
+//   O[query][d] += P V          with v_mfma_f32_16x16x16_f16: A = P as hi + lo halves of 2^10 p (p <= 1; the factor
+//                               is carried as m - 10 in the partial sums), B = V (exact f16), D/16 tiles x 2 halves.
+// The operand layouts are chosen so that nothing moves between lanes: as A operand, lane (c = lane % 16,
+// g = lane / 16) holds row 4*(c % 4) + c / 4 of the block's K, so that the result's lane (query c, g) holds the
+// scores of the tokens 4i + g, i = 0..3 - which is the A operand of the second product as it stands - and the
+// V rows of exactly those tokens, D/16 columns from c * D/16 on, are what the same lane loads (for D = 128 the
+// 16 bytes per lane of the vector form: whole rows per instruction); tile e of the output holds columns
+// c * D/16 + e. Rows of Q beyond G*RG are zero and their results are dropped.
+template <int D, int G, int RG = 1>
+__global__ void __launch_bounds__(256, 3) paged_decode_gqa_kernel(
+    const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix,
+    const int32_t *__restrict__ bt_rows, int max_blocks, const int32_t *__restrict__ kv_lens,
+    float *__restrict__ partial, int num_q_heads, int num_kv_heads, float scale, int max_splits,
+    const int32_t *__restrict__ items, MergeOut mg, int tps) {
+    constexpr int GG = G * RG;
+    static_assert(GG >= 1 && GG <= 16 && (D == 64 || D == 128), "up to 16 queries per K/V row, heads of 64 or 128");
+    constexpr int NS = D / 32;  // steps of the first product (32 head elements each)
+    constexpr int NT = D / 16;  // 16-column tiles of the output = halves per lane and token of V
+    typedef _Float16 halfv __attribute__((ext_vector_type(NT)));
+    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+    const int kvh = blockIdx.x;
+    int split = blockIdx.y, seq = blockIdx.z, kv_len, row;
+    if (items) {
+        if ((int)blockIdx.y >= items[0]) return;
+        const int4 rec = ((const int4 *)(items + 4))[blockIdx.y];  // (sequence, split, kv length, table row)
+        seq = rec.x;
+        split = rec.y;
+        kv_len = rec.z;
+        row = rec.w;
+    } else {
+        kv_len = kv_lens[seq];
+        row = bt_rows ? bt_rows[seq] : seq;
+    }
+    kv_len = min(kv_len, max_splits * tps);
+    const int t_begin = split * tps;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int GD = G * D;
+    constexpr bool MERGES = RG == 1 && (GD % 256 == 0 || 256 % GD == 0);
+    constexpr int CH = GD >= 256 ? GD / 256 : 1;
+    constexpr int HPC = GD >= 256 ? 1 : 256 / GD;
+    if (split >= max_splits || t_begin >= kv_len) {
+        if constexpr (MERGES) {
+            if (mg.cnt && kv_len == 0 && split == 0 && kvh % HPC == 0) {
+                const float zero[4] = {0.f, 0.f, 0.f, 0.f};
+                for (int ch = wave; ch < CH; ch += 4) put_merged(mg, seq, kvh / HPC * CH + ch, zero, num_q_heads * D);
+            }
+        }
+        return;
+    }
+    const int t_end = min(kv_len, t_begin + tps);
+    const int32_t *bt = bt_matrix + (size_t)row * max_blocks + t_begin / HOT_BS;
+    const int c16 = lane & 15, g4 = lane >> 4;
+    const size_t hs = (size_t)num_kv_heads * D;
+    const size_t part = (size_t)HOT_BS * hs;
+
+    // Q^T as the B operand: lane (query c16, head elements g4 * D/4 + 8s .. + 7 in step s), times scale * log2(e)
+    // and the row's power of two, hi + lo
+    half8 qh[NS], ql[NS];
+    float q_inv;  // undoes the power of two on this lane's scores (query c16)
+    {
+        float x[NS][8];
+        float amax = 0.f;
+        const float qs = scale * kLog2e;
+        const float *qp = q + (((size_t)seq * RG + c16 / G) * num_q_heads + (size_t)kvh * G + c16 % G) * D + g4 * (D / 4);
 #pragma unroll
-        for (int w = 0; w < 4; w++) {
-            const float f = (s_m[w][g] == -INFINITY) ? 0.f : exp2f(s_m[w][g] - M);
-            L += s_l[w][g] * f;
-            A += s_acc[w][g][d] * f;
+        for (int s = 0; s < NS; s++) {
+            float4 a = make_float4(0.f, 0.f, 0.f, 0.f), b = a;
+            if (c16 < GG) {
+                a = *(const float4 *)(qp + 8 * s);
+                b = *(const float4 *)(qp + 8 * s + 4);
+            }
+            const float t[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                x[s][e] = t[e] * qs;
+                amax = fmaxf(amax, fabsf(x[s][e]));
+            }
         }
-        const int qh = kvh * G + g % G;
-        float *po = partial + ((((size_t)seq * RG + g / G) * num_q_heads + qh) * max_splits + split) * (D + 2);
-        // (device-scope stores: written through to where a workgroup on another die reads them, see below)
-        __hip_atomic_store(po + 2 + d, A, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (d == 0) {
-            __hip_atomic_store(po, M, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(po + 1, L, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        int ex = 11;
+        if (amax > 0.f && amax < INFINITY) {
+            (void)frexpf(amax, &ex);  // amax = mantissa in [0.5, 1) * 2^ex
+            ex = max(ex, -60);
+        }
+        const float f = ldexpf(1.f, 11 - ex);  // the row's largest element lands in [1024, 2048)
+        q_inv = ldexpf(1.f, ex - 11);
+#pragma unroll
+        for (int s = 0; s < NS; s++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const HalfPair t = split_hl(x[s][e] * f);
+                qh[s][e] = t.h;
+                ql[s][e] = t.l;
+            }
+    }
+    float4v o[NT];
+#pragma unroll
+    for (int e = 0; e < NT; e++) o[e] = (float4v){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;  // of query c16; l_run over this lane's tokens only until the end
+
+    const int n_blocks = (t_end - t_begin + HOT_BS - 1) / HOT_BS;
+    const size_t k_off = (size_t)(4 * (c16 & 3) + (c16 >> 2)) * hs + (size_t)kvh * D + g4 * (D / 4);
+    const size_t v_off = part + (size_t)g4 * hs + (size_t)kvh * D + c16 * NT;
+    half8 kk[NS], kn[NS];
+    halfv vv[4], vn[4];
+    auto issue = [&](int bi, half8 *kd, halfv *vd) {
+        const int blk = __builtin_amdgcn_readfirstlane(bt[bi]);
+        const _Float16 *base = pool + (size_t)blk * 2 * part;
+#pragma unroll
+        for (int s = 0; s < NS; s++) kd[s] = *(const half8 *)(base + k_off + 8 * s);
+#pragma unroll
+        for (int i = 0; i < 4; i++) vd[i] = *(const halfv *)(base + v_off + (size_t)i * 4 * hs);  // token 4i + g4
+    };
+    if (wave < n_blocks) issue(wave, kn, vn);
+    for (int bi = wave; bi < n_blocks; bi += 4) {
+#pragma unroll
+        for (int s = 0; s < NS; s++) kk[s] = kn[s];
+#pragma unroll
+        for (int i = 0; i < 4; i++) vv[i] = vn[i];
+        if (bi + 4 < n_blocks) issue(bi + 4, kn, vn);
+        __builtin_amdgcn_sched_barrier(0);
+        float4v sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk[s], qh[s], sc, 0, 0, 0);
+            sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk[s], ql[s], sc, 0, 0, 0);
+        }
+        const int tok0 = t_begin + bi * HOT_BS + g4;             // sc[i]: token tok0 + 4i
+        const bool whole = t_begin + (bi + 1) * HOT_BS <= t_end;  // (the same for the whole wave)
+        float sv[4], gm = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            sv[i] = (whole || tok0 + 4 * i < t_end) ? sc[i] * q_inv : -INFINITY;
+            gm = fmaxf(gm, sv[i]);
+        }
+        gm = fmaxf(gm, __shfl_xor(gm, 16, 64));
+        gm = fmaxf(gm, __shfl_xor(gm, 32, 64));  // (finite: a block's first token is always valid)
+        if (__builtin_amdgcn_ballot_w64(gm > m_run) != 0) {  // some query's maximum grows: rescale (a factor of 1 otherwise)
+            const float m_new = fmaxf(m_run, gm);
+            const float alpha = exp2f(m_run - m_new);  // exp2(-inf) = 0 on the first block
+            m_run = m_new;
+            l_run *= alpha;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float a = __shfl(alpha, 4 * g4 + i, 64);  // o[.][i] is query 4 g4 + i
+#pragma unroll
+                for (int e = 0; e < NT; e++) o[e][i] *= a;
+            }
+        }
+        half4 ph, pl;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float pw = exp2f(sv[i] - m_run + 10.f);  // 2^10 p; 0 for a masked token
+            l_run += pw;
+            const HalfPair t = split_hl(pw);
+            ph[i] = t.h;
+            pl[i] = t.l;
+        }
+        if (!whole) {  // rows past the end may hold anything
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (tok0 + 4 * i >= t_end)
+#pragma unroll
+                    for (int e = 0; e < NT; e++) vv[i][e] = (_Float16)0.f;
+        }
+#pragma unroll
+        for (int e = 0; e < NT; e++) {
+            const half4 vb = {vv[0][e], vv[1][e], vv[2][e], vv[3][e]};
+            o[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(ph, vb, o[e], 0, 0, 0);
+            o[e] = __builtin_amdgcn_mfma_f32_16x16x16f16(pl, vb, o[e], 0, 0, 0);
         }
     }
-    // The last workgroup to arrive at a (sequence, chunk of 256 output columns) merges the chunk's splits in
-    // index order - the sums do not depend on who that is - and writes it as the next GEMM's operand.
-    if constexpr (MERGES) {
-        if (!mg.cnt) return;
-        // Ordering without device-wide cache write-backs and invalidations (a release / acquire fence pair at
-        // device scope costs this kernel several times its run time: every workgroup would flush and drop its
-        // die's L2): the partial sums above are device-scope stores and are read back by device-scope loads, which
-        // the dies' caches do not hold back or serve stale; each wave waits until its stores are acknowledged
-        // before the workgroup's barrier, thread 0 counts the arrival after the barrier, and whoever counts the
-        // last one reads only after that atomic has returned.
-        __shared__ int s_last;
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();
-        const int ns = (kv_len + tps - 1) / tps;  // workgroups of one kv head that arrive for this sequence
-        const int unit = kvh / HPC;
-        if (tid == 0) {
-            int32_t *cnt = mg.cnt + (size_t)seq * (num_kv_heads / HPC) + unit;
-            const int last = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == ns * HPC - 1;
-            if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // (nobody else comes before the next launch)
-            s_last = last;
-        }
-        __syncthreads();
-        if (!s_last) return;
-        for (int ch = wave; ch < CH; ch += 4) {
-            const int c = unit * CH + ch;
-            float y[4];
-            split_merge4<true>(partial, ns, num_q_heads, D, max_splits, seq, c * 256 + lane * 4, y);
-            put_merged(mg, seq, c, y, num_q_heads * D);
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+
+    __shared__ float s_m[4][GG], s_l[4][GG];
+    __shared__ float s_acc[4][GG][D];
+    if (g4 == 0 && c16 < GG) {
+        s_m[wave][c16] = m_run - 10.f;  // (the sums carry 2^10)
+        s_l[wave][c16] = l_run;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const int qr = 4 * g4 + i;
+        if (qr < GG) {
+#pragma unroll
+            for (int e = 0; e < NT; e++) s_acc[wave][qr][c16 * NT + e] = o[e][i];
         }
     }
+    finish_split<D, G, RG>(s_m, s_l, s_acc, partial, seq, kvh, split, kv_len, num_q_heads, num_kv_heads, max_splits, mg, tps);
 }
 
 // Copies per-sequence block tables given as device pointers into a padded [batch, max_blocks] matrix.
@@ -466,7 +704,7 @@ __global__ void __launch_bounds__(D) paged_merge_kernel(const float *__restrict_
 }
 
 // The rows of candidate trees: query row `row` of head qh has its context (pool positions < start, read by
-// paged_decode_f16_kernel<D, G, RG>) as split partials; this adds the tree's own keys, which sit at pool positions
+// paged_decode_gqa_kernel<D, G, RG>) as split partials; this adds the tree's own keys, which sit at pool positions
 // start .. start + n - 1 of the same sequence and are visible where the row's mask says so (medusa/tree.go:186-202),
 // and normalises. info[row] = (block-table row, start, row index inside its tree, rows of the tree);
 // grid = (num_q_heads, rows); block = D threads.
@@ -534,24 +772,6 @@ __global__ void __launch_bounds__(D) tree_merge_kernel(const float *__restrict__
 // crosses from the MFMA output layout to the operand layout through a wave-private LDS tile. LDS row pitches are
 // an odd number of 16-byte slots, so the 16 lanes of an operand read land in 16 different slots.
 constexpr int FA_BQ = 64, FA_BK = 32;
-
-// x = h + l in two f16 halves. The float32 value, its rounded half and their difference each pass through a register
-// of their own: left to itself the compiler folds the operations that produced x into mixed-precision
-// multiply-adds that round once from the unrounded product, and the halves then add up to less than x's 24 bits
-// (measured: attention outputs off by 3e-5 instead of 1e-6).
-struct HalfPair { _Float16 h, l; };
-__device__ __forceinline__ HalfPair split_hl(float x) {
-    asm volatile("" : "+v"(x));
-    HalfPair r;
-    r.h = (_Float16)x;
-    float hf = (float)r.h;
-    asm volatile("" : "+v"(hf));
-    float d = x - hf;
-    asm volatile("" : "+v"(d));
-    r.l = (_Float16)d;
-    return r;
-}
-typedef float float4v __attribute__((ext_vector_type(4)));
 
 template <int N>
 __device__ __forceinline__ float row16_max(float t) {  // max over the 16 lanes of a row; every lane gets it
@@ -795,6 +1015,9 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
         int n = 0;
         return (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, be->device) == hipSuccess && n > 0) ? n : 256;
     }();
+    // (grouped queries: fewer kv heads, so fewer workgroups per token, and the matrix-core form's per-block work is
+    // small: half the tokens per split measured faster at every batch tried)
+    if (G >= 2 && (D == 64 || D == 128)) tps = TPW / 2;
     while (tps > TPW / 4 && (size_t)batch * num_kv_heads * ceil_div(max_kv_len, tps) < (size_t)2 * cus) tps /= 2;
     int max_splits = ceil_div(max_kv_len, tps);
     const size_t partial_floats = ((size_t)batch * num_q_heads * max_splits * (D + 2) + 3) & ~(size_t)3;
@@ -843,10 +1066,23 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
                 return rc;
         }
     }
-    paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
-                                                                max_blocks, kv_lens, ws, num_q_heads,
-                                                                num_kv_heads, scale, max_splits,
-                                                                listed ? be->items.buf : nullptr, mg, tps);
+    // grouped queries on heads of 64 or 128: the matrix-core form (VEXEL_HIP_ATTN_VECTOR_FORM=1: the vector form, to compare)
+    static const bool vector_form = getenv("VEXEL_HIP_ATTN_VECTOR_FORM") != nullptr;
+    bool launched = false;
+    if constexpr (G >= 2 && (D == 64 || D == 128)) {  // (one query per K/V row: the vector form is the faster one, 110 against 119 us)
+        if (!vector_form) {
+            paged_decode_gqa_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
+                                                                        max_blocks, kv_lens, ws, num_q_heads,
+                                                                        num_kv_heads, scale, max_splits,
+                                                                        listed ? be->items.buf : nullptr, mg, tps);
+            launched = true;
+        }
+    }
+    if (!launched)
+        paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
+                                                                    max_blocks, kv_lens, ws, num_q_heads,
+                                                                    num_kv_heads, scale, max_splits,
+                                                                    listed ? be->items.buf : nullptr, mg, tps);
     VX_CHECK_LAUNCH();
     if (!fixed) be->split.batch = 0;  // (the fixed area is not where vx_decode_ffn looks for a split result)
     if (!out) {  // the caller merges: vx_decode_ffn(attn = NULL)
@@ -1232,7 +1468,7 @@ int vx_sdpa_paged_tree_batched(vx_backend *be, const float *q, const void *kv_po
     if (max_kv_len > 0) {
 #define VX_TREE(DD, GG, RR)                                                                                              \
     if (head_dim == DD && G == GG)                                                                                        \
-        paged_decode_f16_kernel<DD, GG, RR><<<grid, 256, 0, be->stream>>>(q, pool, block_tables, entry_table_rows, max_blocks, \
+        paged_decode_gqa_kernel<DD, GG, RR><<<grid, 256, 0, be->stream>>>(q, pool, block_tables, entry_table_rows, max_blocks, \
                                                                         entry_kv_lens, ws, num_q_heads, num_kv_heads, scale, \
                                                                         max_splits, nullptr, MergeOut{}, TPW);
         VX_TREE(128, 1, 8) VX_TREE(128, 2, 4) VX_TREE(128, 4, 2) VX_TREE(128, 8, 1)
