@@ -58,10 +58,11 @@ def load_synth():
     return s
 
 
-def build_model(be, ctx, extra_tokens, layers, cfg=None, fmts=None, max_batch=None, arch=None):
+def build_model(be, ctx, extra_tokens, layers, cfg=None, fmts=None, max_batch=None, arch=None, spare_tokens=0):
     """Synthetic model (7B-shaped Q4_0 unless cfg / fmts say otherwise) + pre-filled contexts, generated on the
     device. fmts: weight name (wq, wk, wv, wo, w1, w3, w2, head) -> VX_* format, "*" the default.
     arch: the switches of ModelRuntime.set_architecture plus "bias": "qkv" | "all" (small random bias vectors).
+    spare_tokens: free pool blocks (and a free sequence slot) for one more sequence of that many tokens.
     -> (ModelRuntime, ids)"""
     from vexel_amd import lib
     from vexel_amd.runtime import ModelRuntime
@@ -70,9 +71,9 @@ def build_model(be, ctx, extra_tokens, layers, cfg=None, fmts=None, max_batch=No
     c["num_layers"] = layers
     fmts = fmts or {"*": lib.VX_Q4_0, "head": lib.VX_Q8_0}
     fm = lambda name: fmts.get(name, fmts["*"])
-    need_blocks = sum((L + extra_tokens + BLOCK - 1) // BLOCK + 1 for L in ctx)
-    max_bps = (max(ctx) + extra_tokens + BLOCK - 1) // BLOCK + 1
-    mr = ModelRuntime(be, **c, pool_blocks=need_blocks, max_seqs=len(ctx), max_blocks_per_seq=max_bps,
+    need_blocks = sum((L + extra_tokens + BLOCK - 1) // BLOCK + 1 for L in list(ctx) + ([spare_tokens] if spare_tokens else []))
+    max_bps = (max(max(ctx), spare_tokens) + extra_tokens + BLOCK - 1) // BLOCK + 1
+    mr = ModelRuntime(be, **c, pool_blocks=need_blocks, max_seqs=len(ctx) + (1 if spare_tokens else 0), max_blocks_per_seq=max_bps,
                       max_batch=max_batch or len(ctx), kv_fp16=True)
     seed = [0]
     arch = dict(arch or {})
@@ -508,8 +509,8 @@ def configs_report(be):
                rope_theta=500000.0)
     q4km = {"*": lib.VX_Q4_K, "wv": lib.VX_Q6_K, "w2": lib.VX_Q6_K, "head": lib.VX_Q6_K}
 
-    def decode_rate(name, cfg, fmts, ctx, steps):
-        mr, ids = build_model(be, ctx, steps + 16, cfg["num_layers"], cfg, fmts)
+    def decode_rate(name, cfg, fmts, ctx, steps, spare_tokens=0):
+        mr, ids = build_model(be, ctx, steps + 16, cfg["num_layers"], cfg, fmts, spare_tokens=spare_tokens)
         first = np.random.default_rng(3).integers(0, cfg["vocab"], len(ctx)).astype(np.int32)
         mr.decode_graph(first, ids, ctx, 4, use_graph=True)
         be.sync()
@@ -531,9 +532,8 @@ def configs_report(be):
     mr.close()
     ctx4 = [int(x) for x in np.clip(np.exp(rng.normal(math.log(512.0), 0.6, 64)), 16, 4096)]
     mr, ids = decode_rate("config 4 (decode part): 8B-shaped Q8_0, 64 sequences (sum ctx %d)" % sum(ctx4), l8b,
-                          {"*": lib.VX_Q8_0}, ctx4 + [4200], 32)   # the 65th sequence only reserves blocks for the chunks
+                          {"*": lib.VX_Q8_0}, ctx4, 32, spare_tokens=4200)   # (free blocks for the chunks below)
     chunk = rng.integers(0, l8b["vocab"], 512).tolist()
-    mr.delete_sequence(ids[-1])
     mr.prefill_with_paged_kv(chunk[:64], 1000, 0)           # sizes the workspaces
     mr.delete_sequence(1000)
     be.sync()

@@ -1736,14 +1736,18 @@ struct WavePlan {
     int ks;  // K slices
 };
 
-// Depends on the format and the matrix only, never on M, so that a row's bits do not depend on the batch it sits
-// in. One workgroup per compute unit: the plan with the shortest modelled time among those whose workgroups all
+// Depends on the format, the matrix and on whether M is above 32 only, so that a row's bits do not depend on the
+// batch it sits in within 2 .. 32 and within 33 .. 64 rows. One workgroup per compute unit: the plan with the shortest modelled time among those whose workgroups all
 // run at once. VEXEL_HIP_WPLAN="NxK:R,KS;..." overrides (tuning).
-// (up to 32 activation rows: with more, every further 32 rows would stage and unpack the weights again from
+// (up to 64 activation rows: with more, every further group of rows would stage and unpack the weights again from
 // eight waves' separate slices, and qgemm_kernel's shared staging is quicker)
 WavePlan wave_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K, int M) {
     WavePlan none = {0, 1};
-    if (M > 32 && fmt != VX_BF16) return none;  // (BF16 has no other matrix-core kernel: it takes the groups of 32 rows)
+    // 33 .. 64 rows: four activation tiles a step, whose sums and operand ring leave room for 3 weight tiles a
+    // workgroup; tall matrices then take several rounds of workgroups (measured at 64 rows against qgemm_kernel:
+    // 0.79 of its time for Q4_0, 0.87 for Q8_0, 0.75 for Q4_K over the four projections of a 7B / 8B layer)
+    const bool rows64 = M > 32 && M <= 64 && fmt != VX_BF16;
+    if (M > 32 && fmt != VX_BF16 && !rows64) return none;  // (BF16 has no other matrix-core kernel: it takes the groups of 32 rows)
     static const char *off = getenv("VEXEL_HIP_WAVE_OFF");
     if (off && atoi(off)) return none;
     if (fmt != VX_Q4_0 && fmt != VX_Q8_0 && fmt != VX_Q4_K && fmt != VX_BF16) return none;
@@ -1766,8 +1770,9 @@ WavePlan wave_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K, int 
         }
     }
     // more than 6 tiles a workgroup would spill registers: taller matrices (output heads) stay on qgemm_kernel
-    const int max_r = fmt == VX_Q8_0 ? 4 : (fmt == VX_BF16 ? 2 : 6);  // (wider staging leaves room for fewer tiles)
-    if (tiles > max_r * cus && fmt != VX_BF16) return none;
+    const int max_r = rows64 ? 3 : (fmt == VX_Q8_0 ? 4 : (fmt == VX_BF16 ? 2 : 6));  // (wider staging leaves room for fewer tiles)
+    const bool rounds = fmt == VX_BF16 || rows64;
+    if (tiles > max_r * cus && !rounds) return none;
     static const int rs[] = {1, 2, 3, 4, 6};
     WavePlan best = none;
     float best_cost = 0.f;
@@ -1775,7 +1780,7 @@ WavePlan wave_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K, int 
         if (!fits(r) || r > max_r) continue;
         const int rg = ceil_div(tiles, r);
         for (int ks = 1; ks <= std::min(n_chunks, 8); ks++) {
-            if (rg * ks > cus && !(fmt == VX_BF16 && ks == 1 && r == max_r)) continue;  // (a tall BF16 matrix: several rounds of workgroups)
+            if (rg * ks > cus && !(rounds && ks == 1 && r == max_r)) continue;  // (a tall BF16 matrix: several rounds of workgroups)
             const int wg_chunks = ceil_div(n_chunks, ks), wave_chunks = ceil_div(wg_chunks, 8);
             // In cycles, fitted to the 7B shapes at 32 rows: a wave's tile steps share a SIMD with one other
             // wave's (about 220 cycles a tile step for the pair); a compute unit pulls the 32 KB of activation
@@ -1794,13 +1799,18 @@ WavePlan wave_plan(vx_backend *be, int fmt, const Segs &segs, int N, int K, int 
     return best;
 }
 
+constexpr int WAVE_MT4_MAX_R = 3;  // weight tiles per workgroup up to which 64 activation rows' sums fit the registers
+
 template <class W, int R>
 int launch_gemm_wave(vx_backend *be, const Segs &segs, int N, float *out, const float *residual, bool to_partials, int M,
                      int K, int ks, int *ks_out, const QkvEpi &epi) {
     constexpr int NW = 8;
     const int mpad = mpad_for(M);
     const PrepView pv = prep_view(be, mpad, K);
-    const int rg = ceil_div(N, 16 * R), mgroups = mpad <= 16 ? 1 : mpad / 32;
+    // activation rows per workgroup: 16, 32 or (33 .. 64 rows, where the tiles fit the registers) 64; beyond, groups of 32
+    constexpr bool MT4 = R <= (W::PITCH >= 256 ? 1 : WAVE_MT4_MAX_R);
+    const bool four = MT4 && mpad == 64;
+    const int rg = ceil_div(N, 16 * R), mgroups = mpad <= 16 || four ? 1 : mpad / 32;
     float *partial = nullptr;
     if (ks > 1 || to_partials) {
         int rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, (size_t)ks * M * N * sizeof(float), "split-K partial sums");
@@ -1812,8 +1822,10 @@ int launch_gemm_wave(vx_backend *be, const Segs &segs, int N, float *out, const 
     const int n_chunks = K / 256, slices = ((n_chunks / ks) << 16) | (n_chunks % ks);  // the kernel takes the division done
     if (mpad <= 16)
         qgemm_wave_kernel<W, R, 1, NW><<<grid, 64 * NW, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slices, vec ? 1 : 0, epi);
-    else
+    else if (!four)
         qgemm_wave_kernel<W, R, 2, NW><<<grid, 64 * NW, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slices, vec ? 1 : 0, epi);
+    else if constexpr (MT4)
+        qgemm_wave_kernel<W, R, 4, NW><<<grid, 64 * NW, 0, be->stream>>>(segs, pv, out, residual, partial, M, mpad, N, K, slices, vec ? 1 : 0, epi);
     VX_CHECK_LAUNCH();
     if (ks_out) *ks_out = ks;
     if (partial && !to_partials) {

@@ -182,7 +182,7 @@ __global__ void __launch_bounds__(64 * NW, 1) qgemm_wave_kernel(Segs segs, PrepV
     constexpr int ROWS = G::ROWS;
     // steps an activation load runs ahead of its use: a step of few tiles is short, so its operand must be
     // requested more steps ahead to cover the same latency (the ring's size divides the eight steps of a chunk)
-    constexpr int AD = R * MT <= 4 ? 7 : 3;
+    constexpr int AD = MT >= 4 ? 1 : (R * MT <= 4 ? 7 : 3);  // (four tiles a step: two ring slots are 64 registers)
     constexpr int NG = (ROWS + W::GROWS - 1) / W::GROWS;  // load groups per stage
     constexpr int LAST_ROWS = ROWS - (NG - 1) * W::GROWS;
     constexpr int REGION = G::REGION;
