@@ -317,8 +317,9 @@ int vx_sdpa_paged_tree(vx_backend *be, const float *q, const void *kv_pool, int 
                        int query_len);
 
 /* Tree verification for many sequences in two launches. The query rows come in entries of
- * vx_sdpa_paged_tree_rows_per_entry() consecutive rows (0: this geometry has no batched form); the rows of an
- * entry belong to one tree, whose sequence is block-table row entry_table_rows[e] with entry_kv_lens[e] tokens
+ * vx_sdpa_paged_tree_rows_per_entry() consecutive rows (16 / G for G query heads per KV head; 0: this geometry
+ * has no batched form) or, where that number is even, of half as many (rows / entries says which: fewer rows of
+ * padding for small trees, the context read twice as often); the rows of an entry belong to one tree, whose sequence is block-table row entry_table_rows[e] with entry_kv_lens[e] tokens
  * before the tree. A tree's own keys sit at pool positions kv_len .. kv_len + n - 1 of its sequence (stored
  * before the call). row_info: int32[rows][4] = (block-table row, kv_len, row index inside its tree, rows n of the
  * tree); row i of a tree sees key j where tree_masks[mask_offsets[row] + i*n + j] != 0 (medusa/tree.go:186-202).

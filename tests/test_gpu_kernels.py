@@ -983,15 +983,21 @@ def test_paged_multiquery_tiled(be, hq, hk, d, qn, start):
     be.reset_pool()
 
 
-@pytest.mark.parametrize("hq,hk,d", [(8, 8, 128), (8, 2, 64), (16, 2, 128)])
-def test_paged_tree_batched(be, hq, hk, d):
+@pytest.mark.parametrize("hq,hk,d,half", [(8, 8, 128, False), (8, 8, 128, True), (8, 2, 64, False), (8, 2, 64, True),
+                                          (16, 2, 128, False), (16, 2, 128, True), (6, 2, 128, False), (10, 2, 64, False),
+                                          (14, 2, 128, True)])
+def test_paged_tree_batched(be, hq, hk, d, half):
     """Every tree of a batch in two launches: against the oracle's masked multi-query attention per sequence and,
     to rounding, the per-sequence entry point. Ragged contexts (one empty, one a multiple of the 512-token split),
-    trees of different sizes, entries padded with repeated rows."""
+    trees of different sizes, entries padded with repeated rows; entries of 16 / G rows and, where that is even, of
+    half as many."""
     rng = np.random.default_rng(37)
     bs, nblocks = 16, 160
     rg = be._lib.vx_sdpa_paged_tree_rows_per_entry(1, bs, hq, hk, d)
-    assert rg == 8 // (hq // hk)
+    assert rg == 16 // (hq // hk)
+    if half:
+        assert rg % 2 == 0
+        rg //= 2
     pool = _make_pool(rng, True, nblocks, bs, hk, d)
     dpool = be.upload(pool)
     starts = [0, 37, 512, 700]

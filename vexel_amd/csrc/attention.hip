@@ -1433,7 +1433,7 @@ int vx_sdpa_paged_tree_rows_per_entry(int pool_is_f16, int block_size, int num_q
     if (!pool_is_f16 || block_size != HOT_BS || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0) return 0;
     if (head_dim != 128 && head_dim != 64) return 0;
     const int G = num_q_heads / num_kv_heads;
-    return (G == 1 || G == 2 || G == 4 || G == 8) ? 8 / G : 0;
+    return G <= 8 ? 16 / G : 0;  // 16 queries (row, head) per K/V row fill the matrix-core tile: 16, 8, 5, 4, 3, 2, 2, 2 rows
 }
 
 int vx_sdpa_paged_tree_batched(vx_backend *be, const float *q, const void *kv_pool, const int32_t *block_tables,
@@ -1445,13 +1445,16 @@ int vx_sdpa_paged_tree_batched(vx_backend *be, const float *q, const void *kv_po
     if (rc) return rc;
     VX_REQUIRE(q && kv_pool && block_tables && entry_table_rows && entry_kv_lens && row_info && tree_masks && mask_offsets && out,
                "vx_sdpa_paged_tree_batched: null pointer");
-    const int rg = vx_sdpa_paged_tree_rows_per_entry(1, HOT_BS, num_q_heads, num_kv_heads, head_dim);
-    if (rg == 0) {
+    const int rg_max = vx_sdpa_paged_tree_rows_per_entry(1, HOT_BS, num_q_heads, num_kv_heads, head_dim);
+    if (rg_max == 0) {
         set_error("vx_sdpa_paged_tree_batched: head geometry %d/%d x %d has no batched form", num_q_heads, num_kv_heads, head_dim);
         return VX_ERR_UNSUPPORTED;
     }
-    VX_REQUIRE(entries >= 0 && rows == entries * rg, "vx_sdpa_paged_tree_batched: %d rows are not %d entries of %d rows", rows,
-               entries, rg);
+    // entries of rg_max rows, or - for small trees, which would mostly pad them - of half as many where that is whole
+    const int rg = entries > 0 ? rows / entries : rg_max;
+    VX_REQUIRE(entries >= 0 && rows == entries * rg && (rg == rg_max || (rg_max % 2 == 0 && rg == rg_max / 2)),
+               "vx_sdpa_paged_tree_batched: %d rows are not %d entries of %d rows%s", rows, entries, rg_max,
+               rg_max % 2 == 0 ? " or of half as many" : "");
     VX_REQUIRE(max_tree_rows >= 1 && max_tree_rows <= 64 && max_tree_rows <= head_dim,
                "vx_sdpa_paged_tree_batched: a tree of %d rows (at most 64)", max_tree_rows);
     VX_REQUIRE(((uintptr_t)kv_pool % 16) == 0 && max_kv_len >= 0, "vx_sdpa_paged_tree_batched: bad pool alignment / length");
@@ -1467,12 +1470,16 @@ int vx_sdpa_paged_tree_batched(vx_backend *be, const float *q, const void *kv_po
     const dim3 grid(num_kv_heads, max_splits, entries);
     if (max_kv_len > 0) {
 #define VX_TREE(DD, GG, RR)                                                                                              \
-    if (head_dim == DD && G == GG)                                                                                        \
+    if (head_dim == DD && G == GG && rg == RR)                                                                            \
         paged_decode_gqa_kernel<DD, GG, RR><<<grid, 256, 0, be->stream>>>(q, pool, block_tables, entry_table_rows, max_blocks, \
                                                                         entry_kv_lens, ws, num_q_heads, num_kv_heads, scale, \
                                                                         max_splits, nullptr, MergeOut{}, TPW);
-        VX_TREE(128, 1, 8) VX_TREE(128, 2, 4) VX_TREE(128, 4, 2) VX_TREE(128, 8, 1)
-        VX_TREE(64, 1, 8) VX_TREE(64, 2, 4) VX_TREE(64, 4, 2) VX_TREE(64, 8, 1)
+#define VX_TREES(DD)                                                                                                       \
+    VX_TREE(DD, 1, 16) VX_TREE(DD, 1, 8) VX_TREE(DD, 2, 8) VX_TREE(DD, 2, 4) VX_TREE(DD, 3, 5) VX_TREE(DD, 4, 4)         \
+    VX_TREE(DD, 4, 2) VX_TREE(DD, 5, 3) VX_TREE(DD, 6, 2) VX_TREE(DD, 6, 1) VX_TREE(DD, 7, 2) VX_TREE(DD, 7, 1)           \
+    VX_TREE(DD, 8, 2) VX_TREE(DD, 8, 1)
+        VX_TREES(128) VX_TREES(64)
+#undef VX_TREES
 #undef VX_TREE
         VX_CHECK_LAUNCH();
     }

@@ -1046,7 +1046,16 @@ int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_
     // last entry repeat the sequence's last row (same token, position and pool slot), their results are dropped.
     static const bool per_sequence = getenv("VEXEL_HIP_TREE_PER_SEQUENCE") != nullptr;
     const int rg0 = vx_sdpa_paged_tree_rows_per_entry(c.kv_fp16, c.block_size, c.num_heads, c.num_kv_heads, c.head_dim);
-    const int rg = (rg0 > 0 && max_rows <= 64 && max_rows <= c.head_dim && !per_sequence) ? rg0 : 0;
+    int rg = (rg0 > 0 && max_rows <= 64 && max_rows <= c.head_dim && !per_sequence) ? rg0 : 0;
+    if (rg && rg % 2 == 0) {  // entries of half as many rows where the full ones would add rows of padding (small trees)
+        int full = 0, half = 0;
+        for (int i = 0; i < n_seqs; i++) {
+            const int rows = 1 + n_nodes[i];
+            full += (rows + rg - 1) / rg * rg;
+            half += (rows + rg / 2 - 1) / (rg / 2) * (rg / 2);
+        }
+        if (half < full) rg /= 2;
+    }
     for (int i = 0; i < n_seqs; i++) {
         const int rows = 1 + n_nodes[i], pad = rg ? (rows + rg - 1) / rg * rg : rows;
         sr[i] = {total, rows, nodes_total, start_pos[i], -1, pad};
