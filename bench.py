@@ -352,7 +352,7 @@ def kernel_report(be):
     names = {1: "Q4_0", 2: "Q8_0", 3: "Q4_K", 4: "Q6_K", 5: "Q5_0", 6: "Q5_K"}
     shapes = [("Q|K|V", 12288, 4096), ("Wo", 4096, 4096), ("gate|up", 22016, 4096), ("down", 4096, 11008),
               ("lm_head", 32000, 4096)]
-    a = np.random.default_rng(0).standard_normal((32, 11008)).astype(np.float32)
+    a = np.random.default_rng(0).standard_normal((64, 11008)).astype(np.float32)
     da = be.upload(a, permanent=True)
     print("%-8s %-5s %3s %6s %6s %9s %9s %7s" % ("matmul", "fmt", "M", "N", "K", "us/call", "GB/s", "of 8TB"))
     for fmt in (1, 2, 3, 4, 5, 6):
@@ -377,7 +377,7 @@ def kernel_report(be):
                 if rc:
                     raise RuntimeError("synthetic weight generation failed: %d" % rc)
                 ws.append(p)
-            for m in (1, 32):
+            for m in (1, 32, 64):
                 out = be.alloc_permanent(m * n * 4)
                 be.prepare_act(da, m, k)
                 for w in ws[:2]:
@@ -415,6 +415,34 @@ def kernel_report(be):
     print("paged decode attention, 32 ragged sequences (sum ctx %d), one layer: %.1f us, %.0f GB/s, %.3f of 8 TB/s"
           % (sum(ctx), ms * 1e3, nb / ms / 1e6, nb / ms / 1e6 / HBM_PEAK_GBS))
     mr.close()
+    # grouped-query geometries (the matrix-core form of the kernel), result left merged for the output projection
+    for hq, hk, nseq, med in ((32, 8, 64, 512), (32, 8, 32, 1024), (28, 4, 32, 1024)):
+        rng = np.random.default_rng(0)
+        d = 128
+        lens = np.clip(np.exp(rng.normal(math.log(med), 0.6, nseq)), 16, 4096).astype(np.int32)
+        nblk = [(int(L) + BLOCK - 1) // BLOCK for L in lens]
+        perm = rng.permutation(sum(nblk)).astype(np.int32)
+        tables = np.zeros((nseq, 256), dtype=np.int32)
+        off = 0
+        for i in range(nseq):
+            tables[i, :nblk[i]] = perm[off:off + nblk[i]]
+            off += nblk[i]
+        pool = be.alloc_permanent(sum(nblk) * 2 * BLOCK * hk * d * 2)
+        dq = be.upload(rng.standard_normal((nseq, hq * d)).astype(np.float32), permanent=True)
+        dt, dl = be.upload(tables, permanent=True), be.upload(lens, permanent=True)
+        args = (dq, pool, True, dt, dl, None, nseq, 256, BLOCK, hq, hk, d, 1.0 / math.sqrt(d), 4096)
+        for _ in range(3):
+            be.sdpa_paged_decode_ragged(*args)
+        be.sync()
+        be.timer_start()
+        for _ in range(40):
+            be.sdpa_paged_decode_ragged(*args)
+        us = be.timer_stop_ms() * 1e3 / 40
+        nb = sum(2 * int(L) * hk * d * 2 + nblk[i] * 4 for i, L in enumerate(lens)) + 2 * nseq * hq * d * 4
+        print("paged decode attention, %d / %d heads x %d, %d ragged sequences (sum ctx %d), one layer: %.1f us, %.0f GB/s, "
+              "%.3f of 8 TB/s" % (hq, hk, d, nseq, int(lens.sum()), us, nb / us / 1e3, nb / us / 1e3 / HBM_PEAK_GBS))
+        for p_ in (pool, dq, dt, dl):
+            be.free(p_)
     # dense causal prefill attention of one 512-token chunk, 7B head geometry (f16 matrix cores, operands as hi + lo halves)
     S, hq, d = 512, c["num_heads"], c["head_dim"]
     rng = np.random.default_rng(5)
