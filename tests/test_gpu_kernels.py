@@ -948,14 +948,16 @@ def test_paged_multiquery_and_tree(be):
         be.reset_pool()
 
 
-@pytest.mark.parametrize("hq,hk,d,qn,start", [(8, 2, 128, 200, 137), (8, 8, 64, 70, 0), (4, 1, 128, 16, 500),
-                                              (32, 8, 128, 65, 40)])
-def test_paged_multiquery_tiled(be, hq, hk, d, qn, start):
-    """SDPAPagedDecodeMultiquery on the tiled kernel (F16 pool, 16 or more query rows): the later chunk of a prompt
-    (row i sees start + i + 1 keys, runtime/block.go:884-887), with the chunk's rows crossing 64-row tile and 32-key
-    tile boundaries, against the oracle's per-row attention."""
+@pytest.mark.parametrize("hq,hk,d,qn,start,bs", [(8, 2, 128, 200, 137, 16), (8, 8, 64, 70, 0, 16), (4, 1, 128, 16, 500, 16),
+                                                 (32, 8, 128, 65, 40, 16), (28, 4, 128, 50, 77, 16), (4, 4, 128, 100, 300, 16),
+                                                 (8, 2, 128, 200, 137, 32), (8, 8, 64, 70, 0, 8)])
+def test_paged_multiquery_tiled(be, hq, hk, d, qn, start, bs):
+    """SDPAPagedDecodeMultiquery on the matrix-core kernels (F16 pool, 16 or more query rows): the later chunk of a
+    prompt (row i sees start + i + 1 keys, runtime/block.go:884-887), with the chunk's rows crossing tile boundaries,
+    against the oracle's per-row attention. 16-token blocks: the kernel that walks the blocks per wave; other block
+    sizes: the one that stages 32-key tiles in LDS."""
     rng = np.random.default_rng(340 + qn)
-    bs, nblocks = 16, 60
+    nblocks = 960 // bs
     pool = _make_pool(rng, True, nblocks, bs, hk, d)
     dpool = be.upload(pool)
     bt = rng.permutation(nblocks)[:(start + qn + bs - 1) // bs + 1].astype(np.int32)

@@ -13,8 +13,11 @@
 //    output projection the kernel merges its own splits (the last workgroup of a chunk does it).
 //  * paged_decode_gqa_kernel: the same for grouped queries (2 to 16 queries per K/V row, heads of 64 or
 //    128) and for the batched tree attention's entries, on the f16 matrix cores; same splits, same merge.
-//  * prefill_fa2_kernel: tiled causal prefill and paged multi-query attention on the f16
-//    matrix cores (operands as two f16 halves).
+//  * paged_mq_kernel: many query rows of one sequence over its paged F16 context (later prompt
+//    chunks, linear verification), the grouped-query kernel's products with a tile of query rows
+//    per wave; no LDS.
+//  * prefill_fa2_kernel: tiled causal prefill (dense float32 K/V) and paged multi-query attention
+//    for other block sizes on the f16 matrix cores (operands as two f16 halves), K/V tiles in LDS.
 //
 // Arithmetic: float32 dot products and accumulation (the matrix-core kernels: f16 products of
 // two-halves operands, float32 accumulation), softmax through exp2 of the max-subtracted score; the CPU reference (backend/cpu/cpu.go:568-632) normalises the
@@ -671,6 +674,185 @@ __global__ void __launch_bounds__(256, 3) paged_decode_gqa_kernel(
         }
     }
     finish_split<D, G, RG>(s_m, s_l, s_acc, partial, seq, kvh, split, kv_len, num_q_heads, num_kv_heads, max_splits, mg, tps);
+}
+
+// Many query rows of one sequence over its paged F16 context, each row with its own number of visible keys (the
+// later chunks of a prompt, linear verification): paged_decode_gqa_kernel's two matrix-core products and operand
+// layouts, with QT tiles of 16 consecutive query rows of one head per wave instead of 16 (row, head) queries of one
+// KV head, the per-row limits as the mask, no split of the keys and no LDS: a wave walks the 16-token blocks up
+// to the longest of its rows' limits and writes its rows' outputs itself. The four waves of a workgroup take
+// combinations (head of the KV head's group, row group) next to each other - the same rows for up to four heads
+// that share the K/V rows, or neighbouring row groups - so that their loads of a block meet in the cache.
+// grid = (ceil(G * row groups / 4), num_kv_heads); block = 256.
+template <int D, int QT>
+__global__ void __launch_bounds__(256, 2) paged_mq_kernel(const float *__restrict__ q, const _Float16 *__restrict__ pool,
+                                                         const int32_t *__restrict__ table, const int32_t *__restrict__ kv_lens,
+                                                         float *__restrict__ out, int query_len, int max_keys, int num_q_heads,
+                                                         int num_kv_heads, float scale) {
+    constexpr int NS = D / 32, NT = D / 16;
+    typedef _Float16 halfv __attribute__((ext_vector_type(NT)));
+    typedef _Float16 half4 __attribute__((ext_vector_type(4)));
+    const int kvh = blockIdx.y, G = num_q_heads / num_kv_heads;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int combo = blockIdx.x * 4 + wave, row_groups = (query_len + 16 * QT - 1) / (16 * QT);
+    if (combo >= G * row_groups) return;  // (no barrier in this kernel: a wave without work leaves)
+    const int head = kvh * G + combo % G, r0 = (combo / G) * 16 * QT;
+    const int c16 = lane & 15, g4 = lane >> 4;
+    const size_t hs = (size_t)num_kv_heads * D, part = (size_t)HOT_BS * hs, qs = (size_t)num_q_heads * D;
+
+    half8 qh[QT][NS], ql[QT][NS];
+    float q_inv[QT];
+    int lim[QT];  // query row r0 + 16 t + c16 sees the keys 0 .. lim[t] - 1
+    int len_max = 0, len_min = max_keys;
+#pragma unroll
+    for (int t = 0; t < QT; t++) {
+        const int qi = r0 + 16 * t + c16;
+        lim[t] = qi < query_len ? min(max(kv_lens[qi], 0), max_keys) : 0;
+        len_max = max(len_max, lim[t]);
+        if (qi < query_len) len_min = min(len_min, lim[t]);
+        float x[NS][8];
+        float amax = 0.f;
+        const float f0 = scale * kLog2e;
+        const float *qp = q + (size_t)min(qi, query_len - 1) * qs + (size_t)head * D + g4 * (D / 4);
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const float4 a = *(const float4 *)(qp + 8 * s), b = *(const float4 *)(qp + 8 * s + 4);
+            const float v[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                x[s][e] = v[e] * f0;
+                amax = fmaxf(amax, fabsf(x[s][e]));
+            }
+        }
+        amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+        amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+        int ex = 11;
+        if (amax > 0.f && amax < INFINITY) {
+            (void)frexpf(amax, &ex);
+            ex = max(ex, -60);
+        }
+        const float f = ldexpf(1.f, 11 - ex);
+        q_inv[t] = ldexpf(1.f, ex - 11);
+#pragma unroll
+        for (int s = 0; s < NS; s++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const HalfPair hl = split_hl(x[s][e] * f);
+                qh[t][s][e] = hl.h;
+                ql[t][s][e] = hl.l;
+            }
+    }
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {  // over the wave's rows
+        len_max = max(len_max, __shfl_xor(len_max, off, 64));
+        len_min = min(len_min, __shfl_xor(len_min, off, 64));
+    }
+    float4v o[QT][NT];
+    float m_run[QT], l_run[QT];
+#pragma unroll
+    for (int t = 0; t < QT; t++) {
+        m_run[t] = -INFINITY;
+        l_run[t] = 0.f;
+#pragma unroll
+        for (int e = 0; e < NT; e++) o[t][e] = (float4v){0.f, 0.f, 0.f, 0.f};
+    }
+    const int n_blocks = (len_max + HOT_BS - 1) / HOT_BS;
+    const size_t k_off = (size_t)(4 * (c16 & 3) + (c16 >> 2)) * hs + (size_t)kvh * D + g4 * (D / 4);
+    const size_t v_off = part + (size_t)g4 * hs + (size_t)kvh * D + c16 * NT;
+    half8 kk[NS], kn[NS];
+    halfv vv[4], vn[4];
+    auto issue = [&](int bi, half8 *kd, halfv *vd) {
+        const int blk = __builtin_amdgcn_readfirstlane(table[bi]);
+        const _Float16 *base = pool + (size_t)blk * 2 * part;
+#pragma unroll
+        for (int s = 0; s < NS; s++) kd[s] = *(const half8 *)(base + k_off + 8 * s);
+#pragma unroll
+        for (int i = 0; i < 4; i++) vd[i] = *(const halfv *)(base + v_off + (size_t)i * 4 * hs);
+    };
+    if (n_blocks > 0) issue(0, kn, vn);
+    for (int bi = 0; bi < n_blocks; bi++) {
+#pragma unroll
+        for (int s = 0; s < NS; s++) kk[s] = kn[s];
+#pragma unroll
+        for (int i = 0; i < 4; i++) vv[i] = vn[i];
+        if (bi + 1 < n_blocks) issue(bi + 1, kn, vn);
+        __builtin_amdgcn_sched_barrier(0);
+        const int tok0 = bi * HOT_BS + g4;                       // score i of a tile: token tok0 + 4i
+        const bool open = (bi + 1) * HOT_BS <= len_min;          // every row of the wave sees the whole block
+        if ((bi + 1) * HOT_BS > len_max) {                       // rows past the sequence's end may hold anything
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (tok0 + 4 * i >= len_max)
+#pragma unroll
+                    for (int e = 0; e < NT; e++) vv[i][e] = (_Float16)0.f;
+        }
+#pragma unroll
+        for (int t = 0; t < QT; t++) {
+            float4v sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk[s], qh[t][s], sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_16x16x32_f16(kk[s], ql[t][s], sc, 0, 0, 0);
+            }
+            float sv[4], gm = -INFINITY;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                sv[i] = (open || tok0 + 4 * i < lim[t]) ? sc[i] * q_inv[t] : -INFINITY;
+                gm = fmaxf(gm, sv[i]);
+            }
+            gm = fmaxf(gm, __shfl_xor(gm, 16, 64));
+            gm = fmaxf(gm, __shfl_xor(gm, 32, 64));
+            if (__builtin_amdgcn_ballot_w64(gm > m_run[t]) != 0) {
+                const float m_new = fmaxf(m_run[t], gm);
+                const float alpha = exp2f(m_run[t] - m_new);  // (m_new is finite in every lane that gets here with gm > m_run; 1 elsewhere)
+                const float a_own = gm > m_run[t] ? alpha : 1.f;
+                m_run[t] = m_new;
+                l_run[t] *= a_own;
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const float a = __shfl(a_own, 4 * g4 + i, 64);
+#pragma unroll
+                    for (int e = 0; e < NT; e++) o[t][e][i] *= a;
+                }
+            }
+            const float m_use = m_run[t] == -INFINITY ? 0.f : m_run[t];  // (a row that has seen no key yet: every weight 0)
+            half4 ph, pl;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float pw = exp2f(sv[i] - m_use + 10.f);
+                l_run[t] += pw;
+                const HalfPair hl = split_hl(pw);
+                ph[i] = hl.h;
+                pl[i] = hl.l;
+            }
+#pragma unroll
+            for (int e = 0; e < NT; e++) {
+                const half4 vb = {vv[0][e], vv[1][e], vv[2][e], vv[3][e]};
+                o[t][e] = __builtin_amdgcn_mfma_f32_16x16x16f16(ph, vb, o[t][e], 0, 0, 0);
+                o[t][e] = __builtin_amdgcn_mfma_f32_16x16x16f16(pl, vb, o[t][e], 0, 0, 0);
+            }
+        }
+    }
+    // lane (c16, g4) holds O[row 4 g4 + i][columns c16 * NT .. + NT - 1] of every tile; the row's sum of weights is
+    // spread over the four lanes (row, 0..3)
+#pragma unroll
+    for (int t = 0; t < QT; t++) {
+        float l = l_run[t];
+        l += __shfl_xor(l, 16, 64);
+        l += __shfl_xor(l, 32, 64);
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const float w = __shfl(inv, 4 * g4 + i, 64);
+            const int qi = r0 + 16 * t + 4 * g4 + i;
+            if (qi >= query_len) continue;
+            float *op = out + (size_t)qi * qs + (size_t)head * D + c16 * NT;
+#pragma unroll
+            for (int e = 0; e < NT; e += 4)
+                *(float4 *)(op + e) = make_float4(o[t][e][i] * w, o[t][e + 1][i] * w, o[t][e + 2][i] * w, o[t][e + 3][i] * w);
+        }
+    }
 }
 
 // Copies per-sequence block tables given as device pointers into a padded [batch, max_blocks] matrix.
@@ -1373,9 +1555,24 @@ int vx_sdpa_paged_decode_multiquery(vx_backend *be, const float *q, const void *
     VX_REQUIRE(q && kv_pool && block_table && out && kv_lens, "vx_sdpa_paged_decode_multiquery: null pointer");
     VX_REQUIRE(num_blocks >= 1 && block_size >= 1 && query_len >= 0, "vx_sdpa_paged_decode_multiquery: bad counts");
     VX_REQUIRE(head_dim > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0, "vx_sdpa_paged_decode_multiquery: bad head counts");
-    // Chunks of a prompt and verification rows over an F16 pool: the tiled kernel (K/V tiles of 32 keys staged in
-    // LDS for 64 queries, float32 matrix cores). A handful of rows, other head sizes and float32 pools keep the
-    // one-workgroup-per-query kernel.
+    // Chunks of a prompt and verification rows over an F16 pool: the matrix-core kernels (16-token blocks: a tile of
+    // 16 query rows per wave straight from the pool; other block sizes: K/V tiles of 32 keys staged in LDS for 64
+    // queries). A handful of rows, other head sizes and float32 pools keep the one-workgroup-per-query kernel.
+    static const bool lds_tiles = getenv("VEXEL_HIP_MQ_LDS_TILES") != nullptr;  // (the LDS-tiled kernel instead, to compare)
+    if (pool_is_f16 && query_len >= 16 && (head_dim == 64 || head_dim == 128) && ((uintptr_t)kv_pool % 16) == 0 &&
+        block_size == HOT_BS && ((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 16) == 0 && !lds_tiles) {
+        constexpr int QT = 1;
+        const int G = num_q_heads / num_kv_heads, combos = G * ceil_div(query_len, 16 * QT);
+        const dim3 grid(ceil_div(combos, 4), num_kv_heads);
+        if (head_dim == 128)
+            paged_mq_kernel<128, QT><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)kv_pool, block_table, kv_lens, out, query_len,
+                                                                   num_blocks * block_size, num_q_heads, num_kv_heads, scale);
+        else
+            paged_mq_kernel<64, QT><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)kv_pool, block_table, kv_lens, out, query_len,
+                                                                  num_blocks * block_size, num_q_heads, num_kv_heads, scale);
+        VX_CHECK_LAUNCH();
+        return VX_OK;
+    }
     if (pool_is_f16 && query_len >= 16 && (head_dim == 64 || head_dim == 128) && ((uintptr_t)kv_pool % 8) == 0) {
         PagedSrc src = {(const _Float16 *)kv_pool, block_table, kv_lens, block_size};
         dim3 grid(ceil_div(query_len, FA_BQ), num_q_heads);
