@@ -679,13 +679,14 @@ __global__ void __launch_bounds__(256, 3) paged_decode_gqa_kernel(
 // Many query rows of one sequence over its paged F16 context, each row with its own number of visible keys (the
 // later chunks of a prompt, linear verification): paged_decode_gqa_kernel's two matrix-core products and operand
 // layouts, with QT tiles of 16 consecutive query rows of one head per wave instead of 16 (row, head) queries of one
-// KV head, the per-row limits as the mask, no split of the keys and no LDS: a wave walks the 16-token blocks up
-// to the longest of its rows' limits and writes its rows' outputs itself. The four waves of a workgroup take
-// combinations (head of the KV head's group, row group) next to each other - the same rows for up to four heads
-// that share the K/V rows, or neighbouring row groups - so that their loads of a block meet in the cache.
-// grid = (ceil(G * row groups / 4), num_kv_heads); block = 256.
-template <int D, int QT>
-__global__ void __launch_bounds__(256, 2) paged_mq_kernel(const float *__restrict__ q, const _Float16 *__restrict__ pool,
+// KV head and the per-row limits as the mask. A workgroup holds NSUB (head of the KV head's group, row tile) pairs
+// next to each other - the same rows for the heads that share the K/V rows, or neighbouring row tiles - times KS
+// shares of the blocks (block b belongs to share b % KS). The NSUB waves of a share bring each block into LDS
+// together, whole rows per load instruction, and read their operands from there, so the K/V rows pass through the
+// memory system once per workgroup; the shares' (m, l, O) meet in LDS at the end and share 0 writes the rows.
+// grid = (ceil(G * row tiles / NSUB), num_kv_heads); block = 64 * NSUB * KS.
+template <int D, int QT, int KS, int NSUB = 4>
+__global__ void __launch_bounds__(64 * NSUB * KS) paged_mq_kernel(const float *__restrict__ q, const _Float16 *__restrict__ pool,
                                                          const int32_t *__restrict__ table, const int32_t *__restrict__ kv_lens,
                                                          float *__restrict__ out, int query_len, int max_keys, int num_q_heads,
                                                          int num_kv_heads, float scale) {
@@ -695,8 +696,10 @@ __global__ void __launch_bounds__(256, 2) paged_mq_kernel(const float *__restric
     const int kvh = blockIdx.y, G = num_q_heads / num_kv_heads;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int combo = blockIdx.x * 4 + wave, row_groups = (query_len + 16 * QT - 1) / (16 * QT);
-    if (combo >= G * row_groups) return;  // (no barrier in this kernel: a wave without work leaves)
+    const int sub = wave % NSUB, ksub = wave / NSUB;  // which of the workgroup's NSUB (head, row group) pairs, which share of the blocks
+    const int row_groups = (query_len + 16 * QT - 1) / (16 * QT);
+    const bool idle = blockIdx.x * NSUB + sub >= G * row_groups;  // (a wave without work walks no block; it still meets the others)
+    const int combo = min((int)blockIdx.x * NSUB + sub, G * row_groups - 1);
     const int head = kvh * G + combo % G, r0 = (combo / G) * 16 * QT;
     const int c16 = lane & 15, g4 = lane >> 4;
     const size_t hs = (size_t)num_kv_heads * D, part = (size_t)HOT_BS * hs, qs = (size_t)num_q_heads * D;
@@ -757,36 +760,14 @@ __global__ void __launch_bounds__(256, 2) paged_mq_kernel(const float *__restric
 #pragma unroll
         for (int e = 0; e < NT; e++) o[t][e] = (float4v){0.f, 0.f, 0.f, 0.f};
     }
-    const int n_blocks = (len_max + HOT_BS - 1) / HOT_BS;
-    const size_t k_off = (size_t)(4 * (c16 & 3) + (c16 >> 2)) * hs + (size_t)kvh * D + g4 * (D / 4);
-    const size_t v_off = part + (size_t)g4 * hs + (size_t)kvh * D + c16 * NT;
-    half8 kk[NS], kn[NS];
-    halfv vv[4], vn[4];
-    auto issue = [&](int bi, half8 *kd, halfv *vd) {
-        const int blk = __builtin_amdgcn_readfirstlane(table[bi]);
-        const _Float16 *base = pool + (size_t)blk * 2 * part;
-#pragma unroll
-        for (int s = 0; s < NS; s++) kd[s] = *(const half8 *)(base + k_off + 8 * s);
-#pragma unroll
-        for (int i = 0; i < 4; i++) vd[i] = *(const halfv *)(base + v_off + (size_t)i * 4 * hs);
-    };
-    if (n_blocks > 0) issue(0, kn, vn);
-    for (int bi = 0; bi < n_blocks; bi++) {
-#pragma unroll
-        for (int s = 0; s < NS; s++) kk[s] = kn[s];
-#pragma unroll
-        for (int i = 0; i < 4; i++) vv[i] = vn[i];
-        if (bi + 1 < n_blocks) issue(bi + 1, kn, vn);
-        __builtin_amdgcn_sched_barrier(0);
+    const int n_blocks = idle ? 0 : (len_max + HOT_BS - 1) / HOT_BS;
+    const int tok_row = 4 * (c16 & 3) + (c16 >> 2);  // this lane's K row of a block as A operand
+    half8 kk[NS];
+    halfv vv[4];
+    // one block against the wave's query tiles (kk, vv hold the block's operands)
+    auto compute = [&](int bi) __attribute__((always_inline)) {
         const int tok0 = bi * HOT_BS + g4;                       // score i of a tile: token tok0 + 4i
         const bool open = (bi + 1) * HOT_BS <= len_min;          // every row of the wave sees the whole block
-        if ((bi + 1) * HOT_BS > len_max) {                       // rows past the sequence's end may hold anything
-#pragma unroll
-            for (int i = 0; i < 4; i++)
-                if (tok0 + 4 * i >= len_max)
-#pragma unroll
-                    for (int e = 0; e < NT; e++) vv[i][e] = (_Float16)0.f;
-        }
 #pragma unroll
         for (int t = 0; t < QT; t++) {
             float4v sc = {0.f, 0.f, 0.f, 0.f};
@@ -833,24 +814,128 @@ __global__ void __launch_bounds__(256, 2) paged_mq_kernel(const float *__restric
                 o[t][e] = __builtin_amdgcn_mfma_f32_16x16x16f16(pl, vb, o[t][e], 0, 0, 0);
             }
         }
+    };
+    {
+        // The NSUB waves that share a block (same KV head, same share of the blocks) bring it into LDS together, whole
+        // rows per load instruction, once for all of them, and each reads its operands from there: one pass over
+        // the K/V rows per workgroup instead of one per wave. Two buffers, one barrier per block; the loop runs to
+        // the longest of the workgroup's row tiles for every wave.
+        constexpr int KP = D + 8;                      // halves per staged row (rows 4 banks apart)
+        constexpr int TG = NSUB * 64, PIECES = HOT_BS * D / 8, PPT = (PIECES + TG - 1) / TG;
+        __shared__ __attribute__((aligned(16))) _Float16 stg[KS][2][2][HOT_BS * KP];
+        __shared__ int s_wg[2];
+        if (tid == 0) s_wg[0] = s_wg[1] = 0;
+        __syncthreads();
+        if (lane == 0 && !idle) {
+            atomicMax(&s_wg[0], n_blocks);
+            atomicMax(&s_wg[1], len_max);
+        }
+        __syncthreads();
+        const int wg_blocks = s_wg[0], wg_len = s_wg[1];
+        const int tg = sub * 64 + lane;
+        half8 kreg[PPT], vreg[PPT];
+        auto issue = [&](int bi) {
+            const int blk = __builtin_amdgcn_readfirstlane(table[bi]);
+            const _Float16 *base = pool + (size_t)blk * 2 * part + (size_t)kvh * D;
+#pragma unroll
+            for (int j = 0; j < PPT; j++) {
+                const int pc = min(j * TG + tg, PIECES - 1), row = pc / (D / 8), c8 = pc % (D / 8);
+                kreg[j] = *(const half8 *)(base + (size_t)row * hs + c8 * 8);
+                vreg[j] = *(const half8 *)(base + part + (size_t)row * hs + c8 * 8);
+            }
+        };
+        auto commit = [&](int bi, int buf) {
+#pragma unroll
+            for (int j = 0; j < PPT; j++) {
+                const int pc = j * TG + tg, row = pc / (D / 8), c8 = pc % (D / 8);
+                if (PIECES % TG != 0 && pc >= PIECES) continue;
+                half8 v = vreg[j];
+                if (bi * HOT_BS + row >= wg_len) v = (half8){0, 0, 0, 0, 0, 0, 0, 0};  // rows past the sequence's end may hold anything
+                *(half8 *)&stg[ksub][buf][0][row * KP + c8 * 8] = kreg[j];
+                *(half8 *)&stg[ksub][buf][1][row * KP + c8 * 8] = v;
+            }
+        };
+        const int iters = (wg_blocks + KS - 1) / KS;
+        if (ksub < wg_blocks) issue(ksub);
+        for (int it = 0; it < iters; it++) {
+            const int bi = it * KS + ksub, buf = it & 1;
+            if (bi < wg_blocks) commit(bi, buf);
+            if (bi + KS < wg_blocks) issue(bi + KS);
+            __syncthreads();
+            if (bi < n_blocks) {  // (beyond: none of this wave's rows sees a key of the block)
+#pragma unroll
+                for (int s = 0; s < NS; s++) kk[s] = *(const half8 *)&stg[ksub][buf][0][tok_row * KP + g4 * (D / 4) + 8 * s];
+#pragma unroll
+                for (int i = 0; i < 4; i++) vv[i] = *(const halfv *)&stg[ksub][buf][1][(4 * i + g4) * KP + c16 * NT];
+                compute(bi);
+            }
+        }
     }
     // lane (c16, g4) holds O[row 4 g4 + i][columns c16 * NT .. + NT - 1] of every tile; the row's sum of weights is
-    // spread over the four lanes (row, 0..3)
+    // spread over the four lanes (row, 0..3). With KS > 1 the waves that took the other shares of the blocks hand
+    // their (m, l, O) over through LDS - every value in the slot of the lane that holds the same element - and the
+    // wave with share 0 adds them in share order.
+    __shared__ float s_m[KS > 1 ? KS : 1][NSUB][QT][16], s_l[KS > 1 ? KS : 1][NSUB][QT][16];
+    __shared__ float s_o[KS > 1 ? KS - 1 : 1][KS > 1 ? NSUB : 1][QT][4 * NT][64];
 #pragma unroll
     for (int t = 0; t < QT; t++) {
-        float l = l_run[t];
-        l += __shfl_xor(l, 16, 64);
-        l += __shfl_xor(l, 32, 64);
-        const float inv = l > 0.f ? 1.f / l : 0.f;
+        l_run[t] += __shfl_xor(l_run[t], 16, 64);
+        l_run[t] += __shfl_xor(l_run[t], 32, 64);
+    }
+    if constexpr (KS > 1) {
+#pragma unroll
+        for (int t = 0; t < QT; t++) {
+            if (g4 == 0) {
+                s_m[ksub][sub][t][c16] = m_run[t];
+                s_l[ksub][sub][t][c16] = l_run[t];
+            }
+            if (ksub > 0) {
+#pragma unroll
+                for (int e = 0; e < NT; e++)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) s_o[ksub - 1][sub][t][e * 4 + i][lane] = o[t][e][i];
+            }
+        }
+        __syncthreads();
+        if (ksub > 0) return;
+    }
+    if (idle) return;
+#pragma unroll
+    for (int t = 0; t < QT; t++) {
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float w = __shfl(inv, 4 * g4 + i, 64);
-            const int qi = r0 + 16 * t + 4 * g4 + i;
+            const int row = 4 * g4 + i, qi = r0 + 16 * t + row;
+            float L, w[KS];
+            if constexpr (KS > 1) {
+                float M = s_m[0][sub][t][row];
+#pragma unroll
+                for (int k2 = 1; k2 < KS; k2++) M = fmaxf(M, s_m[k2][sub][t][row]);
+                L = 0.f;
+#pragma unroll
+                for (int k2 = 0; k2 < KS; k2++) {
+                    const float mk = s_m[k2][sub][t][row];
+                    w[k2] = mk == -INFINITY ? 0.f : exp2f(mk - M);
+                    L += s_l[k2][sub][t][row] * w[k2];
+                }
+            } else {
+                L = __shfl(l_run[t], row, 64);
+                w[0] = 1.f;
+            }
+            const float inv = L > 0.f ? 1.f / L : 0.f;
             if (qi >= query_len) continue;
             float *op = out + (size_t)qi * qs + (size_t)head * D + c16 * NT;
+            float y[NT];
 #pragma unroll
-            for (int e = 0; e < NT; e += 4)
-                *(float4 *)(op + e) = make_float4(o[t][e][i] * w, o[t][e + 1][i] * w, o[t][e + 2][i] * w, o[t][e + 3][i] * w);
+            for (int e = 0; e < NT; e++) {
+                float acc = o[t][e][i] * w[0];
+                if constexpr (KS > 1) {
+#pragma unroll
+                    for (int k2 = 1; k2 < KS; k2++) acc += s_o[k2 - 1][sub][t][e * 4 + i][lane] * w[k2];
+                }
+                y[e] = acc * inv;
+            }
+#pragma unroll
+            for (int e = 0; e < NT; e += 4) *(float4 *)(op + e) = make_float4(y[e], y[e + 1], y[e + 2], y[e + 3]);
         }
     }
 }
@@ -1563,13 +1648,19 @@ int vx_sdpa_paged_decode_multiquery(vx_backend *be, const float *q, const void *
         block_size == HOT_BS && ((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 16) == 0 && !lds_tiles) {
         constexpr int QT = 1;
         const int G = num_q_heads / num_kv_heads, combos = G * ceil_div(query_len, 16 * QT);
-        const dim3 grid(ceil_div(combos, 4), num_kv_heads);
-        if (head_dim == 128)
-            paged_mq_kernel<128, QT><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)kv_pool, block_table, kv_lens, out, query_len,
-                                                                   num_blocks * block_size, num_q_heads, num_kv_heads, scale);
-        else
-            paged_mq_kernel<64, QT><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)kv_pool, block_table, kv_lens, out, query_len,
-                                                                  num_blocks * block_size, num_q_heads, num_kv_heads, scale);
+        // the blocks of a row tile shared out over 1, 2 or 4 waves: two waves per SIMD and more cover each other's
+        // dependent chains (scores, softmax, weights, values), fewer leave the matrix cores waiting
+        const long waves = (long)combos * num_kv_heads;
+        const int share = waves >= 2048 ? 1 : (waves >= 1024 ? 2 : 4);
+        const _Float16 *pool = (const _Float16 *)kv_pool;
+        const int max_keys = num_blocks * block_size;
+#define VX_MQ(DD, KK, NS)                                                                                                 \
+    if (head_dim == DD && share == KK)                                                                                    \
+        paged_mq_kernel<DD, QT, KK, NS><<<dim3(ceil_div(combos, NS), num_kv_heads), 64 * NS * KK, 0, be->stream>>>(         \
+            q, pool, block_table, kv_lens, out, query_len, max_keys, num_q_heads, num_kv_heads, scale);
+        // (heads of 128 with four shares: two pairs a workgroup, so that a wave keeps 256 registers)
+        VX_MQ(128, 1, 4) VX_MQ(128, 2, 4) VX_MQ(128, 4, 2) VX_MQ(64, 1, 4) VX_MQ(64, 2, 4) VX_MQ(64, 4, 4)
+#undef VX_MQ
         VX_CHECK_LAUNCH();
         return VX_OK;
     }
