@@ -526,10 +526,11 @@ def prefill_probe(be, rows=512, reps=10):
     print(json.dumps(out))
 
 
-def configs_report(be):
+def configs_report(be, only=None):
     """Throughput of the benchmark configs other than the north star, each at its real shape (synthetic weights and
     contexts, greedy decode replayed from a hipGraph; config 4 as its two ingredients; config 5 as one verification
-    step). Informational: the benchmark line is the north-star workload."""
+    step). Informational: the benchmark line is the north-star workload.
+    only: "1" .. "5" runs that config alone ("4": its decode part; "4p": decode and the prefill chunks)."""
     from vexel_amd import lib
     from oracle import host_logic as hl
     tiny = dict(num_layers=22, hidden=2048, num_heads=32, num_kv_heads=4, head_dim=64, ffn=5632, vocab=32000)
@@ -550,18 +551,35 @@ def configs_report(be):
         return mr, ids
 
     rng = np.random.default_rng(0)
-    mr, _ = decode_rate("config 1: TinyLlama-shaped Q4_0, 1 sequence, ctx 32 + 64 steps", tiny, None, [32], 64)
-    mr.close()
-    ctx2 = [int(x) for x in rng.integers(128, 2049, 8)]
-    mr, _ = decode_rate("config 2: TinyLlama-shaped Q4_0, 8 ragged sequences (sum ctx %d)" % sum(ctx2), tiny, None, ctx2, 128)
-    mr.close()
+    want = lambda n: only is None or only[0] == n
+    if want("1"):
+        mr, _ = decode_rate("config 1: TinyLlama-shaped Q4_0, 1 sequence, ctx 32 + 64 steps", tiny, None, [32], 64)
+        mr.close()
+    ctx2 = [int(x) for x in rng.integers(128, 2049, 8)]   # (the contexts are drawn whether or not the config runs: same numbers either way)
+    if want("2"):
+        mr, _ = decode_rate("config 2: TinyLlama-shaped Q4_0, 8 ragged sequences (sum ctx %d)" % sum(ctx2), tiny, None, ctx2, 128)
+        mr.close()
     ctx3 = ragged_contexts()
-    mr, _ = decode_rate("config 3: 7B-shaped Q4_K_M mix, 32 ragged sequences (sum ctx %d)" % sum(ctx3), CFG, q4km, ctx3, 64)
-    mr.close()
+    if want("3"):
+        mr, _ = decode_rate("config 3: 7B-shaped Q4_K_M mix, 32 ragged sequences (sum ctx %d)" % sum(ctx3), CFG, q4km, ctx3, 64)
+        mr.close()
     ctx4 = [int(x) for x in np.clip(np.exp(rng.normal(math.log(512.0), 0.6, 64)), 16, 4096)]
+    if want("4"):
+        _config4(be, rng, ctx4, l8b, decode_rate, prefill=only != "4")
+    else:
+        rng.integers(0, l8b["vocab"], 512)
+    if want("5"):
+        _config5(be, rng)
+
+
+def _config4(be, rng, ctx4, l8b, decode_rate, prefill):
+    from vexel_amd import lib
     mr, ids = decode_rate("config 4 (decode part): 8B-shaped Q8_0, 64 sequences (sum ctx %d)" % sum(ctx4), l8b,
                           {"*": lib.VX_Q8_0}, ctx4, 32, spare_tokens=4200)   # (free blocks for the chunks below)
     chunk = rng.integers(0, l8b["vocab"], 512).tolist()
+    if not prefill:
+        mr.close()
+        return
     mr.prefill_with_paged_kv(chunk[:64], 1000, 0)           # sizes the workspaces
     mr.delete_sequence(1000)
     be.sync()
@@ -592,6 +610,11 @@ def configs_report(be):
                                                       512 / dt, dt * 1e3), flush=True)
         mr.delete_sequence(sid)
     mr.close()
+
+
+def _config5(be, rng):
+    from vexel_amd import lib
+    from oracle import host_logic as hl
     ctx5 = [int(x) for x in rng.integers(256, 2049, 16)]
     mr, ids = build_model(be, ctx5, 64, 32, CFG, {"*": lib.VX_Q6_K}, max_batch=16)
     start, inputs = list(ctx5), rng.integers(0, 32000, 16).tolist()
@@ -691,6 +714,8 @@ def main():
                          "table of achieved GB/s against the 8 TB/s HBM peak, then exit")
     ap.add_argument("--counter-probe", action="store_true",
                     help="for rocprofv3 --pmc runs: one 1 GiB plain copy and 8 attention launches, then exit")
+    ap.add_argument("--only", default=None, choices=["1", "2", "3", "4", "4p", "5"],
+                    help="with --configs-report: that config alone (4: its decode part, 4p: with the prefill chunks)")
     ap.add_argument("--configs-report", action="store_true",
                     help="decode / prefill / verification rates of benchmark configs 1-5 at their real shapes, then exit")
     ap.add_argument("--prefill-probe", action="store_true",
@@ -713,7 +738,7 @@ def main():
         prefill_probe(be)
         return
     if args.configs_report:
-        configs_report(be)
+        configs_report(be, args.only)
         return
     if args.medusa_report:
         medusa_report(be)
