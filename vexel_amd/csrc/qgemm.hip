@@ -1,7 +1,7 @@
-// Quantized matmul C[M,N] = A[M,K] * B^T with B in raw GGUF blocks (Q4_0, Q8_0, Q4_K, Q6_K).
-// Replaces QuantizedMatMul.MatMulQ4_0/Q4_K/Q6_K/Q8_0 (inference/backend/backend.go:47-81).
+// Quantized matmul C[M,N] = A[M,K] * B^T with B in raw GGUF blocks (Q4_0, Q8_0, Q4_K, Q6_K, Q5_0, Q5_K) or BF16.
+// Replaces QuantizedMatMul.MatMulQ4_0/Q4_K/Q6_K/Q8_0/Q5_0/Q5_K/BF16 (inference/backend/backend.go:47-81).
 //
-// Fast path (Q4_0, Q8_0, Q4_K; K a multiple of 256, 16-byte aligned rows), two phases:
+// Fast path (the six block formats; K a multiple of 256, the matrix on a 16-byte boundary), two phases:
 //
 //  1. prepare: every activation row is scaled by a power of two and split into
 //     hi = f16(x), lo = f16(x - hi) (together ~22 significant bits, the float32 level). Both are
@@ -20,9 +20,10 @@
 //     format's integers. With KS > 1 slices the partial sums go to scratch and
 //     qgemm_reduce_kernel adds them in slice order (deterministic), applies the row scale and
 //     the optional residual.
-//     Decode batches (2 to 32 rows) whose weight rows fit one round of workgroups take
-//     qgemm_wave_kernel (qgemm_wave.h) instead: one workgroup per compute unit, its waves split K,
-//     activation tiles go from L2 straight to registers; BF16 matrices take it at any batch size.
+//     Decode batches (2 to 64 rows) of Q4_0, Q8_0 and Q4_K take qgemm_wave_kernel (qgemm_wave.h)
+//     instead: one workgroup per compute unit, its waves split K, activation tiles go from L2
+//     straight to registers (up to 32 rows: matrices whose rows fit one round of workgroups; 33 to
+//     64 rows: four activation tiles a step, several rounds); BF16 matrices take it at any batch size.
 //     Q8_0 batches of more than 96 rows take qgemm_rows_kernel (same header): the waves split the
 //     weight rows and share 64 activation rows' tiles through LDS.
 //  Each output element depends only on its own activation row and weight row and the launch
@@ -30,8 +31,7 @@
 //  the same bits in any two batches of one range (the property the reference keeps by looping
 //  M=1 kernels, backend/metal/backend.go:777-779).
 //
-// Fallback (Q6_K, odd shapes): one wave per output column, float32 FMAs on the exact
-// dequantised values.
+// Fallback (odd shapes): one wave per output column, float32 FMAs on the exact dequantised values.
 #include <stdlib.h>
 
 #include "common.h"
