@@ -489,7 +489,8 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
 // scores of the tokens 4i + g, i = 0..3 - which is the A operand of the second product as it stands - and the
 // V rows of exactly those tokens, D/16 columns from c * D/16 on, are what the same lane loads (for D = 128 the
 // 16 bytes per lane of the vector form: whole rows per instruction); tile e of the output holds columns
-// c * D/16 + e. Rows of Q beyond G*RG are zero and their results are dropped.
+// c * D/16 + e. K reaches its operand layout through the wave's own LDS rows. Rows of Q beyond G*RG are zero and
+// their results are dropped.
 template <int D, int G, int RG = 1>
 __global__ void __launch_bounds__(256, 3) paged_decode_gqa_kernel(
     const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix,
@@ -585,7 +586,16 @@ __global__ void __launch_bounds__(256, 3) paged_decode_gqa_kernel(
     float m_run = -INFINITY, l_run = 0.f;  // of query c16; l_run over this lane's tokens only until the end
 
     const int n_blocks = (t_end - t_begin + HOT_BS - 1) / HOT_BS;
-    const size_t k_off = (size_t)(4 * (c16 & 3) + (c16 >> 2)) * hs + (size_t)kvh * D + g4 * (D / 4);
+    // K is loaded as whole rows per instruction, the way V is (LPT lanes a row, TPI rows an instruction), and turned
+    // into the A operand's layout - one row per 16 lanes, a quarter of it per lane group - through the wave's own
+    // LDS rows: loading it in operand layout straight from the pool (16 bytes per lane at four places of every row)
+    // measured 5 - 9 % slower.
+    constexpr int LPT = D / 8, TPI = 64 / LPT;
+    constexpr int KP = D + 8;  // halves per staged row
+    __shared__ __attribute__((aligned(16))) _Float16 kst[4][HOT_BS * KP];
+    const int tok_row = 4 * (c16 & 3) + (c16 >> 2);
+    const size_t k_off = (size_t)(lane / LPT) * hs + (size_t)kvh * D + (lane % LPT) * 8;
+    const size_t k_step = (size_t)TPI * hs;
     const size_t v_off = part + (size_t)g4 * hs + (size_t)kvh * D + c16 * NT;
     half8 kk[NS], kn[NS];
     halfv vv[4], vn[4];
@@ -593,17 +603,24 @@ __global__ void __launch_bounds__(256, 3) paged_decode_gqa_kernel(
         const int blk = __builtin_amdgcn_readfirstlane(bt[bi]);
         const _Float16 *base = pool + (size_t)blk * 2 * part;
 #pragma unroll
-        for (int s = 0; s < NS; s++) kd[s] = *(const half8 *)(base + k_off + 8 * s);
+        for (int s = 0; s < NS; s++) kd[s] = *(const half8 *)(base + k_off + k_step * s);
 #pragma unroll
         for (int i = 0; i < 4; i++) vd[i] = *(const halfv *)(base + v_off + (size_t)i * 4 * hs);  // token 4i + g4
     };
     if (wave < n_blocks) issue(wave, kn, vn);
     for (int bi = wave; bi < n_blocks; bi += 4) {
 #pragma unroll
-        for (int s = 0; s < NS; s++) kk[s] = kn[s];
+        for (int s = 0; s < NS; s++) *(half8 *)&kst[wave][(s * TPI + lane / LPT) * KP + (lane % LPT) * 8] = kn[s];
 #pragma unroll
         for (int i = 0; i < 4; i++) vv[i] = vn[i];
         if (bi + 4 < n_blocks) issue(bi + 4, kn, vn);
+        // (the wave's own rows: its LDS accesses stay in order, the compiler must keep them so)
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int s = 0; s < NS; s++) kk[s] = *(const half8 *)&kst[wave][tok_row * KP + g4 * (D / 4) + 8 * s];
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_sched_barrier(0);
         float4v sc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
