@@ -530,8 +530,11 @@ def test_decode_attn_qkv_with_v_in_another_format(be, rows, fqk, fv):
 
 
 # (query heads, kv heads, head size): a workgroup's columns are one 256-column chunk, a quarter or half of one,
-# four of them, and (3 query heads of 128 per kv head) no whole number either way
-@pytest.mark.parametrize("hq,hk,d", [(8, 2, 64), (8, 8, 64), (4, 4, 128), (8, 1, 128), (6, 2, 128)])
+# four of them, one and a half / three and a half (two KV heads make whole chunks), five sixteenths (heads of 80:
+# sixteen KV heads make five chunks). (Whenever all heads together are whole chunks, which the fused output
+# projection needs anyway, the KV heads are whole merge units.)
+@pytest.mark.parametrize("hq,hk,d", [(8, 2, 64), (8, 8, 64), (4, 4, 128), (8, 1, 128), (6, 2, 128), (28, 4, 128),
+                                     (16, 16, 80)])
 def test_decode_ffn_merges_split_attention(be, hq, hk, d):
     """vx_sdpa_paged_decode_ragged(out = NULL) + vx_decode_ffn(attn = NULL) equals the merged attention output
     fed to vx_decode_ffn (the split-KV partials are merged by the same formula, by the attention kernel's last

@@ -226,6 +226,15 @@ __device__ __forceinline__ float token_sum(float t) {
 // Where the workgroup that finishes a sequence's 256-column chunk last leaves the chunk merged over its splits,
 // as the prepared activation of the output projection (cnt == nullptr: nobody merges, the partial sums are the
 // result). cnt[sequence * units + unit] counts the arrivals and is zero again when the launch ends.
+// The unit of the in-kernel merge for workgroups of GD = G * D output columns: the fewest KV heads whose columns are
+// a whole number of 256-column chunks (HPC of them, CH chunks).
+constexpr int gcd_c(int a, int b) { return b == 0 ? a : gcd_c(b, a % b); }
+template <int GD>
+struct MergeUnit {
+    static constexpr int HPC = 256 / gcd_c(GD, 256);
+    static constexpr int CH = HPC * GD / 256;
+};
+
 struct MergeOut {
     PrepView pv;
     int32_t *cnt = nullptr;
@@ -254,9 +263,9 @@ __device__ __forceinline__ void finish_split(const float (&s_m)[4][G * RG], cons
                                              int max_splits, const MergeOut &mg, int tps) {
     constexpr int GG = G * RG;
     constexpr int GD = G * D;                          // this workgroup's columns of the output
-    constexpr bool MERGES = RG == 1 && (GD % 256 == 0 || 256 % GD == 0);
-    constexpr int CH = GD >= 256 ? GD / 256 : 1;       // 256-column chunks inside them
-    constexpr int HPC = GD >= 256 ? 1 : 256 / GD;      // kv heads that share a chunk
+    constexpr bool MERGES = RG == 1;
+    constexpr int CH = MergeUnit<GD>::CH;    // 256-column chunks of a merge unit
+    constexpr int HPC = MergeUnit<GD>::HPC;  // kv heads of a merge unit
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     __syncthreads();
@@ -349,9 +358,9 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     constexpr int GD = G * D;                          // this workgroup's columns of the output
-    constexpr bool MERGES = RG == 1 && (GD % 256 == 0 || 256 % GD == 0);
-    constexpr int CH = GD >= 256 ? GD / 256 : 1;       // 256-column chunks inside them
-    constexpr int HPC = GD >= 256 ? 1 : 256 / GD;      // kv heads that share a chunk
+    constexpr bool MERGES = RG == 1;
+    constexpr int CH = MergeUnit<GD>::CH;    // 256-column chunks of a merge unit
+    constexpr int HPC = MergeUnit<GD>::HPC;  // kv heads of a merge unit
     if (split >= max_splits || t_begin >= kv_len) {
         // a sequence without tokens has nobody to merge for it: zeros, as the merge of no splits gives
         if constexpr (MERGES) {
@@ -521,9 +530,9 @@ __global__ void __launch_bounds__(256, 3) paged_decode_gqa_kernel(
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     constexpr int GD = G * D;
-    constexpr bool MERGES = RG == 1 && (GD % 256 == 0 || 256 % GD == 0);
-    constexpr int CH = GD >= 256 ? GD / 256 : 1;
-    constexpr int HPC = GD >= 256 ? 1 : 256 / GD;
+    constexpr bool MERGES = RG == 1;
+    constexpr int CH = MergeUnit<GD>::CH;    // 256-column chunks of a merge unit
+    constexpr int HPC = MergeUnit<GD>::HPC;  // kv heads of a merge unit
     if (split >= max_splits || t_begin >= kv_len) {
         if constexpr (MERGES) {
             if (mg.cnt && kv_len == 0 && split == 0 && kvh % HPC == 0) {
@@ -1333,9 +1342,7 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
     float *plain = nullptr;
     static const bool no_merge = getenv("VEXEL_HIP_NO_ATTN_MERGE") != nullptr;
     constexpr int GD = G * D;
-    constexpr int HPC = (GD < 256 && 256 % GD == 0) ? 256 / GD : 0;  // kv heads that share a chunk
-    bool mergeable = GD % 256 == 0;
-    if constexpr (HPC > 0) mergeable = num_kv_heads % HPC == 0;
+    const bool mergeable = num_kv_heads % MergeUnit<GD>::HPC == 0;  // (whole merge units: chunks of whole KV heads)
     if (!out && !fixed && !no_merge && mergeable && be->attn_cnt && (size_t)batch * num_kv_heads <= VX_ATTN_CNT) {
         if (batch == 1) {
             mg.cnt = be->attn_cnt;
