@@ -523,6 +523,25 @@ def prefill_probe(be, rows=512, reps=10):
     ms = be.timer_stop_ms() / reps
     flops = 4.0 * hq * d * rows * (rows + 1) / 2
     out["prefill_attention"] = {"tokens": rows, "ms": ms, "tflops": flops / ms / 1e9}
+    # a later chunk of a prompt: `rows` query rows at position 3584 over the paged f16 pool, 8B head geometry (32 / 8)
+    hk, start = 8, 3584
+    nb = (start + rows + BLOCK - 1) // BLOCK
+    pool = be.alloc_permanent(nb * 2 * BLOCK * hk * d * 2)
+    if synth.vxs_gaussian_f16(pool, nb * 2 * BLOCK * hk * d, 1.0, 7):
+        raise RuntimeError("synthetic KV generation failed")
+    dbt = be.upload(rng.permutation(nb).astype(np.int32), permanent=True)
+    kvl = np.arange(start + 1, start + rows + 1, dtype=np.int32)
+    dk = be.upload(kvl, permanent=True)
+    args = (bufs[0], pool, dbt, do, dk, nb, BLOCK, hq, hk, d, scale, rows)
+    be.sdpa_paged_decode_multiquery(*args, pool_is_f16=True)
+    be.sync()
+    be.timer_start()
+    for _ in range(reps):
+        be.sdpa_paged_decode_multiquery(*args, pool_is_f16=True)
+    ms = be.timer_stop_ms() / reps
+    flops = 4.0 * hq * d * float(kvl.sum())
+    out["paged_multiquery_attention"] = {"rows": rows, "position": start, "heads": "%d/%d x %d" % (hq, hk, d), "ms": ms,
+                                         "tflops": flops / ms / 1e9}
     print(json.dumps(out))
 
 
