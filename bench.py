@@ -428,6 +428,8 @@ def kernel_report(be):
             tables[i, :nblk[i]] = perm[off:off + nblk[i]]
             off += nblk[i]
         pool = be.alloc_permanent(sum(nblk) * 2 * BLOCK * hk * d * 2)
+        if synth.vxs_gaussian_f16(pool, sum(nblk) * 2 * BLOCK * hk * d, 1.0, 11):
+            raise RuntimeError("synthetic KV generation failed")
         dq = be.upload(rng.standard_normal((nseq, hq * d)).astype(np.float32), permanent=True)
         dt, dl = be.upload(tables, permanent=True), be.upload(lens, permanent=True)
         args = (dq, pool, True, dt, dl, None, nseq, 256, BLOCK, hq, hk, d, 1.0 / math.sqrt(d), 4096)

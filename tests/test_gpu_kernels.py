@@ -530,9 +530,9 @@ def test_decode_attn_qkv_with_v_in_another_format(be, rows, fqk, fv):
 
 
 # (query heads, kv heads, head size): a workgroup's columns are one 256-column chunk, a quarter or half of one,
-# four of them, one and a half / three and a half (two KV heads make whole chunks), five sixteenths (heads of 80:
-# sixteen KV heads make five chunks). (Whenever all heads together are whole chunks, which the fused output
-# projection needs anyway, the KV heads are whole merge units.)
+# four of them, one and a half (two KV heads make three chunks: merged in the kernel), three and a half and five
+# sixteenths (7 chunks per two KV heads, 5 per sixteen heads of 80: more than a workgroup merges at once, the
+# prepare kernel does it)
 @pytest.mark.parametrize("hq,hk,d", [(8, 2, 64), (8, 8, 64), (4, 4, 128), (8, 1, 128), (6, 2, 128), (28, 4, 128),
                                      (16, 16, 80)])
 def test_decode_ffn_merges_split_attention(be, hq, hk, d):

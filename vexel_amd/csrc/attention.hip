@@ -1342,7 +1342,9 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
     float *plain = nullptr;
     static const bool no_merge = getenv("VEXEL_HIP_NO_ATTN_MERGE") != nullptr;
     constexpr int GD = G * D;
-    const bool mergeable = num_kv_heads % MergeUnit<GD>::HPC == 0;  // (whole merge units: chunks of whole KV heads)
+    // whole merge units, of at most one chunk per wave of the merging workgroup (with more - 7 chunks per two KV heads
+    // at 28 / 4 heads of 128 - the merge at the launch's tail costs what the separate merge launch does)
+    const bool mergeable = num_kv_heads % MergeUnit<GD>::HPC == 0 && MergeUnit<GD>::CH <= 4;
     if (!out && !fixed && !no_merge && mergeable && be->attn_cnt && (size_t)batch * num_kv_heads <= VX_ATTN_CNT) {
         if (batch == 1) {
             mg.cnt = be->attn_cnt;
