@@ -966,49 +966,84 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
     VXC(vx_embedding(be, d_tok, n, m->embedding, x, c.vocab, c.hidden));               // decode.go:1005-1010
     VHC(g_scale_embedding(m, x, n));                                                   // decode.go:1030
     const float scale = (float)(1.0 / sqrt((double)c.head_dim));
+    // A later chunk reads every key from the pool (block.go:881-890), so its projections can take the decode step's
+    // fused form: Q|K|V in one launch that rotates and stores K/V itself; the fused tail serves every chunk.
+    const bool later = n > 1 && start_pos > 0;
+    const bool tails_fusable = n > 1 && m->fused && (!m->general || m->fused_ok);
+    int32_t *d_pos = nullptr, *d_slot = nullptr;
+    if (later) {
+        std::vector<int32_t> pos(n), slot(n);
+        for (int i = 0; i < n; i++) {
+            pos[i] = start_pos + i;
+            slot[i] = page[i] * c.block_size + offs[i];
+        }
+        d_pos = ia(n), d_slot = ia(n);
+        if (!d_pos || !d_slot) return fail("prefill buffers: %s", vx_last_error());
+        VXC(vx_to_device(be, d_pos, pos.data(), (size_t)n * 4));
+        VXC(vx_to_device(be, d_slot, slot.data(), (size_t)n * 4));
+    }
+    bool chained = false;  // the backend's prepared slot holds RMSNorm(x) * attn_norm of the layer about to run
     for (int l = 0; l < c.num_layers; l++) {
         const vh_layer_weights &w = m->layers[l];
-        if (m->general) {
-            VHC(g_qkv(m, l, x, norm, q, k, v, n));
-        } else {
-            bool prep;
-            const vh_qweight *qkv[3] = {&w.wq, &w.wk, &w.wv};
-            VHC(norm_for(m, x, w.attn_norm, norm, n, qkv, 3, &prep));
-            VHC(mm(m, prep, norm, w.wq, q, nullptr, n));
-            VHC(mm(m, prep, norm, w.wk, k, nullptr, n));
-            VHC(mm(m, prep, norm, w.wv, v, nullptr, n));
-        }
-        VXC(vx_rope(be, q, k, c.head_dim, c.num_heads, c.num_kv_heads, n, start_pos, m->arch.rope_dim, c.rope_theta,
-                    m->arch.rope_neox));                                               // block.go:858 (applyRoPE, :497-503)
-        if (c.kv_fp16) {                                                               // gpu_block_pool.go:262-272
-            VXC(vx_reshape_paged_kv_f16(be, k, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 0));
-            VXC(vx_reshape_paged_kv_f16(be, v, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 1));
-        } else {
-            VXC(vx_reshape_paged_kv(be, k, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 0));
-            VXC(vx_reshape_paged_kv(be, v, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 1));
-        }
-        if (n == 1) {                                                                  // block.go:866-874
-            const int nb = (seq_len + c.block_size - 1) / c.block_size;
-            const int til = seq_len - (nb - 1) * c.block_size;                        // gpu_block_pool.go:359-363
-            if (c.kv_fp16)
-                VXC(vx_sdpa_paged_decode_f16(be, q, m->kv[l], d_bt, attn, nb, c.block_size, c.num_heads,
-                                             c.num_kv_heads, c.head_dim, scale, til));
-            else
-                VXC(vx_sdpa_paged_decode(be, q, m->kv[l], d_bt, attn, nb, c.block_size, c.num_heads, c.num_kv_heads,
-                                         c.head_dim, scale, til));
-        } else if (start_pos > 0) {                                                    // block.go:881-890
+        const bool attn_fused = later && attn_fusable(m, l);
+        if (attn_fused) {
+            const vh_layer_extras &e = m->extras[l];
+            VXC(vx_decode_attn_qkv_ex(be, x, w.attn_norm, c.eps, chained ? 1 : 0, &w.wq, &w.wk, &w.wv, e.wq_bias, e.wk_bias,
+                                      e.wv_bias, n, d_pos, d_slot, m->kv[l], c.kv_fp16, c.num_heads, c.num_kv_heads, c.head_dim,
+                                      c.block_size, c.rope_theta, m->arch.rope_dim, m->arch.rope_neox, q));
+            chained = false;
             VXC(vx_sdpa_paged_decode_multiquery(be, q, m->kv[l], c.kv_fp16, d_bt, attn, d_kvl, (int)table.size(),
                                                 c.block_size, c.num_heads, c.num_kv_heads, c.head_dim, scale, n));
-        } else if (m->arch.attn_softcap > 0.f) {                                       // block.go:891-892
-            VXC(vx_sdpa_prefill_softcap(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale,
-                                        m->arch.attn_softcap));
-        } else {                                                                       // block.go:893-895
-            VXC(vx_sdpa_prefill(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale));
+        } else {
+            if (chained) return fail("internal: prepared activation handed to an unfused layer");
+            if (m->general) {
+                VHC(g_qkv(m, l, x, norm, q, k, v, n));
+            } else {
+                bool prep;
+                const vh_qweight *qkv[3] = {&w.wq, &w.wk, &w.wv};
+                VHC(norm_for(m, x, w.attn_norm, norm, n, qkv, 3, &prep));
+                VHC(mm(m, prep, norm, w.wq, q, nullptr, n));
+                VHC(mm(m, prep, norm, w.wk, k, nullptr, n));
+                VHC(mm(m, prep, norm, w.wv, v, nullptr, n));
+            }
+            VXC(vx_rope(be, q, k, c.head_dim, c.num_heads, c.num_kv_heads, n, start_pos, m->arch.rope_dim, c.rope_theta,
+                        m->arch.rope_neox));                                               // block.go:858 (applyRoPE, :497-503)
+            if (c.kv_fp16) {                                                               // gpu_block_pool.go:262-272
+                VXC(vx_reshape_paged_kv_f16(be, k, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 0));
+                VXC(vx_reshape_paged_kv_f16(be, v, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 1));
+            } else {
+                VXC(vx_reshape_paged_kv(be, k, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 0));
+                VXC(vx_reshape_paged_kv(be, v, m->kv[l], d_page, d_offs, n, c.num_kv_heads, c.head_dim, c.block_size, 1));
+            }
+            if (n == 1) {                                                                  // block.go:866-874
+                const int nb = (seq_len + c.block_size - 1) / c.block_size;
+                const int til = seq_len - (nb - 1) * c.block_size;                        // gpu_block_pool.go:359-363
+                if (c.kv_fp16)
+                    VXC(vx_sdpa_paged_decode_f16(be, q, m->kv[l], d_bt, attn, nb, c.block_size, c.num_heads,
+                                                 c.num_kv_heads, c.head_dim, scale, til));
+                else
+                    VXC(vx_sdpa_paged_decode(be, q, m->kv[l], d_bt, attn, nb, c.block_size, c.num_heads, c.num_kv_heads,
+                                             c.head_dim, scale, til));
+            } else if (start_pos > 0) {                                                    // block.go:881-890
+                VXC(vx_sdpa_paged_decode_multiquery(be, q, m->kv[l], c.kv_fp16, d_bt, attn, d_kvl, (int)table.size(),
+                                                    c.block_size, c.num_heads, c.num_kv_heads, c.head_dim, scale, n));
+            } else if (m->arch.attn_softcap > 0.f) {                                       // block.go:891-892
+                VXC(vx_sdpa_prefill_softcap(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale,
+                                            m->arch.attn_softcap));
+            } else {                                                                       // block.go:893-895
+                VXC(vx_sdpa_prefill(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale));
+            }
         }
-        if (m->general)
+        if (tails_fusable && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
+            vx_decode_ffn_supported(&w.wo, &w.w1, &w.w3, &w.w2)) {                      // block.go:981-1077
+            const float *next_norm = l + 1 < c.num_layers && later && attn_fusable(m, l + 1) ? m->layers[l + 1].attn_norm : nullptr;
+            VXC(vx_decode_ffn(be, attn, x, &w.wo, w.ffn_norm, c.eps, &w.w1, &w.w3, &w.w2, n, next_norm));
+            chained = next_norm != nullptr;
+        } else if (m->general) {
             VHC(g_tail(m, l, x, norm, attn, gate, up, n));
-        else
+        } else {
             VHC(layer_tail(m, w, x, norm, attn, gate, up, n));
+        }
     }
     const float *last = all_logits ? x : x + (size_t)(n - 1) * c.hidden;                // decode.go:1057-1066
     if (m->general) {
