@@ -782,7 +782,8 @@ def test_reshape_paged_kv_exact_layout(be, f16):
 
 @pytest.mark.parametrize("f16", [False, True])
 @pytest.mark.parametrize("shape", [(32, 4, 64), (32, 32, 128), (8, 8, 128), (4, 2, 32), (28, 4, 128), (24, 8, 128),
-                                   (12, 2, 64), (10, 2, 128), (14, 2, 64), (8, 4, 256), (4, 4, 256), (32, 32, 80), (6, 6, 96)])
+                                   (12, 2, 64), (10, 2, 128), (14, 2, 64), (8, 4, 256), (4, 4, 256), (32, 32, 80), (6, 6, 96),
+                                   (32, 2, 128), (24, 2, 128)])
 def test_paged_decode_single_batched_ragged(be, f16, shape):
     hq, hk, d = shape
     rng = np.random.default_rng(32 + hq + d)

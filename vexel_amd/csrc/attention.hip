@@ -1363,7 +1363,7 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
     static const bool vector_form = getenv("VEXEL_HIP_ATTN_VECTOR_FORM") != nullptr;
     bool launched = false;
     if constexpr (G >= 2 && (D == 64 || D == 128)) {  // (one query per K/V row: the vector form is the faster one, 110 against 119 us)
-        if (!vector_form) {
+        if (!vector_form || G > 8) {
             paged_decode_gqa_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
                                                                         max_blocks, kv_lens, ws, num_q_heads,
                                                                         num_kv_heads, scale, max_splits,
@@ -1371,11 +1371,13 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
             launched = true;
         }
     }
-    if (!launched)
-        paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
-                                                                    max_blocks, kv_lens, ws, num_q_heads,
-                                                                    num_kv_heads, scale, max_splits,
-                                                                    listed ? be->items.buf : nullptr, mg, tps);
+    if constexpr (G <= 8) {  // (wider groups have the matrix-core form only)
+        if (!launched)
+            paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
+                                                                        max_blocks, kv_lens, ws, num_q_heads,
+                                                                        num_kv_heads, scale, max_splits,
+                                                                        listed ? be->items.buf : nullptr, mg, tps);
+    }
     VX_CHECK_LAUNCH();
     if (!fixed) be->split.batch = 0;  // (the fixed area is not where vx_decode_ffn looks for a split result)
     if (!out) {  // the caller merges: vx_decode_ffn(attn = NULL)
@@ -1423,6 +1425,8 @@ int run_ragged(vx_backend *be, const float *q, const void *pool, int pool_is_f16
     // group sizes that are no power of two (Qwen 2 7B: 28 / 4 heads, LLaMA 3.2 3B: 24 / 8, Qwen 2 1.5B: 12 / 2)
     VX_HOT(128, 3) VX_HOT(128, 5) VX_HOT(128, 6) VX_HOT(128, 7)
     VX_HOT(64, 3) VX_HOT(64, 5) VX_HOT(64, 6) VX_HOT(64, 7)
+    // wide groups (12 and 16 query heads per KV head: the matrix-core tile's 16 rows)
+    VX_HOT(128, 12) VX_HOT(128, 16)
     // heads of 256 (Gemma): 32 lanes per token; the K/V registers of a 16-token block leave room for 1 or 2 query heads
     VX_HOT(256, 1) VX_HOT(256, 2)
     // heads of 80 (Phi-2) and 96 (Phi-3 mini) on 16 lanes per token, 10 or 12 of them live
@@ -1653,7 +1657,8 @@ int vx_sdpa_paged_decode_split_supported(int pool_is_f16, int block_size, int nu
                                          int head_dim) {
     if (!pool_is_f16 || block_size != HOT_BS || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0) return 0;
     const int G = num_q_heads / num_kv_heads;
-    return ((head_dim == 128 || head_dim == 64) && G >= 1 && G <= 8) || (head_dim == 256 && G <= 2) ||
+    return ((head_dim == 128 || head_dim == 64) && G >= 1 && G <= 8) || (head_dim == 128 && (G == 12 || G == 16)) ||
+           (head_dim == 256 && G <= 2) ||
            ((head_dim == 80 || head_dim == 96) && G == 1);
 }
 
