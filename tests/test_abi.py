@@ -52,3 +52,21 @@ def test_error_text_is_available_without_a_gpu():
 def test_every_entry_point_cites_the_reference():
     text = open(os.path.join(ROOT, "include", "vexel_hip.h")).read()
     assert text.count("backend.go") >= 10 and "gpu_block_pool.go" in text
+
+
+def test_geometry_queries_answer_without_a_gpu():
+    """The capability queries are plain functions of the head geometry: which shapes the streaming decode attention
+    takes (and leaves split for the fused tail), and how many rows of a candidate tree share one pass over the
+    context (16 queries per K/V row: 16 / G rows, whole)."""
+    dll = lib.load()
+    split = dll.vx_sdpa_paged_decode_split_supported
+    rows = dll.vx_sdpa_paged_tree_rows_per_entry
+    # (pool is f16, block size, query heads, kv heads, head size)
+    assert split(1, 16, 32, 32, 128) == 1 and split(1, 16, 32, 8, 128) == 1 and split(1, 16, 28, 4, 128) == 1
+    assert split(1, 16, 32, 2, 128) == 1 and split(1, 16, 24, 2, 128) == 1      # 16 and 12 query heads per kv head
+    assert split(1, 16, 36, 4, 128) == 0 and split(1, 16, 32, 2, 64) == 0        # 9 per kv head; 16 at heads of 64
+    assert split(1, 16, 8, 4, 256) == 1 and split(1, 16, 12, 4, 256) == 0 and split(1, 16, 32, 32, 80) == 1
+    assert split(0, 16, 32, 32, 128) == 0 and split(1, 32, 32, 32, 128) == 0    # float32 pool; 32-token blocks
+    assert [rows(1, 16, g * 2, 2, 128) for g in range(1, 9)] == [16, 8, 5, 4, 3, 2, 2, 2]
+    assert rows(1, 16, 18, 2, 128) == 0 and rows(1, 16, 8, 4, 256) == 0 and rows(0, 16, 8, 8, 128) == 0
+    assert rows(1, 16, 8, 2, 64) == 4 and rows(1, 8, 8, 8, 128) == 0
