@@ -219,6 +219,20 @@ typedef struct vx_qweight {
     int n, k;
 } vx_qweight;
 
+/* Load-time repack for decode batches. No counterpart in the reference, whose loader hands GGUF rows to the kernels
+ * as they are (runtime/loader.go:79-200): vx_qweight_pack makes a second copy of a Q4_0 matrix (n % 16 == 0,
+ * k % 256 == 0; VX_ERR_UNSUPPORTED otherwise, nothing changed) whose bytes are the rows' bytes in the order the matrix
+ * cores consume them (18 bytes per 32 elements either way), kept by the backend under the matrix' address until
+ * vx_qweight_unpack, vx_free of the matrix or vx_backend_destroy. While it exists, every quantized matmul entry
+ * point and fused decode block that is given the matrix (by the same data pointer, alone or as part of a Q|K|V or
+ * gate|up group) with 2 .. 32 activation rows streams the packed copy; other row counts read the GGUF rows, which
+ * stay where they are. vx_dequantize_packed: gguf.Dequantize of the packed copy (pkg/gguf/dequant.go:16-56), bit
+ * for bit what vx_dequantize gives for the rows. */
+int vx_qweight_pack(vx_backend *be, const vx_qweight *w);
+int vx_qweight_unpack(vx_backend *be, const vx_qweight *w);
+int vx_qweight_is_packed(vx_backend *be, const vx_qweight *w);
+int vx_dequantize_packed(vx_backend *be, const vx_qweight *w, float *dst);
+
 /* RMSNorm(x, norm_weight) -> Q|K|V projections (one launch) -> RoPE at positions[r] -> rotated Q to
  * q_out [rows,Hq*D], rotated K and V scattered into the pool at slot_mapping[r]
  * (runtime/block.go:834-868). With x_prepared != 0 the normalised activation left prepared by the

@@ -1,0 +1,189 @@
+"""GPU parity of the decode-batch GEMM over load-time packed Q4_0 matrices (vx_qweight_pack): the packed copy
+dequantises to the reference's values bit for bit, the products match the CPU oracle's MatMulQ4_0
+(backend/cpu/cpu.go:842-911) to float32 summation order on every cut of the matrix the planner makes, a row's bits
+do not depend on the batch it sits in, and the fused decode blocks give the oracle's layer with packed weights."""
+import numpy as np
+import pytest
+
+from oracle import numerics as nx
+from oracle import quantize as qz
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def be():
+    from vexel_amd.backend import HipBackend
+    b = HipBackend(0)
+    yield b
+    b.close()
+
+
+def _close(got, want, rtol, atol, what=""):
+    err = np.abs(got.astype(np.float64) - want.astype(np.float64))
+    lim = atol + rtol * np.abs(want.astype(np.float64))
+    assert np.all(err <= lim), "%s: max err %.3e (limit %.3e at worst element)" % (
+        what, err.max(), lim.reshape(-1)[err.argmax()])
+
+
+def _packed(be, w, n, k):
+    dw = be.upload(w, permanent=True)
+    qw = be.qweight(nx.FMT_Q4_0, dw, n, k)
+    assert be.qweight_pack(qw)
+    assert be.qweight_is_packed(qw)
+    return dw, qw
+
+
+@pytest.mark.parametrize("n,k", [(16, 256), (48, 1024), (1040, 512)])
+def test_packed_copy_dequantises_bit_exact(be, n, k):
+    rng = np.random.default_rng(n + k)
+    w = qz.random_quant(nx.FMT_Q4_0, rng, n, k)
+    w.reshape(-1)[2:18] = rng.integers(0, 256, 16, dtype=np.uint8)   # every nibble position carries arbitrary codes
+    dw, qw = _packed(be, w, n, k)
+    dst = be.alloc(n * k * 4)
+    be.dequantize_packed(qw, dst)
+    got = be.download(dst, (n * k,), np.float32)
+    want = nx.dequantize(nx.FMT_Q4_0, w, n * k)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    be.free(dw)
+    assert not be.qweight_is_packed(qw)                          # the copy goes with the matrix
+    be.reset_pool()
+
+
+def test_pack_refuses_other_formats_and_shapes(be):
+    rng = np.random.default_rng(0)
+    w = qz.random_quant(nx.FMT_Q8_0, rng, 32, 256)
+    dw = be.upload(w, permanent=True)
+    assert not be.qweight_pack(be.qweight(nx.FMT_Q8_0, dw, 32, 256))
+    assert not be.qweight_pack(be.qweight(nx.FMT_Q4_0, dw, 24, 256))     # rows not a multiple of 16
+    assert not be.qweight_pack(be.qweight(nx.FMT_Q4_0, dw, 32, 128))     # K not a multiple of 256
+    be.free(dw)
+
+
+# (n, k): one tile; K slices of one and two half chunks per wave; slices with an odd share of half chunks;
+# more tiles than workgroups in a slice; a 7B down-projection's K
+@pytest.mark.parametrize("n,k", [(16, 256), (80, 1024), (96, 2048), (1040, 2304), (4112, 512), (64, 4352), (208, 11008)])
+@pytest.mark.parametrize("m", [2, 5, 16, 17, 32])
+def test_matmul_packed_vs_oracle(be, n, k, m):
+    rng = np.random.default_rng(n * 7 + k + m)
+    w = qz.random_quant(nx.FMT_Q4_0, rng, n, k)
+    a = (rng.standard_normal((m, k)) * (1.0 + 3.0 * (rng.random((1, k)) < 0.1))).astype(np.float32)
+    want = nx.matmul_quant(nx.FMT_Q4_0, a, w, m, n, k)
+    dw, qw = _packed(be, w, n, k)
+    da = be.upload(a)
+    dout = be.alloc(m * n * 4)
+    be.matmul_q4_0(da, dw, dout, m, n, k)
+    got = be.download(dout, (m, n), np.float32)
+    scale = np.abs(want).max()
+    _close(got, want, 2e-5, 2e-6 * scale + 1e-7, "packed matmul %dx%dx%d" % (m, n, k))
+    # the unpacked path on the same inputs: float32 summation order apart
+    be.qweight_unpack(qw)
+    be.matmul_q4_0(da, dw, dout, m, n, k)
+    plain = be.download(dout, (m, n), np.float32)
+    _close(got, plain, 0, 3e-6 * scale + 1e-7, "packed vs unpacked")
+    be.free(dw)
+    be.reset_pool()
+
+
+def test_matmul_packed_rows_independent_of_batch(be):
+    """A row has the same bits in a batch of 2, of 16, of 17 and of 32 rows (the cut of the matrix depends on its
+    shape and the device only; 16 rows and fewer run the one-tile form of the kernel)."""
+    rng = np.random.default_rng(11)
+    n, k = 208, 4096
+    w = qz.random_quant(nx.FMT_Q4_0, rng, n, k)
+    a = rng.standard_normal((32, k)).astype(np.float32)
+    dw, qw = _packed(be, w, n, k)
+    da = be.upload(a)
+
+    def batch(first, rows):
+        d = be.alloc(rows * n * 4)
+        be.matmul_quant(nx.FMT_Q4_0, da + first * k * 4, dw, d, None, rows, n, k)
+        return be.download(d, (rows, n), np.float32)
+
+    full = batch(0, 32)
+    for first, rows in ((0, 2), (5, 2), (30, 2), (0, 16), (3, 17), (16, 16), (9, 7)):
+        part = batch(first, rows)
+        assert np.array_equal(part.view(np.uint32), full[first:first + rows].view(np.uint32)), (first, rows)
+    res = rng.standard_normal((32, n)).astype(np.float32)
+    dres, d = be.upload(res), be.alloc(32 * n * 4)
+    be.matmul_quant(nx.FMT_Q4_0, da, dw, d, dres, 32, n, k)
+    assert np.array_equal(be.download(d, (32, n), np.float32).view(np.uint32), (res + full).view(np.uint32))
+    be.free(dw)
+    be.reset_pool()
+
+
+def test_rewriting_the_matrix_drops_the_packed_copy(be):
+    rng = np.random.default_rng(5)
+    n, k, m = 64, 512, 8
+    w1, w2 = qz.random_quant(nx.FMT_Q4_0, rng, n, k), qz.random_quant(nx.FMT_Q4_0, rng, n, k)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    dw, qw = _packed(be, w1, n, k)
+    da, dout = be.upload(a), be.alloc(m * n * 4)
+    be.to_device(dw, w2)                                         # new rows under the same address
+    assert not be.qweight_is_packed(qw)
+    be.matmul_q4_0(da, dw, dout, m, n, k)
+    want = nx.matmul_quant(nx.FMT_Q4_0, a, w2, m, n, k)
+    _close(be.download(dout, (m, n), np.float32), want, 2e-5, 2e-6 * np.abs(want).max() + 1e-7, "after rewrite")
+    be.free(dw)
+    be.reset_pool()
+
+
+@pytest.mark.parametrize("rows", [2, 7, 32])
+@pytest.mark.parametrize("hq,hk,d,hidden,ffn", [(8, 8, 64, 512, 1024), (8, 2, 128, 1024, 2816), (32, 32, 128, 4096, 1024)])
+def test_fused_decode_blocks_with_packed_weights(be, rows, hq, hk, d, hidden, ffn):
+    """RMSNorm -> Q|K|V -> RoPE -> KV store (one launch with the table of angles) and Wo -> residual -> RMSNorm ->
+    gate|up -> SiLU*up -> down -> residual on packed weights against the oracle's operators."""
+    rng = np.random.default_rng(rows + hq + hidden)
+    bs, nblocks, theta, eps = 16, 8, 10000.0, 1e-5
+    qd, kvd = hq * d, hk * d
+    mk = lambda n, k: qz.quantize_q4_0((rng.standard_normal((n, k)) * 0.05).astype(np.float32)).reshape(-1)
+    raw = {"wq": (mk(qd, hidden), qd, hidden), "wk": (mk(kvd, hidden), kvd, hidden), "wv": (mk(kvd, hidden), kvd, hidden),
+           "wo": (mk(hidden, qd), hidden, qd), "w1": (mk(ffn, hidden), ffn, hidden), "w3": (mk(ffn, hidden), ffn, hidden),
+           "w2": (mk(hidden, ffn), hidden, ffn)}
+    dev, qws = {}, {}
+    for name, (w, n, k) in raw.items():
+        dev[name], qws[name] = _packed(be, w, n, k)
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    nw_attn = (1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    nw_ffn = (1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    positions = rng.integers(0, 100, rows).astype(np.int32)
+    slots = rng.permutation(nblocks * bs)[:rows].astype(np.int32)
+    per_block = 2 * bs * kvd
+    pool0 = nx.f32_to_f16_array(rng.standard_normal(nblocks * per_block).astype(np.float32))
+
+    # oracle
+    h = nx.rmsnorm(x, nw_attn, rows, hidden, eps)
+    q = nx.matmul_quant(nx.FMT_Q4_0, h, raw["wq"][0], rows, qd, hidden)
+    kk = nx.matmul_quant(nx.FMT_Q4_0, h, raw["wk"][0], rows, kvd, hidden)
+    vv = nx.matmul_quant(nx.FMT_Q4_0, h, raw["wv"][0], rows, kvd, hidden)
+    want_q, want_k = nx.rope_positions(q, kk, d, hq, hk, positions, d, theta, False)
+    attn = rng.standard_normal((rows, qd)).astype(np.float32)
+    x1 = nx.add(x, nx.matmul_quant(nx.FMT_Q4_0, attn, raw["wo"][0], rows, hidden, qd))
+    h2 = nx.rmsnorm(x1, nw_ffn, rows, hidden, eps)
+    g = nx.matmul_quant(nx.FMT_Q4_0, h2, raw["w1"][0], rows, ffn, hidden)
+    u = nx.matmul_quant(nx.FMT_Q4_0, h2, raw["w3"][0], rows, ffn, hidden)
+    want_x = nx.add(x1, nx.matmul_quant(nx.FMT_Q4_0, nx.silu_mul(g, u), raw["w2"][0], rows, hidden, ffn))
+
+    # GPU
+    dx, dnw, dnf = be.upload(x, permanent=True), be.upload(nw_attn, permanent=True), be.upload(nw_ffn, permanent=True)
+    dpos, dslots = be.upload(positions, permanent=True), be.upload(slots, permanent=True)
+    dpool, dq = be.upload(pool0, permanent=True), be.alloc_permanent(rows * qd * 4)
+    be.rope_table_prepare(dpos, rows, d, theta)
+    be.decode_attn_qkv(dx, dnw, eps, False, qws["wq"], qws["wk"], qws["wv"], rows, dpos, dslots, dpool, True, hq, hk, d, bs,
+                       theta, dq)
+    got_q = be.download(dq, (rows, qd), np.float32)
+    _close(got_q, want_q, 2e-4, 2e-5 * np.abs(want_q).max(), "Q")
+    pool = nx.f16_to_f32_array(be.download(dpool, (nblocks * per_block,), np.uint16))
+    for r in range(rows):
+        blk, off = divmod(int(slots[r]), bs)
+        gk = pool[blk * per_block + off * kvd: blk * per_block + (off + 1) * kvd]
+        gv = pool[blk * per_block + bs * kvd + off * kvd: blk * per_block + bs * kvd + (off + 1) * kvd]
+        _close(gk, nx.f16_to_f32_array(nx.f32_to_f16_array(want_k[r])), 2e-3, 2e-3 * np.abs(want_k).max(), "K row %d" % r)
+        _close(gv, nx.f16_to_f32_array(nx.f32_to_f16_array(vv[r])), 2e-3, 2e-3 * np.abs(vv).max(), "V row %d" % r)
+    dattn = be.upload(attn, permanent=True)
+    be.decode_ffn(dattn, dx, qws["wo"], dnf, eps, qws["w1"], qws["w3"], qws["w2"], rows)
+    got_x = be.download(dx, (rows, hidden), np.float32)
+    _close(got_x, want_x, 2e-4, 2e-5 * np.abs(want_x).max(), "layer output")
+    for p in list(dev.values()) + [dx, dnw, dnf, dpos, dslots, dpool, dq, dattn]:
+        be.free(p)
+    be.reset_pool()

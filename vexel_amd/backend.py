@@ -276,6 +276,23 @@ class HipBackend:
         """vx_qweight for the fused decode entry points (data: device pointer of the raw blocks)."""
         return VxQWeight(fmt, data, n, k)
 
+    def qweight_pack(self, w):
+        """vx_qweight_pack: True when a packed copy was made, False when the format or shape has none."""
+        rc = self._lib.vx_qweight_pack(self._h, C.byref(w))
+        if rc == _l.VX_ERR_UNSUPPORTED:
+            return False
+        self._ck(rc)
+        return True
+
+    def qweight_unpack(self, w):
+        self.call("vx_qweight_unpack", C.byref(w))
+
+    def qweight_is_packed(self, w):
+        return bool(self._lib.vx_qweight_is_packed(self._h, C.byref(w)))
+
+    def dequantize_packed(self, w, dst):
+        self.call("vx_dequantize_packed", C.byref(w), dst)
+
     def decode_attn_qkv_supported(self, wq, wk, wv, head_dim):
         return bool(self._lib.vx_decode_attn_qkv_supported(C.byref(wq), C.byref(wk), C.byref(wv), head_dim))
 

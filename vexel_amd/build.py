@@ -12,7 +12,7 @@ HOST_LIB = os.path.join(HERE, "libvexel_host.so")
 SYNTH_LIB = os.path.join(HERE, "libvexel_synth.so")
 OBJ_DIR = os.path.join(HERE, "build")
 
-SOURCES = ["backend.hip", "elementwise.hip", "attention.hip", "qgemm.hip", "qmatvec.hip", "pack.hip", "sampler.hip", "medusa.hip"]
+SOURCES = ["backend.hip", "elementwise.hip", "attention.hip", "qgemm.hip", "qstream.hip", "qmatvec.hip", "pack.hip", "sampler.hip", "medusa.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-fvisibility=default",

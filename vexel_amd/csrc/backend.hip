@@ -106,6 +106,7 @@ void vx_backend_destroy(vx_backend *be) {
     if (!be) return;
     (void)hipSetDevice(be->device);
     (void)hipStreamSynchronize(be->stream);
+    stream_drop_all(be);
     for (auto &c : be->chunks) (void)hipFree(c.base);
     for (auto &kv : be->permanent) (void)hipFree(kv.first);
     if (be->gemm_ws) (void)hipFree(be->gemm_ws);
@@ -179,6 +180,7 @@ void vx_free(vx_backend *be, void *ptr) {
     if (it == be->permanent.end()) return;  // pool buffer: recycled by vx_reset_pool
     items_written(be, ptr, it->second);
     (void)hipStreamSynchronize(be->stream);
+    stream_drop_packed(be, ptr);  // a packed copy of a matrix that started here goes with it
     (void)hipFree(ptr);
     be->permanent.erase(it);
 }

@@ -62,6 +62,10 @@ struct vx_backend {
     // permanent allocations (vx_alloc_permanent / vx_free)
     std::unordered_map<void *, size_t> permanent;
 
+    // load-time repacked copies of quantized matrices for the decode-batch GEMM (qstream.hip), keyed by the raw
+    // matrix' device address; each value is that file's record of the copy
+    std::unordered_map<const void *, void *> packed;
+
     // library-owned scratch, grown on demand outside graph capture; scratch_gen counts the reallocations
     // (a captured graph holds the old addresses)
     uint64_t scratch_gen = 0;
@@ -125,11 +129,18 @@ struct vx_graph {
 
 namespace vx {
 
+// qstream.hip: drops the packed copy of the raw matrix at `raw` (if any) / every packed copy of the backend / the
+// copies of matrices that [dst, dst + bytes) overlaps.
+void stream_drop_packed(vx_backend *be, const void *raw);
+void stream_drop_all(vx_backend *be);
+void stream_written(vx_backend *be, const void *dst, size_t bytes);
+
 constexpr int ATTN_TPW = 512;  // tokens of one (sequence, kv head) that one attention workgroup takes
 
 // Drops the attention work list when [dst, dst + bytes) overlaps the kv_lens array it was built from.
 inline void items_written(vx_backend *be, const void *dst, size_t bytes) {
     be->write_epoch++;  // the library wrote into a caller's buffer: a kept RoPE table may describe other positions now
+    if (!be->packed.empty()) stream_written(be, dst, bytes);  // a packed copy of rewritten rows is stale
     if (!be->items.valid) return;
     const char *a = (const char *)dst, *k = (const char *)be->items.kv_lens;
     if (a < k + (size_t)be->items.batch * 4 && k < a + bytes) be->items.valid = false;

@@ -39,6 +39,7 @@
 #include <algorithm>
 
 #include "prep_tiles.h"
+#include "qgemm_shared.h"
 
 using namespace vx;
 
@@ -1295,48 +1296,11 @@ __global__ void __launch_bounds__(PREP_THREADS) merge_prepare_kernel(const float
 // a row to arrive adds the partials in chunk order (so the result does not depend on who arrives last) and
 // writes the row factor 1/rms; nobody waits for anybody. The prepared values are x*w (not yet divided by rms)
 // scaled per chunk; the GEMM multiplies each chunk's dot product by cscale and the row's result by inv_scale.
-// The sums of squares of a row's chunks, from which whoever consumes the activation's products takes 1/rms.
-struct RowNorm {
-    const float *sspart;  // [VX_PREP_SYNC_CHUNKS][VX_PREP_SYNC_ROWS], NULL when the rows carry no pending RMSNorm
-    int n_chunks;
-    float inv_k, eps;
-};
-
-__device__ __forceinline__ float wave_sum(float v) {
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
-
-// Factor of row r's finished dot products: the stored row factor times, for a pending RMSNorm, 1/rms from the
-// chunks' sums of squares (added by a fixed butterfly over the wave, so every caller gets the same bits).
-// Must be called by all 64 lanes of a wave.
-__device__ __forceinline__ float row_factor(const float *__restrict__ inv_rows, const RowNorm &rn, int r) {
-    float f = inv_rows[r];
-    if (rn.sspart) {
-        const int lane = threadIdx.x & 63;
-        const float ss = wave_sum(lane < rn.n_chunks ? rn.sspart[lane * VX_PREP_SYNC_ROWS + r] : 0.f);
-        const float rms = (float)sqrt((double)(ss * rn.inv_k + rn.eps));  // backend/cpu/cpu.go:214
-        f = f / rms;
-    }
-    return f;
-}
-
 // Writes inv_scale[r] *= 1/rms for every row, for consumers that read plain row factors. grid = rows, block = 64.
 __global__ void __launch_bounds__(64) finalize_row_norm_kernel(float *__restrict__ inv_rows, RowNorm rn) {
     const float f = row_factor(inv_rows, rn, blockIdx.x);
     if (threadIdx.x == 0) inv_rows[blockIdx.x] = f;
 }
-
-// What the Q|K|V launch needs to finish its rows itself (RoPE, the rotated Q to q_out, K and V into the paged
-// pool: rope_store_partials_kernel's work) when one K slice holds the whole sum. q_out == NULL: not in use.
-struct QkvEpi {
-    float *q_out;
-    void *pool;
-    const int32_t *slots;
-    const float2 *cs_tab;  // [row][head_dim / 2] (cos, sin) of the row's position
-    RowNorm rn;
-    int qd, kvd, head_dim, block_size, pool_f16;
-};
 
 #include "qgemm_wave.h"
 
@@ -1921,6 +1885,25 @@ int launch_gemm_rows_r(vx_backend *be, const WavePlan &pl, const Segs &segs, int
 
 int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out, const float *residual,
                     bool to_partials, int M, int K, int *ks_out, const QkvEpi *epi_in = nullptr) {
+    // packed copies of the matrices (vx_qweight_pack) and a decode-sized batch: the streaming kernel
+    const bool fin = epi_in && epi_in->q_out;
+    if (stream_gemm_ok(be, fmt, segs.w, segs.n_end, 3, N, K, M, fin)) {
+        int ks = 1;
+        const int mpad = mpad_for(M);
+        const PrepView spv = prep_view(be, mpad, K);
+        int rc = stream_gemm(be, fmt, segs.w, segs.n_end, 3, N, K, M, mpad, spv, epi_in, &ks);
+        if (rc != VX_ERR_UNSUPPORTED) {
+            if (rc) return rc;
+            if (ks_out) *ks_out = ks;
+            if (!fin && !to_partials) {
+                const size_t total = (size_t)M * N;
+                qgemm_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const float *)be->part_ws, spv.inv_scale, out,
+                                                                                              residual, M, N, ks);
+                VX_CHECK_LAUNCH();
+            }
+            return VX_OK;
+        }
+    }
     const WavePlan rp = rows_plan(be, fmt, segs, N, K, M);
     if (rp.r > 0) {
         return launch_gemm_rows_r<WQ8_0>(be, rp, segs, N, out, residual, to_partials, M, K, ks_out);
@@ -2319,7 +2302,8 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
         const bool table = be->rope_tab_pos == positions && be->rope_tab_rows >= rows && be->rope_tab_dim == head_dim &&
                            be->rope_tab_theta == theta && be->rope_tab_epoch == be->write_epoch;
         static const bool no_epi = getenv("VEXEL_HIP_NO_QKV_EPILOGUE") != nullptr;
-        if (!no_epi && !gen && table && pl.r > 0 && pl.ks == 1 && mpad_for(rows) <= 32 && (head_dim & (head_dim - 1)) == 0 &&
+        const bool one_launch = (pl.r > 0 && pl.ks == 1) || stream_gemm_ok(be, wq->fmt, segs.w, segs.n_end, 3, ntot, k, rows, true);
+        if (!no_epi && !gen && table && one_launch && mpad_for(rows) <= 32 && (head_dim & (head_dim - 1)) == 0 &&
             head_dim >= 4 && ((uintptr_t)kv_pool % 16) == 0 && ((uintptr_t)q_out % 16) == 0) {
             QkvEpi epi;
             epi.q_out = q_out;

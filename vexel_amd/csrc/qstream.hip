@@ -1,0 +1,602 @@
+// Decode-batch GEMM (2 .. 32 activation rows) over Q4_0 weights repacked at load time into the order the matrix
+// cores consume them: C[M,N] = A[M,K] * B^T with B [N,K] as backend.go:47-52 (MatMulQ4_0) has it, the arithmetic
+// of backend/cpu/cpu.go:842-911 up to float32 summation order.
+//
+// Packed layout (vx_qweight_pack): the matrix is cut into tiles of 16 rows and half chunks of 128 columns. One
+// (tile, half chunk) is a unit of 1152 bytes, units of a tile follow one another along K:
+//   bytes [0, 1024): lane l = 16 * g + r of a wave owns 16 bytes, dword j of them the eight 4-bit codes of row r's
+//     block 4 * hc + j that lane group g feeds to the matrix core: nibble i of the dword is block element
+//     ELT[g][SLOT[i]] (the slot order of the prepared activation tiles, prep_tiles.h), so that two masks, one shift
+//     and four packed f16 operations turn the dword into the operand;
+//   bytes [1024, 1152): row r's four f16 block scales at 1024 + 8 r.
+// The bytes are a permutation of the GGUF rows' bytes (18 per 32 elements either way); vx_dequantize_packed gives
+// back gguf.DequantizeQ4_0's values bit for bit (pkg/gguf/dequant.go:16-56).
+//
+// Kernel: one workgroup of eight waves per compute unit owns a range of tiles and one K slice. Wave w keeps the
+// activation operand of half chunk h0 + w (and h0 + 8 + w) of the slice in registers for the whole pass and streams
+// the weight units of those half chunks through them, tile after tile, from a ring of requests that runs ahead of
+// the arithmetic: a unit goes from memory to registers with one 16-byte and one 8-byte load per lane and nowhere
+// else. Per 32-column step: 9 vector instructions unpack the codes to exact integers in f16, four
+// v_mfma_f32_16x16x32_f16 multiply them with the hi and lo halves of two activation tiles, 8 fused multiply-adds
+// apply the block scale. After every RG tiles the eight waves' sums meet in LDS and are added in wave order. A slice
+// wider than 16 half chunks is walked in passes of 16 (the sums wait in LDS), which is how the Q|K|V launch
+// keeps the whole K in one workgroup and finishes its rows itself (RoPE, K/V store).
+// Which tiles and half chunks a workgroup takes depends on (N, K, device, epilogue) only and every sum is added in
+// a fixed order, so a row has the same bits in any batch of 2 .. 32 rows.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+
+#include "common.h"
+#include "qgemm_shared.h"
+
+using namespace vx;
+
+namespace {
+
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr int HUNIT = 1152;      // bytes of one (tile, half chunk)
+constexpr int NW = 8;            // waves per workgroup
+constexpr int ACC_TILES = 8;     // tiles whose sums can wait in LDS between the passes of a wide slice
+
+// block element held by slot i of lane group g (the prepared tiles' order), and the slot that nibble j feeds
+__host__ __device__ inline int elt_of(int g, int slot) {
+    const int base[8] = {0, 2, 16, 18, 1, 3, 17, 19};
+    return 4 * g + base[slot];
+}
+__host__ __device__ inline int slot_of_nibble(int j) { return j < 4 ? 2 * j : 2 * (j - 4) + 1; }
+
+__device__ __forceinline__ half2v as_h2(uint32_t u) {
+    half2v v;
+    __builtin_memcpy(&v, &u, 4);
+    return v;
+}
+__device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t k) {
+    uint32_t r;
+    asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "s"(mask), "v"(k));
+    return r;
+}
+// A load through the global address space (pointers that arrive inside a by-value kernel argument are generic, and
+// a generic load also waits on the LDS counter), and a pointer known to be the same in every lane.
+template <class T> __device__ __forceinline__ T gload(const void *p) {
+    return *(const __attribute__((address_space(1))) T *)(uintptr_t)p;
+}
+__device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
+    const uint64_t v = (uint64_t)(uintptr_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const uint8_t *)(uintptr_t)(((uint64_t)hi << 32) | lo);
+}
+
+// Eight nibbles of one dword -> the step's operand: exact integers q - 8 as f16. A nibble under 0x6400's exponent is
+// the f16 1024 + q; one four bits higher is 1024 + 16 q, which one fused multiply-add brings to q - 8 as well.
+__device__ __forceinline__ half8 unpack_q4(uint32_t w, uint32_t k64) {
+    const uint32_t w8 = w >> 8;
+    const half2v a = as_h2(and_or(w, 0x000F000Fu, k64)), b = as_h2(and_or(w, 0x00F000F0u, k64));
+    const half2v c = as_h2(and_or(w8, 0x000F000Fu, k64)), d = as_h2(and_or(w8, 0x00F000F0u, k64));
+    const half2v m1032 = {(_Float16)-1032.f, (_Float16)-1032.f}, m72 = {(_Float16)-72.f, (_Float16)-72.f};
+    const half2v s16 = {(_Float16)0.0625f, (_Float16)0.0625f};
+    const half2v h0 = a + m1032, h1 = b * s16 + m72, h2 = c + m1032, h3 = d * s16 + m72;
+    half8 r;
+    r[0] = h0[0]; r[1] = h0[1]; r[2] = h1[0]; r[3] = h1[1];
+    r[4] = h2[0]; r[5] = h2[1]; r[6] = h3[0]; r[7] = h3[1];
+    return r;
+}
+
+// ------------------------------------------------------------------------------------------------ pack / unpack
+// grid = (tiles, half chunks), block = 64: lane l writes its 16 code bytes, lanes 0 .. 15 their row's scales.
+__global__ void __launch_bounds__(64) pack_q4_0_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ packed, int n_hc) {
+    const int T = blockIdx.x, hc = blockIdx.y, lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+    const size_t row_bytes = (size_t)n_hc * 4 * 18;
+    const uint8_t *row = raw + (size_t)(T * 16 + r) * row_bytes + (size_t)hc * 4 * 18;
+    uint8_t *u = packed + ((size_t)T * n_hc + hc) * HUNIT;
+    uint32_t out[4];
+    for (int j = 0; j < 4; j++) {
+        const uint8_t *blk = row + j * 18;
+        uint32_t w = 0;
+        for (int nib = 0; nib < 8; nib++) {
+            const int e = elt_of(g, slot_of_nibble(nib));
+            const uint32_t q = e < 16 ? (blk[2 + e] & 0xFu) : (blk[2 + e - 16] >> 4);
+            w |= q << (4 * nib);
+        }
+        out[j] = w;
+    }
+    *(u32x4 *)(u + lane * 16) = (u32x4){out[0], out[1], out[2], out[3]};
+    if (g == 0) {
+        uint16_t d[4];
+        for (int j = 0; j < 4; j++) d[j] = (uint16_t)(row[j * 18] | (row[j * 18 + 1] << 8));
+        *(u32x2 *)(u + 1024 + r * 8) = (u32x2){(uint32_t)d[0] | ((uint32_t)d[1] << 16), (uint32_t)d[2] | ((uint32_t)d[3] << 16)};
+    }
+}
+
+// One thread per element: scale * float32(q - 8) as gguf.DequantizeQ4_0 computes it, read from the packed form.
+__global__ void __launch_bounds__(256) dequant_packed_q4_0_kernel(const uint8_t *__restrict__ packed, float *__restrict__ dst, int n,
+                                                                  int k) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)n * k) return;
+    const int row = (int)(idx / k), col = (int)(idx % k);
+    const int T = row >> 4, r = row & 15, hc = col >> 7, j = (col >> 5) & 3, e = col & 31;
+    const int n_hc = k >> 7;
+    const uint8_t *u = packed + ((size_t)T * n_hc + hc) * HUNIT;
+    int g = 0, nib = 0;
+    for (int gg = 0; gg < 4; gg++)
+        for (int i = 0; i < 8; i++)
+            if (elt_of(gg, slot_of_nibble(i)) == e) {
+                g = gg;
+                nib = i;
+            }
+    const uint32_t w = *(const uint32_t *)(u + (g * 16 + r) * 16 + j * 4);
+    const int q = (int)((w >> (4 * nib)) & 0xFu);
+    _Float16 d;
+    __builtin_memcpy(&d, u + 1024 + r * 8 + j * 2, 2);
+    dst[idx] = __fmul_rn((float)d, (float)(q - 8));
+}
+
+// ------------------------------------------------------------------------------------------------ the GEMM
+// First unit of tile T among up to three packed matrices (all arguments the same in every lane). A plain function of
+// values: the same selection written over a lambda's captures is compiled into an indexed load of the closure
+// object, which then lives in scratch memory.
+__device__ __forceinline__ const uint8_t *tile_base(int T, const uint8_t *w0, const uint8_t *w1, const uint8_t *w2, int e0, int e1,
+                                                    size_t tile_stride) {
+    uint64_t b = (uint64_t)(uintptr_t)w0;
+    int local = T;
+    if (T >= e0) {
+        b = (uint64_t)(uintptr_t)w1;
+        local = T - e0;
+    }
+    if (T >= e1) {
+        b = (uint64_t)(uintptr_t)w2;
+        local = T - e1;
+    }
+    return (const uint8_t *)(uintptr_t)(b + (uint64_t)local * tile_stride);
+}
+
+struct PackedSegs {  // up to three packed matrices whose rows follow one another in the output
+    const uint8_t *w[3];
+    int t_end[3];  // tiles before the end of each
+};
+
+template <int MT> struct APhase {
+    half8 h[4][MT], l[4][MT];
+    float4v cs[MT];
+};
+struct WHalf {
+    u32x4 c;
+    u32x2 s;
+};
+
+struct StreamShape {
+    int M, Mpad, N, n_hc, npass, t_end0, t_end1;
+};
+
+// grid = (row groups, K slices), block = 512. PH: half chunks a wave holds per pass (1 or 2); RG: tiles per
+// reduction; EPI: finish Q|K|V rows (one slice).
+template <int PH, int RG, int MT, bool EPI>
+__global__ void __launch_bounds__(64 * NW, 1)
+qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, const uint8_t *__restrict__ pw2,
+               const half8 *__restrict__ a_tiles, const float *__restrict__ a_cscale, const float *__restrict__ a_inv_scale,
+               float *__restrict__ partial, const StreamShape a, const QkvEpi epi) {
+    constexpr int D = RG * PH;            // requests in flight per wave
+    constexpr int TP = 16 * RG + 4;       // floats per row of a wave's block in LDS
+    __shared__ __attribute__((aligned(16))) float red[2][NW][16 * MT * TP];
+    __shared__ __attribute__((aligned(16))) float wait_sums[EPI ? ACC_TILES * 16 * 16 * MT : 4];
+    __shared__ float s_fac[16 * MT];
+
+    const int tid = threadIdx.x, lane = tid & 63, ln = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n_tiles = a.N >> 4, mtiles = a.Mpad >> 4, n_hc = a.n_hc;
+    const int gb = n_tiles / (int)gridDim.x, gr = n_tiles % (int)gridDim.x;
+    const int t0 = blockIdx.x * gb + min((int)blockIdx.x, gr), nt = gb + ((int)blockIdx.x < gr ? 1 : 0);
+    const int sb = n_hc / (int)gridDim.y, sr = n_hc % (int)gridDim.y;
+    const int h0 = blockIdx.y * sb + min((int)blockIdx.y, sr), nh = sb + ((int)blockIdx.y < sr ? 1 : 0);
+
+    const size_t tile_stride = (size_t)n_hc * HUNIT;
+    const int lane_c = lane * 16, lane_s = 1024 + ln * 8;
+    // the packed matrices' addresses and tile ends as scalars (the same in every lane)
+    // (through readfirstlane: selecting among plain kernel arguments becomes an indexed load of the argument
+    // block, copied to scratch memory for it)
+    const uint8_t *const w0 = uniform_ptr(pw0), *const w1 = uniform_ptr(pw1), *const w2 = uniform_ptr(pw2);
+    const int e0 = __builtin_amdgcn_readfirstlane(a.t_end0), e1 = __builtin_amdgcn_readfirstlane(a.t_end1);
+    uint32_t k64;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(k64));
+
+    if (EPI) {
+        // row factors with the pending 1/rms of the RMSNorm that fed the activation: whole-wave computations
+        for (int r = wave; r < 16 * MT; r += NW) {
+            const float f = row_factor(a_inv_scale, epi.rn, r);
+            if (lane == 0) s_fac[r] = f;
+        }
+    }
+
+    int buf = 0;
+    for (int pass = 0; pass < a.npass; pass++) {
+        const int hp = h0 + pass * NW * PH, nhp = min(nh - pass * NW * PH, NW * PH);  // this pass's half chunks
+        // (separate scalars, not arrays: an array indexed in an unrolled loop can end up in scratch memory)
+        const bool valid0 = wave < nhp, valid1 = PH > 1 && NW + wave < nhp;
+        const int hc0 = hp + min(wave, nhp - 1), hc1 = hp + min(NW + wave, nhp - 1);
+        auto ldw = [&](int tile, int p) __attribute__((always_inline)) {
+            const uint8_t *u = uniform_ptr(tile_base(t0 + min(tile, nt - 1), w0, w1, w2, e0, e1, tile_stride) + (size_t)(p == 0 ? hc0 : hc1) * HUNIT);
+            WHalf x;
+            x.c = gload<u32x4>(u + lane_c);
+            x.s = gload<u32x2>(u + lane_s);
+            return x;
+        };
+        APhase<MT> A[PH];
+#pragma unroll
+        for (int p = 0; p < PH; p++) {
+            const int hc = p == 0 ? hc0 : hc1;
+            const half8 *base = a_tiles + ((size_t)(hc * 4) * mtiles * 2) * 64 + lane;
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    A[p].h[j][t] = gload<half8>(base + ((size_t)(j * mtiles + t) * 2 + 0) * 64);
+                    A[p].l[j][t] = gload<half8>(base + ((size_t)(j * mtiles + t) * 2 + 1) * 64);
+                }
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+                A[p].cs[t] = gload<float4v>(a_cscale + (size_t)(hc >> 1) * a.Mpad + t * 16 + 4 * g);
+        }
+        WHalf ring[D];
+#pragma unroll
+        for (int i = 0; i < D; i++) ring[i] = ldw(i / PH, i % PH);
+
+        for (int tb = 0; tb < nt; tb += RG) {
+            float4v acc[RG][MT];
+#pragma unroll
+            for (int r = 0; r < RG; r++) {
+#pragma unroll
+                for (int m = 0; m < MT; m++) acc[r][m] = (float4v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int p = 0; p < PH; p++) {
+                    const WHalf x = ring[r * PH + p];
+                    ring[r * PH + p] = ldw(tb + RG + r, p);
+                    if (p == 0 ? valid0 : valid1) {
+                        float4v tmp[MT];
+#pragma unroll
+                        for (int m = 0; m < MT; m++) tmp[m] = (float4v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const half8 wb = unpack_q4(x.c[j], k64);
+                            const uint32_t sw = x.s[j >> 1];
+                            _Float16 dh;
+                            const uint16_t d16 = (uint16_t)((j & 1) ? (sw >> 16) : (sw & 0xFFFFu));
+                            __builtin_memcpy(&dh, &d16, 2);
+                            const float d = (float)dh;
+                            float4v P[MT];
+#pragma unroll
+                            for (int m = 0; m < MT; m++)
+                                P[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[p].h[j][m], wb, (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                            for (int m = 0; m < MT; m++) P[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[p].l[j][m], wb, P[m], 0, 0, 0);
+#pragma unroll
+                            for (int m = 0; m < MT; m++)
+#pragma unroll
+                                for (int e = 0; e < 4; e++) tmp[m][e] = __builtin_fmaf(d, P[m][e], tmp[m][e]);
+                        }
+#pragma unroll
+                        for (int m = 0; m < MT; m++)
+#pragma unroll
+                            for (int e = 0; e < 4; e++) acc[r][m][e] = __builtin_fmaf(A[p].cs[m][e], tmp[m][e], acc[r][m][e]);
+                    }
+                }
+            }
+            // the waves' sums of these RG tiles: lane (g, ln) of tile r holds C[16 m + 4 g + e][16 r + ln]
+            float *T = &red[buf][wave][0];
+#pragma unroll
+            for (int r = 0; r < RG; r++)
+#pragma unroll
+                for (int m = 0; m < MT; m++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) T[(m * 16 + 4 * g + e) * TP + r * 16 + ln] = acc[r][m][e];
+            __syncthreads();
+            const int ntile = min(RG, nt - tb);
+            constexpr int F4 = 16 * MT * RG * 4;  // float4 groups of a full block
+#pragma unroll
+            for (int f0 = 0; f0 < F4; f0 += 64 * NW) {
+                const int f = f0 + tid;
+                const int ml = f / (RG * 4), nl = (f % (RG * 4)) * 4;
+                if (f < F4 && nl < ntile * 16) {
+                    float4 c = *(const float4 *)(&red[buf][0][0] + ml * TP + nl);
+#pragma unroll
+                    for (int w = 1; w < NW; w++) {
+                        const float4 d = *(const float4 *)(&red[buf][w][0] + ml * TP + nl);
+                        c.x += d.x; c.y += d.y; c.z += d.z; c.w += d.w;
+                    }
+                    if (!EPI) {
+                        if (ml < a.M)
+                            *(float4 *)(partial + ((size_t)blockIdx.y * a.M + ml) * a.N + (size_t)(t0 + tb) * 16 + nl) = c;
+                    } else {
+                        // sums of the earlier passes wait in LDS, [tile][row][16 columns]
+                        float4 *ws = (float4 *)(wait_sums + ((size_t)(tb * 16 * MT + ml * RG) * 16 + nl));
+                        if (a.npass > 1) {
+                            if (pass > 0) {
+                                const float4 p = *ws;
+                                c.x += p.x; c.y += p.y; c.z += p.z; c.w += p.w;
+                            }
+                            if (pass + 1 < a.npass) *ws = c;
+                        }
+                        if (pass + 1 == a.npass && ml < a.M) {
+                            // columns n .. n+3 of row m: two RoPE pairs of a Q or K head, or four V values
+                            // (the arithmetic of rope_store_partials_kernel)
+                            const int m = ml, n = (t0 + tb) * 16 + nl;
+                            const float inv = s_fac[ml];
+                            const float a0 = __fmul_rn(c.x, inv), b0 = __fmul_rn(c.y, inv), a1 = __fmul_rn(c.z, inv), b1 = __fmul_rn(c.w, inv);
+                            const bool is_q = n < epi.qd, is_v = n >= epi.qd + epi.kvd;
+                            const int o = is_q ? n : (is_v ? n - epi.qd - epi.kvd : n - epi.qd);
+                            float4 r4 = make_float4(a0, b0, a1, b1);
+                            if (!is_v) {
+                                const float2 *cs = epi.cs_tab + (size_t)m * (epi.head_dim >> 1) + ((o & (epi.head_dim - 1)) >> 1);
+                                const float2 c0 = cs[0], c1 = cs[1];
+                                r4.x = __fsub_rn(__fmul_rn(a0, c0.x), __fmul_rn(b0, c0.y));
+                                r4.y = __fadd_rn(__fmul_rn(a0, c0.y), __fmul_rn(b0, c0.x));
+                                r4.z = __fsub_rn(__fmul_rn(a1, c1.x), __fmul_rn(b1, c1.y));
+                                r4.w = __fadd_rn(__fmul_rn(a1, c1.y), __fmul_rn(b1, c1.x));
+                            }
+                            if (is_q) {
+                                *(float4 *)(epi.q_out + (size_t)m * epi.qd + o) = r4;
+                            } else {
+                                const int slot = epi.slots[m], blk = slot / epi.block_size, off = slot - blk * epi.block_size;
+                                const size_t part = (size_t)epi.block_size * epi.kvd;
+                                const size_t at = (size_t)blk * 2 * part + (size_t)off * epi.kvd + (is_v ? part : 0) + o;
+                                if (epi.pool_f16) {
+                                    typedef _Float16 half4w __attribute__((ext_vector_type(4)));
+                                    const half4w h4 = {(_Float16)r4.x, (_Float16)r4.y, (_Float16)r4.z, (_Float16)r4.w};
+                                    *(half4w *)((_Float16 *)epi.pool + at) = h4;
+                                } else {
+                                    *(float4 *)((float *)epi.pool + at) = r4;
+                                }
+                            }
+                        }
+                    }
+                }
+            }
+            buf ^= 1;
+        }
+    }
+}
+
+struct StreamPlan {
+    int g, s, ph, npass;  // row groups, K slices, half chunks per wave and pass, passes; g == 0: not served
+};
+
+// The cut of an [n_tiles * 16, n_hc * 128] matrix for a device of `cus` compute units. With the epilogue the whole
+// K stays in one workgroup (passes of 16 half chunks); otherwise K is sliced so that a slice is one pass, and
+// further while a workgroup would own fewer than four tiles and slices stay at least four half chunks wide: every
+// workgroup first pulls its slice of the activation (128 bytes per column) through its compute unit's L1, which
+// costs as much as the weights of a few tiles. VEXEL_HIP_SPLAN="NxK:G,S;..." overrides the choice (tuning).
+StreamPlan stream_plan(int n_tiles, int n_hc, int cus, bool epi, int N, int K) {
+    StreamPlan pl = {0, 1, 1, 1};
+    if (n_tiles < 1 || n_hc < 1) return pl;
+    static const char *env = getenv("VEXEL_HIP_SPLAN");
+    int s = epi ? 1 : ceil_div(n_hc, 16), g = 0;
+    if (!epi) {
+        while (true) {
+            const int gg = std::max(1, std::min(cus / s, n_tiles));
+            const int nh = ceil_div(n_hc, s);
+            if (n_tiles / gg >= 4 || nh < 8 || s * 2 > cus) break;
+            s *= 2;
+        }
+    }
+    g = std::max(1, std::min(cus / s, n_tiles));
+    if (env && !epi) {
+        char key[64];
+        snprintf(key, sizeof key, "%dx%d:", N, K);
+        const char *p = strstr(env, key);
+        int eg = 0, es = 0;
+        if (p && sscanf(p + strlen(key), "%d,%d", &eg, &es) == 2 && eg >= 1 && es >= 1 && es <= n_hc && eg <= n_tiles &&
+            ceil_div(n_hc, es) <= 16) {
+            g = eg;
+            s = es;
+        }
+    }
+    const int nh = ceil_div(n_hc, s);
+    pl.g = g;
+    pl.s = s;
+    pl.ph = nh > 8 ? 2 : 1;
+    pl.npass = ceil_div(nh, 8 * pl.ph);
+    if (!epi && pl.npass != 1) pl.g = 0;
+    if (epi && pl.npass > 1 && ceil_div(n_tiles, g) > ACC_TILES) pl.g = 0;
+    return pl;
+}
+
+struct PackedW {
+    void *data;
+    int fmt, n, k;
+    size_t bytes;
+};
+
+}  // namespace
+
+namespace vx {
+
+// Registry of packed copies, keyed by the raw matrix' device address (the backend's map stores them type-erased).
+static PackedW *find_packed(vx_backend *be, const void *raw) {
+    auto it = be->packed.find(raw);
+    return it == be->packed.end() ? nullptr : (PackedW *)it->second;
+}
+
+void stream_drop_packed(vx_backend *be, const void *raw) {
+    auto it = be->packed.find(raw);
+    if (it == be->packed.end()) return;
+    PackedW *pw = (PackedW *)it->second;
+    (void)hipFree(pw->data);
+    delete pw;
+    be->packed.erase(it);
+}
+
+void stream_written(vx_backend *be, const void *dst, size_t bytes) {
+    const char *a = (const char *)dst;
+    std::vector<const void *> stale;
+    for (auto &kv : be->packed) {
+        const PackedW *pw = (const PackedW *)kv.second;
+        const char *r = (const char *)kv.first;
+        if (a < r + pw->bytes && r < a + bytes) stale.push_back(kv.first);
+    }
+    if (stale.empty()) return;
+    (void)hipStreamSynchronize(be->stream);  // a launch may still read the copies
+    for (const void *r : stale) stream_drop_packed(be, r);
+}
+
+void stream_drop_all(vx_backend *be) {
+    while (!be->packed.empty()) stream_drop_packed(be, be->packed.begin()->first);
+}
+
+// Resolves up to three row segments of raw matrices (each a run of registered matrices laid end to end) into packed
+// matrices; false when any part has no packed copy.
+static bool resolve(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, PackedSegs *out) {
+    if (fmt != VX_Q4_0 || be->packed.empty()) return false;
+    const size_t row_bytes = (size_t)K / 32 * 18;
+    int np = 0, rows_done = 0;
+    for (int i = 0; i < nseg && rows_done < N; i++) {
+        const int seg_rows = n_end[i] - rows_done;
+        if (seg_rows <= 0) continue;
+        const uint8_t *p = w[i];
+        int left = seg_rows;
+        while (left > 0) {
+            PackedW *pw = find_packed(be, p);
+            if (!pw || pw->fmt != fmt || pw->k != K || pw->n > left || np == 3) return false;
+            out->w[np] = (const uint8_t *)pw->data;
+            out->t_end[np] = (rows_done + pw->n) / 16;
+            np++;
+            rows_done += pw->n;
+            left -= pw->n;
+            p += (size_t)pw->n * row_bytes;
+        }
+    }
+    if (rows_done != N || np == 0) return false;
+    for (int i = np; i < 3; i++) {
+        out->w[i] = out->w[np - 1];
+        out->t_end[i] = N / 16;
+    }
+    return true;
+}
+
+bool stream_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M, bool epi) {
+    static const char *off = getenv("VEXEL_HIP_STREAM_OFF");
+    if (off && atoi(off)) return false;
+    if (M < 2 || M > 32 || N % 16 != 0 || K % 256 != 0 || N < 16) return false;
+    // With the epilogue the whole K stays in one workgroup, which walks it in passes of 16 half chunks; every pass
+    // starts its requests anew, and for two passes and more the launch takes longer than the wave-private kernel's
+    // (7B Q|K|V, 32 rows: 23.8 against 20.9 us). VEXEL_HIP_STREAM_EPI=1 takes it anyway (measurements).
+    static const bool epi_any = getenv("VEXEL_HIP_STREAM_EPI") != nullptr;
+    if (epi && K / 128 > 16 && !epi_any) return false;
+    PackedSegs ps;
+    if (!resolve(be, fmt, w, n_end, nseg, N, K, &ps)) return false;
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0) cus = 256;
+    return stream_plan(N / 16, K / 128, cus, epi, N, K).g > 0;
+}
+
+// Launches the streaming kernel; the K slices' sums go to be->part_ws as [slice][M][N] (raw: no row factors), or, with
+// an epilogue, the finished rows to where it says. *ks_out: the number of slices.
+int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M, int mpad,
+                const PrepView &pv, const QkvEpi *epi, int *ks_out) {
+    PackedSegs ps;
+    if (!resolve(be, fmt, w, n_end, nseg, N, K, &ps)) return VX_ERR_UNSUPPORTED;
+    static int cus = 0;
+    if (cus == 0 && (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0)) cus = 256;
+    const bool fin = epi && epi->q_out;
+    const StreamPlan pl = stream_plan(N / 16, K / 128, cus, fin, N, K);
+    if (pl.g == 0) return VX_ERR_UNSUPPORTED;
+    StreamShape a;
+    a.M = M;
+    a.Mpad = mpad;
+    a.N = N;
+    a.n_hc = K / 128;
+    a.npass = pl.npass;
+    a.t_end0 = ps.t_end[0];
+    a.t_end1 = ps.t_end[1];
+    const QkvEpi e = fin ? *epi : QkvEpi{};
+    float *partial = nullptr;
+    if (!fin) {
+        int rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, (size_t)pl.s * M * N * sizeof(float), "split-K partial sums");
+        if (rc) return rc;
+        partial = (float *)be->part_ws;
+    }
+    dim3 grid(pl.g, pl.s);
+    const int mt = mpad / 16;
+#define VX_STREAM_LAUNCH(PH_, RG_, MT_, EPI_)                                                                                  \
+    qstream_kernel<PH_, RG_, MT_, EPI_><<<grid, 64 * NW, 0, be->stream>>>(ps.w[0], ps.w[1], ps.w[2], pv.tiles, pv.cscale, pv.inv_scale, \
+                                                                           partial, a, e)
+    if (fin) {
+        if (pl.ph == 2) {
+            if (mt == 2) VX_STREAM_LAUNCH(2, 2, 2, true);
+            else VX_STREAM_LAUNCH(2, 2, 1, true);
+        } else {
+            if (mt == 2) VX_STREAM_LAUNCH(1, 2, 2, true);
+            else VX_STREAM_LAUNCH(1, 2, 1, true);
+        }
+    } else if (pl.ph == 2) {
+        if (mt == 2) VX_STREAM_LAUNCH(2, 2, 2, false);
+        else VX_STREAM_LAUNCH(2, 2, 1, false);
+    } else {
+        if (mt == 2) VX_STREAM_LAUNCH(1, 4, 2, false);
+        else VX_STREAM_LAUNCH(1, 4, 1, false);
+    }
+#undef VX_STREAM_LAUNCH
+    VX_CHECK_LAUNCH();
+    if (ks_out) *ks_out = pl.s;
+    return VX_OK;
+}
+
+}  // namespace vx
+
+extern "C" {
+
+int vx_qweight_pack(vx_backend *be, const vx_qweight *w) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(w && w->data, "vx_qweight_pack: null weight");
+    VX_REQUIRE(!be->capturing, "vx_qweight_pack during graph capture");
+    if (w->fmt != VX_Q4_0 || w->n < 16 || w->n % 16 != 0 || w->k < 256 || w->k % 256 != 0) return VX_ERR_UNSUPPORTED;
+    if (find_packed(be, w->data)) stream_drop_packed(be, w->data);
+    PackedW *pw = new PackedW{nullptr, w->fmt, w->n, w->k, (size_t)w->n * (w->k / 32) * 18};
+    if (hipMalloc(&pw->data, pw->bytes) != hipSuccess) {
+        delete pw;
+        set_error("vx_qweight_pack: out of device memory (%zu bytes)", (size_t)w->n * (w->k / 32) * 18);
+        return VX_ERR_OOM;
+    }
+    pack_q4_0_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) {
+        (void)hipFree(pw->data);
+        delete pw;
+        set_error("vx_qweight_pack: launch failed: %s", hipGetErrorString(e));
+        return VX_ERR_HIP;
+    }
+    be->packed[w->data] = pw;
+    return VX_OK;
+}
+
+int vx_qweight_unpack(vx_backend *be, const vx_qweight *w) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(w && w->data, "vx_qweight_unpack: null weight");
+    VX_CHECK_HIP(hipStreamSynchronize(be->stream));  // a launch may still read the copy
+    stream_drop_packed(be, w->data);
+    return VX_OK;
+}
+
+int vx_qweight_is_packed(vx_backend *be, const vx_qweight *w) {
+    if (!be || !w || !w->data) return 0;
+    PackedW *pw = find_packed(be, w->data);
+    return pw && pw->fmt == w->fmt && pw->n == w->n && pw->k == w->k ? 1 : 0;
+}
+
+int vx_dequantize_packed(vx_backend *be, const vx_qweight *w, float *dst) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(w && w->data && dst, "vx_dequantize_packed: null pointer");
+    PackedW *pw = find_packed(be, w->data);
+    VX_REQUIRE(pw && pw->fmt == w->fmt && pw->n == w->n && pw->k == w->k, "vx_dequantize_packed: the matrix has no packed copy");
+    const size_t total = (size_t)w->n * w->k;
+    dequant_packed_q4_0_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+}  // extern "C"

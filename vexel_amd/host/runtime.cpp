@@ -526,6 +526,17 @@ int vh_model_set_layer(vh_model *m, int layer, const vh_layer_weights *w) {
         w->wo.k != qd || w->w1.n != c.ffn || (w->w3.data && w->w3.n != c.ffn) || w->w2.n != c.hidden || w->w2.k != c.ffn)
         return fail("layer %d: weight shapes do not match the configuration", layer);
     m->layers[layer] = *w;
+    // Decode batches stream load-time packed copies of the projections (formats and shapes without one stay as
+    // they are); a model that never runs more than one row at a time has no use for them.
+    static const bool no_pack = getenv("VEXEL_HIP_NO_PACK") != nullptr;
+    if (c.max_batch >= 2 && !no_pack) {
+        const vh_qweight *all[7] = {&w->wq, &w->wk, &w->wv, &w->wo, &w->w1, &w->w3, &w->w2};
+        for (const vh_qweight *q : all) {
+            if (!q->data) continue;
+            const int rc = vx_qweight_pack(m->be, q);
+            if (rc != VX_OK && rc != VX_ERR_UNSUPPORTED) return fail("layer %d: %s", layer, vx_last_error());
+        }
+    }
     return VH_OK;
 }
 

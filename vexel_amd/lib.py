@@ -80,6 +80,10 @@ SIGNATURES = {
                                    _f, _i, _i, _vp]),
     "vx_decode_attn_qkv": (_i, [_vp, _vp, _vp, _f, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
     "vx_decode_ffn_supported": (_i, [_vp, _vp, _vp, _vp]),
+    "vx_qweight_pack": (_i, [_vp, _vp]),
+    "vx_qweight_unpack": (_i, [_vp, _vp]),
+    "vx_qweight_is_packed": (_i, [_vp, _vp]),
+    "vx_dequantize_packed": (_i, [_vp, _vp, _vp]),
     "vx_decode_ffn": (_i, [_vp, _vp, _vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _vp]),
     "vx_rope_store_paged": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f]),
     "vx_rope_store_paged_ex": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i, _i]),
