@@ -313,14 +313,23 @@ int vx_sdpa_paged_decode_ragged(vx_backend *be, const float *q, const void *kv_p
  * the per-split partial sums in a fixed 8 MiB area that every device holds from the moment the library is loaded
  * until the process ends, instead of the backend's growable scratch. It has no counterpart in the reference. The
  * call allocates and frees nothing. It needs out != NULL and a geometry of the streaming kernel
- * (vx_sdpa_paged_decode_split_supported() == 1), else VX_ERR_UNSUPPORTED; batch * num_q_heads *
- * ceil(max_kv_len / 512) * (head_dim + 2) * 4 bytes must fit the area (32 sequences x 32 heads of 128 up to 4096
- * tokens take 4.3 MB), else VX_ERR_INVALID with the sizes in vx_last_error(). All calls on one device, from any
- * backend, share the area: two of them in flight at once race. */
+ * (vx_sdpa_paged_decode_split_supported() == 1), else VX_ERR_UNSUPPORTED; batch * num_q_heads * splits *
+ * (head_dim + 2) * 4 bytes must fit the area, else VX_ERR_INVALID with the sizes in vx_last_error(). splits =
+ * ceil(max_kv_len / t), where t, the tokens one workgroup takes, is what the allocating entry point uses for the
+ * same call (so that the results are the same bits): 512; 256 with two or more query heads per KV head at heads
+ * of 64 or 128; and halved again, down to 128, while batch * num_kv_heads * splits would be under twice the
+ * device's compute units. Examples: 32 sequences x 32 heads of 128 up to 4096 tokens take 4.3 MB; 32 sequences
+ * x 32 / 8 heads of 128 up to 4096 tokens take 8.5 MB and are refused. vx_sdpa_paged_decode_ragged_noalloc_bytes
+ * gives the exact need of a call (0 for a geometry the entry point does not take) and, through *capacity when
+ * that is not NULL, the size of the area. All calls on one device, from any backend, share the area: two of
+ * them in flight at once race. */
 int vx_sdpa_paged_decode_ragged_noalloc(vx_backend *be, const float *q, const void *kv_pool, int pool_is_f16,
                                         const int32_t *block_tables, const int32_t *table_rows, const int32_t *kv_lens,
                                         float *out, int batch, int max_blocks, int block_size, int num_q_heads,
                                         int num_kv_heads, int head_dim, float scale, int max_kv_len);
+
+size_t vx_sdpa_paged_decode_ragged_noalloc_bytes(vx_backend *be, int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                                                 int max_kv_len, size_t *capacity);
 
 /* Tree verification (medusa/tree.go:186-202 mask rule): query i attends to every pool
  * position < tree_base and to position tree_base+j iff tree_mask[i*query_len+j] != 0
@@ -410,11 +419,13 @@ int vx_graph_begin_capture(vx_backend *be);
 int vx_graph_end_capture(vx_backend *be, vx_graph **out);
 int vx_graph_launch(vx_backend *be, vx_graph *g);
 /* A recording holds the addresses of the library's own scratch buffers (prepared activations, split-K and
- * split-KV partial sums, the attention work list). They move when a later eager call needs more room than any
- * call before it; the counter returned here goes up by one each time that happens. A caller that keeps a graph
+ * split-KV partial sums, the attention work list) and of the packed copies of quantized matrices. The buffers move
+ * when a later eager call needs more room than any call before it, the copies come and go with vx_qweight_pack /
+ * vx_qweight_unpack / vx_free; the counter returned here goes up by one each time either happens. A caller that keeps a graph
  * records the counter after vx_graph_end_capture and captures again, instead of launching, once it has changed.
  * No counterpart in the reference (its command buffers are rebuilt every step). */
 uint64_t vx_scratch_generation(const vx_backend *be);
+/* The caller makes sure no replay of the graph is still running (vx_sync). */
 void vx_graph_destroy(vx_graph *g);
 
 /* Wall-clock helpers on the backend stream (HIP events), for benchmarks. */

@@ -580,14 +580,65 @@ def test_batched_greedy_64_steps_c2_shape(be):
     mr.close()
 
 
+def _f64_logit_gap(omodel, token, seq_id, pos, a, b):
+    """logit[a] - logit[b] of one decode step of a LLaMA-type oracle model, evaluated in float64 from the oracle's
+    inputs: the exactly dequantised weights and the K/V rows its pool holds for positions 0 .. pos (the step's own
+    row included, as the oracle stored it). RoPE angles are the reference's float32 angles (cpu.go:256-260)."""
+    c = omodel.cfg
+    deq = lambda q: nx.dequantize(q.fmt, q.data, q.n * q.k).reshape(q.n, q.k).astype(np.float64)
+    rms = lambda v, w: v / np.sqrt((v * v).mean() + c.eps) * w.astype(np.float64)
+    x = omodel.embedding[token].astype(np.float64)
+    D, Hq, Hk, bs = c.head_dim, c.num_heads, c.num_kv_heads, c.block_size
+    j = np.arange(D // 2)
+    freq = (1.0 / np.power(np.float64(c.rope_theta), 2.0 * j / D)).astype(np.float32)
+    ang = (np.float32(pos) * freq).astype(np.float64)
+    cs, sn = np.cos(ang), np.sin(ang)
+    for l, lw in enumerate(omodel.layers):
+        h = rms(x, lw.attn_norm)
+        q = (deq(lw.wq) @ h).reshape(Hq, D)
+        qr = q.copy()
+        qr[:, 0::2] = q[:, 0::2] * cs - q[:, 1::2] * sn
+        qr[:, 1::2] = q[:, 0::2] * sn + q[:, 1::2] * cs
+        bt = omodel.pool.seqs[seq_id].block_tables[l]
+        kv = omodel.kv[l]
+        per_block = 2 * bs * Hk * D
+        K = np.empty((pos + 1, Hk, D))
+        V = np.empty((pos + 1, Hk, D))
+        for t in range(pos + 1):
+            base = bt[t // bs] * per_block + (t % bs) * Hk * D
+            K[t] = nx.f16_to_f32_array(kv[base:base + Hk * D]).reshape(Hk, D)
+            V[t] = nx.f16_to_f32_array(kv[base + bs * Hk * D:base + bs * Hk * D + Hk * D]).reshape(Hk, D)
+        out = np.empty((Hq, D))
+        for hq in range(Hq):
+            hk = hq // (Hq // Hk)
+            sc = K[:, hk, :] @ qr[hq] / np.sqrt(np.float64(D))
+            w = np.exp(sc - sc.max())
+            out[hq] = (w / w.sum()) @ V[:, hk, :]
+        x = x + deq(lw.wo) @ out.reshape(-1)
+        h2 = rms(x, lw.ffn_norm)
+        g, u = deq(lw.w1) @ h2, deq(lw.w3) @ h2
+        x = x + deq(lw.w2) @ (g / (1.0 + np.exp(-g)) * u)
+    hn = rms(x, omodel.final_norm)
+    head = omodel.lm_head
+    rows = head.data.reshape(head.n, -1)
+    la = nx.dequantize(head.fmt, rows[a], head.k).astype(np.float64) @ hn
+    lb = nx.dequantize(head.fmt, rows[b], head.k).astype(np.float64) @ hn
+    return float(la - lb)
+
+
 def test_batched_greedy_64_steps_7b_geometry_32_sequences(be):
     """The north-star batch shape, one layer deep: hidden 4096, 32 heads of 128, FFN 11008, Q4_0, 32 ragged
     sequences, 64 greedy steps through the graph-captured batched path (2048 tokens). The oracle is run over the
     tokens the GPU produced: at every step and sequence the GPU's token must be the oracle's argmax. With 2048
-    draws from 4096 near-flat random-init logits a few top-two gaps fall below the float32 summation noise of the
-    reference loop itself (its K = 11008 sequential sums differ from the exact value by up to ~5e-4 here, as much
-    as the two implementations differ from each other); at such a tie, and only there, the GPU may take the
-    oracle's runner-up, which has to be within 5e-4 of the maximum. At most three such ties are accepted."""
+    draws from 4096 near-flat random-init logits a top-two gap can fall below the float32 summation noise of the
+    reference loop itself (K = 11008 sequential float32 sums). Where the GPU took the oracle's runner-up, the pair
+    of logits is evaluated in float64 from the oracle's inputs, and the pick stands only if (a) it is the float64
+    maximum of the two, or (b) the oracle's own float32 gap at that pair is off the float64 gap by more than the gap
+    itself (the reference's arithmetic cannot tell the two apart), or (c) the float64 gap is under 1e-4: the size of
+    the differences that a change of float32 summation order makes in logits of magnitude 1 to 4 here (the library
+    sums 256-column chunks on the matrix cores, the reference one column after the other), a hundredth of the
+    north star's 1e-2 logit tolerance. Anything else fails, and at most three picks may need (b) or (c). The
+    smallest top-1 margin of every step and every settled pick are printed."""
     cfg = om.ModelConfig(num_layers=1, hidden=4096, num_heads=32, num_kv_heads=32, head_dim=128, ffn=11008, vocab=4096)
     rng0 = np.random.default_rng(61)
     ctx = [int(x) for x in np.clip(np.exp(rng0.normal(np.log(150), 0.6, 32)), 16, 400)]
@@ -597,23 +648,30 @@ def test_batched_greedy_64_steps_7b_geometry_32_sequences(be):
     out, _ = mr.decode_graph(first, ids, ctx, 64, use_graph=True)
     assert mr.device_matches_host()
     nx.set_row_threads(16)
-    ties = []
+    ties, margins = [], []
     try:
         toks, pos = list(first), list(ctx)
         for s in range(64):
             lg = omodel.decode_batched(toks, ids, pos)
             assert np.isfinite(lg).all()
+            top2 = np.sort(lg, axis=1)[:, -2:]
+            margins.append(float((top2[:, 1] - top2[:, 0]).min()))
             for i in range(32):
                 best, got = nx.argmax(lg[i]), int(out[s][i])
                 if got != best:
-                    gap = float(lg[i][best] - lg[i][got])
-                    assert gap <= 5e-4, "step %d sequence %d: token %d is %.3e below the oracle's %d" % (s, i, got, gap, best)
-                    ties.append((s, i, gap))
+                    gap32 = float(lg[i][best] - lg[i][got])
+                    gap64 = _f64_logit_gap(omodel, toks[i], ids[i], pos[i], best, got)
+                    rule = "a" if gap64 <= 0.0 else ("b" if abs(gap32 - gap64) >= gap32 else ("c" if gap64 < 1e-4 else None))
+                    assert rule, ("step %d sequence %d: token %d is %.3e below the oracle's %d in float32 and %.3e in float64"
+                                  % (s, i, got, gap32, best, gap64))
+                    ties.append((s, i, gap32, gap64, rule))
             toks = [int(t) for t in out[s]]
             pos = [p + 1 for p in pos]
     finally:
         nx.set_row_threads(1)
-    assert len(ties) <= 3, ties
+    print("smallest top-1 margin per step: %s" % " ".join("%.1e" % m for m in margins))
+    print("picks settled in float64 (step, sequence, float32 gap, float64 gap, rule): %s" % ties)
+    assert len([t for t in ties if t[4] != "a"]) <= 3, ties
     for sid in ids:
         assert mr.block_table(sid) == omodel.pool.seqs[sid].block_tables[0]
     mr.close()

@@ -20,10 +20,10 @@ def be():
     b.close()
 
 
-def _case(rng, be, lens, hq, hk, d, nblocks, dpool, pool):
+def _case(rng, be, lens, hq, hk, d, nblocks, dpool, pool, mb=None):
     bs = 16
     B = len(lens)
-    mb = max((L + bs - 1) // bs for L in lens) + 2
+    mb = mb or max((L + bs - 1) // bs for L in lens) + 2
     perm = rng.permutation(nblocks)
     mat = np.zeros((B, mb), dtype=np.int32)
     off = 0
@@ -71,9 +71,40 @@ def test_noalloc_refuses_what_does_not_fit(be):
     do = be.alloc(B * hq * d * 4)
     with pytest.raises(VexelError, match="fixed area holds"):
         be.sdpa_paged_decode_ragged_noalloc(dq, dpool, True, dmat, dl, do, B, mb, bs, hq, hk, d, 0.1, mb * bs)
+    need, cap = be.sdpa_paged_decode_ragged_noalloc_bytes(B, hq, hk, d, mb * bs)
+    assert cap == 8 << 20 and need == B * hq * 16 * (d + 2) * 4
     # a float32 pool has no streaming kernel: refused rather than sent to the allocating path
     with pytest.raises(VexelError, match="streaming kernel"):
         be.sdpa_paged_decode_ragged_noalloc(dq, dpool, False, dmat, dl, do, 2, mb, bs, hq, hk, d, 0.1, 64)
     with pytest.raises(VexelError, match="null pointer"):
         be.sdpa_paged_decode_ragged_noalloc(dq, dpool, True, dmat, dl, None, 2, mb, bs, hq, hk, d, 0.1, 64)
+    be.reset_pool()
+
+
+def test_noalloc_grouped_queries_at_the_limit_of_the_area(be):
+    """Grouped queries run on splits of 256 tokens (128 for small batches), so they need two to four times the
+    partial sums of one query head per KV head: the query function gives the exact figure, a call just inside the
+    area runs and matches the allocating entry point bit for bit, the 8B shape at 32 x 4096 tokens is refused."""
+    from vexel_amd.backend import VexelError
+    rng = np.random.default_rng(79)
+    hq, hk, d, bs = 32, 8, 128, 16
+    need, cap = be.sdpa_paged_decode_ragged_noalloc_bytes(32, hq, hk, d, 4096)
+    assert need == 32 * hq * 16 * (d + 2) * 4 and need > cap          # 16 splits of 256 tokens: 8.5 MB
+    # the largest batch of 3800-token tables that fits: 15 splits of 256 tokens
+    B = cap // (hq * 15 * (d + 2) * 4)
+    mb = 3800 // bs + 1
+    need, _ = be.sdpa_paged_decode_ragged_noalloc_bytes(B, hq, hk, d, mb * bs)
+    assert need <= cap < be.sdpa_paged_decode_ragged_noalloc_bytes(B + 1, hq, hk, d, mb * bs)[0]
+    lens = [int(x) for x in rng.integers(1, 3800, B)]
+    lens[0], lens[1] = 3800, 256
+    nblocks = sum((L + bs - 1) // bs for L in lens) + 4
+    pool = nx.f32_to_f16_array(rng.standard_normal(nblocks * 2 * bs * hk * d).astype(np.float32))
+    dpool = be.upload(pool)
+    _case(rng, be, lens, hq, hk, d, nblocks, dpool, pool, mb=mb)
+    dq = be.upload(np.zeros((32, hq, d), dtype=np.float32))
+    dmat = be.upload(np.zeros((32, 256), dtype=np.int32))
+    dl = be.upload(np.ones(32, dtype=np.int32))
+    do = be.alloc(32 * hq * d * 4)
+    with pytest.raises(VexelError, match="fixed area holds"):
+        be.sdpa_paged_decode_ragged_noalloc(dq, dpool, True, dmat, dl, do, 32, 256, bs, hq, hk, d, 0.1, 4096)
     be.reset_pool()

@@ -335,6 +335,13 @@ class HipBackend:
         self.call("vx_sdpa_paged_decode_ragged_noalloc", q, kv_pool, int(bool(pool_is_f16)), block_tables, table_rows,
                   kv_lens, out, batch, max_blocks, block_size, num_q_heads, num_kv_heads, head_dim, scale, max_kv_len)
 
+    def sdpa_paged_decode_ragged_noalloc_bytes(self, batch, num_q_heads, num_kv_heads, head_dim, max_kv_len):
+        """(bytes of partial sums the call needs, size of the fixed area)."""
+        cap = C.c_size_t(0)
+        need = self._lib.vx_sdpa_paged_decode_ragged_noalloc_bytes(self._h, batch, num_q_heads, num_kv_heads, head_dim,
+                                                                    max_kv_len, C.byref(cap))
+        return int(need), int(cap.value)
+
     def sdpa_paged_tree(self, q, kv_pool, pool_is_f16, block_table, out, tree_mask, tree_base, block_size,
                         num_q_heads, num_kv_heads, head_dim, scale, query_len):
         self.call("vx_sdpa_paged_tree", q, kv_pool, int(bool(pool_is_f16)), block_table, out, tree_mask,

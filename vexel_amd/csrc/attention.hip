@@ -1296,6 +1296,27 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
 constexpr size_t FIXED_WS_BYTES = (size_t)8 << 20;
 static __device__ __align__(256) unsigned char scratch[FIXED_WS_BYTES];
 
+// Tokens per split of the streaming kernels: ATTN_TPW; half of it for grouped queries at heads of 64 / 128 (fewer
+// kv heads, so fewer workgroups per token, and the matrix-core form's per-block work is small: measured faster at
+// every batch tried); and down to a quarter of ATTN_TPW while that many splits would leave most of the chip idle
+// (a single sequence). The work list from vx_pack_batch is cut in ATTN_TPW tokens, so it serves the first only.
+int split_tokens(vx_backend *be, int D, int G, int batch, int num_kv_heads, int max_kv_len) {
+    static const int cus = [&] {
+        int n = 0;
+        return (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, be->device) == hipSuccess && n > 0) ? n : 256;
+    }();
+    int tps = TPW;
+    if (G >= 2 && (D == 64 || D == 128)) tps = TPW / 2;
+    while (tps > TPW / 4 && (size_t)batch * num_kv_heads * ceil_div(max_kv_len, tps) < (size_t)2 * cus) tps /= 2;
+    return tps;
+}
+// Bytes of partial sums for that many splits: (maximum, sum, D values) per sequence, head and split; a single
+// sequence's merged row behind them.
+size_t split_bytes(int D, int batch, int num_q_heads, int max_splits) {
+    const size_t partial_floats = ((size_t)batch * num_q_heads * max_splits * (D + 2) + 3) & ~(size_t)3;
+    return (partial_floats + (batch == 1 ? (size_t)num_q_heads * D : 0)) * sizeof(float);
+}
+
 // fixed: the call takes the fixed area (and fails when it is too small) instead of the growable one
 template <int D, int G>
 int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *bt_matrix, const int32_t *bt_rows,
@@ -1303,18 +1324,10 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
                float scale, int max_kv_len, bool fixed) {
     // Tokens per split: ATTN_TPW; a quarter of it at least when that many splits would leave most of the chip
     // idle (a single sequence). The work list from vx_pack_batch is cut in ATTN_TPW tokens, so it serves the first only.
-    int tps = TPW;
-    static const int cus = [&] {
-        int n = 0;
-        return (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, be->device) == hipSuccess && n > 0) ? n : 256;
-    }();
-    // (grouped queries: fewer kv heads, so fewer workgroups per token, and the matrix-core form's per-block work is
-    // small: half the tokens per split measured faster at every batch tried)
-    if (G >= 2 && (D == 64 || D == 128)) tps = TPW / 2;
-    while (tps > TPW / 4 && (size_t)batch * num_kv_heads * ceil_div(max_kv_len, tps) < (size_t)2 * cus) tps /= 2;
+    const int tps = split_tokens(be, D, G, batch, num_kv_heads, max_kv_len);
     int max_splits = ceil_div(max_kv_len, tps);
+    const size_t need = split_bytes(D, batch, num_q_heads, max_splits);
     const size_t partial_floats = ((size_t)batch * num_q_heads * max_splits * (D + 2) + 3) & ~(size_t)3;
-    const size_t need = (partial_floats + (batch == 1 ? (size_t)num_q_heads * D : 0)) * sizeof(float);
     float *ws;
     if (fixed) {
         if (need > FIXED_WS_BYTES || !be->attn_fixed_ws) {
@@ -1651,6 +1664,16 @@ int vx_sdpa_paged_decode_ragged_noalloc(vx_backend *be, const float *q, const vo
                "vx_sdpa_paged_decode_ragged_noalloc: max_kv_len %d not in 1..table capacity %d", max_kv_len, max_blocks * block_size);
     return run_ragged(be, q, kv_pool, pool_is_f16, nullptr, block_tables, table_rows, max_blocks, kv_lens, out, batch,
                       block_size, num_q_heads, num_kv_heads, head_dim, scale, max_kv_len, true);
+}
+
+size_t vx_sdpa_paged_decode_ragged_noalloc_bytes(vx_backend *be, int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                                                 int max_kv_len, size_t *capacity) {
+    if (capacity) *capacity = FIXED_WS_BYTES;
+    if (!be || batch < 1 || max_kv_len < 1 || !vx_sdpa_paged_decode_split_supported(1, HOT_BS, num_q_heads, num_kv_heads, head_dim))
+        return 0;
+    if (enter(be) != VX_OK) return 0;
+    const int tps = split_tokens(be, head_dim, num_q_heads / num_kv_heads, batch, num_kv_heads, max_kv_len);
+    return split_bytes(head_dim, batch, num_q_heads, ceil_div(max_kv_len, tps));
 }
 
 int vx_sdpa_paged_decode_split_supported(int pool_is_f16, int block_size, int num_q_heads, int num_kv_heads,

@@ -426,6 +426,7 @@ void stream_drop_packed(vx_backend *be, const void *raw) {
     (void)hipFree(pw->data);
     delete pw;
     be->packed.erase(it);
+    be->scratch_gen++;  // a recorded graph may hold the copy's address
 }
 
 void stream_written(vx_backend *be, const void *dst, size_t bytes) {
@@ -569,6 +570,7 @@ int vx_qweight_pack(vx_backend *be, const vx_qweight *w) {
         return VX_ERR_HIP;
     }
     be->packed[w->data] = pw;
+    be->scratch_gen++;  // a graph recorded before streams the GGUF rows: the holder records again
     return VX_OK;
 }
 

@@ -506,9 +506,11 @@ int vh_model_create(vx_backend *be, const vh_config *cfg, vh_model **out) {
     return VH_OK;
 }
 
+static void drop_graph(vh_model *m);
+
 void vh_model_destroy(vh_model *m) {
     if (!m) return;
-    if (m->graph) vx_graph_destroy(m->graph);
+    drop_graph(m);
     for (void *p : m->kv) vx_free(m->be, p);
     void *bufs[] = {m->d_tables, m->d_num_blocks, m->d_free, m->d_free_count, m->d_slots, m->d_positions, m->d_tokens,
                     m->d_next, m->d_cu, m->d_token_pos, m->d_slot_map, m->d_kv_lens, m->d_pos_in, m->d_status, m->d_step, m->d_log,
@@ -525,6 +527,7 @@ int vh_model_set_layer(vh_model *m, int layer, const vh_layer_weights *w) {
     if (w->wq.n != qd || w->wq.k != c.hidden || w->wk.n != kvd || w->wv.n != kvd || w->wo.n != c.hidden ||
         w->wo.k != qd || w->w1.n != c.ffn || (w->w3.data && w->w3.n != c.ffn) || w->w2.n != c.hidden || w->w2.k != c.ffn)
         return fail("layer %d: weight shapes do not match the configuration", layer);
+    drop_graph(m);  // a recorded step holds the previous matrices' addresses
     m->layers[layer] = *w;
     // Decode batches stream load-time packed copies of the projections (formats and shapes without one stay as
     // they are); a model that never runs more than one row at a time has no use for them.
@@ -543,14 +546,18 @@ int vh_model_set_layer(vh_model *m, int layer, const vh_layer_weights *w) {
 int vh_model_set_head(vh_model *m, const float *embedding, const float *final_norm, const vh_qweight *lm_head) {
     if (!m || !embedding || !final_norm || !lm_head) return fail("null argument");
     if (lm_head->n != m->cfg.vocab || lm_head->k != m->cfg.hidden) return fail("lm_head shape mismatch");
+    drop_graph(m);
     m->embedding = embedding;
     m->final_norm = final_norm;
     m->lm_head = *lm_head;
     return VH_OK;
 }
 
-static void drop_graph(vh_model *m) {  // a captured step was recorded with another kernel sequence
+// A recorded step goes away: because it was recorded with another kernel sequence or other addresses, or with its
+// model. The stream is drained first, so that no replay is in flight when the executable graph is destroyed.
+static void drop_graph(vh_model *m) {
     if (m->graph) {
+        (void)vx_sync(m->be);
         vx_graph_destroy(m->graph);
         m->graph = nullptr;
         m->graph_batch = 0;
@@ -620,11 +627,7 @@ int vh_model_set_final_norm_bias(vh_model *m, const float *bias) {
 void vh_model_set_fused(vh_model *m, int on) {
     if (!m) return;
     m->fused = on != 0;
-    if (m->graph) {  // the captured step was recorded with the other kernel sequence
-        vx_graph_destroy(m->graph);
-        m->graph = nullptr;
-        m->graph_batch = 0;
-    }
+    drop_graph(m);  // the captured step was recorded with the other kernel sequence
 }
 
 void *vh_kv_pool(vh_model *m, int layer) {
@@ -1384,10 +1387,7 @@ int vh_decode_graph(vh_model *m, const int32_t *first_tokens, const int64_t *seq
         m->d_log = nullptr;
         VHC(dev_alloc(m, &m->d_log, (size_t)steps * c.max_batch));
         m->log_cap = steps;
-        if (m->graph) {  // the graph holds the old log pointer
-            vx_graph_destroy(m->graph);
-            m->graph = nullptr;
-        }
+        drop_graph(m);  // the graph holds the old log pointer
     }
     int32_t zero = 0;
     VXC(vx_to_device(m->be, m->d_step, &zero, 4));
@@ -1396,15 +1396,17 @@ int vh_decode_graph(vh_model *m, const int32_t *first_tokens, const int64_t *seq
     // a recording holds the library's scratch addresses: once an eager call in between (a longer prefill, a tree
     // verification, a larger batch) has made one of them grow, it is stale
     if (use_graph && (!m->graph || m->graph_batch != batch || m->graph_scratch_gen != vx_scratch_generation(m->be))) {
-        if (m->graph) vx_graph_destroy(m->graph);
-        m->graph = nullptr;
+        drop_graph(m);
         VHC(device_step(m, batch));  // eager: sizes the library scratch; it is step 0 of this call
         done = 1;
         VXC(vx_graph_begin_capture(m->be));
         int rc = device_step(m, batch);
         vx_graph *gr = nullptr;
         int rc2 = vx_graph_end_capture(m->be, &gr);
-        if (rc != VH_OK) return VH_ERR;
+        if (rc != VH_OK) {
+            if (gr) vx_graph_destroy(gr);
+            return VH_ERR;
+        }
         if (rc2 != VX_OK) return fail("graph capture: %s", vx_last_error());
         m->graph = gr;
         m->graph_batch = batch;

@@ -90,6 +90,7 @@ SIGNATURES = {
     "vx_sdpa_paged_decode_split_supported": (_i, [_i, _i, _i, _i, _i]),
     "vx_sdpa_paged_decode_ragged": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i]),
     "vx_sdpa_paged_decode_ragged_noalloc": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _f, _i]),
+    "vx_sdpa_paged_decode_ragged_noalloc_bytes": (_sz, [_vp, _i, _i, _i, _i, _i, C.POINTER(_sz)]),
     "vx_sdpa_paged_tree": (_i, [_vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _i]),
     "vx_argmax_rows": (_i, [_vp, _vp, _i, _i, _vp]),
     "vx_sdpa_paged_tree_rows_per_entry": (_i, [_i, _i, _i, _i, _i]),
