@@ -43,6 +43,13 @@ enum { VX_Q4_0 = 1, VX_Q8_0 = 2, VX_Q4_K = 3, VX_Q6_K = 4, VX_Q5_0 = 5, VX_Q5_K 
 /* metal.NewBackend (backend/metal/backend.go:238-409); Backend.Device (backend.go:311) */
 int vx_backend_create(int device_id, vx_backend **out);
 void vx_backend_destroy(vx_backend *be);
+/* Whether the ragged decode attention kernel merges the partial results of a sequence's splits itself (the workgroup
+ * that finishes a sequence's columns last does it; default) or leaves them to a merge step of the consumer
+ * (on = 0). Both give the same bits; the in-kernel form saves a launch per layer and orders its memory traffic by
+ * properties of this GPU family's caches rather than by HIP's memory model, so the switch exists to fall back and
+ * to compare. The environment variable VEXEL_HIP_NO_ATTN_MERGE, read at vx_backend_create, sets the initial value
+ * to off. No counterpart in the reference. */
+int vx_backend_set_attn_merge(vx_backend *be, int on);
 int vx_backend_device(const vx_backend *be);
 const char *vx_last_error(void);
 

@@ -1482,3 +1482,66 @@ def test_decode_attn_qkv_with_bias_and_rope_forms(be, rows, rope_dim, neox, bias
         untouched[b * per_blk + bs * hk * d + o * hk * d: b * per_blk + bs * hk * d + (o + 1) * hk * d] = False
     assert np.array_equal(be.download(dpool, pool.shape, pool.dtype)[untouched], pool[untouched])
     be.reset_pool()
+
+
+@pytest.mark.parametrize("hq,hk,d,hidden", [(32, 32, 128, 4096), (32, 8, 128, 4096), (24, 8, 128, 3072)])
+def test_in_kernel_merge_equals_the_separate_merge_and_the_oracle(be, hq, hk, d, hidden):
+    """The attention kernel's own merge of its splits (vx_backend_set_attn_merge, the default) against the merge left
+    to vx_decode_ffn, at the north-star head geometry and two grouped-query ones: over 24 launches with changing
+    ragged lengths (up to nine splits per sequence, sequences without tokens, lengths on split boundaries) the
+    layer outputs of the two forms are the same bits, launch after launch; and the first launch's attention output,
+    merged in the kernel and fed through Wo, matches the oracle's paged attention and MatMulQ4_0."""
+    rng = np.random.default_rng(hq * 7 + hk)
+    fmt, rows, ffn = nx.FMT_Q4_0, 32, 1024
+    bs, eps = 16, 1e-5
+    max_blocks = 290
+    nblocks = 32 * 140
+    dims = dict(wo=(hidden, hq * d), w1=(ffn, hidden), w3=(ffn, hidden), w2=(hidden, ffn))
+    raw = {n: qz.random_quant(fmt, rng, *dims[n]) for n in dims}
+    dW = {n: be.upload(raw[n], permanent=True) for n in dims}
+    qw = {n: be.qweight(fmt, dW[n], *dims[n]) for n in dims}
+    pool = _make_pool(rng, True, nblocks, bs, hk, d)
+    q = rng.standard_normal((rows, hq * d)).astype(np.float32)
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    nw = (1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    dpool, dq, dnw = be.upload(pool, permanent=True), be.upload(q, permanent=True), be.upload(nw, permanent=True)
+    scale = np.float32(1.0 / math.sqrt(d))
+    dl, dt = be.alloc_permanent(rows * 4), be.alloc_permanent(rows * max_blocks * 4)
+    dx = be.alloc_permanent(rows * hidden * 4)
+    try:
+        for launch in range(24):
+            lens = np.clip(np.exp(rng.normal(math.log(600), 0.9, rows)), 1, max_blocks * bs).astype(np.int32)
+            lens[launch % rows] = 0
+            lens[(launch + 3) % rows] = 512 * (1 + launch % 4)
+            lens[(launch + 7) % rows] = 512 * (1 + launch % 3) + 1
+            perm = rng.permutation(nblocks).astype(np.int32)
+            tables = np.zeros((rows, max_blocks), dtype=np.int32)
+            off = 0
+            for i, L in enumerate(lens):
+                nb = (int(L) + bs - 1) // bs
+                tables[i, :nb] = perm[off:off + nb]
+                off += nb
+            be.to_device(dl, lens)
+            be.to_device(dt, tables)
+            outs = []
+            for merge in (True, False):
+                be.set_attn_merge(merge)
+                be.to_device(dx, x)
+                be.sdpa_paged_decode_ragged(dq, dpool, True, dt, dl, None, rows, max_blocks, bs, hq, hk, d, scale, max_blocks * bs)
+                be.decode_ffn(None, dx, qw["wo"], dnw, eps, qw["w1"], qw["w3"], qw["w2"], rows, None)
+                outs.append(be.download(dx, (rows, hidden), np.float32))
+            assert np.array_equal(outs[0].view(np.uint32), outs[1].view(np.uint32)), "launch %d" % launch
+            if launch == 0:
+                attn = nx.sdpa_paged_decode_batched(q.reshape(rows, hq, d), pool, tables, bs, hq, hk, d, scale, lens)
+                attn = np.where((lens > 0)[:, None], attn.reshape(rows, hq * d), 0.0).astype(np.float32)
+                x1 = nx.add(x, nx.matmul_quant(fmt, attn, raw["wo"], rows, hidden, hq * d))
+                h2 = nx.rmsnorm(x1, nw, rows, hidden, eps)
+                g = nx.matmul_quant(fmt, h2, raw["w1"], rows, ffn, hidden)
+                u = nx.matmul_quant(fmt, h2, raw["w3"], rows, ffn, hidden)
+                want = nx.add(x1, nx.matmul_quant(fmt, nx.silu_mul(g, u), raw["w2"], rows, hidden, ffn))
+                _close(outs[0], want, 2e-4, 2e-5 * np.abs(want).max(), "merged in the kernel, against the oracle")
+    finally:
+        be.set_attn_merge(True)
+        for p in list(dW.values()) + [dpool, dq, dnw, dl, dt, dx]:
+            be.free(p)
+        be.reset_pool()

@@ -56,6 +56,10 @@ class HipBackend:
         """Calls C-ABI function `name` with the backend handle prepended; raises on error."""
         self._ck(getattr(self._lib, name)(self._h, *args))
 
+    def set_attn_merge(self, on):
+        """vx_backend_set_attn_merge: the decode attention kernel merges its own splits (default) or not."""
+        self.call("vx_backend_set_attn_merge", int(bool(on)))
+
     def scratch_generation(self):
         """How often the library's own scratch buffers have moved (a kept graph is stale once this changes)."""
         return int(self._lib.vx_scratch_generation(self._h))

@@ -353,7 +353,7 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     // The caller's max_kv_len sized the partial sums (max_splits per sequence and head). A length above it is
     // attended over its first max_splits * TPW tokens by every kernel of the path alike: defined, and inside the
     // buffers.
-    kv_len = min(kv_len, max_splits * tps);  // (tps: tokens per split, a multiple of the block size; ATTN_TPW with a work list)
+    kv_len = min(kv_len, max_splits * tps);  // (tps: tokens per split, a multiple of the block size)
     const int t_begin = split * tps;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1299,7 +1299,7 @@ static __device__ __align__(256) unsigned char scratch[FIXED_WS_BYTES];
 // Tokens per split of the streaming kernels: ATTN_TPW; half of it for grouped queries at heads of 64 / 128 (fewer
 // kv heads, so fewer workgroups per token, and the matrix-core form's per-block work is small: measured faster at
 // every batch tried); and down to a quarter of ATTN_TPW while that many splits would leave most of the chip idle
-// (a single sequence). The work list from vx_pack_batch is cut in ATTN_TPW tokens, so it serves the first only.
+// (a single sequence). vx_pack_batch leaves a work list for each of the first two.
 int split_tokens(vx_backend *be, int D, int G, int batch, int num_kv_heads, int max_kv_len) {
     static const int cus = [&] {
         int n = 0;
@@ -1322,8 +1322,6 @@ template <int D, int G>
 int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *bt_matrix, const int32_t *bt_rows,
                int max_blocks, const int32_t *kv_lens, float *out, int batch, int num_q_heads, int num_kv_heads,
                float scale, int max_kv_len, bool fixed) {
-    // Tokens per split: ATTN_TPW; a quarter of it at least when that many splits would leave most of the chip
-    // idle (a single sequence). The work list from vx_pack_batch is cut in ATTN_TPW tokens, so it serves the first only.
     const int tps = split_tokens(be, D, G, batch, num_kv_heads, max_kv_len);
     int max_splits = ceil_div(max_kv_len, tps);
     const size_t need = split_bytes(D, batch, num_q_heads, max_splits);
@@ -1343,17 +1341,19 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
     }
     // With a work list from vx_pack_batch for these lengths the grid's second dimension runs over its items
     // (at most max_splits per sequence, as max_kv_len bounds every length); otherwise over (split, sequence).
-    const bool listed = tps == TPW && be->items.valid && be->items.kv_lens == kv_lens && be->items.table_rows == bt_rows &&
-                        be->items.batch == batch &&
-                        ((size_t)batch * max_splits + 1) * 4 <= be->items.bytes / sizeof(int32_t) &&
+    const bool half_list = tps == TPW / 2;
+    const size_t list_off = half_list ? (be->items.cap + 1) * 4 : 0, list_cap = half_list ? 2 * be->items.cap : be->items.cap;
+    const bool listed = (tps == TPW || half_list) && be->items.valid && be->items.kv_lens == kv_lens &&
+                        be->items.table_rows == bt_rows && be->items.batch == batch && (size_t)batch * max_splits <= list_cap &&
                         (size_t)batch * max_splits <= 65535;
+    const int32_t *const list = listed ? be->items.buf + list_off : nullptr;
     dim3 grid(num_kv_heads, listed ? batch * max_splits : max_splits, listed ? 1 : batch);
     // out == NULL leaves the result to vx_decode_ffn(attn = NULL): as split partial sums, and - where the shape
     // allows - already merged by the workgroups that finish last: prepared as that call's first operand, or, for
     // a single row, as plain floats behind the partial sums (what the matrix-vector product reads).
     MergeOut mg;
     float *plain = nullptr;
-    static const bool no_merge = getenv("VEXEL_HIP_NO_ATTN_MERGE") != nullptr;
+    const bool no_merge = !be->attn_merge;
     constexpr int GD = G * D;
     // whole merge units, of at most one chunk per wave of the merging workgroup (with more - 7 chunks per two KV heads
     // at 28 / 4 heads of 128 - the merge at the launch's tail costs what the separate merge launch does)
@@ -1380,7 +1380,7 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
             paged_decode_gqa_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
                                                                         max_blocks, kv_lens, ws, num_q_heads,
                                                                         num_kv_heads, scale, max_splits,
-                                                                        listed ? be->items.buf : nullptr, mg, tps);
+                                                                        list, mg, tps);
             launched = true;
         }
     }
@@ -1389,7 +1389,7 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
             paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
                                                                         max_blocks, kv_lens, ws, num_q_heads,
                                                                         num_kv_heads, scale, max_splits,
-                                                                        listed ? be->items.buf : nullptr, mg, tps);
+                                                                        list, mg, tps);
     }
     VX_CHECK_LAUNCH();
     if (!fixed) be->split.batch = 0;  // (the fixed area is not where vx_decode_ffn looks for a split result)

@@ -98,7 +98,14 @@ int vx_backend_create(int device_id, vx_backend **out) {
         VX_CHECK_HIP(hipMalloc((void **)&be->ones, sizeof ones));
         VX_CHECK_HIP(hipMemcpy(be->ones, ones, sizeof ones, hipMemcpyHostToDevice));
     }
+    be->attn_merge = getenv("VEXEL_HIP_NO_ATTN_MERGE") == nullptr;
     *out = be;
+    return VX_OK;
+}
+
+int vx_backend_set_attn_merge(vx_backend *be, int on) {
+    if (!be) return VX_ERR_INVALID;
+    be->attn_merge = on != 0;
     return VX_OK;
 }
 

@@ -96,12 +96,16 @@ struct vx_backend {
         int merged = 0;  // the attention kernel also left the merged rows as the prepared activation (gemm_ws)
         const float *plain = nullptr;  // a single row: the attention kernel also left the merged row here, as floats
     } split;
+    // the decode attention kernel merges its own splits where the geometry allows (vx_backend_set_attn_merge; the
+    // initial value is off when VEXEL_HIP_NO_ATTN_MERGE is set in the environment at vx_backend_create)
+    bool attn_merge = true;
     int32_t *attn_cnt = nullptr;  // arrival counters of the merging attention kernel, VX_ATTN_CNT of them, zero between launches
     size_t attn_ws_bytes = 0;
-    // Work list of the ragged decode attention, written on the device by vx_pack_batch next to kv_lens:
+    // Work lists of the ragged decode attention, written on the device by vx_pack_batch next to kv_lens:
     // buf[0] = number of items, then from buf[4] one record of four ints per item (batch index, split, kv
     // length, block-table row), full splits first, then the sequences' partial last splits from the longest
-    // down. Valid for attention calls that pass the same kv_lens and table-row pointers and batch, until the
+    // down; items of ATTN_TPW tokens, with room for `cap` of them, and behind that room (from buf[4 (cap + 1)])
+    // the same for items of ATTN_TPW / 2 tokens. Valid for attention calls that pass the same kv_lens and table-row pointers and batch, until the
     // library is asked to write into the kv_lens array by other means.
     struct {
         int32_t *buf = nullptr;
@@ -109,6 +113,7 @@ struct vx_backend {
         const int32_t *kv_lens = nullptr;
         const int32_t *table_rows = nullptr;
         int batch = 0;
+        size_t cap = 0;
         bool valid = false;
     } items;
     float *ones = nullptr;       // 64 floats of 1.0 on the device (row factors of an unscaled activation)

@@ -71,34 +71,43 @@ __global__ void __launch_bounds__(PK_THREADS) pack_batch_kernel(
     if (any_fail) {
         if (tid == 0) {
             *status = 1;
-            if (items) items[0] = 0;
+            if (items) {
+                items[0] = 0;
+                items[(items_cap + 1) * 4] = 0;
+            }
         }
         return;
     }
     if (items) {
-        // The attention work list: one item per ATTN_TPW tokens of a sequence. Equal (full) items first, in
-        // batch order; then the partial last items from the longest down, so that the kernel's last
-        // workgroups are its smallest.
+        // The attention work lists: one item per ATTN_TPW tokens of a sequence, and a second list in items of half
+        // that for the kernels that take half as many tokens per workgroup (grouped queries). Equal (full) items
+        // first, in batch order; then the partial last items from the longest down, so that the kernel's last
+        // workgroups are its smallest. The second list sits behind the first one's capacity.
         const int len = act ? pos + ql : 0;
-        const int full = len / ATTN_TPW, rest = len % ATTN_TPW;
-        int total_full;
-        const int off = block_exclusive_scan(full, sm, &total_full);
-        sm[tid] = rest;
-        __syncthreads();
-        int before = 0, partials = 0;  // partial items ahead of this one; partial items in all
-        for (int j = 0; j < batch; j++) {
-            const int rj = sm[j];
-            partials += rj > 0;
-            before += (rj > rest) || (rj == rest && rj > 0 && j < tid);
+        for (int which = 0; which < 2; which++) {
+            const int tpw = which == 0 ? ATTN_TPW : ATTN_TPW / 2;
+            const int cap = which == 0 ? items_cap : 2 * items_cap;
+            int32_t *list = which == 0 ? items : items + (items_cap + 1) * 4;
+            const int full = len / tpw, rest = len % tpw;
+            int total_full;
+            const int off = block_exclusive_scan(full, sm, &total_full);
+            sm[tid] = rest;
+            __syncthreads();
+            int before = 0, partials = 0;  // partial items ahead of this one; partial items in all
+            for (int j = 0; j < batch; j++) {
+                const int rj = sm[j];
+                partials += rj > 0;
+                before += (rj > rest) || (rj == rest && rj > 0 && j < tid);
+            }
+            __syncthreads();
+            const int n_items = total_full + partials;
+            if (n_items <= cap) {
+                int4 *rec = (int4 *)(list + 4);  // one 16-byte record per item: everything a workgroup needs to start
+                for (int s2 = 0; s2 < full; s2++) rec[off + s2] = make_int4(tid, s2, len, slot);
+                if (rest > 0) rec[total_full + before] = make_int4(tid, full, len, slot);
+            }
+            if (tid == 0) list[0] = n_items <= cap ? n_items : -1;  // -1: the list did not fit, not to be used
         }
-        __syncthreads();
-        const int n_items = total_full + partials;
-        if (n_items <= items_cap) {
-            int4 *rec = (int4 *)(items + 4);  // one 16-byte record per item: everything a workgroup needs to start
-            for (int s2 = 0; s2 < full; s2++) rec[off + s2] = make_int4(tid, s2, len, slot);
-            if (rest > 0) rec[total_full + before] = make_int4(tid, full, len, slot);
-        }
-        if (tid == 0) items[0] = n_items <= items_cap ? n_items : -1;  // -1: the list did not fit, not to be used
     }
     if (act) {
         for (int j = 0; j < need; j++)
@@ -153,7 +162,7 @@ extern "C" int vx_pack_batch(vx_backend *be, const int32_t *seq_slots, const int
     int32_t *items = nullptr;
     be->items.valid = false;
     if (batch <= 32767 && per_seq <= 65535 &&
-        ensure_ws(be, (void **)&be->items.buf, &be->items.bytes, (cap + 1) * 4 * sizeof(int32_t), "attention work list") == VX_OK)
+        ensure_ws(be, (void **)&be->items.buf, &be->items.bytes, (3 * cap + 2) * 4 * sizeof(int32_t), "attention work list") == VX_OK)
         items = be->items.buf;
     pack_batch_kernel<<<1, PK_THREADS, 0, be->stream>>>(seq_slots, positions, q_lens, batch, total_tokens,
                                                         block_tables, max_blocks, num_blocks, free_list, free_count,
@@ -164,6 +173,7 @@ extern "C" int vx_pack_batch(vx_backend *be, const int32_t *seq_slots, const int
         be->items.kv_lens = kv_lens;
         be->items.table_rows = seq_slots;
         be->items.batch = batch;
+        be->items.cap = cap;
         be->items.valid = true;
     }
     return VX_OK;

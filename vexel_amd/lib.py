@@ -17,6 +17,7 @@ SIGNATURES = {
     "vx_backend_create": (_i, [_i, C.POINTER(_vp)]),
     "vx_backend_destroy": (None, [_vp]),
     "vx_backend_device": (_i, [_vp]),
+    "vx_backend_set_attn_merge": (_i, [_vp, _i]),
     "vx_last_error": (C.c_char_p, []),
     "vx_scratch_generation": (C.c_uint64, [_vp]),
     "vx_alloc": (_vp, [_vp, _sz]),
