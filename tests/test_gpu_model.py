@@ -812,6 +812,34 @@ def test_pool_errors_and_lifecycle(be):
     mr.close()
 
 
+def test_fragment_insert_that_runs_out_of_blocks_leaves_the_sequence_as_it_was(be):
+    """A fragment of 3 blocks is put behind a 13-token prompt in a pool with one free block: the insertion fails, and the
+    sequence keeps its table, its length and its logits, the pool its counts (host-forced failure, no kernel involved);
+    after room is made the same insertion succeeds and, undone again, leaves the logits of the next step unchanged."""
+    from vexel_amd.backend import VexelError
+    cfg = om.ModelConfig(num_layers=2, hidden=256, num_heads=4, num_kv_heads=2, head_dim=64, ffn=256, vocab=256)
+    omodel = om.random_model(cfg, 43, nx.FMT_Q4_0, nx.FMT_Q4_0, max_blocks=8)
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=8, max_seqs=4, max_blocks_per_seq=8, max_batch=4)
+    mr.prefill_with_paged_kv(list(range(37)), 1, 0)            # 3 blocks
+    mr.cache_fragment("doc", 1)
+    mr.delete_sequence(1)
+    mr.prefill_with_paged_kv(list(range(64)), 3, 0)            # 4 more: one block left
+    mr.create_sequence(2)
+    mr.prefill_with_paged_kv(list(range(13)), 2, 0)            # the last one
+    table, stats = mr.block_table(2), mr.block_stats()
+    with pytest.raises(VexelError, match="no free blocks"):
+        mr.insert_fragment(2, "doc", 13)
+    assert mr.block_table(2) == table and mr.block_stats() == stats and mr.seq_len(2) == 13
+    before, _ = mr.decode_with_paged_kv_batched([7], [2], [13])
+    mr.truncate_sequence(2, 13)
+    mr.delete_sequence(3)
+    assert mr.insert_fragment(2, "doc", 13) == 37 and mr.seq_len(2) == 50 and len(mr.block_table(2)) == 4
+    mr.truncate_sequence(2, 13)
+    again, _ = mr.decode_with_paged_kv_batched([7], [2], [13])
+    assert np.array_equal(before.view(np.uint32), again.view(np.uint32))
+    mr.close()
+
+
 # ------------------------------------------------------------------ the architectures beside LLaMA
 def _arch_config(name):
     """Small models with the layer shapes of Phi-2 (LayerNorm, biases, 32 of 80 head dimensions rotated in split

@@ -125,6 +125,7 @@ void vx_backend_destroy(vx_backend *be) {
     if (be->misc_ws) (void)hipFree(be->misc_ws);
     if (be->prep_sync) (void)hipFree(be->prep_sync);
     if (be->rope_tab) (void)hipFree(be->rope_tab);
+    if (be->shift_tab) (void)hipFree(be->shift_tab);
     if (be->attn_cnt) (void)hipFree(be->attn_cnt);
     if (be->ones) (void)hipFree(be->ones);
     if (be->host_stage) (void)hipHostFree(be->host_stage);

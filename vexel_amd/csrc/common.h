@@ -87,6 +87,10 @@ struct vx_backend {
     int rope_tab_rows = 0, rope_tab_dim = 0;
     float rope_tab_theta = 0.f;
     uint64_t rope_tab_epoch = 0, write_epoch = 1;
+    // cos / sin of vx_paged_kv_copy_shifted's rotation per pair, kept while (shift, theta, head_dim) stay the same
+    void *shift_tab = nullptr;
+    int shift_tab_shift = 0, shift_tab_dim = 0;
+    float shift_tab_theta = 0.f;
     void *attn_ws = nullptr;     // split-KV partial results
     void *attn_fixed_ws = nullptr;  // this device's copy of the fixed-size partial-sum area (never allocated or freed)
     // attention left in split form by vx_sdpa_paged_decode_ragged(out = NULL), to be merged by vx_decode_ffn

@@ -626,12 +626,13 @@ int vx_paged_kv_copy_shifted(vx_backend *be, void *kv_pool, int pool_is_f16, con
     VX_REQUIRE(head_dim > 0 && head_dim % 2 == 0 && num_kv_heads > 0 && block_size > 0, "vx_paged_kv_copy_shifted: bad shape");
     if (num_tokens == 0) return VX_OK;
     const int half = head_dim / 2;
-    VX_REQUIRE((size_t)half * sizeof(float2) <= be->host_stage_bytes && (size_t)half * sizeof(float2) <= be->misc_ws_bytes,
-               "vx_paged_kv_copy_shifted: head_dim %d too large", head_dim);
-    if (shift != 0) {
-        // the table must not change under a copy still in flight from the call before
-        VX_CHECK_HIP(hipStreamSynchronize(be->stream));
-        float2 *t = (float2 *)be->host_stage;
+    VX_REQUIRE(half <= VX_ROPE_TAB_PAIRS * 2, "vx_paged_kv_copy_shifted: head_dim %d too large", head_dim);
+    if (shift != 0 && !(be->shift_tab && be->shift_tab_shift == shift && be->shift_tab_theta == theta && be->shift_tab_dim == head_dim)) {
+        // The angles depend on (shift, theta, head_dim) only: worked out and uploaded when that changes (once per
+        // fragment insertion, not once per layer), into a table of their own that nothing else writes.
+        VX_REQUIRE(!be->capturing, "vx_paged_kv_copy_shifted: a new shift table during graph capture");
+        if (!be->shift_tab) VX_CHECK_HIP(hipMalloc(&be->shift_tab, (size_t)VX_ROPE_TAB_PAIRS * 2 * sizeof(float2)));
+        std::vector<float2> t(half);
         for (int j = 0; j < half; j++) {                       // backend/cpu/backend.go:262-266
             const double ex = (double)(2 * j) / (double)head_dim;
             const float freq = (float)(1.0 / pow((double)theta, ex));
@@ -641,16 +642,19 @@ int vx_paged_kv_copy_shifted(vx_backend *be, void *kv_pool, int pool_is_f16, con
             volatile double cd = cos((double)angle), sd = sin((double)angle);
             t[j] = make_float2((float)cd, (float)sd);
         }
-        VX_CHECK_HIP(hipMemcpyAsync(be->misc_ws, t, (size_t)half * sizeof(float2), hipMemcpyHostToDevice, be->stream));
-        VX_CHECK_HIP(hipStreamSynchronize(be->stream));        // the staging buffer is free again for the next caller
+        VX_CHECK_HIP(hipStreamSynchronize(be->stream));        // a copy in flight may still read the previous table
+        VX_CHECK_HIP(hipMemcpy(be->shift_tab, t.data(), (size_t)half * sizeof(float2), hipMemcpyHostToDevice));
+        be->shift_tab_shift = shift;
+        be->shift_tab_theta = theta;
+        be->shift_tab_dim = head_dim;
     }
     if (pool_is_f16)
         copy_shift_paged_kv_kernel<_Float16><<<num_tokens, 256, 0, be->stream>>>((_Float16 *)kv_pool, src_slots, dst_slots,
-                                                                                 (const float2 *)be->misc_ws, num_kv_heads,
+                                                                                 (const float2 *)be->shift_tab, num_kv_heads,
                                                                                  head_dim, block_size, shift != 0);
     else
         copy_shift_paged_kv_kernel<float><<<num_tokens, 256, 0, be->stream>>>((float *)kv_pool, src_slots, dst_slots,
-                                                                              (const float2 *)be->misc_ws, num_kv_heads,
+                                                                              (const float2 *)be->shift_tab, num_kv_heads,
                                                                               head_dim, block_size, shift != 0);
     VX_CHECK_LAUNCH();
     return VX_OK;

@@ -766,7 +766,20 @@ int vh_fragment_insert(vh_model *m, int64_t seq_id, const char *name, int insert
     if ((insert_pos + n - 1) / bs + 1 > c.max_blocks_per_seq && n > 0)
         return fail("sequence %lld: %d tokens at position %d exceed max_blocks_per_seq %d", (long long)seq_id, n, insert_pos,
                     c.max_blocks_per_seq);
-    VHC(m->pool.ensure_blocks(*s, insert_pos + n));
+    const size_t blocks_before = s->table.size();
+    // what the sequence gained goes back when a later step fails (the reference's InsertFragment has no failing step
+    // after its allocation, paged_cache.go:302-314)
+    auto roll_back = [&]() {
+        while (s->table.size() > blocks_before) {
+            m->pool.release_block(s->table.back());
+            s->table.pop_back();
+        }
+        s->dirty = true;
+    };
+    if (m->pool.ensure_blocks(*s, insert_pos + n) != VH_OK) {
+        roll_back();
+        return VH_ERR;
+    }
     if (n > 0) {
         std::vector<int32_t> slots(2 * (size_t)n);
         for (int t = 0; t < n; t++) {
@@ -774,13 +787,23 @@ int vh_fragment_insert(vh_model *m, int64_t seq_id, const char *name, int insert
             const int p = insert_pos + t;
             slots[n + t] = s->table[p / bs] * bs + p % bs;
         }
-        int32_t *d_slots = (int32_t *)vx_alloc(m->be, slots.size() * 4);
-        if (!d_slots) return fail("vx_alloc: %s", vx_last_error());
-        VXC(vx_to_device(m->be, d_slots, slots.data(), slots.size() * 4));
-        for (int l = 0; l < c.num_layers; l++)
-            VXC(vx_paged_kv_copy_shifted(m->be, m->kv[l], c.kv_fp16, d_slots, d_slots + n, n, c.num_kv_heads, c.head_dim, bs,
-                                         insert_pos, c.rope_theta));
-        VXC(vx_sync(m->be));
+        // a buffer of its own, freed below: the per-step pool is only recycled by the next decode call
+        int32_t *d_slots = (int32_t *)vx_alloc_permanent(m->be, slots.size() * 4);
+        if (!d_slots) {
+            roll_back();
+            return fail("vx_alloc_permanent: %s", vx_last_error());
+        }
+        int rc = vx_to_device(m->be, d_slots, slots.data(), slots.size() * 4);
+        // (the K rotation's table of angles is the same for every layer: the library keeps it from the first call)
+        for (int l = 0; l < c.num_layers && rc == VX_OK; l++)
+            rc = vx_paged_kv_copy_shifted(m->be, m->kv[l], c.kv_fp16, d_slots, d_slots + n, n, c.num_kv_heads, c.head_dim, bs,
+                                          insert_pos, c.rope_theta);
+        if (rc == VX_OK) rc = vx_sync(m->be);
+        vx_free(m->be, d_slots);  // (drains the stream first)
+        if (rc != VX_OK) {
+            roll_back();
+            return fail("fragment copy: %s", vx_last_error());
+        }
     }
     s->seq_len = insert_pos + n;  // paged_cache.go:316-319
     s->dirty = true;
