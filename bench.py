@@ -317,30 +317,83 @@ def time_step_gemms(be, mr, c, rows):
     res, total_us, total_bytes = {}, 0.0, 0
     for name, (fmt, ptrs, n, k) in shapes:
         be.prepare_act(acts[k], rows, k)
-        for p in ptrs[:2]:
-            be.matmul_quant_prepared(fmt, p, out, None, rows, n, k)
-        be.sync()
         reps = 3
-        be.timer_start()
-        for _ in range(reps):
-            for p in ptrs:
-                be.matmul_quant_prepared(fmt, p, out, None, rows, n, k)
-        us = be.timer_stop_ms() * 1e3 / (reps * len(ptrs))
+        timed = []
+        for dst in (None, out):       # the launch alone, as the step issues it; then with its reduction kernel
+            for p in ptrs[:2]:
+                be.matmul_quant_prepared(fmt, p, dst, None, rows, n, k)
+            be.sync()
+            be.timer_start()
+            for _ in range(reps):
+                for p in ptrs:
+                    be.matmul_quant_prepared(fmt, p, dst, None, rows, n, k)
+            timed.append(be.timer_stop_ms() * 1e3 / (reps * len(ptrs)))
+        us = timed[0]
         nbytes = int(n * k * bpe[fmt]) + rows * k * 4 + rows * n * 4
-        res[name] = {"n": n, "k": k, "us": round(us, 2), "bytes": nbytes, "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        res[name] = {"n": n, "k": k, "us": round(us, 2), "us_with_reduction": round(timed[1], 2), "bytes": nbytes,
+                     "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+        if name == "Q|K|V":
+            fused = time_fused_qkv(be, lw, c, rows, acts[k])
+            if fused is not None:   # what the step launches for Q|K|V: the projection with RoPE and the KV store in its epilogue
+                res[name]["us_projection_alone"] = res[name]["us"]
+                res[name]["us"] = us = round(fused, 2)
+                res[name]["frac"] = round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)
         total_us += us
         total_bytes += nbytes
     be.free(out)
     for p in acts.values():
         be.free(p)
-    return {"bound": "hbm", "kernel": "qgemm_wave_kernel (the step's four projection launches per layer, M=%d)" % rows,
+    return {"bound": "hbm", "kernel": "qstream_kernel / qgemm_wave_kernel (the step's four projection launches per layer, M=%d)" % rows,
             "achieved": total_bytes / total_us / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": total_bytes / total_us / 1e3 / HBM_PEAK_GBS,
             "traffic": GEMM_TRAFFIC_PER_ALGORITHMIC_BYTE * total_bytes if rows == BATCH else None,
             "bytes_per_layer": total_bytes,
             "us_per_layer": total_us, "launches": res,
-            "note": "HIP events around back-to-back launches over all layers' weights; a launch with split K "
-                    "includes its reduction kernel"}
+            "note": "HIP events around back-to-back launches over all layers' weights; us: the projection launch alone, "
+                    "as the fused decode blocks issue it (K slices' sums consumed by the next prepare kernel; Q|K|V: "
+                    "with its RoPE + KV-store epilogue, timed as vx_decode_attn_qkv minus the prepare kernel alone); "
+                    "us_with_reduction: with the separate reduction kernel of the unfused call"}
+
+
+def time_fused_qkv(be, lw, c, rows, x):
+    """The decode step's Q|K|V launch by itself: vx_decode_attn_qkv (RMSNorm prepare, then the projection that rotates
+    Q and K from the step's table of angles and stores K and V into a paged pool) over every layer's weights, minus
+    the prepare kernel timed alone. A scratch pool of 2 * rows slots takes the stores. None when the fused entry point
+    does not take these weights."""
+    from vexel_amd import lib
+    hq, hk, d, h = c["num_heads"], c["num_kv_heads"], c["head_dim"], c["hidden"]
+    qws = [[be.qweight(*l[n]) for n in ("wq", "wk", "wv")] for l in lw]
+    if rows > 32 or not be.decode_attn_qkv_supported(*qws[0], d):
+        return None
+    kvd = hk * d
+    nblocks = (2 * rows + BLOCK - 1) // BLOCK
+    pool = be.alloc_permanent(nblocks * 2 * BLOCK * kvd * 2)
+    dq = be.alloc_permanent(rows * hq * d * 4)
+    ones = be.upload(np.ones(h, dtype=np.float32), permanent=True)
+    dpos = be.upload(np.arange(100, 100 + rows, dtype=np.int32), permanent=True)
+    dslots = be.upload(np.arange(rows, dtype=np.int32), permanent=True)
+    theta = float(c.get("rope_theta", 10000.0))
+    reps = 3
+
+    def fused(q):
+        be.decode_attn_qkv(x, ones, 1e-5, False, q[0], q[1], q[2], rows, dpos, dslots, pool, True, hq, hk, d, BLOCK, theta, dq)
+
+    be.rope_table_prepare(dpos, rows, d, theta)
+    for q in qws[:2]:
+        fused(q)
+    be.sync()
+    be.timer_start()
+    for _ in range(reps):
+        for q in qws:
+            fused(q)
+    both = be.timer_stop_ms() * 1e3 / (reps * len(qws))
+    be.timer_start()
+    for _ in range(reps * len(qws)):
+        be.rmsnorm_prepare(x, ones, None, rows, h, 1e-5)
+    prep = be.timer_stop_ms() * 1e3 / (reps * len(qws))
+    for p in (pool, dq, ones, dpos, dslots):
+        be.free(p)
+    return both - prep
 
 
 def kernel_report(be):

@@ -202,7 +202,10 @@ int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, floa
  * 16-byte aligned. Results equal vx_matmul_quant on the same values bit for bit.
  *   vx_prepare_act       a itself
  *   vx_rmsnorm_prepare   Backend.RMSNorm(x, weight) (backend.go:345); also stored to out when out != NULL
- *   vx_silu_mul_prepare  Backend.SiLUMul(gate, up) (backend.go:360); also stored to out when out != NULL */
+ *   vx_silu_mul_prepare  Backend.SiLUMul(gate, up) (backend.go:360); also stored to out when out != NULL
+ * vx_matmul_quant_prepared with out == NULL (and residual == NULL) issues the projection's launch alone, as the
+ * fused decode blocks do: the sums of its K slices stay in a backend workspace that only the library reads. That
+ * form exists to time the launch by itself; it returns nothing to the caller. */
 int vx_prepare_act(vx_backend *be, const float *a, int m, int k);
 int vx_rmsnorm_prepare(vx_backend *be, const float *x, const float *weight, float *out, int rows, int cols, float eps);
 int vx_silu_mul_prepare(vx_backend *be, const float *gate, const float *up, float *out, int rows, int cols);

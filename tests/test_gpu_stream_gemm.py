@@ -1,7 +1,8 @@
-"""GPU parity of the decode-batch GEMM over load-time packed Q4_0 matrices (vx_qweight_pack): the packed copy
-dequantises to the reference's values bit for bit, the products match the CPU oracle's MatMulQ4_0
+"""GPU parity of the decode-batch GEMM over load-time packed Q4_0 and Q8_0 matrices (vx_qweight_pack): the packed
+copy dequantises to the reference's values bit for bit, the products match the CPU oracle's MatMulQ4_0 / MatMulQ8_0
 (backend/cpu/cpu.go:842-911) to float32 summation order on every cut of the matrix the planner makes, a row's bits
-do not depend on the batch it sits in, and the fused decode blocks give the oracle's layer with packed weights."""
+do not depend on the batch it sits in (2 .. 32 rows; 33 .. 64 rows), and the fused decode blocks give the oracle's
+layer with packed weights."""
 import numpy as np
 import pytest
 
@@ -26,24 +27,28 @@ def _close(got, want, rtol, atol, what=""):
         what, err.max(), lim.reshape(-1)[err.argmax()])
 
 
-def _packed(be, w, n, k):
+FMTS = [nx.FMT_Q4_0, nx.FMT_Q8_0]
+
+
+def _packed(be, w, n, k, fmt=nx.FMT_Q4_0):
     dw = be.upload(w, permanent=True)
-    qw = be.qweight(nx.FMT_Q4_0, dw, n, k)
+    qw = be.qweight(fmt, dw, n, k)
     assert be.qweight_pack(qw)
     assert be.qweight_is_packed(qw)
     return dw, qw
 
 
+@pytest.mark.parametrize("fmt", FMTS)
 @pytest.mark.parametrize("n,k", [(16, 256), (48, 1024), (1040, 512)])
-def test_packed_copy_dequantises_bit_exact(be, n, k):
+def test_packed_copy_dequantises_bit_exact(be, n, k, fmt):
     rng = np.random.default_rng(n + k)
-    w = qz.random_quant(nx.FMT_Q4_0, rng, n, k)
-    w.reshape(-1)[2:18] = rng.integers(0, 256, 16, dtype=np.uint8)   # every nibble position carries arbitrary codes
-    dw, qw = _packed(be, w, n, k)
+    w = qz.random_quant(fmt, rng, n, k)
+    w.reshape(-1)[2:34] = rng.integers(0, 256, 32, dtype=np.uint8)   # every code position carries arbitrary codes
+    dw, qw = _packed(be, w, n, k, fmt)
     dst = be.alloc(n * k * 4)
     be.dequantize_packed(qw, dst)
     got = be.download(dst, (n * k,), np.float32)
-    want = nx.dequantize(nx.FMT_Q4_0, w, n * k)
+    want = nx.dequantize(fmt, w, n * k)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
     be.free(dw)
     assert not be.qweight_is_packed(qw)                          # the copy goes with the matrix
@@ -52,9 +57,9 @@ def test_packed_copy_dequantises_bit_exact(be, n, k):
 
 def test_pack_refuses_other_formats_and_shapes(be):
     rng = np.random.default_rng(0)
-    w = qz.random_quant(nx.FMT_Q8_0, rng, 32, 256)
+    w = qz.random_quant(nx.FMT_Q4_K, rng, 32, 256)
     dw = be.upload(w, permanent=True)
-    assert not be.qweight_pack(be.qweight(nx.FMT_Q8_0, dw, 32, 256))
+    assert not be.qweight_pack(be.qweight(nx.FMT_Q4_K, dw, 32, 256))
     assert not be.qweight_pack(be.qweight(nx.FMT_Q4_0, dw, 24, 256))     # rows not a multiple of 16
     assert not be.qweight_pack(be.qweight(nx.FMT_Q4_0, dw, 32, 128))     # K not a multiple of 256
     be.free(dw)
@@ -63,50 +68,59 @@ def test_pack_refuses_other_formats_and_shapes(be):
 # (n, k): one tile; K slices of one and two half chunks per wave; slices with an odd share of half chunks;
 # more tiles than workgroups in a slice; a 7B down-projection's K
 @pytest.mark.parametrize("n,k", [(16, 256), (80, 1024), (96, 2048), (1040, 2304), (4112, 512), (64, 4352), (208, 11008)])
-@pytest.mark.parametrize("m", [2, 5, 16, 17, 32])
-def test_matmul_packed_vs_oracle(be, n, k, m):
+@pytest.mark.parametrize("m", [2, 5, 16, 17, 32, 33, 48, 64])
+@pytest.mark.parametrize("fmt", FMTS)
+def test_matmul_packed_vs_oracle(be, n, k, m, fmt):
     rng = np.random.default_rng(n * 7 + k + m)
-    w = qz.random_quant(nx.FMT_Q4_0, rng, n, k)
+    w = qz.random_quant(fmt, rng, n, k)
     a = (rng.standard_normal((m, k)) * (1.0 + 3.0 * (rng.random((1, k)) < 0.1))).astype(np.float32)
-    want = nx.matmul_quant(nx.FMT_Q4_0, a, w, m, n, k)
-    dw, qw = _packed(be, w, n, k)
+    want = nx.matmul_quant(fmt, a, w, m, n, k)
+    dw, qw = _packed(be, w, n, k, fmt)
     da = be.upload(a)
     dout = be.alloc(m * n * 4)
-    be.matmul_q4_0(da, dw, dout, m, n, k)
+    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
     got = be.download(dout, (m, n), np.float32)
     scale = np.abs(want).max()
     _close(got, want, 2e-5, 2e-6 * scale + 1e-7, "packed matmul %dx%dx%d" % (m, n, k))
     # the unpacked path on the same inputs: float32 summation order apart
     be.qweight_unpack(qw)
-    be.matmul_q4_0(da, dw, dout, m, n, k)
+    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
     plain = be.download(dout, (m, n), np.float32)
     _close(got, plain, 0, 3e-6 * scale + 1e-7, "packed vs unpacked")
     be.free(dw)
     be.reset_pool()
 
 
-def test_matmul_packed_rows_independent_of_batch(be):
+@pytest.mark.parametrize("fmt", FMTS)
+def test_matmul_packed_rows_independent_of_batch(be, fmt):
     """A row has the same bits in a batch of 2, of 16, of 17 and of 32 rows (the cut of the matrix depends on its
-    shape and the device only; 16 rows and fewer run the one-tile form of the kernel)."""
+    shape and the device only; 16 rows and fewer run the one-tile form of the kernel), and in a batch of 33, of 40
+    and of 64 rows (four activation tiles a step: K is cut into narrower slices there)."""
     rng = np.random.default_rng(11)
     n, k = 208, 4096
-    w = qz.random_quant(nx.FMT_Q4_0, rng, n, k)
-    a = rng.standard_normal((32, k)).astype(np.float32)
-    dw, qw = _packed(be, w, n, k)
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((64, k)).astype(np.float32)
+    dw, qw = _packed(be, w, n, k, fmt)
     da = be.upload(a)
 
     def batch(first, rows):
         d = be.alloc(rows * n * 4)
-        be.matmul_quant(nx.FMT_Q4_0, da + first * k * 4, dw, d, None, rows, n, k)
+        be.matmul_quant(fmt, da + first * k * 4, dw, d, None, rows, n, k)
         return be.download(d, (rows, n), np.float32)
 
     full = batch(0, 32)
     for first, rows in ((0, 2), (5, 2), (30, 2), (0, 16), (3, 17), (16, 16), (9, 7)):
         part = batch(first, rows)
         assert np.array_equal(part.view(np.uint32), full[first:first + rows].view(np.uint32)), (first, rows)
+    full64 = batch(0, 64)
+    for first, rows in ((0, 33), (20, 40), (31, 33), (7, 57)):
+        part = batch(first, rows)
+        assert np.array_equal(part.view(np.uint32), full64[first:first + rows].view(np.uint32)), (first, rows)
+    scale = np.abs(full).max()
+    _close(full64[:32], full, 0, 3e-6 * scale, "a row in 64 against the same row in 32")
     res = rng.standard_normal((32, n)).astype(np.float32)
     dres, d = be.upload(res), be.alloc(32 * n * 4)
-    be.matmul_quant(nx.FMT_Q4_0, da, dw, d, dres, 32, n, k)
+    be.matmul_quant(fmt, da, dw, d, dres, 32, n, k)
     assert np.array_equal(be.download(d, (32, n), np.float32).view(np.uint32), (res + full).view(np.uint32))
     be.free(dw)
     be.reset_pool()
@@ -128,21 +142,23 @@ def test_rewriting_the_matrix_drops_the_packed_copy(be):
     be.reset_pool()
 
 
-@pytest.mark.parametrize("rows", [2, 7, 32])
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("rows", [2, 7, 32, 64])
 @pytest.mark.parametrize("hq,hk,d,hidden,ffn", [(8, 8, 64, 512, 1024), (8, 2, 128, 1024, 2816), (32, 32, 128, 4096, 1024)])
-def test_fused_decode_blocks_with_packed_weights(be, rows, hq, hk, d, hidden, ffn):
+def test_fused_decode_blocks_with_packed_weights(be, rows, hq, hk, d, hidden, ffn, fmt):
     """RMSNorm -> Q|K|V -> RoPE -> KV store (one launch with the table of angles) and Wo -> residual -> RMSNorm ->
     gate|up -> SiLU*up -> down -> residual on packed weights against the oracle's operators."""
     rng = np.random.default_rng(rows + hq + hidden)
     bs, nblocks, theta, eps = 16, 8, 10000.0, 1e-5
     qd, kvd = hq * d, hk * d
-    mk = lambda n, k: qz.quantize_q4_0((rng.standard_normal((n, k)) * 0.05).astype(np.float32)).reshape(-1)
+    quant = qz.quantize_q4_0 if fmt == nx.FMT_Q4_0 else qz.quantize_q8_0
+    mk = lambda n, k: quant((rng.standard_normal((n, k)) * 0.05).astype(np.float32)).reshape(-1)
     raw = {"wq": (mk(qd, hidden), qd, hidden), "wk": (mk(kvd, hidden), kvd, hidden), "wv": (mk(kvd, hidden), kvd, hidden),
            "wo": (mk(hidden, qd), hidden, qd), "w1": (mk(ffn, hidden), ffn, hidden), "w3": (mk(ffn, hidden), ffn, hidden),
            "w2": (mk(hidden, ffn), hidden, ffn)}
     dev, qws = {}, {}
     for name, (w, n, k) in raw.items():
-        dev[name], qws[name] = _packed(be, w, n, k)
+        dev[name], qws[name] = _packed(be, w, n, k, fmt)
     x = rng.standard_normal((rows, hidden)).astype(np.float32)
     nw_attn = (1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
     nw_ffn = (1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
@@ -153,16 +169,16 @@ def test_fused_decode_blocks_with_packed_weights(be, rows, hq, hk, d, hidden, ff
 
     # oracle
     h = nx.rmsnorm(x, nw_attn, rows, hidden, eps)
-    q = nx.matmul_quant(nx.FMT_Q4_0, h, raw["wq"][0], rows, qd, hidden)
-    kk = nx.matmul_quant(nx.FMT_Q4_0, h, raw["wk"][0], rows, kvd, hidden)
-    vv = nx.matmul_quant(nx.FMT_Q4_0, h, raw["wv"][0], rows, kvd, hidden)
+    q = nx.matmul_quant(fmt, h, raw["wq"][0], rows, qd, hidden)
+    kk = nx.matmul_quant(fmt, h, raw["wk"][0], rows, kvd, hidden)
+    vv = nx.matmul_quant(fmt, h, raw["wv"][0], rows, kvd, hidden)
     want_q, want_k = nx.rope_positions(q, kk, d, hq, hk, positions, d, theta, False)
     attn = rng.standard_normal((rows, qd)).astype(np.float32)
-    x1 = nx.add(x, nx.matmul_quant(nx.FMT_Q4_0, attn, raw["wo"][0], rows, hidden, qd))
+    x1 = nx.add(x, nx.matmul_quant(fmt, attn, raw["wo"][0], rows, hidden, qd))
     h2 = nx.rmsnorm(x1, nw_ffn, rows, hidden, eps)
-    g = nx.matmul_quant(nx.FMT_Q4_0, h2, raw["w1"][0], rows, ffn, hidden)
-    u = nx.matmul_quant(nx.FMT_Q4_0, h2, raw["w3"][0], rows, ffn, hidden)
-    want_x = nx.add(x1, nx.matmul_quant(nx.FMT_Q4_0, nx.silu_mul(g, u), raw["w2"][0], rows, hidden, ffn))
+    g = nx.matmul_quant(fmt, h2, raw["w1"][0], rows, ffn, hidden)
+    u = nx.matmul_quant(fmt, h2, raw["w3"][0], rows, ffn, hidden)
+    want_x = nx.add(x1, nx.matmul_quant(fmt, nx.silu_mul(g, u), raw["w2"][0], rows, hidden, ffn))
 
     # GPU
     dx, dnw, dnf = be.upload(x, permanent=True), be.upload(nw_attn, permanent=True), be.upload(nw_ffn, permanent=True)

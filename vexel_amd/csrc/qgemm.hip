@@ -1975,7 +1975,9 @@ int run_prepared(vx_backend *be, int fmt, const void *b, float *out, const float
     segs.n_end[0] = segs.n_end[1] = segs.n_end[2] = n;
     int rc = finalize_row_norm(be);  // the GEMM epilogue and the reduce kernel read plain row factors
     if (rc) return rc;
-    return launch_gemm_fmt(be, fmt, segs, n, out, residual, false, m, k, nullptr);
+    // without an output: the projection launch as the fused decode blocks issue it, its K slices' sums left in the
+    // workspace for the consumer that follows there
+    return launch_gemm_fmt(be, fmt, segs, n, out, residual, out == nullptr, m, k, nullptr);
 }
 
 }  // namespace
@@ -2031,7 +2033,7 @@ int vx_matmul_quant_prepared(vx_backend *be, int fmt, const void *b, float *out,
                              int k) {
     int rc = enter(be);
     if (rc) return rc;
-    VX_REQUIRE(b && out && n >= 1, "vx_matmul_quant_prepared: bad arguments");
+    VX_REQUIRE(b && n >= 1 && (out || !residual), "vx_matmul_quant_prepared: bad arguments");
     rc = check_fmt(fmt, k);
     if (rc) return rc;
     VX_REQUIRE(be->prep_m == m && be->prep_k == k, "vx_matmul_quant_prepared: the prepared activation is %dx%d, not %dx%d",

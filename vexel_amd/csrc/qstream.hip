@@ -39,7 +39,6 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr int HUNIT = 1152;      // bytes of one (tile, half chunk)
 constexpr int NW = 8;            // waves per workgroup
 constexpr int ACC_TILES = 8;     // tiles whose sums can wait in LDS between the passes of a wide slice
 
@@ -86,13 +85,74 @@ __device__ __forceinline__ half8 unpack_q4(uint32_t w, uint32_t k64) {
     return r;
 }
 
+// Eight biased bytes (q + 128, two dwords) -> exact integers q as f16: a byte under 0x64 is the f16 1024 + byte. Byte
+// positions 0, 2, 1, 3 of a dword hold consecutive slots, so that each byte permute yields a finished pair.
+__device__ __forceinline__ half8 unpack_q8(uint32_t w0, uint32_t w1) {
+    const uint32_t c64 = 0x64646464u;
+    const half2v off = {(_Float16)1152.f, (_Float16)1152.f};  // 1024 + 128
+    const half2v h0 = as_h2(__builtin_amdgcn_perm(w0, c64, 0x00060004u)) - off, h1 = as_h2(__builtin_amdgcn_perm(w0, c64, 0x00070005u)) - off;
+    const half2v h2 = as_h2(__builtin_amdgcn_perm(w1, c64, 0x00060004u)) - off, h3 = as_h2(__builtin_amdgcn_perm(w1, c64, 0x00070005u)) - off;
+    half8 r;
+    r[0] = h0[0]; r[1] = h0[1]; r[2] = h1[0]; r[3] = h1[1];
+    r[4] = h2[0]; r[5] = h2[1]; r[6] = h3[0]; r[7] = h3[1];
+    return r;
+}
+__device__ __forceinline__ float half_of(uint32_t w, int hi) {
+    _Float16 dh;
+    const uint16_t d16 = (uint16_t)(hi ? (w >> 16) : (w & 0xFFFFu));
+    __builtin_memcpy(&dh, &d16, 2);
+    return (float)dh;
+}
+
+// What the kernel needs to know of a packed format: the unit's size, what a lane requests of it (Ring), and how the
+// request becomes block j's operand and scale.
+struct SQ4_0 {
+    static constexpr int FMT = VX_Q4_0, UNIT = 1152, SCALES_AT = 1024, BLOCK_BYTES = 18;
+    struct Ring {
+        u32x4 c;
+        u32x2 s;
+    };
+    static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
+        Ring x;
+        x.c = gload<u32x4>(u + lane * 16);
+        x.s = gload<u32x2>(u + SCALES_AT + ln * 8);
+        return x;
+    }
+    static __device__ __forceinline__ half8 codes(const Ring &x, int j, uint32_t k64) { return unpack_q4(x.c[j], k64); }
+    static __device__ __forceinline__ float scale(const Ring &x, int j) { return half_of(x.s[j >> 1], j & 1); }
+};
+// Q8_0: a unit is 2176 bytes, lane l = 16 g + r owns 32 of the first 2048: block j's eight codes at 8 j, as q + 128,
+// slot s at byte (s & 4) + {0, 2, 1, 3}[s & 3]; row r's four f16 scales at 2048 + 8 r. 34 bytes per block as in GGUF.
+struct SQ8_0 {
+    static constexpr int FMT = VX_Q8_0, UNIT = 2176, SCALES_AT = 2048, BLOCK_BYTES = 34;
+    struct Ring {
+        u32x4 c0, c1;
+        u32x2 s;
+    };
+    static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
+        Ring x;
+        x.c0 = gload<u32x4>(u + lane * 32);
+        x.c1 = gload<u32x4>(u + lane * 32 + 16);
+        x.s = gload<u32x2>(u + SCALES_AT + ln * 8);
+        return x;
+    }
+    static __device__ __forceinline__ half8 codes(const Ring &x, int j, uint32_t) {
+        return j == 0 ? unpack_q8(x.c0[0], x.c0[1]) : j == 1 ? unpack_q8(x.c0[2], x.c0[3]) : j == 2 ? unpack_q8(x.c1[0], x.c1[1]) : unpack_q8(x.c1[2], x.c1[3]);
+    }
+    static __device__ __forceinline__ float scale(const Ring &x, int j) { return half_of(x.s[j >> 1], j & 1); }
+};
+__host__ __device__ inline int q8_byte_of_slot(int slot) {
+    const int pos[4] = {0, 2, 1, 3};
+    return (slot & 4) + pos[slot & 3];
+}
+
 // ------------------------------------------------------------------------------------------------ pack / unpack
 // grid = (tiles, half chunks), block = 64: lane l writes its 16 code bytes, lanes 0 .. 15 their row's scales.
 __global__ void __launch_bounds__(64) pack_q4_0_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ packed, int n_hc) {
     const int T = blockIdx.x, hc = blockIdx.y, lane = threadIdx.x, r = lane & 15, g = lane >> 4;
     const size_t row_bytes = (size_t)n_hc * 4 * 18;
     const uint8_t *row = raw + (size_t)(T * 16 + r) * row_bytes + (size_t)hc * 4 * 18;
-    uint8_t *u = packed + ((size_t)T * n_hc + hc) * HUNIT;
+    uint8_t *u = packed + ((size_t)T * n_hc + hc) * SQ4_0::UNIT;
     uint32_t out[4];
     for (int j = 0; j < 4; j++) {
         const uint8_t *blk = row + j * 18;
@@ -120,7 +180,7 @@ __global__ void __launch_bounds__(256) dequant_packed_q4_0_kernel(const uint8_t 
     const int row = (int)(idx / k), col = (int)(idx % k);
     const int T = row >> 4, r = row & 15, hc = col >> 7, j = (col >> 5) & 3, e = col & 31;
     const int n_hc = k >> 7;
-    const uint8_t *u = packed + ((size_t)T * n_hc + hc) * HUNIT;
+    const uint8_t *u = packed + ((size_t)T * n_hc + hc) * SQ4_0::UNIT;
     int g = 0, nib = 0;
     for (int gg = 0; gg < 4; gg++)
         for (int i = 0; i < 8; i++)
@@ -133,6 +193,53 @@ __global__ void __launch_bounds__(256) dequant_packed_q4_0_kernel(const uint8_t 
     _Float16 d;
     __builtin_memcpy(&d, u + 1024 + r * 8 + j * 2, 2);
     dst[idx] = __fmul_rn((float)d, (float)(q - 8));
+}
+
+__global__ void __launch_bounds__(64) pack_q8_0_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ packed, int n_hc) {
+    const int T = blockIdx.x, hc = blockIdx.y, lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+    const size_t row_bytes = (size_t)n_hc * 4 * 34;
+    const uint8_t *row = raw + (size_t)(T * 16 + r) * row_bytes + (size_t)hc * 4 * 34;
+    uint8_t *u = packed + ((size_t)T * n_hc + hc) * SQ8_0::UNIT;
+    uint32_t out[8];
+    for (int j = 0; j < 4; j++) {
+        const uint8_t *blk = row + j * 34;
+        uint32_t w[2] = {0, 0};
+        for (int slot = 0; slot < 8; slot++) {
+            const int at = q8_byte_of_slot(slot);
+            w[at >> 2] |= (uint32_t)(uint8_t)(blk[2 + elt_of(g, slot)] ^ 0x80u) << (8 * (at & 3));
+        }
+        out[2 * j] = w[0];
+        out[2 * j + 1] = w[1];
+    }
+    *(u32x4 *)(u + lane * 32) = (u32x4){out[0], out[1], out[2], out[3]};
+    *(u32x4 *)(u + lane * 32 + 16) = (u32x4){out[4], out[5], out[6], out[7]};
+    if (g == 0) {
+        uint16_t d[4];
+        for (int j = 0; j < 4; j++) d[j] = (uint16_t)(row[j * 34] | (row[j * 34 + 1] << 8));
+        *(u32x2 *)(u + SQ8_0::SCALES_AT + r * 8) = (u32x2){(uint32_t)d[0] | ((uint32_t)d[1] << 16), (uint32_t)d[2] | ((uint32_t)d[3] << 16)};
+    }
+}
+
+// scale * float32(q) as gguf.DequantizeQ8_0 computes it (pkg/gguf/dequant.go:58-95), read from the packed form.
+__global__ void __launch_bounds__(256) dequant_packed_q8_0_kernel(const uint8_t *__restrict__ packed, float *__restrict__ dst, int n,
+                                                                  int k) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)n * k) return;
+    const int row = (int)(idx / k), col = (int)(idx % k);
+    const int T = row >> 4, r = row & 15, hc = col >> 7, j = (col >> 5) & 3, e = col & 31;
+    const int n_hc = k >> 7;
+    const uint8_t *u = packed + ((size_t)T * n_hc + hc) * SQ8_0::UNIT;
+    int g = 0, slot = 0;
+    for (int gg = 0; gg < 4; gg++)
+        for (int i = 0; i < 8; i++)
+            if (elt_of(gg, i) == e) {
+                g = gg;
+                slot = i;
+            }
+    const int q = (int)(int8_t)(u[(g * 16 + r) * 32 + j * 8 + q8_byte_of_slot(slot)] ^ 0x80u);
+    _Float16 d;
+    __builtin_memcpy(&d, u + SQ8_0::SCALES_AT + r * 8 + j * 2, 2);
+    dst[idx] = __fmul_rn((float)d, (float)q);
 }
 
 // ------------------------------------------------------------------------------------------------ the GEMM
@@ -163,18 +270,13 @@ template <int MT> struct APhase {
     half8 h[4][MT], l[4][MT];
     float4v cs[MT];
 };
-struct WHalf {
-    u32x4 c;
-    u32x2 s;
-};
-
 struct StreamShape {
     int M, Mpad, N, n_hc, npass, t_end0, t_end1;
 };
 
 // grid = (row groups, K slices), block = 512. PH: half chunks a wave holds per pass (1 or 2); RG: tiles per
 // reduction; EPI: finish Q|K|V rows (one slice).
-template <int PH, int RG, int MT, bool EPI>
+template <class W, int PH, int RG, int MT, bool EPI>
 __global__ void __launch_bounds__(64 * NW, 1)
 qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, const uint8_t *__restrict__ pw2,
                const half8 *__restrict__ a_tiles, const float *__restrict__ a_cscale, const float *__restrict__ a_inv_scale,
@@ -193,8 +295,8 @@ qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1,
     const int sb = n_hc / (int)gridDim.y, sr = n_hc % (int)gridDim.y;
     const int h0 = blockIdx.y * sb + min((int)blockIdx.y, sr), nh = sb + ((int)blockIdx.y < sr ? 1 : 0);
 
-    const size_t tile_stride = (size_t)n_hc * HUNIT;
-    const int lane_c = lane * 16, lane_s = 1024 + ln * 8;
+    const size_t tile_stride = (size_t)n_hc * W::UNIT;
+    typedef typename W::Ring WHalf;
     // the packed matrices' addresses and tile ends as scalars (the same in every lane)
     // (through readfirstlane: selecting among plain kernel arguments becomes an indexed load of the argument
     // block, copied to scratch memory for it)
@@ -218,11 +320,8 @@ qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1,
         const bool valid0 = wave < nhp, valid1 = PH > 1 && NW + wave < nhp;
         const int hc0 = hp + min(wave, nhp - 1), hc1 = hp + min(NW + wave, nhp - 1);
         auto ldw = [&](int tile, int p) __attribute__((always_inline)) {
-            const uint8_t *u = uniform_ptr(tile_base(t0 + min(tile, nt - 1), w0, w1, w2, e0, e1, tile_stride) + (size_t)(p == 0 ? hc0 : hc1) * HUNIT);
-            WHalf x;
-            x.c = gload<u32x4>(u + lane_c);
-            x.s = gload<u32x2>(u + lane_s);
-            return x;
+            const uint8_t *u = uniform_ptr(tile_base(t0 + min(tile, nt - 1), w0, w1, w2, e0, e1, tile_stride) + (size_t)(p == 0 ? hc0 : hc1) * W::UNIT);
+            return W::load(u, lane, ln);
         };
         APhase<MT> A[PH];
 #pragma unroll
@@ -260,12 +359,8 @@ qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1,
                         for (int m = 0; m < MT; m++) tmp[m] = (float4v){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int j = 0; j < 4; j++) {
-                            const half8 wb = unpack_q4(x.c[j], k64);
-                            const uint32_t sw = x.s[j >> 1];
-                            _Float16 dh;
-                            const uint16_t d16 = (uint16_t)((j & 1) ? (sw >> 16) : (sw & 0xFFFFu));
-                            __builtin_memcpy(&dh, &d16, 2);
-                            const float d = (float)dh;
+                            const half8 wb = W::codes(x, j, k64);
+                            const float d = W::scale(x, j);
                             float4v P[MT];
 #pragma unroll
                             for (int m = 0; m < MT; m++)
@@ -363,16 +458,18 @@ struct StreamPlan {
     int g, s, ph, npass;  // row groups, K slices, half chunks per wave and pass, passes; g == 0: not served
 };
 
-// The cut of an [n_tiles * 16, n_hc * 128] matrix for a device of `cus` compute units. With the epilogue the whole
+// The cut of an [n_tiles * 16, n_hc * 128] matrix for a device of `cus` compute units; max_ph: how many half chunks'
+// operands a wave's registers hold (2; 1 at four activation tiles). With the epilogue the whole
 // K stays in one workgroup (passes of 16 half chunks); otherwise K is sliced so that a slice is one pass, and
 // further while a workgroup would own fewer than four tiles and slices stay at least four half chunks wide: every
 // workgroup first pulls its slice of the activation (128 bytes per column) through its compute unit's L1, which
 // costs as much as the weights of a few tiles. VEXEL_HIP_SPLAN="NxK:G,S;..." overrides the choice (tuning).
-StreamPlan stream_plan(int n_tiles, int n_hc, int cus, bool epi, int N, int K) {
+StreamPlan stream_plan(int n_tiles, int n_hc, int cus, bool epi, int N, int K, int max_ph) {
     StreamPlan pl = {0, 1, 1, 1};
-    if (n_tiles < 1 || n_hc < 1) return pl;
+    if (n_tiles < 1 || n_hc < 1 || (epi && max_ph < 2)) return pl;
     static const char *env = getenv("VEXEL_HIP_SPLAN");
-    int s = epi ? 1 : ceil_div(n_hc, 16), g = 0;
+    const int cap = NW * max_ph;  // half chunks a workgroup's registers hold
+    int s = epi ? 1 : ceil_div(n_hc, cap), g = 0;
     if (!epi) {
         while (true) {
             const int gg = std::max(1, std::min(cus / s, n_tiles));
@@ -388,7 +485,7 @@ StreamPlan stream_plan(int n_tiles, int n_hc, int cus, bool epi, int N, int K) {
         const char *p = strstr(env, key);
         int eg = 0, es = 0;
         if (p && sscanf(p + strlen(key), "%d,%d", &eg, &es) == 2 && eg >= 1 && es >= 1 && es <= n_hc && eg <= n_tiles &&
-            ceil_div(n_hc, es) <= 16) {
+            ceil_div(n_hc, es) <= cap) {
             g = eg;
             s = es;
         }
@@ -449,8 +546,8 @@ void stream_drop_all(vx_backend *be) {
 // Resolves up to three row segments of raw matrices (each a run of registered matrices laid end to end) into packed
 // matrices; false when any part has no packed copy.
 static bool resolve(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, PackedSegs *out) {
-    if (fmt != VX_Q4_0 || be->packed.empty()) return false;
-    const size_t row_bytes = (size_t)K / 32 * 18;
+    if ((fmt != VX_Q4_0 && fmt != VX_Q8_0) || be->packed.empty()) return false;
+    const size_t row_bytes = (size_t)K / 32 * (fmt == VX_Q4_0 ? 18 : 34);
     int np = 0, rows_done = 0;
     for (int i = 0; i < nseg && rows_done < N; i++) {
         const int seg_rows = n_end[i] - rows_done;
@@ -479,7 +576,8 @@ static bool resolve(vx_backend *be, int fmt, const uint8_t *const *w, const int 
 bool stream_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M, bool epi) {
     static const char *off = getenv("VEXEL_HIP_STREAM_OFF");
     if (off && atoi(off)) return false;
-    if (M < 2 || M > 32 || N % 16 != 0 || K % 256 != 0 || N < 16) return false;
+    if (M < 2 || M > 64 || N % 16 != 0 || K % 256 != 0 || N < 16) return false;
+    if (epi && M > 32) return false;
     // With the epilogue the whole K stays in one workgroup, which walks it in passes of 16 half chunks; every pass
     // starts its requests anew, and for two passes and more the launch takes longer than the wave-private kernel's
     // (7B Q|K|V, 32 rows: 23.8 against 20.9 us). VEXEL_HIP_STREAM_EPI=1 takes it anyway (measurements).
@@ -489,7 +587,33 @@ bool stream_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int 
     if (!resolve(be, fmt, w, n_end, nseg, N, K, &ps)) return false;
     int cus = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0) cus = 256;
-    return stream_plan(N / 16, K / 128, cus, epi, N, K).g > 0;
+    return stream_plan(N / 16, K / 128, cus, epi, N, K, M > 32 ? 1 : 2).g > 0;
+}
+
+template <class W>
+static void launch_stream(vx_backend *be, const StreamPlan &pl, dim3 grid, int mt, bool fin, const PackedSegs &ps, const PrepView &pv,
+                          float *partial, const StreamShape &a, const QkvEpi &e) {
+#define VX_STREAM_LAUNCH(PH_, RG_, MT_, EPI_)                                                                                  \
+    qstream_kernel<W, PH_, RG_, MT_, EPI_><<<grid, 64 * NW, 0, be->stream>>>(ps.w[0], ps.w[1], ps.w[2], pv.tiles, pv.cscale, pv.inv_scale, \
+                                                                              partial, a, e)
+    if (mt == 4) {
+        VX_STREAM_LAUNCH(1, 2, 4, false);
+    } else if (fin) {
+        if (pl.ph == 2) {
+            if (mt == 2) VX_STREAM_LAUNCH(2, 2, 2, true);
+            else VX_STREAM_LAUNCH(2, 2, 1, true);
+        } else {
+            if (mt == 2) VX_STREAM_LAUNCH(1, 2, 2, true);
+            else VX_STREAM_LAUNCH(1, 2, 1, true);
+        }
+    } else if (pl.ph == 2) {
+        if (mt == 2) VX_STREAM_LAUNCH(2, 2, 2, false);
+        else VX_STREAM_LAUNCH(2, 2, 1, false);
+    } else {
+        if (mt == 2) VX_STREAM_LAUNCH(1, 4, 2, false);
+        else VX_STREAM_LAUNCH(1, 4, 1, false);
+    }
+#undef VX_STREAM_LAUNCH
 }
 
 // Launches the streaming kernel; the K slices' sums go to be->part_ws as [slice][M][N] (raw: no row factors), or, with
@@ -501,8 +625,10 @@ int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_e
     static int cus = 0;
     if (cus == 0 && (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0)) cus = 256;
     const bool fin = epi && epi->q_out;
-    const StreamPlan pl = stream_plan(N / 16, K / 128, cus, fin, N, K);
-    if (pl.g == 0) return VX_ERR_UNSUPPORTED;
+    const int mt = mpad / 16;
+    if (mt != 1 && mt != 2 && mt != 4) return VX_ERR_UNSUPPORTED;
+    const StreamPlan pl = stream_plan(N / 16, K / 128, cus, fin, N, K, mt == 4 ? 1 : 2);
+    if (pl.g == 0 || (mt == 4 && (fin || pl.ph != 1))) return VX_ERR_UNSUPPORTED;
     StreamShape a;
     a.M = M;
     a.Mpad = mpad;
@@ -519,26 +645,8 @@ int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_e
         partial = (float *)be->part_ws;
     }
     dim3 grid(pl.g, pl.s);
-    const int mt = mpad / 16;
-#define VX_STREAM_LAUNCH(PH_, RG_, MT_, EPI_)                                                                                  \
-    qstream_kernel<PH_, RG_, MT_, EPI_><<<grid, 64 * NW, 0, be->stream>>>(ps.w[0], ps.w[1], ps.w[2], pv.tiles, pv.cscale, pv.inv_scale, \
-                                                                           partial, a, e)
-    if (fin) {
-        if (pl.ph == 2) {
-            if (mt == 2) VX_STREAM_LAUNCH(2, 2, 2, true);
-            else VX_STREAM_LAUNCH(2, 2, 1, true);
-        } else {
-            if (mt == 2) VX_STREAM_LAUNCH(1, 2, 2, true);
-            else VX_STREAM_LAUNCH(1, 2, 1, true);
-        }
-    } else if (pl.ph == 2) {
-        if (mt == 2) VX_STREAM_LAUNCH(2, 2, 2, false);
-        else VX_STREAM_LAUNCH(2, 2, 1, false);
-    } else {
-        if (mt == 2) VX_STREAM_LAUNCH(1, 4, 2, false);
-        else VX_STREAM_LAUNCH(1, 4, 1, false);
-    }
-#undef VX_STREAM_LAUNCH
+    if (fmt == VX_Q4_0) launch_stream<SQ4_0>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
+    else launch_stream<SQ8_0>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
     VX_CHECK_LAUNCH();
     if (ks_out) *ks_out = pl.s;
     return VX_OK;
@@ -553,15 +661,19 @@ int vx_qweight_pack(vx_backend *be, const vx_qweight *w) {
     if (rc) return rc;
     VX_REQUIRE(w && w->data, "vx_qweight_pack: null weight");
     VX_REQUIRE(!be->capturing, "vx_qweight_pack during graph capture");
-    if (w->fmt != VX_Q4_0 || w->n < 16 || w->n % 16 != 0 || w->k < 256 || w->k % 256 != 0) return VX_ERR_UNSUPPORTED;
+    if ((w->fmt != VX_Q4_0 && w->fmt != VX_Q8_0) || w->n < 16 || w->n % 16 != 0 || w->k < 256 || w->k % 256 != 0) return VX_ERR_UNSUPPORTED;
     if (find_packed(be, w->data)) stream_drop_packed(be, w->data);
-    PackedW *pw = new PackedW{nullptr, w->fmt, w->n, w->k, (size_t)w->n * (w->k / 32) * 18};
+    const size_t bytes = (size_t)w->n * (w->k / 32) * (w->fmt == VX_Q4_0 ? 18 : 34);
+    PackedW *pw = new PackedW{nullptr, w->fmt, w->n, w->k, bytes};
     if (hipMalloc(&pw->data, pw->bytes) != hipSuccess) {
         delete pw;
-        set_error("vx_qweight_pack: out of device memory (%zu bytes)", (size_t)w->n * (w->k / 32) * 18);
+        set_error("vx_qweight_pack: out of device memory (%zu bytes)", bytes);
         return VX_ERR_OOM;
     }
-    pack_q4_0_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
+    if (w->fmt == VX_Q4_0)
+        pack_q4_0_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
+    else
+        pack_q8_0_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         (void)hipFree(pw->data);
@@ -596,7 +708,10 @@ int vx_dequantize_packed(vx_backend *be, const vx_qweight *w, float *dst) {
     PackedW *pw = find_packed(be, w->data);
     VX_REQUIRE(pw && pw->fmt == w->fmt && pw->n == w->n && pw->k == w->k, "vx_dequantize_packed: the matrix has no packed copy");
     const size_t total = (size_t)w->n * w->k;
-    dequant_packed_q4_0_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
+    if (pw->fmt == VX_Q4_0)
+        dequant_packed_q4_0_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
+    else
+        dequant_packed_q8_0_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }

@@ -550,6 +550,11 @@ int vh_model_set_head(vh_model *m, const float *embedding, const float *final_no
     m->embedding = embedding;
     m->final_norm = final_norm;
     m->lm_head = *lm_head;
+    // (the output head of a batched model streams a packed copy like the projections)
+    if (m->cfg.max_batch >= 2 && getenv("VEXEL_HIP_NO_PACK") == nullptr) {
+        const int rc = vx_qweight_pack(m->be, lm_head);
+        if (rc != VX_OK && rc != VX_ERR_UNSUPPORTED) return fail("lm_head: %s", vx_last_error());
+    }
     return VH_OK;
 }
 
