@@ -601,11 +601,12 @@ def prefill_probe(be, rows=512, reps=10):
     print(json.dumps(out))
 
 
-def configs_report(be, only=None):
+def configs_report(be, only=None, use_graph=True):
     """Throughput of the benchmark configs other than the north star, each at its real shape (synthetic weights and
     contexts, greedy decode replayed from a hipGraph; config 4 as its two ingredients; config 5 as one verification
     step). Informational: the benchmark line is the north-star workload.
-    only: "1" .. "5" runs that config alone ("4": its decode part; "4p": decode and the prefill chunks)."""
+    only: "1" .. "5" runs that config alone ("4": its decode part; "4p": decode and the prefill chunks).
+    use_graph=False (--no-graph) issues the same device-driven steps launch by launch (for kernel traces)."""
     from vexel_amd import lib
     from oracle import host_logic as hl
     tiny = dict(num_layers=22, hidden=2048, num_heads=32, num_kv_heads=4, head_dim=64, ffn=5632, vocab=32000)
@@ -616,10 +617,10 @@ def configs_report(be, only=None):
     def decode_rate(name, cfg, fmts, ctx, steps, spare_tokens=0):
         mr, ids = build_model(be, ctx, steps + 16, cfg["num_layers"], cfg, fmts, spare_tokens=spare_tokens)
         first = np.random.default_rng(3).integers(0, cfg["vocab"], len(ctx)).astype(np.int32)
-        mr.decode_graph(first, ids, ctx, 4, use_graph=True)
+        mr.decode_graph(first, ids, ctx, 4, use_graph=use_graph)
         be.sync()
         t0 = time.perf_counter()
-        mr.decode_graph(None, None, None, steps, use_graph=True, batch=len(ctx))
+        mr.decode_graph(None, None, None, steps, use_graph=use_graph, batch=len(ctx))
         be.sync()
         dt = time.perf_counter() - t0
         print("%-64s %8.1f tok/s  %7.3f ms/step" % (name, len(ctx) * steps / dt, dt * 1e3 / steps), flush=True)
@@ -813,7 +814,7 @@ def main():
         prefill_probe(be)
         return
     if args.configs_report:
-        configs_report(be, args.only)
+        configs_report(be, args.only, use_graph=not args.no_graph)
         return
     if args.medusa_report:
         medusa_report(be)

@@ -72,11 +72,12 @@ __device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
 
 // Eight nibbles of one dword -> the step's operand: exact integers q - 8 as f16. A nibble under 0x6400's exponent is
 // the f16 1024 + q; one four bits higher is 1024 + 16 q, which one fused multiply-add brings to q - 8 as well.
-__device__ __forceinline__ half8 unpack_q4(uint32_t w, uint32_t k64) {
+// BIAS: what is subtracted from the code (8 for Q4_0, 0 for Q4_K's unsigned codes).
+template <int BIAS> __device__ __forceinline__ half8 unpack_q4(uint32_t w, uint32_t k64) {
     const uint32_t w8 = w >> 8;
     const half2v a = as_h2(and_or(w, 0x000F000Fu, k64)), b = as_h2(and_or(w, 0x00F000F0u, k64));
     const half2v c = as_h2(and_or(w8, 0x000F000Fu, k64)), d = as_h2(and_or(w8, 0x00F000F0u, k64));
-    const half2v m1032 = {(_Float16)-1032.f, (_Float16)-1032.f}, m72 = {(_Float16)-72.f, (_Float16)-72.f};
+    const half2v m1032 = {(_Float16)(-1024.f - BIAS), (_Float16)(-1024.f - BIAS)}, m72 = {(_Float16)(-64.f - BIAS), (_Float16)(-64.f - BIAS)};
     const half2v s16 = {(_Float16)0.0625f, (_Float16)0.0625f};
     const half2v h0 = a + m1032, h1 = b * s16 + m72, h2 = c + m1032, h3 = d * s16 + m72;
     half8 r;
@@ -108,6 +109,7 @@ __device__ __forceinline__ float half_of(uint32_t w, int hi) {
 // request becomes block j's operand and scale.
 struct SQ4_0 {
     static constexpr int FMT = VX_Q4_0, UNIT = 1152, SCALES_AT = 1024, BLOCK_BYTES = 18;
+    static constexpr bool TWO_SCALES = false, HAS_MIN = false;
     struct Ring {
         u32x4 c;
         u32x2 s;
@@ -118,13 +120,38 @@ struct SQ4_0 {
         x.s = gload<u32x2>(u + SCALES_AT + ln * 8);
         return x;
     }
-    static __device__ __forceinline__ half8 codes(const Ring &x, int j, uint32_t k64) { return unpack_q4(x.c[j], k64); }
+    static __device__ __forceinline__ half8 codes(const Ring &x, int j, uint32_t k64) { return unpack_q4<8>(x.c[j], k64); }
     static __device__ __forceinline__ float scale(const Ring &x, int j) { return half_of(x.s[j >> 1], j & 1); }
+    static __device__ __forceinline__ float minimum(const Ring &, int) { return 0.f; }
+};
+// Q4_K (144-byte super-blocks of 8 sub-blocks of 32, pkg/gguf/dequant.go:333-409): element = d1 * q - m1 with
+// d1 = d * sc and m1 = dmin * m per sub-block (both exact float32 products). A half chunk is half a super-block. A
+// unit is 1536 bytes: the codes as in the Q4_0 unit (unsigned), then row r's d1[4] at 1024 + 32 r and m1[4] at
+// 1040 + 32 r. The m1 term multiplies the activation's block sums (prepared with the tiles): one more FMA per output
+// and block. 6 bits per weight against GGUF's 4.5.
+struct SQ4_K {
+    static constexpr int FMT = VX_Q4_K, UNIT = 1536, SCALES_AT = 1024;
+    static constexpr bool TWO_SCALES = false, HAS_MIN = true;
+    struct Ring {
+        u32x4 c;
+        float4v d1, m1;
+    };
+    static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
+        Ring x;
+        x.c = gload<u32x4>(u + lane * 16);
+        x.d1 = gload<float4v>(u + SCALES_AT + ln * 32);
+        x.m1 = gload<float4v>(u + SCALES_AT + ln * 32 + 16);
+        return x;
+    }
+    static __device__ __forceinline__ half8 codes(const Ring &x, int j, uint32_t k64) { return unpack_q4<0>(x.c[j], k64); }
+    static __device__ __forceinline__ float scale(const Ring &x, int j) { return x.d1[j]; }
+    static __device__ __forceinline__ float minimum(const Ring &x, int j) { return x.m1[j]; }
 };
 // Q8_0: a unit is 2176 bytes, lane l = 16 g + r owns 32 of the first 2048: block j's eight codes at 8 j, as q + 128,
 // slot s at byte (s & 4) + {0, 2, 1, 3}[s & 3]; row r's four f16 scales at 2048 + 8 r. 34 bytes per block as in GGUF.
 struct SQ8_0 {
     static constexpr int FMT = VX_Q8_0, UNIT = 2176, SCALES_AT = 2048, BLOCK_BYTES = 34;
+    static constexpr bool TWO_SCALES = false, HAS_MIN = false;
     struct Ring {
         u32x4 c0, c1;
         u32x2 s;
@@ -141,6 +168,48 @@ struct SQ8_0 {
     }
     static __device__ __forceinline__ float scale(const Ring &x, int j) { return half_of(x.s[j >> 1], j & 1); }
 };
+// Q6_K (210-byte super-blocks of 256 elements, pkg/gguf/dequant.go:272-331): a half chunk is half a super-block, and
+// every 16 of its elements carry a scale of their own, so a 32-column step is two v_mfma_f32_16x16x16_f16 per
+// activation half instead of one x32. A unit is 2560 bytes: lane l = 16 g + r owns 32 of the first 2048 — block j's
+// codes at 8 j, one byte each (q, 0 .. 63): elements 4 g .. 4 g + 3, then 16 + 4 g .. 16 + 4 g + 3 — and row r's eight
+// float32 scales d * sc (exact products; element = scale * float32(q - 32) as the reference rounds it) at 2048 + 32 r,
+// scale 2 j + h for elements 16 h .. 16 h + 15 of block j. 10 bits per weight against GGUF's 6.5625.
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ half4v unpack_q6(uint32_t w) {
+    const uint32_t c64 = 0x64646464u;
+    const half2v off = {(_Float16)1056.f, (_Float16)1056.f};  // 1024 + 32
+    const half2v h0 = as_h2(__builtin_amdgcn_perm(w, c64, 0x00060004u)) - off, h1 = as_h2(__builtin_amdgcn_perm(w, c64, 0x00070005u)) - off;
+    half4v r;
+    r[0] = h0[0]; r[1] = h0[1]; r[2] = h1[0]; r[3] = h1[1];  // elements 0, 2, 1, 3 of the four: the activation halves' order
+    return r;
+}
+struct SQ6_K {
+    static constexpr int FMT = VX_Q6_K, UNIT = 2560, SCALES_AT = 2048;
+    static constexpr bool TWO_SCALES = true, HAS_MIN = false;
+    struct Ring {
+        u32x4 c0, c1;
+        float4v s0, s1;
+    };
+    static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
+        Ring x;
+        x.c0 = gload<u32x4>(u + lane * 32);
+        x.c1 = gload<u32x4>(u + lane * 32 + 16);
+        x.s0 = gload<float4v>(u + SCALES_AT + ln * 32);
+        x.s1 = gload<float4v>(u + SCALES_AT + ln * 32 + 16);
+        return x;
+    }
+    // h: which 16 elements of block j
+    static __device__ __forceinline__ half4v codes16(const Ring &x, int j, int h) {
+        const uint32_t w = j < 2 ? x.c0[2 * j + h] : x.c1[2 * (j - 2) + h];
+        return unpack_q6(w);
+    }
+    static __device__ __forceinline__ float scale16(const Ring &x, int j, int h) { return j < 2 ? x.s0[2 * j + h] : x.s1[2 * (j - 2) + h]; }
+    // (unused forms of the one-scale interface)
+    static __device__ __forceinline__ half8 codes(const Ring &, int, uint32_t) { return half8{}; }
+    static __device__ __forceinline__ float scale(const Ring &, int) { return 0.f; }
+    static __device__ __forceinline__ float minimum(const Ring &, int) { return 0.f; }
+};
+
 __host__ __device__ inline int q8_byte_of_slot(int slot) {
     const int pos[4] = {0, 2, 1, 3};
     return (slot & 4) + pos[slot & 3];
@@ -242,6 +311,124 @@ __global__ void __launch_bounds__(256) dequant_packed_q8_0_kernel(const uint8_t 
     dst[idx] = __fmul_rn((float)d, (float)q);
 }
 
+// Q4_K: scale and min of sub-block j of a super-block (get_scale_min_k4, pkg/gguf/dequant.go:400-409)
+__host__ __device__ inline void q4k_scale_min(const uint8_t *q, int j, int *sc, int *mn) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *mn = q[j + 4] & 63;
+    } else {
+        *sc = (q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4);
+        *mn = (q[j + 4] >> 4) | ((q[j] >> 6) << 4);
+    }
+}
+__global__ void __launch_bounds__(64) pack_q4_k_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ packed, int n_hc) {
+    const int T = blockIdx.x, hc = blockIdx.y, lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+    const size_t row_bytes = (size_t)(n_hc / 2) * 144;
+    const uint8_t *sb = raw + (size_t)(T * 16 + r) * row_bytes + (size_t)(hc >> 1) * 144;
+    uint8_t *u = packed + ((size_t)T * n_hc + hc) * SQ4_K::UNIT;
+    uint32_t out[4];
+    for (int j = 0; j < 4; j++) {
+        const int sbi = 4 * (hc & 1) + j;  // sub-block: pair sbi / 2 of 32 bytes, low or high nibbles
+        const uint8_t *qs = sb + 16 + 32 * (sbi >> 1);
+        uint32_t w = 0;
+        for (int nib = 0; nib < 8; nib++) {
+            const int e = elt_of(g, slot_of_nibble(nib));
+            const uint32_t q = (sbi & 1) ? (qs[e] >> 4) : (qs[e] & 0xFu);
+            w |= q << (4 * nib);
+        }
+        out[j] = w;
+    }
+    *(u32x4 *)(u + lane * 16) = (u32x4){out[0], out[1], out[2], out[3]};
+    if (g == 0) {
+        _Float16 dh, mh;
+        const uint16_t d16 = (uint16_t)(sb[0] | (sb[1] << 8)), m16 = (uint16_t)(sb[2] | (sb[3] << 8));
+        __builtin_memcpy(&dh, &d16, 2);
+        __builtin_memcpy(&mh, &m16, 2);
+        float d1[4], m1[4];
+        for (int j = 0; j < 4; j++) {
+            int sc, mn;
+            q4k_scale_min(sb + 4, 4 * (hc & 1) + j, &sc, &mn);
+            d1[j] = __fmul_rn((float)dh, (float)sc);
+            m1[j] = __fmul_rn((float)mh, (float)mn);
+        }
+        *(float4v *)(u + SQ4_K::SCALES_AT + r * 32) = (float4v){d1[0], d1[1], d1[2], d1[3]};
+        *(float4v *)(u + SQ4_K::SCALES_AT + r * 32 + 16) = (float4v){m1[0], m1[1], m1[2], m1[3]};
+    }
+}
+
+// d1 * float32(q) - m1 as gguf.DequantizeQ4_K rounds it (pkg/gguf/dequant.go:333-398), from the packed form.
+__global__ void __launch_bounds__(256) dequant_packed_q4_k_kernel(const uint8_t *__restrict__ packed, float *__restrict__ dst, int n,
+                                                                  int k) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)n * k) return;
+    const int row = (int)(idx / k), col = (int)(idx % k);
+    const int T = row >> 4, r = row & 15, hc = col >> 7, j = (col >> 5) & 3, e = col & 31;
+    const int n_hc = k >> 7;
+    const uint8_t *u = packed + ((size_t)T * n_hc + hc) * SQ4_K::UNIT;
+    int g = 0, nib = 0;
+    for (int gg = 0; gg < 4; gg++)
+        for (int i = 0; i < 8; i++)
+            if (elt_of(gg, slot_of_nibble(i)) == e) {
+                g = gg;
+                nib = i;
+            }
+    const uint32_t w = *(const uint32_t *)(u + (g * 16 + r) * 16 + j * 4);
+    const int q = (int)((w >> (4 * nib)) & 0xFu);
+    float d1, m1;
+    __builtin_memcpy(&d1, u + SQ4_K::SCALES_AT + r * 32 + j * 4, 4);
+    __builtin_memcpy(&m1, u + SQ4_K::SCALES_AT + r * 32 + 16 + j * 4, 4);
+    dst[idx] = __fsub_rn(__fmul_rn(d1, (float)q), m1);
+}
+
+// Q6_K code and scale of element e (0 .. 127) of half nn of a super-block (dequant.go:272-331)
+__host__ __device__ inline int q6k_code(const uint8_t *sb, int nn, int e) {
+    const int j = e >> 5, l = e & 31;
+    const uint8_t ql = sb[64 * nn + 32 * (j & 1) + l], qh = sb[128 + 32 * nn + l];
+    return (int)(((j & 2) ? (ql >> 4) : (ql & 0xF)) | (((qh >> (2 * j)) & 3) << 4));
+}
+__global__ void __launch_bounds__(64) pack_q6_k_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ packed, int n_hc) {
+    const int T = blockIdx.x, hc = blockIdx.y, lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+    const size_t row_bytes = (size_t)(n_hc / 2) * 210;
+    const uint8_t *sb = raw + (size_t)(T * 16 + r) * row_bytes + (size_t)(hc >> 1) * 210;
+    const int nn = hc & 1;
+    uint8_t *u = packed + ((size_t)T * n_hc + hc) * SQ6_K::UNIT;
+    uint32_t out[8];
+    for (int j = 0; j < 4; j++)
+        for (int h = 0; h < 2; h++) {
+            uint32_t w = 0;
+            for (int i = 0; i < 4; i++) w |= (uint32_t)q6k_code(sb, nn, 32 * j + 16 * h + 4 * g + i) << (8 * i);
+            out[2 * j + h] = w;
+        }
+    *(u32x4 *)(u + lane * 32) = (u32x4){out[0], out[1], out[2], out[3]};
+    *(u32x4 *)(u + lane * 32 + 16) = (u32x4){out[4], out[5], out[6], out[7]};
+    if (g == 0) {
+        _Float16 dh;
+        const uint16_t d16 = (uint16_t)(sb[208] | (sb[209] << 8));
+        __builtin_memcpy(&dh, &d16, 2);
+        const float d = (float)dh;
+        float sc[8];
+        for (int i = 0; i < 8; i++) sc[i] = __fmul_rn(d, (float)(int8_t)sb[192 + 8 * nn + i]);
+        *(float4v *)(u + SQ6_K::SCALES_AT + r * 32) = (float4v){sc[0], sc[1], sc[2], sc[3]};
+        *(float4v *)(u + SQ6_K::SCALES_AT + r * 32 + 16) = (float4v){sc[4], sc[5], sc[6], sc[7]};
+    }
+}
+
+// d * float32(sc) * float32(q - 32) as gguf.DequantizeQ6_K rounds it (pkg/gguf/dequant.go:272-331), from the packed form.
+__global__ void __launch_bounds__(256) dequant_packed_q6_k_kernel(const uint8_t *__restrict__ packed, float *__restrict__ dst, int n,
+                                                                  int k) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)n * k) return;
+    const int row = (int)(idx / k), col = (int)(idx % k);
+    const int T = row >> 4, r = row & 15, hc = col >> 7, j = (col >> 5) & 3, e = col & 31;
+    const int n_hc = k >> 7;
+    const uint8_t *u = packed + ((size_t)T * n_hc + hc) * SQ6_K::UNIT;
+    const int h = e >> 4, g = (e & 15) >> 2, i = e & 3;
+    const int q = (int)u[(g * 16 + r) * 32 + j * 8 + h * 4 + i];
+    float s;
+    __builtin_memcpy(&s, u + SQ6_K::SCALES_AT + r * 32 + (2 * j + h) * 4, 4);
+    dst[idx] = __fmul_rn(s, (float)(q - 32));
+}
+
 // ------------------------------------------------------------------------------------------------ the GEMM
 // First unit of tile T among up to three packed matrices (all arguments the same in every lane). A plain function of
 // values: the same selection written over a lambda's captures is compiled into an indexed load of the closure
@@ -266,10 +453,16 @@ struct PackedSegs {  // up to three packed matrices whose rows follow one anothe
     int t_end[3];  // tiles before the end of each
 };
 
-template <int MT> struct APhase {
+template <int MT, bool TWO> struct APhase {
     half8 h[4][MT], l[4][MT];
     float4v cs[MT];
 };
+template <int MT> struct APhase<MT, true> {  // the halves of each operand that belong to the first and the second 16 elements
+    half4v h[4][MT][2], l[4][MT][2];
+    float4v cs[MT];
+};
+__device__ __forceinline__ half4v first16(half8 v) { return __builtin_shufflevector(v, v, 0, 1, 4, 5); }
+__device__ __forceinline__ half4v second16(half8 v) { return __builtin_shufflevector(v, v, 2, 3, 6, 7); }
 struct StreamShape {
     int M, Mpad, N, n_hc, npass, t_end0, t_end1;
 };
@@ -280,7 +473,7 @@ template <class W, int PH, int RG, int MT, bool EPI>
 __global__ void __launch_bounds__(64 * NW, 1)
 qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, const uint8_t *__restrict__ pw2,
                const half8 *__restrict__ a_tiles, const float *__restrict__ a_cscale, const float *__restrict__ a_inv_scale,
-               float *__restrict__ partial, const StreamShape a, const QkvEpi epi) {
+               const float *__restrict__ a_bsum, float *__restrict__ partial, const StreamShape a, const QkvEpi epi) {
     constexpr int D = RG * PH;            // requests in flight per wave
     constexpr int TP = 16 * RG + 4;       // floats per row of a wave's block in LDS
     __shared__ __attribute__((aligned(16))) float red[2][NW][16 * MT * TP];
@@ -323,7 +516,8 @@ qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1,
             const uint8_t *u = uniform_ptr(tile_base(t0 + min(tile, nt - 1), w0, w1, w2, e0, e1, tile_stride) + (size_t)(p == 0 ? hc0 : hc1) * W::UNIT);
             return W::load(u, lane, ln);
         };
-        APhase<MT> A[PH];
+        APhase<MT, W::TWO_SCALES> A[PH];
+        float4v bsum[W::HAS_MIN ? PH : 1][4][MT];
 #pragma unroll
         for (int p = 0; p < PH; p++) {
             const int hc = p == 0 ? hc0 : hc1;
@@ -332,12 +526,27 @@ qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1,
             for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
-                    A[p].h[j][t] = gload<half8>(base + ((size_t)(j * mtiles + t) * 2 + 0) * 64);
-                    A[p].l[j][t] = gload<half8>(base + ((size_t)(j * mtiles + t) * 2 + 1) * 64);
+                    const half8 vh = gload<half8>(base + ((size_t)(j * mtiles + t) * 2 + 0) * 64);
+                    const half8 vl = gload<half8>(base + ((size_t)(j * mtiles + t) * 2 + 1) * 64);
+                    if constexpr (W::TWO_SCALES) {
+                        A[p].h[j][t][0] = first16(vh);
+                        A[p].h[j][t][1] = second16(vh);
+                        A[p].l[j][t][0] = first16(vl);
+                        A[p].l[j][t][1] = second16(vl);
+                    } else {
+                        A[p].h[j][t] = vh;
+                        A[p].l[j][t] = vl;
+                    }
                 }
 #pragma unroll
             for (int t = 0; t < MT; t++)
                 A[p].cs[t] = gload<float4v>(a_cscale + (size_t)(hc >> 1) * a.Mpad + t * 16 + 4 * g);
+            if constexpr (W::HAS_MIN) {  // the activation's block sums of this half chunk, rows 16 t + 4 g + e
+#pragma unroll
+                for (int j = 0; j < 4; j++)
+#pragma unroll
+                    for (int t = 0; t < MT; t++) bsum[p][j][t] = gload<float4v>(a_bsum + (size_t)(hc * 4 + j) * a.Mpad + t * 16 + 4 * g);
+            }
         }
         WHalf ring[D];
 #pragma unroll
@@ -359,18 +568,43 @@ qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1,
                         for (int m = 0; m < MT; m++) tmp[m] = (float4v){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                         for (int j = 0; j < 4; j++) {
-                            const half8 wb = W::codes(x, j, k64);
-                            const float d = W::scale(x, j);
-                            float4v P[MT];
+                            if constexpr (W::TWO_SCALES) {
 #pragma unroll
-                            for (int m = 0; m < MT; m++)
-                                P[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[p].h[j][m], wb, (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                                for (int h = 0; h < 2; h++) {
+                                    const half4v wb = W::codes16(x, j, h);
+                                    const float d = W::scale16(x, j, h);
+                                    float4v P[MT];
 #pragma unroll
-                            for (int m = 0; m < MT; m++) P[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[p].l[j][m], wb, P[m], 0, 0, 0);
+                                    for (int m = 0; m < MT; m++)
+                                        P[m] = __builtin_amdgcn_mfma_f32_16x16x16f16(A[p].h[j][m][h], wb, (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
-                            for (int m = 0; m < MT; m++)
+                                    for (int m = 0; m < MT; m++) P[m] = __builtin_amdgcn_mfma_f32_16x16x16f16(A[p].l[j][m][h], wb, P[m], 0, 0, 0);
 #pragma unroll
-                                for (int e = 0; e < 4; e++) tmp[m][e] = __builtin_fmaf(d, P[m][e], tmp[m][e]);
+                                    for (int m = 0; m < MT; m++)
+#pragma unroll
+                                        for (int e = 0; e < 4; e++) tmp[m][e] = __builtin_fmaf(d, P[m][e], tmp[m][e]);
+                                }
+                            } else {
+                                const half8 wb = W::codes(x, j, k64);
+                                const float d = W::scale(x, j);
+                                float4v P[MT];
+#pragma unroll
+                                for (int m = 0; m < MT; m++)
+                                    P[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[p].h[j][m], wb, (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                                for (int m = 0; m < MT; m++) P[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[p].l[j][m], wb, P[m], 0, 0, 0);
+#pragma unroll
+                                for (int m = 0; m < MT; m++)
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) tmp[m][e] = __builtin_fmaf(d, P[m][e], tmp[m][e]);
+                                if constexpr (W::HAS_MIN) {
+                                    const float mn = -W::minimum(x, j);
+#pragma unroll
+                                    for (int m = 0; m < MT; m++)
+#pragma unroll
+                                        for (int e = 0; e < 4; e++) tmp[m][e] = __builtin_fmaf(mn, bsum[p][j][m][e], tmp[m][e]);
+                                }
+                            }
                         }
 #pragma unroll
                         for (int m = 0; m < MT; m++)
@@ -503,8 +737,28 @@ StreamPlan stream_plan(int n_tiles, int n_hc, int cus, bool epi, int N, int K, i
 struct PackedW {
     void *data;
     int fmt, n, k;
-    size_t bytes;
+    size_t bytes;  // of the raw matrix (what a write into it is checked against)
 };
+
+bool packable(int fmt) { return fmt == VX_Q4_0 || fmt == VX_Q8_0 || fmt == VX_Q6_K || fmt == VX_Q4_K; }
+size_t raw_row_bytes(int fmt, int K) {
+    switch (fmt) {
+    case VX_Q4_0: return (size_t)K / 32 * 18;
+    case VX_Q8_0: return (size_t)K / 32 * 34;
+    case VX_Q4_K: return (size_t)K / 256 * 144;
+    default: return (size_t)K / 256 * 210;
+    }
+}
+int unit_bytes(int fmt) {
+    switch (fmt) {
+    case VX_Q4_0: return SQ4_0::UNIT;
+    case VX_Q8_0: return SQ8_0::UNIT;
+    case VX_Q4_K: return SQ4_K::UNIT;
+    default: return SQ6_K::UNIT;
+    }
+}
+// half chunks whose operands a wave's registers hold beside the format's requests in flight
+int max_ph_of(int fmt, int M) { return (M > 32 || fmt == VX_Q6_K || fmt == VX_Q4_K) ? 1 : 2; }
 
 }  // namespace
 
@@ -546,8 +800,8 @@ void stream_drop_all(vx_backend *be) {
 // Resolves up to three row segments of raw matrices (each a run of registered matrices laid end to end) into packed
 // matrices; false when any part has no packed copy.
 static bool resolve(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, PackedSegs *out) {
-    if ((fmt != VX_Q4_0 && fmt != VX_Q8_0) || be->packed.empty()) return false;
-    const size_t row_bytes = (size_t)K / 32 * (fmt == VX_Q4_0 ? 18 : 34);
+    if (!packable(fmt) || be->packed.empty()) return false;
+    const size_t row_bytes = raw_row_bytes(fmt, K);
     int np = 0, rows_done = 0;
     for (int i = 0; i < nseg && rows_done < N; i++) {
         const int seg_rows = n_end[i] - rows_done;
@@ -578,6 +832,7 @@ bool stream_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int 
     if (off && atoi(off)) return false;
     if (M < 2 || M > 64 || N % 16 != 0 || K % 256 != 0 || N < 16) return false;
     if (epi && M > 32) return false;
+    if (fmt == VX_Q4_K && M > 32) return false;  // the block sums of four activation tiles do not fit the registers
     // With the epilogue the whole K stays in one workgroup, which walks it in passes of 16 half chunks; every pass
     // starts its requests anew, and for two passes and more the launch takes longer than the wave-private kernel's
     // (7B Q|K|V, 32 rows: 23.8 against 20.9 us). VEXEL_HIP_STREAM_EPI=1 takes it anyway (measurements).
@@ -587,7 +842,7 @@ bool stream_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int 
     if (!resolve(be, fmt, w, n_end, nseg, N, K, &ps)) return false;
     int cus = 0;
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0) cus = 256;
-    return stream_plan(N / 16, K / 128, cus, epi, N, K, M > 32 ? 1 : 2).g > 0;
+    return stream_plan(N / 16, K / 128, cus, epi, N, K, max_ph_of(fmt, M)).g > 0;
 }
 
 template <class W>
@@ -595,9 +850,12 @@ static void launch_stream(vx_backend *be, const StreamPlan &pl, dim3 grid, int m
                           float *partial, const StreamShape &a, const QkvEpi &e) {
 #define VX_STREAM_LAUNCH(PH_, RG_, MT_, EPI_)                                                                                  \
     qstream_kernel<W, PH_, RG_, MT_, EPI_><<<grid, 64 * NW, 0, be->stream>>>(ps.w[0], ps.w[1], ps.w[2], pv.tiles, pv.cscale, pv.inv_scale, \
-                                                                              partial, a, e)
+                                                                              pv.bsum, partial, a, e)
     if (mt == 4) {
-        VX_STREAM_LAUNCH(1, 2, 4, false);
+        if constexpr (!W::HAS_MIN) VX_STREAM_LAUNCH(1, 2, 4, false);  // (refused by stream_gemm_ok for a format with a min term)
+    } else if constexpr (W::TWO_SCALES || W::HAS_MIN) {
+        if (mt == 2) VX_STREAM_LAUNCH(1, 4, 2, false);
+        else VX_STREAM_LAUNCH(1, 4, 1, false);
     } else if (fin) {
         if (pl.ph == 2) {
             if (mt == 2) VX_STREAM_LAUNCH(2, 2, 2, true);
@@ -627,8 +885,9 @@ int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_e
     const bool fin = epi && epi->q_out;
     const int mt = mpad / 16;
     if (mt != 1 && mt != 2 && mt != 4) return VX_ERR_UNSUPPORTED;
-    const StreamPlan pl = stream_plan(N / 16, K / 128, cus, fin, N, K, mt == 4 ? 1 : 2);
-    if (pl.g == 0 || (mt == 4 && (fin || pl.ph != 1))) return VX_ERR_UNSUPPORTED;
+    const int max_ph = max_ph_of(fmt, M);
+    const StreamPlan pl = stream_plan(N / 16, K / 128, cus, fin, N, K, max_ph);
+    if (pl.g == 0 || (max_ph == 1 && (fin || pl.ph != 1)) || (fmt == VX_Q4_K && mt == 4)) return VX_ERR_UNSUPPORTED;
     StreamShape a;
     a.M = M;
     a.Mpad = mpad;
@@ -646,7 +905,9 @@ int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_e
     }
     dim3 grid(pl.g, pl.s);
     if (fmt == VX_Q4_0) launch_stream<SQ4_0>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
-    else launch_stream<SQ8_0>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
+    else if (fmt == VX_Q8_0) launch_stream<SQ8_0>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
+    else if (fmt == VX_Q4_K) launch_stream<SQ4_K>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
+    else launch_stream<SQ6_K>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
     VX_CHECK_LAUNCH();
     if (ks_out) *ks_out = pl.s;
     return VX_OK;
@@ -661,19 +922,23 @@ int vx_qweight_pack(vx_backend *be, const vx_qweight *w) {
     if (rc) return rc;
     VX_REQUIRE(w && w->data, "vx_qweight_pack: null weight");
     VX_REQUIRE(!be->capturing, "vx_qweight_pack during graph capture");
-    if ((w->fmt != VX_Q4_0 && w->fmt != VX_Q8_0) || w->n < 16 || w->n % 16 != 0 || w->k < 256 || w->k % 256 != 0) return VX_ERR_UNSUPPORTED;
+    if (!packable(w->fmt) || w->n < 16 || w->n % 16 != 0 || w->k < 256 || w->k % 256 != 0) return VX_ERR_UNSUPPORTED;
     if (find_packed(be, w->data)) stream_drop_packed(be, w->data);
-    const size_t bytes = (size_t)w->n * (w->k / 32) * (w->fmt == VX_Q4_0 ? 18 : 34);
-    PackedW *pw = new PackedW{nullptr, w->fmt, w->n, w->k, bytes};
-    if (hipMalloc(&pw->data, pw->bytes) != hipSuccess) {
+    const size_t bytes = (size_t)(w->n / 16) * (w->k / 128) * unit_bytes(w->fmt);
+    PackedW *pw = new PackedW{nullptr, w->fmt, w->n, w->k, (size_t)w->n * raw_row_bytes(w->fmt, w->k)};
+    if (hipMalloc(&pw->data, bytes) != hipSuccess) {
         delete pw;
         set_error("vx_qweight_pack: out of device memory (%zu bytes)", bytes);
         return VX_ERR_OOM;
     }
     if (w->fmt == VX_Q4_0)
         pack_q4_0_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
-    else
+    else if (w->fmt == VX_Q8_0)
         pack_q8_0_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
+    else if (w->fmt == VX_Q4_K)
+        pack_q4_k_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
+    else
+        pack_q6_k_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) {
         (void)hipFree(pw->data);
@@ -710,8 +975,12 @@ int vx_dequantize_packed(vx_backend *be, const vx_qweight *w, float *dst) {
     const size_t total = (size_t)w->n * w->k;
     if (pw->fmt == VX_Q4_0)
         dequant_packed_q4_0_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
-    else
+    else if (pw->fmt == VX_Q8_0)
         dequant_packed_q8_0_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
+    else if (pw->fmt == VX_Q4_K)
+        dequant_packed_q4_k_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
+    else
+        dequant_packed_q6_k_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }
