@@ -554,6 +554,7 @@ def prefill_probe(be, rows=512, reps=10):
         if synth.vxs_gaussian_quant(1, w, n * (k // 32), 0.02, 91):
             raise RuntimeError("synthetic weight generation failed")
         o = be.alloc_permanent(rows * n * 4)
+        be.qweight_pack(be.qweight(1, w, n, k))      # as the host runtime does at load time
         be.prepare_act(da, rows, k)
         be.matmul_quant_prepared(1, w, o, None, rows, n, k)
         be.sync()

@@ -96,6 +96,59 @@ def test_matmul_packed_vs_oracle(be, n, k, m, fmt):
     be.reset_pool()
 
 
+# more than 64 rows: the kernel whose waves own weight tiles and share the activation through LDS
+# (n, k): fewer tiles than a workgroup's waves own; tiles not a multiple of a wave's; many K slices; a long K
+@pytest.mark.parametrize("n,k", [(16, 256), (80, 1024), (1040, 2304), (4112, 512), (208, 11008)])
+@pytest.mark.parametrize("m", [65, 96, 130, 256])
+@pytest.mark.parametrize("fmt", FMTS)
+def test_matmul_packed_many_rows_vs_oracle(be, n, k, m, fmt):
+    rng = np.random.default_rng(n * 5 + k + m)
+    w = qz.random_quant(fmt, rng, n, k)
+    a = (rng.standard_normal((m, k)) * (1.0 + 3.0 * (rng.random((1, k)) < 0.1))).astype(np.float32)
+    want = nx.matmul_quant(fmt, a, w, m, n, k)
+    dw, qw = _packed(be, w, n, k, fmt)
+    da = be.upload(a)
+    dout = be.alloc(m * n * 4)
+    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
+    got = be.download(dout, (m, n), np.float32)
+    scale = np.abs(want).max()
+    _close(got, want, 2e-5, 2e-6 * scale + 1e-7, "packed matmul %dx%dx%d" % (m, n, k))
+    res = rng.standard_normal((m, n)).astype(np.float32)
+    dres = be.upload(res)
+    be.matmul_quant(fmt, da, dw, dout, dres, m, n, k)
+    assert np.array_equal(be.download(dout, (m, n), np.float32).view(np.uint32), (res + got).view(np.uint32))
+    be.qweight_unpack(qw)
+    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
+    plain = be.download(dout, (m, n), np.float32)
+    _close(got, plain, 0, 3e-6 * scale + 1e-7, "packed vs unpacked")
+    be.free(dw)
+    be.reset_pool()
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_matmul_packed_many_rows_independent_of_batch(be, fmt):
+    """A row has the same bits in any batch with the same number of 64-row groups (the K slicing depends on that
+    number beside the matrix' shape): 65 .. 128 rows here."""
+    rng = np.random.default_rng(12)
+    n, k = 208, 4096
+    w = qz.random_quant(fmt, rng, n, k)
+    a = rng.standard_normal((128, k)).astype(np.float32)
+    dw, qw = _packed(be, w, n, k, fmt)
+    da = be.upload(a)
+
+    def batch(first, rows):
+        d = be.alloc(rows * n * 4)
+        be.matmul_quant(fmt, da + first * k * 4, dw, d, None, rows, n, k)
+        return be.download(d, (rows, n), np.float32)
+
+    full = batch(0, 128)
+    for first, rows in ((0, 65), (11, 90), (40, 88), (1, 127)):
+        part = batch(first, rows)
+        assert np.array_equal(part.view(np.uint32), full[first:first + rows].view(np.uint32)), (first, rows)
+    be.free(dw)
+    be.reset_pool()
+
+
 @pytest.mark.parametrize("fmt", FMTS)
 def test_matmul_packed_rows_independent_of_batch(be, fmt):
     """A row has the same bits in a batch of 2, of 16, of 17 and of 32 rows (the cut of the matrix depends on its

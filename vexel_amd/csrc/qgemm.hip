@@ -1904,6 +1904,23 @@ int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out
             return VX_OK;
         }
     }
+    if (tiles_gemm_ok(be, fmt, segs.w, segs.n_end, 3, N, K, M)) {  // packed copies and a batch beyond the streaming kernel's
+        int ks = 1;
+        const int mpad = mpad_for(M);
+        const PrepView spv = prep_view(be, mpad, K);
+        int rc = tiles_gemm(be, fmt, segs.w, segs.n_end, 3, N, K, M, mpad, spv, out, residual, to_partials, &ks);
+        if (rc != VX_ERR_UNSUPPORTED) {
+            if (rc) return rc;
+            if (ks_out) *ks_out = ks;
+            if (!to_partials && ks > 1) {
+                const size_t total = (size_t)M * N;
+                qgemm_reduce_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const float *)be->part_ws, spv.inv_scale, out,
+                                                                                              residual, M, N, ks);
+                VX_CHECK_LAUNCH();
+            }
+            return VX_OK;
+        }
+    }
     const WavePlan rp = rows_plan(be, fmt, segs, N, K, M);
     if (rp.r > 0) {
         return launch_gemm_rows_r<WQ8_0>(be, rp, segs, N, out, residual, to_partials, M, K, ks_out);

@@ -41,12 +41,18 @@ struct QkvEpi {
     int qd, kvd, head_dim, block_size, pool_f16;
 };
 
-// qstream.hip: the decode-batch GEMM over load-time packed copies of Q4_0 matrices. w / n_end: up to nseg row
+// qstream.hip: the GEMMs over load-time packed copies of Q4_0 / Q8_0 / Q4_K / Q6_K matrices. w / n_end: up to nseg row
 // segments of raw matrices (device addresses, cumulative row ends); served when every matrix in them has a packed
-// copy (vx_qweight_pack), 2 <= M <= 32 and the shape fits. stream_gemm leaves the K slices' raw sums in
+// copy (vx_qweight_pack), 2 <= M <= 64 and the shape fits. stream_gemm leaves the K slices' raw sums in
 // be->part_ws as [slice][M][N] (*ks_out slices) or, given an epilogue, finishes the Q|K|V rows itself.
 bool stream_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M, bool epi);
 int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M, int mpad,
                 const PrepView &pv, const QkvEpi *epi, int *ks_out);
+
+// More than 64 rows over the same packed copies. With one K slice and to_partials false the finished rows (row
+// factors, residual) go to out; otherwise the slices' sums to be->part_ws, *ks_out of them.
+bool tiles_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M);
+int tiles_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M, int mpad,
+               const PrepView &pv, float *out, const float *residual, bool to_partials, int *ks_out);
 
 }  // namespace vx

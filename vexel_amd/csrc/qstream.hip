@@ -1,28 +1,30 @@
-// Decode-batch GEMM (2 .. 32 activation rows) over Q4_0 weights repacked at load time into the order the matrix
-// cores consume them: C[M,N] = A[M,K] * B^T with B [N,K] as backend.go:47-52 (MatMulQ4_0) has it, the arithmetic
-// of backend/cpu/cpu.go:842-911 up to float32 summation order.
+// Decode-batch GEMM (2 .. 64 activation rows) over quantized weights repacked at load time into the order the matrix
+// cores consume them: C[M,N] = A[M,K] * B^T with B [N,K] as backend.go:47-81 (MatMulQ4_0 / Q8_0 / Q4_K / Q6_K) has
+// it, the arithmetic of backend/cpu/cpu.go:842-911 up to float32 summation order.
 //
 // Packed layout (vx_qweight_pack): the matrix is cut into tiles of 16 rows and half chunks of 128 columns. One
-// (tile, half chunk) is a unit of 1152 bytes, units of a tile follow one another along K:
+// (tile, half chunk) is a unit, units of a tile follow one another along K. The Q4_0 unit, 1152 bytes:
 //   bytes [0, 1024): lane l = 16 * g + r of a wave owns 16 bytes, dword j of them the eight 4-bit codes of row r's
 //     block 4 * hc + j that lane group g feeds to the matrix core: nibble i of the dword is block element
 //     ELT[g][SLOT[i]] (the slot order of the prepared activation tiles, prep_tiles.h), so that two masks, one shift
 //     and four packed f16 operations turn the dword into the operand;
 //   bytes [1024, 1152): row r's four f16 block scales at 1024 + 8 r.
-// The bytes are a permutation of the GGUF rows' bytes (18 per 32 elements either way); vx_dequantize_packed gives
-// back gguf.DequantizeQ4_0's values bit for bit (pkg/gguf/dequant.go:16-56).
+// Its bytes are a permutation of the GGUF rows' bytes (18 per 32 elements either way), as are the Q8_0 unit's; the
+// Q4_K and Q6_K units carry their scales as float32 products (see SQ4_K, SQ6_K). vx_dequantize_packed gives back
+// gguf.Dequantize's values bit for bit for every format (pkg/gguf/dequant.go:16-95, 272-409).
 //
 // Kernel: one workgroup of eight waves per compute unit owns a range of tiles and one K slice. Wave w keeps the
 // activation operand of half chunk h0 + w (and h0 + 8 + w) of the slice in registers for the whole pass and streams
 // the weight units of those half chunks through them, tile after tile, from a ring of requests that runs ahead of
-// the arithmetic: a unit goes from memory to registers with one 16-byte and one 8-byte load per lane and nowhere
-// else. Per 32-column step: 9 vector instructions unpack the codes to exact integers in f16, four
+// the arithmetic: a unit goes from memory to registers with one 16-byte and one 8-byte load per lane (Q4_0) and nowhere
+// else. Per 32-column step (Q4_0): 9 vector instructions unpack the codes to exact integers in f16, four
 // v_mfma_f32_16x16x32_f16 multiply them with the hi and lo halves of two activation tiles, 8 fused multiply-adds
 // apply the block scale. After every RG tiles the eight waves' sums meet in LDS and are added in wave order. A slice
 // wider than 16 half chunks is walked in passes of 16 (the sums wait in LDS), which is how the Q|K|V launch
 // keeps the whole K in one workgroup and finishes its rows itself (RoPE, K/V store).
-// Which tiles and half chunks a workgroup takes depends on (N, K, device, epilogue) only and every sum is added in
-// a fixed order, so a row has the same bits in any batch of 2 .. 32 rows.
+// Which tiles and half chunks a workgroup takes depends on (N, K, device, epilogue, format) and on whether the batch
+// has up to 32 or up to 64 rows; every sum is added in a fixed order, so a row has the same bits in any batch of
+// 2 .. 32 rows, and in any batch of 33 .. 64.
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
@@ -688,6 +690,227 @@ qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1,
     }
 }
 
+
+// ------------------------------------------------------------------------------------------------ many rows
+// More than 64 activation rows (prefill chunks, tree verification) over the same packed units. The activation no
+// longer fits the registers, so the roles turn: a wave owns R weight tiles (16 R rows) and keeps their sums for 64
+// activation rows (R x 4 tiles of 16 x 16) in registers; the eight waves of a workgroup share the activation tiles of
+// those 64 rows, which all threads bring into LDS half chunk by half chunk (double buffered, one barrier each), and
+// every wave requests its R units of the next half chunk straight into registers meanwhile. Per 32-column step a
+// wave reads 8 operands from LDS for 8 R MFMAs (the form with two tiles a wave reads them for 16 and is bound by LDS
+// bandwidth). grid = (groups of 8 R tiles, K slices, groups of 64 rows); the sums of one K slice carry the chunk
+// factor of the chunk they are in and move to the next chunk's by a ratio of two powers of two.
+__device__ __forceinline__ float pow2_ratio_s(float num, float den) {
+    return __uint_as_float(__float_as_uint(num) - __float_as_uint(den) + 0x3F800000u);
+}
+
+template <class W, int R>
+__global__ void __launch_bounds__(64 * NW, 1)
+qtiles_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, const uint8_t *__restrict__ pw2,
+              const half8 *__restrict__ a_tiles, const float *__restrict__ a_cscale, const float *__restrict__ a_inv_scale,
+              const float *__restrict__ a_bsum, float *__restrict__ out, const float *__restrict__ residual,
+              float *__restrict__ partial, const StreamShape a, const int slices) {
+    constexpr int MT = 4;
+    __shared__ half8 a_lds[2][4 * 512];
+    typedef typename W::Ring Unit;
+
+    const int tid = threadIdx.x, lane = tid & 63, ln = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n_tiles = a.N >> 4, mtiles = a.Mpad >> 4, n_hc = a.n_hc;
+    const int t_own = (blockIdx.x * NW + wave) * R;          // first tile this wave writes
+    const int t0 = max(min(t_own, n_tiles - R), 0);          // (a wave past the end works on the last tiles and writes nothing)
+    const int ks = blockIdx.y, mg = blockIdx.z, m0 = mg * 16 * MT;
+    const int sl_base = slices >> 16, sl_rem = slices & 0xFFFF;
+    const int h_begin = ks * sl_base + min(ks, sl_rem), n_half = sl_base + (ks < sl_rem ? 1 : 0);
+
+    const size_t tile_stride = (size_t)n_hc * W::UNIT;
+    const uint8_t *const w0 = uniform_ptr(pw0), *const w1 = uniform_ptr(pw1), *const w2 = uniform_ptr(pw2);
+    const int e0 = __builtin_amdgcn_readfirstlane(a.t_end0), e1 = __builtin_amdgcn_readfirstlane(a.t_end1);
+    const uint8_t *tb[R];
+#pragma unroll
+    for (int r = 0; r < R; r++) tb[r] = uniform_ptr(tile_base(t0 + r, w0, w1, w2, e0, e1, tile_stride));
+    uint32_t k64;
+    asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(k64));
+
+    // this thread's piece of a step's activation tiles: tile tid / 128 of the group (hi and lo halves, 64 lanes each);
+    // a tile past the padded rows repeats the last one (its products are not stored)
+    const int a_tile = min(mg * MT + tid / 128, mtiles - 1);
+    const half8 *a_src = a_tiles + ((size_t)a_tile * 2) * 64 + (tid & 127);
+
+    float4v run[R][MT];
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int t = 0; t < MT; t++) run[r][t] = (float4v){0.f, 0.f, 0.f, 0.f};
+    if (n_half <= 0) return;
+
+    Unit ring[R];
+    half8 areg[4];
+    auto fetch = [&](int q) __attribute__((always_inline)) {
+        const int hc = h_begin + min(q, n_half - 1);
+#pragma unroll
+        for (int r = 0; r < R; r++) ring[r] = W::load(tb[r] + (size_t)hc * W::UNIT, lane, ln);
+#pragma unroll
+        for (int sp = 0; sp < 4; sp++) areg[sp] = gload<half8>(a_src + (size_t)(hc * 4 + sp) * mtiles * 128);
+    };
+    auto commit = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int sp = 0; sp < 4; sp++) a_lds[buf][sp * 512 + tid] = areg[sp];
+    };
+    auto load_cs = [&](int chunk, float4v (&cs)[MT]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            const int mt = min(mg * MT + t, mtiles - 1);
+            cs[t] = gload<float4v>(a_cscale + (size_t)chunk * a.Mpad + mt * 16 + 4 * g);
+        }
+    };
+
+    float4v cs[MT];
+    fetch(0);
+    load_cs(h_begin >> 1, cs);
+    commit(0);
+    __syncthreads();
+    for (int q = 0; q < n_half; q++) {
+        const int hc = h_begin + q;
+        Unit cur[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) cur[r] = ring[r];
+        fetch(q + 1);
+        if (q > 0 && (hc & 1) == 0) {  // a new chunk: the sums move to its activation scale
+            float4v cn[MT];
+            load_cs(hc >> 1, cn);
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                float4v f;
+#pragma unroll
+                for (int e = 0; e < 4; e++) f[e] = pow2_ratio_s(cs[t][e], cn[t][e]);
+#pragma unroll
+                for (int r = 0; r < R; r++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) run[r][t][e] *= f[e];
+                cs[t] = cn[t];
+            }
+        }
+        const half8 *ab = &a_lds[q & 1][0];
+#pragma unroll
+        for (int sp = 0; sp < 4; sp++) {
+            half8 ah[MT], al[MT];
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                ah[t] = ab[sp * 512 + (t * 2 + 0) * 64 + lane];
+                al[t] = ab[sp * 512 + (t * 2 + 1) * 64 + lane];
+            }
+            float4v bs[MT];
+            if constexpr (W::HAS_MIN) {
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    const int mt = min(mg * MT + t, mtiles - 1);
+                    bs[t] = gload<float4v>(a_bsum + (size_t)(hc * 4 + sp) * a.Mpad + mt * 16 + 4 * g);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                if constexpr (W::TWO_SCALES) {
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const half4v wb = W::codes16(cur[r], sp, h);
+                        const float d = W::scale16(cur[r], sp, h);
+                        float4v P[MT];
+#pragma unroll
+                        for (int t = 0; t < MT; t++)
+                            P[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(h ? second16(ah[t]) : first16(ah[t]), wb, (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                        for (int t = 0; t < MT; t++)
+                            P[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(h ? second16(al[t]) : first16(al[t]), wb, P[t], 0, 0, 0);
+#pragma unroll
+                        for (int t = 0; t < MT; t++)
+#pragma unroll
+                            for (int e = 0; e < 4; e++) run[r][t][e] = __builtin_fmaf(d, P[t][e], run[r][t][e]);
+                    }
+                } else {
+                    const half8 wb = W::codes(cur[r], sp, k64);
+                    const float d = W::scale(cur[r], sp);
+                    float4v P[MT];
+#pragma unroll
+                    for (int t = 0; t < MT; t++) P[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ah[t], wb, (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+#pragma unroll
+                    for (int t = 0; t < MT; t++) P[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(al[t], wb, P[t], 0, 0, 0);
+#pragma unroll
+                    for (int t = 0; t < MT; t++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) run[r][t][e] = __builtin_fmaf(d, P[t][e], run[r][t][e]);
+                    if constexpr (W::HAS_MIN) {
+                        const float mn = -W::minimum(cur[r], sp);
+#pragma unroll
+                        for (int t = 0; t < MT; t++)
+#pragma unroll
+                            for (int e = 0; e < 4; e++) run[r][t][e] = __builtin_fmaf(mn, bs[t][e], run[r][t][e]);
+                    }
+                }
+            }
+        }
+        // the next half chunk's activation tiles into the buffer every wave finished with before the previous barrier
+        commit((q + 1) & 1);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int r = 0; r < R; r++)
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) run[r][t][e] *= cs[t][e];
+
+    // lane (g, ln) of tile (r, t) holds C[m0 + 16 t + 4 g + e][16 (t0 + r) + ln]
+#pragma unroll
+    for (int t = 0; t < MT; t++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int m = m0 + 16 * t + 4 * g + e;
+            if (m >= a.M) continue;
+            const float inv = partial ? 1.f : a_inv_scale[m];
+#pragma unroll
+            for (int r = 0; r < R; r++) {
+                if (t0 + r < t_own) continue;
+                const int n = 16 * (t0 + r) + ln;
+                if (partial) {
+                    partial[((size_t)ks * a.M + m) * a.N + n] = run[r][t][e];
+                } else {
+                    float v = __fmul_rn(run[r][t][e], inv);
+                    if (residual) v = __fadd_rn(residual[(size_t)m * a.N + n], v);
+                    out[(size_t)m * a.N + n] = v;
+                }
+            }
+        }
+}
+
+struct TilesPlan {
+    int r, s;  // weight tiles a wave, K slices; r == 0: not served
+};
+// Tiles per wave by what the format's units leave of the registers; K slices so that the grid fills the device in
+// whole rounds where it can (efficiency = workgroups / (rounds x compute units)), each slice at least two half chunks.
+TilesPlan tiles_plan(int fmt, int n_tiles, int n_hc, int mgroups, int cus) {
+    TilesPlan pl = {0, 1};
+    // (four tiles a wave: 64 more accumulators than there are registers; Q6_K's units and Q4_K's block sums leave room for two)
+    int r = (fmt == VX_Q6_K || fmt == VX_Q4_K) ? 2 : 3;
+    while (r > 1 && (n_tiles < r || ceil_div(n_tiles, NW * r) * mgroups * 4 < cus)) r--;  // few rows: more, smaller workgroups
+    if (n_tiles < r) return pl;
+    const int base = ceil_div(n_tiles, NW * r) * mgroups;
+    int best = 1;
+    float best_cost = 1e30f;
+    for (int s = 1; s <= std::min(16, std::max(1, n_hc / 2)); s++) {
+        const int wgs = base * s, rounds = ceil_div(wgs, cus);
+        // time of a round ~ half chunks per slice + a fixed part; the slices' sums cost their round trip
+        const float cost = (float)rounds * ((float)ceil_div(n_hc, s) + 3.f) + (s > 1 ? 0.15f * (float)s * (float)n_hc / 16.f : 0.f);
+        if (cost < best_cost) {
+            best_cost = cost;
+            best = s;
+        }
+    }
+    pl.r = r;
+    pl.s = best;
+    return pl;
+}
+
 struct StreamPlan {
     int g, s, ph, npass;  // row groups, K slices, half chunks per wave and pass, passes; g == 0: not served
 };
@@ -908,6 +1131,69 @@ int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_e
     else if (fmt == VX_Q8_0) launch_stream<SQ8_0>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
     else if (fmt == VX_Q4_K) launch_stream<SQ4_K>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
     else launch_stream<SQ6_K>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
+    VX_CHECK_LAUNCH();
+    if (ks_out) *ks_out = pl.s;
+    return VX_OK;
+}
+
+
+bool tiles_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M) {
+    static const char *off = getenv("VEXEL_HIP_TILES_OFF");
+    if (off && atoi(off)) return false;
+    if (M <= 64 || N % 16 != 0 || K % 256 != 0 || N < 16) return false;
+    PackedSegs ps;
+    return resolve(be, fmt, w, n_end, nseg, N, K, &ps);
+}
+
+template <class W>
+static void launch_tiles(vx_backend *be, const TilesPlan &pl, dim3 grid, const PackedSegs &ps, const PrepView &pv, float *out,
+                         const float *residual, float *partial, const StreamShape &a, int slices) {
+#define VX_TILES_LAUNCH(R_)                                                                                                    \
+    qtiles_kernel<W, R_><<<grid, 64 * NW, 0, be->stream>>>(ps.w[0], ps.w[1], ps.w[2], pv.tiles, pv.cscale, pv.inv_scale, pv.bsum, out, \
+                                                           residual, partial, a, slices)
+    if (pl.r == 3) {
+        if constexpr (!W::TWO_SCALES && !W::HAS_MIN) VX_TILES_LAUNCH(3);
+    } else if (pl.r == 2) {
+        VX_TILES_LAUNCH(2);
+    } else {
+        VX_TILES_LAUNCH(1);
+    }
+#undef VX_TILES_LAUNCH
+}
+
+// More than 64 rows over packed matrices. One K slice and no request for the slices' sums: the finished rows go to
+// out (row factors and the residual applied); otherwise [slice][M][N] sums go to be->part_ws and *ks_out says how many.
+int tiles_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M, int mpad,
+               const PrepView &pv, float *out, const float *residual, bool to_partials, int *ks_out) {
+    PackedSegs ps;
+    if (!resolve(be, fmt, w, n_end, nseg, N, K, &ps)) return VX_ERR_UNSUPPORTED;
+    static int cus = 0;
+    if (cus == 0 && (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0)) cus = 256;
+    const int n_hc = K / 128, mgroups = ceil_div(mpad, 64);
+    const TilesPlan pl = tiles_plan(fmt, N / 16, n_hc, mgroups, cus);
+    if (pl.r == 0) return VX_ERR_UNSUPPORTED;
+    StreamShape a;
+    a.M = M;
+    a.Mpad = mpad;
+    a.N = N;
+    a.n_hc = n_hc;
+    a.npass = 1;
+    a.t_end0 = ps.t_end[0];
+    a.t_end1 = ps.t_end[1];
+    float *partial = nullptr;
+    if (pl.s > 1 || to_partials) {
+        int rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, (size_t)pl.s * M * N * sizeof(float), "split-K partial sums");
+        if (rc) return rc;
+        partial = (float *)be->part_ws;
+    }
+    const int slices = ((n_hc / pl.s) << 16) | (n_hc % pl.s);
+    dim3 grid(ceil_div(N / 16, NW * pl.r), pl.s, mgroups);
+    switch (fmt) {
+    case VX_Q4_0: launch_tiles<SQ4_0>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
+    case VX_Q8_0: launch_tiles<SQ8_0>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
+    case VX_Q4_K: launch_tiles<SQ4_K>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
+    default: launch_tiles<SQ6_K>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
+    }
     VX_CHECK_LAUNCH();
     if (ks_out) *ks_out = pl.s;
     return VX_OK;
