@@ -400,13 +400,16 @@ def time_fused_qkv(be, lw, c, rows, x):
 def kernel_report(be):
     """Per-kernel timings through the C ABI, inputs resident in HBM, HIP events on the backend stream. Every
     weight shape cycles over enough distinct copies (> 400 MB) that nothing is served from the 256 MB
-    memory-side cache. Algorithmic bytes of a quantized matmul: N*K*bytes_per_element + M*K*4 + M*N*4."""
+    memory-side cache. Algorithmic bytes of a quantized matmul: N*K*bytes_per_element + M*K*4 + M*N*4 with the GGUF
+    bytes per element. The matrices are packed at load time as the host runtime packs a batched model's (formats
+    with a packed form; one row reads the GGUF rows either way); several rows are timed as the unfused call: the
+    projection launch and the reduction of its K slices."""
     synth = load_synth()
     bpe = {1: 18 / 32, 2: 34 / 32, 3: 144 / 256, 4: 210 / 256, 5: 22 / 32, 6: 176 / 256}
     names = {1: "Q4_0", 2: "Q8_0", 3: "Q4_K", 4: "Q6_K", 5: "Q5_0", 6: "Q5_K"}
     shapes = [("Q|K|V", 12288, 4096), ("Wo", 4096, 4096), ("gate|up", 22016, 4096), ("down", 4096, 11008),
               ("lm_head", 32000, 4096)]
-    a = np.random.default_rng(0).standard_normal((64, 11008)).astype(np.float32)
+    a = np.random.default_rng(0).standard_normal((256, 11008)).astype(np.float32)
     da = be.upload(a, permanent=True)
     print("%-8s %-5s %3s %6s %6s %9s %9s %7s" % ("matmul", "fmt", "M", "N", "K", "us/call", "GB/s", "of 8TB"))
     for fmt in (1, 2, 3, 4, 5, 6):
@@ -430,8 +433,9 @@ def kernel_report(be):
                     rc = synth.vxs_random_kquant(fmt, p, n * (k // 256), 77 + i)
                 if rc:
                     raise RuntimeError("synthetic weight generation failed: %d" % rc)
+                be.qweight_pack(be.qweight(fmt, p, n, k))
                 ws.append(p)
-            for m in (1, 32, 64):
+            for m in (1, 32, 64, 256):
                 out = be.alloc_permanent(m * n * 4)
                 be.prepare_act(da, m, k)
                 for w in ws[:2]:
