@@ -230,16 +230,17 @@ typedef struct vx_qweight {
 } vx_qweight;
 
 /* Load-time repack for decode batches. No counterpart in the reference, whose loader hands GGUF rows to the kernels
- * as they are (runtime/loader.go:79-200): vx_qweight_pack makes a second copy of a Q4_0, Q8_0, Q4_K or Q6_K matrix
+ * as they are (runtime/loader.go:79-200): vx_qweight_pack makes a second copy of a Q4_0, Q8_0, Q4_K, Q6_K, Q5_0 or Q5_K matrix
  * (n % 16 == 0, k % 256 == 0; VX_ERR_UNSUPPORTED otherwise, nothing changed) in the order the matrix cores consume it
  * (Q4_0 and Q8_0: a permutation of the rows' bytes, 18 / 34 per 32 elements either way; Q4_K: the codes with the
  * sub-blocks' scale and min products d * sc, dmin * m as float32, 6 bits per weight; Q6_K: one byte per code and the
- * float32 products d * sc per 16 elements, 10 bits per weight), kept by the backend under the matrix' address until
+ * float32 products d * sc per 16 elements, 10 bits per weight; Q5_0: one byte per code in the Q8_0 form, 8.5 bits;
+ * Q5_K: one byte per code and the products as for Q4_K, 10 bits), kept by the backend under the matrix' address until
  * vx_qweight_unpack, vx_free of the matrix, a library write into its bytes or vx_backend_destroy. While it exists,
  * every quantized matmul entry point and fused decode block that is given the matrix (by the same data pointer, alone
- * or as part of a Q|K|V or gate|up group) with 2 .. 64 activation rows (Q4_K: 2 .. 32) streams the packed copy; other
- * row counts read the GGUF rows, which stay where they are. vx_dequantize_packed: gguf.Dequantize of the packed copy
- * (pkg/gguf/dequant.go:16-95, 272-409), bit for bit what vx_dequantize gives for the rows. */
+ * or as part of a Q|K|V or gate|up group) with 2 .. 64 activation rows (Q4_K, Q5_K: 2 .. 32) streams the packed copy, and with more than 64 rows reads
+ * it tile by tile; other row counts read the GGUF rows, which stay where they are. vx_dequantize_packed: gguf.Dequantize of the packed copy
+ * (pkg/gguf/dequant.go:16-145, 272-470), bit for bit what vx_dequantize gives for the rows. */
 int vx_qweight_pack(vx_backend *be, const vx_qweight *w);
 int vx_qweight_unpack(vx_backend *be, const vx_qweight *w);
 int vx_qweight_is_packed(vx_backend *be, const vx_qweight *w);

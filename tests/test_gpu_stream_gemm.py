@@ -1,5 +1,5 @@
-"""GPU parity of the decode-batch GEMM over load-time packed Q4_0, Q8_0, Q6_K and Q4_K matrices (vx_qweight_pack): the packed
-copy dequantises to the reference's values bit for bit, the products match the CPU oracle's MatMulQ4_0 / Q8_0 / Q6_K
+"""GPU parity of the decode-batch GEMM over load-time packed matrices of the six block formats (vx_qweight_pack): the packed
+copy dequantises to the reference's values bit for bit, the products match the CPU oracle's MatMulQ4_0 / Q8_0 / Q4_K / Q6_K / Q5_0 / Q5_K
 (backend/cpu/cpu.go:842-911) to float32 summation order on every cut of the matrix the planner makes, a row's bits
 do not depend on the batch it sits in (2 .. 32 rows; 33 .. 64 rows), and the fused decode blocks give the oracle's
 layer with packed weights."""
@@ -27,7 +27,7 @@ def _close(got, want, rtol, atol, what=""):
         what, err.max(), lim.reshape(-1)[err.argmax()])
 
 
-FMTS = [nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q6_K, nx.FMT_Q4_K]
+FMTS = [nx.FMT_Q4_0, nx.FMT_Q8_0, nx.FMT_Q6_K, nx.FMT_Q4_K, nx.FMT_Q5_0, nx.FMT_Q5_K]
 
 
 def _packed(be, w, n, k, fmt=nx.FMT_Q4_0):
@@ -43,7 +43,11 @@ def _packed(be, w, n, k, fmt=nx.FMT_Q4_0):
 def test_packed_copy_dequantises_bit_exact(be, n, k, fmt):
     rng = np.random.default_rng(n + k)
     w = qz.random_quant(fmt, rng, n, k)
-    if fmt == nx.FMT_Q4_K:
+    if fmt == nx.FMT_Q5_0:
+        w.reshape(-1)[2:22] = rng.integers(0, 256, 20, dtype=np.uint8)     # arbitrary fifth bits and nibbles in one block
+    elif fmt == nx.FMT_Q5_K:
+        w.reshape(-1)[4:176] = rng.integers(0, 256, 172, dtype=np.uint8)   # arbitrary scale / min fields, fifth bits and nibbles
+    elif fmt == nx.FMT_Q4_K:
         w.reshape(-1)[4:144] = rng.integers(0, 256, 140, dtype=np.uint8)   # arbitrary scale / min fields and codes in one super-block
     elif fmt == nx.FMT_Q6_K:
         w.reshape(-1)[0:208] = rng.integers(0, 256, 208, dtype=np.uint8)   # arbitrary codes and scale bytes in one super-block
@@ -62,9 +66,9 @@ def test_packed_copy_dequantises_bit_exact(be, n, k, fmt):
 
 def test_pack_refuses_other_formats_and_shapes(be):
     rng = np.random.default_rng(0)
-    w = qz.random_quant(nx.FMT_Q5_K, rng, 32, 256)
+    w = qz.random_quant(nx.FMT_BF16, rng, 32, 256)
     dw = be.upload(w, permanent=True)
-    assert not be.qweight_pack(be.qweight(nx.FMT_Q5_K, dw, 32, 256))
+    assert not be.qweight_pack(be.qweight(nx.FMT_BF16, dw, 32, 256))
     assert not be.qweight_pack(be.qweight(nx.FMT_Q4_0, dw, 24, 256))     # rows not a multiple of 16
     assert not be.qweight_pack(be.qweight(nx.FMT_Q4_0, dw, 32, 128))     # K not a multiple of 256
     be.free(dw)
@@ -209,8 +213,8 @@ def test_fused_decode_blocks_with_packed_weights(be, rows, hq, hk, d, hidden, ff
     rng = np.random.default_rng(rows + hq + hidden)
     bs, nblocks, theta, eps = 16, 8, 10000.0, 1e-5
     qd, kvd = hq * d, hk * d
-    quant = qz.quantize_q4_0 if fmt == nx.FMT_Q4_0 else qz.quantize_q8_0
-    if fmt in (nx.FMT_Q6_K, nx.FMT_Q4_K):
+    quant = {nx.FMT_Q4_0: qz.quantize_q4_0, nx.FMT_Q8_0: qz.quantize_q8_0, nx.FMT_Q5_0: qz.quantize_q5_0}.get(fmt)
+    if fmt in (nx.FMT_Q6_K, nx.FMT_Q4_K, nx.FMT_Q5_K):
         mk = lambda n, k: qz.random_quant(fmt, rng, n, k, std=0.05).reshape(-1)
     else:
         mk = lambda n, k: quant((rng.standard_normal((n, k)) * 0.05).astype(np.float32)).reshape(-1)

@@ -90,9 +90,9 @@ template <int BIAS> __device__ __forceinline__ half8 unpack_q4(uint32_t w, uint3
 
 // Eight biased bytes (q + 128, two dwords) -> exact integers q as f16: a byte under 0x64 is the f16 1024 + byte. Byte
 // positions 0, 2, 1, 3 of a dword hold consecutive slots, so that each byte permute yields a finished pair.
-__device__ __forceinline__ half8 unpack_q8(uint32_t w0, uint32_t w1) {
+template <int BIAS> __device__ __forceinline__ half8 unpack_q8(uint32_t w0, uint32_t w1) {
     const uint32_t c64 = 0x64646464u;
-    const half2v off = {(_Float16)1152.f, (_Float16)1152.f};  // 1024 + 128
+    const half2v off = {(_Float16)(1024.f + BIAS), (_Float16)(1024.f + BIAS)};
     const half2v h0 = as_h2(__builtin_amdgcn_perm(w0, c64, 0x00060004u)) - off, h1 = as_h2(__builtin_amdgcn_perm(w0, c64, 0x00070005u)) - off;
     const half2v h2 = as_h2(__builtin_amdgcn_perm(w1, c64, 0x00060004u)) - off, h3 = as_h2(__builtin_amdgcn_perm(w1, c64, 0x00070005u)) - off;
     half8 r;
@@ -166,9 +166,35 @@ struct SQ8_0 {
         return x;
     }
     static __device__ __forceinline__ half8 codes(const Ring &x, int j, uint32_t) {
-        return j == 0 ? unpack_q8(x.c0[0], x.c0[1]) : j == 1 ? unpack_q8(x.c0[2], x.c0[3]) : j == 2 ? unpack_q8(x.c1[0], x.c1[1]) : unpack_q8(x.c1[2], x.c1[3]);
+        return j == 0 ? unpack_q8<128>(x.c0[0], x.c0[1]) : j == 1 ? unpack_q8<128>(x.c0[2], x.c0[3]) : j == 2 ? unpack_q8<128>(x.c1[0], x.c1[1]) : unpack_q8<128>(x.c1[2], x.c1[3]);
     }
     static __device__ __forceinline__ float scale(const Ring &x, int j) { return half_of(x.s[j >> 1], j & 1); }
+    static __device__ __forceinline__ float minimum(const Ring &, int) { return 0.f; }
+};
+// Q5_0 (22-byte blocks, pkg/gguf/dequant.go:100-145: element = float32(q - 16) * d) is packed into Q8_0 units with
+// q - 16 as the code: the same kernel, the same product. Q5_K (176-byte super-blocks, dequant.go:411-470: element =
+// d1 * q - m1 with 5-bit q) gets a unit of 2560 bytes: the codes one byte each in the Q8_0 unit's order (unsigned),
+// then row r's d1[4] at 2048 + 32 r and m1[4] at 2064 + 32 r; its min term as Q4_K's. 10 bits per weight against 5.5.
+struct SQ5_K {
+    static constexpr int FMT = VX_Q5_K, UNIT = 2560, SCALES_AT = 2048;
+    static constexpr bool TWO_SCALES = false, HAS_MIN = true;
+    struct Ring {
+        u32x4 c0, c1;
+        float4v d1, m1;
+    };
+    static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
+        Ring x;
+        x.c0 = gload<u32x4>(u + lane * 32);
+        x.c1 = gload<u32x4>(u + lane * 32 + 16);
+        x.d1 = gload<float4v>(u + SCALES_AT + ln * 32);
+        x.m1 = gload<float4v>(u + SCALES_AT + ln * 32 + 16);
+        return x;
+    }
+    static __device__ __forceinline__ half8 codes(const Ring &x, int j, uint32_t) {
+        return j == 0 ? unpack_q8<0>(x.c0[0], x.c0[1]) : j == 1 ? unpack_q8<0>(x.c0[2], x.c0[3]) : j == 2 ? unpack_q8<0>(x.c1[0], x.c1[1]) : unpack_q8<0>(x.c1[2], x.c1[3]);
+    }
+    static __device__ __forceinline__ float scale(const Ring &x, int j) { return x.d1[j]; }
+    static __device__ __forceinline__ float minimum(const Ring &x, int j) { return x.m1[j]; }
 };
 // Q6_K (210-byte super-blocks of 256 elements, pkg/gguf/dequant.go:272-331): a half chunk is half a super-block, and
 // every 16 of its elements carry a scale of their own, so a 32-column step is two v_mfma_f32_16x16x16_f16 per
@@ -291,6 +317,35 @@ __global__ void __launch_bounds__(64) pack_q8_0_kernel(const uint8_t *__restrict
     }
 }
 
+// Q5_0 rows into Q8_0 units: code q - 16 (dequant.go:100-145: low nibbles and bits 0 .. 15 of qh are elements 0 .. 15,
+// high nibbles and bits 16 .. 31 elements 16 .. 31)
+__global__ void __launch_bounds__(64) pack_q5_0_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ packed, int n_hc) {
+    const int T = blockIdx.x, hc = blockIdx.y, lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+    const size_t row_bytes = (size_t)n_hc * 4 * 22;
+    const uint8_t *row = raw + (size_t)(T * 16 + r) * row_bytes + (size_t)hc * 4 * 22;
+    uint8_t *u = packed + ((size_t)T * n_hc + hc) * SQ8_0::UNIT;
+    uint32_t out[8];
+    for (int j = 0; j < 4; j++) {
+        const uint8_t *blk = row + j * 22;
+        const uint32_t qh = (uint32_t)blk[2] | ((uint32_t)blk[3] << 8) | ((uint32_t)blk[4] << 16) | ((uint32_t)blk[5] << 24);
+        uint32_t w[2] = {0, 0};
+        for (int slot = 0; slot < 8; slot++) {
+            const int e = elt_of(g, slot), at = q8_byte_of_slot(slot);
+            const int q = (int)(e < 16 ? (blk[6 + e] & 0xFu) : (blk[6 + e - 16] >> 4)) | (int)(((qh >> e) & 1u) << 4);
+            w[at >> 2] |= (uint32_t)(uint8_t)(q - 16 + 128) << (8 * (at & 3));
+        }
+        out[2 * j] = w[0];
+        out[2 * j + 1] = w[1];
+    }
+    *(u32x4 *)(u + lane * 32) = (u32x4){out[0], out[1], out[2], out[3]};
+    *(u32x4 *)(u + lane * 32 + 16) = (u32x4){out[4], out[5], out[6], out[7]};
+    if (g == 0) {
+        uint16_t d[4];
+        for (int j = 0; j < 4; j++) d[j] = (uint16_t)(row[j * 22] | (row[j * 22 + 1] << 8));
+        *(u32x2 *)(u + SQ8_0::SCALES_AT + r * 8) = (u32x2){(uint32_t)d[0] | ((uint32_t)d[1] << 16), (uint32_t)d[2] | ((uint32_t)d[3] << 16)};
+    }
+}
+
 // scale * float32(q) as gguf.DequantizeQ8_0 computes it (pkg/gguf/dequant.go:58-95), read from the packed form.
 __global__ void __launch_bounds__(256) dequant_packed_q8_0_kernel(const uint8_t *__restrict__ packed, float *__restrict__ dst, int n,
                                                                   int k) {
@@ -379,6 +434,67 @@ __global__ void __launch_bounds__(256) dequant_packed_q4_k_kernel(const uint8_t 
     float d1, m1;
     __builtin_memcpy(&d1, u + SQ4_K::SCALES_AT + r * 32 + j * 4, 4);
     __builtin_memcpy(&m1, u + SQ4_K::SCALES_AT + r * 32 + 16 + j * 4, 4);
+    dst[idx] = __fsub_rn(__fmul_rn(d1, (float)q), m1);
+}
+
+// Q5_K (dequant.go:411-470): sub-block sbi's element e is nibble (sbi & 1) of qs[32 (sbi / 2) + e] plus 16 times bit
+// sbi of qh[e]
+__global__ void __launch_bounds__(64) pack_q5_k_kernel(const uint8_t *__restrict__ raw, uint8_t *__restrict__ packed, int n_hc) {
+    const int T = blockIdx.x, hc = blockIdx.y, lane = threadIdx.x, r = lane & 15, g = lane >> 4;
+    const size_t row_bytes = (size_t)(n_hc / 2) * 176;
+    const uint8_t *sb = raw + (size_t)(T * 16 + r) * row_bytes + (size_t)(hc >> 1) * 176;
+    uint8_t *u = packed + ((size_t)T * n_hc + hc) * SQ5_K::UNIT;
+    uint32_t out[8];
+    for (int j = 0; j < 4; j++) {
+        const int sbi = 4 * (hc & 1) + j;
+        const uint8_t *qs = sb + 48 + 32 * (sbi >> 1), *qh = sb + 16;
+        uint32_t w[2] = {0, 0};
+        for (int slot = 0; slot < 8; slot++) {
+            const int e = elt_of(g, slot), at = q8_byte_of_slot(slot);
+            const uint32_t q = ((sbi & 1) ? (qs[e] >> 4) : (qs[e] & 0xFu)) + (((qh[e] >> sbi) & 1u) << 4);
+            w[at >> 2] |= q << (8 * (at & 3));
+        }
+        out[2 * j] = w[0];
+        out[2 * j + 1] = w[1];
+    }
+    *(u32x4 *)(u + lane * 32) = (u32x4){out[0], out[1], out[2], out[3]};
+    *(u32x4 *)(u + lane * 32 + 16) = (u32x4){out[4], out[5], out[6], out[7]};
+    if (g == 0) {
+        _Float16 dh, mh;
+        const uint16_t d16 = (uint16_t)(sb[0] | (sb[1] << 8)), m16 = (uint16_t)(sb[2] | (sb[3] << 8));
+        __builtin_memcpy(&dh, &d16, 2);
+        __builtin_memcpy(&mh, &m16, 2);
+        float d1[4], m1[4];
+        for (int j = 0; j < 4; j++) {
+            int sc, mn;
+            q4k_scale_min(sb + 4, 4 * (hc & 1) + j, &sc, &mn);
+            d1[j] = __fmul_rn((float)dh, (float)sc);
+            m1[j] = __fmul_rn((float)mh, (float)mn);
+        }
+        *(float4v *)(u + SQ5_K::SCALES_AT + r * 32) = (float4v){d1[0], d1[1], d1[2], d1[3]};
+        *(float4v *)(u + SQ5_K::SCALES_AT + r * 32 + 16) = (float4v){m1[0], m1[1], m1[2], m1[3]};
+    }
+}
+
+__global__ void __launch_bounds__(256) dequant_packed_q5_k_kernel(const uint8_t *__restrict__ packed, float *__restrict__ dst, int n,
+                                                                  int k) {
+    const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= (size_t)n * k) return;
+    const int row = (int)(idx / k), col = (int)(idx % k);
+    const int T = row >> 4, r = row & 15, hc = col >> 7, j = (col >> 5) & 3, e = col & 31;
+    const int n_hc = k >> 7;
+    const uint8_t *u = packed + ((size_t)T * n_hc + hc) * SQ5_K::UNIT;
+    int g = 0, slot = 0;
+    for (int gg = 0; gg < 4; gg++)
+        for (int i = 0; i < 8; i++)
+            if (elt_of(gg, i) == e) {
+                g = gg;
+                slot = i;
+            }
+    const int q = (int)u[(g * 16 + r) * 32 + j * 8 + q8_byte_of_slot(slot)];
+    float d1, m1;
+    __builtin_memcpy(&d1, u + SQ5_K::SCALES_AT + r * 32 + j * 4, 4);
+    __builtin_memcpy(&m1, u + SQ5_K::SCALES_AT + r * 32 + 16 + j * 4, 4);
     dst[idx] = __fsub_rn(__fmul_rn(d1, (float)q), m1);
 }
 
@@ -883,6 +999,7 @@ qtiles_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, 
         }
 }
 
+bool has_min(int fmt) { return fmt == VX_Q4_K || fmt == VX_Q5_K; }
 struct TilesPlan {
     int r, s;  // weight tiles a wave, K slices; r == 0: not served
 };
@@ -891,7 +1008,7 @@ struct TilesPlan {
 TilesPlan tiles_plan(int fmt, int n_tiles, int n_hc, int mgroups, int cus) {
     TilesPlan pl = {0, 1};
     // (four tiles a wave: 64 more accumulators than there are registers; Q6_K's units and Q4_K's block sums leave room for two)
-    int r = (fmt == VX_Q6_K || fmt == VX_Q4_K) ? 2 : 3;
+    int r = (fmt == VX_Q6_K || has_min(fmt)) ? 2 : 3;
     while (r > 1 && (n_tiles < r || ceil_div(n_tiles, NW * r) * mgroups * 4 < cus)) r--;  // few rows: more, smaller workgroups
     if (n_tiles < r) return pl;
     const int base = ceil_div(n_tiles, NW * r) * mgroups;
@@ -963,12 +1080,14 @@ struct PackedW {
     size_t bytes;  // of the raw matrix (what a write into it is checked against)
 };
 
-bool packable(int fmt) { return fmt == VX_Q4_0 || fmt == VX_Q8_0 || fmt == VX_Q6_K || fmt == VX_Q4_K; }
+bool packable(int fmt) { return fmt == VX_Q4_0 || fmt == VX_Q8_0 || fmt == VX_Q6_K || fmt == VX_Q4_K || fmt == VX_Q5_0 || fmt == VX_Q5_K; }
 size_t raw_row_bytes(int fmt, int K) {
     switch (fmt) {
     case VX_Q4_0: return (size_t)K / 32 * 18;
     case VX_Q8_0: return (size_t)K / 32 * 34;
     case VX_Q4_K: return (size_t)K / 256 * 144;
+    case VX_Q5_0: return (size_t)K / 32 * 22;
+    case VX_Q5_K: return (size_t)K / 256 * 176;
     default: return (size_t)K / 256 * 210;
     }
 }
@@ -976,12 +1095,14 @@ int unit_bytes(int fmt) {
     switch (fmt) {
     case VX_Q4_0: return SQ4_0::UNIT;
     case VX_Q8_0: return SQ8_0::UNIT;
+    case VX_Q5_0: return SQ8_0::UNIT;
     case VX_Q4_K: return SQ4_K::UNIT;
+    case VX_Q5_K: return SQ5_K::UNIT;
     default: return SQ6_K::UNIT;
     }
 }
 // half chunks whose operands a wave's registers hold beside the format's requests in flight
-int max_ph_of(int fmt, int M) { return (M > 32 || fmt == VX_Q6_K || fmt == VX_Q4_K) ? 1 : 2; }
+int max_ph_of(int fmt, int M) { return (M > 32 || fmt == VX_Q6_K || fmt == VX_Q4_K || fmt == VX_Q5_K) ? 1 : 2; }
 
 }  // namespace
 
@@ -1055,7 +1176,7 @@ bool stream_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int 
     if (off && atoi(off)) return false;
     if (M < 2 || M > 64 || N % 16 != 0 || K % 256 != 0 || N < 16) return false;
     if (epi && M > 32) return false;
-    if (fmt == VX_Q4_K && M > 32) return false;  // the block sums of four activation tiles do not fit the registers
+    if (has_min(fmt) && M > 32) return false;  // the block sums of four activation tiles do not fit the registers
     // With the epilogue the whole K stays in one workgroup, which walks it in passes of 16 half chunks; every pass
     // starts its requests anew, and for two passes and more the launch takes longer than the wave-private kernel's
     // (7B Q|K|V, 32 rows: 23.8 against 20.9 us). VEXEL_HIP_STREAM_EPI=1 takes it anyway (measurements).
@@ -1110,7 +1231,7 @@ int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_e
     if (mt != 1 && mt != 2 && mt != 4) return VX_ERR_UNSUPPORTED;
     const int max_ph = max_ph_of(fmt, M);
     const StreamPlan pl = stream_plan(N / 16, K / 128, cus, fin, N, K, max_ph);
-    if (pl.g == 0 || (max_ph == 1 && (fin || pl.ph != 1)) || (fmt == VX_Q4_K && mt == 4)) return VX_ERR_UNSUPPORTED;
+    if (pl.g == 0 || (max_ph == 1 && (fin || pl.ph != 1)) || (has_min(fmt) && mt == 4)) return VX_ERR_UNSUPPORTED;
     StreamShape a;
     a.M = M;
     a.Mpad = mpad;
@@ -1128,8 +1249,9 @@ int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_e
     }
     dim3 grid(pl.g, pl.s);
     if (fmt == VX_Q4_0) launch_stream<SQ4_0>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
-    else if (fmt == VX_Q8_0) launch_stream<SQ8_0>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
+    else if (fmt == VX_Q8_0 || fmt == VX_Q5_0) launch_stream<SQ8_0>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
     else if (fmt == VX_Q4_K) launch_stream<SQ4_K>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
+    else if (fmt == VX_Q5_K) launch_stream<SQ5_K>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
     else launch_stream<SQ6_K>(be, pl, grid, mt, fin, ps, pv, partial, a, e);
     VX_CHECK_LAUNCH();
     if (ks_out) *ks_out = pl.s;
@@ -1190,7 +1312,9 @@ int tiles_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_en
     dim3 grid(ceil_div(N / 16, NW * pl.r), pl.s, mgroups);
     switch (fmt) {
     case VX_Q4_0: launch_tiles<SQ4_0>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
-    case VX_Q8_0: launch_tiles<SQ8_0>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
+    case VX_Q8_0:
+    case VX_Q5_0: launch_tiles<SQ8_0>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
+    case VX_Q5_K: launch_tiles<SQ5_K>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
     case VX_Q4_K: launch_tiles<SQ4_K>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
     default: launch_tiles<SQ6_K>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
     }
@@ -1221,6 +1345,10 @@ int vx_qweight_pack(vx_backend *be, const vx_qweight *w) {
         pack_q4_0_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
     else if (w->fmt == VX_Q8_0)
         pack_q8_0_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
+    else if (w->fmt == VX_Q5_0)
+        pack_q5_0_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
+    else if (w->fmt == VX_Q5_K)
+        pack_q5_k_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
     else if (w->fmt == VX_Q4_K)
         pack_q4_k_kernel<<<dim3(w->n / 16, w->k / 128), 64, 0, be->stream>>>((const uint8_t *)w->data, (uint8_t *)pw->data, w->k / 128);
     else
@@ -1261,7 +1389,9 @@ int vx_dequantize_packed(vx_backend *be, const vx_qweight *w, float *dst) {
     const size_t total = (size_t)w->n * w->k;
     if (pw->fmt == VX_Q4_0)
         dequant_packed_q4_0_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
-    else if (pw->fmt == VX_Q8_0)
+    else if (pw->fmt == VX_Q5_K)
+        dequant_packed_q5_k_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
+    else if (pw->fmt == VX_Q8_0 || pw->fmt == VX_Q5_0)
         dequant_packed_q8_0_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
     else if (pw->fmt == VX_Q4_K)
         dequant_packed_q4_k_kernel<<<(unsigned)((total + 255) / 256), 256, 0, be->stream>>>((const uint8_t *)pw->data, dst, w->n, w->k);
