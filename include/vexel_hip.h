@@ -214,6 +214,11 @@ int vx_matmul_quant_prepared(vx_backend *be, int fmt, const void *b, float *out,
 /* 1 when the [n,k] matrix can take the prepared MFMA path: k % 256 == 0, a 16-byte aligned pointer, and rows
  * that are a multiple of 16 bytes (Q6_K: the whole matrix is, e.g. n % 8 == 0). */
 int vx_matmul_quant_has_fast_path(int fmt, const void *b, int n, int k);
+/* Which kernel family the backend's last quantized matmul launch took ("qmatvec_kernel", "qstream_kernel",
+ * "qtiles_kernel", "qgemm_wave_kernel", "qgemm_rows_kernel", "qgemm_kernel", "qrow4_kernel",
+ * "qgemm_fallback_kernel"; "" before the first). No counterpart in the reference; for tests and reports that must
+ * know that the path they measure is the one a default configuration runs. */
+const char *vx_last_matmul_kernel(vx_backend *be);
 
 /* Fused decode blocks (the reference's FusedOps idea, backend.go:128-158, re-cut for the batched
  * paged path). They compute what the unfused call sequence computes, with each projection group

@@ -188,6 +188,31 @@ def test_matmul_packed_rows_independent_of_batch(be, fmt):
     be.reset_pool()
 
 
+def test_default_configuration_takes_the_kernels_the_benchmark_reports(be):
+    """With no environment switch set, a packed matrix runs the streaming kernel at 2 .. 64 rows and the many-rows
+    kernel beyond, one row the matrix-vector kernel, and an unpacked matrix the kernels over the GGUF rows: the paths
+    bench.py times are the paths a default process takes."""
+    import os
+    if [k for k in os.environ if k.startswith("VEXEL_HIP_")]:
+        pytest.skip("a VEXEL_HIP_* switch is set: this is not the default configuration")
+    rng = np.random.default_rng(21)
+    n, k = 256, 4096
+    w = qz.random_quant(nx.FMT_Q4_0, rng, n, k)
+    a = rng.standard_normal((256, k)).astype(np.float32)
+    dw, qw = _packed(be, w, n, k)
+    da, dout = be.upload(a), be.alloc(256 * n * 4)
+    for m, want in ((1, "qmatvec_kernel"), (2, "qstream_kernel"), (32, "qstream_kernel"), (64, "qstream_kernel"),
+                    (65, "qtiles_kernel"), (256, "qtiles_kernel")):
+        be.matmul_quant(nx.FMT_Q4_0, da, dw, dout, None, m, n, k)
+        assert be.last_matmul_kernel() == want, (m, be.last_matmul_kernel())
+    be.qweight_unpack(qw)
+    for m, want in ((1, "qmatvec_kernel"), (32, "qgemm_wave_kernel"), (256, "qgemm_kernel")):
+        be.matmul_quant(nx.FMT_Q4_0, da, dw, dout, None, m, n, k)
+        assert be.last_matmul_kernel() == want, (m, be.last_matmul_kernel())
+    be.free(dw)
+    be.reset_pool()
+
+
 def test_rewriting_the_matrix_drops_the_packed_copy(be):
     rng = np.random.default_rng(5)
     n, k, m = 64, 512, 8

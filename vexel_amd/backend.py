@@ -60,6 +60,10 @@ class HipBackend:
         """vx_backend_set_attn_merge: the decode attention kernel merges its own splits (default) or not."""
         self.call("vx_backend_set_attn_merge", int(bool(on)))
 
+    def last_matmul_kernel(self):
+        """vx_last_matmul_kernel: the kernel family of the last quantized matmul launch."""
+        return self._lib.vx_last_matmul_kernel(self._h).decode()
+
     def scratch_generation(self):
         """How often the library's own scratch buffers have moved (a kept graph is stale once this changes)."""
         return int(self._lib.vx_scratch_generation(self._h))

@@ -55,6 +55,7 @@ struct vx_backend {
     int device = 0;
     hipStream_t stream = nullptr;
     bool capturing = false;
+    const char *last_matmul = "";  // kernel family of the last quantized matmul launch (vx_last_matmul_kernel)
 
     // per-step pool (vx_alloc / vx_reset_pool)
     std::vector<vx::PoolChunk> chunks;

@@ -1894,6 +1894,7 @@ int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out
         int rc = stream_gemm(be, fmt, segs.w, segs.n_end, 3, N, K, M, mpad, spv, epi_in, &ks);
         if (rc != VX_ERR_UNSUPPORTED) {
             if (rc) return rc;
+            be->last_matmul = "qstream_kernel";
             if (ks_out) *ks_out = ks;
             if (!fin && !to_partials) {
                 const size_t total = (size_t)M * N;
@@ -1911,6 +1912,7 @@ int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out
         int rc = tiles_gemm(be, fmt, segs.w, segs.n_end, 3, N, K, M, mpad, spv, out, residual, to_partials, &ks);
         if (rc != VX_ERR_UNSUPPORTED) {
             if (rc) return rc;
+            be->last_matmul = "qtiles_kernel";
             if (ks_out) *ks_out = ks;
             if (!to_partials && ks > 1) {
                 const size_t total = (size_t)M * N;
@@ -1923,16 +1925,19 @@ int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out
     }
     const WavePlan rp = rows_plan(be, fmt, segs, N, K, M);
     if (rp.r > 0) {
+        be->last_matmul = "qgemm_rows_kernel";
         return launch_gemm_rows_r<WQ8_0>(be, rp, segs, N, out, residual, to_partials, M, K, ks_out);
     }
     const QkvEpi epi = epi_in ? *epi_in : QkvEpi{};  // (with an epilogue the caller has checked that the wave plan applies)
     const WavePlan pl = wave_plan(be, fmt, segs, N, K, M);
     if (pl.r > 0) {
+        be->last_matmul = "qgemm_wave_kernel";
         if (fmt == VX_Q4_0) return launch_gemm_wave_r<WQ4_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
         if (fmt == VX_Q8_0) return launch_gemm_wave_r<WQ8_0>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
         if (fmt == VX_BF16) return launch_gemm_wave_r<WBF16>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
         return launch_gemm_wave_r<WQ4_K>(be, pl, segs, N, out, residual, to_partials, M, K, ks_out, epi);
     }
+    be->last_matmul = "qgemm_kernel";
     switch (fmt) {
     case VX_Q4_0: return launch_gemm<PQ4_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
     case VX_Q8_0: return launch_gemm<PQ8_0>(be, segs, N, out, residual, to_partials, M, K, ks_out);
@@ -2061,6 +2066,8 @@ int vx_matmul_quant_prepared(vx_backend *be, int fmt, const void *b, float *out,
 
 int vx_matmul_quant_has_fast_path(int fmt, const void *b, int n, int k) { return fast_ok(fmt, b, n, k) ? 1 : 0; }
 
+const char *vx_last_matmul_kernel(vx_backend *be) { return be ? be->last_matmul : ""; }
+
 int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, float *out, const float *residual, int m,
                     int n, int k) {
     int rc = enter(be);
@@ -2073,7 +2080,10 @@ int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, floa
     static const bool no_matvec = getenv("VEXEL_HIP_NO_MATVEC") != nullptr;  // keeps M = 1 on the batched kernel
     if (m == 1 && !no_matvec) {  // a single row: the streaming matrix-vector kernel
         rc = run_matvec(be, fmt, a, b, out, residual, n, k);
-        if (rc != VX_ERR_UNSUPPORTED) return rc;
+        if (rc != VX_ERR_UNSUPPORTED) {
+            be->last_matmul = "qmatvec_kernel";
+            return rc;
+        }
     }
     if (fmt == VX_BF16 && m >= 2 && k % 256 == 0 && ((uintptr_t)a % 16) == 0 && ((uintptr_t)b % 16) == 0) {
         // the matrix cores: bf16 -> f16 is exact for weights, the activations enter as hi + lo as everywhere
@@ -2097,10 +2107,12 @@ int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, floa
             else if (fmt == VX_Q5_K) qrow4_kernel<VX_Q5_K><<<grid, 64, 0, be->stream>>>(w, a, out, residual, m, n, k, rb);
             else qrow4_kernel<VX_BF16><<<grid, 64, 0, be->stream>>>(w, a, out, residual, m, n, k, rb);
             VX_CHECK_LAUNCH();
+            be->last_matmul = "qrow4_kernel";
             return VX_OK;
         }
         qgemm_fallback_kernel<<<grid, 64, 0, be->stream>>>(fmt, (const uint8_t *)b, a, out, residual, m, n, k, rb);
         VX_CHECK_LAUNCH();
+        be->last_matmul = "qgemm_fallback_kernel";
         return VX_OK;
     }
     rc = vx_prepare_act(be, a, m, k);

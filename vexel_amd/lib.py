@@ -75,6 +75,7 @@ SIGNATURES = {
     "vx_silu_mul_prepare": (_i, [_vp, _vp, _vp, _vp, _i, _i]),
     "vx_matmul_quant_prepared": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i]),
     "vx_matmul_quant_has_fast_path": (_i, [_i, _vp, _i, _i]),
+    "vx_last_matmul_kernel": (C.c_char_p, [_vp]),
     "vx_rope_table_prepare": (_i, [_vp, _vp, _i, _i, _f]),
     "vx_decode_attn_qkv_supported": (_i, [_vp, _vp, _vp, _i]),
     "vx_decode_attn_qkv_ex": (_i, [_vp, _vp, _vp, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i,
