@@ -329,14 +329,17 @@ def time_step_gemms(be, mr, c, rows):
                 for p in ptrs:
                     be.matmul_quant_prepared(fmt, p, dst, None, rows, n, k)
             timed.append(be.timer_stop_ms() * 1e3 / (reps * len(ptrs)))
+        kernel = be.last_matmul_kernel()
         us = timed[0]
         nbytes = int(n * k * bpe[fmt]) + rows * k * 4 + rows * n * 4
         res[name] = {"n": n, "k": k, "us": round(us, 2), "us_with_reduction": round(timed[1], 2), "bytes": nbytes,
-                     "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)}
+                     "frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "kernel": kernel}
         if name == "Q|K|V":
             fused = time_fused_qkv(be, lw, c, rows, acts[k])
             if fused is not None:   # what the step launches for Q|K|V: the projection with RoPE and the KV store in its epilogue
                 res[name]["us_projection_alone"] = res[name]["us"]
+                res[name]["kernel_projection_alone"] = res[name]["kernel"]
+                res[name]["kernel"] = be.last_matmul_kernel()
                 res[name]["us"] = us = round(fused, 2)
                 res[name]["frac"] = round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)
         total_us += us
@@ -344,7 +347,8 @@ def time_step_gemms(be, mr, c, rows):
     be.free(out)
     for p in acts.values():
         be.free(p)
-    return {"bound": "hbm", "kernel": "qstream_kernel / qgemm_wave_kernel (the step's four projection launches per layer, M=%d)" % rows,
+    return {"bound": "hbm", "kernel": "%s (the step's four projection launches per layer, M=%d)"
+                                      % (" / ".join(sorted({v["kernel"] for v in res.values()})), rows),
             "achieved": total_bytes / total_us / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
             "frac": total_bytes / total_us / 1e3 / HBM_PEAK_GBS,
             "traffic": GEMM_TRAFFIC_PER_ALGORITHMIC_BYTE * total_bytes if rows == BATCH else None,

@@ -329,12 +329,12 @@ __device__ __forceinline__ void finish_split(const float (&s_m)[4][G * RG], cons
 
 // RG > 1: an entry of the batch is RG consecutive query rows that share one sequence's context (the rows of a
 // candidate tree): the workgroup serves the G*RG queries (row, head) of its kv head from one pass over the K/V.
-template <int D, int G, int RG = 1>
-__global__ void __launch_bounds__(256) paged_decode_f16_kernel(
-    const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix,
-    const int32_t *__restrict__ bt_rows, int max_blocks, const int32_t *__restrict__ kv_lens,
-    float *__restrict__ partial, int num_q_heads, int num_kv_heads, float scale, int max_splits,
-    const int32_t *__restrict__ items, MergeOut mg, int tps) {
+// One item of the work: the tokens of split `split` of sequence `seq` for kv head `kvh` (all of the workgroup).
+template <int D, int G, int RG>
+__device__ __forceinline__ void paged_decode_f16_item(
+    const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix, int max_blocks,
+    float *__restrict__ partial, int num_q_heads, int num_kv_heads, float scale, int max_splits, const MergeOut &mg, int tps,
+    const int kvh, const int split, const int seq, int kv_len, const int row) {
     constexpr int GG = G * RG;       // queries per K/V row
     constexpr int DL = D / 8;        // 8-element slices of a head vector
     // lanes per token: the next power of two; the lanes past DL (heads of 80 or 96) repeat the last slice's loads
@@ -344,19 +344,6 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
     constexpr int TPI = 64 / LPT;    // tokens per load instruction
     constexpr int NL = HOT_BS / TPI; // load instructions per block and per K or V
     typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-    const int kvh = blockIdx.x;
-    int split = blockIdx.y, seq = blockIdx.z, kv_len, row;
-    if (items) {  // work list: grid.y runs over the items, the workgroups past the list's end are the grid's last
-        if ((int)blockIdx.y >= items[0]) return;
-        const int4 rec = ((const int4 *)(items + 4))[blockIdx.y];  // (sequence, split, kv length, table row)
-        seq = rec.x;
-        split = rec.y;
-        kv_len = rec.z;
-        row = rec.w;
-    } else {
-        kv_len = kv_lens[seq];
-        row = bt_rows ? bt_rows[seq] : seq;
-    }
     // The caller's max_kv_len sized the partial sums (max_splits per sequence and head). A length above it is
     // attended over its first max_splits * TPW tokens by every kernel of the path alike: defined, and inside the
     // buffers.
@@ -490,6 +477,34 @@ __global__ void __launch_bounds__(256) paged_decode_f16_kernel(
         }
     }
     finish_split<D, G, RG>(s_m, s_l, s_acc, partial, seq, kvh, split, kv_len, num_q_heads, num_kv_heads, max_splits, mg, tps);
+}
+
+// grid = (kv heads, items or splits, 1 or sequences). With a work list a workgroup walks the items y, y + grid.y, ...;
+// the grid's second dimension normally covers the most items the list can hold, so that every workgroup takes one
+// item or none (the host cannot know how many the packing kernel listed; the empty workgroups are the grid's last and
+// cost nothing measurable). A grid of just the workgroups the device holds at once, each walking several items
+// (VEXEL_HIP_ATTN_WG_PER_CU=n), measured slower at 4, 5, 6 and 8 per compute unit (110.6 - 118.7 us against 105.5):
+// the dispatcher hands the next item to whichever slot frees first, a fixed stride does not.
+template <int D, int G, int RG = 1>
+__global__ void __launch_bounds__(256) paged_decode_f16_kernel(
+    const float *__restrict__ q, const _Float16 *__restrict__ pool, const int32_t *__restrict__ bt_matrix,
+    const int32_t *__restrict__ bt_rows, int max_blocks, const int32_t *__restrict__ kv_lens,
+    float *__restrict__ partial, int num_q_heads, int num_kv_heads, float scale, int max_splits,
+    const int32_t *__restrict__ items, MergeOut mg, int tps) {
+    const int kvh = blockIdx.x;
+    if (items) {
+        const int n = __builtin_amdgcn_readfirstlane(items[0]);
+        for (int it = blockIdx.y; it < n; it += gridDim.y) {
+            const int4 rec = ((const int4 *)(items + 4))[it];  // (sequence, split, kv length, table row)
+            paged_decode_f16_item<D, G, RG>(q, pool, bt_matrix, max_blocks, partial, num_q_heads, num_kv_heads, scale, max_splits, mg,
+                                            tps, kvh, rec.y, rec.x, rec.z, rec.w);
+            __syncthreads();  // (the next item reuses the workgroup's LDS)
+        }
+    } else {
+        const int seq = blockIdx.z;
+        paged_decode_f16_item<D, G, RG>(q, pool, bt_matrix, max_blocks, partial, num_q_heads, num_kv_heads, scale, max_splits, mg, tps,
+                                        kvh, blockIdx.y, seq, kv_lens[seq], bt_rows ? bt_rows[seq] : seq);
+    }
 }
 
 // The same split of the work for grouped queries (G*RG = 2 .. 16 queries per K/V row) on the matrix cores: the vector
@@ -1355,6 +1370,14 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
                         (size_t)batch * max_splits <= 65535;
     const int32_t *const list = listed ? be->items.buf + list_off : nullptr;
     dim3 grid(num_kv_heads, listed ? batch * max_splits : max_splits, listed ? 1 : batch);
+    // (for measurements: the vector kernel walking the list with n workgroups per compute unit instead)
+    static const int gy_env = getenv("VEXEL_HIP_ATTN_WG_PER_CU") ? atoi(getenv("VEXEL_HIP_ATTN_WG_PER_CU")) : 0;
+    dim3 grid_walk = grid;
+    if (listed && gy_env > 0) {
+        static int cus = 0;
+        if (cus == 0 && (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0)) cus = 256;
+        grid_walk.y = (unsigned)std::max(1, std::min(batch * max_splits, ceil_div(cus * gy_env, num_kv_heads)));
+    }
     // out == NULL leaves the result to vx_decode_ffn(attn = NULL): as split partial sums, and - where the shape
     // allows - already merged by the workgroups that finish last: prepared as that call's first operand, or, for
     // a single row, as plain floats behind the partial sums (what the matrix-vector product reads).
@@ -1393,7 +1416,7 @@ int launch_hot(vx_backend *be, const float *q, const void *pool, const int32_t *
     }
     if constexpr (G <= 8) {  // (wider groups have the matrix-core form only)
         if (!launched)
-            paged_decode_f16_kernel<D, G><<<grid, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
+            paged_decode_f16_kernel<D, G><<<grid_walk, 256, 0, be->stream>>>(q, (const _Float16 *)pool, bt_matrix, bt_rows,
                                                                         max_blocks, kv_lens, ws, num_q_heads,
                                                                         num_kv_heads, scale, max_splits,
                                                                         list, mg, tps);
