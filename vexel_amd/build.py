@@ -17,6 +17,9 @@ SOURCES = ["backend.hip", "elementwise.hip", "attention.hip", "qgemm.hip", "qstr
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-fvisibility=default",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         # float32 operations round one by one, as the reference's Go on amd64 does (cpu.go never fuses a multiply
+         # with an add); where a fused multiply-add is meant the kernels call fmaf themselves
+         "-ffp-contract=off",
          "-Wall", "-Wno-unused-function",
          "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
 
