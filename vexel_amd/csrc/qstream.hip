@@ -860,18 +860,24 @@ qtiles_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, 
         for (int t = 0; t < MT; t++) run[r][t] = (float4v){0.f, 0.f, 0.f, 0.f};
     if (n_half <= 0) return;
 
-    Unit ring[R];
     half8 areg[4];
-    auto fetch = [&](int q) __attribute__((always_inline)) {
+    // half chunk q of the slice (past the end: the last again): the wave's R units into `dst`, this thread's pieces of
+    // the activation tiles into areg
+    auto fetch = [&](int q, Unit (&dst)[R]) __attribute__((always_inline)) {
         const int hc = h_begin + min(q, n_half - 1);
 #pragma unroll
-        for (int r = 0; r < R; r++) ring[r] = W::load(tb[r] + (size_t)hc * W::UNIT, lane, ln);
+        for (int r = 0; r < R; r++) dst[r] = W::load(tb[r] + (size_t)hc * W::UNIT, lane, ln);
 #pragma unroll
         for (int sp = 0; sp < 4; sp++) areg[sp] = gload<half8>(a_src + (size_t)(hc * 4 + sp) * mtiles * 128);
     };
     auto commit = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
-        for (int sp = 0; sp < 4; sp++) a_lds[buf][sp * 512 + tid] = areg[sp];
+        for (int sp = 0; sp < 4; sp++) {
+            if constexpr (W::TWO_SCALES)  // elements 0 - 15 of the step (dwords 0, 2) in front of elements 16 - 31
+                a_lds[buf][sp * 512 + tid] = __builtin_shufflevector(areg[sp], areg[sp], 0, 1, 4, 5, 2, 3, 6, 7);
+            else
+                a_lds[buf][sp * 512 + tid] = areg[sp];
+        }
     };
     auto load_cs = [&](int chunk, float4v (&cs)[MT]) __attribute__((always_inline)) {
 #pragma unroll
@@ -882,16 +888,11 @@ qtiles_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, 
     };
 
     float4v cs[MT];
-    fetch(0);
-    load_cs(h_begin >> 1, cs);
-    commit(0);
-    __syncthreads();
-    for (int q = 0; q < n_half; q++) {
+    // One half chunk: the units in `cur` against the tiles in LDS buffer q & 1, while the next half chunk's units go to
+    // `nxt` (two sets of registers that swap roles from one half chunk to the next, so nothing is copied).
+    auto half_chunk = [&](int q, const Unit (&cur)[R], Unit (&nxt)[R]) __attribute__((always_inline)) {
         const int hc = h_begin + q;
-        Unit cur[R];
-#pragma unroll
-        for (int r = 0; r < R; r++) cur[r] = ring[r];
-        fetch(q + 1);
+        fetch(q + 1, nxt);
         if (q > 0 && (hc & 1) == 0) {  // a new chunk: the sums move to its activation scale
             float4v cn[MT];
             load_cs(hc >> 1, cn);
@@ -911,10 +912,24 @@ qtiles_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, 
 #pragma unroll
         for (int sp = 0; sp < 4; sp++) {
             half8 ah[MT], al[MT];
+            half4v ah16[MT][2], al16[MT][2];  // (two scales a step) the operand halves of elements 0 - 15 and 16 - 31
+            if constexpr (W::TWO_SCALES) {
+                // (commit() has put each tile's dwords 0, 2 in front of its dwords 1, 3: the two halves of the 16 bytes
+                // a lane reads are the two operands as they stand, no register copies)
 #pragma unroll
-            for (int t = 0; t < MT; t++) {
-                ah[t] = ab[sp * 512 + (t * 2 + 0) * 64 + lane];
-                al[t] = ab[sp * 512 + (t * 2 + 1) * 64 + lane];
+                for (int t = 0; t < MT; t++) {
+                    const half8 vh = ab[sp * 512 + (t * 2 + 0) * 64 + lane], vl = ab[sp * 512 + (t * 2 + 1) * 64 + lane];
+                    ah16[t][0] = __builtin_shufflevector(vh, vh, 0, 1, 2, 3);
+                    ah16[t][1] = __builtin_shufflevector(vh, vh, 4, 5, 6, 7);
+                    al16[t][0] = __builtin_shufflevector(vl, vl, 0, 1, 2, 3);
+                    al16[t][1] = __builtin_shufflevector(vl, vl, 4, 5, 6, 7);
+                }
+            } else {
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    ah[t] = ab[sp * 512 + (t * 2 + 0) * 64 + lane];
+                    al[t] = ab[sp * 512 + (t * 2 + 1) * 64 + lane];
+                }
             }
             float4v bs[MT];
             if constexpr (W::HAS_MIN) {
@@ -934,10 +949,9 @@ qtiles_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, 
                         float4v P[MT];
 #pragma unroll
                         for (int t = 0; t < MT; t++)
-                            P[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(h ? second16(ah[t]) : first16(ah[t]), wb, (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                            P[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(ah16[t][h], wb, (float4v){0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
 #pragma unroll
-                        for (int t = 0; t < MT; t++)
-                            P[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(h ? second16(al[t]) : first16(al[t]), wb, P[t], 0, 0, 0);
+                        for (int t = 0; t < MT; t++) P[t] = __builtin_amdgcn_mfma_f32_16x16x16f16(al16[t][h], wb, P[t], 0, 0, 0);
 #pragma unroll
                         for (int t = 0; t < MT; t++)
 #pragma unroll
@@ -968,6 +982,24 @@ qtiles_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, 
         // the next half chunk's activation tiles into the buffer every wave finished with before the previous barrier
         commit((q + 1) & 1);
         __syncthreads();
+    };
+    Unit ua[R], ub[R];
+    fetch(0, ua);
+    load_cs(h_begin >> 1, cs);
+    commit(0);
+    __syncthreads();
+    if constexpr (W::HAS_MIN) {
+        // (with the block sums' loads in the step the twice-unrolled loop runs out of registers: one set, copied)
+        for (int q = 0; q < n_half; q++) {
+#pragma unroll
+            for (int r = 0; r < R; r++) ub[r] = ua[r];
+            half_chunk(q, ub, ua);
+        }
+    } else {
+        for (int q = 0; q < n_half; q += 2) {
+            half_chunk(q, ua, ub);
+            if (q + 1 < n_half) half_chunk(q + 1, ub, ua);
+        }
     }
 #pragma unroll
     for (int r = 0; r < R; r++)
