@@ -1035,28 +1035,30 @@ bool has_min(int fmt) { return fmt == VX_Q4_K || fmt == VX_Q5_K; }
 struct TilesPlan {
     int r, s;  // weight tiles a wave, K slices; r == 0: not served
 };
-// Tiles per wave by what the format's units leave of the registers; K slices so that the grid fills the device in
-// whole rounds where it can (efficiency = workgroups / (rounds x compute units)), each slice at least two half chunks.
+// Weight tiles a wave (at most what the format's units leave of the registers: four tiles are 64 more accumulators
+// than there are; Q6_K's units and the block sums of the formats with a min term leave room for two) and K slices,
+// chosen together by a small cost model in units of about a microsecond: rounds of workgroups over the device x (a
+// half chunk's time, which grows with the tiles a wave owns, x half chunks per slice + a fixed part) + the round trip
+// of the slices' sums. Depends on the format, the matrix' shape and the number of 64-row groups only.
 TilesPlan tiles_plan(int fmt, int n_tiles, int n_hc, int mgroups, int cus) {
     TilesPlan pl = {0, 1};
-    // (four tiles a wave: 64 more accumulators than there are registers; Q6_K's units and Q4_K's block sums leave room for two)
-    int r = (fmt == VX_Q6_K || has_min(fmt)) ? 2 : 3;
-    while (r > 1 && (n_tiles < r || ceil_div(n_tiles, NW * r) * mgroups * 4 < cus)) r--;  // few rows: more, smaller workgroups
-    if (n_tiles < r) return pl;
-    const int base = ceil_div(n_tiles, NW * r) * mgroups;
-    int best = 1;
+    const int rmax = (fmt == VX_Q6_K || has_min(fmt)) ? 2 : 3;
+    // a tile's time per half chunk relative to Q4_0's: Q6_K issues twice the MFMAs and scale FMAs, a min term adds FMAs
+    const float unit = fmt == VX_Q6_K ? 1.9f : (has_min(fmt) ? 1.3f : 1.f);
     float best_cost = 1e30f;
-    for (int s = 1; s <= std::min(16, std::max(1, n_hc / 2)); s++) {
-        const int wgs = base * s, rounds = ceil_div(wgs, cus);
-        // time of a round ~ half chunks per slice + a fixed part; the slices' sums cost their round trip
-        const float cost = (float)rounds * ((float)ceil_div(n_hc, s) + 3.f) + (s > 1 ? 0.15f * (float)s * (float)n_hc / 16.f : 0.f);
-        if (cost < best_cost) {
-            best_cost = cost;
-            best = s;
+    for (int r = std::min(rmax, n_tiles); r >= 1; r--) {
+        const int base = ceil_div(n_tiles, NW * r) * mgroups;
+        for (int s = 1; s <= std::min(16, std::max(1, n_hc / 2)); s++) {
+            const int rounds = ceil_div(base * s, cus);
+            const float sums = s > 1 ? (float)s * 64.f * (float)mgroups * 16.f * (float)n_tiles * 1.0e-6f : 0.f;
+            const float cost = (float)rounds * (((float)r * unit + 0.4f) * (float)ceil_div(n_hc, s) + 4.f) + sums;
+            if (cost < best_cost) {
+                best_cost = cost;
+                pl.r = r;
+                pl.s = s;
+            }
         }
     }
-    pl.r = r;
-    pl.s = best;
     return pl;
 }
 
