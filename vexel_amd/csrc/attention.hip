@@ -209,6 +209,10 @@ __device__ __forceinline__ HalfPair split_hl(float x) {
 }
 typedef float float4v __attribute__((ext_vector_type(4)));
 
+// A read of K/V pool bytes, which a launch reads once: the non-temporal form does not keep the line in the die's L2
+// and streams measurably faster (570 MB: 6.6 - 6.7 TB/s against 5.9 with plain loads).
+template <class T> __device__ __forceinline__ T stream_load(const T *p) { return __builtin_nontemporal_load(p); }
+
 // Sum over the N adjacent lanes (N = 8, 16 or 32, aligned) that hold one token's head vector, by DPP inside a
 // 16-lane row (no LDS traffic): quads, then the mirrored quad of the half, then the mirrored half; heads of 256
 // span two rows, joined by one cross-row exchange.
@@ -400,8 +404,8 @@ __device__ __forceinline__ void paged_decode_f16_item(
         const _Float16 *base = pool + (size_t)blk * 2 * part + lane_off;
 #pragma unroll
         for (int u = 0; u < NL; u++) {
-            kd[u] = *(const half8 *)(base + (size_t)u * TPI * hs);
-            vd[u] = *(const half8 *)(base + part + (size_t)u * TPI * hs);
+            kd[u] = stream_load((const half8 *)(base + (size_t)u * TPI * hs));
+            vd[u] = stream_load((const half8 *)(base + part + (size_t)u * TPI * hs));
         }
     };
     if (wave < n_blocks) issue(wave, kn, vn);
@@ -634,9 +638,9 @@ __global__ void __launch_bounds__(256, 3) paged_decode_gqa_kernel(
         const int blk = __builtin_amdgcn_readfirstlane(bt[bi]);
         const _Float16 *base = pool + (size_t)blk * 2 * part;
 #pragma unroll
-        for (int s = 0; s < NS; s++) kd[s] = *(const half8 *)(base + k_off + k_step * s);
+        for (int s = 0; s < NS; s++) kd[s] = stream_load((const half8 *)(base + k_off + k_step * s));
 #pragma unroll
-        for (int i = 0; i < 4; i++) vd[i] = *(const halfv *)(base + v_off + (size_t)i * 4 * hs);  // token 4i + g4
+        for (int i = 0; i < 4; i++) vd[i] = stream_load((const halfv *)(base + v_off + (size_t)i * 4 * hs));  // token 4i + g4
     };
     if (wave < n_blocks) issue(wave, kn, vn);
     for (int bi = wave; bi < n_blocks; bi += 4) {
@@ -888,8 +892,8 @@ __global__ void __launch_bounds__(64 * NSUB * KS) paged_mq_kernel(const float *_
 #pragma unroll
             for (int j = 0; j < PPT; j++) {
                 const int pc = min(j * TG + tg, PIECES - 1), row = pc / (D / 8), c8 = pc % (D / 8);
-                kreg[j] = *(const half8 *)(base + (size_t)row * hs + c8 * 8);
-                vreg[j] = *(const half8 *)(base + part + (size_t)row * hs + c8 * 8);
+                kreg[j] = stream_load((const half8 *)(base + (size_t)row * hs + c8 * 8));
+                vreg[j] = stream_load((const half8 *)(base + part + (size_t)row * hs + c8 * 8));
             }
         };
         auto commit = [&](int bi, int buf) {
