@@ -372,7 +372,7 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec_kernel(const MvArgs p) {
             const uint8_t *first = row_base(row) + (start & ~(size_t)15);
             const uint32_t last_piece = (uint32_t)(((start & 15) + (size_t)seg_bytes - 1) >> 4);
             const uint32_t c = min((uint32_t)(((i & (PASSES - 1)) << 6) + lane), last_piece);
-            pc[i] = *(const u32x4 *)(first + c * 16u);
+            pc[i] = __builtin_nontemporal_load((const u32x4 *)(first + c * 16u));
         }
     };
     int grp = blockIdx.x;
@@ -556,7 +556,7 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec2_kernel(const MvArgs p, in
         for (int i = 0; i < NPL; i++) {
             const int c = min(lane + 64 * i, total - 1);
             const uint8_t *b = (pair > 0 && c >= half_pieces) ? b1 : b0;
-            pc[i] = *(const u32x4 *)(b + (size_t)c * 16);
+            pc[i] = __builtin_nontemporal_load((const u32x4 *)(b + (size_t)c * 16));
         }
     };
     const int n_waves = gridDim.x * MV_WAVES;
@@ -776,8 +776,8 @@ __global__ void __launch_bounds__(MV_THREADS) bf16_matvec_kernel(const uint8_t *
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const int pc = min(p0 + 64 * u + lane, pieces - 1);  // (past the row's end: the last piece again, not added)
-                q0[u] = *(const u32x4 *)(w0 + (size_t)pc * 16);
-                q1[u] = *(const u32x4 *)(w1 + (size_t)pc * 16);
+                q0[u] = __builtin_nontemporal_load((const u32x4 *)(w0 + (size_t)pc * 16));
+                q1[u] = __builtin_nontemporal_load((const u32x4 *)(w1 + (size_t)pc * 16));
             }
 #pragma unroll
             for (int u = 0; u < U; u++) {
