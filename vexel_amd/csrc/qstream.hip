@@ -87,7 +87,8 @@ template <int BIAS> __device__ __forceinline__ half8 unpack_q4(uint32_t w, uint3
     const half2v c = as_h2(and_or(w8, 0x000F000Fu, k64)), d = as_h2(and_or(w8, 0x00F000F0u, k64));
     const half2v m1032 = {(_Float16)(-1024.f - BIAS), (_Float16)(-1024.f - BIAS)}, m72 = {(_Float16)(-64.f - BIAS), (_Float16)(-64.f - BIAS)};
     const half2v s16 = {(_Float16)0.0625f, (_Float16)0.0625f};
-    const half2v h0 = a + m1032, h1 = b * s16 + m72, h2 = c + m1032, h3 = d * s16 + m72;
+    // (explicitly fused: the library is built without contraction of a * b + c)
+    const half2v h0 = a + m1032, h1 = __builtin_elementwise_fma(b, s16, m72), h2 = c + m1032, h3 = __builtin_elementwise_fma(d, s16, m72);
     half8 r;
     r[0] = h0[0]; r[1] = h0[1]; r[2] = h1[0]; r[3] = h1[1];
     r[4] = h2[0]; r[5] = h2[1]; r[6] = h3[0]; r[7] = h3[1];
