@@ -209,8 +209,10 @@ __device__ __forceinline__ HalfPair split_hl(float x) {
 }
 typedef float float4v __attribute__((ext_vector_type(4)));
 
-// A read of K/V pool bytes, which a launch reads once: the non-temporal form does not keep the line in the die's L2
-// and streams measurably faster (570 MB: 6.6 - 6.7 TB/s against 5.9 with plain loads).
+// A read of K/V pool bytes that a launch reads once (the decode kernels: one workgroup per KV head and token range):
+// the non-temporal form does not keep the line in the die's L2 and streams measurably faster (570 MB: 6.6 - 6.7 TB/s
+// against 5.9 with plain loads). Not for bytes that several workgroups or two instructions share a line of (the
+// multi-query kernel's rows, weight units of 32 bytes per lane): those measured slower with it.
 template <class T> __device__ __forceinline__ T stream_load(const T *p) { return __builtin_nontemporal_load(p); }
 
 // Sum over the N adjacent lanes (N = 8, 16 or 32, aligned) that hold one token's head vector, by DPP inside a
@@ -892,8 +894,9 @@ __global__ void __launch_bounds__(64 * NSUB * KS) paged_mq_kernel(const float *_
 #pragma unroll
             for (int j = 0; j < PPT; j++) {
                 const int pc = min(j * TG + tg, PIECES - 1), row = pc / (D / 8), c8 = pc % (D / 8);
-                kreg[j] = stream_load((const half8 *)(base + (size_t)row * hs + c8 * 8));
-                vreg[j] = stream_load((const half8 *)(base + part + (size_t)row * hs + c8 * 8));
+                // (plain loads: the workgroups of other row tiles and heads read the same rows, from the die's L2)
+                kreg[j] = *(const half8 *)(base + (size_t)row * hs + c8 * 8);
+                vreg[j] = *(const half8 *)(base + part + (size_t)row * hs + c8 * 8);
             }
         };
         auto commit = [&](int bi, int buf) {

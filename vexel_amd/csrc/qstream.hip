@@ -66,12 +66,6 @@ __device__ __forceinline__ uint32_t and_or(uint32_t x, uint32_t mask, uint32_t k
 template <class T> __device__ __forceinline__ T gload(const void *p) {
     return *(const __attribute__((address_space(1))) T *)(uintptr_t)p;
 }
-// The same for bytes that a launch reads once (weight units in the decode kernel): NT = true makes it a non-temporal
-// load, which leaves the line out of the die's L2 and streams faster.
-template <bool NT, class T> __device__ __forceinline__ T gload_s(const void *p) {
-    if constexpr (NT) return __builtin_nontemporal_load((const __attribute__((address_space(1))) T *)(uintptr_t)p);
-    else return gload<T>(p);
-}
 __device__ __forceinline__ const uint8_t *uniform_ptr(const uint8_t *p) {
     const uint64_t v = (uint64_t)(uintptr_t)p;
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
@@ -123,10 +117,10 @@ struct SQ4_0 {
         u32x4 c;
         u32x2 s;
     };
-    template <bool NT = false> static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
+    static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
         Ring x;
-        x.c = gload_s<NT, u32x4>(u + lane * 16);
-        x.s = gload_s<NT, u32x2>(u + SCALES_AT + ln * 8);
+        x.c = gload<u32x4>(u + lane * 16);
+        x.s = gload<u32x2>(u + SCALES_AT + ln * 8);
         return x;
     }
     static __device__ __forceinline__ half8 codes(const Ring &x, int j, uint32_t k64) { return unpack_q4<8>(x.c[j], k64); }
@@ -145,11 +139,11 @@ struct SQ4_K {
         u32x4 c;
         float4v d1, m1;
     };
-    template <bool NT = false> static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
+    static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
         Ring x;
-        x.c = gload_s<NT, u32x4>(u + lane * 16);
-        x.d1 = gload_s<NT, float4v>(u + SCALES_AT + ln * 32);
-        x.m1 = gload_s<NT, float4v>(u + SCALES_AT + ln * 32 + 16);
+        x.c = gload<u32x4>(u + lane * 16);
+        x.d1 = gload<float4v>(u + SCALES_AT + ln * 32);
+        x.m1 = gload<float4v>(u + SCALES_AT + ln * 32 + 16);
         return x;
     }
     static __device__ __forceinline__ half8 codes(const Ring &x, int j, uint32_t k64) { return unpack_q4<0>(x.c[j], k64); }
@@ -165,11 +159,11 @@ struct SQ8_0 {
         u32x4 c0, c1;
         u32x2 s;
     };
-    template <bool NT = false> static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
+    static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
         Ring x;
-        x.c0 = gload_s<NT, u32x4>(u + lane * 32);
-        x.c1 = gload_s<NT, u32x4>(u + lane * 32 + 16);
-        x.s = gload_s<NT, u32x2>(u + SCALES_AT + ln * 8);
+        x.c0 = gload<u32x4>(u + lane * 32);
+        x.c1 = gload<u32x4>(u + lane * 32 + 16);
+        x.s = gload<u32x2>(u + SCALES_AT + ln * 8);
         return x;
     }
     static __device__ __forceinline__ half8 codes(const Ring &x, int j, uint32_t) {
@@ -189,12 +183,12 @@ struct SQ5_K {
         u32x4 c0, c1;
         float4v d1, m1;
     };
-    template <bool NT = false> static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
+    static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
         Ring x;
-        x.c0 = gload_s<NT, u32x4>(u + lane * 32);
-        x.c1 = gload_s<NT, u32x4>(u + lane * 32 + 16);
-        x.d1 = gload_s<NT, float4v>(u + SCALES_AT + ln * 32);
-        x.m1 = gload_s<NT, float4v>(u + SCALES_AT + ln * 32 + 16);
+        x.c0 = gload<u32x4>(u + lane * 32);
+        x.c1 = gload<u32x4>(u + lane * 32 + 16);
+        x.d1 = gload<float4v>(u + SCALES_AT + ln * 32);
+        x.m1 = gload<float4v>(u + SCALES_AT + ln * 32 + 16);
         return x;
     }
     static __device__ __forceinline__ half8 codes(const Ring &x, int j, uint32_t) {
@@ -225,12 +219,12 @@ struct SQ6_K {
         u32x4 c0, c1;
         float4v s0, s1;
     };
-    template <bool NT = false> static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
+    static __device__ __forceinline__ Ring load(const uint8_t *u, int lane, int ln) {
         Ring x;
-        x.c0 = gload_s<NT, u32x4>(u + lane * 32);
-        x.c1 = gload_s<NT, u32x4>(u + lane * 32 + 16);
-        x.s0 = gload_s<NT, float4v>(u + SCALES_AT + ln * 32);
-        x.s1 = gload_s<NT, float4v>(u + SCALES_AT + ln * 32 + 16);
+        x.c0 = gload<u32x4>(u + lane * 32);
+        x.c1 = gload<u32x4>(u + lane * 32 + 16);
+        x.s0 = gload<float4v>(u + SCALES_AT + ln * 32);
+        x.s1 = gload<float4v>(u + SCALES_AT + ln * 32 + 16);
         return x;
     }
     // h: which 16 elements of block j
@@ -639,7 +633,7 @@ qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1,
         const int hc0 = hp + min(wave, nhp - 1), hc1 = hp + min(NW + wave, nhp - 1);
         auto ldw = [&](int tile, int p) __attribute__((always_inline)) {
             const uint8_t *u = uniform_ptr(tile_base(t0 + min(tile, nt - 1), w0, w1, w2, e0, e1, tile_stride) + (size_t)(p == 0 ? hc0 : hc1) * W::UNIT);
-            return W::template load<true>(u, lane, ln);
+            return W::load(u, lane, ln);
         };
         APhase<MT, W::TWO_SCALES> A[PH];
         float4v bsum[W::HAS_MIN ? PH : 1][4][MT];
