@@ -576,6 +576,31 @@ __global__ void __launch_bounds__(256, 3) paged_decode_gqa_kernel(
     const size_t hs = (size_t)num_kv_heads * D;
     const size_t part = (size_t)HOT_BS * hs;
 
+    const int n_blocks = (t_end - t_begin + HOT_BS - 1) / HOT_BS;
+    // K is loaded as whole rows per instruction, the way V is (LPT lanes a row, TPI rows an instruction), and turned
+    // into the A operand's layout - one row per 16 lanes, a quarter of it per lane group - through the wave's own
+    // LDS rows: loading it in operand layout straight from the pool (16 bytes per lane at four places of every row)
+    // measured 5 - 9 % slower.
+    constexpr int LPT = D / 8, TPI = 64 / LPT;
+    constexpr int KP = D + 8;  // halves per staged row
+    __shared__ __attribute__((aligned(16))) _Float16 kst[4][HOT_BS * KP];
+    const int tok_row = 4 * (c16 & 3) + (c16 >> 2);
+    const size_t k_off = (size_t)(lane / LPT) * hs + (size_t)kvh * D + (lane % LPT) * 8;
+    const size_t k_step = (size_t)TPI * hs;
+    const size_t v_off = part + (size_t)g4 * hs + (size_t)kvh * D + c16 * NT;
+    half8 kk[NS], kn[NS];
+    halfv vv[4], vn[4];
+    auto issue = [&](int bi, half8 *kd, halfv *vd) {
+        const int blk = __builtin_amdgcn_readfirstlane(bt[bi]);
+        const _Float16 *base = pool + (size_t)blk * 2 * part;
+#pragma unroll
+        for (int s = 0; s < NS; s++) kd[s] = stream_load((const half8 *)(base + k_off + k_step * s));
+#pragma unroll
+        for (int i = 0; i < 4; i++) vd[i] = stream_load((const halfv *)(base + v_off + (size_t)i * 4 * hs));  // token 4i + g4
+    };
+    // (the wave's first block is on its way while the query operand is built: the launch waits for K/V bytes)
+    if (wave < n_blocks) issue(wave, kn, vn);
+    __builtin_amdgcn_sched_barrier(0);
     // Q^T as the B operand: lane (query c16, head elements g4 * D/4 + 8s .. + 7 in step s), times scale * log2(e)
     // and the row's power of two, hi + lo
     half8 qh[NS], ql[NS];
@@ -622,29 +647,6 @@ __global__ void __launch_bounds__(256, 3) paged_decode_gqa_kernel(
     for (int e = 0; e < NT; e++) o[e] = (float4v){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;  // of query c16; l_run over this lane's tokens only until the end
 
-    const int n_blocks = (t_end - t_begin + HOT_BS - 1) / HOT_BS;
-    // K is loaded as whole rows per instruction, the way V is (LPT lanes a row, TPI rows an instruction), and turned
-    // into the A operand's layout - one row per 16 lanes, a quarter of it per lane group - through the wave's own
-    // LDS rows: loading it in operand layout straight from the pool (16 bytes per lane at four places of every row)
-    // measured 5 - 9 % slower.
-    constexpr int LPT = D / 8, TPI = 64 / LPT;
-    constexpr int KP = D + 8;  // halves per staged row
-    __shared__ __attribute__((aligned(16))) _Float16 kst[4][HOT_BS * KP];
-    const int tok_row = 4 * (c16 & 3) + (c16 >> 2);
-    const size_t k_off = (size_t)(lane / LPT) * hs + (size_t)kvh * D + (lane % LPT) * 8;
-    const size_t k_step = (size_t)TPI * hs;
-    const size_t v_off = part + (size_t)g4 * hs + (size_t)kvh * D + c16 * NT;
-    half8 kk[NS], kn[NS];
-    halfv vv[4], vn[4];
-    auto issue = [&](int bi, half8 *kd, halfv *vd) {
-        const int blk = __builtin_amdgcn_readfirstlane(bt[bi]);
-        const _Float16 *base = pool + (size_t)blk * 2 * part;
-#pragma unroll
-        for (int s = 0; s < NS; s++) kd[s] = stream_load((const half8 *)(base + k_off + k_step * s));
-#pragma unroll
-        for (int i = 0; i < 4; i++) vd[i] = stream_load((const halfv *)(base + v_off + (size_t)i * 4 * hs));  // token 4i + g4
-    };
-    if (wave < n_blocks) issue(wave, kn, vn);
     for (int bi = wave; bi < n_blocks; bi += 4) {
 #pragma unroll
         for (int s = 0; s < NS; s++) *(half8 *)&kst[wave][(s * TPI + lane / LPT) * KP + (lane % LPT) * 8] = kn[s];
