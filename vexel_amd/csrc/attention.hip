@@ -212,8 +212,12 @@ typedef float float4v __attribute__((ext_vector_type(4)));
 // A read of K/V pool bytes that a launch reads once (the decode kernels: one workgroup per KV head and token range):
 // the non-temporal form does not keep the line in the die's L2 and streams measurably faster (570 MB: 6.6 - 6.7 TB/s
 // against 5.9 with plain loads). Not for bytes that several workgroups or two instructions share a line of (the
-// multi-query kernel's rows, weight units of 32 bytes per lane): those measured slower with it.
-template <class T> __device__ __forceinline__ T stream_load(const T *p) { return __builtin_nontemporal_load(p); }
+// multi-query kernel's rows, weight units of 32 bytes per lane, head vectors of 160 or 192 bytes, whose lines straddle
+// the heads of neighbouring workgroups): those measured slower with it.
+template <bool NT = true, class T> __device__ __forceinline__ T stream_load(const T *p) {
+    if constexpr (NT) return __builtin_nontemporal_load(p);
+    else return *p;
+}
 
 // Sum over the N adjacent lanes (N = 8, 16 or 32, aligned) that hold one token's head vector, by DPP inside a
 // 16-lane row (no LDS traffic): quads, then the mirrored quad of the half, then the mirrored half; heads of 256
@@ -406,8 +410,8 @@ __device__ __forceinline__ void paged_decode_f16_item(
         const _Float16 *base = pool + (size_t)blk * 2 * part + lane_off;
 #pragma unroll
         for (int u = 0; u < NL; u++) {
-            kd[u] = stream_load((const half8 *)(base + (size_t)u * TPI * hs));
-            vd[u] = stream_load((const half8 *)(base + part + (size_t)u * TPI * hs));
+            kd[u] = stream_load<D % 64 == 0>((const half8 *)(base + (size_t)u * TPI * hs));
+            vd[u] = stream_load<D % 64 == 0>((const half8 *)(base + part + (size_t)u * TPI * hs));
         }
     };
     if (wave < n_blocks) issue(wave, kn, vn);
