@@ -1327,7 +1327,12 @@ int tiles_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_en
     static int cus = 0;
     if (cus == 0 && (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0)) cus = 256;
     const int n_hc = K / 128, mgroups = ceil_div(mpad, 64);
-    const TilesPlan pl = tiles_plan(fmt, N / 16, n_hc, mgroups, cus);
+    TilesPlan pl = tiles_plan(fmt, N / 16, n_hc, mgroups, cus);
+    if (const char *env = getenv("VEXEL_HIP_TPLAN")) {  // "r,s" for every shape (tuning)
+        int r = 0, s2 = 0;
+        const int rmax = (fmt == VX_Q6_K || has_min(fmt)) ? 2 : 3;
+        if (sscanf(env, "%d,%d", &r, &s2) == 2 && r >= 1 && r <= rmax && s2 >= 1 && s2 <= std::max(1, n_hc / 2)) pl = {r, s2};
+    }
     if (pl.r == 0) return VX_ERR_UNSUPPORTED;
     StreamShape a;
     a.M = M;
