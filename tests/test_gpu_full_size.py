@@ -76,6 +76,47 @@ def test_7b_and_8b_projection_shapes_q4_0(be, name, n, k):
     _sampled_matmul_check(be, nx.FMT_Q4_0, 1, n, k, rng, name + ", 1 row", 0.02 / 4)
 
 
+# The packed kernels at the configs' real shapes and row counts: the streaming kernel at 32 rows (two activation
+# tiles) and 64 rows (four), the many-rows kernel at 256 rows (a verification step) and 512 (a prompt chunk), in the
+# formats the configs hold there. Full-size GPU product, oracle on a sample of the weight rows.
+@pytest.mark.parametrize("what,fmt,n,k,m", [
+    ("7B gate|up, Q4_0, 32 rows", nx.FMT_Q4_0, 22016, 4096, 32),
+    ("7B gate|up, Q4_0, 512 rows", nx.FMT_Q4_0, 22016, 4096, 512),
+    ("7B down, Q4_0, 512 rows", nx.FMT_Q4_0, 4096, 11008, 512),
+    ("8B gate|up, Q8_0, 64 rows", nx.FMT_Q8_0, 28672, 4096, 64),
+    ("8B down, Q8_0, 64 rows", nx.FMT_Q8_0, 4096, 14336, 64),
+    ("8B down, Q8_0, 512 rows", nx.FMT_Q8_0, 4096, 14336, 512),
+    ("7B gate|up, Q4_K, 32 rows", nx.FMT_Q4_K, 22016, 4096, 32),
+    ("7B down, Q6_K, 32 rows", nx.FMT_Q6_K, 4096, 11008, 32),
+    ("7B gate|up, Q6_K, 256 rows", nx.FMT_Q6_K, 22016, 4096, 256),
+    ("7B down, Q6_K, 256 rows", nx.FMT_Q6_K, 4096, 11008, 256),
+])
+def test_packed_projections_at_the_configs_shapes(be, what, fmt, n, k, m):
+    from oracle import quantize as qz
+    rng = np.random.default_rng(n + k + m + fmt)
+    if fmt in (nx.FMT_Q4_0, nx.FMT_Q8_0):
+        w = _random_blocks(rng, fmt, n, k, 0.02 / (4 if fmt == nx.FMT_Q4_0 else 64))
+    else:
+        w = qz.random_quant(fmt, rng, n, k)
+    a = (rng.standard_normal((m, k)) * (1.0 + 3.0 * (rng.random((1, k)) < 0.1))).astype(np.float32)
+    da, dw = be.upload(a, permanent=True), be.upload(w, permanent=True)
+    qw = be.qweight(fmt, dw, n, k)
+    assert be.qweight_pack(qw)
+    dout = be.alloc_permanent(m * n * 4)
+    be.matmul_quant(fmt, da, dw, dout, None, m, n, k)
+    kernel = be.last_matmul_kernel()
+    assert kernel == ("qtiles_kernel" if m > 64 else "qstream_kernel"), kernel
+    got = be.download(dout, (m, n), np.float32)
+    assert np.all(np.isfinite(got))
+    rows = np.unique(np.concatenate([rng.integers(0, n, 45), [0, 15, 16, n - 17, n - 1]]))
+    mrows = np.unique(np.concatenate([rng.integers(0, m, 12), [0, m - 1]]))  # (the oracle's rows are independent)
+    want = nx.matmul_quant(fmt, a[mrows], w[rows], len(mrows), len(rows), k)
+    _close(got[np.ix_(mrows, rows)], want, 2e-5, 3e-6 * np.abs(want).max() + 1e-7, what)
+    for p_ in (da, dw, dout):
+        be.free(p_)
+    be.reset_pool()
+
+
 def test_paged_attention_at_full_context_and_head_geometry(be):
     """7B geometry (32 x 128 heads, MHA) with contexts at the configs' upper clip (4096), one short of it, a
     multiple of the 512-token split and the lower clip; 8B geometry (32 / 8 heads) likewise. Whole heads of
