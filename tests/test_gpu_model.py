@@ -995,6 +995,12 @@ def _gguf_from_oracle(omodel, arch, extra_md=()):
             tensors += [f32(b + "attn_norm.bias", lw.attn_norm_bias), f32(b + "attn_output.bias", lw.wo_bias),
                         f32(b + "ffn_up.bias", lw.w1_bias), f32(b + "ffn_down.bias", lw.w2_bias)]
             tensors.append(mat(b + "ffn_up.weight", lw.w1))
+        elif arch == "phi3":   # fused attn_qkv (no bias) and the gate+up matrix as ffn_up, gate rows first
+            fused = np.concatenate([lw.wq.data, lw.wk.data, lw.wv.data], axis=0)
+            tensors.append((b + "attn_qkv.weight", [lw.wq.k, lw.wq.n + 2 * lw.wk.n], GGUF_TYPE[lw.wq.fmt], fused.tobytes()))
+            both = np.concatenate([lw.w1.data, lw.w3.data], axis=0)
+            tensors.append((b + "ffn_up.weight", [lw.w1.k, 2 * lw.w1.n], GGUF_TYPE[lw.w1.fmt], both.tobytes()))
+            tensors.append(f32(b + "ffn_norm.weight", lw.ffn_norm))
         else:
             tensors += [mat(b + "attn_q.weight", lw.wq), mat(b + "attn_k.weight", lw.wk), mat(b + "attn_v.weight", lw.wv),
                         mat(b + "ffn_gate.weight", lw.w1), mat(b + "ffn_up.weight", lw.w3),
@@ -1020,16 +1026,17 @@ def _gguf_from_oracle(omodel, arch, extra_md=()):
     return og.build(md, tensors)
 
 
-@pytest.mark.parametrize("arch", ["phi2", "gemma2", "qwen2"])
+@pytest.mark.parametrize("arch", ["phi2", "gemma2", "qwen2", "phi3"])
 def test_load_gguf_other_architectures(be, tmp_path, arch):
     """general.architecture selects the switches as ModelConfigFromGGUF does (runtime/config.go:388-470) and the
     loader finds each architecture's tensors (runtime/loader.go:290-385): the loaded model gives the oracle's logits
-    and greedy tokens. Gemma 2 takes interleaved RoPE pairs here, as the reference's table has it."""
+    and greedy tokens. Gemma 2 takes interleaved RoPE pairs here, as the reference's table has it. Phi-3: the fused
+    attn_qkv matrix and the gate+up matrix (gate rows first, loader.go:1147-1218) are used in place as row ranges."""
     import copy, os
     from oracle import gguf as og
     from vexel_amd.backend import VexelError
     from vexel_amd.runtime import ModelRuntime
-    cfg = _arch_config({"phi2": "phi", "gemma2": "gemma", "qwen2": "qwen"}[arch])
+    cfg = _arch_config({"phi2": "phi", "gemma2": "gemma", "qwen2": "qwen", "phi3": "qwen"}[arch])  # (Phi-3: Qwen 2's layer without biases)
     extra = []
     if arch == "gemma2":
         cfg.rope_neox, cfg.final_softcap = False, 30.0

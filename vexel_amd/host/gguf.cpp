@@ -561,7 +561,7 @@ extern "C" int vh_model_load_gguf(vx_backend *be, const char *path, const vh_loa
     const std::string archname = gc.architecture;
     vh_arch a;
     memset(&a, 0, sizeof a);
-    bool qkv_bias = false, all_bias = false, fused_qkv = false;
+    bool qkv_bias = false, all_bias = false, fused_qkv = false, fused_gate_up = false;
     if (archname.empty() || archname == "llama" || archname == "mistral") {
     } else if (archname == "qwen2") {
         qkv_bias = true;
@@ -580,8 +580,12 @@ extern "C" int vh_model_load_gguf(vx_backend *be, const char *path, const vh_loa
         a.parallel_residual = 1;
         a.rope_neox = 1;
         all_bias = fused_qkv = true;
+    } else if (archname == "phi3") {
+        // config.go:419-424: RMSNorm, SwiGLU over a pre-fused gate+up tensor, serial residual, split RoPE pairs
+        a.rope_neox = 1;
+        fused_qkv = fused_gate_up = true;
     } else {
-        return done(gfail("%s: architecture '%s' has no loader here (llama, mistral, qwen2, gemma, gemma2, phi, phi2 do)", path,
+        return done(gfail("%s: architecture '%s' has no loader here (llama, mistral, qwen2, gemma, gemma2, phi, phi2, phi3 do)", path,
                           archname.c_str()));
     }
     if (gc.rope_dim_count < 0 || gc.rope_dim_count > c.head_dim || gc.rope_dim_count % 2 != 0)
@@ -628,6 +632,21 @@ extern "C" int vh_model_load_gguf(vx_backend *be, const char *path, const vh_loa
         }
         if (!rc && a.mlp_type == VH_MLP_GELU) {  // fc1 = ffn_up, fc2 = ffn_down (pkg/gguf/loader.go:190-198)
             rc = L.matrix(b + "ffn_up.weight", c.ffn, c.hidden, &w.w1);
+        } else if (!rc && fused_gate_up) {
+            // Phi-3's gate+up matrix [2 ffn rows, hidden], gate rows first: W1 and W3 are its halves, in place
+            // (splitGateUpWeight, loader.go:1147-1218, which the reference reaches under the tensor's safetensors
+            // name mlp.gate_up_proj; GGUF files of the architecture carry it as ffn_up)
+            vh_qweight both;
+            memset(&both, 0, sizeof both);
+            rc = L.matrix(b + "ffn_up.weight", 2 * c.ffn, c.hidden, &both);
+            if (!rc) {
+                vh_gguf_tensor t;
+                L.find(b + "ffn_up.weight", &t);
+                const size_t row_bytes = (size_t)t.n_bytes / (size_t)(2 * c.ffn);
+                const uint8_t *base = (const uint8_t *)both.data;
+                w.w1 = vh_qweight{both.fmt, base, c.ffn, c.hidden};
+                w.w3 = vh_qweight{both.fmt, base + (size_t)c.ffn * row_bytes, c.ffn, c.hidden};
+            }
         } else if (!rc) {
             rc = L.matrix(b + "ffn_gate.weight", c.ffn, c.hidden, &w.w1) || L.matrix(b + "ffn_up.weight", c.ffn, c.hidden, &w.w3);
         }
