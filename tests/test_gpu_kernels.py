@@ -373,6 +373,17 @@ def test_prepared_activation_paths(be):
         be.matmul_quant_prepared(nx.FMT_Q4_0, dw2, do, None, 3, 48, kk)
         want = nx.matmul_q4_0(act, w2, 3, 48, kk)
         _close(be.download(do, (3, 48), np.float32), want, 3e-5, 3e-6 * np.abs(want).max(), "silu_mul_prepare + matmul")
+        # the GeGLU form of the same launch: the bits of the separate GELU * up kernel
+        be.gelu_mul_prepare(dg, du, dact, 3, kk)
+        act = nx.gelu_mul(g, u)
+        got_act = be.download(dact, (3, kk), np.float32)
+        _close(got_act, act, 1e-6, 1e-9, "gelu_mul_prepare f32 output")
+        dsep = be.alloc(3 * kk * 4)
+        be.gelu_mul(dg, du, dsep, 3 * kk)
+        assert np.array_equal(got_act.view(np.uint32), be.download(dsep, (3, kk), np.float32).view(np.uint32))
+        be.matmul_quant_prepared(nx.FMT_Q4_0, dw2, do, None, 3, 48, kk)
+        want = nx.matmul_q4_0(act, w2, 3, 48, kk)
+        _close(be.download(do, (3, 48), np.float32), want, 3e-5, 3e-6 * np.abs(want).max(), "gelu_mul_prepare + matmul")
     # shape mismatch is an error, not a wrong answer
     from vexel_amd.backend import VexelError
     with pytest.raises(VexelError):

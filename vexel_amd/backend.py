@@ -276,6 +276,9 @@ class HipBackend:
     def silu_mul_prepare(self, gate, up, out, rows, cols):
         self.call("vx_silu_mul_prepare", gate, up, out, rows, cols)
 
+    def gelu_mul_prepare(self, gate, up, out, rows, cols):
+        self.call("vx_gelu_mul_prepare", gate, up, out, rows, cols)
+
     def matmul_quant_prepared(self, fmt, b, out, residual, m, n, k):
         self.call("vx_matmul_quant_prepared", fmt, b, out, residual, m, n, k)
 

@@ -137,6 +137,7 @@ struct vh_model {
     float *zeros = nullptr;               // [hidden] zeros: the bias of a LayerNorm whose bias tensor is absent
     bool general = false;                 // some switch or extra tensor is set: the one-call-per-operation sequence
     bool fused_ok = true;                 // the layer differs from LLaMA's at most by Q/K/V biases and the RoPE form
+    bool attn_fused_ok = true;            // the attention half does (RMSNorm without a bias in front of Q|K|V): its fused block serves it
                                           // (Qwen 2): decode may still take the fused entry points
 
     vx_graph *graph = nullptr;
@@ -295,22 +296,36 @@ int g_tail(vh_model *m, int layer, float *x, float *norm, const float *attn, flo
     float *o = a.parallel_residual ? up : norm;                                        // :972-978
     VHC(g_mm(m, attn, w.wo, e.wo_bias, o, rows));                                      // :981-983
     if (a.post_norms && e.post_attn_norm) VXC(vx_rmsnorm(be, o, e.post_attn_norm, o, rows, c.hidden, c.eps));  // :985-987
+    bool gated_prepared = false;  // RMSNorm in front of a gated MLP: one launch normalises and prepares W1's and W3's operand
     if (!a.parallel_residual) {
         VXC(vx_add(be, x, o, x, rows * c.hidden));                                     // :989-991
-        if (w.ffn_norm) VHC(g_norm(m, x, w.ffn_norm, e.ffn_norm_bias, norm, rows));    // :996-998
+        if (w.ffn_norm && a.norm_type != VH_NORM_LAYER && a.mlp_type != VH_MLP_GELU) {
+            const vh_qweight *w13[2] = {&w.w1, &w.w3};
+            VHC(norm_for(m, x, w.ffn_norm, norm, rows, w13, 2, &gated_prepared));      // :996-998
+        } else if (w.ffn_norm) {
+            VHC(g_norm(m, x, w.ffn_norm, e.ffn_norm_bias, norm, rows));                // :996-998
+        }
     }
     if (a.mlp_type == VH_MLP_GELU) {                                                   // :1004-1037
         VHC(g_mm(m, norm, w.w1, e.w1_bias, gate, rows));
         VXC(vx_gelu(be, gate, gate, rows * c.ffn));
         VHC(g_mm(m, gate, w.w2, e.w2_bias, norm, rows));
     } else {                                                                           // :1040-1062
-        VHC(mm(m, false, norm, w.w1, gate, nullptr, rows));
-        VHC(mm(m, false, norm, w.w3, up, nullptr, rows));
-        if (a.mlp_type == VH_MLP_GEGLU)
-            VXC(vx_gelu_mul(be, gate, up, gate, rows * c.ffn));
-        else
-            VXC(vx_silu_mul(be, gate, up, gate, rows * c.ffn));
-        VHC(mm(m, false, gate, w.w2, norm, nullptr, rows));
+        VHC(mm(m, gated_prepared, norm, w.w1, gate, nullptr, rows));
+        VHC(mm(m, gated_prepared, norm, w.w3, up, nullptr, rows));
+        if (rows > 1 && fast(w.w2) && c.ffn % 256 == 0) {   // the activation leaves its kernel as W2's prepared operand
+            if (a.mlp_type == VH_MLP_GEGLU)
+                VXC(vx_gelu_mul_prepare(be, gate, up, nullptr, rows, c.ffn));
+            else
+                VXC(vx_silu_mul_prepare(be, gate, up, nullptr, rows, c.ffn));
+            VHC(mm(m, true, nullptr, w.w2, norm, nullptr, rows));
+        } else {
+            if (a.mlp_type == VH_MLP_GEGLU)
+                VXC(vx_gelu_mul(be, gate, up, gate, rows * c.ffn));
+            else
+                VXC(vx_silu_mul(be, gate, up, gate, rows * c.ffn));
+            VHC(mm(m, false, gate, w.w2, norm, nullptr, rows));
+        }
     }
     if (a.post_norms && e.post_ffn_norm) VXC(vx_rmsnorm(be, norm, e.post_ffn_norm, norm, rows, c.hidden, c.eps));  // :1066-1069
     if (a.parallel_residual) VXC(vx_add(be, x, o, x, rows * c.hidden));                // :1072-1075
@@ -325,7 +340,7 @@ int g_scale_embedding(vh_model *m, float *x, int rows) {
 }
 
 bool attn_fusable(const vh_model *m, int layer) {
-    if (!m->fused || (m->general && !m->fused_ok) || layer >= m->cfg.num_layers) return false;
+    if (!m->fused || (m->general && !m->attn_fused_ok) || layer >= m->cfg.num_layers) return false;
     const vh_layer_weights &w = m->layers[layer];
     return w.wq.data && w.wk.data && w.wv.data && vx_decode_attn_qkv_supported(&w.wq, &w.wk, &w.wv, m->cfg.head_dim) != 0;
 }
@@ -365,7 +380,9 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
         VXC(vx_rope_store_paged(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
                                 c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta));  // :858, :868
     }
-    const bool ffn_fused = m->fused && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
+    // (a layer whose second half is not LLaMA's - post-norms, GeGLU: Gemma - keeps the general sequence there)
+    const bool tail_general = m->general && !m->fused_ok;
+    const bool ffn_fused = !tail_general && m->fused && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
                            vx_decode_ffn_supported(&w.wo, &w.w1, &w.w3, &w.w2);
     // the fused tail can merge the attention's split-KV partials itself
     const bool split = ffn_fused && (size_t)w.wo.k * 4 <= 64 * 1024 && c.head_dim % 4 == 0 &&
@@ -380,6 +397,7 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
         *chained = next_norm != nullptr;
         return VH_OK;
     }
+    if (tail_general) return g_tail(m, layer, m->x, m->norm, m->attn, m->gate, m->up, rows);
     return layer_tail(m, w, m->x, m->norm, m->attn, m->gate, m->up, rows);
 }
 
@@ -580,9 +598,12 @@ static void refresh_general(vh_model *m) {
     for (const vh_layer_extras &e : m->extras)
         f = f && !e.attn_norm_bias && !e.ffn_norm_bias && !e.wo_bias && !e.w1_bias && !e.w2_bias && !e.post_attn_norm &&
             !e.post_ffn_norm;
-    if (g != m->general || f != m->fused_ok) drop_graph(m);
+    bool af = !a.norm_type;
+    for (const vh_layer_extras &e : m->extras) af = af && !e.attn_norm_bias;
+    if (g != m->general || f != m->fused_ok || af != m->attn_fused_ok) drop_graph(m);
     m->general = g;
     m->fused_ok = f;
+    m->attn_fused_ok = af;
 }
 
 int vh_model_set_architecture(vh_model *m, const vh_arch *arch) {
