@@ -34,7 +34,7 @@ BLOCK = 16
 
 # HBM bytes per algorithmic byte of the attention launch, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs
 # scaled by a plain copy of known size (summary: profiles/paged_decode_attention_7b_x32_hbm_traffic.txt).
-ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.013
+ATTN_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.012
 # the same for the step's four projection launches per layer at 32 rows
 # (summary: profiles/decode_gemm_7b_q4_0_x32_issue_and_traffic_counters.txt)
 GEMM_TRAFFIC_PER_ALGORITHMIC_BYTE = 1.23
