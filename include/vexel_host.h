@@ -77,8 +77,10 @@ void vh_model_get_config(const vh_model *m, vh_config *out);  /* the configurati
 void vh_model_set_fused(vh_model *m, int on);
 int vh_model_set_layer(vh_model *m, int layer, const vh_layer_weights *w);
 /* A model with any switch or extra tensor set runs ExecuteWithPagedKV's general sequence, one backend call per
- * operation (block.go:834-1077), in vh_prefill, vh_decode_batched, vh_decode_graph and the scheduler; the fused
- * decode entry points and vh_verify_tree are for the LLaMA arm. With the GELU MLP a layer's w3 may be empty.
+ * operation (block.go:834-1077), in vh_prefill, vh_decode_batched, vh_decode_graph, vh_verify_tree and the scheduler,
+ * except where a half of the layer is LLaMA's up to Q/K/V biases and the RoPE form: an RMSNorm in front of Q|K|V
+ * without a bias lets the fused attention block serve the first half, and a second half without post-norms, biases,
+ * GELU / GeGLU or a parallel residual takes the fused FFN block. With the GELU MLP a layer's w3 may be empty.
  * All pointers are float32 device vectors that outlive the model's use of them. */
 int vh_model_set_architecture(vh_model *m, const vh_arch *arch);
 void vh_model_get_architecture(const vh_model *m, vh_arch *out);

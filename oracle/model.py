@@ -163,6 +163,12 @@ class OracleModel:
         else:                                                                  # :893-895 dense causal on F32 K/V
             attn = nx.sdpa_prefill(q, k, v, seq_len, c.num_heads, c.num_kv_heads, c.head_dim,
                                    scale).reshape(seq_len, -1)
+        return self._tail(x, norm, attn, lw, seq_len)
+
+    def _tail(self, x, norm, attn, lw, seq_len):
+        """block.go:981-1077: output projection, post-norm, residual(s), FFN norm, MLP. `norm` is the attention
+        norm's output (what the parallel residual's MLP reads)."""
+        c = self.cfg
         o = _mm_bias(attn, lw.wo, lw.wo_bias, seq_len)                         # :981-983
         if c.post_norms and lw.post_attn_norm is not None:                     # :985-987
             o = nx.rmsnorm(o, lw.post_attn_norm, seq_len, c.hidden, c.eps)
@@ -235,15 +241,17 @@ class OracleModel:
     def _execute_tree_layer(self, x, seq_id, layer_idx, start_pos, positions, mask):
         """block.go:763-1081 for the rows [input token, candidate nodes]: row r is stored at pool position
         start_pos + r, rotated at positions[r] (start_pos + its depth in the tree) and attends to every earlier
-        pool position and to the rows the mask names (tree.go:186-202)."""
+        pool position and to the rows the mask names (tree.go:186-202). The architecture's switches act as in
+        execute_with_paged_kv's multi-query arm (a chunk behind a context: no soft cap on the scores)."""
         c = self.cfg
         lw = self.layers[layer_idx]
         rows = x.shape[0]
-        norm = nx.rmsnorm(x, lw.attn_norm, rows, c.hidden, c.eps)
-        q = _mm(norm, lw.wq, rows)
-        k = _mm(norm, lw.wk, rows)
-        v = _mm(norm, lw.wv, rows)
-        q, k = nx.rope_positions(q, k, c.head_dim, c.num_heads, c.num_kv_heads, positions, 0, c.rope_theta, False)
+        norm = self._norm(x, lw.attn_norm, lw.attn_norm_bias, rows)
+        q = _mm_bias(norm, lw.wq, lw.wq_bias, rows)
+        k = _mm_bias(norm, lw.wk, lw.wk_bias, rows)
+        v = _mm_bias(norm, lw.wv, lw.wv_bias, rows)
+        q, k = nx.rope_positions(q, k, c.head_dim, c.num_heads, c.num_kv_heads, positions, c.rope_dim, c.rope_theta,
+                                 c.rope_neox)
         scale = np.float32(1.0 / math.sqrt(float(c.head_dim)))
         slots = self.pool.store_kv_slots(layer_idx, seq_id, start_pos, rows)
         bi = [s[0] for s in slots]
@@ -253,11 +261,7 @@ class OracleModel:
         bt = self.pool.seqs[seq_id].block_tables[layer_idx]
         attn = nx.sdpa_paged_multiquery(q, self.kv[layer_idx], bt, None, c.block_size, c.num_heads, c.num_kv_heads,
                                         c.head_dim, scale, tree_mask=mask, tree_base=start_pos).reshape(rows, -1)
-        o = _mm(attn, lw.wo, rows)
-        x = nx.add(x, o)
-        norm = nx.rmsnorm(x, lw.ffn_norm, rows, c.hidden, c.eps)
-        act = nx.silu_mul(_mm(norm, lw.w1, rows), _mm(norm, lw.w3, rows))
-        return nx.add(x, _mm(act, lw.w2, rows))
+        return self._tail(x, norm, attn, lw, rows)
 
     def verify_tree(self, input_token, node_tokens, parent_idx, seq_id, start_pos):
         """Logits [1 + nodes, vocab] of one pass over the input token and a candidate tree given as
@@ -267,7 +271,6 @@ class OracleModel:
         start_pos .. start_pos + nodes."""
         from .host_logic import build_tree_attention_mask, tree_depths
         c = self.cfg
-        assert is_llama(c), "tree verification is restated for the LLaMA arm only"
         self._ensure_seq(seq_id)
         n = len(node_tokens)
         rows = n + 1
@@ -275,7 +278,7 @@ class OracleModel:
         parents = [-1] + [p + 1 for p in parent_idx]
         mask = np.array(build_tree_attention_mask(rows, parents), dtype=np.uint8).reshape(rows, rows)
         positions = [start_pos + d for d in tree_depths(parents)]
-        x = nx.embedding([input_token] + list(node_tokens), self.embedding, c.vocab, c.hidden)
+        x = self._embed([input_token] + list(node_tokens))
         for i in range(c.num_layers):
             x = self._execute_tree_layer(x, seq_id, i, start_pos, positions, mask)
         return self._head(x, rows)

@@ -863,7 +863,8 @@ def _arch_config(name):
 @pytest.mark.parametrize("name", ["phi", "gemma", "qwen", "qwen_g7"])
 def test_other_architectures_prefill_decode_graph(be, name):
     """ExecuteWithPagedKV's general sequence (block.go:834-1077) through vh_prefill (first chunk and a later one),
-    vh_decode_batched and the device-driven vh_decode_graph, against the oracle's layer for the same switches."""
+    vh_decode_batched, the device-driven vh_decode_graph and vh_verify_tree, against the oracle's layer for the same
+    switches."""
     cfg = _arch_config(name)
     omodel = om.random_model(cfg, 21, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=24)
     if name.startswith("qwen"):
@@ -904,8 +905,38 @@ def test_other_architectures_prefill_decode_graph(be, name):
         assert out[step].tolist() == cur, "graph step %d" % step
     assert mr.block_table(1) == omodel.pool.seqs[1].block_tables[0]
     assert mr.device_matches_host()
-    with pytest.raises(RuntimeError, match="LLaMA arm only"):
-        mr.verify_tree([1], [cur[0]], [pos[0]], [([5, 6], [-1, 0])])
+    # tree verification under the same switches: a 10-node tree per sequence, sequence 1's own greedy continuation
+    # planted two levels deep, acceptance and rollback against the oracle's pass, then a decode step on the result
+    import copy
+    from oracle import host_logic as hl
+    rng = np.random.default_rng(24)
+    probe, tok, plant = copy.deepcopy(omodel), cur[0], []
+    for d in range(2):
+        tok = nx.argmax(probe.decode_with_paged_kv(tok, 1, pos[0] + d))
+        plant.append(tok)
+    trees = []
+    for i in range(2):
+        tk = [rng.choice(cfg.vocab, 2, replace=False).tolist() for _ in range(4)]
+        if i == 0:
+            for h, t in enumerate(plant):
+                tk[h][(h + 1) % 2] = t
+                if tk[h][0] == tk[h][1]:
+                    tk[h][h % 2] = (t + 1) % cfg.vocab
+        trees.append(hl.build_candidate_tree_from_topk(tk, [[2.0, 1.0]] * 4, 10).linearize())
+    want = omodel.tree_step_batched(cur, trees, ids, pos)
+    acc, fin, logits = mr.verify_tree(ids, cur, pos, trees)
+    for i, sid in enumerate(ids):
+        worst = max(worst, assert_logits_close(logits[i], want[i][2], "%s tree rows of sequence %d" % (name, sid)))
+        assert acc[i] == want[i][0] and fin[i] == want[i][1]
+        assert mr.seq_len(sid) == omodel.pool.seqs[sid].seq_len == pos[i] + 1 + len(acc[i])
+        assert mr.block_table(sid) == omodel.pool.seqs[sid].block_tables[0]
+    assert len(acc[0]) >= 2
+    cur, pos = list(fin), [pos[i] + 1 + len(acc[i]) for i in range(2)]
+    want = omodel.decode_batched(cur, ids, pos)
+    got, am = mr.decode_with_paged_kv_batched(cur, ids, pos)
+    worst = max(worst, assert_logits_close(got, want, "%s decode after the rollback" % name))
+    assert [nx.argmax(w) for w in want] == [int(a) for a in am]
+    assert mr.device_matches_host()
     print("%s: worst logit error %.3e" % (name, worst))
     mr.close()
 

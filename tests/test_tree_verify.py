@@ -109,3 +109,40 @@ def test_tree_step_with_nothing_accepted_keeps_only_the_input_token():
     want = copy.deepcopy(base)
     want.prefill_with_paged_kv([9], 7, 21)
     assert m.pool.seqs[7].block_tables == want.pool.seqs[7].block_tables
+
+
+def _arch_cfg(name):
+    import math
+    if name == "phi":     # LayerNorm, biases, partial split-pair RoPE, GELU MLP, parallel residual
+        return om.ModelConfig(num_layers=2, hidden=256, num_heads=4, num_kv_heads=4, head_dim=64, ffn=512, vocab=512,
+                              norm_type="layer", mlp_type="gelu", parallel_residual=True, rope_dim=32, rope_neox=True)
+    if name == "gemma":   # scaled embeddings, GeGLU, post-norms, soft-capped first chunk
+        return om.ModelConfig(num_layers=2, hidden=256, num_heads=4, num_kv_heads=2, head_dim=64, ffn=512, vocab=512,
+                              eps=1e-6, mlp_type="geglu", post_norms=True, attn_softcap=50.0,
+                              embedding_scale=float(np.float32(math.sqrt(256.0))))
+    return om.ModelConfig(num_layers=2, hidden=256, num_heads=4, num_kv_heads=2, head_dim=64, ffn=512, vocab=512,
+                          eps=1e-6, rope_neox=True, rope_theta=1000000.0)   # Qwen 2: split pairs, Q/K/V biases below
+
+
+def test_every_path_sees_its_linear_verification_in_the_other_architectures():
+    """The same property under ExecuteWithPagedKV's switches (block.go:834-1077): the tree pass takes the layer's
+    multi-query arm row by row, so each path must still equal the linear verification bit for bit."""
+    for name in ("phi", "gemma", "qwen"):
+        cfg = _arch_cfg(name)
+        m = om.random_model(cfg, 15, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=16)
+        rng = np.random.default_rng(16)
+        if name == "qwen":
+            for lw in m.layers:
+                lw.wq_bias = (0.05 * rng.standard_normal(256)).astype(np.float32)
+                lw.wk_bias = (0.05 * rng.standard_normal(128)).astype(np.float32)
+                lw.wv_bias = (0.05 * rng.standard_normal(128)).astype(np.float32)
+        m.prefill_with_paged_kv(rng.integers(0, cfg.vocab, 21).tolist(), 7, 0)
+        base = copy.deepcopy(m)
+        tokens, parent = _tree(rng, max_nodes=10)
+        logits = m.verify_tree(9, tokens, parent, 7, 21)
+        leaves = [i for i in range(len(tokens)) if i not in parent]
+        for leaf in leaves:
+            path = _path(parent, leaf)
+            lin = copy.deepcopy(base).verify_with_paged_kv([9] + [tokens[i] for i in path], 7, 21)
+            for j, row in enumerate([0] + [i + 1 for i in path]):
+                assert np.array_equal(logits[row].view(np.uint32), lin[j].view(np.uint32)), (name, leaf, j)

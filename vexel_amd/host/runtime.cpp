@@ -1127,7 +1127,6 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
 int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_t *input_tokens, const int32_t *start_pos,
                    const int32_t *n_nodes, const int32_t *node_tokens, const int32_t *parent_idx, int32_t *num_accepted,
                    int32_t *accepted_nodes, int32_t *final_tokens, float *logits_out) {
-    if (m && m->general) return fail("vh_verify_tree: the LLaMA arm only");
     if (!m || n_seqs < 0 || !seq_ids || !input_tokens || !start_pos || !n_nodes || !num_accepted || !final_tokens)
         return fail("bad arguments");
     if (n_seqs == 0) return VH_OK;
@@ -1258,16 +1257,25 @@ int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_
         VXC(vx_to_device(be, d_moff, moff.data(), (size_t)n * 4));
     }
     VXC(vx_embedding(be, d_tok, n, m->embedding, x, c.vocab, c.hidden));
+    VHC(g_scale_embedding(m, x, n));
     const float scale = (float)(1.0 / sqrt((double)c.head_dim));
     // the layers as in forward_decode: fused projection groups where the weights allow them, each fused tail
-    // leaving the next norm's activation prepared
-    const bool head_prepared = n > 1 && m->fused && fast(m->lm_head) && c.hidden % 256 == 0;
+    // leaving the next norm's activation prepared; the other architectures' switches as in execute_layer_decode
+    const bool tail_general = m->general && !m->fused_ok;
+    const bool head_prepared = n > 1 && m->fused && !tail_general && fast(m->lm_head) && c.hidden % 256 == 0;
     bool chained = false;
     for (int l = 0; l < c.num_layers; l++) {
         const vh_layer_weights &w = m->layers[l];
         if (attn_fusable(m, l)) {
-            VXC(vx_decode_attn_qkv(be, x, w.attn_norm, c.eps, chained ? 1 : 0, &w.wq, &w.wk, &w.wv, n, d_pos, d_slot, m->kv[l],
-                                   c.kv_fp16, c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta, q));
+            const vh_layer_extras &e = m->extras[l];
+            VXC(vx_decode_attn_qkv_ex(be, x, w.attn_norm, c.eps, chained ? 1 : 0, &w.wq, &w.wk, &w.wv, e.wq_bias, e.wk_bias,
+                                      e.wv_bias, n, d_pos, d_slot, m->kv[l], c.kv_fp16, c.num_heads, c.num_kv_heads, c.head_dim,
+                                      c.block_size, c.rope_theta, m->arch.rope_dim, m->arch.rope_neox, q));
+        } else if (m->general) {
+            if (chained) return fail("internal: prepared activation handed to a general layer");
+            VHC(g_qkv(m, l, x, norm, q, k, v, n));
+            VXC(vx_rope_store_paged_ex(be, q, k, v, d_pos, d_slot, m->kv[l], c.kv_fp16, n, c.num_heads, c.num_kv_heads,
+                                       c.head_dim, c.block_size, c.rope_theta, m->arch.rope_dim, m->arch.rope_neox));
         } else {
             if (chained) return fail("internal: prepared activation handed to an unfused layer");
             bool prep;
@@ -1293,6 +1301,10 @@ int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_
             }
         }
         chained = false;
+        if (tail_general) {
+            VHC(g_tail(m, l, x, norm, attn, gate, up, n));
+            continue;
+        }
         const bool ffn_fused = m->fused && n > 1 && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
                                vx_decode_ffn_supported(&w.wo, &w.w1, &w.w3, &w.w2);
         if (ffn_fused) {
@@ -1306,6 +1318,9 @@ int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_
     }
     if (chained) {
         VHC(mm(m, true, nullptr, m->lm_head, logits, nullptr, n));
+    } else if (tail_general) {                                                            // model.go:207-226
+        VHC(g_norm(m, x, m->final_norm, m->final_norm_bias, norm, n));
+        VHC(mm(m, false, norm, m->lm_head, logits, nullptr, n));
     } else {
         bool prep;
         const vh_qweight *hw[1] = {&m->lm_head};
