@@ -204,6 +204,7 @@ int vx_matmul_quant(vx_backend *be, int fmt, const float *a, const void *b, floa
  *   vx_rmsnorm_prepare   Backend.RMSNorm(x, weight) (backend.go:345); also stored to out when out != NULL
  *   vx_silu_mul_prepare  Backend.SiLUMul(gate, up) (backend.go:360); also stored to out when out != NULL
  *   vx_gelu_mul_prepare  GELUMul(gate, up) (backend.go:222-224; GeGLU layers); also stored to out when out != NULL
+ *   vx_gelu_prepare      GELU(x) (backend.go:216-220; the GELU MLP's fc1 output); also stored to out when out != NULL
  * vx_matmul_quant_prepared with out == NULL (and residual == NULL) issues the projection's launch alone, as the
  * fused decode blocks do: the sums of its K slices stay in a backend workspace that only the library reads. That
  * form exists to time the launch by itself; it returns nothing to the caller. */
@@ -211,6 +212,7 @@ int vx_prepare_act(vx_backend *be, const float *a, int m, int k);
 int vx_rmsnorm_prepare(vx_backend *be, const float *x, const float *weight, float *out, int rows, int cols, float eps);
 int vx_silu_mul_prepare(vx_backend *be, const float *gate, const float *up, float *out, int rows, int cols);
 int vx_gelu_mul_prepare(vx_backend *be, const float *gate, const float *up, float *out, int rows, int cols);
+int vx_gelu_prepare(vx_backend *be, const float *x, float *out, int rows, int cols);
 int vx_matmul_quant_prepared(vx_backend *be, int fmt, const void *b, float *out, const float *residual, int m,
                              int n, int k);
 /* 1 when the [n,k] matrix can take the prepared MFMA path: k % 256 == 0, a 16-byte aligned pointer, and rows

@@ -384,6 +384,15 @@ def test_prepared_activation_paths(be):
         be.matmul_quant_prepared(nx.FMT_Q4_0, dw2, do, None, 3, 48, kk)
         want = nx.matmul_q4_0(act, w2, 3, 48, kk)
         _close(be.download(do, (3, 48), np.float32), want, 3e-5, 3e-6 * np.abs(want).max(), "gelu_mul_prepare + matmul")
+        # GELU alone (the GELU MLP's fc1 output as fc2's operand): the bits of vx_gelu
+        be.gelu_prepare(dg, dact, 3, kk)
+        got_act = be.download(dact, (3, kk), np.float32)
+        be.gelu(dg, dsep, 3 * kk)
+        assert np.array_equal(got_act.view(np.uint32), be.download(dsep, (3, kk), np.float32).view(np.uint32))
+        _close(got_act, nx.gelu(g), 1e-6, 1e-9, "gelu_prepare f32 output")
+        be.matmul_quant_prepared(nx.FMT_Q4_0, dw2, do, None, 3, 48, kk)
+        want = nx.matmul_q4_0(nx.gelu(g), w2, 3, 48, kk)
+        _close(be.download(do, (3, 48), np.float32), want, 3e-5, 3e-6 * np.abs(want).max(), "gelu_prepare + matmul")
     # shape mismatch is an error, not a wrong answer
     from vexel_amd.backend import VexelError
     with pytest.raises(VexelError):

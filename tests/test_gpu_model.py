@@ -866,7 +866,7 @@ def test_other_architectures_prefill_decode_graph(be, name):
     vh_decode_batched, the device-driven vh_decode_graph and vh_verify_tree, against the oracle's layer for the same
     switches."""
     cfg = _arch_config(name)
-    omodel = om.random_model(cfg, 21, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=24)
+    omodel = om.random_model(cfg, 21, nx.FMT_Q4_0, nx.FMT_Q8_0, max_blocks=40)
     if name.startswith("qwen"):
         rng = np.random.default_rng(22)
         qd, kvd = cfg.num_heads * cfg.head_dim, cfg.num_kv_heads * cfg.head_dim
@@ -874,8 +874,14 @@ def test_other_architectures_prefill_decode_graph(be, name):
             lw.wq_bias = (0.05 * rng.standard_normal(qd)).astype(np.float32)
             lw.wk_bias = (0.05 * rng.standard_normal(kvd)).astype(np.float32)
             lw.wv_bias = (0.05 * rng.standard_normal(kvd)).astype(np.float32)
-    mr = gpu_model_from_oracle(be, omodel, pool_blocks=24, max_seqs=4, max_batch=8)
+    mr = gpu_model_from_oracle(be, omodel, pool_blocks=40, max_seqs=4, max_batch=8)
     rng = np.random.default_rng(23)
+    # a chunk of 130 rows: the general sequence then takes its activation kernels that leave W2's prepared operand
+    long_prompt = rng.integers(0, cfg.vocab, 130).tolist()
+    assert_logits_close(mr.prefill_with_paged_kv(long_prompt, 3, 0), omodel.prefill_with_paged_kv(long_prompt, 3, 0),
+                        "%s 130-row chunk" % name)
+    mr.delete_sequence(3)
+    omodel.pool.delete_sequence(3)
     prompts = {1: rng.integers(0, cfg.vocab, 21).tolist(), 2: rng.integers(0, cfg.vocab, 35).tolist()}
     toks, worst = {}, 0.0
     for sid, p in prompts.items():

@@ -279,6 +279,9 @@ class HipBackend:
     def gelu_mul_prepare(self, gate, up, out, rows, cols):
         self.call("vx_gelu_mul_prepare", gate, up, out, rows, cols)
 
+    def gelu_prepare(self, x, out, rows, cols):
+        self.call("vx_gelu_prepare", x, out, rows, cols)
+
     def matmul_quant_prepared(self, fmt, b, out, residual, m, n, k):
         self.call("vx_matmul_quant_prepared", fmt, b, out, residual, m, n, k)
 

@@ -62,7 +62,7 @@ __device__ __forceinline__ float h2f(uint16_t h) {
 // ---------------------------------------------------------------- activation prepare
 // (PrepView, the workspace layout and write_chunk: prep_tiles.h)
 
-enum { PREP_PLAIN = 0, PREP_RMSNORM = 1, PREP_SILU_MUL = 2, PREP_GELU_MUL = 3 };
+enum { PREP_PLAIN = 0, PREP_RMSNORM = 1, PREP_SILU_MUL = 2, PREP_GELU_MUL = 3, PREP_GELU = 4 };
 
 __device__ __forceinline__ float sigmoid_ref(float v) { return 1.0f / (1.0f + (float)exp((double)(-v))); }
 // GELU, tanh form, with the reference's operation order (backend/cpu/cpu.go:440-473; the arithmetic of vx_gelu)
@@ -73,16 +73,19 @@ __device__ __forceinline__ float gelu_tanh_ref(float v) {
     const float th = (float)tanh((double)arg);
     return 0.5f * v * (1.0f + th);
 }
-// the gated activation of the two-operand modes: SiLU(a) * b or GELU(a) * b
+// the activation modes: SiLU(a) * b, GELU(a) * b, or GELU(a) alone (b unused)
 template <int MODE> __device__ __forceinline__ float gated(float a, float b) {
+    if (MODE == PREP_GELU) return gelu_tanh_ref(a);
     return MODE == PREP_GELU_MUL ? __fmul_rn(gelu_tanh_ref(a), b) : __fmul_rn(__fmul_rn(a, sigmoid_ref(a)), b);
 }
+template <int MODE> constexpr bool is_act_mode() { return MODE == PREP_SILU_MUL || MODE == PREP_GELU_MUL || MODE == PREP_GELU; }
 
 // grid = Mpad rows, block = 256.
 //   PREP_PLAIN:    y = a
 //   PREP_RMSNORM:  y = (a / rms) * w            (backend/cpu/cpu.go:200-220), optional f32 copy to `fout`
 //   PREP_SILU_MUL: y = (a*sigmoid(a)) * b       (backend/cpu/cpu.go:390-400), optional f32 copy to `fout`
 //   PREP_GELU_MUL: y = gelu(a) * b              (backend/cpu/cpu.go:462-473), optional f32 copy to `fout`
+//   PREP_GELU:     y = gelu(a)                  (backend/cpu/cpu.go:440-460), optional f32 copy to `fout`
 // STAGE: keep the row's output values in LDS between the two passes (K*4 bytes of dynamic LDS);
 // otherwise pass 2 recomputes them.
 constexpr int PREP_THREADS = 1024;  // shared by every kernel that writes prepared tiles: the row statistics
@@ -146,14 +149,14 @@ __global__ void __launch_bounds__(PREP_THREADS) prepare_kernel(const float *__re
         float y[4] = {x.x, x.y, x.z, x.w};
         if (MODE == PREP_RMSNORM) {
             ss = sumsq4(ss, x.x, x.y, x.z, x.w);
-        } else if (MODE == PREP_SILU_MUL || MODE == PREP_GELU_MUL) {
-            const float4 u = *(const float4 *)(br + k);
+        } else if (is_act_mode<MODE>()) {
+            const float4 u = MODE == PREP_GELU ? make_float4(0.f, 0.f, 0.f, 0.f) : *(const float4 *)(br + k);
             y[0] = gated<MODE>(x.x, u.x);
             y[1] = gated<MODE>(x.y, u.y);
             y[2] = gated<MODE>(x.z, u.z);
             y[3] = gated<MODE>(x.w, u.w);
         }
-        if (STAGE && (MODE == PREP_SILU_MUL || MODE == PREP_GELU_MUL)) *(float4 *)(ybuf + k) = make_float4(y[0], y[1], y[2], y[3]);
+        if (STAGE && is_act_mode<MODE>()) *(float4 *)(ybuf + k) = make_float4(y[0], y[1], y[2], y[3]);
         if (MODE == PREP_RMSNORM) {
             const float4 w = *(const float4 *)(br + k);
             y[0] *= w.x; y[1] *= w.y; y[2] *= w.z; y[3] *= w.w;
@@ -179,7 +182,7 @@ __global__ void __launch_bounds__(PREP_THREADS) prepare_kernel(const float *__re
     for (int p = tid; p < npairs; p += PREP_THREADS) {
         const int ks = p >> 2, g = p & 3;
         const int k0 = ks * 32 + 4 * g;
-        const float *src = (STAGE && (MODE == PREP_SILU_MUL || MODE == PREP_GELU_MUL)) ? ybuf : ar;
+        const float *src = (STAGE && is_act_mode<MODE>()) ? ybuf : ar;
         float4 xa = *(const float4 *)(src + k0), xb = *(const float4 *)(src + k0 + 16);
         float ya[4] = {xa.x, xa.y, xa.z, xa.w}, yb[4] = {xb.x, xb.y, xb.z, xb.w};
         if (MODE == PREP_RMSNORM) {
@@ -190,8 +193,9 @@ __global__ void __launch_bounds__(PREP_THREADS) prepare_kernel(const float *__re
                 ya[i] = __fmul_rn(ya[i] / rms, wv[i]);
                 yb[i] = __fmul_rn(yb[i] / rms, wv[4 + i]);
             }
-        } else if ((MODE == PREP_SILU_MUL || MODE == PREP_GELU_MUL) && !STAGE) {
-            const float4 ua = *(const float4 *)(br + k0), ub = *(const float4 *)(br + k0 + 16);
+        } else if (is_act_mode<MODE>() && !STAGE) {
+            const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 ua = MODE == PREP_GELU ? zero4 : *(const float4 *)(br + k0), ub = MODE == PREP_GELU ? zero4 : *(const float4 *)(br + k0 + 16);
             const float uv[8] = {ua.x, ua.y, ua.z, ua.w, ub.x, ub.y, ub.z, ub.w};
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -2078,6 +2082,22 @@ int vx_gelu_mul_prepare(vx_backend *be, const float *gate, const float *up, floa
                                                                                           pv, mpad);
     else
         prepare_kernel<PREP_GELU_MUL, false><<<mpad, PREP_THREADS, 0, be->stream>>>(gate, up, out, rows, cols, 0.f, pv, mpad);
+    VX_CHECK_LAUNCH();
+    return VX_OK;
+}
+
+int vx_gelu_prepare(vx_backend *be, const float *x, float *out, int rows, int cols) {
+    int rc = enter(be);
+    if (rc) return rc;
+    VX_REQUIRE(x && ((uintptr_t)x % 16 == 0) && ((uintptr_t)out % 16 == 0), "vx_gelu_prepare: null or unaligned pointer");
+    PrepView pv;
+    rc = prep_begin(be, rows, cols, &pv);
+    if (rc) return rc;
+    const int mpad = mpad_for(rows);
+    if ((size_t)cols * 4 <= 48 * 1024)
+        prepare_kernel<PREP_GELU, true><<<mpad, PREP_THREADS, (size_t)cols * 4, be->stream>>>(x, nullptr, out, rows, cols, 0.f, pv, mpad);
+    else
+        prepare_kernel<PREP_GELU, false><<<mpad, PREP_THREADS, 0, be->stream>>>(x, nullptr, out, rows, cols, 0.f, pv, mpad);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }

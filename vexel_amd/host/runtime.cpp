@@ -268,9 +268,9 @@ int g_norm(vh_model *m, const float *x, const float *w, const float *b, float *o
     return VH_OK;
 }
 
-// matMulTransposedWithBias (block.go:555-560)
-int g_mm(vh_model *m, const float *a, const vh_qweight &w, const float *bias, float *out, int rows) {
-    VHC(mm(m, false, a, w, out, nullptr, rows));
+// matMulTransposedWithBias (block.go:555-560); prepared: the activation is in the backend's prepared slot already
+int g_mm(vh_model *m, const float *a, const vh_qweight &w, const float *bias, float *out, int rows, bool prepared = false) {
+    VHC(mm(m, prepared, a, w, out, nullptr, rows));
     if (bias) VXC(vx_add_bias(m->be, out, bias, out, rows, w.n));
     return VH_OK;
 }
@@ -280,9 +280,12 @@ int g_qkv(vh_model *m, int layer, const float *x, float *norm, float *q, float *
     const vh_layer_weights &w = m->layers[layer];
     const vh_layer_extras &e = m->extras[layer];
     VHC(g_norm(m, x, w.attn_norm, e.attn_norm_bias, norm, rows));
-    VHC(g_mm(m, norm, w.wq, e.wq_bias, q, rows));
-    VHC(g_mm(m, norm, w.wk, e.wk_bias, k, rows));
-    VHC(g_mm(m, norm, w.wv, e.wv_bias, v, rows));
+    // (the three projections read one prepared copy of the normalised rows)
+    const bool prep = rows > 1 && m->cfg.hidden % 256 == 0 && fast(w.wq) && fast(w.wk) && fast(w.wv);
+    if (prep) VXC(vx_prepare_act(m->be, norm, rows, m->cfg.hidden));
+    VHC(g_mm(m, norm, w.wq, e.wq_bias, q, rows, prep));
+    VHC(g_mm(m, norm, w.wk, e.wk_bias, k, rows, prep));
+    VHC(g_mm(m, norm, w.wv, e.wv_bias, v, rows, prep));
     return VH_OK;
 }
 
@@ -296,6 +299,9 @@ int g_tail(vh_model *m, int layer, float *x, float *norm, const float *attn, flo
     float *o = a.parallel_residual ? up : norm;                                        // :972-978
     VHC(g_mm(m, attn, w.wo, e.wo_bias, o, rows));                                      // :981-983
     if (a.post_norms && e.post_attn_norm) VXC(vx_rmsnorm(be, o, e.post_attn_norm, o, rows, c.hidden, c.eps));  // :985-987
+    // The activation can leave its kernel as W2's prepared operand (one launch less). That kernel takes a workgroup per
+    // row, and GELU's double-precision tanh makes it slow where the rows are few: a prompt chunk's rows only.
+    const bool act_prepared = rows >= 128 && fast(w.w2) && c.ffn % 256 == 0;
     bool gated_prepared = false;  // RMSNorm in front of a gated MLP: one launch normalises and prepares W1's and W3's operand
     if (!a.parallel_residual) {
         VXC(vx_add(be, x, o, x, rows * c.hidden));                                     // :989-991
@@ -308,12 +314,17 @@ int g_tail(vh_model *m, int layer, float *x, float *norm, const float *attn, flo
     }
     if (a.mlp_type == VH_MLP_GELU) {                                                   // :1004-1037
         VHC(g_mm(m, norm, w.w1, e.w1_bias, gate, rows));
-        VXC(vx_gelu(be, gate, gate, rows * c.ffn));
-        VHC(g_mm(m, gate, w.w2, e.w2_bias, norm, rows));
+        if (act_prepared) {
+            VXC(vx_gelu_prepare(be, gate, nullptr, rows, c.ffn));
+            VHC(g_mm(m, nullptr, w.w2, e.w2_bias, norm, rows, true));
+        } else {
+            VXC(vx_gelu(be, gate, gate, rows * c.ffn));
+            VHC(g_mm(m, gate, w.w2, e.w2_bias, norm, rows));
+        }
     } else {                                                                           // :1040-1062
         VHC(mm(m, gated_prepared, norm, w.w1, gate, nullptr, rows));
         VHC(mm(m, gated_prepared, norm, w.w3, up, nullptr, rows));
-        if (rows > 1 && fast(w.w2) && c.ffn % 256 == 0) {   // the activation leaves its kernel as W2's prepared operand
+        if (act_prepared) {
             if (a.mlp_type == VH_MLP_GEGLU)
                 VXC(vx_gelu_mul_prepare(be, gate, up, nullptr, rows, c.ffn));
             else

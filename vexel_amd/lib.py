@@ -74,6 +74,7 @@ SIGNATURES = {
     "vx_rmsnorm_prepare": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f]),
     "vx_silu_mul_prepare": (_i, [_vp, _vp, _vp, _vp, _i, _i]),
     "vx_gelu_mul_prepare": (_i, [_vp, _vp, _vp, _vp, _i, _i]),
+    "vx_gelu_prepare": (_i, [_vp, _vp, _vp, _i, _i]),
     "vx_matmul_quant_prepared": (_i, [_vp, _i, _vp, _vp, _vp, _i, _i, _i]),
     "vx_matmul_quant_has_fast_path": (_i, [_i, _vp, _i, _i]),
     "vx_last_matmul_kernel": (C.c_char_p, [_vp]),
