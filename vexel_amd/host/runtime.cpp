@@ -289,6 +289,29 @@ int g_qkv(vh_model *m, int layer, const float *x, float *norm, float *q, float *
     return VH_OK;
 }
 
+// block.go:834-868 for rows whose K/V go to the pool at given slots (decode batches, later prompt chunks, tree rows) in an
+// architecture whose norm the fused attention block does not have (LayerNorm, a norm bias): the norm by its own
+// kernel, one prepared copy of its output, then that block's grouped projection, biases, RoPE form and KV store.
+// false: the weights or the row count have no such path (the caller takes g_qkv and the separate RoPE + store).
+bool g_qkv_fusable(const vh_model *m, int layer, int rows) {
+    if (!m->fused || rows < 2 || layer >= m->cfg.num_layers || m->cfg.hidden % 256 != 0) return false;
+    const vh_layer_weights &w = m->layers[layer];
+    return w.wq.data && w.wk.data && w.wv.data && fast(w.wq) && fast(w.wk) && fast(w.wv) &&
+           vx_decode_attn_qkv_supported(&w.wq, &w.wk, &w.wv, m->cfg.head_dim) != 0;
+}
+int g_qkv_store(vh_model *m, int layer, const float *x, float *norm, float *q, int rows, const int32_t *d_pos,
+                const int32_t *d_slot) {
+    const vh_config &c = m->cfg;
+    const vh_layer_weights &w = m->layers[layer];
+    const vh_layer_extras &e = m->extras[layer];
+    VHC(g_norm(m, x, w.attn_norm, e.attn_norm_bias, norm, rows));
+    VXC(vx_prepare_act(m->be, norm, rows, c.hidden));
+    VXC(vx_decode_attn_qkv_ex(m->be, nullptr, nullptr, c.eps, 1, &w.wq, &w.wk, &w.wv, e.wq_bias, e.wk_bias, e.wv_bias, rows, d_pos,
+                              d_slot, m->kv[layer], c.kv_fp16, c.num_heads, c.num_kv_heads, c.head_dim, c.block_size,
+                              c.rope_theta, m->arch.rope_dim, m->arch.rope_neox, q));
+    return VH_OK;
+}
+
 // block.go:972-1077: Wo, post-norm, residual(s), FFN norm, MLP. `norm` holds the attention norm's output on entry.
 int g_tail(vh_model *m, int layer, float *x, float *norm, const float *attn, float *gate, float *up, int rows) {
     const vh_config &c = m->cfg;
@@ -365,10 +388,14 @@ int execute_layer_decode(vh_model *m, int layer, int rows, int max_kv_len, const
     const float scale = (float)(1.0 / sqrt((double)c.head_dim));                          // block.go:862
     if (m->general && !attn_fusable(m, layer)) {
         if (*chained) return fail("internal: prepared activation handed to a general layer");
-        VHC(g_qkv(m, layer, m->x, m->norm, m->q, m->k, m->v, rows));
-        VXC(vx_rope_store_paged_ex(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
-                                   c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta, m->arch.rope_dim,
-                                   m->arch.rope_neox));                               // :858, :868
+        if (g_qkv_fusable(m, layer, rows)) {
+            VHC(g_qkv_store(m, layer, m->x, m->norm, m->q, rows, m->d_token_pos, m->d_slot_map));
+        } else {
+            VHC(g_qkv(m, layer, m->x, m->norm, m->q, m->k, m->v, rows));
+            VXC(vx_rope_store_paged_ex(m->be, m->q, m->k, m->v, m->d_token_pos, m->d_slot_map, m->kv[layer], c.kv_fp16, rows,
+                                       c.num_heads, c.num_kv_heads, c.head_dim, c.block_size, c.rope_theta, m->arch.rope_dim,
+                                       m->arch.rope_neox));                           // :858, :868
+        }
         VXC(vx_sdpa_paged_decode_ragged(m->be, m->q, m->kv[layer], c.kv_fp16, m->d_tables, m->d_slots, m->d_kv_lens,
                                         m->attn, rows, c.max_blocks_per_seq, c.block_size, c.num_heads, c.num_kv_heads,
                                         c.head_dim, scale, max_kv_len));               // :872 (no soft cap on this arm)
@@ -1068,6 +1095,11 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
             chained = false;
             VXC(vx_sdpa_paged_decode_multiquery(be, q, m->kv[l], c.kv_fp16, d_bt, attn, d_kvl, (int)table.size(),
                                                 c.block_size, c.num_heads, c.num_kv_heads, c.head_dim, scale, n));
+        } else if (later && m->general && g_qkv_fusable(m, l, n)) {   // (a LayerNorm in front of the same fused projections)
+            if (chained) return fail("internal: prepared activation handed to a general layer");
+            VHC(g_qkv_store(m, l, x, norm, q, n, d_pos, d_slot));
+            VXC(vx_sdpa_paged_decode_multiquery(be, q, m->kv[l], c.kv_fp16, d_bt, attn, d_kvl, (int)table.size(),
+                                                c.block_size, c.num_heads, c.num_kv_heads, c.head_dim, scale, n));
         } else {
             if (chained) return fail("internal: prepared activation handed to an unfused layer");
             if (m->general) {
@@ -1284,9 +1316,13 @@ int vh_verify_tree(vh_model *m, int n_seqs, const int64_t *seq_ids, const int32_
                                       c.block_size, c.rope_theta, m->arch.rope_dim, m->arch.rope_neox, q));
         } else if (m->general) {
             if (chained) return fail("internal: prepared activation handed to a general layer");
-            VHC(g_qkv(m, l, x, norm, q, k, v, n));
-            VXC(vx_rope_store_paged_ex(be, q, k, v, d_pos, d_slot, m->kv[l], c.kv_fp16, n, c.num_heads, c.num_kv_heads,
-                                       c.head_dim, c.block_size, c.rope_theta, m->arch.rope_dim, m->arch.rope_neox));
+            if (g_qkv_fusable(m, l, n)) {
+                VHC(g_qkv_store(m, l, x, norm, q, n, d_pos, d_slot));
+            } else {
+                VHC(g_qkv(m, l, x, norm, q, k, v, n));
+                VXC(vx_rope_store_paged_ex(be, q, k, v, d_pos, d_slot, m->kv[l], c.kv_fp16, n, c.num_heads, c.num_kv_heads,
+                                           c.head_dim, c.block_size, c.rope_theta, m->arch.rope_dim, m->arch.rope_neox));
+            }
         } else {
             if (chained) return fail("internal: prepared activation handed to an unfused layer");
             bool prep;
