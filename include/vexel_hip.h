@@ -259,8 +259,9 @@ int vx_dequantize_packed(vx_backend *be, const vx_qweight *w, float *dst);
  * q_out [rows,Hq*D], rotated K and V scattered into the pool at slot_mapping[r]
  * (runtime/block.go:834-868). With x_prepared != 0 the normalised activation left prepared by the
  * previous vx_decode_ffn (next_norm_weight) is used and x / norm_weight are ignored. wq and wk share a format;
- * wv may have another one (the Q4_K_M mixes keep attn_v in Q6_K): it then is a launch of its own between the shared
- * prepare and the shared RoPE + store. */
+ * wv may have another one (the K-quant mixes keep attn_v in Q6_K): with packed copies of Q4_K or Q5_K beside Q6_K and at
+ * most 32 rows one launch still computes the three (its row groups shared out between the two formats), otherwise V is
+ * a launch of its own between the shared prepare and the shared RoPE + store. */
 int vx_decode_attn_qkv_supported(const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, int head_dim);
 /* Optional, once per decode step before the layers' vx_decode_attn_qkv calls: works out cos / sin of every (row,
  * dimension pair) for positions[0 .. rows-1] (up to 64 rows, heads up to 256) and keeps them in the backend. While the

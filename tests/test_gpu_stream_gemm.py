@@ -293,3 +293,59 @@ def test_fused_decode_blocks_with_packed_weights(be, rows, hq, hk, d, hidden, ff
     for p in list(dev.values()) + [dx, dnw, dnf, dpos, dslots, dpool, dq, dattn]:
         be.free(p)
     be.reset_pool()
+
+
+@pytest.mark.parametrize("fqk", [nx.FMT_Q4_K, nx.FMT_Q5_K])
+@pytest.mark.parametrize("rows", [2, 7, 17, 32, 40])
+@pytest.mark.parametrize("hq,hk,d,hidden", [(8, 2, 128, 1024), (32, 32, 128, 4096), (32, 8, 128, 4096), (24, 1, 64, 2048)])
+def test_fused_qkv_with_packed_v_in_q6_k(be, rows, hq, hk, d, hidden, fqk):
+    """attn_q and attn_k in Q4_K or Q5_K beside attn_v in Q6_K, as the K-quant mixes of GGUF files hold them, all
+    three packed: up to 32 rows one launch computes the three (row groups shared out between the two formats),
+    beyond that V takes a launch of its own; either way RMSNorm -> Q|K|V -> RoPE -> KV store gives what the oracle's
+    operators give."""
+    import os
+    rng = np.random.default_rng(rows * 31 + hq + hidden + fqk)
+    bs, nblocks, theta, eps = 16, 8, 10000.0, 1e-5
+    qd, kvd = hq * d, hk * d
+    fm = {"wq": fqk, "wk": fqk, "wv": nx.FMT_Q6_K}
+    shapes = {"wq": (qd, hidden), "wk": (kvd, hidden), "wv": (kvd, hidden)}
+    raw = {n: qz.random_quant(fm[n], rng, *shapes[n], std=0.05).reshape(-1) for n in shapes}
+    dev, qws = {}, {}
+    for name in shapes:
+        dev[name], qws[name] = _packed(be, raw[name], *shapes[name], fm[name])
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    nw = (1.0 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    positions = rng.integers(0, 100, rows).astype(np.int32)
+    slots = rng.permutation(nblocks * bs)[:rows].astype(np.int32)
+    per_block = 2 * bs * kvd
+    pool0 = nx.f32_to_f16_array(rng.standard_normal(nblocks * per_block).astype(np.float32))
+
+    h = nx.rmsnorm(x, nw, rows, hidden, eps)
+    q = nx.matmul_quant(fqk, h, raw["wq"], rows, qd, hidden)
+    kk = nx.matmul_quant(fqk, h, raw["wk"], rows, kvd, hidden)
+    vv = nx.matmul_quant(nx.FMT_Q6_K, h, raw["wv"], rows, kvd, hidden)
+    want_q, want_k = nx.rope_positions(q, kk, d, hq, hk, positions, d, theta, False)
+
+    dx, dnw = be.upload(x, permanent=True), be.upload(nw, permanent=True)
+    dpos, dslots = be.upload(positions, permanent=True), be.upload(slots, permanent=True)
+    dpool, dq = be.upload(pool0, permanent=True), be.alloc_permanent(rows * qd * 4)
+    be.rope_table_prepare(dpos, rows, d, theta)
+    be.decode_attn_qkv(dx, dnw, eps, False, qws["wq"], qws["wk"], qws["wv"], rows, dpos, dslots, dpool, True, hq, hk, d, bs,
+                       theta, dq)
+    if not [k for k in os.environ if k.startswith("VEXEL_HIP_")] and rows <= 32 and hidden % 1024 == 0:
+        assert be.last_matmul_kernel() == "qstream_mixed_kernel", be.last_matmul_kernel()
+    got_q = be.download(dq, (rows, qd), np.float32)
+    _close(got_q, want_q, 2e-4, 2e-5 * np.abs(want_q).max(), "Q")
+    pool = nx.f16_to_f32_array(be.download(dpool, (nblocks * per_block,), np.uint16))
+    untouched = np.ones(nblocks * per_block, dtype=bool)
+    for r in range(rows):
+        blk, off = divmod(int(slots[r]), bs)
+        ko, vo = blk * per_block + off * kvd, blk * per_block + bs * kvd + off * kvd
+        untouched[ko:ko + kvd] = False
+        untouched[vo:vo + kvd] = False
+        _close(pool[ko:ko + kvd], nx.f16_to_f32_array(nx.f32_to_f16_array(want_k[r])), 2e-3, 2e-3 * np.abs(want_k).max(), "K row %d" % r)
+        _close(pool[vo:vo + kvd], nx.f16_to_f32_array(nx.f32_to_f16_array(vv[r])), 2e-3, 2e-3 * np.abs(vv).max(), "V row %d" % r)
+    assert np.array_equal(pool[untouched], nx.f16_to_f32_array(pool0)[untouched])
+    for p in list(dev.values()) + [dx, dnw, dpos, dslots, dpool, dq]:
+        be.free(p)
+    be.reset_pool()

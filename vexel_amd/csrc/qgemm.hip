@@ -2364,7 +2364,12 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
     int ntot, ks;
     const Segs segs = make_segs(ws, mixed ? 2 : 3, &ntot);
     VSrc vs = {nullptr, 0, 0};
-    if (mixed) {
+    // Q and K of one format and V of another, all three with packed copies: one launch leaves the K slices' sums of
+    // the three side by side.
+    const bool one_mixed = mixed && wk->fmt == wq->fmt && mpad_for(rows) <= 32 &&
+                           stream_gemm_mixed_ok(be, wq->fmt, (const uint8_t *)wq->data, (const uint8_t *)wk->data, wq->n, wk->n,
+                                                wv->fmt, (const uint8_t *)wv->data, wv->n, k, rows);
+    if (mixed && !one_mixed) {
         // V first, into the second partial-sum area (the two change places around its launch), then Q|K as usual
         const vx_qweight *wvs[1] = {wv};
         int nv, ksv;
@@ -2401,9 +2406,14 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
             return launch_gemm_fmt(be, wq->fmt, segs, ntot, nullptr, nullptr, false, rows, k, nullptr, &epi);
         }
     }
-    rc = launch_gemm_fmt(be, wq->fmt, segs, ntot, nullptr, nullptr, true, rows, k, &ks);
-    if (rc) return rc;
     const PrepView pv = prep_view(be, mpad_for(rows), k);
+    if (one_mixed)
+        rc = stream_gemm_mixed(be, wq->fmt, (const uint8_t *)wq->data, (const uint8_t *)wk->data, wq->n, wk->n, wv->fmt,
+                               (const uint8_t *)wv->data, wv->n, k, rows, mpad_for(rows), pv, &ks);
+    else
+        rc = launch_gemm_fmt(be, wq->fmt, segs, ntot, nullptr, nullptr, true, rows, k, &ks);
+    if (rc) return rc;
+    if (one_mixed) be->last_matmul = "qstream_mixed_kernel";
     const int half = head_dim / 2;
     const int lanes = 256 / half > 0 ? 256 / half : 1;
     if ((lanes * half) % 64 != 0) {  // the row factor is a whole-wave computation

@@ -49,6 +49,13 @@ bool stream_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int 
 int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M, int mpad,
                 const PrepView &pv, const QkvEpi *epi, int *ks_out);
 
+// A Q|K|V group whose V matrix (format fb) differs from Q and K (format fa), each with a packed copy, in one launch:
+// the K slices' raw sums of all three as [slice][M][nq + nk + nv] in be->part_ws.
+bool stream_gemm_mixed_ok(vx_backend *be, int fa, const uint8_t *wq, const uint8_t *wk, int nq, int nk, int fb, const uint8_t *wv,
+                          int nv, int K, int M);
+int stream_gemm_mixed(vx_backend *be, int fa, const uint8_t *wq, const uint8_t *wk, int nq, int nk, int fb, const uint8_t *wv, int nv,
+                      int K, int M, int mpad, const PrepView &pv, int *ks_out);
+
 // More than 64 rows over the same packed copies. With one K slice and to_partials false the finished rows (row
 // factors, residual) go to out; otherwise the slices' sums to be->part_ws, *ks_out of them.
 bool tiles_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M);

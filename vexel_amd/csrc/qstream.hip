@@ -584,26 +584,28 @@ __device__ __forceinline__ half4v first16(half8 v) { return __builtin_shufflevec
 __device__ __forceinline__ half4v second16(half8 v) { return __builtin_shufflevector(v, v, 2, 3, 6, 7); }
 struct StreamShape {
     int M, Mpad, N, n_hc, npass, t_end0, t_end1;
+    int split_groups;  // (the two-format launch: row groups of the first format)
 };
 
 // grid = (row groups, K slices), block = 512. PH: half chunks a wave holds per pass (1 or 2); RG: tiles per
 // reduction; EPI: finish Q|K|V rows (one slice).
+// The workgroup's share: row group gx of gdx over the tiles [tile_lo, tile_lo + tile_cnt) (of format W), K slice
+// blockIdx.y. The LDS areas come from the kernel (red: [2][NW][16 * MT * (16 RG + 4)] floats).
 template <class W, int PH, int RG, int MT, bool EPI>
-__global__ void __launch_bounds__(64 * NW, 1)
-qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, const uint8_t *__restrict__ pw2,
-               const half8 *__restrict__ a_tiles, const float *__restrict__ a_cscale, const float *__restrict__ a_inv_scale,
-               const float *__restrict__ a_bsum, float *__restrict__ partial, const StreamShape a, const QkvEpi epi) {
+__device__ __forceinline__ void
+qstream_body(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, const uint8_t *__restrict__ pw2,
+             const half8 *__restrict__ a_tiles, const float *__restrict__ a_cscale, const float *__restrict__ a_inv_scale,
+             const float *__restrict__ a_bsum, float *__restrict__ partial, const StreamShape &a, const QkvEpi &epi,
+             float (*red)[NW][16 * MT * (16 * RG + 4)], float *wait_sums, float *s_fac, const int gx, const int gdx,
+             const int tile_lo, const int tile_cnt) {
     constexpr int D = RG * PH;            // requests in flight per wave
     constexpr int TP = 16 * RG + 4;       // floats per row of a wave's block in LDS
-    __shared__ __attribute__((aligned(16))) float red[2][NW][16 * MT * TP];
-    __shared__ __attribute__((aligned(16))) float wait_sums[EPI ? ACC_TILES * 16 * 16 * MT : 4];
-    __shared__ float s_fac[16 * MT];
 
     const int tid = threadIdx.x, lane = tid & 63, ln = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int n_tiles = a.N >> 4, mtiles = a.Mpad >> 4, n_hc = a.n_hc;
-    const int gb = n_tiles / (int)gridDim.x, gr = n_tiles % (int)gridDim.x;
-    const int t0 = blockIdx.x * gb + min((int)blockIdx.x, gr), nt = gb + ((int)blockIdx.x < gr ? 1 : 0);
+    const int mtiles = a.Mpad >> 4, n_hc = a.n_hc;
+    const int gb = tile_cnt / gdx, gr = tile_cnt % gdx;
+    const int t0 = tile_lo + gx * gb + min(gx, gr), nt = gb + (gx < gr ? 1 : 0);
     const int sb = n_hc / (int)gridDim.y, sr = n_hc % (int)gridDim.y;
     const int h0 = blockIdx.y * sb + min((int)blockIdx.y, sr), nh = sb + ((int)blockIdx.y < sr ? 1 : 0);
 
@@ -805,6 +807,39 @@ qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1,
             buf ^= 1;
         }
     }
+}
+
+// grid = (row groups, K slices), block = 512.
+template <class W, int PH, int RG, int MT, bool EPI>
+__global__ void __launch_bounds__(64 * NW, 1)
+qstream_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, const uint8_t *__restrict__ pw2,
+               const half8 *__restrict__ a_tiles, const float *__restrict__ a_cscale, const float *__restrict__ a_inv_scale,
+               const float *__restrict__ a_bsum, float *__restrict__ partial, const StreamShape a, const QkvEpi epi) {
+    __shared__ __attribute__((aligned(16))) float red[2][NW][16 * MT * (16 * RG + 4)];
+    __shared__ __attribute__((aligned(16))) float wait_sums[EPI ? ACC_TILES * 16 * 16 * MT : 4];
+    __shared__ float s_fac[16 * MT];
+    qstream_body<W, PH, RG, MT, EPI>(pw0, pw1, pw2, a_tiles, a_cscale, a_inv_scale, a_bsum, partial, a, epi, red, wait_sums, s_fac,
+                                     (int)blockIdx.x, (int)gridDim.x, 0, a.N >> 4);
+}
+
+// Two formats in one launch (a Q|K|V group whose V matrix has another format than Q and K, as the Q4_K_M mixes keep
+// attn_v in Q6_K): the first a.split_groups row groups take the tiles below a.t_end1 in format W1, the others the
+// tiles from there on in format W2; one half chunk per wave, K slices of 8 half chunks, no epilogue.
+template <class W1, class W2, int RG, int MT>
+__global__ void __launch_bounds__(64 * NW, 1)
+qstream_mixed_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, const uint8_t *__restrict__ pw2,
+                     const half8 *__restrict__ a_tiles, const float *__restrict__ a_cscale, const float *__restrict__ a_inv_scale,
+                     const float *__restrict__ a_bsum, float *__restrict__ partial, const StreamShape a) {
+    __shared__ __attribute__((aligned(16))) float red[2][NW][16 * MT * (16 * RG + 4)];
+    __shared__ float unused[4];
+    const QkvEpi none = {};
+    const int split = __builtin_amdgcn_readfirstlane(a.split_groups);
+    if ((int)blockIdx.x < split)
+        qstream_body<W1, 1, RG, MT, false>(pw0, pw1, pw2, a_tiles, a_cscale, a_inv_scale, a_bsum, partial, a, none, red, unused,
+                                           unused, (int)blockIdx.x, split, 0, a.t_end1);
+    else
+        qstream_body<W2, 1, RG, MT, false>(pw0, pw1, pw2, a_tiles, a_cscale, a_inv_scale, a_bsum, partial, a, none, red, unused,
+                                           unused, (int)blockIdx.x - split, (int)gridDim.x - split, a.t_end1, (a.N >> 4) - a.t_end1);
 }
 
 
@@ -1275,6 +1310,7 @@ int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_e
     a.npass = pl.npass;
     a.t_end0 = ps.t_end[0];
     a.t_end1 = ps.t_end[1];
+    a.split_groups = 0;
     const QkvEpi e = fin ? *epi : QkvEpi{};
     float *partial = nullptr;
     if (!fin) {
@@ -1293,6 +1329,101 @@ int stream_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_e
     return VX_OK;
 }
 
+
+// ---- a Q|K|V group whose V matrix has another format: one launch over both
+// Q and K (format fa, rows na) and V (format fb, rows nb) with packed copies; 2 .. 32 rows (the formats with a min term
+// hold no more), K in slices of 8 half chunks, the row groups shared out by what a tile of each format costs.
+static bool mixed_resolve(vx_backend *be, int fa, const uint8_t *wq, const uint8_t *wk, int nq, int nk, int fb, const uint8_t *wv,
+                          int nv, int K, PackedSegs *out) {
+    PackedW *pq = find_packed(be, wq), *pk = find_packed(be, wk), *pv = find_packed(be, wv);
+    if (!pq || !pk || !pv || pq->fmt != fa || pk->fmt != fa || pv->fmt != fb) return false;
+    if (pq->k != K || pk->k != K || pv->k != K || pq->n != nq || pk->n != nk || pv->n != nv) return false;
+    out->w[0] = (const uint8_t *)pq->data;
+    out->w[1] = (const uint8_t *)pk->data;
+    out->w[2] = (const uint8_t *)pv->data;
+    out->t_end[0] = nq / 16;
+    out->t_end[1] = (nq + nk) / 16;
+    out->t_end[2] = (nq + nk + nv) / 16;
+    return true;
+}
+
+// The row groups of a two-format launch and how many of them the first format takes. A group works in rounds of four
+// tiles (a started round costs a whole one), and a round costs what its format's tiles cost (relative to Q4_0's: the
+// many-rows kernel's plan uses the same figures): the split with the shortest longer side, then the least work.
+static bool mixed_plan(vx_backend *be, int ta, int tb, int slices, int *groups_out, int *ga_out) {
+    static int cus = 0;
+    if (cus == 0 && (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0)) cus = 256;
+    const int groups = std::max(2, std::min(cus / slices, ta + tb));
+    auto rounds = [](int tiles, int g) { return (ceil_div(tiles, g) + 3) / 4; };
+    float best = 0.f, best_sum = 0.f;
+    int best_ga = 0;
+    for (int ga = 1; ga < groups; ga++) {
+        const int gb = groups - ga;
+        if (ga > ta || gb > tb) continue;  // (no group without a tile)
+        const float ra = 1.3f * (float)rounds(ta, ga), rb = 1.9f * (float)rounds(tb, gb);
+        const float longer = std::max(ra, rb), sum = ra * (float)ga + rb * (float)gb;
+        if (best_ga == 0 || longer < best || (longer == best && sum < best_sum)) {
+            best = longer;
+            best_sum = sum;
+            best_ga = ga;
+        }
+    }
+    if (best_ga == 0) return false;
+    *groups_out = groups;
+    *ga_out = best_ga;
+    return true;
+}
+
+bool stream_gemm_mixed_ok(vx_backend *be, int fa, const uint8_t *wq, const uint8_t *wk, int nq, int nk, int fb, const uint8_t *wv,
+                          int nv, int K, int M) {
+    static const char *off = getenv("VEXEL_HIP_STREAM_OFF");
+    if (off && atoi(off)) return false;
+    static const bool mixed_off = getenv("VEXEL_HIP_MIXED_OFF") != nullptr;  // (measurements: V in a launch of its own)
+    if (mixed_off) return false;
+    if (!((fa == VX_Q4_K || fa == VX_Q5_K) && fb == VX_Q6_K)) return false;  // (the pairs the K-quant mixes hold)
+    if (M < 2 || M > 32 || K % 1024 != 0 || nq % 16 || nk % 16 || nv % 16 || nq < 16 || nk < 16 || nv < 16) return false;
+    if (be->packed.empty()) return false;
+    PackedSegs ps;
+    int groups, ga;
+    return mixed_resolve(be, fa, wq, wk, nq, nk, fb, wv, nv, K, &ps) && mixed_plan(be, (nq + nk) / 16, nv / 16, K / 128 / NW, &groups, &ga);
+}
+
+int stream_gemm_mixed(vx_backend *be, int fa, const uint8_t *wq, const uint8_t *wk, int nq, int nk, int fb, const uint8_t *wv, int nv,
+                      int K, int M, int mpad, const PrepView &pv, int *ks_out) {
+    PackedSegs ps;
+    if (!mixed_resolve(be, fa, wq, wk, nq, nk, fb, wv, nv, K, &ps)) return VX_ERR_UNSUPPORTED;
+    const int N = nq + nk + nv, n_hc = K / 128, slices = n_hc / NW, mt = mpad / 16;
+    if (mt != 1 && mt != 2) return VX_ERR_UNSUPPORTED;
+    int groups, ga;
+    if (!mixed_plan(be, (nq + nk) / 16, nv / 16, slices, &groups, &ga)) return VX_ERR_UNSUPPORTED;
+    StreamShape a;
+    a.M = M;
+    a.Mpad = mpad;
+    a.N = N;
+    a.n_hc = n_hc;
+    a.npass = 1;
+    a.t_end0 = ps.t_end[0];
+    a.t_end1 = ps.t_end[1];
+    a.split_groups = ga;
+    int rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, (size_t)slices * M * N * sizeof(float), "split-K partial sums");
+    if (rc) return rc;
+    float *partial = (float *)be->part_ws;
+    dim3 grid(groups, slices);
+#define VX_MIXED_LAUNCH(W1_, MT_)                                                                                              \
+    qstream_mixed_kernel<W1_, SQ6_K, 4, MT_><<<grid, 64 * NW, 0, be->stream>>>(ps.w[0], ps.w[1], ps.w[2], pv.tiles, pv.cscale,    \
+                                                                                pv.inv_scale, pv.bsum, partial, a)
+    if (fa == VX_Q4_K) {
+        if (mt == 2) VX_MIXED_LAUNCH(SQ4_K, 2);
+        else VX_MIXED_LAUNCH(SQ4_K, 1);
+    } else {
+        if (mt == 2) VX_MIXED_LAUNCH(SQ5_K, 2);
+        else VX_MIXED_LAUNCH(SQ5_K, 1);
+    }
+#undef VX_MIXED_LAUNCH
+    VX_CHECK_LAUNCH();
+    if (ks_out) *ks_out = slices;
+    return VX_OK;
+}
 
 bool tiles_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M) {
     static const char *off = getenv("VEXEL_HIP_TILES_OFF");
@@ -1342,6 +1473,7 @@ int tiles_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_en
     a.npass = 1;
     a.t_end0 = ps.t_end[0];
     a.t_end1 = ps.t_end[1];
+    a.split_groups = 0;
     float *partial = nullptr;
     if (pl.s > 1 || to_partials) {
         int rc = ensure_ws(be, &be->part_ws, &be->part_ws_bytes, (size_t)pl.s * M * N * sizeof(float), "split-K partial sums");
