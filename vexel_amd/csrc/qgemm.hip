@@ -1490,7 +1490,7 @@ __global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, 
                                            float *__restrict__ q_out, const int32_t *__restrict__ positions,
                                            const int32_t *__restrict__ slot_mapping, void *__restrict__ pool,
                                            int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta,
-                                           VSrc vs) {
+                                           VSrc vs, const float2 *__restrict__ cs_tab = nullptr) {
     const int row = blockIdx.x, half = head_dim / 2;
     const int qd = num_q_heads * head_dim, kvd = num_kv_heads * head_dim, ncols = vs.P ? qd + kvd : qd + 2 * kvd;
     const size_t slice_elems = (size_t)M * ncols;
@@ -1502,10 +1502,18 @@ __global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, 
     const int lanes = blockDim.x / half, hl = threadIdx.x / half, j = threadIdx.x % half;
     if (hl >= lanes) return;
     const int hstride = lanes * gridDim.y, h0 = blockIdx.y * lanes + hl;
-    const double ex = (double)(2 * j) / (double)head_dim;
-    const float freq = (float)(1.0 / pow((double)theta, ex));
-    const float angle = __fmul_rn((float)pos, freq);
-    const float c = (float)cos((double)angle), sn = (float)sin((double)angle);
+    float c, sn;
+    if (cs_tab) {  // the step's table of angles (rope_table_kernel: the arithmetic below, once per row and pair)
+        const float2 cs = cs_tab[(size_t)row * half + j];
+        c = cs.x;
+        sn = cs.y;
+    } else {
+        const double ex = (double)(2 * j) / (double)head_dim;
+        const float freq = (float)(1.0 / pow((double)theta, ex));
+        const float angle = __fmul_rn((float)pos, freq);
+        c = (float)cos((double)angle);
+        sn = (float)sin((double)angle);
+    }
     auto pair = [&](int col, float &a, float &b) {
         const float *p0 = P + (size_t)row * ncols + col;
         float2 v = *(const float2 *)p0;
@@ -2422,6 +2430,10 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
     }
     const RowNorm rn = cur_row_norm(be);
     const int max_heads = num_q_heads > num_kv_heads ? num_q_heads : num_kv_heads;
+    // the step's table of angles, where it stands for these positions (vx_rope_table_prepare)
+    const bool have_table = be->rope_tab_pos == positions && be->rope_tab_rows >= rows && be->rope_tab_dim == head_dim &&
+                            be->rope_tab_theta == theta && be->rope_tab_epoch == be->write_epoch;
+    const float2 *cs_tab = have_table ? (const float2 *)be->rope_tab : nullptr;
     dim3 grid(rows, ceil_div(max_heads, lanes));
     if (gen && pool_is_f16)
         rope_store_general_kernel<true, true><<<grid, lanes * half, 0, be->stream>>>(
@@ -2434,11 +2446,11 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
     else if (pool_is_f16)
         rope_store_partials_kernel<true><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-            num_kv_heads, head_dim, block_size, theta, vs);
+            num_kv_heads, head_dim, block_size, theta, vs, cs_tab);
     else
         rope_store_partials_kernel<false><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-            num_kv_heads, head_dim, block_size, theta, vs);
+            num_kv_heads, head_dim, block_size, theta, vs, cs_tab);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }

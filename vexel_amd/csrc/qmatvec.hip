@@ -639,7 +639,8 @@ __global__ void __launch_bounds__(MV_THREADS) qmatvec2_kernel(const MvArgs p, in
         float acc[NR];
 #pragma unroll
         for (int r = 0; r < NR; r++) acc[r] = 0.f;
-#pragma unroll
+        constexpr int UNROLL_T = TT > 0 ? TT : 1;  // (a trip count known only at run time: as written)
+#pragma unroll UNROLL_T
         for (int t = 0; t < (TT > 0 ? TT : T); t++) {
             const int j = t * 64 + lane;
             const int jx = j < nblocks ? j : nblocks;   // past the row's end: the zero planes

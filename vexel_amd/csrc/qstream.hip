@@ -111,7 +111,7 @@ __device__ __forceinline__ float half_of(uint32_t w, int hi) {
 // What the kernel needs to know of a packed format: the unit's size, what a lane requests of it (Ring), and how the
 // request becomes block j's operand and scale.
 struct SQ4_0 {
-    static constexpr int FMT = VX_Q4_0, UNIT = 1152, SCALES_AT = 1024, BLOCK_BYTES = 18;
+    static constexpr int UNIT = 1152, SCALES_AT = 1024;
     static constexpr bool TWO_SCALES = false, HAS_MIN = false;
     struct Ring {
         u32x4 c;
@@ -133,7 +133,7 @@ struct SQ4_0 {
 // 1040 + 32 r. The m1 term multiplies the activation's block sums (prepared with the tiles): one more FMA per output
 // and block. 6 bits per weight against GGUF's 4.5.
 struct SQ4_K {
-    static constexpr int FMT = VX_Q4_K, UNIT = 1536, SCALES_AT = 1024;
+    static constexpr int UNIT = 1536, SCALES_AT = 1024;
     static constexpr bool TWO_SCALES = false, HAS_MIN = true;
     struct Ring {
         u32x4 c;
@@ -153,7 +153,7 @@ struct SQ4_K {
 // Q8_0: a unit is 2176 bytes, lane l = 16 g + r owns 32 of the first 2048: block j's eight codes at 8 j, as q + 128,
 // slot s at byte (s & 4) + {0, 2, 1, 3}[s & 3]; row r's four f16 scales at 2048 + 8 r. 34 bytes per block as in GGUF.
 struct SQ8_0 {
-    static constexpr int FMT = VX_Q8_0, UNIT = 2176, SCALES_AT = 2048, BLOCK_BYTES = 34;
+    static constexpr int UNIT = 2176, SCALES_AT = 2048;
     static constexpr bool TWO_SCALES = false, HAS_MIN = false;
     struct Ring {
         u32x4 c0, c1;
@@ -177,7 +177,7 @@ struct SQ8_0 {
 // d1 * q - m1 with 5-bit q) gets a unit of 2560 bytes: the codes one byte each in the Q8_0 unit's order (unsigned),
 // then row r's d1[4] at 2048 + 32 r and m1[4] at 2064 + 32 r; its min term as Q4_K's. 10 bits per weight against 5.5.
 struct SQ5_K {
-    static constexpr int FMT = VX_Q5_K, UNIT = 2560, SCALES_AT = 2048;
+    static constexpr int UNIT = 2560, SCALES_AT = 2048;
     static constexpr bool TWO_SCALES = false, HAS_MIN = true;
     struct Ring {
         u32x4 c0, c1;
@@ -213,7 +213,7 @@ __device__ __forceinline__ half4v unpack_q6(uint32_t w) {
     return r;
 }
 struct SQ6_K {
-    static constexpr int FMT = VX_Q6_K, UNIT = 2560, SCALES_AT = 2048;
+    static constexpr int UNIT = 2560, SCALES_AT = 2048;
     static constexpr bool TWO_SCALES = true, HAS_MIN = false;
     struct Ring {
         u32x4 c0, c1;
