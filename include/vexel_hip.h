@@ -267,7 +267,9 @@ int vx_decode_attn_qkv_supported(const vx_qweight *wq, const vx_qweight *wk, con
  * dimension pair) for positions[0 .. rows-1] (up to 64 rows, heads up to 256) and keeps them in the backend. While the
  * table stands, a vx_decode_attn_qkv call with the same positions pointer, at most 32 rows, an unbiased interleaved
  * whole-head RoPE and weights laid out for a single K slice rotates and stores its rows inside the projection launch
- * (one launch per layer less), with the same arithmetic. The table falls when the library writes to a caller's
+ * (one launch per layer less), with the same arithmetic; a call whose projection leaves K slices' sums (more rows, the
+ * formats with a min term, V in another format) reads its cos / sin from the table in the RoPE + store launch that
+ * follows. The table falls when the library writes to a caller's
  * buffer (vx_pack_batch, vx_decode_advance, vx_to_device, vx_copy_buffer); a caller that changes the positions by
  * other means must call this again (or not at all: without a table nothing changes). No counterpart in the reference,
  * which recomputes the angles in every layer (backend/cpu/cpu.go:226-303). */
