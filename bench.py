@@ -654,7 +654,7 @@ def _config4(be, rng, ctx4, l8b, decode_rate, prefill):
     if not prefill:
         mr.close()
         return
-    mr.prefill_with_paged_kv(chunk[:64], 1000, 0)           # sizes the workspaces
+    mr.prefill_with_paged_kv(chunk, 1000, 0)                # (untimed: sizes the workspaces for 512 rows)
     mr.delete_sequence(1000)
     be.sync()
     t0 = time.perf_counter()

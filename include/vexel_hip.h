@@ -286,6 +286,16 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
                           const float *k_bias, const float *v_bias, int rows, const int32_t *positions,
                           const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int num_q_heads, int num_kv_heads,
                           int head_dim, int block_size, float theta, int rope_dim, int rope_neox, float *q_out);
+/* vx_decode_attn_qkv_ex for the first chunk of a prompt (runtime/block.go:834-868 at startPos 0): the same block, and
+ * the rotated K rows and the V rows also as dense floats, k_out / v_out [rows, Hkv*D] (not yet rounded to the pool's
+ * type), which the causal attention of that chunk reads (SDPAPrefill, block.go:893-895). k_out = v_out = NULL: exactly
+ * vx_decode_attn_qkv_ex. */
+int vx_prefill_attn_qkv(vx_backend *be, const float *x, const float *norm_weight, float eps, int x_prepared,
+                        const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, const float *q_bias,
+                        const float *k_bias, const float *v_bias, int rows, const int32_t *positions,
+                        const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int num_q_heads, int num_kv_heads,
+                        int head_dim, int block_size, float theta, int rope_dim, int rope_neox, float *q_out, float *k_out,
+                        float *v_out);
 
 /* x += attn*Wo^T; h = RMSNorm(x, ffn_norm_weight); x += (SiLU(h*W1^T) * (h*W3^T)) * W2^T
  * (runtime/block.go:981-1077), x [rows,hidden] updated in place. attn may be NULL when the call follows a

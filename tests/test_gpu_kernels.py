@@ -1504,6 +1504,64 @@ def test_decode_attn_qkv_with_bias_and_rope_forms(be, rows, rope_dim, neox, bias
     be.reset_pool()
 
 
+@pytest.mark.parametrize("fmt", [nx.FMT_Q4_0, nx.FMT_Q6_K])
+@pytest.mark.parametrize("rows,f16,general", [(1, True, False), (5, True, False), (40, False, True), (130, True, False),
+                                              (130, False, False), (200, True, True)])
+def test_prefill_attn_qkv_leaves_dense_k_and_v(be, fmt, rows, f16, general):
+    """vx_prefill_attn_qkv (a prompt's first chunk, block.go:834-868 + 891-895): Q and the pool as
+    vx_decode_attn_qkv_ex leaves them, bit for bit, and the rotated K rows and the V rows as dense floats - the values
+    the pool holds (exactly for a float pool, rounded to f16 for an f16 pool) -, against the oracle's operation
+    sequence; both RoPE + store kernels (the interleaved whole-head form, and the general one with biases and a
+    partial NeoX rotation)."""
+    rng = np.random.default_rng(500 + rows + fmt)
+    hq, hk, d, hidden, bs, nblocks = 8, 2, 64, 1024, 16, 40
+    qd, kvd = hq * d, hk * d
+    rope_dim, neox = (32, True) if general else (0, False)
+    x = rng.standard_normal((rows, hidden)).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
+    ws = [qz.random_quant(fmt, rng, n, hidden) for n in (qd, kvd, kvd)]
+    bs_ = [(0.1 * rng.standard_normal(n)).astype(np.float32) if general else None for n in (qd, kvd, kvd)]
+    pos = np.arange(rows, dtype=np.int32)
+    slots = rng.permutation(nblocks * bs)[:rows].astype(np.int32)
+    pool = _make_pool(rng, f16, nblocks, bs, hk, d)
+    norm = nx.rmsnorm(x, nw, rows, hidden, 1e-5)
+    proj = [nx.matmul_quant(fmt, norm, w, rows, n, hidden) for w, n in zip(ws, (qd, kvd, kvd))]
+    if general:
+        proj = [nx.add_bias(p, b, rows, n) for p, b, n in zip(proj, bs_, (qd, kvd, kvd))]
+    want_q, want_k = nx.rope_positions(proj[0], proj[1], d, hq, hk, pos, rope_dim if rope_dim else d, 10000.0, neox)
+    dx, dn = be.upload(x), be.upload(nw)
+    dws = [be.qweight(fmt, be.upload(w), n, hidden) for w, n in zip(ws, (qd, kvd, kvd))]
+    dbs = [be.upload(b) if b is not None else None for b in bs_]
+    dp, ds = be.upload(pos), be.upload(slots)
+    dpool1, dpool2 = be.upload(pool), be.upload(pool)
+    dq1, dq2, dk, dv = be.alloc(rows * qd * 4), be.alloc(rows * qd * 4), be.alloc(rows * kvd * 4), be.alloc(rows * kvd * 4)
+    be.decode_attn_qkv_ex(dx, dn, 1e-5, False, dws[0], dws[1], dws[2], dbs[0], dbs[1], dbs[2], rows, dp, ds, dpool1, f16,
+                          hq, hk, d, bs, 10000.0, rope_dim, neox, dq1)
+    be.prefill_attn_qkv(dx, dn, 1e-5, False, dws[0], dws[1], dws[2], dbs[0], dbs[1], dbs[2], rows, dp, ds, dpool2, f16,
+                        hq, hk, d, bs, 10000.0, rope_dim, neox, dq2, dk, dv)
+    q1, q2 = be.download(dq1, (rows, qd), np.float32), be.download(dq2, (rows, qd), np.float32)
+    p1, p2 = be.download(dpool1, pool.shape, pool.dtype), be.download(dpool2, pool.shape, pool.dtype)
+    k, v = be.download(dk, (rows, kvd), np.float32), be.download(dv, (rows, kvd), np.float32)
+    if rows > 1:   # (one row: the decode entry point takes the matrix-vector kernels, whose sums are added in another order)
+        assert np.array_equal(q1.view(np.uint32), q2.view(np.uint32))
+        assert np.array_equal(p1, p2)
+    scale = np.abs(want_q).max()
+    _close(q2, want_q.reshape(rows, qd), 2e-5, 3e-6 * scale + 1e-7, "q")
+    _close(k, want_k.reshape(rows, kvd), 2e-5, 3e-6 * np.abs(want_k).max() + 1e-7, "dense k")
+    _close(v, proj[2].reshape(rows, kvd), 2e-5, 3e-6 * np.abs(proj[2]).max() + 1e-7, "dense v")
+    per_blk = 2 * bs * kvd
+    for r, sl in enumerate(slots):
+        b, o = int(sl) // bs, int(sl) % bs
+        pk = p2[b * per_blk + o * kvd: b * per_blk + (o + 1) * kvd]
+        pv_ = p2[b * per_blk + bs * kvd + o * kvd: b * per_blk + bs * kvd + (o + 1) * kvd]
+        if f16:
+            assert np.array_equal(pk, nx.f32_to_f16_array(k[r])) and np.array_equal(pv_, nx.f32_to_f16_array(v[r])), r
+        else:
+            assert np.array_equal(pk.view(np.uint32), k[r].view(np.uint32)), r
+            assert np.array_equal(pv_.view(np.uint32), v[r].view(np.uint32)), r
+    be.reset_pool()
+
+
 @pytest.mark.parametrize("hq,hk,d,hidden", [(32, 32, 128, 4096), (32, 8, 128, 4096), (24, 8, 128, 3072)])
 def test_in_kernel_merge_equals_the_separate_merge_and_the_oracle(be, hq, hk, d, hidden):
     """The attention kernel's own merge of its splits (vx_backend_set_attn_merge, the default) against the merge left

@@ -326,6 +326,14 @@ class HipBackend:
                   C.byref(wv), q_bias, k_bias, v_bias, rows, positions, slot_mapping, kv_pool, int(bool(pool_is_f16)),
                   num_q_heads, num_kv_heads, head_dim, block_size, theta, rope_dim, int(bool(rope_neox)), q_out)
 
+    def prefill_attn_qkv(self, x, norm_weight, eps, x_prepared, wq, wk, wv, q_bias, k_bias, v_bias, rows, positions,
+                         slot_mapping, kv_pool, pool_is_f16, num_q_heads, num_kv_heads, head_dim, block_size, theta,
+                         rope_dim, rope_neox, q_out, k_out, v_out):
+        self.call("vx_prefill_attn_qkv", x, norm_weight, eps, int(bool(x_prepared)), C.byref(wq), C.byref(wk),
+                  C.byref(wv), q_bias, k_bias, v_bias, rows, positions, slot_mapping, kv_pool, int(bool(pool_is_f16)),
+                  num_q_heads, num_kv_heads, head_dim, block_size, theta, rope_dim, int(bool(rope_neox)), q_out, k_out,
+                  v_out)
+
     def decode_ffn_supported(self, wo, w1, w3, w2):
         return bool(self._lib.vx_decode_ffn_supported(C.byref(wo), C.byref(w1), C.byref(w3), C.byref(w2)))
 

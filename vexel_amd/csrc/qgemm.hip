@@ -1417,7 +1417,8 @@ __global__ void rope_store_general_kernel(const float *__restrict__ P, int KS, i
                                           float *__restrict__ q_out, const int32_t *__restrict__ positions,
                                           const int32_t *__restrict__ slot_mapping, void *__restrict__ pool,
                                           int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta,
-                                          QkvExtra ex, VSrc vs) {
+                                          QkvExtra ex, VSrc vs, float *__restrict__ k_out = nullptr,
+                                          float *__restrict__ v_out = nullptr) {
     static_assert(GEN, "the interleaved whole-head form is rope_store_partials_kernel");
     const int row = blockIdx.x, half = head_dim / 2, he = ex.eff_dim / 2;
     const int qd = num_q_heads * head_dim, kvd = num_kv_heads * head_dim, ncols = vs.P ? qd + kvd : qd + 2 * kvd;
@@ -1469,6 +1470,12 @@ __global__ void rope_store_general_kernel(const float *__restrict__ P, int KS, i
         const float va = velem(b0), vb = velem(b1);
         const float ka = turn ? __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, sn)) : a;
         const float kb = turn ? __fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, c)) : b;
+        if (k_out) {  // (a prompt's first chunk: the rows also as dense floats for the attention that follows)
+            k_out[(size_t)row * kvd + b0] = ka;
+            k_out[(size_t)row * kvd + b1] = kb;
+            v_out[(size_t)row * kvd + b0] = va;
+            v_out[(size_t)row * kvd + b1] = vb;
+        }
         if (F16) {
             _Float16 *pp = (_Float16 *)pool;
             pp[kbase + b0] = (_Float16)ka;
@@ -1490,7 +1497,8 @@ __global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, 
                                            float *__restrict__ q_out, const int32_t *__restrict__ positions,
                                            const int32_t *__restrict__ slot_mapping, void *__restrict__ pool,
                                            int num_q_heads, int num_kv_heads, int head_dim, int block_size, float theta,
-                                           VSrc vs, const float2 *__restrict__ cs_tab = nullptr) {
+                                           VSrc vs, const float2 *__restrict__ cs_tab = nullptr, float *__restrict__ k_out = nullptr,
+                                           float *__restrict__ v_out = nullptr) {
     const int row = blockIdx.x, half = head_dim / 2;
     const int qd = num_q_heads * head_dim, kvd = num_kv_heads * head_dim, ncols = vs.P ? qd + kvd : qd + 2 * kvd;
     const size_t slice_elems = (size_t)M * ncols;
@@ -1555,6 +1563,10 @@ __global__ void rope_store_partials_kernel(const float *__restrict__ P, int KS, 
         const float ka = __fsub_rn(__fmul_rn(a, c), __fmul_rn(b, sn));
         const float kb = __fadd_rn(__fmul_rn(a, sn), __fmul_rn(b, c));
         const size_t o = (size_t)h * head_dim + 2 * j;
+        if (k_out) {  // (a prompt's first chunk: the rows also as dense floats for the attention that follows)
+            *(float2 *)(k_out + (size_t)row * kvd + o) = make_float2(ka, kb);
+            *(float2 *)(v_out + (size_t)row * kvd + o) = make_float2(va, vb);
+        }
         if (F16) {
             _Float16 *pp = (_Float16 *)pool;
             pp[kbase + o] = (_Float16)ka;
@@ -2265,8 +2277,21 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
                           const float *k_bias, const float *v_bias, int rows, const int32_t *positions,
                           const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int num_q_heads, int num_kv_heads,
                           int head_dim, int block_size, float theta, int rope_dim, int rope_neox, float *q_out) {
+    return vx_prefill_attn_qkv(be, x, norm_weight, eps, x_prepared, wq, wk, wv, q_bias, k_bias, v_bias, rows, positions,
+                               slot_mapping, kv_pool, pool_is_f16, num_q_heads, num_kv_heads, head_dim, block_size, theta,
+                               rope_dim, rope_neox, q_out, nullptr, nullptr);
+}
+
+int vx_prefill_attn_qkv(vx_backend *be, const float *x, const float *norm_weight, float eps, int x_prepared,
+                        const vx_qweight *wq, const vx_qweight *wk, const vx_qweight *wv, const float *q_bias,
+                        const float *k_bias, const float *v_bias, int rows, const int32_t *positions,
+                        const int32_t *slot_mapping, void *kv_pool, int pool_is_f16, int num_q_heads, int num_kv_heads,
+                        int head_dim, int block_size, float theta, int rope_dim, int rope_neox, float *q_out, float *k_out,
+                        float *v_out) {
     int rc = enter(be);
     if (rc) return rc;
+    VX_REQUIRE((k_out == nullptr) == (v_out == nullptr), "vx_prefill_attn_qkv: k_out and v_out go together");
+    VX_REQUIRE(!k_out || (((uintptr_t)k_out % 8) == 0 && ((uintptr_t)v_out % 8) == 0), "vx_prefill_attn_qkv: unaligned output");
     const int eff_dim = rope_dim == 0 ? head_dim : rope_dim;
     VX_REQUIRE(eff_dim > 0 && eff_dim <= head_dim && eff_dim % 2 == 0, "vx_decode_attn_qkv: rope_dim %d invalid for head_dim %d",
                rope_dim, head_dim);
@@ -2282,7 +2307,7 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
                "vx_decode_attn_qkv: weight shapes do not match the head geometry");
     const int k = wq->k;
     static const bool no_matvec = getenv("VEXEL_HIP_NO_MATVEC") != nullptr;
-    if (rows == 1 && !x_prepared && !no_matvec && pool_is_f16 && head_dim % 2 == 0) {
+    if (rows == 1 && !x_prepared && !no_matvec && pool_is_f16 && head_dim % 2 == 0 && !k_out) {
         // A single row: Q|K|V by one matrix-vector launch with the RMSNorm folded in (the row enters as x * w,
         // the dot products are divided by rms(x)), then RoPE and the KV store from that launch's output.
         const void *mw[3] = {wq->data, wk->data, wv->data};
@@ -2392,7 +2417,7 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
     }
     // One K slice, one activation group, the plain RoPE form and a table of this step's angles: the GEMM's workgroups
     // finish their own rows (no partial sums, no second launch).
-    if (!mixed) {
+    if (!mixed && !k_out) {
         const WavePlan pl = wave_plan(be, wq->fmt, segs, ntot, k, rows);
         const bool table = be->rope_tab_pos == positions && be->rope_tab_rows >= rows && be->rope_tab_dim == head_dim &&
                            be->rope_tab_theta == theta && be->rope_tab_epoch == be->write_epoch;
@@ -2438,19 +2463,19 @@ int vx_decode_attn_qkv_ex(vx_backend *be, const float *x, const float *norm_weig
     if (gen && pool_is_f16)
         rope_store_general_kernel<true, true><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-            num_kv_heads, head_dim, block_size, theta, ex, vs);
+            num_kv_heads, head_dim, block_size, theta, ex, vs, k_out, v_out);
     else if (gen)
         rope_store_general_kernel<false, true><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-            num_kv_heads, head_dim, block_size, theta, ex, vs);
+            num_kv_heads, head_dim, block_size, theta, ex, vs, k_out, v_out);
     else if (pool_is_f16)
         rope_store_partials_kernel<true><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-            num_kv_heads, head_dim, block_size, theta, vs, cs_tab);
+            num_kv_heads, head_dim, block_size, theta, vs, cs_tab, k_out, v_out);
     else
         rope_store_partials_kernel<false><<<grid, lanes * half, 0, be->stream>>>(
             (const float *)be->part_ws, ks, rows, pv.inv_scale, rn, q_out, positions, slot_mapping, kv_pool, num_q_heads,
-            num_kv_heads, head_dim, block_size, theta, vs, cs_tab);
+            num_kv_heads, head_dim, block_size, theta, vs, cs_tab, k_out, v_out);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }

@@ -1070,9 +1070,12 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
     // A later chunk reads every key from the pool (block.go:881-890), so its projections can take the decode step's
     // fused form: Q|K|V in one launch that rotates and stores K/V itself; the fused tail serves every chunk.
     const bool later = n > 1 && start_pos > 0;
+    // The first chunk attends over its own rows as dense floats (block.go:891-895): the same fused projection block
+    // leaves the rotated K and V rows in that form too, beside the pool store.
+    const bool first = n > 1 && start_pos == 0;
     const bool tails_fusable = n > 1 && m->fused && (!m->general || m->fused_ok);
     int32_t *d_pos = nullptr, *d_slot = nullptr;
-    if (later) {
+    if (later || first) {
         std::vector<int32_t> pos(n), slot(n);
         for (int i = 0; i < n; i++) {
             pos[i] = start_pos + i;
@@ -1095,6 +1098,17 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
             chained = false;
             VXC(vx_sdpa_paged_decode_multiquery(be, q, m->kv[l], c.kv_fp16, d_bt, attn, d_kvl, (int)table.size(),
                                                 c.block_size, c.num_heads, c.num_kv_heads, c.head_dim, scale, n));
+        } else if (first && attn_fusable(m, l)) {
+            const vh_layer_extras &e = m->extras[l];
+            VXC(vx_prefill_attn_qkv(be, x, w.attn_norm, c.eps, chained ? 1 : 0, &w.wq, &w.wk, &w.wv, e.wq_bias, e.wk_bias,
+                                    e.wv_bias, n, d_pos, d_slot, m->kv[l], c.kv_fp16, c.num_heads, c.num_kv_heads, c.head_dim,
+                                    c.block_size, c.rope_theta, m->arch.rope_dim, m->arch.rope_neox, q, k, v));
+            chained = false;
+            if (m->arch.attn_softcap > 0.f)                                               // block.go:891-892
+                VXC(vx_sdpa_prefill_softcap(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale,
+                                            m->arch.attn_softcap));
+            else                                                                           // block.go:893-895
+                VXC(vx_sdpa_prefill(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale));
         } else if (later && m->general && g_qkv_fusable(m, l, n)) {   // (a LayerNorm in front of the same fused projections)
             if (chained) return fail("internal: prepared activation handed to a general layer");
             VHC(g_qkv_store(m, l, x, norm, q, n, d_pos, d_slot));
@@ -1142,7 +1156,7 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
         }
         if (tails_fusable && w.wo.data && w.w1.data && w.w2.data && w.w3.data &&
             vx_decode_ffn_supported(&w.wo, &w.w1, &w.w3, &w.w2)) {                      // block.go:981-1077
-            const float *next_norm = l + 1 < c.num_layers && later && attn_fusable(m, l + 1) ? m->layers[l + 1].attn_norm : nullptr;
+            const float *next_norm = l + 1 < c.num_layers && (later || first) && attn_fusable(m, l + 1) ? m->layers[l + 1].attn_norm : nullptr;
             VXC(vx_decode_ffn(be, attn, x, &w.wo, w.ffn_norm, c.eps, &w.w1, &w.w3, &w.w2, n, next_norm));
             chained = next_norm != nullptr;
         } else if (m->general) {

@@ -83,6 +83,8 @@ SIGNATURES = {
     "vx_decode_attn_qkv_ex": (_i, [_vp, _vp, _vp, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i,
                                    _f, _i, _i, _vp]),
     "vx_decode_attn_qkv": (_i, [_vp, _vp, _vp, _f, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _f, _vp]),
+    "vx_prefill_attn_qkv": (_i, [_vp, _vp, _vp, _f, _i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _i,
+                                 _f, _i, _i, _vp, _vp, _vp]),
     "vx_decode_ffn_supported": (_i, [_vp, _vp, _vp, _vp]),
     "vx_qweight_pack": (_i, [_vp, _vp]),
     "vx_qweight_unpack": (_i, [_vp, _vp]),
