@@ -1185,24 +1185,54 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
     const int last_q = min(qt * FA_BQ + FA_BQ - 1, S - 1);
     const int n_keys = PAGED ? len_max[4] : last_q + 1;  // keys 0 .. n_keys-1 are visible to some query of the tile
     const int n_tiles = (n_keys + FA_BK - 1) / FA_BK;
-    for (int kt = 0; kt < n_tiles; kt++) {
-        __syncthreads();  // the previous tile's reads are done
-        for (int idx = tid; idx < FA_BK * (D / 8); idx += 256) {
+    // A tile's rows as they come from memory: requested a tile ahead, so that their way is covered by the
+    // arithmetic of the tile before (a thread's pieces: key idx % 32, columns 8 (idx / 32) .. + 7).
+    constexpr int NIDX = FA_BK * (D / 8) / 256;
+    static_assert(NIDX * 256 == FA_BK * (D / 8), "whole trips of the 256 threads over a tile");
+    float4 rk[PAGED ? 1 : NIDX][2], rv[PAGED ? 1 : NIDX][2];
+    half8 rkh[PAGED ? NIDX : 1], rvh[PAGED ? NIDX : 1];
+    auto fetch = [&](int kt) __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < NIDX; t++) {
+            const int idx = tid + 256 * t;
             const int key = idx % FA_BK, d8 = (idx / FA_BK) * 8;  // (lanes run over keys: V^T's 2-byte stores fill whole rows)
             const int ki = kt * FA_BK + key;
-            half8 kh = {0, 0, 0, 0, 0, 0, 0, 0}, vh = kh, kl = kh, vl = kh;
-            if (PAGED) {
+            if constexpr (PAGED) {
+                const half8 z = {0, 0, 0, 0, 0, 0, 0, 0};
+                rkh[t] = z;
+                rvh[t] = z;
                 if (ki < n_keys) {
                     const size_t part = (size_t)paged.block_size * ks;  // a block's K rows, then its V rows
                     const _Float16 *kp = paged.pool + (size_t)paged.table[ki / paged.block_size] * 2 * part +
                                          (size_t)(ki % paged.block_size) * ks + (size_t)kvh * D + d8;
-                    kh = *(const half8 *)kp;
-                    vh = *(const half8 *)(kp + part);
+                    rkh[t] = *(const half8 *)kp;
+                    rvh[t] = *(const half8 *)(kp + part);
                 }
-            } else if (ki < S) {
-                const float *kp = k + (size_t)ki * ks + (size_t)kvh * D + d8, *vp = v + (size_t)ki * ks + (size_t)kvh * D + d8;
-                const float4 k0 = *(const float4 *)kp, k1 = *(const float4 *)(kp + 4);
-                const float4 v0 = *(const float4 *)vp, v1 = *(const float4 *)(vp + 4);
+            } else {
+                const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
+                rk[t][0] = rk[t][1] = rv[t][0] = rv[t][1] = z;
+                if (ki < S) {
+                    const float *kp = k + (size_t)ki * ks + (size_t)kvh * D + d8, *vp = v + (size_t)ki * ks + (size_t)kvh * D + d8;
+                    rk[t][0] = *(const float4 *)kp;
+                    rk[t][1] = *(const float4 *)(kp + 4);
+                    rv[t][0] = *(const float4 *)vp;
+                    rv[t][1] = *(const float4 *)(vp + 4);
+                }
+            }
+        }
+    };
+    // what fetch() brought, as f16 halves into the LDS tiles (K rows, V transposed)
+    auto stash = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int t = 0; t < NIDX; t++) {
+            const int idx = tid + 256 * t;
+            const int key = idx % FA_BK, d8 = (idx / FA_BK) * 8;
+            half8 kh = {0, 0, 0, 0, 0, 0, 0, 0}, vh = kh, kl = kh, vl = kh;
+            if constexpr (PAGED) {
+                kh = rkh[t];
+                vh = rvh[t];
+            } else {
+                const float4 k0 = rk[t][0], k1 = rk[t][1], v0 = rv[t][0], v1 = rv[t][1];
                 const float kx[8] = {k0.x, k0.y, k0.z, k0.w, k1.x, k1.y, k1.z, k1.w};
                 const float vx[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
 #pragma unroll
@@ -1221,6 +1251,12 @@ __global__ void __launch_bounds__(256) prefill_fa2_kernel(const float *__restric
                 for (int e = 0; e < 8; e++) Vt[NLO - 1][(d8 + e) * VP + key] = vl[e];
             }
         }
+    };
+    if (n_tiles > 0) fetch(0);
+    for (int kt = 0; kt < n_tiles; kt++) {
+        __syncthreads();  // the previous tile's reads are done
+        stash();
+        if (kt + 1 < n_tiles) fetch(kt + 1);
         __syncthreads();
         if (kt * FA_BK >= wave_keys) continue;  // every key of the tile is beyond what the wave's queries see
         // S = Q K^T for the wave's 16 queries x 32 keys: lane holds S[row 4g+i][key cb*16 + c16]
