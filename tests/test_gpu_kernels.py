@@ -734,6 +734,21 @@ def test_rmsnorm_rope_silu_add_softmax_embedding_argmax(be):
     got = be.download(di, (6,), np.int32)
     assert list(got) == [nx.argmax(lg[r]) for r in range(6)]
     assert be.argmax(dl + 4 * 32000 * 4, 32000) == 31999
+    # ties between the columns one thread scans (4 t .. 4 t + 3, then 4096 further on), and rows that the vector
+    # scan does not take (a width that is no multiple of four: every second row also starts off a 16-byte boundary)
+    lg2 = rng.standard_normal((4, 8200)).astype(np.float32)
+    lg2[0, 9] = lg2[0, 4105] = lg2[0, 8] = 40.0
+    lg2[1, 4106] = lg2[1, 11] = 40.0
+    lg2[2, 8199] = lg2[2, 4103] = 40.0
+    lg2[3, 8196] = 40.0
+    d2, di2 = be.upload(lg2), be.alloc(4 * 4)
+    be.argmax_rows(d2, 4, 8200, di2)
+    assert list(be.download(di2, (4,), np.int32)) == [8, 11, 4103, 8196]
+    lg3 = rng.standard_normal((3, 333)).astype(np.float32)
+    lg3[1, 332] = lg3[1, 7] = 30.0
+    d3, di3 = be.upload(lg3), be.alloc(3 * 4)
+    be.argmax_rows(d3, 3, 333, di3)
+    assert list(be.download(di3, (3,), np.int32)) == [nx.argmax(lg3[r]) for r in range(3)]
     be.reset_pool()
 
 

@@ -303,11 +303,36 @@ __global__ void __launch_bounds__(1024) argmax_rows_kernel(const float *x, int n
     const float *xr = x + (size_t)blockIdx.x * n;
     float bv = -FLT_MAX;
     int bi = 0;
-    for (int j = threadIdx.x; j < n; j += blockDim.x) {
-        float v = xr[j];
-        if (v > bv) {
-            bv = v;
-            bi = j;
+    if (((uintptr_t)xr % 16) == 0 && n % 4 == 0) {
+        // four pieces of four columns in flight per thread (the comparisons form a chain; the loads need not wait for
+        // it), a thread's columns in rising order, so that its first maximum is the one with the lowest index
+        const int n4 = n / 4, step = (int)blockDim.x;
+        for (int j0 = threadIdx.x; j0 < n4; j0 += 4 * step) {
+            float4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int j = j0 + u * step;
+                v[u] = j < n4 ? ((const float4 *)xr)[j] : make_float4(-FLT_MAX, -FLT_MAX, -FLT_MAX, -FLT_MAX);
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int j = 4 * (j0 + u * step);
+                const float e[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+                for (int i = 0; i < 4; i++)
+                    if (e[i] > bv) {
+                        bv = e[i];
+                        bi = j + i;
+                    }
+            }
+        }
+    } else {
+        for (int j = threadIdx.x; j < n; j += blockDim.x) {
+            float v = xr[j];
+            if (v > bv) {
+                bv = v;
+                bi = j;
+            }
         }
     }
 #pragma unroll
