@@ -17,21 +17,34 @@ namespace {
 constexpr int PK_THREADS = 1024;
 
 // Exclusive scan over blockDim.x values held one per thread; returns the exclusive prefix and
-// writes the total to *total (same value in every thread).
+// writes the total to *total (same value in every thread). Each wave scans its 64 values by shuffles, the first wave
+// then the 16 waves' sums (sm: at least PK_THREADS / 64 ints).
 __device__ int block_exclusive_scan(int v, int *sm, int *total) {
-    const int tid = threadIdx.x;
-    sm[tid] = v;
-    __syncthreads();
-    for (int off = 1; off < PK_THREADS; off <<= 1) {
-        int t = (tid >= off) ? sm[tid - off] : 0;
-        __syncthreads();
-        sm[tid] += t;
-        __syncthreads();
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    constexpr int NWAVES = PK_THREADS / 64;
+    int incl = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int t = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += t;
     }
-    int incl = sm[tid];
-    *total = sm[PK_THREADS - 1];
+    __syncthreads();  // (whoever still reads sm from an earlier use is done)
+    if (lane == 63) sm[wave] = incl;
     __syncthreads();
-    return incl - v;
+    if (wave == 0) {
+        int w = lane < NWAVES ? sm[lane] : 0;
+#pragma unroll
+        for (int off = 1; off < NWAVES; off <<= 1) {
+            const int t = __shfl_up(w, off, 64);
+            if (lane >= off) w += t;
+        }
+        if (lane < NWAVES) sm[lane] = w;          // inclusive sums of the waves
+    }
+    __syncthreads();
+    const int before = wave > 0 ? sm[wave - 1] : 0;
+    *total = sm[NWAVES - 1];
+    __syncthreads();  // (the caller may write sm next)
+    return before + incl - v;
 }
 
 __global__ void __launch_bounds__(PK_THREADS) pack_batch_kernel(
@@ -60,14 +73,7 @@ __global__ void __launch_bounds__(PK_THREADS) pack_batch_kernel(
     bool fail = total_need > F || total_q != total_tokens;
     if (act && have + need > max_blocks) fail = true;
     // any thread's failure fails the step
-    sm[tid] = fail ? 1 : 0;
-    __syncthreads();
-    for (int off = PK_THREADS / 2; off > 0; off >>= 1) {
-        if (tid < off) sm[tid] |= sm[tid + off];
-        __syncthreads();
-    }
-    const bool any_fail = sm[0] != 0;
-    __syncthreads();
+    const bool any_fail = __syncthreads_or(fail ? 1 : 0) != 0;
     if (any_fail) {
         if (tid == 0) {
             *status = 1;
@@ -94,14 +100,16 @@ __global__ void __launch_bounds__(PK_THREADS) pack_batch_kernel(
             sm[tid] = rest;
             __syncthreads();
             int before = 0, partials = 0;  // partial items ahead of this one; partial items in all
-            for (int j = 0; j < batch; j++) {
-                const int rj = sm[j];
-                partials += rj > 0;
-                before += (rj > rest) || (rj == rest && rj > 0 && j < tid);
+            if (act || tid == 0) {  // (the threads without a sequence write nothing below)
+                for (int j = 0; j < batch; j++) {
+                    const int rj = sm[j];
+                    partials += rj > 0;
+                    before += (rj > rest) || (rj == rest && rj > 0 && j < tid);
+                }
             }
             __syncthreads();
             const int n_items = total_full + partials;
-            if (n_items <= cap) {
+            if (act && n_items <= cap) {
                 int4 *rec = (int4 *)(list + 4);  // one 16-byte record per item: everything a workgroup needs to start
                 for (int s2 = 0; s2 < full; s2++) rec[off + s2] = make_int4(tid, s2, len, slot);
                 if (rest > 0) rec[total_full + before] = make_int4(tid, full, len, slot);
