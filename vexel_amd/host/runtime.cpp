@@ -299,16 +299,17 @@ bool g_qkv_fusable(const vh_model *m, int layer, int rows) {
     return w.wq.data && w.wk.data && w.wv.data && fast(w.wq) && fast(w.wk) && fast(w.wv) &&
            vx_decode_attn_qkv_supported(&w.wq, &w.wk, &w.wv, m->cfg.head_dim) != 0;
 }
+// k_dense / v_dense (a prompt's first chunk): the rotated K and the V rows also as dense floats.
 int g_qkv_store(vh_model *m, int layer, const float *x, float *norm, float *q, int rows, const int32_t *d_pos,
-                const int32_t *d_slot) {
+                const int32_t *d_slot, float *k_dense = nullptr, float *v_dense = nullptr) {
     const vh_config &c = m->cfg;
     const vh_layer_weights &w = m->layers[layer];
     const vh_layer_extras &e = m->extras[layer];
     VHC(g_norm(m, x, w.attn_norm, e.attn_norm_bias, norm, rows));
     VXC(vx_prepare_act(m->be, norm, rows, c.hidden));
-    VXC(vx_decode_attn_qkv_ex(m->be, nullptr, nullptr, c.eps, 1, &w.wq, &w.wk, &w.wv, e.wq_bias, e.wk_bias, e.wv_bias, rows, d_pos,
-                              d_slot, m->kv[layer], c.kv_fp16, c.num_heads, c.num_kv_heads, c.head_dim, c.block_size,
-                              c.rope_theta, m->arch.rope_dim, m->arch.rope_neox, q));
+    VXC(vx_prefill_attn_qkv(m->be, nullptr, nullptr, c.eps, 1, &w.wq, &w.wk, &w.wv, e.wq_bias, e.wk_bias, e.wv_bias, rows, d_pos,
+                            d_slot, m->kv[layer], c.kv_fp16, c.num_heads, c.num_kv_heads, c.head_dim, c.block_size,
+                            c.rope_theta, m->arch.rope_dim, m->arch.rope_neox, q, k_dense, v_dense));
     return VH_OK;
 }
 
@@ -1108,6 +1109,14 @@ int vh_prefill(vh_model *m, const int32_t *tokens, int n, int64_t seq_id, int st
                 VXC(vx_sdpa_prefill_softcap(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale,
                                             m->arch.attn_softcap));
             else                                                                           // block.go:893-895
+                VXC(vx_sdpa_prefill(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale));
+        } else if (first && m->general && g_qkv_fusable(m, l, n)) {   // (a LayerNorm in front of the same fused projections)
+            if (chained) return fail("internal: prepared activation handed to a general layer");
+            VHC(g_qkv_store(m, l, x, norm, q, n, d_pos, d_slot, k, v));
+            if (m->arch.attn_softcap > 0.f)
+                VXC(vx_sdpa_prefill_softcap(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale,
+                                            m->arch.attn_softcap));
+            else
                 VXC(vx_sdpa_prefill(be, q, k, v, attn, n, c.num_heads, c.num_kv_heads, c.head_dim, scale));
         } else if (later && m->general && g_qkv_fusable(m, l, n)) {   // (a LayerNorm in front of the same fused projections)
             if (chained) return fail("internal: prepared activation handed to a general layer");
