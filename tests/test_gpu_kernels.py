@@ -405,7 +405,8 @@ def test_prepared_activation_paths(be):
                                                  (nx.FMT_Q6_K, 32, 512, 2816), (nx.FMT_Q6_K, 3, 1024, 1024),
                                                  (nx.FMT_Q8_0, 1, 512, 1024), (nx.FMT_Q4_K, 1, 1024, 2048),
                                                  (nx.FMT_Q6_K, 1, 1024, 2816), (nx.FMT_Q4_0, 1, 4096, 11008),
-                                                 (nx.FMT_Q4_0, 100, 512, 1024), (nx.FMT_Q6_K, 256, 512, 1024)])
+                                                 (nx.FMT_Q4_0, 100, 512, 1024), (nx.FMT_Q6_K, 256, 512, 1024),
+                                                 (nx.FMT_Q8_0, 300, 512, 2816), (nx.FMT_Q4_0, 512, 1024, 1024)])
 def test_fused_decode_blocks_equal_the_unfused_sequence(be, fmt, rows, hidden, ffn):
     """vx_decode_attn_qkv / vx_decode_ffn give what the one-call-per-operation sequence of
     runtime/block.go:834-1077 gives (float32 activations, F16 and F32 pools; one row goes through the
@@ -414,7 +415,9 @@ def test_fused_decode_blocks_equal_the_unfused_sequence(be, fmt, rows, hidden, f
     width, so its split-K slices differ from the separate launches': values agree to float32 summation
     order (1e-5 of the row magnitude), not bit for bit; a chained call equals a fresh one exactly."""
     rng = np.random.default_rng(77 + rows)
-    hq, hk, d, bs, nblocks, eps, theta = hidden // 64, 2, 64, 16, 24, 1e-5, 10000.0
+    hq, hk, d, bs, eps, theta = hidden // 64, 2, 64, 16, 1e-5, 10000.0
+    nblocks = max(24, (rows + bs - 1) // bs + 8)      # (a slot for every row)
+    assert nblocks * bs >= rows
     kvd = hk * d
     W = {name: qz.random_quant(fmt, rng, n, k) for name, (n, k) in
          dict(wq=(hidden, hidden), wk=(kvd, hidden), wv=(kvd, hidden), wo=(hidden, hidden), w1=(ffn, hidden),
