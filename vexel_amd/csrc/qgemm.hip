@@ -1385,6 +1385,18 @@ __global__ void __launch_bounds__(64) chunk_merge_kernel(const float *__restrict
     if (c == 0 && lane == 0) pv.inv_scale[r] = r < M ? 1.f : 0.f;
 }
 
+//   a plain activation row by row and chunk by chunk, row factor 1 (big prompt chunks: see vx_prepare_act)
+__global__ void __launch_bounds__(64) chunk_plain_kernel(const float *__restrict__ a, int M, int K, PrepView pv, int Mpad) {
+    const int c = blockIdx.x, r = blockIdx.y, lane = threadIdx.x;
+    float y[4] = {0.f, 0.f, 0.f, 0.f};
+    if (r < M) {
+        const float4 v = *(const float4 *)(a + (size_t)r * K + c * 256 + lane * 4);
+        y[0] = v.x; y[1] = v.y; y[2] = v.z; y[3] = v.w;
+    }
+    write_chunk(pv, r, c, y, Mpad);
+    if (c == 0 && lane == 0) pv.inv_scale[r] = r < M ? 1.f : 0.f;
+}
+
 // x <- x + inv_in * sum_ks P (residual add only; used after the last layer's down projection)
 __global__ void __launch_bounds__(256) add_partials_kernel(float *__restrict__ x, const float *__restrict__ P, int KS,
                                                            int M, int K, const float *__restrict__ inv_scale) {
@@ -2051,7 +2063,12 @@ int vx_prepare_act(vx_backend *be, const float *a, int m, int k) {
     rc = prep_begin(be, m, k, &pv);
     if (rc) return rc;
     const int mpad = mpad_for(m);
-    prepare_kernel<PREP_PLAIN, false><<<mpad, PREP_THREADS, 0, be->stream>>>(a, nullptr, nullptr, m, k, 0.f, pv, mpad);
+    // beyond 256 rows a wave per row and 256-column chunk (each chunk with its own power-of-two factor): many small
+    // workgroups instead of one of 1024 threads per row; up to there the row kernel, whose bits the decode paths share
+    if (m > 256)
+        chunk_plain_kernel<<<dim3(k / 256, mpad), 64, 0, be->stream>>>(a, m, k, pv, mpad);
+    else
+        prepare_kernel<PREP_PLAIN, false><<<mpad, PREP_THREADS, 0, be->stream>>>(a, nullptr, nullptr, m, k, 0.f, pv, mpad);
     VX_CHECK_LAUNCH();
     return VX_OK;
 }
