@@ -43,11 +43,11 @@ struct PoolChunk {
 
 }  // namespace vx
 
-// chunk-parallel prepares: up to 64 rows x 64 chunks of 256 columns; two [64][64] float arrays of per-chunk sums of squares
+// chunk-parallel prepares: up to 512 rows x 64 chunks of 256 columns; two [64][512] float arrays of per-chunk sums of squares
 #define VX_ROPE_TAB_ROWS 64
 #define VX_ATTN_CNT 16384
 #define VX_ROPE_TAB_PAIRS 128
-#define VX_PREP_SYNC_ROWS 64
+#define VX_PREP_SYNC_ROWS 512
 #define VX_PREP_SYNC_CHUNKS 64
 #define VX_PREP_SYNC_BYTES (2 * VX_PREP_SYNC_CHUNKS * VX_PREP_SYNC_ROWS * 4)
 

@@ -1932,6 +1932,8 @@ int launch_gemm_rows_r(vx_backend *be, const WavePlan &pl, const Segs &segs, int
     return launch_gemm_rows<W, 2>(be, segs, N, out, residual, to_partials, M, K, pl.ks, ks_out);
 }
 
+RowNorm cur_row_norm(const vx_backend *be);
+
 int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out, const float *residual,
                     bool to_partials, int M, int K, int *ks_out, const QkvEpi *epi_in = nullptr) {
     // packed copies of the matrices (vx_qweight_pack) and a decode-sized batch: the streaming kernel
@@ -1958,9 +1960,14 @@ int launch_gemm_fmt(vx_backend *be, int fmt, const Segs &segs, int N, float *out
         int ks = 1;
         const int mpad = mpad_for(M);
         const PrepView spv = prep_view(be, mpad, K);
-        int rc = tiles_gemm(be, fmt, segs.w, segs.n_end, 3, N, K, M, mpad, spv, out, residual, to_partials, &ks);
+        // (a pending 1/rms: this launch folds it into the plain row factors beside its own work, for whoever
+        // consumes its K slices' sums)
+        const bool fold = to_partials && be->prep_norm_k > 0;
+        const RowNorm fin = cur_row_norm(be);
+        int rc = tiles_gemm(be, fmt, segs.w, segs.n_end, 3, N, K, M, mpad, spv, out, residual, to_partials, &ks, fold ? &fin : nullptr);
         if (rc != VX_ERR_UNSUPPORTED) {
             if (rc) return rc;
+            if (fold) be->prep_norm_k = 0;
             be->last_matmul = "qtiles_kernel";
             if (ks_out) *ks_out = ks;
             if (!to_partials && ks > 1) {
@@ -2244,13 +2251,19 @@ static Segs make_segs(const vx_qweight *const *ws, int nw, int *ntot) {
     return sg;
 }
 
-// The chunk-parallel prepares cover decode-sized batches; larger ones keep the one-workgroup-per-row kernels.
-bool chunk_prepare_ok(int rows, int k) { return mpad_for(rows) <= VX_PREP_SYNC_ROWS && k / 256 <= VX_PREP_SYNC_CHUNKS; }
+// The chunk-parallel prepares (a wave per row and 256-column chunk) cover decode batches, prompt chunks and trees of
+// up to 512 rows; larger ones keep the one-workgroup-per-row kernels. VEXEL_HIP_PREP_ROW_KERNELS=1 (measurements):
+// those from 65 rows on, as before the many-rows GEMM folded the pending 1/rms in.
+bool chunk_prepare_ok(int rows, int k) {
+    static const bool row_kernels = getenv("VEXEL_HIP_PREP_ROW_KERNELS") != nullptr;
+    return mpad_for(rows) <= (row_kernels ? 64 : VX_PREP_SYNC_ROWS) && k / 256 <= VX_PREP_SYNC_CHUNKS;
+}
 
 extern "C++" {
 namespace vx {
 int prep_begin_chunked(vx_backend *be, int m, int k, PrepView *pv, int *mpad) {
-    if (k < 256 || k % 256 != 0 || !chunk_prepare_ok(m, k)) return VX_ERR_UNSUPPORTED;
+    // (the attention kernel that merges its own splits into this form: decode batches of up to 64 rows)
+    if (k < 256 || k % 256 != 0 || !chunk_prepare_ok(m, k) || mpad_for(m) > 64) return VX_ERR_UNSUPPORTED;
     *mpad = mpad_for(m);
     return prep_begin(be, m, k, pv);
 }

@@ -60,6 +60,7 @@ int stream_gemm_mixed(vx_backend *be, int fa, const uint8_t *wq, const uint8_t *
 // factors, residual) go to out; otherwise the slices' sums to be->part_ws, *ks_out of them.
 bool tiles_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M);
 int tiles_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M, int mpad,
-               const PrepView &pv, float *out, const float *residual, bool to_partials, int *ks_out);
+               const PrepView &pv, float *out, const float *residual, bool to_partials, int *ks_out,
+               const RowNorm *fin_norm = nullptr);  // fin_norm (to_partials only): a pending 1/rms the launch folds into pv.inv_scale
 
 }  // namespace vx

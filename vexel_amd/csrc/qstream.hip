@@ -861,13 +861,29 @@ __global__ void __launch_bounds__(64 * NW, 1)
 qtiles_kernel(const uint8_t *__restrict__ pw0, const uint8_t *__restrict__ pw1, const uint8_t *__restrict__ pw2,
               const half8 *__restrict__ a_tiles, const float *__restrict__ a_cscale, const float *__restrict__ a_inv_scale,
               const float *__restrict__ a_bsum, float *__restrict__ out, const float *__restrict__ residual,
-              float *__restrict__ partial, const StreamShape a, const int slices) {
+              float *__restrict__ partial, const StreamShape a, const int slices, const RowNorm fin, float *__restrict__ fin_rows) {
     constexpr int MT = 4;
     __shared__ half8 a_lds[2][4 * 512];
     typedef typename W::Ring Unit;
 
     const int tid = threadIdx.x, lane = tid & 63, ln = lane & 15, g = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    // A side job of a launch that leaves K slices' sums (it reads no row factors itself): the activation's pending
+    // 1/rms is folded into its plain row factors - finalize_row_norm_kernel's work, by up to eight workgroups of
+    // the first K slice per 64 rows, a row per wave and turn - so that whoever consumes the sums reads plain
+    // factors instead of adding up the chunks' sums of squares in every one of its waves.
+    if (fin.sspart && blockIdx.y == 0) {
+        const int nx = min((int)gridDim.x, 8);
+        if ((int)blockIdx.x < nx) {
+            for (int i = blockIdx.x + nx * wave; i < 64; i += nx * NW) {
+                const int r = blockIdx.z * 64 + i;
+                if (r < a.Mpad) {
+                    const float f = row_factor(fin_rows, fin, r);
+                    if (lane == 0) fin_rows[r] = f;
+                }
+            }
+        }
+    }
     const int n_tiles = a.N >> 4, mtiles = a.Mpad >> 4, n_hc = a.n_hc;
     const int t_own = (blockIdx.x * NW + wave) * R;          // first tile this wave writes
     const int t0 = max(min(t_own, n_tiles - R), 0);          // (a wave past the end works on the last tiles and writes nothing)
@@ -1435,10 +1451,10 @@ bool tiles_gemm_ok(vx_backend *be, int fmt, const uint8_t *const *w, const int *
 
 template <class W>
 static void launch_tiles(vx_backend *be, const TilesPlan &pl, dim3 grid, const PackedSegs &ps, const PrepView &pv, float *out,
-                         const float *residual, float *partial, const StreamShape &a, int slices) {
+                         const float *residual, float *partial, const StreamShape &a, int slices, const RowNorm &fin) {
 #define VX_TILES_LAUNCH(R_)                                                                                                    \
     qtiles_kernel<W, R_><<<grid, 64 * NW, 0, be->stream>>>(ps.w[0], ps.w[1], ps.w[2], pv.tiles, pv.cscale, pv.inv_scale, pv.bsum, out, \
-                                                           residual, partial, a, slices)
+                                                           residual, partial, a, slices, fin, pv.inv_scale)
     if (pl.r == 3) {
         if constexpr (!W::TWO_SCALES && !W::HAS_MIN) VX_TILES_LAUNCH(3);
     } else if (pl.r == 2) {
@@ -1452,9 +1468,12 @@ static void launch_tiles(vx_backend *be, const TilesPlan &pl, dim3 grid, const P
 // More than 64 rows over packed matrices. One K slice and no request for the slices' sums: the finished rows go to
 // out (row factors and the residual applied); otherwise [slice][M][N] sums go to be->part_ws and *ks_out says how many.
 int tiles_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_end, int nseg, int N, int K, int M, int mpad,
-               const PrepView &pv, float *out, const float *residual, bool to_partials, int *ks_out) {
+               const PrepView &pv, float *out, const float *residual, bool to_partials, int *ks_out, const RowNorm *fin_norm) {
     PackedSegs ps;
     if (!resolve(be, fmt, w, n_end, nseg, N, K, &ps)) return VX_ERR_UNSUPPORTED;
+    // (a pending 1/rms is folded in by the launch only where the launch itself reads no row factors)
+    if (fin_norm && !to_partials) return VX_ERR_UNSUPPORTED;
+    const RowNorm fin = fin_norm ? *fin_norm : RowNorm{nullptr, 0, 0.f, 0.f};
     static int cus = 0;
     if (cus == 0 && (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, be->device) != hipSuccess || cus <= 0)) cus = 256;
     const int n_hc = K / 128, mgroups = ceil_div(mpad, 64);
@@ -1483,12 +1502,12 @@ int tiles_gemm(vx_backend *be, int fmt, const uint8_t *const *w, const int *n_en
     const int slices = ((n_hc / pl.s) << 16) | (n_hc % pl.s);
     dim3 grid(ceil_div(N / 16, NW * pl.r), pl.s, mgroups);
     switch (fmt) {
-    case VX_Q4_0: launch_tiles<SQ4_0>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
+    case VX_Q4_0: launch_tiles<SQ4_0>(be, pl, grid, ps, pv, out, residual, partial, a, slices, fin); break;
     case VX_Q8_0:
-    case VX_Q5_0: launch_tiles<SQ8_0>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
-    case VX_Q5_K: launch_tiles<SQ5_K>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
-    case VX_Q4_K: launch_tiles<SQ4_K>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
-    default: launch_tiles<SQ6_K>(be, pl, grid, ps, pv, out, residual, partial, a, slices); break;
+    case VX_Q5_0: launch_tiles<SQ8_0>(be, pl, grid, ps, pv, out, residual, partial, a, slices, fin); break;
+    case VX_Q5_K: launch_tiles<SQ5_K>(be, pl, grid, ps, pv, out, residual, partial, a, slices, fin); break;
+    case VX_Q4_K: launch_tiles<SQ4_K>(be, pl, grid, ps, pv, out, residual, partial, a, slices, fin); break;
+    default: launch_tiles<SQ6_K>(be, pl, grid, ps, pv, out, residual, partial, a, slices, fin); break;
     }
     VX_CHECK_LAUNCH();
     if (ks_out) *ks_out = pl.s;
